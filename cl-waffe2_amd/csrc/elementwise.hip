@@ -1,0 +1,511 @@
+// elementwise.hip -- fp32 element-wise kernels over offset/stride/broadcast
+// views: a <- a op b, a <- b (copy), out <- f(x).
+//
+// Reference semantics: cl-waffe2-simd.c:153-250 (x[i*incx] <- x[i*incx] op
+// y[i*incy], in place in x), :586-768 (out <- f(x), out <- x^p), BLAS scopy
+// for MoveTensorNode (source/backends/cpu/arithmetic.lisp:39-61,125-144).
+// The reference reaches N-D views by wrapping those 1-D kernels in host loops
+// (call-with-view.lisp:112-229) -- thousands of calls for a row-broadcast or a
+// sliced operand; here a node is ONE launch over the normalised space.
+//
+// All of these are HBM-bound (8 or 12 bytes per element against a handful of
+// VALU instructions), so the kernels are organised around 16-byte coalesced
+// accesses: the "rows" kernel walks an innermost contiguous axis with float4
+// loads, several independent loads in flight per thread, and resolves the
+// outer axes (arbitrary strides, broadcast, slices) once per thread; the
+// "tile" kernel turns a transposed operand into coalesced reads AND writes
+// through an LDS tile; the "generic" kernel covers what is left.
+//
+// Arithmetic is IEEE binary32 with contraction disabled at build time
+// (-ffp-contract=off) so a+b, a*b ... are bit-identical to _mm256_*_ps.
+#include "wf2_common.h"
+#include "wf2_math.h"
+#include "wf2_view.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+// ---- functors: operator()(dst_value, src_value) ---------------------------
+struct OpAdd { __device__ __forceinline__ float operator()(float d, float s) const { return d + s; } };
+struct OpSub { __device__ __forceinline__ float operator()(float d, float s) const { return d - s; } };
+struct OpMul { __device__ __forceinline__ float operator()(float d, float s) const { return d * s; } };
+struct OpDiv { __device__ __forceinline__ float operator()(float d, float s) const { return d / s; } };
+struct OpMove { __device__ __forceinline__ float operator()(float, float s) const { return s; } };
+struct OpSin { __device__ __forceinline__ float operator()(float, float s) const { return sinf_(s); } };
+struct OpCos { __device__ __forceinline__ float operator()(float, float s) const { return cosf_(s); } };
+struct OpTanh { __device__ __forceinline__ float operator()(float, float s) const { return tanhf_(s); } };
+struct OpLog { __device__ __forceinline__ float operator()(float, float s) const { return logf_(s); } };
+struct OpExp { __device__ __forceinline__ float operator()(float, float s) const { return expf_(s); } };
+struct OpSqrt { __device__ __forceinline__ float operator()(float, float s) const { return sqrtf_(s); } };
+struct OpAbs { __device__ __forceinline__ float operator()(float, float s) const { return absf_(s); } };
+struct OpGelu { __device__ __forceinline__ float operator()(float, float s) const { return gelu_tanh_f(s); } };
+struct OpPow {
+  float p;
+  __device__ __forceinline__ float operator()(float, float s) const { return powf_(s, p); }
+};
+
+// ---- rows kernel ------------------------------------------------------------
+constexpr int kMaxOuter = WF2HIP_MAX_RANK - 1;
+
+struct RowsParams {
+  float* dst;
+  const float* src;
+  int64_t n0;     // extent of the innermost (contiguous) axis
+  uint32_t nrows; // product of the outer extents
+  int32_t src_inner;  // 1: src contiguous along the inner axis, 0: broadcast
+  int32_t nouter;
+  int32_t tpr_log2;  // threads that share one row segment
+  uint32_t chunks_per_row;
+  uint32_t oshape[kMaxOuter];  // outer axes, innermost of them first
+  int64_t odst[kMaxOuter];
+  int64_t osrc[kMaxOuter];
+};
+
+template <class F, bool ReadDst, int VEC, int U>
+__global__ __launch_bounds__(kBlock) void ew_rows(RowsParams p, F f) {
+  const int tpr = 1 << p.tpr_log2;
+  const int rpb = kBlock >> p.tpr_log2;
+  const int lane = threadIdx.x & (tpr - 1);
+  const int sub = threadIdx.x >> p.tpr_log2;
+  const uint32_t rblock = blockIdx.x / p.chunks_per_row;
+  const uint32_t chunk = blockIdx.x - rblock * p.chunks_per_row;
+  const uint32_t row = rblock * rpb + sub;
+  if (row >= p.nrows) return;
+
+  int64_t doff = 0, soff = 0;
+  uint32_t rem = row;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t idx;
+    if (i == p.nouter - 1) {
+      idx = rem;
+    } else {
+      uint32_t q = rem / p.oshape[i];
+      idx = rem - q * p.oshape[i];
+      rem = q;
+    }
+    doff += (int64_t)idx * p.odst[i];
+    soff += (int64_t)idx * p.osrc[i];
+  }
+  float* __restrict__ d = p.dst + doff;
+  const float* __restrict__ s = p.src + soff;
+  const int64_t col0 = (int64_t)chunk * U * tpr * VEC + (int64_t)lane * VEC;
+
+  if constexpr (VEC == 4) {
+    f4 dv[U], sv[U];
+    float sb = 0.0f;
+    if (!p.src_inner) sb = s[0];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t col = col0 + (int64_t)u * tpr * 4;
+      if (col + 4 <= p.n0) {
+        if constexpr (ReadDst) dv[u] = *reinterpret_cast<const f4*>(d + col);
+        if (p.src_inner) sv[u] = *reinterpret_cast<const f4*>(s + col);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t col = col0 + (int64_t)u * tpr * 4;
+      if (col + 4 <= p.n0) {
+        f4 a = ReadDst ? dv[u] : f4{0.f, 0.f, 0.f, 0.f};
+        f4 b = p.src_inner ? sv[u] : f4{sb, sb, sb, sb};
+        f4 r;
+        r.x = f(a.x, b.x);
+        r.y = f(a.y, b.y);
+        r.z = f(a.z, b.z);
+        r.w = f(a.w, b.w);
+        *reinterpret_cast<f4*>(d + col) = r;
+      } else if (col < p.n0) {  // ragged end of the row
+        for (int64_t c = col; c < p.n0; c++) {
+          float a = ReadDst ? d[c] : 0.0f;
+          float b = p.src_inner ? s[c] : sb;
+          d[c] = f(a, b);
+        }
+      }
+    }
+  } else {
+    float dv[U], sv[U];
+    float sb = 0.0f;
+    if (!p.src_inner) sb = s[0];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t col = col0 + (int64_t)u * tpr;
+      if (col < p.n0) {
+        if constexpr (ReadDst) dv[u] = d[col];
+        if (p.src_inner) sv[u] = s[col];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t col = col0 + (int64_t)u * tpr;
+      if (col < p.n0) {
+        float a = ReadDst ? dv[u] : 0.0f;
+        float b = p.src_inner ? sv[u] : sb;
+        d[col] = f(a, b);
+      }
+    }
+  }
+}
+
+// ---- generic kernel -----------------------------------------------------------
+struct GenParams {
+  float* dst;
+  const float* src;
+  int32_t rank;
+  int64_t total;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t sd[WF2HIP_MAX_RANK];
+  int64_t ss[WF2HIP_MAX_RANK];
+};
+
+template <class F, bool ReadDst, class Index>
+__global__ __launch_bounds__(kBlock) void ew_generic(GenParams p, F f) {
+  const Index total = (Index)p.total;
+  const Index step = (Index)gridDim.x * kBlock;
+  for (Index i = (Index)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    Index rem = i;
+    int64_t doff = 0, soff = 0;
+    for (int r = p.rank - 1; r > 0; r--) {
+      Index extent = (Index)p.shape[r];
+      Index q = rem / extent;
+      Index idx = rem - q * extent;
+      rem = q;
+      doff += (int64_t)idx * p.sd[r];
+      soff += (int64_t)idx * p.ss[r];
+    }
+    doff += (int64_t)rem * p.sd[0];
+    soff += (int64_t)rem * p.ss[0];
+    float a = ReadDst ? p.dst[doff] : 0.0f;
+    p.dst[doff] = f(a, p.src[soff]);
+  }
+}
+
+// ---- tile kernel: dst contiguous along one axis, src along another ------------
+// dst[..., j, ..., i] <- f(dst, src) where dst has stride 1 along axis I (the
+// innermost) and src has stride 1 along another axis J.  A 64x64 tile is read
+// with threads running along J (coalesced for src), parked in LDS, and written
+// with threads running along I (coalesced for dst).  The +1 padding keeps the
+// column reads free of LDS bank conflicts.
+constexpr int kTile = 64;
+
+struct TileParams {
+  float* dst;
+  const float* src;
+  int64_t ni, nj;        // extents of axis I and J
+  int64_t d_j;           // dst stride along J   (dst stride along I is 1)
+  int64_t s_i;           // src stride along I   (src stride along J is 1)
+  uint32_t tiles_i, tiles_j;
+  int32_t nouter;
+  uint32_t oshape[kMaxOuter];
+  int64_t odst[kMaxOuter];
+  int64_t osrc[kMaxOuter];
+};
+
+template <class F, bool ReadDst>
+__global__ __launch_bounds__(kBlock) void ew_tile(TileParams p, F f) {
+  __shared__ float tile[kTile][kTile + 1];
+  uint32_t bid = blockIdx.x;
+  const uint32_t ti = bid % p.tiles_i;
+  bid /= p.tiles_i;
+  const uint32_t tj = bid % p.tiles_j;
+  uint32_t rem = bid / p.tiles_j;
+  int64_t doff = 0, soff = 0;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t q = rem / p.oshape[i];
+    uint32_t idx = rem - q * p.oshape[i];
+    rem = q;
+    doff += (int64_t)idx * p.odst[i];
+    soff += (int64_t)idx * p.osrc[i];
+  }
+  const int64_t i0 = (int64_t)ti * kTile;
+  const int64_t j0 = (int64_t)tj * kTile;
+  const int tx = threadIdx.x & (kTile - 1);  // 0..63
+  const int ty = threadIdx.x >> 6;           // 0..3
+  // read: tx runs along J (src contiguous), rows of the tile are I
+  for (int r = ty; r < kTile; r += kBlock / kTile) {
+    int64_t i = i0 + r, j = j0 + tx;
+    if (i < p.ni && j < p.nj) tile[r][tx] = p.src[soff + i * p.s_i + j];
+  }
+  __syncthreads();
+  // write: tx runs along I (dst contiguous), rows are J
+  for (int r = ty; r < kTile; r += kBlock / kTile) {
+    int64_t i = i0 + tx, j = j0 + r;
+    if (i < p.ni && j < p.nj) {
+      float* dp = p.dst + doff + j * p.d_j + i;
+      float a = ReadDst ? *dp : 0.0f;
+      *dp = f(a, tile[tx][r]);
+    }
+  }
+}
+
+// ---- dispatch -------------------------------------------------------------------
+static inline int ilog2_ceil(int64_t v) {
+  int l = 0;
+  while (((int64_t)1 << l) < v) l++;
+  return l;
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <class F, bool ReadDst>
+static int launch_rows(const Space& s, float* dst, const float* src, F f) {
+  const int last = s.rank - 1;
+  RowsParams p;
+  p.dst = dst + s.off_a;
+  p.src = src + s.off_b;
+  p.n0 = s.shape[last];
+  p.src_inner = (int32_t)s.sb[last];
+  p.nouter = s.rank - 1;
+  int64_t nrows = 1;
+  bool vec_ok = aligned16(p.dst) && (!p.src_inner || aligned16(p.src));
+  for (int i = 0; i < p.nouter; i++) {
+    int r = last - 1 - i;
+    p.oshape[i] = (uint32_t)s.shape[r];
+    p.odst[i] = s.sa[r];
+    p.osrc[i] = s.sb[r];
+    nrows *= s.shape[r];
+    if (s.sa[r] % 4 != 0) vec_ok = false;
+    if (p.src_inner && s.sb[r] % 4 != 0) vec_ok = false;
+  }
+  p.nrows = (uint32_t)nrows;
+  const int vec = vec_ok ? 4 : 1;
+  const int64_t n0v = ceil_div(p.n0, vec);
+  int tl = ilog2_ceil(n0v);
+  if (tl > 8) tl = 8;
+  p.tpr_log2 = tl;
+  const int tpr = 1 << tl;
+  const int rpb = kBlock >> tl;
+  const bool deep = p.n0 >= (int64_t)tpr * vec * 4;
+  const int u = deep ? 4 : 1;
+  const int64_t chunks = ceil_div(p.n0, (int64_t)tpr * vec * u);
+  const int64_t blocks = ceil_div(nrows, rpb) * chunks;
+  if (blocks <= 0 || blocks >= ((int64_t)1 << 31))
+    return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+  p.chunks_per_row = (uint32_t)chunks;
+  hipStream_t st = rt().stream;
+  if (vec == 4 && deep)
+    ew_rows<F, ReadDst, 4, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p, f);
+  else if (vec == 4)
+    ew_rows<F, ReadDst, 4, 1><<<(uint32_t)blocks, kBlock, 0, st>>>(p, f);
+  else if (deep)
+    ew_rows<F, ReadDst, 1, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p, f);
+  else
+    ew_rows<F, ReadDst, 1, 1><<<(uint32_t)blocks, kBlock, 0, st>>>(p, f);
+  return after_launch("ew_rows");
+}
+
+template <class F, bool ReadDst>
+static int launch_generic(const Space& s, float* dst, const float* src, F f) {
+  GenParams p;
+  p.dst = dst + s.off_a;
+  p.src = src + s.off_b;
+  p.rank = s.rank;
+  p.total = s.total;
+  for (int r = 0; r < s.rank; r++) {
+    p.shape[r] = s.shape[r];
+    p.sd[r] = s.sa[r];
+    p.ss[r] = s.sb[r];
+  }
+  int64_t want = ceil_div(s.total, kBlock);
+  int64_t cap = (int64_t)rt().num_cus * 64;
+  uint32_t blocks = (uint32_t)(want < cap ? want : cap);
+  hipStream_t st = rt().stream;
+  if (s.total < ((int64_t)1 << 31))
+    ew_generic<F, ReadDst, uint32_t><<<blocks, kBlock, 0, st>>>(p, f);
+  else
+    ew_generic<F, ReadDst, int64_t><<<blocks, kBlock, 0, st>>>(p, f);
+  return after_launch("ew_generic");
+}
+
+// dst stride 1 on the last axis; src stride 1 on another axis J whose dst
+// stride is positive; both extents large enough for a tile to pay off.
+template <class F, bool ReadDst>
+static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, int* rc) {
+  const int last = s.rank - 1;
+  if (s.rank < 2 || s.sa[last] != 1 || s.sb[last] <= 1) return false;
+  int J = -1;
+  for (int r = 0; r < last; r++)
+    if (s.sb[r] == 1 && s.sa[r] > 0) J = r;
+  if (J < 0 || s.shape[last] < 16 || s.shape[J] < 16) return false;
+  TileParams p;
+  p.dst = dst + s.off_a;
+  p.src = src + s.off_b;
+  p.ni = s.shape[last];
+  p.nj = s.shape[J];
+  p.d_j = s.sa[J];
+  p.s_i = s.sb[last];
+  p.tiles_i = (uint32_t)ceil_div(p.ni, kTile);
+  p.tiles_j = (uint32_t)ceil_div(p.nj, kTile);
+  p.nouter = 0;
+  int64_t blocks = (int64_t)p.tiles_i * p.tiles_j;
+  for (int r = last - 1; r >= 0; r--) {
+    if (r == J) continue;
+    p.oshape[p.nouter] = (uint32_t)s.shape[r];
+    p.odst[p.nouter] = s.sa[r];
+    p.osrc[p.nouter] = s.sb[r];
+    p.nouter++;
+    blocks *= s.shape[r];
+  }
+  if (blocks >= ((int64_t)1 << 31)) return false;
+  ew_tile<F, ReadDst><<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(p, f);
+  *rc = after_launch("ew_tile");
+  return true;
+}
+
+// `s` describes dst through (sa, off_a) and src through (sb, off_b); dst has
+// no broadcast axis.
+template <class F, bool ReadDst>
+static int launch_elementwise(const Space& s, float* dst, const float* src, F f) {
+  const int last = s.rank - 1;
+  int64_t nrows = s.total / (s.shape[last] ? s.shape[last] : 1);
+  bool rows_ok = s.sa[last] == 1 && (s.sb[last] == 1 || s.sb[last] == 0) &&
+                 nrows < ((int64_t)1 << 31);
+  for (int r = 0; r < last; r++)
+    if (s.shape[r] >= ((int64_t)1 << 32)) rows_ok = false;
+  if (rows_ok) return launch_rows<F, ReadDst>(s, dst, src, f);
+  int rc = 0;
+  if (try_launch_tile<F, ReadDst>(s, dst, src, f, &rc)) return rc;
+  return launch_generic<F, ReadDst>(s, dst, src, f);
+}
+
+// For ops that overwrite dst (copy, unary) a broadcast dst axis means "the
+// last write wins", exactly what the reference's sequential loops leave
+// behind: keep only the last index of such axes.
+static void keep_last_write(Space* s) {
+  for (int r = 0; r < s->rank; r++) {
+    if (s->sa[r] == 0 && s->shape[r] > 1) {
+      s->off_b += s->sb[r] * (s->shape[r] - 1);
+      s->shape[r] = 1;
+    }
+  }
+  s->total = 1;
+  for (int r = 0; r < s->rank; r++) s->total *= s->shape[r];
+  normalise(s);
+}
+
+int launch_accumulate(int op, const Space& s, float* a, const float* b);  // reduce.hip
+
+int binary_nd(int op, Space s, float* a, const float* b) {
+  if (op < WF2HIP_ADD || op > WF2HIP_MOVE) return fail(WF2HIP_EINVAL, "unknown binary op %d", op);
+  if (s.total == 0) return 0;
+  if (!a || !b) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  normalise(&s);
+  if (hazardous_overlap(s, a, b))
+    return fail(WF2HIP_EOVERLAP,
+                "in-place op on partially overlapping windows of one buffer; "
+                "copy one operand first");
+  if (has_broadcast_axis(s, s.sa)) {
+    if (op != WF2HIP_MOVE) return launch_accumulate(op, s, a, b);
+    keep_last_write(&s);
+  }
+  switch (op) {
+    case WF2HIP_ADD: return launch_elementwise<OpAdd, true>(s, a, b, OpAdd{});
+    case WF2HIP_SUB: return launch_elementwise<OpSub, true>(s, a, b, OpSub{});
+    case WF2HIP_MUL: return launch_elementwise<OpMul, true>(s, a, b, OpMul{});
+    case WF2HIP_DIV: return launch_elementwise<OpDiv, true>(s, a, b, OpDiv{});
+    default: return launch_elementwise<OpMove, false>(s, a, b, OpMove{});
+  }
+}
+
+// x = source (described by the view's `a` side), out = destination (`b` side).
+int unary_nd(int op, Space s, const float* x, float* out, float p) {
+  if (s.total == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  // launch_elementwise wants dst on the `a` side
+  for (int r = 0; r < s.rank; r++) {
+    int64_t t = s.sa[r];
+    s.sa[r] = s.sb[r];
+    s.sb[r] = t;
+  }
+  int64_t t = s.off_a;
+  s.off_a = s.off_b;
+  s.off_b = t;
+  normalise(&s);
+  if (hazardous_overlap(s, out, x))
+    return fail(WF2HIP_EOVERLAP, "unary op between partially overlapping windows");
+  if (has_broadcast_axis(s, s.sa)) keep_last_write(&s);
+  switch (op) {
+    case WF2HIP_SIN: return launch_elementwise<OpSin, false>(s, out, x, OpSin{});
+    case WF2HIP_COS: return launch_elementwise<OpCos, false>(s, out, x, OpCos{});
+    case WF2HIP_TANH: return launch_elementwise<OpTanh, false>(s, out, x, OpTanh{});
+    case WF2HIP_LOG: return launch_elementwise<OpLog, false>(s, out, x, OpLog{});
+    case WF2HIP_EXP: return launch_elementwise<OpExp, false>(s, out, x, OpExp{});
+    case WF2HIP_SQRT: return launch_elementwise<OpSqrt, false>(s, out, x, OpSqrt{});
+    case WF2HIP_ABS: return launch_elementwise<OpAbs, false>(s, out, x, OpAbs{});
+    case WF2HIP_GELU: return launch_elementwise<OpGelu, false>(s, out, x, OpGelu{});
+    case WF2HIP_POW: return launch_elementwise<OpPow, false>(s, out, x, OpPow{p});
+    default: return fail(WF2HIP_EINVAL, "unknown unary op %d", op);
+  }
+}
+
+static int space_1d(long n, long inca, long incb, Space* s) {
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
+  s->rank = 1;
+  s->shape[0] = n;
+  s->sa[0] = inca;
+  s->sb[0] = incb;
+  s->off_a = s->off_b = 0;
+  s->total = n;
+  return 0;
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  return binary_nd(op, s, a, b);
+}
+
+WF2_API int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  return unary_nd(op, s, a, b, p);
+}
+
+#define WF2_DEFINE_BINARY_1D(name, OP)                                                   \
+  WF2_API int wf2hip_s##name(long n, float* x, long incx, const float* y, long incy) {  \
+    WF2_TRY(require_init());                                                             \
+    Space s;                                                                             \
+    WF2_TRY(space_1d(n, incx, incy, &s));                                                \
+    return binary_nd(OP, s, x, y);                                                       \
+  }
+
+WF2_DEFINE_BINARY_1D(add, WF2HIP_ADD)
+WF2_DEFINE_BINARY_1D(sub, WF2HIP_SUB)
+WF2_DEFINE_BINARY_1D(mul, WF2HIP_MUL)
+WF2_DEFINE_BINARY_1D(div, WF2HIP_DIV)
+
+WF2_API int wf2hip_scopy(long n, const float* y, long incy, float* x, long incx) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(space_1d(n, incx, incy, &s));
+  return binary_nd(WF2HIP_MOVE, s, x, y);
+}
+
+#define WF2_DEFINE_UNARY_1D(name, OP)                                                        \
+  WF2_API int wf2hip_s##name(long n, const float* x, long incx, float* out, long inco) {    \
+    WF2_TRY(require_init());                                                                 \
+    Space s;                                                                                 \
+    WF2_TRY(space_1d(n, incx, inco, &s));                                                    \
+    return unary_nd(OP, s, x, out, 0.0f);                                                    \
+  }
+
+WF2_DEFINE_UNARY_1D(sin, WF2HIP_SIN)
+WF2_DEFINE_UNARY_1D(cos, WF2HIP_COS)
+WF2_DEFINE_UNARY_1D(tanh, WF2HIP_TANH)
+WF2_DEFINE_UNARY_1D(log, WF2HIP_LOG)
+WF2_DEFINE_UNARY_1D(exp, WF2HIP_EXP)
+WF2_DEFINE_UNARY_1D(sqrt, WF2HIP_SQRT)
+WF2_DEFINE_UNARY_1D(abs, WF2HIP_ABS)
+
+WF2_API int wf2hip_spow(long n, const float* x, long incx, float p, float* out, long inco) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(space_1d(n, incx, inco, &s));
+  return unary_nd(WF2HIP_POW, s, x, out, p);
+}

@@ -1,0 +1,301 @@
+// gemm.hip -- fp32 gemm on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// Replaces the BLAS sgemm_ call behind MatMulNode
+// (source/backends/cpu/matrix-ops.lisp:12-237; binding
+// source/backends/cpu/blas-functions.lisp:34-38).  The public entry keeps
+// sgemm_'s column-major argument meaning so the Lisp side ports unchanged
+// (expand-gemm-form-column swaps operands: sgemm_(transB, transA, n, m, k, 1,
+// B, ldb, A, lda, 0, C, ldc) for a row-major C = A.B).
+//
+// Internally everything is row-major.  A column-major C(m x n, ldc) is the
+// row-major matrix Cr[n][m]; Cr = op(B)^T . op(A)^T, so the LEFT row-major
+// operand comes from B and the RIGHT one from A:
+//   transb 'N'  ->  left  stored [rows][k]   (k innermost)
+//   transb 'T'  ->  left  stored [k][rows]   (rows innermost)
+//   transa 'N'  ->  right stored [k][cols]   (cols innermost)
+//   transa 'T'  ->  right stored [cols][k]   (k innermost)
+// cl-waffe2's plain row-major matmul lands on (left k-innermost, right
+// cols-innermost), where both global reads are contiguous.
+//
+// Tiling: 128x128 per workgroup, K-step 16, 4 wavefronts in 2x2, each owning a
+// 64x64 block = 2x2 MFMA tiles of 32x32 (64 accumulator registers per lane).
+// Operand tiles are staged global -> registers -> LDS with two LDS buffers, so
+// one barrier per K-step; a k-innermost tile is kept [128][16+4] and read back
+// with one 128-bit LDS load per four MFMA steps (the +4 pad makes eight
+// consecutive lanes cover all 32 banks), an x-innermost tile is kept [16][128]
+// and read with conflict-free 32-bit loads.  Within a group of 8 k values,
+// MFMA step s takes k = s from lanes 0-31 and k = 4+s from lanes 32-63 for
+// both operands, which is what makes the 128-bit read usable.
+//
+// Bound: fp32 MFMA peak (157.3 TFLOP/s on MI355X); 2 m n k flop per product.
+#include "wf2_common.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int KPITCH = BK + 4;       // row pitch of a k-innermost LDS tile
+constexpr int TILE_FLOATS = BM * KPITCH;  // >= BK*BM, size of one operand buffer
+
+struct GemmParams {
+  const float* L;  // left operand  (rows = M)
+  const float* R;  // right operand (cols = N)
+  float* C;
+  int64_t M, N, K;
+  int64_t ldl, ldr, ldc;
+  int64_t sL, sR, sC;  // batch strides
+  float alpha, beta;
+  uint32_t tiles_m, tiles_n;
+};
+
+// Loads this thread's share of a 128 x 16 operand tile into registers.
+// KIN: operand stored [x][k] (k innermost) else [k][x].
+// FAST: 16-byte loads (pointer, pitch and extents checked on the host).
+template <bool KIN, bool FAST>
+__device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_t ld, int64_t x0,
+                                          int64_t k0, int64_t X, int64_t K, f4 (&reg)[2]) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int f = t + kBlock * j;  // float4 slot 0..511
+    int64_t x, k;
+    if (KIN) {
+      x = x0 + (f >> 2);
+      k = k0 + (f & 3) * 4;
+    } else {
+      k = k0 + (f >> 5);
+      x = x0 + (f & 31) * 4;
+    }
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    if (FAST) {
+      if (x < X && k < K) v = *reinterpret_cast<const f4*>(KIN ? base + x * ld + k : base + k * ld + x);
+    } else {
+      float e[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        int64_t xx = KIN ? x : x + c;
+        int64_t kk = KIN ? k + c : k;
+        if (xx < X && kk < K) e[c] = KIN ? base[xx * ld + kk] : base[kk * ld + xx];
+      }
+      v = f4{e[0], e[1], e[2], e[3]};
+    }
+    reg[j] = v;
+  }
+}
+
+template <bool KIN>
+__device__ __forceinline__ void store_tile(float* __restrict__ lds, const f4 (&reg)[2]) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int f = t + kBlock * j;
+    float* dst = KIN ? lds + (f >> 2) * KPITCH + (f & 3) * 4 : lds + (f >> 5) * BM + (f & 31) * 4;
+    *reinterpret_cast<f4*>(dst) = reg[j];
+  }
+}
+
+// Fragment for MFMA steps s = 0..3 of k-group `kb` (0 or 8): frag[s] is the
+// operand value for row/col (x0 + lane%32) at k = kb + 4*(lane/32) + s.
+template <bool KIN>
+__device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0, int kb, int lane,
+                                          float (&frag)[4]) {
+  const int xi = x0 + (lane & 31);
+  const int half = lane >> 5;
+  if (KIN) {
+    f4 v = *reinterpret_cast<const f4*>(lds + xi * KPITCH + kb + half * 4);
+    frag[0] = v.x; frag[1] = v.y; frag[2] = v.z; frag[3] = v.w;
+  } else {
+#pragma unroll
+    for (int s = 0; s < 4; s++) frag[s] = lds[(kb + half * 4 + s) * BM + xi];
+  }
+}
+
+template <bool LKIN, bool RKIN, bool FAST>
+__global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) float ldsL[2][TILE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float ldsR[2][TILE_FLOATS];
+
+  // Tile order: consecutive workgroups land on different XCDs (round robin),
+  // so give each XCD a contiguous band of tiles, and walk a band column-major
+  // in groups of 8 row-tiles so neighbours share operand panels in that L2.
+  const uint32_t ntiles = p.tiles_m * p.tiles_n;
+  uint32_t pid = blockIdx.x;
+  {
+    const uint32_t xcds = 8;
+    const uint32_t per = ntiles / xcds;
+    if (per > 0 && pid < per * xcds) pid = (pid % xcds) * per + pid / xcds;
+  }
+  const uint32_t group = 8;
+  const uint32_t width = group * p.tiles_n;
+  const uint32_t gid = pid / width;
+  const uint32_t first_m = gid * group;
+  const uint32_t gsize = (p.tiles_m - first_m) < group ? (p.tiles_m - first_m) : group;
+  const uint32_t tm = first_m + (pid % width) % gsize;
+  const uint32_t tn = (pid % width) / gsize;
+
+  const int64_t m0 = (int64_t)tm * BM;
+  const int64_t n0 = (int64_t)tn * BN;
+  const float* L = p.L + (int64_t)blockIdx.y * p.sL;
+  const float* R = p.R + (int64_t)blockIdx.y * p.sR;
+  float* C = p.C + (int64_t)blockIdx.y * p.sC;
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int wm = (wave >> 1) * 64;
+  const int wn = (wave & 1) * 64;
+
+  f16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  f4 regL[2], regR[2];
+  const int64_t ksteps = (p.K + BK - 1) / BK;
+  load_tile<LKIN, FAST>(L, p.ldl, m0, 0, p.M, p.K, regL);
+  load_tile<RKIN, FAST>(R, p.ldr, n0, 0, p.N, p.K, regR);
+  store_tile<LKIN>(ldsL[0], regL);
+  store_tile<RKIN>(ldsR[0], regR);
+  __syncthreads();
+
+  for (int64_t ks = 0; ks < ksteps; ks++) {
+    const int cur = (int)(ks & 1);
+    if (ks + 1 < ksteps) {
+      load_tile<LKIN, FAST>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
+      load_tile<RKIN, FAST>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
+    }
+#pragma unroll
+    for (int kb = 0; kb < BK; kb += 8) {
+      float a[2][4], b[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; i++) read_frag<LKIN>(ldsL[cur], wm + i * 32, kb, lane, a[i]);
+#pragma unroll
+      for (int j = 0; j < 2; j++) read_frag<RKIN>(ldsR[cur], wn + j * 32, kb, lane, b[j]);
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+    }
+    if (ks + 1 < ksteps) {
+      // The other buffer was last read in iteration ks-1, and every wave has
+      // passed the barrier that ended it.
+      store_tile<LKIN>(ldsL[cur ^ 1], regL);
+      store_tile<RKIN>(ldsR[cur ^ 1], regR);
+    }
+    __syncthreads();
+  }
+
+  // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int64_t col = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < p.M && col < p.N) {
+          float* c = C + row * p.ldc + col;
+          float v = p.alpha * acc[i][j][r];
+          if (p.beta != 0.0f) v += p.beta * *c;
+          *c = v;
+        }
+      }
+    }
+}
+
+static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; }
+
+static bool is_n(char c) { return c == 'N' || c == 'n'; }
+static bool is_t(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
+
+int sgemm_batched(char transa, char transb, long m, long n, long k, float alpha, const float* A,
+                  long lda, long strideA, const float* B, long ldb, long strideB, float beta,
+                  float* C, long ldc, long strideC, long batch) {
+  if (!(is_n(transa) || is_t(transa)) || !(is_n(transb) || is_t(transb)))
+    return fail(WF2HIP_EINVAL, "trans must be N, T or C");
+  if (m < 0 || n < 0 || k < 0 || batch < 0) return fail(WF2HIP_EINVAL, "negative dimension");
+  // sgemm_'s own leading-dimension rules (column-major)
+  const long rows_a = is_n(transa) ? m : k;
+  const long rows_b = is_n(transb) ? k : n;
+  if (lda < (rows_a > 1 ? rows_a : 1) || ldb < (rows_b > 1 ? rows_b : 1) || ldc < (m > 1 ? m : 1))
+    return fail(WF2HIP_EINVAL, "leading dimension too small (lda %ld ldb %ld ldc %ld)", lda, ldb,
+                ldc);
+  if (m == 0 || n == 0 || batch == 0) return 0;
+  if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
+  if (batch > 65535) return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+
+  GemmParams p;
+  // row-major view: Cr[n][m] = Left[n][k] . Right[k][m]
+  p.L = B;
+  p.R = A;
+  p.C = C;
+  p.M = n;
+  p.N = m;
+  p.K = k;
+  p.ldl = ldb;
+  p.ldr = lda;
+  p.ldc = ldc;
+  p.sL = strideB;
+  p.sR = strideA;
+  p.sC = strideC;
+  p.alpha = alpha;
+  p.beta = beta;
+  p.tiles_m = (uint32_t)ceil_div(p.M, BM);
+  p.tiles_n = (uint32_t)ceil_div(p.N, BN);
+  const bool lkin = is_n(transb);   // left stored [rows][k]
+  const bool rkin = !is_n(transa);  // right stored [cols][k]
+  int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
+  bool fast = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && strideA % 4 == 0 &&
+              strideB % 4 == 0;
+  // every 4-wide load must be wholly inside or wholly outside the matrix
+  fast = fast && (lkin ? k % 4 == 0 : p.M % 4 == 0) && (rkin ? k % 4 == 0 : p.N % 4 == 0);
+  dim3 grid((uint32_t)blocks, (uint32_t)batch);
+  hipStream_t st = rt().stream;
+#define WF2_GEMM_LAUNCH(LK, RK)                                                   \
+  do {                                                                            \
+    if (fast)                                                                     \
+      sgemm_kernel<LK, RK, true><<<grid, kBlock, 0, st>>>(p);                     \
+    else                                                                          \
+      sgemm_kernel<LK, RK, false><<<grid, kBlock, 0, st>>>(p);                    \
+  } while (0)
+  if (lkin && rkin)
+    WF2_GEMM_LAUNCH(true, true);
+  else if (lkin)
+    WF2_GEMM_LAUNCH(true, false);
+  else if (rkin)
+    WF2_GEMM_LAUNCH(false, true);
+  else
+    WF2_GEMM_LAUNCH(false, false);
+#undef WF2_GEMM_LAUNCH
+  return after_launch("sgemm_kernel");
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_sgemm(char transa, char transb, long m, long n, long k, float alpha,
+                         const float* A, long lda, const float* B, long ldb, float beta, float* C,
+                         long ldc) {
+  WF2_TRY(require_init());
+  return sgemm_batched(transa, transb, m, n, k, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1);
+}
+
+WF2_API int wf2hip_sgemm_strided_batched(char transa, char transb, long m, long n, long k,
+                                         float alpha, const float* A, long lda, long strideA,
+                                         const float* B, long ldb, long strideB, float beta,
+                                         float* C, long ldc, long strideC, long batch) {
+  WF2_TRY(require_init());
+  return sgemm_batched(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C,
+                       ldc, strideC, batch);
+}

@@ -1,0 +1,693 @@
+// reduce.hip -- accumulation into stride-0 destinations (cl-waffe2's !sum /
+// !mean), max/min, and the fused row kernels (softmax, causal softmax,
+// LayerNorm).
+//
+// cl-waffe2 has no reduction node: (!sum x :axis k) zero-fills `out`, views it
+// with (:broadcast n) on the reduced axes and runs AddNode into that view
+// (source/base-impl/reduction.lisp:5-79), so the CPU kernel is called with
+// incx == 0 and adds sequentially into one float (cl-waffe2-simd.c:159,
+// 205-212).  On the GPU the same node becomes a parallel reduction:
+// wavefront shuffles inside a 64-lane wave, LDS across the four waves of a
+// workgroup, and a second tiny pass when a row has to be split over
+// workgroups.  Partial sums are kept in binary64 (binary64 adds issue at the
+// binary32 rate on CDNA) and rounded once, so the result is closer to the
+// exact sum than the reference's own sequential binary32 order; reduce mode 1
+// reproduces that order exactly for bit-parity checks.
+//
+// All kernels here are HBM-bound: 4 bytes read per element reduced, 8 bytes
+// per element for softmax/LayerNorm (one read, one write).
+#include "wf2_common.h"
+#include "wf2_math.h"
+#include "wf2_view.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+constexpr int kMaxOuter = WF2HIP_MAX_RANK - 1;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
+  return v;
+}
+
+// Sum over the workgroup in a fixed order; valid in thread 0.
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
+  __syncthreads();
+  double t = 0.0;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < kWavesPerBlock; i++) t += lds[i];
+  }
+  return t;
+}
+
+// ---- row reduction: a[row] += sum_c b[row, c] ---------------------------------
+struct RowRedParams {
+  float* a;
+  const float* b;
+  int64_t n0;       // reduced (innermost, contiguous) extent
+  uint32_t nrows;
+  int32_t nouter;
+  uint32_t oshape[kMaxOuter];  // kept axes, innermost of them first
+  int64_t oa[kMaxOuter];
+  int64_t ob[kMaxOuter];
+  uint32_t splits;  // workgroups per row
+  int64_t seg;      // elements per split (multiple of 4)
+  double* partials; // nrows*splits, used when splits > 1
+};
+
+__device__ __forceinline__ void row_offsets(const RowRedParams& p, uint32_t row, int64_t* aoff,
+                                            int64_t* boff) {
+  int64_t ao = 0, bo = 0;
+  uint32_t rem = row;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t idx;
+    if (i == p.nouter - 1) {
+      idx = rem;
+    } else {
+      uint32_t q = rem / p.oshape[i];
+      idx = rem - q * p.oshape[i];
+      rem = q;
+    }
+    ao += (int64_t)idx * p.oa[i];
+    bo += (int64_t)idx * p.ob[i];
+  }
+  *aoff = ao;
+  *boff = bo;
+}
+
+// Sum of b[lo, hi) by `nthreads` cooperating threads; `t` is this thread's
+// rank among them.  VEC == 4 needs b + lo 16-byte aligned.
+template <int VEC>
+__device__ __forceinline__ double strided_sum(const float* __restrict__ b, int64_t lo, int64_t hi,
+                                              int t, int nthreads) {
+  double acc0 = 0.0, acc1 = 0.0;
+  if constexpr (VEC == 4) {
+    int64_t nvec = (hi - lo) / 4;
+    const f4* bv = reinterpret_cast<const f4*>(b + lo);
+    int64_t i = t;
+    for (; i + nthreads < nvec; i += 2 * (int64_t)nthreads) {
+      f4 v0 = bv[i];
+      f4 v1 = bv[i + nthreads];
+      acc0 += ((double)v0.x + (double)v0.y) + ((double)v0.z + (double)v0.w);
+      acc1 += ((double)v1.x + (double)v1.y) + ((double)v1.z + (double)v1.w);
+    }
+    if (i < nvec) {
+      f4 v0 = bv[i];
+      acc0 += ((double)v0.x + (double)v0.y) + ((double)v0.z + (double)v0.w);
+    }
+    for (int64_t c = lo + nvec * 4 + t; c < hi; c += nthreads) acc1 += (double)b[c];
+  } else {
+    for (int64_t c = lo + t; c < hi; c += nthreads) acc0 += (double)b[c];
+  }
+  return acc0 + acc1;
+}
+
+// One workgroup per (row, split).
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_rows_block(RowRedParams p) {
+  __shared__ double lds[kWavesPerBlock];
+  const uint32_t row = blockIdx.x / p.splits;
+  const uint32_t split = blockIdx.x - row * p.splits;
+  int64_t aoff, boff;
+  row_offsets(p, row, &aoff, &boff);
+  int64_t lo = (int64_t)split * p.seg;
+  int64_t hi = lo + p.seg < p.n0 ? lo + p.seg : p.n0;
+  double v = strided_sum<VEC>(p.b + boff, lo, hi, threadIdx.x, kBlock);
+  double total = block_sum(v, lds);
+  if (threadIdx.x == 0) {
+    if (p.splits == 1)
+      p.a[aoff] = (float)((double)p.a[aoff] + total);
+    else
+      p.partials[(int64_t)row * p.splits + split] = total;
+  }
+}
+
+// One wavefront per row, four rows per workgroup.
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_rows_wave(RowRedParams p) {
+  const uint32_t row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= p.nrows) return;
+  int64_t aoff, boff;
+  row_offsets(p, row, &aoff, &boff);
+  double v = strided_sum<VEC>(p.b + boff, 0, p.n0, threadIdx.x & (kWave - 1), kWave);
+  v = wave_sum(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) p.a[aoff] = (float)((double)p.a[aoff] + v);
+}
+
+__global__ __launch_bounds__(kBlock) void reduce_rows_finish(RowRedParams p) {
+  const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
+  if (row >= p.nrows) return;
+  int64_t aoff, boff;
+  row_offsets(p, row, &aoff, &boff);
+  double t = 0.0;
+  for (uint32_t s = 0; s < p.splits; s++) t += p.partials[(int64_t)row * p.splits + s];
+  p.a[aoff] = (float)((double)p.a[aoff] + t);
+}
+
+// ---- generic accumulation: one wavefront per destination element ----------------
+struct AccParams {
+  float* a;
+  const float* b;
+  int32_t nk, nr;                       // kept / reduced axis counts
+  int64_t nout, nred;
+  int64_t kshape[WF2HIP_MAX_RANK], ka[WF2HIP_MAX_RANK], kb[WF2HIP_MAX_RANK];
+  int64_t rshape[WF2HIP_MAX_RANK], rb[WF2HIP_MAX_RANK];  // outermost first
+};
+
+__device__ __forceinline__ void kept_offsets(const AccParams& p, int64_t out, int64_t* aoff,
+                                             int64_t* boff) {
+  int64_t ao = 0, bo = 0, rem = out;
+  for (int i = p.nk - 1; i >= 0; i--) {
+    int64_t q = rem / p.kshape[i];
+    int64_t idx = rem - q * p.kshape[i];
+    rem = q;
+    ao += idx * p.ka[i];
+    bo += idx * p.kb[i];
+  }
+  *aoff = ao;
+  *boff = bo;
+}
+
+__device__ __forceinline__ int64_t reduced_offset(const AccParams& p, int64_t j) {
+  int64_t off = 0, rem = j;
+  for (int i = p.nr - 1; i >= 0; i--) {
+    int64_t q = rem / p.rshape[i];
+    int64_t idx = rem - q * p.rshape[i];
+    rem = q;
+    off += idx * p.rb[i];
+  }
+  return off;
+}
+
+__global__ __launch_bounds__(kBlock) void accumulate_generic(AccParams p) {
+  const int64_t out = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (out >= p.nout) return;
+  int64_t aoff, boff;
+  kept_offsets(p, out, &aoff, &boff);
+  const int lane = threadIdx.x & (kWave - 1);
+  double acc = 0.0;
+  for (int64_t j = lane; j < p.nred; j += kWave) acc += (double)p.b[boff + reduced_offset(p, j)];
+  acc = wave_sum(acc);
+  if (lane == 0) p.a[aoff] = (float)((double)p.a[aoff] + acc);
+}
+
+// The reference's order: for one destination element, visit the reduced index
+// space in row-major order and apply a <- a op b in binary32 each time.
+template <class F>
+__global__ __launch_bounds__(kBlock) void accumulate_sequential(AccParams p, F f) {
+  const int64_t out = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (out >= p.nout) return;
+  int64_t aoff, boff;
+  kept_offsets(p, out, &aoff, &boff);
+  float acc = p.a[aoff];
+  const int64_t inner = p.rshape[p.nr - 1];
+  const int64_t inner_stride = p.rb[p.nr - 1];
+  const int64_t outer = p.nred / inner;
+  for (int64_t o = 0; o < outer; o++) {
+    int64_t base = boff + reduced_offset(p, o * inner);
+    for (int64_t i = 0; i < inner; i++) acc = f(acc, p.b[base + i * inner_stride]);
+  }
+  p.a[aoff] = acc;
+}
+
+struct SeqAdd { __device__ __forceinline__ float operator()(float d, float s) const { return d + s; } };
+struct SeqSub { __device__ __forceinline__ float operator()(float d, float s) const { return d - s; } };
+struct SeqMul { __device__ __forceinline__ float operator()(float d, float s) const { return d * s; } };
+struct SeqDiv { __device__ __forceinline__ float operator()(float d, float s) const { return d / s; } };
+
+static void split_axes(const Space& s, AccParams* p) {
+  p->nk = p->nr = 0;
+  p->nout = p->nred = 1;
+  for (int r = 0; r < s.rank; r++) {
+    if (s.sa[r] == 0 && s.shape[r] > 1) {
+      p->rshape[p->nr] = s.shape[r];
+      p->rb[p->nr] = s.sb[r];
+      p->nr++;
+      p->nred *= s.shape[r];
+    } else {
+      p->kshape[p->nk] = s.shape[r];
+      p->ka[p->nk] = s.sa[r];
+      p->kb[p->nk] = s.sb[r];
+      p->nk++;
+      p->nout *= s.shape[r];
+    }
+  }
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+static int launch_row_reduce(const Space& s, float* a, const float* b) {
+  const int last = s.rank - 1;
+  RowRedParams p;
+  p.a = a + s.off_a;
+  p.b = b + s.off_b;
+  p.n0 = s.shape[last];
+  p.nouter = s.rank - 1;
+  int64_t nrows = 1;
+  bool vec_ok = aligned16(p.b);
+  for (int i = 0; i < p.nouter; i++) {
+    int r = last - 1 - i;
+    p.oshape[i] = (uint32_t)s.shape[r];
+    p.oa[i] = s.sa[r];
+    p.ob[i] = s.sb[r];
+    nrows *= s.shape[r];
+    if (s.sb[r] % 4 != 0) vec_ok = false;
+  }
+  p.nrows = (uint32_t)nrows;
+  p.partials = reinterpret_cast<double*>(rt().partials);
+  p.splits = 1;
+  p.seg = p.n0;
+  hipStream_t st = rt().stream;
+  const int64_t target_blocks = (int64_t)rt().num_cus * 8;
+  if (p.n0 < 2048 && nrows * 1 >= 1) {
+    // short rows: a wavefront each
+    if (nrows >= target_blocks || p.n0 < 8192) {
+      uint32_t blocks = (uint32_t)ceil_div(nrows, kWavesPerBlock);
+      if (vec_ok)
+        reduce_rows_wave<4><<<blocks, kBlock, 0, st>>>(p);
+      else
+        reduce_rows_wave<1><<<blocks, kBlock, 0, st>>>(p);
+      return after_launch("reduce_rows_wave");
+    }
+  }
+  if (nrows < target_blocks) {
+    int64_t by_work = ceil_div(p.n0, 16384);
+    int64_t by_fill = ceil_div(target_blocks, nrows);
+    int64_t by_cap = (kPartialCapacity / 2) / nrows;
+    int64_t splits = by_work < by_fill ? by_work : by_fill;
+    if (splits > by_cap) splits = by_cap;
+    if (splits < 1) splits = 1;
+    int64_t seg = ceil_div(ceil_div(p.n0, splits), 1024) * 1024;
+    splits = ceil_div(p.n0, seg);
+    p.splits = (uint32_t)splits;
+    p.seg = seg;
+  }
+  int64_t blocks = nrows * p.splits;
+  if (blocks >= ((int64_t)1 << 31))
+    return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+  if (vec_ok)
+    reduce_rows_block<4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else
+    reduce_rows_block<1><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  WF2_TRY(after_launch("reduce_rows_block"));
+  if (p.splits > 1) {
+    reduce_rows_finish<<<(uint32_t)ceil_div(nrows, kBlock), kBlock, 0, st>>>(p);
+    WF2_TRY(after_launch("reduce_rows_finish"));
+  }
+  return 0;
+}
+
+// a <- a op b where `a` has broadcast (stride-0) axes.  `s` is normalised.
+int launch_accumulate(int op, const Space& s, float* a, const float* b) {
+  hipStream_t st = rt().stream;
+  const bool sequential = op != WF2HIP_ADD || rt().reduce_mode == 1;
+  AccParams p;
+  p.a = a + s.off_a;
+  p.b = b + s.off_b;
+  split_axes(s, &p);
+  if (sequential) {
+    if (p.nout >= ((int64_t)1 << 31) * kBlock)
+      return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+    uint32_t blocks = (uint32_t)ceil_div(p.nout, kBlock);
+    switch (op) {
+      case WF2HIP_ADD: accumulate_sequential<SeqAdd><<<blocks, kBlock, 0, st>>>(p, SeqAdd{}); break;
+      case WF2HIP_SUB: accumulate_sequential<SeqSub><<<blocks, kBlock, 0, st>>>(p, SeqSub{}); break;
+      case WF2HIP_MUL: accumulate_sequential<SeqMul><<<blocks, kBlock, 0, st>>>(p, SeqMul{}); break;
+      case WF2HIP_DIV: accumulate_sequential<SeqDiv><<<blocks, kBlock, 0, st>>>(p, SeqDiv{}); break;
+      default: return fail(WF2HIP_EINVAL, "op %d cannot accumulate", op);
+    }
+    return after_launch("accumulate_sequential");
+  }
+  // Row form: the only reduced axis is the innermost one and b is contiguous
+  // along it; every other axis is kept.
+  const int last = s.rank - 1;
+  bool row_form = s.sa[last] == 0 && s.sb[last] == 1 && p.nr == 1 &&
+                  p.nout < ((int64_t)1 << 31);
+  for (int r = 0; r < last; r++)
+    if (s.shape[r] >= ((int64_t)1 << 32)) row_form = false;
+  if (row_form) return launch_row_reduce(s, a, b);
+  int64_t blocks = ceil_div(p.nout, kWavesPerBlock);
+  if (blocks >= ((int64_t)1 << 31))
+    return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+  accumulate_generic<<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  return after_launch("accumulate_generic");
+}
+
+// ---- max / min ------------------------------------------------------------------
+template <bool IsMax>
+__global__ __launch_bounds__(kBlock) void maxmin_pass(const float* __restrict__ x, int64_t n,
+                                                      int64_t incx, float* __restrict__ out) {
+  __shared__ float lds[kWavesPerBlock];
+  float best = x[0];
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    float v = x[i * incx];
+    best = IsMax ? fmaxf(best, v) : fminf(best, v);
+  }
+  best = IsMax ? wave_max(best) : wave_min(best);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < kWavesPerBlock; i++) best = IsMax ? fmaxf(best, lds[i]) : fminf(best, lds[i]);
+    out[blockIdx.x] = best;
+  }
+}
+
+template <bool IsMax>
+static int launch_maxmin(long n, const float* x, long incx, float* out) {
+  if (n <= 0) return fail(WF2HIP_EINVAL, "max/min of an empty range");
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null pointer");
+  hipStream_t st = rt().stream;
+  int64_t blocks = ceil_div(n, kBlock * 16);
+  if (blocks > 1024) blocks = 1024;
+  if (blocks == 1) {
+    maxmin_pass<IsMax><<<1, kBlock, 0, st>>>(x, n, incx, out);
+    return after_launch("maxmin");
+  }
+  float* partial = rt().partials;
+  maxmin_pass<IsMax><<<(uint32_t)blocks, kBlock, 0, st>>>(x, n, incx, partial);
+  WF2_TRY(after_launch("maxmin pass 1"));
+  maxmin_pass<IsMax><<<1, kBlock, 0, st>>>(partial, blocks, 1, out);
+  return after_launch("maxmin pass 2");
+}
+
+// ---- fused row kernels: one wavefront per row, the row held in registers --------
+// Lane l of the wave owns NV groups of 4 consecutive columns, group g starting
+// at column (g*64 + l)*4 (16-byte coalesced) or, when the row cannot be read
+// with 16-byte loads, columns (g*4 + c)*64 + l.
+template <int NV, bool VEC>
+struct RowRegs {
+  float v[NV][4];
+
+  __device__ __forceinline__ static int64_t col(int g, int c, int lane) {
+    return VEC ? ((int64_t)(g * kWave + lane) * 4 + c) : ((int64_t)(g * 4 + c) * kWave + lane);
+  }
+
+  __device__ __forceinline__ void load(const float* __restrict__ row, int64_t ncols, int lane,
+                                       float fill) {
+#pragma unroll
+    for (int g = 0; g < NV; g++) {
+      if (VEC && col(g, 3, lane) < ncols) {
+        f4 t = *reinterpret_cast<const f4*>(row + col(g, 0, lane));
+        v[g][0] = t.x; v[g][1] = t.y; v[g][2] = t.z; v[g][3] = t.w;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          int64_t cc = col(g, c, lane);
+          v[g][c] = cc < ncols ? row[cc] : fill;
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(float* __restrict__ row, int64_t ncols, int lane) const {
+#pragma unroll
+    for (int g = 0; g < NV; g++) {
+      if (VEC && col(g, 3, lane) < ncols) {
+        f4 t = {v[g][0], v[g][1], v[g][2], v[g][3]};
+        *reinterpret_cast<f4*>(row + col(g, 0, lane)) = t;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          int64_t cc = col(g, c, lane);
+          if (cc < ncols) row[cc] = v[g][c];
+        }
+      }
+    }
+  }
+};
+
+// softmax over the first `valid` columns of a row; columns valid..ncols-1 of
+// the output are set to 0 (used by the causal form).
+template <int NV, bool VEC>
+__global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restrict__ x, int64_t ldx,
+                                                            float* __restrict__ out, int64_t ldo,
+                                                            int64_t nrows, int64_t ncols,
+                                                            int64_t causal_seq, float scale) {
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= nrows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
+  const float ninf = -__builtin_inff();
+  RowRegs<NV, VEC> r;
+  r.load(x + row * ldx, valid, lane, ninf);
+  float m = ninf;
+#pragma unroll
+  for (int g = 0; g < NV; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      if (causal_seq > 0) {
+        // binary32 product, like a MulNode; padding stays -inf whatever the sign of scale
+        bool in = RowRegs<NV, VEC>::col(g, c, lane) < valid;
+        r.v[g][c] = in ? r.v[g][c] * scale : ninf;
+      }
+      m = fmaxf(m, r.v[g][c]);
+    }
+  m = wave_max(m);
+  double e[NV][4];
+  double sum = 0.0;
+#pragma unroll
+  for (int g = 0; g < NV; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      float d = r.v[g][c] - m;  // binary32 subtraction, like a SubNode
+      // exp underflows to +0 below -104; -inf (padding) must give exactly 0
+      double ed = (d < -104.0f) ? 0.0 : exp_core((double)d);
+      e[g][c] = ed;
+      sum += ed;
+    }
+  sum = wave_sum(sum);
+  const double inv = 1.0 / sum;
+#pragma unroll
+  for (int g = 0; g < NV; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) r.v[g][c] = (float)(e[g][c] * inv);
+  r.store(out + row * ldo, ncols, lane);
+}
+
+// Rows too long for registers: one workgroup per row, three passes (the second
+// and third hit L2).
+__global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __restrict__ x, int64_t ldx,
+                                                             float* __restrict__ out, int64_t ldo,
+                                                             int64_t ncols) {
+  __shared__ float lmax[kWavesPerBlock];
+  __shared__ double lsum[kWavesPerBlock];
+  const float* xr = x + (int64_t)blockIdx.x * ldx;
+  float* orow = out + (int64_t)blockIdx.x * ldo;
+  float m = -__builtin_inff();
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) m = fmaxf(m, xr[c]);
+  m = wave_max(m);
+  if ((threadIdx.x & (kWave - 1)) == 0) lmax[threadIdx.x / kWave] = m;
+  __syncthreads();
+  m = lmax[0];
+  for (int i = 1; i < kWavesPerBlock; i++) m = fmaxf(m, lmax[i]);
+  double s = 0.0;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
+    float d = xr[c] - m;
+    s += (d < -104.0f) ? 0.0 : exp_core((double)d);
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & (kWave - 1)) == 0) lsum[threadIdx.x / kWave] = s;
+  __syncthreads();
+  s = 0.0;
+  for (int i = 0; i < kWavesPerBlock; i++) s += lsum[i];
+  const double inv = 1.0 / s;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
+    float d = xr[c] - m;
+    double ed = (d < -104.0f) ? 0.0 : exp_core((double)d);
+    orow[c] = (float)(ed * inv);
+  }
+}
+
+template <int NV, bool VEC>
+__global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __restrict__ x,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta,
+                                                              float eps, float* __restrict__ out,
+                                                              int64_t nrows, int64_t ncols) {
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= nrows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  RowRegs<NV, VEC> r, g, b;
+  r.load(x + row * ncols, ncols, lane, 0.0f);
+  g.load(gamma, ncols, lane, 0.0f);
+  b.load(beta, ncols, lane, 0.0f);
+  double sum = 0.0;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) sum += (double)r.v[i][c];
+  const double mean = wave_sum(sum) / (double)ncols;
+  double sq = 0.0;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      bool in = RowRegs<NV, VEC>::col(i, c, lane) < ncols;
+      double d = in ? (double)r.v[i][c] - mean : 0.0;
+      sq += d * d;
+    }
+  const double var = wave_sum(sq) / (double)ncols;
+  const double rstd = 1.0 / __builtin_sqrt(var + (double)eps);
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      r.v[i][c] = (float)(((double)r.v[i][c] - mean) * rstd * (double)g.v[i][c] + (double)b.v[i][c]);
+  r.store(out + row * ncols, ncols, lane);
+}
+
+template <bool VEC>
+static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t ldx, float* out,
+                               int64_t ldo, int64_t nrows, int64_t ncols, int64_t causal_seq,
+                               float scale) {
+  hipStream_t st = rt().stream;
+#define WF2_SOFTMAX_CASE(N)                                                                   \
+  case N:                                                                                     \
+    softmax_rows_wave<N, VEC><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,       \
+                                                         causal_seq, scale);                  \
+    break;
+  switch (nv) {
+    WF2_SOFTMAX_CASE(1)
+    WF2_SOFTMAX_CASE(2)
+    WF2_SOFTMAX_CASE(4)
+    WF2_SOFTMAX_CASE(8)
+    WF2_SOFTMAX_CASE(16)
+    default: return fail(WF2HIP_EINVAL, "bad register tile");
+  }
+#undef WF2_SOFTMAX_CASE
+  return after_launch("softmax_rows_wave");
+}
+
+static int pick_nv(int64_t ncols) {
+  for (int nv = 1; nv <= 16; nv *= 2)
+    if ((int64_t)nv * kWave * 4 >= ncols) return nv;
+  return 0;
+}
+
+static int softmax_dispatch(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
+                            int64_t ldo, int64_t causal_seq, float scale) {
+  if (nrows < 0 || ncols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if (nrows == 0 || ncols == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null pointer");
+  if (ldx < ncols || ldo < ncols) return fail(WF2HIP_EINVAL, "row pitch smaller than the row");
+  const int nv = pick_nv(ncols);
+  if (nv == 0) {
+    if (causal_seq > 0) return fail(WF2HIP_EUNSUPPORTED, "causal softmax rows longer than 4096");
+    if (nrows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+    softmax_rows_block<<<(uint32_t)nrows, kBlock, 0, rt().stream>>>(x, ldx, out, ldo, ncols);
+    return after_launch("softmax_rows_block");
+  }
+  int64_t blocks = ceil_div(nrows, kWavesPerBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+  const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0;
+  if (vec)
+    return launch_softmax_wave<true>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                     causal_seq, scale);
+  return launch_softmax_wave<false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                    causal_seq, scale);
+}
+
+template <bool VEC>
+static int launch_layernorm_wave(int nv, uint32_t blocks, const float* x, const float* g,
+                                 const float* b, float eps, float* out, int64_t nrows,
+                                 int64_t ncols) {
+  hipStream_t st = rt().stream;
+#define WF2_LN_CASE(N)                                                                          \
+  case N:                                                                                       \
+    layernorm_rows_wave<N, VEC><<<blocks, kBlock, 0, st>>>(x, g, b, eps, out, nrows, ncols);     \
+    break;
+  switch (nv) {
+    WF2_LN_CASE(1)
+    WF2_LN_CASE(2)
+    WF2_LN_CASE(4)
+    WF2_LN_CASE(8)
+    default: return fail(WF2HIP_EUNSUPPORTED, "LayerNorm rows longer than 2048 are not supported");
+  }
+#undef WF2_LN_CASE
+  return after_launch("layernorm_rows_wave");
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_smax(long n, const float* x, long incx, float* out) {
+  WF2_TRY(require_init());
+  return launch_maxmin<true>(n, x, incx, out);
+}
+
+WF2_API int wf2hip_smin(long n, const float* x, long incx, float* out) {
+  WF2_TRY(require_init());
+  return launch_maxmin<false>(n, x, incx, out);
+}
+
+namespace wf2 {
+int binary_nd(int op, Space s, float* a, const float* b);  // elementwise.hip
+}
+
+WF2_API int wf2hip_reduce_add_rows_f32(long rows, long cols, const float* x, long ldx, float* out,
+                                       long inco) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  Space s;
+  s.rank = 2;
+  s.shape[0] = rows;
+  s.shape[1] = cols;
+  s.sa[0] = inco;
+  s.sa[1] = 0;
+  s.sb[0] = ldx;
+  s.sb[1] = 1;
+  s.off_a = s.off_b = 0;
+  s.total = (int64_t)rows * cols;
+  return binary_nd(WF2HIP_ADD, s, out, x);
+}
+
+WF2_API int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long ldx, float* out,
+                                    long ldo) {
+  WF2_TRY(require_init());
+  return softmax_dispatch(rows, cols, x, ldx, out, ldo, 0, 1.0f);
+}
+
+WF2_API int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
+                                      float scale) {
+  WF2_TRY(require_init());
+  if (batch < 0 || seq < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  return softmax_dispatch((int64_t)batch * seq, seq, x, seq, out, seq, seq > 0 ? seq : 0, scale);
+}
+
+WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
+                                      const float* beta, float eps, float* out) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if (rows == 0 || cols == 0) return 0;
+  if (!x || !gamma || !beta || !out) return fail(WF2HIP_EINVAL, "null pointer");
+  int nv = pick_nv(cols);
+  if (nv == 0 || nv > 8)
+    return fail(WF2HIP_EUNSUPPORTED, "LayerNorm rows longer than 2048 are not supported");
+  int64_t blocks = ceil_div(rows, kWavesPerBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+  const bool vec = aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta) &&
+                   cols % 4 == 0;
+  if (vec)
+    return launch_layernorm_wave<true>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
+  return launch_layernorm_wave<false>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
+}

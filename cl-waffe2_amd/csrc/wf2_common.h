@@ -1,0 +1,51 @@
+// wf2_common.h -- shared state, error channel and launch helpers of
+// libwaffe2-hip.so (internal; the public ABI is include/waffe2_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/waffe2_hip.h"
+
+#define WF2_API extern "C" __attribute__((visibility("default")))
+
+namespace wf2 {
+
+constexpr int kWave = 64;            // CDNA wavefront width
+constexpr int kBlock = 256;          // 4 wavefronts, one per SIMD of a CU
+constexpr int kPartialCapacity = 1 << 16;  // floats of reduction scratch
+
+struct Runtime {
+  bool initialised = false;
+  int device = -1;
+  int num_cus = 0;
+  hipStream_t stream = nullptr;
+  int reduce_mode = 0;
+  float* partials = nullptr;  // kPartialCapacity floats, owned by the library
+  char name[128] = {0};
+  char arch[64] = {0};
+  size_t total_mem = 0;
+};
+
+Runtime& rt();
+
+// Records a message in the thread-local error slot and returns `code`.
+int fail(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+int require_init();
+
+// Every launch goes through this: catches launch-configuration errors at the
+// call that caused them.
+inline int after_launch(const char* what) { return check_hip(hipGetLastError(), what); }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace wf2
+
+#define WF2_TRY(expr)            \
+  do {                           \
+    int _rc = (expr);            \
+    if (_rc != 0) return _rc;    \
+  } while (0)

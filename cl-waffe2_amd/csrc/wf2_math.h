@@ -1,0 +1,253 @@
+// wf2_math.h -- scalar math cores of the element-wise kernels.
+//
+// Contract being replaced: cl-waffe2-simd's unary kernels call SLEEF's
+// Sleef_{sin,cos,tanh,log,exp,pow}f8_u10avx2 (<= 1.0 ulp) and
+// Sleef_sqrtf8_u05avx2 (cl-waffe2-simd/kernels/simd/x86_64/avx2.h:264-332,
+// cl-waffe2-simd.c:586-768).  The device versions below must stay within
+// 2 ulp of those results.
+//
+// Design: CDNA3/CDNA4 issue a binary64 FMA at the same rate as a non-packed
+// binary32 FMA, so every core is evaluated in binary64 with a short
+// polynomial (relative error < 2^-35) and rounded to binary32 once at the
+// end.  The result is within 0.5 + 2^-10 ulp of the exact value, hence within
+// 1.5 ulp of any 1.0-ulp implementation.  Only IEEE operations and fma are
+// used (plus one reciprocal seed that is refined by two Newton steps), so the
+// same header compiles for the host and a CPU build can check every binary32
+// input against libm.
+//
+// Coefficients come from gen_math_coeffs.py (Chebyshev fits in 60-digit
+// arithmetic).
+#pragma once
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#include <hip/hip_runtime.h>
+#define WF2_MATH_FN __device__ __forceinline__
+#define WF2_FMA(a, b, c) __builtin_fma((a), (b), (c))
+#define WF2_RCP_SEED(f) __builtin_amdgcn_rcpf(f)
+#define WF2_SLOW_SINF(x) sinf(x)
+#define WF2_SLOW_COSF(x) cosf(x)
+#define WF2_SLOW_POW(x, p) pow((x), (p))
+#define WF2_SQRTF(x) __builtin_sqrtf(x)
+#else
+#include <math.h>
+#define WF2_MATH_FN static inline
+#define WF2_FMA(a, b, c) __builtin_fma((a), (b), (c))
+#define WF2_RCP_SEED(f) (1.0f / (f))
+#define WF2_SLOW_SINF(x) ((float)sin((double)(x)))
+#define WF2_SLOW_COSF(x) ((float)cos((double)(x)))
+#define WF2_SLOW_POW(x, p) pow((x), (p))
+#define WF2_SQRTF(x) sqrtf(x)
+#endif
+
+namespace wf2 {
+
+WF2_MATH_FN uint64_t bits_of(double d) { return __builtin_bit_cast(uint64_t, d); }
+WF2_MATH_FN double double_of(uint64_t u) { return __builtin_bit_cast(double, u); }
+WF2_MATH_FN uint32_t bits_of(float f) { return __builtin_bit_cast(uint32_t, f); }
+WF2_MATH_FN float float_of(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// Adding 1.5*2^52 rounds a |value| < 2^31 to the nearest-even integer in the
+// fma's own rounding; the integer is then the low 32 bits of the sum.
+constexpr double kRoundMagic = 6755399441055744.0;
+constexpr double kLog2e = 1.442695040888963407359925;
+constexpr double kLn2 = 0.6931471805599453094172321;
+constexpr double kLn2Head = 0.6931471803691238164901733;   // 33 significant bits
+constexpr double kLn2Tail = 1.908214929270587816144266e-10;
+constexpr double kTwoOverPi = 0.6366197723675813430755351;
+constexpr double kPio2Head = 1.57079632673412561416626;    // 33 significant bits
+constexpr double kPio2Tail = 6.077100506506192601475144e-11;
+
+// exp(r) = 1 + r + r^2 Q(r) on |r| <= 0.35; relative error 4.7e-12 (exp),
+// 1.1e-11 (expm1).
+WF2_MATH_FN double expm1_poly(double r) {
+  double q = 0.00002486073188584067535;
+  q = WF2_FMA(q, r, 0.00019900428151915095571);
+  q = WF2_FMA(q, r, 0.0013888852650225144401);
+  q = WF2_FMA(q, r, 0.008333297083738308707);
+  q = WF2_FMA(q, r, 0.041666666722163555503);
+  q = WF2_FMA(q, r, 0.16666666722181582537);
+  q = WF2_FMA(q, r, 0.5);
+  return WF2_FMA(r * r, q, r);
+}
+
+// Splits x = n ln2 + r, |r| <= ln2/2; returns expm1(r) and 2^n.
+// Valid for |x| < 700.
+WF2_MATH_FN void exp_reduce(double x, double* em1_r, double* scale) {
+  double t = WF2_FMA(x, kLog2e, kRoundMagic);
+  double n = t - kRoundMagic;
+  int32_t ni = (int32_t)(uint32_t)bits_of(t);
+  double r = WF2_FMA(n, -kLn2Head, x);
+  r = WF2_FMA(n, -kLn2Tail, r);
+  *em1_r = expm1_poly(r);
+  *scale = double_of((uint64_t)(uint32_t)(ni + 1023) << 52);
+}
+
+// e^x in binary64 for x in [-104, 89] (relative error < 1e-11).
+WF2_MATH_FN double exp_core(double x) {
+  double p, s;
+  exp_reduce(x, &p, &s);
+  return WF2_FMA(s, p, s);
+}
+
+WF2_MATH_FN float expf_(float x) {
+  // Below -104 the result rounds to +0 and above 89 to +inf, as e^-104 and
+  // e^89 already do, so clamping is exact.  fmin/fmax drop a NaN operand.
+  double xd = __builtin_fmin(__builtin_fmax((double)x, -104.0), 89.0);
+  float r = (float)exp_core(xd);
+  return (x != x) ? x : r;
+}
+
+// 1/d for d >= 1 representable in binary32 range: a binary32 seed refined by
+// two Newton steps in binary64 (relative error ~2^-50 whatever the seed's
+// last bit).
+WF2_MATH_FN double rcp_refined(double d) {
+  double y = (double)WF2_RCP_SEED((float)d);
+  double e = WF2_FMA(-d, y, 1.0);
+  y = WF2_FMA(y, e, y);
+  e = WF2_FMA(-d, y, 1.0);
+  return WF2_FMA(y, e, y);
+}
+
+// tanh(x) = expm1(2|x|) / (expm1(2|x|) + 2); saturates to 1 from |x| = 10
+// (1 - tanh(10) = 4.1e-9 < 2^-25).
+WF2_MATH_FN double tanh_core(double ax) {
+  double p, s;
+  exp_reduce(ax + ax, &p, &s);
+  double em1 = WF2_FMA(s, p, s - 1.0);
+  return em1 * rcp_refined(em1 + 2.0);
+}
+
+WF2_MATH_FN float tanhf_(float x) {
+  double ax = __builtin_fmin(__builtin_fabs((double)x), 10.0);
+  float r = __builtin_copysignf((float)tanh_core(ax), x);
+  return (x != x) ? x : r;
+}
+
+// log(m) for m in [sqrt(1/2), sqrt(2)): f = m - 1,
+// log(1+f) = f - f^2/2 + f^3 R(f); relative error 1.3e-11.
+WF2_MATH_FN double log1p_poly(double f) {
+  double r = -0.05005748841457288547;
+  r = WF2_FMA(r, f, 0.09036934208961060298);
+  r = WF2_FMA(r, f, -0.09109982945851015244);
+  r = WF2_FMA(r, f, 0.09031005007965443269);
+  r = WF2_FMA(r, f, -0.09922837010255326152);
+  r = WF2_FMA(r, f, 0.1110948193429464372);
+  r = WF2_FMA(r, f, -0.1250321982641986753);
+  r = WF2_FMA(r, f, 0.1428586067850288431);
+  r = WF2_FMA(r, f, -0.1666661173195466807);
+  r = WF2_FMA(r, f, 0.1999999784866672395);
+  r = WF2_FMA(r, f, -0.2500000026716445387);
+  r = WF2_FMA(r, f, 0.3333333333749120236);
+  double f2 = f * f;
+  return WF2_FMA(f2 * f, r, WF2_FMA(-0.5, f2, f));
+}
+
+// log of a positive finite binary64 that is normal (every positive binary32,
+// subnormals included, converts to one).
+WF2_MATH_FN double log_core(double xd) {
+  uint64_t b = bits_of(xd);
+  int32_t hi = (int32_t)(b >> 32);
+  hi += 0x3ff00000 - 0x3fe6a09e;  // moves the binade boundary to sqrt(1/2)
+  int32_t k = (hi >> 20) - 0x3ff;
+  hi = (hi & 0x000fffff) + 0x3fe6a09e;
+  double m = double_of(((uint64_t)(uint32_t)hi << 32) | (b & 0xffffffffu));
+  return WF2_FMA((double)k, kLn2, log1p_poly(m - 1.0));
+}
+
+WF2_MATH_FN float logf_(float x) {
+  const float inf = __builtin_inff();
+  bool ok = (x > 0.0f) && (x < inf);
+  float r = (float)log_core(ok ? (double)x : 1.0);
+  // x == +inf -> +inf; x == +-0 -> -inf; x < 0 or NaN -> NaN
+  float special = (x == inf) ? inf : ((x == 0.0f) ? -inf : __builtin_nanf(""));
+  return ok ? r : special;
+}
+
+// sin/cos on |r| <= pi/4: sin r = r + r^3 S(r^2) (1.9e-11),
+// cos r = 1 - z/2 + z^2 C(z) (1.3e-12).
+WF2_MATH_FN double sin_poly(double r, double z) {
+  double s = 2.7249146796813166492e-6;
+  s = WF2_FMA(s, z, -0.0001984008071991224356);
+  s = WF2_FMA(s, z, 0.008333331863560767561);
+  s = WF2_FMA(s, z, -0.1666666666382658236);
+  return WF2_FMA(r * z, s, r);
+}
+
+WF2_MATH_FN double cos_poly(double z) {
+  double c = -2.7300309020522219532e-7;
+  c = WF2_FMA(c, z, 0.000024800595356594503473);
+  c = WF2_FMA(c, z, -0.0013888887662711772101);
+  c = WF2_FMA(c, z, 0.041666666664297246826);
+  return WF2_FMA(z * z, c, WF2_FMA(-0.5, z, 1.0));
+}
+
+// Quadrant reduction x = q*pi/2 + r in binary64.  q*kPio2Head is exact for
+// |q| < 2^20, i.e. |x| <= 1e6.
+constexpr float kTrigFastLimit = 1.0e6f;
+
+WF2_MATH_FN double trig_core(double xd, int32_t quadrant_shift) {
+  double t = WF2_FMA(xd, kTwoOverPi, kRoundMagic);
+  double q = t - kRoundMagic;
+  int32_t qi = (int32_t)(uint32_t)bits_of(t) + quadrant_shift;
+  double r = WF2_FMA(q, -kPio2Head, xd);
+  r = WF2_FMA(q, -kPio2Tail, r);
+  double z = r * r;
+  double s = sin_poly(r, z);
+  double c = cos_poly(z);
+  double v = (qi & 1) ? c : s;
+  return (qi & 2) ? -v : v;
+}
+
+WF2_MATH_FN float sinf_(float x) {
+  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_SINF(x);
+  return (float)trig_core((double)x, 0);
+}
+
+WF2_MATH_FN float cosf_(float x) {
+  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_COSF(x);
+  return (float)trig_core((double)x, 1);
+}
+
+WF2_MATH_FN float sqrtf_(float x) { return WF2_SQRTF(x); }
+WF2_MATH_FN float absf_(float x) { return __builtin_fabsf(x); }
+
+// x^p.  The exponent is the same for every element of a launch (it is the
+// host scalar of ExptNode, base-impl/mathematics.lisp:267-303), so the branch
+// is uniform.  Integral exponents (GELU's x^3, LayerNorm's (x-u)^2) are
+// repeated products in binary64, exact to ~2^-48 and rounded once.
+WF2_MATH_FN float powf_(float x, float p) {
+  float ap = __builtin_fabsf(p);
+  if (ap <= 1024.0f && p == __builtin_truncf(p)) {
+    uint32_t e = (uint32_t)ap;
+    double base = (double)x, acc = 1.0;
+    while (e) {
+      if (e & 1u) acc *= base;
+      base *= base;
+      e >>= 1;
+    }
+    if (p < 0.0f) acc = 1.0 / acc;
+    return (float)acc;
+  }
+  if (p == 0.5f) return WF2_SQRTF(x);
+  return (float)WF2_SLOW_POW((double)x, (double)p);
+}
+
+// tanh-form GELU, 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3)
+// (nn/activation.lisp:45-66), in binary64 and rounded once.  0.5 (1 + tanh u)
+// equals sigmoid(2u), evaluated with e = exp(-2|u|) in (0, 1] as 1/(1+e) for
+// u >= 0 and e/(1+e) for u < 0: no cancellation on either side.
+WF2_MATH_FN float gelu_tanh_f(float x) {
+  double xd = (double)x;
+  double u = 0.7978845608028654 * WF2_FMA(0.044715 * xd * xd, xd, xd);
+  double au = __builtin_fmin(__builtin_fabs(u), 350.0);
+  double e = exp_core(-(au + au));
+  double num = (u >= 0.0) ? 1.0 : e;
+  float r = (float)(xd * num * rcp_refined(1.0 + e));
+  // x = -inf: the limit is -0 (x e^{2u} -> 0), not -inf * tiny.
+  r = (x == -__builtin_inff()) ? -0.0f : r;
+  return (x != x) ? x : r;
+}
+
+}  // namespace wf2

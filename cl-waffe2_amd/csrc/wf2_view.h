@@ -1,0 +1,118 @@
+// wf2_view.h -- host-side normalisation of a two-tensor iteration space.
+//
+// cl-waffe2 hands a kernel per-axis (offset, size, stride) triplets
+// (ViewInstruction, source/vm/generic-tensor/view.lisp:50-69) and wraps the
+// 1-D kernel in host loops (call-with-view.lisp:112-229).  Here the whole
+// space arrives in one wf2hip_view2 and is reduced to the fewest axes that
+// describe the same address pattern, so that one launch covers the node.
+#pragma once
+
+#include <stdint.h>
+
+#include "wf2_common.h"
+
+namespace wf2 {
+
+struct Space {
+  int rank = 0;                       // >= 1 after normalise() unless empty
+  int64_t shape[WF2HIP_MAX_RANK];     // outermost first
+  int64_t sa[WF2HIP_MAX_RANK];
+  int64_t sb[WF2HIP_MAX_RANK];
+  int64_t off_a = 0, off_b = 0;
+  int64_t total = 0;
+};
+
+// Validates the descriptor and copies it.  total == 0 means nothing to do.
+inline int load_space(const wf2hip_view2* v, Space* s) {
+  if (!v) return fail(WF2HIP_EINVAL, "null view descriptor");
+  if (v->rank < 1 || v->rank > WF2HIP_MAX_RANK)
+    return fail(WF2HIP_EINVAL, "view rank %d outside 1..%d", v->rank, WF2HIP_MAX_RANK);
+  s->rank = v->rank;
+  s->total = 1;
+  for (int r = 0; r < v->rank; r++) {
+    if (v->shape[r] < 0) return fail(WF2HIP_EINVAL, "negative extent on axis %d", r);
+    s->shape[r] = v->shape[r];
+    s->sa[r] = v->stride_a[r];
+    s->sb[r] = v->stride_b[r];
+    s->total *= v->shape[r];
+  }
+  if (v->off_a < 0 || v->off_b < 0) return fail(WF2HIP_EINVAL, "negative offset");
+  s->off_a = v->off_a;
+  s->off_b = v->off_b;
+  return 0;
+}
+
+// Drops extent-1 axes and merges neighbours that are one linear run for both
+// tensors (stride_outer == stride_inner * extent_inner, which also merges
+// 0/0 broadcast pairs).
+inline void normalise(Space* s) {
+  int w = 0;
+  for (int r = 0; r < s->rank; r++) {
+    if (s->shape[r] == 1) continue;
+    s->shape[w] = s->shape[r];
+    s->sa[w] = s->sa[r];
+    s->sb[w] = s->sb[r];
+    w++;
+  }
+  if (w == 0) {  // a single element
+    s->shape[0] = 1;
+    s->sa[0] = 0;
+    s->sb[0] = 0;
+    w = 1;
+  }
+  s->rank = w;
+  int out = 0;
+  for (int r = 1; r < s->rank; r++) {
+    bool merge = s->sa[out] == s->sa[r] * s->shape[r] && s->sb[out] == s->sb[r] * s->shape[r];
+    if (merge) {
+      s->shape[out] *= s->shape[r];
+      s->sa[out] = s->sa[r];
+      s->sb[out] = s->sb[r];
+    } else {
+      out++;
+      s->shape[out] = s->shape[r];
+      s->sa[out] = s->sa[r];
+      s->sb[out] = s->sb[r];
+    }
+  }
+  s->rank = out + 1;
+}
+
+// Lowest and highest element offset a strided window touches.
+inline void extent_of(const Space& s, const int64_t* stride, int64_t off, int64_t* lo,
+                      int64_t* hi) {
+  *lo = off;
+  *hi = off;
+  for (int r = 0; r < s.rank; r++) {
+    int64_t span = stride[r] * (s.shape[r] - 1);
+    if (span >= 0)
+      *hi += span;
+    else
+      *lo += span;
+  }
+}
+
+// True when the two windows may touch a common element without being the
+// same element-for-element mapping.
+inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {
+  int64_t alo, ahi, blo, bhi;
+  extent_of(s, s.sa, s.off_a, &alo, &ahi);
+  extent_of(s, s.sb, s.off_b, &blo, &bhi);
+  const float* a0 = a + alo;
+  const float* a1 = a + ahi;
+  const float* b0 = b + blo;
+  const float* b1 = b + bhi;
+  if (a1 < b0 || b1 < a0) return false;
+  if (a + s.off_a != b + s.off_b) return true;
+  for (int r = 0; r < s.rank; r++)
+    if (s.sa[r] != s.sb[r]) return true;
+  return false;  // identical mapping: every element depends on itself only
+}
+
+inline bool has_broadcast_axis(const Space& s, const int64_t* stride) {
+  for (int r = 0; r < s.rank; r++)
+    if (stride[r] == 0 && s.shape[r] > 1) return true;
+  return false;
+}
+
+}  // namespace wf2

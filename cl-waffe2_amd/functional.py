@@ -1,0 +1,406 @@
+"""User-level tensor functions, decomposed into nodes the way cl-waffe2 does.
+
+Eager mirror of ``source/base-impl`` (``!add`` ... ``!matmul``), ``!sum`` /
+``!mean`` (``base-impl/reduction.lisp``) and the ``source/nn`` recipes used by a
+transformer block.  Each function issues the same node sequence the reference
+builds lazily and runs through ``proceed``; the nodes land on whatever device
+``nodes.USING_BACKEND`` selects.
+
+Naming: ``!add`` -> ``add``, ``A+=B`` -> ``add_``, ``!loge`` -> ``loge``,
+``->contiguous`` -> ``to_contiguous``.
+"""
+from __future__ import annotations
+
+import math
+from typing import Sequence
+
+import numpy as np
+
+from . import lib as _lib
+from . import nodes
+from .tensor import HIPTensor
+
+Number = (int, float, np.integer, np.floating)
+
+
+# ---------------------------------------------------------------------------
+# construction / movement
+# ---------------------------------------------------------------------------
+
+def make_tensor(shape: Sequence[int], initial_element: float = 0.0) -> HIPTensor:
+    """``(make-tensor shape :initial-element x)``"""
+    return HIPTensor(shape, initial_element=initial_element)
+
+
+def from_numpy(a) -> HIPTensor:
+    return HIPTensor.from_numpy(a)
+
+
+def move_(dst: HIPTensor, src: HIPTensor) -> HIPTensor:
+    """``(!move dst src)``: MoveTensorNode, ``dst <- src``
+    (``base-impl/fundamental.lisp:9-43,80-120``)."""
+    return nodes.forward("MoveTensorNode", dst, src)
+
+
+def copy(x: HIPTensor) -> HIPTensor:
+    """``(!copy x)``: a fresh contiguous tensor of x's visible shape filled by
+    MoveTensorNode (``fundamental.lisp:122-163``)."""
+    return move_(HIPTensor(x.shape), x)
+
+
+def to_contiguous(x: HIPTensor) -> HIPTensor:
+    """``(->contiguous x)`` (``fundamental.lisp:1059-1107``): copies only when
+    the tensor is viewed, permuted or broadcast."""
+    return x if x.is_contiguous() else copy(x)
+
+
+def view(x: HIPTensor, *subscripts) -> HIPTensor:
+    return x.view(*subscripts)
+
+
+def permute(x: HIPTensor, *order: int) -> HIPTensor:
+    return x.permute(*order)
+
+
+def reshape(x: HIPTensor, *shape: int) -> HIPTensor:
+    """``(!reshape x ...)`` (``fundamental.lisp:273-350``): same storage, new
+    shape; a non-contiguous source is materialised first.  One extent may be
+    -1."""
+    shape = list(shape)
+    if shape.count(-1) == 1:
+        known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+        shape[shape.index(-1)] = x.size // max(known, 1)
+    if int(np.prod(shape, dtype=np.int64)) != x.size:
+        raise ValueError(f"reshape: cannot reshape {x.shape} into {shape}")
+    src = to_contiguous(x)
+    return HIPTensor(shape, vec=src.vec)
+
+
+class Transposed:
+    """Marker returned by ``t``: the last two axes are swapped lazily and the
+    flag is consumed by ``matmul`` (``LazyTransposeNode``,
+    ``base-impl/matrix-ops.lisp:34-78``)."""
+
+    def __init__(self, tensor: HIPTensor):
+        self.tensor = tensor
+
+    @property
+    def shape(self):
+        s = self.tensor.shape
+        return s[:-2] + [s[-1], s[-2]]
+
+
+def t(x: HIPTensor) -> Transposed:
+    """``(!t x)``"""
+    return Transposed(x)
+
+
+# ---------------------------------------------------------------------------
+# broadcasting helpers
+# ---------------------------------------------------------------------------
+
+def scalar_tensor(value: float, like: HIPTensor) -> HIPTensor:
+    """A ``(1 ... 1)`` tensor viewed ``(:broadcast n)`` on every axis, which is
+    how ``!scalar-add`` & co. feed a scalar to a tensor node
+    (``base-impl/arithmetic.lisp:31-51,216-262``)."""
+    s = HIPTensor([1] * like.ndim, initial_element=float(value))
+    return s.view(*[(":broadcast", n) if n != 1 else True for n in like.shape])
+
+
+def flexible(y: HIPTensor, like: HIPTensor) -> HIPTensor:
+    """Rank-extend ``y`` on the left and broadcast its size-1 axes against
+    ``like`` (what ``!flexible`` + the automatic broadcast of ``forward
+    :around`` do, ``vm/nodes/node.lisp:171-182``, ``broadcast.lisp:22``)."""
+    ys, ls = y.shape, like.shape
+    if ys == ls:
+        return y
+    if len(ys) > len(ls):
+        raise ValueError(f"cannot broadcast {ys} to {ls}")
+    if len(ys) < len(ls):
+        if not y.is_contiguous():
+            y = copy(y)
+        y = HIPTensor([1] * (len(ls) - len(ys)) + ys, vec=y.vec)
+        ys = y.shape
+    subs = []
+    for a, b in zip(ys, ls):
+        if a == b:
+            subs.append(True)
+        elif a == 1:
+            subs.append((":broadcast", b))
+        else:
+            raise ValueError(f"cannot broadcast {ys} to {ls}")
+    # T would reset an existing slice; only touch axes that need broadcasting
+    if all(s is True for s in subs):
+        return y
+    views = list(y.views)
+    from .tensor import parse_view
+    for i, s in enumerate(subs):
+        if s is not True:
+            views[i] = parse_view(y.orig_shape[i], y.views[i], s)
+    return HIPTensor(y.orig_shape, vec=y.vec, strides=y.stride, views=views, offset=y.initial_offset)
+
+
+def _operand(y, like: HIPTensor) -> HIPTensor:
+    if isinstance(y, Number):
+        return scalar_tensor(float(y), like)
+    return flexible(y, like)
+
+
+# ---------------------------------------------------------------------------
+# arithmetic
+# ---------------------------------------------------------------------------
+
+def add_(x: HIPTensor, y) -> HIPTensor:
+    """``(A+=B x y)``: AddNode in place in x."""
+    return nodes.forward("AddNode", x, _operand(y, x))
+
+
+def sub_(x: HIPTensor, y) -> HIPTensor:
+    return nodes.forward("SubNode", x, _operand(y, x))
+
+
+def mul_(x: HIPTensor, y) -> HIPTensor:
+    return nodes.forward("MulNode", x, _operand(y, x))
+
+
+def div_(x: HIPTensor, y) -> HIPTensor:
+    return nodes.forward("DivNode", x, _operand(y, x))
+
+
+def _out_of_place(node: str, x, y) -> HIPTensor:
+    """``!add``-family (``base-impl/arithmetic.lisp:114-177,367-434``): the left
+    operand is copied, the node runs in place on the copy."""
+    if isinstance(x, Number):
+        # scalar op tensor: s + T, s * T commute; s - T = s + (-1 * T);
+        # s / T = s * (1 / T)   (arithmetic.lisp:180-209,407-434)
+        if node == "AddNode":
+            return add_(copy(y), x)
+        if node == "MulNode":
+            return mul_(copy(y), x)
+        if node == "SubNode":
+            return add_(mul_(copy(y), -1.0), x)
+        return mul_(reciprocal(y), x)
+    if isinstance(y, Number):
+        return nodes.forward(node, copy(x), scalar_tensor(float(y), x))
+    if x.shape == y.shape:
+        return nodes.forward(node, copy(x), y)
+    out_shape = list(np.broadcast_shapes(tuple(x.shape), tuple(y.shape)))
+    if x.shape == out_shape:
+        left = copy(x)
+    else:  # x is the smaller operand: expand it into a full-size tensor first
+        left = move_(HIPTensor(out_shape), flexible(x, _ShapeOnly(out_shape)))
+    return nodes.forward(node, left, flexible(y, left))
+
+
+def add(x, y) -> HIPTensor:
+    return _out_of_place("AddNode", x, y)
+
+
+def sub(x, y) -> HIPTensor:
+    return _out_of_place("SubNode", x, y)
+
+
+def mul(x, y) -> HIPTensor:
+    return _out_of_place("MulNode", x, y)
+
+
+def div(x, y) -> HIPTensor:
+    return _out_of_place("DivNode", x, y)
+
+
+def reciprocal(x: HIPTensor) -> HIPTensor:
+    """``(!reciprocal x)`` = DivNode(ones, x) (``arithmetic.lisp:180-209``)."""
+    return nodes.forward("DivNode", HIPTensor(x.shape, initial_element=1.0), x)
+
+
+# ---------------------------------------------------------------------------
+# mathematics
+# ---------------------------------------------------------------------------
+
+def _math(node: str, x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!exp x :-> out)``: ``out`` defaults to a fresh tensor (the pruned
+    ``(!copy x :maybe-in-place t)`` of ``base-impl/mathematics.lisp:13-120``)."""
+    if out is None:
+        out = HIPTensor(x.shape)
+    return nodes.forward(node, x, out)
+
+
+def sin(x, out=None): return _math("SinNode", x, out)
+def cos(x, out=None): return _math("CosNode", x, out)
+def tanh(x, out=None): return _math("TanhNode", x, out)
+def exp(x, out=None): return _math("ExpNode", x, out)
+def loge(x, out=None): return _math("LogENode", x, out)
+def sqrt(x, out=None): return _math("SqrtNode", x, out)
+def abs(x, out=None): return _math("AbsNode", x, out)  # noqa: A001 - mirrors !abs
+
+
+def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!expt x n)`` (``mathematics.lisp:267-303``)."""
+    if out is None:
+        out = HIPTensor(x.shape)
+    return nodes.forward("ExptNode", x, out, float(n))
+
+
+# ---------------------------------------------------------------------------
+# reductions
+# ---------------------------------------------------------------------------
+
+def _axes(axis, ndim: int) -> list[int]:
+    if axis is True:
+        return list(range(ndim))
+    if isinstance(axis, (int, np.integer)):
+        axis = [int(axis)]
+    return sorted(a + ndim if a < 0 else a for a in axis)
+
+
+def sum(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = False,  # noqa: A001
+        div_by=None) -> HIPTensor:
+    """``(!sum tensor :axis :-> :keepdims)`` exactly as
+    ``base-impl/reduction.lisp:5-79`` composes it: zero-fill ``out`` by
+    multiplying with 0, view it ``(:broadcast n)`` on the reduced axes, AddNode
+    ``x`` into that stride-0 view, then undo (or keep) the broadcast."""
+    axes = _axes(axis, x.ndim)
+    shape = list(x.shape)
+    out_shape = [1 if i in axes else n for i, n in enumerate(shape)]
+    if out is None:
+        out = HIPTensor(out_shape)
+    elif out.shape != out_shape:
+        raise ValueError(f"!sum: the given out's shape is {out.shape}, but expected: {out_shape}")
+    out = mul_(out, 0.0)  # A*=scal out 0  (reduction.lisp:63)
+    view_args = [(":broadcast", shape[i]) if (i in axes and shape[i] != 1) else True
+                 for i in range(x.ndim)]
+    # keep existing (non-broadcast) views on `out` intact: only re-view reduced axes
+    from .tensor import parse_view
+    views = list(out.views)
+    for i, s in enumerate(view_args):
+        if s is not True:
+            views[i] = parse_view(out.orig_shape[i], out.views[i], s)
+    out_bc = HIPTensor(out.orig_shape, vec=out.vec, strides=out.stride, views=views,
+                       offset=out.initial_offset)
+    add_(out_bc, x)  # A+=B out* tensor: accumulation into a stride-0 destination
+    result = out_bc if keepdims else out
+    if div_by is not None:
+        div_(out, float(div_by))
+    return result
+
+
+def mean(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = False) -> HIPTensor:
+    """``(!mean ...)`` = ``!sum`` with ``:div-by`` the number of reduced
+    elements (``reduction.lisp:81-136``)."""
+    n = 1
+    for a in _axes(axis, x.ndim):
+        n *= x.shape[a]
+    return sum(x, axis=axis, out=out, keepdims=keepdims, div_by=float(n))
+
+
+# ---------------------------------------------------------------------------
+# matmul
+# ---------------------------------------------------------------------------
+
+def matmul(a, b, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!matmul a b)`` (``base-impl/matrix-ops.lisp:80-173``): ``!t`` operands
+    become transpose flags, any other non-trivial layout of the last two axes is
+    materialised with ``->contiguous``, a lower-rank operand is broadcast over
+    the batch axes, and the output is a fresh ``(~ i k)`` tensor."""
+    trans_a = isinstance(a, Transposed)
+    trans_b = isinstance(b, Transposed)
+    at = a.tensor if trans_a else a
+    bt = b.tensor if trans_b else b
+
+    def ready(x: HIPTensor) -> HIPTensor:
+        shape, strides, _ = x.geometry()
+        ok = (shape[-1] == 1 or strides[-1] == 1) and (shape[-2] == 1 or strides[-2] >= shape[-1])
+        return x if ok else copy(x)
+
+    at, bt = ready(at), ready(bt)
+    ashape = a.shape if trans_a else at.shape
+    bshape = b.shape if trans_b else bt.shape
+    batch = ashape[:-2] if len(ashape) >= len(bshape) else bshape[:-2]
+    if out is None:
+        out = HIPTensor(list(batch) + [ashape[-2], bshape[-1]])
+
+    def with_batch(x: HIPTensor) -> HIPTensor:
+        if x.shape[:-2] == list(batch):
+            return x
+        return flexible(x, _ShapeOnly(list(batch) + x.shape[-2:]))
+
+    return nodes.forward("MatMulNode", with_batch(at), with_batch(bt), out,
+                         trans_a=trans_a, trans_b=trans_b)
+
+
+class _ShapeOnly:
+    def __init__(self, shape):
+        self.shape = list(shape)
+        self.ndim = len(shape)
+
+
+# ---------------------------------------------------------------------------
+# nn recipes
+# ---------------------------------------------------------------------------
+
+def softmax(x: HIPTensor, avoid_overflow: bool = True, axis=1) -> HIPTensor:
+    """``(!softmax x :avoid-overflow t :axis 1)`` node for node
+    (``source/nn/activation.lisp:126-159``).  Note that the reference subtracts
+    the MEAN along ``axis``, not the max."""
+    if avoid_overflow:
+        x1 = sub(x, mean(x, axis=axis, keepdims=True))
+        expx1 = exp(x1)
+        z = sum(expx1, axis=axis, keepdims=True)
+        return div(expx1, z)
+    x1 = exp(x)
+    return div(x1, sum(x1, axis=axis, keepdims=True))
+
+
+def softmax_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
+    """Max-subtracted softmax over the last axis in one kernel
+    (``wf2hip_softmax_rows_f32``)."""
+    import ctypes as C
+    x = to_contiguous(x)
+    if out is None:
+        out = HIPTensor(x.shape)
+    cols = x.shape[-1]
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols,
+                                                 C.c_void_p(out.ptr), cols))
+    return out
+
+
+def gelu(x: HIPTensor) -> HIPTensor:
+    """``(!gelu x)`` node for node (``source/nn/activation.lisp:45-66``):
+    0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))."""
+    inner = add(x, mul(expt(x, 3), 0.044715))
+    th = tanh(mul(inner, float(np.float32(math.sqrt(2.0 / math.pi)))))
+    return mul(mul(x, 0.5), add(th, 1.0))
+
+
+def gelu_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
+    import ctypes as C
+    if out is None:
+        out = HIPTensor(x.shape)
+    v = nodes.view2(x, out)
+    _lib.check(_lib.get().wf2hip_unary_nd(_lib.GELU, C.byref(v), C.c_void_p(x.ptr),
+                                         C.c_void_p(out.ptr), 0.0))
+    return out
+
+
+def layer_norm(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e-5) -> HIPTensor:
+    """``LayerNorm-Revisit`` node for node (``examples/gpt-2/utils.lisp:114-127``;
+    same recipe as ``source/nn/norms.lisp:72-82``)."""
+    u = mean(x, axis=-1, keepdims=True)
+    xc = sub(x, u)
+    s = mean(expt(xc, 2), axis=-1, keepdims=True)
+    xn = div(xc, sqrt(add(to_contiguous(s), eps)))
+    return add(mul(xn, g), b)
+
+
+def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e-5,
+                     out: HIPTensor | None = None) -> HIPTensor:
+    import ctypes as C
+    x = to_contiguous(x)
+    if out is None:
+        out = HIPTensor(x.shape)
+    cols = x.shape[-1]
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_layernorm_rows_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),
+                                                   C.c_void_p(b.ptr), float(eps), C.c_void_p(out.ptr)))
+    return out

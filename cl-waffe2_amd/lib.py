@@ -1,0 +1,189 @@
+"""ctypes binding of ``libwaffe2-hip.so`` (the C ABI in ``include/waffe2_hip.h``).
+
+Mirrors the role of ``cl-waffe2-simd/shared-object.lisp`` + ``api.lisp`` in the
+reference: find the shared object next to the package, load it, declare every
+foreign function.  Unlike the reference's soft-failing loader
+(``shared-object.lisp:4-13`` warns and returns NIL so that CPUTensor falls back
+to LispTensor), a missing library here is an error: there is no CPU fallback
+behind the HIP backend.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwaffe2-hip.so")
+MAX_RANK = 8
+
+# enum wf2hip_binary_op / wf2hip_unary_op
+ADD, SUB, MUL, DIV, MOVE = 0, 1, 2, 3, 4
+SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
+POW, GELU = 32, 40
+
+EOVERLAP = -3
+
+
+class HIPExtensionMissing(RuntimeError):
+    """libwaffe2-hip.so is not built or cannot be loaded."""
+
+
+class HIPError(RuntimeError):
+    """A wf2hip_* call returned a non-zero code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"wf2hip error {code}: {message}")
+        self.code = code
+
+
+class View2(C.Structure):
+    """``struct wf2hip_view2``"""
+
+    _fields_ = [
+        ("rank", C.c_int32),
+        ("reserved", C.c_int32),
+        ("shape", C.c_int64 * MAX_RANK),
+        ("stride_a", C.c_int64 * MAX_RANK),
+        ("stride_b", C.c_int64 * MAX_RANK),
+        ("off_a", C.c_int64),
+        ("off_b", C.c_int64),
+    ]
+
+
+_P = C.c_void_p
+_L = C.c_long
+_F = C.c_float
+
+_SIGNATURES = {
+    "wf2hip_abi_version": ([], C.c_int),
+    "wf2hip_init": ([C.c_int], C.c_int),
+    "wf2hip_shutdown": ([], C.c_int),
+    "wf2hip_last_error": ([], C.c_char_p),
+    "wf2hip_device_info": ([C.c_char_p, C.c_size_t], C.c_int),
+    "wf2hip_malloc": ([C.POINTER(_P), C.c_size_t], C.c_int),
+    "wf2hip_free": ([_P], C.c_int),
+    "wf2hip_memcpy_h2d": ([_P, _P, C.c_size_t], C.c_int),
+    "wf2hip_memcpy_d2h": ([_P, _P, C.c_size_t], C.c_int),
+    "wf2hip_memcpy_d2d": ([_P, _P, C.c_size_t], C.c_int),
+    "wf2hip_fill_f32": ([_P, C.c_size_t, _F], C.c_int),
+    "wf2hip_sync": ([], C.c_int),
+    "wf2hip_set_stream": ([_P], C.c_int),
+    "wf2hip_get_stream": ([], _P),
+    "wf2hip_event_create": ([C.POINTER(_P)], C.c_int),
+    "wf2hip_event_record": ([_P], C.c_int),
+    "wf2hip_event_elapsed_ms": ([_P, _P, C.POINTER(_F)], C.c_int),
+    "wf2hip_event_destroy": ([_P], C.c_int),
+    "wf2hip_sadd": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_ssub": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_smul": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sdiv": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_scopy": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_ssin": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_scos": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_stanh": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_slog": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sexp": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_ssqrt": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sabs": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_spow": ([_L, _P, _L, _F, _P, _L], C.c_int),
+    "wf2hip_smax": ([_L, _P, _L, _P], C.c_int),
+    "wf2hip_smin": ([_L, _P, _L, _P], C.c_int),
+    "wf2hip_binary_nd": ([C.c_int, C.POINTER(View2), _P, _P], C.c_int),
+    "wf2hip_unary_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F], C.c_int),
+    "wf2hip_set_reduce_mode": ([C.c_int], C.c_int),
+    "wf2hip_get_reduce_mode": ([], C.c_int),
+    "wf2hip_reduce_add_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_softmax_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_causal_softmax_f32": ([_L, _L, _P, _P, _F], C.c_int),
+    "wf2hip_layernorm_rows_f32": ([_L, _L, _P, _P, _P, _F, _P], C.c_int),
+    "wf2hip_sgemm": ([C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _P, _L, _F, _P, _L], C.c_int),
+    "wf2hip_sgemm_strided_batched": (
+        [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _P, _L, _L, _F, _P, _L, _L, _L],
+        C.c_int,
+    ),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+_lib = None
+_initialised_device = None
+
+
+def load():
+    """Load the shared library and declare its functions (no GPU touched)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HIPExtensionMissing(
+            f"{LIB_PATH} is not built; run `make -C {os.path.join(_HERE, 'csrc')}` "
+            "(or __graft_entry__.build()). The HIP backend has no CPU fallback."
+        )
+    try:
+        lib = C.CDLL(LIB_PATH)
+    except OSError as e:  # pragma: no cover - depends on the machine
+        raise HIPExtensionMissing(f"cannot load {LIB_PATH}: {e}") from e
+    for name, (argtypes, restype) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = restype
+    _lib = lib
+    return lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        msg = load().wf2hip_last_error()
+        raise HIPError(code, msg.decode() if msg else "")
+
+
+def init(device: int = 0):
+    """Initialise the runtime on ``device`` (idempotent) and return the library."""
+    global _initialised_device
+    lib = load()
+    if _initialised_device != device:
+        check(lib.wf2hip_init(device))
+        _initialised_device = device
+    return lib
+
+
+def get():
+    """The initialised library; initialises device 0 on first use."""
+    if _initialised_device is None:
+        return init(0)
+    return _lib
+
+
+def device_info() -> dict:
+    buf = C.create_string_buffer(256)
+    check(get().wf2hip_device_info(buf, 256))
+    name, arch, cus, mem = buf.value.decode().split("|")
+    return {"name": name, "arch": arch, "compute_units": int(cus), "memory_bytes": int(mem)}
+
+
+def synchronize() -> None:
+    check(get().wf2hip_sync())
+
+
+class Event:
+    """HIP event on the library's stream (for timing kernels where they run)."""
+
+    def __init__(self):
+        self._h = _P()
+        check(get().wf2hip_event_create(C.byref(self._h)))
+
+    def record(self) -> "Event":
+        check(get().wf2hip_event_record(self._h))
+        return self
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = _F()
+        check(get().wf2hip_event_elapsed_ms(self._h, stop._h, C.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self._h and _lib is not None:
+                _lib.wf2hip_event_destroy(self._h)
+        except Exception:
+            pass

@@ -1,0 +1,221 @@
+"""Node dispatch and the HIPTensor implementations (the ``define-impl`` layer).
+
+Mirror of how a cl-waffe2 backend plugs in (``source/vm/nodes/defnode.lisp``):
+
+* ``define_impl(node, device, reject_p)`` registers an implementation in
+  ``DEVICE_FEATURES[device][node]`` (``defnode.lisp:428-571``, ``:535-538``);
+* ``forward(node, *tensors)`` walks the priority list ``USING_BACKEND`` and
+  takes the first device that has an implementation whose ``reject_p`` does not
+  reject the dtype (``determine-facet-of-nodes``, ``defnode.lisp:215-232``);
+  nothing matching raises ``NodeNotFound`` -- there is no silent fallback;
+* each implementation returns its output tensor, as the VM requires
+  (``source/vm/vm.lisp:144-150``).
+
+The implementations below are what ``(define-impl (AddNode :device HIPTensor)
+...)`` etc. do on the Lisp side: turn the tensors' views into one
+``wf2hip_view2`` and make ONE library call per node, where the CPU backend emits
+host loops around 1-D kernels (``source/backends/cpu/arithmetic.lisp:32-144``,
+``mathematics.lisp:8-76``, ``matrix-ops.lisp:12-237``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from contextlib import contextmanager
+
+from . import lib as _lib
+from .tensor import HIPTensor
+
+NODE_NAMES = (
+    "AddNode", "SubNode", "MulNode", "DivNode", "MoveTensorNode",
+    "SinNode", "CosNode", "TanhNode", "LogENode", "ExpNode", "SqrtNode", "AbsNode",
+    "ExptNode", "MatMulNode",
+)
+
+DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
+USING_BACKEND: list[type] = [HIPTensor]
+
+
+class NodeNotFound(LookupError):
+    """No device in the backend list implements the node (``node-not-found``)."""
+
+
+def define_impl(node: str, device: type, reject_p=None):
+    if node not in NODE_NAMES:
+        raise ValueError(f"unknown AbstractNode {node}")
+
+    def register(fn):
+        DEVICE_FEATURES.setdefault(device, {})[node] = (fn, reject_p)
+        return fn
+
+    return register
+
+
+@contextmanager
+def with_devices(*devices):
+    """``(with-devices (D1 D2 ...) ...)`` (``source/utils.lisp:7-17``)."""
+    global USING_BACKEND
+    saved = USING_BACKEND
+    USING_BACKEND = list(devices)
+    try:
+        yield
+    finally:
+        USING_BACKEND = saved
+
+
+def find_impl(node: str, dtype: str = "float"):
+    for device in USING_BACKEND:
+        entry = DEVICE_FEATURES.get(device, {}).get(node)
+        if entry is None:
+            continue
+        fn, reject_p = entry
+        if reject_p is not None and reject_p(dtype):
+            continue
+        return fn
+    raise NodeNotFound(f"{node}: no implementation for dtype {dtype} among "
+                       f"{[d.__name__ for d in USING_BACKEND]}")
+
+
+def forward(node: str, *args, **kwargs):
+    dtype = getattr(args[0], "dtype", "float")
+    return find_impl(node, dtype)(*args, **kwargs)
+
+
+# ---------------------------------------------------------------------------
+# HIPTensor implementations
+# ---------------------------------------------------------------------------
+
+def _only_float(dtype) -> bool:
+    """reject-p: only ``:float`` runs on the device (``supported-dtypes-are``,
+    ``source/vm/nodes/utils.lisp:71-93``)."""
+    return dtype != "float"
+
+
+def view2(a: HIPTensor, b: HIPTensor) -> _lib.View2:
+    sa, sta, oa = a.geometry()
+    sb, stb, ob = b.geometry()
+    if sa != sb:
+        raise ValueError(f"shape mismatch: {sa} and {sb} (the node's :where is A[~] B[~] -> A[~])")
+    v = _lib.View2()
+    v.rank = len(sa)
+    for r, (n, x, y) in enumerate(zip(sa, sta, stb)):
+        v.shape[r] = n
+        v.stride_a[r] = x
+        v.stride_b[r] = y
+    v.off_a = oa
+    v.off_b = ob
+    return v
+
+
+def _binary(op):
+    def impl(x: HIPTensor, y: HIPTensor) -> HIPTensor:
+        v = view2(x, y)
+        _lib.check(_lib.get().wf2hip_binary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(y.ptr)))
+        return x
+
+    return impl
+
+
+def _unary(op):
+    def impl(x: HIPTensor, out: HIPTensor) -> HIPTensor:
+        v = view2(x, out)
+        _lib.check(_lib.get().wf2hip_unary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), 0.0))
+        return out
+
+    return impl
+
+
+for _name, _op in (("AddNode", _lib.ADD), ("SubNode", _lib.SUB), ("MulNode", _lib.MUL),
+                   ("DivNode", _lib.DIV), ("MoveTensorNode", _lib.MOVE)):
+    define_impl(_name, HIPTensor, _only_float)(_binary(_op))
+
+for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _lib.TANH),
+                   ("LogENode", _lib.LOG), ("ExpNode", _lib.EXP), ("SqrtNode", _lib.SQRT),
+                   ("AbsNode", _lib.ABS)):
+    define_impl(_name, HIPTensor, _only_float)(_unary(_op))
+
+
+@define_impl("ExptNode", HIPTensor, _only_float)
+def _expt(x: HIPTensor, out: HIPTensor, n: float) -> HIPTensor:
+    v = view2(x, out)
+    _lib.check(_lib.get().wf2hip_unary_nd(_lib.POW, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(n)))
+    return out
+
+
+def _matrix_geometry(t: HIPTensor, what: str):
+    """Batch shape/strides, start offset and the leading dimension of the last
+    two axes.  The last axis must be unit-stride (the CPU backend reads ldX as
+    the last-axis size of the untransposed tensor, matrix-ops.lisp:40-47)."""
+    shape, strides, off = t.geometry()
+    if len(shape) < 2:
+        raise ValueError(f"MatMulNode: {what} needs rank >= 2")
+    if shape[-1] > 1 and strides[-1] != 1:
+        raise ValueError(f"MatMulNode: {what} must be contiguous along its last axis; "
+                         "materialise it with to_contiguous first")
+    ld = strides[-2] if shape[-2] > 1 else max(shape[-1], 1)
+    if ld < shape[-1]:
+        raise ValueError(f"MatMulNode: {what} rows overlap (broadcast rows are not supported)")
+    return shape, strides, off, ld
+
+
+@define_impl("MatMulNode", HIPTensor, _only_float)
+def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
+            trans_b: bool = False) -> HIPTensor:
+    """``C[~ i k] = A[~ i j] . B[~ j k]`` through the operand-swapped
+    column-major call of ``expand-gemm-form-column``
+    (``backends/cpu/matrix-ops.lisp:12-112``): sgemm(transB, transA, n, m, k, 1,
+    B, ldb, A, lda, 0, C, ldc).  ``a``/``b`` are the tensors as stored (i.e.
+    untransposed); batch axes may be broadcast (stride 0) on either operand."""
+    sa, sta, oa, lda = _matrix_geometry(a, "A")
+    sb, stb, ob, ldb = _matrix_geometry(b, "B")
+    sc, stc, oc, ldc = _matrix_geometry(out, "C")
+    m, n = sc[-2], sc[-1]
+    k = sa[-2] if trans_a else sa[-1]
+    if (sa[-1] if trans_a else sa[-2]) != m or (sb[-1] if trans_b else sb[-2]) != k or \
+            (sb[-2] if trans_b else sb[-1]) != n:
+        raise ValueError(f"MatMulNode: shapes {sa} {'T' if trans_a else ''} x {sb} "
+                         f"{'T' if trans_b else ''} -> {sc} do not agree")
+    batch_shape = sc[:-2]
+    if sa[:-2] != batch_shape or sb[:-2] != batch_shape:
+        raise ValueError("MatMulNode: batch axes differ; view the smaller operand with (:broadcast n)")
+    lib = _lib.get()
+    ta = b"C" if trans_a else b"N"
+    tb = b"C" if trans_b else b"N"
+
+    def launch(offa, offb, offc, strides3, count):
+        _lib.check(lib.wf2hip_sgemm_strided_batched(
+            tb, ta, n, m, k, 1.0,
+            C.c_void_p(b.ptr + 4 * offb), ldb, strides3[1],
+            C.c_void_p(a.ptr + 4 * offa), lda, strides3[0],
+            0.0, C.c_void_p(out.ptr + 4 * offc), ldc, strides3[2], count))
+
+    # Collapse the batch axes into one strided axis when all three tensors
+    # allow it; otherwise loop over the outer ones on the host like the CPU
+    # backend does for every batch index.
+    nb = len(batch_shape)
+    if nb == 0:
+        launch(oa, ob, oc, (0, 0, 0), 1)
+        return out
+    inner = nb - 1
+    count = batch_shape[inner]
+    strides3 = [sta[inner], stb[inner], stc[inner]]
+    while inner > 0:
+        o = inner - 1
+        # axis o continues the run when its stride is (merged stride x merged count),
+        # which also holds for 0 == 0 x count on a broadcast operand
+        if not all(st[o] == s3 * count for st, s3 in zip((sta, stb, stc), strides3)):
+            break
+        count *= batch_shape[o]
+        inner = o
+    outer_shape = batch_shape[:inner]
+    if count > 65535:
+        raise ValueError("MatMulNode: more than 65535 matrices in one strided batch")
+
+    def rec(axis, offa, offb, offc):
+        if axis == len(outer_shape):
+            launch(offa, offb, offc, strides3, count)
+            return
+        for i in range(outer_shape[axis]):
+            rec(axis + 1, offa + i * sta[axis], offb + i * stb[axis], offc + i * stc[axis])
+
+    rec(0, oa, ob, oc)
+    return out

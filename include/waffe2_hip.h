@@ -1,0 +1,204 @@
+/*
+ * waffe2_hip.h -- C ABI of libwaffe2-hip.so, the MI355X (gfx950) tensor-kernel
+ * library behind cl-waffe2's HIPTensor backend.
+ *
+ * The library takes the place that cl-waffe2-simd.so plus the system BLAS hold
+ * for the CPUTensor backend: a host language (Common Lisp through CFFI, or any
+ * FFI) passes element counts, raw DEVICE pointers, offsets and strides.  Every
+ * entry point cites the reference interface it replaces (paths relative to the
+ * cl-waffe2 checkout).
+ *
+ * Conventions
+ *   - All data pointers are device pointers obtained from wf2hip_malloc (or
+ *     any other HIP allocation of the current device).  fp32 only.
+ *   - Strides/increments and offsets are in ELEMENTS.  inc == 0 broadcasts.
+ *   - Every function returns 0 on success or a negative WF2HIP_E* code / a
+ *     positive hipError_t; wf2hip_last_error() returns a thread-local message.
+ *     (The reference's kernels return void and have no error channel.)
+ *   - Kernels are enqueued on one stream (wf2hip_set_stream, default: the null
+ *     stream) and return without waiting; wf2hip_memcpy_d2h, wf2hip_sync and
+ *     wf2hip_event_elapsed_ms block.
+ *   - The library keeps no pointer after a call returns and never frees or
+ *     reallocates a caller's buffer.
+ */
+#ifndef WAFFE2_HIP_H
+#define WAFFE2_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WF2HIP_ABI_VERSION 1
+#define WF2HIP_MAX_RANK 8
+
+/* error codes (negative: raised by the library before any launch) */
+#define WF2HIP_OK 0
+#define WF2HIP_EINVAL (-1)     /* bad rank, negative size, null pointer          */
+#define WF2HIP_ENOTINIT (-2)   /* wf2hip_init has not succeeded                  */
+#define WF2HIP_EOVERLAP (-3)   /* in-place op on partially overlapping views     */
+#define WF2HIP_EUNSUPPORTED (-4)
+#define WF2HIP_ENOMEM (-5)
+
+/* ---- runtime ----------------------------------------------------------- */
+/* No counterpart in cl-waffe2-simd (host memory needs none); the loader
+ * pattern it follows is cl-waffe2-simd/shared-object.lisp:4-13 and the
+ * allocation hook is AbstractTensor's initialize-instance
+ * (source/vm/generic-tensor/tensor.lisp:146-210). */
+int wf2hip_abi_version(void);
+int wf2hip_init(int device);
+int wf2hip_shutdown(void);
+const char* wf2hip_last_error(void);
+/* "name|gcnArch|CUs|memory bytes" of the initialised device */
+int wf2hip_device_info(char* buf, size_t buflen);
+/* Zero-initialised device memory: cl-waffe2 relies on fresh tensors being 0
+ * (backends/lisp/tensor.lisp:12-28; !sum zero-fills by multiplying by 0,
+ * base-impl/reduction.lisp:63). */
+int wf2hip_malloc(void** ptr, size_t bytes);
+int wf2hip_free(void* ptr);
+int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int wf2hip_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int wf2hip_memcpy_d2d(void* dst, const void* src, size_t bytes);
+int wf2hip_fill_f32(float* x, size_t n, float value);
+int wf2hip_sync(void);
+/* Adopt an externally created hipStream_t (NULL = the null stream). */
+int wf2hip_set_stream(void* hip_stream);
+void* wf2hip_get_stream(void);
+/* Events on the library's stream, for timing kernels where they run. */
+int wf2hip_event_create(void** event);
+int wf2hip_event_record(void* event);
+int wf2hip_event_elapsed_ms(void* start, void* stop, float* ms);
+int wf2hip_event_destroy(void* event);
+
+/* ---- BLAS-like 1-D kernels (one-for-one with waffe2_s*) ---------------- */
+/* x[i*incx] <- x[i*incx] op y[i*incy], i < n.
+ * Replaces waffe2_s{add,sub,mul,div} (cl-waffe2-simd.c:153-250; CFFI binding
+ * cl-waffe2-simd/api.lisp:63-82).  IEEE binary32, no FMA contraction.
+ * incx == 0 makes x[0] an accumulator (x[0] <- x[0] op y[0] op y[incy] ...):
+ * add is tree-reduced unless wf2hip_set_reduce_mode(1); the others always run
+ * in the reference's sequential order. */
+int wf2hip_sadd(long n, float* x, long incx, const float* y, long incy);
+int wf2hip_ssub(long n, float* x, long incx, const float* y, long incy);
+int wf2hip_smul(long n, float* x, long incx, const float* y, long incy);
+int wf2hip_sdiv(long n, float* x, long incx, const float* y, long incy);
+/* x[i*incx] <- y[i*incy].  Replaces BLAS scopy_ as called by
+ * expand-move-form (source/backends/cpu/arithmetic.lisp:39-61): source first. */
+int wf2hip_scopy(long n, const float* y, long incy, float* x, long incx);
+/* out[i*inco] <- f(x[i*incx]).  Replaces waffe2_s{sin,cos,tanh,log,exp,sqrt,abs}
+ * (cl-waffe2-simd.c:586-706; api.lisp:212-251).  <= 2 ulp from SLEEF u10. */
+int wf2hip_ssin(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_scos(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_stanh(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_slog(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_sexp(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_ssqrt(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_sabs(long n, const float* x, long incx, float* out, long inco);
+/* out <- x^p.  Replaces waffe2_spow (cl-waffe2-simd.c:708-768; api.lisp:257-273). */
+int wf2hip_spow(long n, const float* x, long incx, float p, float* out, long inco);
+/* out[0] <- max/min_i x[i*incx].  Replaces waffe2_s{max,min}
+ * (cl-waffe2-simd.c:316-365; api.lisp:126-141). */
+int wf2hip_smax(long n, const float* x, long incx, float* out);
+int wf2hip_smin(long n, const float* x, long incx, float* out);
+
+/* ---- N-D view form: one launch per node -------------------------------- */
+/* Replaces the host loops call-with-view emits around the 1-D kernels
+ * (source/vm/generic-tensor/call-with-view.lisp:112-229,
+ * do-compiled-loop.lisp:76-164): the whole iteration space of a node in one
+ * descriptor.  For each axis r: extent shape[r]; stride_a/stride_b are the
+ * EFFECTIVE strides of the two tensors (storage stride x view step, 0 for a
+ * broadcast axis); off_a/off_b are the start offsets (tensor-initial-offset
+ * plus stride x range-nth(view, 0) per axis). */
+typedef struct wf2hip_view2 {
+  int32_t rank; /* 1..WF2HIP_MAX_RANK */
+  int32_t reserved;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t stride_a[WF2HIP_MAX_RANK];
+  int64_t stride_b[WF2HIP_MAX_RANK];
+  int64_t off_a;
+  int64_t off_b;
+} wf2hip_view2;
+
+enum wf2hip_binary_op {
+  WF2HIP_ADD = 0, /* AddNode  source/base-impl/arithmetic.lisp:57-103 */
+  WF2HIP_SUB = 1, /* SubNode  */
+  WF2HIP_MUL = 2, /* MulNode  */
+  WF2HIP_DIV = 3, /* DivNode  */
+  WF2HIP_MOVE = 4 /* MoveTensorNode source/base-impl/fundamental.lisp:9-43 */
+};
+
+enum wf2hip_unary_op {
+  WF2HIP_SIN = 16, /* SinNode  source/base-impl/mathematics.lisp:13-120 */
+  WF2HIP_COS = 17,
+  WF2HIP_TANH = 18,
+  WF2HIP_LOG = 19, /* LogENode */
+  WF2HIP_EXP = 20,
+  WF2HIP_SQRT = 21,
+  WF2HIP_ABS = 22,
+  WF2HIP_POW = 32, /* ExptNode mathematics.lisp:267-303 */
+  WF2HIP_GELU = 40 /* fused tanh-form GELU (nn/activation.lisp:45-66) */
+};
+
+/* a <- a op b over the view (a = X, the in-place destination; b = Y).
+ * Replaces the define-impl forwards of Add/Sub/Mul/Div/MoveTensorNode for
+ * CPUTensor (source/backends/cpu/arithmetic.lisp:65-144).
+ * Axes where stride_a == 0 and the extent is > 1 make `a` an accumulator:
+ * that is how cl-waffe2 expresses !sum / !mean (base-impl/reduction.lisp:5-79).
+ * WF2HIP_ADD reduces them in parallel (fp32 tree) unless reduce mode 1 is set;
+ * SUB/MUL/DIV use the sequential order of the reference; MOVE keeps the last
+ * element written, as a sequential loop would.
+ * Returns WF2HIP_EOVERLAP when a and b are different, partially overlapping
+ * windows of one buffer (the CPU result then depends on loop order). */
+int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b);
+/* b <- f(a) over the view (a = X source, b = OUT).  Replaces the
+ * define-math-impl forwards and ExptNode (source/backends/cpu/mathematics.lisp:
+ * 8-76).  `p` is the exponent for WF2HIP_POW and ignored otherwise. */
+int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p);
+
+/* 0 (default): parallel tree reduction for accumulate-into-stride-0 ADD.
+ * 1: the reference's strictly sequential fp32 order (slow; for bit parity). */
+int wf2hip_set_reduce_mode(int mode);
+int wf2hip_get_reduce_mode(void);
+
+/* ---- reductions and softmax as direct entry points ---------------------- */
+/* out[r*inco] <- out[r*inco] + sum_c x[r*ldx + c], r < rows, c < cols.
+ * What (!sum x :axis -1) lowers to after its zero-fill
+ * (base-impl/reduction.lisp:5-79). */
+int wf2hip_reduce_add_rows_f32(long rows, long cols, const float* x, long ldx,
+                               float* out, long inco);
+/* out[r*ldo + c] <- softmax over c of x[r*ldx + c], max-subtracted.
+ * One fused kernel for what !softmax composes from mean/sub/exp/sum/div
+ * (source/nn/activation.lisp:126-159). */
+int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long ldx,
+                            float* out, long ldo);
+/* Causal variant for attention scores: row r of each (seq x seq) matrix keeps
+ * columns c <= r; x is (batch, seq, seq) contiguous, scaled by `scale` first. */
+int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
+                              float scale);
+/* LayerNorm over the last axis: out = (x - mean)/sqrt(var + eps) * g + b
+ * (source/nn/norms.lisp:44-82; examples/gpt-2/utils.lisp:114-127). */
+int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
+                              const float* beta, float eps, float* out);
+
+/* ---- gemm ---------------------------------------------------------------- */
+/* Column-major C(m x n) <- alpha op(A) op(B) + beta C with the argument
+ * meaning of Fortran sgemm_, scalars by value.  Replaces the BLAS call of
+ * expand-gemm-form-column/-row (source/backends/cpu/matrix-ops.lisp:12-212;
+ * binding source/backends/cpu/blas-functions.lisp:34-38).  fp32 MFMA. */
+int wf2hip_sgemm(char transa, char transb, long m, long n, long k, float alpha,
+                 const float* A, long lda, const float* B, long ldb, float beta,
+                 float* C, long ldc);
+/* Same product for `batch` matrices strideA/strideB/strideC elements apart
+ * (stride 0 re-uses one operand): the host loop over batch axes that
+ * call-with-view :at-least-dim 2 emits (matrix-ops.lisp:214-237), in one
+ * launch. */
+int wf2hip_sgemm_strided_batched(char transa, char transb, long m, long n, long k,
+                                 float alpha, const float* A, long lda, long strideA,
+                                 const float* B, long ldb, long strideB, float beta,
+                                 float* C, long ldc, long strideC, long batch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WAFFE2_HIP_H */

@@ -1,0 +1,265 @@
+"""ctypes front end of the CPU oracle (``libwaffe2_oracle.so``) and of the
+compiled reference kernels (``_ref/libwaffe2_simd_ref.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the
+CPU-baseline leg of the benchmark.  The product package never imports it.
+
+The oracle restates cl-waffe2's CPUTensor + cl-waffe2-simd path; see the header
+of ``waffe2_oracle.c`` for the reference file:line each function follows.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ORACLE_SO = os.path.join(_HERE, "libwaffe2_oracle.so")
+_REF_SO = os.path.join(_HERE, "_ref", "libwaffe2_simd_ref.so")
+
+MAX_RANK = 8
+MAX_TENSORS = 3
+
+# view kinds of orc_views.kind
+KIND_T, KIND_BROADCAST, KIND_OTHER = 0, 1, 2
+
+OPS = {
+    "add": 0, "sub": 1, "mul": 2, "div": 3, "move": 4,
+    "sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21,
+    "abs": 22, "pow": 32,
+}
+
+
+class OrcViews(C.Structure):
+    _fields_ = [
+        ("rank", C.c_int),
+        ("ntensors", C.c_int),
+        ("shape", C.c_long * MAX_RANK),
+        ("stride", (C.c_long * MAX_RANK) * MAX_TENSORS),
+        ("kind", (C.c_int * MAX_RANK) * MAX_TENSORS),
+        ("first", (C.c_long * MAX_RANK) * MAX_TENSORS),
+        ("step", (C.c_long * MAX_RANK) * MAX_TENSORS),
+        ("offset", C.c_long * MAX_TENSORS),
+    ]
+
+
+class OrcCall(C.Structure):
+    _fields_ = [
+        ("n", C.c_long),
+        ("off", C.c_long * MAX_TENSORS),
+        ("inc", C.c_long * MAX_TENSORS),
+    ]
+
+
+def build(force: bool = False) -> None:
+    """Compile the oracle (and ``_ref`` when the reference checkout exists)."""
+    if force or not os.path.exists(_ORACLE_SO) or (
+        os.path.getmtime(_ORACLE_SO)
+        < os.path.getmtime(os.path.join(_HERE, "waffe2_oracle.c"))
+    ):
+        subprocess.check_call(["make", "-C", _HERE, "oracle"], stdout=subprocess.DEVNULL)
+    if force or not os.path.exists(_REF_SO):
+        subprocess.call(["make", "-C", _HERE, "ref"], stdout=subprocess.DEVNULL,
+                        stderr=subprocess.DEVNULL)
+
+
+def _torch_cpu_lib() -> str | None:
+    import importlib.util
+
+    spec = importlib.util.find_spec("torch")
+    if spec is None or spec.origin is None:
+        return None
+    path = os.path.join(os.path.dirname(spec.origin), "lib", "libtorch_cpu.so")
+    return path if os.path.exists(path) else None
+
+
+_lib = None
+_ref = None
+_F = C.POINTER(C.c_float)
+
+
+def _fp(a: np.ndarray, offset: int = 0):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return C.cast(a.ctypes.data + 4 * offset, _F)
+
+
+def lib():
+    """The oracle library, with SLEEF resolved when a provider is present."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_ORACLE_SO):
+        build()
+    L = C.CDLL(_ORACLE_SO)
+    for name in ("add", "sub", "mul", "div"):
+        f = getattr(L, "orc_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
+        f.restype = None
+    L.orc_scopy.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
+    L.orc_scopy.restype = None
+    for name in ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs"):
+        f = getattr(L, "orc_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
+        f.restype = None
+    L.orc_spow.argtypes = [C.c_long, _F, C.c_long, C.c_float, _F, C.c_long]
+    L.orc_spow.restype = None
+    for name in ("max", "min"):
+        f = getattr(L, "orc_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F]
+        f.restype = None
+    L.orc_schedule.argtypes = [C.POINTER(OrcViews), C.POINTER(OrcCall), C.c_long]
+    L.orc_schedule.restype = C.c_long
+    L.orc_node_nd.argtypes = [C.c_int, C.POINTER(OrcViews), _F, _F, C.c_float]
+    L.orc_node_nd.restype = C.c_long
+    L.orc_sgemm.argtypes = [C.c_char, C.c_char, C.c_long, C.c_long, C.c_long,
+                            C.c_float, _F, C.c_long, _F, C.c_long, C.c_float,
+                            _F, C.c_long]
+    L.orc_sgemm.restype = None
+    L.orc_matmul_rowmajor.argtypes = [C.c_int, C.c_int, C.c_long, C.c_long,
+                                      C.c_long, _F, C.c_long, _F, C.c_long, _F,
+                                      C.c_long]
+    L.orc_matmul_rowmajor.restype = None
+    L.orc_sleef_open.argtypes = [C.c_char_p]
+    L.orc_sleef_open.restype = C.c_int
+    L.orc_sleef_available.restype = C.c_int
+    tl = _torch_cpu_lib()
+    if tl is not None:
+        L.orc_sleef_open(tl.encode())
+    _lib = L
+    return L
+
+
+def sleef_available() -> bool:
+    return bool(lib().orc_sleef_available())
+
+
+def ref():
+    """The reference's own C kernels compiled into ``_ref`` (or None)."""
+    global _ref
+    if _ref is not None:
+        return _ref
+    if not os.path.exists(_REF_SO):
+        return None
+    try:
+        R = C.CDLL(_REF_SO)
+    except OSError:
+        return None
+    for name in ("add", "sub", "mul", "div", "sin", "cos", "tanh", "log", "exp",
+                 "sqrt", "abs"):
+        f = getattr(R, "waffe2_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
+        f.restype = None
+    R.waffe2_spow.argtypes = [C.c_long, _F, C.c_long, C.c_float, _F, C.c_long]
+    R.waffe2_spow.restype = None
+    for name in ("max", "min"):
+        f = getattr(R, "waffe2_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F]
+        f.restype = None
+    _ref = R
+    return R
+
+
+# ---------------------------------------------------------------------------
+# 1-D kernels on numpy storage (in place on `x`, like the reference)
+# ---------------------------------------------------------------------------
+
+def binary_1d(op: str, n: int, x: np.ndarray, incx: int, y: np.ndarray, incy: int,
+              offx: int = 0, offy: int = 0, use_ref: bool = False) -> None:
+    L = ref() if use_ref else lib()
+    name = ("waffe2_s" if use_ref else "orc_s") + op
+    getattr(L, name)(n, _fp(x, offx), incx, _fp(y, offy), incy)
+
+
+def copy_1d(n: int, y: np.ndarray, incy: int, x: np.ndarray, incx: int,
+            offy: int = 0, offx: int = 0) -> None:
+    lib().orc_scopy(n, _fp(y, offy), incy, _fp(x, offx), incx)
+
+
+def unary_1d(op: str, n: int, x: np.ndarray, incx: int, out: np.ndarray, inco: int,
+             offx: int = 0, offo: int = 0, use_ref: bool = False) -> None:
+    L = ref() if use_ref else lib()
+    name = ("waffe2_s" if use_ref else "orc_s") + op
+    getattr(L, name)(n, _fp(x, offx), incx, _fp(out, offo), inco)
+
+
+def pow_1d(n: int, x: np.ndarray, incx: int, p: float, out: np.ndarray, inco: int,
+           use_ref: bool = False) -> None:
+    L = ref() if use_ref else lib()
+    name = "waffe2_spow" if use_ref else "orc_spow"
+    getattr(L, name)(n, _fp(x), incx, C.c_float(p), _fp(out), inco)
+
+
+def maxmin_1d(op: str, n: int, x: np.ndarray, incx: int, use_ref: bool = False) -> float:
+    L = ref() if use_ref else lib()
+    out = np.zeros(1, np.float32)
+    getattr(L, ("waffe2_s" if use_ref else "orc_s") + op)(n, _fp(x), incx, _fp(out))
+    return float(out[0])
+
+
+# ---------------------------------------------------------------------------
+# Views / scheduler
+# ---------------------------------------------------------------------------
+
+def make_views(shape, tensors) -> OrcViews:
+    """``tensors``: list of dicts with keys stride, kind, first, step, offset
+    (per-axis lists; see waffe2_oracle.c for their meaning)."""
+    v = OrcViews()
+    v.rank = len(shape)
+    v.ntensors = len(tensors)
+    for r, s in enumerate(shape):
+        v.shape[r] = int(s)
+    for t, d in enumerate(tensors):
+        v.offset[t] = int(d.get("offset", 0))
+        for r in range(len(shape)):
+            v.stride[t][r] = int(d["stride"][r])
+            v.kind[t][r] = int(d["kind"][r])
+            v.first[t][r] = int(d["first"][r])
+            v.step[t][r] = int(d["step"][r])
+    return v
+
+
+def schedule(views: OrcViews, cap: int = 1 << 16):
+    """List of (n, offs, incs) 1-D calls the reference's compiled loop makes."""
+    buf = (OrcCall * cap)()
+    cnt = lib().orc_schedule(C.byref(views), buf, cap)
+    out = []
+    for i in range(min(cnt, cap)):
+        c = buf[i]
+        out.append((c.n, tuple(c.off[: views.ntensors]), tuple(c.inc[: views.ntensors])))
+    return cnt, out
+
+
+def node_nd(op: str, views: OrcViews, t0: np.ndarray, t1: np.ndarray, p: float = 0.0) -> None:
+    """Run a node over N-D views exactly as the CPU backend would: binary/move
+    ops write into ``t0`` (x <- x op y); unary/pow read ``t0`` and write ``t1``."""
+    rc = lib().orc_node_nd(OPS[op], C.byref(views), _fp(t0), _fp(t1), C.c_float(p))
+    if rc != 0:
+        raise ValueError("orc_node_nd rejected the views")
+
+
+# ---------------------------------------------------------------------------
+# gemm
+# ---------------------------------------------------------------------------
+
+def sgemm(transa: str, transb: str, m: int, n: int, k: int, alpha: float,
+          A: np.ndarray, lda: int, B: np.ndarray, ldb: int, beta: float,
+          Cm: np.ndarray, ldc: int) -> None:
+    lib().orc_sgemm(transa.encode(), transb.encode(), m, n, k, C.c_float(alpha),
+                    _fp(A), lda, _fp(B), ldb, C.c_float(beta), _fp(Cm), ldc)
+
+
+def matmul_rowmajor(A: np.ndarray, B: np.ndarray, trans_a: bool = False,
+                    trans_b: bool = False) -> np.ndarray:
+    """Row-major ``op(A) @ op(B)`` through the reference's operand-swapped
+    column-major sgemm call (backends/cpu/matrix-ops.lisp:12-112)."""
+    A = np.ascontiguousarray(A, np.float32)
+    B = np.ascontiguousarray(B, np.float32)
+    m, k = (A.shape[1], A.shape[0]) if trans_a else A.shape
+    k2, n = (B.shape[1], B.shape[0]) if trans_b else B.shape
+    assert k == k2
+    out = np.zeros((m, n), np.float32)
+    lib().orc_matmul_rowmajor(int(trans_a), int(trans_b), m, n, k, _fp(A), A.shape[1],
+                              _fp(B), B.shape[1], _fp(out), n)
+    return out

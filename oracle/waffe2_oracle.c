@@ -1,0 +1,471 @@
+/*
+ * waffe2_oracle.c -- CPU restatement of cl-waffe2's CPUTensor + cl-waffe2-simd
+ * tensor-kernel path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP kernels are
+ * compared against (tests, the smoke check and the CPU-baseline leg of the
+ * benchmark).  Nothing in the shipped library may call, link or fall back to
+ * it.
+ *
+ * Every function cites the reference file:line it follows (paths relative to
+ * the cl-waffe2 checkout).  The arithmetic is plain C compiled with
+ * -ffp-contract=off so that + - * / are single IEEE-754 binary32 operations,
+ * exactly as _mm256_{add,sub,mul,div}_ps are in the reference.
+ *
+ * Third-party arithmetic that is NOT in the reference checkout:
+ *   - SLEEF (un-vendored submodule third_party/sleef, no commit pin): the
+ *     unary math kernels call Sleef_<f>f8_u10avx2.  The oracle resolves those
+ *     very symbols at run time from a library that exports SLEEF 3.8.0
+ *     (PyTorch's libtorch_cpu.so); when none is found it falls back to libm in
+ *     double precision and orc_sleef_available() returns 0 so that the caller
+ *     can say so.
+ *   - BLAS sgemm_/scopy_ (system libblas, unpinned; CI installs netlib
+ *     reference BLAS): restated here from the published netlib reference
+ *     algorithm (column-major, j-l-i loop nest for 'N','N').
+ *
+ * Pinning status (which independent check covers each function) is recorded
+ * in tests/test_oracle_*.py:
+ *   orc_s{add,sub,mul,div}, orc_scopy  : golden vectors from the compiled
+ *       reference C (tests/golden), numpy IEEE closed form, reference test
+ *       vectors 10 op 1 -> 11/9/10/10.
+ *   orc_s{exp,log,tanh,sin,sqrt}, orc_spow : golden vectors from the compiled
+ *       reference C; float64 truth within 1 ulp; special values.
+ *   orc_s{max,min}                     : golden vectors, numpy max/min.
+ *   orc_schedule / orc_*_nd            : worked schedules derived by hand from
+ *       do-compiled-loop.lisp, exactly-once coverage invariant, brute-force
+ *       N-D index walk on random tiny views.
+ *   orc_sgemm                          : the reference's integer gemm vectors
+ *       (base-impl/t/arithmetic.lisp:120,135,142,148), float64 truth.
+ */
+#define _GNU_SOURCE
+#include <dlfcn.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+#define ORC_SIMD 8 /* SIMD_SINGLE_STRIDE, simd/x86_64/avx2.h:26 */
+
+/* ------------------------------------------------------------------ */
+/* SLEEF resolution                                                    */
+/* ------------------------------------------------------------------ */
+
+typedef float v8f __attribute__((vector_size(32)));
+typedef v8f (*sleef_f8_1)(v8f);
+typedef v8f (*sleef_f8_2)(v8f, v8f);
+
+static void *g_sleef_handle = NULL;
+static int g_sleef_tried = 0;
+
+ORC_API int orc_sleef_open(const char *path) {
+  g_sleef_tried = 1;
+  g_sleef_handle = dlopen(path, RTLD_NOW | RTLD_GLOBAL);
+  if (!g_sleef_handle) return 0;
+  if (!dlsym(g_sleef_handle, "Sleef_expf8_u10avx2")) {
+    g_sleef_handle = NULL;
+    return 0;
+  }
+  return 1;
+}
+
+ORC_API int orc_sleef_available(void) { return g_sleef_handle != NULL; }
+
+static void *sleef_sym(const char *name) {
+  if (!g_sleef_handle) return NULL;
+  return dlsym(g_sleef_handle, name);
+}
+
+/* ------------------------------------------------------------------ */
+/* x <- x op y   (cl-waffe2-simd.c:153-250, define_arithmetic_func)     */
+/* ------------------------------------------------------------------ */
+/* The reference handles incx >= 1 in blocks of 8 (load 8 x, load 8 y,
+ * compute, store 8) and everything else -- the n%8 tail, and the whole range
+ * when incx <= 0 -- with a sequential scalar loop (:205-212).  incx == 0 is
+ * therefore a strictly sequential accumulate into x[0]. */
+#define ORC_DEFINE_ARITH(name, OP)                                            \
+  ORC_API void orc_s##name(long n, float *x, long incx, const float *y,      \
+                           long incy) {                                       \
+    long count = 0;                                                           \
+    const long simd_end = (n / ORC_SIMD) * ORC_SIMD;                          \
+    if (incx >= 1) {                                                          \
+      while (count != simd_end) {                                             \
+        float vx[ORC_SIMD], vy[ORC_SIMD];                                     \
+        for (int i = 0; i < ORC_SIMD; i++) vx[i] = x[(count + i) * incx];     \
+        for (int i = 0; i < ORC_SIMD; i++) vy[i] = y[(count + i) * incy];     \
+        for (int i = 0; i < ORC_SIMD; i++) vx[i] = vx[i] OP vy[i];            \
+        for (int i = 0; i < ORC_SIMD; i++) x[(count + i) * incx] = vx[i];     \
+        count += ORC_SIMD;                                                    \
+      }                                                                       \
+    }                                                                         \
+    x += count * incx;                                                        \
+    y += count * incy;                                                        \
+    while (count != n) {                                                      \
+      count += 1;                                                             \
+      x[0] = x[0] OP y[0];                                                    \
+      x += incx;                                                              \
+      y += incy;                                                              \
+    }                                                                         \
+  }
+
+ORC_DEFINE_ARITH(add, +)
+ORC_DEFINE_ARITH(sub, -)
+ORC_DEFINE_ARITH(mul, *)
+ORC_DEFINE_ARITH(div, /)
+
+/* x <- y strided copy.  backends/cpu/arithmetic.lisp:39-61 passes
+ * (n, y, incy, x, incx) to BLAS scopy_, i.e. source first.  Netlib scopy
+ * with non-negative increments is a plain strided copy. */
+ORC_API void orc_scopy(long n, const float *y, long incy, float *x, long incx) {
+  for (long i = 0; i < n; i++) x[i * incx] = y[i * incy];
+}
+
+/* ------------------------------------------------------------------ */
+/* out <- f(x)   (cl-waffe2-simd.c:586-706, define_math_func)           */
+/* ------------------------------------------------------------------ */
+/* Blocks of 8 go through SLEEF u10 when incx >= 1; the tail and the whole
+ * range when incx <= 0 use libm in double precision, narrowed to float
+ * (:636-641: `y[0] = sin(x[0])` with float operands promotes to double). */
+static void unary_apply(long n, const float *x, long incx, float *out,
+                        long inco, const char *sleef_name,
+                        double (*libm_f)(double)) {
+  long count = 0;
+  const long simd_end = (n / ORC_SIMD) * ORC_SIMD;
+  sleef_f8_1 vf = (sleef_f8_1)sleef_sym(sleef_name);
+  if (incx >= 1) {
+    while (count != simd_end) {
+      float in[ORC_SIMD] __attribute__((aligned(32)));
+      float res[ORC_SIMD] __attribute__((aligned(32)));
+      for (int i = 0; i < ORC_SIMD; i++) in[i] = x[(count + i) * incx];
+      if (vf) {
+        v8f v;
+        memcpy(&v, in, sizeof v);
+        v = vf(v);
+        memcpy(res, &v, sizeof v);
+      } else {
+        for (int i = 0; i < ORC_SIMD; i++) res[i] = (float)libm_f((double)in[i]);
+      }
+      for (int i = 0; i < ORC_SIMD; i++) out[(count + i) * inco] = res[i];
+      count += ORC_SIMD;
+    }
+  }
+  x += count * incx;
+  out += count * inco;
+  while (count != n) {
+    count += 1;
+    out[0] = (float)libm_f((double)x[0]);
+    x += incx;
+    out += inco;
+  }
+}
+
+#define ORC_DEFINE_UNARY(name, sleef, libm)                                  \
+  ORC_API void orc_s##name(long n, const float *x, long incx, float *out,   \
+                           long inco) {                                      \
+    unary_apply(n, x, incx, out, inco, sleef, libm);                         \
+  }
+
+/* avx2.h:265,291,308,322,325 and cl-waffe2-simd.c:645,670,685,697,703 */
+ORC_DEFINE_UNARY(sin, "Sleef_sinf8_u10avx2", sin)
+ORC_DEFINE_UNARY(cos, "Sleef_cosf8_u10avx2", cos)
+ORC_DEFINE_UNARY(tanh, "Sleef_tanhf8_u10avx2", tanh)
+ORC_DEFINE_UNARY(log, "Sleef_logf8_u10avx2", log)
+ORC_DEFINE_UNARY(exp, "Sleef_expf8_u10avx2", exp)
+ORC_DEFINE_UNARY(sqrt, "Sleef_sqrtf8_u05avx2", sqrt)
+ORC_DEFINE_UNARY(abs, "Sleef_fabsf8_avx2", fabs)
+
+/* out <- x^p  (cl-waffe2-simd.c:708-768; avx2.h:304) */
+ORC_API void orc_spow(long n, const float *x, long incx, float p, float *out,
+                      long inco) {
+  long count = 0;
+  const long simd_end = (n / ORC_SIMD) * ORC_SIMD;
+  sleef_f8_2 vf = (sleef_f8_2)sleef_sym("Sleef_powf8_u10avx2");
+  if (incx >= 1) {
+    while (count != simd_end) {
+      float in[ORC_SIMD], res[ORC_SIMD];
+      for (int i = 0; i < ORC_SIMD; i++) in[i] = x[(count + i) * incx];
+      if (vf) {
+        v8f v, pv;
+        memcpy(&v, in, sizeof v);
+        for (int i = 0; i < ORC_SIMD; i++) pv[i] = p;
+        v = vf(v, pv);
+        memcpy(res, &v, sizeof v);
+      } else {
+        for (int i = 0; i < ORC_SIMD; i++)
+          res[i] = (float)pow((double)in[i], (double)p);
+      }
+      for (int i = 0; i < ORC_SIMD; i++) out[(count + i) * inco] = res[i];
+      count += ORC_SIMD;
+    }
+  }
+  x += count * incx;
+  out += count * inco;
+  while (count != n) {
+    count += 1;
+    out[0] = (float)pow((double)x[0], (double)p);
+    x += incx;
+    out += inco;
+  }
+}
+
+/* out[0] <- max/min over x  (cl-waffe2-simd.c:316-365).  _mm256_max_ps(a,b)
+ * returns b when either operand is NaN; MAX(a,b) = a > b ? a : b. */
+#define ORC_DEFINE_MAXMIN(name, CMP)                                          \
+  ORC_API void orc_s##name(long n, const float *x, long incx, float *out) {  \
+    float best = x[0];                                                        \
+    float lanes[ORC_SIMD];                                                    \
+    long count = 0;                                                           \
+    const long simd_end = (n / ORC_SIMD) * ORC_SIMD;                          \
+    for (int i = 0; i < ORC_SIMD; i++) lanes[i] = best;                       \
+    while (count != simd_end) {                                               \
+      for (int i = 0; i < ORC_SIMD; i++) {                                    \
+        float v = x[(count + i) * incx];                                      \
+        lanes[i] = (lanes[i] CMP v) ? lanes[i] : v;                           \
+      }                                                                       \
+      count += ORC_SIMD;                                                      \
+    }                                                                         \
+    for (int i = 0; i < ORC_SIMD; i++)                                        \
+      best = (best CMP lanes[i]) ? best : lanes[i];                           \
+    x += count * incx;                                                        \
+    while (count != n) {                                                      \
+      count += 1;                                                             \
+      best = (best CMP x[0]) ? best : x[0];                                   \
+      x += incx;                                                              \
+    }                                                                         \
+    out[0] = best;                                                            \
+  }
+
+ORC_DEFINE_MAXMIN(max, >)
+ORC_DEFINE_MAXMIN(min, <)
+
+/* ------------------------------------------------------------------ */
+/* Loop scheduler                                                      */
+/* ------------------------------------------------------------------ */
+/* Restates solve-loop-order (vm/generic-tensor/do-compiled-loop.lisp:76-164)
+ * with rest-contiguous-p (:46-73) and the emitter call-with-view
+ * (call-with-view.lisp:112-229) for kernel rank 1 (element-wise), all tensors
+ * sharing one permute order.
+ *
+ * A tensor axis is described by
+ *   stride   the storage stride of the axis in elements
+ *            (tensor-stride, utils.lisp:50-67)
+ *   kind     0 = T (whole axis), 1 = (:broadcast n), 2 = anything else
+ *            (index, slice, stepped slice; view.lisp:120-138)
+ *   first    range-nth(view, 0)                 (iterator/range.lisp:74-98)
+ *   step     range-nth(view, 1) - range-nth(view, 0)
+ * and a tensor by its axes plus tensor-initial-offset.
+ *
+ * The result is the list of 1-D calls the compiled loop makes:
+ *   (n, off_0, inc_0, off_1, inc_1, ...) per call, offsets in elements. */
+
+#define ORC_MAX_RANK 8
+#define ORC_MAX_TENSORS 3
+
+typedef struct {
+  int rank;
+  int ntensors;
+  long shape[ORC_MAX_RANK];
+  long stride[ORC_MAX_TENSORS][ORC_MAX_RANK];
+  int kind[ORC_MAX_TENSORS][ORC_MAX_RANK];
+  long first[ORC_MAX_TENSORS][ORC_MAX_RANK];
+  long step[ORC_MAX_TENSORS][ORC_MAX_RANK];
+  long offset[ORC_MAX_TENSORS];
+} orc_views;
+
+typedef struct {
+  long n;
+  long off[ORC_MAX_TENSORS];
+  long inc[ORC_MAX_TENSORS];
+} orc_call;
+
+/* rest-contiguous-p: from `rank` on, every view of every tensor is T or
+ * broadcast, and within one tensor they all have the same type. */
+static int rest_contiguous_p(const orc_views *v, int rank) {
+  for (int t = 0; t < v->ntensors; t++) {
+    for (int r = rank; r < v->rank; r++) {
+      if (v->kind[t][r] != 0 && v->kind[t][r] != 1) return 0;
+      if (v->kind[t][r] != v->kind[t][rank]) return 0;
+    }
+  }
+  return 1;
+}
+
+typedef void (*orc_emit_fn)(const orc_call *c, void *ctx);
+
+static void emit_rec(const orc_views *v, int rank, long *offsets,
+                     orc_emit_fn emit, void *ctx) {
+  if (rest_contiguous_p(v, rank)) {
+    /* :apply-flatten (do-compiled-loop.lisp:113-137, call-with-view.lisp:
+     * 160-195): one call over the product of the remaining extents; stride 1,
+     * or 0 for a broadcast tensor.  Offsets add stride*range-nth(0) of every
+     * remaining non-broadcast axis (all T here, so zero). */
+    orc_call c;
+    c.n = 1;
+    for (int r = rank; r < v->rank; r++) c.n *= v->shape[r];
+    for (int t = 0; t < v->ntensors; t++) {
+      long off = offsets[t];
+      for (int r = rank; r < v->rank; r++)
+        if (v->kind[t][r] != 1) off += v->stride[t][r] * v->first[t][r];
+      c.off[t] = off;
+      c.inc[t] = (v->kind[t][rank] == 1) ? 0 : 1;
+    }
+    emit(&c, ctx);
+    return;
+  }
+  if (v->rank - rank == 1) {
+    /* :apply (do-compiled-loop.lisp:141-155): the innermost axis as one call
+     * with size shape[last], stride = stride*step or 0 if broadcast. */
+    orc_call c;
+    c.n = v->shape[rank];
+    for (int t = 0; t < v->ntensors; t++) {
+      int bc = v->kind[t][rank] == 1;
+      c.off[t] = offsets[t] + (bc ? 0 : v->stride[t][rank] * v->first[t][rank]);
+      c.inc[t] = bc ? 0 : v->stride[t][rank] * v->step[t][rank];
+    }
+    emit(&c, ctx);
+    return;
+  }
+  /* :batch (call-with-view.lisp:120-159): host loop over this axis; each
+   * tensor's offset starts at stride*range-nth(0) and advances by
+   * stride*(range-nth(1)-range-nth(0)) unless the axis is broadcast. */
+  long local[ORC_MAX_TENSORS];
+  for (int t = 0; t < v->ntensors; t++) {
+    local[t] = offsets[t];
+    if (v->kind[t][rank] != 1) local[t] += v->stride[t][rank] * v->first[t][rank];
+  }
+  for (long i = 0; i < v->shape[rank]; i++) {
+    emit_rec(v, rank + 1, local, emit, ctx);
+    for (int t = 0; t < v->ntensors; t++)
+      if (v->kind[t][rank] != 1) local[t] += v->stride[t][rank] * v->step[t][rank];
+  }
+}
+
+typedef struct {
+  orc_call *out;
+  long cap;
+  long count;
+} collect_ctx;
+
+static void collect_emit(const orc_call *c, void *p) {
+  collect_ctx *ctx = (collect_ctx *)p;
+  if (ctx->count < ctx->cap) ctx->out[ctx->count] = *c;
+  ctx->count++;
+}
+
+/* Returns the number of 1-D calls; writes at most `cap` of them. */
+ORC_API long orc_schedule(const orc_views *v, orc_call *out, long cap) {
+  collect_ctx ctx = {out, cap, 0};
+  long offsets[ORC_MAX_TENSORS];
+  for (int t = 0; t < v->ntensors; t++) offsets[t] = v->offset[t];
+  if (v->rank == 0) return 0;
+  emit_rec(v, 0, offsets, collect_emit, &ctx);
+  return ctx.count;
+}
+
+/* N-D node execution = schedule + the 1-D kernel per call
+ * (backends/cpu/arithmetic.lisp:32-37, 39-61; mathematics.lisp:8-32,55-76). */
+typedef struct {
+  int op;
+  float *a;
+  float *b;
+  float p;
+} exec_ctx;
+
+enum {
+  ORC_ADD = 0,
+  ORC_SUB,
+  ORC_MUL,
+  ORC_DIV,
+  ORC_MOVE,
+  ORC_SIN = 16,
+  ORC_COS,
+  ORC_TANH,
+  ORC_LOG,
+  ORC_EXP,
+  ORC_SQRT,
+  ORC_ABS,
+  ORC_POW = 32
+};
+
+static void exec_emit(const orc_call *c, void *p) {
+  exec_ctx *e = (exec_ctx *)p;
+  float *a = e->a + c->off[0];
+  float *b = e->b + c->off[1];
+  switch (e->op) {
+    case ORC_ADD: orc_sadd(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_SUB: orc_ssub(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_MUL: orc_smul(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_DIV: orc_sdiv(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_MOVE: orc_scopy(c->n, b, c->inc[1], a, c->inc[0]); break;
+    /* unary: tensor 0 = x (source), tensor 1 = out */
+    case ORC_SIN: orc_ssin(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_COS: orc_scos(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_TANH: orc_stanh(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_LOG: orc_slog(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_EXP: orc_sexp(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_SQRT: orc_ssqrt(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_ABS: orc_sabs(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_POW: orc_spow(c->n, a, c->inc[0], e->p, b, c->inc[1]); break;
+    default: break;
+  }
+}
+
+/* Binary/move: tensor 0 = x (destination, in place), tensor 1 = y.
+ * Unary/pow: tensor 0 = x (source), tensor 1 = out. */
+ORC_API long orc_node_nd(int op, const orc_views *v, float *t0, float *t1,
+                         float p) {
+  exec_ctx e = {op, t0, t1, p};
+  long offsets[ORC_MAX_TENSORS];
+  collect_ctx unused = {NULL, 0, 0};
+  (void)unused;
+  if (v->rank == 0 || v->ntensors != 2) return -1;
+  for (int t = 0; t < v->ntensors; t++) offsets[t] = v->offset[t];
+  emit_rec(v, 0, offsets, exec_emit, &e);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* sgemm                                                               */
+/* ------------------------------------------------------------------ */
+/* Column-major C(m x n) <- alpha*op(A)*op(B) + beta*C with Fortran sgemm_
+ * argument meaning (backends/cpu/blas-functions.lisp:34-38,
+ * backends/cpu/blas.lisp:76-92), restated from the netlib reference BLAS loop
+ * nests (fp32 accumulation in the order l = 0..k-1). */
+ORC_API void orc_sgemm(char transa, char transb, long m, long n, long k,
+                       float alpha, const float *A, long lda, const float *B,
+                       long ldb, float beta, float *C, long ldc) {
+  const int nota = (transa == 'N' || transa == 'n');
+  const int notb = (transb == 'N' || transb == 'n');
+  for (long j = 0; j < n; j++) {
+    if (nota) {
+      for (long i = 0; i < m; i++)
+        C[i + j * ldc] = (beta == 0.0f) ? 0.0f : beta * C[i + j * ldc];
+      for (long l = 0; l < k; l++) {
+        float temp = alpha * (notb ? B[l + j * ldb] : B[j + l * ldb]);
+        for (long i = 0; i < m; i++) C[i + j * ldc] += temp * A[i + l * lda];
+      }
+    } else {
+      for (long i = 0; i < m; i++) {
+        float temp = 0.0f;
+        for (long l = 0; l < k; l++)
+          temp += A[l + i * lda] * (notb ? B[l + j * ldb] : B[j + l * ldb]);
+        C[i + j * ldc] =
+            (beta == 0.0f) ? alpha * temp : alpha * temp + beta * C[i + j * ldc];
+      }
+    }
+  }
+}
+
+/* Row-major C[m,n] = A[m,k] . B[k,n] the way expand-gemm-form-column calls
+ * it (backends/cpu/matrix-ops.lisp:12-112): operands swapped,
+ * sgemm_(transB, transA, n, m, k, 1, B, ldb, A, lda, 0, C, ldc), where the
+ * leading dimensions are the last-axis sizes of the untransposed tensors. */
+ORC_API void orc_matmul_rowmajor(int trans_a, int trans_b, long m, long n,
+                                 long k, const float *A, long lda,
+                                 const float *B, long ldb, float *C, long ldc) {
+  orc_sgemm(trans_b ? 'C' : 'N', trans_a ? 'C' : 'N', n, m, k, 1.0f, B, ldb, A,
+            lda, 0.0f, C, ldc);
+}
+
+ORC_API int orc_abi_version(void) { return 1; }

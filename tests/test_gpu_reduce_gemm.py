@@ -1,0 +1,322 @@
+"""GPU parity of reductions, softmax, LayerNorm and gemm.
+
+Bar (BASELINE north_star): <= 1e-5 relative error for reductions and gemm
+(relative to the sum of magnitudes, because a sum of N(0,1) values is itself
+~0); bit-exact against the oracle in the sequential reduce mode; the
+reference's own integer test vectors exactly.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import assert_bit_equal, oracle_views, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-5
+
+
+def dptr(t, offset=0):
+    return C.c_void_p(t.ptr + 4 * offset)
+
+
+def test_sum_tester_vectors(gpu):
+    """sum-tester / mean-tester of the reference
+    (base-impl/t/reduction.lisp:9-48): ones(100,100,100) -> 1e6 for axis t,
+    100 for axis 0 / 1 / -1, 10000 for axes (0 1); mean -> 1.0."""
+    F = gpu.functional
+    ones = F.make_tensor((100, 100, 100), initial_element=1.0)
+    assert F.sum(ones).numpy().ravel().tolist() == [1000000.0]
+    for axis in (0, 1, -1):
+        out = F.sum(ones, axis=axis)
+        assert out.size == 10000 and np.all(out.numpy() == 100.0)
+    out = F.sum(ones, axis=(0, 1))
+    assert out.shape == [1, 1, 100] and np.all(out.numpy() == 10000.0)
+    assert np.all(F.mean(ones, axis=1).numpy() == 1.0)
+    assert F.mean(ones).numpy().ravel().tolist() == [1.0]
+    kd = F.sum(ones, axis=1, keepdims=True)
+    assert kd.shape == [100, 100, 100] and np.all(kd.numpy() == 100.0)
+
+
+def test_config4_row_and_full_sum(gpu, O):
+    """BASELINE config 4: row sum and full sum of (8192, 4096) N(0,1), seed 4.
+    Tree mode against float64 truth; a slice of it in sequential mode against
+    the oracle's strictly ordered fp32 accumulation, bit for bit."""
+    W = gpu
+    F = W.functional
+    rng = np.random.Generator(np.random.PCG64(4))
+    A = rng.standard_normal((8192, 4096)).astype(np.float32)
+    dA = F.from_numpy(A)
+    A64 = A.astype(np.float64)
+    mag_rows = np.abs(A64).sum(axis=1)
+    got = F.sum(dA, axis=1).numpy().ravel()
+    assert np.all(np.abs(got - A64.sum(axis=1)) <= REL * mag_rows)
+    got = F.sum(dA).numpy().ravel()[0]
+    assert abs(got - A64.sum()) <= REL * np.abs(A64).sum()
+    # the GPU tree result must also be at least as close to the truth as the
+    # reference's own sequential fp32 order is
+    seq = np.zeros(1, np.float32)
+    O.binary_1d("add", A.size, seq, 0, A.ravel(), 1)
+    assert abs(got - A64.sum()) <= abs(float(seq[0]) - A64.sum()) + 1e-3
+
+    lib = W.lib.get()
+    W.lib.check(lib.wf2hip_set_reduce_mode(1))
+    try:
+        small = dA.view((0, 64), True)
+        got = F.sum(small, axis=1).numpy().ravel()
+        want = np.zeros(64, np.float32)
+        for r in range(64):
+            O.binary_1d("add", 4096, want, 0, A[r], 1, offx=r)
+        assert_bit_equal(got, want, "sequential row sums")
+        got = F.sum(small).numpy().ravel()
+        want = np.zeros(1, np.float32)
+        O.binary_1d("add", 64 * 4096, want, 0, np.ascontiguousarray(A[:64]).ravel(), 1)
+        assert_bit_equal(got, want, "sequential full sum")
+    finally:
+        W.lib.check(lib.wf2hip_set_reduce_mode(0))
+
+
+@pytest.mark.parametrize("shape,axis", [((7, 13), 1), ((7, 13), 0), ((5, 6, 7), (0, 2)), ((5, 6, 7), 1),
+                                        ((3000,), True), ((1, 70000), 1), ((3, 1 << 18), 1),
+                                        ((2, 3, 4, 5), (1, 3)), ((300, 300), True), ((64, 1000), 0),
+                                        ((513, 2049), 1), ((4, 5000, 3), 1)])
+def test_reduce_shapes(gpu, shape, axis):
+    """Row, column, mixed and split-row reductions against float64."""
+    F = gpu.functional
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal(shape).astype(np.float32)
+    npaxis = None if axis is True else axis
+    want = x.astype(np.float64).sum(axis=npaxis, keepdims=True)
+    mag = np.abs(x.astype(np.float64)).sum(axis=npaxis, keepdims=True)
+    got = F.sum(F.from_numpy(x), axis=axis).numpy()
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= REL * mag)
+    gotm = F.mean(F.from_numpy(x), axis=axis).numpy()
+    cnt = x.size / want.size
+    assert np.all(np.abs(gotm - want / cnt) <= REL * mag / cnt + 1e-7)
+
+
+def test_accumulate_adds_to_existing_value(gpu):
+    """AddNode into a stride-0 destination is x += sum(y), not x = sum(y)."""
+    W = gpu
+    x = W.HIPTensor.from_numpy(np.array([[10.0], [20.0]], np.float32))
+    y = W.HIPTensor.from_numpy(np.arange(12, dtype=np.float32).reshape(2, 6))
+    W.forward("AddNode", x.view(True, (":broadcast", 6)), y)
+    assert x.numpy().ravel().tolist() == [25.0, 71.0]
+    out = np.zeros(3, np.float32) + 5
+    d = W.HIPTensor.from_numpy(out)
+    W.lib.check(W.lib.get().wf2hip_reduce_add_rows_f32(3, 4, dptr(W.HIPTensor.from_numpy(np.ones((3, 4), np.float32))),
+                                                      4, dptr(d), 1))
+    assert d.numpy().tolist() == [9.0, 9.0, 9.0]
+
+
+def test_max_min(gpu, O):
+    W = gpu
+    rng = np.random.default_rng(3)
+    for n, inc in [(1, 1), (5, 1), (8, 1), (1000, 1), (1000, 3), (100000, 1), (3000000, 1)]:
+        x = rng.standard_normal(n * inc).astype(np.float32)
+        dx = W.HIPTensor.from_numpy(x)
+        out = W.HIPTensor([1])
+        W.lib.check(W.lib.get().wf2hip_smax(n, dptr(dx), inc, dptr(out)))
+        assert out.numpy()[0] == O.maxmin_1d("max", n, x, inc) == x[::inc][:n].max()
+        W.lib.check(W.lib.get().wf2hip_smin(n, dptr(dx), inc, dptr(out)))
+        assert out.numpy()[0] == O.maxmin_1d("min", n, x, inc) == x[::inc][:n].min()
+
+
+def _softmax64(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+def test_config4_softmax(gpu):
+    """BASELINE config 4: max-subtracted row softmax of (32768, 1024) N(0, 3^2)
+    logits, seed 4 -- fused kernel against the float64 closed form; invariants
+    of the reference's tests (rows sum to 1, nn/t/activation.lisp:9-12) and
+    shift invariance."""
+    W = gpu
+    F = W.functional
+    rng = np.random.Generator(np.random.PCG64(4))
+    rng.standard_normal((8192, 4096))  # config 4 draws the sum tensor first
+    X = (rng.standard_normal((32768, 1024)) * 3.0).astype(np.float32)
+    got = F.softmax_fused(F.from_numpy(X)).numpy()
+    want = _softmax64(X)
+    assert ulp_distance(got, want.astype(np.float32)).max() <= 2
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
+    shifted = F.softmax_fused(F.from_numpy(X[:256] + np.float32(8.0))).numpy()
+    np.testing.assert_allclose(shifted, _softmax64(X[:256] + np.float32(8.0)), rtol=1e-5, atol=1e-12)
+
+
+@pytest.mark.parametrize("cols", [1, 3, 64, 100, 255, 256, 1000, 1024, 2050, 4096, 5000, 20000])
+def test_softmax_widths(gpu, cols):
+    F = gpu.functional
+    rng = np.random.default_rng(cols)
+    X = (rng.standard_normal((37, cols)) * 4).astype(np.float32)
+    got = F.softmax_fused(F.from_numpy(X)).numpy()
+    assert ulp_distance(got, _softmax64(X).astype(np.float32)).max() <= 2
+
+
+def test_softmax_reference_composition(gpu, O):
+    """!softmax exactly as the reference composes it (mean-subtract, axis 1):
+    each node against the oracle running the same node on the CPU."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(9)
+    X = rng.standard_normal((64, 96)).astype(np.float32)
+    got = F.softmax(F.from_numpy(X)).numpy()
+    # oracle: same decomposition, sequential CPU semantics
+    s = np.zeros(64, np.float32)
+    for r in range(64):
+        O.binary_1d("add", 96, s, 0, X[r], 1, offx=r)
+    mean = s / np.float32(96.0)
+    x1 = X - mean[:, None]
+    e = np.zeros_like(x1)
+    O.unary_1d("exp", x1.size, x1.ravel(), 1, e.reshape(-1), 1)
+    z = np.zeros(64, np.float32)
+    for r in range(64):
+        O.binary_1d("add", 96, z, 0, e[r], 1, offx=r)
+    want = e / z[:, None]
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-9)
+    np.testing.assert_allclose(got, _softmax64(X), rtol=1e-5)
+    assert np.abs(got.sum(axis=1) - 1).max() < 1e-5
+
+
+def test_causal_softmax(gpu):
+    W = gpu
+    rng = np.random.default_rng(6)
+    for batch, seq in [(3, 64), (2, 100), (2, 1024), (1, 7)]:
+        X = rng.standard_normal((batch, seq, seq)).astype(np.float32) * 5
+        scale = np.float32(0.125)
+        dx = W.HIPTensor.from_numpy(X)
+        out = W.HIPTensor(X.shape)
+        W.lib.check(W.lib.get().wf2hip_causal_softmax_f32(batch, seq, dptr(dx), dptr(out), float(scale)))
+        s = (X * scale).astype(np.float64)
+        mask = np.tril(np.ones((seq, seq), bool))
+        s = np.where(mask, s, -np.inf)
+        want = _softmax64(s)
+        got = out.numpy()
+        assert np.all(got[:, ~mask] == 0.0)
+        assert ulp_distance(got, want.astype(np.float32)).max() <= 2
+
+
+def test_layernorm(gpu):
+    """Fused LayerNorm against float64, and the node-for-node recipe of
+    LayerNorm-Revisit (examples/gpt-2/utils.lisp:114-127) against it."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(7)
+    for rows, cols in [(64, 768), (10, 100), (5, 1), (33, 2048), (7, 255)]:
+        X = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+        g = rng.standard_normal(cols).astype(np.float32)
+        b = rng.standard_normal(cols).astype(np.float32)
+        X64 = X.astype(np.float64)
+        mu = X64.mean(axis=1, keepdims=True)
+        var = ((X64 - mu) ** 2).mean(axis=1, keepdims=True)
+        want = (X64 - mu) / np.sqrt(var + 1e-5) * g + b
+        got = F.layer_norm_fused(F.from_numpy(X), F.from_numpy(g), F.from_numpy(b)).numpy()
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=2e-6)
+        got = F.layer_norm(F.from_numpy(X), F.from_numpy(g), F.from_numpy(b)).numpy()
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+# ---------------------------------------------------------------------------
+# gemm
+# ---------------------------------------------------------------------------
+
+def test_matmul_reference_vectors(gpu):
+    """matmul-tester, -mnk, -mnk1, matmul-both-transposed
+    (base-impl/t/arithmetic.lisp:116-149): integer-valued, exact under any
+    correct gemm."""
+    F = gpu.functional
+    a33 = F.from_numpy(np.arange(9, dtype=np.float32).reshape(3, 3))
+    a34 = F.from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4))
+    assert F.matmul(a33, a33).numpy().ravel().tolist() == [15, 18, 21, 42, 54, 66, 69, 90, 111]
+    assert F.matmul(a34, F.t(a34)).numpy().ravel().tolist() == [14, 38, 62, 38, 126, 214, 62, 214, 366]
+    assert F.matmul(F.t(a34), a34).numpy().ravel().tolist() == [80, 92, 104, 116, 92, 107, 122, 137, 104, 122,
+                                                               140, 158, 116, 137, 158, 179]
+    assert F.matmul(F.t(a33), F.t(a33)).numpy().ravel().tolist() == [15, 42, 69, 18, 54, 90, 21, 66, 111]
+
+
+def _gemm_check(got, A64, B64):
+    want = A64 @ B64
+    bound = REL * (np.abs(A64) @ np.abs(B64)) + 1e-30
+    assert np.all(np.abs(got - want) <= bound), float(np.max(np.abs(got - want) / bound))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 5, 7), (128, 128, 16), (129, 127, 33), (256, 384, 64),
+                                   (100, 260, 1000), (64, 64, 4), (512, 768, 768), (1000, 10, 3), (2, 300, 130)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_random(gpu, m, n, k, ta, tb):
+    F = gpu.functional
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    A = rng.standard_normal((m, k)).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    dA = F.t(F.from_numpy(np.ascontiguousarray(A.T))) if ta else F.from_numpy(A)
+    dB = F.t(F.from_numpy(np.ascontiguousarray(B.T))) if tb else F.from_numpy(B)
+    got = F.matmul(dA, dB).numpy()
+    _gemm_check(got, A.astype(np.float64), B.astype(np.float64))
+
+
+def test_sgemm_column_major_contract(gpu, O):
+    """wf2hip_sgemm keeps Fortran sgemm_ semantics (column-major, alpha/beta,
+    leading dimensions larger than the matrix), checked against the oracle's
+    netlib restatement."""
+    W = gpu
+    rng = np.random.default_rng(77)
+    lib = W.lib.get()
+    for ta, tb in [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")]:
+        m, n, k = 37, 29, 53
+        lda = (m if ta == "N" else k) + 3
+        ldb = (k if tb == "N" else n) + 5
+        ldc = m + 2
+        A = rng.standard_normal(lda * (k if ta == "N" else m)).astype(np.float32)
+        B = rng.standard_normal(ldb * (n if tb == "N" else k)).astype(np.float32)
+        Cm = rng.standard_normal(ldc * n).astype(np.float32)
+        want = Cm.copy()
+        O.sgemm(ta, tb, m, n, k, 0.75, A, lda, B, ldb, -1.5, want, ldc)
+        dA, dB, dC = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B), W.HIPTensor.from_numpy(Cm)
+        W.lib.check(lib.wf2hip_sgemm(ta.encode(), tb.encode(), m, n, k, 0.75, dptr(dA), lda, dptr(dB), ldb,
+                                     -1.5, dptr(dC), ldc))
+        got = dC.numpy()
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+        # padding rows of C (ldc > m) are never written
+        pad = np.arange(got.size) % ldc >= m
+        assert_bit_equal(got[pad], Cm[pad], "ldc padding")
+    # beta == 0 must not read C (NaN in C stays out of the result)
+    nanC = W.HIPTensor.from_numpy(np.full(16, np.nan, np.float32))
+    eye = W.HIPTensor.from_numpy(np.eye(4, dtype=np.float32).ravel())
+    W.lib.check(lib.wf2hip_sgemm(b"N", b"N", 4, 4, 4, 1.0, dptr(eye), 4, dptr(eye), 4, 0.0, dptr(nanC), 4))
+    assert nanC.numpy().tolist() == np.eye(4).ravel().tolist()
+    assert lib.wf2hip_sgemm(b"X", b"N", 4, 4, 4, 1.0, dptr(eye), 4, dptr(eye), 4, 0.0, dptr(nanC), 4) == -1
+    assert lib.wf2hip_sgemm(b"N", b"N", 4, 4, 4, 1.0, dptr(eye), 2, dptr(eye), 4, 0.0, dptr(nanC), 4) == -1
+
+
+def test_matmul_batched_and_broadcast(gpu):
+    """Batch axes, a rank-2 weight against a rank-3 activation (the !flexible
+    broadcast of nn/regression.lisp:14-18), permuted head layouts."""
+    F = gpu.functional
+    rng = np.random.default_rng(31)
+    X = rng.standard_normal((4, 50, 24)).astype(np.float32)
+    Wt = rng.standard_normal((24, 36)).astype(np.float32)
+    got = F.matmul(F.from_numpy(X), F.from_numpy(Wt)).numpy()
+    for b in range(4):
+        _gemm_check(got[b], X[b].astype(np.float64), Wt.astype(np.float64))
+    Q = rng.standard_normal((2, 3, 40, 16)).astype(np.float32)
+    K = rng.standard_normal((2, 3, 40, 16)).astype(np.float32)
+    got = F.matmul(F.from_numpy(Q), F.t(F.from_numpy(K))).numpy()
+    assert got.shape == (2, 3, 40, 40)
+    for b in range(2):
+        for h in range(3):
+            _gemm_check(got[b, h], Q[b, h].astype(np.float64), K[b, h].T.astype(np.float64))
+    # heads read straight out of a fused (B, T, 3, H, hd) projection: batch
+    # strides that do not merge -> host loop over the outer batch axis
+    qkv = rng.standard_normal((2, 40, 3, 3, 16)).astype(np.float32)
+    d = F.from_numpy(qkv)
+    q = d.view(True, True, 0, True, True)
+    q = F.reshape(F.copy(q.permute(0, 2, 3, 1, 4)), 2, 3, 40, 16)
+    got = F.matmul(q, F.t(q)).numpy()
+    for b in range(2):
+        for h in range(3):
+            M = qkv[b, :, 0, h, :].astype(np.float64)
+            _gemm_check(got[b, h], M, M.T)
