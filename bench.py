@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIPTensor kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the hot path over one batch of synthetic fp32 input
+at the metric size, 2^26 elements = (8192, 8192), seed 6:
+
+    x <- x + y      AddNode, in place, both operands full      12 B/elem
+    x <- x * y      MulNode, in place                          12 B/elem
+    o <- exp(y)     ExpNode                                     8 B/elem
+    r <- r + sum_c y[:, c]   (!sum y :axis 1)                   4 B/elem
+
+`value` is the algorithmic bytes of a step divided by its time (GB/s), with all
+inputs resident in HBM before the timed region.  Every launch works on a
+different buffer set of a ring much larger than the 256 MB Infinity Cache, so
+no launch finds its operands cached from the previous one.
+
+Extra fields: per-kernel GB/s, the roofline of the dominant kernel (the
+in-place binary kernel) from HIP events recorded on the library's stream, the
+GPT-2-small block forward time, and the CPU baseline (the reference's own C
+kernels compiled under oracle/_ref when present, else the oracle port) timed
+on one host core -- cl-waffe2 runs these kernels single-threaded
+(`*num-cores*` = 1, no define-impl passes :lparallel).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N = 1 << 26
+SIDE = 8192
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+BYTES = {"add": 12 * N, "mul": 12 * N, "exp": 8 * N, "rowsum": 4 * N + 4 * SIDE}
+RING = 8  # buffer sets: 8 x (x, y, o) x 256 MiB = 6 GiB
+
+
+def p(t):
+    return C.c_void_p(t.ptr)
+
+
+def gpu_steps(W, steps: int, warmup: int):
+    lib = W.lib.get()
+    rng = np.random.Generator(np.random.PCG64(6))
+    hx = rng.standard_normal(N).astype(np.float32)
+    hy = rng.standard_normal(N).astype(np.float32)
+    x0, y0 = W.HIPTensor.from_numpy(hx), W.HIPTensor.from_numpy(hy)
+    del hx, hy
+    ring = []
+    for i in range(RING):
+        xs, ys, os_ = (W.HIPTensor([N]) for _ in range(3))
+        W.lib.check(lib.wf2hip_memcpy_d2d(p(xs), p(x0), 4 * N))
+        W.lib.check(lib.wf2hip_memcpy_d2d(p(ys), p(y0), 4 * N))
+        ring.append((xs, ys, os_, W.HIPTensor([SIDE])))
+    W.lib.synchronize()
+
+    def launch(name, slot):
+        xs, ys, os_, rs = ring[slot % RING]
+        if name == "add":
+            W.lib.check(lib.wf2hip_sadd(N, p(xs), 1, p(ys), 1))
+        elif name == "mul":
+            W.lib.check(lib.wf2hip_smul(N, p(xs), 1, p(ys), 1))
+        elif name == "exp":
+            W.lib.check(lib.wf2hip_sexp(N, p(ys), 1, p(os_), 1))
+        else:
+            W.lib.check(lib.wf2hip_reduce_add_rows_f32(SIDE, SIDE, p(ys), SIDE, p(rs), 1))
+
+    order = ["add", "mul", "exp", "rowsum"]
+    slot = 0
+    for _ in range(warmup):
+        for name in order:
+            launch(name, slot)
+            slot += 1
+    W.lib.synchronize()
+
+    # timed region: K steps; events between the kernels attribute time per kernel
+    marks = [[W.lib.Event() for _ in range(len(order) + 1)] for _ in range(steps)]
+    W.lib.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        marks[s][0].record()
+        for k, name in enumerate(order):
+            launch(name, slot)
+            slot += 1
+            marks[s][k + 1].record()
+    W.lib.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per_kernel = {name: 0.0 for name in order}
+    step_ms = 0.0
+    for s in range(steps):
+        for k, name in enumerate(order):
+            per_kernel[name] += marks[s][k].elapsed_ms(marks[s][k + 1])
+        step_ms += marks[s][0].elapsed_ms(marks[s][-1])
+    per_kernel = {k: v / steps for k, v in per_kernel.items()}
+    # the binary kernel alone, back to back, for the roofline entry
+    reps = max(steps, 20)
+    e0, e1 = W.lib.Event(), W.lib.Event()
+    e0.record()
+    for _ in range(reps):
+        launch("add", slot)
+        slot += 1
+    e1.record()
+    binary_ms = e0.elapsed_ms(e1) / reps
+    return step_ms / steps, wall_ms / steps, per_kernel, binary_ms
+
+
+def block_forward_ms(W, reps: int = 5):
+    try:
+        gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
+    except ImportError:
+        return None
+    params = gpt2.make_block_params(seed=5)
+    x = gpt2.make_block_input(seed=5)
+    dparams = gpt2.to_device(params)
+    dx = W.HIPTensor.from_numpy(x)
+    out = {}
+    for mode in ("nodes", "fused"):
+        for _ in range(2):
+            gpt2.block_forward(dx, dparams, mode=mode)
+        e0, e1 = W.lib.Event(), W.lib.Event()
+        e0.record()
+        for _ in range(reps):
+            gpt2.block_forward(dx, dparams, mode=mode)
+        e1.record()
+        out[mode] = e0.elapsed_ms(e1) / reps
+    return out
+
+
+def cpu_baseline():
+    """The same step on one host core over the full 2^26 sample, through the
+    reference's compiled C kernels when oracle/_ref is present."""
+    from oracle import oracle as O
+
+    O.build()
+    use_ref = O.ref() is not None
+    rng = np.random.Generator(np.random.PCG64(6))
+    x = rng.standard_normal(N).astype(np.float32)
+    y = rng.standard_normal(N).astype(np.float32)
+    o = np.zeros(N, np.float32)
+    r = np.zeros(SIDE, np.float32)
+    t0 = time.perf_counter()
+    reps = 0
+    while reps < 2 or time.perf_counter() - t0 < 10.0:
+        O.binary_1d("add", N, x, 1, y, 1, use_ref=use_ref)
+        O.binary_1d("mul", N, x, 1, y, 1, use_ref=use_ref)
+        O.unary_1d("exp", N, y, 1, o, 1, use_ref=use_ref)
+        for row in range(SIDE):  # the reference's schedule: one incx = 0 call per row
+            O.binary_1d("add", SIDE, r, 0, y, 1, offx=row, offy=row * SIDE, use_ref=use_ref)
+        reps += 1
+        if time.perf_counter() - t0 > 30.0:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    gbs = sum(BYTES.values()) / dt / 1e9
+    return {
+        "value": round(gbs, 3),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "reference" if use_ref else "port",
+        "sample": f"{reps} full steps at 2^26 elements (add, mul, exp, 8192 row sums), "
+                  f"{dt:.2f} s each, 1 thread as in the reference (lparallel off, *num-cores* 1), "
+                  f"SLEEF {'from libtorch_cpu.so' if O.sleef_available() else 'absent: libm'}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-block", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on ONE GPU (no collectives, no sharding); "
+                 "--gpus must be 1")
+
+    W = importlib.import_module("cl-waffe2_amd")
+    W.lib.init(0)  # raises if libwaffe2-hip.so is missing: there is no CPU fallback
+    info = W.lib.device_info()
+
+    step_ms, wall_ms, per_kernel, binary_ms = gpu_steps(W, args.steps, args.warmup)
+    total_bytes = sum(BYTES.values())
+    value = total_bytes / step_ms / 1e6
+    kernels = {k: {"ms": round(v, 5), "GB/s": round(BYTES[k] / v / 1e6, 1),
+                   "frac_hbm_peak": round(BYTES[k] / v / 1e6 / HBM_PEAK_GBS, 4)}
+               for k, v in per_kernel.items()}
+    achieved = BYTES["add"] / binary_ms / 1e6
+    result = {
+        "metric": "fp32 elem-wise/reduce GB/s (% HBM peak) @2^26 elems; GPT-2 block fwd ms",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 5),
+        "wall_ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "x+=y, x*=y, o=exp(y), row-sum(y) on fp32 (8192,8192)=2^26 elements, N(0,1) seed 6; "
+                        "cold-cache ring of 8 buffer sets",
+            "elements": N,
+            "bytes_per_step": total_bytes,
+            "device": info["name"] or info["arch"],
+            "arch": info["arch"],
+        },
+        "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "kernels": kernels,
+        "roofline": {
+            "kernel": "ew_rows<OpAdd, ReadDst, VEC 4, U 4, NT> (x <- x + y, 2^26 elements)",
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": BYTES["add"],
+            "avg_launch_ms": round(binary_ms, 5),
+        },
+    }
+    if not args.no_block:
+        blk = block_forward_ms(W)
+        if blk is not None:
+            flop = 141.7e9
+            result["gpt2_block_fwd_ms"] = {k: round(v, 4) for k, v in blk.items()}
+            result["gpt2_block_gemm_tflops_if_all_gemm"] = {
+                k: round(flop / v / 1e9, 1) for k, v in blk.items()}
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

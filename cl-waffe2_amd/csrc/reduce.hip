@@ -95,7 +95,7 @@ __device__ __forceinline__ void row_offsets(const RowRedParams& p, uint32_t row,
 
 // Sum of b[lo, hi) by `nthreads` cooperating threads; `t` is this thread's
 // rank among them.  VEC == 4 needs b + lo 16-byte aligned.
-template <int VEC>
+template <int VEC, bool NT = false>
 __device__ __forceinline__ double strided_sum(const float* __restrict__ b, int64_t lo, int64_t hi,
                                               int t, int nthreads) {
   double acc0 = 0.0, acc1 = 0.0;
@@ -104,13 +104,13 @@ __device__ __forceinline__ double strided_sum(const float* __restrict__ b, int64
     const f4* bv = reinterpret_cast<const f4*>(b + lo);
     int64_t i = t;
     for (; i + nthreads < nvec; i += 2 * (int64_t)nthreads) {
-      f4 v0 = bv[i];
-      f4 v1 = bv[i + nthreads];
+      f4 v0 = NT ? __builtin_nontemporal_load(bv + i) : bv[i];
+      f4 v1 = NT ? __builtin_nontemporal_load(bv + i + nthreads) : bv[i + nthreads];
       acc0 += ((double)v0.x + (double)v0.y) + ((double)v0.z + (double)v0.w);
       acc1 += ((double)v1.x + (double)v1.y) + ((double)v1.z + (double)v1.w);
     }
     if (i < nvec) {
-      f4 v0 = bv[i];
+      f4 v0 = NT ? __builtin_nontemporal_load(bv + i) : bv[i];
       acc0 += ((double)v0.x + (double)v0.y) + ((double)v0.z + (double)v0.w);
     }
     for (int64_t c = lo + nvec * 4 + t; c < hi; c += nthreads) acc1 += (double)b[c];
@@ -121,7 +121,7 @@ __device__ __forceinline__ double strided_sum(const float* __restrict__ b, int64
 }
 
 // One workgroup per (row, split).
-template <int VEC>
+template <int VEC, bool NT = false>
 __global__ __launch_bounds__(kBlock) void reduce_rows_block(RowRedParams p) {
   __shared__ double lds[kWavesPerBlock];
   const uint32_t row = blockIdx.x / p.splits;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block(RowRedParams p) {
   row_offsets(p, row, &aoff, &boff);
   int64_t lo = (int64_t)split * p.seg;
   int64_t hi = lo + p.seg < p.n0 ? lo + p.seg : p.n0;
-  double v = strided_sum<VEC>(p.b + boff, lo, hi, threadIdx.x, kBlock);
+  double v = strided_sum<VEC, NT>(p.b + boff, lo, hi, threadIdx.x, kBlock);
   double total = block_sum(v, lds);
   if (threadIdx.x == 0) {
     if (p.splits == 1)
@@ -153,13 +153,15 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_wave(RowRedParams p) {
 }
 
 __global__ __launch_bounds__(kBlock) void reduce_rows_finish(RowRedParams p) {
-  const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
-  if (row >= p.nrows) return;
+  __shared__ double lds[kWavesPerBlock];
+  const uint32_t row = blockIdx.x;
   int64_t aoff, boff;
   row_offsets(p, row, &aoff, &boff);
   double t = 0.0;
-  for (uint32_t s = 0; s < p.splits; s++) t += p.partials[(int64_t)row * p.splits + s];
-  p.a[aoff] = (float)((double)p.a[aoff] + t);
+  for (uint32_t s = threadIdx.x; s < p.splits; s += kBlock)
+    t += p.partials[(int64_t)row * p.splits + s];
+  double total = block_sum(t, lds);
+  if (threadIdx.x == 0) p.a[aoff] = (float)((double)p.a[aoff] + total);
 }
 
 // ---- generic accumulation: one wavefront per destination element ----------------
@@ -303,13 +305,16 @@ static int launch_row_reduce(const Space& s, float* a, const float* b) {
   int64_t blocks = nrows * p.splits;
   if (blocks >= ((int64_t)1 << 31))
     return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
-  if (vec_ok)
+  // far beyond the Infinity Cache: stream with non-temporal loads
+  if (vec_ok && nrows * p.n0 * 4 >= ((int64_t)192 << 20))
+    reduce_rows_block<4, true><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else if (vec_ok)
     reduce_rows_block<4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   else
     reduce_rows_block<1><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   WF2_TRY(after_launch("reduce_rows_block"));
   if (p.splits > 1) {
-    reduce_rows_finish<<<(uint32_t)ceil_div(nrows, kBlock), kBlock, 0, st>>>(p);
+    reduce_rows_finish<<<(uint32_t)nrows, kBlock, 0, st>>>(p);
     WF2_TRY(after_launch("reduce_rows_finish"));
   }
   return 0;
@@ -468,9 +473,10 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
   for (int g = 0; g < NV; g++)
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      float d = r.v[g][c] - m;  // binary32 subtraction, like a SubNode
-      // exp underflows to +0 below -104; -inf (padding) must give exactly 0
-      double ed = (d < -104.0f) ? 0.0 : exp_core((double)d);
+      // x - max is exact in binary64, so the only rounding is the final one;
+      // exp underflows to +0 below -104 and -inf (padding) must give exactly 0
+      double d = (double)r.v[g][c] - (double)m;
+      double ed = (d < -104.0) ? 0.0 : exp_core(d);
       e[g][c] = ed;
       sum += ed;
     }
@@ -501,8 +507,8 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __rest
   for (int i = 1; i < kWavesPerBlock; i++) m = fmaxf(m, lmax[i]);
   double s = 0.0;
   for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
-    float d = xr[c] - m;
-    s += (d < -104.0f) ? 0.0 : exp_core((double)d);
+    double d = (double)xr[c] - (double)m;
+    s += (d < -104.0) ? 0.0 : exp_core(d);
   }
   s = wave_sum(s);
   if ((threadIdx.x & (kWave - 1)) == 0) lsum[threadIdx.x / kWave] = s;
@@ -511,8 +517,8 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __rest
   for (int i = 0; i < kWavesPerBlock; i++) s += lsum[i];
   const double inv = 1.0 / s;
   for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
-    float d = xr[c] - m;
-    double ed = (d < -104.0f) ? 0.0 : exp_core((double)d);
+    double d = (double)xr[c] - (double)m;
+    double ed = (d < -104.0) ? 0.0 : exp_core(d);
     orow[c] = (float)(ed * inv);
   }
 }

@@ -1,0 +1,119 @@
+"""GPT-2-small-style transformer block forward on HIPTensor nodes.
+
+Op decomposition follows the reference's GPT-2 example
+(``examples/gpt-2/model.lisp:95-137`` block wiring, ``utils.lisp:114-127``
+LayerNorm-Revisit, ``:204-239`` split-heads / SelfAttention / merge-heads,
+``source/nn/activation.lisp:45-66`` GELU) with the standard definitions the
+benchmark configuration asks for where the example deviates: causal mask,
+scores scaled by 1/sqrt(head_dim), softmax over the key axis, max-subtracted.
+Weights are stored ``[in, out]`` and applied as ``x @ W + b`` like the example
+(``model.lisp:118-122``).
+
+Two modes:
+
+``nodes``  every step is one of the backend's AbstractNode implementations:
+           LayerNorm and GELU node for node, heads materialised with
+           MoveTensorNode copies of sliced/permuted views, scaling and masking
+           as MulNode / AddNode with broadcast operands, row softmax kernel.
+``fused``  the same mathematics with the fused row kernels (LayerNorm, GELU,
+           scale+mask+softmax) and zero-copy heads: the attention gemms read
+           q/k/v straight out of the (B, T, 3, H, hd) projection through
+           strides and write the context straight into (B, T, H*hd).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+
+from . import functional as F
+from . import lib as _lib
+from .tensor import HIPTensor
+
+CONFIG = dict(batch=8, seq=1024, d_model=768, n_head=12, head_dim=64, d_ff=3072, eps=1e-5)
+
+
+def make_block_params(seed: int = 5, cfg: dict = CONFIG) -> dict:
+    """Weights ~ N(0, 0.02^2), zero biases, LayerNorm gamma 1 / beta 0; drawn
+    after the input from one PCG64 stream (see make_block_input)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, ff = cfg["d_model"], cfg["d_ff"]
+    rng.standard_normal((cfg["batch"], cfg["seq"], d))  # the input comes first
+    w = lambda *s: (rng.standard_normal(s) * 0.02).astype(np.float32)  # noqa: E731
+    return {
+        "w_qkv": w(d, 3 * d), "w_o": w(d, d), "w_fc": w(d, ff), "w_proj": w(ff, d),
+        "b_qkv": np.zeros(3 * d, np.float32), "b_o": np.zeros(d, np.float32),
+        "b_fc": np.zeros(ff, np.float32), "b_proj": np.zeros(d, np.float32),
+        "ln1_g": np.ones(d, np.float32), "ln1_b": np.zeros(d, np.float32),
+        "ln2_g": np.ones(d, np.float32), "ln2_b": np.zeros(d, np.float32),
+    }
+
+
+def make_block_input(seed: int = 5, cfg: dict = CONFIG) -> np.ndarray:
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rng.standard_normal((cfg["batch"], cfg["seq"], cfg["d_model"])).astype(np.float32)
+
+
+def to_device(params: dict) -> dict:
+    return {k: HIPTensor.from_numpy(v) for k, v in params.items()}
+
+
+def causal_mask(seq: int) -> HIPTensor:
+    """(1, 1, T, T) additive mask: 0 on and below the diagonal, -inf above."""
+    m = np.where(np.tril(np.ones((seq, seq), bool)), 0.0, -np.inf).astype(np.float32)
+    return HIPTensor.from_numpy(m.reshape(1, 1, seq, seq))
+
+
+def _linear(x: HIPTensor, w: HIPTensor, b: HIPTensor) -> HIPTensor:
+    """``(!add (!matmul x w) (%transform b[i] -> [~ i]))``; the product is a
+    fresh tensor, so the bias is added in place."""
+    return F.add_(F.matmul(x, w), b)
+
+
+def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG,
+                  mask: HIPTensor | None = None) -> HIPTensor:
+    B, T, D = x.shape
+    H = cfg["n_head"]
+    hd = D // H
+    scale = 1.0 / math.sqrt(hd)
+    eps = cfg["eps"]
+    fused = mode == "fused"
+    if mode not in ("fused", "nodes"):
+        raise ValueError("mode must be 'fused' or 'nodes'")
+    ln = F.layer_norm_fused if fused else F.layer_norm
+    act = F.gelu_fused if fused else F.gelu
+
+    h = ln(x, p["ln1_g"], p["ln1_b"], eps)
+    qkv = _linear(h, p["w_qkv"], p["b_qkv"])                       # (B, T, 3D)
+
+    if fused:
+        five = F.reshape(qkv, B, T, 3, H, hd)
+        # (B, 1, H, T, hd) strided windows of the projection, no copy
+        q, k, v = (five.view(True, True, i, True, True).permute(0, 2, 3, 1, 4) for i in range(3))
+        scores = F.matmul(q, F.t(k))                                # (B, 1, H, T, T)
+        probs = HIPTensor(scores.shape)
+        _lib.check(_lib.get().wf2hip_causal_softmax_f32(B * H, T, C.c_void_p(scores.ptr),
+                                                       C.c_void_p(probs.ptr), scale))
+        ctx_store = HIPTensor([B, T, 1, H, hd])
+        F.matmul(probs, v, out=ctx_store.permute(0, 2, 3, 1, 4))    # written as (B, T, H*hd)
+        ctx = F.reshape(ctx_store, B, T, D)
+    else:
+        def heads(i):  # split-heads: slice, reshape, permute, materialise
+            part = qkv.view(True, True, (i * D, (i + 1) * D))
+            return F.copy(F.reshape(part, B, T, H, hd).permute(0, 2, 1, 3))  # (B, H, T, hd)
+        q, k, v = heads(0), heads(1), heads(2)
+        scores = F.mul_(F.matmul(q, F.t(k)), scale)                 # (B, H, T, T)
+        if mask is None:
+            mask = causal_mask(T)
+        F.add_(scores, mask)                                        # broadcast over (B, H)
+        probs = F.softmax_fused(scores)
+        ctx = F.matmul(probs, v)                                    # (B, H, T, hd)
+        ctx = F.reshape(ctx.permute(0, 2, 1, 3), B, T, D)           # merge-heads (copies)
+
+    attn = _linear(ctx, p["w_o"], p["b_o"])
+    x1 = F.add(x, attn)                                             # residual
+    h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)
+    f = act(_linear(h2, p["w_fc"], p["b_fc"]))
+    m = _linear(f, p["w_proj"], p["b_proj"])
+    return F.add_(m, x1)                                            # residual, in place in m

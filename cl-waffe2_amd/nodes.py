@@ -190,7 +190,10 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
 
     # Collapse the batch axes into one strided axis when all three tensors
     # allow it; otherwise loop over the outer ones on the host like the CPU
-    # backend does for every batch index.
+    # backend does for every batch index.  Extent-1 axes carry no information.
+    keep = [i for i, n in enumerate(batch_shape) if n != 1]
+    batch_shape = [batch_shape[i] for i in keep]
+    sta, stb, stc = ([st[i] for i in keep] for st in (sta, stb, stc))
     nb = len(batch_shape)
     if nb == 0:
         launch(oa, ob, oc, (0, 0, 0), 1)
