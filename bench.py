@@ -115,6 +115,34 @@ def gpu_steps(W, steps: int, warmup: int):
     return step_ms / steps, wall_ms / steps, per_kernel, binary_ms
 
 
+def counter_probe(W, reps: int = 5):
+    """A short fixed sequence for `rocprofv3 --pmc` runs: `reps` launches each of
+    a plain copy of known size (2^26 floats: 256 MiB read, 256 MiB written; the
+    calibration for FETCH_SIZE / WRITE_SIZE) and of the four metric kernels, each
+    on a different buffer set so that no launch finds its data in cache."""
+    lib = W.lib.get()
+    ring = [(W.HIPTensor([N], initial_element=1.0), W.HIPTensor([N], initial_element=1.0),
+             W.HIPTensor([N]), W.HIPTensor([SIDE])) for _ in range(RING)]
+    W.lib.synchronize()
+    slot = 0
+    for name in ("copy", "add", "mul", "exp", "rowsum"):
+        for _ in range(reps):
+            xs, ys, os_, rs = ring[slot % RING]
+            slot += 1
+            if name == "copy":
+                W.lib.check(lib.wf2hip_scopy(N, p(ys), 1, p(os_), 1))
+            elif name == "add":
+                W.lib.check(lib.wf2hip_sadd(N, p(xs), 1, p(ys), 1))
+            elif name == "mul":
+                W.lib.check(lib.wf2hip_smul(N, p(xs), 1, p(ys), 1))
+            elif name == "exp":
+                W.lib.check(lib.wf2hip_sexp(N, p(ys), 1, p(os_), 1))
+            else:
+                W.lib.check(lib.wf2hip_reduce_add_rows_f32(SIDE, SIDE, p(ys), SIDE, p(rs), 1))
+    W.lib.synchronize()
+    print(json.dumps({"probe": "copy, add, mul, exp, rowsum", "launches_each": reps, "elements": N}))
+
+
 def block_forward_ms(W, reps: int = 5):
     try:
         gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
@@ -180,6 +208,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-block", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on ONE GPU (no collectives, no sharding); "
@@ -188,6 +218,9 @@ def main():
     W = importlib.import_module("cl-waffe2_amd")
     W.lib.init(0)  # raises if libwaffe2-hip.so is missing: there is no CPU fallback
     info = W.lib.device_info()
+    if args.probe:
+        counter_probe(W)
+        return
 
     step_ms, wall_ms, per_kernel, binary_ms = gpu_steps(W, args.steps, args.warmup)
     total_bytes = sum(BYTES.values())

@@ -7,8 +7,11 @@
 // tensor.lisp:146-210), tensor-finalizer (:323-329), vref (:719-746) and
 // convert-tensor-facet (source/array-converter.lisp:15-197) map onto
 // malloc/free/memcpy below.
+#include <map>
 #include <mutex>
+#include <stdlib.h>
 #include <string.h>
+#include <unordered_map>
 
 #include "wf2_common.h"
 
@@ -36,6 +39,82 @@ int check_hip(hipError_t e, const char* what) {
 int require_init() {
   if (!g_rt.initialised) return fail(WF2HIP_ENOTINIT, "wf2hip_init has not been called");
   return 0;
+}
+
+// ---- caching allocator -------------------------------------------------------
+// cl-waffe2 allocates a compiled model's temporaries once and reuses them on
+// every forward (maybe-allocate!, source/vm/allocation.lisp:121-145); a host
+// that allocates per call gets the same steady state from this pool.  Blocks
+// are recycled without synchronising: every kernel and copy of the library
+// runs on one stream, so a recycled block's new user is ordered after its old
+// one.  hipFree (which does synchronise) only happens on trim/shutdown or when
+// the device is out of memory.
+struct Pool {
+  std::mutex mu;
+  std::multimap<size_t, void*> idle;          // size class -> block
+  std::unordered_map<void*, size_t> size_of;  // every block handed out or idle
+  size_t idle_bytes = 0;
+  bool enabled = true;
+};
+static Pool g_pool;
+
+static size_t size_class(size_t bytes) {
+  const size_t small = 512, large = (size_t)2 << 20;
+  if (bytes < ((size_t)1 << 20)) return (bytes + small - 1) / small * small;
+  return (bytes + large - 1) / large * large;
+}
+
+static void pool_release_idle_locked() {
+  for (auto& kv : g_pool.idle) {
+    (void)hipFree(kv.second);
+    g_pool.size_of.erase(kv.second);
+  }
+  g_pool.idle.clear();
+  g_pool.idle_bytes = 0;
+}
+
+static int pool_alloc(void** ptr, size_t bytes) {
+  const size_t cls = size_class(bytes);
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  if (g_pool.enabled) {
+    auto it = g_pool.idle.find(cls);
+    if (it != g_pool.idle.end()) {
+      *ptr = it->second;
+      g_pool.idle.erase(it);
+      g_pool.idle_bytes -= cls;
+      return 0;
+    }
+  }
+  hipError_t e = hipMalloc(ptr, cls);
+  if (e == hipErrorOutOfMemory && !g_pool.idle.empty()) {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(g_rt.stream);
+    pool_release_idle_locked();
+    e = hipMalloc(ptr, cls);
+  }
+  if (e == hipErrorOutOfMemory) {
+    (void)hipGetLastError();
+    *ptr = nullptr;
+    return fail(WF2HIP_ENOMEM, "out of device memory allocating %zu bytes", bytes);
+  }
+  WF2_TRY(check_hip(e, "hipMalloc"));
+  g_pool.size_of[*ptr] = cls;
+  return 0;
+}
+
+static int pool_free(void* ptr) {
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  auto it = g_pool.size_of.find(ptr);
+  if (it == g_pool.size_of.end())
+    return fail(WF2HIP_EINVAL, "wf2hip_free: %p was not allocated by wf2hip_malloc", ptr);
+  if (g_pool.enabled) {
+    g_pool.idle.emplace(it->second, ptr);
+    g_pool.idle_bytes += it->second;
+    return 0;
+  }
+  g_pool.size_of.erase(it);
+  WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
+  return check_hip(hipFree(ptr), "hipFree");
 }
 
 __global__ void fill_kernel(float* __restrict__ x, size_t n, float v) {
@@ -78,6 +157,8 @@ WF2_API int wf2hip_init(int device) {
   snprintf(g_rt.arch, sizeof g_rt.arch, "%s", prop.gcnArchName);
   g_rt.stream = nullptr;
   g_rt.initialised = true;
+  const char* pool_env = getenv("WF2HIP_POOL");
+  g_pool.enabled = !(pool_env && pool_env[0] == '0');
   return 0;
 }
 
@@ -85,9 +166,26 @@ WF2_API int wf2hip_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mu);
   if (!g_rt.initialised) return 0;
   (void)hipStreamSynchronize(g_rt.stream);
+  {
+    std::lock_guard<std::mutex> pool_lock(g_pool.mu);
+    pool_release_idle_locked();
+  }
   if (g_rt.partials) (void)hipFree(g_rt.partials);
   g_rt = Runtime();
   return 0;
+}
+
+WF2_API int wf2hip_pool_trim(void) {
+  WF2_TRY(require_init());
+  WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  pool_release_idle_locked();
+  return 0;
+}
+
+WF2_API size_t wf2hip_pool_idle_bytes(void) {
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  return g_pool.idle_bytes;
 }
 
 WF2_API int wf2hip_device_info(char* buf, size_t buflen) {
@@ -97,39 +195,31 @@ WF2_API int wf2hip_device_info(char* buf, size_t buflen) {
   return 0;
 }
 
-WF2_API int wf2hip_malloc(void** ptr, size_t bytes) {
+WF2_API int wf2hip_malloc_uninitialized(void** ptr, size_t bytes) {
   WF2_TRY(require_init());
   if (!ptr) return fail(WF2HIP_EINVAL, "null result pointer");
   *ptr = nullptr;
   if (bytes == 0) return 0;
-  hipError_t e = hipMalloc(ptr, bytes);
-  if (e == hipErrorOutOfMemory) {
-    (void)hipGetLastError();
-    return fail(WF2HIP_ENOMEM, "out of device memory allocating %zu bytes", bytes);
-  }
-  WF2_TRY(check_hip(e, "hipMalloc"));
+  return pool_alloc(ptr, bytes);
+}
+
+WF2_API int wf2hip_malloc(void** ptr, size_t bytes) {
+  WF2_TRY(wf2hip_malloc_uninitialized(ptr, bytes));
+  if (bytes == 0) return 0;
   // Zero fill on the library's stream so it is ordered with the kernels that
-  // will use the buffer.
-  size_t words = bytes / 4;
-  if (words) {
-    int blocks = (int)(ceil_div((int64_t)words, kBlock * 8) < 16384
-                           ? ceil_div((int64_t)words, kBlock * 8)
-                           : 16384);
-    fill_kernel<<<blocks, kBlock, 0, g_rt.stream>>>((float*)*ptr, words, 0.0f);
-    WF2_TRY(after_launch("zero fill"));
-  }
-  if (bytes % 4)
-    WF2_TRY(check_hip(hipMemsetAsync((char*)*ptr + words * 4, 0, bytes % 4, g_rt.stream),
-                      "hipMemsetAsync"));
-  return 0;
+  // will use the buffer (a fill kernel rather than a memset node, so callers
+  // may capture it).  Blocks are multiples of 512 bytes: whole words.
+  const size_t words = (bytes + 3) / 4;
+  int64_t want = ceil_div((int64_t)words, kBlock * 8);
+  int blocks = (int)(want < 16384 ? want : 16384);
+  fill_kernel<<<blocks, kBlock, 0, g_rt.stream>>>((float*)*ptr, words, 0.0f);
+  return after_launch("zero fill");
 }
 
 WF2_API int wf2hip_free(void* ptr) {
   WF2_TRY(require_init());
   if (!ptr) return 0;
-  // Kernels still reading the buffer must finish first.
-  WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
-  return check_hip(hipFree(ptr), "hipFree");
+  return pool_free(ptr);
 }
 
 WF2_API int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
@@ -176,6 +266,8 @@ WF2_API int wf2hip_sync(void) {
 
 WF2_API int wf2hip_set_stream(void* hip_stream) {
   WF2_TRY(require_init());
+  // recycled blocks rely on single-stream ordering: drain the old stream first
+  WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
   g_rt.stream = (hipStream_t)hip_stream;
   return 0;
 }

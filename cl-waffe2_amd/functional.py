@@ -45,7 +45,7 @@ def move_(dst: HIPTensor, src: HIPTensor) -> HIPTensor:
 def copy(x: HIPTensor) -> HIPTensor:
     """``(!copy x)``: a fresh contiguous tensor of x's visible shape filled by
     MoveTensorNode (``fundamental.lisp:122-163``)."""
-    return move_(HIPTensor(x.shape), x)
+    return move_(HIPTensor(x.shape, initial_element=None), x)
 
 
 def to_contiguous(x: HIPTensor) -> HIPTensor:
@@ -188,7 +188,7 @@ def _out_of_place(node: str, x, y) -> HIPTensor:
     if x.shape == out_shape:
         left = copy(x)
     else:  # x is the smaller operand: expand it into a full-size tensor first
-        left = move_(HIPTensor(out_shape), flexible(x, _ShapeOnly(out_shape)))
+        left = move_(HIPTensor(out_shape, initial_element=None), flexible(x, _ShapeOnly(out_shape)))
     return nodes.forward(node, left, flexible(y, left))
 
 
@@ -221,7 +221,7 @@ def _math(node: str, x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     """``(!exp x :-> out)``: ``out`` defaults to a fresh tensor (the pruned
     ``(!copy x :maybe-in-place t)`` of ``base-impl/mathematics.lisp:13-120``)."""
     if out is None:
-        out = HIPTensor(x.shape)
+        out = HIPTensor(x.shape, initial_element=None)
     return nodes.forward(node, x, out)
 
 
@@ -237,7 +237,7 @@ def abs(x, out=None): return _math("AbsNode", x, out)  # noqa: A001 - mirrors !a
 def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:
     """``(!expt x n)`` (``mathematics.lisp:267-303``)."""
     if out is None:
-        out = HIPTensor(x.shape)
+        out = HIPTensor(x.shape, initial_element=None)
     return nodes.forward("ExptNode", x, out, float(n))
 
 
@@ -317,7 +317,7 @@ def matmul(a, b, out: HIPTensor | None = None) -> HIPTensor:
     bshape = b.shape if trans_b else bt.shape
     batch = ashape[:-2] if len(ashape) >= len(bshape) else bshape[:-2]
     if out is None:
-        out = HIPTensor(list(batch) + [ashape[-2], bshape[-1]])
+        out = HIPTensor(list(batch) + [ashape[-2], bshape[-1]], initial_element=None)
 
     def with_batch(x: HIPTensor) -> HIPTensor:
         if x.shape[:-2] == list(batch):
@@ -357,7 +357,7 @@ def softmax_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     import ctypes as C
     x = to_contiguous(x)
     if out is None:
-        out = HIPTensor(x.shape)
+        out = HIPTensor(x.shape, initial_element=None)
     cols = x.shape[-1]
     rows = x.size // max(cols, 1)
     _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols,
@@ -376,7 +376,7 @@ def gelu(x: HIPTensor) -> HIPTensor:
 def gelu_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     import ctypes as C
     if out is None:
-        out = HIPTensor(x.shape)
+        out = HIPTensor(x.shape, initial_element=None)
     v = nodes.view2(x, out)
     _lib.check(_lib.get().wf2hip_unary_nd(_lib.GELU, C.byref(v), C.c_void_p(x.ptr),
                                          C.c_void_p(out.ptr), 0.0))
@@ -398,7 +398,7 @@ def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e
     import ctypes as C
     x = to_contiguous(x)
     if out is None:
-        out = HIPTensor(x.shape)
+        out = HIPTensor(x.shape, initial_element=None)
     cols = x.shape[-1]
     rows = x.size // max(cols, 1)
     _lib.check(_lib.get().wf2hip_layernorm_rows_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),

@@ -92,10 +92,10 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         # (B, 1, H, T, hd) strided windows of the projection, no copy
         q, k, v = (five.view(True, True, i, True, True).permute(0, 2, 3, 1, 4) for i in range(3))
         scores = F.matmul(q, F.t(k))                                # (B, 1, H, T, T)
-        probs = HIPTensor(scores.shape)
+        probs = HIPTensor(scores.shape, initial_element=None)
         _lib.check(_lib.get().wf2hip_causal_softmax_f32(B * H, T, C.c_void_p(scores.ptr),
                                                        C.c_void_p(probs.ptr), scale))
-        ctx_store = HIPTensor([B, T, 1, H, hd])
+        ctx_store = HIPTensor([B, T, 1, H, hd], initial_element=None)
         F.matmul(probs, v, out=ctx_store.permute(0, 2, 3, 1, 4))    # written as (B, T, H*hd)
         ctx = F.reshape(ctx_store, B, T, D)
     else:

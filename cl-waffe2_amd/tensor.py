@@ -32,10 +32,11 @@ from .ranges import Range, compose, make_range
 class DeviceBuffer:
     """Zero-initialised device memory owned by one or more tensors."""
 
-    def __init__(self, nbytes: int):
+    def __init__(self, nbytes: int, zero: bool = True):
         self.nbytes = int(nbytes)
         p = C.c_void_p()
-        _lib.check(_lib.get().wf2hip_malloc(C.byref(p), self.nbytes))
+        alloc = _lib.get().wf2hip_malloc if zero else _lib.get().wf2hip_malloc_uninitialized
+        _lib.check(alloc(C.byref(p), self.nbytes))
         self.ptr = p.value or 0
 
     def __del__(self):  # tensor-finalizer
@@ -131,7 +132,7 @@ class HIPTensor:
 
     def __init__(self, shape: Sequence[int], *, vec: DeviceBuffer | None = None,
                  strides: Sequence[int] | None = None, views: Sequence[Subscript] | None = None,
-                 offset: int = 0, initial_element: float = 0.0):
+                 offset: int = 0, initial_element: float | None = 0.0):
         self.orig_shape = [int(s) for s in shape]
         if len(self.orig_shape) < 1 or len(self.orig_shape) > _lib.MAX_RANK:
             raise ValueError(f"HIPTensor rank must be 1..{_lib.MAX_RANK}")
@@ -143,8 +144,10 @@ class HIPTensor:
         self.initial_offset = int(offset)
         if vec is None:
             n = int(np.prod(self.orig_shape, dtype=np.int64))
-            vec = DeviceBuffer(4 * n)
-            if initial_element != 0.0 and n:
+            # initial_element None = an InputTensor temporary (make-input): its
+            # first use overwrites it, so it is not zero-filled
+            vec = DeviceBuffer(4 * n, zero=initial_element == 0.0)
+            if initial_element and n:
                 _lib.check(_lib.get().wf2hip_fill_f32(C.c_void_p(vec.ptr), n, float(initial_element)))
         self.vec = vec
 

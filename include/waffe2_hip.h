@@ -57,7 +57,18 @@ int wf2hip_device_info(char* buf, size_t buflen);
  * (backends/lisp/tensor.lisp:12-28; !sum zero-fills by multiplying by 0,
  * base-impl/reduction.lisp:63). */
 int wf2hip_malloc(void** ptr, size_t bytes);
+/* Same without the zero fill, for tensors whose first use overwrites them
+ * (cl-waffe2's InputTensor temporaries from make-input,
+ * source/vm/generic-tensor/tensor.lisp:613-717). */
+int wf2hip_malloc_uninitialized(void** ptr, size_t bytes);
+/* Returns the block to the library's pool: no synchronisation, the block is
+ * recycled in stream order (the steady state cl-waffe2 gets from allocating a
+ * compiled model's temporaries once, source/vm/allocation.lisp:121-145).
+ * WF2HIP_POOL=0 in the environment makes every free a hipFree. */
 int wf2hip_free(void* ptr);
+/* Give idle pooled blocks back to the device (synchronises). */
+int wf2hip_pool_trim(void);
+size_t wf2hip_pool_idle_bytes(void);
 int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes);
 int wf2hip_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int wf2hip_memcpy_d2d(void* dst, const void* src, size_t bytes);
