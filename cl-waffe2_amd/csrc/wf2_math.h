@@ -202,7 +202,8 @@ WF2_MATH_FN double trig_core(double xd, int32_t quadrant_shift) {
 
 WF2_MATH_FN float sinf_(float x) {
   if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_SINF(x);
-  return (float)trig_core((double)x, 0);
+  float r = (float)trig_core((double)x, 0);
+  return (x == 0.0f) ? x : r;  // sin(-0) = -0: the polynomial's sign of zero is not x's
 }
 
 WF2_MATH_FN float cosf_(float x) {

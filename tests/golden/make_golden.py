@@ -1,0 +1,94 @@
+#!/usr/bin/env python3
+"""Writes the golden vectors under tests/golden/ from the reference's own C
+kernels (cl-waffe2-simd/kernels/cl-waffe2-simd.c) compiled into
+oracle/_ref/libwaffe2_simd_ref.so by `make -C oracle ref`.
+
+Run in a container that has the reference checkout; the fixtures are data
+(inputs and the outputs the reference kernels produced), small enough to
+commit, and are what pins the oracle and the device math where the reference
+itself cannot travel.
+
+    python tests/golden/make_golden.py
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from oracle import oracle as O  # noqa: E402
+
+REGIMES = [(1, 1), (1, 0), (2, 1), (1, 3), (2, 2), (3, 0), (0, 1), (0, 0), (0, 2)]
+SIZES = [1, 7, 8, 9, 31, 64, 67]
+EDGE = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 1.0, -1.0, np.inf, -np.inf, np.nan, 88.72, 88.73,
+                 -87.4, -103.9, -104.5, 1e10, -1e10, 3.4e38, 1e6, 1.5e6, 9.01, -9.01, 0.5, 2.0,
+                 1e-3, 123456.7, 1e-20, 0.99999994, 1.0000001, 3.1415927, 1.5707964, 6.2831855,
+                 102.1, 355.0, 710.0, 1e5, 65536.0, 20.0, -20.0, 0.1], np.float32)
+UNARY = {"exp": (-10, 10), "tanh": (-10, 10), "sin": (-100, 100), "cos": (-100, 100),
+         "log": (1e-3, 1e3), "sqrt": (0, 1e3), "abs": (-5, 5)}
+
+
+def main():
+    assert O.ref() is not None, "oracle/_ref/libwaffe2_simd_ref.so is missing: run `make -C oracle ref`"
+    rng = np.random.Generator(np.random.PCG64(2024))
+    out = {}
+    # x <- x op y for every (incx, incy) regime incl. incx == 0 accumulation
+    for op in ("add", "sub", "mul", "div"):
+        for n in SIZES:
+            for incx, incy in REGIMES:
+                size = max(1, n) * 3 + 1
+                x = rng.standard_normal(size).astype(np.float32)
+                y = (rng.standard_normal(size) + (1.5 if op in ("mul", "div") and incx == 0 else 0)).astype(np.float32)
+                if op in ("mul", "div") and incx == 0:
+                    y = rng.uniform(0.9, 1.1, size).astype(np.float32)
+                res = x.copy()
+                O.binary_1d(op, n, res, incx, y, incy, use_ref=True)
+                key = f"bin_{op}_{n}_{incx}_{incy}"
+                out[key + "_x"], out[key + "_y"], out[key + "_out"] = x, y, res
+    # out <- f(x): BASELINE ranges (n = 2048 + 5 so that the libm tail is hit),
+    # edge values, strided in/out, broadcast source
+    for op, (lo, hi) in UNARY.items():
+        x = rng.uniform(lo, hi, 2053).astype(np.float32)
+        res = np.zeros_like(x)
+        O.unary_1d(op, x.size, x, 1, res, 1, use_ref=True)
+        out[f"un_{op}_range_x"], out[f"un_{op}_range_out"] = x, res
+        res = np.zeros(EDGE.size, np.float32)
+        with np.errstate(all="ignore"):
+            O.unary_1d(op, EDGE.size, EDGE, 1, res, 1, use_ref=True)
+        out[f"un_{op}_edge_out"] = res
+        for n, incx, inco in [(13, 2, 1), (16, 1, 3), (9, 0, 1)]:
+            res = np.full(64, 7.0, np.float32)
+            O.unary_1d(op, n, x, incx, res, inco, use_ref=True)
+            out[f"un_{op}_{n}_{incx}_{inco}_out"] = res
+    out["edge_x"] = EDGE
+    for p in (2.0, 3.0, 0.5, 2.5, -1.0):
+        x = rng.uniform(0.01, 30.0, 1029).astype(np.float32)
+        if p == int(p):
+            x[::2] *= -1
+        res = np.zeros_like(x)
+        O.pow_1d(x.size, x, 1, p, res, 1, use_ref=True)
+        out[f"pow_{p}_x"], out[f"pow_{p}_out"] = x, res
+    for n, inc in [(1, 1), (5, 1), (8, 1), (67, 1), (40, 3)]:
+        x = rng.standard_normal(n * inc + 1).astype(np.float32)
+        out[f"max_{n}_{inc}_x"] = x
+        out[f"max_{n}_{inc}_out"] = np.float32(O.maxmin_1d("max", n, x, inc, use_ref=True))
+        out[f"min_{n}_{inc}_out"] = np.float32(O.maxmin_1d("min", n, x, inc, use_ref=True))
+    np.savez_compressed(os.path.join(HERE, "simd_kernels.npz"), **out)
+    manifest = {
+        "source": "cl-waffe2-simd/kernels/cl-waffe2-simd.c compiled by oracle/Makefile target `ref`",
+        "compiler": "ROCm clang -O3 -mavx2 -mfma -flax-vector-conversions=all",
+        "sleef": "3.8.0 symbols exported by PyTorch's libtorch_cpu.so (Sleef_*f8_u10avx2, sqrt u05)",
+        "seed": "PCG64(2024)",
+        "arrays": len(out),
+        "regimes": REGIMES,
+        "sizes": SIZES,
+    }
+    with open(os.path.join(HERE, "simd_kernels.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "simd_kernels.npz")), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -55,3 +55,18 @@ def oracle_views(O, tensors):
         descs.append(dict(stride=list(t.stride), kind=kind, first=first, step=step,
                           offset=t.initial_offset))
     return O.make_views(shape, descs)
+
+
+class NoBuffer:
+    """Stands in for device storage so that view geometry can be exercised on a
+    machine without a GPU."""
+
+    def __init__(self, nbytes):
+        self.ptr = 0
+        self.nbytes = int(nbytes)
+
+
+def host_tensor(W, shape):
+    """A HIPTensor whose storage is never touched (geometry only)."""
+    n = int(np.prod(shape, dtype=np.int64))
+    return W.HIPTensor(shape, vec=NoBuffer(4 * n))

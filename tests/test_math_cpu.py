@@ -1,0 +1,100 @@
+"""The device math cores (cl-waffe2_amd/csrc/wf2_math.h) compiled for the host:
+accuracy against float64 over strided sweeps of ALL binary32 inputs, agreement
+with the oracle's SLEEF u10 results within 2 ulp on the benchmark ranges, and
+with the golden vectors of the reference's compiled kernels.
+
+The header uses only IEEE operations and fma, so the host build computes what
+the GPU computes (up to the reciprocal seed, refined to ~2^-50 either way)."""
+import ctypes as C
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+from helpers import ulp_distance
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+OPS = {"sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21, "abs": 22, "gelu": 40}
+
+
+@pytest.fixture(scope="module")
+def M():
+    so = os.path.join(HERE, "native", "libwf2_math_cpu.so")
+    src = os.path.join(HERE, "native", "math_cpu.cpp")
+    hdr = os.path.join(HERE, "..", "cl-waffe2_amd", "csrc", "wf2_math.h")
+    if not os.path.exists(so) or os.path.getmtime(so) < max(os.path.getmtime(src), os.path.getmtime(hdr)):
+        subprocess.check_call(["make", "-C", os.path.join(HERE, "native"), "-B"], stdout=subprocess.DEVNULL)
+    L = C.CDLL(so)
+    L.wf2cpu_unary.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_void_p]
+    L.wf2cpu_pow.argtypes = [C.c_long, C.c_void_p, C.c_float, C.c_void_p]
+    L.wf2cpu_scan.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_double),
+                              C.POINTER(C.c_uint32)]
+    return L
+
+
+def apply(M, op, x):
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty_like(x)
+    M.wf2cpu_unary(OPS[op], x.size, x.ctypes.data, out.ctypes.data)
+    return out
+
+
+def fbits(v):
+    return struct.unpack("I", struct.pack("f", v))[0]
+
+
+@pytest.mark.parametrize("op", ["exp", "tanh", "log", "sqrt", "gelu", "sin", "cos"])
+def test_sweep_of_all_binary32_inputs(M, op):
+    """Every 997th bit pattern of the whole binary32 line (positive and
+    negative): error <= 0.5003 ulp, i.e. correctly rounded except for
+    near-ties.  (A stride-1 sweep gives the same maxima.)"""
+    spans = [(0, 0x7F800000)] if op in ("log", "sqrt") else [(0, 0x7F800000), (0x80000000, 0xFF800000)]
+    for lo, hi in spans:
+        if op in ("sin", "cos"):  # beyond 1e6 the slow path is the platform's own routine
+            hi = lo + fbits(1.0e6)
+        m, w = C.c_double(), C.c_uint32()
+        M.wf2cpu_scan(OPS[op], lo, hi, 997, C.byref(m), C.byref(w))
+        assert m.value <= 0.5003, (op, m.value, struct.unpack("f", struct.pack("I", w.value))[0])
+
+
+@pytest.mark.parametrize("op,lo,hi", [("exp", -10, 10), ("tanh", -10, 10), ("sin", -100, 100),
+                                      ("log", 1e-3, 1e3), ("cos", -100, 100)])
+def test_within_two_ulp_of_sleef(M, O, op, lo, hi):
+    if not O.sleef_available():
+        pytest.skip("no SLEEF provider")
+    rng = np.random.Generator(np.random.PCG64(3))
+    x = rng.uniform(lo, hi, 1 << 21).astype(np.float32)
+    want = np.zeros_like(x)
+    O.unary_1d(op, x.size, x, 1, want, 1)
+    assert ulp_distance(apply(M, op, x), want).max() <= 2
+
+
+def test_against_golden_vectors(M):
+    gold = np.load(os.path.join(HERE, "golden", "simd_kernels.npz"))
+    for op in ("exp", "tanh", "sin", "cos", "log", "sqrt", "abs"):
+        limit = 0 if op in ("sqrt", "abs") else 2
+        got = apply(M, op, gold[f"un_{op}_range_x"])
+        assert ulp_distance(got, gold[f"un_{op}_range_out"]).max() <= limit, op
+        got = apply(M, op, gold["edge_x"])
+        assert ulp_distance(got, gold[f"un_{op}_edge_out"]).max() <= limit, op
+    for p in (2.0, 3.0, 0.5, 2.5, -1.0):
+        x = gold[f"pow_{p}_x"]
+        out = np.empty_like(x)
+        M.wf2cpu_pow(x.size, x.ctypes.data, p, out.ctypes.data)
+        assert ulp_distance(out, gold[f"pow_{p}_out"]).max() <= 2, p
+
+
+def test_special_values(M):
+    f = lambda op, v: apply(M, op, np.array([v], np.float32))[0]  # noqa: E731
+    assert f("exp", 0.0) == 1.0 and f("exp", -np.inf) == 0.0 and f("exp", np.inf) == np.inf
+    assert f("exp", 88.8) == np.inf and f("exp", -104.0) == 0.0 and np.isnan(f("exp", np.nan))
+    assert f("log", 1.0) == 0.0 and f("log", 0.0) == -np.inf and np.isnan(f("log", -1.0))
+    assert f("log", np.inf) == np.inf and f("log", 1e-45) == np.float32(np.log(np.float64(np.float32(1e-45))))
+    assert f("tanh", np.inf) == 1.0 and f("tanh", -np.inf) == -1.0 and f("tanh", 0.0) == 0.0
+    assert np.signbit(f("tanh", -0.0)) and np.signbit(f("sin", -0.0))
+    assert f("sin", 0.0) == 0.0 and f("cos", 0.0) == 1.0 and np.isnan(f("sin", np.inf))
+    assert f("sqrt", 4.0) == 2.0 and np.isnan(f("sqrt", -1.0))
+    assert abs(f("gelu", 1.0) - 0.841192) < 5e-7   # vm/nodes/t/composite.lisp:119
+    assert f("gelu", 0.0) == 0.0 and f("gelu", -30.0) == 0.0 and f("gelu", 30.0) == 30.0

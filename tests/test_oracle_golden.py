@@ -1,0 +1,197 @@
+"""Pins the CPU oracle (oracle/waffe2_oracle.c) before anything trusts it:
+
+* golden vectors produced by the reference's own compiled C kernels
+  (tests/golden/simd_kernels.npz, written by tests/golden/make_golden.py);
+* the compiled reference itself (oracle/_ref) on fresh random inputs where it
+  is present;
+* what the mathematics fixes: IEEE binary32 closed forms (numpy), float64
+  truth within 1 ulp for the SLEEF u10 functions, exact special values;
+* the reference's own test vectors (10 op 1 -> 11/9/10/10,
+  base-impl/t/arithmetic.lisp:26-51; gemm vectors :120,135,142,148).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from helpers import assert_bit_equal, ulp_distance
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "simd_kernels.npz")
+REGIMES = [(1, 1), (1, 0), (2, 1), (1, 3), (2, 2), (3, 0), (0, 1), (0, 0), (0, 2)]
+SIZES = [1, 7, 8, 9, 31, 64, 67]
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLD)
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_binary_golden(O, gold, op):
+    for n in SIZES:
+        for incx, incy in REGIMES:
+            key = f"bin_{op}_{n}_{incx}_{incy}"
+            x = gold[key + "_x"].copy()
+            O.binary_1d(op, n, x, incx, gold[key + "_y"].copy(), incy)
+            assert_bit_equal(x, gold[key + "_out"], key)
+
+
+@pytest.mark.parametrize("op,f", [("add", np.add), ("sub", np.subtract), ("mul", np.multiply),
+                                  ("div", np.divide)])
+def test_binary_closed_form(O, op, f):
+    """IEEE binary32: one correctly rounded operation per element (numpy)."""
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(1001).astype(np.float32)
+    y = rng.standard_normal(1001).astype(np.float32)
+    got = x.copy()
+    O.binary_1d(op, 1001, got, 1, y, 1)
+    assert_bit_equal(got, f(x, y), op)
+    got = x.copy()
+    O.binary_1d(op, 500, got, 2, y, 0)  # strided x, scalar y
+    want = x.copy()
+    want[:1000:2] = f(x[:1000:2], y[0])
+    assert_bit_equal(got, want, op + " strided/broadcast")
+    # incx == 0: strictly sequential accumulation into x[0]
+    got = x.copy()
+    O.binary_1d(op, 100, got, 0, y, 1)
+    acc = x[0]
+    for i in range(100):
+        acc = f(acc, y[i])
+    assert got[0] == acc and np.array_equal(got[1:], x[1:])
+
+
+def test_reference_tester_vectors(O):
+    """add/sub/mul/div-tester: (100,100) of 10 op (100,100) of 1 -> 11/9/10/10;
+    scalar testers likewise (base-impl/t/arithmetic.lisp:26-79)."""
+    for op, want in [("add", 11.0), ("sub", 9.0), ("mul", 10.0), ("div", 10.0)]:
+        x = np.full(10000, 10.0, np.float32)
+        O.binary_1d(op, 10000, x, 1, np.ones(10000, np.float32), 1)
+        assert np.all(x == want)
+        x = np.full(10000, 10.0, np.float32)
+        O.binary_1d(op, 10000, x, 1, np.ones(1, np.float32), 0)
+        assert np.all(x == want)
+
+
+@pytest.mark.skipif(not os.path.exists(os.path.join(os.path.dirname(__file__), "..", "oracle", "_ref",
+                                                    "libwaffe2_simd_ref.so")),
+                    reason="oracle/_ref not built (needs the reference checkout)")
+def test_oracle_equals_compiled_reference(O):
+    if O.ref() is None:
+        pytest.skip("oracle/_ref does not load here")
+    rng = np.random.default_rng(7)
+    for op in ("add", "sub", "mul", "div"):
+        for n in (5, 8, 100, 1003):
+            for incx, incy in REGIMES:
+                x = rng.standard_normal(3100).astype(np.float32)
+                y = rng.uniform(0.5, 1.5, 3100).astype(np.float32)
+                a, b = x.copy(), x.copy()
+                O.binary_1d(op, n, a, incx, y, incy)
+                O.binary_1d(op, n, b, incx, y, incy, use_ref=True)
+                assert_bit_equal(a, b, f"{op} {n} {incx} {incy}")
+    for op, lo, hi in [("exp", -10, 10), ("tanh", -10, 10), ("sin", -100, 100), ("log", 1e-3, 1e3),
+                       ("sqrt", 0, 100), ("cos", -100, 100), ("abs", -1, 1)]:
+        for n, incx, inco in [(1003, 1, 1), (500, 2, 1), (500, 1, 2), (77, 0, 1)]:
+            x = rng.uniform(lo, hi, 1100).astype(np.float32)
+            a = np.zeros(1100, np.float32)
+            b = np.zeros(1100, np.float32)
+            O.unary_1d(op, n, x, incx, a, inco)
+            O.unary_1d(op, n, x, incx, b, inco, use_ref=True)
+            assert_bit_equal(a, b, f"{op} {n} {incx} {inco}")
+
+
+UNARY = ["exp", "tanh", "sin", "cos", "log", "sqrt", "abs"]
+
+
+@pytest.mark.parametrize("op", UNARY)
+def test_unary_golden(O, gold, op):
+    if not O.sleef_available():
+        pytest.skip("no SLEEF provider: the oracle runs on libm and is only within 1 ulp of the goldens")
+    x = gold[f"un_{op}_range_x"]
+    got = np.zeros_like(x)
+    O.unary_1d(op, x.size, x, 1, got, 1)
+    assert_bit_equal(got, gold[f"un_{op}_range_out"], op)
+    got = np.zeros(gold["edge_x"].size, np.float32)
+    with np.errstate(all="ignore"):
+        O.unary_1d(op, got.size, gold["edge_x"], 1, got, 1)
+    assert_bit_equal(got, gold[f"un_{op}_edge_out"], op + " edge")
+    for n, incx, inco in [(13, 2, 1), (16, 1, 3), (9, 0, 1)]:
+        got = np.full(64, 7.0, np.float32)
+        O.unary_1d(op, n, x, incx, got, inco)
+        assert_bit_equal(got, gold[f"un_{op}_{n}_{incx}_{inco}_out"], f"{op} {n} {incx} {inco}")
+
+
+@pytest.mark.parametrize("op", UNARY)
+def test_unary_against_float64_truth(O, gold, op):
+    """SLEEF u10 promises <= 1.0 ulp (sqrt u05: correctly rounded); the goldens
+    and the oracle must honour it against numpy float64."""
+    x = gold[f"un_{op}_range_x"]
+    truth = getattr(np, "abs" if op == "abs" else op)(x.astype(np.float64)).astype(np.float32)
+    limit = 0 if op in ("sqrt", "abs") else 1
+    assert ulp_distance(gold[f"un_{op}_range_out"], truth).max() <= limit
+    got = np.zeros_like(x)
+    O.unary_1d(op, x.size, x, 1, got, 1)
+    assert ulp_distance(got, truth).max() <= limit
+
+
+def test_unary_special_values(O):
+    def f(op, v):
+        out = np.zeros(1, np.float32)
+        with np.errstate(all="ignore"):
+            O.unary_1d(op, 1, np.array([v], np.float32), 1, out, 1)
+        return out[0]
+    assert f("exp", 0.0) == 1.0 and f("log", 1.0) == 0.0 and f("sin", 0.0) == 0.0
+    assert f("tanh", np.inf) == 1.0 and f("tanh", -np.inf) == -1.0 and f("cos", 0.0) == 1.0
+    assert f("log", 0.0) == -np.inf and np.isnan(f("log", -1.0)) and f("exp", -np.inf) == 0.0
+    assert f("sqrt", 4.0) == 2.0 and f("abs", -3.5) == 3.5
+
+
+def test_pow_and_maxmin_golden(O, gold):
+    for p in (2.0, 3.0, 0.5, 2.5, -1.0):
+        x = gold[f"pow_{p}_x"]
+        got = np.zeros_like(x)
+        O.pow_1d(x.size, x, 1, p, got, 1)
+        if O.sleef_available():
+            assert_bit_equal(got, gold[f"pow_{p}_out"], f"pow {p}")
+        with np.errstate(all="ignore"):
+            truth = np.power(x.astype(np.float64), p).astype(np.float32)
+        assert ulp_distance(gold[f"pow_{p}_out"], truth).max() <= 1
+    for n, inc in [(1, 1), (5, 1), (8, 1), (67, 1), (40, 3)]:
+        x = gold[f"max_{n}_{inc}_x"]
+        assert O.maxmin_1d("max", n, x, inc) == gold[f"max_{n}_{inc}_out"] == x[::inc][:n].max()
+        assert O.maxmin_1d("min", n, x, inc) == gold[f"min_{n}_{inc}_out"] == x[::inc][:n].min()
+
+
+def test_copy(O):
+    y = np.arange(40, dtype=np.float32)
+    x = np.zeros(40, np.float32)
+    O.copy_1d(10, y, 3, x, 2)
+    assert x[:20:2].tolist() == y[:30:3].tolist() and np.all(x[1::2] == 0)
+
+
+def test_gemm_reference_vectors(O):
+    """matmul-tester vectors (base-impl/t/arithmetic.lisp:120,135,142,148) and
+    the column == row-major equivalence (backends/cpu/t/arithmetic.lisp:53-68)."""
+    a33 = np.arange(9, dtype=np.float32).reshape(3, 3)
+    a34 = np.arange(12, dtype=np.float32).reshape(3, 4)
+    assert O.matmul_rowmajor(a33, a33).ravel().tolist() == [15, 18, 21, 42, 54, 66, 69, 90, 111]
+    assert O.matmul_rowmajor(a34, a34, trans_b=True).ravel().tolist() == [14, 38, 62, 38, 126, 214, 62, 214, 366]
+    assert O.matmul_rowmajor(a34, a34, trans_a=True).ravel().tolist() == [
+        80, 92, 104, 116, 92, 107, 122, 137, 104, 122, 140, 158, 116, 137, 158, 179]
+    assert O.matmul_rowmajor(a33, a33, trans_a=True, trans_b=True).ravel().tolist() == [
+        15, 42, 69, 18, 54, 90, 21, 66, 111]
+
+
+def test_gemm_against_float64(O):
+    rng = np.random.default_rng(3)
+    for ta in ("N", "T"):
+        for tb in ("N", "T"):
+            m, n, k = 13, 9, 21
+            A = rng.standard_normal((k, m) if ta == "N" else (m, k)).astype(np.float32)  # column-major storage
+            B = rng.standard_normal((n, k) if tb == "N" else (k, n)).astype(np.float32)
+            Cm = rng.standard_normal((n, m)).astype(np.float32)
+            opA = A.T if ta == "N" else A          # (m, k)
+            opB = B.T if tb == "N" else B          # (k, n)
+            want = 0.5 * (opA.astype(np.float64) @ opB.astype(np.float64)) + 2.0 * Cm.T.astype(np.float64)
+            got = Cm.copy().ravel()
+            O.sgemm(ta, tb, m, n, k, 0.5, A.ravel(), A.shape[1], B.ravel(), B.shape[1], 2.0, got, m)
+            np.testing.assert_allclose(got.reshape(n, m).T, want, rtol=1e-5, atol=1e-5)
