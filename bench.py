@@ -44,6 +44,11 @@ HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BYTES = {"add": 12 * N, "mul": 12 * N, "exp": 8 * N, "rowsum": 4 * N + 4 * SIDE}
 RING = 8  # buffer sets: 8 x (x, y, o) x 256 MiB = 6 GiB
+# HBM bytes per launch of the in-place binary kernel at 2^26 elements, from two
+# `rocprofv3 --pmc` runs of `bench.py --probe` (FETCH_SIZE 262173.8 KiB, WRITE_SIZE
+# 262144.3 KiB per dispatch), each scaled by what the same counter reads for the plain
+# copy of 2^26 floats in the same run (x1.9996 and x0.9996); summary under profiles/.
+BINARY_TRAFFIC_BYTES = 805_150_000
 
 
 def p(t):
@@ -84,35 +89,34 @@ def gpu_steps(W, steps: int, warmup: int):
             slot += 1
     W.lib.synchronize()
 
-    # timed region: K steps; events between the kernels attribute time per kernel
-    marks = [[W.lib.Event() for _ in range(len(order) + 1)] for _ in range(steps)]
+    # timed region: exactly K steps, launched back to back, bracketed by a
+    # synchronisation and one HIP event on the library's stream at each end
     W.lib.synchronize()
+    e0, e1 = W.lib.Event(), W.lib.Event()
     t0 = time.perf_counter()
+    e0.record()
     for s in range(steps):
-        marks[s][0].record()
-        for k, name in enumerate(order):
+        for name in order:
             launch(name, slot)
             slot += 1
-            marks[s][k + 1].record()
+    e1.record()
     W.lib.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    per_kernel = {name: 0.0 for name in order}
-    step_ms = 0.0
-    for s in range(steps):
-        for k, name in enumerate(order):
-            per_kernel[name] += marks[s][k].elapsed_ms(marks[s][k + 1])
-        step_ms += marks[s][0].elapsed_ms(marks[s][-1])
-    per_kernel = {k: v / steps for k, v in per_kernel.items()}
-    # the binary kernel alone, back to back, for the roofline entry
+    step_ms = e0.elapsed_ms(e1) / steps
+
+    # per-kernel average launch duration: each kernel alone, back to back on the
+    # ring (cold operands), event pair around the run
     reps = max(steps, 20)
-    e0, e1 = W.lib.Event(), W.lib.Event()
-    e0.record()
-    for _ in range(reps):
-        launch("add", slot)
-        slot += 1
-    e1.record()
-    binary_ms = e0.elapsed_ms(e1) / reps
-    return step_ms / steps, wall_ms / steps, per_kernel, binary_ms
+    per_kernel = {}
+    for name in order:
+        a, b = W.lib.Event(), W.lib.Event()
+        a.record()
+        for _ in range(reps):
+            launch(name, slot)
+            slot += 1
+        b.record()
+        per_kernel[name] = a.elapsed_ms(b) / reps
+    return step_ms, wall_ms / steps, per_kernel, per_kernel["add"]
 
 
 def counter_probe(W, reps: int = 5):
@@ -260,7 +264,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": BINARY_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": BYTES["add"],
             "avg_launch_ms": round(binary_ms, 5),
         },

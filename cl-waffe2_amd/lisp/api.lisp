@@ -1,0 +1,77 @@
+(in-package :cl-waffe2/backends.hip)
+
+;; CFFI bindings of include/waffe2_hip.h.  Counterpart of cl-waffe2-simd/api.lisp: where that
+;; file declares `(defcfun "waffe2_sadd" :void (n :long) (x (:pointer :float)) (incx :long) ...)`
+;; (api.lisp:63-82), the device library returns an int status that `check` turns into a Lisp
+;; error, so that the VM's handler reports the failing instruction (source/vm/vm.lisp:230-256).
+
+(define-condition hip-error (error)
+  ((code :initarg :code :reader hip-error-code)
+   (message :initarg :message :reader hip-error-message))
+  (:report (lambda (c s)
+             (format s "libwaffe2-hip: error ~a: ~a" (hip-error-code c) (hip-error-message c)))))
+
+(defmacro check (form)
+  "Evaluates a wf2hip_* call and signals HIP-ERROR unless it returned 0."
+  (let ((code (gensym "CODE")))
+    `(let ((,code ,form))
+       (unless (zerop ,code)
+         (error 'hip-error :code ,code :message (wf2hip-last-error)))
+       ,code)))
+
+(defun ensure-extension ()
+  (unless *hip-extension-p*
+    (error "HIPTensor: libwaffe2-hip.so is not loaded; there is no CPU fallback for device tensors.")))
+
+(defcfun "wf2hip_last_error" :string)
+(defcfun "wf2hip_malloc" :int (ptr :pointer) (bytes :size))
+(defcfun "wf2hip_malloc_uninitialized" :int (ptr :pointer) (bytes :size))
+(defcfun "wf2hip_free" :int (ptr :pointer))
+(defcfun "wf2hip_memcpy_h2d" :int (dst :pointer) (src :pointer) (bytes :size))
+(defcfun "wf2hip_memcpy_d2h" :int (dst :pointer) (src :pointer) (bytes :size))
+(defcfun "wf2hip_memcpy_d2d" :int (dst :pointer) (src :pointer) (bytes :size))
+(defcfun "wf2hip_fill_f32" :int (x :pointer) (n :size) (value :float))
+(defcfun "wf2hip_sync" :int)
+(defcfun "wf2hip_device_info" :int (buf :pointer) (len :size))
+(defcfun "wf2hip_set_reduce_mode" :int (mode :int))
+(defcfun "wf2hip_get_reduce_mode" :int)
+
+;; struct wf2hip_view2
+(defcstruct view2
+  (rank :int32)
+  (reserved :int32)
+  (shape :int64 :count 8)
+  (stride-a :int64 :count 8)
+  (stride-b :int64 :count 8)
+  (off-a :int64)
+  (off-b :int64))
+
+(defcfun "wf2hip_binary_nd" :int (op :int) (view (:pointer (:struct view2))) (a :pointer) (b :pointer))
+(defcfun "wf2hip_unary_nd" :int (op :int) (view (:pointer (:struct view2))) (a :pointer) (b :pointer) (p :float))
+(defcfun "wf2hip_sgemm_strided_batched" :int
+  (transa :char) (transb :char) (m :long) (n :long) (k :long) (alpha :float)
+  (a :pointer) (lda :long) (stride-a :long)
+  (b :pointer) (ldb :long) (stride-b :long)
+  (beta :float) (c :pointer) (ldc :long) (stride-c :long) (batch :long))
+(defcfun "wf2hip_softmax_rows_f32" :int (rows :long) (cols :long) (x :pointer) (ldx :long) (out :pointer) (ldo :long))
+(defcfun "wf2hip_layernorm_rows_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (b :pointer) (eps :float) (out :pointer))
+
+;; enum wf2hip_binary_op / wf2hip_unary_op
+(defconstant +add+ 0) (defconstant +sub+ 1) (defconstant +mul+ 2) (defconstant +div+ 3) (defconstant +move+ 4)
+(defconstant +sin+ 16) (defconstant +cos+ 17) (defconstant +tanh+ 18) (defconstant +log+ 19)
+(defconstant +exp+ 20) (defconstant +sqrt+ 21) (defconstant +abs+ 22) (defconstant +pow+ 32)
+
+(defun hip-synchronize ()
+  "Blocks until every kernel enqueued so far has finished (needed around wall-clock timing such
+as proceed-bench, source/base-impl/fundamental.lisp:706-777)."
+  (ensure-extension)
+  (check (wf2hip-sync)))
+
+(defmacro with-sequential-reductions (&body body)
+  "Runs BODY with AddNode-into-broadcast accumulations in the CPU backend's strictly sequential
+fp32 order (bit parity with CPUTensor; slow)."
+  (let ((old (gensym "OLD")))
+    `(let ((,old (wf2hip-get-reduce-mode)))
+       (check (wf2hip-set-reduce-mode 1))
+       (unwind-protect (progn ,@body)
+         (wf2hip-set-reduce-mode ,old)))))

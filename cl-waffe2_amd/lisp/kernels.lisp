@@ -1,0 +1,156 @@
+(in-package :cl-waffe2/backends.hip)
+
+;; define-impl-op registrations: closures that read the tensors' views at run time and make
+;; ONE library call per node.  The CPU backend instead generates loops with call-with-view at
+;; graph-construction time and compiles them per shape
+;; (source/backends/cpu/arithmetic.lisp:32-144); ExptNode-CPUTensor already uses the run-time
+;; form (source/backends/cpu/mathematics.lisp:55-76), which is the one followed here.
+
+(defun only-float-p (dtype &rest more)
+  "reject-p: everything but :float falls through to the next device in *using-backend*
+(cf. supported-dtypes-are, source/vm/nodes/utils.lisp:71-93)."
+  (declare (ignore more))
+  (not (eql dtype :float)))
+
+(defun fill-view2 (view a b)
+  "Writes the iteration space shared by tensors A and B into the foreign struct VIEW: per axis
+the visible extent and each tensor's effective stride (storage stride x view step, 0 when the
+axis is (:broadcast n)), plus the start offsets (tensor-initial-offset + stride x range-nth 0).
+These are exactly the numbers call-with-view computes per axis
+(source/vm/generic-tensor/call-with-view.lisp:120-137,168-195)."
+  (let ((rank (length (shape a))))
+    (assert (<= 1 rank 8) () "HIPTensor kernels take rank 1..8 tensors, got ~a" rank)
+    (setf (foreign-slot-value view '(:struct view2) 'rank) rank)
+    (flet ((geometry (tensor stride-slot)
+             (let ((offset (tensor-initial-offset tensor)))
+               (loop for axis from 0
+                     for extent in (shape tensor)
+                     for stride in (tensor-stride tensor)
+                     for subscript in (tensor-view tensor)
+                     for range = (subscript-range subscript)
+                     for first = (wf/iter:range-nth range 0)
+                     do (setf (mem-aref (foreign-slot-pointer view '(:struct view2) 'shape) :int64 axis)
+                              (cl-waffe2/vm:maybe-observe-axis extent))
+                        (incf offset (* stride first))
+                        (setf (mem-aref (foreign-slot-pointer view '(:struct view2) stride-slot) :int64 axis)
+                              (if (subscript-broadcast subscript)
+                                  0
+                                  (* stride (- (wf/iter:range-nth range 1) first)))))
+               offset)))
+      (setf (foreign-slot-value view '(:struct view2) 'off-a) (geometry a 'stride-a)
+            (foreign-slot-value view '(:struct view2) 'off-b) (geometry b 'stride-b)))
+    view))
+
+(defun run-binary (op x y)
+  (ensure-extension)
+  (with-foreign-object (view '(:struct view2))
+    (fill-view2 view x y)
+    (check (wf2hip-binary-nd op view (tensor-device-pointer x) (tensor-device-pointer y))))
+  x)
+
+(defun run-unary (op x out &optional (p 0.0))
+  (ensure-extension)
+  (with-foreign-object (view '(:struct view2))
+    (fill-view2 view x out)
+    (check (wf2hip-unary-nd op view (tensor-device-pointer x) (tensor-device-pointer out)
+                            (coerce p 'single-float))))
+  out)
+
+;; X <- X op Y, returns X (:where A[~] B[~] -> A[~], source/base-impl/arithmetic.lisp:57-103).
+;; A stride-0 destination axis -- how !sum and !mean arrive (base-impl/reduction.lisp:5-79) --
+;; is reduced in parallel by the library.
+(macrolet ((define-arith (node op)
+             `(define-impl-op (,node :device HIPTensor :reject-p #'only-float-p)
+                              :forward ((self x y) (declare (ignore self)) (run-binary ,op x y)))))
+  (define-arith AddNode +add+)
+  (define-arith SubNode +sub+)
+  (define-arith MulNode +mul+)
+  (define-arith DivNode +div+))
+
+;; X <- Y (source/base-impl/fundamental.lisp:9-43).  Without this impl every !copy on a device
+;; tensor would fall through to CPUTensor's scopy on a device handle.
+(define-impl-op (MoveTensorNode :device HIPTensor :reject-p #'only-float-p)
+                :forward ((self x y)
+                          (if (cl-waffe2/base-impl::movetensor-ignore-me self)
+                              y
+                              (run-binary +move+ x y))))
+
+;; OUT <- f(X) (:where X[~] OUT[~] -> OUT[~], source/base-impl/mathematics.lisp:13-120)
+(macrolet ((define-math (node op)
+             `(define-impl-op (,node :device HIPTensor :reject-p #'only-float-p)
+                              :forward ((self x out) (declare (ignore self)) (run-unary ,op x out)))))
+  (define-math SinNode +sin+)
+  (define-math CosNode +cos+)
+  (define-math TanhNode +tanh+)
+  (define-math LogENode +log+)
+  (define-math ExpNode +exp+)
+  (define-math SqrtNode +sqrt+)
+  (define-math AbsNode +abs+))
+
+;; OUT <- X^N with N a host ScalarTensor (source/base-impl/mathematics.lisp:267-303)
+(define-impl-op (ExptNode :device HIPTensor :reject-p #'only-float-p)
+                :forward ((self x out n)
+                          (declare (ignore self))
+                          (run-unary +pow+ x out (tensor-vec n))))
+
+;; C[~ i k] = A[~ i j] . B[~ j k].  Same operand swap as expand-gemm-form-column
+;; (source/backends/cpu/matrix-ops.lisp:12-112): a row-major product is the column-major
+;; sgemm(transB, transA, n, m, k, 1, B, ldb, A, lda, 0, C, ldc).  Batch axes are walked on the
+;; host exactly like call-with-view :at-least-dim 2 does, except that the innermost batch axis
+;; goes to the library as one strided batch.
+(defun matrix-geometry (tensor)
+  (let* ((view (foreign-alloc '(:struct view2))))
+    (unwind-protect
+         (progn
+           (fill-view2 view tensor tensor)
+           (let* ((rank (length (shape tensor)))
+                  (strides (loop for i below rank
+                                 collect (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-a) :int64 i)))
+                  (extents (loop for i below rank
+                                 collect (mem-aref (foreign-slot-pointer view '(:struct view2) 'shape) :int64 i))))
+             (assert (or (= 1 (nth (1- rank) extents)) (= 1 (nth (1- rank) strides))) ()
+                     "MatMulNode-HIPTensor: operands must be contiguous along the last axis (use ->contiguous)")
+             (values extents strides (foreign-slot-value view '(:struct view2) 'off-a))))
+      (foreign-free view))))
+
+(define-impl-op (MatMulNode :device HIPTensor :reject-p #'only-float-p)
+                :forward ((self a b out)
+                          (ensure-extension)
+                          (let ((trans-a (trans-a? self))
+                                (trans-b (trans-b? self))
+                                (a (if (trans-a? self) (read-untransposed a) a))
+                                (b (if (trans-b? self) (read-untransposed b) b)))
+                            (multiple-value-bind (ea sa oa) (matrix-geometry a)
+                              (multiple-value-bind (eb sb ob) (matrix-geometry b)
+                                (multiple-value-bind (ec sc oc) (matrix-geometry out)
+                                  (let* ((rank (length ec))
+                                         (m (nth (- rank 2) ec))
+                                         (n (nth (- rank 1) ec))
+                                         (k (if trans-a (nth (- rank 2) ea) (nth (- rank 1) ea)))
+                                         (lda (max 1 (nth (- rank 2) sa)))
+                                         (ldb (max 1 (nth (- rank 2) sb)))
+                                         (ldc (max 1 (nth (- rank 2) sc)))
+                                         (batch-rank (- rank 2)))
+                                    (labels ((launch (oa ob oc stride-a stride-b stride-c count)
+                                               (check (wf2hip-sgemm-strided-batched
+                                                       (char-code (if trans-b #\C #\N))
+                                                       (char-code (if trans-a #\C #\N))
+                                                       n m k 1.0
+                                                       (tensor-device-pointer b ob) ldb stride-b
+                                                       (tensor-device-pointer a oa) lda stride-a
+                                                       0.0
+                                                       (tensor-device-pointer out oc) ldc stride-c count)))
+                                             (walk (axis oa ob oc)
+                                               (cond
+                                                 ((= batch-rank 0) (launch oa ob oc 0 0 0 1))
+                                                 ((= axis (1- batch-rank))
+                                                  (launch oa ob oc (nth axis sa) (nth axis sb) (nth axis sc)
+                                                          (nth axis ec)))
+                                                 (t
+                                                  (dotimes (i (nth axis ec))
+                                                    (walk (1+ axis)
+                                                          (+ oa (* i (nth axis sa)))
+                                                          (+ ob (* i (nth axis sb)))
+                                                          (+ oc (* i (nth axis sc)))))))))
+                                      (walk 0 oa ob oc))))))
+                            out)))
