@@ -45,8 +45,8 @@ def qexp(r):
     return (mp.exp(r) - 1 - r) / (r * r) if r != 0 else mp.mpf(1) / 2
 
 
-Q = fit(qexp, -0.35, 0.35, 6)
-show("EXP_Q: exp(r) = 1 + r + r^2*Q(r), |r| <= 0.35, degree 6", Q)
+Q = fit(qexp, -0.35, 0.35, 5)
+show("EXP_Q: exp(r) = 1 + r + r^2*Q(r), |r| <= 0.35, degree 5", Q)
 print("// max rel err exp  :", mp.nstr(maxrel(lambda r: 1 + r + r * r * horner(Q, r), mp.exp, -0.35, 0.35), 5))
 print("// max rel err expm1:", mp.nstr(maxrel(lambda r: r + r * r * horner(Q, r), mp.expm1, -0.35, 0.35), 5))
 

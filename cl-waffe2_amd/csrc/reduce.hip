@@ -398,7 +398,7 @@ static int launch_maxmin(long n, const float* x, long incx, float* out) {
 // Lane l of the wave owns NV groups of 4 consecutive columns, group g starting
 // at column (g*64 + l)*4 (16-byte coalesced) or, when the row cannot be read
 // with 16-byte loads, columns (g*4 + c)*64 + l.
-template <int NV, bool VEC>
+template <int NV, bool VEC, bool NT = false>
 struct RowRegs {
   float v[NV][4];
 
@@ -408,6 +408,16 @@ struct RowRegs {
 
   __device__ __forceinline__ void load(const float* __restrict__ row, int64_t ncols, int lane,
                                        float fill) {
+    if (VEC && ncols == (int64_t)NV * kWave * 4) {
+      // the row fills the register tile exactly: unguarded loads, all in flight
+#pragma unroll
+      for (int g = 0; g < NV; g++) {
+        const f4* q = reinterpret_cast<const f4*>(row + col(g, 0, lane));
+        f4 t = NT ? __builtin_nontemporal_load(q) : *q;
+        v[g][0] = t.x; v[g][1] = t.y; v[g][2] = t.z; v[g][3] = t.w;
+      }
+      return;
+    }
 #pragma unroll
     for (int g = 0; g < NV; g++) {
       if (VEC && col(g, 3, lane) < ncols) {
@@ -424,6 +434,18 @@ struct RowRegs {
   }
 
   __device__ __forceinline__ void store(float* __restrict__ row, int64_t ncols, int lane) const {
+    if (VEC && ncols == (int64_t)NV * kWave * 4) {
+#pragma unroll
+      for (int g = 0; g < NV; g++) {
+        f4 t = {v[g][0], v[g][1], v[g][2], v[g][3]};
+        f4* q = reinterpret_cast<f4*>(row + col(g, 0, lane));
+        if (NT)
+          __builtin_nontemporal_store(t, q);
+        else
+          *q = t;
+      }
+      return;
+    }
 #pragma unroll
     for (int g = 0; g < NV; g++) {
       if (VEC && col(g, 3, lane) < ncols) {
@@ -442,7 +464,7 @@ struct RowRegs {
 
 // softmax over the first `valid` columns of a row; columns valid..ncols-1 of
 // the output are set to 0 (used by the causal form).
-template <int NV, bool VEC>
+template <int NV, bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restrict__ x, int64_t ldx,
                                                             float* __restrict__ out, int64_t ldo,
                                                             int64_t nrows, int64_t ncols,
@@ -452,7 +474,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
   const float ninf = -__builtin_inff();
-  RowRegs<NV, VEC> r;
+  RowRegs<NV, VEC, NT> r;
   r.load(x + row * ldx, valid, lane, ninf);
   float m = ninf;
 #pragma unroll
@@ -461,7 +483,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
     for (int c = 0; c < 4; c++) {
       if (causal_seq > 0) {
         // binary32 product, like a MulNode; padding stays -inf whatever the sign of scale
-        bool in = RowRegs<NV, VEC>::col(g, c, lane) < valid;
+        bool in = RowRegs<NV, VEC, NT>::col(g, c, lane) < valid;
         r.v[g][c] = in ? r.v[g][c] * scale : ninf;
       }
       m = fmaxf(m, r.v[g][c]);
@@ -523,7 +545,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __rest
   }
 }
 
-template <int NV, bool VEC>
+template <int NV, bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __restrict__ x,
                                                               const float* __restrict__ gamma,
                                                               const float* __restrict__ beta,
@@ -532,7 +554,8 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __res
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (row >= nrows) return;
   const int lane = threadIdx.x & (kWave - 1);
-  RowRegs<NV, VEC> r, g, b;
+  RowRegs<NV, VEC, NT> r;
+  RowRegs<NV, VEC, false> g, b;
   r.load(x + row * ncols, ncols, lane, 0.0f);
   g.load(gamma, ncols, lane, 0.0f);
   b.load(beta, ncols, lane, 0.0f);
@@ -547,7 +570,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __res
   for (int i = 0; i < NV; i++)
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      bool in = RowRegs<NV, VEC>::col(i, c, lane) < ncols;
+      bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
       double d = in ? (double)r.v[i][c] - mean : 0.0;
       sq += d * d;
     }
@@ -561,32 +584,39 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __res
   r.store(out + row * ncols, ncols, lane);
 }
 
-template <bool VEC>
+// Register tiles: NV groups of 256 columns per wavefront.  Sizes 3, 6 and 12
+// make rows of 768, 1536 and 3072 columns (transformer widths) fill the tile
+// exactly, which selects the unguarded load path.
+static int pick_nv(int64_t ncols) {
+  static const int sizes[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  for (int nv : sizes)
+    if ((int64_t)nv * kWave * 4 >= ncols) return nv;
+  return 0;
+}
+
+template <bool VEC, bool NT>
 static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t ldx, float* out,
                                int64_t ldo, int64_t nrows, int64_t ncols, int64_t causal_seq,
                                float scale) {
   hipStream_t st = rt().stream;
 #define WF2_SOFTMAX_CASE(N)                                                                   \
   case N:                                                                                     \
-    softmax_rows_wave<N, VEC><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,       \
-                                                         causal_seq, scale);                  \
+    softmax_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,   \
+                                                             causal_seq, scale);              \
     break;
   switch (nv) {
     WF2_SOFTMAX_CASE(1)
     WF2_SOFTMAX_CASE(2)
+    WF2_SOFTMAX_CASE(3)
     WF2_SOFTMAX_CASE(4)
+    WF2_SOFTMAX_CASE(6)
     WF2_SOFTMAX_CASE(8)
+    WF2_SOFTMAX_CASE(12)
     WF2_SOFTMAX_CASE(16)
     default: return fail(WF2HIP_EINVAL, "bad register tile");
   }
 #undef WF2_SOFTMAX_CASE
   return after_launch("softmax_rows_wave");
-}
-
-static int pick_nv(int64_t ncols) {
-  for (int nv = 1; nv <= 16; nv *= 2)
-    if ((int64_t)nv * kWave * 4 >= ncols) return nv;
-  return 0;
 }
 
 static int softmax_dispatch(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
@@ -605,26 +635,32 @@ static int softmax_dispatch(int64_t nrows, int64_t ncols, const float* x, int64_
   int64_t blocks = ceil_div(nrows, kWavesPerBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
   const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0;
+  const bool streaming = nrows * ncols * 8 >= ((int64_t)192 << 20);
+  if (vec && streaming)
+    return launch_softmax_wave<true, true>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                           causal_seq, scale);
   if (vec)
-    return launch_softmax_wave<true>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
-                                     causal_seq, scale);
-  return launch_softmax_wave<false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
-                                    causal_seq, scale);
+    return launch_softmax_wave<true, false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                            causal_seq, scale);
+  return launch_softmax_wave<false, false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                           causal_seq, scale);
 }
 
-template <bool VEC>
+template <bool VEC, bool NT>
 static int launch_layernorm_wave(int nv, uint32_t blocks, const float* x, const float* g,
                                  const float* b, float eps, float* out, int64_t nrows,
                                  int64_t ncols) {
   hipStream_t st = rt().stream;
-#define WF2_LN_CASE(N)                                                                          \
-  case N:                                                                                       \
-    layernorm_rows_wave<N, VEC><<<blocks, kBlock, 0, st>>>(x, g, b, eps, out, nrows, ncols);     \
+#define WF2_LN_CASE(N)                                                                            \
+  case N:                                                                                         \
+    layernorm_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, g, b, eps, out, nrows, ncols);   \
     break;
   switch (nv) {
     WF2_LN_CASE(1)
     WF2_LN_CASE(2)
+    WF2_LN_CASE(3)
     WF2_LN_CASE(4)
+    WF2_LN_CASE(6)
     WF2_LN_CASE(8)
     default: return fail(WF2HIP_EUNSUPPORTED, "LayerNorm rows longer than 2048 are not supported");
   }
@@ -693,7 +729,10 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
   const bool vec = aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta) &&
                    cols % 4 == 0;
+  const bool streaming = (int64_t)rows * cols * 8 >= ((int64_t)192 << 20);
+  if (vec && streaming)
+    return launch_layernorm_wave<true, true>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
   if (vec)
-    return launch_layernorm_wave<true>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
-  return launch_layernorm_wave<false>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
+    return launch_layernorm_wave<true, false>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
+  return launch_layernorm_wave<false, false>(nv, (uint32_t)blocks, x, gamma, beta, eps, out, rows, cols);
 }

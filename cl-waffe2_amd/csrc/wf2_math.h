@@ -8,10 +8,11 @@
 //
 // Design: CDNA3/CDNA4 issue a binary64 FMA at the same rate as a non-packed
 // binary32 FMA, so every core is evaluated in binary64 with a short
-// polynomial (relative error < 2^-35) and rounded to binary32 once at the
-// end.  The result is within 0.5 + 2^-10 ulp of the exact value, hence within
-// 1.5 ulp of any 1.0-ulp implementation.  Only IEEE operations and fma are
-// used (plus one reciprocal seed that is refined by two Newton steps), so the
+// polynomial (relative error < 2^-30) and rounded to binary32 once at the
+// end.  The result is within 0.506 ulp of the exact value for every binary32
+// input (exhaustive host run), hence within 1.51 ulp of any 1.0-ulp
+// implementation.  Only IEEE operations and fma are
+// used (plus one reciprocal seed that is refined by a Newton step), so the
 // same header compiles for the host and a CPU build can check every binary32
 // input against libm.
 //
@@ -59,16 +60,15 @@ constexpr double kTwoOverPi = 0.6366197723675813430755351;
 constexpr double kPio2Head = 1.57079632673412561416626;    // 33 significant bits
 constexpr double kPio2Tail = 6.077100506506192601475144e-11;
 
-// exp(r) = 1 + r + r^2 Q(r) on |r| <= 0.35; relative error 4.7e-12 (exp),
-// 1.1e-11 (expm1).
+// exp(r) = 1 + r + r^2 Q(r) on |r| <= 0.35, Q of degree 5; relative error
+// 2.4e-10 (exp), 5.7e-10 (expm1): 2^-31, i.e. at most 0.004 ulp of binary32.
 WF2_MATH_FN double expm1_poly(double r) {
-  double q = 0.00002486073188584067535;
-  q = WF2_FMA(q, r, 0.00019900428151915095571);
-  q = WF2_FMA(q, r, 0.0013888852650225144401);
-  q = WF2_FMA(q, r, 0.008333297083738308707);
-  q = WF2_FMA(q, r, 0.041666666722163555503);
-  q = WF2_FMA(q, r, 0.16666666722181582537);
-  q = WF2_FMA(q, r, 0.5);
+  double q = 0.00019891969905683136498;
+  q = WF2_FMA(q, r, 0.0013934531655088020325);
+  q = WF2_FMA(q, r, 0.0083333100347068682249);
+  q = WF2_FMA(q, r, 0.041666456904062640998);
+  q = WF2_FMA(q, r, 0.16666666682523656912);
+  q = WF2_FMA(q, r, 0.50000000142765894076);
   return WF2_FMA(r * r, q, r);
 }
 
@@ -84,7 +84,7 @@ WF2_MATH_FN void exp_reduce(double x, double* em1_r, double* scale) {
   *scale = double_of((uint64_t)(uint32_t)(ni + 1023) << 52);
 }
 
-// e^x in binary64 for x in [-104, 89] (relative error < 1e-11).
+// e^x in binary64 for x in [-104, 89] (relative error < 2.5e-10).
 WF2_MATH_FN double exp_core(double x) {
   double p, s;
   exp_reduce(x, &p, &s);
@@ -94,19 +94,17 @@ WF2_MATH_FN double exp_core(double x) {
 WF2_MATH_FN float expf_(float x) {
   // Below -104 the result rounds to +0 and above 89 to +inf, as e^-104 and
   // e^89 already do, so clamping is exact.  fmin/fmax drop a NaN operand.
-  double xd = __builtin_fmin(__builtin_fmax((double)x, -104.0), 89.0);
-  float r = (float)exp_core(xd);
+  float xc = __builtin_fminf(__builtin_fmaxf(x, -104.0f), 89.0f);  // one v_med3_f32
+  float r = (float)exp_core((double)xc);
   return (x != x) ? x : r;
 }
 
-// 1/d for d >= 1 representable in binary32 range: a binary32 seed refined by
-// two Newton steps in binary64 (relative error ~2^-50 whatever the seed's
-// last bit).
+// 1/d for d >= 1 in binary32 range: a binary32 seed (relative error <= 2^-22
+// for v_rcp_f32, 2^-24 for a correctly rounded host division) refined by one
+// Newton step in binary64, which squares the error: <= 2^-44.
 WF2_MATH_FN double rcp_refined(double d) {
   double y = (double)WF2_RCP_SEED((float)d);
   double e = WF2_FMA(-d, y, 1.0);
-  y = WF2_FMA(y, e, y);
-  e = WF2_FMA(-d, y, 1.0);
   return WF2_FMA(y, e, y);
 }
 
