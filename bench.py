@@ -258,7 +258,7 @@ def main():
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "kernels": kernels,
         "roofline": {
-            "kernel": "ew_rows<OpAdd, ReadDst, VEC 4, U 4, NT> (x <- x + y, 2^26 elements)",
+            "kernel": "ew_flat<OpAdd, ReadDst, NT, wave-contiguous, 4 vectors/thread> (x <- x + y, 2^26 elements)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,

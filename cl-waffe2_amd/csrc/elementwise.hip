@@ -80,10 +80,9 @@ struct OpPow {
 // 6.59 with layout 0; two streams (copy, unary) 6.45 with layout 0 against 6.25.
 // Functors with a long binary64 body (transcendentals) take two vectors per
 // thread instead of four: measured 4-7 % faster at 2^26 (exp 5.91 -> 6.36 TB/s).
-template <class F, bool ReadDst, bool SrcBroadcast, bool NT, int LAYOUT>
+template <class F, bool ReadDst, bool SrcBroadcast, bool NT, int LAYOUT, int kFlatU>
 __global__ __launch_bounds__(kBlock) void ew_flat(float* __restrict__ dst,
                                                   const float* __restrict__ src, size_t nvec, F f) {
-  constexpr int kFlatU = F::kFlatU;
   size_t base;
   if (LAYOUT == 0) {
     base = (size_t)blockIdx.x * kBlock * kFlatU + threadIdx.x;
@@ -433,22 +432,32 @@ static bool try_launch_flat(const Space& s, float* dst, const float* src, F f, i
   const bool bcast = s.sb[0] == 0;
   if (!aligned16(d) || (!bcast && !aligned16(q))) return false;
   const size_t nvec = (size_t)(s.total / 4);
-  const int64_t blocks = ceil_div((int64_t)nvec, kBlock * F::kFlatU);
-  if (blocks >= ((int64_t)1 << 31)) return false;
+  // vectors per thread: 4 for x <- x op y (three streams), 2 for functors with
+  // a long binary64 body, 1 for the light two-stream forms (copy, fill, scalar
+  // operand, sqrt, abs) -- each the best of a sweep at 2^26 on MI355X.
+  constexpr int u3 = 4;
+  constexpr int u2 = F::kFlatU == 2 ? 2 : 1;
   const int64_t streams = 1 + (ReadDst ? 1 : 0) + (bcast ? 0 : 1);
   const bool nt = s.total * 4 * streams >= kStreamingBytes;
   hipStream_t st = rt().stream;
-  constexpr int layout = ReadDst ? 1 : 0;
+  const bool three = ReadDst && !bcast;
+  const int64_t blocks = ceil_div((int64_t)nvec, kBlock * (three ? u3 : u2));
+  if (blocks >= ((int64_t)1 << 31)) return false;
   if (bcast) {
     if (nt)
-      ew_flat<F, ReadDst, true, true, 0><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, true, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
     else
-      ew_flat<F, ReadDst, true, false, 0><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, true, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+  } else if (ReadDst) {
+    if (nt)
+      ew_flat<F, ReadDst, false, true, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+    else
+      ew_flat<F, ReadDst, false, false, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
   } else {
     if (nt)
-      ew_flat<F, ReadDst, false, true, layout><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
     else
-      ew_flat<F, ReadDst, false, false, layout><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
   }
   *rc = after_launch("ew_flat");
   const int64_t done = (int64_t)nvec * 4;

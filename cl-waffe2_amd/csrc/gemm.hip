@@ -17,8 +17,8 @@
 // cl-waffe2's plain row-major matmul lands on (left k-innermost, right
 // cols-innermost), where both global reads are contiguous.
 //
-// Tiling: 128x128 per workgroup, K-step 16, 4 wavefronts in 2x2, each owning a
-// 64x64 block = 2x2 MFMA tiles of 32x32 (64 accumulator registers per lane).
+// Tiling: 128x128 (or 128x64) per workgroup, K-step 16, 4 wavefronts in 2x2,
+// each owning 2x2 (or 2x1) MFMA tiles of 32x32 (64 or 32 accumulator registers).
 // Operand tiles are staged global -> registers -> LDS with two LDS buffers, so
 // one barrier per K-step; a k-innermost tile is kept [128][16+4] and read back
 // with one 128-bit LDS load per four MFMA steps (the +4 pad makes eight
@@ -35,9 +35,8 @@ namespace wf2 {
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 16;
-constexpr int KPITCH = BK + 4;       // row pitch of a k-innermost LDS tile
-constexpr int TILE_FLOATS = BM * KPITCH;  // >= BK*BM, size of one operand buffer
+constexpr int BK = 16;
+constexpr int KPITCH = BK + 4;  // row pitch of a k-innermost LDS tile
 
 struct GemmParams {
   const float* L;  // left operand  (rows = M)
@@ -45,28 +44,31 @@ struct GemmParams {
   float* C;
   int64_t M, N, K;
   int64_t ldl, ldr, ldc;
-  int64_t sL, sR, sC;  // batch strides
+  int64_t sL, sR, sC;     // strides of the inner batch axis
+  int64_t sL2, sR2, sC2;  // strides of the outer batch axis
+  uint32_t batch_inner;   // blockIdx.y = outer * batch_inner + inner
   float alpha, beta;
   uint32_t tiles_m, tiles_n;
 };
 
-// Loads this thread's share of a 128 x 16 operand tile into registers.
+// Loads this thread's share of a ROWS x 16 operand tile into registers
+// (ROWS/64 float4 per thread).
 // KIN: operand stored [x][k] (k innermost) else [k][x].
 // FAST: 16-byte loads (pointer, pitch and extents checked on the host).
-template <bool KIN, bool FAST>
+template <bool KIN, bool FAST, int ROWS>
 __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_t ld, int64_t x0,
-                                          int64_t k0, int64_t X, int64_t K, f4 (&reg)[2]) {
+                                          int64_t k0, int64_t X, int64_t K, f4 (&reg)[ROWS / 64]) {
   const int t = threadIdx.x;
 #pragma unroll
-  for (int j = 0; j < 2; j++) {
-    const int f = t + kBlock * j;  // float4 slot 0..511
+  for (int j = 0; j < ROWS / 64; j++) {
+    const int f = t + kBlock * j;  // float4 slot
     int64_t x, k;
     if (KIN) {
       x = x0 + (f >> 2);
       k = k0 + (f & 3) * 4;
     } else {
-      k = k0 + (f >> 5);
-      x = x0 + (f & 31) * 4;
+      k = k0 + f / (ROWS / 4);
+      x = x0 + (f % (ROWS / 4)) * 4;
     }
     f4 v = {0.f, 0.f, 0.f, 0.f};
     if (FAST) {
@@ -85,20 +87,21 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
   }
 }
 
-template <bool KIN>
-__device__ __forceinline__ void store_tile(float* __restrict__ lds, const f4 (&reg)[2]) {
+template <bool KIN, int ROWS>
+__device__ __forceinline__ void store_tile(float* __restrict__ lds, const f4 (&reg)[ROWS / 64]) {
   const int t = threadIdx.x;
 #pragma unroll
-  for (int j = 0; j < 2; j++) {
+  for (int j = 0; j < ROWS / 64; j++) {
     const int f = t + kBlock * j;
-    float* dst = KIN ? lds + (f >> 2) * KPITCH + (f & 3) * 4 : lds + (f >> 5) * BM + (f & 31) * 4;
+    float* dst = KIN ? lds + (f >> 2) * KPITCH + (f & 3) * 4
+                     : lds + (f / (ROWS / 4)) * ROWS + (f % (ROWS / 4)) * 4;
     *reinterpret_cast<f4*>(dst) = reg[j];
   }
 }
 
 // Fragment for MFMA steps s = 0..3 of k-group `kb` (0 or 8): frag[s] is the
 // operand value for row/col (x0 + lane%32) at k = kb + 4*(lane/32) + s.
-template <bool KIN>
+template <bool KIN, int ROWS>
 __device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0, int kb, int lane,
                                           float (&frag)[4]) {
   const int xi = x0 + (lane & 31);
@@ -108,14 +111,21 @@ __device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0,
     frag[0] = v.x; frag[1] = v.y; frag[2] = v.z; frag[3] = v.w;
   } else {
 #pragma unroll
-    for (int s = 0; s < 4; s++) frag[s] = lds[(kb + half * 4 + s) * BM + xi];
+    for (int s = 0; s < 4; s++) frag[s] = lds[(kb + half * 4 + s) * ROWS + xi];
   }
 }
 
-template <bool LKIN, bool RKIN, bool FAST>
+// TM x TN MFMA tiles (32x32) per wavefront, wavefronts 2 x 2: the workgroup
+// tile is (64 TM) x (64 TN).  2x2 -> 128x128 (64 accumulator registers), 2x1
+// -> 128x64 for narrow outputs and for shapes whose 128x128 tiling would leave
+// a partial last round of workgroups.
+template <bool LKIN, bool RKIN, bool FAST, int TM, int TN>
 __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(16))) float ldsL[2][TILE_FLOATS];
-  __shared__ __attribute__((aligned(16))) float ldsR[2][TILE_FLOATS];
+  constexpr int BMt = 64 * TM, BNt = 64 * TN;
+  constexpr int LFLOATS = LKIN ? BMt * KPITCH : BK * BMt;
+  constexpr int RFLOATS = RKIN ? BNt * KPITCH : BK * BNt;
+  __shared__ __attribute__((aligned(16))) float ldsL[2][LFLOATS];
+  __shared__ __attribute__((aligned(16))) float ldsR[2][RFLOATS];
 
   // Tile order: consecutive workgroups land on different XCDs (round robin),
   // so give each XCD a contiguous band of tiles, and walk a band column-major
@@ -135,59 +145,61 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   const uint32_t tm = first_m + (pid % width) % gsize;
   const uint32_t tn = (pid % width) / gsize;
 
-  const int64_t m0 = (int64_t)tm * BM;
-  const int64_t n0 = (int64_t)tn * BN;
-  const float* L = p.L + (int64_t)blockIdx.y * p.sL;
-  const float* R = p.R + (int64_t)blockIdx.y * p.sR;
-  float* C = p.C + (int64_t)blockIdx.y * p.sC;
+  const int64_t m0 = (int64_t)tm * BMt;
+  const int64_t n0 = (int64_t)tn * BNt;
+  const uint32_t zo = blockIdx.y / p.batch_inner;
+  const uint32_t zi = blockIdx.y - zo * p.batch_inner;
+  const float* L = p.L + (int64_t)zo * p.sL2 + (int64_t)zi * p.sL;
+  const float* R = p.R + (int64_t)zo * p.sR2 + (int64_t)zi * p.sR;
+  float* C = p.C + (int64_t)zo * p.sC2 + (int64_t)zi * p.sC;
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  const int wm = (wave >> 1) * 64;
-  const int wn = (wave & 1) * 64;
+  const int wm = (wave >> 1) * 32 * TM;
+  const int wn = (wave & 1) * 32 * TN;
 
-  f16v acc[2][2];
+  f16v acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  f4 regL[2], regR[2];
+  f4 regL[BMt / 64], regR[BNt / 64];
   const int64_t ksteps = (p.K + BK - 1) / BK;
-  load_tile<LKIN, FAST>(L, p.ldl, m0, 0, p.M, p.K, regL);
-  load_tile<RKIN, FAST>(R, p.ldr, n0, 0, p.N, p.K, regR);
-  store_tile<LKIN>(ldsL[0], regL);
-  store_tile<RKIN>(ldsR[0], regR);
+  load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, 0, p.M, p.K, regL);
+  load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, 0, p.N, p.K, regR);
+  store_tile<LKIN, BMt>(ldsL[0], regL);
+  store_tile<RKIN, BNt>(ldsR[0], regR);
   __syncthreads();
 
   for (int64_t ks = 0; ks < ksteps; ks++) {
     const int cur = (int)(ks & 1);
     if (ks + 1 < ksteps) {
-      load_tile<LKIN, FAST>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
-      load_tile<RKIN, FAST>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
+      load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
+      load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
     }
 #pragma unroll
     for (int kb = 0; kb < BK; kb += 8) {
-      float a[2][4], b[2][4];
+      float a[TM][4], b[TN][4];
 #pragma unroll
-      for (int i = 0; i < 2; i++) read_frag<LKIN>(ldsL[cur], wm + i * 32, kb, lane, a[i]);
+      for (int i = 0; i < TM; i++) read_frag<LKIN, BMt>(ldsL[cur], wm + i * 32, kb, lane, a[i]);
 #pragma unroll
-      for (int j = 0; j < 2; j++) read_frag<RKIN>(ldsR[cur], wn + j * 32, kb, lane, b[j]);
+      for (int j = 0; j < TN; j++) read_frag<RKIN, BNt>(ldsR[cur], wn + j * 32, kb, lane, b[j]);
 #pragma unroll
       for (int s = 0; s < 4; s++)
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int j = 0; j < 2; j++)
+          for (int j = 0; j < TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
     }
     if (ks + 1 < ksteps) {
       // The other buffer was last read in iteration ks-1, and every wave has
       // passed the barrier that ended it.
-      store_tile<LKIN>(ldsL[cur ^ 1], regL);
-      store_tile<RKIN>(ldsR[cur ^ 1], regR);
+      store_tile<LKIN, BMt>(ldsL[cur ^ 1], regL);
+      store_tile<RKIN, BNt>(ldsR[cur ^ 1], regR);
     }
     __syncthreads();
   }
@@ -195,9 +207,9 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < TN; j++) {
       const int64_t col = n0 + wn + j * 32 + (lane & 31);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -217,21 +229,53 @@ static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; 
 static bool is_n(char c) { return c == 'N' || c == 'n'; }
 static bool is_t(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
-int sgemm_batched(char transa, char transb, long m, long n, long k, float alpha, const float* A,
-                  long lda, long strideA, const float* B, long ldb, long strideB, float beta,
-                  float* C, long ldc, long strideC, long batch) {
+template <bool LK, bool RK, int TM, int TN>
+static void launch_variant(const GemmParams& p, bool fast, dim3 grid, hipStream_t st) {
+  if (fast)
+    sgemm_kernel<LK, RK, true, TM, TN><<<grid, kBlock, 0, st>>>(p);
+  else
+    sgemm_kernel<LK, RK, false, TM, TN><<<grid, kBlock, 0, st>>>(p);
+}
+
+template <int TM, int TN>
+static void launch_layout(const GemmParams& p, bool lkin, bool rkin, bool fast, dim3 grid,
+                          hipStream_t st) {
+  if (lkin && rkin)
+    launch_variant<true, true, TM, TN>(p, fast, grid, st);
+  else if (lkin)
+    launch_variant<true, false, TM, TN>(p, fast, grid, st);
+  else if (rkin)
+    launch_variant<false, true, TM, TN>(p, fast, grid, st);
+  else
+    launch_variant<false, false, TM, TN>(p, fast, grid, st);
+}
+
+// Workgroups are spread evenly over the CUs, and the ones resident on a CU
+// share its matrix cores, so the launch takes about as long as the busiest CU:
+// ceil(tiles / CUs) tiles, one after the other.
+static double busiest_cu_tiles(int64_t tiles) {
+  const int64_t cus = rt().num_cus;
+  return (double)((tiles + cus - 1) / cus);
+}
+
+int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha, const float* A,
+                   long lda, long strideA, long strideA2, const float* B, long ldb, long strideB,
+                   long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
+                   long batch, long batch2) {
   if (!(is_n(transa) || is_t(transa)) || !(is_n(transb) || is_t(transb)))
     return fail(WF2HIP_EINVAL, "trans must be N, T or C");
-  if (m < 0 || n < 0 || k < 0 || batch < 0) return fail(WF2HIP_EINVAL, "negative dimension");
+  if (m < 0 || n < 0 || k < 0 || batch < 0 || batch2 < 0)
+    return fail(WF2HIP_EINVAL, "negative dimension");
   // sgemm_'s own leading-dimension rules (column-major)
   const long rows_a = is_n(transa) ? m : k;
   const long rows_b = is_n(transb) ? k : n;
   if (lda < (rows_a > 1 ? rows_a : 1) || ldb < (rows_b > 1 ? rows_b : 1) || ldc < (m > 1 ? m : 1))
     return fail(WF2HIP_EINVAL, "leading dimension too small (lda %ld ldb %ld ldc %ld)", lda, ldb,
                 ldc);
-  if (m == 0 || n == 0 || batch == 0) return 0;
+  if (m == 0 || n == 0 || batch == 0 || batch2 == 0) return 0;
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
-  if (batch > 65535) return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  if ((int64_t)batch * batch2 > 65535)
+    return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
 
   GemmParams p;
   // row-major view: Cr[n][m] = Left[n][k] . Right[k][m]
@@ -247,36 +291,39 @@ int sgemm_batched(char transa, char transb, long m, long n, long k, float alpha,
   p.sL = strideB;
   p.sR = strideA;
   p.sC = strideC;
+  p.sL2 = strideB2;
+  p.sR2 = strideA2;
+  p.sC2 = strideC2;
+  p.batch_inner = (uint32_t)batch;
   p.alpha = alpha;
   p.beta = beta;
-  p.tiles_m = (uint32_t)ceil_div(p.M, BM);
-  p.tiles_n = (uint32_t)ceil_div(p.N, BN);
   const bool lkin = is_n(transb);   // left stored [rows][k]
   const bool rkin = !is_n(transa);  // right stored [cols][k]
-  int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
-  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
   bool fast = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && strideA % 4 == 0 &&
-              strideB % 4 == 0;
+              strideB % 4 == 0 && strideA2 % 4 == 0 && strideB2 % 4 == 0;
   // every 4-wide load must be wholly inside or wholly outside the matrix
   fast = fast && (lkin ? k % 4 == 0 : p.M % 4 == 0) && (rkin ? k % 4 == 0 : p.N % 4 == 0);
-  dim3 grid((uint32_t)blocks, (uint32_t)batch);
+
+  // Tile choice: time ~ tiles on the busiest CU x work per tile.
+  // The narrow tile does 15 % less work per cycle (one operand is re-read from
+  // LDS twice as often) but wastes nothing on N <= 64 and evens out the last
+  // round.
+  const int64_t nb = (int64_t)batch * batch2;
+  const int64_t tiles_wide = ceil_div(p.M, 128) * ceil_div(p.N, 128) * nb;
+  const int64_t tiles_narrow = ceil_div(p.M, 128) * ceil_div(p.N, 64) * nb;
+  const double cost_wide = busiest_cu_tiles(tiles_wide) * 1.0;
+  const double cost_narrow = busiest_cu_tiles(tiles_narrow) * 0.5 / 0.85;
+  const bool narrow = cost_narrow < cost_wide;
+  p.tiles_m = (uint32_t)ceil_div(p.M, 128);
+  p.tiles_n = (uint32_t)ceil_div(p.N, narrow ? 64 : 128);
+  const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
+  dim3 grid((uint32_t)blocks, (uint32_t)nb);
   hipStream_t st = rt().stream;
-#define WF2_GEMM_LAUNCH(LK, RK)                                                   \
-  do {                                                                            \
-    if (fast)                                                                     \
-      sgemm_kernel<LK, RK, true><<<grid, kBlock, 0, st>>>(p);                     \
-    else                                                                          \
-      sgemm_kernel<LK, RK, false><<<grid, kBlock, 0, st>>>(p);                    \
-  } while (0)
-  if (lkin && rkin)
-    WF2_GEMM_LAUNCH(true, true);
-  else if (lkin)
-    WF2_GEMM_LAUNCH(true, false);
-  else if (rkin)
-    WF2_GEMM_LAUNCH(false, true);
+  if (narrow)
+    launch_layout<2, 1>(p, lkin, rkin, fast, grid, st);
   else
-    WF2_GEMM_LAUNCH(false, false);
-#undef WF2_GEMM_LAUNCH
+    launch_layout<2, 2>(p, lkin, rkin, fast, grid, st);
   return after_launch("sgemm_kernel");
 }
 
@@ -288,7 +335,8 @@ WF2_API int wf2hip_sgemm(char transa, char transb, long m, long n, long k, float
                          const float* A, long lda, const float* B, long ldb, float beta, float* C,
                          long ldc) {
   WF2_TRY(require_init());
-  return sgemm_batched(transa, transb, m, n, k, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1);
+  return sgemm_batched2(transa, transb, m, n, k, alpha, A, lda, 0, 0, B, ldb, 0, 0, beta, C, ldc, 0,
+                        0, 1, 1);
 }
 
 WF2_API int wf2hip_sgemm_strided_batched(char transa, char transb, long m, long n, long k,
@@ -296,6 +344,16 @@ WF2_API int wf2hip_sgemm_strided_batched(char transa, char transb, long m, long 
                                          const float* B, long ldb, long strideB, float beta,
                                          float* C, long ldc, long strideC, long batch) {
   WF2_TRY(require_init());
-  return sgemm_batched(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C,
-                       ldc, strideC, batch);
+  return sgemm_batched2(transa, transb, m, n, k, alpha, A, lda, strideA, 0, B, ldb, strideB, 0,
+                        beta, C, ldc, strideC, 0, batch, 1);
+}
+
+WF2_API int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, long n, long k,
+                                            float alpha, const float* A, long lda, long strideA,
+                                            long strideA2, const float* B, long ldb, long strideB,
+                                            long strideB2, float beta, float* C, long ldc,
+                                            long strideC, long strideC2, long batch, long batch2) {
+  WF2_TRY(require_init());
+  return sgemm_batched2(transa, transb, m, n, k, alpha, A, lda, strideA, strideA2, B, ldb, strideB,
+                        strideB2, beta, C, ldc, strideC, strideC2, batch, batch2);
 }

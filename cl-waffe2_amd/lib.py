@@ -104,6 +104,10 @@ _SIGNATURES = {
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _P, _L, _L, _F, _P, _L, _L, _L],
         C.c_int,
     ),
+    "wf2hip_sgemm_strided_batched_2d": (
+        [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],
+        C.c_int,
+    ),
 }
 
 EXPORTS = tuple(_SIGNATURES)

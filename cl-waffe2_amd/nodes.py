@@ -181,41 +181,48 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     ta = b"C" if trans_a else b"N"
     tb = b"C" if trans_b else b"N"
 
-    def launch(offa, offb, offc, strides3, count):
-        _lib.check(lib.wf2hip_sgemm_strided_batched(
+    def launch(offa, offb, offc, inner, outer):
+        (count, s3), (count2, s3o) = inner, outer
+        _lib.check(lib.wf2hip_sgemm_strided_batched_2d(
             tb, ta, n, m, k, 1.0,
-            C.c_void_p(b.ptr + 4 * offb), ldb, strides3[1],
-            C.c_void_p(a.ptr + 4 * offa), lda, strides3[0],
-            0.0, C.c_void_p(out.ptr + 4 * offc), ldc, strides3[2], count))
+            C.c_void_p(b.ptr + 4 * offb), ldb, s3[1], s3o[1],
+            C.c_void_p(a.ptr + 4 * offa), lda, s3[0], s3o[0],
+            0.0, C.c_void_p(out.ptr + 4 * offc), ldc, s3[2], s3o[2], count, count2))
 
-    # Collapse the batch axes into one strided axis when all three tensors
-    # allow it; otherwise loop over the outer ones on the host like the CPU
-    # backend does for every batch index.  Extent-1 axes carry no information.
-    keep = [i for i, n in enumerate(batch_shape) if n != 1]
+    # Fold the batch axes, innermost first, into at most two strided axes per
+    # launch (the library takes two batch levels); anything beyond that is
+    # walked on the host like the CPU backend walks every batch index.
+    # Extent-1 axes carry no information.
+    keep = [i for i, n_ in enumerate(batch_shape) if n_ != 1]
     batch_shape = [batch_shape[i] for i in keep]
     sta, stb, stc = ([st[i] for i in keep] for st in (sta, stb, stc))
-    nb = len(batch_shape)
-    if nb == 0:
-        launch(oa, ob, oc, (0, 0, 0), 1)
+
+    def fold(last):
+        """Merge axes last, last-1, ... while they form one strided run for all
+        three tensors (0 == 0 x count holds for a broadcast operand)."""
+        count = batch_shape[last]
+        s3 = [sta[last], stb[last], stc[last]]
+        first = last
+        while first > 0 and all(st[first - 1] == s * count for st, s in zip((sta, stb, stc), s3)):
+            first -= 1
+            count *= batch_shape[first]
+        return first, (count, s3)
+
+    none = (1, [0, 0, 0])
+    if not batch_shape:
+        launch(oa, ob, oc, none, none)
         return out
-    inner = nb - 1
-    count = batch_shape[inner]
-    strides3 = [sta[inner], stb[inner], stc[inner]]
-    while inner > 0:
-        o = inner - 1
-        # axis o continues the run when its stride is (merged stride x merged count),
-        # which also holds for 0 == 0 x count on a broadcast operand
-        if not all(st[o] == s3 * count for st, s3 in zip((sta, stb, stc), strides3)):
-            break
-        count *= batch_shape[o]
-        inner = o
-    outer_shape = batch_shape[:inner]
-    if count > 65535:
-        raise ValueError("MatMulNode: more than 65535 matrices in one strided batch")
+    first, inner = fold(len(batch_shape) - 1)
+    outer = none
+    if first > 0:
+        first, outer = fold(first - 1)
+    if inner[0] * outer[0] > 65535:
+        raise ValueError("MatMulNode: more than 65535 matrices in one launch")
+    outer_shape = batch_shape[:first]
 
     def rec(axis, offa, offb, offc):
         if axis == len(outer_shape):
-            launch(offa, offb, offc, strides3, count)
+            launch(offa, offb, offc, inner, outer)
             return
         for i in range(outer_shape[axis]):
             rec(axis + 1, offa + i * sta[axis], offb + i * stb[axis], offc + i * stc[axis])

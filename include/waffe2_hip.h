@@ -209,6 +209,15 @@ int wf2hip_sgemm_strided_batched(char transa, char transb, long m, long n, long 
                                  const float* B, long ldb, long strideB, float beta,
                                  float* C, long ldc, long strideC, long batch);
 
+/* Two batch axes (matrix z = outer * batch + inner; strides *2 belong to the
+ * outer axis): heads read in place from a fused (B, T, 3, H, hd) projection
+ * have batch strides that do not merge into one. */
+int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, long n, long k,
+                                    float alpha, const float* A, long lda, long strideA,
+                                    long strideA2, const float* B, long ldb, long strideB,
+                                    long strideB2, float beta, float* C, long ldc, long strideC,
+                                    long strideC2, long batch, long batch2);
+
 #ifdef __cplusplus
 }
 #endif
