@@ -17,17 +17,19 @@
 // cl-waffe2's plain row-major matmul lands on (left k-innermost, right
 // cols-innermost), where both global reads are contiguous.
 //
-// Tiling: 128x128 (or 128x64) per workgroup, K-step 16, 4 wavefronts in 2x2,
+// Tiling: 128x128 (or 128x64) per workgroup, K-step 32, 4 wavefronts in 2x2,
 // each owning 2x2 (or 2x1) MFMA tiles of 32x32 (64 or 32 accumulator registers).
 // Operand tiles are staged global -> registers -> LDS with two LDS buffers, so
-// one barrier per K-step; a k-innermost tile is kept [128][16+4] and read back
+// one barrier per K-step; a k-innermost tile is kept [128][32+4] and read back
 // with one 128-bit LDS load per four MFMA steps (the +4 pad makes eight
-// consecutive lanes cover all 32 banks), an x-innermost tile is kept [16][128]
+// consecutive lanes cover all 32 banks), an x-innermost tile is kept [32][128]
 // and read with conflict-free 32-bit loads.  Within a group of 8 k values,
 // MFMA step s takes k = s from lanes 0-31 and k = 4+s from lanes 32-63 for
 // both operands, which is what makes the 128-bit read usable.
 //
 // Bound: fp32 MFMA peak (157.3 TFLOP/s on MI355X); 2 m n k flop per product.
+#include <stdlib.h>
+
 #include "wf2_common.h"
 
 namespace wf2 {
@@ -35,8 +37,8 @@ namespace wf2 {
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 16;
-constexpr int KPITCH = BK + 4;  // row pitch of a k-innermost LDS tile
+constexpr int BK = 32;
+constexpr int KPITCH = BK + 4;  // row pitch of a k-innermost LDS tile (36: b128 reads of 8 lanes cover all 32 banks)
 
 struct GemmParams {
   const float* L;  // left operand  (rows = M)
@@ -51,21 +53,21 @@ struct GemmParams {
   uint32_t tiles_m, tiles_n;
 };
 
-// Loads this thread's share of a ROWS x 16 operand tile into registers
-// (ROWS/64 float4 per thread).
+// Loads this thread's share of a ROWS x BK operand tile into registers
+// (ROWS/32 float4 per thread).
 // KIN: operand stored [x][k] (k innermost) else [k][x].
 // FAST: 16-byte loads (pointer, pitch and extents checked on the host).
 template <bool KIN, bool FAST, int ROWS>
 __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_t ld, int64_t x0,
-                                          int64_t k0, int64_t X, int64_t K, f4 (&reg)[ROWS / 64]) {
+                                          int64_t k0, int64_t X, int64_t K, f4 (&reg)[ROWS / 32]) {
   const int t = threadIdx.x;
 #pragma unroll
-  for (int j = 0; j < ROWS / 64; j++) {
+  for (int j = 0; j < ROWS / 32; j++) {
     const int f = t + kBlock * j;  // float4 slot
     int64_t x, k;
     if (KIN) {
-      x = x0 + (f >> 2);
-      k = k0 + (f & 3) * 4;
+      x = x0 + (f >> 3);
+      k = k0 + (f & 7) * 4;
     } else {
       k = k0 + f / (ROWS / 4);
       x = x0 + (f % (ROWS / 4)) * 4;
@@ -88,18 +90,18 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
 }
 
 template <bool KIN, int ROWS>
-__device__ __forceinline__ void store_tile(float* __restrict__ lds, const f4 (&reg)[ROWS / 64]) {
+__device__ __forceinline__ void store_tile(float* __restrict__ lds, const f4 (&reg)[ROWS / 32]) {
   const int t = threadIdx.x;
 #pragma unroll
-  for (int j = 0; j < ROWS / 64; j++) {
+  for (int j = 0; j < ROWS / 32; j++) {
     const int f = t + kBlock * j;
-    float* dst = KIN ? lds + (f >> 2) * KPITCH + (f & 3) * 4
+    float* dst = KIN ? lds + (f >> 3) * KPITCH + (f & 7) * 4
                      : lds + (f / (ROWS / 4)) * ROWS + (f % (ROWS / 4)) * 4;
     *reinterpret_cast<f4*>(dst) = reg[j];
   }
 }
 
-// Fragment for MFMA steps s = 0..3 of k-group `kb` (0 or 8): frag[s] is the
+// Fragment for MFMA steps s = 0..3 of k-group `kb` (0, 8, 16 or 24): frag[s] is the
 // operand value for row/col (x0 + lane%32) at k = kb + 4*(lane/32) + s.
 template <bool KIN, int ROWS>
 __device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0, int kb, int lane,
@@ -124,8 +126,10 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   constexpr int BMt = 64 * TM, BNt = 64 * TN;
   constexpr int LFLOATS = LKIN ? BMt * KPITCH : BK * BMt;
   constexpr int RFLOATS = RKIN ? BNt * KPITCH : BK * BNt;
-  __shared__ __attribute__((aligned(16))) float ldsL[2][LFLOATS];
-  __shared__ __attribute__((aligned(16))) float ldsR[2][RFLOATS];
+  // two stages of both operand tiles: up to 73.7 KB, beyond the static limit
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  auto ldsL = [&](int stage) { return smem + stage * LFLOATS; };
+  auto ldsR = [&](int stage) { return smem + 2 * LFLOATS + stage * RFLOATS; };
 
   // Tile order: consecutive workgroups land on different XCDs (round robin),
   // so give each XCD a contiguous band of tiles, and walk a band column-major
@@ -166,12 +170,12 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  f4 regL[BMt / 64], regR[BNt / 64];
+  f4 regL[BMt / 32], regR[BNt / 32];
   const int64_t ksteps = (p.K + BK - 1) / BK;
   load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, 0, p.M, p.K, regL);
   load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, 0, p.N, p.K, regR);
-  store_tile<LKIN, BMt>(ldsL[0], regL);
-  store_tile<RKIN, BNt>(ldsR[0], regR);
+  store_tile<LKIN, BMt>(ldsL(0), regL);
+  store_tile<RKIN, BNt>(ldsR(0), regR);
   __syncthreads();
 
   for (int64_t ks = 0; ks < ksteps; ks++) {
@@ -184,9 +188,9 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
     for (int kb = 0; kb < BK; kb += 8) {
       float a[TM][4], b[TN][4];
 #pragma unroll
-      for (int i = 0; i < TM; i++) read_frag<LKIN, BMt>(ldsL[cur], wm + i * 32, kb, lane, a[i]);
+      for (int i = 0; i < TM; i++) read_frag<LKIN, BMt>(ldsL(cur), wm + i * 32, kb, lane, a[i]);
 #pragma unroll
-      for (int j = 0; j < TN; j++) read_frag<RKIN, BNt>(ldsR[cur], wn + j * 32, kb, lane, b[j]);
+      for (int j = 0; j < TN; j++) read_frag<RKIN, BNt>(ldsR(cur), wn + j * 32, kb, lane, b[j]);
 #pragma unroll
       for (int s = 0; s < 4; s++)
 #pragma unroll
@@ -198,8 +202,8 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
     if (ks + 1 < ksteps) {
       // The other buffer was last read in iteration ks-1, and every wave has
       // passed the barrier that ended it.
-      store_tile<LKIN, BMt>(ldsL[cur ^ 1], regL);
-      store_tile<RKIN, BNt>(ldsR[cur ^ 1], regR);
+      store_tile<LKIN, BMt>(ldsL(cur ^ 1), regL);
+      store_tile<RKIN, BNt>(ldsR(cur ^ 1), regR);
     }
     __syncthreads();
   }
@@ -229,25 +233,35 @@ static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; 
 static bool is_n(char c) { return c == 'N' || c == 'n'; }
 static bool is_t(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
+template <bool LK, bool RK, bool FAST, int TM, int TN>
+static int launch_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
+  constexpr int lfloats = LK ? 64 * TM * KPITCH : BK * 64 * TM;
+  constexpr int rfloats = RK ? 64 * TN * KPITCH : BK * 64 * TN;
+  constexpr size_t bytes = 2 * (size_t)(lfloats + rfloats) * sizeof(float);
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_kernel<LK, RK, FAST, TM, TN>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+                      "hipFuncSetAttribute(sgemm_kernel)"));
+    configured = true;
+  }
+  sgemm_kernel<LK, RK, FAST, TM, TN><<<grid, kBlock, bytes, st>>>(p);
+  return 0;
+}
+
 template <bool LK, bool RK, int TM, int TN>
-static void launch_variant(const GemmParams& p, bool fast, dim3 grid, hipStream_t st) {
-  if (fast)
-    sgemm_kernel<LK, RK, true, TM, TN><<<grid, kBlock, 0, st>>>(p);
-  else
-    sgemm_kernel<LK, RK, false, TM, TN><<<grid, kBlock, 0, st>>>(p);
+static int launch_variant(const GemmParams& p, bool fast, dim3 grid, hipStream_t st) {
+  if (fast) return launch_kernel<LK, RK, true, TM, TN>(p, grid, st);
+  return launch_kernel<LK, RK, false, TM, TN>(p, grid, st);
 }
 
 template <int TM, int TN>
-static void launch_layout(const GemmParams& p, bool lkin, bool rkin, bool fast, dim3 grid,
-                          hipStream_t st) {
-  if (lkin && rkin)
-    launch_variant<true, true, TM, TN>(p, fast, grid, st);
-  else if (lkin)
-    launch_variant<true, false, TM, TN>(p, fast, grid, st);
-  else if (rkin)
-    launch_variant<false, true, TM, TN>(p, fast, grid, st);
-  else
-    launch_variant<false, false, TM, TN>(p, fast, grid, st);
+static int launch_layout(const GemmParams& p, bool lkin, bool rkin, bool fast, dim3 grid,
+                         hipStream_t st) {
+  if (lkin && rkin) return launch_variant<true, true, TM, TN>(p, fast, grid, st);
+  if (lkin) return launch_variant<true, false, TM, TN>(p, fast, grid, st);
+  if (rkin) return launch_variant<false, true, TM, TN>(p, fast, grid, st);
+  return launch_variant<false, false, TM, TN>(p, fast, grid, st);
 }
 
 // Workgroups are spread evenly over the CUs, and the ones resident on a CU
@@ -305,15 +319,16 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   fast = fast && (lkin ? k % 4 == 0 : p.M % 4 == 0) && (rkin ? k % 4 == 0 : p.N % 4 == 0);
 
   // Tile choice: time ~ tiles on the busiest CU x work per tile.
-  // The narrow tile does 15 % less work per cycle (one operand is re-read from
+  // The narrow tile does 10 % less work per cycle (one operand is re-read from
   // LDS twice as often) but wastes nothing on N <= 64 and evens out the last
   // round.
   const int64_t nb = (int64_t)batch * batch2;
   const int64_t tiles_wide = ceil_div(p.M, 128) * ceil_div(p.N, 128) * nb;
   const int64_t tiles_narrow = ceil_div(p.M, 128) * ceil_div(p.N, 64) * nb;
   const double cost_wide = busiest_cu_tiles(tiles_wide) * 1.0;
-  const double cost_narrow = busiest_cu_tiles(tiles_narrow) * 0.5 / 0.85;
-  const bool narrow = cost_narrow < cost_wide;
+  const double cost_narrow = busiest_cu_tiles(tiles_narrow) * 0.5 / 0.9;
+  bool narrow = cost_narrow < cost_wide;
+  if (const char* force = getenv("WF2HIP_GEMM_TILE")) narrow = force[0] == 'n';  // tuning knob
   p.tiles_m = (uint32_t)ceil_div(p.M, 128);
   p.tiles_n = (uint32_t)ceil_div(p.N, narrow ? 64 : 128);
   const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
@@ -321,9 +336,9 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   dim3 grid((uint32_t)blocks, (uint32_t)nb);
   hipStream_t st = rt().stream;
   if (narrow)
-    launch_layout<2, 1>(p, lkin, rkin, fast, grid, st);
+    WF2_TRY((launch_layout<2, 1>(p, lkin, rkin, fast, grid, st)));
   else
-    launch_layout<2, 2>(p, lkin, rkin, fast, grid, st);
+    WF2_TRY((launch_layout<2, 2>(p, lkin, rkin, fast, grid, st)));
   return after_launch("sgemm_kernel");
 }
 
