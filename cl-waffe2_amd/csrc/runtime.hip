@@ -49,6 +49,17 @@ int require_init() {
 // runs on one stream, so a recycled block's new user is ordered after its old
 // one.  hipFree (which does synchronise) only happens on trim/shutdown or when
 // the device is out of memory.
+// A captured graph keeps the blocks its kernels were recorded with: blocks
+// freed while capturing are parked here (re-usable by later allocations of the
+// same capture, since a replay preserves the recorded order) and only return to
+// the pool when the graph is destroyed.
+struct Graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::multimap<size_t, void*> held;
+};
+static Graph* g_capture = nullptr;  // non-null between graph_begin and graph_end
+
 struct Pool {
   std::mutex mu;
   std::multimap<size_t, void*> idle;          // size class -> block
@@ -76,6 +87,14 @@ static void pool_release_idle_locked() {
 static int pool_alloc(void** ptr, size_t bytes) {
   const size_t cls = size_class(bytes);
   std::lock_guard<std::mutex> lock(g_pool.mu);
+  if (g_capture) {
+    auto held = g_capture->held.find(cls);
+    if (held != g_capture->held.end()) {
+      *ptr = held->second;
+      g_capture->held.erase(held);
+      return 0;
+    }
+  }
   if (g_pool.enabled) {
     auto it = g_pool.idle.find(cls);
     if (it != g_pool.idle.end()) {
@@ -84,6 +103,12 @@ static int pool_alloc(void** ptr, size_t bytes) {
       g_pool.idle_bytes -= cls;
       return 0;
     }
+  }
+  if (g_capture) {
+    *ptr = nullptr;
+    return fail(WF2HIP_ECAPTURE,
+                "a %zu-byte block is not in the pool and hipMalloc cannot run during graph "
+                "capture: run the sequence once before capturing it", bytes);
   }
   hipError_t e = hipMalloc(ptr, cls);
   if (e == hipErrorOutOfMemory && !g_pool.idle.empty()) {
@@ -107,6 +132,10 @@ static int pool_free(void* ptr) {
   auto it = g_pool.size_of.find(ptr);
   if (it == g_pool.size_of.end())
     return fail(WF2HIP_EINVAL, "wf2hip_free: %p was not allocated by wf2hip_malloc", ptr);
+  if (g_capture) {
+    g_capture->held.emplace(it->second, ptr);
+    return 0;
+  }
   if (g_pool.enabled) {
     g_pool.idle.emplace(it->second, ptr);
     g_pool.idle_bytes += it->second;
@@ -155,7 +184,12 @@ WF2_API int wf2hip_init(int device) {
   g_rt.total_mem = prop.totalGlobalMem;
   snprintf(g_rt.name, sizeof g_rt.name, "%s", prop.name);
   snprintf(g_rt.arch, sizeof g_rt.arch, "%s", prop.gcnArchName);
-  g_rt.stream = nullptr;
+  // The library's own stream (default priority).  A real stream rather than
+  // the null stream so that it can be captured into a graph.
+  if (!g_rt.own_stream)
+    WF2_TRY(check_hip(hipStreamCreateWithFlags(&g_rt.own_stream, hipStreamNonBlocking),
+                      "hipStreamCreateWithFlags"));
+  g_rt.stream = g_rt.own_stream;
   g_rt.initialised = true;
   const char* pool_env = getenv("WF2HIP_POOL");
   g_pool.enabled = !(pool_env && pool_env[0] == '0');
@@ -171,6 +205,7 @@ WF2_API int wf2hip_shutdown(void) {
     pool_release_idle_locked();
   }
   if (g_rt.partials) (void)hipFree(g_rt.partials);
+  if (g_rt.own_stream) (void)hipStreamDestroy(g_rt.own_stream);
   g_rt = Runtime();
   return 0;
 }
@@ -224,6 +259,7 @@ WF2_API int wf2hip_free(void* ptr) {
 
 WF2_API int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
   WF2_TRY(require_init());
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "host transfers block and cannot be captured");
   if (bytes == 0) return 0;
   if (!dst || !src) return fail(WF2HIP_EINVAL, "null pointer");
   WF2_TRY(check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_rt.stream),
@@ -234,6 +270,7 @@ WF2_API int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
 
 WF2_API int wf2hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
   WF2_TRY(require_init());
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "host transfers block and cannot be captured");
   if (bytes == 0) return 0;
   if (!dst || !src) return fail(WF2HIP_EINVAL, "null pointer");
   WF2_TRY(check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_rt.stream),
@@ -261,14 +298,16 @@ WF2_API int wf2hip_fill_f32(float* x, size_t n, float value) {
 
 WF2_API int wf2hip_sync(void) {
   WF2_TRY(require_init());
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "cannot synchronise during graph capture");
   return check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize");
 }
 
 WF2_API int wf2hip_set_stream(void* hip_stream) {
   WF2_TRY(require_init());
   // recycled blocks rely on single-stream ordering: drain the old stream first
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "cannot change the stream during graph capture");
   WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
-  g_rt.stream = (hipStream_t)hip_stream;
+  g_rt.stream = hip_stream ? (hipStream_t)hip_stream : g_rt.own_stream;
   return 0;
 }
 
@@ -308,3 +347,76 @@ WF2_API int wf2hip_set_reduce_mode(int mode) {
 }
 
 WF2_API int wf2hip_get_reduce_mode(void) { return g_rt.reduce_mode; }
+
+// ---- graph capture ------------------------------------------------------------
+// cl-waffe2 compiles a model into an instruction sequence once and replays it on
+// every forward (source/vm/generic-tensor/acceptor.lisp:409-508, vm.lisp:260).
+// The device-side analogue: record the kernel sequence of one forward on the
+// library's stream into a HIP graph and replay it with a single launch, which
+// removes the per-node host cost.  Zero fills are fill kernels, never memset
+// nodes, so everything the library enqueues is a kernel or a copy node.
+
+WF2_API int wf2hip_graph_begin(void) {
+  WF2_TRY(require_init());
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "a capture is already in progress");
+  if (g_rt.stream == nullptr)
+    return fail(WF2HIP_ECAPTURE, "the null stream cannot be captured; use the library's own stream");
+  Graph* g = new Graph();
+  int rc = check_hip(hipStreamBeginCapture(g_rt.stream, hipStreamCaptureModeThreadLocal),
+                     "hipStreamBeginCapture");
+  if (rc != 0) {
+    delete g;
+    return rc;
+  }
+  g_capture = g;
+  return 0;
+}
+
+WF2_API int wf2hip_graph_end(void** graph) {
+  WF2_TRY(require_init());
+  if (!graph) return fail(WF2HIP_EINVAL, "null result pointer");
+  *graph = nullptr;
+  Graph* g;
+  {
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    g = g_capture;
+    g_capture = nullptr;
+  }
+  if (!g) return fail(WF2HIP_ECAPTURE, "no capture in progress");
+  int rc = check_hip(hipStreamEndCapture(g_rt.stream, &g->graph), "hipStreamEndCapture");
+  if (rc == 0) rc = check_hip(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0),
+                              "hipGraphInstantiate");
+  if (rc != 0) {
+    wf2hip_graph_destroy(g);
+    return rc;
+  }
+  *graph = g;
+  return 0;
+}
+
+WF2_API int wf2hip_graph_launch(void* graph) {
+  WF2_TRY(require_init());
+  Graph* g = (Graph*)graph;
+  if (!g || !g->exec) return fail(WF2HIP_EINVAL, "not an instantiated graph");
+  if (g_capture) return fail(WF2HIP_ECAPTURE, "cannot launch a graph while capturing");
+  return check_hip(hipGraphLaunch(g->exec, g_rt.stream), "hipGraphLaunch");
+}
+
+WF2_API int wf2hip_graph_destroy(void* graph) {
+  Graph* g = (Graph*)graph;
+  if (!g) return 0;
+  // replays still in flight read and write the held blocks
+  if (g_rt.initialised) (void)hipStreamSynchronize(g_rt.stream);
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  if (g->graph) (void)hipGraphDestroy(g->graph);
+  {
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    for (auto& kv : g->held) {
+      g_pool.idle.emplace(kv.first, kv.second);
+      g_pool.idle_bytes += kv.first;
+    }
+  }
+  delete g;
+  return 0;
+}

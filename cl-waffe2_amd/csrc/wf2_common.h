@@ -21,7 +21,8 @@ struct Runtime {
   bool initialised = false;
   int device = -1;
   int num_cus = 0;
-  hipStream_t stream = nullptr;
+  hipStream_t stream = nullptr;      // where every kernel and copy is enqueued
+  hipStream_t own_stream = nullptr;  // created by wf2hip_init, the default
   int reduce_mode = 0;
   float* partials = nullptr;  // kPartialCapacity floats, owned by the library
   char name[128] = {0};

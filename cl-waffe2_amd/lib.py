@@ -22,6 +22,7 @@ SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
 POW, GELU = 32, 40
 
 EOVERLAP = -3
+ECAPTURE = -6
 
 
 class HIPExtensionMissing(RuntimeError):
@@ -76,6 +77,10 @@ _SIGNATURES = {
     "wf2hip_event_record": ([_P], C.c_int),
     "wf2hip_event_elapsed_ms": ([_P, _P, C.POINTER(_F)], C.c_int),
     "wf2hip_event_destroy": ([_P], C.c_int),
+    "wf2hip_graph_begin": ([], C.c_int),
+    "wf2hip_graph_end": ([C.POINTER(_P)], C.c_int),
+    "wf2hip_graph_launch": ([_P], C.c_int),
+    "wf2hip_graph_destroy": ([_P], C.c_int),
     "wf2hip_sadd": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_ssub": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_smul": ([_L, _P, _L, _P, _L], C.c_int),
@@ -192,5 +197,44 @@ class Event:
         try:
             if self._h and _lib is not None:
                 _lib.wf2hip_event_destroy(self._h)
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded kernel sequence (``wf2hip_graph_*``).
+
+        run()                       # once, so that the pool holds the temporaries
+        with Graph() as g:          # record
+            out = run()
+        g.launch()                  # replay: one launch, no per-node host cost
+
+    Keep the tensors the replay reads or writes (inputs, ``out``) alive while the
+    graph is in use."""
+
+    def __init__(self):
+        self._h = _P()
+
+    def __enter__(self) -> "Graph":
+        check(get().wf2hip_graph_begin())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        code = get().wf2hip_graph_end(C.byref(self._h))
+        if exc_type is None:
+            check(code)
+        return False
+
+    def launch(self) -> None:
+        check(get().wf2hip_graph_launch(self._h))
+
+    def destroy(self) -> None:
+        if self._h and _lib is not None:
+            _lib.wf2hip_graph_destroy(self._h)
+            self._h = _P()
+
+    def __del__(self):
+        try:
+            self.destroy()
         except Exception:
             pass

@@ -15,8 +15,8 @@
  *   - Every function returns 0 on success or a negative WF2HIP_E* code / a
  *     positive hipError_t; wf2hip_last_error() returns a thread-local message.
  *     (The reference's kernels return void and have no error channel.)
- *   - Kernels are enqueued on one stream (wf2hip_set_stream, default: the null
- *     stream) and return without waiting; wf2hip_memcpy_d2h, wf2hip_sync and
+ *   - Kernels are enqueued on one stream (created by wf2hip_init; another one
+ *     can be adopted with wf2hip_set_stream) and return without waiting; wf2hip_memcpy_d2h, wf2hip_sync and
  *     wf2hip_event_elapsed_ms block.
  *   - The library keeps no pointer after a call returns and never frees or
  *     reallocates a caller's buffer.
@@ -41,6 +41,7 @@ extern "C" {
 #define WF2HIP_EOVERLAP (-3)   /* in-place op on partially overlapping views     */
 #define WF2HIP_EUNSUPPORTED (-4)
 #define WF2HIP_ENOMEM (-5)
+#define WF2HIP_ECAPTURE (-6)   /* not possible during / outside a graph capture    */
 
 /* ---- runtime ----------------------------------------------------------- */
 /* No counterpart in cl-waffe2-simd (host memory needs none); the loader
@@ -74,7 +75,7 @@ int wf2hip_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int wf2hip_memcpy_d2d(void* dst, const void* src, size_t bytes);
 int wf2hip_fill_f32(float* x, size_t n, float value);
 int wf2hip_sync(void);
-/* Adopt an externally created hipStream_t (NULL = the null stream). */
+/* Adopt an externally created hipStream_t (NULL = back to the library's own). */
 int wf2hip_set_stream(void* hip_stream);
 void* wf2hip_get_stream(void);
 /* Events on the library's stream, for timing kernels where they run. */
@@ -82,6 +83,21 @@ int wf2hip_event_create(void** event);
 int wf2hip_event_record(void* event);
 int wf2hip_event_elapsed_ms(void* start, void* stop, float* ms);
 int wf2hip_event_destroy(void* event);
+
+/* ---- graph capture ------------------------------------------------------- */
+/* Record everything enqueued between begin and end into a HIP graph and replay
+ * it with one launch: the device-side counterpart of cl-waffe2 compiling a
+ * model once and re-running its instruction sequence on every forward
+ * (source/vm/generic-tensor/acceptor.lisp:409-508, source/vm/vm.lisp:260).
+ * Rules: run the sequence once before capturing (allocations during capture
+ * are served from the pool only: WF2HIP_ECAPTURE otherwise); host transfers and
+ * wf2hip_sync are refused while capturing; tensors the replay reads or writes
+ * (inputs, outputs) must stay allocated for as long as the graph is used; new
+ * inputs are written into the same buffers. */
+int wf2hip_graph_begin(void);
+int wf2hip_graph_end(void** graph);
+int wf2hip_graph_launch(void* graph);
+int wf2hip_graph_destroy(void* graph);
 
 /* ---- BLAS-like 1-D kernels (one-for-one with waffe2_s*) ---------------- */
 /* x[i*incx] <- x[i*incx] op y[i*incy], i < n.

@@ -1,0 +1,69 @@
+"""Graph capture and replay of a node sequence (wf2hip_graph_*).
+
+A replay must reproduce the eager result bit for bit on every launch, with the
+program's own eager work and synchronisations between the replays, and must
+follow new contents written into the captured input buffer."""
+import importlib
+
+import numpy as np
+import pytest
+
+from helpers import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(batch=2, seq=40, d_model=64, n_head=2, head_dim=32, d_ff=96, eps=1e-5)
+
+
+@pytest.mark.parametrize("mode", ["nodes", "fused"])
+def test_block_forward_replay(gpu, mode):
+    W = gpu
+    F = W.functional
+    gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
+    params = gpt2.to_device(gpt2.make_block_params(3, CFG))
+    x_host = gpt2.make_block_input(3, CFG)
+    x = F.from_numpy(x_host)
+    mask = gpt2.causal_mask(CFG["seq"])
+
+    def run():
+        return gpt2.block_forward(x, params, mode=mode, cfg=CFG, mask=mask)
+
+    eager = run().numpy()            # also warms the pool with every temporary
+    with W.lib.Graph() as g:
+        out = run()
+    for i in range(3):
+        g.launch()
+        assert_bit_equal(out.numpy(), eager, f"replay {i}")
+        # eager work between replays, recycling pool blocks
+        junk = F.exp(F.from_numpy(np.full((64, 64), float(i), np.float32)))
+        assert junk.numpy()[0, 0] == np.float32(np.exp(np.float64(i)))
+        W.lib.synchronize()
+    # new contents in the same input buffer
+    x2 = (x_host * np.float32(0.5) + np.float32(0.25)).astype(np.float32)
+    F.move_(x, F.from_numpy(x2))
+    g.launch()
+    replayed = out.numpy()
+    want = run().numpy()
+    assert_bit_equal(replayed, want, "replay on new input")
+    assert not np.array_equal(replayed, eager)
+    g.destroy()
+
+
+def test_capture_rules(gpu):
+    W = gpu
+    F = W.functional
+    a = F.from_numpy(np.ones((33, 77), np.float32))
+    with pytest.raises(W.HIPError) as e:
+        with W.lib.Graph():
+            F.exp(W.HIPTensor([12345, 7]))  # a size the pool has never seen: would need hipMalloc
+    assert e.value.code == W.lib.ECAPTURE
+    with pytest.raises(W.HIPError) as e:
+        with W.lib.Graph():
+            a.numpy()                        # a blocking host transfer
+    assert e.value.code == W.lib.ECAPTURE
+    lib = W.lib.get()
+    import ctypes as C
+    h = C.c_void_p()
+    assert lib.wf2hip_graph_end(C.byref(h)) == W.lib.ECAPTURE   # nothing to end
+    # the library still works afterwards
+    assert F.add(a, a).numpy()[0, 0] == 2.0
