@@ -31,6 +31,7 @@
 #include <stdlib.h>
 
 #include "wf2_common.h"
+#include "wf2_math.h"
 
 namespace wf2 {
 
@@ -51,6 +52,15 @@ struct GemmParams {
   uint32_t batch_inner;   // blockIdx.y = outer * batch_inner + inner
   float alpha, beta;
   uint32_t tiles_m, tiles_n;
+  // fused epilogue (row-major terms): C = act(alpha acc + bias[col]) + residual
+  const float* bias;       // N floats or null
+  const float* residual;   // laid out like C (own pitch and batch strides) or null
+  int64_t ldres, sRes, sRes2;
+  int32_t activation;      // 0 none, 1 tanh-form GELU
+  // 1: only tiles that touch the lower triangle (col <= row) are computed;
+  // 2: the left operand is lower-triangular (L[i][l] = 0 for l > i), so the
+  //    K loop of a row tile stops at its last row
+  int32_t causal;
 };
 
 // Loads this thread's share of a ROWS x BK operand tile into registers
@@ -151,6 +161,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 
   const int64_t m0 = (int64_t)tm * BMt;
   const int64_t n0 = (int64_t)tn * BNt;
+  if (p.causal == 1 && n0 > m0 + BMt - 1) return;  // tile wholly above the diagonal
   const uint32_t zo = blockIdx.y / p.batch_inner;
   const uint32_t zi = blockIdx.y - zo * p.batch_inner;
   const float* L = p.L + (int64_t)zo * p.sL2 + (int64_t)zi * p.sL;
@@ -171,7 +182,9 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
   f4 regL[BMt / 32], regR[BNt / 32];
-  const int64_t ksteps = (p.K + BK - 1) / BK;
+  int64_t klimit = p.K;
+  if (p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
+  const int64_t ksteps = (klimit + BK - 1) / BK;
   load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, 0, p.M, p.K, regL);
   load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, 0, p.N, p.K, regR);
   store_tile<LKIN, BMt>(ldsL(0), regL);
@@ -222,6 +235,10 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
           float* c = C + row * p.ldc + col;
           float v = p.alpha * acc[i][j][r];
           if (p.beta != 0.0f) v += p.beta * *c;
+          if (p.bias) v += p.bias[col];
+          if (p.activation == 1) v = gelu_tanh_f(v);
+          if (p.residual)
+            v += p.residual[(int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes + row * p.ldres + col];
           *c = v;
         }
       }
@@ -272,10 +289,18 @@ static double busiest_cu_tiles(int64_t tiles) {
   return (double)((tiles + cus - 1) / cus);
 }
 
+struct Epilogue {
+  const float* bias = nullptr;
+  const float* residual = nullptr;
+  int64_t ldres = 0, sRes = 0, sRes2 = 0;
+  int activation = 0;
+  int causal = 0;
+};
+
 int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha, const float* A,
                    long lda, long strideA, long strideA2, const float* B, long ldb, long strideB,
                    long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
-                   long batch, long batch2) {
+                   long batch, long batch2, const Epilogue& ep = Epilogue()) {
   if (!(is_n(transa) || is_t(transa)) || !(is_n(transb) || is_t(transb)))
     return fail(WF2HIP_EINVAL, "trans must be N, T or C");
   if (m < 0 || n < 0 || k < 0 || batch < 0 || batch2 < 0)
@@ -311,6 +336,13 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   p.batch_inner = (uint32_t)batch;
   p.alpha = alpha;
   p.beta = beta;
+  p.bias = ep.bias;
+  p.residual = ep.residual;
+  p.ldres = ep.ldres;
+  p.sRes = ep.sRes;
+  p.sRes2 = ep.sRes2;
+  p.activation = ep.activation;
+  p.causal = ep.causal;
   const bool lkin = is_n(transb);   // left stored [rows][k]
   const bool rkin = !is_n(transa);  // right stored [cols][k]
   bool fast = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && strideA % 4 == 0 &&
@@ -371,4 +403,31 @@ WF2_API int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, lo
   WF2_TRY(require_init());
   return sgemm_batched2(transa, transb, m, n, k, alpha, A, lda, strideA, strideA2, B, ldb, strideB,
                         strideB2, beta, C, ldc, strideC, strideC2, batch, batch2);
+}
+
+// Row-major C[m,n] = act(alpha A.B + bias) + residual: the operand swap of
+// expand-gemm-form-column done here, so that bias is per output column.
+WF2_API int wf2hip_matmul_fused(const wf2hip_matmul_desc* d, const float* A, const float* B,
+                                float* C) {
+  WF2_TRY(require_init());
+  if (!d) return fail(WF2HIP_EINVAL, "null descriptor");
+  if (d->activation < 0 || d->activation > 1) return fail(WF2HIP_EINVAL, "unknown activation");
+  if (d->causal < 0 || d->causal > 2) return fail(WF2HIP_EINVAL, "unknown causal mode");
+  if (d->causal == 1 && d->m != d->n)
+    return fail(WF2HIP_EINVAL, "lower-triangular output needs a square product");
+  if (d->causal == 2 && d->m != d->k)
+    return fail(WF2HIP_EINVAL, "a lower-triangular left operand must be square");
+  if (d->residual && d->ld_residual < d->n)
+    return fail(WF2HIP_EINVAL, "residual pitch smaller than the row");
+  Epilogue ep;
+  ep.bias = d->bias;
+  ep.residual = d->residual;
+  ep.ldres = d->ld_residual;
+  ep.sRes = d->stride_residual;
+  ep.sRes2 = d->stride_residual2;
+  ep.activation = d->activation;
+  ep.causal = d->causal;
+  return sgemm_batched2(d->trans_b ? 'C' : 'N', d->trans_a ? 'C' : 'N', d->n, d->m, d->k, d->alpha,
+                        B, d->ldb, d->stride_b, d->stride_b2, A, d->lda, d->stride_a, d->stride_a2,
+                        0.0f, C, d->ldc, d->stride_c, d->stride_c2, d->batch, d->batch2, ep);
 }

@@ -297,11 +297,18 @@ def mean(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool =
 # matmul
 # ---------------------------------------------------------------------------
 
-def matmul(a, b, out: HIPTensor | None = None) -> HIPTensor:
+def matmul(a, b, out: HIPTensor | None = None, bias: HIPTensor | None = None,
+           residual: HIPTensor | None = None, activation: str | None = None,
+           causal: int = 0) -> HIPTensor:
     """``(!matmul a b)`` (``base-impl/matrix-ops.lisp:80-173``): ``!t`` operands
     become transpose flags, any other non-trivial layout of the last two axes is
     materialised with ``->contiguous``, a lower-rank operand is broadcast over
-    the batch axes, and the output is a fresh ``(~ i k)`` tensor."""
+    the batch axes, and the output is a fresh ``(~ i k)`` tensor.
+
+    The keyword options fuse what would otherwise be separate nodes into the
+    product's epilogue: ``act(a @ b + bias) + residual`` (``activation='gelu'``),
+    ``causal=1`` when only the lower triangle of a square product is needed,
+    ``causal=2`` when ``a`` is lower-triangular."""
     trans_a = isinstance(a, Transposed)
     trans_b = isinstance(b, Transposed)
     at = a.tensor if trans_a else a
@@ -325,7 +332,8 @@ def matmul(a, b, out: HIPTensor | None = None) -> HIPTensor:
         return flexible(x, _ShapeOnly(list(batch) + x.shape[-2:]))
 
     return nodes.forward("MatMulNode", with_batch(at), with_batch(bt), out,
-                         trans_a=trans_a, trans_b=trans_b)
+                         trans_a=trans_a, trans_b=trans_b, bias=bias, residual=residual,
+                         activation=activation, causal=causal)
 
 
 class _ShapeOnly:

@@ -15,8 +15,9 @@ Two modes:
            LayerNorm and GELU node for node, heads materialised with
            MoveTensorNode copies of sliced/permuted views, scaling and masking
            as MulNode / AddNode with broadcast operands, row softmax kernel.
-``fused``  the same mathematics with the fused row kernels (LayerNorm, GELU,
-           scale+mask+softmax) and zero-copy heads: the attention gemms read
+``fused``  the same mathematics with the fused row kernels (LayerNorm,
+           scale+mask+softmax), bias / GELU / residual in the gemm epilogues,
+           causal tile skipping in both attention products, and zero-copy heads: the attention gemms read
            q/k/v straight out of the (B, T, 3, H, hd) projection through
            strides and write the context straight into (B, T, H*hd).
 """
@@ -85,18 +86,21 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
     act = F.gelu_fused if fused else F.gelu
 
     h = ln(x, p["ln1_g"], p["ln1_b"], eps)
-    qkv = _linear(h, p["w_qkv"], p["b_qkv"])                       # (B, T, 3D)
+    if fused:
+        qkv = F.matmul(h, p["w_qkv"], bias=p["b_qkv"])             # (B, T, 3D)
+    else:
+        qkv = _linear(h, p["w_qkv"], p["b_qkv"])
 
     if fused:
         five = F.reshape(qkv, B, T, 3, H, hd)
         # (B, 1, H, T, hd) strided windows of the projection, no copy
         q, k, v = (five.view(True, True, i, True, True).permute(0, 2, 3, 1, 4) for i in range(3))
-        scores = F.matmul(q, F.t(k))                                # (B, 1, H, T, T)
+        scores = F.matmul(q, F.t(k), causal=1)                      # (B, 1, H, T, T), lower triangle
         probs = HIPTensor(scores.shape, initial_element=None)
         _lib.check(_lib.get().wf2hip_causal_softmax_f32(B * H, T, C.c_void_p(scores.ptr),
                                                        C.c_void_p(probs.ptr), scale))
         ctx_store = HIPTensor([B, T, 1, H, hd], initial_element=None)
-        F.matmul(probs, v, out=ctx_store.permute(0, 2, 3, 1, 4))    # written as (B, T, H*hd)
+        F.matmul(probs, v, out=ctx_store.permute(0, 2, 3, 1, 4), causal=2)  # written as (B, T, H*hd)
         ctx = F.reshape(ctx_store, B, T, D)
     else:
         def heads(i):  # split-heads: slice, reshape, permute, materialise
@@ -111,6 +115,12 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         ctx = F.matmul(probs, v)                                    # (B, H, T, hd)
         ctx = F.reshape(ctx.permute(0, 2, 1, 3), B, T, D)           # merge-heads (copies)
 
+    if fused:
+        # bias, GELU and the residual adds ride in the products' epilogues
+        x1 = F.matmul(ctx, p["w_o"], bias=p["b_o"], residual=x)
+        h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)
+        f = F.matmul(h2, p["w_fc"], bias=p["b_fc"], activation="gelu")
+        return F.matmul(f, p["w_proj"], bias=p["b_proj"], residual=x1)
     attn = _linear(ctx, p["w_o"], p["b_o"])
     x1 = F.add(x, attn)                                             # residual
     h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)

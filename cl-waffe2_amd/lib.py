@@ -55,6 +55,23 @@ _P = C.c_void_p
 _L = C.c_long
 _F = C.c_float
 
+
+class MatmulDesc(C.Structure):
+    """``struct wf2hip_matmul_desc``"""
+
+    _fields_ = [
+        ("trans_a", C.c_int32), ("trans_b", C.c_int32), ("activation", C.c_int32), ("causal", C.c_int32),
+        ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64),
+        ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
+        ("batch", C.c_int64), ("batch2", C.c_int64),
+        ("stride_a", C.c_int64), ("stride_a2", C.c_int64), ("stride_b", C.c_int64),
+        ("stride_b2", C.c_int64), ("stride_c", C.c_int64), ("stride_c2", C.c_int64),
+        ("bias", C.c_void_p), ("residual", C.c_void_p),
+        ("ld_residual", C.c_int64), ("stride_residual", C.c_int64), ("stride_residual2", C.c_int64),
+        ("alpha", C.c_float), ("reserved", C.c_int32),
+    ]
+
+
 _SIGNATURES = {
     "wf2hip_abi_version": ([], C.c_int),
     "wf2hip_init": ([C.c_int], C.c_int),
@@ -109,6 +126,7 @@ _SIGNATURES = {
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _P, _L, _L, _F, _P, _L, _L, _L],
         C.c_int,
     ),
+    "wf2hip_matmul_fused": ([C.POINTER(MatmulDesc), _P, _P, _P], C.c_int),
     "wf2hip_sgemm_strided_batched_2d": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],
         C.c_int,

@@ -20,6 +20,7 @@ host loops around 1-D kernels (``source/backends/cpu/arithmetic.lisp:32-144``,
 from __future__ import annotations
 
 import ctypes as C
+import itertools
 from contextlib import contextmanager
 
 from . import lib as _lib
@@ -159,12 +160,18 @@ def _matrix_geometry(t: HIPTensor, what: str):
 
 @define_impl("MatMulNode", HIPTensor, _only_float)
 def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
-            trans_b: bool = False) -> HIPTensor:
+            trans_b: bool = False, bias: HIPTensor | None = None,
+            residual: HIPTensor | None = None, activation: str | None = None,
+            causal: int = 0) -> HIPTensor:
     """``C[~ i k] = A[~ i j] . B[~ j k]`` through the operand-swapped
     column-major call of ``expand-gemm-form-column``
     (``backends/cpu/matrix-ops.lisp:12-112``): sgemm(transB, transA, n, m, k, 1,
     B, ldb, A, lda, 0, C, ldc).  ``a``/``b`` are the tensors as stored (i.e.
-    untransposed); batch axes may be broadcast (stride 0) on either operand."""
+    untransposed); batch axes may be broadcast (stride 0) on either operand.
+
+    ``bias`` / ``activation`` / ``residual`` / ``causal`` select the fused
+    epilogue of ``wf2hip_matmul_fused`` (not part of MatMulNode: what a
+    ``define-bypass`` fusion of MatMulNode + AddNode (+ !gelu) would call)."""
     sa, sta, oa, lda = _matrix_geometry(a, "A")
     sb, stb, ob, ldb = _matrix_geometry(b, "B")
     sc, stc, oc, ldc = _matrix_geometry(out, "C")
@@ -177,17 +184,49 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     batch_shape = sc[:-2]
     if sa[:-2] != batch_shape or sb[:-2] != batch_shape:
         raise ValueError("MatMulNode: batch axes differ; view the smaller operand with (:broadcast n)")
+    fused = bias is not None or residual is not None or activation is not None or causal
+    tensors = [sta, stb, stc]
+    ores = ldres = 0
+    if residual is not None:
+        sr, strd, ores, ldres = _matrix_geometry(residual, "residual")
+        if sr != sc:
+            raise ValueError(f"residual shape {sr} differs from the product's {sc}")
+        tensors.append(strd)
+    if bias is not None and (bias.shape != [n] or not bias.is_contiguous()):
+        raise ValueError(f"bias must be a contiguous vector of {n} elements")
+    if activation not in (None, "gelu"):
+        raise ValueError("activation must be None or 'gelu'")
     lib = _lib.get()
     ta = b"C" if trans_a else b"N"
     tb = b"C" if trans_b else b"N"
 
-    def launch(offa, offb, offc, inner, outer):
+    def launch(offs, inner, outer):
         (count, s3), (count2, s3o) = inner, outer
-        _lib.check(lib.wf2hip_sgemm_strided_batched_2d(
-            tb, ta, n, m, k, 1.0,
-            C.c_void_p(b.ptr + 4 * offb), ldb, s3[1], s3o[1],
-            C.c_void_p(a.ptr + 4 * offa), lda, s3[0], s3o[0],
-            0.0, C.c_void_p(out.ptr + 4 * offc), ldc, s3[2], s3o[2], count, count2))
+        if not fused:
+            _lib.check(lib.wf2hip_sgemm_strided_batched_2d(
+                tb, ta, n, m, k, 1.0,
+                C.c_void_p(b.ptr + 4 * offs[1]), ldb, s3[1], s3o[1],
+                C.c_void_p(a.ptr + 4 * offs[0]), lda, s3[0], s3o[0],
+                0.0, C.c_void_p(out.ptr + 4 * offs[2]), ldc, s3[2], s3o[2], count, count2))
+            return
+        d = _lib.MatmulDesc()
+        d.trans_a, d.trans_b = int(trans_a), int(trans_b)
+        d.activation = 1 if activation == "gelu" else 0
+        d.causal = int(causal)
+        d.m, d.n, d.k = m, n, k
+        d.lda, d.ldb, d.ldc = lda, ldb, ldc
+        d.batch, d.batch2 = count, count2
+        d.stride_a, d.stride_a2 = s3[0], s3o[0]
+        d.stride_b, d.stride_b2 = s3[1], s3o[1]
+        d.stride_c, d.stride_c2 = s3[2], s3o[2]
+        d.bias = bias.ptr if bias is not None else None
+        if residual is not None:
+            d.residual = residual.ptr + 4 * offs[3]
+            d.ld_residual, d.stride_residual, d.stride_residual2 = ldres, s3[3], s3o[3]
+        d.alpha = 1.0
+        _lib.check(lib.wf2hip_matmul_fused(C.byref(d), C.c_void_p(a.ptr + 4 * offs[0]),
+                                           C.c_void_p(b.ptr + 4 * offs[1]),
+                                           C.c_void_p(out.ptr + 4 * offs[2])))
 
     # Fold the batch axes, innermost first, into at most two strided axes per
     # launch (the library takes two batch levels); anything beyond that is
@@ -195,22 +234,23 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     # Extent-1 axes carry no information.
     keep = [i for i, n_ in enumerate(batch_shape) if n_ != 1]
     batch_shape = [batch_shape[i] for i in keep]
-    sta, stb, stc = ([st[i] for i in keep] for st in (sta, stb, stc))
+    tensors = [[st[i] for i in keep] for st in tensors]
+    start = [oa, ob, oc] + ([ores] if residual is not None else [])
 
     def fold(last):
-        """Merge axes last, last-1, ... while they form one strided run for all
-        three tensors (0 == 0 x count holds for a broadcast operand)."""
+        """Merge axes last, last-1, ... while they form one strided run for
+        every tensor (0 == 0 x count holds for a broadcast operand)."""
         count = batch_shape[last]
-        s3 = [sta[last], stb[last], stc[last]]
+        s3 = [st[last] for st in tensors]
         first = last
-        while first > 0 and all(st[first - 1] == s * count for st, s in zip((sta, stb, stc), s3)):
+        while first > 0 and all(st[first - 1] == s * count for st, s in zip(tensors, s3)):
             first -= 1
             count *= batch_shape[first]
         return first, (count, s3)
 
-    none = (1, [0, 0, 0])
+    none = (1, [0] * len(tensors))
     if not batch_shape:
-        launch(oa, ob, oc, none, none)
+        launch(start, none, none)
         return out
     first, inner = fold(len(batch_shape) - 1)
     outer = none
@@ -220,12 +260,10 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
         raise ValueError("MatMulNode: more than 65535 matrices in one launch")
     outer_shape = batch_shape[:first]
 
-    def rec(axis, offa, offb, offc):
-        if axis == len(outer_shape):
-            launch(offa, offb, offc, inner, outer)
-            return
-        for i in range(outer_shape[axis]):
-            rec(axis + 1, offa + i * sta[axis], offb + i * stb[axis], offc + i * stc[axis])
-
-    rec(0, oa, ob, oc)
+    # (an explicit product instead of a recursive closure: a function that
+    # refers to itself is a reference cycle, which would keep the operands --
+    # and their device memory -- alive until the cyclic collector runs)
+    for index in itertools.product(*[range(n_) for n_ in outer_shape]):
+        launch([o + sum(i * st[ax] for ax, i in enumerate(index)) for o, st in zip(start, tensors)],
+               inner, outer)
     return out

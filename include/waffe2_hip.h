@@ -234,6 +234,35 @@ int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, long n, lo
                                     long strideB2, float beta, float* C, long ldc, long strideC,
                                     long strideC2, long batch, long batch2);
 
+/* ---- fused matmul (extension; no BLAS counterpart) ------------------------- */
+/* Row-major C[m,n] = act(alpha * op(A)[m,k] . op(B)[k,n] + bias[n]) + residual[m,n]
+ * in one kernel: the bias add, GELU and residual add that cl-waffe2 runs as
+ * separate AddNode / !gelu passes after MatMulNode (examples/gpt-2/model.lisp:
+ * 109-137), applied in the same order and the same binary32 arithmetic, so the
+ * result is bit-identical to the unfused sequence.  The route for it on the
+ * Lisp side is define-bypass (source/vm/nodes/symbolic.lisp:118-131).
+ * causal 1: only entries with col <= row are needed (attention scores before a
+ * causal softmax): tiles wholly above the diagonal are neither computed nor
+ * written.  causal 2: op(A) is lower-triangular (causal attention
+ * probabilities): the K loop of each row tile stops at its last row.
+ * Leading dimensions are row pitches; stride_*2 belong to the outer batch axis. */
+typedef struct wf2hip_matmul_desc {
+  int32_t trans_a;    /* A stored [k][m] */
+  int32_t trans_b;    /* B stored [n][k] */
+  int32_t activation; /* 0 none, 1 tanh-form GELU (nn/activation.lisp:45-66) */
+  int32_t causal;     /* 0, 1 or 2, see above */
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc;
+  int64_t batch, batch2;
+  int64_t stride_a, stride_a2, stride_b, stride_b2, stride_c, stride_c2;
+  const float* bias;     /* n floats or NULL */
+  const float* residual; /* [m][ld_residual] per matrix or NULL */
+  int64_t ld_residual, stride_residual, stride_residual2;
+  float alpha;
+  int32_t reserved;
+} wf2hip_matmul_desc;
+int wf2hip_matmul_fused(const wf2hip_matmul_desc* desc, const float* A, const float* B, float* C);
+
 #ifdef __cplusplus
 }
 #endif

@@ -320,3 +320,47 @@ def test_matmul_batched_and_broadcast(gpu):
         for h in range(3):
             M = qkv[b, :, 0, h, :].astype(np.float64)
             _gemm_check(got[b, h], M, M.T)
+
+
+def test_matmul_fused_epilogue_is_bit_identical_to_the_node_sequence(gpu):
+    """act(a @ w + bias) + residual in the gemm epilogue against MatMulNode,
+    AddNode, fused GELU kernel, AddNode run one after the other."""
+    F = gpu.functional
+    rng = np.random.default_rng(51)
+    for shape_a, n in [((3, 70, 48), 100), ((130, 64), 256), ((2, 2, 33, 20), 7)]:
+        a = rng.standard_normal(shape_a).astype(np.float32)
+        w = (rng.standard_normal((shape_a[-1], n)) * 0.2).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        res = rng.standard_normal(shape_a[:-1] + (n,)).astype(np.float32)
+        da, dw, db, dr = (F.from_numpy(v) for v in (a, w, bias, res))
+        plain = F.add_(F.matmul(da, dw), db)
+        assert_bit_equal(F.matmul(da, dw, bias=db).numpy(), plain.numpy(), "bias")
+        act = F.gelu_fused(plain)
+        assert_bit_equal(F.matmul(da, dw, bias=db, activation="gelu").numpy(), act.numpy(), "bias+gelu")
+        want = F.add(plain, dr)
+        assert_bit_equal(F.matmul(da, dw, bias=db, residual=dr).numpy(), want.numpy(), "bias+residual")
+        want = F.add(act, dr)
+        assert_bit_equal(F.matmul(da, dw, bias=db, activation="gelu", residual=dr).numpy(), want.numpy(),
+                         "bias+gelu+residual")
+
+
+def test_matmul_causal_modes(gpu):
+    """causal=1: the lower triangle of q k^T equals the full product's (entries
+    above the diagonal are unspecified); causal=2: a lower-triangular left
+    operand gives the full product."""
+    F = gpu.functional
+    rng = np.random.default_rng(52)
+    for t, hd in [(300, 16), (128, 64), (129, 8), (1024, 64)]:
+        q = rng.standard_normal((2, 3, t, hd)).astype(np.float32)
+        k = rng.standard_normal((2, 3, t, hd)).astype(np.float32)
+        v = rng.standard_normal((2, 3, t, hd)).astype(np.float32)
+        dq, dk, dv = F.from_numpy(q), F.from_numpy(k), F.from_numpy(v)
+        full = F.matmul(dq, F.t(dk)).numpy()
+        tri = F.matmul(dq, F.t(dk), causal=1).numpy()
+        low = np.tril(np.ones((t, t), bool))
+        assert_bit_equal(tri[..., low], full[..., low], f"lower triangle t={t}")
+        p = np.tril(rng.standard_normal((2, 3, t, t))).astype(np.float32)
+        dp = F.from_numpy(p)
+        assert_bit_equal(F.matmul(dp, dv, causal=2).numpy(), F.matmul(dp, dv).numpy(), f"triangular left t={t}")
+    with pytest.raises(gpu.HIPError):
+        F.matmul(F.from_numpy(q[0, 0]), F.from_numpy(np.ones((hd, 5), np.float32)), causal=1)
