@@ -131,7 +131,7 @@ __device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0,
 // tile is (64 TM) x (64 TN).  2x2 -> 128x128 (64 accumulator registers), 2x1
 // -> 128x64 for narrow outputs and for shapes whose 128x128 tiling would leave
 // a partial last round of workgroups.
-template <bool LKIN, bool RKIN, bool FAST, int TM, int TN>
+template <bool LKIN, bool RKIN, bool FAST, int TM, int TN, bool FUSED>
 __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   constexpr int BMt = 64 * TM, BNt = 64 * TN;
   constexpr int LFLOATS = LKIN ? BMt * KPITCH : BK * BMt;
@@ -146,10 +146,21 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   // in groups of 8 row-tiles so neighbours share operand panels in that L2.
   const uint32_t ntiles = p.tiles_m * p.tiles_n;
   uint32_t pid = blockIdx.x;
+  // Triangular problems have cheap and expensive tiles, and workgroups start
+  // in dispatch order (x fastest).  Re-read the linear workgroup number as
+  // (tile rank, matrix) with the matrix index fastest and the most expensive
+  // tile rank first: every CU then works through expensive tiles early and
+  // fills up with cheap ones (longest-processing-time-first).
+  uint32_t batch_index = blockIdx.y;
+  if (FUSED && p.causal) {
+    const uint32_t linear = blockIdx.y * ntiles + blockIdx.x;
+    batch_index = linear % gridDim.y;
+    pid = ntiles - 1 - linear / gridDim.y;  // large tile rows (long K loops) first
+  }
   {
     const uint32_t xcds = 8;
     const uint32_t per = ntiles / xcds;
-    if (per > 0 && pid < per * xcds) pid = (pid % xcds) * per + pid / xcds;
+    if (!(FUSED && p.causal) && per > 0 && pid < per * xcds) pid = (pid % xcds) * per + pid / xcds;
   }
   const uint32_t group = 8;
   const uint32_t width = group * p.tiles_n;
@@ -161,9 +172,9 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 
   const int64_t m0 = (int64_t)tm * BMt;
   const int64_t n0 = (int64_t)tn * BNt;
-  if (p.causal == 1 && n0 > m0 + BMt - 1) return;  // tile wholly above the diagonal
-  const uint32_t zo = blockIdx.y / p.batch_inner;
-  const uint32_t zi = blockIdx.y - zo * p.batch_inner;
+  if (FUSED && p.causal == 1 && n0 > m0 + BMt - 1) return;  // tile wholly above the diagonal
+  const uint32_t zo = batch_index / p.batch_inner;
+  const uint32_t zi = batch_index - zo * p.batch_inner;
   const float* L = p.L + (int64_t)zo * p.sL2 + (int64_t)zi * p.sL;
   const float* R = p.R + (int64_t)zo * p.sR2 + (int64_t)zi * p.sR;
   float* C = p.C + (int64_t)zo * p.sC2 + (int64_t)zi * p.sC;
@@ -183,7 +194,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 
   f4 regL[BMt / 32], regR[BNt / 32];
   int64_t klimit = p.K;
-  if (p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
+  if (FUSED && p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
   const int64_t ksteps = (klimit + BK - 1) / BK;
   load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, 0, p.M, p.K, regL);
   load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, 0, p.N, p.K, regR);
@@ -235,10 +246,12 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
           float* c = C + row * p.ldc + col;
           float v = p.alpha * acc[i][j][r];
           if (p.beta != 0.0f) v += p.beta * *c;
-          if (p.bias) v += p.bias[col];
-          if (p.activation == 1) v = gelu_tanh_f(v);
-          if (p.residual)
-            v += p.residual[(int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes + row * p.ldres + col];
+          if constexpr (FUSED) {
+            if (p.bias) v += p.bias[col];
+            if (p.activation == 1) v = gelu_tanh_f(v);
+            if (p.residual)
+              v += p.residual[(int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes + row * p.ldres + col];
+          }
           *c = v;
         }
       }
@@ -250,26 +263,34 @@ static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; 
 static bool is_n(char c) { return c == 'N' || c == 'n'; }
 static bool is_t(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
-template <bool LK, bool RK, bool FAST, int TM, int TN>
+template <bool LK, bool RK, bool FAST, int TM, int TN, bool FUSED>
 static int launch_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
   constexpr int lfloats = LK ? 64 * TM * KPITCH : BK * 64 * TM;
   constexpr int rfloats = RK ? 64 * TN * KPITCH : BK * 64 * TN;
   constexpr size_t bytes = 2 * (size_t)(lfloats + rfloats) * sizeof(float);
   static bool configured = false;  // per instantiation
   if (!configured) {
-    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_kernel<LK, RK, FAST, TM, TN>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
-                      "hipFuncSetAttribute(sgemm_kernel)"));
+    WF2_TRY(check_hip(
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_kernel<LK, RK, FAST, TM, TN, FUSED>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+        "hipFuncSetAttribute(sgemm_kernel)"));
     configured = true;
   }
-  sgemm_kernel<LK, RK, FAST, TM, TN><<<grid, kBlock, bytes, st>>>(p);
+  sgemm_kernel<LK, RK, FAST, TM, TN, FUSED><<<grid, kBlock, bytes, st>>>(p);
   return 0;
 }
 
 template <bool LK, bool RK, int TM, int TN>
 static int launch_variant(const GemmParams& p, bool fast, dim3 grid, hipStream_t st) {
-  if (fast) return launch_kernel<LK, RK, true, TM, TN>(p, grid, st);
-  return launch_kernel<LK, RK, false, TM, TN>(p, grid, st);
+  // the plain product keeps a lean epilogue; bias / activation / residual /
+  // triangular skipping live in a separate instantiation
+  const bool fused = p.bias || p.residual || p.activation || p.causal;
+  if (fused) {
+    if (fast) return launch_kernel<LK, RK, true, TM, TN, true>(p, grid, st);
+    return launch_kernel<LK, RK, false, TM, TN, true>(p, grid, st);
+  }
+  if (fast) return launch_kernel<LK, RK, true, TM, TN, false>(p, grid, st);
+  return launch_kernel<LK, RK, false, TM, TN, false>(p, grid, st);
 }
 
 template <int TM, int TN>
