@@ -290,6 +290,51 @@ def test_config3_transcendentals(gpu, O, op, lo, hi):
     assert ulp_distance(got, truth).max() <= 1
 
 
+@pytest.mark.parametrize("op,lo,hi", CFG3[:4])
+def test_config3_full_size(gpu, O, op, lo, hi):
+    """BASELINE config 3 at its full size, 2^26 elements in one flat call (the
+    non-temporal streaming kernel): same bars as above."""
+    W = gpu
+    rng = np.random.Generator(np.random.PCG64(3))
+    n = 1 << 26
+    x = rng.uniform(lo, hi, n).astype(np.float32)
+    want = np.zeros(n, np.float32)
+    O.unary_1d(op, n, x, 1, want, 1)
+    dx = W.HIPTensor.from_numpy(x)
+    out = W.HIPTensor([n])
+    W.lib.check(getattr(W.lib.get(), "wf2hip_s" + op)(n, dptr(dx), 1, dptr(out), 1))
+    got = out.numpy()
+    del dx, out
+    assert ulp_distance(got, want).max() <= 2
+    truth = getattr(np, op)(x.astype(np.float64)).astype(np.float32)
+    assert ulp_distance(got, truth).max() <= 1
+
+
+def test_metric_size_binary_and_rowsum(gpu, O):
+    """The benchmark's workload, (8192, 8192) = 2^26 elements from seed 6:
+    x += y and x *= y bit-exact against the oracle, row sums <= 1e-5 relative
+    to the float64 sums (relative to sum |x|, the forward error scale)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.Generator(np.random.PCG64(6))
+    X = rng.standard_normal((8192, 8192)).astype(np.float32)
+    Y = rng.standard_normal((8192, 8192)).astype(np.float32)
+    dX, dY = F.from_numpy(X), F.from_numpy(Y)
+    for op in ("add", "mul"):
+        want = X.copy().ravel()
+        O.binary_1d(op, want.size, want, 1, Y.ravel(), 1)
+        work = F.copy(dX)
+        getattr(F, op + "_")(work, dY)
+        assert_bit_equal(work.numpy().ravel(), want, op)
+        del work, want
+    got = F.sum(dY, axis=1).numpy().ravel().astype(np.float64)
+    truth = Y.astype(np.float64).sum(axis=1)
+    scale = np.abs(Y).astype(np.float64).sum(axis=1)
+    assert np.max(np.abs(got - truth) / scale) <= 1e-5
+    # one rounding of the float64 sum is the best any fp32 result can do
+    assert np.max(np.abs(got - truth) / np.maximum(np.abs(truth), 1e-30) * (np.abs(truth) > 1)) <= 1e-6
+
+
 def test_unary_edge_values_and_tails(gpu, O):
     """+-0, denormals, +-inf, NaN, huge arguments, n % 8 != 0 tails, strided
     in/out."""
