@@ -158,7 +158,7 @@ def block_forward_ms(W, reps: int = 5):
     dx = W.HIPTensor.from_numpy(x)
     mask = gpt2.causal_mask(gpt2.CONFIG["seq"])
     out = {}
-    for mode in ("nodes", "fused"):
+    for mode in ("nodes", "fused_matmul_attention", "fused"):
         for _ in range(2):
             gpt2.block_forward(dx, dparams, mode=mode, mask=mask)
         e0, e1 = W.lib.Event(), W.lib.Event()

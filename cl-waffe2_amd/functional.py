@@ -373,6 +373,39 @@ def softmax_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     return out
 
 
+def attention(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor | None = None,
+              scale: float | None = None, causal: bool = False) -> HIPTensor:
+    """softmax(scale q k^T [+ causal mask]) v for (batch, heads, seq, 64) views in
+    one kernel (``wf2hip_attention_f32``): the fused form of SelfAttention's
+    !matmul / !softmax / !matmul chain (``examples/gpt-2/utils.lisp:222-243``).
+    Operands may be any views whose last axis is contiguous (heads read in
+    place from a fused projection); ``out`` defaults to a fresh (B, H, T, 64)
+    tensor."""
+    import ctypes as C
+    if not (len(q.shape) == len(k.shape) == len(v.shape) == 4) or \
+            not (list(q.shape) == list(k.shape) == list(v.shape)):
+        raise ValueError("attention expects three (batch, heads, seq, head_dim) tensors of one shape")
+    B, H, T, hd = q.shape
+    if out is None:
+        out = HIPTensor([B, H, T, hd], initial_element=None)
+    if list(out.shape) != [B, H, T, hd]:
+        raise ValueError("attention: out must have the operands' shape")
+    d = _lib.AttentionDesc()
+    d.batch, d.heads, d.seq, d.head_dim = B, H, T, hd
+    ptrs = []
+    for t, field in ((q, d.q_stride), (k, d.k_stride), (v, d.v_stride), (out, d.o_stride)):
+        _, strides, off = t.geometry()
+        if hd > 1 and strides[3] != 1:
+            raise ValueError("attention: the head_dim axis must be contiguous")
+        for a in range(3):
+            field[a] = strides[a]
+        ptrs.append(C.c_void_p(t.ptr + 4 * off))
+    d.scale = float(1.0 / math.sqrt(hd) if scale is None else scale)
+    d.causal = 1 if causal else 0
+    _lib.check(_lib.get().wf2hip_attention_f32(C.byref(d), *ptrs))
+    return out
+
+
 def gelu(x: HIPTensor) -> HIPTensor:
     """``(!gelu x)`` node for node (``source/nn/activation.lisp:45-66``):
     0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))."""

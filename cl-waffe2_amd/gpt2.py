@@ -15,11 +15,15 @@ Two modes:
            LayerNorm and GELU node for node, heads materialised with
            MoveTensorNode copies of sliced/permuted views, scaling and masking
            as MulNode / AddNode with broadcast operands, row softmax kernel.
-``fused``  the same mathematics with the fused row kernels (LayerNorm,
-           scale+mask+softmax), bias / GELU / residual in the gemm epilogues,
-           causal tile skipping in both attention products, and zero-copy heads: the attention gemms read
-           q/k/v straight out of the (B, T, 3, H, hd) projection through
-           strides and write the context straight into (B, T, H*hd).
+``fused``  the same mathematics with fused kernels: LayerNorm in one pass,
+           bias / GELU / residual in the gemm epilogues, and causal attention
+           as a single kernel that reads q/k/v straight out of the
+           (B, T, 3, H, hd) projection through strides, never materialises the
+           (B, H, T, T) scores and writes the context straight into
+           (B, T, H*hd).
+``fused_matmul_attention``  as ``fused`` but attention built from two batched
+           products with causal tile skipping and the fused scale+mask+softmax
+           row kernel (scores materialised once).
 """
 from __future__ import annotations
 
@@ -79,9 +83,9 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
     hd = D // H
     scale = 1.0 / math.sqrt(hd)
     eps = cfg["eps"]
-    fused = mode == "fused"
-    if mode not in ("fused", "nodes"):
-        raise ValueError("mode must be 'fused' or 'nodes'")
+    fused = mode in ("fused", "fused_matmul_attention")
+    if mode not in ("fused", "fused_matmul_attention", "nodes"):
+        raise ValueError("mode must be 'fused', 'fused_matmul_attention' or 'nodes'")
     ln = F.layer_norm_fused if fused else F.layer_norm
     act = F.gelu_fused if fused else F.gelu
 
@@ -91,7 +95,18 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
     else:
         qkv = _linear(h, p["w_qkv"], p["b_qkv"])
 
-    if fused:
+    if mode == "fused" and (hd % 4 != 0 or hd > 64):
+        mode = "fused_matmul_attention"   # the attention kernel is built for heads up to 64 wide
+    if mode == "fused":
+        four = F.reshape(qkv, B, T, 3 * H, hd)
+        # (B, H, T, hd) strided windows of the projection, no copy; the context is
+        # written straight into its merged (B, T, H*hd) layout
+        q, k, v = (four.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3)
+                   for i in range(3))
+        ctx_store = HIPTensor([B, T, H, hd], initial_element=None)
+        F.attention(q, k, v, out=ctx_store.permute(0, 2, 1, 3), scale=scale, causal=True)
+        ctx = F.reshape(ctx_store, B, T, D)
+    elif fused:
         five = F.reshape(qkv, B, T, 3, H, hd)
         # (B, 1, H, T, hd) strided windows of the projection, no copy
         q, k, v = (five.view(True, True, i, True, True).permute(0, 2, 3, 1, 4) for i in range(3))

@@ -72,6 +72,17 @@ class MatmulDesc(C.Structure):
     ]
 
 
+class AttentionDesc(C.Structure):
+    """``struct wf2hip_attention_desc``"""
+
+    _fields_ = [
+        ("batch", C.c_int64), ("heads", C.c_int64), ("seq", C.c_int64), ("head_dim", C.c_int64),
+        ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3),
+        ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
+        ("scale", C.c_float), ("causal", C.c_int32),
+    ]
+
+
 _SIGNATURES = {
     "wf2hip_abi_version": ([], C.c_int),
     "wf2hip_init": ([C.c_int], C.c_int),
@@ -127,6 +138,7 @@ _SIGNATURES = {
         C.c_int,
     ),
     "wf2hip_matmul_fused": ([C.POINTER(MatmulDesc), _P, _P, _P], C.c_int),
+    "wf2hip_attention_f32": ([C.POINTER(AttentionDesc), _P, _P, _P, _P], C.c_int),
     "wf2hip_sgemm_strided_batched_2d": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],
         C.c_int,

@@ -263,6 +263,27 @@ typedef struct wf2hip_matmul_desc {
 } wf2hip_matmul_desc;
 int wf2hip_matmul_fused(const wf2hip_matmul_desc* desc, const float* A, const float* B, float* C);
 
+/* ---- attention (extension; no BLAS counterpart) ---------------------------- */
+/* O[b,h,i,:] = sum_j softmax_j(scale * Q[b,h,i,:].K[b,h,j,:] (+ causal mask j <= i)) V[b,h,j,:]
+ * in one kernel, replacing the node sequence !matmul, scalar multiply, mask add,
+ * !softmax, !matmul of cl-waffe2's SelfAttention (examples/gpt-2/utils.lisp:
+ * 222-243) without materialising the (batch, heads, seq, seq) scores.  Softmax is
+ * the max-subtracted form.  head_dim: a multiple of 4, at most 64 (narrower heads
+ * run zero-padded to 64).  Each operand is addressed as
+ * base[b * stride[0] + h * stride[1] + i * stride[2] + c], c < head_dim with unit
+ * stride, so heads can be read in place from a fused (B, T, 3, H, 64) projection
+ * and O written directly as (B, T, H * 64).  Pointers 16-byte aligned, strides
+ * multiples of 4 elements; O may not overlap an input (WF2HIP_EOVERLAP).
+ * Result: within 1e-5 of the float64 value relative to max |V|. */
+typedef struct wf2hip_attention_desc {
+  int64_t batch, heads, seq, head_dim;
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3]; /* batch, head, position */
+  float scale;    /* multiplies Q.K before the softmax, e.g. 1/sqrt(head_dim) */
+  int32_t causal; /* 1: position i attends to j <= i only */
+} wf2hip_attention_desc;
+int wf2hip_attention_f32(const wf2hip_attention_desc* desc, const float* q, const float* k,
+                         const float* v, float* o);
+
 #ifdef __cplusplus
 }
 #endif

@@ -3,7 +3,8 @@
 Tolerance: the block chains six fp32 gemms (K up to 3072) and two LayerNorms;
 each gemm is held to 1e-5 relative to its magnitude sum elsewhere, here the
 output (O(1) values) is held to 2e-4 absolute + 2e-4 relative, and the two
-modes (node-for-node vs fused kernels) to each other at the same bar.
+modes (node-for-node vs fused kernels, attention as one kernel or as two
+products) to each other at the same bar.
 """
 import importlib
 
@@ -13,7 +14,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def _run(W, cfg, seed, modes=("nodes", "fused")):
+def _run(W, cfg, seed, modes=("nodes", "fused", "fused_matmul_attention")):
     from oracle import gpt2_block_ref as ref
     gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
     params = gpt2.make_block_params(seed, cfg)
@@ -33,8 +34,8 @@ def _run(W, cfg, seed, modes=("nodes", "fused")):
         assert got.shape == want.shape
         np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4, err_msg=mode)
         outs[mode] = got
-    if len(outs) == 2:
-        np.testing.assert_allclose(outs["nodes"], outs["fused"], rtol=2e-4, atol=2e-4)
+    for mode in modes[1:]:
+        np.testing.assert_allclose(outs[modes[0]], outs[mode], rtol=2e-4, atol=2e-4, err_msg=mode)
 
 
 def test_block_small(gpu):
