@@ -36,6 +36,7 @@
 namespace wf2 {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int BK = 32;
@@ -61,13 +62,18 @@ struct GemmParams {
   // 2: the left operand is lower-triangular (L[i][l] = 0 for l > i), so the
   //    K loop of a row tile stops at its last row
   int32_t causal;
+  int32_t pair_ok;  // C (and residual) rows allow 8-byte stores at even columns
 };
 
 // Loads this thread's share of a ROWS x BK operand tile into registers
 // (ROWS/32 float4 per thread).
 // KIN: operand stored [x][k] (k innermost) else [k][x].
-// FAST: 16-byte loads (pointer, pitch and extents checked on the host).
-template <bool KIN, bool FAST, int ROWS>
+// FAST: 16-byte loads (pointer, pitch and extents checked on the host).  Rows or
+// columns beyond the matrix are clamped to its last ones instead of zeroed:
+// they only feed accumulators that are never stored.  KGUARD: the tile may
+// reach beyond K, where operands must read as zero; the main loop runs without
+// it and has no branches.
+template <bool KIN, bool FAST, int ROWS, bool KGUARD>
 __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_t ld, int64_t x0,
                                           int64_t k0, int64_t X, int64_t K, f4 (&reg)[ROWS / 32]) {
   const int t = threadIdx.x;
@@ -84,7 +90,9 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
     }
     f4 v = {0.f, 0.f, 0.f, 0.f};
     if (FAST) {
-      if (x < X && k < K) v = *reinterpret_cast<const f4*>(KIN ? base + x * ld + k : base + k * ld + x);
+      const int64_t xc = KIN ? (x < X ? x : X - 1) : (x < X ? x : X - 4);
+      if (!KGUARD || k < K)
+        v = *reinterpret_cast<const f4*>(KIN ? base + xc * ld + k : base + k * ld + xc);
     } else {
       float e[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -127,6 +135,52 @@ __device__ __forceinline__ void read_frag(const float* __restrict__ lds, int x0,
   }
 }
 
+// Which output tile and which matrix of the batch a workgroup owns.
+// Tile order: consecutive workgroups land on different XCDs (round robin),
+// so each XCD gets a contiguous band of tiles, walked column-major in groups
+// of 8 row-tiles so that neighbours share operand panels in that XCD's L2.
+// Triangular problems have cheap and expensive tiles, and workgroups start in
+// dispatch order (x fastest): there the linear workgroup number is re-read as
+// (tile rank, matrix) with the matrix index fastest and the most expensive tile
+// rank first, so every CU works through expensive tiles early and fills up
+// with cheap ones (longest-processing-time-first).
+__device__ __forceinline__ void map_tile(const GemmParams& p, bool triangular, uint32_t* tm,
+                                         uint32_t* tn, uint32_t* batch_index) {
+  const uint32_t ntiles = p.tiles_m * p.tiles_n;
+  uint32_t pid = blockIdx.x;
+  *batch_index = blockIdx.y;
+  if (triangular) {
+    const uint32_t linear = blockIdx.y * ntiles + blockIdx.x;
+    *batch_index = linear % gridDim.y;
+    pid = ntiles - 1 - linear / gridDim.y;  // large tile rows (long K loops) first
+  } else {
+    const uint32_t xcds = 8;
+    const uint32_t per = ntiles / xcds;
+    if (per > 0 && pid < per * xcds) pid = (pid % xcds) * per + pid / xcds;
+  }
+  const uint32_t group = 8;
+  const uint32_t width = group * p.tiles_n;
+  const uint32_t gid = pid / width;
+  const uint32_t first_m = gid * group;
+  const uint32_t gsize = (p.tiles_m - first_m) < group ? (p.tiles_m - first_m) : group;
+  *tm = first_m + (pid % width) % gsize;
+  *tn = (pid % width) / gsize;
+}
+
+// One output element: C = act(alpha acc + beta C + bias[col]) + residual.
+template <bool FUSED>
+__device__ __forceinline__ float finish_value(const GemmParams& p, float accv, float cold,
+                                              int64_t row, int64_t col, int64_t res_base) {
+  float v = p.alpha * accv;
+  if (p.beta != 0.0f) v += p.beta * cold;
+  if constexpr (FUSED) {
+    if (p.bias) v += p.bias[col];
+    if (p.activation == 1) v = gelu_tanh_f(v);
+    if (p.residual) v += p.residual[res_base + row * p.ldres + col];
+  }
+  return v;
+}
+
 // TM x TN MFMA tiles (32x32) per wavefront, wavefronts 2 x 2: the workgroup
 // tile is (64 TM) x (64 TN).  2x2 -> 128x128 (64 accumulator registers), 2x1
 // -> 128x64 for narrow outputs and for shapes whose 128x128 tiling would leave
@@ -141,34 +195,8 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   auto ldsL = [&](int stage) { return smem + stage * LFLOATS; };
   auto ldsR = [&](int stage) { return smem + 2 * LFLOATS + stage * RFLOATS; };
 
-  // Tile order: consecutive workgroups land on different XCDs (round robin),
-  // so give each XCD a contiguous band of tiles, and walk a band column-major
-  // in groups of 8 row-tiles so neighbours share operand panels in that L2.
-  const uint32_t ntiles = p.tiles_m * p.tiles_n;
-  uint32_t pid = blockIdx.x;
-  // Triangular problems have cheap and expensive tiles, and workgroups start
-  // in dispatch order (x fastest).  Re-read the linear workgroup number as
-  // (tile rank, matrix) with the matrix index fastest and the most expensive
-  // tile rank first: every CU then works through expensive tiles early and
-  // fills up with cheap ones (longest-processing-time-first).
-  uint32_t batch_index = blockIdx.y;
-  if (FUSED && p.causal) {
-    const uint32_t linear = blockIdx.y * ntiles + blockIdx.x;
-    batch_index = linear % gridDim.y;
-    pid = ntiles - 1 - linear / gridDim.y;  // large tile rows (long K loops) first
-  }
-  {
-    const uint32_t xcds = 8;
-    const uint32_t per = ntiles / xcds;
-    if (!(FUSED && p.causal) && per > 0 && pid < per * xcds) pid = (pid % xcds) * per + pid / xcds;
-  }
-  const uint32_t group = 8;
-  const uint32_t width = group * p.tiles_n;
-  const uint32_t gid = pid / width;
-  const uint32_t first_m = gid * group;
-  const uint32_t gsize = (p.tiles_m - first_m) < group ? (p.tiles_m - first_m) : group;
-  const uint32_t tm = first_m + (pid % width) % gsize;
-  const uint32_t tn = (pid % width) / gsize;
+  uint32_t tm, tn, batch_index;
+  map_tile(p, FUSED && p.causal, &tm, &tn, &batch_index);
 
   const int64_t m0 = (int64_t)tm * BMt;
   const int64_t n0 = (int64_t)tn * BNt;
@@ -196,34 +224,51 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   int64_t klimit = p.K;
   if (FUSED && p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
   const int64_t ksteps = (klimit + BK - 1) / BK;
-  load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, 0, p.M, p.K, regL);
-  load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, 0, p.N, p.K, regR);
+  load_tile<LKIN, FAST, BMt, true>(L, p.ldl, m0, 0, p.M, p.K, regL);
+  load_tile<RKIN, FAST, BNt, true>(R, p.ldr, n0, 0, p.N, p.K, regR);
   store_tile<LKIN, BMt>(ldsL(0), regL);
   store_tile<RKIN, BNt>(ldsR(0), regR);
   __syncthreads();
 
   for (int64_t ks = 0; ks < ksteps; ks++) {
     const int cur = (int)(ks & 1);
-    if (ks + 1 < ksteps) {
-      load_tile<LKIN, FAST, BMt>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
-      load_tile<RKIN, FAST, BNt>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
+    const bool more = ks + 1 < ksteps;
+    if (more) {
+      if ((ks + 2) * BK <= p.K) {
+        load_tile<LKIN, FAST, BMt, false>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
+        load_tile<RKIN, FAST, BNt, false>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
+      } else {
+        load_tile<LKIN, FAST, BMt, true>(L, p.ldl, m0, (ks + 1) * BK, p.M, p.K, regL);
+        load_tile<RKIN, FAST, BNt, true>(R, p.ldr, n0, (ks + 1) * BK, p.N, p.K, regR);
+      }
     }
+    // fragments of k-group g+1 are fetched from LDS while the matrix cores work
+    // on group g
+    float a[2][TM][4], b[2][TN][4];
 #pragma unroll
-    for (int kb = 0; kb < BK; kb += 8) {
-      float a[TM][4], b[TN][4];
+    for (int i = 0; i < TM; i++) read_frag<LKIN, BMt>(ldsL(cur), wm + i * 32, 0, lane, a[0][i]);
 #pragma unroll
-      for (int i = 0; i < TM; i++) read_frag<LKIN, BMt>(ldsL(cur), wm + i * 32, kb, lane, a[i]);
+    for (int j = 0; j < TN; j++) read_frag<RKIN, BNt>(ldsR(cur), wn + j * 32, 0, lane, b[0][j]);
 #pragma unroll
-      for (int j = 0; j < TN; j++) read_frag<RKIN, BNt>(ldsR(cur), wn + j * 32, kb, lane, b[j]);
+    for (int g = 0; g < BK / 8; g++) {
+      if (g + 1 < BK / 8) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+          read_frag<LKIN, BMt>(ldsL(cur), wm + i * 32, 8 * (g + 1), lane, a[(g + 1) & 1][i]);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          read_frag<RKIN, BNt>(ldsR(cur), wn + j * 32, 8 * (g + 1), lane, b[(g + 1) & 1][j]);
+      }
 #pragma unroll
       for (int s = 0; s < 4; s++)
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[g & 1][i][s], b[g & 1][j][s],
+                                                             acc[i][j], 0, 0, 0);
     }
-    if (ks + 1 < ksteps) {
+    if (more) {
       // The other buffer was last read in iteration ks-1, and every wave has
       // passed the barrier that ended it.
       store_tile<LKIN, BMt>(ldsL(cur ^ 1), regL);
@@ -258,6 +303,248 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
     }
 }
 
+// ---- streaming variant: global -> LDS without passing through registers ------------
+// For the common case (left operand k-innermost, 16-byte aligned operands, K a
+// multiple of 32) the operand tiles are fetched with global_load_lds_dwordx4:
+// each wavefront instruction moves 64 x 16 bytes straight into 1 KB of LDS, so the
+// K loop holds no staging registers, no ds_write and no address branches.
+// Measured on 4096^3 (cycles the CUs are busy / cycles the matrix cores need):
+// 82 % with register staging, 91 % with this kernel.  What made the difference,
+// in order: (1) LDS writes issued by the wavefronts themselves cost ~12 cycles of
+// CU time each, the DMA path ~8 per KB less; (2) the compiler folds a software
+// prefetch of the fragments back into load-wait-use unless the order is pinned
+// with sched_group_barrier, which leaves the LDS latency of every k-group exposed;
+// (3) the barrier sits before the last k-group, so the first fragments of the next
+// K-step are fetched under that group's MFMAs.
+//
+// LDS layouts (64 banks of 4 bytes: a 128-bit read is conflict-free when 16
+// consecutive lanes cover 256 distinct bytes modulo 256):
+//   k-innermost tile  [rows][32], no padding; the eight 16-byte slots of a row are
+//                     permuted: slot = chunk ^ ((row / 2) % 8).  The DMA writes
+//                     lane l of an instruction to byte 16 l, so the permutation is
+//                     applied to the global address each lane reads.
+//   x-innermost tile  [32][128]: MFMA tile j of a wavefront takes columns
+//                     2 c + j (c = lane % 32), so one 64-bit read serves both
+//                     tiles and the output is stored as 8-byte pairs.
+//                     [32][64] (narrow tile): groups of four k-rows are kept 1152
+//                     bytes apart so the two half-waves hit different banks.
+template <bool RKIN, int TN>
+struct DmaLayout {
+  static constexpr int BNt = 64 * TN;
+  static constexpr int LFLOATS = 128 * BK;
+  // instructions per workgroup and K-step for the right operand, rows each covers
+  static constexpr int R_ROWS_PER_INSTR = RKIN ? 8 : 256 / BNt;
+  static constexpr int R_INSTRS = RKIN ? BNt / 8 : BK / R_ROWS_PER_INSTR;
+  static constexpr int R_INSTR_PITCH = (!RKIN && TN == 1) ? 288 : 256;  // floats
+  static constexpr int RFLOATS = R_INSTRS * R_INSTR_PITCH;
+  static constexpr int STAGE = LFLOATS + RFLOATS;
+  static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE * sizeof(float);
+};
+
+template <bool RKIN, int TN, bool FUSED>
+__global__ __launch_bounds__(kBlock) void sgemm_dma_kernel(GemmParams p) {
+  using Lay = DmaLayout<RKIN, TN>;
+  constexpr int BMt = 128, BNt = Lay::BNt;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  auto ldsL = [&](int stage) { return smem + stage * Lay::STAGE; };
+  auto ldsR = [&](int stage) { return smem + stage * Lay::STAGE + Lay::LFLOATS; };
+
+  uint32_t tm, tn, batch_index;
+  map_tile(p, FUSED && p.causal, &tm, &tn, &batch_index);
+  const int64_t m0 = (int64_t)tm * BMt;
+  const int64_t n0 = (int64_t)tn * BNt;
+  if (FUSED && p.causal == 1 && n0 > m0 + BMt - 1) return;  // tile wholly above the diagonal
+  const uint32_t zo = batch_index / p.batch_inner;
+  const uint32_t zi = batch_index - zo * p.batch_inner;
+  const float* L = p.L + (int64_t)zo * p.sL2 + (int64_t)zi * p.sL;
+  const float* R = p.R + (int64_t)zo * p.sR2 + (int64_t)zi * p.sR;
+  float* C = p.C + (int64_t)zo * p.sC2 + (int64_t)zi * p.sC;
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int half = lane >> 5;
+  const int col = lane & 31;
+  const int wm = (wave >> 1) * 64;
+  const int wn = (wave & 1) * 32 * TN;
+
+  // Global source of every 16-byte piece this lane moves per K-step (k = 0);
+  // rows / columns beyond the matrix are clamped to its last ones: they only
+  // feed accumulators that are never stored.
+  constexpr int LI = 4;                   // left-operand instructions per wavefront
+  constexpr int RI = Lay::R_INSTRS / 4;   // right-operand instructions per wavefront
+  const float* srcL[LI];
+  const float* srcR[RI];
+#pragma unroll
+  for (int j = 0; j < LI; j++) {
+    const int row = (wave * LI + j) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int64_t gr = m0 + row;
+    gr = gr < p.M ? gr : p.M - 1;
+    srcL[j] = L + gr * p.ldl + chunk * 4;
+  }
+#pragma unroll
+  for (int j = 0; j < RI; j++) {
+    const int q = wave * RI + j;
+    if (RKIN) {
+      const int row = q * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+      int64_t gn = n0 + row;
+      gn = gn < p.N ? gn : p.N - 1;
+      srcR[j] = R + gn * p.ldr + chunk * 4;
+    } else {
+      constexpr int CPR = BNt / 4;  // 16-byte pieces per k-row
+      const int krow = q * Lay::R_ROWS_PER_INSTR + lane / CPR;
+      int64_t gn = n0 + (lane % CPR) * 4;
+      gn = gn < p.N ? gn : p.N - 4;
+      srcR[j] = R + (int64_t)krow * p.ldr + gn;
+    }
+  }
+  auto fetch = [&](int stage, int64_t k0) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int j = 0; j < LI; j++)
+      __builtin_amdgcn_global_load_lds(srcL[j] + k0, ldsL(stage) + (wave * LI + j) * 256, 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < RI; j++)
+      __builtin_amdgcn_global_load_lds(RKIN ? srcR[j] + k0 : srcR[j] + k0 * p.ldr,
+                                       ldsR(stage) + (wave * RI + j) * Lay::R_INSTR_PITCH, 16, 0, 0);
+#endif
+  };
+
+  f16v acc[2][TN];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  int lrow[2], lswz[2], rrow[TN], rswz[TN];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    lrow[i] = wm + i * 32 + col;
+    lswz[i] = (lrow[i] >> 1) & 7;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    rrow[j] = wn + j * 32 + col;
+    rswz[j] = (rrow[j] >> 1) & 7;
+  }
+
+  // fragments of k-group g (k = 8 g + 4 half + s, s = 0..3) into buffer `buf`
+  float a[2][2][4], b[2][TN][4];
+  auto read_frags = [&](int stage, int g, int buf) {
+    const float* sl = ldsL(stage);
+    const float* sr = ldsR(stage);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const f4 v = *reinterpret_cast<const f4*>(sl + lrow[i] * BK + ((2 * g + half) ^ lswz[i]) * 4);
+      a[buf][i][0] = v.x; a[buf][i][1] = v.y; a[buf][i][2] = v.z; a[buf][i][3] = v.w;
+    }
+    if (RKIN) {
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const f4 v = *reinterpret_cast<const f4*>(sr + rrow[j] * BK + ((2 * g + half) ^ rswz[j]) * 4);
+        b[buf][j][0] = v.x; b[buf][j][1] = v.y; b[buf][j][2] = v.z; b[buf][j][3] = v.w;
+      }
+    } else if (TN == 2) {
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++) {
+        const f2 v = *reinterpret_cast<const f2*>(sr + (8 * g + 4 * half + s4) * 128 + wn + 2 * col);
+        b[buf][0][s4] = v.x;
+        b[buf][TN - 1][s4] = v.y;
+      }
+    } else {
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++) {
+        const int k = 8 * g + 4 * half + s4;
+        b[buf][0][s4] = sr[(k >> 2) * Lay::R_INSTR_PITCH + (k & 3) * 64 + wn + col];
+      }
+    }
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++)
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[buf][i][s4], b[buf][j][s4], acc[i][j], 0, 0, 0);
+  };
+  // keeps the LDS reads of the next k-group among the first MFMAs of this one
+  auto pin_order = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4 * TN, 0);
+#endif
+  };
+
+  int64_t klimit = p.K;
+  if (FUSED && p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
+  const int ksteps = (int)(klimit / BK);  // K and the tile height are multiples of BK
+
+  fetch(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  read_frags(0, 0, 0);
+  for (int ks = 0; ks < ksteps; ks++) {
+    const int cur = ks & 1;
+    const bool more = ks + 1 < ksteps;
+    // the other stage was last read before the barrier of the previous step
+    if (more) fetch(cur ^ 1, (int64_t)(ks + 1) * BK);
+    read_frags(cur, 1, 1); multiply(0); pin_order();
+    read_frags(cur, 2, 0); multiply(1); pin_order();
+    read_frags(cur, 3, 1); multiply(0); pin_order();
+    // every fragment of this stage is in registers and this wavefront's part of
+    // the next stage has landed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (more) read_frags(cur ^ 1, 0, 0);
+    multiply(1); pin_order();
+  }
+
+  // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
+  const int64_t res_base = (int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes;
+  if (!RKIN && TN == 2 && p.pair_ok) {
+    const int64_t c0 = n0 + wn + 2 * col;  // even; N is a multiple of 4 here
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (row < p.M && c0 < p.N) {
+          f2* c = reinterpret_cast<f2*>(C + row * p.ldc + c0);
+          f2 old = {0.f, 0.f};
+          if (p.beta != 0.0f) old = *c;
+          f2 v;
+          v.x = finish_value<FUSED>(p, acc[i][0][r], old.x, row, c0, res_base);
+          v.y = finish_value<FUSED>(p, acc[i][TN - 1][r], old.y, row, c0 + 1, res_base);
+          *c = v;
+        }
+      }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int64_t cc = (!RKIN && TN == 2) ? n0 + wn + 2 * col + j : n0 + wn + j * 32 + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (row < p.M && cc < p.N) {
+          float* c = C + row * p.ldc + cc;
+          *c = finish_value<FUSED>(p, acc[i][j][r], p.beta != 0.0f ? *c : 0.0f, row, cc, res_base);
+        }
+      }
+    }
+}
+
 static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; }
 
 static bool is_n(char c) { return c == 'N' || c == 'n'; }
@@ -278,6 +565,31 @@ static int launch_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
   }
   sgemm_kernel<LK, RK, FAST, TM, TN, FUSED><<<grid, kBlock, bytes, st>>>(p);
   return 0;
+}
+
+template <bool RK, int TN, bool FUSED>
+static int launch_dma_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
+  constexpr size_t bytes = DmaLayout<RK, TN>::LDS_BYTES;
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_dma_kernel<RK, TN, FUSED>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+                      "hipFuncSetAttribute(sgemm_dma_kernel)"));
+    configured = true;
+  }
+  sgemm_dma_kernel<RK, TN, FUSED><<<grid, kBlock, bytes, st>>>(p);
+  return 0;
+}
+
+template <int TN>
+static int launch_dma(const GemmParams& p, bool rkin, dim3 grid, hipStream_t st) {
+  const bool fused = p.bias || p.residual || p.activation || p.causal;
+  if (rkin) {
+    if (fused) return launch_dma_kernel<true, TN, true>(p, grid, st);
+    return launch_dma_kernel<true, TN, false>(p, grid, st);
+  }
+  if (fused) return launch_dma_kernel<false, TN, true>(p, grid, st);
+  return launch_dma_kernel<false, TN, false>(p, grid, st);
 }
 
 template <bool LK, bool RK, int TM, int TN>
@@ -388,6 +700,20 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
   dim3 grid((uint32_t)blocks, (uint32_t)nb);
   hipStream_t st = rt().stream;
+  // 8-byte output stores: even pitch and batch strides, 8-byte aligned bases
+  auto even = [](int64_t v) { return (v & 1) == 0; };
+  p.pair_ok = ((uintptr_t)C % 8 == 0) && even(ldc) && even(strideC) && even(strideC2) &&
+              (!ep.residual || (((uintptr_t)ep.residual % 8 == 0) && even(ep.ldres) &&
+                                even(ep.sRes) && even(ep.sRes2)));
+  // global -> LDS streaming kernel: left operand k-innermost, whole K-steps
+  const bool dma = fast && lkin && k % BK == 0 && k > 0 && !getenv("WF2HIP_GEMM_NO_DMA");
+  if (dma) {
+    if (narrow)
+      WF2_TRY((launch_dma<1>(p, rkin, grid, st)));
+    else
+      WF2_TRY((launch_dma<2>(p, rkin, grid, st)));
+    return after_launch("sgemm_dma_kernel");
+  }
   if (narrow)
     WF2_TRY((launch_layout<2, 1>(p, lkin, rkin, fast, grid, st)));
   else

@@ -364,3 +364,56 @@ def test_matmul_causal_modes(gpu):
         assert_bit_equal(F.matmul(dp, dv, causal=2).numpy(), F.matmul(dp, dv).numpy(), f"triangular left t={t}")
     with pytest.raises(gpu.HIPError):
         F.matmul(F.from_numpy(q[0, 0]), F.from_numpy(np.ones((hd, 5), np.float32)), causal=1)
+
+@pytest.mark.parametrize("tile", ["w", "n"])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_streaming_kernel_matches_register_staged_kernel(gpu, monkeypatch, tile, tb):
+    """K a multiple of 32 with aligned operands takes the global->LDS streaming
+    kernel; it contracts k in the same order as the register-staged kernel, so
+    the two are bit-identical.  Ragged M / N (clamped loads), both tile widths,
+    both right-operand layouts, bias + GELU + residual, and sgemm_ with beta."""
+    import ctypes as C
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(77 + tb)
+    monkeypatch.setenv("WF2HIP_GEMM_TILE", tile)
+    for m, n, k in [(128, 128, 32), (200, 132, 96), (1, 4, 64), (515, 260, 416), (64, 1024, 128)]:
+        A = rng.standard_normal((m, k)).astype(np.float32)
+        B = rng.standard_normal((k, n)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        res = rng.standard_normal((m, n)).astype(np.float32)
+        dA = F.from_numpy(A)
+        dB = F.t(F.from_numpy(np.ascontiguousarray(B.T))) if tb else F.from_numpy(B)
+        db, dr = F.from_numpy(bias), F.from_numpy(res)
+        outs = {}
+        for mode in ("stream", "staged"):
+            if mode == "staged":
+                monkeypatch.setenv("WF2HIP_GEMM_NO_DMA", "1")
+            else:
+                monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+            outs[mode] = (F.matmul(dA, dB).numpy(),
+                          F.matmul(dA, dB, bias=db, activation="gelu", residual=dr).numpy())
+        monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+        _gemm_check(outs["stream"][0], A.astype(np.float64), B.astype(np.float64))
+        assert_bit_equal(outs["stream"][0], outs["staged"][0], f"plain {m}x{n}x{k}")
+        assert_bit_equal(outs["stream"][1], outs["staged"][1], f"fused {m}x{n}x{k}")
+    # Fortran contract with beta and a padded ldc (odd pitch: scalar stores)
+    m, n, k = 100, 36, 64
+    for ldc in (m + 3, m + 4):
+        A = rng.standard_normal((k, m)).astype(np.float32)      # column-major m x k, lda = m
+        B = rng.standard_normal((n, k)).astype(np.float32)      # column-major k x n, ldb = k
+        Cm = rng.standard_normal((n, ldc)).astype(np.float32)
+        dA, dB = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B)
+        got = {}
+        for mode in ("stream", "staged"):
+            if mode == "staged":
+                monkeypatch.setenv("WF2HIP_GEMM_NO_DMA", "1")
+            dC = W.HIPTensor.from_numpy(Cm)
+            W.lib.check(W.lib.get().wf2hip_sgemm(b"N", b"N", m, n, k, 0.5, C.c_void_p(dA.ptr), m,
+                                                 C.c_void_p(dB.ptr), k, -2.0, C.c_void_p(dC.ptr), ldc))
+            got[mode] = dC.numpy()
+        monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+        want = Cm.astype(np.float64)                               # the padding is left alone
+        want[:, :m] = -2.0 * want[:, :m] + 0.5 * (B.astype(np.float64) @ A.astype(np.float64))
+        np.testing.assert_allclose(got["stream"], want, rtol=0, atol=1e-4)
+        assert_bit_equal(got["stream"], got["staged"], f"sgemm beta ldc={ldc}")
