@@ -147,7 +147,7 @@ def counter_probe(W, reps: int = 5):
     print(json.dumps({"probe": "copy, add, mul, exp, rowsum", "launches_each": reps, "elements": N}))
 
 
-def block_forward_ms(W, reps: int = 5):
+def block_forward_ms(W, reps: int = 20, warm: int = 10):
     try:
         gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
     except ImportError:
@@ -159,7 +159,7 @@ def block_forward_ms(W, reps: int = 5):
     mask = gpt2.causal_mask(gpt2.CONFIG["seq"])
     out = {}
     for mode in ("nodes", "fused_matmul_attention", "fused"):
-        for _ in range(2):
+        for _ in range(warm):  # the core clock takes tens of milliseconds of load to settle
             gpt2.block_forward(dx, dparams, mode=mode, mask=mask)
         e0, e1 = W.lib.Event(), W.lib.Event()
         e0.record()

@@ -167,16 +167,18 @@ __device__ __forceinline__ void map_tile(const GemmParams& p, bool triangular, u
   *tn = (pid % width) / gsize;
 }
 
-// One output element: C = act(alpha acc + beta C + bias[col]) + residual.
+// One output element: C = act(alpha acc + beta C + bias) + residual; the caller
+// fetches bias and residual (once per column, and in batches) so that the
+// loads are not strung out one dependent access per element.
 template <bool FUSED>
 __device__ __forceinline__ float finish_value(const GemmParams& p, float accv, float cold,
-                                              int64_t row, int64_t col, int64_t res_base) {
+                                              float biasv, float resv) {
   float v = p.alpha * accv;
   if (p.beta != 0.0f) v += p.beta * cold;
   if constexpr (FUSED) {
-    if (p.bias) v += p.bias[col];
+    if (p.bias) v += biasv;
     if (p.activation == 1) v = gelu_tanh_f(v);
-    if (p.residual) v += p.residual[res_base + row * p.ldres + col];
+    if (p.residual) v += resv;
   }
   return v;
 }
@@ -328,13 +330,14 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 //                     tiles and the output is stored as 8-byte pairs.
 //                     [32][64] (narrow tile): groups of four k-rows are kept 1152
 //                     bytes apart so the two half-waves hit different banks.
+//                     [32][192] (128 x 192 tile): columns 0-63 of a wavefront's 96
+//                     are shared by tiles 0 and 1 as above, 64-95 belong to tile 2.
 template <bool RKIN, int TN>
 struct DmaLayout {
   static constexpr int BNt = 64 * TN;
   static constexpr int LFLOATS = 128 * BK;
   // instructions per workgroup and K-step for the right operand, rows each covers
-  static constexpr int R_ROWS_PER_INSTR = RKIN ? 8 : 256 / BNt;
-  static constexpr int R_INSTRS = RKIN ? BNt / 8 : BK / R_ROWS_PER_INSTR;
+  static constexpr int R_INSTRS = BNt * BK / 256;  // 64 pieces of 16 bytes each
   static constexpr int R_INSTR_PITCH = (!RKIN && TN == 1) ? 288 : 256;  // floats
   static constexpr int RFLOATS = R_INSTRS * R_INSTR_PITCH;
   static constexpr int STAGE = LFLOATS + RFLOATS;
@@ -342,7 +345,8 @@ struct DmaLayout {
 };
 
 template <bool RKIN, int TN, bool FUSED>
-__global__ __launch_bounds__(kBlock) void sgemm_dma_kernel(GemmParams p) {
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void sgemm_dma_kernel(
+    GemmParams p) {  // two workgroups per CU: at most 256 registers per lane
   using Lay = DmaLayout<RKIN, TN>;
   constexpr int BMt = 128, BNt = Lay::BNt;
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -392,9 +396,10 @@ __global__ __launch_bounds__(kBlock) void sgemm_dma_kernel(GemmParams p) {
       gn = gn < p.N ? gn : p.N - 1;
       srcR[j] = R + gn * p.ldr + chunk * 4;
     } else {
-      constexpr int CPR = BNt / 4;  // 16-byte pieces per k-row
-      const int krow = q * Lay::R_ROWS_PER_INSTR + lane / CPR;
-      int64_t gn = n0 + (lane % CPR) * 4;
+      constexpr int CPR = BNt / 4;  // 16-byte pieces per k-row; LDS keeps [k][BNt] densely
+      const int piece = q * 64 + lane;
+      const int krow = piece / CPR;
+      int64_t gn = n0 + (piece % CPR) * 4;
       gn = gn < p.N ? gn : p.N - 4;
       srcR[j] = R + (int64_t)krow * p.ldr + gn;
     }
@@ -447,12 +452,14 @@ __global__ __launch_bounds__(kBlock) void sgemm_dma_kernel(GemmParams p) {
         const f4 v = *reinterpret_cast<const f4*>(sr + rrow[j] * BK + ((2 * g + half) ^ rswz[j]) * 4);
         b[buf][j][0] = v.x; b[buf][j][1] = v.y; b[buf][j][2] = v.z; b[buf][j][3] = v.w;
       }
-    } else if (TN == 2) {
+    } else if (TN >= 2) {
 #pragma unroll
       for (int s4 = 0; s4 < 4; s4++) {
-        const f2 v = *reinterpret_cast<const f2*>(sr + (8 * g + 4 * half + s4) * 128 + wn + 2 * col);
+        const float* krow = sr + (8 * g + 4 * half + s4) * BNt + wn;
+        const f2 v = *reinterpret_cast<const f2*>(krow + 2 * col);
         b[buf][0][s4] = v.x;
-        b[buf][TN - 1][s4] = v.y;
+        b[buf][1][s4] = v.y;
+        if (TN == 3) b[buf][TN - 1][s4] = krow[64 + col];
       }
     } else {
 #pragma unroll
@@ -510,37 +517,83 @@ __global__ __launch_bounds__(kBlock) void sgemm_dma_kernel(GemmParams p) {
   // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
   const int64_t res_base = (int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes;
-  if (!RKIN && TN == 2 && p.pair_ok) {
+  const bool pairs = !RKIN && TN >= 2 && p.pair_ok;
+  const float* res = (FUSED && p.residual) ? p.residual + res_base : nullptr;
+  if (pairs) {
     const int64_t c0 = n0 + wn + 2 * col;  // even; N is a multiple of 4 here
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (row < p.M && c0 < p.N) {
-          f2* c = reinterpret_cast<f2*>(C + row * p.ldc + c0);
-          f2 old = {0.f, 0.f};
-          if (p.beta != 0.0f) old = *c;
-          f2 v;
-          v.x = finish_value<FUSED>(p, acc[i][0][r], old.x, row, c0, res_base);
-          v.y = finish_value<FUSED>(p, acc[i][TN - 1][r], old.y, row, c0 + 1, res_base);
-          *c = v;
-        }
+    if (c0 < p.N) {
+      float bias0 = 0.f, bias1 = 0.f;
+      if (FUSED && p.bias) {
+        bias0 = p.bias[c0];
+        bias1 = p.bias[c0 + 1];
       }
-    return;
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {  // eight rows at a time: loads first, then arithmetic and stores
+          f2 old[8], rs[8];
+#pragma unroll
+          for (int q = 0; q < 8; q++) {
+            const int r = 8 * h + q;
+            const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            old[q] = f2{0.f, 0.f};
+            rs[q] = f2{0.f, 0.f};
+            if (row < p.M) {
+              if (p.beta != 0.0f) old[q] = *reinterpret_cast<const f2*>(C + row * p.ldc + c0);
+              if (res) rs[q] = *reinterpret_cast<const f2*>(res + row * p.ldres + c0);
+            }
+          }
+#pragma unroll
+          for (int q = 0; q < 8; q++) {
+            const int r = 8 * h + q;
+            const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (row < p.M) {
+              f2 v;
+              v.x = finish_value<FUSED>(p, acc[i][0][r], old[q].x, bias0, rs[q].x);
+              v.y = finish_value<FUSED>(p, acc[i][TN >= 2 ? 1 : 0][r], old[q].y, bias1, rs[q].y);
+              *reinterpret_cast<f2*>(C + row * p.ldc + c0) = v;
+            }
+          }
+#if defined(__HIP_DEVICE_COMPILE__)
+          __builtin_amdgcn_sched_barrier(0);
+#endif
+        }
+    }
+    if (TN < 3) return;
   }
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int64_t cc = (!RKIN && TN == 2) ? n0 + wn + 2 * col + j : n0 + wn + j * 32 + col;
+      if (pairs && j < 2) continue;  // stored above
+      // tiles 0 and 1 of an n-innermost right operand own interleaved columns
+      const int64_t cc = (!RKIN && TN >= 2) ? (j < 2 ? n0 + wn + 2 * col + j : n0 + wn + 64 + col)
+                                            : n0 + wn + j * 32 + col;
+      if (cc >= p.N) continue;
+      const float biasv = (FUSED && p.bias) ? p.bias[cc] : 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (row < p.M && cc < p.N) {
-          float* c = C + row * p.ldc + cc;
-          *c = finish_value<FUSED>(p, acc[i][j][r], p.beta != 0.0f ? *c : 0.0f, row, cc, res_base);
+      for (int h = 0; h < 2; h++) {
+        float old[8], rs[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+          const int r = 8 * h + q;
+          const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          old[q] = 0.f;
+          rs[q] = 0.f;
+          if (row < p.M) {
+            if (p.beta != 0.0f) old[q] = C[row * p.ldc + cc];
+            if (res) rs[q] = res[row * p.ldres + cc];
+          }
         }
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+          const int r = 8 * h + q;
+          const int64_t row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          if (row < p.M) C[row * p.ldc + cc] = finish_value<FUSED>(p, acc[i][j][r], old[q], biasv, rs[q]);
+        }
+#if defined(__HIP_DEVICE_COMPILE__)
+        __builtin_amdgcn_sched_barrier(0);
+#endif
       }
     }
 }
@@ -581,6 +634,7 @@ static int launch_dma_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
   return 0;
 }
 
+// TN = 1, 2, 3: 128 x 64, 128 x 128, 128 x 192 output tiles
 template <int TN>
 static int launch_dma(const GemmParams& p, bool rkin, dim3 grid, hipStream_t st) {
   const bool fused = p.bias || p.residual || p.activation || p.causal;
@@ -683,38 +737,60 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   // every 4-wide load must be wholly inside or wholly outside the matrix
   fast = fast && (lkin ? k % 4 == 0 : p.M % 4 == 0) && (rkin ? k % 4 == 0 : p.N % 4 == 0);
 
-  // Tile choice: time ~ tiles on the busiest CU x work per tile.
-  // The narrow tile does 10 % less work per cycle (one operand is re-read from
-  // LDS twice as often) but wastes nothing on N <= 64 and evens out the last
-  // round.
-  const int64_t nb = (int64_t)batch * batch2;
-  const int64_t tiles_wide = ceil_div(p.M, 128) * ceil_div(p.N, 128) * nb;
-  const int64_t tiles_narrow = ceil_div(p.M, 128) * ceil_div(p.N, 64) * nb;
-  const double cost_wide = busiest_cu_tiles(tiles_wide) * 1.0;
-  const double cost_narrow = busiest_cu_tiles(tiles_narrow) * 0.5 / 0.9;
-  bool narrow = cost_narrow < cost_wide;
-  if (const char* force = getenv("WF2HIP_GEMM_TILE")) narrow = force[0] == 'n';  // tuning knob
-  p.tiles_m = (uint32_t)ceil_div(p.M, 128);
-  p.tiles_n = (uint32_t)ceil_div(p.N, narrow ? 64 : 128);
-  const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
-  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
-  dim3 grid((uint32_t)blocks, (uint32_t)nb);
-  hipStream_t st = rt().stream;
   // 8-byte output stores: even pitch and batch strides, 8-byte aligned bases
   auto even = [](int64_t v) { return (v & 1) == 0; };
   p.pair_ok = ((uintptr_t)C % 8 == 0) && even(ldc) && even(strideC) && even(strideC2) &&
               (!ep.residual || (((uintptr_t)ep.residual % 8 == 0) && even(ep.ldres) &&
                                 even(ep.sRes) && even(ep.sRes2)));
   // global -> LDS streaming kernel: left operand k-innermost, whole K-steps
-  const bool dma = fast && lkin && k % BK == 0 && k > 0 && !getenv("WF2HIP_GEMM_NO_DMA");
+  // (with only a few K-steps per tile the set-up of the streaming kernel costs more
+  // than it saves: 96 x 1024x1024x64 runs in 187 us staged, 243 us streamed)
+  bool dma = fast && lkin && k % BK == 0 && k >= 256;
+  if (const char* force = getenv("WF2HIP_GEMM_STREAM"))  // testing knob: 0 never, 1 whenever possible
+    dma = force[0] == '1' ? (fast && lkin && k % BK == 0 && k > 0) : false;
+
+  // Tile choice: time ~ tiles on the busiest CU x tile width / efficiency.
+  // Measured per unit of work 128x128 is about 6 % ahead of 128x64 (which
+  // re-reads one operand from LDS twice as often but keeps three workgroups on a
+  // CU), so what decides is how evenly the tile count divides over the CUs
+  // (8192 x 768 outputs: 768 or 384 tiles on 256 CUs).  A width that leaves one
+  // tile per CU loses the overlap of one workgroup's prologue and epilogue with
+  // another's K loop.  The 128x192 tile of the streaming kernel matches the
+  // others back to back but ran 25 % slower between other kernels (8192 x 2304
+  // x 768: 316 us against 245 us), so it is only reachable through the knob.
+  const int64_t nb = (int64_t)batch * batch2;
+  const int widths[2] = {64, 128};
+  const double eff[2] = {0.94, 1.0};
+  int tn_tiles = 2;
+  double best = 0.0;
+  for (int c = 0; c < 2; c++) {
+    const int64_t tiles = ceil_div(p.M, 128) * ceil_div(p.N, widths[c]) * nb;
+    const double rounds = busiest_cu_tiles(tiles);
+    const double cost = rounds * widths[c] / (eff[c] * (rounds < 2.0 ? 0.85 : 1.0));
+    if (c == 0 || cost < best) {
+      best = cost;
+      tn_tiles = c + 1;
+    }
+  }
+  if (const char* force = getenv("WF2HIP_GEMM_TILE")) {  // tuning knob: n(arrow), w(ide), x(tra wide)
+    tn_tiles = force[0] == 'n' ? 1 : (force[0] == 'x' && dma ? 3 : 2);
+  }
+  p.tiles_m = (uint32_t)ceil_div(p.M, 128);
+  p.tiles_n = (uint32_t)ceil_div(p.N, 64 * tn_tiles);
+  const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
+  dim3 grid((uint32_t)blocks, (uint32_t)nb);
+  hipStream_t st = rt().stream;
   if (dma) {
-    if (narrow)
+    if (tn_tiles == 1)
       WF2_TRY((launch_dma<1>(p, rkin, grid, st)));
-    else
+    else if (tn_tiles == 2)
       WF2_TRY((launch_dma<2>(p, rkin, grid, st)));
+    else
+      WF2_TRY((launch_dma<3>(p, rkin, grid, st)));
     return after_launch("sgemm_dma_kernel");
   }
-  if (narrow)
+  if (tn_tiles == 1)
     WF2_TRY((launch_layout<2, 1>(p, lkin, rkin, fast, grid, st)));
   else
     WF2_TRY((launch_layout<2, 2>(p, lkin, rkin, fast, grid, st)));

@@ -365,11 +365,11 @@ def test_matmul_causal_modes(gpu):
     with pytest.raises(gpu.HIPError):
         F.matmul(F.from_numpy(q[0, 0]), F.from_numpy(np.ones((hd, 5), np.float32)), causal=1)
 
-@pytest.mark.parametrize("tile", ["w", "n"])
+@pytest.mark.parametrize("tile", ["w", "n", "x"])
 @pytest.mark.parametrize("tb", [False, True])
 def test_matmul_streaming_kernel_matches_register_staged_kernel(gpu, monkeypatch, tile, tb):
-    """K a multiple of 32 with aligned operands takes the global->LDS streaming
-    kernel; it contracts k in the same order as the register-staged kernel, so
+    """K a multiple of 32 (from 256 on, or always with WF2HIP_GEMM_STREAM=1) and
+    aligned operands takes the global->LDS streaming kernel; it contracts k in the same order as the register-staged kernel, so
     the two are bit-identical.  Ragged M / N (clamped loads), both tile widths,
     both right-operand layouts, bias + GELU + residual, and sgemm_ with beta."""
     import ctypes as C
@@ -387,13 +387,10 @@ def test_matmul_streaming_kernel_matches_register_staged_kernel(gpu, monkeypatch
         db, dr = F.from_numpy(bias), F.from_numpy(res)
         outs = {}
         for mode in ("stream", "staged"):
-            if mode == "staged":
-                monkeypatch.setenv("WF2HIP_GEMM_NO_DMA", "1")
-            else:
-                monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+            monkeypatch.setenv("WF2HIP_GEMM_STREAM", "0" if mode == "staged" else "1")
             outs[mode] = (F.matmul(dA, dB).numpy(),
                           F.matmul(dA, dB, bias=db, activation="gelu", residual=dr).numpy())
-        monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+        monkeypatch.delenv("WF2HIP_GEMM_STREAM", raising=False)
         _gemm_check(outs["stream"][0], A.astype(np.float64), B.astype(np.float64))
         assert_bit_equal(outs["stream"][0], outs["staged"][0], f"plain {m}x{n}x{k}")
         assert_bit_equal(outs["stream"][1], outs["staged"][1], f"fused {m}x{n}x{k}")
@@ -406,13 +403,12 @@ def test_matmul_streaming_kernel_matches_register_staged_kernel(gpu, monkeypatch
         dA, dB = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B)
         got = {}
         for mode in ("stream", "staged"):
-            if mode == "staged":
-                monkeypatch.setenv("WF2HIP_GEMM_NO_DMA", "1")
+            monkeypatch.setenv("WF2HIP_GEMM_STREAM", "0" if mode == "staged" else "1")
             dC = W.HIPTensor.from_numpy(Cm)
             W.lib.check(W.lib.get().wf2hip_sgemm(b"N", b"N", m, n, k, 0.5, C.c_void_p(dA.ptr), m,
                                                  C.c_void_p(dB.ptr), k, -2.0, C.c_void_p(dC.ptr), ldc))
             got[mode] = dC.numpy()
-        monkeypatch.delenv("WF2HIP_GEMM_NO_DMA", raising=False)
+        monkeypatch.delenv("WF2HIP_GEMM_STREAM", raising=False)
         want = Cm.astype(np.float64)                               # the padding is left alone
         want[:, :m] = -2.0 * want[:, :m] + 0.5 * (B.astype(np.float64) @ A.astype(np.float64))
         np.testing.assert_allclose(got["stream"], want, rtol=0, atol=1e-4)
