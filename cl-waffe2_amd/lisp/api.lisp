@@ -56,6 +56,56 @@
 (defcfun "wf2hip_softmax_rows_f32" :int (rows :long) (cols :long) (x :pointer) (ldx :long) (out :pointer) (ldo :long))
 (defcfun "wf2hip_layernorm_rows_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (b :pointer) (eps :float) (out :pointer))
 
+;; Extensions without a BLAS / SIMD-extension counterpart.  cl-waffe2 reaches them through its own
+;; extension points: a define-bypass rule (source/vm/nodes/symbolic.lisp:118-131) or a define-op node
+;; like Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90).
+(defcfun "wf2hip_sgemm_strided_batched_2d" :int
+  (transa :char) (transb :char) (m :long) (n :long) (k :long) (alpha :float)
+  (a :pointer) (lda :long) (stride-a :long) (stride-a2 :long)
+  (b :pointer) (ldb :long) (stride-b :long) (stride-b2 :long)
+  (beta :float) (c :pointer) (ldc :long) (stride-c :long) (stride-c2 :long) (batch :long) (batch2 :long))
+
+;; struct wf2hip_matmul_desc
+(defcstruct matmul-desc
+  (trans-a :int32) (trans-b :int32) (activation :int32) (causal :int32)
+  (m :int64) (n :int64) (k :int64)
+  (lda :int64) (ldb :int64) (ldc :int64)
+  (batch :int64) (batch2 :int64)
+  (stride-a :int64) (stride-a2 :int64) (stride-b :int64) (stride-b2 :int64) (stride-c :int64) (stride-c2 :int64)
+  (bias :pointer) (residual :pointer)
+  (ld-residual :int64) (stride-residual :int64) (stride-residual2 :int64)
+  (alpha :float) (reserved :int32))
+(defcfun "wf2hip_matmul_fused" :int (desc (:pointer (:struct matmul-desc))) (a :pointer) (b :pointer) (c :pointer))
+
+;; struct wf2hip_attention_desc
+(defcstruct attention-desc
+  (batch :int64) (heads :int64) (seq :int64) (head-dim :int64)
+  (q-stride :int64 :count 3) (k-stride :int64 :count 3) (v-stride :int64 :count 3) (o-stride :int64 :count 3)
+  (scale :float) (causal :int32))
+(defcfun "wf2hip_attention_f32" :int
+  (desc (:pointer (:struct attention-desc))) (q :pointer) (k :pointer) (v :pointer) (o :pointer))
+(defcfun "wf2hip_causal_softmax_f32" :int (matrices :long) (seq :long) (x :pointer) (out :pointer) (scale :float))
+
+;; HIP graphs: record the launches of one compiled forward, replay them with one call.
+(defcfun "wf2hip_graph_begin" :int)
+(defcfun "wf2hip_graph_end" :int (graph (:pointer :pointer)))
+(defcfun "wf2hip_graph_launch" :int (graph :pointer))
+(defcfun "wf2hip_graph_destroy" :int (graph :pointer))
+(defcfun "wf2hip_pool_trim" :int)
+
+(defmacro with-captured-graph ((graph) &body body)
+  "Runs BODY once with every kernel launch recorded instead of executed and binds GRAPH to the
+recorded graph handle (replay with (check (wf2hip-graph-launch graph)), release with
+wf2hip-graph-destroy).  BODY must have run once eagerly before, so that its temporaries can be
+served from the library's pool; transfers and vref are refused while recording."
+  (let ((slot (gensym "SLOT")))
+    `(cffi:with-foreign-object (,slot :pointer)
+       (check (wf2hip-graph-begin))
+       (unwind-protect (progn ,@body)
+         (check (wf2hip-graph-end ,slot)))
+       (let ((,graph (cffi:mem-ref ,slot :pointer)))
+         ,graph))))
+
 ;; enum wf2hip_binary_op / wf2hip_unary_op
 (defconstant +add+ 0) (defconstant +sub+ 1) (defconstant +mul+ 2) (defconstant +div+ 3) (defconstant +move+ 4)
 (defconstant +sin+ 16) (defconstant +cos+ 17) (defconstant +tanh+ 18) (defconstant +log+ 19)

@@ -10,7 +10,9 @@ kernels are the hand-written gfx950 kernels of libwaffe2-hip.so.")
    #:*hip-device*
    #:try-loading-hip-extension
    #:hip-synchronize
-   #:with-sequential-reductions))
+   #:with-sequential-reductions
+   #:with-captured-graph
+   #:hip-error))
 
 (in-package :cl-waffe2/backends.hip)
 
