@@ -1,0 +1,279 @@
+// compare.hip -- out <- (x OP y) ? then : else over three tensors.
+//
+// Compare-Operation-Node (source/base-impl/logical.lisp:35-62) compares two
+// tensors element by element and writes one of two constants; the CPU backend
+// runs it as one waffe2_s{eq,lt,le,gt,ge} call per row
+// (source/backends/cpu/logical.lisp:62-84, cl-waffe2-simd.c:385-468).  Here the
+// node is one launch: a 16-byte-vector kernel when all three views collapse to
+// contiguous runs, an index-decomposing kernel otherwise.  HBM-bound: 12 bytes
+// per element (two reads, one write).  The scalar right-hand side
+// (Where-Operation-Node) is an element-wise functor in elementwise.hip.
+#include "wf2_common.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct Space3 {
+  int rank = 0;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t sa[WF2HIP_MAX_RANK], sb[WF2HIP_MAX_RANK], sc[WF2HIP_MAX_RANK];
+  int64_t off_a = 0, off_b = 0, off_c = 0;
+  int64_t total = 0;
+};
+
+__device__ __forceinline__ bool holds(int op, float a, float b) {
+  switch (op) {
+    case WF2HIP_EQ: return a == b;
+    case WF2HIP_LT: return a < b;
+    case WF2HIP_LE: return a <= b;
+    case WF2HIP_GT: return a > b;
+    default: return a >= b;
+  }
+}
+
+// all three contiguous and 16-byte aligned.  Three streams, like x <- x + y:
+// each wavefront owns 4 KB contiguous per stream and every thread issues its four
+// 16-byte loads per operand before the first use (the layout that measured best
+// for three-stream kernels, see elementwise.hip).
+template <bool NT>
+__global__ __launch_bounds__(kBlock) void compare_flat(const float* __restrict__ x,
+                                                       const float* __restrict__ y,
+                                                       float* __restrict__ out, size_t n, int op,
+                                                       float then_value, float else_value) {
+  constexpr int U = 4;
+  const size_t nvec = n / 4;
+  const f4* xv = reinterpret_cast<const f4*>(x);
+  const f4* yv = reinterpret_cast<const f4*>(y);
+  f4* ov = reinterpret_cast<f4*>(out);
+  const unsigned wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + wave) * kWave * U + lane;
+  f4 a[U], b[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const size_t i = base + (size_t)u * kWave;
+    if (i < nvec) {
+      a[u] = NT ? __builtin_nontemporal_load(xv + i) : xv[i];
+      b[u] = NT ? __builtin_nontemporal_load(yv + i) : yv[i];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const size_t i = base + (size_t)u * kWave;
+    if (i < nvec) {
+      f4 r;
+      r.x = holds(op, a[u].x, b[u].x) ? then_value : else_value;
+      r.y = holds(op, a[u].y, b[u].y) ? then_value : else_value;
+      r.z = holds(op, a[u].z, b[u].z) ? then_value : else_value;
+      r.w = holds(op, a[u].w, b[u].w) ? then_value : else_value;
+      if (NT)
+        __builtin_nontemporal_store(r, ov + i);
+      else
+        ov[i] = r;
+    }
+  }
+  // the last n % 4 elements
+  if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    const size_t i = nvec * 4 + threadIdx.x;
+    out[i] = holds(op, x[i], y[i]) ? then_value : else_value;
+  }
+}
+
+struct Cmp3Params {
+  const float* x;
+  const float* y;
+  float* out;
+  int32_t rank, op;
+  int64_t total;
+  int64_t shape[WF2HIP_MAX_RANK], sa[WF2HIP_MAX_RANK], sb[WF2HIP_MAX_RANK], sc[WF2HIP_MAX_RANK];
+  float then_value, else_value;
+};
+
+// any strides: one element per thread, innermost axis fastest so that unit
+// inner strides stay coalesced
+__global__ __launch_bounds__(kBlock) void compare_generic(Cmp3Params p) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= p.total) return;
+  int64_t rem = i, ao = 0, bo = 0, co = 0;
+  for (int r = p.rank - 1; r > 0; r--) {
+    const int64_t q = rem / p.shape[r];
+    const int64_t idx = rem - q * p.shape[r];
+    rem = q;
+    ao += idx * p.sa[r];
+    bo += idx * p.sb[r];
+    co += idx * p.sc[r];
+  }
+  ao += rem * p.sa[0];
+  bo += rem * p.sb[0];
+  co += rem * p.sc[0];
+  p.out[co] = holds(p.op, p.x[ao], p.y[bo]) ? p.then_value : p.else_value;
+}
+
+static void normalise3(Space3* s) {
+  int w = 0;
+  for (int r = 0; r < s->rank; r++) {
+    if (s->shape[r] == 1) continue;
+    s->shape[w] = s->shape[r];
+    s->sa[w] = s->sa[r];
+    s->sb[w] = s->sb[r];
+    s->sc[w] = s->sc[r];
+    w++;
+  }
+  if (w == 0) {
+    s->shape[0] = 1;
+    s->sa[0] = s->sb[0] = s->sc[0] = 0;
+    w = 1;
+  }
+  s->rank = w;
+  int out = 0;
+  for (int r = 1; r < s->rank; r++) {
+    const bool merge = s->sa[out] == s->sa[r] * s->shape[r] && s->sb[out] == s->sb[r] * s->shape[r] &&
+                       s->sc[out] == s->sc[r] * s->shape[r];
+    if (merge) {
+      s->shape[out] *= s->shape[r];
+    } else {
+      out++;
+      s->shape[out] = s->shape[r];
+    }
+    s->sa[out] = s->sa[r];
+    s->sb[out] = s->sb[r];
+    s->sc[out] = s->sc[r];
+  }
+  s->rank = out + 1;
+  s->total = 1;
+  for (int r = 0; r < s->rank; r++) s->total *= s->shape[r];
+}
+
+// lowest / highest element a strided window touches
+static void span_of(const Space3& s, const int64_t* stride, int64_t off, int64_t* lo, int64_t* hi) {
+  *lo = *hi = off;
+  for (int r = 0; r < s.rank; r++) {
+    const int64_t span = stride[r] * (s.shape[r] - 1);
+    if (span >= 0)
+      *hi += span;
+    else
+      *lo += span;
+  }
+}
+
+// `out` may coincide with an input element for element (in-place compare);
+// any other overlap makes the result depend on the order of the writes
+static bool hazardous(const Space3& s, const float* out, const int64_t* sin, int64_t off_in,
+                      const float* in) {
+  int64_t olo, ohi, ilo, ihi;
+  span_of(s, s.sc, s.off_c, &olo, &ohi);
+  span_of(s, sin, off_in, &ilo, &ihi);
+  if (out + ohi < in + ilo || in + ihi < out + olo) return false;
+  if (out + s.off_c != in + off_in) return true;
+  for (int r = 0; r < s.rank; r++)
+    if (s.sc[r] != sin[r]) return true;
+  return false;
+}
+
+int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, float then_value,
+               float else_value) {
+  if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
+  if (s.total == 0) return 0;
+  if (!x || !y || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  // a stride-0 axis of `out` keeps what the sequential loop writes last
+  for (int r = 0; r < s.rank; r++)
+    if (s.sc[r] == 0 && s.shape[r] > 1) {
+      s.off_a += s.sa[r] * (s.shape[r] - 1);
+      s.off_b += s.sb[r] * (s.shape[r] - 1);
+      s.shape[r] = 1;
+    }
+  normalise3(&s);
+  if (hazardous(s, out, s.sa, s.off_a, x) || hazardous(s, out, s.sb, s.off_b, y))
+    return fail(WF2HIP_EOVERLAP, "compare writes into a window that partially overlaps an input");
+  hipStream_t st = rt().stream;
+  const float* xp = x + s.off_a;
+  const float* yp = y + s.off_b;
+  float* op_ = out + s.off_c;
+  const bool flat = s.rank == 1 && (s.total == 1 || (s.sa[0] == 1 && s.sb[0] == 1 && s.sc[0] == 1)) &&
+                    (((uintptr_t)xp | (uintptr_t)yp | (uintptr_t)op_) & 15u) == 0;
+  if (flat) {
+    const int64_t nvec = s.total / 4;
+    const int64_t blocks = ceil_div(nvec > 0 ? nvec : 1, (int64_t)kBlock * 4);
+    if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+    if (s.total * 12 >= ((int64_t)192 << 20))
+      compare_flat<true><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, yp, op_, (size_t)s.total, op,
+                                                              then_value, else_value);
+    else
+      compare_flat<false><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, yp, op_, (size_t)s.total, op,
+                                                               then_value, else_value);
+    return after_launch("compare_flat");
+  }
+  Cmp3Params p;
+  p.x = xp;
+  p.y = yp;
+  p.out = op_;
+  p.rank = s.rank;
+  p.op = op;
+  p.total = s.total;
+  for (int r = 0; r < s.rank; r++) {
+    p.shape[r] = s.shape[r];
+    p.sa[r] = s.sa[r];
+    p.sb[r] = s.sb[r];
+    p.sc[r] = s.sc[r];
+  }
+  p.then_value = then_value;
+  p.else_value = else_value;
+  const int64_t blocks = ceil_div(s.total, kBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+  compare_generic<<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  return after_launch("compare_generic");
+}
+
+static int load_space3(const wf2hip_view3* v, Space3* s) {
+  if (!v) return fail(WF2HIP_EINVAL, "null view descriptor");
+  if (v->rank < 1 || v->rank > WF2HIP_MAX_RANK)
+    return fail(WF2HIP_EINVAL, "view rank %d outside 1..%d", v->rank, WF2HIP_MAX_RANK);
+  s->rank = v->rank;
+  s->total = 1;
+  for (int r = 0; r < v->rank; r++) {
+    if (v->shape[r] < 0) return fail(WF2HIP_EINVAL, "negative extent on axis %d", r);
+    s->shape[r] = v->shape[r];
+    s->sa[r] = v->stride_a[r];
+    s->sb[r] = v->stride_b[r];
+    s->sc[r] = v->stride_c[r];
+    s->total *= v->shape[r];
+  }
+  if (v->off_a < 0 || v->off_b < 0 || v->off_c < 0) return fail(WF2HIP_EINVAL, "negative offset");
+  s->off_a = v->off_a;
+  s->off_b = v->off_b;
+  s->off_c = v->off_c;
+  return 0;
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_compare_nd(int op, const wf2hip_view3* v, const float* x, const float* y,
+                              float* out, float then_value, float else_value) {
+  WF2_TRY(require_init());
+  Space3 s;
+  WF2_TRY(load_space3(v, &s));
+  return compare_nd(op, s, x, y, out, then_value, else_value);
+}
+
+#define WF2_DEFINE_COMPARE_1D(name, OP)                                                          \
+  WF2_API int wf2hip_s##name(long n, const float* x, long incx, const float* y, long incy,       \
+                             float* out, long inco, float then_value, float else_value) {        \
+    WF2_TRY(require_init());                                                                     \
+    if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");                             \
+    Space3 s;                                                                                    \
+    s.rank = 1;                                                                                  \
+    s.shape[0] = n;                                                                              \
+    s.sa[0] = incx;                                                                              \
+    s.sb[0] = incy;                                                                              \
+    s.sc[0] = inco;                                                                              \
+    s.total = n;                                                                                 \
+    return compare_nd(OP, s, x, y, out, then_value, else_value);                                 \
+  }
+
+WF2_DEFINE_COMPARE_1D(eq, WF2HIP_EQ)
+WF2_DEFINE_COMPARE_1D(lt, WF2HIP_LT)
+WF2_DEFINE_COMPARE_1D(le, WF2HIP_LE)
+WF2_DEFINE_COMPARE_1D(gt, WF2HIP_GT)
+WF2_DEFINE_COMPARE_1D(ge, WF2HIP_GE)

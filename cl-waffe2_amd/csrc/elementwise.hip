@@ -67,6 +67,26 @@ struct OpPow {
   __device__ __forceinline__ float operator()(float, float s) const { return powf_(s, p); }
 };
 
+// (x OP y) ? then : else with a scalar y: Where-Operation-Node's kernel
+// (cl-waffe2-simd.c:474-513).  All five predicates are the ordered ones: false
+// when x or y is NaN.
+struct OpWhere {
+  static constexpr int kFlatU = 4;
+  int op;
+  float y, then_value, else_value;
+  __device__ __forceinline__ float operator()(float, float s) const {
+    bool t;
+    switch (op) {
+      case WF2HIP_EQ: t = s == y; break;
+      case WF2HIP_LT: t = s < y; break;
+      case WF2HIP_LE: t = s <= y; break;
+      case WF2HIP_GT: t = s > y; break;
+      default: t = s >= y; break;
+    }
+    return t ? then_value : else_value;
+  }
+};
+
 // ---- flat kernel -------------------------------------------------------------
 // Both tensors one contiguous run (or src a single broadcast value): the node
 // the reference flattens to a single 1-D call (do-compiled-loop.lisp:113-137).
@@ -663,6 +683,27 @@ int unary_nd(int op, Space s, const float* x, float* out, float p) {
   }
 }
 
+// out <- (x OP scal) ? then : else; x on the view's `a` side, out on `b`.
+int where_nd(int op, Space s, const float* x, float* out, float scal, float then_value,
+             float else_value) {
+  if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
+  if (s.total == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  for (int r = 0; r < s.rank; r++) {
+    int64_t t = s.sa[r];
+    s.sa[r] = s.sb[r];
+    s.sb[r] = t;
+  }
+  int64_t t = s.off_a;
+  s.off_a = s.off_b;
+  s.off_b = t;
+  normalise(&s);
+  if (hazardous_overlap(s, out, x))
+    return fail(WF2HIP_EOVERLAP, "compare between partially overlapping windows");
+  if (has_broadcast_axis(s, s.sa)) keep_last_write(&s);
+  return launch_elementwise<OpWhere, false>(s, out, x, OpWhere{op, scal, then_value, else_value});
+}
+
 static int space_1d(long n, long inca, long incb, Space* s) {
   if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
   s->rank = 1;
@@ -734,3 +775,26 @@ WF2_API int wf2hip_spow(long n, const float* x, long incx, float p, float* out, 
   WF2_TRY(space_1d(n, incx, inco, &s));
   return unary_nd(WF2HIP_POW, s, x, out, p);
 }
+
+WF2_API int wf2hip_where_nd(int op, const wf2hip_view2* v, const float* x, float* out, float scal,
+                            float then_value, float else_value) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  return where_nd(op, s, x, out, scal, then_value, else_value);
+}
+
+#define WF2_DEFINE_WHERE_1D(name, OP)                                                            \
+  WF2_API int wf2hip_s##name##_scal(long n, const float* x, long incx, float* out, long inco,   \
+                                    float y, float then_value, float else_value) {              \
+    WF2_TRY(require_init());                                                                     \
+    Space s;                                                                                     \
+    WF2_TRY(space_1d(n, incx, inco, &s));                                                        \
+    return where_nd(OP, s, x, out, y, then_value, else_value);                                   \
+  }
+
+WF2_DEFINE_WHERE_1D(eq, WF2HIP_EQ)
+WF2_DEFINE_WHERE_1D(lt, WF2HIP_LT)
+WF2_DEFINE_WHERE_1D(le, WF2HIP_LE)
+WF2_DEFINE_WHERE_1D(gt, WF2HIP_GT)
+WF2_DEFINE_WHERE_1D(ge, WF2HIP_GE)

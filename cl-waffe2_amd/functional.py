@@ -242,6 +242,59 @@ def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:
 
 
 # ---------------------------------------------------------------------------
+# compare / where (source/base-impl/logical.lisp)
+# ---------------------------------------------------------------------------
+
+def where(x: HIPTensor, condition: str, scal: float, true_then: float = 1.0, false_then: float = 0.0,
+          out: HIPTensor | None = None) -> HIPTensor:
+    """``(!where x #'(lambda (e) (condition e scal)) ...)`` for the five
+    predicates with a device kernel (``logical.lisp:65-110``): ``out_i`` is
+    ``true_then`` where ``x_i condition scal`` holds, else ``false_then``."""
+    if out is None:
+        out = HIPTensor(x.shape, initial_element=None)
+    return nodes.forward("Where-Operation-Node", x, out, condition, float(scal), true_then, false_then)
+
+
+def compare(x: HIPTensor, y: HIPTensor, condition: str, true_then: float = 1.0,
+            false_then: float = 0.0, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!compare x y condition ...)`` (``logical.lisp:112-156``)."""
+    if out is None:
+        out = HIPTensor(x.shape, initial_element=None)
+    return nodes.forward("Compare-Operation-Node", x, y, out, condition, true_then, false_then)
+
+
+def _scal_cmp(condition):
+    def f(a: HIPTensor, scal: float, out: HIPTensor | None = None, true_then: float = 1.0,
+          false_then: float = 0.0) -> HIPTensor:
+        return where(a, condition, scal, true_then, false_then, out)
+    f.__doc__ = f"``(A{condition}scal A scal)`` (``logical.lisp:162-194``)."
+    return f
+
+
+def _mat_cmp(condition):
+    def f(a: HIPTensor, b: HIPTensor, out: HIPTensor | None = None, true_then: float = 1.0,
+          false_then: float = 0.0) -> HIPTensor:
+        return compare(a, b, condition, true_then, false_then, out)
+    f.__doc__ = f"``(A{condition}B A B)`` (``logical.lisp:196-225``)."
+    return f
+
+
+a_gt_scal, a_lt_scal, a_ge_scal, a_le_scal, a_eq_scal = (_scal_cmp(c) for c in (">", "<", ">=", "<=", "="))
+a_gt_b, a_lt_b, a_ge_b, a_le_b, a_eq_b = (_mat_cmp(c) for c in (">", "<", ">=", "<=", "="))
+
+
+def relu(x: HIPTensor) -> HIPTensor:
+    """``(!relu x)`` = ``(!mul x (A>scal x 0.0))`` (``source/nn/activation.lisp:15-26``)."""
+    return mul(x, a_gt_scal(x, 0.0))
+
+
+def sigmoid(x: HIPTensor) -> HIPTensor:
+    """``(!sigmoid x)`` = ``(!div 1 (!add 1 (!exp (!mul -1 x))))``
+    (``source/nn/activation.lisp:28-43``)."""
+    return div(1.0, add(1.0, exp(mul(-1.0, x))))
+
+
+# ---------------------------------------------------------------------------
 # reductions
 # ---------------------------------------------------------------------------
 

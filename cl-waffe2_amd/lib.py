@@ -20,6 +20,8 @@ MAX_RANK = 8
 ADD, SUB, MUL, DIV, MOVE = 0, 1, 2, 3, 4
 SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
 POW, GELU = 32, 40
+EQ, LT, LE, GT, GE = 0, 1, 2, 3, 4  # enum wf2hip_compare_op
+COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")
 
 EOVERLAP = -3
 ECAPTURE = -6
@@ -54,6 +56,17 @@ class View2(C.Structure):
 _P = C.c_void_p
 _L = C.c_long
 _F = C.c_float
+
+
+class View3(C.Structure):
+    """``struct wf2hip_view3``"""
+
+    _fields_ = [
+        ("rank", C.c_int32), ("reserved", C.c_int32),
+        ("shape", C.c_int64 * 8), ("stride_a", C.c_int64 * 8), ("stride_b", C.c_int64 * 8),
+        ("stride_c", C.c_int64 * 8),
+        ("off_a", C.c_int64), ("off_b", C.c_int64), ("off_c", C.c_int64),
+    ]
 
 
 class MatmulDesc(C.Structure):
@@ -138,6 +151,12 @@ _SIGNATURES = {
         C.c_int,
     ),
     "wf2hip_matmul_fused": ([C.POINTER(MatmulDesc), _P, _P, _P], C.c_int),
+    "wf2hip_where_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F, _F, _F], C.c_int),
+    "wf2hip_compare_nd": ([C.c_int, C.POINTER(View3), _P, _P, _P, _F, _F], C.c_int),
+    **{f"wf2hip_s{n}": ([_L, _P, _L, _P, _L, _P, _L, _F, _F], C.c_int)
+       for n in ("eq", "lt", "le", "gt", "ge")},
+    **{f"wf2hip_s{n}_scal": ([_L, _P, _L, _P, _L, _F, _F, _F], C.c_int)
+       for n in ("eq", "lt", "le", "gt", "ge")},
     "wf2hip_attention_f32": ([C.POINTER(AttentionDesc), _P, _P, _P, _P], C.c_int),
     "wf2hip_sgemm_strided_batched_2d": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],

@@ -56,6 +56,26 @@
 (defcfun "wf2hip_softmax_rows_f32" :int (rows :long) (cols :long) (x :pointer) (ldx :long) (out :pointer) (ldo :long))
 (defcfun "wf2hip_layernorm_rows_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (b :pointer) (eps :float) (out :pointer))
 
+;; struct wf2hip_view3 and the compare kernels (counterparts of waffe2_s{eq,lt,le,gt,ge}[_scal],
+;; cl-waffe2-simd/api.lisp:143-209)
+(defcstruct view3
+  (rank :int32)
+  (reserved :int32)
+  (shape :int64 :count 8)
+  (stride-a :int64 :count 8)
+  (stride-b :int64 :count 8)
+  (stride-c :int64 :count 8)
+  (off-a :int64)
+  (off-b :int64)
+  (off-c :int64))
+(defcfun "wf2hip_where_nd" :int
+  (op :int) (view (:pointer (:struct view2))) (x :pointer) (out :pointer)
+  (scal :float) (then-value :float) (else-value :float))
+(defcfun "wf2hip_compare_nd" :int
+  (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
+  (then-value :float) (else-value :float))
+(defconstant +eq+ 0) (defconstant +lt+ 1) (defconstant +le+ 2) (defconstant +gt+ 3) (defconstant +ge+ 4)
+
 ;; Extensions without a BLAS / SIMD-extension counterpart.  cl-waffe2 reaches them through its own
 ;; extension points: a define-bypass rule (source/vm/nodes/symbolic.lisp:118-131) or a define-op node
 ;; like Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90).

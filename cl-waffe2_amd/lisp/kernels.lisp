@@ -93,6 +93,70 @@ These are exactly the numbers call-with-view computes per axis
                           (declare (ignore self))
                           (run-unary +pow+ x out (tensor-vec n))))
 
+;; OUT <- (X cond scal) ? then : else and OUT <- (X cond Y) ? then : else
+;; (source/base-impl/logical.lisp:12-62).  Like the CPU backend's SIMD path
+;; (source/backends/cpu/logical.lisp:3-84) only the predicates < <= > >= = have a kernel; any
+;; other condition is rejected so that the node falls through to the next device.
+(defun condition->op (condition)
+  (cond ((eql condition #'<) +lt+) ((eql condition #'<=) +le+) ((eql condition #'>) +gt+)
+        ((eql condition #'>=) +ge+) ((eql condition #'=) +eq+)))
+
+(defun where-reject-p (&rest args &key &allow-other-keys)
+  "Where-Operation-Node carries its predicate and scalar in :compiler-info (logical.lisp:162-194)."
+  (let ((info (car (last args))))
+    (not (and (consp info) (condition->op (car info))))))
+
+(defun compare-reject-p (&rest args)
+  (not (condition->op (car args))))
+
+(define-impl-op (Where-Operation-Node :device HIPTensor :reject-p #'where-reject-p)
+                :forward ((self x out)
+                          (ensure-extension)
+                          (destructuring-bind (condition scal &rest more)
+                              (cl-waffe2/base-impl::logical-compiler-info self)
+                            (declare (ignore more))
+                            (with-foreign-object (view '(:struct view2))
+                              (fill-view2 view x out)
+                              (check (wf2hip-where-nd
+                                      (condition->op condition) view
+                                      (tensor-device-pointer x) (tensor-device-pointer out)
+                                      (coerce scal 'single-float)
+                                      (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
+                                      (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float)))))
+                          out))
+
+(defun fill-view3 (view x y out)
+  "Like fill-view2 for three tensors: X and Y go through a view2 each paired with OUT."
+  (with-foreign-objects ((xo '(:struct view2)) (yo '(:struct view2)))
+    (fill-view2 xo x out)
+    (fill-view2 yo y out)
+    (setf (foreign-slot-value view '(:struct view3) 'rank) (foreign-slot-value xo '(:struct view2) 'rank))
+    (dotimes (axis (length (shape out)))
+      (flet ((copy-slot (to from-view from)
+               (setf (mem-aref (foreign-slot-pointer view '(:struct view3) to) :int64 axis)
+                     (mem-aref (foreign-slot-pointer from-view '(:struct view2) from) :int64 axis))))
+        (copy-slot 'shape xo 'shape)
+        (copy-slot 'stride-a xo 'stride-a)
+        (copy-slot 'stride-b yo 'stride-a)
+        (copy-slot 'stride-c xo 'stride-b)))
+    (setf (foreign-slot-value view '(:struct view3) 'off-a) (foreign-slot-value xo '(:struct view2) 'off-a)
+          (foreign-slot-value view '(:struct view3) 'off-b) (foreign-slot-value yo '(:struct view2) 'off-a)
+          (foreign-slot-value view '(:struct view3) 'off-c) (foreign-slot-value xo '(:struct view2) 'off-b)))
+  view)
+
+(define-impl-op (Compare-Operation-Node :device HIPTensor :reject-p #'compare-reject-p)
+                :forward ((self x y out)
+                          (ensure-extension)
+                          (with-foreign-object (view '(:struct view3))
+                            (fill-view3 view x y out)
+                            (check (wf2hip-compare-nd
+                                    (condition->op (cl-waffe2/base-impl::logical-condition self)) view
+                                    (tensor-device-pointer x) (tensor-device-pointer y)
+                                    (tensor-device-pointer out)
+                                    (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
+                                    (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float))))
+                          out))
+
 ;; C[~ i k] = A[~ i j] . B[~ j k].  Same operand swap as expand-gemm-form-column
 ;; (source/backends/cpu/matrix-ops.lisp:12-112): a row-major product is the column-major
 ;; sgemm(transB, transA, n, m, k, 1, B, ldb, A, lda, 0, C, ldc).  Batch axes are walked on the

@@ -30,6 +30,7 @@ NODE_NAMES = (
     "AddNode", "SubNode", "MulNode", "DivNode", "MoveTensorNode",
     "SinNode", "CosNode", "TanhNode", "LogENode", "ExpNode", "SqrtNode", "AbsNode",
     "ExptNode", "MatMulNode",
+    "Where-Operation-Node", "Compare-Operation-Node",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -139,6 +140,58 @@ for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _l
 def _expt(x: HIPTensor, out: HIPTensor, n: float) -> HIPTensor:
     v = view2(x, out)
     _lib.check(_lib.get().wf2hip_unary_nd(_lib.POW, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(n)))
+    return out
+
+
+_CONDITIONS = {"=": _lib.EQ, "==": _lib.EQ, "<": _lib.LT, "<=": _lib.LE, ">": _lib.GT, ">=": _lib.GE}
+
+
+def _condition(op) -> int:
+    """The five predicates the SIMD extension implements
+    (``backends/cpu/logical.lisp:26-33``); anything else has no device kernel."""
+    if op in _CONDITIONS:
+        return _CONDITIONS[op]
+    raise NodeNotFound(f"no HIPTensor kernel for condition {op!r} (supported: = < <= > >=)")
+
+
+@define_impl("Where-Operation-Node", HIPTensor, _only_float)
+def _where(x: HIPTensor, out: HIPTensor, condition, scal: float, true_then: float = 1.0,
+           false_then: float = 0.0) -> HIPTensor:
+    """``out <- (x condition scal) ? true-then : false-then``
+    (``backends/cpu/logical.lisp:37-60``)."""
+    v = view2(x, out)
+    _lib.check(_lib.get().wf2hip_where_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
+                                          C.c_void_p(out.ptr), float(scal), float(true_then),
+                                          float(false_then)))
+    return out
+
+
+def view3(a: HIPTensor, b: HIPTensor, c: HIPTensor) -> _lib.View3:
+    sa, sta, oa = a.geometry()
+    sb, stb, ob = b.geometry()
+    sc, stc, oc = c.geometry()
+    if not (sa == sb == sc):
+        raise ValueError(f"shape mismatch: {sa}, {sb} and {sc}")
+    v = _lib.View3()
+    v.rank = len(sa)
+    for r, (n, x, y, z) in enumerate(zip(sa, sta, stb, stc)):
+        v.shape[r] = n
+        v.stride_a[r] = x
+        v.stride_b[r] = y
+        v.stride_c[r] = z
+    v.off_a, v.off_b, v.off_c = oa, ob, oc
+    return v
+
+
+@define_impl("Compare-Operation-Node", HIPTensor, _only_float)
+def _compare(x: HIPTensor, y: HIPTensor, out: HIPTensor, condition, true_then: float = 1.0,
+             false_then: float = 0.0) -> HIPTensor:
+    """``out <- (x condition y) ? true-then : false-then``
+    (``backends/cpu/logical.lisp:62-84``)."""
+    v = view3(x, y, out)
+    _lib.check(_lib.get().wf2hip_compare_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
+                                            C.c_void_p(y.ptr), C.c_void_p(out.ptr),
+                                            float(true_then), float(false_then)))
     return out
 
 

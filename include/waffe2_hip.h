@@ -183,6 +183,56 @@ int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b);
  * 8-76).  `p` is the exponent for WF2HIP_POW and ignored otherwise. */
 int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p);
 
+/* ---- compare / where ---------------------------------------------------- */
+/* out <- (x OP y) ? then_value : else_value.  OP is ordered: false when an
+ * operand is NaN (the reference uses _CMP_*_OQ, avx2.h:179-230). */
+enum wf2hip_compare_op { WF2HIP_EQ = 0, WF2HIP_LT = 1, WF2HIP_LE = 2, WF2HIP_GT = 3, WF2HIP_GE = 4 };
+
+/* 1-D forms.  Replace waffe2_s{eq,lt,le,gt,ge} (cl-waffe2-simd.c:385-468;
+ * api.lisp:143-175) and waffe2_s{eq,lt,le,gt,ge}_scal (cl-waffe2-simd.c:474-560;
+ * api.lisp:177-209), same argument order.  With inco == 0 `out` keeps the last
+ * element's result, as the reference's sequential loop leaves it. */
+int wf2hip_seq(long n, const float* x, long incx, const float* y, long incy, float* out, long inco,
+               float then_value, float else_value);
+int wf2hip_slt(long n, const float* x, long incx, const float* y, long incy, float* out, long inco,
+               float then_value, float else_value);
+int wf2hip_sle(long n, const float* x, long incx, const float* y, long incy, float* out, long inco,
+               float then_value, float else_value);
+int wf2hip_sgt(long n, const float* x, long incx, const float* y, long incy, float* out, long inco,
+               float then_value, float else_value);
+int wf2hip_sge(long n, const float* x, long incx, const float* y, long incy, float* out, long inco,
+               float then_value, float else_value);
+int wf2hip_seq_scal(long n, const float* x, long incx, float* out, long inco, float y,
+                    float then_value, float else_value);
+int wf2hip_slt_scal(long n, const float* x, long incx, float* out, long inco, float y,
+                    float then_value, float else_value);
+int wf2hip_sle_scal(long n, const float* x, long incx, float* out, long inco, float y,
+                    float then_value, float else_value);
+int wf2hip_sgt_scal(long n, const float* x, long incx, float* out, long inco, float y,
+                    float then_value, float else_value);
+int wf2hip_sge_scal(long n, const float* x, long incx, float* out, long inco, float y,
+                    float then_value, float else_value);
+
+/* Three tensors over one iteration space (a = X, b = Y, c = OUT), in elements. */
+typedef struct wf2hip_view3 {
+  int32_t rank; /* 1..WF2HIP_MAX_RANK */
+  int32_t reserved;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t stride_a[WF2HIP_MAX_RANK];
+  int64_t stride_b[WF2HIP_MAX_RANK];
+  int64_t stride_c[WF2HIP_MAX_RANK];
+  int64_t off_a, off_b, off_c;
+} wf2hip_view3;
+
+/* N-D forms, one launch per node.  wf2hip_where_nd replaces the forward of
+ * Where-Operation-Node (source/backends/cpu/logical.lisp:37-60; view: a = X,
+ * b = OUT), wf2hip_compare_nd that of Compare-Operation-Node (logical.lisp:
+ * 62-84).  Stride-0 axes of OUT keep the last element written. */
+int wf2hip_where_nd(int op, const wf2hip_view2* v, const float* x, float* out, float scal,
+                    float then_value, float else_value);
+int wf2hip_compare_nd(int op, const wf2hip_view3* v, const float* x, const float* y, float* out,
+                      float then_value, float else_value);
+
 /* 0 (default): parallel tree reduction for accumulate-into-stride-0 ADD.
  * 1: the reference's strictly sequential fp32 order (slow; for bit parity). */
 int wf2hip_set_reduce_mode(int mode);

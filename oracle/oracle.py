@@ -109,6 +109,16 @@ def lib():
         f = getattr(L, "orc_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F]
         f.restype = None
+    L.orc_scmp.argtypes = [C.c_int, C.c_long, _F, C.c_long, _F, C.c_long, _F, C.c_long,
+                           C.c_float, C.c_float]
+    L.orc_scmp.restype = None
+    L.orc_scmp_scal.argtypes = [C.c_int, C.c_long, _F, C.c_long, _F, C.c_long, C.c_float,
+                                C.c_float, C.c_float]
+    L.orc_scmp_scal.restype = None
+    L.orc_where_nd.argtypes = [C.c_int, C.POINTER(OrcViews), _F, _F, C.c_float, C.c_float, C.c_float]
+    L.orc_where_nd.restype = C.c_long
+    L.orc_compare_nd.argtypes = [C.c_int, C.POINTER(OrcViews), _F, _F, _F, C.c_float, C.c_float]
+    L.orc_compare_nd.restype = C.c_long
     L.orc_schedule.argtypes = [C.POINTER(OrcViews), C.POINTER(OrcCall), C.c_long]
     L.orc_schedule.restype = C.c_long
     L.orc_node_nd.argtypes = [C.c_int, C.POINTER(OrcViews), _F, _F, C.c_float]
@@ -153,6 +163,13 @@ def ref():
         f.restype = None
     R.waffe2_spow.argtypes = [C.c_long, _F, C.c_long, C.c_float, _F, C.c_long]
     R.waffe2_spow.restype = None
+    for name in CMP_OPS:
+        f = getattr(R, "waffe2_s" + name)
+        f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long, _F, C.c_long, C.c_float, C.c_float]
+        f.restype = None
+        f = getattr(R, "waffe2_s" + name + "_scal")
+        f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long, C.c_float, C.c_float, C.c_float]
+        f.restype = None
     for name in ("max", "min"):
         f = getattr(R, "waffe2_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F]
@@ -189,6 +206,45 @@ def pow_1d(n: int, x: np.ndarray, incx: int, p: float, out: np.ndarray, inco: in
     L = ref() if use_ref else lib()
     name = "waffe2_spow" if use_ref else "orc_spow"
     getattr(L, name)(n, _fp(x), incx, C.c_float(p), _fp(out), inco)
+
+
+CMP_OPS = ("eq", "lt", "le", "gt", "ge")  # enum order of orc_scmp / wf2hip compare ops
+
+
+def cmp_1d(op: str, n: int, x: np.ndarray, incx: int, y: np.ndarray, incy: int, out: np.ndarray,
+           inco: int, then: float = 1.0, els: float = 0.0, use_ref: bool = False) -> None:
+    """out <- (x OP y) ? then : els (waffe2_s{eq,lt,le,gt,ge})."""
+    if use_ref:
+        getattr(ref(), "waffe2_s" + op)(n, _fp(x), incx, _fp(y), incy, _fp(out), inco,
+                                        C.c_float(then), C.c_float(els))
+    else:
+        lib().orc_scmp(CMP_OPS.index(op), n, _fp(x), incx, _fp(y), incy, _fp(out), inco,
+                       C.c_float(then), C.c_float(els))
+
+
+def cmp_scal_1d(op: str, n: int, x: np.ndarray, incx: int, out: np.ndarray, inco: int, y: float,
+                then: float = 1.0, els: float = 0.0, use_ref: bool = False) -> None:
+    """out <- (x OP y) ? then : els with a scalar y (waffe2_s{eq,...}_scal)."""
+    if use_ref:
+        getattr(ref(), "waffe2_s" + op + "_scal")(n, _fp(x), incx, _fp(out), inco, C.c_float(y),
+                                                  C.c_float(then), C.c_float(els))
+    else:
+        lib().orc_scmp_scal(CMP_OPS.index(op), n, _fp(x), incx, _fp(out), inco, C.c_float(y),
+                            C.c_float(then), C.c_float(els))
+
+
+def where_nd(op: str, views: OrcViews, x: np.ndarray, out: np.ndarray, scal: float,
+             then: float = 1.0, els: float = 0.0) -> None:
+    rc = lib().orc_where_nd(CMP_OPS.index(op), C.byref(views), _fp(x), _fp(out), C.c_float(scal),
+                            C.c_float(then), C.c_float(els))
+    assert rc == 0
+
+
+def compare_nd(op: str, views: OrcViews, x: np.ndarray, y: np.ndarray, out: np.ndarray,
+               then: float = 1.0, els: float = 0.0) -> None:
+    rc = lib().orc_compare_nd(CMP_OPS.index(op), C.byref(views), _fp(x), _fp(y), _fp(out),
+                              C.c_float(then), C.c_float(els))
+    assert rc == 0
 
 
 def maxmin_1d(op: str, n: int, x: np.ndarray, incx: int, use_ref: bool = False) -> float:

@@ -426,6 +426,104 @@ ORC_API long orc_node_nd(int op, const orc_views *v, float *t0, float *t1,
 }
 
 /* ------------------------------------------------------------------ */
+/* compare / where                                                     */
+/* ------------------------------------------------------------------ */
+/* out[i] = (x[i] OP y[i]) ? then : else  (cl-waffe2-simd.c:385-425, define_cmp)
+ * and the scalar-right-hand-side form (cl-waffe2-simd.c:474-513, define_scmp).
+ * The SIMD predicates are the ordered, quiet ones (avx2.h:179,192,205,218,230:
+ * _CMP_EQ_OQ 0, _CMP_LT_OQ 17, _CMP_LE_OQ 18, _CMP_GE_OQ 29, _CMP_GT_OQ 30), i.e. what
+ * the C operators of the scalar tail give: false whenever an operand is NaN.
+ * With inco < 1 the block-of-8 part is skipped and every element is written
+ * through the scalar loop, so a stride-0 `out` ends up holding the last one. */
+enum { ORC_EQ = 0, ORC_LT, ORC_LE, ORC_GT, ORC_GE };
+
+static int orc_cmp1(int op, float a, float b) {
+  switch (op) {
+    case ORC_EQ: return a == b;
+    case ORC_LT: return a < b;
+    case ORC_LE: return a <= b;
+    case ORC_GT: return a > b;
+    default: return a >= b;
+  }
+}
+
+ORC_API void orc_scmp(int op, long n, const float *x, long incx, const float *y, long incy,
+                      float *out, long inco, float then_value, float else_value) {
+  long count = 0;
+  if (inco >= 1) {
+    const long blocks_end = (n / 8) * 8;
+    for (; count != blocks_end; count += 8) {
+      float res[8];
+      for (int l = 0; l < 8; l++)
+        res[l] = orc_cmp1(op, x[(count + l) * incx], y[(count + l) * incy]) ? then_value : else_value;
+      for (int l = 0; l < 8; l++) out[(count + l) * inco] = res[l];
+    }
+  }
+  for (; count != n; count++)
+    out[count * inco] = orc_cmp1(op, x[count * incx], y[count * incy]) ? then_value : else_value;
+}
+
+ORC_API void orc_scmp_scal(int op, long n, const float *x, long incx, float *out, long inco,
+                           float y, float then_value, float else_value) {
+  long count = 0;
+  if (inco >= 1) {
+    const long blocks_end = (n / 8) * 8;
+    for (; count != blocks_end; count += 8) {
+      float res[8];
+      for (int l = 0; l < 8; l++)
+        res[l] = orc_cmp1(op, x[(count + l) * incx], y) ? then_value : else_value;
+      for (int l = 0; l < 8; l++) out[(count + l) * inco] = res[l];
+    }
+  }
+  for (; count != n; count++)
+    out[count * inco] = orc_cmp1(op, x[count * incx], y) ? then_value : else_value;
+}
+
+/* Where-Operation-Node / Compare-Operation-Node over N-D views: the schedule of
+ * do-compiled-loop with one 1-D call per row (backends/cpu/logical.lisp:37-84). */
+typedef struct {
+  int op;
+  const float *x;
+  const float *y;
+  float *out;
+  float scal, then_value, else_value;
+} cmp_ctx;
+
+static void where_emit(const orc_call *c, void *p) {
+  cmp_ctx *e = (cmp_ctx *)p;
+  orc_scmp_scal(e->op, c->n, e->x + c->off[0], c->inc[0], e->out + c->off[1], c->inc[1], e->scal,
+                e->then_value, e->else_value);
+}
+
+static void compare_emit(const orc_call *c, void *p) {
+  cmp_ctx *e = (cmp_ctx *)p;
+  orc_scmp(e->op, c->n, e->x + c->off[0], c->inc[0], e->y + c->off[1], c->inc[1],
+           e->out + c->off[2], c->inc[2], e->then_value, e->else_value);
+}
+
+/* tensors of `v`: 0 = x, 1 = out */
+ORC_API long orc_where_nd(int op, const orc_views *v, const float *x, float *out, float scal,
+                          float then_value, float else_value) {
+  cmp_ctx e = {op, x, NULL, out, scal, then_value, else_value};
+  long offsets[ORC_MAX_TENSORS];
+  if (v->rank == 0 || v->ntensors != 2) return -1;
+  for (int t = 0; t < v->ntensors; t++) offsets[t] = v->offset[t];
+  emit_rec(v, 0, offsets, where_emit, &e);
+  return 0;
+}
+
+/* tensors of `v`: 0 = x, 1 = y, 2 = out */
+ORC_API long orc_compare_nd(int op, const orc_views *v, const float *x, const float *y, float *out,
+                            float then_value, float else_value) {
+  cmp_ctx e = {op, x, y, out, 0.0f, then_value, else_value};
+  long offsets[ORC_MAX_TENSORS];
+  if (v->rank == 0 || v->ntensors != 3) return -1;
+  for (int t = 0; t < v->ntensors; t++) offsets[t] = v->offset[t];
+  emit_rec(v, 0, offsets, compare_emit, &e);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
 /* sgemm                                                               */
 /* ------------------------------------------------------------------ */
 /* Column-major C(m x n) <- alpha*op(A)*op(B) + beta*C with Fortran sgemm_

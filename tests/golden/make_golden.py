@@ -90,5 +90,43 @@ def main():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "simd_kernels.npz")), "bytes")
 
 
+CMP_REGIMES = [(1, 1, 1), (1, 0, 1), (2, 1, 1), (1, 3, 2), (2, 2, 3), (0, 1, 1), (1, 1, 0), (3, 0, 0)]
+CMP_EDGE = np.array([0.0, -0.0, 1.0, -1.0, np.nan, np.inf, -np.inf, 1e-45, -1e-45, 3.4e38, 0.5, 2.0,
+                     -2.0, 1.0000001, 0.99999994, 7.0], np.float32)
+
+
+def compare_goldens():
+    """out <- (x OP y) ? then : else for the five predicates, tensor and scalar
+    right-hand sides (waffe2_s{eq,lt,le,gt,ge}[_scal]), every stride regime
+    incl. a stride-0 `out`, and a table of special values against each other."""
+    rng = np.random.Generator(np.random.PCG64(2025))
+    out = {}
+    for op in O.CMP_OPS:
+        for n in (1, 7, 8, 9, 31, 67):
+            for incx, incy, inco in CMP_REGIMES:
+                size = n * 3 + 1
+                # small integers so that equality happens
+                x = rng.integers(-3, 4, size).astype(np.float32)
+                y = rng.integers(-3, 4, size).astype(np.float32)
+                res = np.full(size, 9.0, np.float32)
+                O.cmp_1d(op, n, x, incx, y, incy, res, inco, 2.5, -1.5, use_ref=True)
+                key = f"cmp_{op}_{n}_{incx}_{incy}_{inco}"
+                out[key + "_x"], out[key + "_y"], out[key + "_out"] = x, y, res
+                res = np.full(size, 9.0, np.float32)
+                O.cmp_scal_1d(op, n, x, incx, res, inco, 1.0, 2.5, -1.5, use_ref=True)
+                out[key + "_scal_out"] = res
+        # every special value against every other one
+        xs = np.repeat(CMP_EDGE, CMP_EDGE.size)
+        ys = np.tile(CMP_EDGE, CMP_EDGE.size)
+        res = np.zeros(xs.size, np.float32)
+        O.cmp_1d(op, xs.size, xs, 1, ys, 1, res, 1, 1.0, 0.0, use_ref=True)
+        out[f"cmp_{op}_edge_out"] = res
+    out["cmp_edge"] = CMP_EDGE
+    np.savez_compressed(os.path.join(HERE, "compare_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "compare_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
-    main()
+    if "--compare-only" not in sys.argv:
+        main()
+    compare_goldens()

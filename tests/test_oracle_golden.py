@@ -195,3 +195,53 @@ def test_gemm_against_float64(O):
             got = Cm.copy().ravel()
             O.sgemm(ta, tb, m, n, k, 0.5, A.ravel(), A.shape[1], B.ravel(), B.shape[1], 2.0, got, m)
             np.testing.assert_allclose(got.reshape(n, m).T, want, rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# compare / where (cl-waffe2-simd.c:385-513)
+# ---------------------------------------------------------------------------
+CMP_GOLD = os.path.join(os.path.dirname(__file__), "golden", "compare_kernels.npz")
+CMP_REGIMES = [(1, 1, 1), (1, 0, 1), (2, 1, 1), (1, 3, 2), (2, 2, 3), (0, 1, 1), (1, 1, 0), (3, 0, 0)]
+CMP_NUMPY = {"eq": np.equal, "lt": np.less, "le": np.less_equal, "gt": np.greater, "ge": np.greater_equal}
+
+
+@pytest.fixture(scope="module")
+def cmp_gold():
+    return np.load(CMP_GOLD)
+
+
+@pytest.mark.parametrize("op", ["eq", "lt", "le", "gt", "ge"])
+def test_compare_golden(O, cmp_gold, op):
+    """Tensor and scalar right-hand sides, every stride regime (a stride-0 `out`
+    keeps the last element's result), bitwise against the compiled reference's
+    outputs."""
+    for n in (1, 7, 8, 9, 31, 67):
+        for incx, incy, inco in CMP_REGIMES:
+            key = f"cmp_{op}_{n}_{incx}_{incy}_{inco}"
+            x, y = cmp_gold[key + "_x"], cmp_gold[key + "_y"]
+            got = np.full(x.size, 9.0, np.float32)
+            O.cmp_1d(op, n, x, incx, y, incy, got, inco, 2.5, -1.5)
+            assert_bit_equal(got, cmp_gold[key + "_out"], key)
+            got = np.full(x.size, 9.0, np.float32)
+            O.cmp_scal_1d(op, n, x, incx, got, inco, 1.0, 2.5, -1.5)
+            assert_bit_equal(got, cmp_gold[key + "_scal_out"], key + " scal")
+            # what the definition fixes, where `out` is not collapsed
+            if inco >= 1:
+                xs = x[::incx][:n] if incx else np.repeat(x[0], n)
+                ys = y[::incy][:n] if incy else np.repeat(y[0], n)
+                want = np.where(CMP_NUMPY[op](xs, ys), np.float32(2.5), np.float32(-1.5))
+                assert_bit_equal(cmp_gold[key + "_out"][::inco][:n], want, key + " numpy")
+
+
+@pytest.mark.parametrize("op", ["eq", "lt", "le", "gt", "ge"])
+def test_compare_special_values(O, cmp_gold, op):
+    """NaN compares false under every predicate, -0 == +0, infinities order."""
+    edge = cmp_gold["cmp_edge"]
+    xs, ys = np.repeat(edge, edge.size), np.tile(edge, edge.size)
+    got = np.zeros(xs.size, np.float32)
+    O.cmp_1d(op, xs.size, xs, 1, ys, 1, got, 1, 1.0, 0.0)
+    assert_bit_equal(got, cmp_gold[f"cmp_{op}_edge_out"], op)
+    with np.errstate(invalid="ignore"):
+        assert_bit_equal(got, CMP_NUMPY[op](xs, ys).astype(np.float32), op + " numpy")
+    nan_rows = np.isnan(xs) | np.isnan(ys)
+    assert not got[nan_rows].any()
