@@ -1,0 +1,266 @@
+// rowselect.hip -- largest / smallest value of a row and where it sits.
+//
+// MaxValue-Node, MinValue-Node, ArgMax-Node and ArgMin-Node
+// (source/base-impl/matrix-ops.lisp:197-470) reduce the trailing run of A and
+// write one element per row of OUT; the CPU backend calls waffe2_s{max,min} or
+// BLAS i?max / i?min once per row
+// (source/backends/cpu/matrix-ops.lisp:240-369).  Here a node is one launch: a
+// wavefront per short row, a workgroup per long row, and (row, split)
+// workgroups plus a small second pass when there are too few rows to fill the
+// chip.  HBM-bound: 4 bytes per element.
+//
+// Ties go to the lowest index (the first occurrence, what a sequential scan
+// with a strict comparison finds); NaN elements are never selected; a row of
+// NaNs gives -inf / +inf and index 0.
+#include <math.h>
+
+#include "wf2_common.h"
+#include "wf2_view.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+constexpr int kSelMaxOuter = WF2HIP_MAX_RANK;
+
+struct Best {
+  float v;
+  uint32_t i;
+};
+
+template <bool IsMax>
+__device__ __forceinline__ bool better(float v, uint32_t i, const Best& b) {
+  return IsMax ? (v > b.v || (v == b.v && i < b.i)) : (v < b.v || (v == b.v && i < b.i));
+}
+
+template <bool IsMax>
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(b.v, o);
+    const uint32_t oi = __shfl_xor(b.i, o);
+    if (better<IsMax>(ov, oi, b)) {
+      b.v = ov;
+      b.i = oi;
+    }
+  }
+  return b;
+}
+
+struct SelParams {
+  const float* x;
+  void* out;        // float for value ops, uint32_t for index ops
+  int64_t n, incx;  // the reduced run
+  uint32_t nrows;
+  int32_t nouter;
+  uint32_t oshape[kSelMaxOuter];  // kept axes, innermost of them first
+  int64_t ox[kSelMaxOuter], oo[kSelMaxOuter];
+  int32_t want_index;
+  uint32_t splits;  // workgroups per row
+  int64_t seg;      // elements per split (multiple of 4)
+  Best* partials;   // nrows * splits
+};
+
+__device__ __forceinline__ void sel_offsets(const SelParams& p, uint32_t row, int64_t* xoff,
+                                            int64_t* ooff) {
+  int64_t xo = 0, oo = 0;
+  uint32_t rem = row;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t idx;
+    if (i == p.nouter - 1) {
+      idx = rem;
+    } else {
+      const uint32_t q = rem / p.oshape[i];
+      idx = rem - q * p.oshape[i];
+      rem = q;
+    }
+    xo += (int64_t)idx * p.ox[i];
+    oo += (int64_t)idx * p.oo[i];
+  }
+  *xoff = xo;
+  *ooff = oo;
+}
+
+// best of x[lo, hi) seen by thread `t` of `nthreads`; a lane scans increasing
+// indices with a strict comparison, so it keeps the first occurrence
+template <bool IsMax, bool VEC>
+__device__ __forceinline__ Best scan(const float* __restrict__ x, int64_t incx, int64_t lo,
+                                     int64_t hi, int t, int nthreads) {
+  Best b = {IsMax ? -INFINITY : INFINITY, 0u};
+  if (VEC) {  // incx == 1, x + lo 16-byte aligned
+    const int64_t nvec = (hi - lo) / 4;
+    const f4* xv = reinterpret_cast<const f4*>(x + lo);
+    auto take = [&](const f4& v, uint32_t at) {
+      if (IsMax ? v.x > b.v : v.x < b.v) { b.v = v.x; b.i = at; }
+      if (IsMax ? v.y > b.v : v.y < b.v) { b.v = v.y; b.i = at + 1; }
+      if (IsMax ? v.z > b.v : v.z < b.v) { b.v = v.z; b.i = at + 2; }
+      if (IsMax ? v.w > b.v : v.w < b.v) { b.v = v.w; b.i = at + 3; }
+    };
+    int64_t i = t;
+    for (; i + nthreads < nvec; i += 2 * (int64_t)nthreads) {  // two loads in flight
+      const f4 v0 = __builtin_nontemporal_load(xv + i);
+      const f4 v1 = __builtin_nontemporal_load(xv + i + nthreads);
+      take(v0, (uint32_t)(lo + 4 * i));
+      take(v1, (uint32_t)(lo + 4 * (i + nthreads)));
+    }
+    if (i < nvec) take(__builtin_nontemporal_load(xv + i), (uint32_t)(lo + 4 * i));
+    for (int64_t c = lo + nvec * 4 + t; c < hi; c += nthreads) {
+      const float v = x[c];
+      if (IsMax ? v > b.v : v < b.v) { b.v = v; b.i = (uint32_t)c; }
+    }
+  } else {
+    for (int64_t c = lo + t; c < hi; c += nthreads) {
+      const float v = x[c * incx];
+      if (IsMax ? v > b.v : v < b.v) { b.v = v; b.i = (uint32_t)c; }
+    }
+  }
+  return b;
+}
+
+__device__ __forceinline__ void emit(const SelParams& p, int64_t ooff, const Best& b) {
+  if (p.want_index)
+    static_cast<uint32_t*>(p.out)[ooff] = b.i;
+  else
+    static_cast<float*>(p.out)[ooff] = b.v;
+}
+
+// one wavefront per row, four rows per workgroup
+template <bool IsMax, bool VEC>
+__global__ __launch_bounds__(kBlock) void select_rows_wave(SelParams p) {
+  const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (row >= p.nrows) return;
+  int64_t xoff, ooff;
+  sel_offsets(p, row, &xoff, &ooff);
+  Best b = scan<IsMax, VEC>(p.x + xoff, p.incx, 0, p.n, threadIdx.x & (kWave - 1), kWave);
+  b = wave_best<IsMax>(b);
+  if ((threadIdx.x & (kWave - 1)) == 0) emit(p, ooff, b);
+}
+
+// one workgroup per (row, split)
+template <bool IsMax, bool VEC>
+__global__ __launch_bounds__(kBlock) void select_rows_block(SelParams p) {
+  __shared__ Best lds[kBlock / kWave];
+  const uint32_t row = blockIdx.x / p.splits;
+  const uint32_t split = blockIdx.x - row * p.splits;
+  int64_t xoff, ooff;
+  sel_offsets(p, row, &xoff, &ooff);
+  const int64_t lo = (int64_t)split * p.seg;
+  const int64_t hi = lo + p.seg < p.n ? lo + p.seg : p.n;
+  Best b = scan<IsMax, VEC>(p.x + xoff, p.incx, lo, hi, threadIdx.x, kBlock);
+  b = wave_best<IsMax>(b);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = b;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; w++)
+      if (better<IsMax>(lds[w].v, lds[w].i, b)) b = lds[w];
+    if (p.splits == 1)
+      emit(p, ooff, b);
+    else
+      p.partials[(int64_t)row * p.splits + split] = b;
+  }
+}
+
+template <bool IsMax>
+__global__ __launch_bounds__(kBlock) void select_rows_finish(SelParams p) {
+  __shared__ Best lds[kBlock / kWave];
+  const uint32_t row = blockIdx.x;
+  int64_t xoff, ooff;
+  sel_offsets(p, row, &xoff, &ooff);
+  Best b = {IsMax ? -INFINITY : INFINITY, 0u};
+  for (uint32_t s = threadIdx.x; s < p.splits; s += kBlock) {
+    const Best c = p.partials[(int64_t)row * p.splits + s];
+    if (better<IsMax>(c.v, c.i, b)) b = c;
+  }
+  b = wave_best<IsMax>(b);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = b;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; w++)
+      if (better<IsMax>(lds[w].v, lds[w].i, b)) b = lds[w];
+    emit(p, ooff, b);
+  }
+}
+
+template <bool IsMax, bool VEC>
+static int launch_select(SelParams& p) {
+  hipStream_t st = rt().stream;
+  const int64_t target = (int64_t)rt().num_cus * 8;
+  if (p.n <= 2048 || (p.n < 8192 && p.nrows >= target)) {
+    const uint32_t blocks = (uint32_t)ceil_div(p.nrows, kBlock / kWave);
+    select_rows_wave<IsMax, VEC><<<blocks, kBlock, 0, st>>>(p);
+    return after_launch("select_rows_wave");
+  }
+  p.splits = 1;
+  p.seg = p.n;
+  if (p.nrows < target) {
+    int64_t by_work = ceil_div(p.n, 16384);
+    int64_t by_fill = ceil_div(target, p.nrows);
+    int64_t by_cap = (int64_t)(kPartialCapacity / 2) / p.nrows;  // a Best is two floats wide
+    int64_t splits = by_work < by_fill ? by_work : by_fill;
+    if (splits > by_cap) splits = by_cap;
+    if (splits < 1) splits = 1;
+    const int64_t seg = ceil_div(ceil_div(p.n, splits), 1024) * 1024;
+    p.splits = (uint32_t)ceil_div(p.n, seg);
+    p.seg = seg;
+  }
+  const int64_t blocks = (int64_t)p.nrows * p.splits;
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows for one launch");
+  select_rows_block<IsMax, VEC><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  WF2_TRY(after_launch("select_rows_block"));
+  if (p.splits > 1) {
+    select_rows_finish<IsMax><<<p.nrows, kBlock, 0, st>>>(p);
+    WF2_TRY(after_launch("select_rows_finish"));
+  }
+  return 0;
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long incx, const float* x,
+                             void* out) {
+  WF2_TRY(require_init());
+  if (op < WF2HIP_MAXVALUE || op > WF2HIP_ARGMIN) return fail(WF2HIP_EINVAL, "unknown selection op %d", op);
+  Space s;
+  WF2_TRY(load_space(outer, &s));
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative run length");
+  if (s.total == 0) return 0;
+  if (n == 0) return fail(WF2HIP_EINVAL, "cannot select from an empty run");
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  if (n >= ((int64_t)1 << 32)) return fail(WF2HIP_EUNSUPPORTED, "run longer than 2^32 - 1 elements");
+  if (s.total >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+  // a stride-0 axis of OUT keeps what the sequential loop writes last
+  for (int r = 0; r < s.rank; r++)
+    if (s.sb[r] == 0 && s.shape[r] > 1) {
+      s.off_a += s.sa[r] * (s.shape[r] - 1);
+      s.shape[r] = 1;
+    }
+  normalise(&s);
+  SelParams p;
+  p.x = x + s.off_a;
+  p.out = static_cast<char*>(out) + 4 * s.off_b;
+  p.n = n;
+  p.incx = incx;
+  p.nouter = s.rank;
+  int64_t nrows = 1;
+  bool vec = incx == 1 && ((uintptr_t)p.x & 15u) == 0;
+  for (int i = 0; i < s.rank; i++) {
+    const int r = s.rank - 1 - i;
+    if (s.shape[r] >= ((int64_t)1 << 32)) return fail(WF2HIP_EUNSUPPORTED, "axis too long");
+    p.oshape[i] = (uint32_t)s.shape[r];
+    p.ox[i] = s.sa[r];
+    p.oo[i] = s.sb[r];
+    nrows *= s.shape[r];
+    if (s.shape[r] > 1 && s.sa[r] % 4 != 0) vec = false;
+  }
+  p.nrows = (uint32_t)nrows;
+  p.want_index = op == WF2HIP_ARGMAX || op == WF2HIP_ARGMIN;
+  p.splits = 1;
+  p.seg = n;
+  p.partials = reinterpret_cast<Best*>(rt().partials);
+  const bool is_max = op == WF2HIP_MAXVALUE || op == WF2HIP_ARGMAX;
+  if (is_max) return vec ? launch_select<true, true>(p) : launch_select<true, false>(p);
+  return vec ? launch_select<false, true>(p) : launch_select<false, false>(p);
+}

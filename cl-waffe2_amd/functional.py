@@ -11,6 +11,7 @@ Naming: ``!add`` -> ``add``, ``A+=B`` -> ``add_``, ``!loge`` -> ``loge``,
 """
 from __future__ import annotations
 
+import builtins as _builtins
 import math
 from typing import Sequence
 
@@ -69,7 +70,7 @@ def reshape(x: HIPTensor, *shape: int) -> HIPTensor:
     shape = list(shape)
     if shape.count(-1) == 1:
         known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
-        shape[shape.index(-1)] = x.size // max(known, 1)
+        shape[shape.index(-1)] = x.size // _builtins.max(known, 1)
     if int(np.prod(shape, dtype=np.int64)) != x.size:
         raise ValueError(f"reshape: cannot reshape {x.shape} into {shape}")
     src = to_contiguous(x)
@@ -295,6 +296,55 @@ def sigmoid(x: HIPTensor) -> HIPTensor:
 
 
 # ---------------------------------------------------------------------------
+# max / min / argmax / argmin (source/base-impl/matrix-ops.lisp:197-470)
+# ---------------------------------------------------------------------------
+
+def _select(node: str, x: HIPTensor, axis: int, out: HIPTensor | None, dtype: str) -> HIPTensor:
+    """The reference keeps the leading ``rank - axis`` axes -- ``(butlast (shape
+    tensor) axis)`` -- and reduces over everything behind them, viewed as one run:
+    ``x`` is reshaped to ``(kept..., t)`` and ``out`` is ``(kept..., 1)``.  For
+    the default ``axis = -1`` of a matrix that is the usual row-wise result."""
+    rank = len(x.shape)
+    axis = axis + rank if axis < 0 else axis
+    kept = list(x.shape[:rank - axis]) if axis > 0 else list(x.shape)
+    flat = reshape(x, *kept, -1)
+    if out is None:
+        out = HIPTensor(kept + [1], initial_element=None, dtype=dtype)
+    return nodes.forward(node, flat, out)
+
+
+def _keepdims(result: HIPTensor, base: HIPTensor) -> HIPTensor:
+    """``keepdims`` of ``matrix-ops.lisp:385-393``: size-1 axes of the result are
+    broadcast back to the extent the source has there."""
+    subs = [(":broadcast", s2) if (s1 == 1 and s2 != 1) else True
+            for s1, s2 in zip(result.shape, base.shape)]
+    return result.view(*subs)
+
+
+def max(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None, keepdims: bool = False):  # noqa: A001
+    """``(!max tensor :axis :out :keepdims)``."""
+    r = _select("MaxValue-Node", x, axis, out, "float")
+    return _keepdims(r, x) if keepdims else r
+
+
+def min(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None, keepdims: bool = False):  # noqa: A001
+    """``(!min tensor :axis :out :keepdims)``."""
+    r = _select("MinValue-Node", x, axis, out, "float")
+    return _keepdims(r, x) if keepdims else r
+
+
+def argmax(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!argmax tensor :axis :out)``: a :uint32 tensor of positions within the
+    reduced run."""
+    return _select("ArgMax-Node", x, axis, out, "uint32")
+
+
+def argmin(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None) -> HIPTensor:
+    """``(!argmin tensor :axis :out)``."""
+    return _select("ArgMin-Node", x, axis, out, "uint32")
+
+
+# ---------------------------------------------------------------------------
 # reductions
 # ---------------------------------------------------------------------------
 
@@ -420,7 +470,7 @@ def softmax_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     if out is None:
         out = HIPTensor(x.shape, initial_element=None)
     cols = x.shape[-1]
-    rows = x.size // max(cols, 1)
+    rows = x.size // _builtins.max(cols, 1)
     _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols,
                                                  C.c_void_p(out.ptr), cols))
     return out
@@ -494,7 +544,7 @@ def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e
     if out is None:
         out = HIPTensor(x.shape, initial_element=None)
     cols = x.shape[-1]
-    rows = x.size // max(cols, 1)
+    rows = x.size // _builtins.max(cols, 1)
     _lib.check(_lib.get().wf2hip_layernorm_rows_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),
                                                    C.c_void_p(b.ptr), float(eps), C.c_void_p(out.ptr)))
     return out

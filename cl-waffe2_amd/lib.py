@@ -22,6 +22,7 @@ SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
 POW, GELU = 32, 40
 EQ, LT, LE, GT, GE = 0, 1, 2, 3, 4  # enum wf2hip_compare_op
 COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")
+MAXVALUE, MINVALUE, ARGMAX, ARGMIN = 48, 49, 50, 51  # enum wf2hip_select_op
 
 EOVERLAP = -3
 ECAPTURE = -6
@@ -151,6 +152,7 @@ _SIGNATURES = {
         C.c_int,
     ),
     "wf2hip_matmul_fused": ([C.POINTER(MatmulDesc), _P, _P, _P], C.c_int),
+    "wf2hip_select_nd": ([C.c_int, C.POINTER(View2), _L, _L, _P, _P], C.c_int),
     "wf2hip_where_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F, _F, _F], C.c_int),
     "wf2hip_compare_nd": ([C.c_int, C.POINTER(View3), _P, _P, _P, _F, _F], C.c_int),
     **{f"wf2hip_s{n}": ([_L, _P, _L, _P, _L, _P, _L, _F, _F], C.c_int)

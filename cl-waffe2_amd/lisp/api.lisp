@@ -74,6 +74,9 @@
 (defcfun "wf2hip_compare_nd" :int
   (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
   (then-value :float) (else-value :float))
+(defcfun "wf2hip_select_nd" :int
+  (op :int) (outer (:pointer (:struct view2))) (n :long) (incx :long) (x :pointer) (out :pointer))
+(defconstant +maxvalue+ 48) (defconstant +minvalue+ 49) (defconstant +argmax+ 50) (defconstant +argmin+ 51)
 (defconstant +eq+ 0) (defconstant +lt+ 1) (defconstant +le+ 2) (defconstant +gt+ 3) (defconstant +ge+ 4)
 
 ;; Extensions without a BLAS / SIMD-extension counterpart.  cl-waffe2 reaches them through its own

@@ -157,6 +157,35 @@ These are exactly the numbers call-with-view computes per axis
                                     (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float))))
                           out))
 
+;; A[~] OUT[out-size] -> OUT: largest / smallest value of every trailing run of A, or its index
+;; (source/base-impl/matrix-ops.lisp:197-383).  !max / !argmax hand over A reshaped to
+;; (kept... t) and OUT shaped (kept... 1); the outer axes go to the library as one view2 with the
+;; last axis of A cut off, the run as (n, incx).  ArgMax / ArgMin write :uint32 into OUT, which is
+;; therefore allocated by the device class as 4-byte elements like :float.
+(defun run-select (op x out)
+  (ensure-extension)
+  (with-foreign-object (view '(:struct view2))
+    (fill-view2 view x out)   ; shape slots come from X; only the outer axes are read below
+    (let* ((rank (length (shape x)))
+           (last-axis (1- rank))
+           (n (mem-aref (foreign-slot-pointer view '(:struct view2) 'shape) :int64 last-axis))
+           (incx (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-a) :int64 last-axis)))
+      (if (= rank 1)
+          (setf (mem-aref (foreign-slot-pointer view '(:struct view2) 'shape) :int64 0) 1
+                (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-a) :int64 0) 0
+                (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-b) :int64 0) 0)
+          (setf (foreign-slot-value view '(:struct view2) 'rank) (1- rank)))
+      (check (wf2hip-select-nd op view n incx (tensor-device-pointer x) (tensor-device-pointer out)))))
+  out)
+
+(macrolet ((define-select (node op)
+             `(define-impl-op (,node :device HIPTensor :reject-p #'(lambda (&rest args) (declare (ignore args)) nil))
+                              :forward ((self x out) (declare (ignore self)) (run-select ,op x out)))))
+  (define-select MaxValue-Node +maxvalue+)
+  (define-select MinValue-Node +minvalue+)
+  (define-select ArgMax-Node +argmax+)
+  (define-select ArgMin-Node +argmin+))
+
 ;; C[~ i k] = A[~ i j] . B[~ j k].  Same operand swap as expand-gemm-form-column
 ;; (source/backends/cpu/matrix-ops.lisp:12-112): a row-major product is the column-major
 ;; sgemm(transB, transA, n, m, k, 1, B, ldb, A, lda, 0, C, ldc).  Batch axes are walked on the

@@ -31,6 +31,7 @@ NODE_NAMES = (
     "SinNode", "CosNode", "TanhNode", "LogENode", "ExpNode", "SqrtNode", "AbsNode",
     "ExptNode", "MatMulNode",
     "Where-Operation-Node", "Compare-Operation-Node",
+    "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -193,6 +194,36 @@ def _compare(x: HIPTensor, y: HIPTensor, out: HIPTensor, condition, true_then: f
                                             C.c_void_p(y.ptr), C.c_void_p(out.ptr),
                                             float(true_then), float(false_then)))
     return out
+
+
+def _select(op, index: bool):
+    def impl(x: HIPTensor, out: HIPTensor) -> HIPTensor:
+        """``A[~] OUT[out-size] -> OUT``: one element of OUT per trailing run of A
+        (``base-impl/matrix-ops.lisp:200-383``; CPU forwards
+        ``backends/cpu/matrix-ops.lisp:240-369``)."""
+        xs, xst, xo = x.geometry()
+        os_, ost, oo = out.geometry()
+        if len(xs) != len(os_) or xs[:-1] != os_[:-1] or os_[-1] != 1:
+            raise ValueError(f"{x.shape} selects into {xs[:-1] + [1]}, not {out.shape}")
+        if out.dtype != ("uint32" if index else "float"):
+            raise ValueError("ArgMax/ArgMin write :uint32, MaxValue/MinValue :float")
+        v = _lib.View2()
+        v.rank = max(len(xs) - 1, 1)
+        v.shape[0], v.stride_a[0], v.stride_b[0] = 1, 0, 0
+        for r in range(len(xs) - 1):
+            v.shape[r], v.stride_a[r], v.stride_b[r] = xs[r], xst[r], ost[r]
+        v.off_a, v.off_b = xo, oo
+        _lib.check(_lib.get().wf2hip_select_nd(op, C.byref(v), xs[-1], xst[-1], C.c_void_p(x.ptr),
+                                               C.c_void_p(out.ptr)))
+        return out
+
+    return impl
+
+
+define_impl("MaxValue-Node", HIPTensor, _only_float)(_select(_lib.MAXVALUE, False))
+define_impl("MinValue-Node", HIPTensor, _only_float)(_select(_lib.MINVALUE, False))
+define_impl("ArgMax-Node", HIPTensor, _only_float)(_select(_lib.ARGMAX, True))
+define_impl("ArgMin-Node", HIPTensor, _only_float)(_select(_lib.ARGMIN, True))
 
 
 def _matrix_geometry(t: HIPTensor, what: str):

@@ -128,11 +128,14 @@ def column_major_strides(shape: Sequence[int]) -> list[int]:
 class HIPTensor:
     """An fp32 tensor on the GPU, possibly a view of another one's storage."""
 
-    dtype = "float"
-
     def __init__(self, shape: Sequence[int], *, vec: DeviceBuffer | None = None,
                  strides: Sequence[int] | None = None, views: Sequence[Subscript] | None = None,
-                 offset: int = 0, initial_element: float | None = 0.0):
+                 offset: int = 0, initial_element: float | None = 0.0, dtype: str = "float"):
+        # "uint32" exists only to hold the indices ArgMax-Node / ArgMin-Node write
+        # (matrix-ops.lisp:238-307); every arithmetic node rejects it
+        if dtype not in ("float", "uint32"):
+            raise ValueError(f"HIPTensor holds :float (and :uint32 indices), not {dtype}")
+        self.dtype = dtype
         self.orig_shape = [int(s) for s in shape]
         if len(self.orig_shape) < 1 or len(self.orig_shape) > _lib.MAX_RANK:
             raise ValueError(f"HIPTensor rank must be 1..{_lib.MAX_RANK}")
@@ -220,7 +223,8 @@ class HIPTensor:
         for ax, (n, st) in enumerate(zip(shape, strides)):
             ix = np.arange(n, dtype=np.int64) * st
             idx += ix.reshape([-1 if i == ax else 1 for i in range(len(shape))])
-        return flat[idx]
+        out = flat[idx]
+        return out.view(np.uint32) if self.dtype == "uint32" else out
 
     # -- element access -------------------------------------------------------
     def vref(self, index: int) -> float:
@@ -243,7 +247,7 @@ class HIPTensor:
         subs = list(subscripts) + [True] * (self.ndim - len(subscripts))
         new = [parse_view(base, past, s) for base, past, s in zip(self.orig_shape, self.views, subs)]
         return HIPTensor(self.orig_shape, vec=self.vec, strides=self.stride, views=new,
-                         offset=self.initial_offset)
+                         offset=self.initial_offset, dtype=self.dtype)
 
     def permute(self, *order: int) -> "HIPTensor":
         """Zero-copy axis permutation; ``order[i]`` is the current axis that
@@ -253,7 +257,8 @@ class HIPTensor:
             raise ValueError(f"permute: {order} is not a permutation of 0..{self.ndim - 1}")
         return HIPTensor([self.orig_shape[i] for i in order], vec=self.vec,
                          strides=[self.stride[i] for i in order],
-                         views=[self.views[i] for i in order], offset=self.initial_offset)
+                         views=[self.views[i] for i in order], offset=self.initial_offset,
+                         dtype=self.dtype)
 
     def __repr__(self):
         return f"<HIPTensor {self.shape} views={[v.view for v in self.views]}>"

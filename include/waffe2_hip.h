@@ -183,6 +183,16 @@ int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b);
  * 8-76).  `p` is the exponent for WF2HIP_POW and ignored otherwise. */
 int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p);
 
+/* ---- row selection: max / min value and index ----------------------------- */
+/* For every row of the `outer` space (a = X, b = OUT, in elements; use rank 1,
+ * extent 1 for a single run): OUT <- max / min of the run x[i * incx], i < n, or
+ * its index as a uint32.  Replaces the forwards of MaxValue-Node, MinValue-Node,
+ * ArgMax-Node and ArgMin-Node (source/backends/cpu/matrix-ops.lisp:240-369), which
+ * call waffe2_s{max,min} (cl-waffe2-simd.c:316-365) or BLAS i?max / i?min once
+ * per row.  Ties go to the lowest index; NaN elements are never selected. */
+enum wf2hip_select_op { WF2HIP_MAXVALUE = 48, WF2HIP_MINVALUE = 49, WF2HIP_ARGMAX = 50, WF2HIP_ARGMIN = 51 };
+int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long incx, const float* x, void* out);
+
 /* ---- compare / where ---------------------------------------------------- */
 /* out <- (x OP y) ? then_value : else_value.  OP is ordered: false when an
  * operand is NaN (the reference uses _CMP_*_OQ, avx2.h:179-230). */

@@ -109,6 +109,10 @@ def lib():
         f = getattr(L, "orc_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F]
         f.restype = None
+    for name in ("orc_ismax", "orc_ismin"):
+        f = getattr(L, name)
+        f.argtypes = [C.c_long, _F, C.c_long]
+        f.restype = C.c_long
     L.orc_scmp.argtypes = [C.c_int, C.c_long, _F, C.c_long, _F, C.c_long, _F, C.c_long,
                            C.c_float, C.c_float]
     L.orc_scmp.restype = None
@@ -206,6 +210,12 @@ def pow_1d(n: int, x: np.ndarray, incx: int, p: float, out: np.ndarray, inco: in
     L = ref() if use_ref else lib()
     name = "waffe2_spow" if use_ref else "orc_spow"
     getattr(L, name)(n, _fp(x), incx, C.c_float(p), _fp(out), inco)
+
+
+def argmaxmin_1d(op: str, n: int, x: np.ndarray, incx: int, offx: int = 0) -> int:
+    """0-based index of the first largest / smallest element of the run, i.e.
+    ``(1- (blas-ismax n x incx))`` as ArgMax-Node uses it."""
+    return int(getattr(lib(), "orc_is" + op)(n, _fp(x, offx), incx)) - 1
 
 
 CMP_OPS = ("eq", "lt", "le", "gt", "ge")  # enum order of orc_scmp / wf2hip compare ops

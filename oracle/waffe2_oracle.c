@@ -426,6 +426,32 @@ ORC_API long orc_node_nd(int op, const orc_views *v, float *t0, float *t1,
 }
 
 /* ------------------------------------------------------------------ */
+/* index of the largest / smallest value                               */
+/* ------------------------------------------------------------------ */
+/* ArgMax-Node / ArgMin-Node call BLAS i?max / i?min
+ * (backends/cpu/blas-functions.lisp:16-21, matrix-ops.lisp:240-290): `ismax_` and
+ * `ismin_` are OpenBLAS extensions (netlib BLAS only has isamax), the library is
+ * whatever `libblas` the host provides and is not part of the reference tree.
+ * Restated from their published behaviour: the 1-based position of the first
+ * element holding the largest (smallest) value, found with a strict comparison.
+ * Pinned by the definition (first occurrence on tie-rich data, numpy.argmax). */
+ORC_API long orc_ismax(long n, const float *x, long incx) {
+  if (n < 1) return 0;
+  long best = 0;
+  for (long i = 1; i < n; i++)
+    if (x[i * incx] > x[best * incx]) best = i;
+  return best + 1;
+}
+
+ORC_API long orc_ismin(long n, const float *x, long incx) {
+  if (n < 1) return 0;
+  long best = 0;
+  for (long i = 1; i < n; i++)
+    if (x[i * incx] < x[best * incx]) best = i;
+  return best + 1;
+}
+
+/* ------------------------------------------------------------------ */
 /* compare / where                                                     */
 /* ------------------------------------------------------------------ */
 /* out[i] = (x[i] OP y[i]) ? then : else  (cl-waffe2-simd.c:385-425, define_cmp)

@@ -182,3 +182,81 @@ def test_compare_argument_checks(gpu):
     assert e.value.code == W.lib.EOVERLAP
     F.compare(lo, lo, "=", out=lo)
     assert np.array_equal(buf.numpy()[:8], np.ones(8, np.float32))
+
+
+# ---------------------------------------------------------------------------
+# MaxValue / MinValue / ArgMax / ArgMin nodes
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(5, 7), (1, 1), (3, 1000), (300, 33), (4, 5, 6), (2, 3, 4, 50), (64, 4096),
+                                   (2, 40000), (1, 300000)])
+def test_select_rows(gpu, O, shape):
+    """Row-wise max / min / argmax / argmin through the nodes: values bitwise
+    equal to the oracle's waffe2_s{max,min} restatement per row, indices equal to
+    the first occurrence (small integers make ties frequent)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(sum(shape))
+    x = rng.integers(-50, 51, shape).astype(np.float32)
+    dx = F.from_numpy(x)
+    rows = x.reshape(-1, shape[-1])
+    want_max = np.array([O.maxmin_1d("max", r.size, np.ascontiguousarray(r), 1) for r in rows[:64]], np.float32)
+    got = F.max(dx).numpy()
+    kept = got.shape
+    assert kept == (shape[0], 1)
+    flat = x.reshape(shape[0], -1)  # the reference reduces everything behind the kept axes
+    assert_bit_equal(got.ravel(), flat.max(axis=1), "max")
+    assert_bit_equal(F.min(dx).numpy().ravel(), flat.min(axis=1), "min")
+    if len(shape) == 2:
+        assert_bit_equal(got.ravel()[:64], want_max, "max vs oracle")
+    am = F.argmax(dx).numpy()
+    assert am.dtype == np.uint32 and am.shape == (shape[0], 1)
+    assert np.array_equal(am.ravel(), flat.argmax(axis=1))
+    assert np.array_equal(F.argmin(dx).numpy().ravel(), flat.argmin(axis=1))
+    for r in range(min(shape[0], 8)):
+        row = np.ascontiguousarray(flat[r])
+        assert am.ravel()[r] == O.argmaxmin_1d("max", row.size, row, 1)
+
+
+def test_select_axis_views_and_keepdims(gpu, O):
+    """axis semantics of the reference ((butlast shape axis) kept), strided and
+    offset sources, keepdims broadcast view."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((6, 5, 8)).astype(np.float32)
+    dx = F.from_numpy(x)
+    assert_bit_equal(F.max(dx, axis=1).numpy(), x.reshape(6, 5, 8).max(axis=2, keepdims=True), "axis=1 keeps two")
+    assert_bit_equal(F.max(dx, axis=2).numpy(), x.reshape(6, 40).max(axis=1, keepdims=True), "axis=2 keeps one")
+    k = F.max(dx, axis=1, keepdims=True)
+    assert k.shape == [6, 5, 8]
+    assert_bit_equal(k.numpy(), np.broadcast_to(x.max(axis=2, keepdims=True), x.shape), "keepdims")
+    # a strided window as the source of the node itself (no reshape in between)
+    big = rng.standard_normal((10, 64)).astype(np.float32)
+    db = F.from_numpy(big)
+    win = db.view((2, 9), (3, 60, 2))
+    out = W.HIPTensor([7, 1])
+    W.forward("MaxValue-Node", win, out)
+    sub = win.numpy()   # 28 columns: the reference's range size is floor(|from - to| / step)
+    assert sub.shape == (7, 28) and np.array_equal(sub, big[2:9, 3:59:2])
+    assert_bit_equal(out.numpy().ravel(), sub.max(axis=1), "strided max")
+    iout = W.HIPTensor([7, 1], dtype="uint32")
+    W.forward("ArgMin-Node", win, iout)
+    assert np.array_equal(iout.numpy().ravel(), sub.argmin(axis=1))
+    for r in range(7):
+        assert out.numpy().ravel()[r] == O.maxmin_1d("max", sub.shape[1], np.ascontiguousarray(big[2 + r, 3:]), 2)
+    with pytest.raises(ValueError):
+        W.forward("ArgMax-Node", win, out)          # indices need a :uint32 destination
+
+
+def test_select_full_size(gpu):
+    """(8192, 8192): every row's maximum, and that x[argmax] is that maximum."""
+    F = gpu.functional
+    rng = np.random.Generator(np.random.PCG64(9))
+    x = rng.standard_normal((8192, 8192)).astype(np.float32)
+    dx = F.from_numpy(x)
+    mx = F.max(dx).numpy().ravel()
+    assert_bit_equal(mx, x.max(axis=1), "row max")
+    am = F.argmax(dx).numpy().ravel()
+    assert np.array_equal(x[np.arange(8192), am], mx)
+    assert np.array_equal(am, x.argmax(axis=1))

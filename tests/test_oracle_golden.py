@@ -245,3 +245,17 @@ def test_compare_special_values(O, cmp_gold, op):
         assert_bit_equal(got, CMP_NUMPY[op](xs, ys).astype(np.float32), op + " numpy")
     nan_rows = np.isnan(xs) | np.isnan(ys)
     assert not got[nan_rows].any()
+
+
+def test_index_of_extreme_value(O):
+    """orc_ismax / orc_ismin restate OpenBLAS' ismax_ / ismin_ (1-based, first
+    occurrence).  Pinned by the definition on tie-rich data and strides."""
+    rng = np.random.default_rng(12)
+    for n, inc in [(1, 1), (2, 1), (9, 1), (64, 1), (100, 3), (1000, 2)]:
+        x = rng.integers(-4, 5, n * inc + 1).astype(np.float32)
+        run = x[::inc][:n]
+        assert O.argmaxmin_1d("max", n, x, inc) == int(np.argmax(run))
+        assert O.argmaxmin_1d("min", n, x, inc) == int(np.argmin(run))
+        assert run[O.argmaxmin_1d("max", n, x, inc)] == O.maxmin_1d("max", n, x, inc)
+    x = np.array([1, 5, 5, 0, 0, 5], np.float32)
+    assert O.argmaxmin_1d("max", 6, x, 1) == 1 and O.argmaxmin_1d("min", 6, x, 1) == 3
