@@ -60,6 +60,15 @@ struct OpLog { static constexpr int kFlatU = 2; __device__ __forceinline__ float
 struct OpExp { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return expf_(s); } };
 struct OpSqrt { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return sqrtf_(s); } };
 struct OpAbs { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return absf_(s); } };
+struct OpTan { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return tanf_(s); } };
+struct OpASin { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return asinf_(s); } };
+struct OpACos { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return acosf_(s); } };
+struct OpATan { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return atanf_(s); } };
+struct OpSinH { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return sinhf_(s); } };
+struct OpCosH { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return coshf_(s); } };
+struct OpLog2 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log2f_(s); } };
+struct OpLog10 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log10f_(s); } };
+struct OpLog1p { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log1pf_(s); } };
 struct OpGelu { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return gelu_tanh_f(s); } };
 struct OpPow {
   static constexpr int kFlatU = 2;
@@ -677,6 +686,15 @@ int unary_nd(int op, Space s, const float* x, float* out, float p) {
     case WF2HIP_EXP: return launch_elementwise<OpExp, false>(s, out, x, OpExp{});
     case WF2HIP_SQRT: return launch_elementwise<OpSqrt, false>(s, out, x, OpSqrt{});
     case WF2HIP_ABS: return launch_elementwise<OpAbs, false>(s, out, x, OpAbs{});
+    case WF2HIP_TAN: return launch_elementwise<OpTan, false>(s, out, x, OpTan{});
+    case WF2HIP_ASIN: return launch_elementwise<OpASin, false>(s, out, x, OpASin{});
+    case WF2HIP_ACOS: return launch_elementwise<OpACos, false>(s, out, x, OpACos{});
+    case WF2HIP_ATAN: return launch_elementwise<OpATan, false>(s, out, x, OpATan{});
+    case WF2HIP_SINH: return launch_elementwise<OpSinH, false>(s, out, x, OpSinH{});
+    case WF2HIP_COSH: return launch_elementwise<OpCosH, false>(s, out, x, OpCosH{});
+    case WF2HIP_LOG2: return launch_elementwise<OpLog2, false>(s, out, x, OpLog2{});
+    case WF2HIP_LOG10: return launch_elementwise<OpLog10, false>(s, out, x, OpLog10{});
+    case WF2HIP_LOG1P: return launch_elementwise<OpLog1p, false>(s, out, x, OpLog1p{});
     case WF2HIP_GELU: return launch_elementwise<OpGelu, false>(s, out, x, OpGelu{});
     case WF2HIP_POW: return launch_elementwise<OpPow, false>(s, out, x, OpPow{p});
     default: return fail(WF2HIP_EINVAL, "unknown unary op %d", op);
@@ -768,6 +786,15 @@ WF2_DEFINE_UNARY_1D(log, WF2HIP_LOG)
 WF2_DEFINE_UNARY_1D(exp, WF2HIP_EXP)
 WF2_DEFINE_UNARY_1D(sqrt, WF2HIP_SQRT)
 WF2_DEFINE_UNARY_1D(abs, WF2HIP_ABS)
+WF2_DEFINE_UNARY_1D(tan, WF2HIP_TAN)
+WF2_DEFINE_UNARY_1D(asin, WF2HIP_ASIN)
+WF2_DEFINE_UNARY_1D(acos, WF2HIP_ACOS)
+WF2_DEFINE_UNARY_1D(atan, WF2HIP_ATAN)
+WF2_DEFINE_UNARY_1D(sinh, WF2HIP_SINH)
+WF2_DEFINE_UNARY_1D(cosh, WF2HIP_COSH)
+WF2_DEFINE_UNARY_1D(log2, WF2HIP_LOG2)
+WF2_DEFINE_UNARY_1D(log10, WF2HIP_LOG10)
+WF2_DEFINE_UNARY_1D(log1p, WF2HIP_LOG1P)
 
 WF2_API int wf2hip_spow(long n, const float* x, long incx, float p, float* out, long inco) {
   WF2_TRY(require_init());

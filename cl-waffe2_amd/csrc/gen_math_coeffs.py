@@ -100,3 +100,20 @@ print("// 2/pi =", mp.nstr(2 / mp.pi, 25), " log2(e) =", mp.nstr(1 / mp.log(2), 
 ln2 = mp.log(2)
 lh = mp.ldexp(mp.floor(mp.ldexp(ln2, 32)), -32)
 print("// LN2_HEAD =", mp.nstr(lh, 25), " LN2_TAIL =", mp.nstr(ln2 - lh, 25), " LN2 =", mp.nstr(ln2, 25))
+
+# atan(t) = t + t^3 * P(t^2), |t| <= tan(pi/8)
+TAN_PIO8 = mp.tan(mp.pi / 8)
+
+
+def patan(z):
+    if z < mp.mpf("1e-20"):
+        return -mp.mpf(1) / 3
+    t = mp.sqrt(z)
+    return (mp.atan(t) - t) / (t * z)
+
+
+P = fit(patan, 0, TAN_PIO8 ** 2, 9)
+show("ATAN_P: atan(t) = t + t^3*P(t^2), |t| <= tan(pi/8), degree 9 in z", P)
+print("// max rel err atan:", mp.nstr(maxrel(lambda t: t + t**3 * horner(P, t * t), mp.atan, mp.mpf("1e-6"), TAN_PIO8), 5))
+print("// 1/ln2 =", mp.nstr(1 / mp.log(2), 25), " 1/ln10 =", mp.nstr(1 / mp.log(10), 25),
+      " pi/2 =", mp.nstr(mp.pi / 2, 25), " pi/4 =", mp.nstr(mp.pi / 4, 25), " tan(pi/8) =", mp.nstr(TAN_PIO8, 20))

@@ -30,6 +30,7 @@
 #define WF2_SLOW_SINF(x) sinf(x)
 #define WF2_SLOW_COSF(x) cosf(x)
 #define WF2_SLOW_POW(x, p) pow((x), (p))
+#define WF2_SLOW_TANF(x) tanf(x)
 #define WF2_SQRTF(x) __builtin_sqrtf(x)
 #else
 #include <math.h>
@@ -39,6 +40,7 @@
 #define WF2_SLOW_SINF(x) ((float)sin((double)(x)))
 #define WF2_SLOW_COSF(x) ((float)cos((double)(x)))
 #define WF2_SLOW_POW(x, p) pow((x), (p))
+#define WF2_SLOW_TANF(x) ((float)tan((double)(x)))
 #define WF2_SQRTF(x) sqrtf(x)
 #endif
 
@@ -207,6 +209,128 @@ WF2_MATH_FN float sinf_(float x) {
 WF2_MATH_FN float cosf_(float x) {
   if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_COSF(x);
   return (float)trig_core((double)x, 1);
+}
+
+// tan = sin / cos of the reduced argument (one binary64 division); odd
+// quadrants give -cos / sin.
+WF2_MATH_FN float tanf_(float x) {
+  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_TANF(x);
+  double xd = (double)x;
+  double t = WF2_FMA(xd, kTwoOverPi, kRoundMagic);
+  double q = t - kRoundMagic;
+  int32_t qi = (int32_t)(uint32_t)bits_of(t);
+  double r = WF2_FMA(q, -kPio2Head, xd);
+  r = WF2_FMA(q, -kPio2Tail, r);
+  double z = r * r;
+  double s = sin_poly(r, z);
+  double c = cos_poly(z);
+  float v = (float)((qi & 1) ? -c / s : s / c);
+  return (x == 0.0f) ? x : v;
+}
+
+// log2, log10: the binary64 logarithm times a constant, rounded once (exact for
+// powers of two: k ln2 / ln2).
+WF2_MATH_FN float log2f_(float x) {
+  const float inf = __builtin_inff();
+  bool ok = (x > 0.0f) && (x < inf);
+  float r = (float)(log_core(ok ? (double)x : 1.0) * 1.4426950408889634074);
+  float special = (x == inf) ? inf : ((x == 0.0f) ? -inf : __builtin_nanf(""));
+  return ok ? r : special;
+}
+
+WF2_MATH_FN float log10f_(float x) {
+  const float inf = __builtin_inff();
+  bool ok = (x > 0.0f) && (x < inf);
+  float r = (float)(log_core(ok ? (double)x : 1.0) * 0.43429448190325182765);
+  float special = (x == inf) ? inf : ((x == 0.0f) ? -inf : __builtin_nanf(""));
+  return ok ? r : special;
+}
+
+// log1p: 1 + x is exact in binary64 from |x| >= 2^-29 on; below that
+// x - x^2/2 is correct to 2^-58 relative.
+WF2_MATH_FN float log1pf_(float x) {
+  const float inf = __builtin_inff();
+  bool ok = (x > -1.0f) && (x < inf);
+  double xd = ok ? (double)x : 0.0;
+  double small = WF2_FMA(-0.5 * xd, xd, xd);
+  double big = log_core(1.0 + xd);
+  float r = (float)((__builtin_fabs(xd) < 0x1p-28) ? small : big);
+  float special = (x == inf) ? inf : ((x == -1.0f) ? -inf : __builtin_nanf(""));
+  r = (x == 0.0f) ? x : r;  // log1p(-0) = -0
+  return ok ? r : special;
+}
+
+// sinh, cosh from E = expm1(|x|): sinh = (E + E / (E + 1)) / 2 (no
+// cancellation for small |x|), cosh = ((E + 1) + 1 / (E + 1)) / 2.  From
+// |x| = 90 on both overflow binary32.
+WF2_MATH_FN float sinhf_(float x) {
+  double ax = __builtin_fmin(__builtin_fabs((double)x), 90.0);
+  double p, s;
+  exp_reduce(ax, &p, &s);
+  double em1 = WF2_FMA(s, p, s - 1.0);
+  double v = 0.5 * (em1 + em1 / (em1 + 1.0));
+  float r = __builtin_copysignf((float)v, x);
+  return (x != x) ? x : r;
+}
+
+WF2_MATH_FN float coshf_(float x) {
+  double ax = __builtin_fmin(__builtin_fabs((double)x), 90.0);
+  double p, s;
+  exp_reduce(ax, &p, &s);
+  double e = WF2_FMA(s, p, s);  // e^|x|
+  float r = (float)(0.5 * (e + 1.0 / e));
+  return (x != x) ? x : r;
+}
+
+// atan in binary64: |x| > 1 is folded by atan x = pi/2 - atan(1/x); on [0, 1]
+// the argument is split once more at tan(pi/8) with
+// atan x = pi/4 + atan((x - 1) / (x + 1)), which leaves |t| <= tan(pi/8) for
+// atan t = t + t^3 P(t^2), P of degree 9 (relative error 1.4e-16).
+WF2_MATH_FN double atan_core(double ax) {  // ax >= 0, finite
+  bool inv = ax > 1.0;
+  double y = inv ? 1.0 / ax : ax;
+  bool mid = y > 0.41421356237309503;
+  double t = mid ? (y - 1.0) / (y + 1.0) : y;
+  double z = t * t;
+  double p = 0.022750526993361672084;
+  p = WF2_FMA(p, z, -0.0448333462227288608);
+  p = WF2_FMA(p, z, 0.057363321659076425088);
+  p = WF2_FMA(p, z, -0.066496136952916693446);
+  p = WF2_FMA(p, z, 0.07691055158393149258);
+  p = WF2_FMA(p, z, -0.090908525571760493567);
+  p = WF2_FMA(p, z, 0.11111109636534361442);
+  p = WF2_FMA(p, z, -0.14285714266096617917);
+  p = WF2_FMA(p, z, 0.1999999999989840813);
+  p = WF2_FMA(p, z, -0.3333333333333324625);
+  double a = WF2_FMA(t * z, p, t);
+  a = mid ? 0.78539816339744830962 + a : a;
+  return inv ? 1.57079632679489661923 - a : a;
+}
+
+WF2_MATH_FN float atanf_(float x) {
+  double ax = __builtin_fabs((double)x);
+  double a = (ax > 0x1p60) ? 1.57079632679489661923 : atan_core(ax);
+  float r = __builtin_copysignf((float)a, x);
+  return (x != x) ? x : r;
+}
+
+// asin x = atan(x / sqrt((1 - x)(1 + x))), acos x = 2 atan(sqrt((1 - x) / (1 + x)));
+// (1 - x) and (1 + x) are exact in binary64 for binary32 x.
+WF2_MATH_FN float asinf_(float x) {
+  double xd = (double)x;
+  double ax = __builtin_fabs(xd);
+  if (!(ax <= 1.0)) return __builtin_nanf("");
+  double a = (ax == 1.0) ? 1.57079632679489661923
+                         : atan_core(ax / __builtin_sqrt((1.0 - ax) * (1.0 + ax)));
+  float r = __builtin_copysignf((float)a, x);
+  return (x == 0.0f) ? x : r;
+}
+
+WF2_MATH_FN float acosf_(float x) {
+  double xd = (double)x;
+  if (!(__builtin_fabs(xd) <= 1.0)) return __builtin_nanf("");
+  if (xd == -1.0) return 3.14159274101257324f;
+  return (float)(2.0 * atan_core(__builtin_sqrt((1.0 - xd) / (1.0 + xd))));
 }
 
 WF2_MATH_FN float sqrtf_(float x) { return WF2_SQRTF(x); }

@@ -233,6 +233,15 @@ def exp(x, out=None): return _math("ExpNode", x, out)
 def loge(x, out=None): return _math("LogENode", x, out)
 def sqrt(x, out=None): return _math("SqrtNode", x, out)
 def abs(x, out=None): return _math("AbsNode", x, out)  # noqa: A001 - mirrors !abs
+def tan(x, out=None): return _math("TanNode", x, out)
+def asin(x, out=None): return _math("ASinNode", x, out)
+def acos(x, out=None): return _math("ACosNode", x, out)
+def atan(x, out=None): return _math("ATanNode", x, out)
+def sinh(x, out=None): return _math("SinHNode", x, out)
+def cosh(x, out=None): return _math("CosHNode", x, out)
+def log2(x, out=None): return _math("Log2Node", x, out)
+def log10(x, out=None): return _math("Log10Node", x, out)
+def log1p(x, out=None): return _math("Log1pNode", x, out)
 
 
 def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:

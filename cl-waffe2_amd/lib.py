@@ -19,6 +19,7 @@ MAX_RANK = 8
 # enum wf2hip_binary_op / wf2hip_unary_op
 ADD, SUB, MUL, DIV, MOVE = 0, 1, 2, 3, 4
 SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
+TAN, ASIN, ACOS, ATAN, SINH, COSH, LOG2, LOG10, LOG1P = 23, 24, 25, 26, 27, 28, 29, 30, 31
 POW, GELU = 32, 40
 EQ, LT, LE, GT, GE = 0, 1, 2, 3, 4  # enum wf2hip_compare_op
 COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")
@@ -135,6 +136,15 @@ _SIGNATURES = {
     "wf2hip_sexp": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_ssqrt": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sabs": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_stan": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sasin": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sacos": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_satan": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_ssinh": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_scosh": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_slog2": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_slog10": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_slog1p": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_spow": ([_L, _P, _L, _F, _P, _L], C.c_int),
     "wf2hip_smax": ([_L, _P, _L, _P], C.c_int),
     "wf2hip_smin": ([_L, _P, _L, _P], C.c_int),

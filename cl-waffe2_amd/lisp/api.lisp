@@ -133,6 +133,8 @@ served from the library's pool; transfers and vref are refused while recording."
 (defconstant +add+ 0) (defconstant +sub+ 1) (defconstant +mul+ 2) (defconstant +div+ 3) (defconstant +move+ 4)
 (defconstant +sin+ 16) (defconstant +cos+ 17) (defconstant +tanh+ 18) (defconstant +log+ 19)
 (defconstant +exp+ 20) (defconstant +sqrt+ 21) (defconstant +abs+ 22) (defconstant +pow+ 32)
+(defconstant +tan+ 23) (defconstant +asin+ 24) (defconstant +acos+ 25) (defconstant +atan+ 26)
+(defconstant +sinh+ 27) (defconstant +cosh+ 28) (defconstant +log2+ 29) (defconstant +log10+ 30) (defconstant +log1p+ 31)
 
 (defun hip-synchronize ()
   "Blocks until every kernel enqueued so far has finished (needed around wall-clock timing such

@@ -85,7 +85,16 @@ These are exactly the numbers call-with-view computes per axis
   (define-math LogENode +log+)
   (define-math ExpNode +exp+)
   (define-math SqrtNode +sqrt+)
-  (define-math AbsNode +abs+))
+  (define-math AbsNode +abs+)
+  (define-math TanNode +tan+)
+  (define-math ASinNode +asin+)
+  (define-math ACosNode +acos+)
+  (define-math ATanNode +atan+)
+  (define-math SinHNode +sinh+)
+  (define-math CosHNode +cosh+)
+  (define-math Log2Node +log2+)
+  (define-math Log10Node +log10+)
+  (define-math Log1pNode +log1p+))
 
 ;; OUT <- X^N with N a host ScalarTensor (source/base-impl/mathematics.lisp:267-303)
 (define-impl-op (ExptNode :device HIPTensor :reject-p #'only-float-p)

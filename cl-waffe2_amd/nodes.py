@@ -29,6 +29,7 @@ from .tensor import HIPTensor
 NODE_NAMES = (
     "AddNode", "SubNode", "MulNode", "DivNode", "MoveTensorNode",
     "SinNode", "CosNode", "TanhNode", "LogENode", "ExpNode", "SqrtNode", "AbsNode",
+    "TanNode", "ASinNode", "ACosNode", "ATanNode", "SinHNode", "CosHNode", "Log2Node", "Log10Node", "Log1pNode",
     "ExptNode", "MatMulNode",
     "Where-Operation-Node", "Compare-Operation-Node",
     "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
@@ -133,7 +134,9 @@ for _name, _op in (("AddNode", _lib.ADD), ("SubNode", _lib.SUB), ("MulNode", _li
 
 for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _lib.TANH),
                    ("LogENode", _lib.LOG), ("ExpNode", _lib.EXP), ("SqrtNode", _lib.SQRT),
-                   ("AbsNode", _lib.ABS)):
+                   ("AbsNode", _lib.ABS), ("TanNode", _lib.TAN), ("ASinNode", _lib.ASIN), ("ACosNode", _lib.ACOS),
+                   ("ATanNode", _lib.ATAN), ("SinHNode", _lib.SINH), ("CosHNode", _lib.COSH),
+                   ("Log2Node", _lib.LOG2), ("Log10Node", _lib.LOG10), ("Log1pNode", _lib.LOG1P)):
     define_impl(_name, HIPTensor, _only_float)(_unary(_op))
 
 

@@ -122,6 +122,17 @@ int wf2hip_slog(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_sexp(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_ssqrt(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_sabs(long n, const float* x, long incx, float* out, long inco);
+/* The rest of define-math-impl's list (source/backends/cpu/mathematics.lisp:33-53): Tan, ASin,
+ * ACos, ATan, SinH, CosH, Log2, Log10, Log1p (cl-waffe2-simd.c:650-694). */
+int wf2hip_stan(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_sasin(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_sacos(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_satan(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_ssinh(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_scosh(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_slog2(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_slog10(long n, const float* x, long incx, float* out, long inco);
+int wf2hip_slog1p(long n, const float* x, long incx, float* out, long inco);
 /* out <- x^p.  Replaces waffe2_spow (cl-waffe2-simd.c:708-768; api.lisp:257-273). */
 int wf2hip_spow(long n, const float* x, long incx, float p, float* out, long inco);
 /* out[0] <- max/min_i x[i*incx].  Replaces waffe2_s{max,min}
@@ -163,6 +174,15 @@ enum wf2hip_unary_op {
   WF2HIP_EXP = 20,
   WF2HIP_SQRT = 21,
   WF2HIP_ABS = 22,
+  WF2HIP_TAN = 23,
+  WF2HIP_ASIN = 24,
+  WF2HIP_ACOS = 25,
+  WF2HIP_ATAN = 26,
+  WF2HIP_SINH = 27,
+  WF2HIP_COSH = 28,
+  WF2HIP_LOG2 = 29,
+  WF2HIP_LOG10 = 30,
+  WF2HIP_LOG1P = 31,
   WF2HIP_POW = 32, /* ExptNode mathematics.lisp:267-303 */
   WF2HIP_GELU = 40 /* fused tanh-form GELU (nn/activation.lisp:45-66) */
 };

@@ -28,8 +28,11 @@ KIND_T, KIND_BROADCAST, KIND_OTHER = 0, 1, 2
 OPS = {
     "add": 0, "sub": 1, "mul": 2, "div": 3, "move": 4,
     "sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21,
-    "abs": 22, "pow": 32,
+    "abs": 22, "tan": 23, "asin": 24, "acos": 25, "atan": 26, "sinh": 27, "cosh": 28, "log2": 29,
+    "log10": 30, "log1p": 31, "pow": 32,
 }
+UNARY_NAMES = ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs", "tan", "asin", "acos", "atan", "sinh", "cosh",
+               "log2", "log10", "log1p")
 
 
 class OrcViews(C.Structure):
@@ -99,7 +102,7 @@ def lib():
         f.restype = None
     L.orc_scopy.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
     L.orc_scopy.restype = None
-    for name in ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs"):
+    for name in UNARY_NAMES:
         f = getattr(L, "orc_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
         f.restype = None
@@ -160,8 +163,7 @@ def ref():
         R = C.CDLL(_REF_SO)
     except OSError:
         return None
-    for name in ("add", "sub", "mul", "div", "sin", "cos", "tanh", "log", "exp",
-                 "sqrt", "abs"):
+    for name in ("add", "sub", "mul", "div") + UNARY_NAMES:
         f = getattr(R, "waffe2_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
         f.restype = None

@@ -174,6 +174,15 @@ ORC_DEFINE_UNARY(log, "Sleef_logf8_u10avx2", log)
 ORC_DEFINE_UNARY(exp, "Sleef_expf8_u10avx2", exp)
 ORC_DEFINE_UNARY(sqrt, "Sleef_sqrtf8_u05avx2", sqrt)
 ORC_DEFINE_UNARY(abs, "Sleef_fabsf8_avx2", fabs)
+ORC_DEFINE_UNARY(tan, "Sleef_tanf8_u10avx2", tan)
+ORC_DEFINE_UNARY(asin, "Sleef_asinf8_u10avx2", asin)
+ORC_DEFINE_UNARY(acos, "Sleef_acosf8_u10avx2", acos)
+ORC_DEFINE_UNARY(atan, "Sleef_atanf8_u10avx2", atan)
+ORC_DEFINE_UNARY(sinh, "Sleef_sinhf8_u10avx2", sinh)
+ORC_DEFINE_UNARY(cosh, "Sleef_coshf8_u10avx2", cosh)
+ORC_DEFINE_UNARY(log2, "Sleef_log2f8_u10avx2", log2)
+ORC_DEFINE_UNARY(log10, "Sleef_log10f8_u10avx2", log10)
+ORC_DEFINE_UNARY(log1p, "Sleef_log1pf8_u10avx2", log1p)
 
 /* out <- x^p  (cl-waffe2-simd.c:708-768; avx2.h:304) */
 ORC_API void orc_spow(long n, const float *x, long incx, float p, float *out,
@@ -385,6 +394,15 @@ enum {
   ORC_EXP,
   ORC_SQRT,
   ORC_ABS,
+  ORC_TAN,
+  ORC_ASIN,
+  ORC_ACOS,
+  ORC_ATAN,
+  ORC_SINH,
+  ORC_COSH,
+  ORC_LOG2,
+  ORC_LOG10,
+  ORC_LOG1P,
   ORC_POW = 32
 };
 
@@ -406,6 +424,15 @@ static void exec_emit(const orc_call *c, void *p) {
     case ORC_EXP: orc_sexp(c->n, a, c->inc[0], b, c->inc[1]); break;
     case ORC_SQRT: orc_ssqrt(c->n, a, c->inc[0], b, c->inc[1]); break;
     case ORC_ABS: orc_sabs(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_TAN: orc_stan(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_ASIN: orc_sasin(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_ACOS: orc_sacos(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_ATAN: orc_satan(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_SINH: orc_ssinh(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_COSH: orc_scosh(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_LOG2: orc_slog2(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_LOG10: orc_slog10(c->n, a, c->inc[0], b, c->inc[1]); break;
+    case ORC_LOG1P: orc_slog1p(c->n, a, c->inc[0], b, c->inc[1]); break;
     case ORC_POW: orc_spow(c->n, a, c->inc[0], e->p, b, c->inc[1]); break;
     default: break;
   }

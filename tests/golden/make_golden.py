@@ -126,7 +126,41 @@ def compare_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "compare_kernels.npz")), "bytes")
 
 
+UNARY_MORE = {"tan": (-100, 100), "asin": (-1, 1), "acos": (-1, 1), "atan": (-100, 100), "sinh": (-10, 10),
+              "cosh": (-10, 10), "log2": (1e-3, 1e3), "log10": (1e-3, 1e3), "log1p": (-0.99, 100)}
+
+
+def unary_more_goldens():
+    """The rest of the SIMD extension's unary list (cl-waffe2-simd.c:650-694):
+    range samples with an n % 8 tail, special values, strides, broadcast source."""
+    rng = np.random.Generator(np.random.PCG64(2026))
+    out = {}
+    for op, (lo, hi) in UNARY_MORE.items():
+        x = rng.uniform(lo, hi, 2053).astype(np.float32)
+        if op == "log1p":
+            x[:256] = (rng.uniform(-1, 1, 256) * 10.0 ** rng.uniform(-12, -1, 256)).astype(np.float32)
+        res = np.zeros_like(x)
+        O.unary_1d(op, x.size, x, 1, res, 1, use_ref=True)
+        out[f"un_{op}_range_x"], out[f"un_{op}_range_out"] = x, res
+        res = np.zeros(EDGE.size, np.float32)
+        with np.errstate(all="ignore"):
+            O.unary_1d(op, EDGE.size, EDGE, 1, res, 1, use_ref=True)
+        out[f"un_{op}_edge_out"] = res
+        for n, incx, inco in [(13, 2, 1), (16, 1, 3), (9, 0, 1)]:
+            res = np.full(64, 7.0, np.float32)
+            O.unary_1d(op, n, x, incx, res, inco, use_ref=True)
+            out[f"un_{op}_{n}_{incx}_{inco}_out"] = res
+    out["edge_x"] = EDGE
+    np.savez_compressed(os.path.join(HERE, "unary_more_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "unary_more_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
-    if "--compare-only" not in sys.argv:
+    if "--compare-only" in sys.argv:
+        compare_goldens()
+    elif "--unary-more-only" in sys.argv:
+        unary_more_goldens()
+    else:
         main()
-    compare_goldens()
+        compare_goldens()
+        unary_more_goldens()

@@ -12,7 +12,8 @@
 
 #include "../../cl-waffe2_amd/csrc/wf2_math.h"
 
-enum { OP_SIN = 16, OP_COS, OP_TANH, OP_LOG, OP_EXP, OP_SQRT, OP_ABS, OP_GELU = 40 };
+enum { OP_SIN = 16, OP_COS, OP_TANH, OP_LOG, OP_EXP, OP_SQRT, OP_ABS, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN,
+       OP_SINH, OP_COSH, OP_LOG2, OP_LOG10, OP_LOG1P, OP_GELU = 40 };
 
 static inline float apply(int op, float x) {
   switch (op) {
@@ -23,6 +24,15 @@ static inline float apply(int op, float x) {
     case OP_EXP: return wf2::expf_(x);
     case OP_SQRT: return wf2::sqrtf_(x);
     case OP_ABS: return wf2::absf_(x);
+    case OP_TAN: return wf2::tanf_(x);
+    case OP_ASIN: return wf2::asinf_(x);
+    case OP_ACOS: return wf2::acosf_(x);
+    case OP_ATAN: return wf2::atanf_(x);
+    case OP_SINH: return wf2::sinhf_(x);
+    case OP_COSH: return wf2::coshf_(x);
+    case OP_LOG2: return wf2::log2f_(x);
+    case OP_LOG10: return wf2::log10f_(x);
+    case OP_LOG1P: return wf2::log1pf_(x);
     case OP_GELU: return wf2::gelu_tanh_f(x);
   }
   return 0.0f;
@@ -37,6 +47,15 @@ static inline double truth(int op, double x) {
     case OP_EXP: return exp(x);
     case OP_SQRT: return sqrt(x);
     case OP_ABS: return fabs(x);
+    case OP_TAN: return tan(x);
+    case OP_ASIN: return asin(x);
+    case OP_ACOS: return acos(x);
+    case OP_ATAN: return atan(x);
+    case OP_SINH: return sinh(x);
+    case OP_COSH: return cosh(x);
+    case OP_LOG2: return log2(x);
+    case OP_LOG10: return log10(x);
+    case OP_LOG1P: return log1p(x);
     case OP_GELU: {
       // 0.5 (1 + tanh u) == 1 / (1 + exp(-2u)), free of cancellation
       double u = 0.7978845608028654 * (x + 0.044715 * x * x * x);

@@ -5,6 +5,7 @@ Bar: bit-exact for add/sub/mul/div/copy (IEEE binary32, no contraction);
 bit-exact for sqrt/abs.  Everything goes through the C ABI.
 """
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -333,6 +334,48 @@ def test_metric_size_binary_and_rowsum(gpu, O):
     assert np.max(np.abs(got - truth) / scale) <= 1e-5
     # one rounding of the float64 sum is the best any fp32 result can do
     assert np.max(np.abs(got - truth) / np.maximum(np.abs(truth), 1e-30) * (np.abs(truth) > 1)) <= 1e-6
+
+
+MORE_UNARY = [("tan", -100, 100), ("asin", -1, 1), ("acos", -1, 1), ("atan", -100, 100), ("sinh", -10, 10),
+              ("cosh", -10, 10), ("log2", 1e-3, 1e3), ("log10", 1e-3, 1e3), ("log1p", -0.99, 100)]
+MORE_TRUTH = {"tan": np.tan, "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan, "sinh": np.sinh,
+              "cosh": np.cosh, "log2": np.log2, "log10": np.log10, "log1p": np.log1p}
+
+
+@pytest.mark.parametrize("op,lo,hi", MORE_UNARY)
+def test_more_unary_functions(gpu, O, op, lo, hi):
+    """Tan, ASin, ACos, ATan, SinH, CosH, Log2, Log10, Log1p through the nodes
+    on 2^22 elements: <= 2 ulp from the oracle's SLEEF u10 results, <= 1 ulp
+    from float64; then the reference's golden special values, strides and an
+    n % 8 tail through the 1-D entry points."""
+    W = gpu
+    F = W.functional
+    rng = np.random.Generator(np.random.PCG64(33))
+    n = 1 << 22
+    x = rng.uniform(lo, hi, n).astype(np.float32)
+    want = np.zeros(n, np.float32)
+    O.unary_1d(op, n, x, 1, want, 1)
+    got = getattr(F, op)(F.from_numpy(x)).numpy()
+    assert O.sleef_available()
+    assert ulp_distance(got, want).max() <= 2
+    assert ulp_distance(got, MORE_TRUTH[op](x.astype(np.float64)).astype(np.float32)).max() <= 1
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "unary_more_kernels.npz"))
+    edge = gold["edge_x"]
+    lib = W.lib.get()
+    dx, dout = W.HIPTensor.from_numpy(edge), W.HIPTensor([edge.size])
+    W.lib.check(getattr(lib, "wf2hip_s" + op)(edge.size, dptr(dx), 1, dptr(dout), 1))
+    ref = gold[f"un_{op}_edge_out"].copy()
+    with np.errstate(all="ignore"):
+        truth = MORE_TRUTH[op](edge.astype(np.float64)).astype(np.float32)
+    early = np.isinf(ref) & np.isfinite(truth)      # SLEEF's sinhf / coshf overflow early (88.72 .. 89.42)
+    ref[early] = truth[early]
+    assert ulp_distance(dout.numpy(), ref).max() <= 2
+    xs = gold[f"un_{op}_range_x"]
+    dxs = W.HIPTensor.from_numpy(xs)
+    for cnt, incx, inco in [(13, 2, 1), (16, 1, 3), (9, 0, 1)]:
+        dst = W.HIPTensor.from_numpy(np.full(64, 7.0, np.float32))
+        W.lib.check(getattr(lib, "wf2hip_s" + op)(cnt, dptr(dxs), incx, dptr(dst), inco))
+        assert ulp_distance(dst.numpy(), gold[f"un_{op}_{cnt}_{incx}_{inco}_out"]).max() <= 2
 
 
 def test_unary_edge_values_and_tails(gpu, O):

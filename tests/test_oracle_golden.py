@@ -133,6 +133,37 @@ def test_unary_against_float64_truth(O, gold, op):
     assert ulp_distance(got, truth).max() <= limit
 
 
+MORE_GOLD = os.path.join(os.path.dirname(__file__), "golden", "unary_more_kernels.npz")
+MORE = ["tan", "asin", "acos", "atan", "sinh", "cosh", "log2", "log10", "log1p"]
+MORE_TRUTH = {"tan": np.tan, "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan, "sinh": np.sinh,
+              "cosh": np.cosh, "log2": np.log2, "log10": np.log10, "log1p": np.log1p}
+
+
+@pytest.mark.parametrize("op", MORE)
+def test_more_unary_golden_and_truth(O, op):
+    """Tan, ASin, ACos, ATan, SinH, CosH, Log2, Log10, Log1p
+    (cl-waffe2-simd.c:650-694): the oracle reproduces the compiled reference bit
+    for bit (same SLEEF symbols, same block/tail structure) and both are within
+    1 ulp of float64."""
+    gold = np.load(MORE_GOLD)
+    x = gold[f"un_{op}_range_x"]
+    truth = MORE_TRUTH[op](x.astype(np.float64)).astype(np.float32)
+    assert ulp_distance(gold[f"un_{op}_range_out"], truth).max() <= 1
+    if not O.sleef_available():
+        pytest.skip("no SLEEF provider")
+    got = np.zeros_like(x)
+    O.unary_1d(op, x.size, x, 1, got, 1)
+    assert_bit_equal(got, gold[f"un_{op}_range_out"], op)
+    got = np.zeros(gold["edge_x"].size, np.float32)
+    with np.errstate(all="ignore"):
+        O.unary_1d(op, got.size, gold["edge_x"], 1, got, 1)
+    assert_bit_equal(got, gold[f"un_{op}_edge_out"], op + " edge")
+    for n, incx, inco in [(13, 2, 1), (16, 1, 3), (9, 0, 1)]:
+        got = np.full(64, 7.0, np.float32)
+        O.unary_1d(op, n, x, incx, got, inco)
+        assert_bit_equal(got, gold[f"un_{op}_{n}_{incx}_{inco}_out"], f"{op} {n} {incx} {inco}")
+
+
 def test_unary_special_values(O):
     def f(op, v):
         out = np.zeros(1, np.float32)
