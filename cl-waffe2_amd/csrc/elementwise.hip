@@ -69,6 +69,7 @@ struct OpCosH { static constexpr int kFlatU = 2; __device__ __forceinline__ floa
 struct OpLog2 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log2f_(s); } };
 struct OpLog10 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log10f_(s); } };
 struct OpLog1p { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log1pf_(s); } };
+struct OpInv { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return 1.0f / s; } };
 struct OpGelu { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return gelu_tanh_f(s); } };
 struct OpPow {
   static constexpr int kFlatU = 2;
@@ -695,6 +696,7 @@ int unary_nd(int op, Space s, const float* x, float* out, float p) {
     case WF2HIP_LOG2: return launch_elementwise<OpLog2, false>(s, out, x, OpLog2{});
     case WF2HIP_LOG10: return launch_elementwise<OpLog10, false>(s, out, x, OpLog10{});
     case WF2HIP_LOG1P: return launch_elementwise<OpLog1p, false>(s, out, x, OpLog1p{});
+    case WF2HIP_INV: return launch_elementwise<OpInv, false>(s, out, x, OpInv{});
     case WF2HIP_GELU: return launch_elementwise<OpGelu, false>(s, out, x, OpGelu{});
     case WF2HIP_POW: return launch_elementwise<OpPow, false>(s, out, x, OpPow{p});
     default: return fail(WF2HIP_EINVAL, "unknown unary op %d", op);
@@ -720,6 +722,13 @@ int where_nd(int op, Space s, const float* x, float* out, float scal, float then
     return fail(WF2HIP_EOVERLAP, "compare between partially overlapping windows");
   if (has_broadcast_axis(s, s.sa)) keep_last_write(&s);
   return launch_elementwise<OpWhere, false>(s, out, x, OpWhere{op, scal, then_value, else_value});
+}
+
+// x[0] <- 1 / x[0], n times over: what the reference's loop does to a stride-0 run
+__global__ void inv_repeated(float* x, long n) {
+  float v = *x;
+  for (long i = 0; i < n; i++) v = 1.0f / v;
+  *x = v;
 }
 
 static int space_1d(long n, long inca, long incb, Space* s) {
@@ -825,3 +834,18 @@ WF2_DEFINE_WHERE_1D(lt, WF2HIP_LT)
 WF2_DEFINE_WHERE_1D(le, WF2HIP_LE)
 WF2_DEFINE_WHERE_1D(gt, WF2HIP_GT)
 WF2_DEFINE_WHERE_1D(ge, WF2HIP_GE)
+
+// x <- 1 / x in place.  Replaces waffe2_sinv (cl-waffe2-simd.c:290-302).
+WF2_API int wf2hip_sinv(long n, float* x, long incx) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
+  if (n == 0) return 0;
+  if (!x) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  if (incx == 0) {
+    inv_repeated<<<1, 1, 0, rt().stream>>>(x, n);
+    return after_launch("inv_repeated");
+  }
+  Space s;
+  WF2_TRY(space_1d(n, incx, incx, &s));
+  return unary_nd(WF2HIP_INV, s, x, x, 0.0f);
+}

@@ -136,6 +136,7 @@ _SIGNATURES = {
     "wf2hip_sexp": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_ssqrt": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sabs": ([_L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_sinv": ([_L, _P, _L], C.c_int),
     "wf2hip_stan": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sasin": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sacos": ([_L, _P, _L, _P, _L], C.c_int),

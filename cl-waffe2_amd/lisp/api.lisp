@@ -74,6 +74,7 @@
 (defcfun "wf2hip_compare_nd" :int
   (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
   (then-value :float) (else-value :float))
+(defcfun "wf2hip_sinv" :int (n :long) (x :pointer) (incx :long))
 (defcfun "wf2hip_select_nd" :int
   (op :int) (outer (:pointer (:struct view2))) (n :long) (incx :long) (x :pointer) (out :pointer))
 (defconstant +maxvalue+ 48) (defconstant +minvalue+ 49) (defconstant +argmax+ 50) (defconstant +argmin+ 51)

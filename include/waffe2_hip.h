@@ -133,6 +133,9 @@ int wf2hip_scosh(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_slog2(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_slog10(long n, const float* x, long incx, float* out, long inco);
 int wf2hip_slog1p(long n, const float* x, long incx, float* out, long inco);
+/* x <- 1 / x in place (IEEE division; with incx == 0 the one element is inverted n times, as the
+ * reference's loop does).  Replaces waffe2_sinv (cl-waffe2-simd.c:290-302; api.lisp:111-124). */
+int wf2hip_sinv(long n, float* x, long incx);
 /* out <- x^p.  Replaces waffe2_spow (cl-waffe2-simd.c:708-768; api.lisp:257-273). */
 int wf2hip_spow(long n, const float* x, long incx, float p, float* out, long inco);
 /* out[0] <- max/min_i x[i*incx].  Replaces waffe2_s{max,min}
@@ -184,6 +187,7 @@ enum wf2hip_unary_op {
   WF2HIP_LOG10 = 30,
   WF2HIP_LOG1P = 31,
   WF2HIP_POW = 32, /* ExptNode mathematics.lisp:267-303 */
+  WF2HIP_INV = 33, /* 1 / x */
   WF2HIP_GELU = 40 /* fused tanh-form GELU (nn/activation.lisp:45-66) */
 };
 

@@ -112,6 +112,8 @@ def lib():
         f = getattr(L, "orc_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F]
         f.restype = None
+    L.orc_sinv.argtypes = [C.c_long, _F, C.c_long]
+    L.orc_sinv.restype = None
     for name in ("orc_ismax", "orc_ismin"):
         f = getattr(L, name)
         f.argtypes = [C.c_long, _F, C.c_long]
@@ -169,6 +171,8 @@ def ref():
         f.restype = None
     R.waffe2_spow.argtypes = [C.c_long, _F, C.c_long, C.c_float, _F, C.c_long]
     R.waffe2_spow.restype = None
+    R.waffe2_sinv.argtypes = [C.c_long, _F, C.c_long]
+    R.waffe2_sinv.restype = None
     for name in CMP_OPS:
         f = getattr(R, "waffe2_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long, _F, C.c_long, C.c_float, C.c_float]
@@ -212,6 +216,11 @@ def pow_1d(n: int, x: np.ndarray, incx: int, p: float, out: np.ndarray, inco: in
     L = ref() if use_ref else lib()
     name = "waffe2_spow" if use_ref else "orc_spow"
     getattr(L, name)(n, _fp(x), incx, C.c_float(p), _fp(out), inco)
+
+
+def inv_1d(n: int, x: np.ndarray, incx: int, use_ref: bool = False) -> None:
+    """x <- 1 / x in place (waffe2_sinv)."""
+    (ref().waffe2_sinv if use_ref else lib().orc_sinv)(n, _fp(x), incx)
 
 
 def argmaxmin_1d(op: str, n: int, x: np.ndarray, incx: int, offx: int = 0) -> int:

@@ -452,6 +452,16 @@ ORC_API long orc_node_nd(int op, const orc_views *v, float *t0, float *t1,
   return 0;
 }
 
+/* x <- 1 / x, element after element (cl-waffe2-simd.c:290-302): the literal
+ * 1.0 is a double, so the division runs in binary64 and is rounded to binary32
+ * (equal to a binary32 division: 53 >= 2 * 24 + 2). */
+ORC_API void orc_sinv(long n, float *x, long incx) {
+  for (long count = 0; count != n; count++) {
+    x[0] = 1.0 / x[0];
+    x += incx;
+  }
+}
+
 /* ------------------------------------------------------------------ */
 /* index of the largest / smallest value                               */
 /* ------------------------------------------------------------------ */

@@ -378,6 +378,21 @@ def test_more_unary_functions(gpu, O, op, lo, hi):
         assert ulp_distance(dst.numpy(), gold[f"un_{op}_{cnt}_{incx}_{inco}_out"]).max() <= 2
 
 
+def test_inv(gpu, O):
+    """wf2hip_sinv against the oracle, bit for bit, strided and stride 0."""
+    W = gpu
+    lib = W.lib.get()
+    rng = np.random.default_rng(6)
+    x = np.concatenate([rng.standard_normal(5000), [0.0, -0.0, np.inf, 1e-45, 3e38, 1.0, 3.0]]).astype(np.float32)
+    for n, inc in [(x.size, 1), (x.size // 2, 2), (100, 7), (6, 0), (0, 1)]:
+        want = x.copy()
+        with np.errstate(all="ignore"):
+            O.inv_1d(n, want, inc)
+        dx = W.HIPTensor.from_numpy(x)
+        W.lib.check(lib.wf2hip_sinv(n, dptr(dx), inc))
+        assert_bit_equal(dx.numpy(), want, f"inv n={n} inc={inc}")
+
+
 def test_unary_edge_values_and_tails(gpu, O):
     """+-0, denormals, +-inf, NaN, huge arguments, n % 8 != 0 tails, strided
     in/out."""

@@ -290,3 +290,30 @@ def test_index_of_extreme_value(O):
         assert run[O.argmaxmin_1d("max", n, x, inc)] == O.maxmin_1d("max", n, x, inc)
     x = np.array([1, 5, 5, 0, 0, 5], np.float32)
     assert O.argmaxmin_1d("max", 6, x, 1) == 1 and O.argmaxmin_1d("min", 6, x, 1) == 3
+
+
+def test_inv(O):
+    """x <- 1 / x (cl-waffe2-simd.c:290-302): equals the IEEE binary32 division,
+    equals the compiled reference where present, and a stride-0 run is inverted
+    n times."""
+    rng = np.random.default_rng(4)
+    x = np.concatenate([rng.standard_normal(1000), [0.0, -0.0, np.inf, 1e-45, 3e38, 1.0, 3.0]]).astype(np.float32)
+    for inc in (1, 2, 3):
+        n = x.size // inc
+        got = x.copy()
+        with np.errstate(all="ignore"):
+            O.inv_1d(n, got, inc)
+            want = x.copy()
+            want[:n * inc:inc] = np.float32(1.0) / x[:n * inc:inc]
+        assert_bit_equal(got, want, f"inv inc={inc}")
+        if O.ref() is not None:
+            r = x.copy()
+            with np.errstate(all="ignore"):
+                O.inv_1d(n, r, inc, use_ref=True)
+            assert_bit_equal(got, r, "inv vs reference")
+    one = np.array([3.0], np.float32)
+    O.inv_1d(5, one, 0)
+    want = np.float32(3.0)
+    for _ in range(5):
+        want = np.float32(1.0) / want
+    assert one[0] == want
