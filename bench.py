@@ -48,7 +48,7 @@ RING = 8  # buffer sets: 8 x (x, y, o) x 256 MiB = 6 GiB
 # `rocprofv3 --pmc` runs of `bench.py --probe` (FETCH_SIZE 262173.8 KiB, WRITE_SIZE
 # 262144.3 KiB per dispatch), each scaled by what the same counter reads for the plain
 # copy of 2^26 floats in the same run (x1.9996 and x0.9996); summary under profiles/.
-BINARY_TRAFFIC_BYTES = 805_160_000
+BINARY_TRAFFIC_BYTES = 805_150_000
 
 
 def p(t):
