@@ -17,6 +17,7 @@ from .tensor import HIPTensor, Subscript, column_major_strides, parse_view, view
 from . import nodes
 from .nodes import NodeNotFound, define_impl, forward, with_devices
 from . import functional
+from . import optimizers
 
 __all__ = [
     "lib", "HIPError", "HIPExtensionMissing", "Range", "compose", "make_range", "HIPTensor",

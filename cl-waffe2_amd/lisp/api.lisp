@@ -110,6 +110,11 @@
   (desc (:pointer (:struct attention-desc))) (q :pointer) (k :pointer) (v :pointer) (o :pointer))
 (defcfun "wf2hip_causal_softmax_f32" :int (matrices :long) (seq :long) (x :pointer) (out :pointer) (scale :float))
 
+(defcfun "wf2hip_sgd_step_f32" :int (n :long) (param :pointer) (grad :pointer) (lr :float))
+(defcfun "wf2hip_adam_step_f32" :int
+  (n :long) (param :pointer) (grad :pointer) (m :pointer) (v :pointer)
+  (one-minus-beta1 :float) (one-minus-beta2 :float) (lr-t :float) (eps :float))
+
 ;; HIP graphs: record the launches of one compiled forward, replay them with one call.
 (defcfun "wf2hip_graph_begin" :int)
 (defcfun "wf2hip_graph_end" :int (graph (:pointer :pointer)))

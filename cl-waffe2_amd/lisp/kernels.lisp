@@ -256,3 +256,39 @@ These are exactly the numbers call-with-view computes per axis
                                                           (+ oc (* i (nth axis sc)))))))))
                                       (walk 0 oa ob oc))))))
                             out)))
+
+;; Optimiser steps in one kernel.  step-optimize of SGD / Adam composes element-wise nodes
+;; (source/optimizers/impls/sgd.lisp:18-34, adam.lisp:45-117); for a contiguous HIPTensor
+;; parameter these :around methods run the same binary32 operations in the same order in one
+;; pass instead (bit-identical result) and fall back to the node composition otherwise.
+(defun contiguous-device-tensor-p (tensor)
+  (and (typep tensor 'HIPTensor)
+       (every #'(lambda (v) (eql (cl-waffe2/vm.generic-tensor::force-list v) t)) (tensor-view tensor))
+       (zerop (tensor-initial-offset tensor))))
+
+(defmethod cl-waffe2/optimizers:step-optimize :around ((optimizer cl-waffe2/optimizers:SGD))
+  (let* ((param (cl-waffe2/optimizers:read-parameter optimizer))
+         (grad (grad param)))
+    (if (and *hip-extension-p* (contiguous-device-tensor-p param) (contiguous-device-tensor-p grad))
+        (check (wf2hip-sgd-step-f32 (apply #'* (shape param))
+                                    (tensor-device-pointer param) (tensor-device-pointer grad)
+                                    (coerce (cl-waffe2/optimizers::sgd-lr optimizer) 'single-float)))
+        (call-next-method))))
+
+(defmethod cl-waffe2/optimizers:step-optimize :around ((optimizer cl-waffe2/optimizers:Adam))
+  (let* ((param (cl-waffe2/optimizers:read-parameter optimizer))
+         (grad (grad param))
+         (m (cl-waffe2/optimizers::adam-m optimizer))
+         (v (cl-waffe2/optimizers::adam-v optimizer)))
+    (if (and *hip-extension-p* (every #'contiguous-device-tensor-p (list param grad m v)))
+        (let ((lr-t (cl-waffe2/optimizers::adam-step-lr optimizer)))   ; also counts the step
+          (check (wf2hip-adam-step-f32
+                  (apply #'* (shape param))
+                  (tensor-device-pointer param) (tensor-device-pointer grad)
+                  (tensor-device-pointer m) (tensor-device-pointer v)
+                  (- 1.0 (cl-waffe2/optimizers::beta1-of optimizer))
+                  (- 1.0 (cl-waffe2/optimizers::beta2-of optimizer))
+                  (coerce lr-t 'single-float)
+                  (cl-waffe2/optimizers::eps-of optimizer))))
+        (call-next-method))))
+

@@ -347,6 +347,21 @@ typedef struct wf2hip_matmul_desc {
 } wf2hip_matmul_desc;
 int wf2hip_matmul_fused(const wf2hip_matmul_desc* desc, const float* A, const float* B, float* C);
 
+/* ---- optimiser steps (extension) ------------------------------------------ */
+/* One pass per parameter tensor, performing the binary32 operations of the
+ * reference's node compositions in the same order, so the result is
+ * bit-identical to running those nodes one by one.  Contiguous, non-overlapping
+ * buffers of n elements.
+ * SGD (source/optimizers/impls/sgd.lisp:18-34): grad <- grad * lr (the reference
+ * scales the gradient in place), param <- param - grad.
+ * Adam (source/optimizers/impls/adam.lisp:45-117): m <- m + (g - m) * (1 - beta1);
+ * v <- v + (1 - beta2) * (g * g - v); param <- param - (m * lr_t) / (eps + sqrt(v)),
+ * with lr_t = lr * sqrt(1 - beta2^t) / (1 - beta1^t) computed by the caller
+ * (adam-step-lr, adam.lisp:78-92) and 1 - beta rounded to binary32 by the caller. */
+int wf2hip_sgd_step_f32(long n, float* param, float* grad, float lr);
+int wf2hip_adam_step_f32(long n, float* param, const float* grad, float* m, float* v,
+                         float one_minus_beta1, float one_minus_beta2, float lr_t, float eps);
+
 /* ---- attention (extension; no BLAS counterpart) ---------------------------- */
 /* O[b,h,i,:] = sum_j softmax_j(scale * Q[b,h,i,:].K[b,h,j,:] (+ causal mask j <= i)) V[b,h,j,:]
  * in one kernel, replacing the node sequence !matmul, scalar multiply, mask add,
