@@ -208,7 +208,9 @@ def cpu_baseline():
             break
     dt = (time.perf_counter() - t0) / reps
     gbs = sum(BYTES.values()) / dt / 1e9
+    block = cpu_block_forward_ms()
     return {
+        "block_fwd_ms": block,
         "value": round(gbs, 3),
         "unit": "GB/s",
         "cores": 1,
@@ -217,6 +219,32 @@ def cpu_baseline():
                   f"{dt:.2f} s each, 1 thread as in the reference (lparallel off, *num-cores* 1), "
                   f"SLEEF {'from libtorch_cpu.so' if O.sleef_available() else 'absent: libm'}",
     }
+
+
+def cpu_block_forward_ms():
+    """The block forward in binary32 on the host (numpy + its BLAS): the
+    reference-equivalent CPU path restated, timed on one thread (what
+    cl-waffe2's CPU backend uses for everything but the gemm) and on all cores
+    given to this process.  A baseline to read the GPU number against, nothing
+    more."""
+    try:
+        from threadpoolctl import threadpool_limits
+    except ImportError:
+        return None
+    from oracle import gpt2_block_ref as ref
+    gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
+    params = gpt2.make_block_params(seed=5)
+    x = gpt2.make_block_input(seed=5)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, 16)
+    out = {"shape": "B 8, T 1024, D 768, 12 x 64, fp32, numpy", "cores_all": cores}
+    for label, threads in (("threads_all", cores), ("threads_1", 1)):
+        with threadpool_limits(limits=threads):
+            ref.block_forward(x[:1], params, 12, dtype=np.float32)  # warm the BLAS
+            t0 = time.perf_counter()
+            ref.block_forward(x, params, 12, dtype=np.float32)
+            out[label] = round((time.perf_counter() - t0) * 1e3, 1)
+    return out
 
 
 def main():

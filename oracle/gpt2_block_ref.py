@@ -18,19 +18,22 @@ def layer_norm(x, g, b, eps):
 
 
 def gelu(x):
-    return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+    c = x.dtype.type
+    return c(0.5) * x * (c(1.0) + np.tanh(c(np.sqrt(2.0 / np.pi)) * (x + c(0.044715) * x ** 3)))
 
 
-def block_forward(x, p, n_head, eps=1e-5):
-    x = x.astype(np.float64)
-    p = {k: v.astype(np.float64) for k, v in p.items()}
+def block_forward(x, p, n_head, eps=1e-5, dtype=np.float64):
+    """dtype float64: the checker.  dtype float32: the same recipe in the
+    arithmetic of the CPU path, used only to time a CPU baseline."""
+    x = x.astype(dtype)
+    p = {k: v.astype(dtype) for k, v in p.items()}
     B, T, D = x.shape
     hd = D // n_head
     h = layer_norm(x, p["ln1_g"], p["ln1_b"], eps)
     qkv = h @ p["w_qkv"] + p["b_qkv"]
     q, k, v = (qkv[..., i * D:(i + 1) * D].reshape(B, T, n_head, hd).transpose(0, 2, 1, 3) for i in range(3))
-    s = (q @ k.transpose(0, 1, 3, 2)) / np.sqrt(hd)
-    s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+    s = (q @ k.transpose(0, 1, 3, 2)) / dtype(np.sqrt(hd))
+    s = np.where(np.tril(np.ones((T, T), bool)), s, dtype(-np.inf))
     e = np.exp(s - s.max(axis=-1, keepdims=True))
     pr = e / e.sum(axis=-1, keepdims=True)
     ctx = (pr @ v).transpose(0, 2, 1, 3).reshape(B, T, D)
