@@ -18,6 +18,7 @@ from . import nodes
 from .nodes import NodeNotFound, define_impl, forward, with_devices
 from . import functional
 from . import optimizers
+from . import io
 
 __all__ = [
     "lib", "HIPError", "HIPExtensionMissing", "Range", "compose", "make_range", "HIPTensor",

@@ -118,3 +118,33 @@ def test_training_loop_converges(gpu):
         if it % 50 == 0 or it == 299:
             losses.append(float(np.mean(err.numpy() ** 2)))
     assert losses[-1] < 1e-4 * losses[0], losses
+
+
+def test_weights_round_trip(gpu, tmp_path):
+    """.npy and :wf2model I/O (examples/gpt-2/utils.lisp:6-9,
+    backends/lisp/wf2model.lisp:5-54): bit-exact round trips, views saved as
+    seen, storage vectors saved flat, non-float files refused."""
+    import json
+    W = gpu
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((5, 7, 3)).astype(f32)
+    np.save(tmp_path / "a.npy", a)
+    t = W.io.load_npy(str(tmp_path / "a.npy"))
+    assert t.shape == [5, 7, 3]
+    assert_bit_equal(t.numpy(), a, "load_npy")
+    W.io.save_npy(t.view((1, 4), True, 2), str(tmp_path / "v.npy"))
+    assert_bit_equal(np.load(tmp_path / "v.npy"), a[1:4, :, 2:3], "save_npy of a view")
+    np.save(tmp_path / "i.npy", np.arange(4))
+    with pytest.raises(TypeError):
+        W.io.load_npy(str(tmp_path / "i.npy"))
+    np.save(tmp_path / "d.npy", a.astype(np.float64))
+    assert_bit_equal(W.io.load_npy(str(tmp_path / "d.npy")).numpy(), a, "float64 file narrows to float")
+    state = {"layer/w": t, "bias": W.HIPTensor.from_numpy(a[0, 0]), "steps": 12, "lr": 0.5}
+    W.io.save_weights(str(tmp_path / "model"), state)
+    table = json.load(open(tmp_path / "model" / "parameters.json"))
+    assert table["steps"] == 12 and table["layer/w"].endswith("layer/w.npy")
+    assert np.load(table["layer/w"]).shape == (105,)      # the storage vector, flat
+    back = W.io.load_weights(str(tmp_path / "model"), shapes={"layer/w": (5, 7, 3)})
+    assert back["steps"] == 12 and back["lr"] == 0.5
+    assert_bit_equal(back["layer/w"].numpy(), a, "wf2model tensor")
+    assert_bit_equal(back["bias"].numpy(), a[0, 0], "wf2model flat tensor")
