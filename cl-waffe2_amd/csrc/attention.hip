@@ -10,9 +10,9 @@
 //
 // Work split: one workgroup per (batch, head, block of 128 queries), four
 // wavefronts of 32 queries each; keys/values stream through LDS in blocks of
-// 64 (two stages, one barrier per block).  Everything is computed transposed so
+// 64 (two stages filled by global -> LDS loads, one barrier per block).  Everything is computed transposed so
 // that a lane owns one query:
-//   S^T = K . Q^T      A operand = K fragment (LDS, 128-bit reads),
+//   S^T = K . Q^T      A operand = K fragment (LDS, conflict-free 128-bit reads),
 //                      B operand = Q fragment (registers for the whole kernel,
 //                      pre-multiplied by scale * log2 e)
 //   O^T += V^T . P^T   A operand = V fragment (LDS, conflict-free 32-bit reads),
@@ -40,10 +40,9 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr int kHeadDim = 64;
 constexpr int kQBlock = 128;         // queries per workgroup
 constexpr int kKBlock = 64;          // keys per LDS stage
-constexpr int kKPitch = kHeadDim + 4;  // 128-bit reads of 8 consecutive lanes cover all 32 banks
-constexpr int kVPitch = kHeadDim;
-constexpr int kStageFloats = kKBlock * kKPitch + kKBlock * kVPitch;
-constexpr size_t kAttnLdsBytes = 2 * (size_t)kStageFloats * sizeof(float);  // 67,584 B
+constexpr int kRowFloats = kHeadDim;  // LDS rows are unpadded: the global -> LDS path writes 1 KB runs
+constexpr int kStageFloats = 2 * kKBlock * kRowFloats;
+constexpr size_t kAttnLdsBytes = 2 * (size_t)kStageFloats * sizeof(float);  // 65,536 B
 
 struct AttnParams {
   const float* q;
@@ -58,35 +57,10 @@ struct AttnParams {
   float scale_log2e;
 };
 
-// This thread's share of a 64 x 64 key (or value) block: four float4.
-// Rows beyond the sequence are clamped (their scores are masked later).
-__device__ __forceinline__ void load_kv(const float* __restrict__ base, int64_t stride_pos,
-                                        int key0, int seq, int head_dim, f4 (&reg)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int f = threadIdx.x + kBlock * j;
-    int key = key0 + (f >> 4);
-    key = key < seq ? key : seq - 1;
-    const int c = (f & 15) * 4;
-    f4 v = {0.f, 0.f, 0.f, 0.f};
-    if (c < head_dim) v = *reinterpret_cast<const f4*>(base + (int64_t)key * stride_pos + c);
-    reg[j] = v;
-  }
-}
-
-template <int PITCH>
-__device__ __forceinline__ void store_kv(float* __restrict__ lds, const f4 (&reg)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int f = threadIdx.x + kBlock * j;
-    *reinterpret_cast<f4*>(lds + (f >> 4) * PITCH + (f & 15) * 4) = reg[j];
-  }
-}
-
 __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   auto lds_k = [&](int stage) { return smem + stage * kStageFloats; };
-  auto lds_v = [&](int stage) { return smem + stage * kStageFloats + kKBlock * kKPitch; };
+  auto lds_v = [&](int stage) { return smem + stage * kStageFloats + kKBlock * kRowFloats; };
 
   // longest query blocks first: with a causal mask block qb needs qb+1 key spans
   const int nbh = p.batch * p.heads;
@@ -108,6 +82,8 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
   const float* qp = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)query_ld * p.qs[2];
   const float* kp = p.k + b * p.ks[0] + h * p.ks[1];
   const float* vp = p.v + b * p.vs[0] + h * p.vs[1];
+  (void)kp;
+  (void)vp;  // only the device pass reads them (global -> LDS builtin)
 
   // Q fragment: qf[4 j + r] = Q[query][8 j + 4 half + r] * scale * log2(e)
   float qf[32];
@@ -131,20 +107,52 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
   float m = -INFINITY;  // running maximum (log2 domain), shared by both halves
   float lsum = 0.f;     // running sum of this half's keys
 
-  f4 kreg[4], vreg[4];
-  load_kv(kp, p.ks[2], 0, p.seq, p.head_dim, kreg);
-  load_kv(vp, p.vs[2], 0, p.seq, p.head_dim, vreg);
-  store_kv<kKPitch>(lds_k(0), kreg);
-  store_kv<kVPitch>(lds_v(0), vreg);
+  // Key / value blocks go global -> LDS without passing through registers: one
+  // instruction moves 64 x 16 bytes into 1 KB of LDS (four rows).  The 16-byte
+  // slots of a row are permuted through the address each lane reads from:
+  //   keys    slot = chunk ^ (row % 16), so that the 128-bit fragment reads of 16
+  //           consecutive rows cover all 64 banks;
+  //   values  the two 128-byte halves of a row are swapped when (row / 4) is odd:
+  //           the half-waves read rows 4 apart and then hit different banks.
+  // Rows beyond the sequence are clamped (their scores are masked later); chunks
+  // beyond head_dim are not loaded and stay zero from the clear below.
+  auto fetch = [&](int stage, int key0) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int q4 = wave * 4 + j;
+      const int row = q4 * 4 + (lane >> 4);
+      const int slot = lane & 15;
+      int key = key0 + row;
+      key = key < p.seq ? key : p.seq - 1;
+      const int kchunk = slot ^ (row & 15);
+      const int vchunk = slot ^ (((row >> 2) & 1) << 3);
+      if (kchunk * 4 < p.head_dim)
+        __builtin_amdgcn_global_load_lds(kp + (int64_t)key * p.ks[2] + kchunk * 4,
+                                         lds_k(stage) + q4 * 256, 16, 0, 0);
+      if (vchunk * 4 < p.head_dim)
+        __builtin_amdgcn_global_load_lds(vp + (int64_t)key * p.vs[2] + vchunk * 4,
+                                         lds_v(stage) + q4 * 256, 16, 0, 0);
+    }
+#endif
+  };
+  if (p.head_dim < kHeadDim) {
+    for (int i = threadIdx.x; i < 2 * kStageFloats / 4; i += kBlock)
+      reinterpret_cast<f4*>(smem)[i] = f4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+  }
+  fetch(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+
+  const int kswz = col & 15;     // rows col and 32 + col share it
+  const int vswap = half << 5;   // keys read by the upper half-wave have (key / 4) odd
 
   for (int kb = 0; kb < nkb; kb++) {
     const int key0 = kb * kKBlock;
     const bool more = kb + 1 < nkb;
-    if (more) {
-      load_kv(kp, p.ks[2], key0 + kKBlock, p.seq, p.head_dim, kreg);
-      load_kv(vp, p.vs[2], key0 + kKBlock, p.seq, p.head_dim, vreg);
-    }
+    // the other stage was last read before the barrier that ended the previous block
+    if (more) fetch((kb + 1) & 1, key0 + kKBlock);
     const float* sk = lds_k(kb & 1);
     const float* sv = lds_v(kb & 1);
 
@@ -154,8 +162,9 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
       f16v s0 = {0}, s1 = {0};
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        f4 k0 = *reinterpret_cast<const f4*>(sk + col * kKPitch + 8 * j + 4 * half);
-        f4 k1 = *reinterpret_cast<const f4*>(sk + (32 + col) * kKPitch + 8 * j + 4 * half);
+        const int slot = ((2 * j + half) ^ kswz) * 4;
+        f4 k0 = *reinterpret_cast<const f4*>(sk + col * kRowFloats + slot);
+        f4 k1 = *reinterpret_cast<const f4*>(sk + (32 + col) * kRowFloats + slot);
         s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[4 * j + 0], s0, 0, 0, 0);
         s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[4 * j + 0], s1, 0, 0, 0);
         s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.y, qf[4 * j + 1], s0, 0, 0, 0);
@@ -202,20 +211,17 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const int key = 8 * (i >> 2) + 4 * half + (i & 3);
-        const float v00 = sv[key * kVPitch + col];
-        const float v01 = sv[key * kVPitch + 32 + col];
-        const float v10 = sv[(32 + key) * kVPitch + col];
-        const float v11 = sv[(32 + key) * kVPitch + 32 + col];
+        const float v00 = sv[key * kRowFloats + (col ^ vswap)];
+        const float v01 = sv[key * kRowFloats + ((32 + col) ^ vswap)];
+        const float v10 = sv[(32 + key) * kRowFloats + (col ^ vswap)];
+        const float v11 = sv[(32 + key) * kRowFloats + ((32 + col) ^ vswap)];
         o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v00, s0[i], o0, 0, 0, 0);
         o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v01, s0[i], o1, 0, 0, 0);
         o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v10, s1[i], o0, 0, 0, 0);
         o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v11, s1[i], o1, 0, 0, 0);
       }
     }
-    if (more) {
-      store_kv<kKPitch>(lds_k((kb + 1) & 1), kreg);
-      store_kv<kVPitch>(lds_v((kb + 1) & 1), vreg);
-    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the next block landed
     __syncthreads();
   }
 
