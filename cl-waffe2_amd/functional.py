@@ -252,6 +252,55 @@ def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:
 
 
 # ---------------------------------------------------------------------------
+# padding / unfold (source/base-impl/utils.lisp:4-140, source/nn/im2col.lisp)
+# ---------------------------------------------------------------------------
+
+def padding(x: HIPTensor, pad_width) -> HIPTensor:
+    """``(padding tensor pad-width)``: a zero tensor of the padded shape, a view of
+    its interior, ``x`` moved into the view.  ``pad_width`` holds ``(before,
+    after)`` per axis, or ``True`` for an axis left alone."""
+    if len(pad_width) != len(x.shape):
+        raise ValueError("padding: one (before, after) pair or True per axis")
+    widths = [(0, 0) if w is True else (int(w[0]), int(w[1])) for w in pad_width]
+    if all(w == (0, 0) for w in widths):
+        return x
+    out = HIPTensor([n + b + a for n, (b, a) in zip(x.shape, widths)])
+    inner = out.view(*[True if w == (0, 0) else (w[0], w[0] + n) for n, w in zip(x.shape, widths)])
+    move_(inner, x)
+    return out
+
+
+def conv_out_size(size: int, pad: int, dilation: int, kernel: int, stride: int) -> int:
+    """``conv-out-size`` (``source/nn/pool.lisp:10-17``)."""
+    return (size + 2 * pad - dilation * (kernel - 1) - 1) // stride + 1
+
+
+def im2col(padded_x: HIPTensor, kernel_size, h_out: int, w_out: int, stride, pad, dilation) -> HIPTensor:
+    """``!im2col`` (``source/nn/im2col.lisp:15-49``): Im2ColNode into a fresh
+    ``[N C k-h k-w h-out w-out]`` tensor, then permuted to (N h-out w-out C k-h k-w)
+    and reshaped to ``[(N h-out w-out) (C k-h k-w)]``."""
+    N, Cc = padded_x.shape[:2]
+    col = HIPTensor([N, Cc, kernel_size[0], kernel_size[1], h_out, w_out])
+    nodes.forward("Im2ColNode", to_contiguous(padded_x), col, stride, pad, dilation)
+    return reshape(col.permute(0, 4, 5, 1, 2, 3), N * h_out * w_out, Cc * kernel_size[0] * kernel_size[1])
+
+
+def unfold(x: HIPTensor, dilation, kernel_size, stride, pad) -> HIPTensor:
+    """``(unfold input dilation kernel-size stride padding)``
+    (``source/nn/im2col.lisp:51-95``): sliding local blocks of a ``[N C H W]``
+    tensor as rows of a ``[(N h-out w-out) (C k-h k-w)]`` matrix.  The input is
+    padded by ``(pad, pad + out mod stride)`` on each spatial axis first, as the
+    reference does."""
+    if len(x.shape) != 4:
+        raise ValueError("unfold takes a [N C H W] tensor")
+    H, W = x.shape[2:]
+    h_out = conv_out_size(H, pad[0], dilation[0], kernel_size[0], stride[0])
+    w_out = conv_out_size(W, pad[1], dilation[0], kernel_size[1], stride[1])   # (car dilation) twice: sic
+    px = padding(x, [True, True, (pad[0], pad[0] + h_out % stride[0]), (pad[1], pad[1] + w_out % stride[1])])
+    return im2col(px, kernel_size, h_out, w_out, stride, pad, dilation)
+
+
+# ---------------------------------------------------------------------------
 # compare / where (source/base-impl/logical.lisp)
 # ---------------------------------------------------------------------------
 

@@ -110,6 +110,12 @@
   (desc (:pointer (:struct attention-desc))) (q :pointer) (k :pointer) (v :pointer) (o :pointer))
 (defcfun "wf2hip_causal_softmax_f32" :int (matrices :long) (seq :long) (x :pointer) (out :pointer) (scale :float))
 
+(defcfun "wf2hip_im2col_f32" :int
+  (col :pointer) (n :long) (c :long) (h :long) (w :long) (h-out :long) (w-out :long) (k-h :long) (k-w :long)
+  (pad-h :long) (pad-w :long) (stride-h :long) (stride-w :long) (dilation-h :long) (dilation-w :long) (im :pointer))
+(defcfun "wf2hip_col2im_f32" :int
+  (col :pointer) (n :long) (c :long) (h :long) (w :long) (h-out :long) (w-out :long) (k-h :long) (k-w :long)
+  (pad-h :long) (pad-w :long) (stride-h :long) (stride-w :long) (dilation-h :long) (dilation-w :long) (im :pointer))
 (defcfun "wf2hip_sgd_step_f32" :int (n :long) (param :pointer) (grad :pointer) (lr :float))
 (defcfun "wf2hip_adam_step_f32" :int
   (n :long) (param :pointer) (grad :pointer) (m :pointer) (v :pointer)

@@ -257,6 +257,28 @@ These are exactly the numbers call-with-view computes per axis
                                       (walk 0 oa ob oc))))))
                             out)))
 
+;; Unfold / fold (source/base-impl/unfold.lisp; CPU forwards source/backends/cpu/im2col.lisp).
+;; Same slots, same argument order as waffe2_im2col_s_column / waffe2_col2im_s_column.
+(macrolet ((define-unfold (node fn first second)
+             `(define-impl-op (,node :device HIPTensor :reject-p #'only-float-p)
+                              :forward ((self ,first ,second)
+                                        (ensure-extension)
+                                        (let ((x ,(if (eq node 'Im2ColNode) first second))
+                                              (col ,(if (eq node 'Im2ColNode) second first)))
+                                          (setf (h-of self) (nth 2 (shape x))
+                                                (w-of self) (nth 3 (shape x)))
+                                          (with-slots (C h-out w-out k-h k-w padding-h padding-w
+                                                       stride-h stride-w dilation-h dilation-w)
+                                              self
+                                            (check (,fn (tensor-device-pointer col)
+                                                        (car (shape x)) C (h-of self) (w-of self)
+                                                        h-out w-out k-h k-w padding-h padding-w
+                                                        stride-h stride-w dilation-h dilation-w
+                                                        (tensor-device-pointer x)))))
+                                        ,second))))
+  (define-unfold Im2ColNode wf2hip-im2col-f32 x col)
+  (define-unfold Col2ImNode wf2hip-col2im-f32 col output-to))
+
 ;; Optimiser steps in one kernel.  step-optimize of SGD / Adam composes element-wise nodes
 ;; (source/optimizers/impls/sgd.lisp:18-34, adam.lisp:45-117); for a contiguous HIPTensor
 ;; parameter these :around methods run the same binary32 operations in the same order in one

@@ -33,6 +33,7 @@ NODE_NAMES = (
     "ExptNode", "MatMulNode",
     "Where-Operation-Node", "Compare-Operation-Node",
     "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
+    "Im2ColNode", "Col2ImNode",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -227,6 +228,36 @@ define_impl("MaxValue-Node", HIPTensor, _only_float)(_select(_lib.MAXVALUE, Fals
 define_impl("MinValue-Node", HIPTensor, _only_float)(_select(_lib.MINVALUE, False))
 define_impl("ArgMax-Node", HIPTensor, _only_float)(_select(_lib.ARGMAX, True))
 define_impl("ArgMin-Node", HIPTensor, _only_float)(_select(_lib.ARGMIN, True))
+
+
+def _unfold_args(x_shape, col_shape, stride, padding, dilation):
+    N, Cc, H, W = x_shape
+    n2, c2, kh, kw, ho, wo = col_shape
+    if (N, Cc) != (n2, c2):
+        raise ValueError(f"X {x_shape} and Col {col_shape} disagree on N, C")
+    return [N, Cc, H, W, ho, wo, kh, kw, padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1]]
+
+
+@define_impl("Im2ColNode", HIPTensor, _only_float)
+def _im2col(x: HIPTensor, col: HIPTensor, stride, padding, dilation) -> HIPTensor:
+    """``X[N C H W] Col[N C k-h k-w h-out w-out] -> Col`` with X already padded
+    (``base-impl/unfold.lisp``; CPU forward ``backends/cpu/im2col.lisp:3-26``)."""
+    if not (x.is_contiguous() and col.is_contiguous()):
+        raise ValueError("Im2ColNode takes contiguous tensors (the CPU kernel indexes the storage directly)")
+    args = _unfold_args(x.shape, col.shape, stride, padding, dilation)
+    _lib.check(_lib.get().wf2hip_im2col_f32(C.c_void_p(col.ptr), *args, C.c_void_p(x.ptr)))
+    return col
+
+
+@define_impl("Col2ImNode", HIPTensor, _only_float)
+def _col2im(col: HIPTensor, x: HIPTensor, stride, padding, dilation) -> HIPTensor:
+    """``Col[N C k-h k-w h-out w-out] X[N C H W] -> X``: X is overwritten with the
+    sum of the columns (``backends/cpu/im2col.lisp:28-50``)."""
+    if not (x.is_contiguous() and col.is_contiguous()):
+        raise ValueError("Col2ImNode takes contiguous tensors")
+    args = _unfold_args(x.shape, col.shape, stride, padding, dilation)
+    _lib.check(_lib.get().wf2hip_col2im_f32(C.c_void_p(col.ptr), *args, C.c_void_p(x.ptr)))
+    return x
 
 
 def _matrix_geometry(t: HIPTensor, what: str):

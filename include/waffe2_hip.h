@@ -347,6 +347,23 @@ typedef struct wf2hip_matmul_desc {
 } wf2hip_matmul_desc;
 int wf2hip_matmul_fused(const wf2hip_matmul_desc* desc, const float* A, const float* B, float* C);
 
+/* ---- unfold / fold --------------------------------------------------------- */
+/* Col[N C K_H K_W H_out W_out] <- X[N C H W] (X already padded) and its adjoint
+ * X <- sum of the columns.  Replace waffe2_im2col_s_column / waffe2_col2im_s_column
+ * (cl-waffe2-simd/kernels/im2col.c:63-115, 395-448), same argument order and the
+ * same walk: for kernel offset k the positions k, k + stride, ... below
+ * dilation * k - pad + stride * out are visited.  Elements of Col the walk does
+ * not reach are left untouched; col2im overwrites X and accumulates in the
+ * reference's order (kernel rows, then kernel columns, ascending).  Geometries
+ * whose walk would leave its plane of Col (dilation > 1) return
+ * WF2HIP_EUNSUPPORTED.  Tensors in cl-waffe2's default (:column) order. */
+int wf2hip_im2col_f32(float* col, long N, long C, long H, long W, long H_out, long W_out, long K_H,
+                      long K_W, long pad_h, long pad_w, long stride_h, long stride_w,
+                      long dilation_h, long dilation_w, const float* im);
+int wf2hip_col2im_f32(const float* col, long N, long C, long H, long W, long H_out, long W_out,
+                      long K_H, long K_W, long pad_h, long pad_w, long stride_h, long stride_w,
+                      long dilation_h, long dilation_w, float* im);
+
 /* ---- optimiser steps (extension) ------------------------------------------ */
 /* One pass per parameter tensor, performing the binary32 operations of the
  * reference's node compositions in the same order, so the result is

@@ -218,6 +218,52 @@ def pow_1d(n: int, x: np.ndarray, incx: int, p: float, out: np.ndarray, inco: in
     getattr(L, name)(n, _fp(x), incx, C.c_float(p), _fp(out), inco)
 
 
+_U64 = C.c_uint64
+_im2col_ref = None
+
+
+def _im2col_lib(use_ref: bool):
+    """(library, prefix): the oracle, or the reference's im2col.c compiled into _ref."""
+    global _im2col_ref
+    if not use_ref:
+        L = lib()
+        for name in ("orc_im2col", "orc_col2im"):
+            getattr(L, name).argtypes = [_F] + [_U64] * 14 + [_F]
+            getattr(L, name).restype = None
+        return L, "orc_"
+    if _im2col_ref is None:
+        path = os.path.join(_HERE, "_ref", "libwaffe2_im2col_ref.so")
+        if not os.path.exists(path):
+            return None, None
+        _im2col_ref = C.CDLL(path)
+        for name in ("waffe2_im2col_s_column", "waffe2_col2im_s_column"):
+            getattr(_im2col_ref, name).argtypes = [_F] + [_U64] * 14 + [_F]
+            getattr(_im2col_ref, name).restype = None
+    return _im2col_ref, "waffe2_"
+
+
+def im2col_ref_available() -> bool:
+    return _im2col_lib(True)[0] is not None
+
+
+def im2col(col: np.ndarray, im: np.ndarray, N, Cc, H, W, H_out, W_out, K_H, K_W, pad, stride, dilation,
+           use_ref: bool = False) -> None:
+    """col[N C K_H K_W H_out W_out] <- im[N C H W] (waffe2_im2col_s_column)."""
+    L, pre = _im2col_lib(use_ref)
+    f = getattr(L, "orc_im2col" if not use_ref else "waffe2_im2col_s_column")
+    f(_fp(col), N, Cc, H, W, H_out, W_out, K_H, K_W, pad[0], pad[1], stride[0], stride[1],
+      dilation[0], dilation[1], _fp(im))
+
+
+def col2im(col: np.ndarray, im: np.ndarray, N, Cc, H, W, H_out, W_out, K_H, K_W, pad, stride, dilation,
+           use_ref: bool = False) -> None:
+    """im[N C H W] <- sum of col (waffe2_col2im_s_column)."""
+    L, pre = _im2col_lib(use_ref)
+    f = getattr(L, "orc_col2im" if not use_ref else "waffe2_col2im_s_column")
+    f(_fp(col), N, Cc, H, W, H_out, W_out, K_H, K_W, pad[0], pad[1], stride[0], stride[1],
+      dilation[0], dilation[1], _fp(im))
+
+
 def inv_1d(n: int, x: np.ndarray, incx: int, use_ref: bool = False) -> None:
     """x <- 1 / x in place (waffe2_sinv)."""
     (ref().waffe2_sinv if use_ref else lib().orc_sinv)(n, _fp(x), incx)

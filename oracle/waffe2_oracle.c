@@ -587,6 +587,57 @@ ORC_API long orc_compare_nd(int op, const orc_views *v, const float *x, const fl
 }
 
 /* ------------------------------------------------------------------ */
+/* im2col / col2im                                                     */
+/* ------------------------------------------------------------------ */
+/* cl-waffe2-simd/kernels/im2col.c:63-115 (waffe2_im2col_s_column) and 395-448
+ * (waffe2_col2im_s_column): X[N C H W] <-> Col[N C K_H K_W H_out W_out].  The walk
+ * over image rows starts at the kernel offset itself and ends below
+ * dilation * k - pad + stride * out (evaluated in uint64 like the reference);
+ * col2im clears X first and accumulates in loop order. */
+typedef unsigned long long orc_u64;
+
+static void orc_unfold_walk(int fold, float *col, orc_u64 N, orc_u64 C, orc_u64 H, orc_u64 W,
+                            orc_u64 H_out, orc_u64 W_out, orc_u64 K_H, orc_u64 K_W, orc_u64 pad_h,
+                            orc_u64 pad_w, orc_u64 s_h, orc_u64 s_w, orc_u64 d_h, orc_u64 d_w,
+                            float *im) {
+  for (orc_u64 n = 0; n < N; n++)
+    for (orc_u64 kh = 0; kh < K_H; kh++) {
+      const orc_u64 h_end = d_h * kh - pad_h + s_h * H_out;
+      for (orc_u64 kw = 0; kw < K_W; kw++) {
+        const orc_u64 w_end = d_w * kw - pad_w + s_w * W_out;
+        orc_u64 i = 0;
+        for (orc_u64 y = kh; y < h_end; y += s_h, i++) {
+          orc_u64 j = 0;
+          for (orc_u64 x = kw; x < w_end; x += s_w, j++)
+            for (orc_u64 c = 0; c < C; c++) {
+              float *cp = col + ((((n * C + c) * K_H + kh) * K_W + kw) * H_out + i) * W_out + j;
+              float *ip = im + ((n * C + c) * H + y) * W + x;
+              if (fold)
+                *ip += *cp;
+              else
+                *cp = *ip;
+            }
+        }
+      }
+    }
+}
+
+ORC_API void orc_im2col(float *col, orc_u64 N, orc_u64 C, orc_u64 H, orc_u64 W, orc_u64 H_out,
+                        orc_u64 W_out, orc_u64 K_H, orc_u64 K_W, orc_u64 pad_h, orc_u64 pad_w,
+                        orc_u64 s_h, orc_u64 s_w, orc_u64 d_h, orc_u64 d_w, const float *im) {
+  orc_unfold_walk(0, col, N, C, H, W, H_out, W_out, K_H, K_W, pad_h, pad_w, s_h, s_w, d_h, d_w,
+                  (float *)im);
+}
+
+ORC_API void orc_col2im(const float *col, orc_u64 N, orc_u64 C, orc_u64 H, orc_u64 W, orc_u64 H_out,
+                        orc_u64 W_out, orc_u64 K_H, orc_u64 K_W, orc_u64 pad_h, orc_u64 pad_w,
+                        orc_u64 s_h, orc_u64 s_w, orc_u64 d_h, orc_u64 d_w, float *im) {
+  for (orc_u64 i = 0; i < N * C * H * W; i++) im[i] = 0.0f;
+  orc_unfold_walk(1, (float *)col, N, C, H, W, H_out, W_out, K_H, K_W, pad_h, pad_w, s_h, s_w, d_h,
+                  d_w, im);
+}
+
+/* ------------------------------------------------------------------ */
 /* sgemm                                                               */
 /* ------------------------------------------------------------------ */
 /* Column-major C(m x n) <- alpha*op(A)*op(B) + beta*C with Fortran sgemm_

@@ -155,8 +155,50 @@ def unary_more_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "unary_more_kernels.npz")), "bytes")
 
 
+IM2COL_CASES = [  # N, C, H_in, W_in, kernel, stride, padding  (dilation 1)
+    (1, 1, 5, 5, (3, 3), (1, 1), (0, 0)),
+    (2, 3, 8, 7, (3, 2), (1, 1), (1, 1)),
+    (1, 2, 9, 9, (3, 3), (2, 2), (1, 1)),
+    (2, 2, 10, 6, (2, 3), (2, 1), (0, 2)),
+    (1, 4, 12, 12, (5, 5), (3, 3), (2, 2)),
+    (3, 1, 6, 11, (1, 1), (1, 2), (0, 0)),
+]
+
+
+def im2col_geometry(case):
+    """The arguments `unfold` hands to Im2ColNode (source/nn/im2col.lisp:51-95):
+    output sizes from conv-out-size, the image padded by (pad, pad + out mod stride)."""
+    N, Cc, H, W, k, s, p = case
+    out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((H, W))]
+    padded = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((H, W))]
+    return N, Cc, padded[0], padded[1], out[0], out[1], k[0], k[1]
+
+
+def im2col_goldens():
+    """waffe2_im2col_s_column / waffe2_col2im_s_column (cl-waffe2-simd/kernels/im2col.c)
+    on the geometries unfold produces."""
+    assert O.im2col_ref_available(), "oracle/_ref/libwaffe2_im2col_ref.so is missing: run `make -C oracle ref`"
+    rng = np.random.Generator(np.random.PCG64(2027))
+    out = {}
+    for idx, case in enumerate(IM2COL_CASES):
+        N, Cc, H, W, Ho, Wo, kh, kw = im2col_geometry(case)
+        _, _, _, _, k, s, p = case
+        im = rng.standard_normal((N, Cc, H, W)).astype(np.float32)
+        col = np.full((N, Cc, kh, kw, Ho, Wo), 7.0, np.float32)      # untouched elements keep the 7
+        O.im2col(col, im, N, Cc, H, W, Ho, Wo, kh, kw, p, s, (1, 1), use_ref=True)
+        out[f"im2col_{idx}_im"], out[f"im2col_{idx}_col"] = im, col
+        cin = rng.standard_normal(col.shape).astype(np.float32)
+        back = np.full(im.shape, 5.0, np.float32)
+        O.col2im(cin, back, N, Cc, H, W, Ho, Wo, kh, kw, p, s, (1, 1), use_ref=True)
+        out[f"col2im_{idx}_col"], out[f"col2im_{idx}_im"] = cin, back
+    np.savez_compressed(os.path.join(HERE, "im2col_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "im2col_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
-    if "--compare-only" in sys.argv:
+    if "--im2col-only" in sys.argv:
+        im2col_goldens()
+    elif "--compare-only" in sys.argv:
         compare_goldens()
     elif "--unary-more-only" in sys.argv:
         unary_more_goldens()
@@ -164,3 +206,4 @@ if __name__ == "__main__":
         main()
         compare_goldens()
         unary_more_goldens()
+        im2col_goldens()

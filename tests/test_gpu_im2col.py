@@ -1,0 +1,104 @@
+"""Im2ColNode / Col2ImNode kernels: bitwise against the oracle (pinned to the
+reference's compiled im2col.c by tests/test_oracle_golden.py) and against the
+golden outputs themselves; the adjoint identity at a larger size; `unfold`
+against the sliding-window closed form."""
+import ctypes as C
+import importlib.util
+import os
+
+import numpy as np
+import pytest
+
+from helpers import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _golden_module():
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(HERE, "golden", "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    return mg
+
+
+def test_im2col_col2im_golden(gpu):
+    W = gpu
+    mg = _golden_module()
+    gold = np.load(os.path.join(HERE, "golden", "im2col_kernels.npz"))
+    for idx, case in enumerate(mg.IM2COL_CASES):
+        N, Cc, H, Wd, Ho, Wo, kh, kw = mg.im2col_geometry(case)
+        _, _, _, _, k, s, p = case
+        x = W.HIPTensor.from_numpy(gold[f"im2col_{idx}_im"])
+        col = W.HIPTensor.from_numpy(np.full((N, Cc, kh, kw, Ho, Wo), 7.0, np.float32))
+        W.forward("Im2ColNode", x, col, s, p, (1, 1))
+        assert_bit_equal(col.numpy(), gold[f"im2col_{idx}_col"], f"im2col case {idx}")
+        back = W.HIPTensor.from_numpy(np.full((N, Cc, H, Wd), 5.0, np.float32))
+        W.forward("Col2ImNode", W.HIPTensor.from_numpy(gold[f"col2im_{idx}_col"]), back, s, p, (1, 1))
+        assert_bit_equal(back.numpy(), gold[f"col2im_{idx}_im"], f"col2im case {idx}")
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_im2col_random_geometries_match_oracle(gpu, O, seed):
+    W = gpu
+    rng = np.random.default_rng(40 + seed)
+    for case in range(10):
+        N, Cc = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        k = (int(rng.integers(1, 5)), int(rng.integers(1, 5)))
+        s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        p = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        Hin, Win = int(rng.integers(k[0], 20)), int(rng.integers(k[1], 20))
+        out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((Hin, Win))]
+        H, Wd = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((Hin, Win))]
+        im = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
+        want = np.full((N, Cc, k[0], k[1], out[0], out[1]), 3.0, np.float32)
+        O.im2col(want, im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
+        col = W.HIPTensor.from_numpy(np.full(want.shape, 3.0, np.float32))
+        W.forward("Im2ColNode", W.HIPTensor.from_numpy(im), col, s, p, (1, 1))
+        assert_bit_equal(col.numpy(), want, f"im2col {N, Cc, H, Wd, k, s, p}")
+        cin = rng.standard_normal(want.shape).astype(np.float32)
+        want_im = np.zeros_like(im)
+        O.col2im(cin, want_im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
+        back = W.HIPTensor([N, Cc, H, Wd])
+        W.forward("Col2ImNode", W.HIPTensor.from_numpy(cin), back, s, p, (1, 1))
+        assert_bit_equal(back.numpy(), want_im, f"col2im {N, Cc, H, Wd, k, s, p}")
+
+
+def test_unfold_and_adjoint(gpu):
+    """unfold(x) for stride 1 without padding is the sliding window of numpy,
+    laid out [(N h-out w-out) (C k-h k-w)]; at a convolution-sized input
+    <im2col(x), c> = <x, col2im(c)> (the two kernels are adjoint)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    got = F.unfold(F.from_numpy(x), (1, 1), (3, 2), (1, 1), (0, 0)).numpy()
+    win = np.lib.stride_tricks.sliding_window_view(x, (3, 2), axis=(2, 3))     # N C ho wo kh kw
+    want = win.transpose(0, 2, 3, 1, 4, 5).reshape(2 * 7 * 7, 3 * 3 * 2)
+    assert_bit_equal(got, np.ascontiguousarray(want), "unfold")
+    N, Cc, H, Wd, k, s = 8, 16, 66, 66, (3, 3), (1, 1)
+    Ho, Wo = H - 2, Wd - 2
+    xi = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
+    ci = rng.standard_normal((N, Cc, 3, 3, Ho, Wo)).astype(np.float32)
+    col = W.HIPTensor([N, Cc, 3, 3, Ho, Wo])
+    W.forward("Im2ColNode", F.from_numpy(xi), col, s, (0, 0), (1, 1))
+    back = W.HIPTensor([N, Cc, H, Wd])
+    W.forward("Col2ImNode", F.from_numpy(ci), back, s, (0, 0), (1, 1))
+    lhs = np.sum(col.numpy().astype(np.float64) * ci)
+    rhs = np.sum(xi.astype(np.float64) * back.numpy())
+    assert abs(lhs - rhs) <= 1e-6 * np.sum(np.abs(xi)) 
+
+
+def test_im2col_argument_checks(gpu):
+    W = gpu
+    lib = W.lib.get()
+    a = W.HIPTensor([1, 1, 8, 8])
+    col = W.HIPTensor([1, 1, 3, 3, 6, 6])
+    args = lambda **kw: [kw.get(n, d) for n, d in (("N", 1), ("C", 1), ("H", 8), ("W", 8), ("Ho", 6), ("Wo", 6), ("kh", 3),  # noqa: E731
+                                                   ("kw", 3), ("ph", 0), ("pw", 0), ("sh", 1), ("sw", 1), ("dh", 1), ("dw", 1))]
+    c, x = C.c_void_p(col.ptr), C.c_void_p(a.ptr)
+    assert lib.wf2hip_im2col_f32(c, *args(), x) == 0
+    assert lib.wf2hip_im2col_f32(c, *args(dh=2), x) == -4          # the walk would leave its plane
+    assert lib.wf2hip_im2col_f32(c, *args(H=7), x) == -1           # the walk leaves the image
+    assert lib.wf2hip_im2col_f32(c, *args(sh=0), x) == -1
+    assert lib.wf2hip_col2im_f32(c, *args(kh=40), x) == -4

@@ -317,3 +317,34 @@ def test_inv(O):
     for _ in range(5):
         want = np.float32(1.0) / want
     assert one[0] == want
+
+
+def test_im2col_golden(O):
+    """orc_im2col / orc_col2im against the outputs of the reference's im2col.c
+    (compiled into oracle/_ref) on the geometries `unfold` produces, bitwise;
+    elements the reference's walk does not reach keep their previous value;
+    with no padding and stride 1 the result is the textbook unfold."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(
+        "make_golden", os.path.join(os.path.dirname(__file__), "golden", "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "im2col_kernels.npz"))
+    for idx, case in enumerate(mg.IM2COL_CASES):
+        N, Cc, H, W, Ho, Wo, kh, kw = mg.im2col_geometry(case)
+        _, _, _, _, k, s, p = case
+        im = gold[f"im2col_{idx}_im"]
+        col = np.full((N, Cc, kh, kw, Ho, Wo), 7.0, np.float32)
+        O.im2col(col, im, N, Cc, H, W, Ho, Wo, kh, kw, p, s, (1, 1))
+        assert_bit_equal(col, gold[f"im2col_{idx}_col"], f"im2col case {idx}")
+        back = np.full(im.shape, 5.0, np.float32)
+        O.col2im(gold[f"col2im_{idx}_col"], back, N, Cc, H, W, Ho, Wo, kh, kw, p, s, (1, 1))
+        assert_bit_equal(back, gold[f"col2im_{idx}_im"], f"col2im case {idx}")
+        if O.im2col_ref_available():
+            col2 = np.full(col.shape, 7.0, np.float32)
+            O.im2col(col2, im, N, Cc, H, W, Ho, Wo, kh, kw, p, s, (1, 1), use_ref=True)
+            assert_bit_equal(col, col2, "oracle vs compiled reference")
+    # closed form: case 0 (5x5, 3x3, stride 1, no padding) is the sliding window
+    im = gold["im2col_0_im"][0, 0]
+    want = np.lib.stride_tricks.sliding_window_view(im, (3, 3)).transpose(2, 3, 0, 1)
+    assert_bit_equal(gold["im2col_0_col"][0, 0], np.ascontiguousarray(want), "sliding window")
