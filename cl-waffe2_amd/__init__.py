@@ -19,6 +19,7 @@ from .nodes import NodeNotFound, define_impl, forward, with_devices
 from . import functional
 from . import optimizers
 from . import io
+from . import nn
 
 __all__ = [
     "lib", "HIPError", "HIPExtensionMissing", "Range", "compose", "make_range", "HIPTensor",

@@ -1,0 +1,58 @@
+"""Convolution and pooling as the reference composes them from unfold.
+
+``source/nn/conv.lisp:90-104`` (apply-conv2d) and ``source/nn/pool.lisp:83-105``
+(MaxPool2D / AvgPool2D): every step is one of the backend's nodes -- padding
+(MoveTensorNode into a view), Im2ColNode, permute / reshape copies, MatMulNode,
+AddNode, MaxValue-Node or the !mean composition -- so the layers run on the
+device without a kernel of their own.
+"""
+from __future__ import annotations
+
+from . import functional as F
+from .tensor import HIPTensor
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
+def conv2d(x: HIPTensor, weight: HIPTensor, bias: HIPTensor | None = None, stride=1, padding=0,
+           dilation=1) -> HIPTensor:
+    """``(call (Conv2D c-in c-out kernel-size ...) x)``: ``x`` is ``[N C_in H W]``,
+    ``weight`` ``[C_out C_in k-h k-w]``, the result ``[N C_out H_out W_out]`` (a
+    permuted view of the ``[N H_out W_out C_out]`` product, as in the reference)."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    N, _, H, W = x.shape
+    c_out, _, kh, kw = weight.shape
+    h_out = F.conv_out_size(H, padding[0], dilation[0], kh, stride[0])
+    w_out = F.conv_out_size(W, padding[1], dilation[1], kw, stride[1])
+    col = F.unfold(x, dilation, (kh, kw), stride, padding)          # [(N h w) (C k-h k-w)]
+    col_w = F.reshape(weight, c_out, -1)
+    out = F.matmul(col, F.t(col_w))                                  # [(N h w) C_out]
+    if bias is not None:
+        out = F.add(out, bias)
+    return F.reshape(out, N, h_out, w_out, c_out).permute(0, 3, 1, 2)
+
+
+def _pool(x: HIPTensor, kernel_size, stride, padding, reduce) -> HIPTensor:
+    kernel_size, stride, padding = _pair(kernel_size), _pair(stride), _pair(padding)
+    N, Cc, H, W = x.shape
+    h_out = (H + 2 * padding[0] - kernel_size[0]) // stride[0] + 1   # pool-out-size, pool.lisp:19-21
+    w_out = (W + 2 * padding[1] - kernel_size[1]) // stride[1] + 1
+    col = F.unfold(x, (1, 1), kernel_size, stride, padding)
+    windows = F.reshape(col, -1, kernel_size[0] * kernel_size[1])   # [(N h w C) (k-h k-w)]
+    red = reduce(windows)
+    return F.reshape(red, N, h_out, w_out, Cc).permute(0, 3, 1, 2)
+
+
+def max_pool2d(x: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
+    """``MaxPool2D`` (pool.lisp:83-93); padded positions hold 0, as in the
+    reference."""
+    return _pool(x, kernel_size, kernel_size if stride is None else stride, padding,
+                 lambda w: F.max(w, axis=1))
+
+
+def avg_pool2d(x: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
+    """``AvgPool2D`` (pool.lisp:95-105)."""
+    return _pool(x, kernel_size, kernel_size if stride is None else stride, padding,
+                 lambda w: F.mean(w, axis=1))

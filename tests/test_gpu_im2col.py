@@ -102,3 +102,47 @@ def test_im2col_argument_checks(gpu):
     assert lib.wf2hip_im2col_f32(c, *args(H=7), x) == -1           # the walk leaves the image
     assert lib.wf2hip_im2col_f32(c, *args(sh=0), x) == -1
     assert lib.wf2hip_col2im_f32(c, *args(kh=40), x) == -4
+
+
+def test_reference_unfold_vectors(gpu):
+    """source/nn/t/conv.lisp:41-56: unfold of (ax+b (2 2 2 2) 1 0) with a 2x2
+    kernel is 0..15, and the backward of sum(out * (ax+b (2 8) 1 0)) through
+    Col2ImNode is 0..15 again; Conv2D 3 -> 6, 2x2 on (3 3 10 10) gives (3 6 9 9)
+    (:6)."""
+    W = gpu
+    F = W.functional
+    img = F.from_numpy(np.arange(16, dtype=np.float32).reshape(2, 2, 2, 2))
+    out = F.unfold(img, (1, 1), (2, 2), (1, 1), (0, 0))
+    assert out.shape == [2, 8]
+    assert np.array_equal(out.numpy().ravel(), np.arange(16, dtype=np.float32))
+    # d/d img of sum(out * g): g laid back as Col[N C kh kw 1 1], folded by Col2ImNode
+    g = np.arange(16, dtype=np.float32).reshape(2, 1, 1, 2, 2, 2).transpose(0, 3, 4, 5, 1, 2)
+    back = W.HIPTensor([2, 2, 2, 2])
+    W.forward("Col2ImNode", F.from_numpy(np.ascontiguousarray(g)), back, (1, 1), (0, 0), (1, 1))
+    assert np.array_equal(back.numpy().ravel(), np.arange(16, dtype=np.float32))
+    rng = np.random.default_rng(0)
+    y = W.nn.conv2d(F.from_numpy(rng.standard_normal((3, 3, 10, 10)).astype(np.float32)),
+                    F.from_numpy(rng.standard_normal((6, 3, 2, 2)).astype(np.float32)),
+                    F.from_numpy(rng.standard_normal(6).astype(np.float32)))
+    assert y.shape == [3, 6, 9, 9]
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_conv_and_pooling_layers(gpu, stride):
+    """Conv2D / MaxPool2D / AvgPool2D composed from the nodes, against float64
+    closed forms (no padding: with padding the reference's walk leaves the last
+    rows of Col untouched, which the im2col tests above pin instead)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(stride)
+    x = rng.standard_normal((2, 3, 12, 11)).astype(np.float32)
+    w = rng.standard_normal((5, 3, 3, 2)).astype(np.float32)
+    b = rng.standard_normal(5).astype(np.float32)
+    y = W.nn.conv2d(F.from_numpy(x), F.from_numpy(w), F.from_numpy(b), stride=stride).numpy()
+    win = np.lib.stride_tricks.sliding_window_view(x.astype(np.float64), (3, 2), axis=(2, 3))[:, :, ::stride, ::stride]
+    want = np.einsum("nchwij,ocij->nohw", win, w.astype(np.float64)) + b[None, :, None, None]
+    np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-5)
+    pw = np.lib.stride_tricks.sliding_window_view(x, (2, 2), axis=(2, 3))[:, :, ::2, ::2]
+    assert_bit_equal(W.nn.max_pool2d(F.from_numpy(x), 2).numpy(), pw.max(axis=(4, 5)), "max pool")
+    np.testing.assert_allclose(W.nn.avg_pool2d(F.from_numpy(x), 2).numpy(),
+                               pw.astype(np.float64).mean(axis=(4, 5)), rtol=1e-6, atol=1e-6)
