@@ -57,7 +57,8 @@ struct AttnParams {
   float scale_log2e;
 };
 
-__global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_kernel(
+    AttnParams p) {  // two workgroups per CU: at most 256 registers per lane
   extern __shared__ __attribute__((aligned(16))) float smem[];
   auto lds_k = [&](int stage) { return smem + stage * kStageFloats; };
   auto lds_v = [&](int stage) { return smem + stage * kStageFloats + kKBlock * kRowFloats; };
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
   //           the half-waves read rows 4 apart and then hit different banks.
   // Rows beyond the sequence are clamped (their scores are masked later); chunks
   // beyond head_dim are not loaded and stay zero from the clear below.
-  auto fetch = [&](int stage, int key0) {
+  auto fetch = [&](bool values, int stage, int key0) {
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -125,14 +126,10 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
       const int slot = lane & 15;
       int key = key0 + row;
       key = key < p.seq ? key : p.seq - 1;
-      const int kchunk = slot ^ (row & 15);
-      const int vchunk = slot ^ (((row >> 2) & 1) << 3);
-      if (kchunk * 4 < p.head_dim)
-        __builtin_amdgcn_global_load_lds(kp + (int64_t)key * p.ks[2] + kchunk * 4,
-                                         lds_k(stage) + q4 * 256, 16, 0, 0);
-      if (vchunk * 4 < p.head_dim)
-        __builtin_amdgcn_global_load_lds(vp + (int64_t)key * p.vs[2] + vchunk * 4,
-                                         lds_v(stage) + q4 * 256, 16, 0, 0);
+      const int chunk = values ? slot ^ (((row >> 2) & 1) << 3) : slot ^ (row & 15);
+      const float* src = values ? vp + (int64_t)key * p.vs[2] : kp + (int64_t)key * p.ks[2];
+      float* dst = (values ? lds_v(stage) : lds_k(stage)) + q4 * 256;
+      if (chunk * 4 < p.head_dim) __builtin_amdgcn_global_load_lds(src + chunk * 4, dst, 16, 0, 0);
     }
 #endif
   };
@@ -141,87 +138,121 @@ __global__ __launch_bounds__(kBlock) void attention_kernel(AttnParams p) {
       reinterpret_cast<f4*>(smem)[i] = f4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
   }
-  fetch(0, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
 
   const int kswz = col & 15;     // rows col and 32 + col share it
   const int vswap = half << 5;   // keys read by the upper half-wave have (key / 4) odd
 
-  for (int kb = 0; kb < nkb; kb++) {
-    const int key0 = kb * kKBlock;
-    const bool more = kb + 1 < nkb;
-    // the other stage was last read before the barrier that ended the previous block
-    if (more) fetch((kb + 1) & 1, key0 + kKBlock);
-    const float* sk = lds_k(kb & 1);
-    const float* sv = lds_v(kb & 1);
-
-    // a wavefront whose queries all precede this key block has nothing to add
-    const bool active = !(p.causal && key0 > q_last_wave);
-    if (active) {
-      f16v s0 = {0}, s1 = {0};
+  // S^T of one key block: two 32 x 32 tiles (keys 0-31 and 32-63 of the block)
+  auto scores = [&](const float* sk, f16v& s0, f16v& s1) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const int slot = ((2 * j + half) ^ kswz) * 4;
-        f4 k0 = *reinterpret_cast<const f4*>(sk + col * kRowFloats + slot);
-        f4 k1 = *reinterpret_cast<const f4*>(sk + (32 + col) * kRowFloats + slot);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[4 * j + 0], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[4 * j + 0], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.y, qf[4 * j + 1], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.y, qf[4 * j + 1], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.z, qf[4 * j + 2], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.z, qf[4 * j + 2], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.w, qf[4 * j + 3], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.w, qf[4 * j + 3], s1, 0, 0, 0);
-      }
-      // register i of tile t holds key key0 + 32 t + 8 (i/4) + 4 half + i%4
-      const bool edge = (p.causal && key0 + kKBlock - 1 > q_first) || key0 + kKBlock > p.seq;
-      if (edge) {
-        const int limit = p.causal ? min(query, p.seq - 1) : p.seq - 1;  // last visible key
+    for (int i = 0; i < 16; i++) {
+      s0[i] = 0.f;
+      s1[i] = 0.f;
+    }
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int key = key0 + 8 * (i >> 2) + 4 * half + (i & 3);
-          if (key > limit) s0[i] = -INFINITY;
-          if (key + 32 > limit) s1[i] = -INFINITY;
-        }
-      }
-      float mloc = s0[0];
-#pragma unroll
-      for (int i = 1; i < 16; i++) mloc = fmaxf(mloc, s0[i]);
-#pragma unroll
-      for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s1[i]);
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-      const float mnew = fmaxf(m, mloc);
-      // key 0 is visible to every query, so mnew is finite from the first block on
-      const float alpha = __builtin_amdgcn_exp2f(m - mnew);
-      m = mnew;
-      float psum = 0.f;
+    for (int j = 0; j < 8; j++) {
+      const int slot = ((2 * j + half) ^ kswz) * 4;
+      f4 k0 = *reinterpret_cast<const f4*>(sk + col * kRowFloats + slot);
+      f4 k1 = *reinterpret_cast<const f4*>(sk + (32 + col) * kRowFloats + slot);
+      s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[4 * j + 0], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[4 * j + 0], s1, 0, 0, 0);
+      s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.y, qf[4 * j + 1], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.y, qf[4 * j + 1], s1, 0, 0, 0);
+      s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.z, qf[4 * j + 2], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.z, qf[4 * j + 2], s1, 0, 0, 0);
+      s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.w, qf[4 * j + 3], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.w, qf[4 * j + 3], s1, 0, 0, 0);
+    }
+  };
+  // masks, running softmax statistics, P = exp2(S - max) in place
+  auto normalise = [&](int key0, f16v& s0, f16v& s1) {
+    // register i of tile t holds key key0 + 32 t + 8 (i/4) + 4 half + i%4
+    const bool edge = (p.causal && key0 + kKBlock - 1 > q_first) || key0 + kKBlock > p.seq;
+    if (edge) {
+      const int limit = p.causal ? min(query, p.seq - 1) : p.seq - 1;  // last visible key
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        s0[i] = __builtin_amdgcn_exp2f(s0[i] - mnew);
-        s1[i] = __builtin_amdgcn_exp2f(s1[i] - mnew);
-        psum += s0[i] + s1[i];
-      }
-      lsum = lsum * alpha + psum;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        o0[i] *= alpha;
-        o1[i] *= alpha;
-      }
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int key = 8 * (i >> 2) + 4 * half + (i & 3);
-        const float v00 = sv[key * kRowFloats + (col ^ vswap)];
-        const float v01 = sv[key * kRowFloats + ((32 + col) ^ vswap)];
-        const float v10 = sv[(32 + key) * kRowFloats + (col ^ vswap)];
-        const float v11 = sv[(32 + key) * kRowFloats + ((32 + col) ^ vswap)];
-        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v00, s0[i], o0, 0, 0, 0);
-        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v01, s0[i], o1, 0, 0, 0);
-        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v10, s1[i], o0, 0, 0, 0);
-        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v11, s1[i], o1, 0, 0, 0);
+        const int key = key0 + 8 * (i >> 2) + 4 * half + (i & 3);
+        if (key > limit) s0[i] = -INFINITY;
+        if (key + 32 > limit) s1[i] = -INFINITY;
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the next block landed
+    float mloc = s0[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mloc = fmaxf(mloc, s0[i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s1[i]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    const float mnew = fmaxf(m, mloc);
+    // key 0 is visible to every query, so mnew is finite from the first block on
+    const float alpha = __builtin_amdgcn_exp2f(m - mnew);
+    m = mnew;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      s0[i] = __builtin_amdgcn_exp2f(s0[i] - mnew);
+      s1[i] = __builtin_amdgcn_exp2f(s1[i] - mnew);
+      psum += s0[i] + s1[i];
+    }
+    lsum = lsum * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      o0[i] *= alpha;
+      o1[i] *= alpha;
+    }
+  };
+  // O^T += V^T . P^T
+  auto accumulate = [&](const float* sv, const f16v& s0, const f16v& s1) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int key = 8 * (i >> 2) + 4 * half + (i & 3);
+      const float v00 = sv[key * kRowFloats + (col ^ vswap)];
+      const float v01 = sv[key * kRowFloats + ((32 + col) ^ vswap)];
+      const float v10 = sv[(32 + key) * kRowFloats + (col ^ vswap)];
+      const float v11 = sv[(32 + key) * kRowFloats + ((32 + col) ^ vswap)];
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v00, s0[i], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v01, s0[i], o1, 0, 0, 0);
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v10, s1[i], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v11, s1[i], o1, 0, 0, 0);
+    }
+  };
+
+  // Software pipeline over key blocks: while the vector units work through the
+  // softmax of block kb, the matrix cores already form the scores of block
+  // kb + 1; then P V of block kb follows.  Keys are therefore staged one block
+  // further ahead than values:
+  //   top of iteration kb   fetch K(kb + 2) into the stage K(kb) left (its scores
+  //                         were formed before the last barrier), V(kb + 1) into
+  //                         the stage V(kb - 1) left
+  //   body                  scores of kb + 1 from K(kb + 1), softmax of kb, P V of
+  //                         kb from V(kb)
+  //   end                   wait for this wavefront's fetches, barrier
+  fetch(false, 0, 0);
+  fetch(true, 0, 0);
+  if (nkb > 1) fetch(false, 1, kKBlock);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  f16v n0, n1;  // scores of the next block
+  scores(lds_k(0), n0, n1);
+  __syncthreads();  // every wavefront has read K(0) before its stage is refilled
+
+  for (int kb = 0; kb < nkb; kb++) {
+    const int key0 = kb * kKBlock;
+    if (kb + 2 < nkb) fetch(false, kb & 1, key0 + 2 * kKBlock);
+    if (kb + 1 < nkb) fetch(true, (kb + 1) & 1, key0 + kKBlock);
+    // a wavefront whose queries all precede a key block has nothing to add there
+    const bool active = !(p.causal && key0 > q_last_wave);
+    const bool next_active = kb + 1 < nkb && !(p.causal && key0 + kKBlock > q_last_wave);
+    f16v s0 = n0, s1 = n1;
+    if (next_active) {  // implies active
+      scores(lds_k((kb + 1) & 1), n0, n1);
+      normalise(key0, s0, s1);
+      accumulate(lds_v(kb & 1), s0, s1);
+    } else if (active) {
+      normalise(key0, s0, s1);
+      accumulate(lds_v(kb & 1), s0, s1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's fetches have landed
     __syncthreads();
   }
 
