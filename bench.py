@@ -147,6 +147,142 @@ def counter_probe(W, reps: int = 5):
     print(json.dumps({"probe": "copy, add, mul, exp, rowsum", "launches_each": reps, "elements": N}))
 
 
+def row_table(W, reps: int = 10, warm: int = 3):
+    """One line per kernel of the path at the shape its configuration names:
+    average launch time from an event pair on the library's stream, the
+    algorithmic bytes (or flop) of one call, and the fraction of the roofline
+    that bounds it.  Each call of a row works on another buffer set of a ring
+    of at least 1 GiB, so operands are cold with respect to the 256 MB
+    Infinity Cache.  `ms` is per call inside a replayed HIP graph of `reps`
+    calls after about 15 ms of the same load (the sustained rate), `eager_ms`
+    the first `reps` calls issued one by one from this process (host time
+    between launches and the clock ramp included).  The rows go through the same host functions a model
+    uses (the time of a row that is several nodes is the sum of its launches)."""
+    F = W.functional
+    T = W.HIPTensor
+    rng = np.random.Generator(np.random.PCG64(6))
+    rows = {}
+
+    def ring_of(make, nbytes):
+        count = max(2, min(16, -(-(1 << 30) // max(nbytes, 1))))
+        return [make() for _ in range(count)]
+
+    def uniform(shape, lo, hi):
+        return T.from_numpy(rng.uniform(lo, hi, size=shape).astype(np.float32))
+
+    def normal(shape, scale=1.0):
+        return T.from_numpy((rng.standard_normal(shape) * scale).astype(np.float32))
+
+    def clone(t):
+        return F.copy(t)
+
+    def measure(label, ring, call, work, bound="hbm", note=None):
+        for i in range(warm):
+            call(ring[i % len(ring)])
+        a, b = W.lib.Event(), W.lib.Event()
+        a.record()
+        for i in range(reps):
+            call(ring[(warm + i) % len(ring)])
+        b.record()
+        eager_ms = a.elapsed_ms(b) / reps
+        # the same `reps` calls recorded once and replayed as one HIP graph: the launch
+        # times without the host work between them (Python here, Lisp in the product)
+        W.lib.synchronize()
+        with W.lib.Graph() as g:
+            for i in range(reps):  # results are dropped: the recording keeps their blocks
+                call(ring[i % len(ring)])
+        # the core clock dips for some milliseconds when a heavy load starts and then
+        # settles: replay about 15 ms of work before the timed replays
+        for _ in range(max(1, min(60, int(15.0 / max(reps * eager_ms, 1e-3)) + 1))):
+            g.launch()
+        a.record()
+        for _ in range(3):
+            g.launch()
+        b.record()
+        ms = a.elapsed_ms(b) / (3 * reps)
+        g.destroy()
+        if bound == "hbm":
+            rate, peak, unit = work / ms / 1e6, HBM_PEAK_GBS, "GB/s"
+        else:
+            rate, peak, unit = work / ms / 1e9, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        rows[label] = {"ms": round(ms, 5), "eager_ms": round(eager_ms, 5), "achieved": round(rate, 1),
+                       "unit": unit, "frac": round(rate / peak, 4), "bound": bound}
+        if note:
+            rows[label]["note"] = note
+        ring.clear()
+
+    # contiguous (1024, 1024): the reference's own CPU-sized case; 12 MiB per call is
+    # launch- and ramp-bound, not bandwidth-bound
+    a0, b0 = normal([1024, 1024]), normal([1024, 1024])
+    ring = ring_of(lambda: (clone(a0), clone(b0)), 8 << 20)
+    measure("add (1024,1024) in place", ring, lambda s: F.add_(s[0], s[1]), 12 << 20)
+
+    # strided / broadcast views on (4096, 8192)
+    R, Cn = 4096, 8192
+    a0, b0 = normal([R, Cn]), normal([1, Cn])
+    ring = ring_of(lambda: clone(a0), 4 * R * Cn)
+    yb = b0.view((":broadcast", R), True)
+    measure("A(4096,8192) += B(1,8192) row broadcast", ring, lambda s: F.add_(s, yb), 8 * R * Cn + 4 * Cn)
+    ring = ring_of(lambda: clone(a0), 4 * R * Cn)
+    measure("A[:, 0:8192:2] *= 0.5", ring, lambda s: F.mul_(s.view(True, (0, Cn, 2)), 0.5), 8 * R * Cn // 2,
+            note="8 B per element of the slice; the hardware moves every 32-byte sector whole, "
+                 "twice these bytes")
+    ring = ring_of(lambda: (clone(a0), T([2048, Cn], initial_element=None)), 4 * R * Cn + 4 * 2048 * Cn)
+    measure("C = A[1024:3072] - A[0:2048] (copy node + in-place sub)", ring,
+            lambda s: F.sub_(F.move_(s[1], s[0].view((1024, 3072), True)), s[0].view((0, 2048), True)),
+            (8 + 12) * 2048 * Cn, note="two launches: MoveTensorNode 8 B/elem, SubNode 12 B/elem")
+    del a0, b0, yb
+
+    # unary functions on 2^26 elements in the ranges of the configuration
+    for label, fn, lo, hi in (("exp", F.exp, -10.0, 10.0), ("tanh", F.tanh, -10.0, 10.0),
+                              ("sin", F.sin, -100.0, 100.0), ("loge", F.loge, 1e-3, 1e3)):
+        x0 = uniform([N], lo, hi)
+        ring = ring_of(lambda: (clone(x0), T([N], initial_element=None)), 8 * N)
+        measure(f"{label} 2^26 in [{lo:g}, {hi:g}]", ring, lambda s, fn=fn: fn(s[0], out=s[1]), 8 * N)
+        del x0
+
+    # reductions and softmax
+    R, Cn = 8192, 4096
+    x0 = normal([R, Cn])
+    ring = ring_of(lambda: (clone(x0), T([R, 1])), 4 * R * Cn)
+    measure("row sum (8192,4096) as !sum composes it", ring,
+            lambda s: F.sum(s[0], axis=1, out=s[1], keepdims=True), 4 * R * Cn + 12 * R,
+            note="zero fill of out + accumulation into the stride-0 view")
+    ring = ring_of(lambda: (clone(x0), T([1, 1])), 4 * R * Cn)
+    measure("full sum (8192,4096)", ring, lambda s: F.sum(s[0], axis=True, out=s[1], keepdims=True),
+            4 * R * Cn, note="two launches: partial sums per block, then their sum")
+    del x0
+    R, Cn = 32768, 1024
+    x0 = normal([R, Cn], 3.0)
+    ring = ring_of(lambda: (clone(x0), T([R, Cn], initial_element=None)), 8 * R * Cn)
+    measure("row softmax (32768,1024), one kernel", ring, lambda s: F.softmax_fused(s[0], out=s[1]), 8 * R * Cn)
+    ring = ring_of(lambda: clone(x0), 4 * R * Cn)
+    measure("row softmax (32768,1024), node for node (!softmax)", ring, lambda s: F.softmax(s), 8 * R * Cn,
+            note="mean, sub, exp, sum, div as separate nodes with their temporaries; "
+                 "rate quoted on the 8 B/elem of the fused form")
+    del x0
+
+    # products on fp32 MFMA, random data
+    for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),
+                    (8192, 768, 3072)):
+        a0, b0 = normal([m, k]), normal([k, n])
+        ring = ring_of(lambda: (clone(a0), clone(b0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
+        measure(f"matmul {m}x{n}x{k}", ring, lambda s: F.matmul(s[0], s[1], out=s[2]), 2.0 * m * n * k,
+                bound="mfma")
+        del a0, b0
+    B, H, S, hd = 8, 12, 1024, 64
+    q0 = normal([B, H, S, hd])
+    for causal in (True, False):
+        ring = ring_of(lambda: (clone(q0), clone(q0), clone(q0), T([B, H, S, hd], initial_element=None)),
+                       16 * B * H * S * hd)
+        flop = 4.0 * B * H * S * S * hd * (0.5 if causal else 1.0)
+        measure(f"attention (8,12,1024,64) {'causal' if causal else 'full'}", ring,
+                lambda s, c=causal: F.attention(s[0], s[1], s[2], out=s[3], causal=c), flop, bound="mfma",
+                note="flop of the useful half of the score matrix" if causal else None)
+    del q0
+    return rows
+
+
 def block_forward_ms(W, reps: int = 20, warm: int = 10):
     try:
         gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
@@ -254,6 +390,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-block", action="store_true")
+    ap.add_argument("--no-rows", action="store_true",
+                    help="skip the table of the other kernels of the path at their configured shapes")
     ap.add_argument("--probe", action="store_true",
                     help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
@@ -311,6 +449,8 @@ def main():
             "avg_launch_ms": round(binary_ms, 5),
         },
     }
+    if not args.no_rows:
+        result["rows"] = row_table(W)
     if not args.no_block:
         blk = block_forward_ms(W)
         if blk is not None:
