@@ -8,6 +8,7 @@
 #pragma once
 
 #include <stdint.h>
+#include <initializer_list>
 
 #include "wf2_common.h"
 
@@ -103,6 +104,22 @@ inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {
   const float* b0 = b + blo;
   const float* b1 = b + bhi;
   if (a1 < b0 || b1 < a0) return false;
+  // Interleaved lattices (the even against the odd elements of one buffer): every
+  // address of a window is its start plus a multiple of g = gcd of all strides of
+  // both windows, so starts that differ modulo g never meet.
+  int64_t g = 0;
+  for (int r = 0; r < s.rank; r++) {
+    if (s.shape[r] <= 1) continue;
+    for (int64_t v : {s.sa[r], s.sb[r]}) {
+      if (v < 0) v = -v;
+      while (v != 0) {
+        int64_t t = g % v;
+        g = v;
+        v = t;
+      }
+    }
+  }
+  if (g > 1 && ((a + s.off_a) - (b + s.off_b)) % g != 0) return false;
   if (a + s.off_a != b + s.off_b) return true;
   for (int r = 0; r < s.rank; r++)
     if (s.sa[r] != s.sb[r]) return true;

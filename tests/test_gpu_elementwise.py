@@ -121,6 +121,61 @@ def test_config2_views(gpu, O):
     assert_bit_equal(got.numpy(), A[1024:3072] - A[0:2048], "offset views")
 
 
+def test_inplace_on_every_second_element(gpu):
+    """In-place ops on [::2] slices (the kernel that stores whole vectors and
+    writes the in-between elements back as read): row pitches and start columns
+    that break the 16-byte alignment of the rows, every kind of second operand,
+    the whole storage compared so that untouched elements are checked too; and
+    the layout where rows interleave (an (n, 2) tensor seen as (2, n)), which must
+    not take that kernel.  Closed form: IEEE binary32 arithmetic in numpy."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(77)
+    f32 = np.float32
+    for rows, pitch, start, count in [(5, 1000, 0, 500), (7, 1001, 1, 450), (3, 4099, 3, 2000),
+                                      (4, 514, 2, 256), (1, 70001, 5, 30000), (6, 300, 0, 150)]:
+        base = rng.standard_normal((rows, pitch)).astype(f32)
+        sel = np.s_[:, start:start + 2 * count:2]
+        for kind in ("scalar", "contiguous", "slice", "row", "column"):
+            t = F.from_numpy(base)
+            v = t.view(True, (start, start + 2 * count, 2))
+            assert v.shape == [rows, count]
+            want = base.copy()
+            if kind == "scalar":
+                F.mul_(v, 0.37)
+                want[sel] *= f32(0.37)
+            elif kind == "contiguous":
+                y = rng.standard_normal((rows, count)).astype(f32)
+                F.add_(v, F.from_numpy(y))
+                want[sel] += y
+            elif kind == "slice":
+                ybase = rng.standard_normal((rows, 2 * count + 3)).astype(f32)
+                F.sub_(v, F.from_numpy(ybase).view(True, (1, 1 + 2 * count, 2)))
+                want[sel] -= ybase[:, 1:1 + 2 * count:2]
+            elif kind == "row":
+                y = (rng.standard_normal((1, count)) + 3.0).astype(f32)
+                F.div_(v, F.from_numpy(y).view((":broadcast", rows), True))
+                want[sel] /= y
+            else:
+                y = rng.standard_normal((rows, 1)).astype(f32)
+                F.mul_(v, F.from_numpy(y).view(True, (":broadcast", count)))
+                want[sel] *= y
+            assert_bit_equal(t.numpy(), want, f"[::2] in place, {kind}, rows {rows} pitch {pitch} start {start}")
+    # even and odd elements of one storage against each other
+    base = rng.standard_normal((8, 2048)).astype(f32)
+    t = F.from_numpy(base)
+    F.add_(t.view(True, (0, 2046, 2)), t.view(True, (1, 2048, 2)))  # 1023 elements each (floor((to-from)/step))
+    want = base.copy()
+    want[:, 0:2046:2] += base[:, 1:2047:2]
+    assert_bit_equal(t.numpy(), want, "even += odd")
+    # interleaved rows
+    base = rng.standard_normal((3000, 2)).astype(f32)
+    y = rng.standard_normal((2, 3000)).astype(f32)
+    t = F.from_numpy(base)
+    F.add_(t.permute(1, 0), F.from_numpy(y))
+    assert_bit_equal(t.numpy(), base + y.T, "(n, 2) seen as (2, n)")
+
+
 def _random_view(rng, n):
     """A random subscript for an axis of extent n."""
     k = rng.integers(0, 6)
