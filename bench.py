@@ -227,6 +227,10 @@ def row_table(W, reps: int = 10, warm: int = 3):
     measure("A[:, 0:8192:2] *= 0.5", ring, lambda s: F.mul_(s.view(True, (0, Cn, 2)), 0.5), 8 * R * Cn // 2,
             note="8 B per element of the slice; the hardware moves every 32-byte sector whole, "
                  "twice these bytes")
+    ring = ring_of(lambda: (clone(a0), T([R, Cn // 2], initial_element=None)), 6 * R * Cn)
+    measure("copy of A[:, 0:8192:2] into a contiguous tensor", ring,
+            lambda s: F.move_(s[1], s[0].view(True, (0, Cn, 2))), 8 * R * Cn // 2,
+            note="8 B per element; the reads move every sector whole (2.5x these bytes in all)")
     ring = ring_of(lambda: (clone(a0), T([2048, Cn], initial_element=None)), 4 * R * Cn + 4 * 2048 * Cn)
     measure("C = A[1024:3072] - A[0:2048] (copy node + in-place sub)", ring,
             lambda s: F.sub_(F.move_(s[1], s[0].view((1024, 3072), True)), s[0].view((0, 2048), True)),
