@@ -130,6 +130,15 @@ def _softmax64(x):
     return e / e.sum(axis=-1, keepdims=True)
 
 
+def _assert_softmax(got, want64, what=""):
+    """The fused kernel's bound: exp(x - max) carries the binary32 rounding of
+    x - max (|x - max| 2^-24 relative: 4e-6 at the underflow edge) plus a few ulp
+    of the exponential, the row sum and the final product; the bar for this
+    configuration is 1e-5 relative.  Results below the normal range are flushed
+    to zero (atol)."""
+    np.testing.assert_allclose(got, want64, rtol=4e-6, atol=1.2e-38, err_msg=what)
+
+
 def test_config4_softmax(gpu):
     """BASELINE config 4: max-subtracted row softmax of (32768, 1024) N(0, 3^2)
     logits, seed 4 -- fused kernel against the float64 closed form; invariants
@@ -142,7 +151,8 @@ def test_config4_softmax(gpu):
     X = (rng.standard_normal((32768, 1024)) * 3.0).astype(np.float32)
     got = F.softmax_fused(F.from_numpy(X)).numpy()
     want = _softmax64(X)
-    assert ulp_distance(got, want.astype(np.float32)).max() <= 2
+    _assert_softmax(got, want, "config 4")
+    assert np.abs(got / want - 1.0)[want > 1e-30].mean() < 4e-7  # typical error: a few ulp
     assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
     shifted = F.softmax_fused(F.from_numpy(X[:256] + np.float32(8.0))).numpy()
     np.testing.assert_allclose(shifted, _softmax64(X[:256] + np.float32(8.0)), rtol=1e-5, atol=1e-12)
@@ -154,7 +164,10 @@ def test_softmax_widths(gpu, cols):
     rng = np.random.default_rng(cols)
     X = (rng.standard_normal((37, cols)) * 4).astype(np.float32)
     got = F.softmax_fused(F.from_numpy(X)).numpy()
-    assert ulp_distance(got, _softmax64(X).astype(np.float32)).max() <= 2
+    if cols <= 4096:
+        _assert_softmax(got, _softmax64(X), f"{cols} columns")
+    else:  # rows too long for registers: the three-pass binary64 kernel
+        assert ulp_distance(got, _softmax64(X).astype(np.float32)).max() <= 2
 
 
 def test_softmax_reference_composition(gpu, O):
@@ -197,7 +210,7 @@ def test_causal_softmax(gpu):
         want = _softmax64(s)
         got = out.numpy()
         assert np.all(got[:, ~mask] == 0.0)
-        assert ulp_distance(got, want.astype(np.float32)).max() <= 2
+        _assert_softmax(got, want, f"causal {batch}x{seq}")
 
 
 def test_layernorm(gpu):
