@@ -170,14 +170,18 @@ __device__ __forceinline__ void map_tile(const GemmParams& p, bool triangular, u
 // One output element: C = act(alpha acc + beta C + bias) + residual; the caller
 // fetches bias and residual (once per column, and in batches) so that the
 // loads are not strung out one dependent access per element.
-template <bool FUSED>
+// FUSED: 0 plain, 1 bias / residual / triangular skipping, 2 the same plus an
+// activation.  The activation's binary64 body is long; keeping it out of the
+// instantiations that never apply it shortens their epilogues by ~12 us at
+// 8192 x 2304 x 768 (48 inlined copies that every element had to branch around).
+template <int FUSED>
 __device__ __forceinline__ float finish_value(const GemmParams& p, float accv, float cold,
                                               float biasv, float resv) {
   float v = p.alpha * accv;
   if (p.beta != 0.0f) v += p.beta * cold;
   if constexpr (FUSED) {
     if (p.bias) v += biasv;
-    if (p.activation == 1) v = gelu_tanh_f(v);
+    if (FUSED == 2 && p.activation == 1) v = gelu_tanh_f(v);
     if (p.residual) v += resv;
   }
   return v;
@@ -187,7 +191,7 @@ __device__ __forceinline__ float finish_value(const GemmParams& p, float accv, f
 // tile is (64 TM) x (64 TN).  2x2 -> 128x128 (64 accumulator registers), 2x1
 // -> 128x64 for narrow outputs and for shapes whose 128x128 tiling would leave
 // a partial last round of workgroups.
-template <bool LKIN, bool RKIN, bool FAST, int TM, int TN, bool FUSED>
+template <bool LKIN, bool RKIN, bool FAST, int TM, int TN, int FUSED>
 __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
   constexpr int BMt = 64 * TM, BNt = 64 * TN;
   constexpr int LFLOATS = LKIN ? BMt * KPITCH : BK * BMt;
@@ -295,7 +299,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
           if (p.beta != 0.0f) v += p.beta * *c;
           if constexpr (FUSED) {
             if (p.bias) v += p.bias[col];
-            if (p.activation == 1) v = gelu_tanh_f(v);
+            if (FUSED == 2 && p.activation == 1) v = gelu_tanh_f(v);
             if (p.residual)
               v += p.residual[(int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes + row * p.ldres + col];
           }
@@ -332,22 +336,31 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 //                     bytes apart so the two half-waves hit different banks.
 //                     [32][192] (128 x 192 tile): columns 0-63 of a wavefront's 96
 //                     are shared by tiles 0 and 1 as above, 64-95 belong to tile 2.
-template <bool RKIN, int TN>
+//   tall layout       the four wavefronts are stacked along M (32 rows x 32 TN columns
+//                     each, TN = 3: a 128 x 96 tile, which divides N = 768 and 2304
+//                     into whole tiles and 8192 x 768 outputs into exactly two tiles
+//                     per CU).  x-innermost right tile: [3 column blocks][32 k][32];
+//                     every DMA instruction fills eight k-rows of a block, stored in
+//                     the order 0 4 1 5 2 6 3 7, so that the value lane l needs for
+//                     k = 8 g + 4 (l / 32) + s sits at float 64 s + l of the
+//                     instruction's 1 KB: plain conflict-free 32-bit reads.
+template <bool RKIN, int TN, bool TALL = false>
 struct DmaLayout {
-  static constexpr int BNt = 64 * TN;
+  static constexpr int BNt = TALL ? 32 * TN : 64 * TN;
   static constexpr int LFLOATS = 128 * BK;
   // instructions per workgroup and K-step for the right operand, rows each covers
   static constexpr int R_INSTRS = BNt * BK / 256;  // 64 pieces of 16 bytes each
-  static constexpr int R_INSTR_PITCH = (!RKIN && TN == 1) ? 288 : 256;  // floats
+  static constexpr int R_INSTR_PITCH = (!RKIN && TN == 1 && !TALL) ? 288 : 256;  // floats
   static constexpr int RFLOATS = R_INSTRS * R_INSTR_PITCH;
   static constexpr int STAGE = LFLOATS + RFLOATS;
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE * sizeof(float);
 };
 
-template <bool RKIN, int TN, bool FUSED>
+template <bool RKIN, int TN, int FUSED, bool TALL = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void sgemm_dma_kernel(
     GemmParams p) {  // two workgroups per CU: at most 256 registers per lane
-  using Lay = DmaLayout<RKIN, TN>;
+  using Lay = DmaLayout<RKIN, TN, TALL>;
+  constexpr int MI = TALL ? 1 : 2;  // 32-row MFMA tiles per wavefront along M
   constexpr int BMt = 128, BNt = Lay::BNt;
   extern __shared__ __attribute__((aligned(16))) float smem[];
   auto ldsL = [&](int stage) { return smem + stage * Lay::STAGE; };
@@ -368,8 +381,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const int wave = threadIdx.x / kWave;
   const int half = lane >> 5;
   const int col = lane & 31;
-  const int wm = (wave >> 1) * 64;
-  const int wn = (wave & 1) * 32 * TN;
+  const int wm = TALL ? wave * 32 : (wave >> 1) * 64;
+  const int wn = TALL ? 0 : (wave & 1) * 32 * TN;
 
   // Global source of every 16-byte piece this lane moves per K-step (k = 0);
   // rows / columns beyond the matrix are clamped to its last ones: they only
@@ -395,6 +408,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       int64_t gn = n0 + row;
       gn = gn < p.N ? gn : p.N - 1;
       srcR[j] = R + gn * p.ldr + chunk * 4;
+    } else if (TALL) {
+      // instruction q: column block q / 4, k-rows 8 (q % 4) + {0 4 1 5 2 6 3 7}[lane / 8]
+      const int slot = lane >> 3;
+      const int krow = 8 * (q & 3) + (slot >> 1) + 4 * (slot & 1);
+      int64_t gn = n0 + 32 * (q >> 2) + 4 * (lane & 7);
+      gn = gn < p.N ? gn : p.N - 4;
+      srcR[j] = R + (int64_t)krow * p.ldr + gn;
     } else {
       constexpr int CPR = BNt / 4;  // 16-byte pieces per k-row; LDS keeps [k][BNt] densely
       const int piece = q * 64 + lane;
@@ -416,17 +436,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #endif
   };
 
-  f16v acc[2][TN];
+  f16v acc[MI][TN];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < MI; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  int lrow[2], lswz[2], rrow[TN], rswz[TN];
+  int lrow[MI], lswz[MI], rrow[TN], rswz[TN];
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < MI; i++) {
     lrow[i] = wm + i * 32 + col;
     lswz[i] = (lrow[i] >> 1) & 7;
   }
@@ -437,22 +457,27 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   }
 
   // fragments of k-group g (k = 8 g + 4 half + s, s = 0..3) into buffer `buf`
-  float a[2][2][4], b[2][TN][4];
+  float a[2][MI][4], b[2][TN][4];
   auto read_frags = [&](int stage, int g, int buf) {
     const float* sl = ldsL(stage);
     const float* sr = ldsR(stage);
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int i = 0; i < MI; i++) {
       const f4 v = *reinterpret_cast<const f4*>(sl + lrow[i] * BK + ((2 * g + half) ^ lswz[i]) * 4);
       a[buf][i][0] = v.x; a[buf][i][1] = v.y; a[buf][i][2] = v.z; a[buf][i][3] = v.w;
     }
-    if (RKIN) {
+    if constexpr (RKIN) {
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const f4 v = *reinterpret_cast<const f4*>(sr + rrow[j] * BK + ((2 * g + half) ^ rswz[j]) * 4);
         b[buf][j][0] = v.x; b[buf][j][1] = v.y; b[buf][j][2] = v.z; b[buf][j][3] = v.w;
       }
-    } else if (TN >= 2) {
+    } else if constexpr (TALL) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int s4 = 0; s4 < 4; s4++) b[buf][j][s4] = sr[(4 * j + g) * 256 + 64 * s4 + lane];
+    } else if constexpr (TN >= 2) {
 #pragma unroll
       for (int s4 = 0; s4 < 4; s4++) {
         const float* krow = sr + (8 * g + 4 * half + s4) * BNt + wn;
@@ -473,7 +498,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 #pragma unroll
     for (int s4 = 0; s4 < 4; s4++)
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[buf][i][s4], b[buf][j][s4], acc[i][j], 0, 0, 0);
@@ -481,12 +506,28 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   // keeps the LDS reads of the next k-group among the first MFMAs of this one
   auto pin_order = [&]() {
 #if defined(__HIP_DEVICE_COMPILE__)
+    if (TALL) {
+      // 4 TN MFMAs; LDS reads of the next group: one 128-bit read for the left
+      // fragment, and for the right one TN 128-bit reads (k-innermost) or 2 TN
+      // ds_read2st64_b32 (the compiler pairs the 4 TN 32-bit reads).  All of them
+      // go among the first MFMAs, the rest of the group runs without.
+      // A read right before the group's first MFMA would sit in front of the wait
+      // for the fragments that MFMA needs, so an MFMA leads.
+      constexpr int NR = 1 + (RKIN ? TN : 2 * TN);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+      for (int q = 0; q < NR; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * TN - NR, 0);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * TN, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4 * TN, 0);
 #endif
   };
 
@@ -517,8 +558,78 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
   const int64_t res_base = (int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes;
-  const bool pairs = !RKIN && TN >= 2 && p.pair_ok;
+  const bool pairs = !TALL && !RKIN && TN >= 2 && p.pair_ok;
   const float* res = (FUSED && p.residual) ? p.residual + res_base : nullptr;
+  if constexpr (!TALL) {
+    // The same for the 2 x 2 wavefront layouts: tiles wholly inside the output
+    // take an epilogue without guards, with one 64-bit multiply per lane and, per
+    // 32-row block, every load ahead of the first store.
+    if (p.beta == 0.0f && m0 + BMt <= p.M && n0 + BNt <= p.N) {
+      constexpr bool INTER = !RKIN && TN >= 2;  // tiles 0 and 1 own columns 2 c, 2 c + 1
+      const int64_t row0 = m0 + wm + 4 * half;
+      if (INTER && p.pair_ok) {
+        float* cl = C + row0 * p.ldc + n0 + wn + 2 * col;
+        const float* rl = res ? res + row0 * p.ldres + n0 + wn + 2 * col : nullptr;
+        float bias0 = 0.f, bias1 = 0.f, bias2 = 0.f;
+        if (FUSED && p.bias) {
+          bias0 = p.bias[n0 + wn + 2 * col];
+          bias1 = p.bias[n0 + wn + 2 * col + 1];
+          if (TN == 3) bias2 = p.bias[n0 + wn + 64 + col];
+        }
+#pragma unroll
+        for (int i = 0; i < MI; i++) {
+          f2 rs[16];
+          float rs2[16];
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int64_t ro = (int64_t)(32 * i + 8 * (r >> 2) + (r & 3));
+            rs[r] = rl ? *reinterpret_cast<const f2*>(rl + ro * p.ldres) : f2{0.f, 0.f};
+            if (TN == 3) rs2[r] = rl ? rl[ro * p.ldres + 64 - col] : 0.f;
+          }
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int64_t ro = (int64_t)(32 * i + 8 * (r >> 2) + (r & 3));
+            f2 v;
+            v.x = finish_value<FUSED>(p, acc[i][0][r], 0.f, bias0, rs[r].x);
+            v.y = finish_value<FUSED>(p, acc[i][TN >= 2 ? 1 : 0][r], 0.f, bias1, rs[r].y);
+            *reinterpret_cast<f2*>(cl + ro * p.ldc) = v;
+            if (TN == 3)
+              cl[ro * p.ldc + 64 - col] = finish_value<FUSED>(p, acc[i][TN - 1][r], 0.f, bias2, rs2[r]);
+          }
+#if defined(__HIP_DEVICE_COMPILE__)
+          __builtin_amdgcn_sched_barrier(0);
+#endif
+        }
+        return;
+      }
+      if (!INTER) {
+        float* cl = C + row0 * p.ldc + n0 + wn + col;
+        const float* rl = res ? res + row0 * p.ldres + n0 + wn + col : nullptr;
+        float biasv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) biasv[j] = (FUSED && p.bias) ? p.bias[n0 + wn + j * 32 + col] : 0.f;
+#pragma unroll
+        for (int i = 0; i < MI; i++) {
+          float rs[TN][16];
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+              rs[j][r] = rl ? rl[(int64_t)(32 * i + 8 * (r >> 2) + (r & 3)) * p.ldres + 32 * j] : 0.f;
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+              cl[(int64_t)(32 * i + 8 * (r >> 2) + (r & 3)) * p.ldc + 32 * j] =
+                  finish_value<FUSED>(p, acc[i][j][r], 0.f, biasv[j], rs[j][r]);
+#if defined(__HIP_DEVICE_COMPILE__)
+          __builtin_amdgcn_sched_barrier(0);
+#endif
+        }
+        return;
+      }
+    }
+  }
   if (pairs) {
     const int64_t c0 = n0 + wn + 2 * col;  // even; N is a multiple of 4 here
     if (c0 < p.N) {
@@ -528,7 +639,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         bias1 = p.bias[c0 + 1];
       }
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int h = 0; h < 2; h++) {  // eight rows at a time: loads first, then arithmetic and stores
           f2 old[8], rs[8];
@@ -561,14 +672,45 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     }
     if (TN < 3) return;
   }
+  if constexpr (TALL) {
+    // Tiles wholly inside the output (all of them when 128 | M and 96 | N): no
+    // per-element guards, one 64-bit multiply per lane (register r of a lane is
+    // 8 (r / 4) + r % 4 rows below the lane's first row: a constant times the
+    // pitch, computed on the scalar unit), and all loads of the epilogue (bias,
+    // residual) before the first store -- loads and stores share one counter on
+    // this hardware, so a load issued after stores is only known to have landed
+    // once those stores have drained.  Measured at 8192 x 2304 x 768 with a bias:
+    // 238 us with the guarded loop below, 225 us without a bias.
+    if (p.beta == 0.0f && m0 + BMt <= p.M && n0 + BNt <= p.N) {
+      const int64_t row0 = m0 + wm + 4 * half;
+      float* cl = C + row0 * p.ldc + n0 + col;
+      const float* rl = res ? res + row0 * p.ldres + n0 + col : nullptr;
+      float biasv[TN], rs[TN][16];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+      for (int j = 0; j < TN; j++) {
+        biasv[j] = (FUSED && p.bias) ? p.bias[n0 + j * 32 + col] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          rs[j][r] = rl ? rl[(int64_t)(8 * (r >> 2) + (r & 3)) * p.ldres + 32 * j] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          cl[(int64_t)(8 * (r >> 2) + (r & 3)) * p.ldc + 32 * j] =
+              finish_value<FUSED>(p, acc[0][j][r], 0.f, biasv[j], rs[j][r]);
+      return;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MI; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       if (pairs && j < 2) continue;  // stored above
       // tiles 0 and 1 of an n-innermost right operand own interleaved columns
-      const int64_t cc = (!RKIN && TN >= 2) ? (j < 2 ? n0 + wn + 2 * col + j : n0 + wn + 64 + col)
-                                            : n0 + wn + j * 32 + col;
+      const int64_t cc = (!TALL && !RKIN && TN >= 2)
+                             ? (j < 2 ? n0 + wn + 2 * col + j : n0 + wn + 64 + col)
+                             : n0 + wn + j * 32 + col;
       if (cc >= p.N) continue;
       const float biasv = (FUSED && p.bias) ? p.bias[cc] : 0.f;
 #pragma unroll
@@ -603,7 +745,7 @@ static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; 
 static bool is_n(char c) { return c == 'N' || c == 'n'; }
 static bool is_t(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
-template <bool LK, bool RK, bool FAST, int TM, int TN, bool FUSED>
+template <bool LK, bool RK, bool FAST, int TM, int TN, int FUSED>
 static int launch_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
   constexpr int lfloats = LK ? 64 * TM * KPITCH : BK * 64 * TM;
   constexpr int rfloats = RK ? 64 * TN * KPITCH : BK * 64 * TN;
@@ -620,30 +762,33 @@ static int launch_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
   return 0;
 }
 
-template <bool RK, int TN, bool FUSED>
+template <bool RK, int TN, int FUSED, bool TALL>
 static int launch_dma_kernel(const GemmParams& p, dim3 grid, hipStream_t st) {
-  constexpr size_t bytes = DmaLayout<RK, TN>::LDS_BYTES;
+  constexpr size_t bytes = DmaLayout<RK, TN, TALL>::LDS_BYTES;
   static bool configured = false;  // per instantiation
   if (!configured) {
-    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_dma_kernel<RK, TN, FUSED>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
-                      "hipFuncSetAttribute(sgemm_dma_kernel)"));
+    WF2_TRY(check_hip(
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_dma_kernel<RK, TN, FUSED, TALL>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+        "hipFuncSetAttribute(sgemm_dma_kernel)"));
     configured = true;
   }
-  sgemm_dma_kernel<RK, TN, FUSED><<<grid, kBlock, bytes, st>>>(p);
+  sgemm_dma_kernel<RK, TN, FUSED, TALL><<<grid, kBlock, bytes, st>>>(p);
   return 0;
 }
 
-// TN = 1, 2, 3: 128 x 64, 128 x 128, 128 x 192 output tiles
-template <int TN>
+// TN = 1, 2, 3: 128 x 64, 128 x 128, 128 x 192 output tiles; TALL with TN = 3: 128 x 96
+template <int TN, bool TALL = false>
 static int launch_dma(const GemmParams& p, bool rkin, dim3 grid, hipStream_t st) {
-  const bool fused = p.bias || p.residual || p.activation || p.causal;
+  const int fused = p.activation ? 2 : ((p.bias || p.residual || p.causal) ? 1 : 0);
   if (rkin) {
-    if (fused) return launch_dma_kernel<true, TN, true>(p, grid, st);
-    return launch_dma_kernel<true, TN, false>(p, grid, st);
+    if (fused == 2) return launch_dma_kernel<true, TN, 2, TALL>(p, grid, st);
+    if (fused == 1) return launch_dma_kernel<true, TN, 1, TALL>(p, grid, st);
+    return launch_dma_kernel<true, TN, 0, TALL>(p, grid, st);
   }
-  if (fused) return launch_dma_kernel<false, TN, true>(p, grid, st);
-  return launch_dma_kernel<false, TN, false>(p, grid, st);
+  if (fused == 2) return launch_dma_kernel<false, TN, 2, TALL>(p, grid, st);
+  if (fused == 1) return launch_dma_kernel<false, TN, 1, TALL>(p, grid, st);
+  return launch_dma_kernel<false, TN, 0, TALL>(p, grid, st);
 }
 
 template <bool LK, bool RK, int TM, int TN>
@@ -652,11 +797,11 @@ static int launch_variant(const GemmParams& p, bool fast, dim3 grid, hipStream_t
   // triangular skipping live in a separate instantiation
   const bool fused = p.bias || p.residual || p.activation || p.causal;
   if (fused) {
-    if (fast) return launch_kernel<LK, RK, true, TM, TN, true>(p, grid, st);
-    return launch_kernel<LK, RK, false, TM, TN, true>(p, grid, st);
+    if (fast) return launch_kernel<LK, RK, true, TM, TN, 2>(p, grid, st);
+    return launch_kernel<LK, RK, false, TM, TN, 2>(p, grid, st);
   }
-  if (fast) return launch_kernel<LK, RK, true, TM, TN, false>(p, grid, st);
-  return launch_kernel<LK, RK, false, TM, TN, false>(p, grid, st);
+  if (fast) return launch_kernel<LK, RK, true, TM, TN, 0>(p, grid, st);
+  return launch_kernel<LK, RK, false, TM, TN, 0>(p, grid, st);
 }
 
 template <int TM, int TN>
@@ -759,38 +904,43 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   // others back to back but ran 25 % slower between other kernels (8192 x 2304
   // x 768: 316 us against 245 us), so it is only reachable through the knob.
   const int64_t nb = (int64_t)batch * batch2;
-  const int widths[2] = {64, 128};
-  const double eff[2] = {0.94, 1.0};
-  int tn_tiles = 2;
+  // The 128x96 tile (streaming kernel only) exists for widths 128 and 64 leave
+  // ragged: N = 768 gives 8 whole tiles per row of tiles, 8192 x 768 outputs two
+  // tiles per CU, 8192 x 2304 six.
+  const int widths[3] = {64, 128, 96};
+  const double eff[3] = {0.94, 1.0, 0.97};
+  int width = 128;
   double best = 0.0;
-  for (int c = 0; c < 2; c++) {
+  for (int c = 0; c < (dma ? 3 : 2); c++) {
     const int64_t tiles = ceil_div(p.M, 128) * ceil_div(p.N, widths[c]) * nb;
     const double rounds = busiest_cu_tiles(tiles);
     const double cost = rounds * widths[c] / (eff[c] * (rounds < 2.0 ? 0.85 : 1.0));
     if (c == 0 || cost < best) {
       best = cost;
-      tn_tiles = c + 1;
+      width = widths[c];
     }
   }
-  if (const char* force = getenv("WF2HIP_GEMM_TILE")) {  // tuning knob: n(arrow), w(ide), x(tra wide)
-    tn_tiles = force[0] == 'n' ? 1 : (force[0] == 'x' && dma ? 3 : 2);
+  if (const char* force = getenv("WF2HIP_GEMM_TILE")) {  // tuning knob: n(arrow), w(ide), x(tra wide), t(all)
+    width = force[0] == 'n' ? 64 : (force[0] == 'x' && dma ? 192 : (force[0] == 't' && dma ? 96 : 128));
   }
   p.tiles_m = (uint32_t)ceil_div(p.M, 128);
-  p.tiles_n = (uint32_t)ceil_div(p.N, 64 * tn_tiles);
+  p.tiles_n = (uint32_t)ceil_div(p.N, width);
   const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many tiles");
   dim3 grid((uint32_t)blocks, (uint32_t)nb);
   hipStream_t st = rt().stream;
   if (dma) {
-    if (tn_tiles == 1)
+    if (width == 64)
       WF2_TRY((launch_dma<1>(p, rkin, grid, st)));
-    else if (tn_tiles == 2)
+    else if (width == 128)
       WF2_TRY((launch_dma<2>(p, rkin, grid, st)));
+    else if (width == 96)
+      WF2_TRY((launch_dma<3, true>(p, rkin, grid, st)));
     else
       WF2_TRY((launch_dma<3>(p, rkin, grid, st)));
     return after_launch("sgemm_dma_kernel");
   }
-  if (tn_tiles == 1)
+  if (width == 64)
     WF2_TRY((launch_layout<2, 1>(p, lkin, rkin, fast, grid, st)));
   else
     WF2_TRY((launch_layout<2, 2>(p, lkin, rkin, fast, grid, st)));

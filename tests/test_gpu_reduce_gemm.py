@@ -378,7 +378,7 @@ def test_matmul_causal_modes(gpu):
     with pytest.raises(gpu.HIPError):
         F.matmul(F.from_numpy(q[0, 0]), F.from_numpy(np.ones((hd, 5), np.float32)), causal=1)
 
-@pytest.mark.parametrize("tile", ["w", "n", "x"])
+@pytest.mark.parametrize("tile", ["w", "n", "x", "t"])
 @pytest.mark.parametrize("tb", [False, True])
 def test_matmul_streaming_kernel_matches_register_staged_kernel(gpu, monkeypatch, tile, tb):
     """K a multiple of 32 (from 256 on, or always with WF2HIP_GEMM_STREAM=1) and
