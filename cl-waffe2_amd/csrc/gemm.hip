@@ -181,7 +181,7 @@ __device__ __forceinline__ float finish_value(const GemmParams& p, float accv, f
   if (p.beta != 0.0f) v += p.beta * cold;
   if constexpr (FUSED) {
     if (p.bias) v += biasv;
-    if (FUSED == 2 && p.activation == 1) v = gelu_tanh_f(v);
+    if (FUSED == 2 && p.activation == 1) v = gelu_tanh_fast(v);
     if (p.residual) v += resv;
   }
   return v;
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
           if (p.beta != 0.0f) v += p.beta * *c;
           if constexpr (FUSED) {
             if (p.bias) v += p.bias[col];
-            if (FUSED == 2 && p.activation == 1) v = gelu_tanh_f(v);
+            if (FUSED == 2 && p.activation == 1) v = gelu_tanh_fast(v);
             if (p.residual)
               v += p.residual[(int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes + row * p.ldres + col];
           }

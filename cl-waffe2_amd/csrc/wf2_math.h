@@ -32,6 +32,8 @@
 #define WF2_SLOW_POW(x, p) pow((x), (p))
 #define WF2_SLOW_TANF(x) tanf(x)
 #define WF2_SQRTF(x) __builtin_sqrtf(x)
+#define WF2_FAST_EXP2F(x) __builtin_amdgcn_exp2f(x)
+#define WF2_FAST_RCPF(x) __builtin_amdgcn_rcpf(x)
 #else
 #include <math.h>
 #define WF2_MATH_FN static inline
@@ -42,6 +44,8 @@
 #define WF2_SLOW_POW(x, p) pow((x), (p))
 #define WF2_SLOW_TANF(x) ((float)tan((double)(x)))
 #define WF2_SQRTF(x) sqrtf(x)
+#define WF2_FAST_EXP2F(x) exp2f(x)
+#define WF2_FAST_RCPF(x) (1.0f / (x))
 #endif
 
 namespace wf2 {
@@ -371,6 +375,23 @@ WF2_MATH_FN float gelu_tanh_f(float x) {
   // x = -inf: the limit is -0 (x e^{2u} -> 0), not -inf * tiny.
   r = (x == -__builtin_inff()) ? -0.0f : r;
   return (x != x) ? x : r;
+}
+
+// The same function in binary32 for gemm epilogues, whose inputs already carry
+// the rounding of a long binary32 accumulation: x / (1 + 2^t) with
+// t = -2 u log2(e) = x (k1 + k2 x^2), through v_exp_f32 and v_rcp_f32 (12 VALU
+// slots against 35).  Error: three roundings of t (|t| 2e-7 absolute, so
+// |t| 1.3e-7 relative in 2^t), one ulp each from the exponential, the
+// reciprocal and the two products: below 4e-6 relative wherever the result is
+// a normal number, below 1e-6 for |x| < 4.
+WF2_MATH_FN float gelu_tanh_fast(float x) {
+  const float k1 = -2.3022082f;    // -2 sqrt(2/pi) log2(e)
+  const float k2 = -0.10294324f;   // k1 * 0.044715
+  const float t = x * __builtin_fmaf(k2, x * x, k1);
+  const float e = WF2_FAST_EXP2F(t < 126.0f ? t : 126.0f);
+  const float r = x * WF2_FAST_RCPF(1.0f + e);
+  // far on the negative side x e^{2u} underflows; x = -inf would give inf / inf
+  return (t > 100.0f) ? -0.0f : r;
 }
 
 }  // namespace wf2
