@@ -237,6 +237,12 @@ def row_table(W, reps: int = 10, warm: int = 3):
             (8 + 12) * 2048 * Cn, note="two launches: MoveTensorNode 8 B/elem, SubNode 12 B/elem")
     del a0, b0, yb
 
+    # transposing copy through LDS tiles
+    a0 = normal([SIDE, SIDE])
+    ring = ring_of(lambda: (clone(a0), T([SIDE, SIDE], initial_element=None)), 8 * N)
+    measure("transposing copy (8192,8192)", ring, lambda s: F.move_(s[1], s[0].permute(1, 0)), 8 * N)
+    del a0
+
     # unary functions on 2^26 elements in the ranges of the configuration
     for label, fn, lo, hi in (("exp", F.exp, -10.0, 10.0), ("tanh", F.tanh, -10.0, 10.0),
                               ("sin", F.sin, -100.0, 100.0), ("loge", F.loge, 1e-3, 1e3)):

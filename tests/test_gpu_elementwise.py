@@ -176,6 +176,31 @@ def test_inplace_on_every_second_element(gpu):
     assert_bit_equal(t.numpy(), base + y.T, "(n, 2) seen as (2, n)")
 
 
+def test_large_transposed_operands(gpu):
+    """Operands whose unit-stride axes differ, large enough for the 128 x 128
+    LDS tiles: copies, an in-place binary op with a transposed second operand
+    and a unary op reading a transposed source, with ragged tile edges and outer
+    (batch) axes.  Closed form: numpy on the same views; bit-exact (exp <= 2 ulp
+    of float64)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(128)
+    for shape, order in [((2052, 2060), (1, 0)), ((3, 1100, 1284), (0, 2, 1)), ((2, 3, 1028, 1032), (0, 1, 3, 2)),
+                         ((1284, 5, 1100), (2, 1, 0))]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        xt = np.transpose(x, order)
+        dx = F.from_numpy(x)
+        got = F.copy(dx.permute(*order))
+        assert got.shape == list(xt.shape)
+        assert_bit_equal(got.numpy(), np.ascontiguousarray(xt), f"copy {shape} -> {order}")
+        y = rng.standard_normal(xt.shape).astype(np.float32)
+        dy = F.from_numpy(y)
+        F.sub_(dy, dx.permute(*order))
+        assert_bit_equal(dy.numpy(), y - xt, f"sub_ {shape} -> {order}")
+        e = F.exp(dx.permute(*order))
+        assert ulp_distance(e.numpy(), np.exp(xt.astype(np.float64)).astype(np.float32)).max() <= 1
+
+
 def _random_view(rng, n):
     """A random subscript for an axis of extent n."""
     k = rng.integers(0, 6)
