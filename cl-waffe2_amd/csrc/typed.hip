@@ -1,0 +1,402 @@
+// typed.hip -- AddNode / SubNode / MulNode / DivNode / MoveTensorNode and inv
+// for the element types of cl-waffe2 other than :float -- :double, :int32,
+// :uint32, :int16, :uint16, :int8, :uint8.
+//
+// Reference: waffe2_d{add,sub,mul,div} (the AVX2 macro of
+// cl-waffe2-simd.c:153-213 instantiated at :247-250), the scalar loops
+// waffe2_{i32,i16,i8,u32,u16,u8}{add,sub,mul,div,copy} (:214-288), dcopy_ from
+// BLAS for :double moves (source/backends/cpu/arithmetic.lisp:39-61) and
+// waffe2_{d,i32,...}inv (:290-310).
+//
+// Integer semantics are C's: int8 / int16 operands are promoted to int and the
+// result is truncated on the store, unsigned types wrap, signed division
+// truncates toward zero.  The reference traps (SIGFPE) on a zero divisor and on
+// INT_MIN / -1; a GPU cannot, so those elements become 0 and INT_MIN.
+//
+// :double has one quirk in the reference that the 1-D entry point reproduces:
+// the scalar remainder of the AVX2 macro goes through `sas_dadd` & co., which
+// are declared to return float (cl-waffe2-simd.c:229-232), so the last n % 4
+// elements of a call -- and every element when incx < 1, which skips the vector
+// body -- are rounded to binary32 and widened again.  The N-D entry point has
+// no notion of "calls" and computes every element in binary64, which is what
+// the reference's vector body does.
+//
+// These are bandwidth kernels like their :float counterparts: 16-byte vectors
+// when both runs are contiguous (or y is one value), one element per lane with
+// four in flight otherwise.  A destination with incx = 0 accumulates in the
+// reference's order on one lane.
+#include "wf2_common.h"
+#include "wf2_view.h"
+
+namespace wf2 {
+
+template <class T>
+struct Wide { using type = T; };
+template <> struct Wide<int8_t> { using type = int; };
+template <> struct Wide<uint8_t> { using type = int; };
+template <> struct Wide<int16_t> { using type = int; };
+template <> struct Wide<uint16_t> { using type = int; };
+
+template <class T>
+constexpr bool kIsInt = !__is_floating_point(T);
+
+template <class T, int OP>
+__device__ __forceinline__ T apply(T a, T b) {
+  using W = typename Wide<T>::type;
+  const W x = (W)a, y = (W)b;
+  if constexpr (OP == WF2HIP_ADD) {
+    if constexpr (kIsInt<T> && sizeof(W) == 4 && (W)(-1) < (W)0)  // signed: wrap, as x86 does
+      return (T)(int32_t)((uint32_t)x + (uint32_t)y);
+    else
+      return (T)(x + y);
+  } else if constexpr (OP == WF2HIP_SUB) {
+    if constexpr (kIsInt<T> && sizeof(W) == 4 && (W)(-1) < (W)0)
+      return (T)(int32_t)((uint32_t)x - (uint32_t)y);
+    else
+      return (T)(x - y);
+  } else if constexpr (OP == WF2HIP_MUL) {
+    if constexpr (kIsInt<T> && sizeof(W) == 4 && (W)(-1) < (W)0)
+      return (T)(int32_t)((uint32_t)x * (uint32_t)y);
+    else
+      return (T)(x * y);
+  } else if constexpr (OP == WF2HIP_DIV) {
+    if constexpr (kIsInt<T>) {
+      if (y == 0) return (T)0;
+      if constexpr ((W)(-1) < (W)0) {
+        if (sizeof(T) == 4 && x == (W)INT32_MIN && y == (W)-1) return (T)x;
+      }
+      return (T)(x / y);
+    } else {
+      return (T)(x / y);
+    }
+  } else {
+    return b;  // MOVE
+  }
+}
+
+// the reference's scalar remainder for :double: through binary32
+template <class T>
+__device__ __forceinline__ T through_float(T v) {
+  if constexpr (__is_same(T, double)) return (double)(float)v;
+  return v;
+}
+
+template <class T, int N>
+struct alignas(16) Pack { T v[N]; };
+
+// contiguous x, y contiguous (or one value): 16 bytes per lane and access
+template <class T, int OP, bool BCAST>
+__global__ __launch_bounds__(kBlock) void typed_flat(T* __restrict__ x, const T* __restrict__ y, size_t nvec) {
+  constexpr int N = 16 / sizeof(T);
+  using P = Pack<T, N>;
+  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= nvec) return;
+  P a, b;
+  if (OP != WF2HIP_MOVE) a = reinterpret_cast<const P*>(x)[i];
+  if (BCAST) {
+    const T s = y[0];
+#pragma unroll
+    for (int k = 0; k < N; k++) b.v[k] = s;
+  } else {
+    b = reinterpret_cast<const P*>(y)[i];
+  }
+  P r;
+#pragma unroll
+  for (int k = 0; k < N; k++) r.v[k] = apply<T, OP>(OP != WF2HIP_MOVE ? a.v[k] : b.v[k], b.v[k]);
+  reinterpret_cast<P*>(x)[i] = r;
+}
+
+// any increments (incx != 0): elements first..n-1; those from `exact_end` on go
+// through binary32 when T is double (the reference's remainder loop)
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void typed_strided(T* x, int64_t incx, const T* y, int64_t incy, int64_t first,
+                                                        int64_t n, int64_t exact_end) {
+  constexpr int U = 4;
+  const int64_t step = (int64_t)gridDim.x * kBlock * U;
+  for (int64_t base = first + (int64_t)blockIdx.x * kBlock * U + threadIdx.x; base < n; base += step) {
+    T a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t i = base + (int64_t)u * kBlock;
+      if (i < n) {
+        a[u] = OP != WF2HIP_MOVE ? x[i * incx] : T(0);
+        b[u] = y[i * incy];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t i = base + (int64_t)u * kBlock;
+      if (i < n) {
+        T r = apply<T, OP>(a[u], b[u]);
+        if (OP != WF2HIP_MOVE && i >= exact_end) r = through_float(r);
+        x[i * incx] = r;
+      }
+    }
+  }
+}
+
+// incx == 0: x[0] <- x[0] op y[i], i = 0..n-1, in that order (one lane)
+template <class T, int OP>
+__global__ void typed_sequential(T* x, const T* y, int64_t incy, int64_t n) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  T acc = x[0];
+  for (int64_t i = 0; i < n; i++) {
+    acc = apply<T, OP>(acc, y[i * incy]);
+    if (OP != WF2HIP_MOVE) acc = through_float(acc);
+  }
+  x[0] = acc;
+}
+
+struct TypedGen {
+  int32_t rank;
+  int64_t total;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t sd[WF2HIP_MAX_RANK];
+  int64_t ss[WF2HIP_MAX_RANK];
+};
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void typed_generic(T* dst, const T* src, TypedGen p) {
+  constexpr int U = 4;
+  const int64_t step = (int64_t)gridDim.x * kBlock * U;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * U + threadIdx.x; base < p.total; base += step) {
+    int64_t doff[U], soff[U];
+    T a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      int64_t rem = base + (int64_t)u * kBlock;
+      if (rem >= p.total) rem = p.total - 1;
+      int64_t d = 0, q = 0;
+      for (int r = p.rank - 1; r > 0; r--) {
+        const int64_t quot = rem / p.shape[r];
+        const int64_t idx = rem - quot * p.shape[r];
+        rem = quot;
+        d += idx * p.sd[r];
+        q += idx * p.ss[r];
+      }
+      doff[u] = d + rem * p.sd[0];
+      soff[u] = q + rem * p.ss[0];
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const bool live = base + (int64_t)u * kBlock < p.total;
+      a[u] = (OP != WF2HIP_MOVE && live) ? dst[doff[u]] : T(0);
+      b[u] = live ? src[soff[u]] : T(0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (base + (int64_t)u * kBlock < p.total) dst[doff[u]] = apply<T, OP>(a[u], b[u]);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_inv(T* x, int64_t incx, int64_t n) {
+  if (incx == 0) {  // the reference's loop inverts the one element n times
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    T v = x[0];
+    for (int64_t i = 0; i < n; i++) v = apply<T, WF2HIP_DIV>(T(1), v);
+    x[0] = v;
+    return;
+  }
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step)
+    x[i * incx] = apply<T, WF2HIP_DIV>(T(1), x[i * incx]);
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+static uint32_t grid_for(int64_t n, int per_thread) {
+  int64_t want = ceil_div(n, (int64_t)kBlock * per_thread);
+  int64_t cap = (int64_t)rt().num_cus * 64;
+  if (want < 1) want = 1;
+  return (uint32_t)(want < cap ? want : cap);
+}
+
+// `quirk`: reproduce the binary32 rounding of the reference's remainder loop (:double only)
+template <class T, int OP>
+static int run_1d(int64_t n, T* x, int64_t incx, const T* y, int64_t incy, bool quirk) {
+  hipStream_t st = rt().stream;
+  if (incx == 0) {
+    if (OP == WF2HIP_MOVE) {  // the last write wins
+      typed_strided<T, OP><<<1, kBlock, 0, st>>>(x, 0, y + (n - 1) * incy, 0, 0, 1, 1);
+      return after_launch("typed_strided");
+    }
+    if (!quirk && __is_same(T, double))
+      return fail(WF2HIP_EUNSUPPORTED, "reductions of :double tensors go through the 1-D entry point");
+    typed_sequential<T, OP><<<1, kWave, 0, st>>>(x, y, incy, n);
+    return after_launch("typed_sequential");
+  }
+  constexpr int N = 16 / (int)sizeof(T);
+  // the reference's vector body covers (n / 4) * 4 elements when incx >= 1
+  const int64_t exact_end = (!quirk || !__is_same(T, double) || OP == WF2HIP_MOVE) ? n : (incx >= 1 ? (n / 4) * 4 : 0);
+  int64_t done = 0;
+  if (incx == 1 && (incy == 1 || incy == 0) && aligned16(x) && (incy == 0 || aligned16(y))) {
+    const int64_t nvec = (exact_end < n ? exact_end : n) / N;
+    if (nvec > 0) {
+      const int64_t blocks = ceil_div(nvec, kBlock);
+      if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "run too long for one launch");
+      if (incy == 0)
+        typed_flat<T, OP, true><<<(uint32_t)blocks, kBlock, 0, st>>>(x, y, (size_t)nvec);
+      else
+        typed_flat<T, OP, false><<<(uint32_t)blocks, kBlock, 0, st>>>(x, y, (size_t)nvec);
+      WF2_TRY(after_launch("typed_flat"));
+      done = nvec * N;
+    }
+  }
+  if (done < n) {
+    typed_strided<T, OP><<<grid_for(n - done, 4), kBlock, 0, st>>>(x, incx, y, incy, done, n, exact_end);
+    return after_launch("typed_strided");
+  }
+  return 0;
+}
+
+template <class T>
+static int dispatch_1d(int op, int64_t n, T* x, int64_t incx, const T* y, int64_t incy, bool quirk) {
+  switch (op) {
+    case WF2HIP_ADD: return run_1d<T, WF2HIP_ADD>(n, x, incx, y, incy, quirk);
+    case WF2HIP_SUB: return run_1d<T, WF2HIP_SUB>(n, x, incx, y, incy, quirk);
+    case WF2HIP_MUL: return run_1d<T, WF2HIP_MUL>(n, x, incx, y, incy, quirk);
+    case WF2HIP_DIV: return run_1d<T, WF2HIP_DIV>(n, x, incx, y, incy, quirk);
+    case WF2HIP_MOVE: return run_1d<T, WF2HIP_MOVE>(n, x, incx, y, incy, quirk);
+    default: return fail(WF2HIP_EINVAL, "unknown binary op %d", op);
+  }
+}
+
+template <class T, int OP>
+static int run_generic(const Space& s, T* a, const T* b) {
+  TypedGen p;
+  p.rank = s.rank;
+  p.total = s.total;
+  for (int r = 0; r < s.rank; r++) {
+    p.shape[r] = s.shape[r];
+    p.sd[r] = s.sa[r];
+    p.ss[r] = s.sb[r];
+  }
+  typed_generic<T, OP><<<grid_for(s.total, 4), kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
+  return after_launch("typed_generic");
+}
+
+// the :float path's test, in elements of `size` bytes
+static bool typed_overlap(const Space& s, const void* a, const void* b, size_t size) {
+  const int64_t bytes = (const char*)b - (const char*)a;
+  if (bytes % (int64_t)size == 0) return hazardous_overlap_at(s, bytes / (int64_t)size);
+  // bases that are not a whole number of elements apart: plain interval test
+  int64_t alo, ahi, blo, bhi;
+  extent_of(s, s.sa, s.off_a, &alo, &ahi);
+  extent_of(s, s.sb, s.off_b, &blo, &bhi);
+  const char* a0 = (const char*)a + alo * (int64_t)size;
+  const char* a1 = (const char*)a + (ahi + 1) * (int64_t)size;
+  const char* b0 = (const char*)b + blo * (int64_t)size;
+  const char* b1 = (const char*)b + (bhi + 1) * (int64_t)size;
+  return !(a1 <= b0 || b1 <= a0);
+}
+
+template <class T>
+static int dispatch_nd(int op, Space s, T* a, const T* b) {
+  if (s.total == 0) return 0;
+  if (!a || !b) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  normalise(&s);
+  if (typed_overlap(s, a, b, sizeof(T)))
+    return fail(WF2HIP_EOVERLAP,
+                "in-place op on partially overlapping windows of one buffer; copy one operand first");
+  if (has_broadcast_axis(s, s.sa)) {
+    if (op != WF2HIP_MOVE)
+      return fail(WF2HIP_EUNSUPPORTED,
+                  "accumulation into a broadcast destination is only built for :float; use the 1-D entry "
+                  "point with incx = 0 per output element");
+    for (int r = 0; r < s.rank; r++)  // the last write wins
+      if (s.sa[r] == 0 && s.shape[r] > 1) {
+        s.off_b += s.sb[r] * (s.shape[r] - 1);
+        s.shape[r] = 1;
+      }
+    s.total = 1;
+    for (int r = 0; r < s.rank; r++) s.total *= s.shape[r];
+    normalise(&s);
+  }
+  if (s.rank == 1 && s.sa[0] != 0)
+    return dispatch_1d<T>(op, s.total, a + s.off_a, s.sa[0], b + s.off_b, s.sb[0], false);
+  switch (op) {
+    case WF2HIP_ADD: return run_generic<T, WF2HIP_ADD>(s, a, b);
+    case WF2HIP_SUB: return run_generic<T, WF2HIP_SUB>(s, a, b);
+    case WF2HIP_MUL: return run_generic<T, WF2HIP_MUL>(s, a, b);
+    case WF2HIP_DIV: return run_generic<T, WF2HIP_DIV>(s, a, b);
+    case WF2HIP_MOVE: return run_generic<T, WF2HIP_MOVE>(s, a, b);
+    default: return fail(WF2HIP_EINVAL, "unknown binary op %d", op);
+  }
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+#define WF2_FOR_DTYPE(dtype, ...)                                                     \
+  switch (dtype) {                                                                      \
+    case WF2HIP_F64: { using T = double; __VA_ARGS__; }                                        \
+    case WF2HIP_I32: { using T = int32_t; __VA_ARGS__; }                                       \
+    case WF2HIP_U32: { using T = uint32_t; __VA_ARGS__; }                                      \
+    case WF2HIP_I16: { using T = int16_t; __VA_ARGS__; }                                       \
+    case WF2HIP_U16: { using T = uint16_t; __VA_ARGS__; }                                      \
+    case WF2HIP_I8: { using T = int8_t; __VA_ARGS__; }                                         \
+    case WF2HIP_U8: { using T = uint8_t; __VA_ARGS__; }                                        \
+    default: return fail(WF2HIP_EINVAL, "unknown element type %d (:float has its own entry points)", dtype); \
+  }
+
+WF2_API int wf2hip_binary_1d_typed(int dtype, int op, long n, void* x, long incx, const void* y, long incy) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative length");
+  if (n == 0) return 0;
+  if (!x || !y) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  WF2_FOR_DTYPE(dtype, return dispatch_1d<T>(op, n, (T*)x, incx, (const T*)y, incy, true));
+}
+
+WF2_API int wf2hip_binary_nd_typed(int dtype, int op, const wf2hip_view2* v, void* a, const void* b) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  WF2_FOR_DTYPE(dtype, return dispatch_nd<T>(op, s, (T*)a, (const T*)b));
+}
+
+WF2_API int wf2hip_inv_1d_typed(int dtype, long n, void* x, long incx) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative length");
+  if (n == 0) return 0;
+  if (!x) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  WF2_FOR_DTYPE(dtype, {
+    typed_inv<T><<<incx == 0 ? 1u : grid_for(n, 1), kBlock, 0, rt().stream>>>((T*)x, incx, n);
+    return after_launch("typed_inv");
+  });
+}
+
+// The reference's own names, one per element type: waffe2_dadd -> wf2hip_dadd, ...
+#define WF2_TYPED_ARITH(prefix, T, code)                                                               \
+  WF2_API int wf2hip_##prefix##add(long n, T* x, long incx, const T* y, long incy) {                   \
+    return wf2hip_binary_1d_typed(code, WF2HIP_ADD, n, x, incx, y, incy);                              \
+  }                                                                                                    \
+  WF2_API int wf2hip_##prefix##sub(long n, T* x, long incx, const T* y, long incy) {                   \
+    return wf2hip_binary_1d_typed(code, WF2HIP_SUB, n, x, incx, y, incy);                              \
+  }                                                                                                    \
+  WF2_API int wf2hip_##prefix##mul(long n, T* x, long incx, const T* y, long incy) {                   \
+    return wf2hip_binary_1d_typed(code, WF2HIP_MUL, n, x, incx, y, incy);                              \
+  }                                                                                                    \
+  WF2_API int wf2hip_##prefix##div(long n, T* x, long incx, const T* y, long incy) {                   \
+    return wf2hip_binary_1d_typed(code, WF2HIP_DIV, n, x, incx, y, incy);                              \
+  }                                                                                                    \
+  WF2_API int wf2hip_##prefix##inv(long n, T* x, long incx) { return wf2hip_inv_1d_typed(code, n, x, incx); }
+
+#define WF2_TYPED_FAMILY(prefix, T, code)                                                              \
+  WF2_TYPED_ARITH(prefix, T, code)                                                                     \
+  WF2_API int wf2hip_##prefix##copy(long n, T* x, long incx, const T* y, long incy) {                  \
+    return wf2hip_binary_1d_typed(code, WF2HIP_MOVE, n, x, incx, y, incy);                             \
+  }
+
+WF2_TYPED_ARITH(d, double, WF2HIP_F64)
+// :double moves are dcopy_ in the reference (source/backends/cpu/arithmetic.lisp:39-61): BLAS argument order
+WF2_API int wf2hip_dcopy(long n, const double* src, long incsrc, double* dst, long incdst) {
+  return wf2hip_binary_1d_typed(WF2HIP_F64, WF2HIP_MOVE, n, dst, incdst, src, incsrc);
+}
+WF2_TYPED_FAMILY(i32, int32_t, WF2HIP_I32)
+WF2_TYPED_FAMILY(u32, uint32_t, WF2HIP_U32)
+WF2_TYPED_FAMILY(i16, int16_t, WF2HIP_I16)
+WF2_TYPED_FAMILY(u16, uint16_t, WF2HIP_U16)
+WF2_TYPED_FAMILY(i8, int8_t, WF2HIP_I8)
+WF2_TYPED_FAMILY(u8, uint8_t, WF2HIP_U8)

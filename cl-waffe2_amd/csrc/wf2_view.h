@@ -94,16 +94,13 @@ inline void extent_of(const Space& s, const int64_t* stride, int64_t off, int64_
 }
 
 // True when the two windows may touch a common element without being the
-// same element-for-element mapping.
-inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {
+// same element-for-element mapping.  `delta` = (base of b - base of a) in
+// elements; the windows start at off_a and delta + off_b.
+inline bool hazardous_overlap_at(const Space& s, int64_t delta) {
   int64_t alo, ahi, blo, bhi;
   extent_of(s, s.sa, s.off_a, &alo, &ahi);
-  extent_of(s, s.sb, s.off_b, &blo, &bhi);
-  const float* a0 = a + alo;
-  const float* a1 = a + ahi;
-  const float* b0 = b + blo;
-  const float* b1 = b + bhi;
-  if (a1 < b0 || b1 < a0) return false;
+  extent_of(s, s.sb, s.off_b + delta, &blo, &bhi);
+  if (ahi < blo || bhi < alo) return false;
   // Interleaved lattices (the even against the odd elements of one buffer): every
   // address of a window is its start plus a multiple of g = gcd of all strides of
   // both windows, so starts that differ modulo g never meet.
@@ -119,11 +116,16 @@ inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {
       }
     }
   }
-  if (g > 1 && ((a + s.off_a) - (b + s.off_b)) % g != 0) return false;
-  if (a + s.off_a != b + s.off_b) return true;
+  const int64_t starts = s.off_a - (s.off_b + delta);
+  if (g > 1 && starts % g != 0) return false;
+  if (starts != 0) return true;
   for (int r = 0; r < s.rank; r++)
     if (s.sa[r] != s.sb[r]) return true;
   return false;  // identical mapping: every element depends on itself only
+}
+
+inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {
+  return hazardous_overlap_at(s, b - a);
 }
 
 inline bool has_broadcast_axis(const Space& s, const int64_t* stride) {

@@ -28,13 +28,13 @@ Number = (int, float, np.integer, np.floating)
 # construction / movement
 # ---------------------------------------------------------------------------
 
-def make_tensor(shape: Sequence[int], initial_element: float = 0.0) -> HIPTensor:
-    """``(make-tensor shape :initial-element x)``"""
-    return HIPTensor(shape, initial_element=initial_element)
+def make_tensor(shape: Sequence[int], initial_element: float = 0.0, dtype: str = "float") -> HIPTensor:
+    """``(make-tensor shape :initial-element x :dtype dtype)``"""
+    return HIPTensor(shape, initial_element=initial_element, dtype=dtype)
 
 
-def from_numpy(a) -> HIPTensor:
-    return HIPTensor.from_numpy(a)
+def from_numpy(a, dtype: str = "float") -> HIPTensor:
+    return HIPTensor.from_numpy(a, dtype=dtype)
 
 
 def move_(dst: HIPTensor, src: HIPTensor) -> HIPTensor:
@@ -46,7 +46,7 @@ def move_(dst: HIPTensor, src: HIPTensor) -> HIPTensor:
 def copy(x: HIPTensor) -> HIPTensor:
     """``(!copy x)``: a fresh contiguous tensor of x's visible shape filled by
     MoveTensorNode (``fundamental.lisp:122-163``)."""
-    return move_(HIPTensor(x.shape, initial_element=None), x)
+    return move_(HIPTensor(x.shape, initial_element=None, dtype=x.dtype), x)
 
 
 def to_contiguous(x: HIPTensor) -> HIPTensor:
@@ -104,7 +104,8 @@ def scalar_tensor(value: float, like: HIPTensor) -> HIPTensor:
     """A ``(1 ... 1)`` tensor viewed ``(:broadcast n)`` on every axis, which is
     how ``!scalar-add`` & co. feed a scalar to a tensor node
     (``base-impl/arithmetic.lisp:31-51,216-262``)."""
-    s = HIPTensor([1] * like.ndim, initial_element=float(value))
+    s = HIPTensor([1] * like.ndim, initial_element=value if like.dtype != "float" else float(value),
+                  dtype=like.dtype)
     return s.view(*[(":broadcast", n) if n != 1 else True for n in like.shape])
 
 
@@ -120,7 +121,7 @@ def flexible(y: HIPTensor, like: HIPTensor) -> HIPTensor:
     if len(ys) < len(ls):
         if not y.is_contiguous():
             y = copy(y)
-        y = HIPTensor([1] * (len(ls) - len(ys)) + ys, vec=y.vec)
+        y = HIPTensor([1] * (len(ls) - len(ys)) + ys, vec=y.vec, dtype=y.dtype)
         ys = y.shape
     subs = []
     for a, b in zip(ys, ls):
@@ -143,7 +144,7 @@ def flexible(y: HIPTensor, like: HIPTensor) -> HIPTensor:
 
 def _operand(y, like: HIPTensor) -> HIPTensor:
     if isinstance(y, Number):
-        return scalar_tensor(float(y), like)
+        return scalar_tensor(y, like)
     return flexible(y, like)
 
 
@@ -182,14 +183,14 @@ def _out_of_place(node: str, x, y) -> HIPTensor:
             return add_(mul_(copy(y), -1.0), x)
         return mul_(reciprocal(y), x)
     if isinstance(y, Number):
-        return nodes.forward(node, copy(x), scalar_tensor(float(y), x))
+        return nodes.forward(node, copy(x), scalar_tensor(y, x))
     if x.shape == y.shape:
         return nodes.forward(node, copy(x), y)
     out_shape = list(np.broadcast_shapes(tuple(x.shape), tuple(y.shape)))
     if x.shape == out_shape:
         left = copy(x)
     else:  # x is the smaller operand: expand it into a full-size tensor first
-        left = move_(HIPTensor(out_shape, initial_element=None), flexible(x, _ShapeOnly(out_shape)))
+        left = move_(HIPTensor(out_shape, initial_element=None, dtype=x.dtype), flexible(x, _ShapeOnly(out_shape)))
     return nodes.forward(node, left, flexible(y, left))
 
 

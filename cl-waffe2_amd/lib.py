@@ -18,6 +18,8 @@ MAX_RANK = 8
 
 # enum wf2hip_binary_op / wf2hip_unary_op
 ADD, SUB, MUL, DIV, MOVE = 0, 1, 2, 3, 4
+# enum wf2hip_dtype: the element types served by the *_typed entry points
+DTYPE_CODES = {"double": 1, "int32": 2, "uint32": 3, "int16": 4, "uint16": 5, "int8": 6, "uint8": 7}
 SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
 TAN, ASIN, ACOS, ATAN, SINH, COSH, LOG2, LOG10, LOG1P = 23, 24, 25, 26, 27, 28, 29, 30, 31
 POW, GELU = 32, 40
@@ -137,6 +139,10 @@ _SIGNATURES = {
     "wf2hip_ssqrt": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sabs": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sinv": ([_L, _P, _L], C.c_int),
+    "wf2hip_binary_1d_typed": ([C.c_int, C.c_int, _L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_binary_nd_typed": ([C.c_int, C.c_int, C.POINTER(View2), _P, _P], C.c_int),
+    "wf2hip_inv_1d_typed": ([C.c_int, _L, _P, _L], C.c_int),
+    "wf2hip_dcopy": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_stan": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sasin": ([_L, _P, _L, _P, _L], C.c_int),
     "wf2hip_sacos": ([_L, _P, _L, _P, _L], C.c_int),
@@ -180,6 +186,12 @@ _SIGNATURES = {
         C.c_int,
     ),
 }
+
+# the reference's own per-dtype names (waffe2_dadd -> wf2hip_dadd, ...): pointers are void* here
+for _prefix in ("d", "i32", "u32", "i16", "u16", "i8", "u8"):
+    for _op in ("add", "sub", "mul", "div") + (() if _prefix == "d" else ("copy",)):
+        _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P, _L], C.c_int)
+    _SIGNATURES[f"wf2hip_{_prefix}inv"] = ([_L, _P, _L], C.c_int)
 
 EXPORTS = tuple(_SIGNATURES)
 

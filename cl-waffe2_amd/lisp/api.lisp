@@ -75,6 +75,13 @@
   (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
   (then-value :float) (else-value :float))
 (defcfun "wf2hip_sinv" :int (n :long) (x :pointer) (incx :long))
+;; :double and the integer dtypes (waffe2_d*, waffe2_{i32,...}*, cl-waffe2-simd/api.lisp:63-124):
+;; one entry point per shape of call, the element type as a code (dtype-info in tensor.lisp)
+(defcfun "wf2hip_binary_1d_typed" :int
+  (dtype :int) (op :int) (n :long) (x :pointer) (incx :long) (y :pointer) (incy :long))
+(defcfun "wf2hip_binary_nd_typed" :int
+  (dtype :int) (op :int) (view (:pointer (:struct view2))) (a :pointer) (b :pointer))
+(defcfun "wf2hip_inv_1d_typed" :int (dtype :int) (n :long) (x :pointer) (incx :long))
 (defcfun "wf2hip_select_nd" :int
   (op :int) (outer (:pointer (:struct view2))) (n :long) (incx :long) (x :pointer) (out :pointer))
 (defconstant +maxvalue+ 48) (defconstant +minvalue+ 49) (defconstant +argmax+ 50) (defconstant +argmin+ 51)

@@ -42,10 +42,18 @@ These are exactly the numbers call-with-view computes per axis
     view))
 
 (defun run-binary (op x y)
+  "X <- X op Y over both views in one call; :float through the kernels of the hot path, any
+other dtype through the typed entry point (the CPU backend dispatches on dtype inside its impl
+too, source/backends/cpu/arithmetic.lisp:65-123)."
   (ensure-extension)
+  (unless (eql (dtype x) (dtype y))
+    (error "HIPTensor: ~a and ~a operands in one node" (dtype x) (dtype y)))
   (with-foreign-object (view '(:struct view2))
     (fill-view2 view x y)
-    (check (wf2hip-binary-nd op view (tensor-device-pointer x) (tensor-device-pointer y))))
+    (if (eql (dtype x) :float)
+        (check (wf2hip-binary-nd op view (tensor-device-pointer x) (tensor-device-pointer y)))
+        (check (wf2hip-binary-nd-typed (nth-value 2 (dtype-info (dtype x))) op view
+                                       (tensor-device-pointer x) (tensor-device-pointer y)))))
   x)
 
 (defun run-unary (op x out &optional (p 0.0))
@@ -60,7 +68,7 @@ These are exactly the numbers call-with-view computes per axis
 ;; A stride-0 destination axis -- how !sum and !mean arrive (base-impl/reduction.lisp:5-79) --
 ;; is reduced in parallel by the library.
 (macrolet ((define-arith (node op)
-             `(define-impl-op (,node :device HIPTensor :reject-p #'only-float-p)
+             `(define-impl-op (,node :device HIPTensor)
                               :forward ((self x y) (declare (ignore self)) (run-binary ,op x y)))))
   (define-arith AddNode +add+)
   (define-arith SubNode +sub+)
@@ -69,7 +77,7 @@ These are exactly the numbers call-with-view computes per axis
 
 ;; X <- Y (source/base-impl/fundamental.lisp:9-43).  Without this impl every !copy on a device
 ;; tensor would fall through to CPUTensor's scopy on a device handle.
-(define-impl-op (MoveTensorNode :device HIPTensor :reject-p #'only-float-p)
+(define-impl-op (MoveTensorNode :device HIPTensor)
                 :forward ((self x y)
                           (if (cl-waffe2/base-impl::movetensor-ignore-me self)
                               y

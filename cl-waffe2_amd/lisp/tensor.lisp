@@ -10,9 +10,25 @@
   (pointer (null-pointer) :type foreign-pointer)
   (bytes 0 :type fixnum))
 
-(defun make-device-buffer (n-elements &key (zero t))
+(defun dtype-info (dtype)
+  "(values CFFI-type bytes-per-element wf2hip_dtype-code) of a cl-waffe2 dtype keyword.  Every
+node of the path runs on :float; the other dtypes have the arithmetic / move nodes (and :uint32
+receives ArgMax-Node / ArgMin-Node results)."
+  (ecase dtype
+    (:float (values :float 4 0))
+    (:double (values :double 8 1))
+    (:int32 (values :int32 4 2))
+    (:uint32 (values :uint32 4 3))
+    (:int16 (values :int16 2 4))
+    (:uint16 (values :uint16 2 5))
+    (:int8 (values :int8 1 6))
+    (:uint8 (values :uint8 1 7))))
+
+(defun dtype-bytes (dtype) (nth-value 1 (dtype-info dtype)))
+
+(defun make-device-buffer (n-elements &key (zero t) (dtype :float))
   (ensure-extension)
-  (let ((bytes (* 4 n-elements)))
+  (let ((bytes (* (dtype-bytes dtype) n-elements)))
     (with-foreign-object (slot :pointer)
       (check (if zero
                  (wf2hip-malloc slot bytes)
@@ -44,32 +60,42 @@ fp32 tensors resident in the HBM of an AMD MI355X; kernels come from libwaffe2-h
         (vec (getf initargs :vec))
         (facet (getf initargs :facet))
         (initial-element (getf initargs :initial-element)))
-    (unless (member (or (getf initargs :dtype) :float) '(:float))
-      (error "HIPTensor supports :float only, got ~a" (getf initargs :dtype)))
+    (dtype-info (or (getf initargs :dtype) :float)) ; signals on an unknown dtype
     (when (eql facet :exist)
       (if vec
           (setf (tensor-vec tensor) vec)
-          (let* ((n (apply #'* shape))
-                 (buffer (make-device-buffer n :zero t)))
+          (let* ((dtype (or (getf initargs :dtype) :float))
+                 (n (apply #'* shape))
+                 (buffer (make-device-buffer n :zero t :dtype dtype)))
             (when (and initial-element (not (zerop initial-element)))
-              (check (wf2hip-fill-f32 (device-buffer-pointer buffer) n (coerce initial-element 'single-float))))
+              (if (eql dtype :float)
+                  (check (wf2hip-fill-f32 (device-buffer-pointer buffer) n (coerce initial-element 'single-float)))
+                  ;; the other dtypes: one element across PCIe, then a stride-0 move spreads it
+                  (multiple-value-bind (ctype bytes code) (dtype-info dtype)
+                    (with-foreign-object (host ctype)
+                      (setf (mem-ref host ctype) (coerce initial-element (dtype->lisp-type dtype)))
+                      (check (wf2hip-memcpy-h2d (device-buffer-pointer buffer) host bytes)))
+                    (check (wf2hip-binary-1d-typed code +move+ n (device-buffer-pointer buffer) 1
+                                                   (device-buffer-pointer buffer) 0)))))
             (setf (tensor-vec tensor) buffer))))))
 
 (defun tensor-device-pointer (tensor &optional (offset 0))
   "Device address of element OFFSET of TENSOR's storage (the analogue of incf-tensor-ptr,
 source/backends/cpu/tensor.lisp:32-40)."
-  (inc-pointer (device-buffer-pointer (tensor-vec tensor)) (* 4 offset)))
+  (inc-pointer (device-buffer-pointer (tensor-vec tensor)) (* (dtype-bytes (dtype tensor)) offset)))
 
 ;; One element across PCIe.  Used by Mat->ScalarNode, tests and printing; never in a loop.
 (defmethod vref ((tensor HIPTensor) index)
-  (with-foreign-object (host :float)
-    (check (wf2hip-memcpy-d2h host (tensor-device-pointer tensor index) 4))
-    (mem-ref host :float)))
+  (multiple-value-bind (ctype bytes) (dtype-info (dtype tensor))
+    (with-foreign-object (host ctype)
+      (check (wf2hip-memcpy-d2h host (tensor-device-pointer tensor index) bytes))
+      (mem-ref host ctype))))
 
 (defmethod (setf vref) (new-value (tensor HIPTensor) index)
-  (with-foreign-object (host :float)
-    (setf (mem-ref host :float) (coerce new-value 'single-float))
-    (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor index) host 4)))
+  (multiple-value-bind (ctype bytes) (dtype-info (dtype tensor))
+    (with-foreign-object (host ctype)
+      (setf (mem-ref host ctype) (coerce new-value (dtype->lisp-type (dtype tensor))))
+      (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor index) host bytes))))
   new-value)
 
 (defmethod tensor-finalizer ((tensor HIPTensor))

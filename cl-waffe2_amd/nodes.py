@@ -129,9 +129,28 @@ def _unary(op):
     return impl
 
 
+def _binary_any_dtype(op):
+    """The arithmetic and move nodes take every dtype (``backends/cpu/
+    arithmetic.lisp:65-144`` dispatches on dtype inside the impl): :float goes to
+    the kernels of the hot path, the rest to the typed entry point."""
+    float_impl = _binary(op)
+
+    def impl(x: HIPTensor, y: HIPTensor) -> HIPTensor:
+        if x.dtype != y.dtype:
+            raise ValueError(f"dtype mismatch: {x.dtype} and {y.dtype}")
+        if x.dtype == "float":
+            return float_impl(x, y)
+        v = view2(x, y)
+        _lib.check(_lib.get().wf2hip_binary_nd_typed(_lib.DTYPE_CODES[x.dtype], op, C.byref(v),
+                                                    C.c_void_p(x.ptr), C.c_void_p(y.ptr)))
+        return x
+
+    return impl
+
+
 for _name, _op in (("AddNode", _lib.ADD), ("SubNode", _lib.SUB), ("MulNode", _lib.MUL),
                    ("DivNode", _lib.DIV), ("MoveTensorNode", _lib.MOVE)):
-    define_impl(_name, HIPTensor, _only_float)(_binary(_op))
+    define_impl(_name, HIPTensor)(_binary_any_dtype(_op))
 
 for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _lib.TANH),
                    ("LogENode", _lib.LOG), ("ExpNode", _lib.EXP), ("SqrtNode", _lib.SQRT),

@@ -125,17 +125,24 @@ def column_major_strides(shape: Sequence[int]) -> list[int]:
     return strides[::-1]
 
 
+# cl-waffe2's dtype keyword -> numpy type of the host copy
+# (``dtype->lisp-type``, ``source/vm/generic-tensor/dtype.lisp``)
+DTYPES = {"float": np.float32, "double": np.float64, "int32": np.int32, "uint32": np.uint32,
+          "int16": np.int16, "uint16": np.uint16, "int8": np.int8, "uint8": np.uint8}
+
+
 class HIPTensor:
-    """An fp32 tensor on the GPU, possibly a view of another one's storage."""
+    """A tensor on the GPU, possibly a view of another one's storage.  Every node
+    of the path runs on :float; the other dtypes have the arithmetic / move
+    nodes only (and :uint32 receives ArgMax-Node / ArgMin-Node results)."""
 
     def __init__(self, shape: Sequence[int], *, vec: DeviceBuffer | None = None,
                  strides: Sequence[int] | None = None, views: Sequence[Subscript] | None = None,
                  offset: int = 0, initial_element: float | None = 0.0, dtype: str = "float"):
-        # "uint32" exists only to hold the indices ArgMax-Node / ArgMin-Node write
-        # (matrix-ops.lisp:238-307); every arithmetic node rejects it
-        if dtype not in ("float", "uint32"):
-            raise ValueError(f"HIPTensor holds :float (and :uint32 indices), not {dtype}")
+        if dtype not in DTYPES:
+            raise ValueError(f"HIPTensor has no dtype {dtype}; known: {sorted(DTYPES)}")
         self.dtype = dtype
+        self.itemsize = np.dtype(DTYPES[dtype]).itemsize
         self.orig_shape = [int(s) for s in shape]
         if len(self.orig_shape) < 1 or len(self.orig_shape) > _lib.MAX_RANK:
             raise ValueError(f"HIPTensor rank must be 1..{_lib.MAX_RANK}")
@@ -149,9 +156,14 @@ class HIPTensor:
             n = int(np.prod(self.orig_shape, dtype=np.int64))
             # initial_element None = an InputTensor temporary (make-input): its
             # first use overwrites it, so it is not zero-filled
-            vec = DeviceBuffer(4 * n, zero=initial_element == 0.0)
+            vec = DeviceBuffer(self.itemsize * n, zero=initial_element is not None and initial_element == 0)
             if initial_element and n:
-                _lib.check(_lib.get().wf2hip_fill_f32(C.c_void_p(vec.ptr), n, float(initial_element)))
+                if dtype == "float":
+                    _lib.check(_lib.get().wf2hip_fill_f32(C.c_void_p(vec.ptr), n, float(initial_element)))
+                else:
+                    host = np.full(n, initial_element, DTYPES[dtype])
+                    _lib.check(_lib.get().wf2hip_memcpy_h2d(C.c_void_p(vec.ptr), host.ctypes.data_as(C.c_void_p),
+                                                           host.nbytes))
         self.vec = vec
 
     # -- geometry -----------------------------------------------------------
@@ -188,7 +200,7 @@ class HIPTensor:
     def is_contiguous(self) -> bool:
         shape, strides, off = self.geometry()
         return off == 0 and strides == column_major_strides(shape) and \
-            int(np.prod(shape, dtype=np.int64)) * 4 == self.vec.nbytes
+            int(np.prod(shape, dtype=np.int64)) * self.itemsize == self.vec.nbytes
 
     @property
     def ptr(self) -> int:
@@ -196,19 +208,20 @@ class HIPTensor:
 
     # -- construction ---------------------------------------------------------
     @classmethod
-    def from_numpy(cls, array) -> "HIPTensor":
-        a = np.ascontiguousarray(array, dtype=np.float32)
-        t = cls(a.shape if a.ndim else (1,))
+    def from_numpy(cls, array, dtype: str = "float") -> "HIPTensor":
+        a = np.ascontiguousarray(array, dtype=DTYPES[dtype])
+        t = cls(a.shape if a.ndim else (1,), initial_element=None, dtype=dtype)
         if a.size:
             _lib.check(_lib.get().wf2hip_memcpy_h2d(C.c_void_p(t.vec.ptr), a.ctypes.data_as(C.c_void_p), a.nbytes))
         return t
 
     def storage_numpy(self) -> np.ndarray:
         """The whole underlying storage, flat."""
-        n = self.vec.nbytes // 4
-        out = np.empty(n, np.float32)
+        n = self.vec.nbytes // self.itemsize
+        out = np.empty(n, DTYPES[self.dtype])
         if n:
-            _lib.check(_lib.get().wf2hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.vec.ptr), 4 * n))
+            _lib.check(_lib.get().wf2hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.vec.ptr),
+                                                   self.itemsize * n))
         return out
 
     def numpy(self) -> np.ndarray:
@@ -218,26 +231,25 @@ class HIPTensor:
         flat = self.storage_numpy()
         shape, strides, off = self.geometry()
         if any(s == 0 for s in shape):
-            return np.empty(shape, np.float32)
+            return np.empty(shape, DTYPES[self.dtype])
         idx = np.full(shape, off, dtype=np.int64)
         for ax, (n, st) in enumerate(zip(shape, strides)):
             ix = np.arange(n, dtype=np.int64) * st
             idx += ix.reshape([-1 if i == ax else 1 for i in range(len(shape))])
-        out = flat[idx]
-        return out.view(np.uint32) if self.dtype == "uint32" else out
+        return flat[idx]
 
     # -- element access -------------------------------------------------------
     def vref(self, index: int) -> float:
         """Element ``index`` of the storage (``tensor.lisp:719-733``)."""
-        out = np.empty(1, np.float32)
+        out = np.empty(1, DTYPES[self.dtype])
         _lib.check(_lib.get().wf2hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p),
-                                               C.c_void_p(self.vec.ptr + 4 * int(index)), 4))
-        return float(out[0])
+                                               C.c_void_p(self.vec.ptr + self.itemsize * int(index)), self.itemsize))
+        return out[0].item()
 
     def set_vref(self, index: int, value: float) -> None:
-        v = np.asarray([value], np.float32)
-        _lib.check(_lib.get().wf2hip_memcpy_h2d(C.c_void_p(self.vec.ptr + 4 * int(index)),
-                                               v.ctypes.data_as(C.c_void_p), 4))
+        v = np.asarray([value], DTYPES[self.dtype])
+        _lib.check(_lib.get().wf2hip_memcpy_h2d(C.c_void_p(self.vec.ptr + self.itemsize * int(index)),
+                                               v.ctypes.data_as(C.c_void_p), self.itemsize))
 
     # -- views ------------------------------------------------------------------
     def view(self, *subscripts) -> "HIPTensor":

@@ -207,6 +207,75 @@ int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b);
  * 8-76).  `p` is the exponent for WF2HIP_POW and ignored otherwise. */
 int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p);
 
+/* ---- the other element types -------------------------------------------- */
+/* AddNode / SubNode / MulNode / DivNode / MoveTensorNode and inv for :double,
+ * :int32, :uint32, :int16, :uint16, :int8 and :uint8 tensors.  Replace
+ * waffe2_d{add,sub,mul,div} (cl-waffe2-simd.c:153-213 instantiated at :247-250),
+ * waffe2_{i32,i16,i8,u32,u16,u8}{add,sub,mul,div,copy} (:214-288; api.lisp:63-109),
+ * waffe2_{d,i32,...}inv (:290-310) and BLAS dcopy_ (source/backends/cpu/
+ * arithmetic.lisp:39-61), same argument order: x[i*incx] <- x[i*incx] OP y[i*incy].
+ * Integer arithmetic is C's (promotion to int, truncation on store, unsigned
+ * wrap-around, division toward zero); where the reference traps -- a zero
+ * divisor, INT_MIN / -1 -- the element becomes 0 / INT_MIN.  The 1-D :double
+ * entry points reproduce the reference's remainder loop, which rounds through
+ * binary32 (sas_dadd & co. return float, :229-232): the last n % 4 elements of a
+ * call, and every element when incx < 1.  The N-D entry point computes every
+ * element in binary64 and refuses accumulation into a broadcast destination. */
+enum wf2hip_dtype {
+  WF2HIP_F64 = 1,
+  WF2HIP_I32 = 2,
+  WF2HIP_U32 = 3,
+  WF2HIP_I16 = 4,
+  WF2HIP_U16 = 5,
+  WF2HIP_I8 = 6,
+  WF2HIP_U8 = 7
+};
+int wf2hip_binary_1d_typed(int dtype, int op, long n, void* x, long incx, const void* y, long incy);
+int wf2hip_binary_nd_typed(int dtype, int op, const wf2hip_view2* v, void* a, const void* b);
+int wf2hip_inv_1d_typed(int dtype, long n, void* x, long incx);
+int wf2hip_dcopy(long n, const double* y, long incy, double* x, long incx);
+int wf2hip_dadd(long n, double* x, long incx, const double* y, long incy);
+int wf2hip_dsub(long n, double* x, long incx, const double* y, long incy);
+int wf2hip_dmul(long n, double* x, long incx, const double* y, long incy);
+int wf2hip_ddiv(long n, double* x, long incx, const double* y, long incy);
+int wf2hip_dinv(long n, double* x, long incx);
+int wf2hip_i32add(long n, int32_t* x, long incx, const int32_t* y, long incy);
+int wf2hip_i32sub(long n, int32_t* x, long incx, const int32_t* y, long incy);
+int wf2hip_i32mul(long n, int32_t* x, long incx, const int32_t* y, long incy);
+int wf2hip_i32div(long n, int32_t* x, long incx, const int32_t* y, long incy);
+int wf2hip_i32copy(long n, int32_t* x, long incx, const int32_t* y, long incy);
+int wf2hip_i32inv(long n, int32_t* x, long incx);
+int wf2hip_u32add(long n, uint32_t* x, long incx, const uint32_t* y, long incy);
+int wf2hip_u32sub(long n, uint32_t* x, long incx, const uint32_t* y, long incy);
+int wf2hip_u32mul(long n, uint32_t* x, long incx, const uint32_t* y, long incy);
+int wf2hip_u32div(long n, uint32_t* x, long incx, const uint32_t* y, long incy);
+int wf2hip_u32copy(long n, uint32_t* x, long incx, const uint32_t* y, long incy);
+int wf2hip_u32inv(long n, uint32_t* x, long incx);
+int wf2hip_i16add(long n, int16_t* x, long incx, const int16_t* y, long incy);
+int wf2hip_i16sub(long n, int16_t* x, long incx, const int16_t* y, long incy);
+int wf2hip_i16mul(long n, int16_t* x, long incx, const int16_t* y, long incy);
+int wf2hip_i16div(long n, int16_t* x, long incx, const int16_t* y, long incy);
+int wf2hip_i16copy(long n, int16_t* x, long incx, const int16_t* y, long incy);
+int wf2hip_i16inv(long n, int16_t* x, long incx);
+int wf2hip_u16add(long n, uint16_t* x, long incx, const uint16_t* y, long incy);
+int wf2hip_u16sub(long n, uint16_t* x, long incx, const uint16_t* y, long incy);
+int wf2hip_u16mul(long n, uint16_t* x, long incx, const uint16_t* y, long incy);
+int wf2hip_u16div(long n, uint16_t* x, long incx, const uint16_t* y, long incy);
+int wf2hip_u16copy(long n, uint16_t* x, long incx, const uint16_t* y, long incy);
+int wf2hip_u16inv(long n, uint16_t* x, long incx);
+int wf2hip_i8add(long n, int8_t* x, long incx, const int8_t* y, long incy);
+int wf2hip_i8sub(long n, int8_t* x, long incx, const int8_t* y, long incy);
+int wf2hip_i8mul(long n, int8_t* x, long incx, const int8_t* y, long incy);
+int wf2hip_i8div(long n, int8_t* x, long incx, const int8_t* y, long incy);
+int wf2hip_i8copy(long n, int8_t* x, long incx, const int8_t* y, long incy);
+int wf2hip_i8inv(long n, int8_t* x, long incx);
+int wf2hip_u8add(long n, uint8_t* x, long incx, const uint8_t* y, long incy);
+int wf2hip_u8sub(long n, uint8_t* x, long incx, const uint8_t* y, long incy);
+int wf2hip_u8mul(long n, uint8_t* x, long incx, const uint8_t* y, long incy);
+int wf2hip_u8div(long n, uint8_t* x, long incx, const uint8_t* y, long incy);
+int wf2hip_u8copy(long n, uint8_t* x, long incx, const uint8_t* y, long incy);
+int wf2hip_u8inv(long n, uint8_t* x, long incx);
+
 /* ---- row selection: max / min value and index ----------------------------- */
 /* For every row of the `outer` space (a = X, b = OUT, in elements; use rank 1,
  * extent 1 for a single run): OUT <- max / min of the run x[i * incx], i < n, or

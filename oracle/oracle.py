@@ -386,3 +386,48 @@ def matmul_rowmajor(A: np.ndarray, B: np.ndarray, trans_a: bool = False,
     lib().orc_matmul_rowmajor(int(trans_a), int(trans_b), m, n, k, _fp(A), A.shape[1],
                               _fp(B), B.shape[1], _fp(out), n)
     return out
+
+
+# ---- the other element types -------------------------------------------------
+DTYPES = {"double": (1, np.float64, "d"), "int32": (2, np.int32, "i32"), "uint32": (3, np.uint32, "u32"),
+          "int16": (4, np.int16, "i16"), "uint16": (5, np.uint16, "u16"), "int8": (6, np.int8, "i8"),
+          "uint8": (7, np.uint8, "u8")}
+TYPED_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "copy": 4}
+
+
+def binary_typed_1d(dtype: str, op: str, n: int, x: np.ndarray, incx: int, y: np.ndarray, incy: int,
+                    offx: int = 0, offy: int = 0, use_ref: bool = False) -> None:
+    """x[offx + i incx] <- x[...] op y[offy + i incy] in place, through the oracle's
+    restatement or (use_ref) the reference's own waffe2_<prefix><op>; :double
+    copies have no reference symbol (BLAS dcopy_) and always take the oracle."""
+    code, npt, prefix = DTYPES[dtype]
+    assert x.dtype == npt and y.dtype == npt
+    size = x.itemsize
+    px = C.c_void_p(x.ctypes.data + size * offx)
+    py = C.c_void_p(y.ctypes.data + size * offy)
+    if use_ref and not (dtype == "double" and op == "copy"):
+        fn = getattr(ref(), f"waffe2_{prefix}{op}")
+        fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long]
+        fn.restype = None
+        fn(n, px, incx, py, incy)
+        return
+    fn = lib().orc_binary_typed
+    fn.argtypes = [C.c_int, C.c_int, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long]
+    fn.restype = C.c_int
+    assert fn(code, TYPED_OPS[op], n, px, incx, py, incy) == 0
+
+
+def inv_typed_1d(dtype: str, n: int, x: np.ndarray, incx: int, use_ref: bool = False) -> None:
+    code, npt, prefix = DTYPES[dtype]
+    assert x.dtype == npt
+    px = C.c_void_p(x.ctypes.data)
+    if use_ref:
+        fn = getattr(ref(), f"waffe2_{prefix}inv")
+        fn.argtypes = [C.c_long, C.c_void_p, C.c_long]
+        fn.restype = None
+        fn(n, px, incx)
+        return
+    fn = lib().orc_inv_typed
+    fn.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_long]
+    fn.restype = C.c_int
+    assert fn(code, n, px, incx) == 0

@@ -34,6 +34,9 @@
  *   orc_schedule / orc_*_nd            : worked schedules derived by hand from
  *       do-compiled-loop.lisp, exactly-once coverage invariant, brute-force
  *       N-D index walk on random tiny views.
+ *   orc_binary_typed, orc_inv_typed    : golden vectors from the compiled
+ *       reference C (waffe2_d*, waffe2_{i32,...}*), numpy closed forms (integer
+ *       wrap-around, binary64 arithmetic, the binary32 round trip of the tail).
  *   orc_sgemm                          : the reference's integer gemm vectors
  *       (base-impl/t/arithmetic.lisp:120,135,142,148), float64 truth.
  */
@@ -678,6 +681,107 @@ ORC_API void orc_matmul_rowmajor(int trans_a, int trans_b, long m, long n,
                                  const float *B, long ldb, float *C, long ldc) {
   orc_sgemm(trans_b ? 'C' : 'N', trans_a ? 'C' : 'N', n, m, k, 1.0f, B, ldb, A,
             lda, 0.0f, C, ldc);
+}
+
+
+/* ------------------------------------------------------------------ */
+/* The other element types                                             */
+/* ------------------------------------------------------------------ */
+/* waffe2_d{add,sub,mul,div}: define_arithmetic_func at SIMD_DOUBLE_STRIDE = 4
+ * (cl-waffe2-simd.c:153-213, instantiated :247-250).  The vector body handles
+ * (n / 4) * 4 elements when incx >= 1 in binary64; the remainder loop calls
+ * sas_d{add,sub,mul,div}, declared `float static inline` (:229-232), so those
+ * elements are rounded to binary32 on the way back.
+ * waffe2_{i32,...}{add,sub,mul,div,copy}: define_arithmetic_scal_func, plain C
+ * loops (:214-288).  Integer overflow wraps (two's complement, what the
+ * reference's compiled code does); a zero divisor and INT_MIN / -1 trap there
+ * and are left to the caller to avoid.
+ * dtype codes: 1 double, 2 int32, 3 uint32, 4 int16, 5 uint16, 6 int8, 7 uint8;
+ * op codes: 0 add, 1 sub, 2 mul, 3 div, 4 copy. */
+static double orc_dop(int op, double a, double b) {
+  switch (op) {
+    case 0: return a + b;
+    case 1: return a - b;
+    case 2: return a * b;
+    case 3: return a / b;
+    default: return b;
+  }
+}
+
+#define ORC_INT_LOOP(T, W, U)                                          \
+  {                                                                    \
+    T *xp = (T *)x;                                                    \
+    const T *yp = (const T *)y;                                        \
+    for (long c = 0; c < n; c++) {                                     \
+      W a = (W)xp[0], b = (W)yp[0];                                    \
+      switch (op) {                                                    \
+        case 0: xp[0] = (T)(U)((U)a + (U)b); break;                    \
+        case 1: xp[0] = (T)(U)((U)a - (U)b); break;                    \
+        case 2: xp[0] = (T)(U)((U)a * (U)b); break;                    \
+        case 3: xp[0] = (T)(a / b); break;                             \
+        default: xp[0] = yp[0]; break;                                 \
+      }                                                                \
+      xp += incx;                                                      \
+      yp += incy;                                                      \
+    }                                                                  \
+  }
+
+ORC_API int orc_binary_typed(int dtype, int op, long n, void *x, long incx, const void *y, long incy) {
+  if (op < 0 || op > 4) return -1;
+  switch (dtype) {
+    case 1: {
+      double *xp = (double *)x;
+      const double *yp = (const double *)y;
+      long count = 0;
+      if (op == 4) { /* dcopy_ (BLAS): no arithmetic */
+        for (long c = 0; c < n; c++) xp[c * incx] = yp[c * incy];
+        return 0;
+      }
+      if (incx >= 1) {
+        const long simd_end = (n / 4) * 4;
+        for (; count < simd_end; count++) xp[count * incx] = orc_dop(op, xp[count * incx], yp[count * incy]);
+      }
+      xp += count * incx;
+      yp += count * incy;
+      for (; count < n; count++) {
+        xp[0] = (double)(float)orc_dop(op, xp[0], yp[0]); /* sas_d*: float return type */
+        xp += incx;
+        yp += incy;
+      }
+      return 0;
+    }
+    case 2: ORC_INT_LOOP(int32_t, int32_t, uint32_t) return 0;
+    case 3: ORC_INT_LOOP(uint32_t, uint32_t, uint32_t) return 0;
+    case 4: ORC_INT_LOOP(int16_t, int, unsigned) return 0;
+    case 5: ORC_INT_LOOP(uint16_t, int, unsigned) return 0;
+    case 6: ORC_INT_LOOP(int8_t, int, unsigned) return 0;
+    case 7: ORC_INT_LOOP(uint8_t, int, unsigned) return 0;
+    default: return -1;
+  }
+}
+
+/* waffe2_{d,i32,...}inv: x[0] = 1 / x[0] (cl-waffe2-simd.c:290-310) */
+ORC_API int orc_inv_typed(int dtype, long n, void *x, long incx) {
+#define ORC_INV(T, ONE)                      \
+  {                                          \
+    T *xp = (T *)x;                          \
+    for (long c = 0; c < n; c++) {           \
+      xp[0] = (T)(ONE / xp[0]);              \
+      xp += incx;                            \
+    }                                        \
+    return 0;                                \
+  }
+  switch (dtype) {
+    case 1: ORC_INV(double, 1.0)
+    case 2: ORC_INV(int32_t, 1)
+    case 3: ORC_INV(uint32_t, 1)
+    case 4: ORC_INV(int16_t, 1)
+    case 5: ORC_INV(uint16_t, 1)
+    case 6: ORC_INV(int8_t, 1)
+    case 7: ORC_INV(uint8_t, 1)
+    default: return -1;
+  }
+#undef ORC_INV
 }
 
 ORC_API int orc_abi_version(void) { return 1; }

@@ -195,6 +195,75 @@ def im2col_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "im2col_kernels.npz")), "bytes")
 
 
+TYPED_REGIMES = [(1, 1), (1, 0), (2, 1), (1, 3), (2, 2), (0, 1), (0, 2)]
+TYPED_SIZES = [1, 4, 5, 13]
+
+
+def typed_operands(rng, dtype, size, op, incx):
+    """Operands that keep the reference out of its traps: no zero divisors, no
+    INT_MIN / -1; everything else (overflow, wrap-around) is fair game."""
+    npt = O.DTYPES[dtype][1]
+    if dtype == "double":
+        x = rng.standard_normal(size)
+        y = rng.standard_normal(size) if incx != 0 or op in ("add", "sub") else rng.uniform(0.9, 1.1, size)
+        return x.astype(npt), y.astype(npt)
+    info = np.iinfo(npt)
+    x = rng.integers(info.min, info.max, size, dtype=np.int64, endpoint=True).astype(npt)
+    y = rng.integers(info.min, info.max, size, dtype=np.int64, endpoint=True).astype(npt)
+    if op == "div":
+        small = rng.integers(1, 12, size).astype(npt)
+        if info.min < 0:
+            small = (small * rng.choice(np.array([1, -1], np.int64), size).astype(npt)).astype(npt)
+            x[x == info.min] = info.min + 1
+        y = np.where(rng.random(size) < 0.7, small, y).astype(npt)
+        y[y == 0] = 3
+    return x, y
+
+
+def typed_goldens():
+    """waffe2_d{add,sub,mul,div}, waffe2_{i32,...}{add,sub,mul,div,copy} and
+    waffe2_*inv of the compiled reference, every increment regime."""
+    assert O.ref() is not None, "oracle/_ref/libwaffe2_simd_ref.so is missing: run `make -C oracle ref`"
+    rng = np.random.Generator(np.random.PCG64(2028))
+    out = {}
+    # per (dtype, op): the cases back to back, `cases` rows = (n, incx, incy, start, size)
+    for dtype in O.DTYPES:
+        for op in ("add", "sub", "mul", "div", "copy"):
+            if dtype == "double" and op == "copy":
+                continue  # BLAS dcopy_, not in the compiled kernels
+            xs, ys, outs, cases, start = [], [], [], [], 0
+            for n in TYPED_SIZES:
+                for incx, incy in TYPED_REGIMES:
+                    size = n * 3 + 1
+                    x, y = typed_operands(rng, dtype, size, op, incx)
+                    res = x.copy()
+                    O.binary_typed_1d(dtype, op, n, res, incx, y, incy, use_ref=True)
+                    xs.append(x), ys.append(y), outs.append(res)
+                    cases.append((n, incx, incy, start, size))
+                    start += size
+            key = f"{dtype}_{op}"
+            out[key + "_x"], out[key + "_y"], out[key + "_out"] = (np.concatenate(v) for v in (xs, ys, outs))
+            out[key + "_cases"] = np.array(cases, np.int64)
+        xs, outs, cases, start = [], [], [], 0
+        for n in (1, 5, 64):
+            for incx in (1, 2):
+                x, _ = typed_operands(rng, dtype, n * 2 + 1, "add", 1)
+                if dtype != "double":  # mostly the values whose inverse is not 0; never 0
+                    info = np.iinfo(x.dtype)
+                    pool = np.array([1, 2, 3, info.max] + ([-1, -2, info.min + 1] if info.min < 0 else []), np.int64)
+                    x = np.where(rng.random(x.size) < 0.8, rng.choice(pool, x.size), x.astype(np.int64)).astype(x.dtype)
+                    x[x == 0] = 1
+                res = x.copy()
+                O.inv_typed_1d(dtype, n, res, incx, use_ref=True)
+                xs.append(x), outs.append(res)
+                cases.append((n, incx, 0, start, x.size))
+                start += x.size
+        out[f"{dtype}_inv_x"], out[f"{dtype}_inv_out"] = np.concatenate(xs), np.concatenate(outs)
+        out[f"{dtype}_inv_cases"] = np.array(cases, np.int64)
+    np.savez_compressed(os.path.join(HERE, "typed_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
     if "--im2col-only" in sys.argv:
         im2col_goldens()
@@ -202,8 +271,11 @@ if __name__ == "__main__":
         compare_goldens()
     elif "--unary-more-only" in sys.argv:
         unary_more_goldens()
+    elif "--typed-only" in sys.argv:
+        typed_goldens()
     else:
         main()
         compare_goldens()
         unary_more_goldens()
         im2col_goldens()
+        typed_goldens()

@@ -1,0 +1,143 @@
+"""GPU parity of the arithmetic / move kernels for :double and the integer
+dtypes: bit-exact against the golden vectors of the compiled reference
+(tests/golden/typed_kernels.npz) and the oracle on larger seeded inputs through
+the 1-D entry points; numpy closed forms through the node layer (N-D views)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "typed_kernels.npz")
+DTYPES = ["double", "int32", "uint32", "int16", "uint16", "int8", "uint8"]
+OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "copy": 4}
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint8)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_1d_entry_points_against_reference_goldens(gpu, O, dtype):
+    W = gpu
+    lib = W.lib.get()
+    gold = np.load(GOLD)
+    code = W.lib.DTYPE_CODES[dtype]
+    size = np.dtype(O.DTYPES[dtype][1]).itemsize
+    for op, opcode in OPS.items():
+        key = f"{dtype}_{op}"
+        if key + "_x" not in gold:
+            continue
+        for n, incx, incy, start, length in gold[key + "_cases"]:
+            sl = slice(int(start), int(start + length))
+            dx = W.HIPTensor.from_numpy(gold[key + "_x"][sl], dtype=dtype)
+            dy = W.HIPTensor.from_numpy(gold[key + "_y"][sl], dtype=dtype)
+            W.lib.check(lib.wf2hip_binary_1d_typed(code, opcode, int(n), C.c_void_p(dx.ptr), int(incx),
+                                                   C.c_void_p(dy.ptr), int(incy)))
+            np.testing.assert_array_equal(_bits(dx.numpy()), _bits(gold[key + "_out"][sl]),
+                                          err_msg=f"{key} n={n} incx={incx} incy={incy}")
+    for n, incx, _, start, length in gold[f"{dtype}_inv_cases"]:
+        sl = slice(int(start), int(start + length))
+        dx = W.HIPTensor.from_numpy(gold[f"{dtype}_inv_x"][sl], dtype=dtype)
+        W.lib.check(lib.wf2hip_inv_1d_typed(code, int(n), C.c_void_p(dx.ptr), int(incx)))
+        np.testing.assert_array_equal(_bits(dx.numpy()), _bits(gold[f"{dtype}_inv_out"][sl]))
+    assert size in (1, 2, 4, 8)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_1d_entry_points_against_oracle_at_size(gpu, O, dtype):
+    """Sizes that reach the 16-byte vector kernel, its scalar remainder, unaligned
+    starts and every increment regime; named wrappers (wf2hip_dadd ...) included."""
+    W = gpu
+    lib = W.lib.get()
+    code, npt, prefix = O.DTYPES[dtype]
+    rng = np.random.default_rng(31 + code)
+    item = np.dtype(npt).itemsize
+
+    def draw(size, op):
+        if dtype == "double":
+            return rng.standard_normal(size), rng.uniform(0.5, 2.0, size) * rng.choice([-1.0, 1.0], size)
+        info = np.iinfo(npt)
+        x = rng.integers(info.min, info.max, size, endpoint=True).astype(npt)
+        y = rng.integers(info.min, info.max, size, endpoint=True).astype(npt)
+        if op == "div":
+            y = np.where(rng.random(size) < 0.6, rng.integers(1, 9, size).astype(npt), y).astype(npt)
+            y[y == 0] = 5
+            x[x == info.min] = info.max
+        return x, y
+
+    for op, opcode in OPS.items():
+        for n, incx, incy, offx, offy in [(100003, 1, 1, 0, 0), (65536, 1, 0, 0, 0), (40001, 1, 1, 1, 0),
+                                          (30000, 2, 1, 0, 3), (30000, 1, 3, 0, 0), (999, 3, 2, 2, 1),
+                                          (777, 0, 1, 5, 0), (0, 1, 1, 0, 0)]:
+            if incx == 0 and dtype != "double" and op in ("mul",):
+                pass  # wrap-around products are fine for integers
+            size = max(n, 1) * 3 + 8
+            x, y = draw(size, op)
+            x, y = x.astype(npt), y.astype(npt)
+            if incx == 0 and op == "div" and dtype != "double":
+                y[:] = 1 + (np.arange(size) % 3)
+            want = x.copy()
+            O.binary_typed_1d(dtype, op, n, want, incx, y, incy, offx=offx, offy=offy)
+            dx, dy = W.HIPTensor.from_numpy(x, dtype=dtype), W.HIPTensor.from_numpy(y, dtype=dtype)
+            px, py = C.c_void_p(dx.ptr + item * offx), C.c_void_p(dy.ptr + item * offy)
+            if op == "copy" and dtype == "double":
+                fn = lib.wf2hip_dcopy
+                fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long]
+                W.lib.check(fn(n, py, incy, px, incx))
+            else:
+                fn = getattr(lib, f"wf2hip_{prefix}{op}")
+                fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long]
+                fn.restype = C.c_int
+                W.lib.check(fn(n, px, incx, py, incy))
+            np.testing.assert_array_equal(_bits(dx.numpy()), _bits(want),
+                                          err_msg=f"{dtype} {op} n={n} incx={incx} incy={incy} off=({offx},{offy})")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_nodes_on_views(gpu, dtype):
+    """AddNode ... MoveTensorNode through the node layer on N-D views (slices,
+    steps, broadcasts, permutes): numpy closed form (binary64 arithmetic for
+    :double -- the N-D entry has no per-call remainder --, wrap-around for ints)."""
+    W = gpu
+    F = W.functional
+    from importlib import import_module
+    npt = import_module("cl-waffe2_amd.tensor").DTYPES[dtype]
+    rng = np.random.default_rng(77)
+
+    def draw(shape, nonzero=False):
+        if dtype == "double":
+            a = rng.standard_normal(shape)
+            return a + np.sign(a) if nonzero else a
+        info = np.iinfo(npt)
+        if nonzero:
+            return rng.integers(1, 9, shape).astype(npt)
+        return rng.integers(info.min // 2, info.max // 2, shape, endpoint=True).astype(npt)
+
+    A = draw((12, 40, 34))
+    dA = F.from_numpy(A, dtype=dtype)
+    with np.errstate(over="ignore"):
+        # contiguous, both operands full
+        B = draw(A.shape)
+        got = F.add(dA, F.from_numpy(B, dtype=dtype))
+        np.testing.assert_array_equal(got.numpy(), (A + B).astype(npt))
+        # slices with steps against a row broadcast
+        v = dA.view((2, 10), (0, 40, 3), (1, 33, 2))
+        R = draw((1, 1, 16))
+        x = F.copy(v)
+        assert x.dtype == dtype and x.shape == [8, 13, 16]  # a range holds floor((to - from) / step) elements
+        F.sub_(x, F.from_numpy(R, dtype=dtype).view((":broadcast", 8), (":broadcast", 13), True))
+        np.testing.assert_array_equal(x.numpy(), (A[2:10, 0:40:3, 1:33:2][:, :13] - R).astype(npt))
+        # permuted source, scalar operand, division by a non-zero tensor
+        p = F.copy(dA.permute(2, 0, 1))
+        np.testing.assert_array_equal(p.numpy(), np.transpose(A, (2, 0, 1)))
+        s = F.mul(dA, 3)
+        np.testing.assert_array_equal(s.numpy(), (A * npt(3)).astype(npt))
+        D = draw(A.shape, nonzero=True)
+        q = F.div(dA, F.from_numpy(D, dtype=dtype))
+        want = A / D if dtype == "double" else np.trunc(A.astype(np.float64) / D).astype(npt)
+        np.testing.assert_array_equal(q.numpy(), want)
+    with pytest.raises(W.HIPError):  # accumulation into a broadcast destination: :float only
+        F.add_(F.from_numpy(draw((1, 4)), dtype=dtype).view((":broadcast", 3), True), F.from_numpy(draw((3, 4)), dtype=dtype))

@@ -94,8 +94,9 @@ def test_dispatch_rules(W):
     with W.with_devices(MyBackend):
         with pytest.raises(W.NodeNotFound):
             W.nodes.find_impl("AddNode")
-    with pytest.raises(W.NodeNotFound):                        # ints are rejected: no device fallback here
-        W.nodes.find_impl("AddNode", dtype="int32")
+    assert W.nodes.find_impl("AddNode", dtype="int32") is not None   # arithmetic and moves take every dtype
+    with pytest.raises(W.NodeNotFound):                        # the rest reject ints: no device fallback here
+        W.nodes.find_impl("ExpNode", dtype="int32")
     with pytest.raises(ValueError):
         W.define_impl("SumNode", W.HIPTensor)                  # cl-waffe2 has no SumNode
     del W.nodes.DEVICE_FEATURES[MyBackendWithImpl]
