@@ -237,6 +237,15 @@ def row_table(W, reps: int = 10, warm: int = 3):
             (8 + 12) * 2048 * Cn, note="two launches: MoveTensorNode 8 B/elem, SubNode 12 B/elem")
     del a0, b0, yb
 
+    # the arithmetic nodes on other element types (16-byte vectors, same traffic per byte)
+    for dtype, count in (("double", N // 2), ("int32", N), ("uint8", 4 * N)):
+        host = (rng.standard_normal(count) * 50).astype(getattr(np, {"double": "float64"}.get(dtype, dtype)))
+        x0 = T.from_numpy(host, dtype=dtype)
+        del host
+        ring = ring_of(lambda: (clone(x0), clone(x0)), 2 * 4 * N)
+        measure(f"x += y, :{dtype}, 256 MiB per tensor", ring, lambda s: F.add_(s[0], s[1]), 12 * N)
+        del x0
+
     # transposing copy through LDS tiles
     a0 = normal([SIDE, SIDE])
     ring = ring_of(lambda: (clone(a0), T([SIDE, SIDE], initial_element=None)), 8 * N)
