@@ -281,6 +281,33 @@ def row_table(W, reps: int = 10, warm: int = 3):
                  "rate quoted on the 8 B/elem of the fused form")
     del x0
 
+    # the next rows of the path: compare / where, row max and argmax, fused GELU and
+    # LayerNorm, optimiser steps
+    x0 = normal([N])
+    ring = ring_of(lambda: (clone(x0), clone(x0), T([N], initial_element=None)), 12 * N)
+    measure("compare x < y -> 1 / 0, 2^26", ring, lambda s: F.compare(s[0], s[1], "<", out=s[2]), 12 * N)
+    ring = ring_of(lambda: (clone(x0), T([N], initial_element=None)), 8 * N)
+    measure("where x > 0.5 -> 1 / 0 (scalar), 2^26", ring, lambda s: F.where(s[0], ">", 0.5, out=s[1]), 8 * N)
+    ring = ring_of(lambda: (clone(x0), T([N], initial_element=None)), 8 * N)
+    measure("GELU, one kernel, 2^26", ring, lambda s: F.gelu_fused(s[0], out=s[1]), 8 * N)
+    del x0
+    R, Cn = 65536, 1024
+    x0 = normal([R, Cn])
+    ring = ring_of(lambda: clone(x0), 4 * R * Cn)
+    measure("row max (65536,1024)", ring, lambda s: F.max(s, axis=1), 4 * R * Cn + 4 * R)
+    ring = ring_of(lambda: clone(x0), 4 * R * Cn)
+    measure("row argmax (65536,1024)", ring, lambda s: F.argmax(s, axis=1), 4 * R * Cn + 4 * R)
+    g0, b0 = normal([Cn]), normal([Cn])
+    ring = ring_of(lambda: (clone(x0), T([R, Cn], initial_element=None)), 8 * R * Cn)
+    measure("LayerNorm (65536,1024), one kernel", ring, lambda s: F.layer_norm_fused(s[0], g0, b0, out=s[1]),
+            8 * R * Cn)
+    del x0, g0, b0
+    p0 = normal([N])
+    for name, make, per in (("Adam", lambda p: W.optimizers.Adam(p, lr=1e-3), 28), ("SGD", lambda p: W.optimizers.SGD(p, lr=1e-3), 16)):
+        ring = ring_of(lambda: (make(clone(p0)), clone(p0)), per * N)
+        measure(f"{name} step, 2^26 parameters, one kernel", ring, lambda s: s[0].step(s[1]), per * N)
+    del p0
+
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),
                     (8192, 768, 3072)):

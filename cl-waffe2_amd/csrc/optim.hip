@@ -33,11 +33,13 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
   if (VEC) {
     constexpr int U = 2;
     const size_t nvec = n / 4;
-    const size_t base = (size_t)blockIdx.x * kBlock * U + threadIdx.x;
+    // each wavefront on 1 KB of its own per access and stream
+    const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWave * U +
+                        (threadIdx.x & (kWave - 1));
     f4 pv[U], gv[U], mv[U], vv[U];
 #pragma unroll
     for (int u = 0; u < U; u++) {
-      const size_t i = base + (size_t)u * kBlock;
+      const size_t i = base + (size_t)u * kWave;
       if (i < nvec) {
         pv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(p) + i) : reinterpret_cast<f4*>(p)[i];
         gv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(g) + i)
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
     }
 #pragma unroll
     for (int u = 0; u < U; u++) {
-      const size_t i = base + (size_t)u * kBlock;
+      const size_t i = base + (size_t)u * kWave;
       if (i < nvec) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
@@ -79,25 +81,51 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
   }
 }
 
-template <bool VEC>
+// VEC: four 16-byte vectors per lane and stream, wave-contiguous, loads first
+// (the shape measured best for x <- x op y); NT as above.
+template <bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void sgd_kernel(float* __restrict__ p, float* __restrict__ g,
                                                      size_t n, float lr) {
-  const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (VEC) {
+    constexpr int U = 4;
     const size_t nvec = n / 4;
-    if (i < nvec) {
-      f4 gv = reinterpret_cast<f4*>(g)[i] * lr;
-      reinterpret_cast<f4*>(g)[i] = gv;
-      reinterpret_cast<f4*>(p)[i] = reinterpret_cast<f4*>(p)[i] - gv;
+    const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWave * U +
+                        (threadIdx.x & (kWave - 1));
+    f4 pv[U], gv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (i < nvec) {
+        pv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(p) + i) : reinterpret_cast<f4*>(p)[i];
+        gv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(g) + i) : reinterpret_cast<f4*>(g)[i];
+      }
     }
-    if (i < (n & 3)) {
-      const size_t j = nvec * 4 + i;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (i < nvec) {
+        gv[u] = gv[u] * lr;
+        pv[u] = pv[u] - gv[u];
+        if (NT) {
+          __builtin_nontemporal_store(gv[u], reinterpret_cast<f4*>(g) + i);
+          __builtin_nontemporal_store(pv[u], reinterpret_cast<f4*>(p) + i);
+        } else {
+          reinterpret_cast<f4*>(g)[i] = gv[u];
+          reinterpret_cast<f4*>(p)[i] = pv[u];
+        }
+      }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+      const size_t j = nvec * 4 + threadIdx.x;
       g[j] = g[j] * lr;
       p[j] = p[j] - g[j];
     }
-  } else if (i < n) {
-    g[i] = g[i] * lr;
-    p[i] = p[i] - g[i];
+  } else {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) {
+      g[i] = g[i] * lr;
+      p[i] = p[i] - g[i];
+    }
   }
 }
 
@@ -145,13 +173,16 @@ WF2_API int wf2hip_sgd_step_f32(long n, float* param, float* grad, float lr) {
   if (!disjoint(param, grad, (size_t)n))
     return fail(WF2HIP_EOVERLAP, "sgd step: parameter and gradient must not overlap");
   const bool vec = aligned16(param) && aligned16(grad);
-  const int64_t threads = vec ? (n / 4 > 3 ? n / 4 : 4) : n;
-  const int64_t blocks = ceil_div(threads, kBlock);
+  const int64_t nvec = n / 4 > 0 ? n / 4 : 1;
+  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 4) : ceil_div(n, kBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
   hipStream_t st = rt().stream;
-  if (vec)
-    sgd_kernel<true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
+  const bool streaming = (int64_t)n * 16 >= ((int64_t)192 << 20);
+  if (vec && streaming)
+    sgd_kernel<true, true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
+  else if (vec)
+    sgd_kernel<true, false><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
   else
-    sgd_kernel<false><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
+    sgd_kernel<false, false><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
   return after_launch("sgd_kernel");
 }
