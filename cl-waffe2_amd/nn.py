@@ -56,3 +56,45 @@ def avg_pool2d(x: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
     """``AvgPool2D`` (pool.lisp:95-105)."""
     return _pool(x, kernel_size, kernel_size if stride is None else stride, padding,
                  lambda w: F.mean(w, axis=1))
+
+
+# ---------------------------------------------------------------------------
+# criteria (source/nn/criterion.lisp), composed from the backend's nodes
+# ---------------------------------------------------------------------------
+
+def _reduce(z: HIPTensor, reduction):
+    if reduction == "sum":
+        return F.sum(z)
+    if reduction == "mean":
+        return F.mean(z)
+    return z
+
+
+def mse(x: HIPTensor, y: HIPTensor, reduction="mean") -> HIPTensor:
+    """``(mse x y :reduction :mean)`` (criterion.lisp:48-80): ``(x - y)^2``."""
+    l = F.sub(x, y)
+    return _reduce(F.mul(l, l), reduction)
+
+
+def cross_entropy_loss(x: HIPTensor, labels: HIPTensor, delta: float = 1e-7, reduction=True) -> HIPTensor:
+    """``(cross-entropy-loss x labels :delta 1e-7)`` (criterion.lisp:128-167):
+    ``-labels * log(x + delta)`` with one-hot ``labels``."""
+    z = F.mul(F.mul(labels, F.loge(F.add(x, delta))), -1.0)
+    return _reduce(z, reduction)
+
+
+def softmax_cross_entropy(x: HIPTensor, labels: HIPTensor, axis: int = 1, delta: float = 1e-7,
+                          avoid_overflow: bool = False, reduction=True):
+    """``(softmax-cross-entropy x labels ...)`` = Softmax-Cross-Entropy-Node
+    (criterion.lisp:90-126,169-196): softmax, then the cross entropy.  Returns
+    ``(loss, z)`` where ``z`` is the softmax the node saves for its backward."""
+    z = F.softmax(x, avoid_overflow=avoid_overflow, axis=axis)
+    return _reduce(cross_entropy_loss(z, labels, delta=delta), reduction), z
+
+
+def softmax_cross_entropy_backward(dy, z: HIPTensor, labels: HIPTensor) -> HIPTensor:
+    """The node's backward, ``sce-diff-static`` (criterion.lisp:82-88):
+    ``dy * (z - labels) / batch`` with ``batch`` the second-to-last extent of
+    ``z``; ``dy`` is the upstream gradient (a tensor of z's shape or a number)."""
+    batch = float(z.shape[-2])
+    return F.div(F.mul(F.sub(z, labels), dy), batch)

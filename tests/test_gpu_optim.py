@@ -148,3 +148,70 @@ def test_weights_round_trip(gpu, tmp_path):
     assert back["steps"] == 12 and back["lr"] == 0.5
     assert_bit_equal(back["layer/w"].numpy(), a, "wf2model tensor")
     assert_bit_equal(back["bias"].numpy(), a[0, 0], "wf2model flat tensor")
+
+
+def test_classifier_training_step_by_step(gpu):
+    """A two-layer classifier trained entirely on the device with the
+    reference's recipes: Linear = matmul + bias (AddNode with a broadcast row),
+    !relu = x * (x > 0), Softmax-Cross-Entropy-Node forward and backward
+    (nn/criterion.lisp:82-126), bias gradients as !sum over the batch, matmul
+    backward products, Adam.  Every step is compared with the same recipe in
+    float64 on the host (loss and weights), and the loss must fall."""
+    W = gpu
+    F = W.functional
+    nn = W.nn
+    rng = np.random.default_rng(33)
+    n, d, h, c = 512, 96, 128, 10
+    centers = rng.standard_normal((c, d)) * 2.0
+    cls = rng.integers(0, c, n)
+    x = (centers[cls] + rng.standard_normal((n, d))).astype(f32)
+    labels = np.eye(c, dtype=f32)[cls]
+    params = {"w1": (rng.standard_normal((d, h)) * 0.1).astype(f32), "b1": np.zeros((1, h), f32),
+              "w2": (rng.standard_normal((h, c)) * 0.1).astype(f32), "b2": np.zeros((1, c), f32)}
+    dev = {k: F.from_numpy(v) for k, v in params.items()}
+    opt = {k: W.optimizers.Adam(dev[k], lr=0.01) for k in dev}
+    dx, dl = F.from_numpy(x), F.from_numpy(labels)
+
+    # float64 mirror of the same recipe (mean-subtracted softmax as the reference's !softmax)
+    ref = {k: v.astype(np.float64) for k, v in params.items()}
+    state = {k: (np.zeros_like(v), np.zeros_like(v)) for k, v in ref.items()}
+
+    def host_step(t):
+        a1 = x @ ref["w1"] + ref["b1"]
+        h1 = a1 * (a1 > 0)
+        a2 = h1 @ ref["w2"] + ref["b2"]
+        e = np.exp(a2 - a2.mean(axis=1, keepdims=True))
+        z = e / e.sum(axis=1, keepdims=True)
+        loss = np.mean(-labels * np.log(z + 1e-7))
+        dz = (z - labels) * (1.0 / labels.size) / n  # d mean / d out, then sce-diff-static: / batch
+        grads = {"w2": h1.T @ dz, "b2": dz.sum(axis=0, keepdims=True)}
+        dh = (dz @ ref["w2"].T) * (a1 > 0)
+        grads["w1"], grads["b1"] = x.T @ dh, dh.sum(axis=0, keepdims=True)
+        for k, g in grads.items():
+            m, v = state[k]
+            m += (g - m) * (1 - 0.9)
+            v += (1 - 0.999) * (g * g - v)
+            lr_t = 0.01 * np.sqrt(1 - 0.999 ** t) / (1 - 0.9 ** t)
+            ref[k] -= (m * lr_t) / (1e-7 + np.sqrt(v))
+        return loss
+
+    losses = []
+    for t in range(1, 41):
+        a1 = F.add(F.matmul(dx, dev["w1"]), dev["b1"])
+        mask = F.where(a1, ">", 0.0)
+        h1 = F.mul(a1, mask)
+        a2 = F.add(F.matmul(h1, dev["w2"]), dev["b2"])
+        loss, z = nn.softmax_cross_entropy(a2, dl, avoid_overflow=True, reduction="mean")
+        dz = nn.softmax_cross_entropy_backward(1.0 / labels.size, z, dl)
+        grads = {"w2": F.matmul(F.t(h1), dz), "b2": F.sum(dz, axis=0)}  # (1, c): the reduced axis stays, size 1
+        dh = F.mul_(F.matmul(dz, F.t(dev["w2"])), mask)
+        grads["w1"], grads["b1"] = F.matmul(F.t(dx), dh), F.sum(dh, axis=0)
+        for k in dev:
+            opt[k].step(grads[k])
+        want = host_step(t)
+        got = float(loss.numpy().ravel()[0])
+        losses.append(got)
+        assert abs(got - want) <= 2e-4 * abs(want) + 1e-6, (t, got, want)
+    for k in dev:
+        np.testing.assert_allclose(dev[k].numpy(), ref[k], rtol=0, atol=5e-3, err_msg=k)
+    assert losses[-1] < 0.5 * losses[0], losses
