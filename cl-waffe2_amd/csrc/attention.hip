@@ -72,7 +72,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const int h = bh - b * p.heads;
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // uniform: DMA destinations, trip counts and
+                                                                         // the causal skipping stay on the scalar unit
   const int half = lane >> 5;
   const int col = lane & 31;
 
