@@ -15,7 +15,8 @@
 //   S^T = K . Q^T      A operand = K fragment (LDS, conflict-free 128-bit reads),
 //                      B operand = Q fragment (registers for the whole kernel,
 //                      pre-multiplied by scale * log2 e)
-//   O^T += V^T . P^T   A operand = V fragment (LDS, conflict-free 32-bit reads),
+//   O^T += V^T . P^T   A operand = V fragment (LDS, conflict-free 64-bit reads: one accumulator
+//                      owns the even head dimensions, the other the odd ones),
 //                      B operand = P^T, which is exactly the S^T accumulator
 //                      after exp2: accumulator register i of a lane holds key
 //                      8 (i/4) + 4 (lane/32) + i%4 of its query, and MFMA step i
@@ -202,19 +203,20 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       o1[i] *= alpha;
     }
   };
-  // O^T += V^T . P^T
+  // O^T += V^T . P^T.  Accumulator o0 owns the even head dimensions, o1 the odd
+  // ones: a lane then needs V[key][2 col] and V[key][2 col + 1], one 64-bit read
+  // (half as many LDS instructions as two tiles of 32 consecutive dimensions).
+  typedef float f2 __attribute__((ext_vector_type(2)));
   auto accumulate = [&](const float* sv, const f16v& s0, const f16v& s1) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int key = 8 * (i >> 2) + 4 * half + (i & 3);
-      const float v00 = sv[key * kRowFloats + (col ^ vswap)];
-      const float v01 = sv[key * kRowFloats + ((32 + col) ^ vswap)];
-      const float v10 = sv[(32 + key) * kRowFloats + (col ^ vswap)];
-      const float v11 = sv[(32 + key) * kRowFloats + ((32 + col) ^ vswap)];
-      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v00, s0[i], o0, 0, 0, 0);
-      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v01, s0[i], o1, 0, 0, 0);
-      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v10, s1[i], o0, 0, 0, 0);
-      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v11, s1[i], o1, 0, 0, 0);
+      const f2 v0 = *reinterpret_cast<const f2*>(sv + key * kRowFloats + ((2 * col) ^ vswap));
+      const f2 v1 = *reinterpret_cast<const f2*>(sv + (32 + key) * kRowFloats + ((2 * col) ^ vswap));
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v0.x, s0[i], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v0.y, s0[i], o1, 0, 0, 0);
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v1.x, s1[i], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v1.y, s1[i], o1, 0, 0, 0);
     }
   };
 
@@ -261,13 +263,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const float inv = 1.0f / total;
   if (query < p.seq) {
     float* op = p.o + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
-    // register i of tile t holds head dimension 32 t + 8 (i/4) + 4 half + i%4
+    // register i of o0 / o1 holds head dimension 2 r / 2 r + 1, r = 8 (i/4) + 4 half + i%4:
+    // four consecutive registers of both make eight consecutive dimensions
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      f4 a = {o0[4 * g] * inv, o0[4 * g + 1] * inv, o0[4 * g + 2] * inv, o0[4 * g + 3] * inv};
-      f4 c = {o1[4 * g] * inv, o1[4 * g + 1] * inv, o1[4 * g + 2] * inv, o1[4 * g + 3] * inv};
-      if (8 * g + 4 * half < p.head_dim) *reinterpret_cast<f4*>(op + 8 * g + 4 * half) = a;
-      if (32 + 8 * g + 4 * half < p.head_dim) *reinterpret_cast<f4*>(op + 32 + 8 * g + 4 * half) = c;
+      const int d0 = 16 * g + 8 * half;
+      f4 a = {o0[4 * g] * inv, o1[4 * g] * inv, o0[4 * g + 1] * inv, o1[4 * g + 1] * inv};
+      f4 c = {o0[4 * g + 2] * inv, o1[4 * g + 2] * inv, o0[4 * g + 3] * inv, o1[4 * g + 3] * inv};
+      if (d0 < p.head_dim) *reinterpret_cast<f4*>(op + d0) = a;
+      if (d0 + 4 < p.head_dim) *reinterpret_cast<f4*>(op + d0 + 4) = c;
     }
   }
 }
