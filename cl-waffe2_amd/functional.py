@@ -354,6 +354,35 @@ def sigmoid(x: HIPTensor) -> HIPTensor:
     return div(1.0, add(1.0, exp(mul(-1.0, x))))
 
 
+def leaky_relu(x: HIPTensor, negative_slope: float = 0.01) -> HIPTensor:
+    """``(!leaky-relu x :negative-slope 0.01)`` = ``x * (A>=scal x 0.0 :true-then 1.0
+    :false-then slope)`` (``source/nn/activation.lisp:68-92``)."""
+    return mul(x, where(x, ">=", 0.0, 1.0, float(np.float32(negative_slope))))
+
+
+def _fused_activation(op: int, x: HIPTensor, out: HIPTensor | None, p: float = 0.0) -> HIPTensor:
+    import ctypes as C
+    if out is None:
+        out = HIPTensor(x.shape, initial_element=None)
+    v = nodes.view2(x, out)
+    _lib.check(_lib.get().wf2hip_unary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(p)))
+    return out
+
+
+def relu_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
+    """!relu in one kernel; bit-identical to the two-node recipe."""
+    return _fused_activation(_lib.RELU, x, out)
+
+
+def sigmoid_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
+    """!sigmoid in one kernel; every step rounded as its node, hence bit-identical."""
+    return _fused_activation(_lib.SIGMOID, x, out)
+
+
+def leaky_relu_fused(x: HIPTensor, negative_slope: float = 0.01, out: HIPTensor | None = None) -> HIPTensor:
+    return _fused_activation(_lib.LEAKY_RELU, x, out, float(np.float32(negative_slope)))
+
+
 # ---------------------------------------------------------------------------
 # max / min / argmax / argmin (source/base-impl/matrix-ops.lisp:197-470)
 # ---------------------------------------------------------------------------

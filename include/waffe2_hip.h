@@ -188,7 +188,10 @@ enum wf2hip_unary_op {
   WF2HIP_LOG1P = 31,
   WF2HIP_POW = 32, /* ExptNode mathematics.lisp:267-303 */
   WF2HIP_INV = 33, /* 1 / x */
-  WF2HIP_GELU = 40 /* fused tanh-form GELU (nn/activation.lisp:45-66) */
+  WF2HIP_GELU = 40, /* fused tanh-form GELU (nn/activation.lisp:45-66) */
+  WF2HIP_RELU = 41, /* fused !relu = x * (x > 0 ? 1 : 0) (nn/activation.lisp:11-25), bit-identical to the two nodes */
+  WF2HIP_SIGMOID = 42, /* fused !sigmoid = 1 / (1 + exp(-1 x)) (nn/activation.lisp:27-43), each step rounded as its node */
+  WF2HIP_LEAKY_RELU = 43 /* fused !leaky-relu = x * (x >= 0 ? 1 : p) (nn/activation.lisp:68-92); p = negative slope */
 };
 
 /* a <- a op b over the view (a = X, the in-place destination; b = Y).
@@ -204,7 +207,8 @@ enum wf2hip_unary_op {
 int wf2hip_binary_nd(int op, const wf2hip_view2* v, float* a, const float* b);
 /* b <- f(a) over the view (a = X source, b = OUT).  Replaces the
  * define-math-impl forwards and ExptNode (source/backends/cpu/mathematics.lisp:
- * 8-76).  `p` is the exponent for WF2HIP_POW and ignored otherwise. */
+ * 8-76).  `p` is the exponent for WF2HIP_POW, the negative slope for
+ * WF2HIP_LEAKY_RELU and ignored otherwise. */
 int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, float p);
 
 /* ---- the other element types -------------------------------------------- */

@@ -260,3 +260,29 @@ def test_select_full_size(gpu):
     am = F.argmax(dx).numpy().ravel()
     assert np.array_equal(x[np.arange(8192), am], mx)
     assert np.array_equal(am, x.argmax(axis=1))
+
+
+def test_fused_activations_match_their_node_recipes(gpu):
+    """!relu, !leaky-relu and !sigmoid as single kernels against the node
+    sequences of nn/activation.lisp:11-92 run one node at a time: bit-identical
+    (the kernels perform the same binary32 operations in the same order), on
+    random data, special values and a strided view; sigmoid also within 2 ulp of
+    float64."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal(100003) * 4).astype(np.float32)
+    x[:16] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 88.0, -88.0, 104.0, -104.0, 1e30, -1e30, 1.0, -1.0, 20.0]
+    dx = F.from_numpy(x)
+    pairs = [(F.relu_fused, F.relu), (F.sigmoid_fused, F.sigmoid),
+             (lambda t: F.leaky_relu_fused(t, 0.2), lambda t: F.leaky_relu(t, 0.2))]
+    for view in (dx, F.reshape(F.from_numpy(x[:99840]), 312, 320).view((3, 300, 2), (5, 305, 3))):
+        for fused, recipe in pairs:
+            a, b = fused(view).numpy(), recipe(view).numpy()
+            nan = np.isnan(b)  # a NaN stays a NaN; its sign bit is not part of the contract
+            assert np.array_equal(np.isnan(a), nan)
+            np.testing.assert_array_equal(a[~nan].view(np.uint32), b[~nan].view(np.uint32))
+    s = F.sigmoid_fused(dx).numpy()[16:]
+    truth = (1.0 / (1.0 + np.exp(-x[16:].astype(np.float64)))).astype(np.float32)
+    assert np.abs(s.view(np.int32).astype(np.int64) - truth.view(np.int32).astype(np.int64)).max() <= 2
+    assert np.array_equal(F.relu_fused(dx).numpy()[16:], np.maximum(x[16:], 0.0))
