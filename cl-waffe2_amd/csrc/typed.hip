@@ -25,6 +25,8 @@
 // when both runs are contiguous (or y is one value), one element per lane with
 // four in flight otherwise.  A destination with incx = 0 accumulates in the
 // reference's order on one lane.
+#include <type_traits>
+
 #include "wf2_common.h"
 #include "wf2_view.h"
 
@@ -84,6 +86,34 @@ __device__ __forceinline__ T through_float(T v) {
 template <class T, int N>
 struct alignas(16) Pack { T v[N]; };
 
+// Four 8-bit or two 16-bit elements per 32-bit word, add / sub / mul modulo the
+// element width: the same bits as widening to int, operating and truncating
+// (signed or not), in a fraction of the instructions -- per-byte unpacking
+// holds the 8-bit kernels at 64 % of the HBM peak, these forms at the 32-bit rate.
+template <class T, int OP>
+constexpr bool kWordOp = kIsInt<T> && sizeof(T) < 4 && (OP == WF2HIP_ADD || OP == WF2HIP_SUB || OP == WF2HIP_MUL);
+
+template <int BYTES, int OP>
+__device__ __forceinline__ uint32_t apply_word(uint32_t a, uint32_t b) {
+  typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+  if constexpr (BYTES == 2) {
+    const us2 x = __builtin_bit_cast(us2, a), y = __builtin_bit_cast(us2, b);
+    if constexpr (OP == WF2HIP_ADD) return __builtin_bit_cast(uint32_t, (us2)(x + y));
+    if constexpr (OP == WF2HIP_SUB) return __builtin_bit_cast(uint32_t, (us2)(x - y));
+    return __builtin_bit_cast(uint32_t, (us2)(x * y));
+  } else {
+    constexpr uint32_t H = 0x80808080u;
+    if constexpr (OP == WF2HIP_ADD) return ((a & ~H) + (b & ~H)) ^ ((a ^ b) & H);
+    if constexpr (OP == WF2HIP_SUB) return ((a | H) - (b & ~H)) ^ ((a ^ ~b) & H);
+    // low bytes: the low byte of a 16-bit product depends on the low bytes only;
+    // high bytes: (a >> 8) * (b with its low byte cleared) = (ah * bh) << 8 modulo 2^16
+    const us2 x = __builtin_bit_cast(us2, a), y = __builtin_bit_cast(us2, b);
+    const us2 lo = (us2)(x * y) & (unsigned short)0x00ff;
+    const us2 hi = (us2)((us2)(x >> (unsigned short)8) * (us2)(y & (unsigned short)0xff00));
+    return __builtin_bit_cast(uint32_t, (us2)(lo | hi));
+  }
+}
+
 // contiguous x, y contiguous (or one value): 16 bytes per lane and access, four
 // accesses per lane issued before the first use, each wavefront on 4 KB of its
 // own per stream, nontemporal from 192 MiB of traffic on -- the shape measured
@@ -97,39 +127,69 @@ __global__ __launch_bounds__(kBlock) void typed_flat(T* __restrict__ x, const T*
   typedef float f4 __attribute__((ext_vector_type(4)));
   const unsigned wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + wave) * kWave * U + lane;
+  // the loaded vectors stay float4 values up to their use: converted to element
+  // arrays where they are loaded, the narrow types lose the nontemporal hint
   auto load = [](const T* p, size_t i) {
     const f4* q = reinterpret_cast<const f4*>(p) + i;
-    f4 raw = NT ? __builtin_nontemporal_load(q) : *q;
-    return __builtin_bit_cast(P, raw);
+    return NT ? __builtin_nontemporal_load(q) : *q;
   };
-  P a[U], b[U];
   T s = T(0);
   if (BCAST) s = y[0];
+  // Two shapes of one body.  Predicated per vector (FULL = false): a branch and a
+  // dozen instructions between the load pairs; that spacing measures best when the
+  // arithmetic is a few instructions (x <- x + y on 256 MiB per tensor: 122 us; with the
+  // eight loads back to back: 127 us).  Branch-free (FULL = true) for a wavefront whose
+  // 4 KB lie inside the run: the scheduler starts on each vector as it arrives, which
+  // hides the longer arithmetic of the 8- and 16-bit types (123 us against 131 us).
+  auto body = [&](auto full) {
+    constexpr bool FULL = decltype(full)::value;
+    f4 a[U], b[U];
 #pragma unroll
-  for (int u = 0; u < U; u++) {
-    const size_t i = base + (size_t)u * kWave;
-    if (i < nvec) {
-      if (OP != WF2HIP_MOVE) a[u] = load(x, i);
-      if (!BCAST) b[u] = load(y, i);
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < U; u++) {
-    const size_t i = base + (size_t)u * kWave;
-    if (i < nvec) {
-      P r;
-#pragma unroll
-      for (int k = 0; k < N; k++) {
-        const T yv = BCAST ? s : b[u].v[k];
-        r.v[k] = apply<T, OP>(OP != WF2HIP_MOVE ? a[u].v[k] : yv, yv);
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        if (OP != WF2HIP_MOVE) a[u] = load(x, i);
+        if (!BCAST) b[u] = load(y, i);
       }
-      f4* q = reinterpret_cast<f4*>(x) + i;
-      if (NT)
-        __builtin_nontemporal_store(__builtin_bit_cast(f4, r), q);
-      else
-        *q = __builtin_bit_cast(f4, r);
     }
-  }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        P r;
+        if constexpr (kWordOp<T, OP>) {
+          typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+          u4 aw = __builtin_bit_cast(u4, a[u]), bw, rw;
+          if (BCAST) {
+            uint32_t w = sizeof(T) == 1 ? (uint32_t)(uint8_t)s * 0x01010101u : (uint32_t)(uint16_t)s * 0x00010001u;
+            bw = (u4){w, w, w, w};
+          } else {
+            bw = __builtin_bit_cast(u4, b[u]);
+          }
+#pragma unroll
+          for (int k = 0; k < 4; k++) rw[k] = apply_word<(int)sizeof(T), OP>(aw[k], bw[k]);
+          r = __builtin_bit_cast(P, rw);
+        } else {
+          const P pa = __builtin_bit_cast(P, a[u]), pb = __builtin_bit_cast(P, b[u]);
+#pragma unroll
+          for (int k = 0; k < N; k++) {
+            const T yv = BCAST ? s : pb.v[k];
+            r.v[k] = apply<T, OP>(OP != WF2HIP_MOVE ? pa.v[k] : yv, yv);
+          }
+        }
+        f4* q = reinterpret_cast<f4*>(x) + i;
+        if (NT)
+          __builtin_nontemporal_store(__builtin_bit_cast(f4, r), q);
+        else
+          *q = __builtin_bit_cast(f4, r);
+      }
+    }
+  };
+  constexpr bool kBranchFree = kIsInt<T> && sizeof(T) < 4 && OP != WF2HIP_MOVE;
+  if (kBranchFree && base - lane + (size_t)kWave * U <= nvec)
+    body(std::true_type{});
+  else
+    body(std::false_type{});
 }
 
 // any increments (incx != 0): elements first..n-1; those from `exact_end` on go
