@@ -9,18 +9,11 @@
 // per element (two reads, one write).  The scalar right-hand side
 // (Where-Operation-Node) is an element-wise functor in elementwise.hip.
 #include "wf2_common.h"
+#include "wf2_view.h"
 
 namespace wf2 {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
-
-struct Space3 {
-  int rank = 0;
-  int64_t shape[WF2HIP_MAX_RANK];
-  int64_t sa[WF2HIP_MAX_RANK], sb[WF2HIP_MAX_RANK], sc[WF2HIP_MAX_RANK];
-  int64_t off_a = 0, off_b = 0, off_c = 0;
-  int64_t total = 0;
-};
 
 __device__ __forceinline__ bool holds(int op, float a, float b) {
   switch (op) {
@@ -109,67 +102,6 @@ __global__ __launch_bounds__(kBlock) void compare_generic(Cmp3Params p) {
   p.out[co] = holds(p.op, p.x[ao], p.y[bo]) ? p.then_value : p.else_value;
 }
 
-static void normalise3(Space3* s) {
-  int w = 0;
-  for (int r = 0; r < s->rank; r++) {
-    if (s->shape[r] == 1) continue;
-    s->shape[w] = s->shape[r];
-    s->sa[w] = s->sa[r];
-    s->sb[w] = s->sb[r];
-    s->sc[w] = s->sc[r];
-    w++;
-  }
-  if (w == 0) {
-    s->shape[0] = 1;
-    s->sa[0] = s->sb[0] = s->sc[0] = 0;
-    w = 1;
-  }
-  s->rank = w;
-  int out = 0;
-  for (int r = 1; r < s->rank; r++) {
-    const bool merge = s->sa[out] == s->sa[r] * s->shape[r] && s->sb[out] == s->sb[r] * s->shape[r] &&
-                       s->sc[out] == s->sc[r] * s->shape[r];
-    if (merge) {
-      s->shape[out] *= s->shape[r];
-    } else {
-      out++;
-      s->shape[out] = s->shape[r];
-    }
-    s->sa[out] = s->sa[r];
-    s->sb[out] = s->sb[r];
-    s->sc[out] = s->sc[r];
-  }
-  s->rank = out + 1;
-  s->total = 1;
-  for (int r = 0; r < s->rank; r++) s->total *= s->shape[r];
-}
-
-// lowest / highest element a strided window touches
-static void span_of(const Space3& s, const int64_t* stride, int64_t off, int64_t* lo, int64_t* hi) {
-  *lo = *hi = off;
-  for (int r = 0; r < s.rank; r++) {
-    const int64_t span = stride[r] * (s.shape[r] - 1);
-    if (span >= 0)
-      *hi += span;
-    else
-      *lo += span;
-  }
-}
-
-// `out` may coincide with an input element for element (in-place compare);
-// any other overlap makes the result depend on the order of the writes
-static bool hazardous(const Space3& s, const float* out, const int64_t* sin, int64_t off_in,
-                      const float* in) {
-  int64_t olo, ohi, ilo, ihi;
-  span_of(s, s.sc, s.off_c, &olo, &ohi);
-  span_of(s, sin, off_in, &ilo, &ihi);
-  if (out + ohi < in + ilo || in + ihi < out + olo) return false;
-  if (out + s.off_c != in + off_in) return true;
-  for (int r = 0; r < s.rank; r++)
-    if (s.sc[r] != sin[r]) return true;
-  return false;
-}
-
 int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, float then_value,
                float else_value) {
   if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
@@ -183,7 +115,7 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
       s.shape[r] = 1;
     }
   normalise3(&s);
-  if (hazardous(s, out, s.sa, s.off_a, x) || hazardous(s, out, s.sb, s.off_b, y))
+  if (hazardous3(s, out, s.sa, s.off_a, x) || hazardous3(s, out, s.sb, s.off_b, y))
     return fail(WF2HIP_EOVERLAP, "compare writes into a window that partially overlaps an input");
   hipStream_t st = rt().stream;
   const float* xp = x + s.off_a;
@@ -222,27 +154,6 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
   compare_generic<<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   return after_launch("compare_generic");
-}
-
-static int load_space3(const wf2hip_view3* v, Space3* s) {
-  if (!v) return fail(WF2HIP_EINVAL, "null view descriptor");
-  if (v->rank < 1 || v->rank > WF2HIP_MAX_RANK)
-    return fail(WF2HIP_EINVAL, "view rank %d outside 1..%d", v->rank, WF2HIP_MAX_RANK);
-  s->rank = v->rank;
-  s->total = 1;
-  for (int r = 0; r < v->rank; r++) {
-    if (v->shape[r] < 0) return fail(WF2HIP_EINVAL, "negative extent on axis %d", r);
-    s->shape[r] = v->shape[r];
-    s->sa[r] = v->stride_a[r];
-    s->sb[r] = v->stride_b[r];
-    s->sc[r] = v->stride_c[r];
-    s->total *= v->shape[r];
-  }
-  if (v->off_a < 0 || v->off_b < 0 || v->off_c < 0) return fail(WF2HIP_EINVAL, "negative offset");
-  s->off_a = v->off_a;
-  s->off_b = v->off_b;
-  s->off_c = v->off_c;
-  return 0;
 }
 
 }  // namespace wf2

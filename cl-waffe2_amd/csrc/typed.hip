@@ -417,6 +417,221 @@ static int dispatch_nd(int op, Space s, T* a, const T* b) {
   }
 }
 
+// ---- compare / where ----------------------------------------------------------
+// out <- (x OP y) ? then : else with all three of one element type
+// (cl-waffe2-simd.c:385-468 define_cmp, :474-560 define_scmp with a scalar y).
+// The reference's AVX2 body orders the lanes of the unsigned types as signed
+// integers (simd/x86_64/avx2.h:198-200, 211-213, 224-226, 237-239: _mm256_cmpgt_epi*
+// under the u32 / u16 / u8 names) while its scalar remainder compares them as
+// unsigned; `signed_end` is the number of leading elements the 1-D entry points
+// order that way to reproduce it.  The N-D entry points always compare in the
+// element type's own order.
+template <class T>
+constexpr T sign_bit_of() {
+  if constexpr (kIsInt<T>) {
+    if constexpr (!((T)(-1) < (T)0)) return (T)((T)1 << (sizeof(T) * 8 - 1));
+  }
+  return (T)0;
+}
+template <class T>
+constexpr T kSignBit = sign_bit_of<T>();
+
+template <class T>
+__device__ __forceinline__ bool holds_t(int op, T a, T b) {
+  switch (op) {
+    case WF2HIP_EQ: return a == b;
+    case WF2HIP_LT: return a < b;
+    case WF2HIP_LE: return a <= b;
+    case WF2HIP_GT: return a > b;
+    default: return a >= b;
+  }
+}
+
+// x XOR bias with bias = the sign bit turns the unsigned order into the signed one
+template <class T>
+__device__ __forceinline__ T biased(T v, T bias) {
+  if constexpr (kIsInt<T>)
+    return (T)(v ^ bias);
+  else
+    return v;
+}
+
+// x, (y,) out contiguous and 16-byte aligned: the layout of typed_flat
+template <class T, bool SCAL, bool NT>
+__global__ __launch_bounds__(kBlock) void typed_cmp_flat(const T* __restrict__ x, const T* __restrict__ y,
+                                                         T* __restrict__ out, size_t nvec, size_t signed_vecs, int op,
+                                                         T ys, T then_value, T else_value) {
+  constexpr int N = 16 / sizeof(T);
+  constexpr int U = 4;
+  using P = Pack<T, N>;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const unsigned wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + wave) * kWave * U + lane;
+  auto load = [](const T* p, size_t i) {
+    const f4* q = reinterpret_cast<const f4*>(p) + i;
+    return NT ? __builtin_nontemporal_load(q) : *q;
+  };
+  auto body = [&](auto full) {
+    constexpr bool FULL = decltype(full)::value;
+    f4 a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        a[u] = load(x, i);
+        if (!SCAL) b[u] = load(y, i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        const T bias = i < signed_vecs ? kSignBit<T> : (T)0;
+        const P pa = __builtin_bit_cast(P, a[u]), pb = __builtin_bit_cast(P, b[u]);
+        const T yb = biased(ys, bias);
+        P r;
+#pragma unroll
+        for (int k = 0; k < N; k++)
+          r.v[k] = holds_t<T>(op, biased(pa.v[k], bias), SCAL ? yb : biased(pb.v[k], bias)) ? then_value : else_value;
+        f4* q = reinterpret_cast<f4*>(out) + i;
+        if (NT)
+          __builtin_nontemporal_store(__builtin_bit_cast(f4, r), q);
+        else
+          *q = __builtin_bit_cast(f4, r);
+      }
+    }
+  };
+  constexpr bool kBranchFree = sizeof(T) < 4;
+  if (kBranchFree && base - lane + (size_t)kWave * U <= nvec)
+    body(std::true_type{});
+  else
+    body(std::false_type{});
+}
+
+template <class T>
+struct TypedCmp {
+  const T* x;
+  const T* y;
+  T* out;
+  int32_t rank, op;
+  int64_t total, signed_end;
+  int64_t shape[WF2HIP_MAX_RANK], sa[WF2HIP_MAX_RANK], sb[WF2HIP_MAX_RANK], sc[WF2HIP_MAX_RANK];
+  T ys, then_value, else_value;
+};
+
+// any strides, one element per thread, innermost axis fastest
+template <class T, bool SCAL>
+__global__ __launch_bounds__(kBlock) void typed_cmp_generic(TypedCmp<T> p) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= p.total) return;
+  int64_t rem = i, ao = 0, bo = 0, co = 0;
+  for (int r = p.rank - 1; r > 0; r--) {
+    const int64_t q = rem / p.shape[r];
+    const int64_t idx = rem - q * p.shape[r];
+    rem = q;
+    ao += idx * p.sa[r];
+    bo += idx * p.sb[r];
+    co += idx * p.sc[r];
+  }
+  ao += rem * p.sa[0];
+  bo += rem * p.sb[0];
+  co += rem * p.sc[0];
+  const T bias = i < p.signed_end ? kSignBit<T> : (T)0;
+  const T b = SCAL ? p.ys : p.y[bo];
+  p.out[co] = holds_t<T>(p.op, biased(p.x[ao], bias), biased(b, bias)) ? p.then_value : p.else_value;
+}
+
+// `signed_end` counts elements of the (rank-1) space in iteration order; 0 for N-D calls
+template <class T, bool SCAL>
+static int run_cmp(int op, Space3 s, const T* x, const T* y, T* out, T ys, T then_value, T else_value,
+                   int64_t signed_end) {
+  if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
+  if (s.total == 0) return 0;
+  if (!x || !out || (!SCAL && !y)) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  if (SCAL) {
+    y = x;
+    for (int r = 0; r < s.rank; r++) s.sb[r] = s.sa[r];
+    s.off_b = s.off_a;
+  }
+  // a stride-0 axis of `out` keeps what the sequential loop writes last (its scalar
+  // loop, which compares in the element type's own order)
+  for (int r = 0; r < s.rank; r++)
+    if (s.sc[r] == 0 && s.shape[r] > 1) {
+      s.off_a += s.sa[r] * (s.shape[r] - 1);
+      s.off_b += s.sb[r] * (s.shape[r] - 1);
+      s.shape[r] = 1;
+      signed_end = 0;
+    }
+  normalise3(&s);
+  if (hazardous3(s, out, s.sa, s.off_a, x) || hazardous3(s, out, s.sb, s.off_b, y))
+    return fail(WF2HIP_EOVERLAP, "compare writes into a window that partially overlaps an input");
+  hipStream_t st = rt().stream;
+  const T* xp = x + s.off_a;
+  const T* yp = y + s.off_b;
+  T* op_ = out + s.off_c;
+  constexpr int N = 16 / (int)sizeof(T);
+  int64_t done = 0;
+  const bool flat = s.rank == 1 && s.total >= N && s.sa[0] == 1 && s.sb[0] == 1 && s.sc[0] == 1 &&
+                    (((uintptr_t)xp | (uintptr_t)yp | (uintptr_t)op_) & 15u) == 0;
+  if (flat) {
+    const int64_t nvec = s.total / N;
+    const int64_t blocks = ceil_div(nvec, (int64_t)kBlock * 4);
+    if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+    const size_t signed_vecs = (size_t)(signed_end / N);  // a multiple of 2 N elements by construction
+    if (nvec * 16 * (SCAL ? 2 : 3) >= ((int64_t)192 << 20))
+      typed_cmp_flat<T, SCAL, true><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, yp, op_, (size_t)nvec, signed_vecs, op, ys,
+                                                                        then_value, else_value);
+    else
+      typed_cmp_flat<T, SCAL, false><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, yp, op_, (size_t)nvec, signed_vecs, op, ys,
+                                                                         then_value, else_value);
+    WF2_TRY(after_launch("typed_cmp_flat"));
+    done = nvec * N;
+    if (done == s.total) return 0;
+  }
+  TypedCmp<T> p;
+  p.rank = s.rank;
+  p.op = op;
+  for (int r = 0; r < s.rank; r++) {
+    p.shape[r] = s.shape[r];
+    p.sa[r] = s.sa[r];
+    p.sb[r] = s.sb[r];
+    p.sc[r] = s.sc[r];
+  }
+  // after the vector kernel only the tail of a rank-1 run is left
+  p.x = xp + done * s.sa[0];
+  p.y = yp + done * s.sb[0];
+  p.out = op_ + done * s.sc[0];
+  if (done > 0) p.shape[0] = s.total - done;
+  p.total = s.total - done;
+  p.signed_end = signed_end > done ? signed_end - done : 0;
+  p.ys = ys;
+  p.then_value = then_value;
+  p.else_value = else_value;
+  const int64_t blocks = ceil_div(p.total, kBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+  typed_cmp_generic<T, SCAL><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  return after_launch("typed_cmp_generic");
+}
+
+// the reference's 1-D kernels: the leading (n / lanes) * lanes elements go through
+// its 256-bit body when inco >= 1 (lanes = 32 bytes / element size)
+template <class T, bool SCAL>
+static int cmp_1d(int op, long n, const T* x, long incx, const T* y, long incy, T* out, long inco, T ys,
+                  T then_value, T else_value) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
+  Space3 s;
+  s.rank = 1;
+  s.shape[0] = n;
+  s.sa[0] = incx;
+  s.sb[0] = SCAL ? incx : incy;
+  s.sc[0] = inco;
+  s.total = n;
+  constexpr long lanes = 32 / (long)sizeof(T);
+  const int64_t signed_end = (kSignBit<T> != (T)0 && inco >= 1) ? (n / lanes) * lanes : 0;
+  return run_cmp<T, SCAL>(op, s, x, y, out, ys, then_value, else_value, signed_end);
+}
+
 }  // namespace wf2
 
 using namespace wf2;
@@ -492,3 +707,56 @@ WF2_TYPED_FAMILY(i16, int16_t, WF2HIP_I16)
 WF2_TYPED_FAMILY(u16, uint16_t, WF2HIP_U16)
 WF2_TYPED_FAMILY(i8, int8_t, WF2HIP_I8)
 WF2_TYPED_FAMILY(u8, uint8_t, WF2HIP_U8)
+
+WF2_API int wf2hip_compare_nd_typed(int dtype, int op, const wf2hip_view3* v, const void* x, const void* y, void* out,
+                                    double then_value, double else_value) {
+  WF2_TRY(require_init());
+  Space3 s;
+  WF2_TRY(load_space3(v, &s));
+  WF2_FOR_DTYPE(dtype, return (run_cmp<T, false>(op, s, (const T*)x, (const T*)y, (T*)out, (T)0, (T)then_value,
+                                                 (T)else_value, 0)));
+}
+
+WF2_API int wf2hip_where_nd_typed(int dtype, int op, const wf2hip_view2* v, const void* x, void* out, double scal,
+                                  double then_value, double else_value) {
+  WF2_TRY(require_init());
+  Space two;
+  WF2_TRY(load_space(v, &two));
+  Space3 s;
+  s.rank = two.rank;
+  s.total = two.total;
+  for (int r = 0; r < two.rank; r++) {
+    s.shape[r] = two.shape[r];
+    s.sa[r] = s.sb[r] = two.sa[r];
+    s.sc[r] = two.sb[r];
+  }
+  s.off_a = s.off_b = two.off_a;
+  s.off_c = two.off_b;
+  WF2_FOR_DTYPE(dtype, return (run_cmp<T, true>(op, s, (const T*)x, nullptr, (T*)out, (T)scal, (T)then_value,
+                                                (T)else_value, 0)));
+}
+
+// the reference's own names: waffe2_<prefix>{eq,lt,le,gt,ge} and ..._scal
+#define WF2_DEFINE_TYPED_CMP(prefix, T, name, OP)                                                                  \
+  WF2_API int wf2hip_##prefix##name(long n, const T* x, long incx, const T* y, long incy, T* out, long inco,      \
+                                    T then_value, T else_value) {                                                  \
+    return cmp_1d<T, false>(OP, n, x, incx, y, incy, out, inco, (T)0, then_value, else_value);                    \
+  }                                                                                                                \
+  WF2_API int wf2hip_##prefix##name##_scal(long n, const T* x, long incx, T* out, long inco, T y, T then_value,  \
+                                           T else_value) {                                                         \
+    return cmp_1d<T, true>(OP, n, x, incx, nullptr, 0, out, inco, y, then_value, else_value);                     \
+  }
+#define WF2_DEFINE_TYPED_CMPS(prefix, T)          \
+  WF2_DEFINE_TYPED_CMP(prefix, T, eq, WF2HIP_EQ)  \
+  WF2_DEFINE_TYPED_CMP(prefix, T, lt, WF2HIP_LT)  \
+  WF2_DEFINE_TYPED_CMP(prefix, T, le, WF2HIP_LE)  \
+  WF2_DEFINE_TYPED_CMP(prefix, T, gt, WF2HIP_GT)  \
+  WF2_DEFINE_TYPED_CMP(prefix, T, ge, WF2HIP_GE)
+
+WF2_DEFINE_TYPED_CMPS(d, double)
+WF2_DEFINE_TYPED_CMPS(i32, int32_t)
+WF2_DEFINE_TYPED_CMPS(u32, uint32_t)
+WF2_DEFINE_TYPED_CMPS(i16, int16_t)
+WF2_DEFINE_TYPED_CMPS(u16, uint16_t)
+WF2_DEFINE_TYPED_CMPS(i8, int8_t)
+WF2_DEFINE_TYPED_CMPS(u8, uint8_t)

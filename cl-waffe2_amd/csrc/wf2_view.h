@@ -134,4 +134,97 @@ inline bool has_broadcast_axis(const Space& s, const int64_t* stride) {
   return false;
 }
 
+
+// ---- three tensors over one iteration space (compare: a = X, b = Y, c = OUT) ----
+struct Space3 {
+  int rank = 0;
+  int64_t shape[WF2HIP_MAX_RANK];
+  int64_t sa[WF2HIP_MAX_RANK], sb[WF2HIP_MAX_RANK], sc[WF2HIP_MAX_RANK];
+  int64_t off_a = 0, off_b = 0, off_c = 0;
+  int64_t total = 0;
+};
+
+inline void normalise3(Space3* s) {
+  int w = 0;
+  for (int r = 0; r < s->rank; r++) {
+    if (s->shape[r] == 1) continue;
+    s->shape[w] = s->shape[r];
+    s->sa[w] = s->sa[r];
+    s->sb[w] = s->sb[r];
+    s->sc[w] = s->sc[r];
+    w++;
+  }
+  if (w == 0) {
+    s->shape[0] = 1;
+    s->sa[0] = s->sb[0] = s->sc[0] = 0;
+    w = 1;
+  }
+  s->rank = w;
+  int out = 0;
+  for (int r = 1; r < s->rank; r++) {
+    const bool merge = s->sa[out] == s->sa[r] * s->shape[r] && s->sb[out] == s->sb[r] * s->shape[r] &&
+                       s->sc[out] == s->sc[r] * s->shape[r];
+    if (merge) {
+      s->shape[out] *= s->shape[r];
+    } else {
+      out++;
+      s->shape[out] = s->shape[r];
+    }
+    s->sa[out] = s->sa[r];
+    s->sb[out] = s->sb[r];
+    s->sc[out] = s->sc[r];
+  }
+  s->rank = out + 1;
+  s->total = 1;
+  for (int r = 0; r < s->rank; r++) s->total *= s->shape[r];
+}
+
+// lowest / highest element a strided window touches
+inline void span_of(const Space3& s, const int64_t* stride, int64_t off, int64_t* lo, int64_t* hi) {
+  *lo = *hi = off;
+  for (int r = 0; r < s.rank; r++) {
+    const int64_t span = stride[r] * (s.shape[r] - 1);
+    if (span >= 0)
+      *hi += span;
+    else
+      *lo += span;
+  }
+}
+
+// `out` may coincide with an input element for element (in-place compare);
+// any other overlap makes the result depend on the order of the writes
+template <class T>
+inline bool hazardous3(const Space3& s, const T* out, const int64_t* sin, int64_t off_in, const T* in) {
+  int64_t olo, ohi, ilo, ihi;
+  span_of(s, s.sc, s.off_c, &olo, &ohi);
+  span_of(s, sin, off_in, &ilo, &ihi);
+  if (out + ohi < in + ilo || in + ihi < out + olo) return false;
+  if (out + s.off_c != in + off_in) return true;
+  for (int r = 0; r < s.rank; r++)
+    if (s.sc[r] != sin[r]) return true;
+  return false;
+}
+
+inline int load_space3(const wf2hip_view3* v, Space3* s) {
+  if (!v) return fail(WF2HIP_EINVAL, "null view descriptor");
+  if (v->rank < 1 || v->rank > WF2HIP_MAX_RANK)
+    return fail(WF2HIP_EINVAL, "view rank %d outside 1..%d", v->rank, WF2HIP_MAX_RANK);
+  s->rank = v->rank;
+  s->total = 1;
+  for (int r = 0; r < v->rank; r++) {
+    if (v->shape[r] < 0) return fail(WF2HIP_EINVAL, "negative extent on axis %d", r);
+    s->shape[r] = v->shape[r];
+    s->sa[r] = v->stride_a[r];
+    s->sb[r] = v->stride_b[r];
+    s->sc[r] = v->stride_c[r];
+    s->total *= v->shape[r];
+  }
+  if (v->off_a < 0 || v->off_b < 0 || v->off_c < 0) return fail(WF2HIP_EINVAL, "negative offset");
+  s->off_a = v->off_a;
+  s->off_b = v->off_b;
+  s->off_c = v->off_c;
+  return 0;
+}
+
+
 }  // namespace wf2

@@ -311,7 +311,7 @@ def where(x: HIPTensor, condition: str, scal: float, true_then: float = 1.0, fal
     predicates with a device kernel (``logical.lisp:65-110``): ``out_i`` is
     ``true_then`` where ``x_i condition scal`` holds, else ``false_then``."""
     if out is None:
-        out = HIPTensor(x.shape, initial_element=None)
+        out = HIPTensor(x.shape, initial_element=None, dtype=x.dtype)
     return nodes.forward("Where-Operation-Node", x, out, condition, float(scal), true_then, false_then)
 
 
@@ -319,7 +319,7 @@ def compare(x: HIPTensor, y: HIPTensor, condition: str, true_then: float = 1.0,
             false_then: float = 0.0, out: HIPTensor | None = None) -> HIPTensor:
     """``(!compare x y condition ...)`` (``logical.lisp:112-156``)."""
     if out is None:
-        out = HIPTensor(x.shape, initial_element=None)
+        out = HIPTensor(x.shape, initial_element=None, dtype=x.dtype)
     return nodes.forward("Compare-Operation-Node", x, y, out, condition, true_then, false_then)
 
 

@@ -194,6 +194,16 @@ for _prefix in ("d", "i32", "u32", "i16", "u16", "i8", "u8"):
         _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P, _L], C.c_int)
     _SIGNATURES[f"wf2hip_{_prefix}inv"] = ([_L, _P, _L], C.c_int)
 
+_SIGNATURES["wf2hip_compare_nd_typed"] = ([C.c_int, C.c_int, C.POINTER(View3), _P, _P, _P, C.c_double, C.c_double], C.c_int)
+_SIGNATURES["wf2hip_where_nd_typed"] = ([C.c_int, C.c_int, C.POINTER(View2), _P, _P, C.c_double, C.c_double, C.c_double],
+                                       C.c_int)
+# waffe2_<prefix>{eq,...} / ..._scal: the scalar and the two constants have the element type
+for _prefix, _ctype in (("d", C.c_double), ("i32", C.c_int32), ("u32", C.c_uint32), ("i16", C.c_int16),
+                        ("u16", C.c_uint16), ("i8", C.c_int8), ("u8", C.c_uint8)):
+    for _op in ("eq", "lt", "le", "gt", "ge"):
+        _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P, _L, _P, _L, _ctype, _ctype], C.c_int)
+        _SIGNATURES[f"wf2hip_{_prefix}{_op}_scal"] = ([_L, _P, _L, _P, _L, _ctype, _ctype, _ctype], C.c_int)
+
 EXPORTS = tuple(_SIGNATURES)
 
 _lib = None

@@ -74,6 +74,12 @@
 (defcfun "wf2hip_compare_nd" :int
   (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
   (then-value :float) (else-value :float))
+(defcfun "wf2hip_where_nd_typed" :int
+  (dtype :int) (op :int) (view (:pointer (:struct view2))) (x :pointer) (out :pointer)
+  (scal :double) (then-value :double) (else-value :double))
+(defcfun "wf2hip_compare_nd_typed" :int
+  (dtype :int) (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
+  (then-value :double) (else-value :double))
 (defcfun "wf2hip_sinv" :int (n :long) (x :pointer) (incx :long))
 ;; :double and the integer dtypes (waffe2_d*, waffe2_{i32,...}*, cl-waffe2-simd/api.lisp:63-124):
 ;; one entry point per shape of call, the element type as a code (dtype-info in tensor.lisp)

@@ -134,12 +134,20 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
                             (declare (ignore more))
                             (with-foreign-object (view '(:struct view2))
                               (fill-view2 view x out)
-                              (check (wf2hip-where-nd
-                                      (condition->op condition) view
-                                      (tensor-device-pointer x) (tensor-device-pointer out)
-                                      (coerce scal 'single-float)
-                                      (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
-                                      (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float)))))
+                              ;; every dtype, as the CPU impl (backends/cpu/logical.lisp:37-60)
+                              (if (eql (dtype x) :float)
+                                  (check (wf2hip-where-nd
+                                          (condition->op condition) view
+                                          (tensor-device-pointer x) (tensor-device-pointer out)
+                                          (coerce scal 'single-float)
+                                          (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
+                                          (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float)))
+                                  (check (wf2hip-where-nd-typed
+                                          (nth-value 2 (dtype-info (dtype x))) (condition->op condition) view
+                                          (tensor-device-pointer x) (tensor-device-pointer out)
+                                          (coerce scal 'double-float)
+                                          (coerce (cl-waffe2/base-impl::logical-true-then self) 'double-float)
+                                          (coerce (cl-waffe2/base-impl::logical-false-then self) 'double-float))))))
                           out))
 
 (defun fill-view3 (view x y out)
@@ -166,12 +174,20 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
                           (ensure-extension)
                           (with-foreign-object (view '(:struct view3))
                             (fill-view3 view x y out)
-                            (check (wf2hip-compare-nd
-                                    (condition->op (cl-waffe2/base-impl::logical-condition self)) view
-                                    (tensor-device-pointer x) (tensor-device-pointer y)
-                                    (tensor-device-pointer out)
-                                    (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
-                                    (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float))))
+                            (if (eql (dtype x) :float)
+                                (check (wf2hip-compare-nd
+                                        (condition->op (cl-waffe2/base-impl::logical-condition self)) view
+                                        (tensor-device-pointer x) (tensor-device-pointer y)
+                                        (tensor-device-pointer out)
+                                        (coerce (cl-waffe2/base-impl::logical-true-then self) 'single-float)
+                                        (coerce (cl-waffe2/base-impl::logical-false-then self) 'single-float)))
+                                (check (wf2hip-compare-nd-typed
+                                        (nth-value 2 (dtype-info (dtype x)))
+                                        (condition->op (cl-waffe2/base-impl::logical-condition self)) view
+                                        (tensor-device-pointer x) (tensor-device-pointer y)
+                                        (tensor-device-pointer out)
+                                        (coerce (cl-waffe2/base-impl::logical-true-then self) 'double-float)
+                                        (coerce (cl-waffe2/base-impl::logical-false-then self) 'double-float)))))
                           out))
 
 ;; A[~] OUT[out-size] -> OUT: largest / smallest value of every trailing run of A, or its index

@@ -178,15 +178,22 @@ def _condition(op) -> int:
     raise NodeNotFound(f"no HIPTensor kernel for condition {op!r} (supported: = < <= > >=)")
 
 
-@define_impl("Where-Operation-Node", HIPTensor, _only_float)
+@define_impl("Where-Operation-Node", HIPTensor)
 def _where(x: HIPTensor, out: HIPTensor, condition, scal: float, true_then: float = 1.0,
            false_then: float = 0.0) -> HIPTensor:
     """``out <- (x condition scal) ? true-then : false-then``
-    (``backends/cpu/logical.lisp:37-60``)."""
+    (``backends/cpu/logical.lisp:37-60``); x and out share one dtype."""
+    if x.dtype != out.dtype:
+        raise ValueError(f"dtype mismatch: {x.dtype} and {out.dtype}")
     v = view2(x, out)
-    _lib.check(_lib.get().wf2hip_where_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
-                                          C.c_void_p(out.ptr), float(scal), float(true_then),
-                                          float(false_then)))
+    if x.dtype == "float":
+        _lib.check(_lib.get().wf2hip_where_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
+                                              C.c_void_p(out.ptr), float(scal), float(true_then),
+                                              float(false_then)))
+    else:
+        _lib.check(_lib.get().wf2hip_where_nd_typed(_lib.DTYPE_CODES[x.dtype], _condition(condition), C.byref(v),
+                                                    C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(scal),
+                                                    float(true_then), float(false_then)))
     return out
 
 
@@ -207,15 +214,22 @@ def view3(a: HIPTensor, b: HIPTensor, c: HIPTensor) -> _lib.View3:
     return v
 
 
-@define_impl("Compare-Operation-Node", HIPTensor, _only_float)
+@define_impl("Compare-Operation-Node", HIPTensor)
 def _compare(x: HIPTensor, y: HIPTensor, out: HIPTensor, condition, true_then: float = 1.0,
              false_then: float = 0.0) -> HIPTensor:
     """``out <- (x condition y) ? true-then : false-then``
-    (``backends/cpu/logical.lisp:62-84``)."""
+    (``backends/cpu/logical.lisp:62-84``); all three share one dtype."""
+    if not (x.dtype == y.dtype == out.dtype):
+        raise ValueError(f"dtype mismatch: {x.dtype}, {y.dtype} and {out.dtype}")
     v = view3(x, y, out)
-    _lib.check(_lib.get().wf2hip_compare_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
-                                            C.c_void_p(y.ptr), C.c_void_p(out.ptr),
-                                            float(true_then), float(false_then)))
+    if x.dtype == "float":
+        _lib.check(_lib.get().wf2hip_compare_nd(_condition(condition), C.byref(v), C.c_void_p(x.ptr),
+                                                C.c_void_p(y.ptr), C.c_void_p(out.ptr),
+                                                float(true_then), float(false_then)))
+    else:
+        _lib.check(_lib.get().wf2hip_compare_nd_typed(_lib.DTYPE_CODES[x.dtype], _condition(condition), C.byref(v),
+                                                      C.c_void_p(x.ptr), C.c_void_p(y.ptr), C.c_void_p(out.ptr),
+                                                      float(true_then), float(false_then)))
     return out
 
 

@@ -340,6 +340,164 @@ int wf2hip_where_nd(int op, const wf2hip_view2* v, const float* x, float* out, f
 int wf2hip_compare_nd(int op, const wf2hip_view3* v, const float* x, const float* y, float* out,
                       float then_value, float else_value);
 
+/* Compare-Operation-Node / Where-Operation-Node on the other element types: x, y,
+ * out, the scalar and the two constants all have the element type `dtype`
+ * (enum wf2hip_dtype).  Replace waffe2_{d,i32,i16,i8,u32,u16,u8}{eq,lt,le,gt,ge}
+ * (cl-waffe2-simd.c:385-468) and ..._scal (:474-560), which the CPU backend calls
+ * for every dtype (source/backends/cpu/logical.lisp:26-84).  The N-D forms take
+ * the constants as double (exact for every element type here) and compare in the
+ * element type's own order.  The 1-D names keep the reference's argument order
+ * and its results bit for bit, including this: its 256-bit body orders :uint32 /
+ * :uint16 / :uint8 lanes as SIGNED integers (simd/x86_64/avx2.h:198-239 bind the
+ * unsigned names to _mm256_cmpgt_epi*), so with inco >= 1 the leading
+ * (n / lanes) * lanes elements of a call (lanes = 32 bytes / element size) compare
+ * that way and only the remainder as unsigned; with inco < 1 every element takes
+ * the scalar loop. */
+int wf2hip_compare_nd_typed(int dtype, int op, const wf2hip_view3* v, const void* x, const void* y, void* out,
+                            double then_value, double else_value);
+int wf2hip_where_nd_typed(int dtype, int op, const wf2hip_view2* v, const void* x, void* out, double scal,
+                          double then_value, double else_value);
+int wf2hip_deq(long n, const double* x, long incx, const double* y, long incy, double* out, long inco,
+               double then_value, double else_value);
+int wf2hip_dlt(long n, const double* x, long incx, const double* y, long incy, double* out, long inco,
+               double then_value, double else_value);
+int wf2hip_dle(long n, const double* x, long incx, const double* y, long incy, double* out, long inco,
+               double then_value, double else_value);
+int wf2hip_dgt(long n, const double* x, long incx, const double* y, long incy, double* out, long inco,
+               double then_value, double else_value);
+int wf2hip_dge(long n, const double* x, long incx, const double* y, long incy, double* out, long inco,
+               double then_value, double else_value);
+int wf2hip_deq_scal(long n, const double* x, long incx, double* out, long inco, double y,
+                    double then_value, double else_value);
+int wf2hip_dlt_scal(long n, const double* x, long incx, double* out, long inco, double y,
+                    double then_value, double else_value);
+int wf2hip_dle_scal(long n, const double* x, long incx, double* out, long inco, double y,
+                    double then_value, double else_value);
+int wf2hip_dgt_scal(long n, const double* x, long incx, double* out, long inco, double y,
+                    double then_value, double else_value);
+int wf2hip_dge_scal(long n, const double* x, long incx, double* out, long inco, double y,
+                    double then_value, double else_value);
+int wf2hip_i32eq(long n, const int32_t* x, long incx, const int32_t* y, long incy, int32_t* out, long inco,
+               int32_t then_value, int32_t else_value);
+int wf2hip_i32lt(long n, const int32_t* x, long incx, const int32_t* y, long incy, int32_t* out, long inco,
+               int32_t then_value, int32_t else_value);
+int wf2hip_i32le(long n, const int32_t* x, long incx, const int32_t* y, long incy, int32_t* out, long inco,
+               int32_t then_value, int32_t else_value);
+int wf2hip_i32gt(long n, const int32_t* x, long incx, const int32_t* y, long incy, int32_t* out, long inco,
+               int32_t then_value, int32_t else_value);
+int wf2hip_i32ge(long n, const int32_t* x, long incx, const int32_t* y, long incy, int32_t* out, long inco,
+               int32_t then_value, int32_t else_value);
+int wf2hip_i32eq_scal(long n, const int32_t* x, long incx, int32_t* out, long inco, int32_t y,
+                    int32_t then_value, int32_t else_value);
+int wf2hip_i32lt_scal(long n, const int32_t* x, long incx, int32_t* out, long inco, int32_t y,
+                    int32_t then_value, int32_t else_value);
+int wf2hip_i32le_scal(long n, const int32_t* x, long incx, int32_t* out, long inco, int32_t y,
+                    int32_t then_value, int32_t else_value);
+int wf2hip_i32gt_scal(long n, const int32_t* x, long incx, int32_t* out, long inco, int32_t y,
+                    int32_t then_value, int32_t else_value);
+int wf2hip_i32ge_scal(long n, const int32_t* x, long incx, int32_t* out, long inco, int32_t y,
+                    int32_t then_value, int32_t else_value);
+int wf2hip_u32eq(long n, const uint32_t* x, long incx, const uint32_t* y, long incy, uint32_t* out, long inco,
+               uint32_t then_value, uint32_t else_value);
+int wf2hip_u32lt(long n, const uint32_t* x, long incx, const uint32_t* y, long incy, uint32_t* out, long inco,
+               uint32_t then_value, uint32_t else_value);
+int wf2hip_u32le(long n, const uint32_t* x, long incx, const uint32_t* y, long incy, uint32_t* out, long inco,
+               uint32_t then_value, uint32_t else_value);
+int wf2hip_u32gt(long n, const uint32_t* x, long incx, const uint32_t* y, long incy, uint32_t* out, long inco,
+               uint32_t then_value, uint32_t else_value);
+int wf2hip_u32ge(long n, const uint32_t* x, long incx, const uint32_t* y, long incy, uint32_t* out, long inco,
+               uint32_t then_value, uint32_t else_value);
+int wf2hip_u32eq_scal(long n, const uint32_t* x, long incx, uint32_t* out, long inco, uint32_t y,
+                    uint32_t then_value, uint32_t else_value);
+int wf2hip_u32lt_scal(long n, const uint32_t* x, long incx, uint32_t* out, long inco, uint32_t y,
+                    uint32_t then_value, uint32_t else_value);
+int wf2hip_u32le_scal(long n, const uint32_t* x, long incx, uint32_t* out, long inco, uint32_t y,
+                    uint32_t then_value, uint32_t else_value);
+int wf2hip_u32gt_scal(long n, const uint32_t* x, long incx, uint32_t* out, long inco, uint32_t y,
+                    uint32_t then_value, uint32_t else_value);
+int wf2hip_u32ge_scal(long n, const uint32_t* x, long incx, uint32_t* out, long inco, uint32_t y,
+                    uint32_t then_value, uint32_t else_value);
+int wf2hip_i16eq(long n, const int16_t* x, long incx, const int16_t* y, long incy, int16_t* out, long inco,
+               int16_t then_value, int16_t else_value);
+int wf2hip_i16lt(long n, const int16_t* x, long incx, const int16_t* y, long incy, int16_t* out, long inco,
+               int16_t then_value, int16_t else_value);
+int wf2hip_i16le(long n, const int16_t* x, long incx, const int16_t* y, long incy, int16_t* out, long inco,
+               int16_t then_value, int16_t else_value);
+int wf2hip_i16gt(long n, const int16_t* x, long incx, const int16_t* y, long incy, int16_t* out, long inco,
+               int16_t then_value, int16_t else_value);
+int wf2hip_i16ge(long n, const int16_t* x, long incx, const int16_t* y, long incy, int16_t* out, long inco,
+               int16_t then_value, int16_t else_value);
+int wf2hip_i16eq_scal(long n, const int16_t* x, long incx, int16_t* out, long inco, int16_t y,
+                    int16_t then_value, int16_t else_value);
+int wf2hip_i16lt_scal(long n, const int16_t* x, long incx, int16_t* out, long inco, int16_t y,
+                    int16_t then_value, int16_t else_value);
+int wf2hip_i16le_scal(long n, const int16_t* x, long incx, int16_t* out, long inco, int16_t y,
+                    int16_t then_value, int16_t else_value);
+int wf2hip_i16gt_scal(long n, const int16_t* x, long incx, int16_t* out, long inco, int16_t y,
+                    int16_t then_value, int16_t else_value);
+int wf2hip_i16ge_scal(long n, const int16_t* x, long incx, int16_t* out, long inco, int16_t y,
+                    int16_t then_value, int16_t else_value);
+int wf2hip_u16eq(long n, const uint16_t* x, long incx, const uint16_t* y, long incy, uint16_t* out, long inco,
+               uint16_t then_value, uint16_t else_value);
+int wf2hip_u16lt(long n, const uint16_t* x, long incx, const uint16_t* y, long incy, uint16_t* out, long inco,
+               uint16_t then_value, uint16_t else_value);
+int wf2hip_u16le(long n, const uint16_t* x, long incx, const uint16_t* y, long incy, uint16_t* out, long inco,
+               uint16_t then_value, uint16_t else_value);
+int wf2hip_u16gt(long n, const uint16_t* x, long incx, const uint16_t* y, long incy, uint16_t* out, long inco,
+               uint16_t then_value, uint16_t else_value);
+int wf2hip_u16ge(long n, const uint16_t* x, long incx, const uint16_t* y, long incy, uint16_t* out, long inco,
+               uint16_t then_value, uint16_t else_value);
+int wf2hip_u16eq_scal(long n, const uint16_t* x, long incx, uint16_t* out, long inco, uint16_t y,
+                    uint16_t then_value, uint16_t else_value);
+int wf2hip_u16lt_scal(long n, const uint16_t* x, long incx, uint16_t* out, long inco, uint16_t y,
+                    uint16_t then_value, uint16_t else_value);
+int wf2hip_u16le_scal(long n, const uint16_t* x, long incx, uint16_t* out, long inco, uint16_t y,
+                    uint16_t then_value, uint16_t else_value);
+int wf2hip_u16gt_scal(long n, const uint16_t* x, long incx, uint16_t* out, long inco, uint16_t y,
+                    uint16_t then_value, uint16_t else_value);
+int wf2hip_u16ge_scal(long n, const uint16_t* x, long incx, uint16_t* out, long inco, uint16_t y,
+                    uint16_t then_value, uint16_t else_value);
+int wf2hip_i8eq(long n, const int8_t* x, long incx, const int8_t* y, long incy, int8_t* out, long inco,
+               int8_t then_value, int8_t else_value);
+int wf2hip_i8lt(long n, const int8_t* x, long incx, const int8_t* y, long incy, int8_t* out, long inco,
+               int8_t then_value, int8_t else_value);
+int wf2hip_i8le(long n, const int8_t* x, long incx, const int8_t* y, long incy, int8_t* out, long inco,
+               int8_t then_value, int8_t else_value);
+int wf2hip_i8gt(long n, const int8_t* x, long incx, const int8_t* y, long incy, int8_t* out, long inco,
+               int8_t then_value, int8_t else_value);
+int wf2hip_i8ge(long n, const int8_t* x, long incx, const int8_t* y, long incy, int8_t* out, long inco,
+               int8_t then_value, int8_t else_value);
+int wf2hip_i8eq_scal(long n, const int8_t* x, long incx, int8_t* out, long inco, int8_t y,
+                    int8_t then_value, int8_t else_value);
+int wf2hip_i8lt_scal(long n, const int8_t* x, long incx, int8_t* out, long inco, int8_t y,
+                    int8_t then_value, int8_t else_value);
+int wf2hip_i8le_scal(long n, const int8_t* x, long incx, int8_t* out, long inco, int8_t y,
+                    int8_t then_value, int8_t else_value);
+int wf2hip_i8gt_scal(long n, const int8_t* x, long incx, int8_t* out, long inco, int8_t y,
+                    int8_t then_value, int8_t else_value);
+int wf2hip_i8ge_scal(long n, const int8_t* x, long incx, int8_t* out, long inco, int8_t y,
+                    int8_t then_value, int8_t else_value);
+int wf2hip_u8eq(long n, const uint8_t* x, long incx, const uint8_t* y, long incy, uint8_t* out, long inco,
+               uint8_t then_value, uint8_t else_value);
+int wf2hip_u8lt(long n, const uint8_t* x, long incx, const uint8_t* y, long incy, uint8_t* out, long inco,
+               uint8_t then_value, uint8_t else_value);
+int wf2hip_u8le(long n, const uint8_t* x, long incx, const uint8_t* y, long incy, uint8_t* out, long inco,
+               uint8_t then_value, uint8_t else_value);
+int wf2hip_u8gt(long n, const uint8_t* x, long incx, const uint8_t* y, long incy, uint8_t* out, long inco,
+               uint8_t then_value, uint8_t else_value);
+int wf2hip_u8ge(long n, const uint8_t* x, long incx, const uint8_t* y, long incy, uint8_t* out, long inco,
+               uint8_t then_value, uint8_t else_value);
+int wf2hip_u8eq_scal(long n, const uint8_t* x, long incx, uint8_t* out, long inco, uint8_t y,
+                    uint8_t then_value, uint8_t else_value);
+int wf2hip_u8lt_scal(long n, const uint8_t* x, long incx, uint8_t* out, long inco, uint8_t y,
+                    uint8_t then_value, uint8_t else_value);
+int wf2hip_u8le_scal(long n, const uint8_t* x, long incx, uint8_t* out, long inco, uint8_t y,
+                    uint8_t then_value, uint8_t else_value);
+int wf2hip_u8gt_scal(long n, const uint8_t* x, long incx, uint8_t* out, long inco, uint8_t y,
+                    uint8_t then_value, uint8_t else_value);
+int wf2hip_u8ge_scal(long n, const uint8_t* x, long incx, uint8_t* out, long inco, uint8_t y,
+                    uint8_t then_value, uint8_t else_value);
+
 /* 0 (default): parallel tree reduction for accumulate-into-stride-0 ADD.
  * 1: the reference's strictly sequential fp32 order (slow; for bit parity). */
 int wf2hip_set_reduce_mode(int mode);

@@ -431,3 +431,40 @@ def inv_typed_1d(dtype: str, n: int, x: np.ndarray, incx: int, use_ref: bool = F
     fn.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_long]
     fn.restype = C.c_int
     assert fn(code, n, px, incx) == 0
+
+
+_CTYPES = {"double": C.c_double, "int32": C.c_int32, "uint32": C.c_uint32, "int16": C.c_int16,
+           "uint16": C.c_uint16, "int8": C.c_int8, "uint8": C.c_uint8}
+
+
+def cmp_typed_1d(dtype: str, op: str, n: int, x: np.ndarray, incx: int, y, incy: int, out: np.ndarray, inco: int,
+                 then=1, els=0, use_ref: bool = False, offx: int = 0, offy: int = 0, offo: int = 0) -> None:
+    """out <- (x OP y) ? then : els for one element type, ``y`` an array
+    (waffe2_<prefix><op>) or a number (waffe2_<prefix><op>_scal), through the
+    oracle's restatement or (use_ref) the compiled reference."""
+    code, npt, prefix = DTYPES[dtype]
+    scal = not isinstance(y, np.ndarray)
+    assert x.dtype == npt and out.dtype == npt and (scal or y.dtype == npt)
+    size = x.itemsize
+    px = C.c_void_p(x.ctypes.data + size * offx)
+    po = C.c_void_p(out.ctypes.data + size * offo)
+    py = None if scal else C.c_void_p(y.ctypes.data + size * offy)
+    ct = _CTYPES[dtype]
+    if use_ref:
+        if scal:
+            fn = getattr(ref(), f"waffe2_{prefix}{op}_scal")
+            fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, ct, ct, ct]
+            fn.restype = None
+            fn(n, px, incx, po, inco, ct(y), ct(then), ct(els))
+        else:
+            fn = getattr(ref(), f"waffe2_{prefix}{op}")
+            fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, ct, ct]
+            fn.restype = None
+            fn(n, px, incx, py, incy, po, inco, ct(then), ct(els))
+        return
+    fn = lib().orc_cmp_typed
+    fn.argtypes = [C.c_int, C.c_int, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long,
+                   C.c_int, C.c_double, C.c_double, C.c_double]
+    fn.restype = C.c_int
+    assert fn(code, CMP_OPS.index(op), n, px, incx, py, 0 if scal else incy, po, inco, int(scal),
+              float(y) if scal else 0.0, float(then), float(els)) == 0

@@ -37,6 +37,10 @@
  *   orc_binary_typed, orc_inv_typed    : golden vectors from the compiled
  *       reference C (waffe2_d*, waffe2_{i32,...}*), numpy closed forms (integer
  *       wrap-around, binary64 arithmetic, the binary32 round trip of the tail).
+ *   orc_cmp_typed                      : golden vectors from the compiled
+ *       reference C (waffe2_{d,i32,...}{eq,...} and ..._scal), numpy closed forms
+ *       (the element type's own order on the remainder, the signed order on the
+ *       leading blocks of the unsigned types).
  *   orc_sgemm                          : the reference's integer gemm vectors
  *       (base-impl/t/arithmetic.lisp:120,135,142,148), float64 truth.
  */
@@ -782,6 +786,58 @@ ORC_API int orc_inv_typed(int dtype, long n, void *x, long incx) {
     default: return -1;
   }
 #undef ORC_INV
+}
+
+/* waffe2_{d,i32,i16,i8,u32,u16,u8}{eq,lt,le,gt,ge} and ..._scal
+ * (cl-waffe2-simd.c:385-468 define_cmp, :474-560 define_scmp): the block part
+ * (inco >= 1, blocks of 32 bytes / element size) compares through the AVX2 lane
+ * predicates, the remainder through the C operators.  For the unsigned types the
+ * lane predicates are the SIGNED ones (simd/x86_64/avx2.h:198-200 lt, :211-213 gt,
+ * :224-226 le = not gt, :237-239 ge = not gt swapped, all on _mm256_cmpgt_epi*);
+ * eq is sign-agnostic.  `scal` != 0 selects the scalar right-hand side `ys`. */
+#define ORC_CMPV(op, a, b) \
+  ((op) == ORC_EQ ? (a) == (b) : (op) == ORC_LT ? (a) < (b) : (op) == ORC_LE ? (a) <= (b) : (op) == ORC_GT ? (a) > (b) : (a) >= (b))
+
+#define ORC_CMP_LOOP(T, S)                                                                     \
+  {                                                                                            \
+    const T *xp = (const T *)x, *yp = (const T *)y;                                            \
+    T *outp = (T *)out;                                                                        \
+    const T tv = (T)then_value, ev = (T)else_value, yv = (T)ys;                                \
+    const long lanes = 32 / (long)sizeof(T);                                                   \
+    long count = 0;                                                                            \
+    if (inco >= 1) {                                                                           \
+      const long blocks_end = (n / lanes) * lanes;                                             \
+      for (; count != blocks_end; count += lanes) {                                            \
+        T res[32];                                                                             \
+        for (long l = 0; l < lanes; l++) {                                                     \
+          const S a = (S)xp[(count + l) * incx];                                               \
+          const S b = (S)(scal ? yv : yp[(count + l) * incy]);                                 \
+          res[l] = ORC_CMPV(op, a, b) ? tv : ev;                                               \
+        }                                                                                      \
+        for (long l = 0; l < lanes; l++) outp[(count + l) * inco] = res[l];                    \
+      }                                                                                        \
+    }                                                                                          \
+    for (; count != n; count++) {                                                              \
+      const T a = xp[count * incx];                                                            \
+      const T b = scal ? yv : yp[count * incy];                                                \
+      outp[count * inco] = ORC_CMPV(op, a, b) ? tv : ev;                                       \
+    }                                                                                          \
+    return 0;                                                                                  \
+  }
+
+ORC_API int orc_cmp_typed(int dtype, int op, long n, const void *x, long incx, const void *y, long incy, void *out,
+                          long inco, int scal, double ys, double then_value, double else_value) {
+  if (op < ORC_EQ || op > ORC_GE) return -1;
+  switch (dtype) {
+    case 1: ORC_CMP_LOOP(double, double)
+    case 2: ORC_CMP_LOOP(int32_t, int32_t)
+    case 3: ORC_CMP_LOOP(uint32_t, int32_t)
+    case 4: ORC_CMP_LOOP(int16_t, int16_t)
+    case 5: ORC_CMP_LOOP(uint16_t, int16_t)
+    case 6: ORC_CMP_LOOP(int8_t, int8_t)
+    case 7: ORC_CMP_LOOP(uint8_t, int8_t)
+    default: return -1;
+  }
 }
 
 ORC_API int orc_abi_version(void) { return 1; }

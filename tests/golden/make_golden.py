@@ -264,6 +264,83 @@ def typed_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_kernels.npz")), "bytes")
 
 
+# (n, incx, incy, inco); lanes = 32 bytes / element size
+CMP_TYPED_REGIMES = [(1, 1, 1, 1), (5, 1, 1, 1), (40, 1, 1, 1), (70, 1, 1, 1), (13, 2, 1, 1), (37, 1, 3, 2),
+                     (40, 1, 1, 0), (33, 2, 3, 0), (9, 3, 2, 1), (70, 1, 0, 1)]
+
+
+def _cmp_case_defined(dtype, n, incx, incy, inco, scal):
+    """The reference builds strided integer lanes by indexing a 4-lane vector up to
+    lane 31 (cl-waffe2-simd.c:54-107, 119-141): undefined unless the block part is
+    skipped (inco < 1, n < lanes) or every increment is 1."""
+    if dtype == "double":
+        return True
+    lanes = 32 // np.dtype(O.DTYPES[dtype][1]).itemsize
+    return inco < 1 or n < lanes or (incx == 1 and inco == 1 and (scal or incy == 1))
+
+
+def _cmp_child(dtype, op, n, x, incx, y, incy, out, inco, then, els, conn):
+    O.cmp_typed_1d(dtype, op, n, x, incx, y, incy, out, inco, then, els, use_ref=True)
+    conn.send(out)
+
+
+def compare_typed_goldens():
+    """waffe2_<prefix>{eq,lt,le,gt,ge} and ..._scal of the compiled reference for
+    :double and the integer types.  Each case runs in a child process: the compiled
+    reference faults or spins on some cases its source leaves undefined; those and
+    the undefined ones are left out and counted in `<dtype>_skipped`."""
+    import multiprocessing as mp
+    assert O.ref() is not None, "oracle/_ref/libwaffe2_simd_ref.so is missing: run `make -C oracle ref`"
+    ctx = mp.get_context("fork")
+    rng = np.random.Generator(np.random.PCG64(2029))
+    out = {}
+    for dtype, (code, npt, prefix) in O.DTYPES.items():
+        xs, ys, outs, cases, start, skipped = [], [], [], [], 0, 0
+        for op_index, op in enumerate(O.CMP_OPS):
+            for n, incx, incy, inco in CMP_TYPED_REGIMES:
+                for scal in (0, 1):
+                    if not _cmp_case_defined(dtype, n, incx, incy, inco, scal):
+                        skipped += 1
+                        continue
+                    size = n * 3 + 1
+                    if dtype == "double":
+                        x = rng.integers(-3, 4, size).astype(npt)
+                        y = rng.integers(-3, 4, size).astype(npt)
+                        x[rng.random(size) < 0.1] = np.nan
+                        y[rng.random(size) < 0.05] = np.inf
+                        then, els = 1.5, -0.25
+                    else:
+                        info = np.iinfo(npt)
+                        pool = np.array([info.min, info.max, 0, 1, 2, info.max // 2, info.max // 2 + 1], np.int64)
+                        x = rng.choice(pool, size).astype(npt)
+                        y = rng.choice(pool, size).astype(npt)
+                        then, els = 3, 5
+                    res = np.full(size, 7, npt)
+                    yy = y[0].item() if scal else y
+                    parent, child = ctx.Pipe(duplex=False)
+                    proc = ctx.Process(target=_cmp_child, args=(dtype, op, n, x, incx, yy, incy, res, inco, then, els, child))
+                    proc.start()
+                    got = parent.recv() if parent.poll(3) else None
+                    proc.join(1)
+                    if proc.is_alive():
+                        proc.kill()
+                        proc.join()
+                    if got is None:
+                        skipped += 1
+                        continue
+                    xs.append(x), ys.append(y), outs.append(got)
+                    cases.append((op_index, n, incx, incy, inco, scal, start, size))
+                    start += size
+        key = f"{dtype}_cmp"
+        if cases:
+            out[key + "_x"], out[key + "_y"], out[key + "_out"] = (np.concatenate(v) for v in (xs, ys, outs))
+        out[key + "_cases"] = np.array(cases, np.int64).reshape(-1, 8)
+        out[key + "_skipped"] = np.array([skipped], np.int64)
+        print(dtype, "cases", len(cases), "skipped", skipped, flush=True)
+    np.savez_compressed(os.path.join(HERE, "typed_compare_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_compare_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
     if "--im2col-only" in sys.argv:
         im2col_goldens()
@@ -273,9 +350,12 @@ if __name__ == "__main__":
         unary_more_goldens()
     elif "--typed-only" in sys.argv:
         typed_goldens()
+    elif "--typed-compare-only" in sys.argv:
+        compare_typed_goldens()
     else:
         main()
         compare_goldens()
         unary_more_goldens()
         im2col_goldens()
         typed_goldens()
+        compare_typed_goldens()
