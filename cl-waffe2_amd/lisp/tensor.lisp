@@ -109,18 +109,30 @@ source/backends/cpu/tensor.lisp:32-40)."
 ;; Bulk transfers.  The generic convert-tensor-facet path copies element by element through
 ;; vref (source/array-converter.lisp:154-197), which is unusable across PCIe; these methods move
 ;; the whole storage in one copy.
+(defun dtype-lisp-type (dtype)
+  "Element type of the host vector that mirrors a tensor of DTYPE (dtype->lisp-type,
+source/vm/generic-tensor/dtype.lisp)."
+  (ecase dtype
+    (:float 'single-float) (:double 'double-float)
+    (:int32 '(signed-byte 32)) (:uint32 '(unsigned-byte 32))
+    (:int16 '(signed-byte 16)) (:uint16 '(unsigned-byte 16))
+    (:int8 '(signed-byte 8)) (:uint8 '(unsigned-byte 8))))
+
 (defmethod cl-waffe2:convert-tensor-facet ((from HIPTensor) (to (eql 'simple-array)))
-  (let* ((n (floor (device-buffer-bytes (tensor-vec from)) 4))
-         (host (make-array n :element-type 'single-float)))
+  (let* ((size (dtype-bytes (dtype from)))
+         (n (floor (device-buffer-bytes (tensor-vec from)) size))
+         (host (make-array n :element-type (dtype-lisp-type (dtype from)))))
     (with-pointer-to-vector-data (p host)
-      (check (wf2hip-memcpy-d2h p (tensor-device-pointer from) (* 4 n))))
+      (check (wf2hip-memcpy-d2h p (tensor-device-pointer from) (* size n))))
     host))
 
-(defun upload (array)
-  "A fresh contiguous HIPTensor holding the contents of a (simple-array single-float)."
-  (let* ((flat (make-array (array-total-size array) :element-type 'single-float :displaced-to array))
-         (storage (coerce flat '(simple-array single-float (*))))
-         (tensor (make-tensor (array-dimensions array) :dtype :float :device 'HIPTensor)))
+(defun upload (array &key (dtype :float))
+  "A fresh contiguous HIPTensor of DTYPE holding the contents of ARRAY, a specialised array whose
+element type is DTYPE's host type (single-float for :float, (unsigned-byte 8) for :uint8 ...)."
+  (let* ((type (dtype-lisp-type dtype))
+         (flat (make-array (array-total-size array) :element-type type :displaced-to array))
+         (storage (coerce flat `(simple-array ,type (*))))
+         (tensor (make-tensor (array-dimensions array) :dtype dtype :device 'HIPTensor)))
     (with-pointer-to-vector-data (p storage)
-      (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor) p (* 4 (length storage)))))
+      (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor) p (* (dtype-bytes dtype) (length storage)))))
     tensor))
