@@ -19,24 +19,44 @@
 
 namespace wf2 {
 
-typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr int kSelMaxOuter = WF2HIP_MAX_RANK;
 
+template <class T>
 struct Best {
-  float v;
+  T v;
   uint32_t i;
 };
 
-template <bool IsMax>
-__device__ __forceinline__ bool better(float v, uint32_t i, const Best& b) {
+// the value no element loses against: -inf / +inf, or the end of the integer range
+template <class T, bool IsMax>
+__device__ __forceinline__ T worst() {
+  if constexpr (__is_floating_point(T)) {
+    return IsMax ? (T)-INFINITY : (T)INFINITY;
+  } else {
+    constexpr bool is_signed = (T)(-1) < (T)0;
+    constexpr T lo = is_signed ? (T)((T)1 << (sizeof(T) * 8 - 1)) : (T)0;
+    return IsMax ? lo : (T)~lo;
+  }
+}
+
+template <bool IsMax, class T>
+__device__ __forceinline__ bool better(T v, uint32_t i, const Best<T>& b) {
   return IsMax ? (v > b.v || (v == b.v && i < b.i)) : (v < b.v || (v == b.v && i < b.i));
 }
 
-template <bool IsMax>
-__device__ __forceinline__ Best wave_best(Best b) {
+template <class T>
+__device__ __forceinline__ T shuffle_xor(T v, int o) {
+  if constexpr (sizeof(T) < 4)
+    return (T)__shfl_xor((int)v, o);
+  else
+    return __shfl_xor(v, o);
+}
+
+template <bool IsMax, class T>
+__device__ __forceinline__ Best<T> wave_best(Best<T> b) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(b.v, o);
+    const T ov = shuffle_xor(b.v, o);
     const uint32_t oi = __shfl_xor(b.i, o);
     if (better<IsMax>(ov, oi, b)) {
       b.v = ov;
@@ -46,9 +66,10 @@ __device__ __forceinline__ Best wave_best(Best b) {
   return b;
 }
 
+template <class T>
 struct SelParams {
-  const float* x;
-  void* out;        // float for value ops, uint32_t for index ops
+  const T* x;
+  void* out;        // T for value ops, uint32_t for index ops
   int64_t n, incx;  // the reduced run
   uint32_t nrows;
   int32_t nouter;
@@ -56,12 +77,12 @@ struct SelParams {
   int64_t ox[kSelMaxOuter], oo[kSelMaxOuter];
   int32_t want_index;
   uint32_t splits;  // workgroups per row
-  int64_t seg;      // elements per split (multiple of 4)
-  Best* partials;   // nrows * splits
+  int64_t seg;      // elements per split (multiple of the 16-byte vector)
+  Best<T>* partials;  // nrows * splits
 };
 
-__device__ __forceinline__ void sel_offsets(const SelParams& p, uint32_t row, int64_t* xoff,
-                                            int64_t* ooff) {
+template <class T>
+__device__ __forceinline__ void sel_offsets(const SelParams<T>& p, uint32_t row, int64_t* xoff, int64_t* ooff) {
   int64_t xo = 0, oo = 0;
   uint32_t rem = row;
   for (int i = 0; i < p.nouter; i++) {
@@ -82,70 +103,74 @@ __device__ __forceinline__ void sel_offsets(const SelParams& p, uint32_t row, in
 
 // best of x[lo, hi) seen by thread `t` of `nthreads`; a lane scans increasing
 // indices with a strict comparison, so it keeps the first occurrence
-template <bool IsMax, bool VEC>
-__device__ __forceinline__ Best scan(const float* __restrict__ x, int64_t incx, int64_t lo,
-                                     int64_t hi, int t, int nthreads) {
-  Best b = {IsMax ? -INFINITY : INFINITY, 0u};
+template <bool IsMax, bool VEC, class T>
+__device__ __forceinline__ Best<T> scan(const T* __restrict__ x, int64_t incx, int64_t lo, int64_t hi, int t,
+                                        int nthreads) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  constexpr int N = 16 / (int)sizeof(T);
+  struct alignas(16) Pack { T v[N]; };
+  Best<T> b = {worst<T, IsMax>(), 0u};
   if (VEC) {  // incx == 1, x + lo 16-byte aligned
-    const int64_t nvec = (hi - lo) / 4;
+    const int64_t nvec = (hi - lo) / N;
     const f4* xv = reinterpret_cast<const f4*>(x + lo);
-    auto take = [&](const f4& v, uint32_t at) {
-      if (IsMax ? v.x > b.v : v.x < b.v) { b.v = v.x; b.i = at; }
-      if (IsMax ? v.y > b.v : v.y < b.v) { b.v = v.y; b.i = at + 1; }
-      if (IsMax ? v.z > b.v : v.z < b.v) { b.v = v.z; b.i = at + 2; }
-      if (IsMax ? v.w > b.v : v.w < b.v) { b.v = v.w; b.i = at + 3; }
+    auto take = [&](const f4& raw, uint32_t at) {
+      const Pack v = __builtin_bit_cast(Pack, raw);
+#pragma unroll
+      for (int k = 0; k < N; k++)
+        if (IsMax ? v.v[k] > b.v : v.v[k] < b.v) { b.v = v.v[k]; b.i = at + k; }
     };
     int64_t i = t;
     for (; i + nthreads < nvec; i += 2 * (int64_t)nthreads) {  // two loads in flight
       const f4 v0 = __builtin_nontemporal_load(xv + i);
       const f4 v1 = __builtin_nontemporal_load(xv + i + nthreads);
-      take(v0, (uint32_t)(lo + 4 * i));
-      take(v1, (uint32_t)(lo + 4 * (i + nthreads)));
+      take(v0, (uint32_t)(lo + N * i));
+      take(v1, (uint32_t)(lo + N * (i + nthreads)));
     }
-    if (i < nvec) take(__builtin_nontemporal_load(xv + i), (uint32_t)(lo + 4 * i));
-    for (int64_t c = lo + nvec * 4 + t; c < hi; c += nthreads) {
-      const float v = x[c];
+    if (i < nvec) take(__builtin_nontemporal_load(xv + i), (uint32_t)(lo + N * i));
+    for (int64_t c = lo + nvec * N + t; c < hi; c += nthreads) {
+      const T v = x[c];
       if (IsMax ? v > b.v : v < b.v) { b.v = v; b.i = (uint32_t)c; }
     }
   } else {
     for (int64_t c = lo + t; c < hi; c += nthreads) {
-      const float v = x[c * incx];
+      const T v = x[c * incx];
       if (IsMax ? v > b.v : v < b.v) { b.v = v; b.i = (uint32_t)c; }
     }
   }
   return b;
 }
 
-__device__ __forceinline__ void emit(const SelParams& p, int64_t ooff, const Best& b) {
+template <class T>
+__device__ __forceinline__ void emit(const SelParams<T>& p, int64_t ooff, const Best<T>& b) {
   if (p.want_index)
     static_cast<uint32_t*>(p.out)[ooff] = b.i;
   else
-    static_cast<float*>(p.out)[ooff] = b.v;
+    static_cast<T*>(p.out)[ooff] = b.v;
 }
 
 // one wavefront per row, four rows per workgroup
-template <bool IsMax, bool VEC>
-__global__ __launch_bounds__(kBlock) void select_rows_wave(SelParams p) {
+template <bool IsMax, bool VEC, class T>
+__global__ __launch_bounds__(kBlock) void select_rows_wave(SelParams<T> p) {
   const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (row >= p.nrows) return;
   int64_t xoff, ooff;
   sel_offsets(p, row, &xoff, &ooff);
-  Best b = scan<IsMax, VEC>(p.x + xoff, p.incx, 0, p.n, threadIdx.x & (kWave - 1), kWave);
+  Best<T> b = scan<IsMax, VEC>(p.x + xoff, p.incx, 0, p.n, threadIdx.x & (kWave - 1), kWave);
   b = wave_best<IsMax>(b);
   if ((threadIdx.x & (kWave - 1)) == 0) emit(p, ooff, b);
 }
 
 // one workgroup per (row, split)
-template <bool IsMax, bool VEC>
-__global__ __launch_bounds__(kBlock) void select_rows_block(SelParams p) {
-  __shared__ Best lds[kBlock / kWave];
+template <bool IsMax, bool VEC, class T>
+__global__ __launch_bounds__(kBlock) void select_rows_block(SelParams<T> p) {
+  __shared__ Best<T> lds[kBlock / kWave];
   const uint32_t row = blockIdx.x / p.splits;
   const uint32_t split = blockIdx.x - row * p.splits;
   int64_t xoff, ooff;
   sel_offsets(p, row, &xoff, &ooff);
   const int64_t lo = (int64_t)split * p.seg;
   const int64_t hi = lo + p.seg < p.n ? lo + p.seg : p.n;
-  Best b = scan<IsMax, VEC>(p.x + xoff, p.incx, lo, hi, threadIdx.x, kBlock);
+  Best<T> b = scan<IsMax, VEC>(p.x + xoff, p.incx, lo, hi, threadIdx.x, kBlock);
   b = wave_best<IsMax>(b);
   if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = b;
   __syncthreads();
@@ -160,15 +185,15 @@ __global__ __launch_bounds__(kBlock) void select_rows_block(SelParams p) {
   }
 }
 
-template <bool IsMax>
-__global__ __launch_bounds__(kBlock) void select_rows_finish(SelParams p) {
-  __shared__ Best lds[kBlock / kWave];
+template <bool IsMax, class T>
+__global__ __launch_bounds__(kBlock) void select_rows_finish(SelParams<T> p) {
+  __shared__ Best<T> lds[kBlock / kWave];
   const uint32_t row = blockIdx.x;
   int64_t xoff, ooff;
   sel_offsets(p, row, &xoff, &ooff);
-  Best b = {IsMax ? -INFINITY : INFINITY, 0u};
+  Best<T> b = {worst<T, IsMax>(), 0u};
   for (uint32_t s = threadIdx.x; s < p.splits; s += kBlock) {
-    const Best c = p.partials[(int64_t)row * p.splits + s];
+    const Best<T> c = p.partials[(int64_t)row * p.splits + s];
     if (better<IsMax>(c.v, c.i, b)) b = c;
   }
   b = wave_best<IsMax>(b);
@@ -182,13 +207,13 @@ __global__ __launch_bounds__(kBlock) void select_rows_finish(SelParams p) {
   }
 }
 
-template <bool IsMax, bool VEC>
-static int launch_select(SelParams& p) {
+template <bool IsMax, bool VEC, class T>
+static int launch_select(SelParams<T>& p) {
   hipStream_t st = rt().stream;
   const int64_t target = (int64_t)rt().num_cus * 8;
   if (p.n <= 2048 || (p.n < 8192 && p.nrows >= target)) {
     const uint32_t blocks = (uint32_t)ceil_div(p.nrows, kBlock / kWave);
-    select_rows_wave<IsMax, VEC><<<blocks, kBlock, 0, st>>>(p);
+    select_rows_wave<IsMax, VEC, T><<<blocks, kBlock, 0, st>>>(p);
     return after_launch("select_rows_wave");
   }
   p.splits = 1;
@@ -196,7 +221,7 @@ static int launch_select(SelParams& p) {
   if (p.nrows < target) {
     int64_t by_work = ceil_div(p.n, 16384);
     int64_t by_fill = ceil_div(target, p.nrows);
-    int64_t by_cap = (int64_t)(kPartialCapacity / 2) / p.nrows;  // a Best is two floats wide
+    int64_t by_cap = (int64_t)(kPartialCapacity * sizeof(float) / sizeof(Best<T>)) / p.nrows;
     int64_t splits = by_work < by_fill ? by_work : by_fill;
     if (splits > by_cap) splits = by_cap;
     if (splits < 1) splits = 1;
@@ -206,21 +231,17 @@ static int launch_select(SelParams& p) {
   }
   const int64_t blocks = (int64_t)p.nrows * p.splits;
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows for one launch");
-  select_rows_block<IsMax, VEC><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  select_rows_block<IsMax, VEC, T><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   WF2_TRY(after_launch("select_rows_block"));
   if (p.splits > 1) {
-    select_rows_finish<IsMax><<<p.nrows, kBlock, 0, st>>>(p);
+    select_rows_finish<IsMax, T><<<p.nrows, kBlock, 0, st>>>(p);
     WF2_TRY(after_launch("select_rows_finish"));
   }
   return 0;
 }
 
-}  // namespace wf2
-
-using namespace wf2;
-
-WF2_API int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long incx, const float* x,
-                             void* out) {
+template <class T>
+static int select_nd(int op, const wf2hip_view2* outer, long n, long incx, const T* x, void* out) {
   WF2_TRY(require_init());
   if (op < WF2HIP_MAXVALUE || op > WF2HIP_ARGMIN) return fail(WF2HIP_EINVAL, "unknown selection op %d", op);
   Space s;
@@ -238,13 +259,15 @@ WF2_API int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long inc
       s.shape[r] = 1;
     }
   normalise(&s);
-  SelParams p;
+  SelParams<T> p;
+  p.want_index = op == WF2HIP_ARGMAX || op == WF2HIP_ARGMIN;
   p.x = x + s.off_a;
-  p.out = static_cast<char*>(out) + 4 * s.off_b;
+  p.out = static_cast<char*>(out) + (p.want_index ? 4 : (int64_t)sizeof(T)) * s.off_b;
   p.n = n;
   p.incx = incx;
   p.nouter = s.rank;
   int64_t nrows = 1;
+  constexpr int64_t N = 16 / (int64_t)sizeof(T);
   bool vec = incx == 1 && ((uintptr_t)p.x & 15u) == 0;
   for (int i = 0; i < s.rank; i++) {
     const int r = s.rank - 1 - i;
@@ -253,14 +276,63 @@ WF2_API int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long inc
     p.ox[i] = s.sa[r];
     p.oo[i] = s.sb[r];
     nrows *= s.shape[r];
-    if (s.shape[r] > 1 && s.sa[r] % 4 != 0) vec = false;
+    if (s.shape[r] > 1 && s.sa[r] % N != 0) vec = false;
   }
   p.nrows = (uint32_t)nrows;
-  p.want_index = op == WF2HIP_ARGMAX || op == WF2HIP_ARGMIN;
   p.splits = 1;
   p.seg = n;
-  p.partials = reinterpret_cast<Best*>(rt().partials);
+  p.partials = reinterpret_cast<Best<T>*>(rt().partials);
   const bool is_max = op == WF2HIP_MAXVALUE || op == WF2HIP_ARGMAX;
   if (is_max) return vec ? launch_select<true, true>(p) : launch_select<true, false>(p);
   return vec ? launch_select<false, true>(p) : launch_select<false, false>(p);
 }
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long incx, const float* x, void* out) {
+  return select_nd<float>(op, outer, n, incx, x, out);
+}
+
+// MaxValue-Node / MinValue-Node on every dtype (the CPU backend calls
+// waffe2_<prefix>{max,min} per row, backends/cpu/matrix-ops.lisp:336-369), ArgMax-Node /
+// ArgMin-Node on :double (BLAS idmax / idmin, :240-283; other dtypes are an error there too)
+WF2_API int wf2hip_select_nd_typed(int dtype, int op, const wf2hip_view2* outer, long n, long incx, const void* x,
+                                   void* out) {
+  const bool index = op == WF2HIP_ARGMAX || op == WF2HIP_ARGMIN;
+  if (index && dtype != WF2HIP_F64)
+    return fail(WF2HIP_EUNSUPPORTED, "argmax / argmin support :float and :double only");
+  switch (dtype) {
+    case WF2HIP_F64: return select_nd<double>(op, outer, n, incx, (const double*)x, out);
+    case WF2HIP_I32: return select_nd<int32_t>(op, outer, n, incx, (const int32_t*)x, out);
+    case WF2HIP_U32: return select_nd<uint32_t>(op, outer, n, incx, (const uint32_t*)x, out);
+    case WF2HIP_I16: return select_nd<int16_t>(op, outer, n, incx, (const int16_t*)x, out);
+    case WF2HIP_U16: return select_nd<uint16_t>(op, outer, n, incx, (const uint16_t*)x, out);
+    case WF2HIP_I8: return select_nd<int8_t>(op, outer, n, incx, (const int8_t*)x, out);
+    case WF2HIP_U8: return select_nd<uint8_t>(op, outer, n, incx, (const uint8_t*)x, out);
+    default: return fail(WF2HIP_EINVAL, "unknown element type %d (:float has its own entry point)", dtype);
+  }
+}
+
+// waffe2_<prefix>{max,min}(n, x, incx, y): y[0] <- the extreme of the run (cl-waffe2-simd.c:316-365)
+#define WF2_DEFINE_TYPED_EXTREME(prefix, T)                                                    \
+  WF2_API int wf2hip_##prefix##max(long n, const T* x, long incx, T* out) {                  \
+    wf2hip_view2 one = {};                                                                    \
+    one.rank = 1;                                                                             \
+    one.shape[0] = 1;                                                                         \
+    return select_nd<T>(WF2HIP_MAXVALUE, &one, n, incx, x, out);                              \
+  }                                                                                           \
+  WF2_API int wf2hip_##prefix##min(long n, const T* x, long incx, T* out) {                  \
+    wf2hip_view2 one = {};                                                                    \
+    one.rank = 1;                                                                             \
+    one.shape[0] = 1;                                                                         \
+    return select_nd<T>(WF2HIP_MINVALUE, &one, n, incx, x, out);                              \
+  }
+WF2_DEFINE_TYPED_EXTREME(d, double)
+WF2_DEFINE_TYPED_EXTREME(i32, int32_t)
+WF2_DEFINE_TYPED_EXTREME(u32, uint32_t)
+WF2_DEFINE_TYPED_EXTREME(i16, int16_t)
+WF2_DEFINE_TYPED_EXTREME(u16, uint16_t)
+WF2_DEFINE_TYPED_EXTREME(i8, int8_t)
+WF2_DEFINE_TYPED_EXTREME(u8, uint8_t)

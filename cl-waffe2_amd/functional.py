@@ -74,7 +74,7 @@ def reshape(x: HIPTensor, *shape: int) -> HIPTensor:
     if int(np.prod(shape, dtype=np.int64)) != x.size:
         raise ValueError(f"reshape: cannot reshape {x.shape} into {shape}")
     src = to_contiguous(x)
-    return HIPTensor(shape, vec=src.vec)
+    return HIPTensor(shape, vec=src.vec, dtype=src.dtype)
 
 
 class Transposed:
@@ -139,7 +139,8 @@ def flexible(y: HIPTensor, like: HIPTensor) -> HIPTensor:
     for i, s in enumerate(subs):
         if s is not True:
             views[i] = parse_view(y.orig_shape[i], y.views[i], s)
-    return HIPTensor(y.orig_shape, vec=y.vec, strides=y.stride, views=views, offset=y.initial_offset)
+    return HIPTensor(y.orig_shape, vec=y.vec, strides=y.stride, views=views, offset=y.initial_offset,
+                     dtype=y.dtype)
 
 
 def _operand(y, like: HIPTensor) -> HIPTensor:
@@ -411,13 +412,13 @@ def _keepdims(result: HIPTensor, base: HIPTensor) -> HIPTensor:
 
 def max(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None, keepdims: bool = False):  # noqa: A001
     """``(!max tensor :axis :out :keepdims)``."""
-    r = _select("MaxValue-Node", x, axis, out, "float")
+    r = _select("MaxValue-Node", x, axis, out, x.dtype)
     return _keepdims(r, x) if keepdims else r
 
 
 def min(x: HIPTensor, axis: int = -1, out: HIPTensor | None = None, keepdims: bool = False):  # noqa: A001
     """``(!min tensor :axis :out :keepdims)``."""
-    r = _select("MinValue-Node", x, axis, out, "float")
+    r = _select("MinValue-Node", x, axis, out, x.dtype)
     return _keepdims(r, x) if keepdims else r
 
 
@@ -467,7 +468,7 @@ def sum(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = 
         if s is not True:
             views[i] = parse_view(out.orig_shape[i], out.views[i], s)
     out_bc = HIPTensor(out.orig_shape, vec=out.vec, strides=out.stride, views=views,
-                       offset=out.initial_offset)
+                       offset=out.initial_offset, dtype=out.dtype)
     add_(out_bc, x)  # A+=B out* tensor: accumulation into a stride-0 destination
     result = out_bc if keepdims else out
     if div_by is not None:

@@ -204,6 +204,11 @@ for _prefix, _ctype in (("d", C.c_double), ("i32", C.c_int32), ("u32", C.c_uint3
         _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P, _L, _P, _L, _ctype, _ctype], C.c_int)
         _SIGNATURES[f"wf2hip_{_prefix}{_op}_scal"] = ([_L, _P, _L, _P, _L, _ctype, _ctype, _ctype], C.c_int)
 
+_SIGNATURES["wf2hip_select_nd_typed"] = ([C.c_int, C.c_int, C.POINTER(View2), _L, _L, _P, _P], C.c_int)
+for _prefix in ("d", "i32", "u32", "i16", "u16", "i8", "u8"):
+    for _op in ("max", "min"):
+        _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P], C.c_int)
+
 EXPORTS = tuple(_SIGNATURES)
 
 _lib = None

@@ -88,6 +88,8 @@
 (defcfun "wf2hip_binary_nd_typed" :int
   (dtype :int) (op :int) (view (:pointer (:struct view2))) (a :pointer) (b :pointer))
 (defcfun "wf2hip_inv_1d_typed" :int (dtype :int) (n :long) (x :pointer) (incx :long))
+(defcfun "wf2hip_select_nd_typed" :int
+  (dtype :int) (op :int) (outer (:pointer (:struct view2))) (n :long) (incx :long) (x :pointer) (out :pointer))
 (defcfun "wf2hip_select_nd" :int
   (op :int) (outer (:pointer (:struct view2))) (n :long) (incx :long) (x :pointer) (out :pointer))
 (defconstant +maxvalue+ 48) (defconstant +minvalue+ 49) (defconstant +argmax+ 50) (defconstant +argmin+ 51)

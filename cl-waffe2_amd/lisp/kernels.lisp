@@ -208,16 +208,25 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
                 (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-a) :int64 0) 0
                 (mem-aref (foreign-slot-pointer view '(:struct view2) 'stride-b) :int64 0) 0)
           (setf (foreign-slot-value view '(:struct view2) 'rank) (1- rank)))
-      (check (wf2hip-select-nd op view n incx (tensor-device-pointer x) (tensor-device-pointer out)))))
+      (if (eql (dtype x) :float)
+          (check (wf2hip-select-nd op view n incx (tensor-device-pointer x) (tensor-device-pointer out)))
+          (check (wf2hip-select-nd-typed (nth-value 2 (dtype-info (dtype x))) op view n incx
+                                         (tensor-device-pointer x) (tensor-device-pointer out))))))
   out)
 
-(macrolet ((define-select (node op)
-             `(define-impl-op (,node :device HIPTensor :reject-p #'(lambda (&rest args) (declare (ignore args)) nil))
+;; The value nodes take every dtype (waffe2_<prefix>{max,min} on the CPU), the index nodes :float
+;; and :double (BLAS i?max / i?min, source/backends/cpu/matrix-ops.lisp:254-266).
+(defun float-or-double-p (dtype &rest more)
+  (declare (ignore more))
+  (not (member dtype '(:float :double))))
+
+(macrolet ((define-select (node op reject)
+             `(define-impl-op (,node :device HIPTensor :reject-p ,reject)
                               :forward ((self x out) (declare (ignore self)) (run-select ,op x out)))))
-  (define-select MaxValue-Node +maxvalue+)
-  (define-select MinValue-Node +minvalue+)
-  (define-select ArgMax-Node +argmax+)
-  (define-select ArgMin-Node +argmin+))
+  (define-select MaxValue-Node +maxvalue+ #'(lambda (&rest args) (declare (ignore args)) nil))
+  (define-select MinValue-Node +minvalue+ #'(lambda (&rest args) (declare (ignore args)) nil))
+  (define-select ArgMax-Node +argmax+ #'float-or-double-p)
+  (define-select ArgMin-Node +argmin+ #'float-or-double-p))
 
 ;; C[~ i k] = A[~ i j] . B[~ j k].  Same operand swap as expand-gemm-form-column
 ;; (source/backends/cpu/matrix-ops.lisp:12-112): a row-major product is the column-major

@@ -242,25 +242,36 @@ def _select(op, index: bool):
         os_, ost, oo = out.geometry()
         if len(xs) != len(os_) or xs[:-1] != os_[:-1] or os_[-1] != 1:
             raise ValueError(f"{x.shape} selects into {xs[:-1] + [1]}, not {out.shape}")
-        if out.dtype != ("uint32" if index else "float"):
-            raise ValueError("ArgMax/ArgMin write :uint32, MaxValue/MinValue :float")
+        if out.dtype != ("uint32" if index else x.dtype):
+            raise ValueError("ArgMax/ArgMin write :uint32, MaxValue/MinValue the dtype of A")
         v = _lib.View2()
         v.rank = max(len(xs) - 1, 1)
         v.shape[0], v.stride_a[0], v.stride_b[0] = 1, 0, 0
         for r in range(len(xs) - 1):
             v.shape[r], v.stride_a[r], v.stride_b[r] = xs[r], xst[r], ost[r]
         v.off_a, v.off_b = xo, oo
-        _lib.check(_lib.get().wf2hip_select_nd(op, C.byref(v), xs[-1], xst[-1], C.c_void_p(x.ptr),
-                                               C.c_void_p(out.ptr)))
+        if x.dtype == "float":
+            _lib.check(_lib.get().wf2hip_select_nd(op, C.byref(v), xs[-1], xst[-1], C.c_void_p(x.ptr),
+                                                   C.c_void_p(out.ptr)))
+        else:
+            _lib.check(_lib.get().wf2hip_select_nd_typed(_lib.DTYPE_CODES[x.dtype], op, C.byref(v), xs[-1], xst[-1],
+                                                         C.c_void_p(x.ptr), C.c_void_p(out.ptr)))
         return out
 
     return impl
 
 
-define_impl("MaxValue-Node", HIPTensor, _only_float)(_select(_lib.MAXVALUE, False))
-define_impl("MinValue-Node", HIPTensor, _only_float)(_select(_lib.MINVALUE, False))
-define_impl("ArgMax-Node", HIPTensor, _only_float)(_select(_lib.ARGMAX, True))
-define_impl("ArgMin-Node", HIPTensor, _only_float)(_select(_lib.ARGMIN, True))
+def _float_or_double(dtype) -> bool:
+    """reject-p of the index nodes: BLAS i?max / i?min exist for :float and :double
+    (``backends/cpu/matrix-ops.lisp:254-266``)."""
+    return dtype not in ("float", "double")
+
+
+# the value nodes take every dtype (waffe2_<prefix>{max,min}, backends/cpu/matrix-ops.lisp:323-369)
+define_impl("MaxValue-Node", HIPTensor)(_select(_lib.MAXVALUE, False))
+define_impl("MinValue-Node", HIPTensor)(_select(_lib.MINVALUE, False))
+define_impl("ArgMax-Node", HIPTensor, _float_or_double)(_select(_lib.ARGMAX, True))
+define_impl("ArgMin-Node", HIPTensor, _float_or_double)(_select(_lib.ARGMIN, True))
 
 
 def _unfold_args(x_shape, col_shape, stride, padding, dilation):

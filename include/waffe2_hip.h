@@ -289,6 +289,29 @@ int wf2hip_u8inv(long n, uint8_t* x, long incx);
  * per row.  Ties go to the lowest index; NaN elements are never selected. */
 enum wf2hip_select_op { WF2HIP_MAXVALUE = 48, WF2HIP_MINVALUE = 49, WF2HIP_ARGMAX = 50, WF2HIP_ARGMIN = 51 };
 int wf2hip_select_nd(int op, const wf2hip_view2* outer, long n, long incx, const float* x, void* out);
+/* The same on the other element types (dtype: enum wf2hip_dtype, declared with the
+ * typed arithmetic below): MaxValue-Node / MinValue-Node for every dtype -- the CPU
+ * backend calls waffe2_<prefix>{max,min} per row (source/backends/cpu/matrix-ops.lisp:
+ * 323-369; cl-waffe2-simd.c:316-365) -- with OUT of the same dtype, ArgMax-Node /
+ * ArgMin-Node for :double only (BLAS idmax / idmin, matrix-ops.lisp:254-266; any other
+ * dtype is an error there and WF2HIP_EUNSUPPORTED here).  The 1-D names keep the
+ * reference's arguments: out[0] <- the extreme of the n elements. */
+int wf2hip_select_nd_typed(int dtype, int op, const wf2hip_view2* outer, long n, long incx, const void* x,
+                           void* out);
+int wf2hip_dmax(long n, const double* x, long incx, double* out);
+int wf2hip_dmin(long n, const double* x, long incx, double* out);
+int wf2hip_i32max(long n, const int32_t* x, long incx, int32_t* out);
+int wf2hip_i32min(long n, const int32_t* x, long incx, int32_t* out);
+int wf2hip_u32max(long n, const uint32_t* x, long incx, uint32_t* out);
+int wf2hip_u32min(long n, const uint32_t* x, long incx, uint32_t* out);
+int wf2hip_i16max(long n, const int16_t* x, long incx, int16_t* out);
+int wf2hip_i16min(long n, const int16_t* x, long incx, int16_t* out);
+int wf2hip_u16max(long n, const uint16_t* x, long incx, uint16_t* out);
+int wf2hip_u16min(long n, const uint16_t* x, long incx, uint16_t* out);
+int wf2hip_i8max(long n, const int8_t* x, long incx, int8_t* out);
+int wf2hip_i8min(long n, const int8_t* x, long incx, int8_t* out);
+int wf2hip_u8max(long n, const uint8_t* x, long incx, uint8_t* out);
+int wf2hip_u8min(long n, const uint8_t* x, long incx, uint8_t* out);
 
 /* ---- compare / where ---------------------------------------------------- */
 /* out <- (x OP y) ? then_value : else_value.  OP is ordered: false when an

@@ -468,3 +468,23 @@ def cmp_typed_1d(dtype: str, op: str, n: int, x: np.ndarray, incx: int, y, incy:
     fn.restype = C.c_int
     assert fn(code, CMP_OPS.index(op), n, px, incx, py, 0 if scal else incy, po, inco, int(scal),
               float(y) if scal else 0.0, float(then), float(els)) == 0
+
+
+def extreme_typed_1d(dtype: str, op: str, n: int, x: np.ndarray, incx: int, use_ref: bool = False, offx: int = 0):
+    """The largest (op "max") / smallest ("min") element of the run, as
+    waffe2_<prefix>{max,min} leave it in y[0]."""
+    code, npt, prefix = DTYPES[dtype]
+    assert x.dtype == npt
+    out = np.zeros(1, npt)
+    px = C.c_void_p(x.ctypes.data + x.itemsize * offx)
+    if use_ref:
+        fn = getattr(ref(), f"waffe2_{prefix}{op}")
+        fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p]
+        fn.restype = None
+        fn(n, px, incx, C.c_void_p(out.ctypes.data))
+    else:
+        fn = lib().orc_extreme_typed
+        fn.argtypes = [C.c_int, C.c_int, C.c_long, C.c_void_p, C.c_long, C.c_void_p]
+        fn.restype = C.c_int
+        assert fn(code, int(op == "max"), n, px, incx, C.c_void_p(out.ctypes.data)) == 0
+    return out[0]

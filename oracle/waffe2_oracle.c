@@ -41,6 +41,8 @@
  *       reference C (waffe2_{d,i32,...}{eq,...} and ..._scal), numpy closed forms
  *       (the element type's own order on the remainder, the signed order on the
  *       leading blocks of the unsigned types).
+ *   orc_extreme_typed                  : golden vectors from the compiled
+ *       reference C (waffe2_{d,i32,...}{max,min}), numpy max / min.
  *   orc_sgemm                          : the reference's integer gemm vectors
  *       (base-impl/t/arithmetic.lisp:120,135,142,148), float64 truth.
  */
@@ -836,6 +838,48 @@ ORC_API int orc_cmp_typed(int dtype, int op, long n, const void *x, long incx, c
     case 5: ORC_CMP_LOOP(uint16_t, int16_t)
     case 6: ORC_CMP_LOOP(int8_t, int8_t)
     case 7: ORC_CMP_LOOP(uint8_t, int8_t)
+    default: return -1;
+  }
+}
+
+/* waffe2_{d,i32,i16,i8,u32,u16,u8}{max,min} (cl-waffe2-simd.c:316-365, define_maxmin):
+ * `lanes` running extremes over blocks of 32 bytes / element size, folded, then the
+ * remainder.  Exact for the integer types in any order; for :double the lane
+ * operation is _mm256_max_pd / _mm256_min_pd (the second operand when either is
+ * NaN) and the folds use MAX / MIN (a > b ? a : b). */
+#define ORC_EXTREME_LOOP(T)                                                          \
+  {                                                                                  \
+    const T *xp = (const T *)x;                                                      \
+    const long lanes = 32 / (long)sizeof(T);                                         \
+    T lane[32], best = xp[0];                                                        \
+    long count = 0;                                                                  \
+    const long blocks_end = (n / lanes) * lanes;                                     \
+    for (long l = 0; l < lanes; l++) lane[l] = best;                                 \
+    for (; count != blocks_end; count += lanes)                                      \
+      for (long l = 0; l < lanes; l++) {                                             \
+        const T v = xp[(count + l) * incx];                                          \
+        lane[l] = is_max ? (lane[l] > v ? lane[l] : v) : (lane[l] < v ? lane[l] : v); \
+      }                                                                              \
+    for (long l = 0; l < lanes; l++)                                                 \
+      best = is_max ? (best > lane[l] ? best : lane[l]) : (best < lane[l] ? best : lane[l]); \
+    for (; count != n; count++) {                                                    \
+      const T v = xp[count * incx];                                                  \
+      best = is_max ? (best > v ? best : v) : (best < v ? best : v);                 \
+    }                                                                                \
+    ((T *)out)[0] = best;                                                            \
+    return 0;                                                                        \
+  }
+
+ORC_API int orc_extreme_typed(int dtype, int is_max, long n, const void *x, long incx, void *out) {
+  if (n < 1) return -1;
+  switch (dtype) {
+    case 1: ORC_EXTREME_LOOP(double)
+    case 2: ORC_EXTREME_LOOP(int32_t)
+    case 3: ORC_EXTREME_LOOP(uint32_t)
+    case 4: ORC_EXTREME_LOOP(int16_t)
+    case 5: ORC_EXTREME_LOOP(uint16_t)
+    case 6: ORC_EXTREME_LOOP(int8_t)
+    case 7: ORC_EXTREME_LOOP(uint8_t)
     default: return -1;
   }
 }

@@ -341,6 +341,60 @@ def compare_typed_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_compare_kernels.npz")), "bytes")
 
 
+def _extreme_child(dtype, op, n, x, incx, conn):
+    conn.send(O.extreme_typed_1d(dtype, op, n, x, incx, use_ref=True))
+
+
+def extreme_typed_goldens():
+    """waffe2_<prefix>{max,min} of the compiled reference; integer runs with
+    incx != 1 that reach the block part are undefined there (strided lanes, see
+    _cmp_case_defined) and left out, as is any case the compiled reference does not
+    finish."""
+    import multiprocessing as mp
+    assert O.ref() is not None, "oracle/_ref/libwaffe2_simd_ref.so is missing: run `make -C oracle ref`"
+    ctx = mp.get_context("fork")
+    rng = np.random.Generator(np.random.PCG64(2030))
+    out = {}
+    for dtype, (code, npt, prefix) in O.DTYPES.items():
+        lanes = 32 // np.dtype(npt).itemsize
+        xs, outs, cases, start, skipped = [], [], [], 0, 0
+        for op_index, op in enumerate(("max", "min")):
+            for n, incx in [(1, 1), (3, 1), (lanes, 1), (2 * lanes + 3, 1), (200, 1), (lanes - 1, 2), (5 * lanes + 1, 3)]:
+                if dtype != "double" and incx != 1 and n >= lanes:
+                    skipped += 1
+                    continue
+                size = n * incx + 1
+                if dtype == "double":
+                    x = (rng.standard_normal(size) * 100).round(1)
+                else:
+                    info = np.iinfo(npt)
+                    x = rng.integers(info.min, info.max, size, endpoint=True).astype(npt)
+                x = x.astype(npt)
+                parent, child = ctx.Pipe(duplex=False)
+                proc = ctx.Process(target=_extreme_child, args=(dtype, op, n, x, incx, child))
+                proc.start()
+                got = parent.recv() if parent.poll(3) else None
+                proc.join(1)
+                if proc.is_alive():
+                    proc.kill()
+                    proc.join()
+                if got is None:
+                    skipped += 1
+                    continue
+                xs.append(x), outs.append(got)
+                cases.append((op_index, n, incx, start, size))
+                start += size
+        key = f"{dtype}_extreme"
+        if cases:
+            out[key + "_x"] = np.concatenate(xs)
+            out[key + "_out"] = np.array(outs, npt)
+        out[key + "_cases"] = np.array(cases, np.int64).reshape(-1, 5)
+        out[key + "_skipped"] = np.array([skipped], np.int64)
+        print(dtype, "cases", len(cases), "skipped", skipped, flush=True)
+    np.savez_compressed(os.path.join(HERE, "typed_extreme_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_extreme_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
     if "--im2col-only" in sys.argv:
         im2col_goldens()
@@ -352,6 +406,8 @@ if __name__ == "__main__":
         typed_goldens()
     elif "--typed-compare-only" in sys.argv:
         compare_typed_goldens()
+    elif "--typed-extreme-only" in sys.argv:
+        extreme_typed_goldens()
     else:
         main()
         compare_goldens()
@@ -359,3 +415,4 @@ if __name__ == "__main__":
         im2col_goldens()
         typed_goldens()
         compare_typed_goldens()
+        extreme_typed_goldens()

@@ -115,3 +115,69 @@ def test_nodes_on_views(gpu, dtype):
         row = F.from_numpy(B[0:1, 0:1, :], dtype=dtype).view(True, (":broadcast", 40), True)
         got = F.compare(dA.view(2, True, True), row, cond, 1, 0)
         np.testing.assert_array_equal(got.numpy(), np.where(fn(A[2:3], B[0:1, 0:1, :]), 1, 0).astype(npt))
+
+
+EXTREME_GOLD = os.path.join(os.path.dirname(__file__), "golden", "typed_extreme_kernels.npz")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_extremes_against_goldens_and_oracle(gpu, O, dtype):
+    """wf2hip_<prefix>{max,min}: the compiled reference's goldens, then the oracle on
+    runs long enough for the split kernel, unit and other increments."""
+    W = gpu
+    lib = W.lib.get()
+    npt, prefix = O.DTYPES[dtype][1], O.DTYPES[dtype][2]
+    gold = np.load(EXTREME_GOLD)
+
+    def run(op, n, x, incx, off=0):
+        dx = W.HIPTensor.from_numpy(x, dtype=dtype)
+        dout = W.HIPTensor.from_numpy(np.zeros(1, npt), dtype=dtype)
+        W.lib.check(getattr(lib, f"wf2hip_{prefix}{op}")(n, C.c_void_p(dx.ptr + dx.itemsize * off), incx,
+                                                         C.c_void_p(dout.ptr)))
+        return dout.numpy()[0]
+
+    for k, (op, n, incx, start, size) in enumerate(gold[f"{dtype}_extreme_cases"]):
+        x = gold[f"{dtype}_extreme_x"][int(start):int(start + size)]
+        assert run(("max", "min")[int(op)], int(n), x, int(incx)) == gold[f"{dtype}_extreme_out"][k]
+    rng = np.random.default_rng(29)
+    for n, incx, off in [(1, 1, 0), (100, 1, 1), (5000, 1, 0), (300001, 1, 4), (70001, 3, 2)]:
+        size = n * incx + off + 1
+        if dtype == "double":
+            x = rng.standard_normal(size)
+        else:
+            info = np.iinfo(npt)
+            x = rng.integers(info.min, info.max, size, endpoint=True).astype(npt)
+        for op in ("max", "min"):
+            assert run(op, n, x, incx, off) == O.extreme_typed_1d(dtype, op, n, x, incx, offx=off), (dtype, op, n, incx)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_max_min_nodes(gpu, dtype):
+    """!max / !min on every dtype, !argmax / !argmin on :double (first occurrence),
+    numpy closed forms; index nodes on integer tensors have no device kernel."""
+    W = gpu
+    F = W.functional
+    from importlib import import_module
+    npt = import_module("cl-waffe2_amd.tensor").DTYPES[dtype]
+    rng = np.random.default_rng(83)
+    if dtype == "double":
+        A = rng.integers(-50, 50, (37, 1000)).astype(npt) / 4
+    else:
+        info = np.iinfo(npt)
+        A = rng.integers(info.min, info.max, (37, 1000), endpoint=True).astype(npt)
+    dA = F.from_numpy(A, dtype=dtype)
+    got = F.max(dA)
+    assert got.dtype == dtype and got.shape == [37, 1]
+    np.testing.assert_array_equal(got.numpy()[:, 0], A.max(axis=1))
+    np.testing.assert_array_equal(F.min(dA).numpy()[:, 0], A.min(axis=1))
+    # strided rows: every second column of a window
+    v = dA.view((3, 30), (1, 999, 2))
+    np.testing.assert_array_equal(F.max(v).numpy()[:, 0], A[3:30, 1:999:2].max(axis=1))
+    # the whole tensor as one run
+    np.testing.assert_array_equal(F.min(dA, axis=2).numpy().ravel(), [A.min()])
+    if dtype == "double":
+        np.testing.assert_array_equal(F.argmax(dA).numpy()[:, 0], A.argmax(axis=1))
+        np.testing.assert_array_equal(F.argmin(dA).numpy()[:, 0], A.argmin(axis=1))
+    else:
+        with pytest.raises(W.nodes.NodeNotFound):
+            F.argmax(dA)
