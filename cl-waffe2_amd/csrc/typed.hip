@@ -383,6 +383,131 @@ static bool typed_overlap(const Space& s, const void* a, const void* b, size_t s
   return !(a1 <= b0 || b1 <= a0);
 }
 
+// ---- accumulation into a broadcast destination (what !sum composes) ------------
+// a[kept] <- a[kept] OP b[kept, reduced] over every reduced index.  Integer sums
+// wrap modulo 2^bits whatever the order, so ADD runs as a tree per destination
+// (one workgroup each) and is exact; :double ADD is the same tree in binary64
+// (within a few ulp of the reference's sequential order).  The other operations
+// keep the reference's order: one lane per destination walks the reduced indices
+// row-major.
+struct TypedAcc {
+  int32_t nk, nr;  // kept / reduced axis counts
+  int64_t nout, nred;
+  int64_t kshape[WF2HIP_MAX_RANK], ka[WF2HIP_MAX_RANK], kb[WF2HIP_MAX_RANK];
+  int64_t rshape[WF2HIP_MAX_RANK], rb[WF2HIP_MAX_RANK];  // outermost first
+};
+
+__device__ __forceinline__ void acc_kept(const TypedAcc& p, int64_t out, int64_t* aoff, int64_t* boff) {
+  int64_t ao = 0, bo = 0, rem = out;
+  for (int i = p.nk - 1; i >= 0; i--) {
+    const int64_t q = rem / p.kshape[i];
+    const int64_t idx = rem - q * p.kshape[i];
+    rem = q;
+    ao += idx * p.ka[i];
+    bo += idx * p.kb[i];
+  }
+  *aoff = ao;
+  *boff = bo;
+}
+
+__device__ __forceinline__ int64_t acc_reduced(const TypedAcc& p, int64_t j) {
+  int64_t off = 0, rem = j;
+  for (int i = p.nr - 1; i >= 0; i--) {
+    const int64_t q = rem / p.rshape[i];
+    const int64_t idx = rem - q * p.rshape[i];
+    rem = q;
+    off += idx * p.rb[i];
+  }
+  return off;
+}
+
+template <class T>
+struct SumOf { using type = uint32_t; };  // wrap-around sums of every integer type
+template <> struct SumOf<double> { using type = double; };
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_add(T* a, const T* b, TypedAcc p) {
+  using S = typename SumOf<T>::type;
+  __shared__ S lds[kBlock / kWave];
+  const int64_t out = blockIdx.x;
+  int64_t aoff, boff;
+  acc_kept(p, out, &aoff, &boff);
+  S acc = S(0);
+  // the innermost reduced axis is walked by the lanes, so a unit stride there coalesces
+  const int64_t inner = p.rshape[p.nr - 1], inner_stride = p.rb[p.nr - 1];
+  const int64_t outer = p.nred / inner;
+  for (int64_t o = threadIdx.x / kWave; o < outer; o += kBlock / kWave) {
+    const int64_t base = boff + acc_reduced(p, o * inner);
+    for (int64_t i = threadIdx.x & (kWave - 1); i < inner; i += kWave) acc += (S)b[base + i * inner_stride];
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    S total = lds[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; w++) total += lds[w];
+    a[aoff] = (T)((S)a[aoff] + total);
+  }
+}
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_sequential(T* a, const T* b, TypedAcc p) {
+  const int64_t out = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (out >= p.nout) return;
+  int64_t aoff, boff;
+  acc_kept(p, out, &aoff, &boff);
+  T acc = a[aoff];
+  const int64_t inner = p.rshape[p.nr - 1], inner_stride = p.rb[p.nr - 1];
+  const int64_t outer = p.nred / inner;
+  for (int64_t o = 0; o < outer; o++) {
+    const int64_t base = boff + acc_reduced(p, o * inner);
+    for (int64_t i = 0; i < inner; i++) acc = apply<T, OP>(acc, b[base + i * inner_stride]);
+  }
+  a[aoff] = acc;
+}
+
+// `s` is normalised and has at least one broadcast axis in `a`
+template <class T>
+static int run_accumulate(int op, const Space& s, T* a, const T* b) {
+  TypedAcc p;
+  p.nk = p.nr = 0;
+  p.nout = p.nred = 1;
+  for (int r = 0; r < s.rank; r++) {
+    if (s.sa[r] == 0 && s.shape[r] > 1) {
+      p.rshape[p.nr] = s.shape[r];
+      p.rb[p.nr] = s.sb[r];
+      p.nr++;
+      p.nred *= s.shape[r];
+    } else {
+      p.kshape[p.nk] = s.shape[r];
+      p.ka[p.nk] = s.sa[r];
+      p.kb[p.nk] = s.sb[r];
+      p.nk++;
+      p.nout *= s.shape[r];
+    }
+  }
+  hipStream_t st = rt().stream;
+  T* ap = a + s.off_a;
+  const T* bp = b + s.off_b;
+  if (op == WF2HIP_ADD && rt().reduce_mode == 0) {
+    if (p.nout >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+    typed_accumulate_add<T><<<(uint32_t)p.nout, kBlock, 0, st>>>(ap, bp, p);
+    return after_launch("typed_accumulate_add");
+  }
+  const int64_t blocks = ceil_div(p.nout, kBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+  switch (op) {
+    case WF2HIP_ADD: typed_accumulate_sequential<T, WF2HIP_ADD><<<(uint32_t)blocks, kBlock, 0, st>>>(ap, bp, p); break;
+    case WF2HIP_SUB: typed_accumulate_sequential<T, WF2HIP_SUB><<<(uint32_t)blocks, kBlock, 0, st>>>(ap, bp, p); break;
+    case WF2HIP_MUL: typed_accumulate_sequential<T, WF2HIP_MUL><<<(uint32_t)blocks, kBlock, 0, st>>>(ap, bp, p); break;
+    case WF2HIP_DIV: typed_accumulate_sequential<T, WF2HIP_DIV><<<(uint32_t)blocks, kBlock, 0, st>>>(ap, bp, p); break;
+    default: return fail(WF2HIP_EINVAL, "op %d cannot accumulate", op);
+  }
+  return after_launch("typed_accumulate_sequential");
+}
+
 template <class T>
 static int dispatch_nd(int op, Space s, T* a, const T* b) {
   if (s.total == 0) return 0;
@@ -392,10 +517,7 @@ static int dispatch_nd(int op, Space s, T* a, const T* b) {
     return fail(WF2HIP_EOVERLAP,
                 "in-place op on partially overlapping windows of one buffer; copy one operand first");
   if (has_broadcast_axis(s, s.sa)) {
-    if (op != WF2HIP_MOVE)
-      return fail(WF2HIP_EUNSUPPORTED,
-                  "accumulation into a broadcast destination is only built for :float; use the 1-D entry "
-                  "point with incx = 0 per output element");
+    if (op != WF2HIP_MOVE) return run_accumulate<T>(op, s, a, b);
     for (int r = 0; r < s.rank; r++)  // the last write wins
       if (s.sa[r] == 0 && s.shape[r] > 1) {
         s.off_b += s.sb[r] * (s.shape[r] - 1);

@@ -455,7 +455,7 @@ def sum(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = 
     shape = list(x.shape)
     out_shape = [1 if i in axes else n for i, n in enumerate(shape)]
     if out is None:
-        out = HIPTensor(out_shape)
+        out = HIPTensor(out_shape, dtype=x.dtype)
     elif out.shape != out_shape:
         raise ValueError(f"!sum: the given out's shape is {out.shape}, but expected: {out_shape}")
     out = mul_(out, 0.0)  # A*=scal out 0  (reduction.lisp:63)

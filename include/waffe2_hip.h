@@ -224,7 +224,11 @@ int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float* b, flo
  * entry points reproduce the reference's remainder loop, which rounds through
  * binary32 (sas_dadd & co. return float, :229-232): the last n % 4 elements of a
  * call, and every element when incx < 1.  The N-D entry point computes every
- * element in binary64 and refuses accumulation into a broadcast destination. */
+ * element in binary64.  A destination with stride-0 axes accumulates (what !sum
+ * composes): ADD as a tree per destination element -- exact for the integer types,
+ * whose sums wrap modulo 2^bits in any order, binary64 partial sums for :double --
+ * and SUB / MUL / DIV (or ADD after wf2hip_set_reduce_mode(1)) in the reference's
+ * sequential order. */
 enum wf2hip_dtype {
   WF2HIP_F64 = 1,
   WF2HIP_I32 = 2,

@@ -139,5 +139,56 @@ def test_nodes_on_views(gpu, dtype):
         q = F.div(dA, F.from_numpy(D, dtype=dtype))
         want = A / D if dtype == "double" else np.trunc(A.astype(np.float64) / D).astype(npt)
         np.testing.assert_array_equal(q.numpy(), want)
-    with pytest.raises(W.HIPError):  # accumulation into a broadcast destination: :float only
-        F.add_(F.from_numpy(draw((1, 4)), dtype=dtype).view((":broadcast", 3), True), F.from_numpy(draw((3, 4)), dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_accumulation_into_broadcast_destinations(gpu, dtype):
+    """!sum as the reference composes it (zero-fill, (:broadcast n) view, AddNode):
+    integer sums wrap modulo 2^bits in any order, so numpy's wrapped sum is the exact
+    answer; :double within 1e-13 relative to the sum of magnitudes.  SubNode into a
+    broadcast destination follows the sequential order (exact for integers)."""
+    W = gpu
+    F = W.functional
+    from importlib import import_module
+    npt = import_module("cl-waffe2_amd.tensor").DTYPES[dtype]
+    rng = np.random.default_rng(91)
+    if dtype == "double":
+        A = rng.standard_normal((7, 300, 41))
+    else:
+        info = np.iinfo(npt)
+        A = rng.integers(info.min, info.max, (7, 300, 41), endpoint=True).astype(npt)
+    dA = F.from_numpy(A, dtype=dtype)
+
+    def check(got, axis):
+        want = A.sum(axis=axis, keepdims=True, dtype=npt if dtype != "double" else np.float64)
+        assert got.dtype == dtype and list(got.shape) == list(want.shape)
+        if dtype == "double":
+            scale = np.abs(A).sum(axis=axis, keepdims=True)
+            assert np.max(np.abs(got.numpy() - want) / scale) < 1e-13
+        else:
+            np.testing.assert_array_equal(got.numpy(), want)
+
+    with np.errstate(over="ignore"):
+        check(F.sum(dA, axis=2), 2)
+        check(F.sum(dA, axis=0), 0)
+        check(F.sum(dA, axis=(0, 2)), (0, 2))
+        check(F.sum(dA), (0, 1, 2))
+        # a strided window
+        v = dA.view((1, 6), (0, 300, 7), (2, 40, 3))
+        W_ = A[1:6, 0:300:7, 2:40:3][:, :42, :12]
+        got = F.sum(v, axis=1)
+        want = W_.sum(axis=1, keepdims=True, dtype=npt if dtype != "double" else np.float64)
+        if dtype == "double":
+            assert np.max(np.abs(got.numpy() - want)) < 1e-11
+        else:
+            np.testing.assert_array_equal(got.numpy(), want)
+        # x[0, j] <- x[0, j] - sum_i y[i, j], sequentially
+        base = A[0, 0:1, :].copy()
+        dst = F.from_numpy(base, dtype=dtype).view((":broadcast", 300), True)
+        F.sub_(dst, F.from_numpy(A[1], dtype=dtype))
+        if dtype == "double":
+            want = base - A[1].sum(axis=0, keepdims=True)
+            assert np.max(np.abs(dst.storage_numpy().reshape(1, 41) - want)) < 1e-10
+        else:
+            want = (base.astype(np.int64) - A[1].astype(np.int64).sum(axis=0, keepdims=True)).astype(npt)
+            np.testing.assert_array_equal(dst.storage_numpy().reshape(1, 41), want)
