@@ -147,7 +147,7 @@ def counter_probe(W, reps: int = 5):
     print(json.dumps({"probe": "copy, add, mul, exp, rowsum", "launches_each": reps, "elements": N}))
 
 
-def row_table(W, reps: int = 10, warm: int = 3):
+def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     """One line per kernel of the path at the shape its configuration names:
     average launch time from an event pair on the library's stream, the
     algorithmic bytes (or flop) of one call, and the fraction of the roofline
@@ -185,22 +185,24 @@ def row_table(W, reps: int = 10, warm: int = 3):
             call(ring[(warm + i) % len(ring)])
         b.record()
         eager_ms = a.elapsed_ms(b) / reps
-        # the same `reps` calls recorded once and replayed as one HIP graph: the launch
-        # times without the host work between them (Python here, Lisp in the product)
-        W.lib.synchronize()
-        with W.lib.Graph() as g:
-            for i in range(reps):  # results are dropped: the recording keeps their blocks
-                call(ring[i % len(ring)])
-        # the core clock dips for some milliseconds when a heavy load starts and then
-        # settles: replay about 15 ms of work before the timed replays
-        for _ in range(max(1, min(60, int(15.0 / max(reps * eager_ms, 1e-3)) + 1))):
-            g.launch()
-        a.record()
-        for _ in range(3):
-            g.launch()
-        b.record()
-        ms = a.elapsed_ms(b) / (3 * reps)
-        g.destroy()
+        ms = eager_ms
+        if replay:
+            # the same `reps` calls recorded once and replayed as one HIP graph: the launch
+            # times without the host work between them (Python here, Lisp in the product)
+            W.lib.synchronize()
+            with W.lib.Graph() as g:
+                for i in range(reps):  # results are dropped: the recording keeps their blocks
+                    call(ring[i % len(ring)])
+            # the core clock dips for some milliseconds when a heavy load starts and then
+            # settles: replay about 15 ms of work before the timed replays
+            for _ in range(max(1, min(60, int(15.0 / max(reps * eager_ms, 1e-3)) + 1))):
+                g.launch()
+            a.record()
+            for _ in range(3):
+                g.launch()
+            b.record()
+            ms = a.elapsed_ms(b) / (3 * reps)
+            g.destroy()
         if bound == "hbm":
             rate, peak, unit = work / ms / 1e6, HBM_PEAK_GBS, "GB/s"
         else:
@@ -436,6 +438,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-block", action="store_true")
+    ap.add_argument("--rows-eager", action="store_true",
+                    help="rows: time the eager calls only, no HIP-graph replay (`ms` = `eager_ms`); for kernel traces")
     ap.add_argument("--no-rows", action="store_true",
                     help="skip the table of the other kernels of the path at their configured shapes")
     ap.add_argument("--probe", action="store_true",
@@ -496,7 +500,7 @@ def main():
         },
     }
     if not args.no_rows:
-        result["rows"] = row_table(W)
+        result["rows"] = row_table(W, replay=not args.rows_eager)
     if not args.no_block:
         blk = block_forward_ms(W)
         if blk is not None:
