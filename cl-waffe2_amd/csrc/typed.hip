@@ -25,6 +25,8 @@
 // when both runs are contiguous (or y is one value), one element per lane with
 // four in flight otherwise.  A destination with incx = 0 accumulates in the
 // reference's order on one lane.
+#include <math.h>
+
 #include <type_traits>
 
 #include "wf2_common.h"
@@ -754,6 +756,154 @@ static int cmp_1d(int op, long n, const T* x, long incx, const T* y, long incy, 
   return run_cmp<T, SCAL>(op, s, x, y, out, ys, then_value, else_value, signed_end);
 }
 
+// ---- :double unary math --------------------------------------------------------
+// out <- f(x) for :double tensors (waffe2_d{sin,...}, cl-waffe2-simd.c:586-706; pow :708-768).
+// The reference mixes SLEEF u10 (blocks of four) and libm (remainder), so its own
+// results vary within an ulp from element to element; here every element goes
+// through the device math library's binary64 routine.
+
+template <int OP>
+__device__ __forceinline__ double dmath(double x, double p) {
+  if constexpr (OP == WF2HIP_SIN) return ::sin(x);
+  else if constexpr (OP == WF2HIP_COS) return ::cos(x);
+  else if constexpr (OP == WF2HIP_TANH) return ::tanh(x);
+  else if constexpr (OP == WF2HIP_LOG) return ::log(x);
+  else if constexpr (OP == WF2HIP_EXP) return ::exp(x);
+  else if constexpr (OP == WF2HIP_SQRT) return ::sqrt(x);
+  else if constexpr (OP == WF2HIP_ABS) return ::fabs(x);
+  else if constexpr (OP == WF2HIP_TAN) return ::tan(x);
+  else if constexpr (OP == WF2HIP_ASIN) return ::asin(x);
+  else if constexpr (OP == WF2HIP_ACOS) return ::acos(x);
+  else if constexpr (OP == WF2HIP_ATAN) return ::atan(x);
+  else if constexpr (OP == WF2HIP_SINH) return ::sinh(x);
+  else if constexpr (OP == WF2HIP_COSH) return ::cosh(x);
+  else if constexpr (OP == WF2HIP_LOG2) return ::log2(x);
+  else if constexpr (OP == WF2HIP_LOG10) return ::log10(x);
+  else if constexpr (OP == WF2HIP_LOG1P) return x == 0.0 ? x : ::log1p(x);  // keeps the sign of -0
+  else if constexpr (OP == WF2HIP_POW) return ::pow(x, p);
+  else return 1.0 / x;  // WF2HIP_INV
+}
+
+// x and out contiguous, 16-byte aligned: two elements per access, four accesses per lane
+template <int OP, bool NT>
+__global__ __launch_bounds__(kBlock) void dunary_flat(const double* __restrict__ x, double* __restrict__ out, size_t nvec,
+                                                      double p) {
+  typedef double d2 __attribute__((ext_vector_type(2)));
+  constexpr int U = 4;
+  const unsigned wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + wave) * kWave * U + lane;
+  const d2* xv = reinterpret_cast<const d2*>(x);
+  d2* ov = reinterpret_cast<d2*>(out);
+  d2 a[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const size_t i = base + (size_t)u * kWave;
+    if (i < nvec) a[u] = NT ? __builtin_nontemporal_load(xv + i) : xv[i];
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const size_t i = base + (size_t)u * kWave;
+    if (i < nvec) {
+      d2 r;
+      r.x = dmath<OP>(a[u].x, p);
+      r.y = dmath<OP>(a[u].y, p);
+      if (NT)
+        __builtin_nontemporal_store(r, ov + i);
+      else
+        ov[i] = r;
+    }
+  }
+}
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void dunary_generic(double* dst, const double* src, TypedGen g, double p) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= g.total) return;
+  int64_t rem = i, d = 0, q = 0;
+  for (int r = g.rank - 1; r > 0; r--) {
+    const int64_t quot = rem / g.shape[r];
+    const int64_t idx = rem - quot * g.shape[r];
+    rem = quot;
+    d += idx * g.sd[r];
+    q += idx * g.ss[r];
+  }
+  d += rem * g.sd[0];
+  q += rem * g.ss[0];
+  dst[d] = dmath<OP>(src[q], p);
+}
+
+// `s`: a = X (source), b = OUT
+template <int OP>
+static int run_dunary(Space s, const double* x, double* out, double p) {
+  if (s.total == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  // a stride-0 axis of OUT keeps what the sequential loop writes last
+  for (int r = 0; r < s.rank; r++)
+    if (s.sb[r] == 0 && s.shape[r] > 1) {
+      s.off_a += s.sa[r] * (s.shape[r] - 1);
+      s.shape[r] = 1;
+    }
+  s.total = 1;
+  for (int r = 0; r < s.rank; r++) s.total *= s.shape[r];
+  normalise(&s);
+  if (typed_overlap(s, x, out, sizeof(double)))
+    return fail(WF2HIP_EOVERLAP, "out partially overlaps x; copy one of them first");
+  hipStream_t st = rt().stream;
+  const double* xp = x + s.off_a;
+  double* op_ = out + s.off_b;
+  int64_t done = 0;
+  if (s.rank == 1 && s.sa[0] == 1 && s.sb[0] == 1 && s.total >= 2 && aligned16(xp) && aligned16(op_)) {
+    const int64_t nvec = s.total / 2;
+    const int64_t blocks = ceil_div(nvec, (int64_t)kBlock * 4);
+    if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+    if (nvec * 32 >= ((int64_t)192 << 20))
+      dunary_flat<OP, true><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, op_, (size_t)nvec, p);
+    else
+      dunary_flat<OP, false><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, op_, (size_t)nvec, p);
+    WF2_TRY(after_launch("dunary_flat"));
+    done = nvec * 2;
+    if (done == s.total) return 0;
+  }
+  TypedGen g;
+  g.rank = s.rank;
+  for (int r = 0; r < s.rank; r++) {
+    g.shape[r] = s.shape[r];
+    g.sd[r] = s.sb[r];
+    g.ss[r] = s.sa[r];
+  }
+  if (done > 0) g.shape[0] = s.total - done;  // the odd last element of a flat run
+  g.total = s.total - done;
+  const int64_t blocks = ceil_div(g.total, kBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+  dunary_generic<OP><<<(uint32_t)blocks, kBlock, 0, st>>>(op_ + done * s.sb[0], xp + done * s.sa[0], g, p);
+  return after_launch("dunary_generic");
+}
+
+static int dispatch_dunary(int op, const Space& s, const double* x, double* out, double p) {
+  switch (op) {
+#define WF2_DUNARY_CASE(OP) case OP: return run_dunary<OP>(s, x, out, p);
+    WF2_DUNARY_CASE(WF2HIP_SIN) WF2_DUNARY_CASE(WF2HIP_COS) WF2_DUNARY_CASE(WF2HIP_TANH) WF2_DUNARY_CASE(WF2HIP_LOG)
+    WF2_DUNARY_CASE(WF2HIP_EXP) WF2_DUNARY_CASE(WF2HIP_SQRT) WF2_DUNARY_CASE(WF2HIP_ABS) WF2_DUNARY_CASE(WF2HIP_TAN)
+    WF2_DUNARY_CASE(WF2HIP_ASIN) WF2_DUNARY_CASE(WF2HIP_ACOS) WF2_DUNARY_CASE(WF2HIP_ATAN) WF2_DUNARY_CASE(WF2HIP_SINH)
+    WF2_DUNARY_CASE(WF2HIP_COSH) WF2_DUNARY_CASE(WF2HIP_LOG2) WF2_DUNARY_CASE(WF2HIP_LOG10)
+    WF2_DUNARY_CASE(WF2HIP_LOG1P) WF2_DUNARY_CASE(WF2HIP_POW)
+#undef WF2_DUNARY_CASE
+    default: return fail(WF2HIP_EINVAL, "unary op %d has no :double kernel", op);
+  }
+}
+
+static int dunary_1d(int op, long n, const double* x, long incx, double* out, long inco, double p) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
+  Space s;
+  s.rank = 1;
+  s.shape[0] = n;
+  s.sa[0] = incx;
+  s.sb[0] = inco;
+  s.total = n;
+  return dispatch_dunary(op, s, x, out, p);
+}
+
 }  // namespace wf2
 
 using namespace wf2;
@@ -882,3 +1032,37 @@ WF2_DEFINE_TYPED_CMPS(i16, int16_t)
 WF2_DEFINE_TYPED_CMPS(u16, uint16_t)
 WF2_DEFINE_TYPED_CMPS(i8, int8_t)
 WF2_DEFINE_TYPED_CMPS(u8, uint8_t)
+
+// OUT <- f(X) on a :double tensor (view: a = X, b = OUT); `p` is the exponent of WF2HIP_POW
+WF2_API int wf2hip_unary_nd_typed(int dtype, int op, const wf2hip_view2* v, const void* x, void* out, double p) {
+  WF2_TRY(require_init());
+  if (dtype != WF2HIP_F64)
+    return fail(WF2HIP_EUNSUPPORTED, "unary math exists for :float and :double only (element type %d)", dtype);
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  return dispatch_dunary(op, s, (const double*)x, (double*)out, p);
+}
+
+#define WF2_DEFINE_DUNARY(name, OP)                                                           \
+  WF2_API int wf2hip_d##name(long n, const double* x, long incx, double* out, long inco) {    \
+    return dunary_1d(OP, n, x, incx, out, inco, 0.0);                                        \
+  }
+WF2_DEFINE_DUNARY(sin, WF2HIP_SIN)
+WF2_DEFINE_DUNARY(cos, WF2HIP_COS)
+WF2_DEFINE_DUNARY(tanh, WF2HIP_TANH)
+WF2_DEFINE_DUNARY(log, WF2HIP_LOG)
+WF2_DEFINE_DUNARY(exp, WF2HIP_EXP)
+WF2_DEFINE_DUNARY(sqrt, WF2HIP_SQRT)
+WF2_DEFINE_DUNARY(abs, WF2HIP_ABS)
+WF2_DEFINE_DUNARY(tan, WF2HIP_TAN)
+WF2_DEFINE_DUNARY(asin, WF2HIP_ASIN)
+WF2_DEFINE_DUNARY(acos, WF2HIP_ACOS)
+WF2_DEFINE_DUNARY(atan, WF2HIP_ATAN)
+WF2_DEFINE_DUNARY(sinh, WF2HIP_SINH)
+WF2_DEFINE_DUNARY(cosh, WF2HIP_COSH)
+WF2_DEFINE_DUNARY(log2, WF2HIP_LOG2)
+WF2_DEFINE_DUNARY(log10, WF2HIP_LOG10)
+WF2_DEFINE_DUNARY(log1p, WF2HIP_LOG1P)
+WF2_API int wf2hip_dpow(long n, const double* x, long incx, double p, double* out, long inco) {
+  return dunary_1d(WF2HIP_POW, n, x, incx, out, inco, p);
+}

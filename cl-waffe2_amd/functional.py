@@ -224,7 +224,7 @@ def _math(node: str, x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
     """``(!exp x :-> out)``: ``out`` defaults to a fresh tensor (the pruned
     ``(!copy x :maybe-in-place t)`` of ``base-impl/mathematics.lisp:13-120``)."""
     if out is None:
-        out = HIPTensor(x.shape, initial_element=None)
+        out = HIPTensor(x.shape, initial_element=None, dtype=x.dtype)
     return nodes.forward(node, x, out)
 
 
@@ -249,7 +249,7 @@ def log1p(x, out=None): return _math("Log1pNode", x, out)
 def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:
     """``(!expt x n)`` (``mathematics.lisp:267-303``)."""
     if out is None:
-        out = HIPTensor(x.shape, initial_element=None)
+        out = HIPTensor(x.shape, initial_element=None, dtype=x.dtype)
     return nodes.forward("ExptNode", x, out, float(n))
 
 

@@ -209,6 +209,12 @@ for _prefix in ("d", "i32", "u32", "i16", "u16", "i8", "u8"):
     for _op in ("max", "min"):
         _SIGNATURES[f"wf2hip_{_prefix}{_op}"] = ([_L, _P, _L, _P], C.c_int)
 
+_SIGNATURES["wf2hip_unary_nd_typed"] = ([C.c_int, C.c_int, C.POINTER(View2), _P, _P, C.c_double], C.c_int)
+for _fn in ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs", "tan", "asin", "acos", "atan", "sinh", "cosh",
+            "log2", "log10", "log1p"):
+    _SIGNATURES[f"wf2hip_d{_fn}"] = ([_L, _P, _L, _P, _L], C.c_int)
+_SIGNATURES["wf2hip_dpow"] = ([_L, _P, _L, C.c_double, _P, _L], C.c_int)
+
 EXPORTS = tuple(_SIGNATURES)
 
 _lib = None

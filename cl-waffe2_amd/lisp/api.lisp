@@ -74,6 +74,8 @@
 (defcfun "wf2hip_compare_nd" :int
   (op :int) (view (:pointer (:struct view3))) (x :pointer) (y :pointer) (out :pointer)
   (then-value :float) (else-value :float))
+(defcfun "wf2hip_unary_nd_typed" :int
+  (dtype :int) (op :int) (view (:pointer (:struct view2))) (x :pointer) (out :pointer) (p :double))
 (defcfun "wf2hip_where_nd_typed" :int
   (dtype :int) (op :int) (view (:pointer (:struct view2))) (x :pointer) (out :pointer)
   (scal :double) (then-value :double) (else-value :double))

@@ -6,6 +6,11 @@
 ;; (source/backends/cpu/arithmetic.lisp:32-144); ExptNode-CPUTensor already uses the run-time
 ;; form (source/backends/cpu/mathematics.lisp:55-76), which is the one followed here.
 
+(defun float-or-double-p (dtype &rest more)
+  "reject-p of the nodes the SIMD extension / BLAS serve for :float and :double only."
+  (declare (ignore more))
+  (not (member dtype '(:float :double))))
+
 (defun only-float-p (dtype &rest more)
   "reject-p: everything but :float falls through to the next device in *using-backend*
 (cf. supported-dtypes-are, source/vm/nodes/utils.lisp:71-93)."
@@ -57,11 +62,17 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
   x)
 
 (defun run-unary (op x out &optional (p 0.0))
+  ":float through the kernels of the hot path, :double through the typed entry point (the SIMD
+extension has both, source/backends/cpu/mathematics.lisp:8-76)."
   (ensure-extension)
   (with-foreign-object (view '(:struct view2))
     (fill-view2 view x out)
-    (check (wf2hip-unary-nd op view (tensor-device-pointer x) (tensor-device-pointer out)
-                            (coerce p 'single-float))))
+    (if (eql (dtype x) :float)
+        (check (wf2hip-unary-nd op view (tensor-device-pointer x) (tensor-device-pointer out)
+                                (coerce p 'single-float)))
+        (check (wf2hip-unary-nd-typed (nth-value 2 (dtype-info (dtype x))) op view
+                                      (tensor-device-pointer x) (tensor-device-pointer out)
+                                      (coerce p 'double-float)))))
   out)
 
 ;; X <- X op Y, returns X (:where A[~] B[~] -> A[~], source/base-impl/arithmetic.lisp:57-103).
@@ -85,7 +96,7 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
 
 ;; OUT <- f(X) (:where X[~] OUT[~] -> OUT[~], source/base-impl/mathematics.lisp:13-120)
 (macrolet ((define-math (node op)
-             `(define-impl-op (,node :device HIPTensor :reject-p #'only-float-p)
+             `(define-impl-op (,node :device HIPTensor :reject-p #'float-or-double-p)
                               :forward ((self x out) (declare (ignore self)) (run-unary ,op x out)))))
   (define-math SinNode +sin+)
   (define-math CosNode +cos+)
@@ -105,7 +116,7 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
   (define-math Log1pNode +log1p+))
 
 ;; OUT <- X^N with N a host ScalarTensor (source/base-impl/mathematics.lisp:267-303)
-(define-impl-op (ExptNode :device HIPTensor :reject-p #'only-float-p)
+(define-impl-op (ExptNode :device HIPTensor :reject-p #'float-or-double-p)
                 :forward ((self x out n)
                           (declare (ignore self))
                           (run-unary +pow+ x out (tensor-vec n))))
@@ -216,10 +227,6 @@ too, source/backends/cpu/arithmetic.lisp:65-123)."
 
 ;; The value nodes take every dtype (waffe2_<prefix>{max,min} on the CPU), the index nodes :float
 ;; and :double (BLAS i?max / i?min, source/backends/cpu/matrix-ops.lisp:254-266).
-(defun float-or-double-p (dtype &rest more)
-  (declare (ignore more))
-  (not (member dtype '(:float :double))))
-
 (macrolet ((define-select (node op reject)
              `(define-impl-op (,node :device HIPTensor :reject-p ,reject)
                               :forward ((self x out) (declare (ignore self)) (run-select ,op x out)))))

@@ -120,11 +120,28 @@ def _binary(op):
     return impl
 
 
+def _float_or_double(dtype) -> bool:
+    """reject-p of the math and index nodes: the SIMD extension and BLAS cover
+    :float and :double (``backends/cpu/mathematics.lisp:8-76``,
+    ``matrix-ops.lisp:254-266``)."""
+    return dtype not in ("float", "double")
+
+
+def _run_unary(op, x: HIPTensor, out: HIPTensor, p: float) -> HIPTensor:
+    if x.dtype != out.dtype:
+        raise ValueError(f"dtype mismatch: {x.dtype} and {out.dtype}")
+    v = view2(x, out)
+    if x.dtype == "float":
+        _lib.check(_lib.get().wf2hip_unary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), p))
+    else:
+        _lib.check(_lib.get().wf2hip_unary_nd_typed(_lib.DTYPE_CODES[x.dtype], op, C.byref(v), C.c_void_p(x.ptr),
+                                                    C.c_void_p(out.ptr), p))
+    return out
+
+
 def _unary(op):
     def impl(x: HIPTensor, out: HIPTensor) -> HIPTensor:
-        v = view2(x, out)
-        _lib.check(_lib.get().wf2hip_unary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), 0.0))
-        return out
+        return _run_unary(op, x, out, 0.0)
 
     return impl
 
@@ -157,14 +174,12 @@ for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _l
                    ("AbsNode", _lib.ABS), ("TanNode", _lib.TAN), ("ASinNode", _lib.ASIN), ("ACosNode", _lib.ACOS),
                    ("ATanNode", _lib.ATAN), ("SinHNode", _lib.SINH), ("CosHNode", _lib.COSH),
                    ("Log2Node", _lib.LOG2), ("Log10Node", _lib.LOG10), ("Log1pNode", _lib.LOG1P)):
-    define_impl(_name, HIPTensor, _only_float)(_unary(_op))
+    define_impl(_name, HIPTensor, _float_or_double)(_unary(_op))
 
 
-@define_impl("ExptNode", HIPTensor, _only_float)
+@define_impl("ExptNode", HIPTensor, _float_or_double)
 def _expt(x: HIPTensor, out: HIPTensor, n: float) -> HIPTensor:
-    v = view2(x, out)
-    _lib.check(_lib.get().wf2hip_unary_nd(_lib.POW, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(n)))
-    return out
+    return _run_unary(_lib.POW, x, out, float(n))
 
 
 _CONDITIONS = {"=": _lib.EQ, "==": _lib.EQ, "<": _lib.LT, "<=": _lib.LE, ">": _lib.GT, ">=": _lib.GE}
@@ -259,12 +274,6 @@ def _select(op, index: bool):
         return out
 
     return impl
-
-
-def _float_or_double(dtype) -> bool:
-    """reject-p of the index nodes: BLAS i?max / i?min exist for :float and :double
-    (``backends/cpu/matrix-ops.lisp:254-266``)."""
-    return dtype not in ("float", "double")
 
 
 # the value nodes take every dtype (waffe2_<prefix>{max,min}, backends/cpu/matrix-ops.lisp:323-369)

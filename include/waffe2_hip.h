@@ -367,6 +367,31 @@ int wf2hip_where_nd(int op, const wf2hip_view2* v, const float* x, float* out, f
 int wf2hip_compare_nd(int op, const wf2hip_view3* v, const float* x, const float* y, float* out,
                       float then_value, float else_value);
 
+/* Unary math on :double tensors: replace waffe2_d{sin,cos,tan,asin,acos,atan,sinh,cosh,
+ * tanh,log,log2,log10,log1p,exp,sqrt,abs} (cl-waffe2-simd.c:586-706, SLEEF u10 on blocks of
+ * four, libm on the remainder) and waffe2_dpow (:708-768), same argument order; `op` of the
+ * N-D form is an enum wf2hip_unary_op (SIN ... POW), view a = X, b = OUT.  Every element
+ * goes through the device math library's binary64 routine: within 2 ulp of SLEEF u10.
+ * Other element types have no unary math in the reference either (WF2HIP_EUNSUPPORTED). */
+int wf2hip_unary_nd_typed(int dtype, int op, const wf2hip_view2* v, const void* x, void* out, double p);
+int wf2hip_dsin(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dcos(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dtanh(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dlog(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dexp(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dsqrt(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dabs(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dtan(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dasin(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dacos(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_datan(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dsinh(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dcosh(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dlog2(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dlog10(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dlog1p(long n, const double* x, long incx, double* out, long inco);
+int wf2hip_dpow(long n, const double* x, long incx, double p, double* out, long inco);
+
 /* Compare-Operation-Node / Where-Operation-Node on the other element types: x, y,
  * out, the scalar and the two constants all have the element type `dtype`
  * (enum wf2hip_dtype).  Replace waffe2_{d,i32,i16,i8,u32,u16,u8}{eq,lt,le,gt,ge}

@@ -488,3 +488,30 @@ def extreme_typed_1d(dtype: str, op: str, n: int, x: np.ndarray, incx: int, use_
         fn.restype = C.c_int
         assert fn(code, int(op == "max"), n, px, incx, C.c_void_p(out.ctypes.data)) == 0
     return out[0]
+
+
+DUNARY_OPS = ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs", "tan", "asin", "acos", "atan", "sinh", "cosh",
+              "log2", "log10", "log1p", "pow")
+
+
+def dunary_1d(op: str, n: int, x: np.ndarray, incx: int, out: np.ndarray, inco: int, p: float = 0.0,
+              use_ref: bool = False, offx: int = 0, offo: int = 0) -> None:
+    """out <- f(x) on binary64 runs (waffe2_d<op>; ``pow`` takes the exponent p)."""
+    assert x.dtype == np.float64 and out.dtype == np.float64
+    px = C.c_void_p(x.ctypes.data + 8 * offx)
+    po = C.c_void_p(out.ctypes.data + 8 * offo)
+    if use_ref:
+        fn = getattr(ref(), f"waffe2_d{op}")
+        if op == "pow":
+            fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_double, C.c_void_p, C.c_long]
+            fn.restype = None
+            fn(n, px, incx, p, po, inco)
+        else:
+            fn.argtypes = [C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long]
+            fn.restype = None
+            fn(n, px, incx, po, inco)
+        return
+    fn = lib().orc_dunary
+    fn.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, C.c_double]
+    fn.restype = C.c_int
+    assert fn(DUNARY_OPS.index(op), n, px, incx, po, inco, p) >= 0

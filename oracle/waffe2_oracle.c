@@ -41,6 +41,9 @@
  *       reference C (waffe2_{d,i32,...}{eq,...} and ..._scal), numpy closed forms
  *       (the element type's own order on the remainder, the signed order on the
  *       leading blocks of the unsigned types).
+ *   orc_dunary                         : golden vectors from the compiled
+ *       reference C (waffe2_d{sin,...,pow}, bit for bit where SLEEF resolves);
+ *       float64 closed forms (numpy / libm within 1 ulp), special values.
  *   orc_extreme_typed                  : golden vectors from the compiled
  *       reference C (waffe2_{d,i32,...}{max,min}), numpy max / min.
  *   orc_sgemm                          : the reference's integer gemm vectors
@@ -882,6 +885,70 @@ ORC_API int orc_extreme_typed(int dtype, int is_max, long n, const void *x, long
     case 7: ORC_EXTREME_LOOP(uint8_t)
     default: return -1;
   }
+}
+
+/* waffe2_d{sin,...} (cl-waffe2-simd.c:586-706 at SIMD_DOUBLE_STRIDE = 4): blocks of four
+ * through Sleef_<f>d4_u10avx2 (avx2.h:264-331; sqrt u05, fabs exact) when incx >= 1, the
+ * remainder -- and everything when incx < 1 -- through libm.  op: 0 sin 1 cos 2 tanh 3 log
+ * 4 exp 5 sqrt 6 abs 7 tan 8 asin 9 acos 10 atan 11 sinh 12 cosh 13 log2 14 log10 15 log1p
+ * 16 pow (waffe2_dpow, :708-768, Sleef_powd4_u10avx2 / pow). */
+typedef double v4d __attribute__((vector_size(32)));
+typedef v4d (*sleef_d4_1)(v4d);
+typedef v4d (*sleef_d4_2)(v4d, v4d);
+
+static const char *const orc_dnames[17] = {
+    "Sleef_sind4_u10avx2",  "Sleef_cosd4_u10avx2",  "Sleef_tanhd4_u10avx2",  "Sleef_logd4_u10avx2",
+    "Sleef_expd4_u10avx2",  "Sleef_sqrtd4_u05avx2", "Sleef_fabsd4_avx2",     "Sleef_tand4_u10avx2",
+    "Sleef_asind4_u10avx2", "Sleef_acosd4_u10avx2", "Sleef_atand4_u10avx2",  "Sleef_sinhd4_u10avx2",
+    "Sleef_coshd4_u10avx2", "Sleef_log2d4_u10avx2", "Sleef_log10d4_u10avx2", "Sleef_log1pd4_u10avx2",
+    "Sleef_powd4_u10avx2"};
+
+static double orc_dlibm(int op, double x, double p) {
+  switch (op) {
+    case 0: return sin(x);
+    case 1: return cos(x);
+    case 2: return tanh(x);
+    case 3: return log(x);
+    case 4: return exp(x);
+    case 5: return sqrt(x);
+    case 6: return fabs(x);
+    case 7: return tan(x);
+    case 8: return asin(x);
+    case 9: return acos(x);
+    case 10: return atan(x);
+    case 11: return sinh(x);
+    case 12: return cosh(x);
+    case 13: return log2(x);
+    case 14: return log10(x);
+    case 15: return log1p(x);
+    default: return pow(x, p);
+  }
+}
+
+/* returns 1 when the blocks went through SLEEF, 0 when libm stood in, -1 on a bad op */
+ORC_API int orc_dunary(int op, long n, const double *x, long incx, double *out, long inco, double p) {
+  if (op < 0 || op > 16) return -1;
+  void *sym = sleef_sym(orc_dnames[op]);
+  long count = 0;
+  if (incx >= 1) {
+    const long blocks_end = (n / 4) * 4;
+    for (; count != blocks_end; count += 4) {
+      double in[4], res[4];
+      for (int l = 0; l < 4; l++) in[l] = x[(count + l) * incx];
+      if (sym) {
+        v4d v, pv, r;
+        memcpy(&v, in, sizeof v);
+        for (int l = 0; l < 4; l++) pv[l] = p;
+        r = op == 16 ? ((sleef_d4_2)sym)(v, pv) : ((sleef_d4_1)sym)(v);
+        memcpy(res, &r, sizeof r);
+      } else {
+        for (int l = 0; l < 4; l++) res[l] = orc_dlibm(op, in[l], p);
+      }
+      for (int l = 0; l < 4; l++) out[(count + l) * inco] = res[l];
+    }
+  }
+  for (; count != n; count++) out[count * inco] = orc_dlibm(op, x[count * incx], p);
+  return sym ? 1 : 0;
 }
 
 ORC_API int orc_abi_version(void) { return 1; }

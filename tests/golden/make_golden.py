@@ -395,6 +395,47 @@ def extreme_typed_goldens():
     print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "typed_extreme_kernels.npz")), "bytes")
 
 
+def dunary_inputs(rng, op, size):
+    """Arguments inside each function's domain, a few special values at the end."""
+    if op in ("asin", "acos"):
+        x = rng.uniform(-1, 1, size)
+    elif op in ("log", "log2", "log10", "sqrt"):
+        x = np.exp(rng.uniform(-30, 30, size))
+    elif op == "log1p":
+        x = np.expm1(rng.uniform(-20, 20, size))
+    elif op in ("exp", "sinh", "cosh"):
+        x = rng.uniform(-40, 40, size)
+    elif op in ("sin", "cos", "tan"):
+        x = rng.uniform(-1, 1, size) * 10.0 ** rng.integers(-3, 6, size)
+    elif op == "pow":
+        x = np.exp(rng.uniform(-5, 5, size))
+    else:
+        x = rng.uniform(-20, 20, size)
+    return x
+
+
+def dunary_goldens():
+    """waffe2_d{sin,...,pow} of the compiled reference: SLEEF u10 on the blocks of
+    four, libm on the remainder (both as this image has them)."""
+    assert O.ref() is not None, "oracle/_ref/libwaffe2_simd_ref.so is missing: run `make -C oracle ref`"
+    rng = np.random.Generator(np.random.PCG64(2031))
+    out = {}
+    for op in O.DUNARY_OPS:
+        xs, outs, cases, start = [], [], [], 0
+        for n, incx, inco in [(1, 1, 1), (4, 1, 1), (23, 1, 1), (64, 1, 1), (13, 2, 1), (13, 1, 3), (9, 3, 2), (7, 0, 1)]:
+            size = n * 3 + 1
+            x = dunary_inputs(rng, op, size)
+            res = np.full(size, 7.0)
+            O.dunary_1d(op, n, x, incx, res, inco, p=2.5, use_ref=True)
+            xs.append(x), outs.append(res)
+            cases.append((n, incx, inco, start, size))
+            start += size
+        out[f"{op}_x"], out[f"{op}_out"] = np.concatenate(xs), np.concatenate(outs)
+        out[f"{op}_cases"] = np.array(cases, np.int64)
+    np.savez_compressed(os.path.join(HERE, "double_unary_kernels.npz"), **out)
+    print("wrote", len(out), "arrays,", os.path.getsize(os.path.join(HERE, "double_unary_kernels.npz")), "bytes")
+
+
 if __name__ == "__main__":
     if "--im2col-only" in sys.argv:
         im2col_goldens()
@@ -408,6 +449,8 @@ if __name__ == "__main__":
         compare_typed_goldens()
     elif "--typed-extreme-only" in sys.argv:
         extreme_typed_goldens()
+    elif "--double-unary-only" in sys.argv:
+        dunary_goldens()
     else:
         main()
         compare_goldens()
@@ -416,3 +459,4 @@ if __name__ == "__main__":
         typed_goldens()
         compare_typed_goldens()
         extreme_typed_goldens()
+        dunary_goldens()
