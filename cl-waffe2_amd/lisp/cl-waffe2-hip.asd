@@ -15,4 +15,5 @@
                (:file "shared-object")
                (:file "api")
                (:file "tensor")
-               (:file "kernels")))
+               (:file "kernels")
+               (:file "fusion")))

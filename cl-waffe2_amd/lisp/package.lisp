@@ -12,7 +12,8 @@ kernels are the hand-written gfx950 kernels of libwaffe2-hip.so.")
    #:hip-synchronize
    #:with-sequential-reductions
    #:with-captured-graph
-   #:hip-error))
+   #:hip-error
+   #:!relu-hip #:!leaky-relu-hip #:!sigmoid-hip #:!gelu-hip #:!softmax-hip #:!layer-norm-hip))
 
 (in-package :cl-waffe2/backends.hip)
 
