@@ -379,6 +379,67 @@ __global__ __launch_bounds__(kBlock) void ew_stride2(RowsParams p, F f) {
   }
 }
 
+// ---- stride-2 source into contiguous rows -------------------------------------
+// x <- x op y (or x <- f(y)) where y takes every second element of its rows and x is
+// contiguous: the copy cl-waffe2 makes of a [::2] slice before any out-of-place
+// op on it.  Each thread reads the 32 contiguous bytes that hold its four source
+// elements as two aligned float4 loads (every fetched sector is used in full by
+// the wavefront; with 4-byte gathers the slice copy of (4096, 8192) sits at 70 %
+// of the sector traffic's roofline) and writes one float4.  `odd` says whether the
+// wanted elements are lanes 1, 3 or 0, 2 of the vectors; the launcher only takes
+// rows whose storage starts 0 or 1 floats past a 16-byte boundary.
+template <class F, bool ReadDst, bool NT>
+__global__ __launch_bounds__(kBlock) void ew_gather2(RowsParams p, F f, int odd) {
+  constexpr int U = 2;
+  const uint32_t row = blockIdx.x / p.chunks_per_row;
+  const uint32_t chunk = blockIdx.x - row * p.chunks_per_row;
+  int64_t doff = 0, soff = 0;
+  uint32_t rem = row;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t idx;
+    if (i == p.nouter - 1) {
+      idx = rem;
+    } else {
+      uint32_t q = rem / p.oshape[i];
+      idx = rem - q * p.oshape[i];
+      rem = q;
+    }
+    doff += (int64_t)idx * p.odst[i];
+    soff += (int64_t)idx * p.osrc[i];
+  }
+  float* d = p.dst + doff;
+  const float* s = p.src + soff - odd;  // 16-byte aligned
+  const int64_t nvec = p.n0 / 4;
+  f4 lo[U], hi[U], old[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const int64_t v = ((int64_t)chunk * U + u) * kBlock + threadIdx.x;
+    if (v < nvec) {
+      lo[u] = load4<NT>(s + 8 * v);
+      hi[u] = load4<NT>(s + 8 * v + 4);
+      if (ReadDst) old[u] = load4<NT>(d + 4 * v);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const int64_t v = ((int64_t)chunk * U + u) * kBlock + threadIdx.x;
+    if (v < nvec) {
+      f4 y = odd ? f4{lo[u].y, lo[u].w, hi[u].y, hi[u].w} : f4{lo[u].x, lo[u].z, hi[u].x, hi[u].z};
+      f4 o;
+      o.x = f(ReadDst ? old[u].x : 0.0f, y.x);
+      o.y = f(ReadDst ? old[u].y : 0.0f, y.y);
+      o.z = f(ReadDst ? old[u].z : 0.0f, y.z);
+      o.w = f(ReadDst ? old[u].w : 0.0f, y.w);
+      store4<NT>(d + 4 * v, o);
+    }
+  }
+  // the last n0 % 4 elements of the row
+  if (chunk == 0 && threadIdx.x < (p.n0 & 3)) {
+    const int64_t c = nvec * 4 + threadIdx.x;
+    d[c] = f(ReadDst ? d[c] : 0.0f, s[2 * c + odd]);
+  }
+}
+
 // ---- generic kernel -----------------------------------------------------------
 struct GenParams {
   float* dst;
@@ -872,6 +933,45 @@ static bool try_launch_stride2(const Space& s, float* dst, const float* src, F f
   }
 }
 
+// Contiguous destination rows, source rows of stride 2.
+template <class F, bool ReadDst>
+static bool try_launch_gather2(const Space& s, float* dst, const float* src, F f, int* rc) {
+  const int last = s.rank - 1;
+  const int64_t n0 = s.shape[last];
+  if (s.sa[last] != 1 || s.sb[last] != 2 || n0 < 128 || s.rank - 1 > kMaxOuter) return false;
+  RowsParams p;
+  p.dst = dst + s.off_a;
+  p.src = src + s.off_b;
+  const int lead = (int)(((uintptr_t)p.src >> 2) & 3);  // floats past a 16-byte boundary
+  if (lead > 1 || !aligned16(p.dst)) return false;
+  p.n0 = n0;
+  p.src_inner = 2;
+  p.nouter = 0;
+  p.tpr_log2 = 8;
+  int64_t nrows = 1;
+  for (int r = last - 1; r >= 0; r--) {
+    if (s.shape[r] >= ((int64_t)1 << 32)) return false;
+    if (s.shape[r] > 1 && (s.sa[r] % 4 != 0 || s.sb[r] % 4 != 0)) return false;  // every row as aligned as the first
+    p.oshape[p.nouter] = (uint32_t)s.shape[r];
+    p.odst[p.nouter] = s.sa[r];
+    p.osrc[p.nouter] = s.sb[r];
+    p.nouter++;
+    nrows *= s.shape[r];
+  }
+  const int64_t chunks = ceil_div(n0 / 4 > 0 ? n0 / 4 : 1, (int64_t)kBlock * 2);
+  if (nrows * chunks >= ((int64_t)1 << 31)) return false;
+  p.nrows = (uint32_t)nrows;
+  p.chunks_per_row = (uint32_t)chunks;
+  const uint32_t blocks = (uint32_t)(nrows * chunks);
+  const bool nt = s.total * (ReadDst ? 16 : 12) >= kStreamingBytes;
+  if (nt)
+    ew_gather2<F, ReadDst, true><<<blocks, kBlock, 0, rt().stream>>>(p, f, lead);
+  else
+    ew_gather2<F, ReadDst, false><<<blocks, kBlock, 0, rt().stream>>>(p, f, lead);
+  *rc = after_launch("ew_gather2");
+  return true;
+}
+
 // `s` describes dst through (sa, off_a) and src through (sb, off_b); dst has
 // no broadcast axis.
 template <class F, bool ReadDst>
@@ -890,6 +990,7 @@ static int launch_elementwise(const Space& s, float* dst, const float* src, F f)
   int rc = 0;
   if (try_launch_tile<F, ReadDst>(s, dst, src, f, &rc)) return rc;
   if (try_launch_stride2<F, ReadDst>(s, dst, src, f, &rc)) return rc;
+  if (try_launch_gather2<F, ReadDst>(s, dst, src, f, &rc)) return rc;
   return launch_generic<F, ReadDst>(s, dst, src, f);
 }
 

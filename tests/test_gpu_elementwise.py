@@ -121,6 +121,38 @@ def test_config2_views(gpu, O):
     assert_bit_equal(got.numpy(), A[1024:3072] - A[0:2048], "offset views")
 
 
+def test_every_second_element_as_source(gpu):
+    """A [::2] slice read into contiguous rows -- the copy behind every out-of-place
+    op on such a view (two aligned 16-byte loads per four elements when the rows
+    start 0 or 1 floats past a 16-byte boundary, the generic kernel otherwise):
+    copies, in-place ops with the slice on the right, unary math; row lengths that
+    are and are not multiples of four.  Closed form: numpy in binary32."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(79)
+    f32 = np.float32
+    for rows, pitch, start, count in [(9, 1000, 0, 500), (7, 1004, 1, 450), (5, 4100, 0, 2049), (3, 4100, 1, 131),
+                                      (4, 1000, 2, 256), (6, 1001, 0, 400), (1, 70004, 1, 35001), (2, 2048, 3, 1000)]:
+        base = rng.standard_normal((rows, pitch)).astype(f32)
+        want_slice = base[:, start:start + 2 * count:2]
+        t = F.from_numpy(base)
+        v = t.view(True, (start, start + 2 * count, 2))
+        assert v.shape == [rows, count]
+        assert_bit_equal(F.copy(v).numpy(), want_slice, f"copy of [::2], rows {rows} pitch {pitch} start {start}")
+        acc = rng.standard_normal((rows, count)).astype(f32)
+        got = F.sub_(F.from_numpy(acc), v)
+        assert_bit_equal(got.numpy(), acc - want_slice, f"x -= [::2], rows {rows} pitch {pitch} start {start}")
+        got = F.mul(v, 0.5)  # the configured case: a copy of the slice, then the scalar product in place
+        assert_bit_equal(got.numpy(), want_slice * f32(0.5), "0.5 * [::2]")
+        got = F.abs(v)
+        assert_bit_equal(got.numpy(), np.abs(want_slice), "abs of [::2]")
+        assert_bit_equal(t.numpy(), base, "the source is untouched")
+    # a 3-D source: slices of every matrix of a batch
+    base = rng.standard_normal((3, 6, 520)).astype(f32)
+    v = F.from_numpy(base).view(True, (1, 5), (0, 520, 2))
+    assert_bit_equal(F.copy(v).numpy(), base[:, 1:5, 0:520:2], "3-D [::2] source")
+
+
 def test_inplace_on_every_second_element(gpu):
     """In-place ops on [::2] slices (the kernel that stores whole vectors and
     writes the in-between elements back as read): row pitches and start columns
