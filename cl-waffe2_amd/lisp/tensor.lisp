@@ -136,3 +136,39 @@ element type is DTYPE's host type (single-float for :float, (unsigned-byte 8) fo
     (with-pointer-to-vector-data (p storage)
       (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor) p (* (dtype-bytes dtype) (length storage)))))
     tensor))
+
+;; The other directions of convert-tensor-facet / device-as (source/array-converter.lisp:93-151).
+;; As with CPUTensor, 'simple-array and 'array expose the whole storage vector in storage order;
+;; views and permutations are properties of the tensor, not of its storage.
+(defmethod cl-waffe2:convert-tensor-facet ((from HIPTensor) (to (eql 'array)))
+  (make-array (cl-waffe2/vm.generic-tensor::original-shape from)
+              :element-type (dtype-lisp-type (dtype from))
+              :displaced-to (cl-waffe2:convert-tensor-facet from 'simple-array)
+              :displaced-index-offset 0))
+
+(defun host-tensor-from (tensor device)
+  "A DEVICE (CPUTensor / LispTensor) tensor of TENSOR's original shape over a downloaded copy of
+its storage."
+  (let ((*using-backend* (list device)))
+    (cl-waffe2/vm.generic-tensor::make-tensor-from-vec
+     (cl-waffe2/vm.generic-tensor::original-shape tensor) (dtype tensor)
+     (cl-waffe2:convert-tensor-facet tensor 'simple-array)
+     :order (order tensor))))
+
+(defmethod cl-waffe2:convert-tensor-facet ((from HIPTensor) (to (eql 'cl-waffe2/backends.cpu:CPUTensor)))
+  (host-tensor-from from 'cl-waffe2/backends.cpu:CPUTensor))
+
+(defmethod cl-waffe2:convert-tensor-facet ((from HIPTensor) (to (eql 'cl-waffe2/backends.lisp:LispTensor)))
+  (host-tensor-from from 'cl-waffe2/backends.lisp:LispTensor))
+
+(defmethod cl-waffe2:convert-tensor-facet ((from AbstractTensor) (to (eql 'HIPTensor)))
+  "(device-as tensor 'HIPTensor): one bulk copy of the host tensor's storage vector."
+  (if (typep from 'HIPTensor)
+      from
+      (let* ((storage (cl-waffe2:convert-tensor-facet from 'simple-array))
+             (tensor (make-tensor (cl-waffe2/vm.generic-tensor::original-shape from)
+                                  :dtype (dtype from) :order (order from) :device 'HIPTensor)))
+        (with-pointer-to-vector-data (p storage)
+          (check (wf2hip-memcpy-h2d (tensor-device-pointer tensor) p
+                                    (* (dtype-bytes (dtype from)) (length storage)))))
+        tensor)))
