@@ -454,6 +454,51 @@ __global__ __launch_bounds__(kBlock) void typed_accumulate_add(T* a, const T* b,
   }
 }
 
+// Few destinations, long reductions: `splits` workgroups per destination each sum a
+// contiguous range of the reduced index space into `partials`, a second launch folds
+// them in a fixed order (deterministic for :double, exact for the integer types).
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_partial(const T* b, TypedAcc p, uint32_t splits, int64_t seg,
+                                                                   typename SumOf<T>::type* partials) {
+  using S = typename SumOf<T>::type;
+  __shared__ S lds[kBlock / kWave];
+  const int64_t out = blockIdx.x / splits;
+  const uint32_t split = blockIdx.x - (uint32_t)out * splits;
+  int64_t aoff, boff;
+  acc_kept(p, out, &aoff, &boff);
+  const int64_t lo = (int64_t)split * seg;
+  const int64_t hi = lo + seg < p.nred ? lo + seg : p.nred;
+  S acc = S(0);
+  if (p.nr == 1) {
+    for (int64_t j = lo + threadIdx.x; j < hi; j += kBlock) acc += (S)b[boff + j * p.rb[0]];
+  } else {
+    for (int64_t j = lo + threadIdx.x; j < hi; j += kBlock) acc += (S)b[boff + acc_reduced(p, j)];
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    S total = lds[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; w++) total += lds[w];
+    partials[blockIdx.x] = total;
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(kWave) void typed_accumulate_fold(T* a, TypedAcc p, uint32_t splits,
+                                                               const typename SumOf<T>::type* partials) {
+  using S = typename SumOf<T>::type;
+  const int64_t out = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  if (out >= p.nout) return;
+  int64_t aoff, boff;
+  acc_kept(p, out, &aoff, &boff);
+  S total = S(0);
+  for (uint32_t s = 0; s < splits; s++) total += partials[out * splits + s];
+  a[aoff] = (T)((S)a[aoff] + total);
+}
+
 template <class T, int OP>
 __global__ __launch_bounds__(kBlock) void typed_accumulate_sequential(T* a, const T* b, TypedAcc p) {
   const int64_t out = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -495,6 +540,22 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
   const T* bp = b + s.off_b;
   if (op == WF2HIP_ADD && rt().reduce_mode == 0) {
     if (p.nout >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+    using S = typename SumOf<T>::type;
+    const int64_t target = (int64_t)rt().num_cus * 8;
+    const int64_t capacity = (int64_t)(kPartialCapacity * sizeof(float) / sizeof(S));
+    if (p.nout < target && p.nred >= 2 * 16384 && p.nout <= capacity / 2) {
+      int64_t splits = ceil_div(p.nred, 16384);
+      const int64_t by_fill = ceil_div(target, p.nout), by_cap = capacity / p.nout;
+      if (splits > by_fill) splits = by_fill;
+      if (splits > by_cap) splits = by_cap;
+      const int64_t seg = ceil_div(p.nred, splits);
+      splits = ceil_div(p.nred, seg);
+      S* partials = reinterpret_cast<S*>(rt().partials);
+      typed_accumulate_partial<T><<<(uint32_t)(p.nout * splits), kBlock, 0, st>>>(bp, p, (uint32_t)splits, seg, partials);
+      WF2_TRY(after_launch("typed_accumulate_partial"));
+      typed_accumulate_fold<T><<<(uint32_t)ceil_div(p.nout, kWave), kWave, 0, st>>>(ap, p, (uint32_t)splits, partials);
+      return after_launch("typed_accumulate_fold");
+    }
     typed_accumulate_add<T><<<(uint32_t)p.nout, kBlock, 0, st>>>(ap, bp, p);
     return after_launch("typed_accumulate_add");
   }

@@ -182,6 +182,17 @@ def test_accumulation_into_broadcast_destinations(gpu, dtype):
             assert np.max(np.abs(got.numpy() - want)) < 1e-11
         else:
             np.testing.assert_array_equal(got.numpy(), want)
+        # long reductions into few destinations (the split kernel): a full sum and two column sums
+        big = (rng.standard_normal((2, 150001)) if dtype == "double"
+               else rng.integers(info.min, info.max, (2, 150001), endpoint=True).astype(npt))
+        dbig = F.from_numpy(big, dtype=dtype)
+        for axis in ((0, 1), 1):
+            got = F.sum(dbig, axis=axis)
+            want = big.sum(axis=axis, keepdims=True, dtype=npt if dtype != "double" else np.float64)
+            if dtype == "double":
+                assert np.max(np.abs(got.numpy() - want)) < 1e-9
+            else:
+                np.testing.assert_array_equal(got.numpy(), want)
         # x[0, j] <- x[0, j] - sum_i y[i, j], sequentially
         base = A[0, 0:1, :].copy()
         dst = F.from_numpy(base, dtype=dtype).view((":broadcast", 300), True)
