@@ -1,6 +1,8 @@
-// typed.hip -- AddNode / SubNode / MulNode / DivNode / MoveTensorNode and inv
-// for the element types of cl-waffe2 other than :float -- :double, :int32,
-// :uint32, :int16, :uint16, :int8, :uint8.
+// typed.hip -- the element types of cl-waffe2 other than :float -- :double, :int32,
+// :uint32, :int16, :uint16, :int8, :uint8: AddNode / SubNode / MulNode / DivNode /
+// MoveTensorNode and inv (below), accumulation into broadcast destinations (!sum),
+// Compare- / Where-Operation-Node, and unary math on :double, each introduced by its
+// own section comment.  MaxValue / MinValue / ArgMax / ArgMin live in rowselect.hip.
 //
 // Reference: waffe2_d{add,sub,mul,div} (the AVX2 macro of
 // cl-waffe2-simd.c:153-213 instantiated at :247-250), the scalar loops
