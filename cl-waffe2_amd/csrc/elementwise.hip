@@ -596,8 +596,10 @@ __global__ __launch_bounds__(kBlock) void ew_tile(TileParams p, F f) {
 constexpr int kBigTile = 128;
 constexpr int kBigTileFloats = kBigTile * (kBigTile + 1) + 4;
 
-template <class F, bool ReadDst, bool NT>
-__global__ __launch_bounds__(kBlock) void ew_tile128(TileParams p, F f) {
+template <class F, bool ReadDst, bool NT, int THREADS>
+__global__ __launch_bounds__(THREADS) void ew_tile128(TileParams p, F f) {
+  constexpr int kWaves = THREADS / kWave;  // 4 or 16
+  constexpr int kPasses = 64 / kWaves;     // row groups per wavefront: 16 or 4
   extern __shared__ float big_tile[];
   uint32_t bid = blockIdx.x;
   const uint32_t ti = bid % p.tiles_i;
@@ -618,21 +620,21 @@ __global__ __launch_bounds__(kBlock) void ew_tile128(TileParams p, F f) {
   const int wave = threadIdx.x / kWave;
   const int q4 = (lane & 31) * 4;       // position along the contiguous axis
   const int rr = 2 * (lane >> 5);       // the two half-waves take rows two apart
-  auto row_of = [&](int pass) {         // pass 0..15: rows 4 (g / 2) + g % 2 + {0, 2}, g = 4 pass + wave
-    const int g = 4 * pass + wave;
+  auto row_of = [&](int pass) {         // rows 4 (g / 2) + g % 2 + {0, 2}, g = kWaves pass + wave in 0..63
+    const int g = kWaves * pass + wave;
     return 4 * (g >> 1) + (g & 1) + rr;
   };
   auto at = [](int a, int b) { return a * (kBigTile + 1) + b + (a >> 6) + (b >> 6); };
-  f4 v[16];
+  f4 v[kPasses];
 #pragma unroll
-  for (int pass = 0; pass < 16; pass++) {
+  for (int pass = 0; pass < kPasses; pass++) {
     const int r = row_of(pass);
     const int64_t i = i0 + r, j = j0 + q4;
     v[pass] = f4{0.f, 0.f, 0.f, 0.f};
     if (i < p.ni && j < p.nj) v[pass] = load4<NT>(p.src + soff + i * p.s_i + j);
   }
 #pragma unroll
-  for (int pass = 0; pass < 16; pass++) {
+  for (int pass = 0; pass < kPasses; pass++) {
     const int r = row_of(pass);
     big_tile[at(r, q4 + 0)] = v[pass].x;
     big_tile[at(r, q4 + 1)] = v[pass].y;
@@ -641,7 +643,7 @@ __global__ __launch_bounds__(kBlock) void ew_tile128(TileParams p, F f) {
   }
   __syncthreads();
 #pragma unroll
-  for (int batch = 0; batch < 4; batch++) {
+  for (int batch = 0; batch < kPasses / 4; batch++) {
     f4 a[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
@@ -666,17 +668,23 @@ __global__ __launch_bounds__(kBlock) void ew_tile128(TileParams p, F f) {
   }
 }
 
+// Sixteen wavefronts per tile: the 66 KB tile allows two workgroups per compute
+// unit whatever their width, so a wide workgroup is what puts enough loads in
+// flight (transposing copy of (8192, 8192): 256 threads 104.1 us, 512 100.1 us,
+// 1024 94.8 us).
+constexpr int kBigTileThreads = 1024;
+
 template <class F, bool ReadDst, bool NT>
 static int launch_tile128(const TileParams& p, uint32_t blocks, F f) {
   constexpr int bytes = kBigTileFloats * (int)sizeof(float);
   static bool configured = false;  // per instantiation
   if (!configured) {
-    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&ew_tile128<F, ReadDst, NT>),
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&ew_tile128<F, ReadDst, NT, kBigTileThreads>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes),
                       "hipFuncSetAttribute(ew_tile128)"));
     configured = true;
   }
-  ew_tile128<F, ReadDst, NT><<<blocks, kBlock, bytes, rt().stream>>>(p, f);
+  ew_tile128<F, ReadDst, NT, kBigTileThreads><<<blocks, kBigTileThreads, bytes, rt().stream>>>(p, f);
   return 0;
 }
 
