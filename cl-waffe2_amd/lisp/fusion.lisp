@@ -5,8 +5,10 @@
 ;;;; node.  The library holds each of them as one kernel; this file makes them reachable the way
 ;;;; the reference intends device-specific fusions to be added:
 ;;;;   * a define-op node per fused kernel (as Softmax-Cross-Entropy-Node, source/nn/criterion.lisp:90),
-;;;;     forward = one library call, backward = the derivative composed from ordinary ! functions,
-;;;;     so it runs on the device through the nodes of kernels.lisp;
+;;;;     forward = one library call, backward = the derivative composed from ordinary ! functions
+;;;;     and evaluated with proceed, so it runs on the device through the nodes of kernels.lisp
+;;;;     (a graph is compiled per backward call: the fused nodes pay off in inference and in
+;;;;     forward-heavy training; a defmodel-as cache is the next step);
 ;;;;   * a define-bypass rule per function (source/vm/nodes/symbolic.lisp:118-131): with HIPTensor
 ;;;;     in *using-backend*, calls of cl-waffe2/nn:!relu & co. compiled after this file is loaded
 ;;;;     build the fused node instead ((setf *enable-symbolic-path* nil) switches that off).
@@ -40,7 +42,10 @@ DERIVATIVE is a function of (x) returning df/dx built from ! functions."
                         (run-unary (activation-op self) x out (activation-parameter self))))
             :backward ((self dout)
                        (with-reading-save4bw ((x x))
-                         (values (!mul dout (funcall (activation-derivative self) x)) nil))))
+                         ;; the body of a define-op backward runs eagerly (it is the forward of the
+                         ;; generated -backward node, source/vm/nodes/static-node.lisp:296-318), so
+                         ;; the composed derivative is evaluated here with proceed
+                         (values (proceed (!mul dout (funcall (activation-derivative self) x))) nil))))
   (setf (activation-op self) op
         (activation-parameter self) p
         (activation-derivative self) derivative))
@@ -105,7 +110,7 @@ DERIVATIVE is a function of (x) returning df/dx built from ! functions."
                        ;; dx = y * (dy - sum(dy * y) over the row)
                        (with-reading-save4bw ((y y))
                          (let ((dot (!sum (!mul dout y) :axis 1 :keepdims t)))
-                           (values (!mul y (!sub dout dot)) nil))))))
+                           (values (proceed (!mul y (!sub dout dot))) nil))))))
 
 (defun !softmax-hip (x &key (avoid-overflow t) (axis 1))
   "(!softmax x :axis 1) on a contiguous :float matrix as one kernel; anything else takes the
