@@ -181,13 +181,13 @@ __global__ __launch_bounds__(kStreamBlock) void reduce_rows_stream(RowRedParams 
 }
 
 // One wavefront per row, four rows per workgroup.
-template <int VEC>
+template <int VEC, bool NT = false>
 __global__ __launch_bounds__(kBlock) void reduce_rows_wave(RowRedParams p) {
   const uint32_t row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (row >= p.nrows) return;
   int64_t aoff, boff;
   row_offsets(p, row, &aoff, &boff);
-  double v = strided_sum<VEC>(p.b + boff, 0, p.n0, threadIdx.x & (kWave - 1), kWave);
+  double v = strided_sum<VEC, NT>(p.b + boff, 0, p.n0, threadIdx.x & (kWave - 1), kWave);
   v = wave_sum(v);
   if ((threadIdx.x & (kWave - 1)) == 0) p.a[aoff] = (float)((double)p.a[aoff] + v);
 }
@@ -323,7 +323,10 @@ static int launch_row_reduce(const Space& s, float* a, const float* b) {
     // short rows: a wavefront each
     if (nrows >= target_blocks || p.n0 < 8192) {
       uint32_t blocks = (uint32_t)ceil_div(nrows, kWavesPerBlock);
-      if (vec_ok)
+      // nontemporal loads beyond the Infinity Cache: (65536, 1024) 40.8 us against 44.4 us
+      if (vec_ok && nrows * p.n0 * 4 >= ((int64_t)192 << 20))
+        reduce_rows_wave<4, true><<<blocks, kBlock, 0, st>>>(p);
+      else if (vec_ok)
         reduce_rows_wave<4><<<blocks, kBlock, 0, st>>>(p);
       else
         reduce_rows_wave<1><<<blocks, kBlock, 0, st>>>(p);
@@ -346,8 +349,16 @@ static int launch_row_reduce(const Space& s, float* a, const float* b) {
   if (blocks >= ((int64_t)1 << 31))
     return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
   // far beyond the Infinity Cache: stream with non-temporal loads
-  if (vec_ok && nrows * p.n0 * 4 >= ((int64_t)192 << 20))
+  // Footprints that do not stay in the 256 MB Infinity Cache: rows (or row segments) of
+  // 4096 elements and more through the streaming kernel; shorter ones, which do not fill
+  // one of its 4096-element batches, through the 256-thread kernel.  Measured cold,
+  // (32768, 2048): 42.1 us against 67.1 us through the streaming kernel; (16384, 4096):
+  // 39.2 us streaming against 45.5 us; (8192, 4096), 128 MiB: 21.6 us against 24.4 us.
+  const int64_t bytes = nrows * p.n0 * 4;
+  if (vec_ok && p.seg >= 4096 && bytes >= ((int64_t)128 << 20))
     reduce_rows_stream<<<(uint32_t)blocks, kStreamBlock, 0, st>>>(p);
+  else if (vec_ok && bytes >= ((int64_t)192 << 20))  // nontemporal loads: (32768, 2048) 39.0 us against 41.7 us
+    reduce_rows_block<4, true><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   else if (vec_ok)
     reduce_rows_block<4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   else
