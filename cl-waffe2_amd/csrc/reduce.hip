@@ -643,6 +643,37 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __res
   r.store(out + row * ncols, ncols, lane);
 }
 
+// Rows beyond the register tile (2048 columns): a workgroup per row, three passes
+// over the row (sum, squared deviations, output); the second and third come from
+// the L2 the first one filled.  Same arithmetic as the wavefront form.
+__global__ __launch_bounds__(kBlock) void layernorm_rows_block(const float* __restrict__ x,
+                                                               const float* __restrict__ gamma,
+                                                               const float* __restrict__ beta, float eps,
+                                                               float* __restrict__ out, int64_t ncols) {
+  __shared__ double lds[kWavesPerBlock];
+  __shared__ double stat;
+  const float* xr = x + (int64_t)blockIdx.x * ncols;
+  float* outr = out + (int64_t)blockIdx.x * ncols;
+  double sum = 0.0;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) sum += (double)xr[c];
+  double total = block_sum(sum, lds);
+  if (threadIdx.x == 0) stat = total / (double)ncols;
+  __syncthreads();
+  const double mean = stat;
+  double sq = 0.0;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
+    const double d = (double)xr[c] - mean;
+    sq += d * d;
+  }
+  __syncthreads();  // everyone has read `stat` and is done with `lds`
+  total = block_sum(sq, lds);
+  if (threadIdx.x == 0) stat = 1.0 / __builtin_sqrt(total / (double)ncols + (double)eps);
+  __syncthreads();
+  const double rstd = stat;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock)
+    outr[c] = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
+}
+
 // Register tiles: NV groups of 256 columns per wavefront.  Sizes 3, 6 and 12
 // make rows of 768, 1536 and 3072 columns (transformer widths) fill the tile
 // exactly, which selects the unguarded load path.
@@ -782,8 +813,11 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   if (rows == 0 || cols == 0) return 0;
   if (!x || !gamma || !beta || !out) return fail(WF2HIP_EINVAL, "null pointer");
   int nv = pick_nv(cols);
-  if (nv == 0 || nv > 8)
-    return fail(WF2HIP_EUNSUPPORTED, "LayerNorm rows longer than 2048 are not supported");
+  if (nv == 0 || nv > 8) {
+    if (rows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+    layernorm_rows_block<<<(uint32_t)rows, kBlock, 0, rt().stream>>>(x, gamma, beta, eps, out, cols);
+    return after_launch("layernorm_rows_block");
+  }
   int64_t blocks = ceil_div(rows, kWavesPerBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
   const bool vec = aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta) &&
