@@ -32,6 +32,12 @@ __device__ __forceinline__ double wave_sum(double v) {
   return v;
 }
 
+__device__ __forceinline__ float wave_sum32(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
@@ -515,59 +521,73 @@ struct RowRegs {
 
 // softmax over the first `valid` columns of a row; columns valid..ncols-1 of
 // the output are set to 0 (used by the causal form).
-template <int NV, bool VEC, bool NT>
+// RW rows per wavefront: with one or two vectors per lane and row a wavefront that
+// takes a single row has 1 - 2 KB in flight and leaves the memory system idle (rows
+// of 256: 68 % of the HBM peak for softmax, 53 % for LayerNorm at 2^26 elements); the
+// rows' loads are all issued first and their reductions interleave.
+template <int NV, bool VEC, bool NT, int RW = 1>
 __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restrict__ x, int64_t ldx,
                                                             float* __restrict__ out, int64_t ldo,
                                                             int64_t nrows, int64_t ncols,
                                                             int64_t causal_seq, float scale) {
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-  if (row >= nrows) return;
+  const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * RW;
+  if (row0 >= nrows) return;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
   const float ninf = -__builtin_inff();
-  RowRegs<NV, VEC, NT> r;
-  r.load(x + row * ldx, valid, lane, ninf);
-  float m = ninf;
+  RowRegs<NV, VEC, NT> r[RW];
+  int64_t valid[RW];
 #pragma unroll
-  for (int g = 0; g < NV; g++)
+  for (int w = 0; w < RW; w++) {
+    const int64_t row = row0 + w < nrows ? row0 + w : nrows - 1;  // a repeated last row is computed and not stored
+    valid[w] = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
+    r[w].load(x + row * ldx, valid[w], lane, ninf);
+  }
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      if (causal_seq > 0) {
-        // binary32 product, like a MulNode; padding stays -inf whatever the sign of scale
-        bool in = RowRegs<NV, VEC, NT>::col(g, c, lane) < valid;
-        r.v[g][c] = in ? r.v[g][c] * scale : ninf;
+  for (int w = 0; w < RW; w++) {
+    float m = ninf;
+#pragma unroll
+    for (int g = 0; g < NV; g++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        if (causal_seq > 0) {
+          // binary32 product, like a MulNode; padding stays -inf whatever the sign of scale
+          bool in = RowRegs<NV, VEC, NT>::col(g, c, lane) < valid[w];
+          r[w].v[g][c] = in ? r[w].v[g][c] * scale : ninf;
+        }
+        m = fmaxf(m, r[w].v[g][c]);
       }
-      m = fmaxf(m, r.v[g][c]);
-    }
-  m = wave_max(m);
-  // exp(x - max) in binary32 through v_exp_f32: 2^(d log2 e) with the rounding
-  // error of the product folded back, so what remains is the rounding of d
-  // itself (|d| 2^-24 relative: 5e-7 at d = -10, 4e-6 at the underflow edge)
-  // and the instruction's own ulp.  The binary64 body this replaces cost 21
-  // VALU slots per element against 12 and left the kernel ALU-bound once the
-  // clock settles (65 % of the HBM peak at (32768, 1024)).  Clamping d at -160
-  // makes padding (-inf) and everything below the denormals an exact 0.
-  float sum = 0.0f;
+    m = wave_max(m);
+    // exp(x - max) in binary32 through v_exp_f32: 2^(d log2 e) with the rounding
+    // error of the product folded back, so what remains is the rounding of d
+    // itself (|d| 2^-24 relative: 5e-7 at d = -10, 4e-6 at the underflow edge)
+    // and the instruction's own ulp.  The binary64 body this replaces cost 21
+    // VALU slots per element against 12 and left the kernel ALU-bound once the
+    // clock settles (65 % of the HBM peak at (32768, 1024)).  Clamping d at -160
+    // makes padding (-inf) and everything below the denormals an exact 0.
+    float sum = 0.0f;
 #pragma unroll
-  for (int g = 0; g < NV; g++)
+    for (int g = 0; g < NV; g++)
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      const float d = fmaxf(r.v[g][c] - m, -160.0f);
-      const float t = d * 1.44269502f;
-      float tl = __builtin_fmaf(d, 1.44269502f, -t);
-      tl = __builtin_fmaf(d, 1.92596299e-8f, tl);
-      const float e = __builtin_amdgcn_exp2f(t);
-      const float ed = __builtin_fmaf(e, tl * 0.693147182f, e);
-      r.v[g][c] = ed;
-      sum += ed;
-    }
-  const double total = wave_sum((double)sum);
-  const float inv = (float)(1.0 / total);
+      for (int c = 0; c < 4; c++) {
+        const float d = fmaxf(r[w].v[g][c] - m, -160.0f);
+        const float t = d * 1.44269502f;
+        float tl = __builtin_fmaf(d, 1.44269502f, -t);
+        tl = __builtin_fmaf(d, 1.92596299e-8f, tl);
+        const float e = __builtin_amdgcn_exp2f(t);
+        const float ed = __builtin_fmaf(e, tl * 0.693147182f, e);
+        r[w].v[g][c] = ed;
+        sum += ed;
+      }
+    const double total = wave_sum((double)sum);
+    const float inv = (float)(1.0 / total);
 #pragma unroll
-  for (int g = 0; g < NV; g++)
+    for (int g = 0; g < NV; g++)
 #pragma unroll
-    for (int c = 0; c < 4; c++) r.v[g][c] *= inv;
-  r.store(out + row * ldo, ncols, lane);
+      for (int c = 0; c < 4; c++) r[w].v[g][c] *= inv;
+  }
+#pragma unroll
+  for (int w = 0; w < RW; w++)
+    if (row0 + w < nrows) r[w].store(out + (row0 + w) * ldo, ncols, lane);
 }
 
 // Rows too long for registers: one workgroup per row, three passes (the second
@@ -604,43 +624,77 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __rest
   }
 }
 
-template <int NV, bool VEC, bool NT>
+template <int NV, bool VEC, bool NT, int RW = 1>
 __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __restrict__ x,
                                                               const float* __restrict__ gamma,
                                                               const float* __restrict__ beta,
                                                               float eps, float* __restrict__ out,
                                                               int64_t nrows, int64_t ncols) {
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-  if (row >= nrows) return;
+  const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * RW;
+  if (row0 >= nrows) return;
   const int lane = threadIdx.x & (kWave - 1);
-  RowRegs<NV, VEC, NT> r;
+  RowRegs<NV, VEC, NT> r[RW];
   RowRegs<NV, VEC, false> g, b;
-  r.load(x + row * ncols, ncols, lane, 0.0f);
+#pragma unroll
+  for (int w = 0; w < RW; w++) r[w].load(x + (row0 + w < nrows ? row0 + w : nrows - 1) * ncols, ncols, lane, 0.0f);
   g.load(gamma, ncols, lane, 0.0f);
   b.load(beta, ncols, lane, 0.0f);
-  double sum = 0.0;
 #pragma unroll
-  for (int i = 0; i < NV; i++)
+  for (int w = 0; w < RW; w++) {
+    if constexpr (RW > 1) {
+      // rows of at most 512 columns: binary32 statistics (each lane adds at most eight
+      // terms, the wavefront folds 64 partial sums as a tree: relative error of the
+      // mean and the variance below 1e-6), a third of the instructions of the binary64 form
+      float sum = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 4; c++) sum += (double)r.v[i][c];
-  const double mean = wave_sum(sum) / (double)ncols;
-  double sq = 0.0;
+      for (int i = 0; i < NV; i++)
 #pragma unroll
-  for (int i = 0; i < NV; i++)
+        for (int c = 0; c < 4; c++) sum += r[w].v[i][c];
+      const float mean = wave_sum32(sum) / (float)ncols;
+      float sq = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
-      double d = in ? (double)r.v[i][c] - mean : 0.0;
-      sq += d * d;
+      for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
+          float d = in ? r[w].v[i][c] - mean : 0.0f;
+          sq = __builtin_fmaf(d, d, sq);
+        }
+      const float var = wave_sum32(sq) / (float)ncols;
+      const float rstd = (float)(1.0 / __builtin_sqrt((double)var + (double)eps));
+#pragma unroll
+      for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          r[w].v[i][c] = __builtin_fmaf((r[w].v[i][c] - mean) * rstd, g.v[i][c], b.v[i][c]);
+    } else {
+      double sum = 0.0;
+#pragma unroll
+      for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) sum += (double)r[w].v[i][c];
+      const double mean = wave_sum(sum) / (double)ncols;
+      double sq = 0.0;
+#pragma unroll
+      for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
+          double d = in ? (double)r[w].v[i][c] - mean : 0.0;
+          sq += d * d;
+        }
+      const double var = wave_sum(sq) / (double)ncols;
+      const double rstd = 1.0 / __builtin_sqrt(var + (double)eps);
+#pragma unroll
+      for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          r[w].v[i][c] = (float)(((double)r[w].v[i][c] - mean) * rstd * (double)g.v[i][c] + (double)b.v[i][c]);
     }
-  const double var = wave_sum(sq) / (double)ncols;
-  const double rstd = 1.0 / __builtin_sqrt(var + (double)eps);
+  }
 #pragma unroll
-  for (int i = 0; i < NV; i++)
-#pragma unroll
-    for (int c = 0; c < 4; c++)
-      r.v[i][c] = (float)(((double)r.v[i][c] - mean) * rstd * (double)g.v[i][c] + (double)b.v[i][c]);
-  r.store(out + row * ncols, ncols, lane);
+  for (int w = 0; w < RW; w++)
+    if (row0 + w < nrows) r[w].store(out + (row0 + w) * ncols, ncols, lane);
 }
 
 // Rows beyond the register tile (2048 columns): a workgroup per row, three passes
@@ -695,8 +749,14 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
                                                              causal_seq, scale);              \
     break;
   switch (nv) {
-    WF2_SOFTMAX_CASE(1)
-    WF2_SOFTMAX_CASE(2)
+    case 1:
+      softmax_rows_wave<1, VEC, NT, 4><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 4), kBlock, 0, st>>>(
+          x, ldx, out, ldo, nrows, ncols, causal_seq, scale);
+      break;
+    case 2:
+      softmax_rows_wave<2, VEC, NT, 2><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 2), kBlock, 0, st>>>(
+          x, ldx, out, ldo, nrows, ncols, causal_seq, scale);
+      break;
     WF2_SOFTMAX_CASE(3)
     WF2_SOFTMAX_CASE(4)
     WF2_SOFTMAX_CASE(6)
@@ -746,8 +806,14 @@ static int launch_layernorm_wave(int nv, uint32_t blocks, const float* x, const 
     layernorm_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, g, b, eps, out, nrows, ncols);   \
     break;
   switch (nv) {
-    WF2_LN_CASE(1)
-    WF2_LN_CASE(2)
+    case 1:
+      layernorm_rows_wave<1, VEC, NT, 4><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 4), kBlock, 0, st>>>(
+          x, g, b, eps, out, nrows, ncols);
+      break;
+    case 2:
+      layernorm_rows_wave<2, VEC, NT, 2><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 2), kBlock, 0, st>>>(
+          x, g, b, eps, out, nrows, ncols);
+      break;
     WF2_LN_CASE(3)
     WF2_LN_CASE(4)
     WF2_LN_CASE(6)
