@@ -39,6 +39,26 @@ def test_sum_tester_vectors(gpu):
     assert kd.shape == [100, 100, 100] and np.all(kd.numpy() == 100.0)
 
 
+def test_many_short_rows(gpu):
+    """Row sums of many rows of at most 512 elements (four rows per wavefront), with
+    row lengths that are not multiples of four through a view: float64 truth, 1e-5
+    relative to the sum of magnitudes."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(97)
+    for rows, pitch, cols in [(10000, 256, 256), (9000, 512, 512), (8200, 100, 100), (12000, 256, 250),
+                              (9001, 384, 321), (8192, 4, 4)]:
+        X = rng.standard_normal((rows, pitch)).astype(np.float32)
+        v = F.from_numpy(X).view(True, (0, cols))
+        got = F.sum(v, axis=1).numpy()
+        want = X[:, :cols].astype(np.float64).sum(axis=1, keepdims=True)
+        scale = np.abs(X[:, :cols]).astype(np.float64).sum(axis=1, keepdims=True)
+        assert got.shape == want.shape
+        assert np.max(np.abs(got - want) / scale) < 1e-5, (rows, pitch, cols)
+        mean = F.mean(v, axis=1).numpy()
+        assert np.max(np.abs(mean - want / cols) / (scale / cols)) < 1e-5
+
+
 def test_config4_row_and_full_sum(gpu, O):
     """BASELINE config 4: row sum and full sum of (8192, 4096) N(0,1), seed 4.
     Tree mode against float64 truth; a slice of it in sequential mode against
