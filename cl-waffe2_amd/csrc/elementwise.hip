@@ -33,18 +33,26 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 // output in cache.
 constexpr int64_t kStreamingBytes = (int64_t)192 << 20;
 
+// Four consecutive floats as one access.  The vector type is declared 4-byte
+// aligned: gfx950 runs with unaligned access enabled, so the compiler still emits a
+// single global_load / global_store_dwordx4 and the hardware takes any float
+// address.  Views that start an odd number of elements into their storage
+// (x[1:], A[:, 1:4097]) therefore use the vector kernels like aligned ones
+// (x[1:] += y at 2^26: 70 % of the HBM peak through scalar accesses).
+typedef f4 f4u __attribute__((aligned(4)));
+
 template <bool NT>
 __device__ __forceinline__ f4 load4(const float* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
-  return *reinterpret_cast<const f4*>(p);
+  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const f4u*>(p));
+  return *reinterpret_cast<const f4u*>(p);
 }
 
 template <bool NT>
 __device__ __forceinline__ void store4(float* p, f4 v) {
   if constexpr (NT)
-    __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+    __builtin_nontemporal_store(v, reinterpret_cast<f4u*>(p));
   else
-    *reinterpret_cast<f4*>(p) = v;
+    *reinterpret_cast<f4u*>(p) = v;
 }
 
 // ---- functors: operator()(dst_value, src_value) ---------------------------
@@ -131,7 +139,15 @@ struct OpWhere {
 // thread instead of four: measured 4-7 % faster at 2^26 (exp 5.91 -> 6.36 TB/s).
 template <class F, bool ReadDst, bool SrcBroadcast, bool NT, int LAYOUT, int kFlatU>
 __global__ __launch_bounds__(kBlock) void ew_flat(float* __restrict__ dst,
-                                                  const float* __restrict__ src, size_t nvec, F f) {
+                                                  const float* __restrict__ src, size_t nvec, F f, int head,
+                                                  int tail) {
+  // the elements before the first whole vector of the body and after the last one
+  if (blockIdx.x == 0 && (int)threadIdx.x < head + tail) {
+    const int t = threadIdx.x;
+    const ptrdiff_t at = t < head ? (ptrdiff_t)t - head : (ptrdiff_t)(4 * nvec) + (t - head);
+    const float a = ReadDst ? dst[at] : 0.0f;
+    dst[at] = f(a, SrcBroadcast ? src[0] : src[at]);
+  }
   size_t base;
   if (LAYOUT == 0) {
     base = (size_t)blockIdx.x * kBlock * kFlatU + threadIdx.x;
@@ -786,18 +802,15 @@ static int launch_rows(const Space& s, float* dst, const float* src, F f) {
   p.src_inner = (int32_t)s.sb[last];
   p.nouter = s.rank - 1;
   int64_t nrows = 1;
-  bool vec_ok = aligned16(p.dst) && (!p.src_inner || aligned16(p.src));
   for (int i = 0; i < p.nouter; i++) {
     int r = last - 1 - i;
     p.oshape[i] = (uint32_t)s.shape[r];
     p.odst[i] = s.sa[r];
     p.osrc[i] = s.sb[r];
     nrows *= s.shape[r];
-    if (s.sa[r] % 4 != 0) vec_ok = false;
-    if (p.src_inner && s.sb[r] % 4 != 0) vec_ok = false;
   }
   p.nrows = (uint32_t)nrows;
-  const int vec = vec_ok ? 4 : 1;
+  const int vec = p.n0 >= 4 ? 4 : 1;  // any row start: the vector accesses need no alignment
   const int64_t n0v = ceil_div(p.n0, vec);
   int tl = ilog2_ceil(n0v);
   if (tl > 8) tl = 8;
@@ -832,16 +845,22 @@ static int launch_rows(const Space& s, float* dst, const float* src, F f) {
   return after_launch("ew_rows");
 }
 
-// Rank-1, unit-stride destination, source unit-stride or broadcast, 16-byte
-// aligned: the flat kernel for the whole vectors, the rows kernel for the
-// (at most three) trailing elements.
+// Rank-1, unit-stride destination, source unit-stride or broadcast: the flat kernel.
 template <class F, bool ReadDst>
 static bool try_launch_flat(const Space& s, float* dst, const float* src, F f, int* rc) {
   float* d = dst + s.off_a;
   const float* q = src + s.off_b;
   const bool bcast = s.sb[0] == 0;
-  if (!aligned16(d) || (!bcast && !aligned16(q))) return false;
-  const size_t nvec = (size_t)(s.total / 4);
+  // The vector body starts where dst reaches a 256-byte boundary, so that the 1 KB a
+  // wavefront stores per access covers whole cache lines: x[1:] += y at 2^26 runs at 70 %
+  // of the HBM peak with dst 4 or 16 bytes past such a boundary, 82 % with only the loads
+  // misaligned.  The up to 63 elements before the body and the up to three after its last
+  // whole vector are done by the first workgroup.
+  const int64_t head = (int64_t)((64 - (((uintptr_t)d >> 2) & 63)) & 63);  // elements up to the next 256-byte boundary
+  d += head;
+  if (!bcast) q += head;
+  const size_t nvec = (size_t)((s.total - head) / 4);
+  const int64_t tail = s.total - head - (int64_t)nvec * 4;
   // vectors per thread: 4 for x <- x op y (three streams), 2 for functors with
   // a long binary64 body, 1 for the light two-stream forms (copy, fill, scalar
   // operand, sqrt, abs) -- each the best of a sweep at 2^26 on MI355X.
@@ -855,30 +874,21 @@ static bool try_launch_flat(const Space& s, float* dst, const float* src, F f, i
   if (blocks >= ((int64_t)1 << 31)) return false;
   if (bcast) {
     if (nt)
-      ew_flat<F, ReadDst, true, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, true, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
     else
-      ew_flat<F, ReadDst, true, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, true, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
   } else if (ReadDst) {
     if (nt)
-      ew_flat<F, ReadDst, false, true, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, true, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
     else
-      ew_flat<F, ReadDst, false, false, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, false, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
   } else {
     if (nt)
-      ew_flat<F, ReadDst, false, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
     else
-      ew_flat<F, ReadDst, false, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f);
+      ew_flat<F, ReadDst, false, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
   }
   *rc = after_launch("ew_flat");
-  const int64_t done = (int64_t)nvec * 4;
-  if (*rc == 0 && done < s.total) {
-    Space tail = s;
-    tail.shape[0] = s.total - done;
-    tail.total = tail.shape[0];
-    tail.off_a += done;
-    if (!bcast) tail.off_b += done;
-    *rc = launch_rows<F, ReadDst>(tail, dst, src, f);
-  }
   return true;
 }
 

@@ -291,6 +291,128 @@ __global__ __launch_bounds__(kBlock) void accumulate_generic(AccParams p) {
   if (lane == 0) p.a[aoff] = (float)((double)p.a[aoff] + acc);
 }
 
+// ---- column form: the kept axis is the contiguous one ----------------------------
+// a[c] += sum_j b[j, c] (sums over the batch axes: bias gradients, !sum :axis 0).  A
+// wavefront per destination element would read with the row pitch as its stride
+// (column sums of (8192, 8192): 7 % of the HBM peak); here a workgroup owns 256
+// columns x a range of the reduced index space, each lane adds four columns of four
+// rows per step in binary64, and the ranges' partial sums are folded in a fixed order
+// by a second launch (scratch from the pool).
+struct ColRedParams {
+  AccParams acc;     // nk == 1: the kept axis is the last, contiguous one
+  int64_t ncols;
+  int64_t seg;       // reduced indices per split
+  uint32_t splits;
+  double* scratch;   // splits x ncols, unused when splits == 1
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kBlock) void reduce_cols_partial(ColRedParams q) {
+  typedef f4 f4u __attribute__((aligned(4)));
+  __shared__ double lds[3][kWave][4];
+  const AccParams& p = q.acc;
+  const int cx = threadIdx.x & (kWave - 1), ry = threadIdx.x / kWave;  // 64 column lanes x 4 row phases
+  const uint32_t ctiles = (uint32_t)((q.ncols + 255) / 256);
+  const uint32_t ctile = blockIdx.x % ctiles;
+  const uint32_t split = blockIdx.x / ctiles;
+  const int64_t c = (int64_t)ctile * 256 + 4 * cx;
+  const int64_t lo = (int64_t)split * q.seg;
+  const int64_t hi = lo + q.seg < p.nred ? lo + q.seg : p.nred;
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  if (c + 4 <= q.ncols) {
+    int64_t j = lo + ry;
+    for (; j + 12 < hi; j += 16) {  // four rows in flight per lane
+      f4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const f4u* src = reinterpret_cast<const f4u*>(p.b + reduced_offset(p, j + 4 * u) + c);
+        v[u] = NT ? __builtin_nontemporal_load(src) : *src;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        acc[0] += (double)v[u].x;
+        acc[1] += (double)v[u].y;
+        acc[2] += (double)v[u].z;
+        acc[3] += (double)v[u].w;
+      }
+    }
+    for (; j < hi; j += 4) {
+      const f4 v = *reinterpret_cast<const f4u*>(p.b + reduced_offset(p, j) + c);
+      acc[0] += (double)v.x;
+      acc[1] += (double)v.y;
+      acc[2] += (double)v.z;
+      acc[3] += (double)v.w;
+    }
+  } else {
+    for (int64_t j = lo + ry; j < hi; j += 4) {
+      const float* row = p.b + reduced_offset(p, j);
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        if (c + k < q.ncols) acc[k] += (double)row[c + k];
+    }
+  }
+  if (ry > 0) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) lds[ry - 1][cx][k] = acc[k];
+  }
+  __syncthreads();
+  if (ry == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const double total = acc[k] + lds[0][cx][k] + lds[1][cx][k] + lds[2][cx][k];
+      if (c + k < q.ncols) {
+        if (q.splits == 1)
+          p.a[c + k] = (float)((double)p.a[c + k] + total);
+        else
+          q.scratch[(int64_t)split * q.ncols + c + k] = total;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void reduce_cols_finish(ColRedParams q) {
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= q.ncols) return;
+  double total = 0.0;
+  for (uint32_t s = 0; s < q.splits; s++) total += q.scratch[(int64_t)s * q.ncols + c];
+  q.acc.a[c] = (float)((double)q.acc.a[c] + total);
+}
+
+static int launch_col_reduce(const AccParams& p, int64_t ncols) {
+  ColRedParams q;
+  q.acc = p;
+  q.ncols = ncols;
+  const int64_t ctiles = ceil_div(ncols, 256);
+  const int64_t target = (int64_t)rt().num_cus * 8;
+  int64_t splits = ceil_div(target, ctiles);
+  if (splits > p.nred / 64) splits = p.nred / 64;  // at least 64 reduced indices per workgroup
+  if (splits < 1) splits = 1;
+  q.seg = ceil_div(ceil_div(p.nred, splits), 16) * 16;
+  splits = ceil_div(p.nred, q.seg);
+  q.splits = (uint32_t)splits;
+  q.scratch = nullptr;
+  if (ctiles * splits >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
+  void* scratch = nullptr;
+  if (splits > 1) {
+    WF2_TRY(wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(double)));
+    q.scratch = static_cast<double*>(scratch);
+  }
+  hipStream_t st = rt().stream;
+  if (p.nred * ncols * 4 >= ((int64_t)192 << 20))
+    reduce_cols_partial<true><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(q);
+  else
+    reduce_cols_partial<false><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(q);
+  int rc = after_launch("reduce_cols_partial");
+  if (rc == 0 && splits > 1) {
+    reduce_cols_finish<<<(uint32_t)ceil_div(ncols, kBlock), kBlock, 0, st>>>(q);
+    rc = after_launch("reduce_cols_finish");
+  }
+  // the block goes back to the pool; later work on the same stream that reuses it is
+  // ordered after these launches
+  if (scratch) (void)wf2hip_free(scratch);
+  return rc;
+}
+
 // The reference's order: for one destination element, visit the reduced index
 // space in row-major order and apply a <- a op b in binary32 each time.
 template <class F>
@@ -448,6 +570,9 @@ int launch_accumulate(int op, const Space& s, float* a, const float* b) {
   for (int r = 0; r < last; r++)
     if (s.shape[r] >= ((int64_t)1 << 32)) row_form = false;
   if (row_form) return launch_row_reduce(s, a, b);
+  // column form: the only kept axis is the last one, contiguous on both sides
+  if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 16)
+    return launch_col_reduce(p, s.shape[last]);
   int64_t blocks = ceil_div(p.nout, kWavesPerBlock);
   if (blocks >= ((int64_t)1 << 31))
     return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");

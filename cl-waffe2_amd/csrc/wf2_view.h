@@ -118,10 +118,49 @@ inline bool hazardous_overlap_at(const Space& s, int64_t delta) {
   }
   const int64_t starts = s.off_a - (s.off_b + delta);
   if (g > 1 && starts % g != 0) return false;
-  if (starts != 0) return true;
+  bool same_strides = true;
   for (int r = 0; r < s.rank; r++)
-    if (s.sa[r] != s.sb[r]) return true;
-  return false;  // identical mapping: every element depends on itself only
+    if (s.sa[r] != s.sb[r]) same_strides = false;
+  if (!same_strides) return true;
+  if (starts == 0) return false;  // identical mapping: every element depends on itself only
+  // One window is the other moved by `starts` elements (x[:, :h] against x[:, h:]): they
+  // share an element iff starts = sum k_r stride_r with |k_r| < extent_r.  With nested
+  // strides (each larger than everything the axes below it span) only the two
+  // neighbouring multiples of a stride can work at each level, so the search is exact;
+  // otherwise stay on the safe side.
+  int order[WF2HIP_MAX_RANK];
+  int n = 0;
+  for (int r = 0; r < s.rank; r++)
+    if (s.shape[r] > 1 && s.sa[r] != 0) order[n++] = r;
+  auto mag = [&](int r) { return s.sa[r] < 0 ? -s.sa[r] : s.sa[r]; };
+  for (int i = 1; i < n; i++)
+    for (int j = i; j > 0 && mag(order[j]) > mag(order[j - 1]); j--) {
+      const int t = order[j];
+      order[j] = order[j - 1];
+      order[j - 1] = t;
+    }
+  int64_t below = 0;
+  for (int i = n - 1; i >= 0; i--) {
+    if (mag(order[i]) <= below) return true;  // not nested
+    below += mag(order[i]) * (s.shape[order[i]] - 1);
+  }
+  struct Search {
+    const Space& s;
+    const int* order;
+    int n;
+    bool hits(int64_t rem, int level) const {
+      if (level == n) return rem == 0;
+      const int r = order[level];
+      const int64_t stride = s.sa[r];
+      int64_t q = rem / stride;  // truncated; the neighbours q - 1, q, q + 1 cover floor and ceiling
+      for (int64_t k = q - 1; k <= q + 1; k++) {
+        const int64_t a = k < 0 ? -k : k;
+        if (a < s.shape[r] && hits(rem - k * stride, level + 1)) return true;
+      }
+      return false;
+    }
+  };
+  return Search{s, order, n}.hits(starts, 0);
 }
 
 inline bool hazardous_overlap(const Space& s, const float* a, const float* b) {

@@ -121,6 +121,33 @@ def test_config2_views(gpu, O):
     assert_bit_equal(got.numpy(), A[1024:3072] - A[0:2048], "offset views")
 
 
+def test_disjoint_windows_of_one_buffer(gpu):
+    """x[:, :h] += x[:, h:] -- two windows of one storage whose address ranges
+    interleave but never share an element -- is an ordinary in-place op; windows
+    that do share elements are refused (the CPU result would depend on loop order)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(81)
+    for rows, cols in [(64, 512), (33, 1030), (7, 10)]:
+        h = cols // 2
+        A = rng.standard_normal((rows, cols)).astype(np.float32)
+        t = F.from_numpy(A)
+        F.add_(t.view(True, (0, h)), t.view(True, (h, 2 * h)))
+        want = A.copy()
+        want[:, :h] += A[:, h:2 * h]
+        assert_bit_equal(t.numpy(), want, f"x[:, :h] += x[:, h:], {rows}x{cols}")
+        t = F.from_numpy(A)
+        F.mul_(t.view((0, rows // 2), True), t.view((rows - rows // 2, rows), True))  # upper rows *= lower rows
+        want = A.copy()
+        want[:rows // 2] *= A[rows - rows // 2:]
+        assert_bit_equal(t.numpy(), want, "rows against later rows")
+        t = F.from_numpy(A)
+        with pytest.raises(W.HIPError):
+            F.add_(t.view(True, (0, h)), t.view(True, (1, h + 1)))
+        with pytest.raises(W.HIPError):
+            F.add_(t.view((0, rows - 1), True), t.view((1, rows), True))
+
+
 def test_every_second_element_as_source(gpu):
     """A [::2] slice read into contiguous rows -- the copy behind every out-of-place
     op on such a view (two aligned 16-byte loads per four elements when the rows

@@ -39,6 +39,32 @@ def test_sum_tester_vectors(gpu):
     assert kd.shape == [100, 100, 100] and np.all(kd.numpy() == 100.0)
 
 
+def test_sums_over_leading_axes(gpu):
+    """!sum over the leading axes with the last axis kept (bias gradients): the column
+    form, whole vectors and ragged column counts, one and several reduced axes, a
+    sliced source; float64 truth, 1e-5 relative to the sum of magnitudes."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(101)
+    for shape, axis in [((3000, 768), 0), ((17, 1000), 0), ((64, 50, 260), (0, 1)), ((4100, 67), 0),
+                        ((9, 33, 1030), (0, 1)), ((20000, 64), 0)]:
+        X = rng.standard_normal(shape).astype(np.float32)
+        got = F.sum(F.from_numpy(X), axis=axis).numpy()
+        want = X.astype(np.float64).sum(axis=axis, keepdims=True)
+        scale = np.abs(X).astype(np.float64).sum(axis=axis, keepdims=True)
+        assert got.shape == want.shape
+        assert np.max(np.abs(got - want) / scale) < 1e-5, (shape, axis)
+    X = rng.standard_normal((5000, 512)).astype(np.float32)
+    v = F.from_numpy(X).view((100, 4100), (3, 259))
+    got = F.sum(v, axis=0).numpy()
+    want = X[100:4100, 3:259].astype(np.float64).sum(axis=0, keepdims=True)
+    assert np.max(np.abs(got - want)) < 1e-3
+    # accumulation adds to what the destination holds
+    acc = F.from_numpy(np.full((1, 512), 2.5, np.float32))
+    F.add_(acc.view((":broadcast", 5000), True), F.from_numpy(X))
+    np.testing.assert_allclose(acc.numpy(), 2.5 + X.astype(np.float64).sum(axis=0, keepdims=True), rtol=0, atol=2e-3)
+
+
 def test_many_short_rows(gpu):
     """Row sums of many rows of at most 512 elements (four rows per wavefront), with
     row lengths that are not multiples of four through a view: float64 truth, 1e-5
