@@ -831,10 +831,60 @@ struct Epilogue {
   int causal = 0;
 };
 
+// C <- beta C + sum over the `splits` partial products of a split-K run (column-major,
+// partials packed m x n each, already scaled by alpha)
+__global__ __launch_bounds__(kBlock) void splitk_fold(const float* __restrict__ partials, int splits, int64_t m,
+                                                      int64_t n, float beta, float* __restrict__ C, int64_t ldc) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= m * n) return;
+  const int64_t j = e / m, i = e - j * m;
+  float acc = 0.0f;
+  for (int s = 0; s < splits; s++) acc += partials[(int64_t)s * m * n + e];
+  float* c = C + i + j * ldc;
+  *c = beta == 0.0f ? acc : beta * *c + acc;
+}
+
 int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha, const float* A,
                    long lda, long strideA, long strideA2, const float* B, long ldb, long strideB,
                    long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
-                   long batch, long batch2, const Epilogue& ep = Epilogue()) {
+                   long batch, long batch2, const Epilogue& ep = Epilogue());
+
+// A single product with few output tiles and a long K (weight gradients: 768 x 3072
+// outputs over K = 8192 are 144 tiles for 256 compute units) runs as `splits` products
+// over slices of K in one batched launch, folded in a fixed order afterwards.
+static bool try_split_k(char transa, char transb, long m, long n, long k, float alpha, const float* A, long lda,
+                        const float* B, long ldb, float beta, float* C, long ldc, int* rc) {
+  const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128);
+  const int64_t cus = rt().num_cus;
+  if (k < 2048 || tiles >= cus || m < 1 || n < 1) return false;
+  int splits = 0;
+  for (int cand : {16, 8, 4, 2})
+    if (k % ((long)cand * 32) == 0 && k / cand >= 512 && tiles * cand <= 4 * cus) {
+      splits = cand;
+      break;
+    }
+  if (splits == 0) return false;
+  const long kc = k / splits;
+  void* scratch = nullptr;
+  if (wf2hip_malloc_uninitialized(&scratch, (size_t)splits * m * n * sizeof(float)) != 0) return false;
+  const long sa = is_n(transa) ? kc * lda : kc;  // op(A) is m x k: a K slice starts kc columns / rows further
+  const long sb = is_n(transb) ? kc : kc * ldb;
+  *rc = sgemm_batched2(transa, transb, m, n, kc, alpha, A, lda, sa, 0, B, ldb, sb, 0, 0.0f,
+                       static_cast<float*>(scratch), m, (long)m * n, 0, splits, 1);
+  if (*rc == 0) {
+    const int64_t blocks = ceil_div((int64_t)m * n, kBlock);
+    splitk_fold<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m, n, beta,
+                                                               C, ldc);
+    *rc = after_launch("splitk_fold");
+  }
+  (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
+  return true;
+}
+
+int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha, const float* A,
+                   long lda, long strideA, long strideA2, const float* B, long ldb, long strideB,
+                   long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
+                   long batch, long batch2, const Epilogue& ep) {
   if (!(is_n(transa) || is_t(transa)) || !(is_n(transb) || is_t(transb)))
     return fail(WF2HIP_EINVAL, "trans must be N, T or C");
   if (m < 0 || n < 0 || k < 0 || batch < 0 || batch2 < 0)
@@ -849,6 +899,10 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
   if ((int64_t)batch * batch2 > 65535)
     return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  if (batch == 1 && batch2 == 1 && !ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
+    int rc = 0;
+    if (try_split_k(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, &rc)) return rc;
+  }
 
   GemmParams p;
   // row-major view: Cr[n][m] = Left[n][k] . Right[k][m]

@@ -317,6 +317,46 @@ def test_matmul_random(gpu, m, n, k, ta, tb):
     _gemm_check(got, A.astype(np.float64), B.astype(np.float64))
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_few_tiles_long_k(gpu, ta, tb):
+    """Products with few output tiles and a long K (weight gradients) run split over K
+    and are folded afterwards: every layout, leading dimensions and beta through the
+    column-major entry point as well."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(303 + ta + 2 * tb)
+    for m, n, k in [(768, 640, 8192), (200, 300, 4096), (130, 1000, 2048)]:
+        A = rng.standard_normal((m, k)).astype(np.float32)
+        B = rng.standard_normal((k, n)).astype(np.float32)
+        dA = F.t(F.from_numpy(np.ascontiguousarray(A.T))) if ta else F.from_numpy(A)
+        dB = F.t(F.from_numpy(np.ascontiguousarray(B.T))) if tb else F.from_numpy(B)
+        _gemm_check(F.matmul(dA, dB).numpy(), A.astype(np.float64), B.astype(np.float64))
+    # column-major contract with beta and padded leading dimensions
+    lib = W.lib.get()
+    m, n, k = 96, 200, 4096
+    ca, cb = ("T" if ta else "N"), ("T" if tb else "N")
+    lda = (m if ca == "N" else k) + 4
+    ldb = (k if cb == "N" else n) + 8
+    ldc = m + 4
+    A = rng.standard_normal(lda * (k if ca == "N" else m)).astype(np.float32)
+    B = rng.standard_normal(ldb * (n if cb == "N" else k)).astype(np.float32)
+    Cm = rng.standard_normal(ldc * n).astype(np.float32)
+    A2 = A.reshape(-1, lda).T.astype(np.float64)  # column-major storage: lda rows
+    B2 = B.reshape(-1, ldb).T.astype(np.float64)
+    opA = A2[:m, :k] if ca == "N" else A2[:k, :m].T
+    opB = B2[:k, :n] if cb == "N" else B2[:n, :k].T
+    C2 = Cm.reshape(-1, ldc).T.astype(np.float64)
+    want = C2.copy()
+    want[:m, :n] = 0.5 * opA @ opB - 2.0 * C2[:m, :n]
+    dA, dB, dC = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B), W.HIPTensor.from_numpy(Cm)
+    W.lib.check(lib.wf2hip_sgemm(ca.encode(), cb.encode(), m, n, k, 0.5, dptr(dA), lda, dptr(dB), ldb, -2.0,
+                                 dptr(dC), ldc))
+    got = dC.numpy().reshape(-1, ldc).T
+    scale = 0.5 * np.abs(opA) @ np.abs(opB) + 2.0 * np.abs(C2[:m, :n])
+    assert np.max(np.abs(got[:m, :n] - want[:m, :n]) / scale) < 1e-5
+    np.testing.assert_array_equal(got[m:, :], C2[m:, :].astype(np.float32))  # padding rows untouched
+
+
 def test_sgemm_column_major_contract(gpu, O):
     """wf2hip_sgemm keeps Fortran sgemm_ semantics (column-major, alpha/beta,
     leading dimensions larger than the matrix), checked against the oracle's
