@@ -102,6 +102,98 @@ __global__ __launch_bounds__(kBlock) void compare_generic(Cmp3Params p) {
   p.out[co] = holds(p.op, p.x[ao], p.y[bo]) ? p.then_value : p.else_value;
 }
 
+// Rows: the innermost axis has unit stride in `out` and unit or zero stride in x and y
+// (windows of matrices, a row or a column compared against a matrix).  A thread takes
+// one 16-byte vector of four rows, all loads before the first store; the vector type
+// needs no alignment (see elementwise.hip).  The index-decomposing kernel below ran
+// two column windows of (8192, 8192) at 48 % of the HBM peak.
+struct CmpRows {
+  const float* x;
+  const float* y;
+  float* out;
+  int64_t n0;
+  int32_t x_inner, y_inner;  // 1 or 0 (one value per row)
+  int32_t nouter, op;
+  uint32_t nrows, chunks;
+  uint32_t oshape[WF2HIP_MAX_RANK];  // outer axes, innermost of them first
+  int64_t ox[WF2HIP_MAX_RANK], oy[WF2HIP_MAX_RANK], oo[WF2HIP_MAX_RANK];
+  float then_value, else_value;
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kBlock) void compare_rows(CmpRows p) {
+  typedef f4 f4u __attribute__((aligned(4)));
+  constexpr int UR = 4;
+  const uint32_t rblock = blockIdx.x / p.chunks;
+  const uint32_t chunk = blockIdx.x - rblock * p.chunks;
+  const int64_t col = ((int64_t)chunk * kBlock + threadIdx.x) * 4;
+  if (col >= p.n0) return;
+  const float *xr[UR], *yr[UR];
+  float* orow[UR];
+  bool live[UR];
+#pragma unroll
+  for (int u = 0; u < UR; u++) {
+    const uint64_t row = (uint64_t)rblock * UR + u;
+    live[u] = row < p.nrows;
+    uint32_t rem = live[u] ? (uint32_t)row : 0u;
+    int64_t xo = 0, yo = 0, oo = 0;
+    for (int i = 0; i < p.nouter; i++) {
+      uint32_t idx;
+      if (i == p.nouter - 1) {
+        idx = rem;
+      } else {
+        const uint32_t q = rem / p.oshape[i];
+        idx = rem - q * p.oshape[i];
+        rem = q;
+      }
+      xo += (int64_t)idx * p.ox[i];
+      yo += (int64_t)idx * p.oy[i];
+      oo += (int64_t)idx * p.oo[i];
+    }
+    xr[u] = p.x + xo;
+    yr[u] = p.y + yo;
+    orow[u] = p.out + oo;
+  }
+  auto pick = [&](float a, float b) { return holds(p.op, a, b) ? p.then_value : p.else_value; };
+  if (col + 4 <= p.n0) {
+    f4 a[UR], b[UR];
+#pragma unroll
+    for (int u = 0; u < UR; u++) {
+      if (!live[u]) continue;
+      if (p.x_inner) {
+        const f4u* q = reinterpret_cast<const f4u*>(xr[u] + col);
+        a[u] = NT ? __builtin_nontemporal_load(q) : *q;
+      } else {
+        const float v = xr[u][0];
+        a[u] = f4{v, v, v, v};
+      }
+      if (p.y_inner) {
+        const f4u* q = reinterpret_cast<const f4u*>(yr[u] + col);
+        b[u] = NT ? __builtin_nontemporal_load(q) : *q;
+      } else {
+        const float v = yr[u][0];
+        b[u] = f4{v, v, v, v};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UR; u++) {
+      if (!live[u]) continue;
+      const f4 r = {pick(a[u].x, b[u].x), pick(a[u].y, b[u].y), pick(a[u].z, b[u].z), pick(a[u].w, b[u].w)};
+      f4u* q = reinterpret_cast<f4u*>(orow[u] + col);
+      if (NT)
+        __builtin_nontemporal_store(r, q);
+      else
+        *q = r;
+    }
+    return;
+  }
+  for (int u = 0; u < UR; u++) {  // ragged end of the rows
+    if (!live[u]) continue;
+    for (int64_t c = col; c < p.n0; c++)
+      orow[u][c] = pick(p.x_inner ? xr[u][c] : xr[u][0], p.y_inner ? yr[u][c] : yr[u][0]);
+  }
+}
+
 int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, float then_value,
                float else_value) {
   if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
@@ -134,6 +226,44 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
       compare_flat<false><<<(uint32_t)blocks, kBlock, 0, st>>>(xp, yp, op_, (size_t)s.total, op,
                                                                then_value, else_value);
     return after_launch("compare_flat");
+  }
+  const int last = s.rank - 1;
+  bool rows_ok = s.rank >= 2 && s.sc[last] == 1 && (s.sa[last] == 1 || s.sa[last] == 0) &&
+                 (s.sb[last] == 1 || s.sb[last] == 0) && s.shape[last] >= 4;
+  int64_t nrows = 1;
+  for (int r = 0; r < last; r++) {
+    if (s.shape[r] >= ((int64_t)1 << 32)) rows_ok = false;
+    nrows *= s.shape[r];
+  }
+  if (rows_ok && nrows < ((int64_t)1 << 32)) {
+    CmpRows q;
+    q.x = xp;
+    q.y = yp;
+    q.out = op_;
+    q.n0 = s.shape[last];
+    q.x_inner = (int32_t)s.sa[last];
+    q.y_inner = (int32_t)s.sb[last];
+    q.op = op;
+    q.nouter = last;
+    for (int i = 0; i < last; i++) {
+      const int r = last - 1 - i;
+      q.oshape[i] = (uint32_t)s.shape[r];
+      q.ox[i] = s.sa[r];
+      q.oy[i] = s.sb[r];
+      q.oo[i] = s.sc[r];
+    }
+    q.nrows = (uint32_t)nrows;
+    q.chunks = (uint32_t)ceil_div(q.n0, (int64_t)kBlock * 4);
+    q.then_value = then_value;
+    q.else_value = else_value;
+    const int64_t row_blocks = ceil_div(nrows, 4) * q.chunks;
+    if (row_blocks < ((int64_t)1 << 31)) {
+      if (s.total * 12 >= ((int64_t)192 << 20))
+        compare_rows<true><<<(uint32_t)row_blocks, kBlock, 0, st>>>(q);
+      else
+        compare_rows<false><<<(uint32_t)row_blocks, kBlock, 0, st>>>(q);
+      return after_launch("compare_rows");
+    }
   }
   Cmp3Params p;
   p.x = xp;
