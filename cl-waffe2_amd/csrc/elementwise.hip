@@ -137,16 +137,24 @@ struct OpWhere {
 // 6.59 with layout 0; two streams (copy, unary) 6.45 with layout 0 against 6.25.
 // Functors with a long binary64 body (transcendentals) take two vectors per
 // thread instead of four: measured 4-7 % faster at 2^26 (exp 5.91 -> 6.36 TB/s).
-template <class F, bool ReadDst, bool SrcBroadcast, bool NT, int LAYOUT, int kFlatU>
+struct FlatEdges {
+  int head, tail;
+};
+struct NoEdges {};
+
+template <class F, bool ReadDst, bool SrcBroadcast, bool NT, int LAYOUT, int kFlatU, class Edges = NoEdges>
 __global__ __launch_bounds__(kBlock) void ew_flat(float* __restrict__ dst,
-                                                  const float* __restrict__ src, size_t nvec, F f, int head,
-                                                  int tail) {
-  // the elements before the first whole vector of the body and after the last one
-  if (blockIdx.x == 0 && (int)threadIdx.x < head + tail) {
-    const int t = threadIdx.x;
-    const ptrdiff_t at = t < head ? (ptrdiff_t)t - head : (ptrdiff_t)(4 * nvec) + (t - head);
-    const float a = ReadDst ? dst[at] : 0.0f;
-    dst[at] = f(a, SrcBroadcast ? src[0] : src[at]);
+                                                  const float* __restrict__ src, size_t nvec, F f, Edges edges = Edges()) {
+  // the elements before the first whole vector of the body and after the last one (the
+  // aligned, whole-vector case is a kernel of its own without this prologue)
+  if constexpr (__is_same(Edges, FlatEdges)) {
+    const int head = edges.head, tail = edges.tail;
+    if (blockIdx.x == 0 && (int)threadIdx.x < head + tail) {
+      const int t = threadIdx.x;
+      const ptrdiff_t at = t < head ? (ptrdiff_t)t - head : (ptrdiff_t)(4 * nvec) + (t - head);
+      const float a = ReadDst ? dst[at] : 0.0f;
+      dst[at] = f(a, SrcBroadcast ? src[0] : src[at]);
+    }
   }
   size_t base;
   if (LAYOUT == 0) {
@@ -872,22 +880,33 @@ static bool try_launch_flat(const Space& s, float* dst, const float* src, F f, i
   const bool three = ReadDst && !bcast;
   const int64_t blocks = ceil_div((int64_t)nvec, kBlock * (three ? u3 : u2));
   if (blocks >= ((int64_t)1 << 31)) return false;
+  const uint32_t grid = (uint32_t)blocks;
+  const FlatEdges edges{(int)head, (int)tail};
+  const bool plain = head == 0 && tail == 0;
+#define WF2_FLAT(BC, NTV, LAY, UV)                                                                   \
+  do {                                                                                               \
+    if (plain)                                                                                       \
+      ew_flat<F, ReadDst, BC, NTV, LAY, UV><<<grid, kBlock, 0, st>>>(d, q, nvec, f);                 \
+    else                                                                                             \
+      ew_flat<F, ReadDst, BC, NTV, LAY, UV, FlatEdges><<<grid, kBlock, 0, st>>>(d, q, nvec, f, edges); \
+  } while (0)
   if (bcast) {
     if (nt)
-      ew_flat<F, ReadDst, true, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(true, true, 0, u2);
     else
-      ew_flat<F, ReadDst, true, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(true, false, 0, u2);
   } else if (ReadDst) {
     if (nt)
-      ew_flat<F, ReadDst, false, true, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(false, true, 1, u3);
     else
-      ew_flat<F, ReadDst, false, false, 1, u3><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(false, false, 1, u3);
   } else {
     if (nt)
-      ew_flat<F, ReadDst, false, true, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(false, true, 0, u2);
     else
-      ew_flat<F, ReadDst, false, false, 0, u2><<<(uint32_t)blocks, kBlock, 0, st>>>(d, q, nvec, f, (int)head, (int)tail);
+      WF2_FLAT(false, false, 0, u2);
   }
+#undef WF2_FLAT
   *rc = after_launch("ew_flat");
   return true;
 }
