@@ -394,8 +394,16 @@ static int launch_col_reduce(const AccParams& p, int64_t ncols) {
   if (ctiles * splits >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
   void* scratch = nullptr;
   if (splits > 1) {
-    WF2_TRY(wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(double)));
-    q.scratch = static_cast<double*>(scratch);
+    // no block to be had (inside a graph capture the pool is the only source): one
+    // workgroup per column tile instead
+    if (wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(double)) != 0) {
+      scratch = nullptr;
+      splits = 1;
+      q.splits = 1;
+      q.seg = p.nred;
+    } else {
+      q.scratch = static_cast<double*>(scratch);
+    }
   }
   hipStream_t st = rt().stream;
   if (p.nred * ncols * 4 >= ((int64_t)192 << 20))
