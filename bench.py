@@ -318,6 +318,20 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         measure(f"matmul {m}x{n}x{k}", ring, lambda s: F.matmul(s[0], s[1], out=s[2]), 2.0 * m * n * k,
                 bound="mfma")
         del a0, b0
+    # the layouts of LinearLayer and of its backward (source/nn/regression.lisp:13-17):
+    # x . W^T with W stored (out, in); dW = dY^T . x over a long K with few output tiles
+    m, n, k = 8192, 3072, 768
+    a0, w0 = normal([m, k]), normal([n, k])
+    ring = ring_of(lambda: (clone(a0), clone(w0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
+    measure(f"matmul {m}x{n}x{k}, right operand stored ({n},{k}) (!t)", ring,
+            lambda s: F.matmul(s[0], F.t(s[1]), out=s[2]), 2.0 * m * n * k, bound="mfma")
+    del a0, w0
+    m, n, k = 768, 3072, 8192
+    a0, b0 = normal([k, m]), normal([k, n])
+    ring = ring_of(lambda: (clone(a0), clone(b0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
+    measure(f"matmul {m}x{n}x{k}, left operand stored ({k},{m}) (!t), split over K", ring,
+            lambda s: F.matmul(F.t(s[0]), s[1], out=s[2]), 2.0 * m * n * k, bound="mfma")
+    del a0, b0
     B, H, S, hd = 8, 12, 1024, 64
     q0 = normal([B, H, S, hd])
     for causal in (True, False):
