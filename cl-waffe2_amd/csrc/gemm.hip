@@ -32,6 +32,7 @@
 
 #include "wf2_common.h"
 #include "wf2_math.h"
+#include "wf2_view.h"
 
 namespace wf2 {
 
@@ -849,6 +850,8 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
                    long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
                    long batch, long batch2, const Epilogue& ep = Epilogue());
 
+int binary_nd(int op, Space s, float* a, const float* b);  // elementwise.hip
+
 // A single product with few output tiles and a long K (weight gradients: 768 x 3072
 // outputs over K = 8192 are 144 tiles for 256 compute units) runs as `splits` products
 // over slices of K in one batched launch, folded in a fixed order afterwards.
@@ -899,6 +902,30 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
   if ((int64_t)batch * batch2 > 65535)
     return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  // x^T . dY (weight gradients): the left operand of the row-major product arrives stored
+  // (k, rows), which only the register-staged kernel reads.  One transposing pass over it
+  // (k x rows elements) puts the product on the streaming kernel.
+  if (batch == 1 && batch2 == 1 && !is_n(transb) && k >= 1024 && k % BK == 0 && n >= 128 && m >= 128 &&
+      aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && (is_n(transa) ? m % 4 == 0 : true)) {
+    void* turned = nullptr;
+    if (wf2hip_malloc_uninitialized(&turned, (size_t)k * n * sizeof(float)) == 0) {
+      Space sp;  // dst (k x n column-major): (kk, j) at kk + j k; src (n x k): j + kk ldb
+      sp.rank = 2;
+      sp.shape[0] = n;
+      sp.shape[1] = k;
+      sp.sa[0] = k;
+      sp.sa[1] = 1;
+      sp.sb[0] = 1;
+      sp.sb[1] = ldb;
+      sp.total = (int64_t)k * n;
+      int rc = binary_nd(WF2HIP_MOVE, sp, static_cast<float*>(turned), B);
+      if (rc == 0)
+        rc = sgemm_batched2(transa, 'N', m, n, k, alpha, A, lda, 0, 0, static_cast<const float*>(turned), k, 0, 0,
+                            beta, C, ldc, 0, 0, 1, 1, ep);
+      (void)wf2hip_free(turned);  // stream order keeps it alive for the launches above
+      return rc;
+    }
+  }
   if (batch == 1 && batch2 == 1 && !ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
     int rc = 0;
     if (try_split_k(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, &rc)) return rc;
