@@ -160,6 +160,31 @@ __global__ __launch_bounds__(kBlock) void select_rows_wave(SelParams<T> p) {
   if ((threadIdx.x & (kWave - 1)) == 0) emit(p, ooff, b);
 }
 
+// four short rows (at most one 16-byte vector per lane) per wavefront: their loads are
+// issued together; a wavefront with one row of 256 floats has 1 KB in flight
+// ((262144, 256): 46 % of the HBM peak)
+template <bool IsMax, bool VEC, class T>
+__global__ __launch_bounds__(kBlock) void select_rows_wave4(SelParams<T> p) {
+  constexpr int RW = 4;
+  const uint32_t row0 = (blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * RW;
+  if (row0 >= p.nrows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  Best<T> b[RW];
+  int64_t ooff[RW];
+#pragma unroll
+  for (int w = 0; w < RW; w++) {
+    const uint32_t row = row0 + w < p.nrows ? row0 + w : p.nrows - 1;
+    int64_t xoff;
+    sel_offsets(p, row, &xoff, &ooff[w]);
+    b[w] = scan<IsMax, VEC>(p.x + xoff, p.incx, 0, p.n, lane, kWave);
+  }
+#pragma unroll
+  for (int w = 0; w < RW; w++) {
+    b[w] = wave_best<IsMax>(b[w]);
+    if (lane == 0 && row0 + w < p.nrows) emit(p, ooff[w], b[w]);
+  }
+}
+
 // one workgroup per (row, split)
 template <bool IsMax, bool VEC, class T>
 __global__ __launch_bounds__(kBlock) void select_rows_block(SelParams<T> p) {
@@ -211,6 +236,11 @@ template <bool IsMax, bool VEC, class T>
 static int launch_select(SelParams<T>& p) {
   hipStream_t st = rt().stream;
   const int64_t target = (int64_t)rt().num_cus * 8;
+  if (p.n <= (int64_t)kWave * (16 / (int64_t)sizeof(T)) && p.nrows >= 4 * target) {
+    const uint32_t blocks = (uint32_t)ceil_div(p.nrows, (kBlock / kWave) * 4);
+    select_rows_wave4<IsMax, VEC, T><<<blocks, kBlock, 0, st>>>(p);
+    return after_launch("select_rows_wave4");
+  }
   if (p.n <= 2048 || (p.n < 8192 && p.nrows >= target)) {
     const uint32_t blocks = (uint32_t)ceil_div(p.nrows, kBlock / kWave);
     select_rows_wave<IsMax, VEC, T><<<blocks, kBlock, 0, st>>>(p);

@@ -249,6 +249,21 @@ def test_select_axis_views_and_keepdims(gpu, O):
         W.forward("ArgMax-Node", win, out)          # indices need a :uint32 destination
 
 
+def test_select_many_short_rows(gpu):
+    """Rows of at most one vector per lane, four to a wavefront: max / min / argmax /
+    argmin against numpy (first occurrence), ragged row counts and lengths."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(113)
+    for rows, cols in [(40000, 10), (33001, 256), (35000, 100), (32768, 64), (33333, 7)]:
+        X = rng.integers(-50, 50, (rows, cols)).astype(np.float32)  # many ties
+        dX = F.from_numpy(X)
+        np.testing.assert_array_equal(F.max(dX).numpy()[:, 0], X.max(axis=1))
+        np.testing.assert_array_equal(F.min(dX).numpy()[:, 0], X.min(axis=1))
+        np.testing.assert_array_equal(F.argmax(dX).numpy()[:, 0], X.argmax(axis=1))
+        np.testing.assert_array_equal(F.argmin(dX).numpy()[:, 0], X.argmin(axis=1))
+
+
 def test_select_full_size(gpu):
     """(8192, 8192): every row's maximum, and that x[argmax] is that maximum."""
     F = gpu.functional
