@@ -437,12 +437,12 @@ __global__ __launch_bounds__(kBlock) void typed_accumulate_add(T* a, const T* b,
   int64_t aoff, boff;
   acc_kept(p, out, &aoff, &boff);
   S acc = S(0);
-  // the innermost reduced axis is walked by the lanes, so a unit stride there coalesces
-  const int64_t inner = p.rshape[p.nr - 1], inner_stride = p.rb[p.nr - 1];
-  const int64_t outer = p.nred / inner;
-  for (int64_t o = threadIdx.x / kWave; o < outer; o += kBlock / kWave) {
-    const int64_t base = boff + acc_reduced(p, o * inner);
-    for (int64_t i = threadIdx.x & (kWave - 1); i < inner; i += kWave) acc += (S)b[base + i * inner_stride];
+  // consecutive threads take consecutive reduced indices: a unit stride on the innermost
+  // reduced axis coalesces, and a single long axis keeps all 256 threads busy
+  if (p.nr == 1) {
+    for (int64_t j = threadIdx.x; j < p.nred; j += kBlock) acc += (S)b[boff + j * p.rb[0]];
+  } else {
+    for (int64_t j = threadIdx.x; j < p.nred; j += kBlock) acc += (S)b[boff + acc_reduced(p, j)];
   }
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
@@ -454,6 +454,50 @@ __global__ __launch_bounds__(kBlock) void typed_accumulate_add(T* a, const T* b,
     for (int w = 1; w < kBlock / kWave; w++) total += lds[w];
     a[aoff] = (T)((S)a[aoff] + total);
   }
+}
+
+// Column form: the only kept axis is contiguous on both sides (sums over the leading
+// axes).  A thread owns one destination column, consecutive threads consecutive columns,
+// so every reduced index is one coalesced row segment; the reduced indices are split
+// over `splits` workgroups per 256 columns and folded by typed_accumulate_fold.
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_cols(T* a, const T* b, TypedAcc p, int64_t ncols,
+                                                                uint32_t splits, int64_t seg,
+                                                                typename SumOf<T>::type* partials) {
+  using S = typename SumOf<T>::type;
+  const uint32_t ctiles = (uint32_t)((ncols + kBlock - 1) / kBlock);
+  const uint32_t ctile = blockIdx.x % ctiles, split = blockIdx.x / ctiles;
+  const int64_t c = (int64_t)ctile * kBlock + threadIdx.x;
+  if (c >= ncols) return;
+  const int64_t lo = (int64_t)split * seg;
+  const int64_t hi = lo + seg < p.nred ? lo + seg : p.nred;
+  S acc0 = S(0), acc1 = S(0), acc2 = S(0), acc3 = S(0);
+  int64_t j = lo;
+  for (; j + 3 < hi; j += 4) {  // four rows in flight per thread
+    const T v0 = b[acc_reduced(p, j) + c], v1 = b[acc_reduced(p, j + 1) + c];
+    const T v2 = b[acc_reduced(p, j + 2) + c], v3 = b[acc_reduced(p, j + 3) + c];
+    acc0 += (S)v0;
+    acc1 += (S)v1;
+    acc2 += (S)v2;
+    acc3 += (S)v3;
+  }
+  for (; j < hi; j++) acc0 += (S)b[acc_reduced(p, j) + c];
+  const S total = (acc0 + acc1) + (acc2 + acc3);
+  if (splits == 1)
+    a[c] = (T)((S)a[c] + total);
+  else
+    partials[(int64_t)split * ncols + c] = total;
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_cols_fold(T* a, int64_t ncols, uint32_t splits,
+                                                                     const typename SumOf<T>::type* partials) {
+  using S = typename SumOf<T>::type;
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= ncols) return;
+  S total = S(0);
+  for (uint32_t s = 0; s < splits; s++) total += partials[(int64_t)s * ncols + c];
+  a[c] = (T)((S)a[c] + total);
 }
 
 // Few destinations, long reductions: `splits` workgroups per destination each sum a
@@ -544,6 +588,35 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
     if (p.nout >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
     using S = typename SumOf<T>::type;
     const int64_t target = (int64_t)rt().num_cus * 8;
+    const int last = s.rank - 1;
+    if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 16) {
+      const int64_t ncols = s.shape[last];
+      const int64_t ctiles = ceil_div(ncols, kBlock);
+      int64_t splits = ceil_div(target, ctiles);
+      if (splits > p.nred / 32) splits = p.nred / 32;
+      if (splits < 1) splits = 1;
+      int64_t seg = ceil_div(p.nred, splits);
+      splits = ceil_div(p.nred, seg);
+      void* scratch = nullptr;
+      if (splits > 1 && wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(S)) != 0) {
+        scratch = nullptr;
+        splits = 1;
+        seg = p.nred;
+      }
+      if (ctiles * splits < ((int64_t)1 << 31)) {
+        typed_accumulate_cols<T><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(ap, bp, p, ncols, (uint32_t)splits, seg,
+                                                                               static_cast<S*>(scratch));
+        int rc = after_launch("typed_accumulate_cols");
+        if (rc == 0 && splits > 1) {
+          typed_accumulate_cols_fold<T><<<(uint32_t)ctiles, kBlock, 0, st>>>(ap, ncols, (uint32_t)splits,
+                                                                            static_cast<const S*>(scratch));
+          rc = after_launch("typed_accumulate_cols_fold");
+        }
+        if (scratch) (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
+        return rc;
+      }
+      if (scratch) (void)wf2hip_free(scratch);
+    }
     const int64_t capacity = (int64_t)(kPartialCapacity * sizeof(float) / sizeof(S));
     if (p.nout < target && p.nred >= 2 * 16384 && p.nout <= capacity / 2) {
       int64_t splits = ceil_div(p.nred, 16384);

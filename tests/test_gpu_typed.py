@@ -193,6 +193,16 @@ def test_accumulation_into_broadcast_destinations(gpu, dtype):
                 assert np.max(np.abs(got.numpy() - want)) < 1e-9
             else:
                 np.testing.assert_array_equal(got.numpy(), want)
+        # sums over the leading axes with a contiguous kept axis of 64 columns or more (column form)
+        for shape, axis in (((700, 130), 0), ((33, 40, 260), (0, 1)), ((5000, 64), 0)):
+            Z = (rng.standard_normal(shape) if dtype == "double"
+                 else rng.integers(info.min, info.max, shape, endpoint=True).astype(npt))
+            got = F.sum(F.from_numpy(Z, dtype=dtype), axis=axis)
+            want = Z.sum(axis=axis, keepdims=True, dtype=npt if dtype != "double" else np.float64)
+            if dtype == "double":
+                assert np.max(np.abs(got.numpy() - want)) < 1e-9
+            else:
+                np.testing.assert_array_equal(got.numpy(), want)
         # x[0, j] <- x[0, j] - sum_i y[i, j], sequentially
         base = A[0, 0:1, :].copy()
         dst = F.from_numpy(base, dtype=dtype).view((":broadcast", 300), True)
