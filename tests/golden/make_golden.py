@@ -47,7 +47,7 @@ def main():
                 O.binary_1d(op, n, res, incx, y, incy, use_ref=True)
                 key = f"bin_{op}_{n}_{incx}_{incy}"
                 out[key + "_x"], out[key + "_y"], out[key + "_out"] = x, y, res
-    # out <- f(x): BASELINE ranges (n = 2048 + 5 so that the libm tail is hit),
+    # out <- f(x): the ranges of the transcendental benchmark configuration (n = 2048 + 5 so that the libm tail is hit),
     # edge values, strided in/out, broadcast source
     for op, (lo, hi) in UNARY.items():
         x = rng.uniform(lo, hi, 2053).astype(np.float32)

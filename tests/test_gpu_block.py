@@ -47,7 +47,7 @@ def test_block_ragged(gpu):
 
 
 def test_block_config5(gpu):
-    """BASELINE config 5: B 8, T 1024, D 768, 12 heads x 64, seed 5."""
+    """benchmark configuration 5: B 8, T 1024, D 768, 12 heads x 64, seed 5."""
     gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
     from oracle import gpt2_block_ref as ref
     W = gpu

@@ -151,7 +151,7 @@ def test_relu_and_sigmoid(gpu):
 
 
 def test_compare_full_size(gpu):
-    """2^26 elements through the streaming kernel; ReLU at BASELINE size via the
+    """2^26 elements through the streaming kernel; ReLU at the benchmark size via the
     identity relu(x) + relu(-x) = |x| (bitwise)."""
     F = gpu.functional
     rng = np.random.Generator(np.random.PCG64(8))

@@ -72,7 +72,7 @@ def test_ieee_special_values(gpu):
 
 
 def test_config1_contiguous(gpu, O):
-    """BASELINE config 1: Z1 = A + B, Z2 = A * B on (1024, 1024) N(0,1), seed 1,
+    """benchmark configuration 1: Z1 = A + B, Z2 = A * B on (1024, 1024) N(0,1), seed 1,
     through !add / !mul (copy + in-place node)."""
     W = gpu
     F = W.functional
@@ -88,7 +88,7 @@ def test_config1_contiguous(gpu, O):
 
 
 def test_config2_views(gpu, O):
-    """BASELINE config 2: row-broadcast add, column-stride-2 slice times 0.5,
+    """benchmark configuration 2: row-broadcast add, column-stride-2 slice times 0.5,
     subtraction of offset views -- against the oracle running the reference's
     own per-row schedule."""
     W = gpu
@@ -412,7 +412,7 @@ CFG3 = [("exp", -10, 10), ("tanh", -10, 10), ("sin", -100, 100), ("log", 1e-3, 1
 
 @pytest.mark.parametrize("op,lo,hi", CFG3)
 def test_config3_transcendentals(gpu, O, op, lo, hi):
-    """BASELINE config 3 ranges (seed 3) on 2^22 elements: <= 2 ulp from the
+    """benchmark configuration 3 ranges (seed 3) on 2^22 elements: <= 2 ulp from the
     oracle's SLEEF u10 results and <= 1 ulp from float64 truth."""
     W = gpu
     rng = np.random.Generator(np.random.PCG64(3))
@@ -432,7 +432,7 @@ def test_config3_transcendentals(gpu, O, op, lo, hi):
 
 @pytest.mark.parametrize("op,lo,hi", CFG3[:4])
 def test_config3_full_size(gpu, O, op, lo, hi):
-    """BASELINE config 3 at its full size, 2^26 elements in one flat call (the
+    """benchmark configuration 3 at its full size, 2^26 elements in one flat call (the
     non-temporal streaming kernel): same bars as above."""
     W = gpu
     rng = np.random.Generator(np.random.PCG64(3))

@@ -1,6 +1,6 @@
 """GPU parity of reductions, softmax, LayerNorm and gemm.
 
-Bar (BASELINE north_star): <= 1e-5 relative error for reductions and gemm
+Bar: <= 1e-5 relative error for reductions and gemm
 (relative to the sum of magnitudes, because a sum of N(0,1) values is itself
 ~0); bit-exact against the oracle in the sequential reduce mode; the
 reference's own integer test vectors exactly.
@@ -86,7 +86,7 @@ def test_many_short_rows(gpu):
 
 
 def test_config4_row_and_full_sum(gpu, O):
-    """BASELINE config 4: row sum and full sum of (8192, 4096) N(0,1), seed 4.
+    """benchmark configuration 4: row sum and full sum of (8192, 4096) N(0,1), seed 4.
     Tree mode against float64 truth; a slice of it in sequential mode against
     the oracle's strictly ordered fp32 accumulation, bit for bit."""
     W = gpu
@@ -186,7 +186,7 @@ def _assert_softmax(got, want64, what=""):
 
 
 def test_config4_softmax(gpu):
-    """BASELINE config 4: max-subtracted row softmax of (32768, 1024) N(0, 3^2)
+    """benchmark configuration 4: max-subtracted row softmax of (32768, 1024) N(0, 3^2)
     logits, seed 4 -- fused kernel against the float64 closed form; invariants
     of the reference's tests (rows sum to 1, nn/t/activation.lisp:9-12) and
     shift invariance."""
