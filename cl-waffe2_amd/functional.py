@@ -516,7 +516,7 @@ def matmul(a, b, out: HIPTensor | None = None, bias: HIPTensor | None = None,
     bshape = b.shape if trans_b else bt.shape
     batch = ashape[:-2] if len(ashape) >= len(bshape) else bshape[:-2]
     if out is None:
-        out = HIPTensor(list(batch) + [ashape[-2], bshape[-1]], initial_element=None)
+        out = HIPTensor(list(batch) + [ashape[-2], bshape[-1]], dtype=at.dtype, initial_element=None)
 
     def with_batch(x: HIPTensor) -> HIPTensor:
         if x.shape[:-2] == list(batch):

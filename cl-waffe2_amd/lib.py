@@ -61,6 +61,7 @@ class View2(C.Structure):
 _P = C.c_void_p
 _L = C.c_long
 _F = C.c_float
+_D = C.c_double
 
 
 class View3(C.Structure):
@@ -184,6 +185,11 @@ _SIGNATURES = {
     "wf2hip_attention_f32": ([C.POINTER(AttentionDesc), _P, _P, _P, _P], C.c_int),
     "wf2hip_sgemm_strided_batched_2d": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],
+        C.c_int,
+    ),
+    "wf2hip_dgemm": ([C.c_char, C.c_char, _L, _L, _L, _D, _P, _L, _P, _L, _D, _P, _L], C.c_int),
+    "wf2hip_dgemm_strided_batched_2d": (
+        [C.c_char, C.c_char, _L, _L, _L, _D, _P, _L, _L, _L, _P, _L, _L, _L, _D, _P, _L, _L, _L, _L, _L],
         C.c_int,
     ),
 }

@@ -106,6 +106,12 @@
   (b :pointer) (ldb :long) (stride-b :long) (stride-b2 :long)
   (beta :float) (c :pointer) (ldc :long) (stride-c :long) (stride-c2 :long) (batch :long) (batch2 :long))
 
+(defcfun "wf2hip_dgemm_strided_batched_2d" :int
+  (transa :char) (transb :char) (m :long) (n :long) (k :long) (alpha :double)
+  (a :pointer) (lda :long) (stride-a :long) (stride-a2 :long)
+  (b :pointer) (ldb :long) (stride-b :long) (stride-b2 :long)
+  (beta :double) (c :pointer) (ldc :long) (stride-c :long) (stride-c2 :long) (batch :long) (batch2 :long))
+
 ;; struct wf2hip_matmul_desc
 (defcstruct matmul-desc
   (trans-a :int32) (trans-b :int32) (activation :int32) (causal :int32)

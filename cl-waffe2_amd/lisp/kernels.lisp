@@ -255,7 +255,7 @@ extension has both, source/backends/cpu/mathematics.lisp:8-76)."
              (values extents strides (foreign-slot-value view '(:struct view2) 'off-a))))
       (foreign-free view))))
 
-(define-impl-op (MatMulNode :device HIPTensor :reject-p #'only-float-p)
+(define-impl-op (MatMulNode :device HIPTensor :reject-p #'float-or-double-p)
                 :forward ((self a b out)
                           (ensure-extension)
                           (let ((trans-a (trans-a? self))
@@ -274,14 +274,25 @@ extension has both, source/backends/cpu/mathematics.lisp:8-76)."
                                          (ldc (max 1 (nth (- rank 2) sc)))
                                          (batch-rank (- rank 2)))
                                     (labels ((launch (oa ob oc stride-a stride-b stride-c count)
-                                               (check (wf2hip-sgemm-strided-batched
-                                                       (char-code (if trans-b #\C #\N))
-                                                       (char-code (if trans-a #\C #\N))
-                                                       n m k 1.0
-                                                       (tensor-device-pointer b ob) ldb stride-b
-                                                       (tensor-device-pointer a oa) lda stride-a
-                                                       0.0
-                                                       (tensor-device-pointer out oc) ldc stride-c count)))
+                                               ;; sgemm_ or dgemm_ by dtype, like expand-gemm-form-column
+                                               ;; (source/backends/cpu/matrix-ops.lisp:12-112)
+                                               (if (eql (dtype out) :double)
+                                                   (check (wf2hip-dgemm-strided-batched-2d
+                                                           (char-code (if trans-b #\C #\N))
+                                                           (char-code (if trans-a #\C #\N))
+                                                           n m k 1.0d0
+                                                           (tensor-device-pointer b ob) ldb stride-b 0
+                                                           (tensor-device-pointer a oa) lda stride-a 0
+                                                           0.0d0
+                                                           (tensor-device-pointer out oc) ldc stride-c 0 count 1))
+                                                   (check (wf2hip-sgemm-strided-batched
+                                                           (char-code (if trans-b #\C #\N))
+                                                           (char-code (if trans-a #\C #\N))
+                                                           n m k 1.0
+                                                           (tensor-device-pointer b ob) ldb stride-b
+                                                           (tensor-device-pointer a oa) lda stride-a
+                                                           0.0
+                                                           (tensor-device-pointer out oc) ldc stride-c count))))
                                              (walk (axis oa ob oc)
                                                (cond
                                                  ((= batch-rank 0) (launch oa ob oc 0 0 0 1))

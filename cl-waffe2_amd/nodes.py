@@ -329,7 +329,7 @@ def _matrix_geometry(t: HIPTensor, what: str):
     return shape, strides, off, ld
 
 
-@define_impl("MatMulNode", HIPTensor, _only_float)
+@define_impl("MatMulNode", HIPTensor, _float_or_double)
 def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
             trans_b: bool = False, bias: HIPTensor | None = None,
             residual: HIPTensor | None = None, activation: str | None = None,
@@ -342,7 +342,12 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
 
     ``bias`` / ``activation`` / ``residual`` / ``causal`` select the fused
     epilogue of ``wf2hip_matmul_fused`` (not part of MatMulNode: what a
-    ``define-bypass`` fusion of MatMulNode + AddNode (+ !gelu) would call)."""
+    ``define-bypass`` fusion of MatMulNode + AddNode (+ !gelu) would call).
+
+    :double operands take ``wf2hip_dgemm_strided_batched_2d`` (the CPU backend's
+    dgemm_ branch of the same expansion); the fused epilogues are :float only."""
+    if not (a.dtype == b.dtype == out.dtype):
+        raise ValueError(f"MatMulNode: dtype mismatch: {a.dtype}, {b.dtype} -> {out.dtype}")
     sa, sta, oa, lda = _matrix_geometry(a, "A")
     sb, stb, ob, ldb = _matrix_geometry(b, "B")
     sc, stc, oc, ldc = _matrix_geometry(out, "C")
@@ -356,6 +361,8 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     if sa[:-2] != batch_shape or sb[:-2] != batch_shape:
         raise ValueError("MatMulNode: batch axes differ; view the smaller operand with (:broadcast n)")
     fused = bias is not None or residual is not None or activation is not None or causal
+    if fused and a.dtype != "float":
+        raise ValueError("MatMulNode: bias / activation / residual / causal epilogues are :float only")
     tensors = [sta, stb, stc]
     ores = ldres = 0
     if residual is not None:
@@ -374,11 +381,14 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     def launch(offs, inner, outer):
         (count, s3), (count2, s3o) = inner, outer
         if not fused:
-            _lib.check(lib.wf2hip_sgemm_strided_batched_2d(
+            gemm = lib.wf2hip_sgemm_strided_batched_2d if a.dtype == "float" \
+                else lib.wf2hip_dgemm_strided_batched_2d
+            w = a.itemsize
+            _lib.check(gemm(
                 tb, ta, n, m, k, 1.0,
-                C.c_void_p(b.ptr + 4 * offs[1]), ldb, s3[1], s3o[1],
-                C.c_void_p(a.ptr + 4 * offs[0]), lda, s3[0], s3o[0],
-                0.0, C.c_void_p(out.ptr + 4 * offs[2]), ldc, s3[2], s3o[2], count, count2))
+                C.c_void_p(b.ptr + w * offs[1]), ldb, s3[1], s3o[1],
+                C.c_void_p(a.ptr + w * offs[0]), lda, s3[0], s3o[0],
+                0.0, C.c_void_p(out.ptr + w * offs[2]), ldc, s3[2], s3o[2], count, count2))
             return
         d = _lib.MatmulDesc()
         d.trans_a, d.trans_b = int(trans_a), int(trans_b)

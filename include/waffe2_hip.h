@@ -601,6 +601,19 @@ int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, long n, lo
                                     long strideB2, float beta, float* C, long ldc, long strideC,
                                     long strideC2, long batch, long batch2);
 
+/* The :double product: Fortran dgemm_ with scalars by value, the other branch
+ * of the same expansion (matrix-ops.lisp:12-112 picks sgemm_ or dgemm_ by
+ * dtype; blas-functions.lisp:34-38).  binary64 FMA on the vector ALUs, one
+ * 64 x 64 tile per workgroup; at most 65535 matrices per call. */
+int wf2hip_dgemm(char transa, char transb, long m, long n, long k, double alpha,
+                 const double* A, long lda, const double* B, long ldb, double beta,
+                 double* C, long ldc);
+int wf2hip_dgemm_strided_batched_2d(char transa, char transb, long m, long n, long k,
+                                    double alpha, const double* A, long lda, long strideA,
+                                    long strideA2, const double* B, long ldb, long strideB,
+                                    long strideB2, double beta, double* C, long ldc, long strideC,
+                                    long strideC2, long batch, long batch2);
+
 /* ---- fused matmul (extension; no BLAS counterpart) ------------------------- */
 /* Row-major C[m,n] = act(alpha * op(A)[m,k] . op(B)[k,n] + bias[n]) + residual[m,n]
  * in one kernel: the bias add, GELU and residual add that cl-waffe2 runs as
