@@ -4,10 +4,11 @@
 // matrix-ops.lisp:12-112 expands to sgemm_ or dgemm_ by dtype; binding
 // blas-functions.lisp:34-38).  This is the same contract as wf2hip_sgemm --
 // column-major C(m x n) <- alpha op(A) op(B) + beta C, scalars by value -- on
-// binary64 with FMA accumulation.  It is a plain LDS-tiled kernel on the vector
-// ALUs (64 x 64 outputs per workgroup, 4 x 4 per thread, K in steps of 16): the
-// :double path is there so that models keep running on the device, the tuned
-// matrix-core kernels are the :float ones in gemm.hip.
+// binary64 on the matrix cores (v_mfma_f64_16x16x4, fused multiply-add).  It is a
+// plain LDS-tiled kernel (128 x 128 or 64 x 64 outputs per workgroup, a quarter
+// per wavefront, K in steps of 16 with the next step prefetched into registers): the :double path is there so that
+// models keep running on the device, the tuned kernels are the :float ones in
+// gemm.hip.
 #include "wf2_common.h"
 
 namespace wf2 {
@@ -22,64 +23,104 @@ struct DgemmParams {
   double alpha, beta;
 };
 
-constexpr int kDT = 64;   // tile edge
+typedef double d4 __attribute__((ext_vector_type(4)));
+
 constexpr int kDK = 16;   // K step
 
-template <bool TA, bool TB>
+// TILE x TILE outputs per workgroup of four wavefronts (2 x 2), TILE / 2 squared per wavefront as
+// (TILE / 32)^2 matrix-core tiles.  The next K step's operands are fetched into registers while the
+// current one is multiplied out of LDS.
+template <bool TA, bool TB, int TILE>
 __global__ __launch_bounds__(kBlock) void dgemm_kernel(DgemmParams p) {
-  __shared__ double As[kDK][kDT + 1];
-  __shared__ double Bs[kDK][kDT + 1];
+  constexpr int NT = TILE / 32;              // matrix-core tiles per wavefront and dimension
+  constexpr int PER = TILE * kDK / kBlock;   // elements of each operand per thread and K step
+  __shared__ double As[kDK][TILE + 1];
+  __shared__ double Bs[kDK][TILE + 1];
   const uint32_t bi = blockIdx.z % p.batch_inner, bo = blockIdx.z / p.batch_inner;
   const double* A = p.A + (int64_t)bi * p.sA + (int64_t)bo * p.sA2;
   const double* B = p.B + (int64_t)bi * p.sB + (int64_t)bo * p.sB2;
   double* C = p.C + (int64_t)bi * p.sC + (int64_t)bo * p.sC2;
-  const int64_t i0 = (int64_t)blockIdx.x * kDT, j0 = (int64_t)blockIdx.y * kDT;
-  const int t = threadIdx.x, tx = t & 15, ty = t >> 4;
-  double acc[4][4] = {};
+  const int64_t i0 = (int64_t)blockIdx.x * TILE, j0 = (int64_t)blockIdx.y * TILE;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wr = (wave & 1) * (TILE / 2), wc = (wave >> 1) * (TILE / 2);
+  const int l16 = lane & 15, lq = lane >> 4;
+  // op(A)(i, kk) and op(B)(kk, j): consecutive threads along the axis that is contiguous in memory
+  auto a_pos = [&](int r, int& i, int& kk) {
+    const int e = t + kBlock * r;
+    if (TA) { kk = e % kDK; i = e / kDK; } else { i = e % TILE; kk = e / TILE; }
+  };
+  auto b_pos = [&](int r, int& j, int& kk) {
+    const int e = t + kBlock * r;
+    if (TB) { j = e % TILE; kk = e / TILE; } else { kk = e % kDK; j = e / kDK; }
+  };
+  double ra[PER], rb[PER];
+  auto fetch = [&](int64_t k0) {
+#pragma unroll
+    for (int r = 0; r < PER; r++) {
+      int i, kk;
+      a_pos(r, i, kk);
+      const int64_t gi = i0 + i, gk = k0 + kk;
+      ra[r] = (gi < p.m && gk < p.k) ? (TA ? A[gk + gi * p.lda] : A[gi + gk * p.lda]) : 0.0;
+      int j, kb;
+      b_pos(r, j, kb);
+      const int64_t gj = j0 + j, gkb = k0 + kb;
+      rb[r] = (gj < p.n && gkb < p.k) ? (TB ? B[gj + gkb * p.ldb] : B[gkb + gj * p.ldb]) : 0.0;
+    }
+  };
+  d4 acc[NT][NT] = {};
+  if (p.k > 0) fetch(0);
   for (int64_t k0 = 0; k0 < p.k; k0 += kDK) {
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      // op(A)(i, kk): consecutive threads along the axis that is contiguous in memory
-      const int i = TA ? (t >> 4) + 16 * r : (t & 63);
-      const int kk = TA ? (t & 15) : (t >> 6) + 4 * r;
-      const int64_t gi = i0 + i, gk = k0 + kk;
-      double v = 0.0;
-      if (gi < p.m && gk < p.k) v = TA ? A[gk + gi * p.lda] : A[gi + gk * p.lda];
-      As[kk][i] = v;
-      // op(B)(kk, j)
-      const int j = TB ? (t & 63) : (t >> 4) + 16 * r;
-      const int kb = TB ? (t >> 6) + 4 * r : (t & 15);
-      const int64_t gj = j0 + j, gkb = k0 + kb;
-      double w = 0.0;
-      if (gj < p.n && gkb < p.k) w = TB ? B[gj + gkb * p.ldb] : B[gkb + gj * p.ldb];
-      Bs[kb][j] = w;
+    for (int r = 0; r < PER; r++) {
+      int i, kk, j, kb;
+      a_pos(r, i, kk);
+      As[kk][i] = ra[r];
+      b_pos(r, j, kb);
+      Bs[kb][j] = rb[r];
     }
     __syncthreads();
+    if (k0 + kDK < p.k) fetch(k0 + kDK);
 #pragma unroll
-    for (int kk = 0; kk < kDK; kk++) {
-      double a[4], b[4];
+    for (int kk = 0; kk < kDK; kk += 4) {
+      // v_mfma_f64_16x16x4: D(16 x 16) += L(16 x 4) R(4 x 16); lane l supplies L[l%16][l/16] and
+      // R[l/16][l%16] and holds D[l/16 + 4 r][l%16] in register r (rows interleaved, unlike the
+      // binary32 forms).  L is taken from op(B) and R from op(A), so that D is the transposed
+      // output tile and l%16 runs along C's contiguous (row) index.
+      double a[NT], b[NT];
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        a[u] = As[kk][tx + 16 * u];
-        b[u] = Bs[kk][ty + 16 * u];
+      for (int u = 0; u < NT; u++) {
+        a[u] = As[kk + lq][wr + 16 * u + l16];
+        b[u] = Bs[kk + lq][wc + 16 * u + l16];
       }
 #pragma unroll
-      for (int u = 0; u < 4; u++)
+      for (int u = 0; u < NT; u++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) acc[u][v] = __builtin_fma(a[u], b[v], acc[u][v]);
+        for (int v = 0; v < NT; v++)
+          acc[u][v] = __builtin_amdgcn_mfma_f64_16x16x4f64(b[v], a[u], acc[u][v], 0, 0, 0);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int u = 0; u < 4; u++)
+  for (int u = 0; u < NT; u++)
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int64_t gi = i0 + tx + 16 * u, gj = j0 + ty + 16 * v;
-      if (gi < p.m && gj < p.n) {
-        double* c = C + gi + gj * p.ldc;
-        *c = p.beta == 0.0 ? p.alpha * acc[u][v] : p.alpha * acc[u][v] + p.beta * *c;
+    for (int v = 0; v < NT; v++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int64_t gi = i0 + wr + 16 * u + l16, gj = j0 + wc + 16 * v + lq + 4 * r;
+        if (gi < p.m && gj < p.n) {
+          double* c = C + gi + gj * p.ldc;
+          const double x = acc[u][v][r];
+          *c = p.beta == 0.0 ? p.alpha * x : p.alpha * x + p.beta * *c;
+        }
       }
-    }
+}
+
+template <int TILE>
+static void launch_dgemm(const DgemmParams& p, bool ta, bool tb, dim3 grid, hipStream_t st) {
+  if (ta && tb) dgemm_kernel<true, true, TILE><<<grid, kBlock, 0, st>>>(p);
+  else if (ta) dgemm_kernel<true, false, TILE><<<grid, kBlock, 0, st>>>(p);
+  else if (tb) dgemm_kernel<false, true, TILE><<<grid, kBlock, 0, st>>>(p);
+  else dgemm_kernel<false, false, TILE><<<grid, kBlock, 0, st>>>(p);
 }
 
 static bool dn(char c) { return c == 'N' || c == 'n'; }
@@ -105,15 +146,16 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
   p.sA2 = strideA2; p.sB2 = strideB2; p.sC2 = strideC2;
   p.batch_inner = (uint32_t)batch;
   p.alpha = alpha; p.beta = beta;
-  const int64_t gx = ceil_div(m, kDT), gy = ceil_div(n, kDT);
+  // 128 x 128 tiles once they fill the chip twice over, 64 x 64 below that
+  const int64_t big = ceil_div(m, 128) * ceil_div(n, 128) * batch * batch2;
+  const int tile = big >= 2 * (int64_t)rt().num_cus ? 128 : 64;
+  const int64_t gx = ceil_div(m, tile), gy = ceil_div(n, tile);
   if (gx >= ((int64_t)1 << 31) || gy > 65535) return fail(WF2HIP_EUNSUPPORTED, "matrix too large for one launch");
   dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)(batch * batch2));
   hipStream_t st = rt().stream;
   const bool ta = !dn(transa), tb = !dn(transb);
-  if (ta && tb) dgemm_kernel<true, true><<<grid, kBlock, 0, st>>>(p);
-  else if (ta) dgemm_kernel<true, false><<<grid, kBlock, 0, st>>>(p);
-  else if (tb) dgemm_kernel<false, true><<<grid, kBlock, 0, st>>>(p);
-  else dgemm_kernel<false, false><<<grid, kBlock, 0, st>>>(p);
+  if (tile == 128) launch_dgemm<128>(p, ta, tb, grid, st);
+  else launch_dgemm<64>(p, ta, tb, grid, st);
   return after_launch("dgemm_kernel");
 }
 

@@ -130,3 +130,25 @@ def test_double_matmul_rejects_mixed_dtypes_and_fused_epilogues(gpu):
         F.matmul(a, b)
     with pytest.raises(ValueError):
         F.matmul(a, a, activation="gelu")
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_double_matmul_large_tiles(gpu, ta, tb):
+    """Enough 128 x 128 tiles to fill the chip twice over select the large-tile
+    form of the kernel; sizes off the tile in every dimension."""
+    F = gpu.functional
+    batch, m, n, k = 26, 500, 515, 70
+    rng = np.random.default_rng(11 + 2 * ta + tb)
+    A = rng.standard_normal((batch, k, m) if ta else (batch, m, k))
+    B = rng.standard_normal((batch, n, k) if tb else (batch, k, n))
+    a, b = D(A), D(B)
+    got = F.matmul(F.t(a) if ta else a, F.t(b) if tb else b).numpy()
+    assert got.shape == (batch, m, n)
+    opA = A.transpose(0, 2, 1) if ta else A
+    opB = B.transpose(0, 2, 1) if tb else B
+    want = opA @ opB
+    scale = np.abs(opA) @ np.abs(opB)
+    assert np.max(np.abs(got - want) / scale) <= 8 * k * EPS
+    _check(got[0], opA[0], opB[0], what="first matrix, extended precision")
+    _check(got[-1], opA[-1], opB[-1], what="last matrix, extended precision")
