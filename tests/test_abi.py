@@ -57,6 +57,7 @@ def test_no_gpu_means_errors_not_fallbacks(W):
     # every compute entry refuses to run before a successful init
     assert lib.wf2hip_sadd(4, None, 1, None, 1) == -2
     assert lib.wf2hip_sgemm(b"N", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0, None, 1) == -2
+    assert lib.wf2hip_dgemm(b"N", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0, None, 1) == -2
     p = C.c_void_p()
     assert lib.wf2hip_malloc(C.byref(p), 16) == -2 and not p.value
     with pytest.raises(W.HIPError):
