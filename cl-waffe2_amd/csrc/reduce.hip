@@ -466,7 +466,9 @@ static void split_axes(const Space& s, AccParams* p) {
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-static int launch_row_reduce(const Space& s, float* a, const float* b) {
+// `partials` holds at least kPartialCapacity / 2 binary64 sums: the library's
+// own buffer, or the static array of the allocation-free entry point.
+static int launch_row_reduce(const Space& s, float* a, const float* b, double* partials) {
   const int last = s.rank - 1;
   RowRedParams p;
   p.a = a + s.off_a;
@@ -484,7 +486,7 @@ static int launch_row_reduce(const Space& s, float* a, const float* b) {
     if (s.sb[r] % 4 != 0) vec_ok = false;
   }
   p.nrows = (uint32_t)nrows;
-  p.partials = reinterpret_cast<double*>(rt().partials);
+  p.partials = partials;
   p.splits = 1;
   p.seg = p.n0;
   hipStream_t st = rt().stream;
@@ -550,7 +552,8 @@ static int launch_row_reduce(const Space& s, float* a, const float* b) {
 }
 
 // a <- a op b where `a` has broadcast (stride-0) axes.  `s` is normalised.
-int launch_accumulate(int op, const Space& s, float* a, const float* b) {
+// `row_partials` replaces the library's partial-sum buffer for the row form.
+static int launch_accumulate_with(int op, const Space& s, float* a, const float* b, double* row_partials) {
   hipStream_t st = rt().stream;
   const bool sequential = op != WF2HIP_ADD || rt().reduce_mode == 1;
   AccParams p;
@@ -577,7 +580,7 @@ int launch_accumulate(int op, const Space& s, float* a, const float* b) {
                   p.nout < ((int64_t)1 << 31);
   for (int r = 0; r < last; r++)
     if (s.shape[r] >= ((int64_t)1 << 32)) row_form = false;
-  if (row_form) return launch_row_reduce(s, a, b);
+  if (row_form) return launch_row_reduce(s, a, b, row_partials);
   // column form: the only kept axis is the last one, contiguous on both sides
   if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 16)
     return launch_col_reduce(p, s.shape[last]);
@@ -586,6 +589,10 @@ int launch_accumulate(int op, const Space& s, float* a, const float* b) {
     return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
   accumulate_generic<<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   return after_launch("accumulate_generic");
+}
+
+int launch_accumulate(int op, const Space& s, float* a, const float* b) {
+  return launch_accumulate_with(op, s, a, b, reinterpret_cast<double*>(rt().partials));
 }
 
 // ---- max / min ------------------------------------------------------------------
@@ -1032,6 +1039,65 @@ WF2_API int wf2hip_reduce_add_rows_f32(long rows, long cols, const float* x, lon
   s.off_a = s.off_b = 0;
   s.total = (int64_t)rows * cols;
   return binary_nd(WF2HIP_ADD, s, out, x);
+}
+
+// ---- row sums without any allocation ---------------------------------------------
+// For callers that cannot allocate device memory (code under graph capture, tight
+// serving loops, harnesses that forbid it): the partial sums of rows split over
+// several workgroups live in a static device array instead of a buffer the library
+// allocates.  Every device holds its own copy of the array at its own address, which
+// wf2hip_init looks up once per device; host code only ever uses that address.
+constexpr int64_t kStaticPartials = kPartialCapacity / 2;  // binary64 sums, 256 KiB
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) double scratch[kStaticPartials];
+static double* g_scratch_ptr[kMaxDevices];
+
+namespace wf2 {
+// Called by wf2hip_init with `device` current.
+int reduce_setup_device(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    return fail(WF2HIP_EUNSUPPORTED, "device ordinal %d beyond the %d this library keeps state for", device,
+                kMaxDevices);
+  if (g_scratch_ptr[device]) return 0;
+  double* ptr = nullptr;
+  WF2_TRY(check_hip(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"));
+  if (!ptr) return fail(WF2HIP_EINVAL, "hipGetSymbolAddress(scratch) returned a null address");
+  g_scratch_ptr[device] = ptr;
+  return 0;
+}
+}  // namespace wf2
+
+WF2_API int wf2hip_reduce_add_rows_f32_noalloc(long rows, long cols, const float* x, long ldx, float* out,
+                                               long inco) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if ((int64_t)rows > WF2HIP_NOALLOC_MAX_ELEMENTS || (int64_t)cols > WF2HIP_NOALLOC_MAX_ELEMENTS ||
+      (rows > 0 && (int64_t)cols > WF2HIP_NOALLOC_MAX_ELEMENTS / rows))
+    return fail(WF2HIP_EUNSUPPORTED,
+                "wf2hip_reduce_add_rows_f32_noalloc: %ld x %ld elements exceed the maximum of %lld this "
+                "entry point accepts; use wf2hip_reduce_add_rows_f32",
+                rows, cols, (long long)WF2HIP_NOALLOC_MAX_ELEMENTS);
+  if (rows == 0 || cols == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  const int device = rt().device;
+  double* partials = device >= 0 && device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
+  if (!partials) return fail(WF2HIP_ENOTINIT, "the static scratch of device %d was not set up by wf2hip_init", device);
+  Space s;
+  s.rank = 2;
+  s.shape[0] = rows;
+  s.shape[1] = cols;
+  s.sa[0] = inco;
+  s.sa[1] = 0;
+  s.sb[0] = ldx;
+  s.sb[1] = 1;
+  s.off_a = s.off_b = 0;
+  s.total = (int64_t)rows * cols;
+  normalise(&s);
+  if (hazardous_overlap(s, out, x))
+    return fail(WF2HIP_EOVERLAP, "row sums into a window that overlaps the source");
+  // cols == 1 leaves no reduced axis: a plain strided add, which uses no scratch
+  if (!has_broadcast_axis(s, s.sa)) return binary_nd(WF2HIP_ADD, s, out, x);
+  return launch_accumulate_with(WF2HIP_ADD, s, out, x, partials);
 }
 
 WF2_API int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long ldx, float* out,

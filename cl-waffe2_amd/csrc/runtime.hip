@@ -23,6 +23,8 @@ static thread_local char g_err[512] = "";
 
 Runtime& rt() { return g_rt; }
 
+int reduce_setup_device(int device);  // reduce.hip: address of its static scratch on this device
+
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -173,6 +175,7 @@ WF2_API int wf2hip_init(int device) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(WF2HIP_EUNSUPPORTED, "kernels are built for gfx950 only, device is %s",
                 prop.gcnArchName);
+  WF2_TRY(reduce_setup_device(device));
   if (g_rt.partials) {
     (void)hipFree(g_rt.partials);
     g_rt.partials = nullptr;

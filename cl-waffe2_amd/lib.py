@@ -29,6 +29,7 @@ COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")
 MAXVALUE, MINVALUE, ARGMAX, ARGMIN = 48, 49, 50, 51  # enum wf2hip_select_op
 
 EOVERLAP = -3
+EUNSUPPORTED = -4
 ECAPTURE = -6
 
 
@@ -162,6 +163,7 @@ _SIGNATURES = {
     "wf2hip_set_reduce_mode": ([C.c_int], C.c_int),
     "wf2hip_get_reduce_mode": ([], C.c_int),
     "wf2hip_reduce_add_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
+    "wf2hip_reduce_add_rows_f32_noalloc": ([_L, _L, _P, _L, _P, _L], C.c_int),
     "wf2hip_softmax_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
     "wf2hip_causal_softmax_f32": ([_L, _L, _P, _P, _F], C.c_int),
     "wf2hip_layernorm_rows_f32": ([_L, _L, _P, _P, _P, _F, _P], C.c_int),

@@ -561,6 +561,20 @@ int wf2hip_get_reduce_mode(void);
  * (base-impl/reduction.lisp:5-79). */
 int wf2hip_reduce_add_rows_f32(long rows, long cols, const float* x, long ldx,
                                float* out, long inco);
+/* The same row sums through an entry point that allocates nothing.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  Same arguments, same kernels and bit-identical results as
+ * wf2hip_reduce_add_rows_f32; the partial sums of rows that are split over
+ * several workgroups go to a 256 KiB static device array (one copy per GPU,
+ * held until the process ends) instead of a buffer the library allocates.
+ * rows * cols above WF2HIP_NOALLOC_MAX_ELEMENTS returns WF2HIP_EUNSUPPORTED.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on
+ * one GPU (two streams, two host threads) race; nothing in the array has to
+ * start at zero, each launch writes every partial sum it later reads. */
+#define WF2HIP_NOALLOC_MAX_ELEMENTS (1LL << 32)
+int wf2hip_reduce_add_rows_f32_noalloc(long rows, long cols, const float* x, long ldx,
+                                       float* out, long inco);
 /* out[r*ldo + c] <- softmax over c of x[r*ldx + c], max-subtracted.
  * One fused kernel for what !softmax composes from mean/sub/exp/sum/div
  * (source/nn/activation.lisp:126-159). */
