@@ -65,7 +65,7 @@ struct OpSin { static constexpr int kFlatU = 2; __device__ __forceinline__ float
 struct OpCos { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return cosf_(s); } };
 struct OpTanh { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return tanhf_(s); } };
 struct OpLog { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return logf_(s); } };
-struct OpExp { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return expf_(s); } };
+struct OpExp { static constexpr int kFlatU = 1; __device__ __forceinline__ float operator()(float, float s) const { return expf_(s); } };
 struct OpSqrt { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return sqrtf_(s); } };
 struct OpAbs { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return absf_(s); } };
 struct OpTan { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return tanf_(s); } };

@@ -6,19 +6,24 @@
 // cl-waffe2-simd.c:586-768).  The device versions below must stay within
 // 2 ulp of those results.
 //
-// Design: CDNA3/CDNA4 issue a binary64 FMA at the same rate as a non-packed
-// binary32 FMA, so every core does its argument reduction and the leading
-// terms of its series in binary64 and rounds to binary32 once at the end.
-// Binary64 FMAs draw much more power, though: beyond ~20 of them per element a
-// streaming kernel leaves the HBM roofline because the clock sags, so the
-// high-order remainders of exp (as used by tanh and GELU), log, sin and cos are
-// evaluated in binary32, where their rounding is below 2^-30 of the result.
-// The result is within 0.52 ulp of the exact value for every binary32 input
-// (0.507 for the functions evaluated wholly in binary64; exhaustive host runs),
-// hence within 1.52 ulp of any 1.0-ulp implementation.  Only IEEE operations and fma are
-// used (plus one reciprocal seed that is refined by a Newton step), so the
-// same header compiles for the host and a CPU build can check every binary32
-// input against libm.
+// Design: two families.
+//  * exp, log, sin, cos, tanh -- the functions of the benchmark configurations, which
+//    run over 2^26 elements at the HBM roofline -- are written in binary32 only:
+//    Cody-Waite reductions with fma, short polynomials, and double-float
+//    (head + tail) arithmetic at the few places that decide the last bit.  A
+//    streaming kernel on MI355X keeps its bandwidth with up to ~48 binary32 VALU
+//    operations per element and one 16-byte vector per thread; binary64 FMAs draw
+//    more power and pull the clock down once the load is sustained (measured: the
+//    binary64 forms of sin and tanh 76-79 % of the HBM peak, the binary32 forms
+//    80-83 %).  Error below 0.9 ulp for every binary32 input (exhaustive host runs;
+//    the bound per function is stated at its definition), hence within 2 ulp of
+//    any 1.0-ulp implementation such as SLEEF u10.
+//  * everything else does its argument reduction and the leading terms of its
+//    series in binary64 (a binary64 FMA issues at the rate of a non-packed
+//    binary32 one on CDNA3/CDNA4) and rounds once: within 0.52 ulp.
+// Only IEEE operations, fma and ldexp are used (plus one reciprocal seed that is
+// refined by a Newton step), so the same header compiles for the host and a CPU
+// build can check every binary32 input against libm.
 //
 // Coefficients come from gen_math_coeffs.py (Chebyshev fits in 60-digit
 // arithmetic).
@@ -29,6 +34,7 @@
 #if defined(__HIPCC__)
 #include <hip/hip_runtime.h>
 #define WF2_MATH_FN __device__ __forceinline__
+#define WF2_MATH_COLD static __device__ __attribute__((noinline))
 #define WF2_FMA(a, b, c) __builtin_fma((a), (b), (c))
 #define WF2_RCP_SEED(f) __builtin_amdgcn_rcpf(f)
 #define WF2_SLOW_SINF(x) sinf(x)
@@ -38,9 +44,13 @@
 #define WF2_SQRTF(x) __builtin_sqrtf(x)
 #define WF2_FAST_EXP2F(x) __builtin_amdgcn_exp2f(x)
 #define WF2_FAST_RCPF(x) __builtin_amdgcn_rcpf(x)
+#define WF2_LDEXPF(x, e) __builtin_ldexpf((x), (e))
+#define WF2_FREXP_MANT(x) __builtin_amdgcn_frexp_mantf(x)
+#define WF2_FREXP_EXP(x) __builtin_amdgcn_frexp_expf(x)
 #else
 #include <math.h>
 #define WF2_MATH_FN static inline
+#define WF2_MATH_COLD static __attribute__((noinline))
 #define WF2_FMA(a, b, c) __builtin_fma((a), (b), (c))
 #define WF2_RCP_SEED(f) (1.0f / (f))
 #define WF2_SLOW_SINF(x) ((float)sin((double)(x)))
@@ -50,6 +60,11 @@
 #define WF2_SQRTF(x) sqrtf(x)
 #define WF2_FAST_EXP2F(x) exp2f(x)
 #define WF2_FAST_RCPF(x) (1.0f / (x))
+#define WF2_LDEXPF(x, e) ldexpf((x), (e))
+static inline float wf2_frexp_mant_host(float x) { int e; return frexpf(x, &e); }
+static inline int wf2_frexp_exp_host(float x) { int e; (void)frexpf(x, &e); return e; }
+#define WF2_FREXP_MANT(x) wf2_frexp_mant_host(x)
+#define WF2_FREXP_EXP(x) wf2_frexp_exp_host(x)
 #endif
 
 namespace wf2 {
@@ -143,12 +158,49 @@ WF2_MATH_FN double exp_core_mixed(double x) {
   return WF2_FMA(s, p, s);
 }
 
+// ---- binary32 cores -----------------------------------------------------------
+// Adding 1.5 * 2^23 rounds |value| < 2^22 to the nearest integer in the fma's own
+// rounding; the integer is then the difference of the bit patterns.
+constexpr float kRoundMagic32 = 12582912.0f;
+constexpr float kLog2e32 = 1.44269502f;
+constexpr float kLn2Head32 = 0.693145751953125f;     // 16 significant bits: n * head is exact for |n| < 2^8
+constexpr float kLn2Tail32 = 1.428606765330187e-06f;
+
+// exp(r) = 1 + r + r^2 Q(r) on |r| <= 0.3475, Q of degree 5 with binary32
+// coefficients fitted one at a time (each rounded, the rest refitted): relative
+// error 1.5e-10 for exp and 4.6e-10 for expm1 before the roundings of the
+// evaluation.
+WF2_MATH_FN float exp_q32(float r) {
+  float q = 0.00019738492846954614f;
+  q = __builtin_fmaf(q, r, 0.0013933394802734256f);
+  q = __builtin_fmaf(q, r, 0.008333572186529636f);
+  q = __builtin_fmaf(q, r, 0.041666481643915176f);
+  q = __builtin_fmaf(q, r, 0.1666666567325592f);
+  return __builtin_fmaf(q, r, 0.5f);
+}
+
+// e^x, binary32 only.  x = n ln2 + r; exp(r) = 1 + w, w = r + r^2 Q(r).  The
+// roundings of r and of w (each up to a quarter ulp of the result) are recovered
+// as tails and added back with the exact remainder of 1 + w, so that one rounding
+// decides the result: error below 0.6 ulp.  Below -104 the result rounds to +0
+// and above 89 to +inf, as e^-104 and e^89 already do, so clamping is exact;
+// fmin / fmax drop a NaN operand.  ldexp rounds once into the subnormals.
+// 28 VALU operations.
 WF2_MATH_FN float expf_(float x) {
-  // Below -104 the result rounds to +0 and above 89 to +inf, as e^-104 and
-  // e^89 already do, so clamping is exact.  fmin/fmax drop a NaN operand.
-  float xc = __builtin_fminf(__builtin_fmaxf(x, -104.0f), 89.0f);  // one v_med3_f32
-  float r = (float)exp_core((double)xc);
-  return (x != x) ? x : r;
+  const float xc = __builtin_fminf(__builtin_fmaxf(x, -104.0f), 89.0f);  // one v_med3_f32
+  const float t = __builtin_fmaf(xc, kLog2e32, kRoundMagic32);
+  const float n = t - kRoundMagic32;
+  const int32_t ni = (int32_t)(bits_of(t) - bits_of(kRoundMagic32));
+  const float r1 = __builtin_fmaf(n, -kLn2Head32, xc);  // exact
+  const float r = __builtin_fmaf(n, -kLn2Tail32, r1);
+  const float rl = __builtin_fmaf(n, -kLn2Tail32, r1 - r);
+  const float r2 = r * r, q = exp_q32(r);
+  const float wh = __builtin_fmaf(r2, q, r);
+  const float wl = __builtin_fmaf(r2, q, r - wh);
+  const float y = 1.0f + wh;
+  const float yl = ((1.0f - y) + wh) + (wl + rl);
+  const float res = WF2_LDEXPF(y + yl, ni);
+  return (x != x) ? x : res;
 }
 
 // 1/d for d >= 1 in binary32 range: a binary32 seed (relative error <= 2^-22
@@ -160,19 +212,35 @@ WF2_MATH_FN double rcp_refined(double d) {
   return WF2_FMA(y, e, y);
 }
 
-// tanh(x) = expm1(2|x|) / (expm1(2|x|) + 2); saturates to 1 from |x| = 10
-// (1 - tanh(10) = 4.1e-9 < 2^-25).
-WF2_MATH_FN double tanh_core(double ax) {
-  double p, s;
-  exp_reduce_mixed(ax + ax, &p, &s);
-  double em1 = WF2_FMA(s, p, s - 1.0);
-  return em1 * rcp_refined(em1 + 2.0);
-}
-
+// tanh(x) = (E - 1) / (E + 1), E = e^{2|x|} = 2^n y, y = 1 + w, as the quotient of
+// N = y - c and D = y + c with c = 2^-n: for n = 0 the numerator is expm1(2|x|)
+// itself, so small arguments need no branch.  w is carried as head + tail (the tail
+// is the rounding error of its last fma), y, N and D are exact two-term sums, and
+// the quotient is one Newton-corrected division, so that the only full rounding is
+// the last one.  Saturates to 1 from |x| = 10 (1 - tanh(10) = 4.1e-9 < 2^-25).
+// 45 VALU operations; error below 0.75 ulp.
 WF2_MATH_FN float tanhf_(float x) {
-  double ax = __builtin_fmin(__builtin_fabs((double)x), 10.0);
-  float r = __builtin_copysignf((float)tanh_core(ax), x);
-  return (x != x) ? x : r;
+  const float a2 = 2.0f * __builtin_fminf(__builtin_fabsf(x), 10.0f);
+  const float t = __builtin_fmaf(a2, kLog2e32, kRoundMagic32);
+  const float n = t - kRoundMagic32;
+  const int32_t ni = (int32_t)(bits_of(t) - bits_of(kRoundMagic32));  // 0 .. 29
+  float r = __builtin_fmaf(n, -kLn2Head32, a2);
+  r = __builtin_fmaf(n, -kLn2Tail32, r);
+  const float r2 = r * r, q = exp_q32(r);
+  const float wh = __builtin_fmaf(r2, q, r);
+  const float wl = __builtin_fmaf(r2, q, r - wh);
+  const float c = float_of((uint32_t)(127 - ni) << 23);
+  // y = 1 + w, N = y - c, D = y + c as exact two-term sums (for n = 0, c = 1 and y >= 1:
+  // y - 1 is exact and 1 <= y orders the other sum)
+  const float yh = 1.0f + wh, yl = ((1.0f - yh) + wh) + wl;
+  const float nh = yh - c, nl = ((yh - nh) - c) + yl;
+  const float dh = yh + c, dl = ((yh - dh) + c) + yl;
+  const float y0 = WF2_FAST_RCPF(dh);
+  const float q0 = nh * y0;
+  float rho = __builtin_fmaf(-q0, dh, nh);
+  rho = __builtin_fmaf(-q0, dl, rho + nl);
+  const float res = __builtin_copysignf(__builtin_fmaf(rho, y0, q0), x);
+  return (x != x) ? x : res;
 }
 
 // log(m) for m in [sqrt(1/2), sqrt(2)): f = m - 1,
@@ -226,12 +294,39 @@ WF2_MATH_FN double log_core(double xd) {
   return WF2_FMA((double)k, kLn2, log1p_mixed(m - 1.0));
 }
 
+// log x = k ln2 + log(1 + f), x = 2^k (1 + f), 1 + f in [sqrt(1/2), sqrt(2)):
+// with s = f / (2 + f), log(1 + f) = 2 atanh(s) = 2 s + s R(s^2), and
+// 2 s = f - f^2/2 + s f^2/2 exactly, so that f, the dominant term, enters
+// unrounded: log(1 + f) = f - (h - s (h + R)), h = f^2/2 (the classical
+// arrangement of 4.4BSD's logf).  R of degree 3 in z = s^2 <= 0.0295 (relative
+// error 2.4e-11).  v_frexp_* handle subnormal arguments.  36 VALU operations;
+// error below 0.87 ulp.
 WF2_MATH_FN float logf_(float x) {
   const float inf = __builtin_inff();
-  bool ok = (x > 0.0f) && (x < inf);
-  float r = (float)log_core(ok ? (double)x : 1.0);
+  const bool ok = (x > 0.0f) && (x < inf);
+  const float xs = ok ? x : 1.0f;
+  float m = WF2_FREXP_MANT(xs);  // [0.5, 1)
+  int32_t e = WF2_FREXP_EXP(xs);
+  const bool low = m < 0.707106769f;
+  m = low ? m + m : m;
+  e = low ? e - 1 : e;
+  const float f = m - 1.0f;
+  const float k = (float)e;
+  const float d = 2.0f + f;
+  const float y0 = WF2_FAST_RCPF(d);
+  const float y = __builtin_fmaf(y0, __builtin_fmaf(-d, y0, 1.0f), y0);
+  const float s = f * y;
+  const float z = s * s;
+  float p = 0.23103581368923187f;
+  p = __builtin_fmaf(p, z, 0.2856609523296356f);
+  p = __builtin_fmaf(p, z, 0.3999979794025421f);
+  p = __builtin_fmaf(p, z, 0.6666666865348816f);
+  const float R = z * p;
+  const float h = (0.5f * f) * f;
+  const float u = __builtin_fmaf(s, h + R, k * kLn2Tail32);
+  const float r = __builtin_fmaf(k, kLn2Head32, -((h - u) - f));
   // x == +inf -> +inf; x == +-0 -> -inf; x < 0 or NaN -> NaN
-  float special = (x == inf) ? inf : ((x == 0.0f) ? -inf : __builtin_nanf(""));
+  const float special = (x == inf) ? inf : ((x == 0.0f) ? -inf : __builtin_nanf(""));
   return ok ? r : special;
 }
 
@@ -284,15 +379,64 @@ WF2_MATH_FN double trig_core(double xd, int32_t quadrant_shift) {
   return (qi & 2) ? -v : v;
 }
 
+// sin and cos in binary32 for |x| <= 128: |x| = q pi/2 + r, |r| <= pi/4, by a
+// three-term Cody-Waite reduction (pi/2 = A + B + C with 17 + 17 + 24 bits, so
+// q A is exact for q <= 82); the roundings of the second and third step are
+// recovered as a tail rl, and sin(r + rl) = sin r + rl (1 - r^2/2), cos(r + rl) =
+// cos r - rl r.  sin r = r + r^3 S(r^2), cos r = 1 - z/2 + z^2 C(z) with S of
+// degree 3 and C of degree 2 (relative errors 1.9e-10 and 1.2e-10).  Error below
+// 0.75 ulp.  From 128 on the binary64 reduction takes over (to 1e6, 0.52 ulp), then
+// the platform's routine.  41 VALU operations on the fast path.
+constexpr float kTrigFast32 = 128.0f;
+constexpr float kPio2A = 1.5707855224609375f, kPio2B = 1.0804273188114166e-05f, kPio2C = 6.07710062827671e-11f;
+
+// value of sin (shift 0) or cos (shift 1) of |x| = ax <= 128, without the sign of x
+WF2_MATH_FN float trig32(float ax, uint32_t shift) {
+  const float t = __builtin_fmaf(ax, 0.636619747f, kRoundMagic32);
+  const float q = t - kRoundMagic32;
+  const uint32_t qi = bits_of(t) + shift;  // low bits: the quadrant
+  const float r1 = __builtin_fmaf(q, -kPio2A, ax);  // exact
+  const float r2 = __builtin_fmaf(q, -kPio2B, r1);
+  const float r2l = __builtin_fmaf(q, -kPio2B, r1 - r2);
+  const float r = __builtin_fmaf(q, -kPio2C, r2);
+  const float rl = __builtin_fmaf(q, -kPio2C, r2 - r) + r2l;
+  const float z = r * r, zl = __builtin_fmaf(r, r, -z);
+  float sp = 2.8040192319167545e-06f;
+  sp = __builtin_fmaf(sp, z, -0.00019850277749355882f);
+  sp = __builtin_fmaf(sp, z, 0.008333372883498669f);
+  sp = __builtin_fmaf(sp, z, -0.1666666716337204f);
+  float cp = 2.443209450575523e-05f;
+  cp = __builtin_fmaf(cp, z, -0.0013887308305129409f);
+  cp = __builtin_fmaf(cp, z, 0.04166664555668831f);
+  // one rounding decides each value: sin = r + (small), cos = (1 + mh) + (small)
+  const float sv = r + __builtin_fmaf(r * z, sp, rl * __builtin_fmaf(z, -0.5f, 1.0f));
+  const float ci = __builtin_fmaf(z, cp, -0.5f);
+  const float mh = z * ci, ml = __builtin_fmaf(z, ci, -mh);
+  const float y = 1.0f + mh;
+  const float cv = y + (((1.0f - y) + mh) + __builtin_fmaf(-rl, r, __builtin_fmaf(-0.5f, zl, ml)));
+  const float v = (qi & 1u) ? cv : sv;
+  return float_of(bits_of(v) ^ ((qi & 2u) << 30));
+}
+
+// Arguments beyond the binary32 fast path; kept out of line so that the rare case
+// does not swell the streaming kernels (inlined four times per vector it cost them
+// two thirds of their bandwidth).
+WF2_MATH_COLD float trig_beyond(float x, int32_t quadrant_shift) {
+  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return quadrant_shift ? WF2_SLOW_COSF(x) : WF2_SLOW_SINF(x);
+  return (float)trig_core((double)x, quadrant_shift);
+}
+
 WF2_MATH_FN float sinf_(float x) {
-  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_SINF(x);
-  float r = (float)trig_core((double)x, 0);
-  return (x == 0.0f) ? x : r;  // sin(-0) = -0: the polynomial's sign of zero is not x's
+  const float ax = __builtin_fabsf(x);
+  if (__builtin_expect(!(ax <= kTrigFast32), 0)) return trig_beyond(x, 0);
+  // sin is odd: -0 stays -0
+  return float_of(bits_of(trig32(ax, 0u)) ^ (bits_of(x) & 0x80000000u));
 }
 
 WF2_MATH_FN float cosf_(float x) {
-  if (!(__builtin_fabsf(x) <= kTrigFastLimit)) return WF2_SLOW_COSF(x);
-  return (float)trig_core((double)x, 1);
+  const float ax = __builtin_fabsf(x);
+  if (__builtin_expect(!(ax <= kTrigFast32), 0)) return trig_beyond(x, 1);
+  return trig32(ax, 1u);
 }
 
 // tan = sin / cos of the reduced argument (one binary64 division); odd
@@ -442,19 +586,42 @@ WF2_MATH_FN float powf_(float x, float p) {
 }
 
 // tanh-form GELU, 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3)
-// (nn/activation.lisp:45-66), in binary64 and rounded once.  0.5 (1 + tanh u)
-// equals sigmoid(2u), evaluated with e = exp(-2|u|) in (0, 1] as 1/(1+e) for
-// u >= 0 and e/(1+e) for u < 0: no cancellation on either side.
+// (nn/activation.lisp:45-66).  0.5 (1 + tanh u) equals sigmoid(2u), evaluated
+// with E = exp(-2|u|) in (0, 1] as 1 / (1 + E) for x >= 0 and E / (1 + E) for
+// x < 0: no cancellation on either side.  a = 2|u| log2(e) = |x| (K1 + K2 x^2)
+// and its split into an integer and |p| <= 1/2 are formed in binary64 (eight
+// operations: a binary32 rounding of a would be multiplied by |a| in the left
+// tail, where the result is x e^{-2|u|}); E = 2^-a through the binary32 exp
+// polynomial, and the quotient (x or x E) / (1 + E) is one Newton-corrected
+// division against 1 + E kept as an exact two-term sum.  Error below 2 ulp
+// (exhaustive host run), far inside the reference's own node composition, whose
+// 1 + tanh u cancels on the left.  48 VALU operations.
 WF2_MATH_FN float gelu_tanh_f(float x) {
-  double xd = (double)x;
-  double u = 0.7978845608028654 * WF2_FMA(0.044715 * xd * xd, xd, xd);
-  double au = __builtin_fmin(__builtin_fabs(u), 80.0);  // e^-160 is far below 2^-30 already; keeps |n| < 2^8
-  double e = exp_core_mixed(-(au + au));
-  double num = (u >= 0.0) ? 1.0 : e;
-  float r = (float)(xd * num * rcp_refined(1.0 + e));
-  // x = -inf: the limit is -0 (x e^{2u} -> 0), not -inf * tiny.
-  r = (x == -__builtin_inff()) ? -0.0f : r;
-  return (x != x) ? x : r;
+  const double K1 = 2.3022081981443249;   // 2 sqrt(2/pi) log2(e)
+  const double K2 = 0.10294323958002349;  // K1 * 0.044715
+  const float Ln2h = 0.6931471824645996f, Ln2l = -1.9046542121259336e-09f;
+  // beyond |x| = 16, E is 0 in binary32; fmin / fmax drop a NaN, which the last line restores
+  const float xc = __builtin_fminf(__builtin_fmaxf(x, -16.0f), 16.0f);
+  const double xd = (double)xc;
+  const double a = __builtin_fabs(xd) * WF2_FMA(K2, xd * xd, K1);  // <= 460
+  const double td = a + kRoundMagic;
+  const int32_t ni = (int32_t)(uint32_t)bits_of(td);
+  const float p = (float)(a - (td - kRoundMagic));  // a = n + p, |p| <= 1/2
+  const float r = __builtin_fmaf(p, -Ln2l, p * -Ln2h);
+  const float w = __builtin_fmaf(r * r, exp_q32(r), r);
+  const float E = WF2_LDEXPF(1.0f + w, -ni);
+  const float D = 1.0f + E, Dl = (1.0f - D) + E;  // exact two-term sum
+  // the numerator without its factor 2^-n, which is applied last: x E may be a normal
+  // number where E alone is subnormal
+  const bool right = xc >= 0.0f;
+  const float num = right ? xc : __builtin_fmaf(xc, w, xc);
+  const float y0 = WF2_FAST_RCPF(D);
+  const float q0 = num * y0;
+  const float q = __builtin_fmaf(__builtin_fmaf(-q0, Dl, __builtin_fmaf(-q0, D, num)), y0, q0);
+  const float res = WF2_LDEXPF(q, right ? 0 : -ni);
+  // |x| >= 16 (or NaN): x on the right, -0 on the left (x e^{2u} underflows)
+  const float far = (x != x) ? x : __builtin_fmaxf(x, -0.0f);
+  return (__builtin_fabsf(x) < 16.0f) ? res : far;
 }
 
 // The same function in binary32 for gemm epilogues, whose inputs already carry
