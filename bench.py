@@ -324,12 +324,16 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     R, Cn = 8192, 4096
     x0 = normal([R, Cn])
     ring = ring_of(lambda: (clone(x0), T([R, 1])), 4 * R * Cn)
-    measure("row sum (8192,4096) as !sum composes it", ring,
-            lambda s: F.sum(s[0], axis=1, out=s[1], keepdims=True), 4 * R * Cn + 12 * R,
-            note="zero fill of out + accumulation into the stride-0 view")
+    measure("row sum (8192,4096), !sum as one node", ring,
+            lambda s: F.sum(s[0], axis=1, out=s[1], keepdims=True), 4 * R * Cn + 4 * R,
+            note="HIP-Sum-Node: out overwritten, no zero fill")
+    ring = ring_of(lambda: (clone(x0), T([R, 1])), 4 * R * Cn)
+    measure("row sum (8192,4096), node for node", ring,
+            lambda s: F.sum_composed(s[0], axis=1, out=s[1], keepdims=True), 4 * R * Cn + 12 * R,
+            note="the reference's composition: zero fill of out (MulNode by 0) + AddNode into the stride-0 view")
     ring = ring_of(lambda: (clone(x0), T([1, 1])), 4 * R * Cn)
-    measure("full sum (8192,4096)", ring, lambda s: F.sum(s[0], axis=True, out=s[1], keepdims=True),
-            4 * R * Cn, note="two launches: partial sums per block, then their sum")
+    measure("full sum (8192,4096), !sum as one node", ring, lambda s: F.sum(s[0], axis=True, out=s[1], keepdims=True),
+            4 * R * Cn, note="two launches: partial sums per workgroup, then their sum")
     del x0
     R, Cn = 32768, 1024
     x0 = normal([R, Cn], 3.0)

@@ -445,8 +445,48 @@ def _axes(axis, ndim: int) -> list[int]:
     return sorted(a + ndim if a < 0 else a for a in axis)
 
 
+# Mirrors cl-waffe2/vm.nodes:*enable-symbolic-path* (vm/nodes/symbolic.lisp:118-131):
+# when true, !sum / !mean on :float tensors build the one-node HIP-Sum-Node instead of
+# the reference's three-node composition, as the define-bypass rules of the Lisp glue do.
+ENABLE_SYMBOLIC_PATH = True
+
+
+def _broadcast_view_of(out: HIPTensor, shape, axes) -> HIPTensor:
+    """`out` viewed ``(:broadcast n)`` on the reduced axes (reduction.lisp:65-69); existing
+    (non-broadcast) views on `out` stay intact."""
+    from .tensor import parse_view
+    view_args = [(":broadcast", shape[i]) if (i in axes and shape[i] != 1) else True
+                 for i in range(len(shape))]
+    views = list(out.views)
+    for i, s in enumerate(view_args):
+        if s is not True:
+            views[i] = parse_view(out.orig_shape[i], out.views[i], s)
+    return HIPTensor(out.orig_shape, vec=out.vec, strides=out.stride, views=views,
+                     offset=out.initial_offset, dtype=out.dtype)
+
+
 def sum(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = False,  # noqa: A001
         div_by=None) -> HIPTensor:
+    """``(!sum tensor :axis :-> :keepdims)``.  On :float tensors with the symbolic path
+    enabled this is ONE node (HIP-Sum-Node: `out` overwritten with the sums, divided by
+    ``div_by`` for !mean), whose bits equal those of the reference's composition on a
+    zeroed `out`; otherwise the composition itself (`sum_composed`)."""
+    if not (ENABLE_SYMBOLIC_PATH and x.dtype == "float" and (out is None or out.dtype == "float")):
+        return sum_composed(x, axis=axis, out=out, keepdims=keepdims, div_by=div_by)
+    axes = _axes(axis, x.ndim)
+    shape = list(x.shape)
+    out_shape = [1 if i in axes else n for i, n in enumerate(shape)]
+    if out is None:
+        out = HIPTensor(out_shape, dtype=x.dtype, initial_element=None)  # overwritten: no zero fill
+    elif out.shape != out_shape:
+        raise ValueError(f"!sum: the given out's shape is {out.shape}, but expected: {out_shape}")
+    out_bc = _broadcast_view_of(out, shape, axes)
+    nodes.forward("HIP-Sum-Node", out_bc, x, 1.0 if div_by is None else float(div_by))
+    return out_bc if keepdims else out
+
+
+def sum_composed(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = False,
+                 div_by=None) -> HIPTensor:
     """``(!sum tensor :axis :-> :keepdims)`` exactly as
     ``base-impl/reduction.lisp:5-79`` composes it: zero-fill ``out`` by
     multiplying with 0, view it ``(:broadcast n)`` on the reduced axes, AddNode
@@ -459,16 +499,7 @@ def sum(x: HIPTensor, axis=True, out: HIPTensor | None = None, keepdims: bool = 
     elif out.shape != out_shape:
         raise ValueError(f"!sum: the given out's shape is {out.shape}, but expected: {out_shape}")
     out = mul_(out, 0.0)  # A*=scal out 0  (reduction.lisp:63)
-    view_args = [(":broadcast", shape[i]) if (i in axes and shape[i] != 1) else True
-                 for i in range(x.ndim)]
-    # keep existing (non-broadcast) views on `out` intact: only re-view reduced axes
-    from .tensor import parse_view
-    views = list(out.views)
-    for i, s in enumerate(view_args):
-        if s is not True:
-            views[i] = parse_view(out.orig_shape[i], out.views[i], s)
-    out_bc = HIPTensor(out.orig_shape, vec=out.vec, strides=out.stride, views=views,
-                       offset=out.initial_offset, dtype=out.dtype)
+    out_bc = _broadcast_view_of(out, shape, axes)
     add_(out_bc, x)  # A+=B out* tensor: accumulation into a stride-0 destination
     result = out_bc if keepdims else out
     if div_by is not None:

@@ -162,6 +162,7 @@ _SIGNATURES = {
     "wf2hip_unary_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F], C.c_int),
     "wf2hip_set_reduce_mode": ([C.c_int], C.c_int),
     "wf2hip_get_reduce_mode": ([], C.c_int),
+    "wf2hip_sum_nd": ([C.POINTER(View2), _P, _P, C.c_float], C.c_int),
     "wf2hip_reduce_add_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
     "wf2hip_reduce_add_rows_f32_noalloc": ([_L, _L, _P, _L, _P, _L], C.c_int),
     "wf2hip_softmax_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),

@@ -34,6 +34,7 @@ NODE_NAMES = (
     "Where-Operation-Node", "Compare-Operation-Node",
     "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
     "Im2ColNode", "Col2ImNode",
+    "HIP-Sum-Node",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -289,6 +290,18 @@ def _unfold_args(x_shape, col_shape, stride, padding, dilation):
     if (N, Cc) != (n2, c2):
         raise ValueError(f"X {x_shape} and Col {col_shape} disagree on N, C")
     return [N, Cc, H, W, ho, wo, kh, kw, padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1]]
+
+
+@define_impl("HIP-Sum-Node", HIPTensor, _only_float)
+def _sum_node(out: HIPTensor, x: HIPTensor, divisor: float = 1.0) -> HIPTensor:
+    """``Out[~] X[~] -> Out[~]`` with `out` viewed ``(:broadcast n)`` on the reduced axes:
+    out <- sum of x over those axes / divisor, overwriting `out`.  One node for the
+    MulNode-by-0, AddNode and DivNode of ``!sum`` / ``!mean``
+    (``base-impl/reduction.lisp:5-136``); its backward is theirs (the gradient
+    broadcast over the reduced axes, divided by `divisor`)."""
+    v = view2(out, x)
+    _lib.check(_lib.get().wf2hip_sum_nd(C.byref(v), C.c_void_p(out.ptr), C.c_void_p(x.ptr), float(divisor)))
+    return out
 
 
 @define_impl("Im2ColNode", HIPTensor, _only_float)

@@ -556,6 +556,16 @@ int wf2hip_set_reduce_mode(int mode);
 int wf2hip_get_reduce_mode(void);
 
 /* ---- reductions and softmax as direct entry points ---------------------- */
+/* a <- (sum of b over the axes on which a has stride 0 and an extent above 1)
+ * / divisor, one node for what (!sum x :axis ..) and (!mean x :axis ..) compose
+ * from a zero fill (MulNode by 0), AddNode into the (:broadcast n) view of
+ * `out` and, for !mean, DivNode by the element count
+ * (base-impl/reduction.lisp:5-79 and :81-136).  `a` is overwritten: its old
+ * content is not read, so it needs no zero fill.  The bits are those of the
+ * composition on a zeroed `out`: the sum rounded to binary32 once (reduce mode
+ * 0) or added in the reference's sequential binary32 order (reduce mode 1),
+ * then an IEEE binary32 division by `divisor` (pass 1 for !sum). */
+int wf2hip_sum_nd(const wf2hip_view2* v, float* a, const float* b, float divisor);
 /* out[r*inco] <- out[r*inco] + sum_c x[r*ldx + c], r < rows, c < cols.
  * What (!sum x :axis -1) lowers to after its zero-fill
  * (base-impl/reduction.lisp:5-79). */

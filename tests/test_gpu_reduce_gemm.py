@@ -143,6 +143,69 @@ def test_reduce_shapes(gpu, shape, axis):
     assert np.all(np.abs(gotm - want / cnt) <= REL * mag / cnt + 1e-7)
 
 
+@pytest.mark.parametrize("shape, axis", [
+    ((8192, 512), 1), ((64, 40000), 1), ((3, 70001), -1), ((1, 1 << 21), True), ((700, 300), True),
+    ((3000, 768), 0), ((17, 1000), 0), ((64, 50, 260), (0, 1)), ((12, 33, 64), 1), ((5, 7, 9, 11), (1, 3)),
+    ((100, 1), 1), ((1, 100), 1), ((6, 1, 8), 1), ((262144, 16), 1),
+])
+def test_one_node_sum_equals_the_composition(gpu, shape, axis):
+    """!sum / !mean as ONE node (HIP-Sum-Node, wf2hip_sum_nd) against the reference's
+    composition (zero fill by MulNode, AddNode into the broadcast view, DivNode) on the
+    same input: bit-identical in both reduce modes, also when `out` holds stale NaNs
+    (the one-node form never reads it), with and without keepdims."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(shape).astype(np.float32)
+    dx = F.from_numpy(x)
+    assert F.ENABLE_SYMBOLIC_PATH
+    for mode in (0, 1):
+        if mode == 1 and x.size > (1 << 21):
+            continue
+        W.lib.check(W.lib.get().wf2hip_set_reduce_mode(mode))
+        try:
+            want = F.sum_composed(dx, axis=axis).numpy()
+            assert_bit_equal(F.sum(dx, axis=axis).numpy(), want, f"sum {shape} {axis} mode {mode}")
+            stale = F.from_numpy(np.full(want.shape, np.nan, np.float32))
+            got = F.sum(dx, axis=axis, out=stale, keepdims=True)
+            assert got.shape == list(shape)
+            assert_bit_equal(stale.numpy(), want, "sum into a NaN-filled out")
+            n = x.size // want.size
+            wantm = F.sum_composed(dx, axis=axis, div_by=float(n)).numpy()
+            assert_bit_equal(F.mean(dx, axis=axis).numpy(), wantm, f"mean {shape} {axis} mode {mode}")
+        finally:
+            W.lib.check(W.lib.get().wf2hip_set_reduce_mode(0))
+    ref = x.astype(np.float64).sum(axis=None if axis is True else axis, keepdims=True)
+    mag = np.abs(x).astype(np.float64).sum(axis=None if axis is True else axis, keepdims=True)
+    assert np.all(np.abs(F.sum(dx, axis=axis).numpy() - ref) <= REL * mag)
+
+
+def test_one_node_sum_on_views_and_switch(gpu):
+    """Sliced sources, an `out` that is itself a view, and the switch back to the
+    composition (ENABLE_SYMBOLIC_PATH, the mirror of *enable-symbolic-path*)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((300, 520)).astype(np.float32)
+    v = F.from_numpy(X).view((10, 290), (3, 515))
+    assert_bit_equal(F.sum(v, axis=1).numpy(), F.sum_composed(v, axis=1).numpy(), "sliced rows")
+    assert_bit_equal(F.sum(v, axis=0).numpy(), F.sum_composed(v, axis=0).numpy(), "sliced columns")
+    big = F.from_numpy(np.full((280, 4), 7.0, np.float32))
+    out = big.view(True, (2, 3))
+    F.sum(v, axis=1, out=out)
+    want = big.numpy().copy()
+    assert np.all(want[:, [0, 1, 3]] == 7.0)  # the neighbours of the viewed column are untouched
+    assert_bit_equal(want[:, 2:3], F.sum_composed(v, axis=1).numpy(), "out as a view")
+    F.ENABLE_SYMBOLIC_PATH = False
+    try:
+        assert_bit_equal(F.sum(v, axis=1).numpy(), F.sum_composed(v, axis=1).numpy(), "composition")
+    finally:
+        F.ENABLE_SYMBOLIC_PATH = True
+    # integer and :double tensors keep the composition (HIP-Sum-Node is :float only)
+    xi = F.from_numpy(np.arange(24, dtype=np.int32).reshape(4, 6), dtype="int32")
+    assert F.sum(xi, axis=1).numpy().ravel().tolist() == [15, 51, 87, 123]
+
+
 def test_accumulate_adds_to_existing_value(gpu):
     """AddNode into a stride-0 destination is x += sum(y), not x = sum(y)."""
     W = gpu
