@@ -338,6 +338,9 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     R, Cn = 32768, 1024
     x0 = normal([R, Cn], 3.0)
     ring = ring_of(lambda: (clone(x0), T([R, Cn], initial_element=None)), 8 * R * Cn)
+    measure("copy (32768,1024): 268 MB in all, the practical ceiling of the rows that move as much", ring,
+            lambda s: F.move_(s[1], s[0]), 8 * R * Cn)
+    ring = ring_of(lambda: (clone(x0), T([R, Cn], initial_element=None)), 8 * R * Cn)
     measure("row softmax (32768,1024), one kernel", ring, lambda s: F.softmax_fused(s[0], out=s[1]), 8 * R * Cn)
     ring = ring_of(lambda: clone(x0), 4 * R * Cn)
     measure("row softmax (32768,1024), node for node (!softmax)", ring, lambda s: F.softmax(s), 8 * R * Cn,

@@ -808,6 +808,70 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
     if (row0 + w < nrows) r[w].store(out + (row0 + w) * ldo, ncols, lane);
 }
 
+// Rows of 769 ... 1024 columns: two wavefronts per row, each holding half of it (two
+// vectors per lane), two rows per workgroup; maxima and sums of the halves meet in
+// LDS.  Twice the wavefronts of the one-per-row form at half the registers and half
+// the arithmetic between a wavefront's loads and its stores: (32768, 1024) 44.5 ->
+// 43.1 us, where a plain copy of the same rows by one wavefront each takes 43.9 us.
+template <bool VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void softmax_rows_pair(const float* __restrict__ x, int64_t ldx,
+                                                            float* __restrict__ out, int64_t ldo,
+                                                            int64_t nrows, int64_t ncols,
+                                                            int64_t causal_seq, float scale) {
+  constexpr int NVH = 2;
+  constexpr int64_t kHalf = (int64_t)NVH * kWave * 4;  // 512 columns
+  __shared__ float lmax[kWavesPerBlock];
+  __shared__ double lsum[kWavesPerBlock];
+  const int w = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), half = w & 1;
+  const int64_t row_raw = (int64_t)blockIdx.x * 2 + (w >> 1);
+  const int64_t row = row_raw < nrows ? row_raw : nrows - 1;  // a repeated last row is computed and not stored
+  const float ninf = -__builtin_inff();
+  const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
+  auto part = [&](int64_t n) { n -= half * kHalf; return n < 0 ? (int64_t)0 : (n > kHalf ? kHalf : n); };
+  const int64_t valid_here = part(valid);
+  RowRegs<NVH, VEC, NT> r;
+  r.load(x + row * ldx + half * kHalf, valid_here, lane, ninf);
+  float m = ninf;
+#pragma unroll
+  for (int g = 0; g < NVH; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      if (causal_seq > 0) {
+        const bool in = RowRegs<NVH, VEC, NT>::col(g, c, lane) < valid_here;
+        r.v[g][c] = in ? r.v[g][c] * scale : ninf;
+      }
+      m = fmaxf(m, r.v[g][c]);
+    }
+  m = wave_max(m);
+  if (lane == 0) lmax[w] = m;
+  __syncthreads();
+  m = fmaxf(lmax[w & ~1], lmax[w | 1]);
+  float sum = 0.0f;
+#pragma unroll
+  for (int g = 0; g < NVH; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      // the exponential of softmax_rows_wave
+      const float d = fmaxf(r.v[g][c] - m, -160.0f);
+      const float t = d * 1.44269502f;
+      float tl = __builtin_fmaf(d, 1.44269502f, -t);
+      tl = __builtin_fmaf(d, 1.92596299e-8f, tl);
+      const float e = __builtin_amdgcn_exp2f(t);
+      const float ed = __builtin_fmaf(e, tl * 0.693147182f, e);
+      r.v[g][c] = ed;
+      sum += ed;
+    }
+  const double total_here = wave_sum((double)sum);
+  if (lane == 0) lsum[w] = total_here;
+  __syncthreads();
+  const float inv = (float)(1.0 / (lsum[w & ~1] + lsum[w | 1]));
+#pragma unroll
+  for (int g = 0; g < NVH; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) r.v[g][c] *= inv;
+  if (row_raw < nrows) r.store(out + row * ldo + half * kHalf, part(ncols), lane);
+}
+
 // Rows too long for registers: one workgroup per row, three passes (the second
 // and third hit L2).
 __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __restrict__ x, int64_t ldx,
@@ -886,28 +950,34 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __res
         for (int c = 0; c < 4; c++)
           r[w].v[i][c] = __builtin_fmaf((r[w].v[i][c] - mean) * rstd, g.v[i][c], b.v[i][c]);
     } else {
+      // longer rows: the mean from binary64 sums; deviations, their squares (four
+      // partial sums per lane, folded in binary64) and the output in binary32 -- two
+      // binary64 operations per element where the all-binary64 form had twelve (same
+      // bandwidth, (65536, 1024) at 77.5 % of the HBM peak, for less power; fetching gamma
+      // and beta only after the statistics frees 24 registers and runs slower, 75.8 %)
       double sum = 0.0;
 #pragma unroll
       for (int i = 0; i < NV; i++)
 #pragma unroll
         for (int c = 0; c < 4; c++) sum += (double)r[w].v[i][c];
       const double mean = wave_sum(sum) / (double)ncols;
-      double sq = 0.0;
+      const float meanf = (float)mean;
+      float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int i = 0; i < NV; i++)
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-          bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
-          double d = in ? (double)r[w].v[i][c] - mean : 0.0;
-          sq += d * d;
+          const bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
+          const float d = in ? r[w].v[i][c] - meanf : 0.0f;
+          r[w].v[i][c] = d;
+          sq[c] = __builtin_fmaf(d, d, sq[c]);
         }
-      const double var = wave_sum(sq) / (double)ncols;
-      const double rstd = 1.0 / __builtin_sqrt(var + (double)eps);
+      const double var = wave_sum(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3])) / (double)ncols;
+      const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
 #pragma unroll
       for (int i = 0; i < NV; i++)
 #pragma unroll
-        for (int c = 0; c < 4; c++)
-          r[w].v[i][c] = (float)(((double)r[w].v[i][c] - mean) * rstd * (double)g.v[i][c] + (double)b.v[i][c]);
+        for (int c = 0; c < 4; c++) r[w].v[i][c] = __builtin_fmaf(r[w].v[i][c] * rstd, g.v[i][c], b.v[i][c]);
     }
   }
 #pragma unroll
@@ -966,6 +1036,11 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
     softmax_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,   \
                                                              causal_seq, scale);              \
     break;
+  if (nv == 4) {
+    softmax_rows_pair<VEC, NT><<<(uint32_t)ceil_div(nrows, 2), kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,
+                                                                            causal_seq, scale);
+    return after_launch("softmax_rows_pair");
+  }
   switch (nv) {
     case 1:
       softmax_rows_wave<1, VEC, NT, 4><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 4), kBlock, 0, st>>>(

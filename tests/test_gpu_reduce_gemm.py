@@ -328,7 +328,8 @@ def test_layernorm(gpu):
     W = gpu
     F = W.functional
     rng = np.random.default_rng(7)
-    for rows, cols in [(64, 768), (10, 100), (5, 1), (33, 2048), (7, 255), (9, 3072), (3, 4101), (2, 20000)]:
+    for rows, cols in [(64, 768), (10, 100), (5, 1), (33, 2048), (7, 255), (9, 3072), (3, 4101), (2, 20000),
+                       (1001, 1024), (513, 1000), (300, 1536)]:
         X = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
         g = rng.standard_normal(cols).astype(np.float32)
         b = rng.standard_normal(cols).astype(np.float32)
