@@ -11,6 +11,7 @@
 #include <mutex>
 #include <stdlib.h>
 #include <string.h>
+#include <iterator>
 #include <unordered_map>
 
 #include "wf2_common.h"
@@ -51,16 +52,21 @@ int require_init() {
 // runs on one stream, so a recycled block's new user is ordered after its old
 // one.  hipFree (which does synchronise) only happens on trim/shutdown or when
 // the device is out of memory.
-// A captured graph keeps the blocks its kernels were recorded with: blocks
-// freed while capturing are parked here (re-usable by later allocations of the
-// same capture, since a replay preserves the recorded order) and only return to
-// the pool when the graph is destroyed.
+// A captured graph keeps the blocks its kernels were recorded with: every block
+// handed out during a capture is registered to that graph, and when such a block is
+// freed -- during the capture or at any time after it, e.g. when the host's collector
+// finalises a result it dropped -- it is parked in the graph's `held` list instead of
+// the idle pool.  Parked blocks are re-usable by later allocations of the same capture
+// (a replay preserves the recorded order) and only return to the pool when the graph
+// is destroyed: until then every replay still writes into them, and an eager
+// allocation that received one would be silently overwritten.
 struct Graph {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   std::multimap<size_t, void*> held;
 };
 static Graph* g_capture = nullptr;  // non-null between graph_begin and graph_end
+static std::unordered_map<void*, Graph*> g_graph_blocks;  // block -> the live graph recorded with it (guarded by g_pool.mu)
 
 struct Pool {
   std::mutex mu;
@@ -103,6 +109,7 @@ static int pool_alloc(void** ptr, size_t bytes) {
       *ptr = it->second;
       g_pool.idle.erase(it);
       g_pool.idle_bytes -= cls;
+      if (g_capture) g_graph_blocks[*ptr] = g_capture;
       return 0;
     }
   }
@@ -135,7 +142,13 @@ static int pool_free(void* ptr) {
   if (it == g_pool.size_of.end())
     return fail(WF2HIP_EINVAL, "wf2hip_free: %p was not allocated by wf2hip_malloc", ptr);
   if (g_capture) {
+    g_graph_blocks[ptr] = g_capture;  // also a block from before the capture: its last use may be recorded
     g_capture->held.emplace(it->second, ptr);
+    return 0;
+  }
+  auto owner = g_graph_blocks.find(ptr);
+  if (owner != g_graph_blocks.end()) {
+    owner->second->held.emplace(it->second, ptr);
     return 0;
   }
   if (g_pool.enabled) {
@@ -415,9 +428,16 @@ WF2_API int wf2hip_graph_destroy(void* graph) {
   if (g->graph) (void)hipGraphDestroy(g->graph);
   {
     std::lock_guard<std::mutex> lock(g_pool.mu);
+    for (auto it = g_graph_blocks.begin(); it != g_graph_blocks.end();)
+      it = it->second == g ? g_graph_blocks.erase(it) : std::next(it);
     for (auto& kv : g->held) {
-      g_pool.idle.emplace(kv.first, kv.second);
-      g_pool.idle_bytes += kv.first;
+      if (g_pool.enabled) {
+        g_pool.idle.emplace(kv.first, kv.second);
+        g_pool.idle_bytes += kv.first;
+      } else {
+        g_pool.size_of.erase(kv.second);
+        (void)hipFree(kv.second);
+      }
     }
   }
   delete g;

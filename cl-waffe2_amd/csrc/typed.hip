@@ -1056,11 +1056,40 @@ using namespace wf2;
     default: return fail(WF2HIP_EINVAL, "unknown element type %d (:float has its own entry points)", dtype); \
   }
 
+static size_t dtype_width(int dtype) {
+  switch (dtype) {
+    case WF2HIP_F64: return 8;
+    case WF2HIP_I32: case WF2HIP_U32: return 4;
+    case WF2HIP_I16: case WF2HIP_U16: return 2;
+    case WF2HIP_I8: case WF2HIP_U8: return 1;
+    default: return 0;
+  }
+}
+
 WF2_API int wf2hip_binary_1d_typed(int dtype, int op, long n, void* x, long incx, const void* y, long incy) {
   WF2_TRY(require_init());
   if (n < 0) return fail(WF2HIP_EINVAL, "negative length");
   if (n == 0) return 0;
   if (!x || !y) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  // The kernels read y while other lanes write x.  Two runs over one buffer are only safe when
+  // they are the same run (x <- x op x); anything else depends on the order of the writes, which
+  // the N-D entry point refuses as well.
+  {
+    const size_t width = dtype_width(dtype);
+    if (width == 0) return fail(WF2HIP_EINVAL, "unknown element type %d (:float has its own entry points)", dtype);
+    auto span = [&](const void* base, long inc, uintptr_t* lo, uintptr_t* hi) {
+      const int64_t reach = (int64_t)(n - 1) * inc * (int64_t)width;
+      const uintptr_t b = (uintptr_t)base;
+      *lo = reach < 0 ? b + reach : b;
+      *hi = (reach < 0 ? b : b + reach) + width;
+    };
+    uintptr_t xlo, xhi, ylo, yhi;
+    span(x, incx, &xlo, &xhi);
+    span(y, incy, &ylo, &yhi);
+    const bool same_run = x == y && incx == incy;
+    if (xlo < yhi && ylo < xhi && !same_run)
+      return fail(WF2HIP_EOVERLAP, "in-place op between overlapping runs of one buffer; copy one operand first");
+  }
   WF2_FOR_DTYPE(dtype, return dispatch_1d<T>(op, n, (T*)x, incx, (const T*)y, incy, true));
 }
 

@@ -70,13 +70,17 @@ fp32 tensors resident in the HBM of an AMD MI355X; kernels come from libwaffe2-h
             (when (and initial-element (not (zerop initial-element)))
               (if (eql dtype :float)
                   (check (wf2hip-fill-f32 (device-buffer-pointer buffer) n (coerce initial-element 'single-float)))
-                  ;; the other dtypes: one element across PCIe, then a stride-0 move spreads it
+                  ;; the other dtypes: one element across PCIe into a buffer of its own, then a
+                  ;; stride-0 move spreads it (source and destination must not be one buffer: the
+                  ;; kernel reads the source while other lanes write the destination, and the
+                  ;; library refuses overlapping runs)
                   (multiple-value-bind (ctype bytes code) (dtype-info dtype)
-                    (with-foreign-object (host ctype)
-                      (setf (mem-ref host ctype) (coerce initial-element (dtype->lisp-type dtype)))
-                      (check (wf2hip-memcpy-h2d (device-buffer-pointer buffer) host bytes)))
-                    (check (wf2hip-binary-1d-typed code +move+ n (device-buffer-pointer buffer) 1
-                                                   (device-buffer-pointer buffer) 0)))))
+                    (let ((one (make-device-buffer 1 :zero nil :dtype dtype)))
+                      (with-foreign-object (host ctype)
+                        (setf (mem-ref host ctype) (coerce initial-element (dtype->lisp-type dtype)))
+                        (check (wf2hip-memcpy-h2d (device-buffer-pointer one) host bytes)))
+                      (check (wf2hip-binary-1d-typed code +move+ n (device-buffer-pointer buffer) 1
+                                                     (device-buffer-pointer one) 0))))))
             (setf (tensor-vec tensor) buffer))))))
 
 (defun tensor-device-pointer (tensor &optional (offset 0))

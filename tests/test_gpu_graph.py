@@ -97,3 +97,32 @@ def test_capture_rules(gpu):
     assert lib.wf2hip_graph_end(C.byref(h)) == W.lib.ECAPTURE   # nothing to end
     # the library still works afterwards
     assert F.add(a, a).numpy()[0, 0] == 2.0
+
+
+def test_block_dropped_after_the_capture_stays_with_the_graph(gpu):
+    """A result allocated during a capture and dropped after it (a host collector
+    finalising it at any later time) must not go back to the pool while the graph
+    lives: the next eager allocation of that size would receive the block every
+    replay still writes into."""
+    W = gpu
+    F = W.functional
+    n = 3 << 18  # its own size class, so that the pool holds exactly the blocks of this test
+    x = F.from_numpy(np.full(n, 1.0, np.float32))
+    warm = F.exp(x)          # the pool learns the size
+    W.lib.synchronize()
+    del warm
+    with W.lib.Graph() as g:
+        out = F.exp(x)       # served from the idle pool during the capture
+    g.launch()
+    W.lib.synchronize()
+    idle_before = W.lib.get().wf2hip_pool_idle_bytes()
+    del out                  # dropped after the capture
+    assert W.lib.get().wf2hip_pool_idle_bytes() == idle_before, "the block went back to the idle pool"
+    fresh = W.HIPTensor([n], initial_element=None)
+    F.move_(fresh, F.from_numpy(np.full(n, 7.0, np.float32)))
+    for _ in range(3):
+        g.launch()
+    W.lib.synchronize()
+    assert np.all(fresh.numpy() == 7.0), "a replay wrote into a tensor allocated after the capture"
+    g.destroy()
+    assert W.lib.get().wf2hip_pool_idle_bytes() > idle_before  # the parked block is back

@@ -213,3 +213,28 @@ def test_accumulation_into_broadcast_destinations(gpu, dtype):
         else:
             want = (base.astype(np.int64) - A[1].astype(np.int64).sum(axis=0, keepdims=True)).astype(npt)
             np.testing.assert_array_equal(dst.storage_numpy().reshape(1, 41), want)
+
+
+@pytest.mark.parametrize("dtype", ["double", "int32", "uint8"])
+def test_1d_entry_refuses_overlapping_runs(gpu, dtype):
+    """x <- x op y reads y while other lanes write x: two different runs over one buffer
+    are refused (as the N-D entry point refuses them); a stride-0 source in a buffer of
+    its own, the way a non-:float tensor is filled with its initial element, is fine, and
+    so is the same run on both sides (x <- x + x)."""
+    W = gpu
+    lib = W.lib.get()
+    code = W.lib.DTYPE_CODES[dtype]
+    npt = {"double": np.float64, "int32": np.int32, "uint8": np.uint8}[dtype]
+    n = 5000
+    dx = W.HIPTensor.from_numpy(np.arange(n) % 50, dtype=dtype)
+    for op in (W.lib.MOVE, W.lib.ADD):
+        rc = lib.wf2hip_binary_1d_typed(code, op, n, C.c_void_p(dx.ptr), 1, C.c_void_p(dx.ptr), 0)
+        assert rc == W.lib.EOVERLAP
+    item = np.dtype(npt).itemsize
+    assert lib.wf2hip_binary_1d_typed(code, W.lib.ADD, n - 1, C.c_void_p(dx.ptr), 1,
+                                      C.c_void_p(dx.ptr + item), 1) == W.lib.EOVERLAP
+    one = W.HIPTensor.from_numpy(np.array([7]), dtype=dtype)
+    W.lib.check(lib.wf2hip_binary_1d_typed(code, W.lib.MOVE, n, C.c_void_p(dx.ptr), 1, C.c_void_p(one.ptr), 0))
+    assert np.all(dx.numpy() == 7)
+    W.lib.check(lib.wf2hip_binary_1d_typed(code, W.lib.ADD, n, C.c_void_p(dx.ptr), 1, C.c_void_p(dx.ptr), 1))
+    assert np.all(dx.numpy() == 14)
