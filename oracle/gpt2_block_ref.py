@@ -41,3 +41,33 @@ def block_forward(x, p, n_head, eps=1e-5, dtype=np.float64):
     h2 = layer_norm(x1, p["ln2_g"], p["ln2_b"], eps)
     m = gelu(h2 @ p["w_fc"] + p["b_fc"]) @ p["w_proj"] + p["b_proj"]
     return x1 + m
+
+
+def block_forward_with_scale(x, p, n_head, eps=1e-5):
+    """The float64 block forward and, per output element, the magnitude the last products
+    of each residual branch sum over: |x| + |ctx| |W_o| + |gelu(..)| |W_proj| (+ biases).
+    An implementation whose products are each within r * sum |a||b| of the exact ones is
+    within about r times this of the exact output: the two last products contribute exactly
+    that, and what the earlier ones pass on arrives through sums of 768 to 3072 terms of
+    either sign and stays well below it (a worst-case propagation, every term aligned, is
+    five orders of magnitude above what any arithmetic produces and tests nothing).
+    One sequence at a time: the float64 score tensors of all eight would be gigabytes."""
+    f8 = np.float64
+    P = {k: v.astype(f8) for k, v in p.items()}
+    outs, scales = [], []
+    for xs in x.astype(f8):
+        T, D = xs.shape
+        hd = D // n_head
+        h = layer_norm(xs, P["ln1_g"], P["ln1_b"], eps)
+        qkv = h @ P["w_qkv"] + P["b_qkv"]
+        q, k, v = (qkv[:, i * D:(i + 1) * D].reshape(T, n_head, hd).transpose(1, 0, 2) for i in range(3))
+        s = (q @ k.transpose(0, 2, 1)) / np.sqrt(hd)
+        s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+        e = np.exp(s - s.max(axis=-1, keepdims=True))
+        ctx = ((e / e.sum(axis=-1, keepdims=True)) @ v).transpose(1, 0, 2).reshape(T, D)
+        x1 = xs + ctx @ P["w_o"] + P["b_o"]
+        a = gelu(layer_norm(x1, P["ln2_g"], P["ln2_b"], eps) @ P["w_fc"] + P["b_fc"])
+        outs.append(x1 + a @ P["w_proj"] + P["b_proj"])
+        scales.append(np.abs(xs) + np.abs(ctx) @ np.abs(P["w_o"]) + np.abs(P["b_o"]) +
+                      np.abs(a) @ np.abs(P["w_proj"]) + np.abs(P["b_proj"]))
+    return np.stack(outs), np.stack(scales)

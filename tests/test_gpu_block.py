@@ -47,15 +47,21 @@ def test_block_ragged(gpu):
 
 
 def test_block_config5(gpu):
-    """benchmark configuration 5: B 8, T 1024, D 768, 12 heads x 64, seed 5."""
+    """benchmark configuration 5: B 8, T 1024, D 768, 12 heads x 64, seed 5; all eight
+    sequences against float64.  The tolerance comes from the bar of the products,
+    1e-5 relative to sum |a||b|: per output element 1e-5 times the magnitude the last
+    product of each residual branch sums over (about 1.6e-4 here, where the output is O(1))."""
     gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
     from oracle import gpt2_block_ref as ref
     W = gpu
     params = gpt2.make_block_params(5)
     x = gpt2.make_block_input(5)
-    want = ref.block_forward(x[:2], params, 12)  # float64 on two sequences keeps the CPU part short
+    want, scale = ref.block_forward_with_scale(x, params, 12)
+    assert np.allclose(want[:1], ref.block_forward(x[:1], params, 12), rtol=0, atol=1e-12)
     dp = gpt2.to_device(params)
-    for mode in ("fused", "nodes"):
+    for mode in ("fused", "fused_matmul_attention", "nodes"):
         got = gpt2.block_forward(W.HIPTensor.from_numpy(x), dp, mode=mode).numpy()
-        np.testing.assert_allclose(got[:2], want, rtol=2e-4, atol=2e-4, err_msg=mode)
-        assert np.isfinite(got).all()
+        assert got.shape == want.shape
+        ratio = np.abs(got - want) / scale
+        print(mode, "worst error / (sum |a||b| of the last products):", ratio.max(), flush=True)
+        assert ratio.max() <= 1e-5, (mode, ratio.max())
