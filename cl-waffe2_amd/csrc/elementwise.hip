@@ -77,6 +77,11 @@ struct OpCosH { static constexpr int kFlatU = 2; __device__ __forceinline__ floa
 struct OpLog2 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log2f_(s); } };
 struct OpLog10 { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log10f_(s); } };
 struct OpLog1p { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return log1pf_(s); } };
+struct OpSign { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return signf_(s); } };
+struct OpSquare { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return s * s; } };
+struct OpASinH { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return asinhf_(s); } };
+struct OpACosH { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return acoshf_(s); } };
+struct OpATanH { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return atanhf_(s); } };
 struct OpInv { static constexpr int kFlatU = 4; __device__ __forceinline__ float operator()(float, float s) const { return 1.0f / s; } };
 struct OpGelu { static constexpr int kFlatU = 2; __device__ __forceinline__ float operator()(float, float s) const { return gelu_tanh_f(s); } };
 // The activation recipes of nn/activation.lisp as single kernels; each performs
@@ -1189,6 +1194,11 @@ int unary_nd(int op, Space s, const float* x, float* out, float p) {
     case WF2HIP_LOG10: return launch_elementwise<OpLog10, false>(s, out, x, OpLog10{});
     case WF2HIP_LOG1P: return launch_elementwise<OpLog1p, false>(s, out, x, OpLog1p{});
     case WF2HIP_INV: return launch_elementwise<OpInv, false>(s, out, x, OpInv{});
+    case WF2HIP_SIGN: return launch_elementwise<OpSign, false>(s, out, x, OpSign{});
+    case WF2HIP_SQUARE: return launch_elementwise<OpSquare, false>(s, out, x, OpSquare{});
+    case WF2HIP_ASINH: return launch_elementwise<OpASinH, false>(s, out, x, OpASinH{});
+    case WF2HIP_ACOSH: return launch_elementwise<OpACosH, false>(s, out, x, OpACosH{});
+    case WF2HIP_ATANH: return launch_elementwise<OpATanH, false>(s, out, x, OpATanH{});
     case WF2HIP_GELU: return launch_elementwise<OpGelu, false>(s, out, x, OpGelu{});
     case WF2HIP_RELU: return launch_elementwise<OpRelu, false>(s, out, x, OpRelu{});
     case WF2HIP_SIGMOID: return launch_elementwise<OpSigmoid, false>(s, out, x, OpSigmoid{});

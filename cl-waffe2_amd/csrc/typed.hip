@@ -917,6 +917,11 @@ __device__ __forceinline__ double dmath(double x, double p) {
   else if constexpr (OP == WF2HIP_LOG10) return ::log10(x);
   else if constexpr (OP == WF2HIP_LOG1P) return x == 0.0 ? x : ::log1p(x);  // keeps the sign of -0
   else if constexpr (OP == WF2HIP_POW) return ::pow(x, p);
+  else if constexpr (OP == WF2HIP_SIGN) return x > 0.0 ? 1.0 : (x < 0.0 ? -1.0 : x);
+  else if constexpr (OP == WF2HIP_SQUARE) return x * x;
+  else if constexpr (OP == WF2HIP_ASINH) return ::asinh(x);
+  else if constexpr (OP == WF2HIP_ACOSH) return ::acosh(x);
+  else if constexpr (OP == WF2HIP_ATANH) return ::atanh(x);
   else return 1.0 / x;  // WF2HIP_INV
 }
 
@@ -1022,7 +1027,9 @@ static int dispatch_dunary(int op, const Space& s, const double* x, double* out,
     WF2_DUNARY_CASE(WF2HIP_EXP) WF2_DUNARY_CASE(WF2HIP_SQRT) WF2_DUNARY_CASE(WF2HIP_ABS) WF2_DUNARY_CASE(WF2HIP_TAN)
     WF2_DUNARY_CASE(WF2HIP_ASIN) WF2_DUNARY_CASE(WF2HIP_ACOS) WF2_DUNARY_CASE(WF2HIP_ATAN) WF2_DUNARY_CASE(WF2HIP_SINH)
     WF2_DUNARY_CASE(WF2HIP_COSH) WF2_DUNARY_CASE(WF2HIP_LOG2) WF2_DUNARY_CASE(WF2HIP_LOG10)
-    WF2_DUNARY_CASE(WF2HIP_LOG1P) WF2_DUNARY_CASE(WF2HIP_POW)
+    WF2_DUNARY_CASE(WF2HIP_LOG1P) WF2_DUNARY_CASE(WF2HIP_POW) WF2_DUNARY_CASE(WF2HIP_SIGN)
+    WF2_DUNARY_CASE(WF2HIP_SQUARE) WF2_DUNARY_CASE(WF2HIP_ASINH) WF2_DUNARY_CASE(WF2HIP_ACOSH)
+    WF2_DUNARY_CASE(WF2HIP_ATANH)
 #undef WF2_DUNARY_CASE
     default: return fail(WF2HIP_EINVAL, "unary op %d has no :double kernel", op);
   }

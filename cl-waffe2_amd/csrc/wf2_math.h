@@ -561,6 +561,47 @@ WF2_MATH_FN float acosf_(float x) {
   return (float)(2.0 * atan_core(__builtin_sqrt((1.0 - xd) / (1.0 + xd))));
 }
 
+// The inverse hyperbolic functions through the binary64 logarithm (0.52 ulp); small
+// arguments, where 1 + y would round y away, through their series.
+WF2_MATH_FN float asinhf_(float x) {
+  const double t = __builtin_fabs((double)x);
+  const double t2 = t * t;
+  double r;
+  if (t < 0x1p-10)
+    r = t * WF2_FMA(t2, WF2_FMA(t2, 0.075, -0.16666666666666666667), 1.0);
+  else if (t > 0x1p30)
+    r = log_core(t) + kLn2;  // sqrt(t^2 + 1) = t to binary64 precision
+  else
+    r = log_core(t + __builtin_sqrt(t2 + 1.0));
+  const float v = __builtin_copysignf((float)r, x);
+  return (x != x || __builtin_fabsf(x) == __builtin_inff()) ? x : v;
+}
+
+WF2_MATH_FN float acoshf_(float x) {
+  if (!(x >= 1.0f)) return __builtin_nanf("");
+  if (x == __builtin_inff()) return x;
+  const double t = (double)x;
+  if (t > 0x1p30) return (float)(log_core(t) + kLn2);
+  // (x - 1)(x + 1) is exact in binary64 for a binary32 x; x = 1 gives log(1) = 0
+  return (float)log_core(t + __builtin_sqrt((t - 1.0) * (t + 1.0)));
+}
+
+WF2_MATH_FN float atanhf_(float x) {
+  const double t = __builtin_fabs((double)x);
+  if (!(t <= 1.0)) return __builtin_nanf("");
+  if (t == 1.0) return __builtin_copysignf(__builtin_inff(), x);
+  const double t2 = t * t;
+  double r;
+  if (t < 0x1p-10)
+    r = t * WF2_FMA(t2, WF2_FMA(t2, 0.2, 0.33333333333333333333), 1.0);
+  else
+    r = 0.5 * log_core((1.0 + t) / (1.0 - t));  // 1 + t and 1 - t are exact
+  return __builtin_copysignf((float)r, x);
+}
+
+// CL's signum on floats: -1, 1, and the argument itself when it is +-0 or NaN
+WF2_MATH_FN float signf_(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : x); }
+
 WF2_MATH_FN float sqrtf_(float x) { return WF2_SQRTF(x); }
 WF2_MATH_FN float absf_(float x) { return __builtin_fabsf(x); }
 

@@ -244,6 +244,11 @@ def cosh(x, out=None): return _math("CosHNode", x, out)
 def log2(x, out=None): return _math("Log2Node", x, out)
 def log10(x, out=None): return _math("Log10Node", x, out)
 def log1p(x, out=None): return _math("Log1pNode", x, out)
+def sign(x, out=None): return _math("SignNode", x, out)
+def square(x, out=None): return _math("SquareNode", x, out)
+def asinh(x, out=None): return _math("ASinHNode", x, out)
+def acosh(x, out=None): return _math("ACosHNode", x, out)
+def atanh(x, out=None): return _math("ATanHNode", x, out)
 
 
 def expt(x: HIPTensor, n: float, out: HIPTensor | None = None) -> HIPTensor:

@@ -23,6 +23,7 @@ DTYPE_CODES = {"double": 1, "int32": 2, "uint32": 3, "int16": 4, "uint16": 5, "i
 SIN, COS, TANH, LOG, EXP, SQRT, ABS = 16, 17, 18, 19, 20, 21, 22
 TAN, ASIN, ACOS, ATAN, SINH, COSH, LOG2, LOG10, LOG1P = 23, 24, 25, 26, 27, 28, 29, 30, 31
 POW, GELU = 32, 40
+SIGN, SQUARE, ASINH, ACOSH, ATANH = 34, 35, 36, 37, 38
 RELU, SIGMOID, LEAKY_RELU = 41, 42, 43  # fused activation recipes
 EQ, LT, LE, GT, GE = 0, 1, 2, 3, 4  # enum wf2hip_compare_op
 COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")

@@ -170,6 +170,7 @@ served from the library's pool; transfers and vref are refused while recording."
 (defconstant +exp+ 20) (defconstant +sqrt+ 21) (defconstant +abs+ 22) (defconstant +pow+ 32)
 (defconstant +tan+ 23) (defconstant +asin+ 24) (defconstant +acos+ 25) (defconstant +atan+ 26)
 (defconstant +sinh+ 27) (defconstant +cosh+ 28) (defconstant +log2+ 29) (defconstant +log10+ 30) (defconstant +log1p+ 31)
+(defconstant +sign+ 34) (defconstant +square+ 35) (defconstant +asinh+ 36) (defconstant +acosh+ 37) (defconstant +atanh+ 38)
 
 (defun hip-synchronize ()
   "Blocks until every kernel enqueued so far has finished (needed around wall-clock timing such

@@ -113,7 +113,16 @@ extension has both, source/backends/cpu/mathematics.lisp:8-76)."
   (define-math CosHNode +cosh+)
   (define-math Log2Node +log2+)
   (define-math Log10Node +log10+)
-  (define-math Log1pNode +log1p+))
+  (define-math Log1pNode +log1p+)
+  ;; The CPU backend has no impl for these five and leaves them to LispTensor
+  ;; (source/backends/lisp/mathematics.lisp:30), whose kernels aref the storage vector: with
+  ;; HIPTensor first in *using-backend* they would be handed a device handle.  !abs's backward
+  ;; multiplies by !sign (source/base-impl/mathematics.lisp:125-131).
+  (define-math SignNode +sign+)
+  (define-math SquareNode +square+)
+  (define-math ASinHNode +asinh+)
+  (define-math ACosHNode +acosh+)
+  (define-math ATanHNode +atanh+))
 
 ;; OUT <- X^N with N a host ScalarTensor (source/base-impl/mathematics.lisp:267-303)
 (define-impl-op (ExptNode :device HIPTensor :reject-p #'float-or-double-p)

@@ -30,6 +30,7 @@ NODE_NAMES = (
     "AddNode", "SubNode", "MulNode", "DivNode", "MoveTensorNode",
     "SinNode", "CosNode", "TanhNode", "LogENode", "ExpNode", "SqrtNode", "AbsNode",
     "TanNode", "ASinNode", "ACosNode", "ATanNode", "SinHNode", "CosHNode", "Log2Node", "Log10Node", "Log1pNode",
+    "SignNode", "SquareNode", "ASinHNode", "ACosHNode", "ATanHNode",
     "ExptNode", "MatMulNode",
     "Where-Operation-Node", "Compare-Operation-Node",
     "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
@@ -174,7 +175,11 @@ for _name, _op in (("SinNode", _lib.SIN), ("CosNode", _lib.COS), ("TanhNode", _l
                    ("LogENode", _lib.LOG), ("ExpNode", _lib.EXP), ("SqrtNode", _lib.SQRT),
                    ("AbsNode", _lib.ABS), ("TanNode", _lib.TAN), ("ASinNode", _lib.ASIN), ("ACosNode", _lib.ACOS),
                    ("ATanNode", _lib.ATAN), ("SinHNode", _lib.SINH), ("CosHNode", _lib.COSH),
-                   ("Log2Node", _lib.LOG2), ("Log10Node", _lib.LOG10), ("Log1pNode", _lib.LOG1P)):
+                   ("Log2Node", _lib.LOG2), ("Log10Node", _lib.LOG10), ("Log1pNode", _lib.LOG1P),
+                   # nodes the CPU backend leaves to LispTensor (base-impl/mathematics.lisp:131,147,217-219):
+                   # with HIPTensor first in the backend list they must stay on the device
+                   ("SignNode", _lib.SIGN), ("SquareNode", _lib.SQUARE), ("ASinHNode", _lib.ASINH),
+                   ("ACosHNode", _lib.ACOSH), ("ATanHNode", _lib.ATANH)):
     define_impl(_name, HIPTensor, _float_or_double)(_unary(_op))
 
 

@@ -188,6 +188,11 @@ enum wf2hip_unary_op {
   WF2HIP_LOG1P = 31,
   WF2HIP_POW = 32, /* ExptNode mathematics.lisp:267-303 */
   WF2HIP_INV = 33, /* 1 / x */
+  WF2HIP_SIGN = 34,   /* SignNode: -1, +-0, 1 (CL signum; NaN stays NaN)  mathematics.lisp:131 */
+  WF2HIP_SQUARE = 35, /* SquareNode: x * x                               mathematics.lisp:147 */
+  WF2HIP_ASINH = 36,  /* ASinHNode, ACosHNode, ATanHNode: the inverse hyperbolic functions */
+  WF2HIP_ACOSH = 37,  /* themselves (mathematics.lisp:217-219), not the hyperbolic ones the   */
+  WF2HIP_ATANH = 38,  /* SIMD extension binds under these names (cl-waffe2-simd.c:672-679)     */
   WF2HIP_GELU = 40, /* fused tanh-form GELU (nn/activation.lisp:45-66) */
   WF2HIP_RELU = 41, /* fused !relu = x * (x > 0 ? 1 : 0) (nn/activation.lisp:11-25), bit-identical to the two nodes */
   WF2HIP_SIGMOID = 42, /* fused !sigmoid = 1 / (1 + exp(-1 x)) (nn/activation.lisp:27-43), each step rounded as its node */

@@ -30,9 +30,12 @@ OPS = {
     "sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21,
     "abs": 22, "tan": 23, "asin": 24, "acos": 25, "atan": 26, "sinh": 27, "cosh": 28, "log2": 29,
     "log10": 30, "log1p": 31, "pow": 32,
+    "sign": 34, "square": 35, "asinh": 36, "acosh": 37, "atanh": 38,
 }
 UNARY_NAMES = ("sin", "cos", "tanh", "log", "exp", "sqrt", "abs", "tan", "asin", "acos", "atan", "sinh", "cosh",
                "log2", "log10", "log1p")
+# nodes that run LispTensor's per-element loop in the reference (no SIMD kernel)
+LISP_UNARY_NAMES = ("sign", "square", "asinh", "acosh", "atanh")
 
 
 class OrcViews(C.Structure):
@@ -102,7 +105,7 @@ def lib():
         f.restype = None
     L.orc_scopy.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
     L.orc_scopy.restype = None
-    for name in UNARY_NAMES:
+    for name in UNARY_NAMES + LISP_UNARY_NAMES:
         f = getattr(L, "orc_s" + name)
         f.argtypes = [C.c_long, _F, C.c_long, _F, C.c_long]
         f.restype = None

@@ -196,6 +196,30 @@ ORC_DEFINE_UNARY(log2, "Sleef_log2f8_u10avx2", log2)
 ORC_DEFINE_UNARY(log10, "Sleef_log10f8_u10avx2", log10)
 ORC_DEFINE_UNARY(log1p, "Sleef_log1pf8_u10avx2", log1p)
 
+/* SignNode, SquareNode, ASinHNode, ACosHNode, ATanHNode have no CPUTensor implementation:
+ * they run LispTensor's per-element loop y[offy + incy i] <- f(x[offx + incx i])
+ * (source/backends/lisp/mathematics.lisp:11-45) with f = signum, (* x x), asinh, acosh,
+ * atanh of Common Lisp (:48,52,:66-68 of the same file).  CL's functions are restated by
+ * their definitions: signum keeps +-0 (and NaN), the inverse hyperbolic functions of a
+ * single-float are the mathematical ones rounded to binary32, evaluated here in binary64
+ * by libm.  PARITY UNPINNED BY THE REFERENCE beyond its own one-point test
+ * (mathematical-test-set at x = 1, source/base-impl/t/mathematical.lisp:37-162): no
+ * Common Lisp implementation is available to produce vectors; pinned by float64 closed
+ * forms (tests/test_oracle_golden.py). */
+static float lisp_signum(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : x); }
+#define ORC_DEFINE_LISP_UNARY(name, expr)                                                       \
+  ORC_API void orc_s##name(long n, const float *x, long incx, float *out, long inco) {          \
+    for (long i = 0; i < n; i++) {                                                              \
+      const float v = x[i * incx];                                                              \
+      out[i * inco] = (expr);                                                                   \
+    }                                                                                           \
+  }
+ORC_DEFINE_LISP_UNARY(sign, lisp_signum(v))
+ORC_DEFINE_LISP_UNARY(square, v * v)
+ORC_DEFINE_LISP_UNARY(asinh, (float)asinh((double)v))
+ORC_DEFINE_LISP_UNARY(acosh, (float)acosh((double)v))
+ORC_DEFINE_LISP_UNARY(atanh, (float)atanh((double)v))
+
 /* out <- x^p  (cl-waffe2-simd.c:708-768; avx2.h:304) */
 ORC_API void orc_spow(long n, const float *x, long incx, float p, float *out,
                       long inco) {

@@ -13,7 +13,8 @@
 #include "../../cl-waffe2_amd/csrc/wf2_math.h"
 
 enum { OP_SIN = 16, OP_COS, OP_TANH, OP_LOG, OP_EXP, OP_SQRT, OP_ABS, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN,
-       OP_SINH, OP_COSH, OP_LOG2, OP_LOG10, OP_LOG1P, OP_GELU = 40 };
+       OP_SINH, OP_COSH, OP_LOG2, OP_LOG10, OP_LOG1P, OP_SIGN = 34, OP_SQUARE, OP_ASINH, OP_ACOSH, OP_ATANH,
+       OP_GELU = 40 };
 
 static inline float apply(int op, float x) {
   switch (op) {
@@ -34,6 +35,11 @@ static inline float apply(int op, float x) {
     case OP_LOG10: return wf2::log10f_(x);
     case OP_LOG1P: return wf2::log1pf_(x);
     case OP_GELU: return wf2::gelu_tanh_f(x);
+    case OP_SIGN: return wf2::signf_(x);
+    case OP_SQUARE: return x * x;
+    case OP_ASINH: return wf2::asinhf_(x);
+    case OP_ACOSH: return wf2::acoshf_(x);
+    case OP_ATANH: return wf2::atanhf_(x);
   }
   return 0.0f;
 }
@@ -56,6 +62,11 @@ static inline double truth(int op, double x) {
     case OP_LOG2: return log2(x);
     case OP_LOG10: return log10(x);
     case OP_LOG1P: return log1p(x);
+    case OP_SIGN: return x > 0 ? 1.0 : (x < 0 ? -1.0 : x);
+    case OP_SQUARE: return x * x;
+    case OP_ASINH: return asinh(x);
+    case OP_ACOSH: return acosh(x);
+    case OP_ATANH: return atanh(x);
     case OP_GELU: {
       // 0.5 (1 + tanh u) == 1 / (1 + exp(-2u)), free of cancellation
       double u = 0.7978845608028654 * (x + 0.044715 * x * x * x);

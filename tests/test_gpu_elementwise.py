@@ -599,3 +599,46 @@ def test_gelu_known_answer(gpu):
     truth = truth / (1.0 + np.exp(-2.0 * 0.7978845608028654 * (truth + 0.044715 * truth ** 3)))
     assert ulp_distance(F.gelu_fused(F.from_numpy(x)).numpy(), truth.astype(np.float32)).max() <= 2
     np.testing.assert_allclose(F.gelu(F.from_numpy(x)).numpy(), truth, rtol=2e-5, atol=2e-6)
+
+
+LISP_LOOP_NODES = [("sign", -3, 3), ("square", -100, 100), ("asinh", -1e4, 1e4), ("acosh", 1, 1e4),
+                   ("atanh", -0.999, 0.999)]
+
+
+@pytest.mark.parametrize("op,lo,hi", LISP_LOOP_NODES)
+def test_nodes_the_cpu_backend_leaves_to_lisptensor(gpu, O, op, lo, hi):
+    """SignNode, SquareNode, ASinHNode, ACosHNode, ATanHNode (the CPU backend has no impl;
+    LispTensor's loop would be handed a device handle): against the oracle's restatement
+    of that loop and against float64 on 2^20 elements -- sign and square bit-exact, the
+    inverse hyperbolic functions within 1 ulp -- on a strided view, on :double, and on
+    the special values."""
+    W = gpu
+    F = W.functional
+    rng = np.random.Generator(np.random.PCG64(34))
+    n = 1 << 20
+    x = rng.uniform(lo, hi, n).astype(np.float32)
+    want = np.zeros(n, np.float32)
+    O.unary_1d(op, n, x, 1, want, 1)
+    got = getattr(F, op)(F.from_numpy(x)).numpy()
+    limit = 0 if op in ("sign", "square") else 1
+    assert ulp_distance(got, want).max() <= limit
+    # CL's signum keeps the sign of a zero, numpy's sign does not
+    truth = {"sign": lambda v: np.where(v == 0, v, np.sign(v)), "square": np.square, "asinh": np.arcsinh,
+             "acosh": np.arccosh, "atanh": np.arctanh}[op]
+    assert ulp_distance(got, truth(x.astype(np.float64)).astype(np.float32)).max() <= limit
+    # a strided, offset view as source and a column of a matrix as destination
+    src = F.from_numpy(x[:6000].reshape(60, 100)).view((5, 55), (3, 99, 2))
+    dst = W.HIPTensor([50, 48])
+    getattr(F, op)(src, out=dst)
+    assert ulp_distance(dst.numpy(), truth(x[:6000].reshape(60, 100)[5:55, 3:99:2].astype(np.float64))
+                        .astype(np.float32)).max() <= limit
+    # :double tensors go through the binary64 routines
+    xd = x[:5000].astype(np.float64)
+    gotd = getattr(F, op)(F.from_numpy(xd, dtype="double")).numpy()
+    np.testing.assert_allclose(gotd, truth(xd), rtol=4e-16, atol=0)
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5, 1e-30, -1e-30, 3e38], np.float32)
+    with np.errstate(all="ignore"):
+        te = truth(edge.astype(np.float64)).astype(np.float32)
+    ge = getattr(F, op)(F.from_numpy(edge)).numpy()
+    assert ulp_distance(ge, te).max() <= limit, (edge, ge, te)
+    assert np.array_equal(np.signbit(ge[~np.isnan(te)]), np.signbit(te[~np.isnan(te)]))

@@ -348,3 +348,32 @@ def test_im2col_golden(O):
     im = gold["im2col_0_im"][0, 0]
     want = np.lib.stride_tricks.sliding_window_view(im, (3, 3)).transpose(2, 3, 0, 1)
     assert_bit_equal(gold["im2col_0_col"][0, 0], np.ascontiguousarray(want), "sliding window")
+
+
+def test_lisp_loop_nodes_follow_their_definitions(O):
+    """SignNode, SquareNode, ASinHNode, ACosHNode, ATanHNode (LispTensor's per-element
+    loop in the reference; no SIMD kernel, no golden vectors): the oracle against the
+    float64 closed forms, strided and with special values."""
+    rng = np.random.default_rng(5)
+    truth = {"sign": np.sign, "square": np.square, "asinh": np.arcsinh, "acosh": np.arccosh, "atanh": np.arctanh}
+    ranges = {"sign": (-3, 3), "square": (-100, 100), "asinh": (-1e4, 1e4), "acosh": (1, 1e4), "atanh": (-0.999, 0.999)}
+    for op in O.LISP_UNARY_NAMES:
+        lo, hi = ranges[op]
+        for n, incx, inco in [(1000, 1, 1), (333, 3, 2), (7, 1, 5)]:
+            x = rng.uniform(lo, hi, n * incx).astype(np.float32)
+            out = np.full(n * inco, 99.0, np.float32)
+            O.unary_1d(op, n, x, incx, out, inco)
+            with np.errstate(all="ignore"):
+                want = truth[op](x[::incx][:n].astype(np.float64)).astype(np.float32)
+            assert np.array_equal(out[::inco][:n], want) or \
+                np.abs(out[::inco][:n].view(np.int32).astype(np.int64) - want.view(np.int32)).max() <= 1, op
+            if inco > 1:
+                assert np.all(out.reshape(-1, inco)[:, 1:] == 99.0)
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5], np.float32)
+    out = np.zeros_like(edge)
+    O.unary_1d("sign", edge.size, edge, 1, out, 1)
+    assert out[:4].tolist() == [0.0, -0.0, 1.0, -1.0] and np.signbit(out[1]) and np.isnan(out[4])
+    O.unary_1d("atanh", edge.size, edge, 1, out, 1)
+    assert out[5] == np.inf and out[6] == -np.inf and np.isnan(out[2]) and out[0] == 0.0
+    O.unary_1d("acosh", edge.size, edge, 1, out, 1)
+    assert out[5] == 0.0 and np.isnan(out[7]) and out[2] == np.inf
