@@ -367,12 +367,9 @@ def leaky_relu(x: HIPTensor, negative_slope: float = 0.01) -> HIPTensor:
 
 
 def _fused_activation(op: int, x: HIPTensor, out: HIPTensor | None, p: float = 0.0) -> HIPTensor:
-    import ctypes as C
     if out is None:
         out = HIPTensor(x.shape, initial_element=None)
-    v = nodes.view2(x, out)
-    _lib.check(_lib.get().wf2hip_unary_nd(op, C.byref(v), C.c_void_p(x.ptr), C.c_void_p(out.ptr), float(p)))
-    return out
+    return nodes.forward("HIP-Activation-Node", x, out, op, float(p))
 
 
 def relu_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
@@ -588,50 +585,65 @@ def softmax(x: HIPTensor, avoid_overflow: bool = True, axis=1) -> HIPTensor:
 
 
 def softmax_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
-    """Max-subtracted softmax over the last axis in one kernel
-    (``wf2hip_softmax_rows_f32``)."""
-    import ctypes as C
+    """Max-subtracted softmax over the last axis in one kernel (HIP-Softmax-Node).  A given
+    ``out`` must be a contiguous :float tensor of x's shape that starts at its storage."""
     x = to_contiguous(x)
     if out is None:
         out = HIPTensor(x.shape, initial_element=None)
-    cols = x.shape[-1]
-    rows = x.size // _builtins.max(cols, 1)
-    _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols,
-                                                 C.c_void_p(out.ptr), cols))
+    return nodes.forward("HIP-Softmax-Node", x, out)
+
+
+def causal_softmax_fused(scores: HIPTensor, scale: float = 1.0, out: HIPTensor | None = None) -> HIPTensor:
+    """softmax over j <= i of ``scale * scores[..., i, j]``, zero above the diagonal, in one
+    kernel (HIP-Causal-Softmax-Node): the scaling MulNode, the mask's AddNode and !softmax of
+    causal attention."""
+    scores = to_contiguous(scores)
+    if out is None:
+        out = HIPTensor(scores.shape, initial_element=None)
+    return nodes.forward("HIP-Causal-Softmax-Node", scores, out, float(scale))
+
+
+def linear(x: HIPTensor, w: HIPTensor, b: HIPTensor, activation: str | None = None,
+           residual: HIPTensor | None = None, out: HIPTensor | None = None) -> HIPTensor:
+    """``act(x . w + b) + residual`` for x[~ k], w[k n], b[n] as ONE node (HIP-Linear-Node /
+    HIP-Linear-Residual-Node; ``!linear-hip`` of the Lisp glue): the MatMulNode, the bias's
+    AddNode, !gelu and the residual's AddNode of ``examples/gpt-2/model.lisp:109-137``.
+    Leading axes of x are folded into rows."""
+    if activation not in (None, "gelu"):
+        raise ValueError("linear: activation must be None or 'gelu'")
+    if residual is not None and activation is not None:
+        raise ValueError("linear: a residual closes a branch without activation")
+    k, n = x.shape[-1], w.shape[-1]
+    x2 = reshape(x, -1, k)
+    if out is None:
+        out = HIPTensor(list(x.shape[:-1]) + [n], initial_element=None)
+    out2 = reshape(out, -1, n) if out.is_contiguous() else None
+    if out2 is None:
+        raise ValueError("linear: out must be contiguous")
+    w2 = to_contiguous(w)
+    if residual is not None:
+        nodes.forward("HIP-Linear-Residual-Node", x2, w2, b, reshape(residual, -1, n), out2)
+    else:
+        nodes.forward("HIP-Linear-Node", x2, w2, b, out2, activation)
     return out
 
 
 def attention(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor | None = None,
               scale: float | None = None, causal: bool = False) -> HIPTensor:
     """softmax(scale q k^T [+ causal mask]) v for (batch, heads, seq, 64) views in
-    one kernel (``wf2hip_attention_f32``): the fused form of SelfAttention's
-    !matmul / !softmax / !matmul chain (``examples/gpt-2/utils.lisp:222-243``).
+    one kernel (HIP-Attention-Node; ``!attention-hip`` of the Lisp glue): the fused form of
+    SelfAttention's !matmul / !softmax / !matmul chain (``examples/gpt-2/utils.lisp:222-243``).
     Operands may be any views whose last axis is contiguous (heads read in
     place from a fused projection); ``out`` defaults to a fresh (B, H, T, 64)
     tensor."""
-    import ctypes as C
     if not (len(q.shape) == len(k.shape) == len(v.shape) == 4) or \
             not (list(q.shape) == list(k.shape) == list(v.shape)):
         raise ValueError("attention expects three (batch, heads, seq, head_dim) tensors of one shape")
     B, H, T, hd = q.shape
     if out is None:
         out = HIPTensor([B, H, T, hd], initial_element=None)
-    if list(out.shape) != [B, H, T, hd]:
-        raise ValueError("attention: out must have the operands' shape")
-    d = _lib.AttentionDesc()
-    d.batch, d.heads, d.seq, d.head_dim = B, H, T, hd
-    ptrs = []
-    for t, field in ((q, d.q_stride), (k, d.k_stride), (v, d.v_stride), (out, d.o_stride)):
-        _, strides, off = t.geometry()
-        if hd > 1 and strides[3] != 1:
-            raise ValueError("attention: the head_dim axis must be contiguous")
-        for a in range(3):
-            field[a] = strides[a]
-        ptrs.append(C.c_void_p(t.ptr + 4 * off))
-    d.scale = float(1.0 / math.sqrt(hd) if scale is None else scale)
-    d.causal = 1 if causal else 0
-    _lib.check(_lib.get().wf2hip_attention_f32(C.byref(d), *ptrs))
-    return out
+    return nodes.forward("HIP-Attention-Node", q, k, v, out, 1.0 / math.sqrt(hd) if scale is None else scale,
+                         causal)
 
 
 def gelu(x: HIPTensor) -> HIPTensor:
@@ -643,13 +655,8 @@ def gelu(x: HIPTensor) -> HIPTensor:
 
 
 def gelu_fused(x: HIPTensor, out: HIPTensor | None = None) -> HIPTensor:
-    import ctypes as C
-    if out is None:
-        out = HIPTensor(x.shape, initial_element=None)
-    v = nodes.view2(x, out)
-    _lib.check(_lib.get().wf2hip_unary_nd(_lib.GELU, C.byref(v), C.c_void_p(x.ptr),
-                                         C.c_void_p(out.ptr), 0.0))
-    return out
+    """!gelu (tanh form) in one kernel (HIP-Activation-Node)."""
+    return _fused_activation(_lib.GELU, x, out)
 
 
 def layer_norm(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e-5) -> HIPTensor:
@@ -664,12 +671,31 @@ def layer_norm(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e-5) ->
 
 def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e-5,
                      out: HIPTensor | None = None) -> HIPTensor:
-    import ctypes as C
+    """LayerNorm over the last axis in one kernel (HIP-LayerNorm-Node; ``!layer-norm-hip``).
+    gamma, beta and a given ``out`` must be contiguous :float tensors that start at their
+    storage, of shapes (cols,), (cols,) and x's."""
     x = to_contiguous(x)
     if out is None:
         out = HIPTensor(x.shape, initial_element=None)
+    return nodes.forward("HIP-LayerNorm-Node", x, g, b, out, float(eps))
+
+
+def layer_norm_backward(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float = 1.0e-5):
+    """(dx, dgamma, dbeta) of LayerNorm over the last axis, composed node for node the way
+    ``layer-norm-gradients`` of the Lisp glue composes the backward of HIP-LayerNorm-Node:
+    with xh = (x - u) rstd and dyh = dout g,
+    dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)), dgamma = sum_rows dout xh, dbeta = sum_rows dout."""
     cols = x.shape[-1]
-    rows = x.size // _builtins.max(cols, 1)
-    _lib.check(_lib.get().wf2hip_layernorm_rows_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),
-                                                   C.c_void_p(b.ptr), float(eps), C.c_void_p(out.ptr)))
-    return out
+    x2, d2 = reshape(x, -1, cols), reshape(dout, -1, cols)
+    u = mean(x2, axis=-1, keepdims=True)
+    xc = sub(x2, u)
+    s = mean(mul(xc, xc), axis=-1, keepdims=True)
+    rstd = reciprocal(sqrt(add(to_contiguous(s), eps)))
+    xh = mul(xc, rstd)
+    dyh = mul(d2, g)
+    m1 = mean(dyh, axis=-1, keepdims=True)
+    m2 = mean(mul(dyh, xh), axis=-1, keepdims=True)
+    dx = mul(sub(sub(dyh, m1), mul(xh, m2)), rstd)
+    dg = sum(mul(d2, xh), axis=0)
+    db = sum(d2, axis=0)
+    return HIPTensor(x.shape, vec=dx.vec), reshape(dg, cols), reshape(db, cols)

@@ -91,7 +91,7 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
 
     h = ln(x, p["ln1_g"], p["ln1_b"], eps)
     if fused:
-        qkv = F.matmul(h, p["w_qkv"], bias=p["b_qkv"])             # (B, T, 3D)
+        qkv = F.linear(h, p["w_qkv"], p["b_qkv"])                  # (B, T, 3D), HIP-Linear-Node
     else:
         qkv = _linear(h, p["w_qkv"], p["b_qkv"])
 
@@ -111,9 +111,7 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         # (B, 1, H, T, hd) strided windows of the projection, no copy
         q, k, v = (five.view(True, True, i, True, True).permute(0, 2, 3, 1, 4) for i in range(3))
         scores = F.matmul(q, F.t(k), causal=1)                      # (B, 1, H, T, T), lower triangle
-        probs = HIPTensor(scores.shape, initial_element=None)
-        _lib.check(_lib.get().wf2hip_causal_softmax_f32(B * H, T, C.c_void_p(scores.ptr),
-                                                       C.c_void_p(probs.ptr), scale))
+        probs = F.causal_softmax_fused(scores, scale)              # HIP-Causal-Softmax-Node
         ctx_store = HIPTensor([B, T, 1, H, hd], initial_element=None)
         F.matmul(probs, v, out=ctx_store.permute(0, 2, 3, 1, 4), causal=2)  # written as (B, T, H*hd)
         ctx = F.reshape(ctx_store, B, T, D)
@@ -132,10 +130,11 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
 
     if fused:
         # bias, GELU and the residual adds ride in the products' epilogues
-        x1 = F.matmul(ctx, p["w_o"], bias=p["b_o"], residual=x)
+        # (HIP-Linear-Residual-Node, HIP-Linear-Node :gelu, HIP-Linear-Residual-Node)
+        x1 = F.linear(ctx, p["w_o"], p["b_o"], residual=x)
         h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)
-        f = F.matmul(h2, p["w_fc"], bias=p["b_fc"], activation="gelu")
-        return F.matmul(f, p["w_proj"], bias=p["b_proj"], residual=x1)
+        f = F.linear(h2, p["w_fc"], p["b_fc"], activation="gelu")
+        return F.linear(f, p["w_proj"], p["b_proj"], residual=x1)
     attn = _linear(ctx, p["w_o"], p["b_o"])
     x1 = F.add(x, attn)                                             # residual
     h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)

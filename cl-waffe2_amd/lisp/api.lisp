@@ -53,6 +53,7 @@
   (a :pointer) (lda :long) (stride-a :long)
   (b :pointer) (ldb :long) (stride-b :long)
   (beta :float) (c :pointer) (ldc :long) (stride-c :long) (batch :long))
+(defcfun "wf2hip_sum_nd" :int (view (:pointer (:struct view2))) (a :pointer) (b :pointer) (divisor :float))
 (defcfun "wf2hip_softmax_rows_f32" :int (rows :long) (cols :long) (x :pointer) (ldx :long) (out :pointer) (ldo :long))
 (defcfun "wf2hip_layernorm_rows_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (b :pointer) (eps :float) (out :pointer))
 

@@ -12,6 +12,11 @@
 ;;;;   * a define-bypass rule per function (source/vm/nodes/symbolic.lisp:118-131): with HIPTensor
 ;;;;     in *using-backend*, calls of cl-waffe2/nn:!relu & co. compiled after this file is loaded
 ;;;;     build the fused node instead ((setf *enable-symbolic-path* nil) switches that off).
+;;;; Also here, on the same two extension points: !sum / !mean as one node (HIP-Sum-Node, bypass rules),
+;;;; LayerNorm with its backward, and the nodes behind the 1.06 ms block forward -- product + bias
+;;;; (+ GELU) (+ residual) as one launch (HIP-Linear-Node, HIP-Linear-Residual-Node, !linear-hip),
+;;;; causal softmax (HIP-Causal-Softmax-Node) and attention as one kernel (HIP-Attention-Node,
+;;;; !attention-hip); the GPT-2 example's call sites they replace are named at each function.
 ;;;; The activation kernels round every step as the node recipe does (bit-identical results);
 ;;;; the softmax kernel subtracts the row maximum where the recipe subtracts the row mean, which
 ;;;; is the same function within the tolerance of the path (1e-5 relative).
@@ -109,7 +114,7 @@ DERIVATIVE is a function of (x) returning df/dx built from ! functions."
             :backward ((self dout)
                        ;; dx = y * (dy - sum(dy * y) over the row)
                        (with-reading-save4bw ((y y))
-                         (let ((dot (!sum (!mul dout y) :axis 1 :keepdims t)))
+                         (let ((dot (!sum-hip (!mul dout y) :axis 1 :keepdims t)))
                            (values (proceed (!mul y (!sub dout dot))) nil))))))
 
 (defun !softmax-hip (x &key (avoid-overflow t) (axis 1))
@@ -124,11 +129,31 @@ composed recipe."
       (call-composed 'cl-waffe2/nn:!softmax x :avoid-overflow avoid-overflow :axis axis)))
 
 ;; ---- LayerNorm over the last axis ------------------------------------------------------------
+(defun layer-norm-gradients (x g dout eps)
+  "Gradients of y = (x - u) / sqrt(s + eps) * g + b per row (source/nn/norms.lisp:72-82) from the
+saved input: with xh = (x - u) rstd and dyh = dout g,
+  dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),  dg = sum over rows of dout xh,  db = sum over rows of dout.
+Composed from ! functions (!mean and !sum are one node each on the device)."
+  (let* ((u    (!mean-hip x :axis -1 :keepdims t))
+         (xc   (!sub x u))
+         (s    (!mean-hip (!mul xc xc) :axis -1 :keepdims t))
+         (rstd (!div 1 (!sqrt (!add (->contiguous s) eps))))
+         (xh   (!mul xc rstd))
+         (dyh  (!mul dout (!flexible g)))
+         (m1   (!mean-hip dyh :axis -1 :keepdims t))
+         (m2   (!mean-hip (!mul dyh xh) :axis -1 :keepdims t))
+         (dx   (!mul rstd (!sub (!sub dyh m1) (!mul xh m2))))
+         (dg   (!sum-hip (!mul dout xh) :axis 0))
+         (db   (!sum-hip dout :axis 0)))
+    (values dx dg db)))
+
 (define-op (HIP-LayerNorm-Node (self eps)
             :slots ((eps :initform 1.0e-5 :accessor layernorm-eps))
+            :save-for-backward-names (x g)
             :where (X[rows cols] G[cols] B[cols] OUT[rows cols] -> OUT[rows cols])
             :documentation "OUT <- (x - mean) / sqrt(var + eps) * g + b per row, one kernel
-(wf2hip_layernorm_rows_f32); forward only (use the composed LayerNorm when training)."
+(wf2hip_layernorm_rows_f32).  Backward: the three gradients composed from the saved input
+(layer-norm-gradients)."
             :forward ((self x g b out)
                       (ensure-extension)
                       (check (wf2hip-layernorm-rows-f32 (first (shape x)) (second (shape x))
@@ -136,14 +161,264 @@ composed recipe."
                                                         (tensor-device-pointer g) (tensor-device-pointer b)
                                                         (coerce (layernorm-eps self) 'single-float)
                                                         (tensor-device-pointer out)))
-                      out))
+                      (with-setting-save4bw ((x x) (g g)) out))
+            :backward ((self dout)
+                       (with-reading-save4bw ((x x) (g g))
+                         (multiple-value-bind (dx dg db) (layer-norm-gradients x g dout (layernorm-eps self))
+                           (values (proceed dx)
+                                   (proceed (!reshape dg (second (shape x))))
+                                   (proceed (!reshape db (second (shape x))))
+                                   nil)))))
   (setf (layernorm-eps self) eps))
 
 (defun !layer-norm-hip (x gamma beta &key (eps 1.0e-5))
-  "LayerNorm of every row of the contiguous :float matrix X with scale GAMMA and shift BETA."
-  (let ((x (->contiguous x)))
-    (call (HIP-LayerNorm-Node eps) x gamma beta
-          (make-input (shape x) nil :dtype :float :order (order x)))))
+  "LayerNorm over the last axis of the :float tensor X with scale GAMMA and shift BETA: what
+LayerNorm-Revisit (examples/gpt-2/utils.lisp:114-127) and LayerNorm2D over one axis
+(source/nn/norms.lisp:72-82) compose from ten nodes.  Leading axes are folded into rows."
+  (let* ((cols (car (last (shape x))))
+         (x2 (!reshape (->contiguous x) t cols))
+         (y (call (HIP-LayerNorm-Node eps) x2 gamma beta
+                  (make-input (shape x2) nil :dtype :float :order (order x)))))
+    (apply #'!reshape y (shape x))))
+
+;; ---- !sum / !mean as one node -------------------------------------------------------------------
+(define-op (HIP-Sum-Node (self divisor)
+            :slots ((divisor :initform 1.0 :accessor sum-divisor))
+            :where (OUT[~] X[~] -> OUT[~])
+            :documentation "OUT <- (sum of X over the axes on which OUT is viewed (:broadcast n)) / divisor,
+overwriting OUT: one node for the A*=scal by 0, the A+=B into the broadcast view and the !div of
+!sum / !mean (source/base-impl/reduction.lisp:5-136), with the bits of that composition
+(wf2hip_sum_nd).  Backward: nothing flows to the overwritten OUT; X receives the gradient of the
+broadcast view, which has X's shape, divided by the divisor."
+            :forward ((self out x)
+                      (ensure-extension)
+                      (with-foreign-object (view '(:struct view2))
+                        (fill-view2 view out x)
+                        (check (wf2hip-sum-nd view (tensor-device-pointer out) (tensor-device-pointer x)
+                                              (coerce (sum-divisor self) 'single-float))))
+                      out)
+            :backward ((self dout)
+                       (values nil
+                               (if (= (sum-divisor self) 1)
+                                   dout
+                                   (proceed (!div dout (sum-divisor self)))))))
+  (setf (sum-divisor self) divisor))
+
+(defun !sum-hip (tensor &key (axis t) (-> nil) (keepdims nil) (div-by nil))
+  "(!sum tensor :axis .. :-> .. :keepdims ..) as one node on :float device tensors; same arguments as
+cl-waffe2/base-impl:!sum, whose argument handling (source/base-impl/reduction.lisp:31-60) is
+repeated here.  A DIV-BY that is not a number (the lazily multiplied scalar tensor !mean passes)
+takes the composed route; !mean-hip passes the count as a number."
+  (if (and (hip-float-tensor-p tensor)
+           (or (null ->) (hip-float-tensor-p ->))
+           (or (null div-by) (numberp div-by)))
+      (let* ((shape (copy-list (shape tensor)))
+             (dims (length shape))
+             (view-args (make-list dims :initial-element t)))
+        (flet ((reduce-axis (ax)
+                 (let ((ax (if (< ax 0) (+ ax dims) ax)))
+                   (setf (nth ax view-args) `(:broadcast ,(nth ax shape))
+                         (nth ax shape) 1))))
+          (typecase axis
+            (fixnum (reduce-axis axis))
+            (list (mapc #'reduce-axis axis))
+            (t (dotimes (ax dims) (reduce-axis ax)))))
+        (let ((out (or -> (make-input shape nil :dtype (dtype tensor) :order (order tensor)))))
+          (assert (equal (shape out) shape) ()
+                  "!sum: Assertion Failed because the given out's shape is ~a, but expected: ~a" (shape out) shape)
+          (multiple-value-bind (out* reverser) (apply #'!view out view-args)
+            (let ((result (call (HIP-Sum-Node (or div-by 1.0)) out* tensor)))
+              (if keepdims
+                  result
+                  (apply #'!view result reverser))))))
+      (call-composed 'cl-waffe2/base-impl:!sum tensor :axis axis :-> -> :keepdims keepdims :div-by div-by)))
+
+(defun !mean-hip (tensor &key (axis t) (-> nil) (keepdims nil))
+  "(!mean tensor ..) as one node: the element count is known from the shape when it is static."
+  (if (and (hip-float-tensor-p tensor) (every #'numberp (shape tensor)))
+      (let* ((dims (length (shape tensor)))
+             (axes (typecase axis
+                     (fixnum (list axis))
+                     (list axis)
+                     (t (loop for i below dims collect i))))
+             (count (reduce #'* (mapcar #'(lambda (ax) (nth (if (< ax 0) (+ ax dims) ax) (shape tensor))) axes))))
+        (!sum-hip tensor :axis axis :-> -> :keepdims keepdims :div-by (coerce count 'single-float)))
+      (call-composed 'cl-waffe2/base-impl:!mean tensor :axis axis :-> -> :keepdims keepdims)))
+
+;; ---- linear layers: product + bias (+ GELU) (+ residual) in the product's epilogue --------------
+(defun fill-matmul-desc (desc rows n k activation bias residual)
+  (macrolet ((field (name) `(foreign-slot-value desc '(:struct matmul-desc) ',name)))
+    (setf (field trans-a) 0 (field trans-b) 0
+          (field activation) (ecase activation ((nil :none) 0) (:gelu 1))
+          (field causal) 0
+          (field m) rows (field n) n (field k) k
+          (field lda) k (field ldb) n (field ldc) n
+          (field batch) 1 (field batch2) 1
+          (field stride-a) 0 (field stride-a2) 0 (field stride-b) 0 (field stride-b2) 0
+          (field stride-c) 0 (field stride-c2) 0
+          (field bias) (if bias (tensor-device-pointer bias) (null-pointer))
+          (field residual) (if residual (tensor-device-pointer residual) (null-pointer))
+          (field ld-residual) n (field stride-residual) 0 (field stride-residual2) 0
+          (field alpha) 1.0 (field reserved) 0))
+  desc)
+
+(defun run-linear (x w b residual out activation)
+  "OUT[rows n] <- act(X[rows k] . W[k n] + B[n]) + RESIDUAL[rows n], one launch (wf2hip_matmul_fused)."
+  (ensure-extension)
+  (with-foreign-object (desc '(:struct matmul-desc))
+    (fill-matmul-desc desc (first (shape x)) (second (shape w)) (second (shape x)) activation b residual)
+    (check (wf2hip-matmul-fused desc (tensor-device-pointer x) (tensor-device-pointer w)
+                                (tensor-device-pointer out))))
+  out)
+
+(defun linear-gradients (x w b dout activation)
+  "dX = dZ W^T, dW = X^T dZ, dB = column sums of dZ, with dZ = dOUT for a plain layer and
+dOUT gelu'(Z), Z = X W + B recomputed, for a GELU layer."
+  (let* ((dz (if (eql activation :gelu)
+                 (!mul dout (gelu-derivative (!add (!matmul x w) (!flexible b))))
+                 dout)))
+    (values (!matmul dz (!t w))
+            (!matmul (!t x) dz)
+            (!reshape (!sum-hip dz :axis 0) (second (shape w))))))
+
+(define-op (HIP-Linear-Node (self activation)
+            :slots ((activation :initform nil :accessor linear-activation))
+            :save-for-backward-names (x w b)
+            :where (X[rows k] W[k n] B[n] OUT[rows n] -> OUT[rows n])
+            :documentation "OUT <- act(X . W + B): MatMulNode, the AddNode of the bias and the
+activation (ACTIVATION nil or :gelu, the tanh form of source/nn/activation.lisp:45-66) as one
+product with an epilogue."
+            :forward ((self x w b out)
+                      (with-setting-save4bw ((x x) (w w) (b b))
+                        (run-linear x w b nil out (linear-activation self))))
+            :backward ((self dout)
+                       (with-reading-save4bw ((x x) (w w) (b b))
+                         (multiple-value-bind (dx dw db) (linear-gradients x w b dout (linear-activation self))
+                           (values (proceed dx) (proceed dw) (proceed db) nil)))))
+  (setf (linear-activation self) activation))
+
+(define-op (HIP-Linear-Residual-Node (self)
+            :save-for-backward-names (x w)
+            :where (X[rows k] W[k n] B[n] R[rows n] OUT[rows n] -> OUT[rows n])
+            :documentation "OUT <- X . W + B + R: the projection that closes a residual branch
+(examples/gpt-2/model.lisp:121-123,134-137) as one product."
+            :forward ((self x w b r out)
+                      (with-setting-save4bw ((x x) (w w))
+                        (run-linear x w b r out nil)))
+            :backward ((self dout)
+                       (with-reading-save4bw ((x x) (w w))
+                         (values (proceed (!matmul dout (!t w)))
+                                 (proceed (!matmul (!t x) dout))
+                                 (proceed (!reshape (!sum-hip dout :axis 0) (second (shape w))))
+                                 dout
+                                 nil)))))
+
+(defun !linear-hip (x w b &key (activation nil) (residual nil))
+  "act(X W + B) + RESIDUAL for X[~ k], W[k n], B[n] on :float device tensors: replaces
+  (asnode #'!matmul w) (asnode #'!add (%transform b[i] -> [~ i])) [(asnode #'!gelu)] [(!add x ..)]
+of examples/gpt-2/model.lisp:109-137 by one node.  Leading axes of X are folded into rows."
+  (let* ((k (car (last (shape x))))
+         (n (second (shape w)))
+         (x2 (!reshape (->contiguous x) t k))
+         (out (make-input (list (first (shape x2)) n) nil :dtype :float :order (order x)))
+         (y (if residual
+                (progn
+                  (assert (null activation) () "!linear-hip: a residual closes a branch without activation")
+                  (call (HIP-Linear-Residual-Node) x2 (->contiguous w) b
+                        (!reshape (->contiguous residual) t n) out))
+                (call (HIP-Linear-Node activation) x2 (->contiguous w) b out))))
+    (apply #'!reshape y `(,@(butlast (shape x)) ,n))))
+
+;; ---- causal softmax and attention -----------------------------------------------------------------
+(define-op (HIP-Causal-Softmax-Node (self scale)
+            :slots ((scale :initform 1.0 :accessor softmax-scale))
+            :save-for-backward-names (y)
+            :where (X[matrices seq seq2] OUT[matrices seq seq2] -> OUT[matrices seq seq2])
+            :documentation "OUT[m, i, :] <- softmax over j <= i of scale X[m, i, j], 0 above the diagonal:
+the MulNode by the scale, the AddNode of the mask and !softmax of causal attention as one kernel
+(wf2hip_causal_softmax_f32) on contiguous square matrices."
+            :forward ((self x out)
+                      (ensure-extension)
+                      (check (wf2hip-causal-softmax-f32 (first (shape x)) (second (shape x))
+                                                        (tensor-device-pointer x) (tensor-device-pointer out)
+                                                        (coerce (softmax-scale self) 'single-float)))
+                      (with-setting-save4bw ((y out)) out))
+            :backward ((self dout)
+                       ;; dx = scale y (dy - sum_j dy y); y is 0 above the diagonal, so is dx
+                       (with-reading-save4bw ((y y))
+                         (let ((dot (!sum-hip (!mul dout y) :axis -1 :keepdims t)))
+                           (values (proceed (!mul (softmax-scale self) (!mul y (!sub dout dot)))) nil)))))
+  (setf (softmax-scale self) scale))
+
+(defun !causal-softmax-hip (scores &key (scale 1.0))
+  "Causal softmax of SCORES[~ seq seq] (any leading axes) times SCALE."
+  (let* ((seq (car (last (shape scores))))
+         (x (!reshape (->contiguous scores) t seq seq))
+         (y (call (HIP-Causal-Softmax-Node scale) x
+                  (make-input (shape x) nil :dtype :float :order (order scores)))))
+    (apply #'!reshape y (shape scores))))
+
+(defun fill-attention-desc (desc q k v out scale causal)
+  (macrolet ((field (name) `(foreign-slot-value desc '(:struct attention-desc) ',name)))
+    (destructuring-bind (batch heads seq head-dim) (shape q)
+      (setf (field batch) batch (field heads) heads (field seq) seq (field head-dim) head-dim
+            (field scale) (coerce scale 'single-float)
+            (field causal) (if causal 1 0))
+      (let ((offsets
+              (loop for tensor in (list q k v out)
+                    for slot in '(q-stride k-stride v-stride o-stride)
+                    collect (multiple-value-bind (extents strides offset) (matrix-geometry tensor)
+                              (declare (ignore extents))
+                              (dotimes (axis 3)
+                                (setf (mem-aref (foreign-slot-pointer desc '(:struct attention-desc) slot) :int64 axis)
+                                      (nth axis strides)))
+                              offset))))
+        offsets))))
+
+(define-op (HIP-Attention-Node (self scale causal)
+            :slots ((scale :initform 1.0 :accessor attention-scale)
+                    (causal :initform nil :accessor attention-causal))
+            :save-for-backward-names (q k v)
+            :where (Q[batch heads seq dim] K[batch heads seq dim] V[batch heads seq dim] OUT[batch heads seq dim]
+                    -> OUT[batch heads seq dim])
+            :documentation "OUT <- softmax(scale Q K^T [+ causal mask]) V per (batch, head) in one kernel that
+never forms the (seq, seq) score matrices (wf2hip_attention_f32; heads up to 64 wide).  The operands may be
+strided windows of a fused projection (last axis contiguous).  Backward: composed, with the
+probabilities recomputed: dV = P^T dO, dP = dO V^T, dS = P (dP - sum_j dP P), dQ = scale dS K,
+dK = scale dS^T Q."
+            :forward ((self q k v out)
+                      (ensure-extension)
+                      (with-foreign-object (desc '(:struct attention-desc))
+                        (destructuring-bind (oq ok ov oo)
+                            (fill-attention-desc desc q k v out (attention-scale self) (attention-causal self))
+                          (check (wf2hip-attention-f32 desc (tensor-device-pointer q oq) (tensor-device-pointer k ok)
+                                                       (tensor-device-pointer v ov) (tensor-device-pointer out oo)))))
+                      (with-setting-save4bw ((q q) (k k) (v v)) out))
+            :backward ((self dout)
+                       (with-reading-save4bw ((q q) (k k) (v v))
+                         (let* ((scale (attention-scale self))
+                                (s (!matmul q (!t k)))
+                                (p (if (attention-causal self)
+                                       (!causal-softmax-hip s :scale scale)
+                                       (!softmax-hip (!reshape (!mul scale s) t (car (last (shape s)))))))
+                                (p (apply #'!reshape p (shape s)))
+                                (dv (!matmul (!t p) dout))
+                                (dp (!matmul dout (!t v)))
+                                (ds (!mul p (!sub dp (!sum-hip (!mul dp p) :axis -1 :keepdims t))))
+                                (dq (!mul scale (!matmul ds k)))
+                                (dk (!mul scale (!matmul (!t ds) q))))
+                           (values (proceed dq) (proceed dk) (proceed dv) nil)))))
+  (setf (attention-scale self) scale
+        (attention-causal self) causal))
+
+(defun !attention-hip (q k v &key (scale nil) (causal nil))
+  "softmax(SCALE Q K^T) V for Q, K, V shaped (batch heads seq head-dim); SCALE defaults to
+1 / sqrt(head-dim).  Replaces the !matmul / !div / !softmax / !matmul chain of SelfAttention
+(examples/gpt-2/utils.lisp:222-243; the example divides by the sequence length and applies no mask:
+pass :scale (/ 1.0 seq) for its numbers, :causal t for a decoder)."
+  (let ((scale (or scale (/ 1.0 (sqrt (coerce (car (last (shape q))) 'single-float))))))
+    (call (HIP-Attention-Node scale causal) q k v
+          (make-input (shape q) nil :dtype :float :order (order q)))))
 
 ;; ---- bypass rules ----------------------------------------------------------------------------
 (define-bypass HIPTensor cl-waffe2/nn:!relu !relu-hip)
@@ -151,3 +426,5 @@ composed recipe."
 (define-bypass HIPTensor cl-waffe2/nn:!sigmoid !sigmoid-hip)
 (define-bypass HIPTensor cl-waffe2/nn:!gelu !gelu-hip)
 (define-bypass HIPTensor cl-waffe2/nn:!softmax !softmax-hip)
+(define-bypass HIPTensor cl-waffe2/base-impl:!sum !sum-hip)
+(define-bypass HIPTensor cl-waffe2/base-impl:!mean !mean-hip)

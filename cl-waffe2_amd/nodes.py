@@ -35,7 +35,9 @@ NODE_NAMES = (
     "Where-Operation-Node", "Compare-Operation-Node",
     "MaxValue-Node", "MinValue-Node", "ArgMax-Node", "ArgMin-Node",
     "Im2ColNode", "Col2ImNode",
-    "HIP-Sum-Node",
+    # the define-op nodes of lisp/fusion.lisp (one kernel each)
+    "HIP-Sum-Node", "HIP-Activation-Node", "HIP-Softmax-Node", "HIP-LayerNorm-Node", "HIP-Linear-Node",
+    "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -465,4 +467,100 @@ def _matmul(a: HIPTensor, b: HIPTensor, out: HIPTensor, trans_a: bool = False,
     for index in itertools.product(*[range(n_) for n_ in outer_shape]):
         launch([o + sum(i * st[ax] for ax, i in enumerate(index)) for o, st in zip(start, tensors)],
                inner, outer)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# the define-op nodes of lisp/fusion.lisp: one kernel per node
+# ---------------------------------------------------------------------------
+
+def _require_rows(what: str, t: HIPTensor, shape=None) -> None:
+    """The row kernels take base pointers and a row count: the tensor must be :float,
+    contiguous and start at its storage (a view would be read or written elsewhere)."""
+    if t.dtype != "float":
+        raise ValueError(f"{what} must be :float, got :{t.dtype}")
+    _, _, off = t.geometry()
+    if not t.is_contiguous() or off != 0:
+        raise ValueError(f"{what} must be a contiguous tensor that starts at its storage; "
+                         "materialise the view with to_contiguous first")
+    if shape is not None and list(t.shape) != list(shape):
+        raise ValueError(f"{what} has shape {t.shape}, expected {list(shape)}")
+
+
+@define_impl("HIP-Activation-Node", HIPTensor, _only_float)
+def _activation_node(x: HIPTensor, out: HIPTensor, op: int, p: float = 0.0) -> HIPTensor:
+    """``X[~] OUT[~] -> OUT[~]``: ReLU / leaky ReLU / sigmoid / GELU as one kernel."""
+    return _run_unary(op, x, out, float(p))
+
+
+@define_impl("HIP-Softmax-Node", HIPTensor, _only_float)
+def _softmax_node(x: HIPTensor, out: HIPTensor) -> HIPTensor:
+    """``X[rows cols] OUT[rows cols] -> OUT``: max-subtracted softmax over the last axis."""
+    _require_rows("HIP-Softmax-Node: x", x)
+    _require_rows("HIP-Softmax-Node: out", out, x.shape)
+    cols = x.shape[-1]
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols, C.c_void_p(out.ptr), cols))
+    return out
+
+
+@define_impl("HIP-LayerNorm-Node", HIPTensor, _only_float)
+def _layernorm_node(x: HIPTensor, g: HIPTensor, b: HIPTensor, out: HIPTensor, eps: float = 1.0e-5) -> HIPTensor:
+    """``X[rows cols] G[cols] B[cols] OUT[rows cols] -> OUT``."""
+    cols = x.shape[-1]
+    _require_rows("HIP-LayerNorm-Node: x", x)
+    _require_rows("HIP-LayerNorm-Node: out", out, x.shape)
+    _require_rows("HIP-LayerNorm-Node: gamma", g, [cols])
+    _require_rows("HIP-LayerNorm-Node: beta", b, [cols])
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_layernorm_rows_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),
+                                                   C.c_void_p(b.ptr), float(eps), C.c_void_p(out.ptr)))
+    return out
+
+
+@define_impl("HIP-Linear-Node", HIPTensor, _only_float)
+def _linear_node(x: HIPTensor, w: HIPTensor, b: HIPTensor, out: HIPTensor, activation: str | None = None) -> HIPTensor:
+    """``X[rows k] W[k n] B[n] OUT[rows n] -> OUT``: act(x . w + b) as one product."""
+    return _matmul(x, w, out, bias=b, activation=activation)
+
+
+@define_impl("HIP-Linear-Residual-Node", HIPTensor, _only_float)
+def _linear_residual_node(x: HIPTensor, w: HIPTensor, b: HIPTensor, r: HIPTensor, out: HIPTensor) -> HIPTensor:
+    """``X[rows k] W[k n] B[n] R[rows n] OUT[rows n] -> OUT``: x . w + b + r as one product."""
+    return _matmul(x, w, out, bias=b, residual=r)
+
+
+@define_impl("HIP-Causal-Softmax-Node", HIPTensor, _only_float)
+def _causal_softmax_node(x: HIPTensor, out: HIPTensor, scale: float = 1.0) -> HIPTensor:
+    """``X[matrices seq seq] OUT[...] -> OUT``: softmax over j <= i of scale x[m, i, j], 0 above the diagonal."""
+    _require_rows("HIP-Causal-Softmax-Node: x", x)
+    _require_rows("HIP-Causal-Softmax-Node: out", out, x.shape)
+    seq = x.shape[-1]
+    if len(x.shape) < 2 or x.shape[-2] != seq:
+        raise ValueError(f"HIP-Causal-Softmax-Node takes square score matrices, got {x.shape}")
+    _lib.check(_lib.get().wf2hip_causal_softmax_f32(x.size // max(seq * seq, 1), seq, C.c_void_p(x.ptr),
+                                                   C.c_void_p(out.ptr), float(scale)))
+    return out
+
+
+@define_impl("HIP-Attention-Node", HIPTensor, _only_float)
+def _attention_node(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor, scale: float,
+                    causal: bool = False) -> HIPTensor:
+    """``Q K V OUT[batch heads seq dim] -> OUT``: softmax(scale q k^T [+ mask]) v in one kernel."""
+    if not (len(q.shape) == 4 and list(q.shape) == list(k.shape) == list(v.shape) == list(out.shape)):
+        raise ValueError("HIP-Attention-Node expects four (batch, heads, seq, head_dim) tensors of one shape")
+    B, H, T, hd = q.shape
+    d = _lib.AttentionDesc()
+    d.batch, d.heads, d.seq, d.head_dim = B, H, T, hd
+    ptrs = []
+    for t, field in ((q, d.q_stride), (k, d.k_stride), (v, d.v_stride), (out, d.o_stride)):
+        _, strides, off = t.geometry()
+        if hd > 1 and strides[3] != 1:
+            raise ValueError("HIP-Attention-Node: the head_dim axis must be contiguous")
+        for a in range(3):
+            field[a] = strides[a]
+        ptrs.append(C.c_void_p(t.ptr + 4 * off))
+    d.scale = float(scale)
+    d.causal = 1 if causal else 0
+    _lib.check(_lib.get().wf2hip_attention_f32(C.byref(d), *ptrs))
     return out

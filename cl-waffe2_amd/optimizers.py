@@ -60,13 +60,28 @@ class Adam:
         self.m = HIPTensor(param.shape)
         self.v = HIPTensor(param.shape)
 
+    @staticmethod
+    def _expt(base: np.float32, power: int) -> np.float32:
+        """``(expt single-float fixnum)``: Common Lisp leaves the algorithm to the
+        implementation; this is exponentiation by squaring in single-float products (what
+        SBCL does), not a binary64 pow rounded once.  The Lisp glue calls the host's own
+        ``expt``, so only this mirror depends on the choice (its last bit is unpinned)."""
+        total = base if power & 1 else np.float32(1.0)
+        power >>= 1
+        while power:
+            base = np.float32(base * base)
+            if power & 1:
+                total = np.float32(base * total)
+            power >>= 1
+        return total
+
     def step_lr(self) -> float:
         """``adam-step-lr`` (adam.lisp:78-92) in single-float arithmetic."""
         self.n += 1
         one = np.float32(1.0)
         b1, b2 = np.float32(self.beta1), np.float32(self.beta2)
-        num = np.sqrt(one - np.float32(math.pow(float(b2), self.n)), dtype=np.float32)
-        den = one - np.float32(math.pow(float(b1), self.n))
+        num = np.sqrt(one - self._expt(b2, self.n), dtype=np.float32)
+        den = one - self._expt(b1, self.n)
         return float(np.float32(self.lr) * (num / den))
 
     def step(self, grad: HIPTensor) -> HIPTensor:

@@ -274,6 +274,30 @@ def test_every_called_binding_is_declared():
     assert used <= declared, sorted(used - declared)
 
 
+def test_every_call_passes_as_many_arguments_as_its_binding_takes():
+    """(wf2hip-foo a b c) in the glue against the defcfun of wf2hip_foo: the same count."""
+    arity = {name.replace("_", "-"): len(classes) for name, (_, classes, _) in defcfuns().items()}
+    calls = 0
+    for f in (x for form in lisp_forms() for x in walk(form)):
+        if f and isinstance(f[0], str) and f[0] in arity:
+            calls += 1
+            assert len(f) - 1 == arity[f[0]], f"({f[0]} ...) is called with {len(f) - 1} arguments, " \
+                                             f"its defcfun takes {arity[f[0]]}"
+    assert calls >= 40
+
+
+def test_nodes_of_the_fused_block_exist_on_both_faces(W):
+    """The define-op nodes of fusion.lisp and the node names the Python mirror dispatches through."""
+    ops = {f[1][0] for form in lisp_forms() for f in walk(form) if f and f[0] == "define-op"}
+    want = {"HIP-Activation-Node", "HIP-Softmax-Node", "HIP-LayerNorm-Node", "HIP-Sum-Node", "HIP-Linear-Node",
+            "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node"}
+    assert want <= ops, want - ops
+    assert want <= set(W.nodes.NODE_NAMES), want - set(W.nodes.NODE_NAMES)
+    bypassed = {f[2] for form in lisp_forms() for f in walk(form) if f and f[0] == "define-bypass"}
+    assert {"cl-waffe2/base-impl:!sum", "cl-waffe2/base-impl:!mean", "cl-waffe2/nn:!softmax",
+            "cl-waffe2/nn:!gelu", "cl-waffe2/nn:!relu"} <= bypassed
+
+
 @pytest.mark.skipif(not os.path.isdir(REFERENCE), reason="the reference checkout is not on this machine")
 def test_internal_symbols_exist_in_the_reference():
     """Symbols the glue reaches with `package::name` are not exported by cl-waffe2, so a
