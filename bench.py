@@ -187,6 +187,79 @@ def counter_probe(W, reps: int = 5):
     print(json.dumps({"probe": "copy, add, mul, exp, rowsum", "launches_each": reps, "elements": N}))
 
 
+def row_probe(W, reps: int = 5):
+    """The launch sequence for `rocprofv3 --pmc` runs of the other kernels of the path: `reps`
+    launches each, in the order printed at the end, every launch on another buffer set (cold
+    cache).  The first case, a plain copy of 2^26 floats, calibrates FETCH_SIZE / WRITE_SIZE."""
+    F = W.functional
+    T = W.HIPTensor
+    rng = np.random.Generator(np.random.PCG64(6))
+    order = []
+
+    def normal(shape, scale=1.0):
+        return T.from_numpy((rng.standard_normal(shape) * scale).astype(np.float32))
+
+    def uniform(shape, lo, hi):
+        return T.from_numpy(rng.uniform(lo, hi, size=shape).astype(np.float32))
+
+    def run(label, nbytes, make, call, launches=1):
+        count = max(2, min(8, -(-(1 << 30) // max(nbytes, 1))))
+        ring = [make() for _ in range(count)]
+        W.lib.synchronize()
+        for i in range(reps):
+            call(ring[i % count])
+        W.lib.synchronize()
+        order.append({"case": label, "launches_per_call": launches, "calls": reps, "algorithmic_bytes": nbytes})
+        ring.clear()
+
+    x0 = normal([N])
+    run("copy 2^26 (calibration)", 8 * N, lambda: (F.copy(x0), T([N], initial_element=None)),
+        lambda s: F.move_(s[1], s[0]))
+    for label, fn, lo, hi in (("exp", F.exp, -10.0, 10.0), ("tanh", F.tanh, -10.0, 10.0),
+                              ("sin", F.sin, -100.0, 100.0), ("loge", F.loge, 1e-3, 1e3)):
+        u0 = uniform([N], lo, hi)
+        run(f"{label} 2^26", 8 * N, lambda: (F.copy(u0), T([N], initial_element=None)),
+            lambda s, fn=fn: fn(s[0], out=s[1]))
+        del u0
+    run("GELU 2^26", 8 * N, lambda: (F.copy(x0), T([N], initial_element=None)), lambda s: F.gelu_fused(s[0], out=s[1]))
+    del x0
+    R, Cn = 4096, 8192
+    a0, b0 = normal([R, Cn]), normal([1, Cn])
+    yb = b0.view((":broadcast", R), True)
+    run("A(4096,8192) += B(1,8192)", 8 * R * Cn + 4 * Cn, lambda: F.copy(a0), lambda s: F.add_(s, yb))
+    run("A[:, ::2] *= 0.5", 8 * R * Cn // 2, lambda: F.copy(a0), lambda s: F.mul_(s.view(True, (0, Cn, 2)), 0.5))
+    run("copy of A[:, ::2]", 8 * R * Cn // 2, lambda: (F.copy(a0), T([R, Cn // 2], initial_element=None)),
+        lambda s: F.move_(s[1], s[0].view(True, (0, Cn, 2))))
+    del a0, b0, yb
+    a0 = normal([SIDE, SIDE])
+    run("transposing copy (8192,8192)", 8 * N, lambda: (F.copy(a0), T([SIDE, SIDE], initial_element=None)),
+        lambda s: F.move_(s[1], s[0].permute(1, 0)))
+    del a0
+    R, Cn = 8192, 4096
+    a0 = normal([R, Cn])
+    run("row sum (8192,4096), one node", 4 * R * Cn + 4 * R, lambda: (F.copy(a0), T([R, 1])),
+        lambda s: F.sum(s[0], axis=1, out=s[1], keepdims=True))
+    run("full sum (8192,4096), one node", 4 * R * Cn, lambda: (F.copy(a0), T([1, 1])),
+        lambda s: F.sum(s[0], axis=True, out=s[1], keepdims=True), launches=2)
+    del a0
+    R, Cn = 32768, 1024
+    a0 = normal([R, Cn], 3.0)
+    run("copy (32768,1024)", 8 * R * Cn, lambda: (F.copy(a0), T([R, Cn], initial_element=None)),
+        lambda s: F.move_(s[1], s[0]))
+    run("row softmax (32768,1024)", 8 * R * Cn, lambda: (F.copy(a0), T([R, Cn], initial_element=None)),
+        lambda s: F.softmax_fused(s[0], out=s[1]))
+    del a0
+    R, Cn = 65536, 1024
+    a0, g0, b0 = normal([R, Cn]), normal([Cn]), normal([Cn])
+    run("LayerNorm (65536,1024)", 8 * R * Cn, lambda: (F.copy(a0), T([R, Cn], initial_element=None)),
+        lambda s: F.layer_norm_fused(s[0], g0, b0, out=s[1]))
+    del a0
+    p0 = normal([N])
+    run("Adam step 2^26", 28 * N, lambda: (W.optimizers.Adam(F.copy(p0), lr=1e-3), F.copy(p0)), lambda s: s[0].step(s[1]))
+    run("SGD step 2^26", 16 * N, lambda: (W.optimizers.SGD(F.copy(p0), lr=1e-3), F.copy(p0)), lambda s: s[0].step(s[1]))
+    print(json.dumps({"probe_rows": order}))
+
+
 def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     """One line per kernel of the path at the shape its configuration names:
     average launch time from an event pair on the library's stream, the
@@ -521,6 +594,8 @@ def main():
                     help="rows: time the eager calls only, no HIP-graph replay (`ms` = `eager_ms`); for kernel traces")
     ap.add_argument("--no-rows", action="store_true",
                     help="skip the table of the other kernels of the path at their configured shapes")
+    ap.add_argument("--probe-rows", action="store_true",
+                    help="run the launch sequence of the other kernels of the path for rocprofv3 --pmc runs and exit")
     ap.add_argument("--probe", action="store_true",
                     help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
@@ -533,6 +608,9 @@ def main():
     info = W.lib.device_info()
     if args.probe:
         counter_probe(W)
+        return
+    if args.probe_rows:
+        row_probe(W)
         return
 
     step_ms, wall_ms, per_kernel, binary_ms, sustained_ms = gpu_steps(W, args.steps, args.warmup)

@@ -10,7 +10,10 @@
  *
  * Conventions
  *   - All data pointers are device pointers obtained from wf2hip_malloc (or
- *     any other HIP allocation of the current device).  fp32 only.
+ *     any other HIP allocation of the current device).  The entry points
+ *     without a dtype argument or prefix take fp32; :double and the integer
+ *     element types have the *_typed entry points and the reference's own
+ *     per-type names (wf2hip_dadd ... wf2hip_u8ge_scal).
  *   - Strides/increments and offsets are in ELEMENTS.  inc == 0 broadcasts.
  *   - Every function returns 0 on success or a negative WF2HIP_E* code / a
  *     positive hipError_t; wf2hip_last_error() returns a thread-local message.
@@ -632,8 +635,9 @@ int wf2hip_sgemm_strided_batched_2d(char transa, char transb, long m, long n, lo
 
 /* The :double product: Fortran dgemm_ with scalars by value, the other branch
  * of the same expansion (matrix-ops.lisp:12-112 picks sgemm_ or dgemm_ by
- * dtype; blas-functions.lisp:34-38).  binary64 FMA on the vector ALUs, one
- * 64 x 64 tile per workgroup; at most 65535 matrices per call. */
+ * dtype; blas-functions.lisp:34-38).  On the binary64 matrix cores
+ * (v_mfma_f64_16x16x4), 128 x 128 (or 64 x 64) x 16 LDS tiles per workgroup; at
+ * most 65535 matrices per call. */
 int wf2hip_dgemm(char transa, char transb, long m, long n, long k, double alpha,
                  const double* A, long lda, const double* B, long ldb, double beta,
                  double* C, long ldc);
