@@ -616,20 +616,50 @@ struct TileParams {
   int64_t d_j;           // dst stride along J   (dst stride along I is 1)
   int64_t s_i;           // src stride along I   (src stride along J is 1)
   uint32_t tiles_i, tiles_j;
+  uint32_t band;         // tiles_i / 8 when that divides, else 0 (see tile_position)
   int32_t nouter;
   uint32_t oshape[kMaxOuter];
   int64_t odst[kMaxOuter];
   int64_t osrc[kMaxOuter];
 };
 
+// Which tile a workgroup takes.  Workgroups go to the eight XCDs round robin
+// (id modulo 8), each with an L2 of its own, so the order is chosen per XCD:
+// XCD x owns the band of tiles_i / 8 tiles x * band .. along I, walks it with I
+// fastest, and steps along J alternately from the two ends towards the middle.
+// The tiles resident on one XCD then read and write runs of band * tile bytes
+// between them, the eight XCDs stay on different parts of every row, and the
+// two column windows in flight keep moving relative to each other instead of
+// sitting a fixed power of two apart.  Transposing copy, 128 x 128 tiles, % of
+// the HBM peak with I fastest over the whole grid -> this order:
+// (8192, 8192) 75.1 -> 79.1, (16384, 4096) 61.8 -> 73.9, (4096, 16384) 71.0 -> 75.0,
+// (8192, 1024) 63.6 -> 74.4, (8192, 3072) 66.6 -> 72.8; 64 x 64 tiles 56.6 -> 71.2.
+// J fastest, 8 x 8 super tiles, bands along J, one contiguous chunk of the
+// linear order per XCD, a per-XCD skew along J and strides of a half or a
+// quarter of tiles_j along J all measured lower.  Without a band (tiles_i not a
+// multiple of 8) the order is I fastest over the whole grid.
+__device__ __forceinline__ void tile_position(const TileParams& p, uint32_t bid, uint32_t& ti, uint32_t& tj,
+                                              uint32_t& rem) {
+  if (p.band != 0) {
+    const uint32_t r = bid >> 3;
+    ti = (bid & 7) * p.band + r % p.band;
+    uint32_t q = r / p.band;
+    rem = q / p.tiles_j;
+    q -= rem * p.tiles_j;
+    tj = (q & 1) ? p.tiles_j - 1 - (q >> 1) : (q >> 1);
+  } else {
+    ti = bid % p.tiles_i;
+    bid /= p.tiles_i;
+    tj = bid % p.tiles_j;
+    rem = bid / p.tiles_j;
+  }
+}
+
 template <class F, bool ReadDst, bool VEC, bool NT = false>
 __global__ __launch_bounds__(kBlock) void ew_tile(TileParams p, F f) {
   __shared__ float tile[kTile][kTile + 1];
-  uint32_t bid = blockIdx.x;
-  const uint32_t ti = bid % p.tiles_i;
-  bid /= p.tiles_i;
-  const uint32_t tj = bid % p.tiles_j;
-  uint32_t rem = bid / p.tiles_j;
+  uint32_t ti, tj, rem;
+  tile_position(p, blockIdx.x, ti, tj, rem);
   int64_t doff = 0, soff = 0;
   for (int i = 0; i < p.nouter; i++) {
     uint32_t q = rem / p.oshape[i];
@@ -698,22 +728,21 @@ __global__ __launch_bounds__(kBlock) void ew_tile(TileParams p, F f) {
 // The same exchange on 128 x 128 tiles for large operands: a workgroup then
 // touches 512 contiguous bytes per row on both sides.  Measured for plain tiled
 // copies of (8192, 8192): 256-byte runs 70 % of the HBM peak, 512-byte runs and
-// longer 80 %.  LDS element (a, b) lives at a * 129 + b + a / 64 + b / 64: with
-// lanes 4 t + k (t = 0..31) along one axis and two rows two apart along the
-// other, both the row-wise writes and the column-wise reads hit 64 distinct banks.
+// longer 80 %.  32 lanes cover a row, a wavefront two neighbouring rows, the
+// workgroup THREADS / 32 rows per pass; LDS element (a, b) lives at a * 129 + b
+// (at most 2-way bank conflicts; the LDS moves 15 % of what it could here).
 constexpr int kBigTile = 128;
 constexpr int kBigTileFloats = kBigTile * (kBigTile + 1) + 4;
 
 template <class F, bool ReadDst, bool NT, int THREADS>
 __global__ __launch_bounds__(THREADS) void ew_tile128(TileParams p, F f) {
-  constexpr int kWaves = THREADS / kWave;  // 4 or 16
-  constexpr int kPasses = 64 / kWaves;     // row groups per wavefront: 16 or 4
+  constexpr int kRowLanes = kBigTile / 4;         // 32 lanes x 4 floats
+  constexpr int kRows = THREADS / kRowLanes;      // rows per pass
+  constexpr int kPasses = kBigTile / kRows;
+  constexpr int kPitch = kBigTile + 1;
   extern __shared__ float big_tile[];
-  uint32_t bid = blockIdx.x;
-  const uint32_t ti = bid % p.tiles_i;
-  bid /= p.tiles_i;
-  const uint32_t tj = bid % p.tiles_j;
-  uint32_t rem = bid / p.tiles_j;
+  uint32_t ti, tj, rem;
+  tile_position(p, blockIdx.x, ti, tj, rem);
   int64_t doff = 0, soff = 0;
   for (int i = 0; i < p.nouter; i++) {
     uint32_t q = rem / p.oshape[i];
@@ -724,54 +753,42 @@ __global__ __launch_bounds__(THREADS) void ew_tile128(TileParams p, F f) {
   }
   const int64_t i0 = (int64_t)ti * kBigTile;
   const int64_t j0 = (int64_t)tj * kBigTile;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  const int q4 = (lane & 31) * 4;       // position along the contiguous axis
-  const int rr = 2 * (lane >> 5);       // the two half-waves take rows two apart
-  auto row_of = [&](int pass) {         // rows 4 (g / 2) + g % 2 + {0, 2}, g = kWaves pass + wave in 0..63
-    const int g = kWaves * pass + wave;
-    return 4 * (g >> 1) + (g & 1) + rr;
-  };
-  auto at = [](int a, int b) { return a * (kBigTile + 1) + b + (a >> 6) + (b >> 6); };
+  const int q4 = (threadIdx.x % kRowLanes) * 4;  // position along the contiguous axis
+  const int r0 = threadIdx.x / kRowLanes;        // row within a pass
   f4 v[kPasses];
 #pragma unroll
   for (int pass = 0; pass < kPasses; pass++) {
-    const int r = row_of(pass);
-    const int64_t i = i0 + r, j = j0 + q4;
+    const int64_t i = i0 + r0 + pass * kRows, j = j0 + q4;
     v[pass] = f4{0.f, 0.f, 0.f, 0.f};
     if (i < p.ni && j < p.nj) v[pass] = load4<NT>(p.src + soff + i * p.s_i + j);
   }
 #pragma unroll
   for (int pass = 0; pass < kPasses; pass++) {
-    const int r = row_of(pass);
-    big_tile[at(r, q4 + 0)] = v[pass].x;
-    big_tile[at(r, q4 + 1)] = v[pass].y;
-    big_tile[at(r, q4 + 2)] = v[pass].z;
-    big_tile[at(r, q4 + 3)] = v[pass].w;
+    float* t = big_tile + (r0 + pass * kRows) * kPitch + q4;
+    t[0] = v[pass].x;
+    t[1] = v[pass].y;
+    t[2] = v[pass].z;
+    t[3] = v[pass].w;
   }
   __syncthreads();
+  f4 a[kPasses];
 #pragma unroll
-  for (int batch = 0; batch < kPasses / 4; batch++) {
-    f4 a[4];
+  for (int pass = 0; pass < kPasses; pass++) {
+    const int64_t i = i0 + q4, j = j0 + r0 + pass * kRows;
+    a[pass] = f4{0.f, 0.f, 0.f, 0.f};
+    if (ReadDst && i < p.ni && j < p.nj) a[pass] = load4<NT>(p.dst + doff + j * p.d_j + i);
+  }
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int r = row_of(4 * batch + u);
-      const int64_t i = i0 + q4, j = j0 + r;
-      a[u] = f4{0.f, 0.f, 0.f, 0.f};
-      if (ReadDst && i < p.ni && j < p.nj) a[u] = load4<NT>(p.dst + doff + j * p.d_j + i);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const int r = row_of(4 * batch + u);
-      const int64_t i = i0 + q4, j = j0 + r;
-      if (i < p.ni && j < p.nj) {
-        f4 o;
-        o.x = f(a[u].x, big_tile[at(q4 + 0, r)]);
-        o.y = f(a[u].y, big_tile[at(q4 + 1, r)]);
-        o.z = f(a[u].z, big_tile[at(q4 + 2, r)]);
-        o.w = f(a[u].w, big_tile[at(q4 + 3, r)]);
-        store4<NT>(p.dst + doff + j * p.d_j + i, o);
-      }
+  for (int pass = 0; pass < kPasses; pass++) {
+    const int r = r0 + pass * kRows;
+    const int64_t i = i0 + q4, j = j0 + r;
+    if (i < p.ni && j < p.nj) {
+      f4 o;
+      o.x = f(a[pass].x, big_tile[(q4 + 0) * kPitch + r]);
+      o.y = f(a[pass].y, big_tile[(q4 + 1) * kPitch + r]);
+      o.z = f(a[pass].z, big_tile[(q4 + 2) * kPitch + r]);
+      o.w = f(a[pass].w, big_tile[(q4 + 3) * kPitch + r]);
+      store4<NT>(p.dst + doff + j * p.d_j + i, o);
     }
   }
 }
@@ -958,6 +975,7 @@ static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, i
   p.s_i = s.sb[last];
   p.tiles_i = (uint32_t)ceil_div(p.ni, kTile);
   p.tiles_j = (uint32_t)ceil_div(p.nj, kTile);
+  p.band = p.tiles_i % 8 == 0 ? p.tiles_i / 8 : 0;
   p.nouter = 0;
   int64_t blocks = (int64_t)p.tiles_i * p.tiles_j;
   for (int r = last - 1; r >= 0; r--) {
@@ -977,6 +995,7 @@ static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, i
   if (vec && p.ni >= kBigTile && p.nj >= kBigTile && s.total >= ((int64_t)1 << 22)) {
     p.tiles_i = (uint32_t)ceil_div(p.ni, kBigTile);
     p.tiles_j = (uint32_t)ceil_div(p.nj, kBigTile);
+    p.band = p.tiles_i % 8 == 0 ? p.tiles_i / 8 : 0;
     int64_t big_blocks = (int64_t)p.tiles_i * p.tiles_j;
     for (int i = 0; i < p.nouter; i++) big_blocks *= p.oshape[i];
     int lrc = streaming ? launch_tile128<F, ReadDst, true>(p, (uint32_t)big_blocks, f)

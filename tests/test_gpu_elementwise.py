@@ -244,8 +244,11 @@ def test_large_transposed_operands(gpu):
     W = gpu
     F = W.functional
     rng = np.random.default_rng(128)
+    # the last three have a multiple of 8 tiles along the destination's contiguous axis, where
+    # the tiles are handed out in bands (128 x 128 tiles twice, 64 x 64 tiles once)
     for shape, order in [((2052, 2060), (1, 0)), ((3, 1100, 1284), (0, 2, 1)), ((2, 3, 1028, 1032), (0, 1, 3, 2)),
-                         ((1284, 5, 1100), (2, 1, 0))]:
+                         ((1284, 5, 1100), (2, 1, 0)), ((2048, 2100), (1, 0)), ((2, 2040, 1100), (0, 2, 1)),
+                         ((3, 1020, 1100), (0, 2, 1))]:
         x = rng.standard_normal(shape).astype(np.float32)
         xt = np.transpose(x, order)
         dx = F.from_numpy(x)
