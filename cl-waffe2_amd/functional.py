@@ -699,3 +699,76 @@ def layer_norm_backward(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float 
     dg = sum(mul(d2, xh), axis=0)
     db = sum(d2, axis=0)
     return HIPTensor(x.shape, vec=dx.vec), reshape(dg, cols), reshape(db, cols)
+
+
+# ---------------------------------------------------------------------------
+# backward of the fused nodes, composed the way the :backward bodies of the Lisp glue
+# (lisp/fusion.lisp) compose them: the same node sequences, so the float64 checks of
+# these functions are checks of those formulas
+# ---------------------------------------------------------------------------
+
+def gelu_derivative(x: HIPTensor) -> HIPTensor:
+    """d/dx of 0.5 x (1 + tanh u), u = c (x + a x^3): 0.5 (1 + t) + 0.5 x (1 - t^2) c (1 + 3 a x^2)
+    (``gelu-derivative`` of the Lisp glue; the recipe of ``source/nn/activation.lisp:45-66``
+    differentiated)."""
+    c = float(np.float32(math.sqrt(2.0 / math.pi)))
+    a = 0.044715
+    x2 = mul(x, x)
+    u = mul(add(x, mul(mul(x2, x), a)), c)
+    th = tanh(u)
+    du = mul(add(mul(x2, 3 * a), 1.0), c)
+    left = mul(add(th, 1.0), 0.5)
+    right = mul(mul(x, 0.5), mul(sub(1.0, mul(th, th)), du))
+    return add_(left, right)
+
+
+def linear_backward(x: HIPTensor, w: HIPTensor, b: HIPTensor, dout: HIPTensor, activation: str | None = None):
+    """(dx, dw, db) of ``act(x . w + b)`` (HIP-Linear-Node, and HIP-Linear-Residual-Node whose
+    residual passes ``dout`` through unchanged): dX = dZ W^T, dW = X^T dZ, dB = column sums of
+    dZ, with dZ = dOUT for a plain layer and dOUT gelu'(Z), Z = X W + B recomputed, for a GELU
+    layer (``linear-gradients`` of the Lisp glue; MatMulNode's backward,
+    ``base-impl/matrix-ops.lisp:10-15``)."""
+    k, n = x.shape[-1], w.shape[-1]
+    x2, d2 = reshape(x, -1, k), reshape(dout, -1, n)
+    if activation == "gelu":
+        z = add_(matmul(x2, w), b)
+        dz = mul_(gelu_derivative(z), d2)
+    elif activation is None:
+        dz = d2
+    else:
+        raise ValueError("linear_backward: activation must be None or 'gelu'")
+    dx = matmul(dz, t(w))
+    dw = matmul(t(x2), dz)
+    db = reshape(sum(dz, axis=0), n)
+    return HIPTensor(list(x.shape), vec=dx.vec), dw, db
+
+
+def softmax_backward(y: HIPTensor, dout: HIPTensor, scale: float = 1.0) -> HIPTensor:
+    """dx = scale y (dy - sum_j dy y) over the last axis, from the saved output y
+    (HIP-Softmax-Node, and HIP-Causal-Softmax-Node whose y is 0 above the diagonal)."""
+    dot = sum(mul(dout, y), axis=-1, keepdims=True)
+    dx = mul_(sub(dout, dot), y)
+    return dx if scale == 1.0 else mul_(dx, float(scale))
+
+
+def attention_backward(q: HIPTensor, k: HIPTensor, v: HIPTensor, dout: HIPTensor, scale: float | None = None,
+                       causal: bool = False, dq: HIPTensor | None = None, dk: HIPTensor | None = None,
+                       dv: HIPTensor | None = None):
+    """(dq, dk, dv) of HIP-Attention-Node with the probabilities recomputed, as its :backward
+    composes them: P = softmax(scale Q K^T [+ mask]), dV = P^T dO, dP = dO V^T,
+    dS = P (dP - sum_j dP P), dQ = scale dS K, dK = scale dS^T Q.  Operands are
+    (batch, heads, seq, head_dim) views whose last axis is contiguous; the optional outputs may be
+    such views too (windows of one fused-projection gradient)."""
+    hd = q.shape[-1]
+    scale = 1.0 / math.sqrt(hd) if scale is None else float(scale)
+    s = matmul(q, t(k))
+    if causal:
+        p = causal_softmax_fused(s, scale)
+    else:
+        p = reshape(softmax_fused(reshape(mul_(s, scale), -1, s.shape[-1])), *s.shape)
+    dv = matmul(t(p), dout, out=dv)
+    dp = matmul(dout, t(v))
+    ds = softmax_backward(p, dp)
+    dq = mul_(matmul(ds, k, out=dq), scale)
+    dk = mul_(matmul(t(ds), q, out=dk), scale)
+    return dq, dk, dv

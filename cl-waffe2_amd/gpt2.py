@@ -77,7 +77,9 @@ def _linear(x: HIPTensor, w: HIPTensor, b: HIPTensor) -> HIPTensor:
 
 
 def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG,
-                  mask: HIPTensor | None = None) -> HIPTensor:
+                  mask: HIPTensor | None = None, saved: dict | None = None) -> HIPTensor:
+    """`saved`, when given (mode 'fused' only), receives what the fused nodes keep for their
+    backward (their inputs: ``:save-for-backward-names`` of the Lisp nodes) for `block_backward`."""
     B, T, D = x.shape
     H = cfg["n_head"]
     hd = D // H
@@ -134,6 +136,10 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         x1 = F.linear(ctx, p["w_o"], p["b_o"], residual=x)
         h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)
         f = F.linear(h2, p["w_fc"], p["b_fc"], activation="gelu")
+        if saved is not None:
+            if mode != "fused":
+                raise ValueError("block_forward: saved tensors are kept for mode 'fused'")
+            saved.update(x=x, h=h, qkv=qkv, ctx=ctx, x1=x1, h2=h2, f=f)
         return F.linear(f, p["w_proj"], p["b_proj"], residual=x1)
     attn = _linear(ctx, p["w_o"], p["b_o"])
     x1 = F.add(x, attn)                                             # residual
@@ -141,3 +147,39 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
     f = act(_linear(h2, p["w_fc"], p["b_fc"]))
     m = _linear(f, p["w_proj"], p["b_proj"])
     return F.add_(m, x1)                                            # residual, in place in m
+
+
+def block_backward(dout: HIPTensor, saved: dict, p: dict, cfg: dict = CONFIG):
+    """Gradients of the fused block from what `block_forward(..., saved=...)` kept: every fused
+    node's backward in reverse order, composed as the Lisp nodes compose theirs (HIP-Linear-Node,
+    HIP-Linear-Residual-Node, HIP-LayerNorm-Node, HIP-Attention-Node with the probabilities
+    recomputed), the gradient adders of the two residual forks as AddNodes.  Returns (dx, grads)
+    with `grads` keyed like the parameters."""
+    x, h, qkv, ctx, x1, h2, f = (saved[k] for k in ("x", "h", "qkv", "ctx", "x1", "h2", "f"))
+    B, T, D = x.shape
+    H = cfg["n_head"]
+    hd = D // H
+    eps = cfg["eps"]
+    g = {}
+    # out = f . w_proj + b_proj + x1
+    df, g["w_proj"], g["b_proj"] = F.linear_backward(f, p["w_proj"], p["b_proj"], dout)
+    # f = gelu(h2 . w_fc + b_fc)
+    dh2, g["w_fc"], g["b_fc"] = F.linear_backward(h2, p["w_fc"], p["b_fc"], df, activation="gelu")
+    # h2 = LayerNorm(x1); x1 also feeds the residual
+    dln2, g["ln2_g"], g["ln2_b"] = F.layer_norm_backward(x1, p["ln2_g"], dh2, eps)
+    dx1 = F.add_(dln2, dout)
+    # x1 = ctx . w_o + b_o + x
+    dctx, g["w_o"], g["b_o"] = F.linear_backward(ctx, p["w_o"], p["b_o"], dx1)
+    # ctx = attention(q, k, v), heads read in place from the projection, their gradients
+    # written in place into the projection's gradient
+    four = F.reshape(qkv, B, T, 3 * H, hd)
+    q, k, v = (four.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3) for i in range(3))
+    dqkv = HIPTensor([B, T, 3 * H, hd], initial_element=None)
+    dq, dk, dv = (dqkv.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3) for i in range(3))
+    dctx_heads = F.reshape(dctx, B, T, H, hd).permute(0, 2, 1, 3)
+    F.attention_backward(q, k, v, dctx_heads, scale=1.0 / math.sqrt(hd), causal=True, dq=dq, dk=dk, dv=dv)
+    # qkv = h . w_qkv + b_qkv
+    dh, g["w_qkv"], g["b_qkv"] = F.linear_backward(h, p["w_qkv"], p["b_qkv"], F.reshape(dqkv, B, T, 3 * D))
+    # h = LayerNorm(x); x also feeds the residual
+    dln1, g["ln1_g"], g["ln1_b"] = F.layer_norm_backward(x, p["ln1_g"], dh, eps)
+    return F.add_(dln1, dx1), g

@@ -1,0 +1,91 @@
+"""Backward of the fused transformer block on the device against the float64 backward.
+
+The device side composes every fused node's backward the way the Lisp nodes do (products through
+the transposed layouts, GELU and attention probabilities recomputed, LayerNorm gradients from the
+saved input).  Tolerance: each gradient is held to 1e-5 times the magnitude its last product or sum
+adds up (sum |a||b|, computed by the float64 reference) -- the bar of the products themselves."""
+import importlib
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(cfg, seed, plain_params=False):
+    gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
+    params = gpt2.make_block_params(seed, cfg)
+    rng = np.random.default_rng(seed)
+    if not plain_params:
+        for k in params:
+            if k.startswith("b_") or k.endswith("_b"):
+                params[k] = (rng.standard_normal(params[k].shape) * 0.1).astype(np.float32)
+            if k.endswith("_g"):
+                params[k] = (1 + rng.standard_normal(params[k].shape) * 0.1).astype(np.float32)
+    x = gpt2.make_block_input(seed, cfg)
+    dout = rng.standard_normal(x.shape).astype(np.float32)
+    return gpt2, params, x, dout
+
+
+def _check(W, cfg, seed, bar, plain_params=False):
+    from oracle import gpt2_block_ref as ref
+    gpt2, params, x, dout = _setup(cfg, seed, plain_params)
+    want, scales = ref.block_backward(x, params, cfg["n_head"], dout, cfg["eps"])
+    dp = gpt2.to_device(params)
+    saved = {}
+    out = gpt2.block_forward(W.HIPTensor.from_numpy(x), dp, mode="fused", cfg=cfg, saved=saved)
+    fwd = ref.block_forward(x, params, cfg["n_head"], cfg["eps"])
+    np.testing.assert_allclose(out.numpy(), fwd, rtol=2e-4, atol=2e-4)
+    dx, grads = gpt2.block_backward(W.HIPTensor.from_numpy(dout), saved, dp, cfg=cfg)
+    got = {k: v.numpy() for k, v in grads.items()}
+    got["x"] = dx.numpy()
+    assert sorted(got) == sorted(want)
+    worst = {}
+    for name in sorted(want):
+        assert got[name].shape == want[name].shape, name
+        ratio = np.abs(got[name] - want[name]) / np.maximum(scales[name], 1e-30)
+        worst[name] = float(ratio.max())
+    print("worst error / (sum |a||b| of the forming product):", {k: f"{v:.2e}" for k, v in worst.items()}, flush=True)
+    for name, r in worst.items():
+        assert r <= bar, (name, r)
+
+
+def test_block_backward_small(gpu):
+    _check(gpu, dict(batch=2, seq=48, d_model=96, n_head=3, head_dim=32, d_ff=384, eps=1e-5), 21, 1e-5)
+
+
+def test_block_backward_ragged(gpu):
+    _check(gpu, dict(batch=3, seq=50, d_model=60, n_head=5, head_dim=12, d_ff=100, eps=1e-5), 22, 1e-5)
+
+
+def test_block_backward_config5_shapes(gpu):
+    """benchmark configuration 5's widths (T 1024, D 768, 12 heads x 64, d_ff 3072) on two sequences."""
+    _check(gpu, dict(batch=2, seq=1024, d_model=768, n_head=12, head_dim=64, d_ff=3072, eps=1e-5), 5, 1e-5,
+           plain_params=True)
+
+
+def test_attention_backward_full_and_causal(gpu):
+    """HIP-Attention-Node's backward composition alone, both mask forms, against float64."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(31)
+    B, H, T, hd = 2, 3, 70, 16
+    q, k, v, do = (rng.standard_normal((B, H, T, hd)).astype(np.float32) for _ in range(4))
+    for causal in (False, True):
+        Q, K, V, DO = (a.astype(np.float64) for a in (q, k, v, do))
+        sc = 1.0 / np.sqrt(hd)
+        s = Q @ K.transpose(0, 1, 3, 2) * sc
+        if causal:
+            s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+        e = np.exp(s - s.max(-1, keepdims=True))
+        p = e / e.sum(-1, keepdims=True)
+        dv = p.transpose(0, 1, 3, 2) @ DO
+        dp = DO @ V.transpose(0, 1, 3, 2)
+        ds = p * (dp - (dp * p).sum(-1, keepdims=True))
+        dq, dk = ds @ K * sc, ds.transpose(0, 1, 3, 2) @ Q * sc
+        gq, gk, gv = F.attention_backward(*(F.from_numpy(a) for a in (q, k, v, do)), causal=causal)
+        for name, got, want, mag in (("dq", gq, dq, np.abs(ds) @ np.abs(K) * sc),
+                                     ("dk", gk, dk, np.abs(ds).transpose(0, 1, 3, 2) @ np.abs(Q) * sc),
+                                     ("dv", gv, dv, p.transpose(0, 1, 3, 2) @ np.abs(DO))):
+            ratio = np.abs(got.numpy() - want) / np.maximum(mag, 1e-30)
+            assert ratio.max() <= 1e-5, (causal, name, ratio.max())
