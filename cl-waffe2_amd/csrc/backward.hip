@@ -1,0 +1,356 @@
+// backward.hip -- the row kernels of the backward pass: softmax (plain and causal)
+// and LayerNorm gradients, each one pass over its rows.
+//
+// cl-waffe2 differentiates these layers through their node compositions
+// (source/nn/activation.lisp:126-159, source/nn/norms.lisp:72-82): some twenty
+// element-wise and reduction passes per layer.  Here a wavefront holds the row of
+// the saved tensor and the row of the upstream gradient in registers, forms the
+// row statistics with shuffles and writes the gradient once:
+//   softmax    dx = scale y (dy - sum_j dy y)                      12 bytes per element
+//   LayerNorm  dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),      12 bytes per element
+//              dgamma = sum_rows dy xh, dbeta = sum_rows dy         (+ the partial sums)
+// with xh = (x - mean) rstd and dyh = dy gamma.  Both are HBM-bound.
+#include <algorithm>
+
+#include "wf2_common.h"
+#include "wf2_rows.h"
+
+namespace wf2 {
+
+__device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- softmax ------------------------------------------------------------------------------------
+// One wavefront per row.  With causal_seq > 0 row r holds (r % causal_seq) + 1 entries:
+// what lies above the diagonal is neither read (dy may be uninitialised there, e.g. the
+// skipped tiles of a triangular product) nor left unwritten (dx is 0 there).
+template <int NV, bool VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_rows_wave(const float* __restrict__ y, int64_t ldy,
+                                                                const float* __restrict__ dy, int64_t lddy,
+                                                                float* __restrict__ dx, int64_t lddx,
+                                                                int64_t nrows, int64_t ncols, int64_t causal_seq,
+                                                                float scale) {
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row >= nrows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
+  RowRegs<NV, VEC, NT> a, b;
+  a.load(y + row * ldy, valid, lane, 0.0f);
+  b.load(dy + row * lddy, valid, lane, 0.0f);
+  float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int g = 0; g < NV; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) part[c] = __builtin_fmaf(b.v[g][c], a.v[g][c], part[c]);
+  const float dot = (float)wave_sum(((double)part[0] + (double)part[1]) + ((double)part[2] + (double)part[3]));
+#pragma unroll
+  for (int g = 0; g < NV; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const bool in = RowRegs<NV, VEC, NT>::col(g, c, lane) < valid;
+      const float t = scale * (a.v[g][c] * (b.v[g][c] - dot));
+      a.v[g][c] = in ? t : 0.0f;
+    }
+  a.store(dx + row * lddx, ncols, lane);
+}
+
+// Rows beyond the register tile: a workgroup per row, two passes (the second one from the L2).
+__global__ __launch_bounds__(kBlock) void softmax_bwd_rows_block(const float* __restrict__ y, int64_t ldy,
+                                                                 const float* __restrict__ dy, int64_t lddy,
+                                                                 float* __restrict__ dx, int64_t lddx,
+                                                                 int64_t ncols, int64_t causal_seq, float scale) {
+  __shared__ double lds[kWavesPerBlock];
+  __shared__ float stat;
+  const int64_t row = blockIdx.x;
+  const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
+  const float* yr = y + row * ldy;
+  const float* dr = dy + row * lddy;
+  float* xr = dx + row * lddx;
+  double acc = 0.0;
+  for (int64_t c = threadIdx.x; c < valid; c += kBlock) acc += (double)(dr[c] * yr[c]);
+  const double total = block_sum(acc, lds);
+  if (threadIdx.x == 0) stat = (float)total;
+  __syncthreads();
+  const float dot = stat;
+  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) xr[c] = c < valid ? scale * (yr[c] * (dr[c] - dot)) : 0.0f;
+}
+
+template <bool VEC, bool NT>
+static int launch_softmax_bwd(int nv, const float* y, int64_t ldy, const float* dy, int64_t lddy, float* dx,
+                              int64_t lddx, int64_t nrows, int64_t ncols, int64_t causal_seq, float scale) {
+  const uint32_t blocks = (uint32_t)ceil_div(nrows, kWavesPerBlock);
+  hipStream_t st = rt().stream;
+#define WF2_CASE(N)                                                                                            \
+  case N:                                                                                                      \
+    softmax_bwd_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, nrows, ncols,      \
+                                                                 causal_seq, scale);                           \
+    break;
+  switch (nv) {
+    WF2_CASE(1)
+    WF2_CASE(2)
+    WF2_CASE(3)
+    WF2_CASE(4)
+    WF2_CASE(6)
+    WF2_CASE(8)
+    default: return fail(WF2HIP_EINVAL, "bad register tile");
+  }
+#undef WF2_CASE
+  return after_launch("softmax_bwd_rows_wave");
+}
+
+// ---- LayerNorm ----------------------------------------------------------------------------------
+// A wavefront walks rows wave, wave + W, wave + 2 W, ... (W = wavefronts of the grid, so that
+// the grid reads a contiguous band of rows at a time), keeps gamma and its share of the two
+// column sums in registers, and the four wavefronts of a workgroup fold their shares through
+// LDS into one row of `partial` ([workgroup][2][ncols]: dgamma, then dbeta); two small kernels
+// then add the workgroups' rows in binary64.  Row statistics as in the forward kernel: the
+// mean from binary64 sums, deviations and squares in binary32 with four partial sums per lane.
+template <int NV, bool VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_rows(const float* __restrict__ x,
+                                                             const float* __restrict__ gamma,
+                                                             const float* __restrict__ dy, float eps,
+                                                             float* __restrict__ dx, float* __restrict__ partial,
+                                                             int64_t nrows, int64_t ncols) {
+  __shared__ float fold[kWavesPerBlock][NV * kWave * 4];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t stride = (int64_t)gridDim.x * kWavesPerBlock;
+  RowRegs<NV, VEC, false> g;
+  g.load(gamma, ncols, lane, 0.0f);
+  float dg[NV][4], db[NV][4];
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) dg[i][c] = db[i][c] = 0.0f;
+  const float inv_n = 1.0f / (float)ncols;
+  // the loads of the wavefront's next row are issued before the arithmetic of this one
+  int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  RowRegs<NV, VEC, NT> xr, dr, xn, dn;
+  if (row < nrows) {
+    xr.load(x + row * ncols, ncols, lane, 0.0f);
+    dr.load(dy + row * ncols, ncols, lane, 0.0f);
+  }
+  for (; row < nrows; row += stride) {
+    const int64_t next = row + stride < nrows ? row + stride : row;  // the last row again: loaded, not used
+    xn.load(x + next * ncols, ncols, lane, 0.0f);
+    dn.load(dy + next * ncols, ncols, lane, 0.0f);
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) sum += (double)xr.v[i][c];
+    const float mean = (float)(wave_sum(sum) / (double)ncols);
+    float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const bool in = RowRegs<NV, VEC, NT>::col(i, c, lane) < ncols;
+        const float d = in ? xr.v[i][c] - mean : 0.0f;
+        xr.v[i][c] = d;
+        sq[c] = __builtin_fmaf(d, d, sq[c]);
+      }
+    const double var = wave_sum(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3])) / (double)ncols;
+    const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
+    // xh, dyh and the two row means
+    float s1[2] = {0.0f, 0.0f}, s2[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float xh = xr.v[i][c] * rstd;
+        const float d = dr.v[i][c];
+        xr.v[i][c] = xh;
+        dg[i][c] = __builtin_fmaf(d, xh, dg[i][c]);
+        db[i][c] += d;
+        const float dyh = d * g.v[i][c];
+        dr.v[i][c] = dyh;
+        s1[c & 1] += dyh;
+        s2[c & 1] = __builtin_fmaf(dyh, xh, s2[c & 1]);
+      }
+    const float m1 = (float)wave_sum((double)s1[0] + (double)s1[1]) * inv_n;
+    const float m2 = (float)wave_sum((double)s2[0] + (double)s2[1]) * inv_n;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) dr.v[i][c] = rstd * ((dr.v[i][c] - m1) - xr.v[i][c] * m2);
+    dr.store(dx + row * ncols, ncols, lane);
+    xr = xn;
+    dr = dn;
+  }
+  // fold the four wavefronts' column sums, dgamma first, then dbeta through the same LDS
+#pragma unroll
+  for (int which = 0; which < 2; which++) {
+    if (which == 1) __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int64_t cc = RowRegs<NV, VEC, NT>::col(i, c, lane);
+        fold[wave][cc] = which == 0 ? dg[i][c] : db[i][c];
+      }
+    __syncthreads();
+    float* out = partial + ((int64_t)blockIdx.x * 2 + which) * ncols;
+    for (int64_t cc = threadIdx.x; cc < ncols; cc += kBlock)
+      out[cc] = (fold[0][cc] + fold[1][cc]) + (fold[2][cc] + fold[3][cc]);
+  }
+}
+
+// Column sums of the workgroups' rows in two small steps, so that the first has enough
+// workgroups to pull the few megabytes of `partial` at speed: the rows are cut into kFoldGroups
+// groups; workgroup (x, g) adds the rows of group g for 64 of the 2 ncols columns (its four
+// wavefronts take every fourth row, eight loads in flight each) into level2[g][.] in binary64;
+// the second step adds the kFoldGroups rows of level2 and rounds once.
+constexpr int kFoldGroups = 16;
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_fold1(const float* __restrict__ partial, int64_t nparts,
+                                                              int64_t width, double* __restrict__ level2) {
+  __shared__ double lds[kWavesPerBlock][kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t col = (int64_t)blockIdx.x * kWave + lane;  // 0 .. width - 1, width = 2 ncols
+  const int64_t per = ceil_div_dev(nparts, kFoldGroups);
+  const int64_t first = (int64_t)blockIdx.y * per;
+  const int64_t last = first + per < nparts ? first + per : nparts;
+  double acc = 0.0;
+  if (col < width) {
+    int64_t w = first + wave;
+    for (; w + 7 * kWavesPerBlock < last; w += 8 * kWavesPerBlock) {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) t[u] = partial[(w + u * kWavesPerBlock) * width + col];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc += (double)t[u];
+    }
+    for (; w < last; w += kWavesPerBlock) acc += (double)partial[w * width + col];
+  }
+  lds[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && col < width)
+    level2[(int64_t)blockIdx.y * width + col] = (lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane]);
+}
+
+__global__ __launch_bounds__(kWave) void layernorm_bwd_fold2(const double* __restrict__ level2, int64_t ncols,
+                                                             float* __restrict__ dgamma, float* __restrict__ dbeta) {
+  const int64_t col = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  if (col >= 2 * ncols) return;
+  double t[kFoldGroups];
+#pragma unroll
+  for (int g = 0; g < kFoldGroups; g++) t[g] = level2[(int64_t)g * 2 * ncols + col];
+  double acc = 0.0;
+#pragma unroll
+  for (int g = 0; g < kFoldGroups; g++) acc += t[g];
+  if (col < ncols)
+    dgamma[col] = (float)acc;
+  else
+    dbeta[col - ncols] = (float)acc;
+}
+
+template <bool VEC, bool NT>
+static int launch_layernorm_bwd(int nv, uint32_t blocks, const float* x, const float* gamma, const float* dy,
+                                float eps, float* dx, float* partial, int64_t nrows, int64_t ncols) {
+  hipStream_t st = rt().stream;
+#define WF2_CASE(N)                                                                                              \
+  case N:                                                                                                        \
+    layernorm_bwd_rows<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, gamma, dy, eps, dx, partial, nrows, ncols);      \
+    break;
+  switch (nv) {
+    WF2_CASE(1)
+    WF2_CASE(2)
+    WF2_CASE(3)
+    WF2_CASE(4)
+    WF2_CASE(6)
+    WF2_CASE(8)
+    default: return fail(WF2HIP_EUNSUPPORTED, "LayerNorm backward: rows longer than 2048 are not built");
+  }
+#undef WF2_CASE
+  return after_launch("layernorm_bwd_rows");
+}
+
+}  // namespace wf2
+
+using namespace wf2;
+
+WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* y, long ldy, const float* dy,
+                                             long lddy, float* dx, long lddx, float scale, long causal_seq) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0 || causal_seq < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if (rows == 0 || cols == 0) return 0;
+  if (!y || !dy || !dx) return fail(WF2HIP_EINVAL, "null pointer");
+  if (ldy < cols || lddy < cols || lddx < cols) return fail(WF2HIP_EINVAL, "row pitch smaller than the row");
+  if (causal_seq > 0 && causal_seq != cols)
+    return fail(WF2HIP_EINVAL, "causal softmax backward takes square (seq, seq) matrices: cols %ld, seq %ld", cols,
+                causal_seq);
+  if (rows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+  // dx may be dy (in place, row by row) but must not overlap anything else
+  const float* ylo = y;
+  const float* yhi = y + (rows - 1) * (int64_t)ldy + cols;
+  const float* dlo = dy;
+  const float* dhi = dy + (rows - 1) * (int64_t)lddy + cols;
+  const float* xlo = dx;
+  const float* xhi = dx + (rows - 1) * (int64_t)lddx + cols;
+  if (xlo < yhi && ylo < xhi) return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps y");
+  if (xlo < dhi && dlo < xhi && !(dx == dy && lddx == lddy))
+    return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps dy without being dy");
+  int nv = pick_nv(cols);
+  if (nv == 0 || nv > 8) {
+    softmax_bwd_rows_block<<<(uint32_t)rows, kBlock, 0, rt().stream>>>(y, ldy, dy, lddy, dx, lddx, cols, causal_seq,
+                                                                     scale);
+    return after_launch("softmax_bwd_rows_block");
+  }
+  const bool vec = aligned16(y) && aligned16(dy) && aligned16(dx) && ldy % 4 == 0 && lddy % 4 == 0 && lddx % 4 == 0;
+  const bool streaming = (int64_t)rows * cols * 12 >= ((int64_t)192 << 20);
+  if (vec && streaming) return launch_softmax_bwd<true, true>(nv, y, ldy, dy, lddy, dx, lddx, rows, cols, causal_seq, scale);
+  if (vec) return launch_softmax_bwd<true, false>(nv, y, ldy, dy, lddy, dx, lddx, rows, cols, causal_seq, scale);
+  return launch_softmax_bwd<false, false>(nv, y, ldy, dy, lddy, dx, lddx, rows, cols, causal_seq, scale);
+}
+
+WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, const float* gamma, const float* dy,
+                                          float eps, float* dx, float* dgamma, float* dbeta) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if (cols == 0) return 0;
+  if (!gamma || !dgamma || !dbeta) return fail(WF2HIP_EINVAL, "null pointer");
+  if (rows == 0) {  // empty sums
+    WF2_TRY(wf2hip_fill_f32(dgamma, (size_t)cols, 0.0f));
+    return wf2hip_fill_f32(dbeta, (size_t)cols, 0.0f);
+  }
+  if (!x || !dy || !dx) return fail(WF2HIP_EINVAL, "null pointer");
+  const int nv = pick_nv(cols);
+  if (nv == 0 || nv > 8)
+    return fail(WF2HIP_EUNSUPPORTED, "LayerNorm backward: rows longer than 2048 are not built (compose it from nodes)");
+  const int64_t total = (int64_t)rows * cols;
+  if ((x < dx + total && dx < x + total) || (dgamma < dbeta + cols && dbeta < dgamma + cols))
+    return fail(WF2HIP_EOVERLAP, "LayerNorm backward: dx overlaps x, or dgamma overlaps dbeta");
+  if (dy < dx + total && dx < dy + total && dx != dy)
+    return fail(WF2HIP_EOVERLAP, "LayerNorm backward: dx overlaps dy without being dy");
+  // two workgroups per compute unit, at most one wavefront per row: (65536, 1024) runs at 74 % of
+  // the HBM peak (both small folds included), 66 % with one workgroup per unit, 65 - 67 % with
+  // three to eight (more rows of `partial` to write and fold)
+  const int64_t blocks = std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
+  const size_t partial_bytes = (size_t)blocks * 2 * cols * sizeof(float);
+  const size_t level2_bytes = (size_t)kFoldGroups * 2 * cols * sizeof(double);
+  void* partial = nullptr;
+  WF2_TRY(wf2hip_malloc_uninitialized(&partial, partial_bytes + level2_bytes));  // partial_bytes is a multiple of 8
+  double* level2 = reinterpret_cast<double*>(static_cast<char*>(partial) + partial_bytes);
+  const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
+  const bool streaming = total * 12 >= ((int64_t)192 << 20);
+  int rc;
+  if (vec && streaming)
+    rc = launch_layernorm_bwd<true, true>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+  else if (vec)
+    rc = launch_layernorm_bwd<true, false>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+  else
+    rc = launch_layernorm_bwd<false, false>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+  if (rc == 0) {
+    const uint32_t strips = (uint32_t)ceil_div(2 * (int64_t)cols, kWave);
+    layernorm_bwd_fold1<<<dim3(strips, kFoldGroups), kBlock, 0, rt().stream>>>((const float*)partial, blocks,
+                                                                              2 * (int64_t)cols, level2);
+    rc = after_launch("layernorm_bwd_fold1");
+  }
+  if (rc == 0) {
+    layernorm_bwd_fold2<<<(uint32_t)ceil_div(2 * (int64_t)cols, kWave), kWave, 0, rt().stream>>>(level2, cols, dgamma,
+                                                                                               dbeta);
+    rc = after_launch("layernorm_bwd_fold2");
+  }
+  (void)wf2hip_free(partial);  // stream order keeps it alive for the launches above
+  return rc;
+}

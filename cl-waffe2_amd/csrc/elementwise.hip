@@ -103,6 +103,31 @@ struct OpSigmoid {
     return 1.0f / (1.0f + e);
   }
 };
+// dOUT <- dOUT f'(X) for the same activations: the MulNode of the upstream gradient with
+// the derivative recipe (A>scal for ReLU, A>=scal with slope for leaky ReLU, s (1 - s) with
+// s recomputed for the sigmoid -- each the binary32 operations of that composition in the
+// same order, so bit-identical to it) in one pass, 12 bytes per element.
+struct OpReluGrad {
+  static constexpr int kFlatU = 4;
+  __device__ __forceinline__ float operator()(float d, float s) const { return d * (s > 0.0f ? 1.0f : 0.0f); }
+};
+struct OpLeakyReluGrad {
+  static constexpr int kFlatU = 4;
+  float slope;
+  __device__ __forceinline__ float operator()(float d, float s) const { return d * (s >= 0.0f ? 1.0f : slope); }
+};
+struct OpSigmoidGrad {
+  static constexpr int kFlatU = 4;
+  __device__ __forceinline__ float operator()(float d, float s) const {
+    const float e = expf_(-1.0f * s);
+    const float sg = 1.0f / (1.0f + e);
+    return d * (sg * (1.0f + -1.0f * sg));  // (!sub 1 s) is 1 + (-1 s)
+  }
+};
+struct OpGeluGrad {
+  static constexpr int kFlatU = 4;
+  __device__ __forceinline__ float operator()(float d, float s) const { return d * gelu_tanh_grad_f(s); }
+};
 struct OpPow {
   static constexpr int kFlatU = 2;
   float p;
@@ -1178,6 +1203,24 @@ int binary_nd(int op, Space s, float* a, const float* b) {
   }
 }
 
+// dout (the `a` side, updated in place) <- dout f'(x) with x on the `b` side.
+int activation_backward_nd(int op, Space s, float* dout, const float* x, float p) {
+  if (s.total == 0) return 0;
+  if (!dout || !x) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  normalise(&s);
+  if (hazardous_overlap(s, dout, x))
+    return fail(WF2HIP_EOVERLAP, "activation backward between partially overlapping windows");
+  if (has_broadcast_axis(s, s.sa))
+    return fail(WF2HIP_EINVAL, "activation backward: the gradient may not be a broadcast view");
+  switch (op) {
+    case WF2HIP_GELU: return launch_elementwise<OpGeluGrad, true>(s, dout, x, OpGeluGrad{});
+    case WF2HIP_RELU: return launch_elementwise<OpReluGrad, true>(s, dout, x, OpReluGrad{});
+    case WF2HIP_SIGMOID: return launch_elementwise<OpSigmoidGrad, true>(s, dout, x, OpSigmoidGrad{});
+    case WF2HIP_LEAKY_RELU: return launch_elementwise<OpLeakyReluGrad, true>(s, dout, x, OpLeakyReluGrad{p});
+    default: return fail(WF2HIP_EINVAL, "activation backward: op %d is not an activation", op);
+  }
+}
+
 // x = source (described by the view's `a` side), out = destination (`b` side).
 int unary_nd(int op, Space s, const float* x, float* out, float p) {
   if (s.total == 0) return 0;
@@ -1282,6 +1325,13 @@ WF2_API int wf2hip_unary_nd(int op, const wf2hip_view2* v, const float* a, float
   Space s;
   WF2_TRY(load_space(v, &s));
   return unary_nd(op, s, a, b, p);
+}
+
+WF2_API int wf2hip_activation_backward_nd(int op, const wf2hip_view2* v, float* dout, const float* x, float p) {
+  WF2_TRY(require_init());
+  Space s;
+  WF2_TRY(load_space(v, &s));
+  return activation_backward_nd(op, s, dout, x, p);
 }
 
 #define WF2_DEFINE_BINARY_1D(name, OP)                                                   \

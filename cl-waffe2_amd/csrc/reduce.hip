@@ -19,50 +19,11 @@
 #include "wf2_common.h"
 #include "wf2_math.h"
 #include "wf2_view.h"
+#include "wf2_rows.h"
 
 namespace wf2 {
 
-typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr int kMaxOuter = WF2HIP_MAX_RANK - 1;
-constexpr int kWavesPerBlock = kBlock / kWave;
-
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
-}
-
-__device__ __forceinline__ float wave_sum32(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-  return v;
-}
-
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
-  return v;
-}
-
-// Sum over the workgroup in a fixed order; valid in thread 0.
-__device__ __forceinline__ double block_sum(double v, double* lds) {
-  v = wave_sum(v);
-  const int w = threadIdx.x / kWave;
-  if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
-  __syncthreads();
-  double t = 0.0;
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int i = 0; i < kWavesPerBlock; i++) t += lds[i];
-  }
-  return t;
-}
 
 // What a reduction leaves in its destination.  Accumulating (AddNode into a
 // stride-0 view): dst + total, rounded once.  Overwriting (the one-node form of
@@ -495,7 +456,6 @@ static void split_axes(const Space& s, AccParams* p) {
   }
 }
 
-static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // `partials` holds at least kPartialCapacity / 2 binary64 sums: the library's
 // own buffer, or the static array of the allocation-free entry point.
@@ -669,74 +629,7 @@ static int launch_maxmin(long n, const float* x, long incx, float* out) {
   return after_launch("maxmin pass 2");
 }
 
-// ---- fused row kernels: one wavefront per row, the row held in registers --------
-// Lane l of the wave owns NV groups of 4 consecutive columns, group g starting
-// at column (g*64 + l)*4 (16-byte coalesced) or, when the row cannot be read
-// with 16-byte loads, columns (g*4 + c)*64 + l.
-template <int NV, bool VEC, bool NT = false>
-struct RowRegs {
-  float v[NV][4];
-
-  __device__ __forceinline__ static int64_t col(int g, int c, int lane) {
-    return VEC ? ((int64_t)(g * kWave + lane) * 4 + c) : ((int64_t)(g * 4 + c) * kWave + lane);
-  }
-
-  __device__ __forceinline__ void load(const float* __restrict__ row, int64_t ncols, int lane,
-                                       float fill) {
-    if (VEC && ncols == (int64_t)NV * kWave * 4) {
-      // the row fills the register tile exactly: unguarded loads, all in flight
-#pragma unroll
-      for (int g = 0; g < NV; g++) {
-        const f4* q = reinterpret_cast<const f4*>(row + col(g, 0, lane));
-        f4 t = NT ? __builtin_nontemporal_load(q) : *q;
-        v[g][0] = t.x; v[g][1] = t.y; v[g][2] = t.z; v[g][3] = t.w;
-      }
-      return;
-    }
-#pragma unroll
-    for (int g = 0; g < NV; g++) {
-      if (VEC && col(g, 3, lane) < ncols) {
-        f4 t = *reinterpret_cast<const f4*>(row + col(g, 0, lane));
-        v[g][0] = t.x; v[g][1] = t.y; v[g][2] = t.z; v[g][3] = t.w;
-      } else {
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          int64_t cc = col(g, c, lane);
-          v[g][c] = cc < ncols ? row[cc] : fill;
-        }
-      }
-    }
-  }
-
-  __device__ __forceinline__ void store(float* __restrict__ row, int64_t ncols, int lane) const {
-    if (VEC && ncols == (int64_t)NV * kWave * 4) {
-#pragma unroll
-      for (int g = 0; g < NV; g++) {
-        f4 t = {v[g][0], v[g][1], v[g][2], v[g][3]};
-        f4* q = reinterpret_cast<f4*>(row + col(g, 0, lane));
-        if (NT)
-          __builtin_nontemporal_store(t, q);
-        else
-          *q = t;
-      }
-      return;
-    }
-#pragma unroll
-    for (int g = 0; g < NV; g++) {
-      if (VEC && col(g, 3, lane) < ncols) {
-        f4 t = {v[g][0], v[g][1], v[g][2], v[g][3]};
-        *reinterpret_cast<f4*>(row + col(g, 0, lane)) = t;
-      } else {
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          int64_t cc = col(g, c, lane);
-          if (cc < ncols) row[cc] = v[g][c];
-        }
-      }
-    }
-  }
-};
-
+// ---- fused row kernels: one wavefront per row, the row held in registers (RowRegs, wf2_rows.h) ----
 // softmax over the first `valid` columns of a row; columns valid..ncols-1 of
 // the output are set to 0 (used by the causal form).
 // RW rows per wavefront: with one or two vectors per lane and row a wavefront that
@@ -1014,16 +907,6 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_block(const float* __re
   const double rstd = stat;
   for (int64_t c = threadIdx.x; c < ncols; c += kBlock)
     outr[c] = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
-}
-
-// Register tiles: NV groups of 256 columns per wavefront.  Sizes 3, 6 and 12
-// make rows of 768, 1536 and 3072 columns (transformer widths) fill the tile
-// exactly, which selects the unguarded load path.
-static int pick_nv(int64_t ncols) {
-  static const int sizes[] = {1, 2, 3, 4, 6, 8, 12, 16};
-  for (int nv : sizes)
-    if ((int64_t)nv * kWave * 4 >= ncols) return nv;
-  return 0;
 }
 
 template <bool VEC, bool NT>

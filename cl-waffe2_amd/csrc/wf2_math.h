@@ -682,4 +682,34 @@ WF2_MATH_FN float gelu_tanh_fast(float x) {
   return (t > 100.0f) ? -0.0f : r;
 }
 
+// d/dx of the tanh-form GELU, x / (1 + E) with E = 2^t, t = x (k1 + k2 x^2):
+//   g'(x) = s (1 + x (1 - s) v),  s = 1 / (1 + E),  v = 2 sqrt(2/pi) (1 + 3 * 0.044715 x^2).
+// s and 1 - s are both formed from e = 2^-|t| <= 1 (no cancellation, no overflow):
+// (s, 1 - s) = (r, e r) for x >= 0 and (e r, r) for x < 0 with r = 1 / (1 + e).
+// Error: three roundings of t (1e-7 |t| absolute in the exponent) and one ulp each
+// from v_exp_f32, v_rcp_f32 and the products: below 1e-6 of |s| + |x s (1 - s) v|
+// for |x| <= 4 (host sweep: 7.7e-7), growing with |t| in the left tail to 1e-5 at
+// x = -10, where g' is 1e-33; g' has a zero near x = -0.75, so no bound relative to
+// g' itself exists.  Beyond |x| = 16, e is 0 in binary32: g' = 1 on the right, 0 on
+// the left; v_exp_f32 returns 0 below 2^-126, so gradients under about 2^-120 (x < -6.9)
+// are flushed to 0.  15 VALU operations.
+WF2_MATH_FN float gelu_tanh_grad_f(float x) {
+  const float k1 = -2.3022082f;    // -2 sqrt(2/pi) log2(e)
+  const float k2 = -0.10294324f;   // k1 * 0.044715
+  const float c1 = 1.5957691f;     // 2 sqrt(2/pi)
+  const float c2 = 0.21406446f;    // c1 * 3 * 0.044715
+  const float xc = __builtin_fminf(__builtin_fmaxf(x, -16.0f), 16.0f);  // drops a NaN, restored below
+  const float x2 = xc * xc;
+  const float t = xc * __builtin_fmaf(k2, x2, k1);
+  const float e = WF2_FAST_EXP2F(-__builtin_fabsf(t));
+  const float r = WF2_FAST_RCPF(1.0f + e);
+  const float er = e * r;
+  const bool right = xc >= 0.0f;
+  const float sg = right ? r : er;
+  const float cs = right ? er : r;
+  const float v = __builtin_fmaf(c2, x2, c1);
+  const float res = sg * __builtin_fmaf(xc * cs, v, 1.0f);
+  return (x != x) ? x : res;
+}
+
 }  // namespace wf2

@@ -681,8 +681,21 @@ def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e
 
 
 def layer_norm_backward(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float = 1.0e-5):
+    """(dx, dgamma, dbeta) of LayerNorm over the last axis from the saved input: one row kernel and a
+    small fold (HIP-LayerNorm-Node-backward) for rows up to 2048 wide, the node composition beyond."""
+    cols = x.shape[-1]
+    if cols > 2048 or x.dtype != "float":
+        return layer_norm_backward_composed(x, g, dout, eps)
+    x2, d2 = to_contiguous(x), to_contiguous(dout)
+    dx = HIPTensor(list(x.shape), initial_element=None)
+    dg, db = HIPTensor([cols], initial_element=None), HIPTensor([cols], initial_element=None)
+    nodes.forward("HIP-LayerNorm-Node-backward", x2, g, d2, dx, dg, db, float(eps))
+    return dx, dg, db
+
+
+def layer_norm_backward_composed(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float = 1.0e-5):
     """(dx, dgamma, dbeta) of LayerNorm over the last axis, composed node for node the way
-    ``layer-norm-gradients`` of the Lisp glue composes the backward of HIP-LayerNorm-Node:
+    ``layer-norm-gradients`` of the Lisp glue composes it for rows beyond the kernel's width:
     with xh = (x - u) rstd and dyh = dout g,
     dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)), dgamma = sum_rows dout xh, dbeta = sum_rows dout."""
     cols = x.shape[-1]
@@ -708,9 +721,9 @@ def layer_norm_backward(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float 
 # ---------------------------------------------------------------------------
 
 def gelu_derivative(x: HIPTensor) -> HIPTensor:
-    """d/dx of 0.5 x (1 + tanh u), u = c (x + a x^3): 0.5 (1 + t) + 0.5 x (1 - t^2) c (1 + 3 a x^2)
-    (``gelu-derivative`` of the Lisp glue; the recipe of ``source/nn/activation.lisp:45-66``
-    differentiated)."""
+    """d/dx of 0.5 x (1 + tanh u), u = c (x + a x^3): 0.5 (1 + t) + 0.5 x (1 - t^2) c (1 + 3 a x^2),
+    node for node (``gelu-derivative`` of the Lisp glue; the recipe of
+    ``source/nn/activation.lisp:45-66`` differentiated).  The one-kernel form is `activation_backward`."""
     c = float(np.float32(math.sqrt(2.0 / math.pi)))
     a = 0.044715
     x2 = mul(x, x)
@@ -722,17 +735,34 @@ def gelu_derivative(x: HIPTensor) -> HIPTensor:
     return add_(left, right)
 
 
-def linear_backward(x: HIPTensor, w: HIPTensor, b: HIPTensor, dout: HIPTensor, activation: str | None = None):
+_ACTIVATIONS = {"relu": _lib.RELU, "leaky_relu": _lib.LEAKY_RELU, "sigmoid": _lib.SIGMOID, "gelu": _lib.GELU}
+
+
+def activation_backward(activation: str, x: HIPTensor, dout: HIPTensor, p: float = 0.0,
+                        in_place: bool = False) -> HIPTensor:
+    """dout f'(x) for 'relu', 'leaky_relu' (slope p), 'sigmoid', 'gelu' from the saved input x in one
+    kernel (HIP-Activation-Node-backward).  With ``in_place`` the result overwrites dout."""
+    d = dout if in_place else copy(dout)
+    return nodes.forward("HIP-Activation-Node-backward", d, x, _ACTIVATIONS[activation], float(p))
+
+
+def linear_backward(x: HIPTensor, w: HIPTensor, b: HIPTensor, dout: HIPTensor, activation: str | None = None,
+                    fused: bool = True):
     """(dx, dw, db) of ``act(x . w + b)`` (HIP-Linear-Node, and HIP-Linear-Residual-Node whose
     residual passes ``dout`` through unchanged): dX = dZ W^T, dW = X^T dZ, dB = column sums of
-    dZ, with dZ = dOUT for a plain layer and dOUT gelu'(Z), Z = X W + B recomputed, for a GELU
-    layer (``linear-gradients`` of the Lisp glue; MatMulNode's backward,
-    ``base-impl/matrix-ops.lisp:10-15``)."""
+    dZ, with dZ = dOUT for a plain layer and dOUT gelu'(Z), Z = X W + B recomputed (one product
+    with the bias in its epilogue), for a GELU layer (``linear-gradients`` of the Lisp glue;
+    MatMulNode's backward, ``base-impl/matrix-ops.lisp:10-15``).  ``fused=False`` composes
+    gelu' node for node."""
     k, n = x.shape[-1], w.shape[-1]
     x2, d2 = reshape(x, -1, k), reshape(dout, -1, n)
     if activation == "gelu":
-        z = add_(matmul(x2, w), b)
-        dz = mul_(gelu_derivative(z), d2)
+        if fused:
+            z = linear(x2, w, b)
+            dz = activation_backward("gelu", z, d2)
+        else:
+            z = add_(matmul(x2, w), b)
+            dz = mul_(gelu_derivative(z), d2)
     elif activation is None:
         dz = d2
     else:
@@ -743,32 +773,51 @@ def linear_backward(x: HIPTensor, w: HIPTensor, b: HIPTensor, dout: HIPTensor, a
     return HIPTensor(list(x.shape), vec=dx.vec), dw, db
 
 
-def softmax_backward(y: HIPTensor, dout: HIPTensor, scale: float = 1.0) -> HIPTensor:
-    """dx = scale y (dy - sum_j dy y) over the last axis, from the saved output y
-    (HIP-Softmax-Node, and HIP-Causal-Softmax-Node whose y is 0 above the diagonal)."""
+def softmax_backward_composed(y: HIPTensor, dout: HIPTensor, scale: float = 1.0) -> HIPTensor:
+    """dx = scale y (dy - sum_j dy y) over the last axis node for node."""
     dot = sum(mul(dout, y), axis=-1, keepdims=True)
     dx = mul_(sub(dout, dot), y)
     return dx if scale == 1.0 else mul_(dx, float(scale))
 
 
+def softmax_backward(y: HIPTensor, dout: HIPTensor, scale: float = 1.0, causal: bool = False,
+                     in_place: bool = False) -> HIPTensor:
+    """dx = scale y (dy - sum_j dy y) over the last axis from the saved output y in one kernel
+    (HIP-Softmax-Node-backward; HIP-Causal-Softmax-Node-backward with ``causal``, which neither
+    reads dout above the diagonal nor leaves dx unwritten there).  With ``in_place`` the result
+    overwrites dout."""
+    y, dout = to_contiguous(y), to_contiguous(dout)
+    dx = dout if in_place else HIPTensor(list(y.shape), initial_element=None)
+    if causal:
+        return nodes.forward("HIP-Causal-Softmax-Node-backward", y, dout, dx, float(scale))
+    nodes.forward("HIP-Softmax-Node-backward", y, dout, dx)
+    return dx if scale == 1.0 else mul_(dx, float(scale))
+
+
 def attention_backward(q: HIPTensor, k: HIPTensor, v: HIPTensor, dout: HIPTensor, scale: float | None = None,
                        causal: bool = False, dq: HIPTensor | None = None, dk: HIPTensor | None = None,
-                       dv: HIPTensor | None = None):
+                       dv: HIPTensor | None = None, fused: bool = True):
     """(dq, dk, dv) of HIP-Attention-Node with the probabilities recomputed, as its :backward
     composes them: P = softmax(scale Q K^T [+ mask]), dV = P^T dO, dP = dO V^T,
-    dS = P (dP - sum_j dP P), dQ = scale dS K, dK = scale dS^T Q.  Operands are
+    dS = scale P (dP - sum_j dP P), dQ = dS K, dK = dS^T Q.  Operands are
     (batch, heads, seq, head_dim) views whose last axis is contiguous; the optional outputs may be
-    such views too (windows of one fused-projection gradient)."""
+    such views too (windows of one fused-projection gradient).  With a mask the two score-shaped
+    products form their lower triangles only and dS K skips the tiles above the diagonal.
+    ``fused=False`` takes the softmax gradient node for node and every product in full."""
     hd = q.shape[-1]
     scale = 1.0 / math.sqrt(hd) if scale is None else float(scale)
-    s = matmul(q, t(k))
+    tri = 1 if (causal and fused) else 0
+    s = matmul(q, t(k), causal=tri)
     if causal:
-        p = causal_softmax_fused(s, scale)
+        p = causal_softmax_fused(s, scale, out=s if fused else None)
     else:
         p = reshape(softmax_fused(reshape(mul_(s, scale), -1, s.shape[-1])), *s.shape)
     dv = matmul(t(p), dout, out=dv)
-    dp = matmul(dout, t(v))
-    ds = softmax_backward(p, dp)
-    dq = mul_(matmul(ds, k, out=dq), scale)
-    dk = mul_(matmul(t(ds), q, out=dk), scale)
+    dp = matmul(dout, t(v), causal=tri)
+    if fused:
+        ds = softmax_backward(p, dp, scale=scale, causal=causal, in_place=True)
+    else:
+        ds = softmax_backward_composed(p, dp, scale)
+    dq = matmul(ds, k, out=dq, causal=2 if tri else 0)
+    dk = matmul(t(ds), q, out=dk)
     return dq, dk, dv

@@ -169,6 +169,9 @@ _SIGNATURES = {
     "wf2hip_softmax_rows_f32": ([_L, _L, _P, _L, _P, _L], C.c_int),
     "wf2hip_causal_softmax_f32": ([_L, _L, _P, _P, _F], C.c_int),
     "wf2hip_layernorm_rows_f32": ([_L, _L, _P, _P, _P, _F, _P], C.c_int),
+    "wf2hip_softmax_backward_rows_f32": ([_L, _L, _P, _L, _P, _L, _P, _L, _F, _L], C.c_int),
+    "wf2hip_layernorm_backward_f32": ([_L, _L, _P, _P, _P, _F, _P, _P, _P], C.c_int),
+    "wf2hip_activation_backward_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F], C.c_int),
     "wf2hip_sgemm": ([C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _P, _L, _F, _P, _L], C.c_int),
     "wf2hip_sgemm_strided_batched": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _P, _L, _L, _F, _P, _L, _L, _L],

@@ -5,10 +5,11 @@
 ;;;; node.  The library holds each of them as one kernel; this file makes them reachable the way
 ;;;; the reference intends device-specific fusions to be added:
 ;;;;   * a define-op node per fused kernel (as Softmax-Cross-Entropy-Node, source/nn/criterion.lisp:90),
-;;;;     forward = one library call, backward = the derivative composed from ordinary ! functions
-;;;;     and evaluated with proceed, so it runs on the device through the nodes of kernels.lisp
-;;;;     (a graph is compiled per backward call: the fused nodes pay off in inference and in
-;;;;     forward-heavy training; a defmodel-as cache is the next step);
+;;;;     forward = one library call; backward = one library call too where the library holds the
+;;;;     gradient as a kernel (activations, softmax, causal softmax, LayerNorm), otherwise the
+;;;;     derivative composed from ordinary ! functions and evaluated with proceed, so it runs on
+;;;;     the device through the nodes of kernels.lisp (a graph is compiled per such backward call;
+;;;;     a defmodel-as cache is the next step);
 ;;;;   * a define-bypass rule per function (source/vm/nodes/symbolic.lisp:118-131): with HIPTensor
 ;;;;     in *using-backend*, calls of cl-waffe2/nn:!relu & co. compiled after this file is loaded
 ;;;;     build the fused node instead ((setf *enable-symbolic-path* nil) switches that off).
@@ -26,8 +27,22 @@
 
 (defconstant +gelu+ 40) (defconstant +relu+ 41) (defconstant +sigmoid+ 42) (defconstant +leaky-relu+ 43)
 
+(defparameter *compose-backward* nil
+  "When true the fused nodes differentiate node for node (the compositions this file also holds)
+instead of through the library's backward kernels.")
+
 (defun hip-float-tensor-p (x)
   (and (typep x 'HIPTensor) (eql (dtype x) :float)))
+
+(defun fresh-like (x)
+  "An uninitialised-content-is-fine :float device tensor of X's shape (every element is written
+by the kernel it is handed to)."
+  (make-tensor (shape x) :dtype :float :order (order x) :device 'HIPTensor))
+
+(defun eager-contiguous (x)
+  "X as a contiguous tensor that starts at its storage, evaluated now: the row kernels take base
+pointers.  Inside a backward body, which runs eagerly."
+  (proceed (->contiguous x)))
 
 (defun call-composed (function &rest args)
   "The reference's own composition; through funcall so that the bypass does not apply again."
@@ -41,16 +56,27 @@
             :save-for-backward-names (x)
             :where (X[~] OUT[~] -> OUT[~])
             :documentation "OUT <- f(X) as one kernel (WF2HIP_RELU / SIGMOID / LEAKY_RELU / GELU).
-DERIVATIVE is a function of (x) returning df/dx built from ! functions."
+Backward: dout f'(x) as one kernel as well (wf2hip_activation_backward_nd, on a copy of dout).
+DERIVATIVE, a function of (x) returning df/dx built from ! functions, is the same gradient node
+for node; it is what the kernel is checked against and what *compose-backward* selects."
             :forward ((self x out)
                       (with-setting-save4bw ((x x))
                         (run-unary (activation-op self) x out (activation-parameter self))))
             :backward ((self dout)
                        (with-reading-save4bw ((x x))
                          ;; the body of a define-op backward runs eagerly (it is the forward of the
-                         ;; generated -backward node, source/vm/nodes/static-node.lisp:296-318), so
-                         ;; the composed derivative is evaluated here with proceed
-                         (values (proceed (!mul dout (funcall (activation-derivative self) x))) nil))))
+                         ;; generated -backward node, source/vm/nodes/static-node.lisp:296-318)
+                         (if *compose-backward*
+                             (values (proceed (!mul dout (funcall (activation-derivative self) x))) nil)
+                             (let ((dx (proceed (!copy dout))))
+                               (ensure-extension)
+                               (with-foreign-object (view '(:struct view2))
+                                 (fill-view2 view dx x)
+                                 (check (wf2hip-activation-backward-nd (activation-op self) view
+                                                                       (tensor-device-pointer dx)
+                                                                       (tensor-device-pointer x)
+                                                                       (coerce (activation-parameter self) 'single-float))))
+                               (values dx nil))))))
   (setf (activation-op self) op
         (activation-parameter self) p
         (activation-derivative self) derivative))
@@ -100,6 +126,21 @@ DERIVATIVE is a function of (x) returning df/dx built from ! functions."
       (call-composed 'cl-waffe2/nn:!gelu x)))
 
 ;; ---- row softmax ---------------------------------------------------------------------------
+(defun softmax-gradient (y dout scale causal)
+  "scale y (dout - sum_j dout y) over the last axis of the saved output Y in one kernel
+(wf2hip_softmax_backward_rows_f32).  CAUSAL: rows of square matrices; dout is not read above
+the diagonal and the gradient is 0 there."
+  (ensure-extension)
+  (let* ((dout (eager-contiguous dout))
+         (dx (fresh-like y))
+         (cols (car (last (shape y))))
+         (rows (/ (apply #'* (shape y)) cols)))
+    (check (wf2hip-softmax-backward-rows-f32 rows cols (tensor-device-pointer y) cols
+                                             (tensor-device-pointer dout) cols
+                                             (tensor-device-pointer dx) cols
+                                             (coerce scale 'single-float) (if causal cols 0)))
+    dx))
+
 (define-op (HIP-Softmax-Node (self)
             :save-for-backward-names (y)
             :where (X[rows cols] OUT[rows cols] -> OUT[rows cols])
@@ -114,8 +155,10 @@ DERIVATIVE is a function of (x) returning df/dx built from ! functions."
             :backward ((self dout)
                        ;; dx = y * (dy - sum(dy * y) over the row)
                        (with-reading-save4bw ((y y))
-                         (let ((dot (!sum-hip (!mul dout y) :axis 1 :keepdims t)))
-                           (values (proceed (!mul y (!sub dout dot))) nil))))))
+                         (if *compose-backward*
+                             (let ((dot (!sum-hip (!mul dout y) :axis 1 :keepdims t)))
+                               (values (proceed (!mul y (!sub dout dot))) nil))
+                             (values (softmax-gradient y dout 1.0 nil) nil))))))
 
 (defun !softmax-hip (x &key (avoid-overflow t) (axis 1))
   "(!softmax x :axis 1) on a contiguous :float matrix as one kernel; anything else takes the
@@ -147,13 +190,29 @@ Composed from ! functions (!mean and !sum are one node each on the device)."
          (db   (!sum-hip dout :axis 0)))
     (values dx dg db)))
 
+(defun layer-norm-gradients-fused (x g dout eps)
+  "The same three gradients from one row kernel and two small folds (wf2hip_layernorm_backward_f32;
+rows up to 2048 wide)."
+  (ensure-extension)
+  (let* ((dout (eager-contiguous dout))
+         (rows (first (shape x)))
+         (cols (second (shape x)))
+         (dx (fresh-like x))
+         (dg (fresh-like g))
+         (db (fresh-like g)))
+    (check (wf2hip-layernorm-backward-f32 rows cols (tensor-device-pointer x) (tensor-device-pointer g)
+                                          (tensor-device-pointer dout) (coerce eps 'single-float)
+                                          (tensor-device-pointer dx) (tensor-device-pointer dg)
+                                          (tensor-device-pointer db)))
+    (values dx dg db)))
+
 (define-op (HIP-LayerNorm-Node (self eps)
             :slots ((eps :initform 1.0e-5 :accessor layernorm-eps))
             :save-for-backward-names (x g)
             :where (X[rows cols] G[cols] B[cols] OUT[rows cols] -> OUT[rows cols])
             :documentation "OUT <- (x - mean) / sqrt(var + eps) * g + b per row, one kernel
-(wf2hip_layernorm_rows_f32).  Backward: the three gradients composed from the saved input
-(layer-norm-gradients)."
+(wf2hip_layernorm_rows_f32).  Backward: the three gradients from the saved input, one kernel for
+rows up to 2048 wide (layer-norm-gradients-fused), composed beyond (layer-norm-gradients)."
             :forward ((self x g b out)
                       (ensure-extension)
                       (check (wf2hip-layernorm-rows-f32 (first (shape x)) (second (shape x))
@@ -164,11 +223,15 @@ Composed from ! functions (!mean and !sum are one node each on the device)."
                       (with-setting-save4bw ((x x) (g g)) out))
             :backward ((self dout)
                        (with-reading-save4bw ((x x) (g g))
-                         (multiple-value-bind (dx dg db) (layer-norm-gradients x g dout (layernorm-eps self))
-                           (values (proceed dx)
-                                   (proceed (!reshape dg (second (shape x))))
-                                   (proceed (!reshape db (second (shape x))))
-                                   nil)))))
+                         (if (or *compose-backward* (> (second (shape x)) 2048))
+                             (multiple-value-bind (dx dg db) (layer-norm-gradients x g dout (layernorm-eps self))
+                               (values (proceed dx)
+                                       (proceed (!reshape dg (second (shape x))))
+                                       (proceed (!reshape db (second (shape x))))
+                                       nil))
+                             (multiple-value-bind (dx dg db)
+                                 (layer-norm-gradients-fused x g dout (layernorm-eps self))
+                               (values dx dg db nil))))))
   (setf (layernorm-eps self) eps))
 
 (defun !layer-norm-hip (x gamma beta &key (eps 1.0e-5))
@@ -274,9 +337,18 @@ takes the composed route; !mean-hip passes the count as a number."
 (defun linear-gradients (x w b dout activation)
   "dX = dZ W^T, dW = X^T dZ, dB = column sums of dZ, with dZ = dOUT for a plain layer and
 dOUT gelu'(Z), Z = X W + B recomputed, for a GELU layer."
-  (let* ((dz (if (eql activation :gelu)
-                 (!mul dout (gelu-derivative (!add (!matmul x w) (!flexible b))))
-                 dout)))
+  (let* ((dz (cond ((not (eql activation :gelu)) dout)
+                   (*compose-backward*
+                    (!mul dout (gelu-derivative (!add (!matmul x w) (!flexible b)))))
+                   (t
+                    ;; Z through the product with the bias in its epilogue, dOUT gelu'(Z) in one kernel
+                    (let ((z (run-linear x w b nil (fresh-like dout) nil))
+                          (dz (proceed (!copy dout))))
+                      (with-foreign-object (view '(:struct view2))
+                        (fill-view2 view dz z)
+                        (check (wf2hip-activation-backward-nd +gelu+ view (tensor-device-pointer dz)
+                                                              (tensor-device-pointer z) 0.0)))
+                      dz)))))
     (values (!matmul dz (!t w))
             (!matmul (!t x) dz)
             (!reshape (!sum-hip dz :axis 0) (second (shape w))))))
@@ -346,8 +418,10 @@ the MulNode by the scale, the AddNode of the mask and !softmax of causal attenti
             :backward ((self dout)
                        ;; dx = scale y (dy - sum_j dy y); y is 0 above the diagonal, so is dx
                        (with-reading-save4bw ((y y))
-                         (let ((dot (!sum-hip (!mul dout y) :axis -1 :keepdims t)))
-                           (values (proceed (!mul (softmax-scale self) (!mul y (!sub dout dot)))) nil)))))
+                         (if *compose-backward*
+                             (let ((dot (!sum-hip (!mul dout y) :axis -1 :keepdims t)))
+                               (values (proceed (!mul (softmax-scale self) (!mul y (!sub dout dot)))) nil))
+                             (values (softmax-gradient y dout (softmax-scale self) t) nil)))))
   (setf (softmax-scale self) scale))
 
 (defun !causal-softmax-hip (scores &key (scale 1.0))
@@ -384,8 +458,8 @@ the MulNode by the scale, the AddNode of the mask and !softmax of causal attenti
             :documentation "OUT <- softmax(scale Q K^T [+ causal mask]) V per (batch, head) in one kernel that
 never forms the (seq, seq) score matrices (wf2hip_attention_f32; heads up to 64 wide).  The operands may be
 strided windows of a fused projection (last axis contiguous).  Backward: composed, with the
-probabilities recomputed: dV = P^T dO, dP = dO V^T, dS = P (dP - sum_j dP P), dQ = scale dS K,
-dK = scale dS^T Q."
+probabilities recomputed: dV = P^T dO, dP = dO V^T, dS = scale P (dP - sum_j dP P) (one kernel),
+dQ = dS K, dK = dS^T Q."
             :forward ((self q k v out)
                       (ensure-extension)
                       (with-foreign-object (desc '(:struct attention-desc))
@@ -404,9 +478,12 @@ dK = scale dS^T Q."
                                 (p (apply #'!reshape p (shape s)))
                                 (dv (!matmul (!t p) dout))
                                 (dp (!matmul dout (!t v)))
-                                (ds (!mul p (!sub dp (!sum-hip (!mul dp p) :axis -1 :keepdims t))))
-                                (dq (!mul scale (!matmul ds k)))
-                                (dk (!mul scale (!matmul (!t ds) q))))
+                                ;; dS carries the factor scale: scale P (dP - sum_j dP P), one kernel
+                                (ds (if *compose-backward*
+                                        (!mul scale (!mul p (!sub dp (!sum-hip (!mul dp p) :axis -1 :keepdims t))))
+                                        (softmax-gradient (proceed p) (proceed dp) scale (attention-causal self))))
+                                (dq (!matmul ds k))
+                                (dk (!matmul (!t ds) q)))
                            (values (proceed dq) (proceed dk) (proceed dv) nil)))))
   (setf (attention-scale self) scale
         (attention-causal self) causal))

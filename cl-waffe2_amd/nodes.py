@@ -38,6 +38,9 @@ NODE_NAMES = (
     # the define-op nodes of lisp/fusion.lisp (one kernel each)
     "HIP-Sum-Node", "HIP-Activation-Node", "HIP-Softmax-Node", "HIP-LayerNorm-Node", "HIP-Linear-Node",
     "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node",
+    # the -backward nodes define-op generates for them, where the backward is one kernel too
+    "HIP-Activation-Node-backward", "HIP-Softmax-Node-backward", "HIP-Causal-Softmax-Node-backward",
+    "HIP-LayerNorm-Node-backward",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -491,6 +494,60 @@ def _require_rows(what: str, t: HIPTensor, shape=None) -> None:
 def _activation_node(x: HIPTensor, out: HIPTensor, op: int, p: float = 0.0) -> HIPTensor:
     """``X[~] OUT[~] -> OUT[~]``: ReLU / leaky ReLU / sigmoid / GELU as one kernel."""
     return _run_unary(op, x, out, float(p))
+
+
+@define_impl("HIP-Activation-Node-backward", HIPTensor, _only_float)
+def _activation_backward_node(dout: HIPTensor, x: HIPTensor, op: int, p: float = 0.0) -> HIPTensor:
+    """``DOUT[~] X[~] -> DOUT[~]``: dout <- dout f'(x) in place, x the saved input."""
+    v = view2(dout, x)
+    _lib.check(_lib.get().wf2hip_activation_backward_nd(op, C.byref(v), C.c_void_p(dout.ptr), C.c_void_p(x.ptr),
+                                                       float(p)))
+    return dout
+
+
+def _softmax_backward(name: str, y: HIPTensor, dout: HIPTensor, dx: HIPTensor, scale: float, causal: bool) -> HIPTensor:
+    _require_rows(f"{name}: y", y)
+    _require_rows(f"{name}: dout", dout, y.shape)
+    _require_rows(f"{name}: dx", dx, y.shape)
+    cols = y.shape[-1]
+    if causal and (len(y.shape) < 2 or y.shape[-2] != cols):
+        raise ValueError(f"{name} takes square score matrices, got {y.shape}")
+    rows = y.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_softmax_backward_rows_f32(rows, cols, C.c_void_p(y.ptr), cols, C.c_void_p(dout.ptr),
+                                                          cols, C.c_void_p(dx.ptr), cols, float(scale),
+                                                          cols if causal else 0))
+    return dx
+
+
+@define_impl("HIP-Softmax-Node-backward", HIPTensor, _only_float)
+def _softmax_backward_node(y: HIPTensor, dout: HIPTensor, dx: HIPTensor) -> HIPTensor:
+    """``Y[rows cols] DOUT[rows cols] DX[rows cols] -> DX``: y (dout - sum_j dout y); dx may be dout."""
+    return _softmax_backward("HIP-Softmax-Node-backward", y, dout, dx, 1.0, False)
+
+
+@define_impl("HIP-Causal-Softmax-Node-backward", HIPTensor, _only_float)
+def _causal_softmax_backward_node(y: HIPTensor, dout: HIPTensor, dx: HIPTensor, scale: float = 1.0) -> HIPTensor:
+    """``Y[matrices seq seq] DOUT[...] DX[...] -> DX``: scale y (dout - sum_j dout y) on and below the
+    diagonal (dout is not read above it), 0 above."""
+    return _softmax_backward("HIP-Causal-Softmax-Node-backward", y, dout, dx, scale, True)
+
+
+@define_impl("HIP-LayerNorm-Node-backward", HIPTensor, _only_float)
+def _layernorm_backward_node(x: HIPTensor, g: HIPTensor, dout: HIPTensor, dx: HIPTensor, dg: HIPTensor,
+                             db: HIPTensor, eps: float = 1.0e-5) -> HIPTensor:
+    """``X[rows cols] G[cols] DOUT[rows cols] DX[rows cols] DG[cols] DB[cols] -> DX DG DB`` (rows up to 2048 wide)."""
+    cols = x.shape[-1]
+    name = "HIP-LayerNorm-Node-backward"
+    _require_rows(f"{name}: x", x)
+    _require_rows(f"{name}: dout", dout, x.shape)
+    _require_rows(f"{name}: dx", dx, x.shape)
+    for what, t in (("gamma", g), ("dgamma", dg), ("dbeta", db)):
+        _require_rows(f"{name}: {what}", t, [cols])
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_layernorm_backward_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(g.ptr),
+                                                       C.c_void_p(dout.ptr), float(eps), C.c_void_p(dx.ptr),
+                                                       C.c_void_p(dg.ptr), C.c_void_p(db.ptr)))
+    return dx
 
 
 @define_impl("HIP-Softmax-Node", HIPTensor, _only_float)

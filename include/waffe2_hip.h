@@ -607,6 +607,39 @@ int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
 int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
                               const float* beta, float eps, float* out);
 
+/* ---- backward of the fused layers ------------------------------------------ */
+/* The reference differentiates !softmax, LayerNorm and the activations through
+ * their node compositions (defnode backward of every node in
+ * source/nn/activation.lisp:11-159 and source/nn/norms.lisp:72-82; the gradient
+ * of a composition is again a composition, source/vm/nodes/defnode.lisp:383-393).
+ * These entries are the backward of the one-kernel forms above, each one pass. */
+/* dx[r*lddx + c] <- scale * y[r*ldy + c] * (dy[r*lddy + c] - sum_k dy[r, k] y[r, k]):
+ * the gradient of y = softmax(scale * x) over the last axis from the saved output.
+ * causal_seq = 0: plain rows.  causal_seq = cols: rows of (seq x seq) matrices whose
+ * row r keeps columns c <= r % seq; dy is not read above the diagonal (it may be
+ * uninitialised there) and dx is 0 there.  dx may be dy (same pitch). */
+int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* y, long ldy,
+                                     const float* dy, long lddy, float* dx, long lddx,
+                                     float scale, long causal_seq);
+/* Gradients of wf2hip_layernorm_rows_f32 from the saved input: with
+ * xh = (x - mean) rstd and dyh = dy gamma,
+ *   dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),
+ *   dgamma[c] = sum over rows of dy xh,  dbeta[c] = sum over rows of dy.
+ * Contiguous (rows, cols) operands, cols <= 2048 (longer rows return
+ * WF2HIP_EUNSUPPORTED: compose them from nodes).  dx may be dy.  Allocates
+ * 8 * cols bytes per workgroup of scratch from the library's pool. */
+int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, const float* gamma,
+                                  const float* dy, float eps, float* dx, float* dgamma,
+                                  float* dbeta);
+/* dout <- dout * f'(x) in place, f one of WF2HIP_RELU, WF2HIP_LEAKY_RELU (slope p),
+ * WF2HIP_SIGMOID, WF2HIP_GELU (tanh form): the MulNode of the upstream gradient
+ * with the derivative recipe of source/nn/activation.lisp:11-92 as one kernel.
+ * The view's `a` side describes dout, its `b` side x.  ReLU, leaky ReLU and the
+ * sigmoid give the bits of the composed recipe; GELU's derivative is
+ * s (1 + x (1 - s) 2 u'), s = sigmoid(2 u), to 1e-6 of |s| + |x s (1 - s) 2 u'|. */
+int wf2hip_activation_backward_nd(int op, const wf2hip_view2* v, float* dout, const float* x,
+                                  float p);
+
 /* ---- gemm ---------------------------------------------------------------- */
 /* Column-major C(m x n) <- alpha op(A) op(B) + beta C with the argument
  * meaning of Fortran sgemm_, scalars by value.  Replaces the BLAS call of

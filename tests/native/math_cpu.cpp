@@ -14,7 +14,7 @@
 
 enum { OP_SIN = 16, OP_COS, OP_TANH, OP_LOG, OP_EXP, OP_SQRT, OP_ABS, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN,
        OP_SINH, OP_COSH, OP_LOG2, OP_LOG10, OP_LOG1P, OP_SIGN = 34, OP_SQUARE, OP_ASINH, OP_ACOSH, OP_ATANH,
-       OP_GELU = 40 };
+       OP_GELU = 40, OP_GELU_GRAD = 44 };
 
 static inline float apply(int op, float x) {
   switch (op) {
@@ -35,6 +35,7 @@ static inline float apply(int op, float x) {
     case OP_LOG10: return wf2::log10f_(x);
     case OP_LOG1P: return wf2::log1pf_(x);
     case OP_GELU: return wf2::gelu_tanh_f(x);
+    case OP_GELU_GRAD: return wf2::gelu_tanh_grad_f(x);
     case OP_SIGN: return wf2::signf_(x);
     case OP_SQUARE: return x * x;
     case OP_ASINH: return wf2::asinhf_(x);

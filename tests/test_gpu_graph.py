@@ -124,5 +124,6 @@ def test_block_dropped_after_the_capture_stays_with_the_graph(gpu):
         g.launch()
     W.lib.synchronize()
     assert np.all(fresh.numpy() == 7.0), "a replay wrote into a tensor allocated after the capture"
+    parked = W.lib.get().wf2hip_pool_idle_bytes()
     g.destroy()
-    assert W.lib.get().wf2hip_pool_idle_bytes() > idle_before  # the parked block is back
+    assert W.lib.get().wf2hip_pool_idle_bytes() >= parked + 4 * n  # the parked block is back

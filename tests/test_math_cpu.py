@@ -18,7 +18,7 @@ from helpers import ulp_distance
 HERE = os.path.dirname(os.path.abspath(__file__))
 OPS = {"sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21, "abs": 22, "tan": 23, "asin": 24,
        "acos": 25, "atan": 26, "sinh": 27, "cosh": 28, "log2": 29, "log10": 30, "log1p": 31, "gelu": 40,
-       "sign": 34, "square": 35, "asinh": 36, "acosh": 37, "atanh": 38}
+       "sign": 34, "square": 35, "asinh": 36, "acosh": 37, "atanh": 38, "gelu_grad": 44}
 
 
 @pytest.fixture(scope="module")
@@ -152,3 +152,35 @@ def test_special_values(M):
     assert f("sqrt", 4.0) == 2.0 and np.isnan(f("sqrt", -1.0))
     assert abs(f("gelu", 1.0) - 0.841192) < 5e-7   # vm/nodes/t/composite.lisp:119
     assert f("gelu", 0.0) == 0.0 and f("gelu", -30.0) == 0.0 and f("gelu", 30.0) == 30.0
+
+
+def gelu_grad_truth(x):
+    """(g', |s| + |x s (1 - s) v|) of the tanh-form GELU in float64: g' = s (1 + x (1 - s) v),
+    s = 1 / (1 + exp(-2u)), 1 - s = 1 / (1 + exp(2u)), v = 2 u'."""
+    x = np.asarray(x, np.float64)
+    c, a = np.sqrt(2.0 / np.pi), 0.044715
+    u2 = 2.0 * c * (x + a * x ** 3)
+    with np.errstate(over="ignore"):
+        s, cs = 1.0 / (1.0 + np.exp(-u2)), 1.0 / (1.0 + np.exp(u2))
+    v = 2.0 * c * (1.0 + 3.0 * a * x * x)
+    return s * (1.0 + x * cs * v), np.abs(s) + np.abs(x * s * cs * v)
+
+
+def test_gelu_gradient_core(M):
+    """gelu_tanh_grad_f against float64 on a dense sweep of [-17, 17] (2^21 points, plus every power of
+    two): within 1e-6 of the magnitude of its two terms for |x| <= 4, 1e-5 in the tails (where the
+    rounding of the exponent shows and g' is below 1e-5 or within 1e-5 of 1); exact limits beyond."""
+    x = np.concatenate([np.linspace(-17, 17, 1 << 21), 2.0 ** np.arange(-140, 5), -(2.0 ** np.arange(-140, 5)),
+                        np.nextafter(np.float32(16), np.float32(0)) * np.array([1, -1]), [0.0, -0.0]]).astype(np.float32)
+    got = apply(M, "gelu_grad", x).astype(np.float64)
+    want, mag = gelu_grad_truth(x)
+    # results below the binary32 subnormals round to 0: an absolute floor of a few subnormal steps
+    ratio = np.abs(got - want) / (mag + 2.0 ** -140 / 1e-6)
+    assert np.max(ratio[np.abs(x) <= 4]) <= 1e-6 and np.max(ratio) <= 1e-5
+    f = lambda v: float(apply(M, "gelu_grad", [v])[0])  # noqa: E731
+    assert f(0.0) == 0.5 and f(np.inf) == 1.0 and f(40.0) == 1.0 and f(-40.0) == 0.0 and f(-np.inf) == 0.0
+    assert np.isnan(f(np.nan))
+    # the numerical derivative of the float64 GELU agrees with the closed form the test uses
+    t = np.linspace(-8, 8, 4001)
+    g = lambda z: z / (1.0 + np.exp(-2.0 * np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))  # noqa: E731
+    assert np.max(np.abs((g(t + 1e-6) - g(t - 1e-6)) / 2e-6 - gelu_grad_truth(t)[0])) < 1e-8
