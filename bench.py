@@ -448,6 +448,27 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         measure(f"{name} step, 2^26 parameters, one kernel", ring, lambda s: s[0].step(s[1]), per * N)
     del p0
 
+    # the backward kernels of the fused layers (the next row: backward on the device)
+    x0 = normal([N])
+    ring = ring_of(lambda: (clone(x0), clone(x0)), 8 * N)
+    measure("GELU backward (dout <- dout gelu'(x)), 2^26", ring,
+            lambda s: F.activation_backward("gelu", s[0], s[1], in_place=True), 12 * N)
+    del x0
+    R, Cn = 32768, 1024
+    x0 = normal([R, Cn], 3.0)
+    y0 = F.softmax_fused(x0)
+    ring = ring_of(lambda: (clone(y0), clone(x0)), 8 * R * Cn)
+    measure("softmax backward (32768,1024), one kernel", ring, lambda s: F.softmax_backward(s[0], s[1], in_place=True),
+            12 * R * Cn)
+    del x0, y0
+    R, Cn = 65536, 1024
+    x0, g0 = normal([R, Cn]), normal([Cn])
+    dg, db = T([Cn], initial_element=None), T([Cn], initial_element=None)
+    ring = ring_of(lambda: (clone(x0), clone(x0), T([R, Cn], initial_element=None)), 12 * R * Cn)
+    measure("LayerNorm backward (65536,1024): dx, dgamma, dbeta (three launches)", ring,
+            lambda s: W.nodes.forward("HIP-LayerNorm-Node-backward", s[0], g0, s[1], s[2], dg, db, 1e-5), 12 * R * Cn)
+    del x0, g0, dg, db
+
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),
                     (8192, 768, 3072)):
@@ -516,6 +537,23 @@ def block_forward_ms(W, reps: int = 20, warm: int = 10):
         out[mode + "_graph"] = e0.elapsed_ms(e1) / reps
         g.destroy()
         del keep
+    # forward keeping what the backward reads, then the backward (every fused node's backward,
+    # attention with the probabilities recomputed); stream launches
+    dout = W.HIPTensor.from_numpy(np.random.Generator(np.random.PCG64(7)).standard_normal(x.shape).astype(np.float32))
+
+    def train_step():
+        saved = {}
+        gpt2.block_forward(dx, dparams, mode="fused", saved=saved)
+        return gpt2.block_backward(dout, saved, dparams)
+
+    for _ in range(3):
+        train_step()
+    e0, e1 = W.lib.Event(), W.lib.Event()
+    e0.record()
+    for _ in range(reps):
+        train_step()
+    e1.record()
+    out["fused_forward_and_backward"] = e0.elapsed_ms(e1) / reps
     return out
 
 
@@ -672,7 +710,7 @@ def main():
             flop = 141.7e9
             result["gpt2_block_fwd_ms"] = {k: round(v, 4) for k, v in blk.items()}
             result["gpt2_block_tflops_on_141.7_gflop"] = {
-                k: round(flop / v / 1e9, 1) for k, v in blk.items()}
+                k: round(flop / v / 1e9, 1) for k, v in blk.items() if k != "fused_forward_and_backward"}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
