@@ -135,11 +135,17 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         # (HIP-Linear-Residual-Node, HIP-Linear-Node :gelu, HIP-Linear-Residual-Node)
         x1 = F.linear(ctx, p["w_o"], p["b_o"], residual=x)
         h2 = ln(x1, p["ln2_g"], p["ln2_b"], eps)
-        f = F.linear(h2, p["w_fc"], p["b_fc"], activation="gelu")
-        if saved is not None:
+        if saved is None:
+            f = F.linear(h2, p["w_fc"], p["b_fc"], activation="gelu")
+        else:
+            # the training form: (!gelu-hip (!linear-hip h2 w b)) keeps the pre-activation as the
+            # activation node's saved input (one more pass of 12 B per element forward) where the
+            # :gelu epilogue would recompute it by a whole product backward
             if mode != "fused":
                 raise ValueError("block_forward: saved tensors are kept for mode 'fused'")
-            saved.update(x=x, h=h, qkv=qkv, ctx=ctx, x1=x1, h2=h2, f=f)
+            z = F.linear(h2, p["w_fc"], p["b_fc"])
+            f = F.gelu_fused(z)
+            saved.update(x=x, h=h, qkv=qkv, ctx=ctx, x1=x1, h2=h2, z=z, f=f)
         return F.linear(f, p["w_proj"], p["b_proj"], residual=x1)
     attn = _linear(ctx, p["w_o"], p["b_o"])
     x1 = F.add(x, attn)                                             # residual
@@ -155,7 +161,7 @@ def block_backward(dout: HIPTensor, saved: dict, p: dict, cfg: dict = CONFIG):
     HIP-Linear-Residual-Node, HIP-LayerNorm-Node, HIP-Attention-Node with the probabilities
     recomputed), the gradient adders of the two residual forks as AddNodes.  Returns (dx, grads)
     with `grads` keyed like the parameters."""
-    x, h, qkv, ctx, x1, h2, f = (saved[k] for k in ("x", "h", "qkv", "ctx", "x1", "h2", "f"))
+    x, h, qkv, ctx, x1, h2, z, f = (saved[k] for k in ("x", "h", "qkv", "ctx", "x1", "h2", "z", "f"))
     B, T, D = x.shape
     H = cfg["n_head"]
     hd = D // H
@@ -163,8 +169,9 @@ def block_backward(dout: HIPTensor, saved: dict, p: dict, cfg: dict = CONFIG):
     g = {}
     # out = f . w_proj + b_proj + x1
     df, g["w_proj"], g["b_proj"] = F.linear_backward(f, p["w_proj"], p["b_proj"], dout)
-    # f = gelu(h2 . w_fc + b_fc)
-    dh2, g["w_fc"], g["b_fc"] = F.linear_backward(h2, p["w_fc"], p["b_fc"], df, activation="gelu")
+    # f = gelu(z), z = h2 . w_fc + b_fc  (HIP-Activation-Node on HIP-Linear-Node; df is not needed again)
+    dz = F.activation_backward("gelu", z, df, in_place=True)
+    dh2, g["w_fc"], g["b_fc"] = F.linear_backward(h2, p["w_fc"], p["b_fc"], dz)
     # h2 = LayerNorm(x1); x1 also feeds the residual
     dln2, g["ln2_g"], g["ln2_b"] = F.layer_norm_backward(x1, p["ln2_g"], dh2, eps)
     dx1 = F.add_(dln2, dout)

@@ -89,3 +89,82 @@ def test_attention_backward_full_and_causal(gpu):
                                      ("dv", gv, dv, p.transpose(0, 1, 3, 2) @ np.abs(DO))):
             ratio = np.abs(got.numpy() - want) / np.maximum(mag, 1e-30)
             assert ratio.max() <= 1e-5, (causal, name, ratio.max())
+
+
+def test_linear_backward_with_the_gelu_epilogue(gpu):
+    """HIP-Linear-Node :gelu recomputes Z = X W + B backward: the kernel form and the node-for-node
+    form against float64, each held to 1e-5 of the magnitude its product adds up."""
+    from oracle import gpt2_block_ref as ref
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(77)
+    rows, k, n = 300, 96, 200
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.3).astype(np.float32)
+    b = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    dout = rng.standard_normal((rows, n)).astype(np.float32)
+    X, Wt, B, D = (a.astype(np.float64) for a in (x, w, b, dout))
+    dz = D * ref.gelu_derivative(X @ Wt + B)
+    want = {"dx": dz @ Wt.T, "dw": X.T @ dz, "db": dz.sum(0)}
+    mag = {"dx": np.abs(dz) @ np.abs(Wt.T), "dw": np.abs(X.T) @ np.abs(dz), "db": np.abs(dz).sum(0)}
+    for fused in (True, False):
+        got = dict(zip(("dx", "dw", "db"), F.linear_backward(F.from_numpy(x), F.from_numpy(w), F.from_numpy(b),
+                                                             F.from_numpy(dout), activation="gelu", fused=fused)))
+        for name in want:
+            ratio = np.abs(got[name].numpy() - want[name]) / mag[name]
+            assert ratio.max() <= 1e-5, (fused, name, ratio.max())
+
+
+def test_block_training_steps_follow_the_float64_recipe(gpu):
+    """Four Adam steps on every parameter of a small block (loss = mean squared error against a
+    fixed target): forward keeping the saved tensors, backward, one fused Adam step per parameter.
+    The float64 recipe takes the same steps (Adam as optimizers/impls/adam.lisp:45-117 states it);
+    the loss must fall and the parameters must stay within 2e-4 of the recipe's."""
+    from oracle import gpt2_block_ref as ref
+    W = gpu
+    F = W.functional
+    gpt2 = importlib.import_module("cl-waffe2_amd.gpt2")
+    cfg = dict(batch=2, seq=40, d_model=64, n_head=4, head_dim=16, d_ff=128, eps=1e-5)
+    rng = np.random.default_rng(9)
+    params = gpt2.make_block_params(9, cfg)
+    for k in params:  # weights large enough for visible gradients
+        if k.startswith("w_"):
+            params[k] = (rng.standard_normal(params[k].shape) * 0.15).astype(np.float32)
+    x = gpt2.make_block_input(9, cfg)
+    target = rng.standard_normal(x.shape).astype(np.float32)
+    lr, b1, b2, eps = 1e-2, 0.9, 0.999, 1e-7
+
+    # float64 recipe
+    P = {k: v.astype(np.float64) for k, v in params.items()}
+    M = {k: np.zeros_like(v) for k, v in P.items()}
+    V = {k: np.zeros_like(v) for k, v in P.items()}
+    ref_losses = []
+    for step in range(1, 5):
+        out = ref.block_forward(x, P, cfg["n_head"], cfg["eps"])
+        diff = out - target
+        ref_losses.append(float((diff ** 2).mean()))
+        grads, _ = ref.block_backward(x, P, cfg["n_head"], 2.0 * diff / diff.size, cfg["eps"])
+        lr_t = lr * np.sqrt(1.0 - b2 ** step) / (1.0 - b1 ** step)
+        for k in P:
+            M[k] += (1.0 - b1) * (grads[k] - M[k])
+            V[k] += (1.0 - b2) * (grads[k] * grads[k] - V[k])
+            P[k] -= lr_t * M[k] / (np.sqrt(V[k]) + eps)
+
+    # the device
+    dp = gpt2.to_device(params)
+    opt = {k: W.optimizers.Adam(dp[k], lr=lr, eps=eps, beta1=b1, beta2=b2) for k in dp}
+    dx, dt = F.from_numpy(x), F.from_numpy(target)
+    losses = []
+    for step in range(4):
+        saved = {}
+        out = gpt2.block_forward(dx, dp, mode="fused", cfg=cfg, saved=saved)
+        diff = F.sub(out, dt)
+        losses.append(float(F.mean(F.mul(diff, diff)).numpy().ravel()[0]))
+        dout = F.mul(diff, 2.0 / diff.size)
+        _, grads = gpt2.block_backward(dout, saved, dp, cfg=cfg)
+        for k in dp:
+            opt[k].step(grads[k])
+    assert losses[-1] < losses[0]
+    np.testing.assert_allclose(losses, ref_losses, rtol=1e-4)
+    for k in dp:
+        np.testing.assert_allclose(dp[k].numpy(), P[k], rtol=0, atol=2e-4, err_msg=k)
