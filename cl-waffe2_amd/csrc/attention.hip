@@ -56,6 +56,7 @@ struct AttnParams {
   int32_t qblocks;
   int32_t causal;
   float scale_log2e;
+  float* lse;  // optional: log2 of the row sums of exp2(scores), (batch * heads, seq); what the backward needs
 };
 
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_kernel(
@@ -261,6 +262,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 
   const float total = lsum + __shfl_xor(lsum, 32);
   const float inv = 1.0f / total;
+  if (p.lse != nullptr && half == 0 && query < p.seq)
+    p.lse[(int64_t)bh * p.seq + query] = m + __builtin_amdgcn_logf(total);  // v_log_f32: log2
   if (query < p.seq) {
     float* op = p.o + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
     // register i of o0 / o1 holds head dimension 2 r / 2 r + 1, r = 8 (i/4) + 4 half + i%4:
@@ -276,6 +279,288 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   }
 }
 
+// ---- backward ---------------------------------------------------------------------------------
+// dQ, dK, dV of O = softmax(scale Q K^T + mask) V from Q, K, V, dO and two numbers per query
+// the forward pass leaves behind or that are cheap to form: L = log2 sum_j exp2(scores) (so that
+// P = exp2(S - L) needs no second pass over the keys) and D = sum_d dO O = sum_j P dP.  Per tile
+//   S = scale log2e Q K^T,  P = exp2(S - L),  dP = dO V^T,  dS = P (dP - D),
+//   dQ += scale dS K,   dK += scale dS^T Q,   dV += P^T dO,
+// and no (seq, seq) tensor is ever written.  One kernel body serves two launches:
+//   KEYS = false  a lane owns a QUERY (Q and dO rows in registers), key / value tiles stream
+//                 through LDS, the accumulator is dQ            (the forward kernel's frame);
+//   KEYS = true   a lane owns a KEY (K and V rows in registers), query / dO tiles stream, the
+//                 accumulators are dK and dV; L and D of the streamed queries come with the tile.
+// Either way the two score-shaped tiles are (streamed tile) . (resident rows)^T, whose accumulator
+// registers are exactly the B operand of (streamed tile)^T . (scores), as in the forward kernel,
+// so dS and P never leave the registers either.  Seven products in all where five are the
+// minimum: S and dP are formed by both launches.
+// Both streamed tiles use the key layout of the forward kernel (16-byte slots XOR row % 16); the
+// 64-bit reads of the accumulation step go through the same permutation.
+struct AttnBwdParams {
+  const float* q;
+  const float* k;
+  const float* v;
+  const float* dout;
+  const float* lse;    // (batch * heads, seq), log2 domain, from the forward kernel
+  const float* delta;  // (batch * heads, seq)
+  float* dq;
+  float* dk;
+  float* dv;
+  int64_t qs[3], ks[3], vs[3], os[3];  // dq, dk, dv are addressed like q, k, v; dout like o
+  int32_t batch, heads, seq, head_dim;
+  int32_t rblocks;  // blocks of 128 resident rows per head
+  int32_t causal;
+  float scale_log2e, scale;
+};
+
+constexpr int kBwdStageFloats = 2 * kKBlock * kRowFloats;  // two tiles of 64 rows
+constexpr int kBwdStatFloats = 2 * kKBlock;                // L and D of 64 streamed queries
+constexpr size_t kAttnBwdLdsBytes = 2 * (size_t)(kBwdStageFloats + kBwdStatFloats) * sizeof(float);  // 66,560 B
+
+// D[b, h, t] = sum_d dO[b, h, t, d] O[b, h, t, d]; sixteen lanes per row.
+__global__ __launch_bounds__(kBlock) void attention_delta_kernel(const float* __restrict__ o,
+                                                                 const float* __restrict__ dout, int64_t s0,
+                                                                 int64_t s1, int64_t s2, int32_t heads, int32_t seq,
+                                                                 int32_t head_dim, int64_t rows,
+                                                                 float* __restrict__ delta) {
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t row = gid >> 4;
+  const int sub = (int)(gid & 15);
+  float acc = 0.0f;
+  if (row < rows && sub * 4 < head_dim) {
+    const int64_t bh = row / seq;
+    const int64_t t = row - bh * seq;
+    const int64_t b = bh / heads;
+    const int64_t h = bh - b * heads;
+    const int64_t off = b * s0 + h * s1 + t * s2 + sub * 4;
+    const f4 x = *reinterpret_cast<const f4*>(o + off);
+    const f4 y = *reinterpret_cast<const f4*>(dout + off);
+    acc = __builtin_fmaf(x.x, y.x, __builtin_fmaf(x.y, y.y, __builtin_fmaf(x.z, y.z, x.w * y.w)));
+  }
+#pragma unroll
+  for (int d = 8; d > 0; d >>= 1) acc += __shfl_xor(acc, d);
+  if (row < rows && sub == 0) delta[row] = acc;
+}
+
+template <bool KEYS>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_bwd_kernel(
+    AttnBwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  auto tile1 = [&](int stage) { return smem + stage * kBwdStageFloats; };
+  auto tile2 = [&](int stage) { return smem + stage * kBwdStageFloats + kKBlock * kRowFloats; };
+  float* const stats = smem + 2 * kBwdStageFloats;  // [stage][L: 64, D: 64]
+
+  // longest first: the last query block walks the most key tiles, the first key block the most query tiles
+  const int nbh = p.batch * p.heads;
+  const int rank = blockIdx.x / nbh;
+  const int bh = blockIdx.x - rank * nbh;
+  const int rb = KEYS ? rank : p.rblocks - 1 - rank;
+  const int b = bh / p.heads;
+  const int h = bh - b * p.heads;
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int half = lane >> 5;
+  const int col = lane & 31;
+
+  const int r_first = rb * kQBlock + wave * 32;  // first resident row of this wavefront
+  const int row = r_first + col;                 // this lane's query (KEYS false) or key (KEYS true)
+  const int row_ld = row < p.seq ? row : p.seq - 1;
+
+  const float* res1 = KEYS ? p.k + b * p.ks[0] + h * p.ks[1] + (int64_t)row_ld * p.ks[2]
+                           : p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)row_ld * p.qs[2];
+  const float* res2 = KEYS ? p.v + b * p.vs[0] + h * p.vs[1] + (int64_t)row_ld * p.vs[2]
+                           : p.dout + b * p.os[0] + h * p.os[1] + (int64_t)row_ld * p.os[2];
+  const float* str1 = KEYS ? p.q + b * p.qs[0] + h * p.qs[1] : p.k + b * p.ks[0] + h * p.ks[1];
+  const float* str2 = KEYS ? p.dout + b * p.os[0] + h * p.os[1] : p.v + b * p.vs[0] + h * p.vs[1];
+  const int64_t pitch1 = KEYS ? p.qs[2] : p.ks[2];
+  const int64_t pitch2 = KEYS ? p.os[2] : p.vs[2];
+  (void)str1;
+  (void)str2;
+  (void)pitch1;
+  (void)pitch2;  // only the device pass reads them (global -> LDS builtin)
+  const float* lse = p.lse + (int64_t)bh * p.seq;
+  const float* delta = p.delta + (int64_t)bh * p.seq;
+
+  // resident fragments: a[4 j + r] = X[row][8 j + 4 half + r]; the first one carries scale * log2(e)
+  float a1[32], a2[32];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    f4 t = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
+    if (8 * j + 4 * half < p.head_dim) {
+      t = *reinterpret_cast<const f4*>(res1 + 8 * j + 4 * half);
+      u = *reinterpret_cast<const f4*>(res2 + 8 * j + 4 * half);
+    }
+    a1[4 * j + 0] = t.x * p.scale_log2e;
+    a1[4 * j + 1] = t.y * p.scale_log2e;
+    a1[4 * j + 2] = t.z * p.scale_log2e;
+    a1[4 * j + 3] = t.w * p.scale_log2e;
+    a2[4 * j + 0] = u.x;
+    a2[4 * j + 1] = u.y;
+    a2[4 * j + 2] = u.z;
+    a2[4 * j + 3] = u.w;
+  }
+  float l_res = 0.f, d_res = 0.f;
+  if (!KEYS) {
+    l_res = lse[row_ld];
+    d_res = delta[row_ld];
+  }
+
+  // streamed tiles of 64 rows: keys 0 .. diagonal (KEYS false), queries diagonal .. end (KEYS true)
+  const int tiles = (p.seq + kKBlock - 1) / kKBlock;
+  int t_begin = 0, t_end = tiles;
+  if (p.causal) {
+    if (KEYS) {
+      t_begin = (rb * kQBlock) / kKBlock;
+    } else {
+      const int key_end = min(rb * kQBlock + kQBlock, p.seq);
+      t_end = (key_end + kKBlock - 1) / kKBlock;
+    }
+  }
+
+  float stat_value = 0.f;
+  auto fetch = [&](int stage, int tile) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int row0 = tile * kKBlock;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int q4 = wave * 4 + j;
+      const int r = q4 * 4 + (lane >> 4);
+      const int slot = lane & 15;
+      int srow = row0 + r;
+      srow = srow < p.seq ? srow : p.seq - 1;
+      const int chunk = slot ^ (r & 15);
+      if (chunk * 4 < p.head_dim) {
+        __builtin_amdgcn_global_load_lds(str1 + (int64_t)srow * pitch1 + chunk * 4, tile1(stage) + q4 * 256, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(str2 + (int64_t)srow * pitch2 + chunk * 4, tile2(stage) + q4 * 256, 16, 0, 0);
+      }
+    }
+    if (KEYS && wave < 2) {  // L (wavefront 0) and D (wavefront 1) of the tile's 64 queries, parked in a register
+      int srow = row0 + lane;
+      srow = srow < p.seq ? srow : p.seq - 1;
+      stat_value = wave == 0 ? lse[srow] : delta[srow];
+    }
+#endif
+  };
+  // ... and written to LDS only after the arithmetic of the current tile, so that waiting for that
+  // load does not also wait for the tile loads issued before it
+  auto publish = [&](int stage) {
+    if (KEYS && wave < 2) stats[stage * kBwdStatFloats + wave * kKBlock + lane] = stat_value;
+  };
+  if (p.head_dim < kHeadDim) {
+    for (int i = threadIdx.x; i < 2 * kBwdStageFloats / 4; i += kBlock)
+      reinterpret_cast<f4*>(smem)[i] = f4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+  }
+
+  f16v g1a = {0}, g1b = {0};  // dQ (KEYS false) or dK (KEYS true): even / odd head dimensions
+  f16v g2a = {0}, g2b = {0};  // dV (KEYS true)
+  const int kswz = col & 15;
+  typedef float f2 __attribute__((ext_vector_type(2)));
+
+  auto compute = [&](int stage, int tile) {
+    const float* s1 = tile1(stage);
+    const float* s2 = tile2(stage);
+    const float* st = stats + stage * kBwdStatFloats;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const int s_first = tile * kKBlock + 32 * t;  // first streamed row of this 32-row sub-tile
+      bool active = s_first < p.seq;
+      if (p.causal) active = active && (KEYS ? s_first + 31 >= r_first : s_first <= r_first + 31);
+      if (!active) continue;  // uniform over the wavefront
+      f16v sc, dp;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        sc[i] = 0.f;
+        dp[i] = 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int slot = ((2 * j + half) ^ kswz) * 4;
+        const f4 x1 = *reinterpret_cast<const f4*>(s1 + (32 * t + col) * kRowFloats + slot);
+        const f4 x2 = *reinterpret_cast<const f4*>(s2 + (32 * t + col) * kRowFloats + slot);
+        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, a1[4 * j + 0], sc, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, a2[4 * j + 0], dp, 0, 0, 0);
+        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, a1[4 * j + 1], sc, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, a2[4 * j + 1], dp, 0, 0, 0);
+        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.z, a1[4 * j + 2], sc, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.z, a2[4 * j + 2], dp, 0, 0, 0);
+        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.w, a1[4 * j + 3], sc, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.w, a2[4 * j + 3], dp, 0, 0, 0);
+      }
+      // register i holds streamed row s_first + 8 (i/4) + 4 half + i%4 against resident row `row`
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f4 lvals = {l_res, l_res, l_res, l_res}, dvals = {d_res, d_res, d_res, d_res};
+        if (KEYS) {
+          lvals = *reinterpret_cast<const f4*>(st + 32 * t + 8 * g + 4 * half);
+          dvals = *reinterpret_cast<const f4*>(st + kKBlock + 32 * t + 8 * g + 4 * half);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const int i = 4 * g + c;
+          const int srow = s_first + 8 * g + 4 * half + c;
+          const int query = KEYS ? srow : row;
+          const int key = KEYS ? row : srow;
+          const bool visible = srow < p.seq && (!p.causal || key <= query);
+          const float pe = visible ? __builtin_amdgcn_exp2f(sc[i] - lvals[c]) : 0.f;
+          sc[i] = pe;
+          dp[i] = pe * (dp[i] - dvals[c]);
+        }
+      }
+      // (streamed tile)^T . dS and, with resident keys, (dO tile)^T . P
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int lr = 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
+        const int pos = (col >> 1) ^ (lr & 15);
+        const int off = lr * kRowFloats + pos * 4 + 2 * (col & 1);
+        const f2 x1 = *reinterpret_cast<const f2*>(s1 + off);
+        g1a = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, dp[i], g1a, 0, 0, 0);
+        g1b = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, dp[i], g1b, 0, 0, 0);
+        if (KEYS) {
+          const f2 x2 = *reinterpret_cast<const f2*>(s2 + off);
+          g2a = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, sc[i], g2a, 0, 0, 0);
+          g2b = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, sc[i], g2b, 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // two stages: the next tile is fetched while this one is worked on; one barrier per tile
+  fetch(t_begin & 1, t_begin);
+  publish(t_begin & 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int tile = t_begin; tile < t_end; tile++) {
+    const bool more = tile + 1 < t_end;
+    if (more) fetch((tile + 1) & 1, tile + 1);
+    compute(tile & 1, tile);
+    if (more) publish((tile + 1) & 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's fetches have landed
+    __syncthreads();
+  }
+
+  auto write = [&](float* out, const f16v& ea, const f16v& eb, float factor) {
+    // register i of ea / eb holds head dimension 2 r / 2 r + 1, r = 8 (i/4) + 4 half + i%4
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const int d0 = 16 * g + 8 * half;
+      f4 x = {ea[4 * g] * factor, eb[4 * g] * factor, ea[4 * g + 1] * factor, eb[4 * g + 1] * factor};
+      f4 y = {ea[4 * g + 2] * factor, eb[4 * g + 2] * factor, ea[4 * g + 3] * factor, eb[4 * g + 3] * factor};
+      if (d0 < p.head_dim) *reinterpret_cast<f4*>(out + d0) = x;
+      if (d0 + 4 < p.head_dim) *reinterpret_cast<f4*>(out + d0 + 4) = y;
+    }
+  };
+  if (row < p.seq) {
+    if (KEYS) {
+      write(p.dk + b * p.ks[0] + h * p.ks[1] + (int64_t)row * p.ks[2], g1a, g1b, p.scale);
+      write(p.dv + b * p.vs[0] + h * p.vs[1] + (int64_t)row * p.vs[2], g2a, g2b, 1.0f);
+    } else {
+      write(p.dq + b * p.qs[0] + h * p.qs[1] + (int64_t)row * p.qs[2], g1a, g1b, p.scale);
+    }
+  }
+}
+
 // [lo, hi) in elements touched through (batch, head, position) strides
 static void extent3(const float* base, const int64_t (&s)[3], int64_t nb, int64_t nh, int64_t nt,
                     int64_t head_dim, const float** lo, const float** hi) {
@@ -287,24 +572,20 @@ static void extent3(const float* base, const int64_t (&s)[3], int64_t nb, int64_
 
 using namespace wf2;
 
-WF2_API int wf2hip_attention_f32(const wf2hip_attention_desc* d, const float* q, const float* k,
-                                 const float* v, float* o) {
-  WF2_TRY(require_init());
-  if (!d || !q || !k || !v || !o) return fail(WF2HIP_EINVAL, "attention: null argument");
+// Checks shared by the forward and the backward entry: extents, alignment, strides.  `ptrs` are the
+// tensors addressed through q / k / v / o strides, in that order (nullptr entries are skipped).
+static int load_attention_desc(const wf2hip_attention_desc* d, const void* const (&ptrs)[4], int64_t (&qs)[3],
+                               int64_t (&ks)[3], int64_t (&vs)[3], int64_t (&os)[3]) {
   if (d->head_dim < 4 || d->head_dim > kHeadDim || d->head_dim % 4 != 0)
     return fail(WF2HIP_EUNSUPPORTED, "attention: head_dim %ld (multiples of 4 up to 64 are built)",
                 (long)d->head_dim);
   if (d->batch < 0 || d->heads < 0 || d->seq < 0)
     return fail(WF2HIP_EINVAL, "attention: negative extent");
-  if (d->batch == 0 || d->heads == 0 || d->seq == 0) return 0;
   if (d->seq > (1 << 24) || d->batch * d->heads > (1 << 20))
     return fail(WF2HIP_EUNSUPPORTED, "attention: extents beyond one launch");
   if (d->causal != 0 && d->causal != 1) return fail(WF2HIP_EINVAL, "attention: causal must be 0 or 1");
-  AttnParams p;
-  p.q = q; p.k = k; p.v = v; p.o = o;
   const int64_t* strides[4] = {d->q_stride, d->k_stride, d->v_stride, d->o_stride};
-  int64_t* dst[4] = {p.qs, p.ks, p.vs, p.os};
-  const void* ptrs[4] = {q, k, v, o};
+  int64_t* dst[4] = {qs, ks, vs, os};
   for (int t = 0; t < 4; t++) {
     if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0)
       return fail(WF2HIP_EINVAL, "attention: operands must be 16-byte aligned");
@@ -314,6 +595,19 @@ WF2_API int wf2hip_attention_f32(const wf2hip_attention_desc* d, const float* q,
       dst[t][a] = strides[t][a];
     }
   }
+  return 0;
+}
+
+WF2_API int wf2hip_attention_forward_f32(const wf2hip_attention_desc* d, const float* q, const float* k,
+                                         const float* v, float* o, float* lse) {
+  WF2_TRY(require_init());
+  if (!d || !q || !k || !v || !o) return fail(WF2HIP_EINVAL, "attention: null argument");
+  AttnParams p;
+  p.q = q; p.k = k; p.v = v; p.o = o;
+  p.lse = lse;
+  const void* const ptrs[4] = {q, k, v, o};
+  WF2_TRY(load_attention_desc(d, ptrs, p.qs, p.ks, p.vs, p.os));
+  if (d->batch == 0 || d->heads == 0 || d->seq == 0) return 0;
   // the output must be a dense-enough set of rows of its own: no two (batch, head,
   // position) triples may share storage, and it may not alias an input
   if (p.os[2] < d->head_dim && d->seq > 1) return fail(WF2HIP_EINVAL, "attention: output rows overlap");
@@ -325,6 +619,11 @@ WF2_API int wf2hip_attention_f32(const wf2hip_attention_desc* d, const float* q,
     const float *lo, *hi;
     extent3(ins[t], *ist[t], d->batch, d->heads, d->seq, d->head_dim, &lo, &hi);
     if (lo < ohi && olo < hi) return fail(WF2HIP_EOVERLAP, "attention: output overlaps an input");
+  }
+  if (lse != nullptr) {
+    const float* llo = lse;
+    const float* lhi = lse + d->batch * d->heads * d->seq;
+    if (llo < ohi && olo < lhi) return fail(WF2HIP_EOVERLAP, "attention: the row statistics overlap the output");
   }
   p.batch = (int32_t)d->batch;
   p.heads = (int32_t)d->heads;
@@ -345,4 +644,88 @@ WF2_API int wf2hip_attention_f32(const wf2hip_attention_desc* d, const float* q,
   }
   attention_kernel<<<(uint32_t)blocks, kBlock, kAttnLdsBytes, rt().stream>>>(p);
   return after_launch("attention_kernel");
+}
+
+WF2_API int wf2hip_attention_f32(const wf2hip_attention_desc* d, const float* q, const float* k,
+                                 const float* v, float* o) {
+  return wf2hip_attention_forward_f32(d, q, k, v, o, nullptr);
+}
+
+WF2_API int wf2hip_attention_backward_f32(const wf2hip_attention_desc* d, const float* q, const float* k,
+                                          const float* v, const float* o, const float* dout, const float* lse,
+                                          float* dq, float* dk, float* dv) {
+  WF2_TRY(require_init());
+  if (!d || !q || !k || !v || !o || !dout || !lse || !dq || !dk || !dv)
+    return fail(WF2HIP_EINVAL, "attention backward: null argument");
+  AttnBwdParams p;
+  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse;
+  p.dq = dq; p.dk = dk; p.dv = dv;
+  const void* const ptrs[4] = {q, k, v, o};
+  WF2_TRY(load_attention_desc(d, ptrs, p.qs, p.ks, p.vs, p.os));
+  const void* const more[6] = {dout, dq, dk, dv, lse, nullptr};
+  for (int t = 0; t < 4; t++)
+    if (reinterpret_cast<uintptr_t>(more[t]) % 16 != 0)
+      return fail(WF2HIP_EINVAL, "attention backward: operands must be 16-byte aligned");
+  if (d->batch == 0 || d->heads == 0 || d->seq == 0) return 0;
+  // gradients are addressed like the tensors they belong to; their rows may not share storage,
+  // and none of them may overlap anything that is read
+  const float* outs[3] = {dq, dk, dv};
+  const int64_t(*ost[3])[3] = {&p.qs, &p.ks, &p.vs};
+  const float* ins[5] = {q, k, v, o, dout};
+  const int64_t(*ist[5])[3] = {&p.qs, &p.ks, &p.vs, &p.os, &p.os};
+  for (int t = 0; t < 3; t++) {
+    if ((*ost[t])[2] < d->head_dim && d->seq > 1)
+      return fail(WF2HIP_EINVAL, "attention backward: gradient rows overlap");
+    const float *olo, *ohi;
+    extent3(outs[t], *ost[t], d->batch, d->heads, d->seq, d->head_dim, &olo, &ohi);
+    for (int u = 0; u < 5; u++) {
+      const float *lo, *hi;
+      extent3(ins[u], *ist[u], d->batch, d->heads, d->seq, d->head_dim, &lo, &hi);
+      if (lo < ohi && olo < hi) return fail(WF2HIP_EOVERLAP, "attention backward: a gradient overlaps an input");
+    }
+    const float* lhi = lse + d->batch * d->heads * d->seq;
+    if (lse < ohi && olo < lhi) return fail(WF2HIP_EOVERLAP, "attention backward: a gradient overlaps the row statistics");
+    for (int u = t + 1; u < 3; u++)
+      if (outs[t] == outs[u]) return fail(WF2HIP_EOVERLAP, "attention backward: two gradients share storage");
+  }
+  p.batch = (int32_t)d->batch;
+  p.heads = (int32_t)d->heads;
+  p.seq = (int32_t)d->seq;
+  p.head_dim = (int32_t)d->head_dim;
+  p.rblocks = (int32_t)ceil_div(d->seq, kQBlock);
+  p.causal = d->causal;
+  p.scale = d->scale;
+  p.scale_log2e = d->scale * 1.44269504088896340736f;
+  const int64_t blocks = (int64_t)p.rblocks * p.batch * p.heads;
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "attention backward: too many workgroups");
+  static bool configured = false;
+  if (!configured) {
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_kernel<false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAttnBwdLdsBytes),
+                      "hipFuncSetAttribute(attention_bwd_kernel<false>)"));
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_kernel<true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAttnBwdLdsBytes),
+                      "hipFuncSetAttribute(attention_bwd_kernel<true>)"));
+    configured = true;
+  }
+  const int64_t rows = d->batch * d->heads * d->seq;
+  if (ceil_div(rows * 16, kBlock) >= ((int64_t)1 << 31))
+    return fail(WF2HIP_EUNSUPPORTED, "attention backward: too many rows for one launch");
+  void* delta = nullptr;
+  WF2_TRY(wf2hip_malloc_uninitialized(&delta, (size_t)rows * sizeof(float)));
+  p.delta = static_cast<const float*>(delta);
+  hipStream_t st = rt().stream;
+  attention_delta_kernel<<<(uint32_t)ceil_div(rows * 16, kBlock), kBlock, 0, st>>>(
+      o, dout, p.os[0], p.os[1], p.os[2], p.heads, p.seq, p.head_dim, rows, static_cast<float*>(delta));
+  int rc = after_launch("attention_delta_kernel");
+  if (rc == 0) {
+    attention_bwd_kernel<false><<<(uint32_t)blocks, kBlock, kAttnBwdLdsBytes, st>>>(p);
+    rc = after_launch("attention_bwd_kernel<false>");
+  }
+  if (rc == 0) {
+    attention_bwd_kernel<true><<<(uint32_t)blocks, kBlock, kAttnBwdLdsBytes, st>>>(p);
+    rc = after_launch("attention_bwd_kernel<true>");
+  }
+  (void)wf2hip_free(delta);  // stream order keeps it alive for the launches above
+  return rc;
 }

@@ -629,7 +629,7 @@ def linear(x: HIPTensor, w: HIPTensor, b: HIPTensor, activation: str | None = No
 
 
 def attention(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor | None = None,
-              scale: float | None = None, causal: bool = False) -> HIPTensor:
+              scale: float | None = None, causal: bool = False, lse: HIPTensor | None = None) -> HIPTensor:
     """softmax(scale q k^T [+ causal mask]) v for (batch, heads, seq, 64) views in
     one kernel (HIP-Attention-Node; ``!attention-hip`` of the Lisp glue): the fused form of
     SelfAttention's !matmul / !softmax / !matmul chain (``examples/gpt-2/utils.lisp:222-243``).
@@ -643,7 +643,7 @@ def attention(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor | None = 
     if out is None:
         out = HIPTensor([B, H, T, hd], initial_element=None)
     return nodes.forward("HIP-Attention-Node", q, k, v, out, 1.0 / math.sqrt(hd) if scale is None else scale,
-                         causal)
+                         causal, lse)
 
 
 def gelu(x: HIPTensor) -> HIPTensor:
@@ -796,16 +796,30 @@ def softmax_backward(y: HIPTensor, dout: HIPTensor, scale: float = 1.0, causal: 
 
 def attention_backward(q: HIPTensor, k: HIPTensor, v: HIPTensor, dout: HIPTensor, scale: float | None = None,
                        causal: bool = False, dq: HIPTensor | None = None, dk: HIPTensor | None = None,
-                       dv: HIPTensor | None = None, fused: bool = True):
+                       dv: HIPTensor | None = None, fused: bool = True, out: HIPTensor | None = None,
+                       lse: HIPTensor | None = None):
     """(dq, dk, dv) of HIP-Attention-Node with the probabilities recomputed, as its :backward
     composes them: P = softmax(scale Q K^T [+ mask]), dV = P^T dO, dP = dO V^T,
     dS = scale P (dP - sum_j dP P), dQ = dS K, dK = dS^T Q.  Operands are
     (batch, heads, seq, head_dim) views whose last axis is contiguous; the optional outputs may be
     such views too (windows of one fused-projection gradient).  With a mask the two score-shaped
     products form their lower triangles only and dS K skips the tiles above the diagonal.
-    ``fused=False`` takes the softmax gradient node for node and every product in full."""
+    ``fused=False`` takes the softmax gradient node for node and every product in full.
+    With the forward pass's output ``out`` and row statistics ``lse`` (`attention(..., lse=)`) the
+    whole backward is HIP-Attention-Node-backward instead: three launches, no (seq, seq) tensor."""
     hd = q.shape[-1]
     scale = 1.0 / math.sqrt(hd) if scale is None else float(scale)
+    if out is not None and lse is not None:
+        dq, dk, dv = (HIPTensor(list(t.shape), initial_element=None) if g is None else g
+                      for t, g in ((q, dq), (k, dk), (v, dv)))
+        same = lambda a, b: a.geometry()[1] == b.geometry()[1]  # noqa: E731
+        if same(dout, out) and same(dq, q) and same(dk, k) and same(dv, v):
+            return nodes.forward("HIP-Attention-Node-backward", q, k, v, out, dout, lse, dq, dk, dv, scale, causal)
+        # operands laid out differently from the tensors they belong to: contiguous copies
+        qc, kc, vc, oc, dc = (to_contiguous(t) for t in (q, k, v, out, dout))
+        gq, gk, gv = (HIPTensor(list(q.shape), initial_element=None) for _ in range(3))
+        nodes.forward("HIP-Attention-Node-backward", qc, kc, vc, oc, dc, lse, gq, gk, gv, scale, causal)
+        return move_(dq, gq), move_(dk, gk), move_(dv, gv)
     tri = 1 if (causal and fused) else 0
     s = matmul(q, t(k), causal=tri)
     if causal:

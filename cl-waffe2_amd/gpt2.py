@@ -106,8 +106,12 @@ def block_forward(x: HIPTensor, p: dict, mode: str = "fused", cfg: dict = CONFIG
         q, k, v = (four.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3)
                    for i in range(3))
         ctx_store = HIPTensor([B, T, H, hd], initial_element=None)
-        F.attention(q, k, v, out=ctx_store.permute(0, 2, 1, 3), scale=scale, causal=True)
+        # training: the row statistics the attention node's backward reads
+        lse = HIPTensor([B, H, T], initial_element=None) if saved is not None else None
+        F.attention(q, k, v, out=ctx_store.permute(0, 2, 1, 3), scale=scale, causal=True, lse=lse)
         ctx = F.reshape(ctx_store, B, T, D)
+        if saved is not None:
+            saved["lse"] = lse
     elif fused:
         five = F.reshape(qkv, B, T, 3, H, hd)
         # (B, 1, H, T, hd) strided windows of the projection, no copy
@@ -184,7 +188,11 @@ def block_backward(dout: HIPTensor, saved: dict, p: dict, cfg: dict = CONFIG):
     dqkv = HIPTensor([B, T, 3 * H, hd], initial_element=None)
     dq, dk, dv = (dqkv.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3) for i in range(3))
     dctx_heads = F.reshape(dctx, B, T, H, hd).permute(0, 2, 1, 3)
-    F.attention_backward(q, k, v, dctx_heads, scale=1.0 / math.sqrt(hd), causal=True, dq=dq, dk=dk, dv=dv)
+    # with the forward's row statistics: one node, no (B, H, T, T) tensor; without them (heads the
+    # attention kernel does not take): the composition with the probabilities recomputed
+    F.attention_backward(q, k, v, dctx_heads, scale=1.0 / math.sqrt(hd), causal=True, dq=dq, dk=dk, dv=dv,
+                         out=F.reshape(ctx, B, T, H, hd).permute(0, 2, 1, 3) if "lse" in saved else None,
+                         lse=saved.get("lse"))
     # qkv = h . w_qkv + b_qkv
     dh, g["w_qkv"], g["b_qkv"] = F.linear_backward(h, p["w_qkv"], p["b_qkv"], F.reshape(dqkv, B, T, 3 * D))
     # h = LayerNorm(x); x also feeds the residual

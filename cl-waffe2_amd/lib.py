@@ -29,6 +29,7 @@ EQ, LT, LE, GT, GE = 0, 1, 2, 3, 4  # enum wf2hip_compare_op
 COMPARE_NAMES = ("eq", "lt", "le", "gt", "ge")
 MAXVALUE, MINVALUE, ARGMAX, ARGMIN = 48, 49, 50, 51  # enum wf2hip_select_op
 
+EINVAL = -1
 EOVERLAP = -3
 EUNSUPPORTED = -4
 ECAPTURE = -6
@@ -190,6 +191,8 @@ _SIGNATURES = {
     "wf2hip_sgd_step_f32": ([_L, _P, _P, _F], C.c_int),
     "wf2hip_adam_step_f32": ([_L, _P, _P, _P, _P, _F, _F, _F, _F], C.c_int),
     "wf2hip_attention_f32": ([C.POINTER(AttentionDesc), _P, _P, _P, _P], C.c_int),
+    "wf2hip_attention_forward_f32": ([C.POINTER(AttentionDesc), _P, _P, _P, _P, _P], C.c_int),
+    "wf2hip_attention_backward_f32": ([C.POINTER(AttentionDesc)] + [_P] * 9, C.c_int),
     "wf2hip_sgemm_strided_batched_2d": (
         [C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _L, _L, _P, _L, _L, _L, _F, _P, _L, _L, _L, _L, _L],
         C.c_int,

@@ -138,6 +138,9 @@
   (scale :float) (causal :int32))
 (defcfun "wf2hip_attention_f32" :int
   (desc (:pointer (:struct attention-desc))) (q :pointer) (k :pointer) (v :pointer) (o :pointer))
+(defcfun "wf2hip_attention_forward_f32" :int (desc :pointer) (q :pointer) (k :pointer) (v :pointer) (o :pointer) (lse :pointer))
+(defcfun "wf2hip_attention_backward_f32" :int (desc :pointer) (q :pointer) (k :pointer) (v :pointer) (o :pointer)
+  (dout :pointer) (lse :pointer) (dq :pointer) (dk :pointer) (dv :pointer))
 (defcfun "wf2hip_causal_softmax_f32" :int (matrices :long) (seq :long) (x :pointer) (out :pointer) (scale :float))
 
 (defcfun "wf2hip_im2col_f32" :int

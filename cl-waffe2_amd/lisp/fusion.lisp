@@ -6,7 +6,7 @@
 ;;;; the reference intends device-specific fusions to be added:
 ;;;;   * a define-op node per fused kernel (as Softmax-Cross-Entropy-Node, source/nn/criterion.lisp:90),
 ;;;;     forward = one library call; backward = one library call too where the library holds the
-;;;;     gradient as a kernel (activations, softmax, causal softmax, LayerNorm), otherwise the
+;;;;     gradient as a kernel (activations, softmax, causal softmax, LayerNorm, attention), otherwise the
 ;;;;     derivative composed from ordinary ! functions and evaluated with proceed, so it runs on
 ;;;;     the device through the nodes of kernels.lisp (a graph is compiled per such backward call;
 ;;;;     a defmodel-as cache is the next step);
@@ -452,39 +452,58 @@ the MulNode by the scale, the AddNode of the mask and !softmax of causal attenti
 (define-op (HIP-Attention-Node (self scale causal)
             :slots ((scale :initform 1.0 :accessor attention-scale)
                     (causal :initform nil :accessor attention-causal))
-            :save-for-backward-names (q k v)
+            :save-for-backward-names (q k v o lse)
             :where (Q[batch heads seq dim] K[batch heads seq dim] V[batch heads seq dim] OUT[batch heads seq dim]
                     -> OUT[batch heads seq dim])
             :documentation "OUT <- softmax(scale Q K^T [+ causal mask]) V per (batch, head) in one kernel that
-never forms the (seq, seq) score matrices (wf2hip_attention_f32; heads up to 64 wide).  The operands may be
-strided windows of a fused projection (last axis contiguous).  Backward: composed, with the
-probabilities recomputed: dV = P^T dO, dP = dO V^T, dS = scale P (dP - sum_j dP P) (one kernel),
-dQ = dS K, dK = dS^T Q."
+never forms the (seq, seq) score matrices (wf2hip_attention_forward_f32; heads up to 64 wide).  The operands
+may be strided windows of a fused projection (last axis contiguous).  The forward also keeps, per query, the
+base-2 logarithm of its row sum; with it the backward is one library call as well
+(wf2hip_attention_backward_f32: D = sum dO O per query, dQ with queries resident, dK and dV with keys resident;
+no (seq, seq) tensor either).  *compose-backward* selects the composition instead, with the probabilities
+recomputed: dV = P^T dO, dP = dO V^T, dS = scale P (dP - sum_j dP P), dQ = dS K, dK = dS^T Q."
             :forward ((self q k v out)
                       (ensure-extension)
-                      (with-foreign-object (desc '(:struct attention-desc))
-                        (destructuring-bind (oq ok ov oo)
-                            (fill-attention-desc desc q k v out (attention-scale self) (attention-causal self))
-                          (check (wf2hip-attention-f32 desc (tensor-device-pointer q oq) (tensor-device-pointer k ok)
-                                                       (tensor-device-pointer v ov) (tensor-device-pointer out oo)))))
-                      (with-setting-save4bw ((q q) (k k) (v v)) out))
+                      (let ((lse (make-tensor (butlast (shape q)) :dtype :float :order (order q) :device 'HIPTensor)))
+                        (with-foreign-object (desc '(:struct attention-desc))
+                          (destructuring-bind (oq ok ov oo)
+                              (fill-attention-desc desc q k v out (attention-scale self) (attention-causal self))
+                            (check (wf2hip-attention-forward-f32 desc
+                                                                 (tensor-device-pointer q oq) (tensor-device-pointer k ok)
+                                                                 (tensor-device-pointer v ov) (tensor-device-pointer out oo)
+                                                                 (tensor-device-pointer lse)))))
+                        (with-setting-save4bw ((q q) (k k) (v v) (o out) (lse lse)) out)))
             :backward ((self dout)
-                       (with-reading-save4bw ((q q) (k k) (v v))
-                         (let* ((scale (attention-scale self))
-                                (s (!matmul q (!t k)))
-                                (p (if (attention-causal self)
-                                       (!causal-softmax-hip s :scale scale)
-                                       (!softmax-hip (!reshape (!mul scale s) t (car (last (shape s)))))))
-                                (p (apply #'!reshape p (shape s)))
-                                (dv (!matmul (!t p) dout))
-                                (dp (!matmul dout (!t v)))
-                                ;; dS carries the factor scale: scale P (dP - sum_j dP P), one kernel
-                                (ds (if *compose-backward*
-                                        (!mul scale (!mul p (!sub dp (!sum-hip (!mul dp p) :axis -1 :keepdims t))))
-                                        (softmax-gradient (proceed p) (proceed dp) scale (attention-causal self))))
-                                (dq (!matmul ds k))
-                                (dk (!matmul (!t ds) q)))
-                           (values (proceed dq) (proceed dk) (proceed dv) nil)))))
+                       (with-reading-save4bw ((q q) (k k) (v v) (o o) (lse lse))
+                         (let ((scale (attention-scale self)))
+                           (if *compose-backward*
+                               (let* ((s (!matmul q (!t k)))
+                                      (p (if (attention-causal self)
+                                             (!causal-softmax-hip s :scale scale)
+                                             (!softmax-hip (!reshape (!mul scale s) t (car (last (shape s)))))))
+                                      (p (apply #'!reshape p (shape s)))
+                                      (dv (!matmul (!t p) dout))
+                                      (dp (!matmul dout (!t v)))
+                                      (ds (!mul scale (!mul p (!sub dp (!sum-hip (!mul dp p) :axis -1 :keepdims t)))))
+                                      (dq (!matmul ds k))
+                                      (dk (!matmul (!t ds) q)))
+                                 (values (proceed dq) (proceed dk) (proceed dv) nil))
+                               ;; the library addresses dO like O and dQ, dK, dV like Q, K, V: contiguous
+                               ;; operands (copies of windows, 25 MB each at the block's shape) and fresh
+                               ;; contiguous gradients share one set of strides
+                               (let* ((q (eager-contiguous q)) (k (eager-contiguous k)) (v (eager-contiguous v))
+                                      (o (eager-contiguous o)) (dout (eager-contiguous dout))
+                                      (dq (fresh-like q)) (dk (fresh-like q)) (dv (fresh-like q)))
+                                 (ensure-extension)
+                                 (with-foreign-object (desc '(:struct attention-desc))
+                                   (fill-attention-desc desc q k v o scale (attention-causal self))
+                                   (check (wf2hip-attention-backward-f32
+                                           desc (tensor-device-pointer q) (tensor-device-pointer k)
+                                           (tensor-device-pointer v) (tensor-device-pointer o)
+                                           (tensor-device-pointer dout) (tensor-device-pointer lse)
+                                           (tensor-device-pointer dq) (tensor-device-pointer dk)
+                                           (tensor-device-pointer dv))))
+                                 (values dq dk dv nil)))))))
   (setf (attention-scale self) scale
         (attention-causal self) causal))
 

@@ -40,7 +40,7 @@ NODE_NAMES = (
     "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node",
     # the -backward nodes define-op generates for them, where the backward is one kernel too
     "HIP-Activation-Node-backward", "HIP-Softmax-Node-backward", "HIP-Causal-Softmax-Node-backward",
-    "HIP-LayerNorm-Node-backward",
+    "HIP-LayerNorm-Node-backward", "HIP-Attention-Node-backward",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -600,24 +600,57 @@ def _causal_softmax_node(x: HIPTensor, out: HIPTensor, scale: float = 1.0) -> HI
     return out
 
 
-@define_impl("HIP-Attention-Node", HIPTensor, _only_float)
-def _attention_node(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor, scale: float,
-                    causal: bool = False) -> HIPTensor:
-    """``Q K V OUT[batch heads seq dim] -> OUT``: softmax(scale q k^T [+ mask]) v in one kernel."""
-    if not (len(q.shape) == 4 and list(q.shape) == list(k.shape) == list(v.shape) == list(out.shape)):
-        raise ValueError("HIP-Attention-Node expects four (batch, heads, seq, head_dim) tensors of one shape")
+def _attention_desc(name: str, q, k, v, o, scale: float, causal: bool):
+    """The descriptor of four (batch, heads, seq, head_dim) views and their start addresses."""
+    if not (len(q.shape) == 4 and list(q.shape) == list(k.shape) == list(v.shape) == list(o.shape)):
+        raise ValueError(f"{name} expects (batch, heads, seq, head_dim) tensors of one shape")
     B, H, T, hd = q.shape
     d = _lib.AttentionDesc()
     d.batch, d.heads, d.seq, d.head_dim = B, H, T, hd
     ptrs = []
-    for t, field in ((q, d.q_stride), (k, d.k_stride), (v, d.v_stride), (out, d.o_stride)):
+    for t, field in ((q, d.q_stride), (k, d.k_stride), (v, d.v_stride), (o, d.o_stride)):
         _, strides, off = t.geometry()
         if hd > 1 and strides[3] != 1:
-            raise ValueError("HIP-Attention-Node: the head_dim axis must be contiguous")
+            raise ValueError(f"{name}: the head_dim axis must be contiguous")
         for a in range(3):
             field[a] = strides[a]
         ptrs.append(C.c_void_p(t.ptr + 4 * off))
     d.scale = float(scale)
     d.causal = 1 if causal else 0
-    _lib.check(_lib.get().wf2hip_attention_f32(C.byref(d), *ptrs))
+    return d, ptrs
+
+
+def _same_layout(name: str, what: str, t: HIPTensor, like: HIPTensor):
+    """`t` must be addressed like `like` (the library reads one set of strides for both)."""
+    if list(t.shape) != list(like.shape) or t.geometry()[1] != like.geometry()[1]:
+        raise ValueError(f"{name}: {what} must have the shape and strides of the tensor it belongs to")
+    return C.c_void_p(t.ptr + 4 * t.geometry()[2])
+
+
+@define_impl("HIP-Attention-Node", HIPTensor, _only_float)
+def _attention_node(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor, scale: float,
+                    causal: bool = False, lse: HIPTensor | None = None) -> HIPTensor:
+    """``Q K V OUT[batch heads seq dim] -> OUT``: softmax(scale q k^T [+ mask]) v in one kernel.  `lse`, a
+    contiguous (batch, heads, seq) tensor, receives the row statistics the backward node reads."""
+    d, ptrs = _attention_desc("HIP-Attention-Node", q, k, v, out, scale, causal)
+    if lse is None:
+        _lib.check(_lib.get().wf2hip_attention_f32(C.byref(d), *ptrs))
+    else:
+        _require_rows("HIP-Attention-Node: lse", lse, list(q.shape[:3]))
+        _lib.check(_lib.get().wf2hip_attention_forward_f32(C.byref(d), *ptrs, C.c_void_p(lse.ptr)))
     return out
+
+
+@define_impl("HIP-Attention-Node-backward", HIPTensor, _only_float)
+def _attention_backward_node(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPTensor, dout: HIPTensor,
+                             lse: HIPTensor, dq: HIPTensor, dk: HIPTensor, dv: HIPTensor, scale: float,
+                             causal: bool = False):
+    """``Q K V OUT DOUT LSE DQ DK DV -> DQ DK DV``: the three gradients without a (seq, seq) tensor.  dout
+    is addressed like out, dq / dk / dv like q / k / v."""
+    name = "HIP-Attention-Node-backward"
+    d, ptrs = _attention_desc(name, q, k, v, out, scale, causal)
+    _require_rows(f"{name}: lse", lse, list(q.shape[:3]))
+    extra = [_same_layout(name, "dout", dout, out), C.c_void_p(lse.ptr), _same_layout(name, "dq", dq, q),
+             _same_layout(name, "dk", dk, k), _same_layout(name, "dv", dv, v)]
+    _lib.check(_lib.get().wf2hip_attention_backward_f32(C.byref(d), *ptrs, *extra))
+    return dq, dk, dv

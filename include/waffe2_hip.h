@@ -761,6 +761,24 @@ typedef struct wf2hip_attention_desc {
 } wf2hip_attention_desc;
 int wf2hip_attention_f32(const wf2hip_attention_desc* desc, const float* q, const float* k,
                          const float* v, float* o);
+/* The same forward pass that also leaves, per (batch, head, query), the base-2 logarithm
+ * of the row sum of exp2(scale log2(e) Q.K) in lse[(b * heads + h) * seq + i] (contiguous;
+ * may be NULL): with it the backward pass forms the probabilities of any tile directly. */
+int wf2hip_attention_forward_f32(const wf2hip_attention_desc* desc, const float* q, const float* k,
+                                 const float* v, float* o, float* lse);
+/* dQ, dK, dV of that forward pass from Q, K, V, its output O, the upstream gradient dO and
+ * lse, without materialising a (seq, seq) tensor: the backward of the !matmul / !softmax /
+ * !matmul chain (MatMulNode's backward, source/base-impl/matrix-ops.lisp:10-15; !softmax's
+ * through its composition, source/nn/activation.lisp:126-159) in three launches
+ * (D = sum_d dO O per query; dQ with queries resident; dK and dV with keys resident).
+ * dO is addressed through o_stride; dQ, dK, dV through q_stride, k_stride, v_stride, so they
+ * can be windows of one fused-projection gradient.  The gradients may not overlap anything
+ * that is read.  Allocates 4 * batch * heads * seq bytes of scratch from the library's pool.
+ * Result: within 1e-5 of the float64 gradients relative to the magnitude their last
+ * product adds up. */
+int wf2hip_attention_backward_f32(const wf2hip_attention_desc* desc, const float* q, const float* k,
+                                  const float* v, const float* o, const float* dout,
+                                  const float* lse, float* dq, float* dk, float* dv);
 
 #ifdef __cplusplus
 }
