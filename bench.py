@@ -257,6 +257,20 @@ def row_probe(W, reps: int = 5):
     p0 = normal([N])
     run("Adam step 2^26", 28 * N, lambda: (W.optimizers.Adam(F.copy(p0), lr=1e-3), F.copy(p0)), lambda s: s[0].step(s[1]))
     run("SGD step 2^26", 16 * N, lambda: (W.optimizers.SGD(F.copy(p0), lr=1e-3), F.copy(p0)), lambda s: s[0].step(s[1]))
+    run("GELU backward 2^26", 12 * N, lambda: (F.copy(p0), F.copy(p0)),
+        lambda s: F.activation_backward("gelu", s[0], s[1], in_place=True))
+    del p0
+    R, Cn = 32768, 1024
+    a0 = normal([R, Cn], 3.0)
+    y0 = F.softmax_fused(a0)
+    run("softmax backward (32768,1024)", 12 * R * Cn, lambda: (F.copy(y0), F.copy(a0)),
+        lambda s: F.softmax_backward(s[0], s[1], in_place=True))
+    del a0, y0
+    R, Cn = 65536, 1024
+    a0, g0 = normal([R, Cn]), normal([Cn])
+    dg, db = T([Cn], initial_element=None), T([Cn], initial_element=None)
+    run("LayerNorm backward (65536,1024)", 12 * R * Cn, lambda: (F.copy(a0), F.copy(a0), T([R, Cn], initial_element=None)),
+        lambda s: W.nodes.forward("HIP-LayerNorm-Node-backward", s[0], g0, s[1], s[2], dg, db, 1e-5), launches=3)
     print(json.dumps({"probe_rows": order}))
 
 
@@ -500,7 +514,17 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         measure(f"attention (8,12,1024,64) {'causal' if causal else 'full'}", ring,
                 lambda s, c=causal: F.attention(s[0], s[1], s[2], out=s[3], causal=c), flop, bound="mfma",
                 note="flop of the useful half of the score matrix" if causal else None)
-    del q0
+    # the backward of the same attention (three launches: D per query, dQ, dK and dV)
+    lse = T([B, H, S], initial_element=None)
+    o0 = F.attention(q0, q0, q0, causal=True, lse=lse)
+    ring = ring_of(lambda: (clone(q0), clone(q0), clone(q0), clone(q0), T([B, H, S, hd], initial_element=None),
+                            T([B, H, S, hd], initial_element=None), T([B, H, S, hd], initial_element=None)),
+                   28 * B * H * S * hd)
+    measure("attention backward (8,12,1024,64) causal: dQ, dK, dV (three launches)", ring,
+            lambda s: F.attention_backward(s[0], s[1], s[2], s[3], causal=True, dq=s[4], dk=s[5], dv=s[6], out=o0, lse=lse),
+            10.0 * B * H * S * S * hd * 0.5, bound="mfma",
+            note="flop of the useful half of the five products a backward needs at least (the kernels form seven)")
+    del q0, o0, lse
     return rows
 
 

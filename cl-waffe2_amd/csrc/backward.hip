@@ -130,9 +130,11 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_rows(const float* __rest
     dr.load(dy + row * ncols, ncols, lane, 0.0f);
   }
   for (; row < nrows; row += stride) {
-    const int64_t next = row + stride < nrows ? row + stride : row;  // the last row again: loaded, not used
-    xn.load(x + next * ncols, ncols, lane, 0.0f);
-    dn.load(dy + next * ncols, ncols, lane, 0.0f);
+    const int64_t next = row + stride;
+    if (next < nrows) {  // uniform over the wavefront
+      xn.load(x + next * ncols, ncols, lane, 0.0f);
+      dn.load(dy + next * ncols, ncols, lane, 0.0f);
+    }
     double sum = 0.0;
 #pragma unroll
     for (int i = 0; i < NV; i++)
