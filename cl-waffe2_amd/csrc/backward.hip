@@ -25,8 +25,8 @@ __device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (
 // skipped tiles of a triangular product) nor left unwritten (dx is 0 there).
 template <int NV, bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_wave(const float* __restrict__ y, int64_t ldy,
-                                                                const float* __restrict__ dy, int64_t lddy,
-                                                                float* __restrict__ dx, int64_t lddx,
+                                                                const float* dy, int64_t lddy,  // dx may be dy
+                                                                float* dx, int64_t lddx,
                                                                 int64_t nrows, int64_t ncols, int64_t causal_seq,
                                                                 float scale) {
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
@@ -55,8 +55,8 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_wave(const float* __r
 
 // Rows beyond the register tile: a workgroup per row, two passes (the second one from the L2).
 __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_block(const float* __restrict__ y, int64_t ldy,
-                                                                 const float* __restrict__ dy, int64_t lddy,
-                                                                 float* __restrict__ dx, int64_t lddx,
+                                                                 const float* dy, int64_t lddy,  // dx may be dy
+                                                                 float* dx, int64_t lddx,
                                                                  int64_t ncols, int64_t causal_seq, float scale) {
   __shared__ double lds[kWavesPerBlock];
   __shared__ float stat;
@@ -107,8 +107,8 @@ static int launch_softmax_bwd(int nv, const float* y, int64_t ldy, const float* 
 template <int NV, bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void layernorm_bwd_rows(const float* __restrict__ x,
                                                              const float* __restrict__ gamma,
-                                                             const float* __restrict__ dy, float eps,
-                                                             float* __restrict__ dx, float* __restrict__ partial,
+                                                             const float* dy, float eps,  // dx may be dy
+                                                             float* dx, float* __restrict__ partial,
                                                              int64_t nrows, int64_t ncols) {
   __shared__ float fold[kWavesPerBlock][NV * kWave * 4];
   const int lane = threadIdx.x & (kWave - 1);
