@@ -155,3 +155,32 @@ def test_layernorm_backward_wide_rows_take_the_composition(gpu):
     dx, dg, db, mag, mag_g = ref.layer_norm_backward(x.astype(np.float64), g.astype(np.float64), dy.astype(np.float64), 1e-5)
     gx, gg, gb = F.layer_norm_backward(tx, tg, td, 1e-5)
     assert np.max(np.abs(gx.numpy() - dx) / mag) <= 5e-6 and np.max(np.abs(gg.numpy() - dg) / mag_g) <= 5e-6
+
+
+def test_backward_entries_on_empty_operands(gpu):
+    """Zero rows, zero columns, zero elements: nothing is launched, column sums of no rows are 0."""
+    import ctypes as C
+    W = gpu
+    lib = W.lib.get()
+    p = lambda t: C.c_void_p(t.ptr)  # noqa: E731
+    a, b, c = (W.HIPTensor([4, 8], initial_element=3.0) for _ in range(3))
+    g = W.HIPTensor([8], initial_element=1.0)
+    dg, db = W.HIPTensor([8], initial_element=5.0), W.HIPTensor([8], initial_element=5.0)
+    assert lib.wf2hip_softmax_backward_rows_f32(0, 8, p(a), 8, p(b), 8, p(c), 8, 1.0, 0) == 0
+    assert lib.wf2hip_softmax_backward_rows_f32(4, 0, p(a), 8, p(b), 8, p(c), 8, 1.0, 0) == 0
+    assert lib.wf2hip_layernorm_backward_f32(0, 8, p(a), p(g), p(b), 1e-5, p(c), p(dg), p(db)) == 0
+    assert np.all(dg.numpy() == 0.0) and np.all(db.numpy() == 0.0)
+    assert np.all(c.numpy() == 3.0)
+    v = W.lib.View2()
+    v.rank = 1
+    v.shape[0] = 0
+    v.stride_a[0] = v.stride_b[0] = 1
+    assert lib.wf2hip_activation_backward_nd(W.lib.GELU, C.byref(v), p(a), p(b), 0.0) == 0
+    assert lib.wf2hip_activation_backward_nd(7, C.byref(v), p(a), p(b), 0.0) == 0  # nothing to do, nothing checked
+    v.shape[0] = 8
+    assert lib.wf2hip_activation_backward_nd(7, C.byref(v), p(a), p(b), 0.0) == W.lib.EINVAL  # not an activation
+    # pitches smaller than the row, a causal form that is not square
+    assert lib.wf2hip_softmax_backward_rows_f32(4, 8, p(a), 4, p(b), 8, p(c), 8, 1.0, 0) == W.lib.EINVAL
+    assert lib.wf2hip_softmax_backward_rows_f32(4, 8, p(a), 8, p(b), 8, p(c), 8, 1.0, 4) == W.lib.EINVAL
+    # dx over y
+    assert lib.wf2hip_softmax_backward_rows_f32(4, 8, p(a), 8, p(b), 8, p(a), 8, 1.0, 0) == W.lib.EOVERLAP
