@@ -198,3 +198,25 @@ def block_backward(dout: HIPTensor, saved: dict, p: dict, cfg: dict = CONFIG):
     # h = LayerNorm(x); x also feeds the residual
     dln1, g["ln1_g"], g["ln1_b"] = F.layer_norm_backward(x, p["ln1_g"], dh, eps)
     return F.add_(dln1, dx1), g
+
+
+def positional_embedding(ctx: HIPTensor, wte: HIPTensor, wpe: HIPTensor) -> HIPTensor:
+    """``(call (GPT2PositionalEmbedding ...) ctx wte wpe out)``: token ids (as :float, N x T) to
+    wte[id] + wpe[position], (N, T, embedding-size) (``examples/gpt-2/utils.lisp:68-110``)."""
+    from . import nodes
+    n, t = ctx.shape
+    out = HIPTensor([n, t, wte.shape[1]], initial_element=None)
+    return nodes.forward("GPT2PositionalEmbedding", ctx, wte, wpe, out)
+
+
+def model_forward(tokens: HIPTensor, model: dict, cfg: dict = CONFIG, mode: str = "fused") -> HIPTensor:
+    """The GPT2 model of the example (``examples/gpt-2/model.lisp:137-196``): positional embedding,
+    the layers, the final LayerNorm and the language-model head ``x . wte^T`` (``lm-head``), with the
+    benchmark's standard attention in the layers.  `model` holds 'wte', 'wpe', 'ln_f_g', 'ln_f_b' and
+    'layers', a list of block parameter dicts.  Returns the logits (N, T, vocab)."""
+    x = positional_embedding(tokens, model["wte"], model["wpe"])
+    for layer in model["layers"]:
+        x = block_forward(x, layer, mode=mode, cfg=cfg)
+    ln = F.layer_norm_fused if mode != "nodes" else F.layer_norm
+    x = ln(x, model["ln_f_g"], model["ln_f_b"], cfg["eps"])
+    return F.matmul(x, F.t(model["wte"]))

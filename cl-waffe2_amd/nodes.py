@@ -41,6 +41,8 @@ NODE_NAMES = (
     # the -backward nodes define-op generates for them, where the backward is one kernel too
     "HIP-Activation-Node-backward", "HIP-Softmax-Node-backward", "HIP-Causal-Softmax-Node-backward",
     "HIP-LayerNorm-Node-backward", "HIP-Attention-Node-backward",
+    # the node of the reference's GPT-2 example (examples/gpt-2/utils.lisp:68-72)
+    "GPT2PositionalEmbedding",
 )
 
 DEVICE_FEATURES: dict[type, dict[str, tuple]] = {}
@@ -654,3 +656,22 @@ def _attention_backward_node(q: HIPTensor, k: HIPTensor, v: HIPTensor, out: HIPT
              _same_layout(name, "dk", dk, k), _same_layout(name, "dv", dv, v)]
     _lib.check(_lib.get().wf2hip_attention_backward_f32(C.byref(d), *ptrs, *extra))
     return dq, dk, dv
+
+
+@define_impl("GPT2PositionalEmbedding", HIPTensor, _only_float)
+def _gpt2_positional_embedding(ctx: HIPTensor, wte: HIPTensor, wpe: HIPTensor, out: HIPTensor) -> HIPTensor:
+    """``ctx[N sentence-length] wte[vocab-size embedding-size] wpe[n-ctx embedding-size]
+    ctx-out[N sentence-length embedding-size] -> ctx-out``: out <- wte[round(ctx)] + wpe[position]
+    (``examples/gpt-2/utils.lisp:68-110``; the example implements it for LispTensor only)."""
+    name = "GPT2PositionalEmbedding"
+    if len(ctx.shape) != 2 or len(wte.shape) != 2 or len(wpe.shape) != 2:
+        raise ValueError(f"{name}: ctx, wte, wpe must be matrices")
+    n, t = ctx.shape
+    vocab, dim = wte.shape
+    _require_rows(f"{name}: ctx", ctx)
+    _require_rows(f"{name}: wte", wte)
+    _require_rows(f"{name}: wpe", wpe, [wpe.shape[0], dim])
+    _require_rows(f"{name}: ctx-out", out, [n, t, dim])
+    _lib.check(_lib.get().wf2hip_embedding_add_f32(n * t, t, dim, C.c_void_p(ctx.ptr), C.c_void_p(wte.ptr), vocab,
+                                                  C.c_void_p(wpe.ptr), wpe.shape[0], C.c_void_p(out.ptr)))
+    return out

@@ -780,6 +780,16 @@ int wf2hip_attention_backward_f32(const wf2hip_attention_desc* desc, const float
                                   const float* v, const float* o, const float* dout,
                                   const float* lse, float* dq, float* dk, float* dv);
 
+/* ---- GPT-2 example: token + position embedding ------------------------------ */
+/* out[r, :] <- wte[round(ctx[r]), :] + wpe[r % seq, :] for r < rows (rows = sentences x seq):
+ * the GPT2PositionalEmbedding node of examples/gpt-2/utils.lisp:19-110, which the example
+ * implements for LispTensor only (a zero fill and two waffe2_sadd calls per position).
+ * ctx holds token ids as floats, rounded to nearest (ties to even, as ROUND) and clamped to
+ * [0, vocab); wte is (vocab, dim), wpe (n_ctx, dim), out (rows, dim), all contiguous;
+ * seq <= n_ctx.  Bit-exact: one binary32 add per element. */
+int wf2hip_embedding_add_f32(long rows, long seq, long dim, const float* ctx, const float* wte,
+                             long vocab, const float* wpe, long n_ctx, float* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -165,3 +165,16 @@ def block_backward(x, p, n_head, dout, eps=1e-5):
     grads["x"] = np.stack(dxs)
     scales["x"] = np.stack(sxs)
     return grads, scales
+
+
+def model_forward(tokens, model, n_head, eps=1e-5):
+    """float64 closed form of the example's GPT2 model with the benchmark's attention in the layers
+    (examples/gpt-2/model.lisp:137-196): wte[token] + wpe[position], the blocks, the final LayerNorm,
+    logits = x . wte^T."""
+    f8 = np.float64
+    ids = np.rint(np.asarray(tokens)).astype(np.int64)
+    x = model["wte"].astype(f8)[ids] + model["wpe"].astype(f8)[np.arange(ids.shape[1])][None]
+    for layer in model["layers"]:
+        x = block_forward(x, layer, n_head, eps)
+    x = layer_norm(x, model["ln_f_g"].astype(f8), model["ln_f_b"].astype(f8), eps)
+    return x @ model["wte"].astype(f8).T

@@ -518,3 +518,22 @@ def dunary_1d(op: str, n: int, x: np.ndarray, incx: int, out: np.ndarray, inco: 
     fn.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_long, C.c_void_p, C.c_long, C.c_double]
     fn.restype = C.c_int
     assert fn(DUNARY_OPS.index(op), n, px, incx, po, inco, p) >= 0
+
+
+def gpt2_positional_embedding(ctx: np.ndarray, wte: np.ndarray, wpe: np.ndarray, use_ref: bool = False) -> np.ndarray:
+    """GPT2PositionalEmbedding of the reference's GPT-2 example on a freshly allocated (zero) output
+    (examples/gpt-2/utils.lisp:19-66): per sentence and position, `waffe2_sadd` of the token's WTE row
+    and then of the position's WPE row onto the output row, embedding-size elements each; the token id
+    is `(round vocab-index)` of the :float context (ties to even).  ctx: (N, T) float32."""
+    n, t = ctx.shape
+    dim = wte.shape[1]
+    out = np.zeros(n * t * dim, np.float32)
+    wte_flat = np.ascontiguousarray(wte, np.float32).ravel()
+    wpe_flat = np.ascontiguousarray(wpe, np.float32).ravel()
+    for s in range(n):
+        for pos in range(t):
+            token = int(np.rint(ctx[s, pos]))
+            offx = (s * t + pos) * dim
+            binary_1d("add", dim, out, 1, wte_flat, 1, offx=offx, offy=token * dim, use_ref=use_ref)
+            binary_1d("add", dim, out, 1, wpe_flat, 1, offx=offx, offy=pos * dim, use_ref=use_ref)
+    return out.reshape(n, t, dim)

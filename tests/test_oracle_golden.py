@@ -377,3 +377,17 @@ def test_lisp_loop_nodes_follow_their_definitions(O):
     assert out[5] == np.inf and out[6] == -np.inf and np.isnan(out[2]) and out[0] == 0.0
     O.unary_1d("acosh", edge.size, edge, 1, out, 1)
     assert out[5] == 0.0 and np.isnan(out[7]) and out[2] == np.inf
+
+
+def test_gpt2_positional_embedding_restatement(O):
+    """The restated loop of examples/gpt-2/utils.lisp:19-66 equals the closed form the node documents,
+    add(WTE[CTX], WPE[position]), exactly; ids round half to even as (round x) does."""
+    rng = np.random.default_rng(3)
+    wte = rng.standard_normal((40, 10)).astype(np.float32)
+    wpe = rng.standard_normal((12, 10)).astype(np.float32)
+    ctx = rng.integers(0, 40, (3, 9)).astype(np.float32)
+    got = O.gpt2_positional_embedding(ctx, wte, wpe)
+    want = wte[ctx.astype(int)] + wpe[np.arange(9)][None]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    halves = O.gpt2_positional_embedding(np.array([[0.5, 1.5, 2.5]], np.float32), wte, np.zeros_like(wpe))
+    assert np.array_equal(halves[0], wte[[0, 2, 2]])
