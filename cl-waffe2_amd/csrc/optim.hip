@@ -25,7 +25,7 @@ __device__ __forceinline__ void adam1(float& p, float g, float& m, float& v, flo
 
 // VEC: two 16-byte vectors per thread and stream, all loads issued before the
 // arithmetic; NT: streaming hint for tensors far beyond the Infinity Cache.
-template <bool VEC, bool NT>
+template <bool VEC, bool NT, bool FULL = false>
 __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, const float* __restrict__ g,
                                                       float* __restrict__ m, float* __restrict__ v,
                                                       size_t n, float omb1, float omb2, float lr_t,
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const size_t i = base + (size_t)u * kWave;
-      if (i < nvec) {
+      if (FULL || i < nvec) {
         pv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(p) + i) : reinterpret_cast<f4*>(p)[i];
         gv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(g) + i)
                    : reinterpret_cast<const f4*>(g)[i];
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const size_t i = base + (size_t)u * kWave;
-      if (i < nvec) {
+      if (FULL || i < nvec) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
           float pe = pv[u][c], me = mv[u][c], ve = vv[u][c];
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
         }
       }
     }
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (!FULL && blockIdx.x == 0 && threadIdx.x < (n & 3)) {
       const size_t j = nvec * 4 + threadIdx.x;
       adam1(p[j], g[j], m[j], v[j], omb1, omb2, lr_t, eps);
     }
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, con
 
 // VEC: four 16-byte vectors per lane and stream, wave-contiguous, loads first
 // (the shape measured best for x <- x op y); NT as above.
-template <bool VEC, bool NT>
+template <bool VEC, bool NT, bool FULL = false>
 __global__ __launch_bounds__(kBlock) void sgd_kernel(float* __restrict__ p, float* __restrict__ g,
                                                      size_t n, float lr) {
   if (VEC) {
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* __restrict__ p, floa
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const size_t i = base + (size_t)u * kWave;
-      if (i < nvec) {
+      if (FULL || i < nvec) {
         pv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(p) + i) : reinterpret_cast<f4*>(p)[i];
         gv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<f4*>(g) + i) : reinterpret_cast<f4*>(g)[i];
       }
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* __restrict__ p, floa
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const size_t i = base + (size_t)u * kWave;
-      if (i < nvec) {
+      if (FULL || i < nvec) {
         gv[u] = gv[u] * lr;
         pv[u] = pv[u] - gv[u];
         if (NT) {
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(float* __restrict__ p, floa
         }
       }
     }
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (!FULL && blockIdx.x == 0 && threadIdx.x < (n & 3)) {
       const size_t j = nvec * 4 + threadIdx.x;
       g[j] = g[j] * lr;
       p[j] = p[j] - g[j];
@@ -153,7 +153,12 @@ WF2_API int wf2hip_adam_step_f32(long n, float* param, const float* grad, float*
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
   hipStream_t st = rt().stream;
   const bool streaming = (int64_t)n * 28 >= ((int64_t)192 << 20);
-  if (vec && streaming)
+  // every workgroup full: no bounds tests, so all eight loads of a thread are issued before its first
+  // wait (2^26 parameters: 315.4 -> 304.2 us, 74.4 -> 77.3 % of the HBM peak)
+  if (vec && streaming && n % (4 * kBlock * 2) == 0)
+    adam_kernel<true, true, true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, m, v, (size_t)n,
+                                                                      one_minus_beta1, one_minus_beta2, lr_t, eps);
+  else if (vec && streaming)
     adam_kernel<true, true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, m, v, (size_t)n,
                                                                 one_minus_beta1, one_minus_beta2, lr_t, eps);
   else if (vec)
@@ -178,6 +183,7 @@ WF2_API int wf2hip_sgd_step_f32(long n, float* param, float* grad, float lr) {
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
   hipStream_t st = rt().stream;
   const bool streaming = (int64_t)n * 16 >= ((int64_t)192 << 20);
+  // (the form without bounds tests that Adam gains 3 points from measures 0.5 - 1.5 points lower here)
   if (vec && streaming)
     sgd_kernel<true, true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, (size_t)n, lr);
   else if (vec)
