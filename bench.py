@@ -274,6 +274,37 @@ def row_probe(W, reps: int = 5):
     print(json.dumps({"probe_rows": order}))
 
 
+def matrix_core_probe(W, reps: int = 4):
+    """The launch sequence for `rocprofv3 --pmc` runs of the kernels bound by the matrix cores, at the block's
+    shapes: `reps` launches each of attention forward (full, then causal), attention backward (causal:
+    D, dQ, dK and dV) and one projection, printed in order at the end."""
+    F = W.functional
+    T = W.HIPTensor
+    rng = np.random.Generator(np.random.PCG64(6))
+    B, S, H, hd = 8, 1024, 12, 64
+    qkv = T.from_numpy(rng.standard_normal((B, S, 3 * H, hd)).astype(np.float32))
+    q, k, v = (qkv.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3) for i in range(3))
+    out = T([B, S, H, hd], initial_element=None).permute(0, 2, 1, 3)
+    lse = T([B, H, S], initial_element=None)
+    dout = T.from_numpy(rng.standard_normal((B, S, H, hd)).astype(np.float32)).permute(0, 2, 1, 3)
+    dqkv = T([B, S, 3 * H, hd], initial_element=None)
+    dq, dk, dv = (dqkv.view(True, True, (i * H, (i + 1) * H), True).permute(0, 2, 1, 3) for i in range(3))
+    for causal in (False, True):
+        for _ in range(reps):
+            F.attention(q, k, v, out=out, causal=causal, lse=lse)
+    for _ in range(reps):
+        F.attention_backward(q, k, v, dout, causal=True, dq=dq, dk=dk, dv=dv, out=out, lse=lse)
+    a = T.from_numpy(rng.standard_normal((B * S, 768)).astype(np.float32))
+    b = T.from_numpy(rng.standard_normal((768, 3072)).astype(np.float32))
+    c = T([B * S, 3072], initial_element=None)
+    for _ in range(reps):
+        F.matmul(a, b, out=c)
+    W.lib.synchronize()
+    print(json.dumps({"probe_matrix_cores": ["attention (8,12,1024,64) full", "attention causal",
+                                             "attention backward causal", "matmul 8192x3072x768"],
+                      "launches_each": reps}))
+
+
 def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     """One line per kernel of the path at the shape its configuration names:
     average launch time from an event pair on the library's stream, the
@@ -671,6 +702,8 @@ def main():
                     help="skip the table of the other kernels of the path at their configured shapes")
     ap.add_argument("--probe-rows", action="store_true",
                     help="run the launch sequence of the other kernels of the path for rocprofv3 --pmc runs and exit")
+    ap.add_argument("--probe-matrix-cores", action="store_true",
+                    help="run the launch sequence of the attention kernels and one projection for rocprofv3 --pmc runs and exit")
     ap.add_argument("--probe", action="store_true",
                     help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
@@ -686,6 +719,9 @@ def main():
         return
     if args.probe_rows:
         row_probe(W)
+        return
+    if args.probe_matrix_cores:
+        matrix_core_probe(W)
         return
 
     step_ms, wall_ms, per_kernel, binary_ms, sustained_ms = gpu_steps(W, args.steps, args.warmup)
