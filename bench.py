@@ -513,6 +513,27 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     measure("LayerNorm backward (65536,1024): dx, dgamma, dbeta (three launches)", ring,
             lambda s: W.nodes.forward("HIP-LayerNorm-Node-backward", s[0], g0, s[1], s[2], dg, db, 1e-5), 12 * R * Cn)
     del x0, g0, dg, db
+    # Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:82-126), forward and backward
+    R, Cn = 32768, 1024
+    x0 = normal([R, Cn], 3.0)
+    t0 = F.softmax_fused(normal([R, Cn]))
+    ring = ring_of(lambda: (clone(x0), clone(t0), T([R, Cn], initial_element=None), T([R, Cn], initial_element=None)),
+                   16 * R * Cn)
+    measure("softmax cross entropy (32768,1024), one kernel: z and the loss per element", ring,
+            lambda s: W.nodes.forward("HIP-Softmax-Cross-Entropy-Node", s[0], s[1], s[2], s[3], 1e-7), 16 * R * Cn)
+    ring = ring_of(lambda: (clone(x0), clone(t0)), 8 * R * Cn)
+    measure("softmax cross entropy (32768,1024), node for node", ring,
+            lambda s: W.nn.softmax_cross_entropy(s[0], s[1], avoid_overflow=True, reduction=True), 16 * R * Cn,
+            note="!softmax (mean, sub, exp, sum, div), then add, loge, mul, mul as separate nodes; "
+                 "rate quoted on the 16 B/elem of the fused form")
+    ring = ring_of(lambda: (clone(x0), clone(t0), clone(t0)), 12 * R * Cn)
+    measure("softmax cross entropy backward (32768,1024), one kernel", ring,
+            lambda s: W.nn.softmax_cross_entropy_backward_fused(s[0], s[1], s[2], in_place=True), 16 * R * Cn)
+    ring = ring_of(lambda: (clone(x0), clone(t0), clone(t0)), 12 * R * Cn)
+    measure("softmax cross entropy backward (32768,1024), node for node", ring,
+            lambda s: W.nn.softmax_cross_entropy_backward(s[0], s[1], s[2]), 16 * R * Cn,
+            note="sub, mul, div as separate nodes; rate quoted on the 16 B/elem of the fused form")
+    del x0, t0
 
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),

@@ -9,7 +9,8 @@
 //   softmax    dx = scale y (dy - sum_j dy y)                      12 bytes per element
 //   LayerNorm  dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),      12 bytes per element
 //              dgamma = sum_rows dy xh, dbeta = sum_rows dy         (+ the partial sums)
-// with xh = (x - mean) rstd and dyh = dy gamma.  Both are HBM-bound.
+//   softmax cross entropy  dx = (dy (z - labels)) / batch          16 bytes per element
+// with xh = (x - mean) rstd and dyh = dy gamma.  All are HBM-bound.
 #include <algorithm>
 
 #include "wf2_common.h"
@@ -267,6 +268,78 @@ static int launch_layernorm_bwd(int nv, uint32_t blocks, const float* x, const f
   return after_launch("layernorm_bwd_rows");
 }
 
+// ---- softmax cross entropy ----------------------------------------------------------------------
+// sce-diff-static of Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:82-88, 103-110): the
+// SubNode, MulNode and DivNode of dx = (dy (z - labels)) / batch in one pass, every operation
+// rounded to binary32 as those nodes round them.  BCAST: dy is one number (the gradient that a
+// !sum or !mean of the loss hands down through its broadcasting view).  Two 16-byte vectors per
+// thread and stream, all loads issued before the arithmetic.
+__device__ __forceinline__ float xent_grad(float dy, float z, float label, float batch) {
+  return (dy * (z - label)) / batch;
+}
+
+template <bool VEC, bool NT, bool BCAST, bool FULL = false>
+__global__ __launch_bounds__(kBlock) void xent_bwd_kernel(const float* dy, const float* z,  // dx may be dy or z
+                                                          const float* __restrict__ labels, float* dx, size_t n,
+                                                          float batch) {
+  const float d0 = BCAST ? dy[0] : 0.0f;
+  if (VEC) {
+    constexpr int U = 2;
+    const size_t nvec = n / 4;
+    const size_t base = ((size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kWave * U + (threadIdx.x & (kWave - 1));
+    f4 dv[U], zv[U], tv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        if (!BCAST) dv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(dy) + i) : reinterpret_cast<const f4*>(dy)[i];
+        zv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(z) + i) : reinterpret_cast<const f4*>(z)[i];
+        tv[u] = NT ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(labels) + i) : reinterpret_cast<const f4*>(labels)[i];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const size_t i = base + (size_t)u * kWave;
+      if (FULL || i < nvec) {
+        f4 r;
+#pragma unroll
+        for (int c = 0; c < 4; c++) r[c] = xent_grad(BCAST ? d0 : dv[u][c], zv[u][c], tv[u][c], batch);
+        if (NT)
+          __builtin_nontemporal_store(r, reinterpret_cast<f4*>(dx) + i);
+        else
+          reinterpret_cast<f4*>(dx)[i] = r;
+      }
+    }
+    if (!FULL && blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+      const size_t j = nvec * 4 + threadIdx.x;
+      dx[j] = xent_grad(BCAST ? d0 : dy[j], z[j], labels[j], batch);
+    }
+  } else {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) dx[i] = xent_grad(BCAST ? d0 : dy[i], z[i], labels[i], batch);
+  }
+}
+
+template <bool BCAST>
+static int launch_xent_bwd(const float* dy, const float* z, const float* labels, float* dx, int64_t n, float batch) {
+  const bool vec = aligned16(z) && aligned16(labels) && aligned16(dx) && (BCAST || aligned16(dy));
+  const int64_t nvec = n / 4 > 0 ? n / 4 : 1;
+  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 2) : ceil_div(n, kBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
+  hipStream_t st = rt().stream;
+  const bool streaming = n * (BCAST ? 12 : 16) >= ((int64_t)192 << 20);
+  // every workgroup full: no bounds tests, so a thread's loads are all issued before its first wait
+  if (vec && streaming && n % (4 * kBlock * 2) == 0)
+    xent_bwd_kernel<true, true, BCAST, true><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);
+  else if (vec && streaming)
+    xent_bwd_kernel<true, true, BCAST><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);
+  else if (vec)
+    xent_bwd_kernel<true, false, BCAST><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);
+  else
+    xent_bwd_kernel<false, false, BCAST><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);
+  return after_launch("xent_bwd_kernel");
+}
+
 }  // namespace wf2
 
 using namespace wf2;
@@ -355,4 +428,20 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   }
   (void)wf2hip_free(partial);  // stream order keeps it alive for the launches above
   return rc;
+}
+
+WF2_API int wf2hip_softmax_cross_entropy_backward_f32(long n, const float* dy, int dy_is_scalar, const float* z,
+                                                      const float* labels, float batch, float* dx) {
+  WF2_TRY(require_init());
+  if (n < 0) return fail(WF2HIP_EINVAL, "negative element count");
+  if (n == 0) return 0;
+  if (!dy || !z || !labels || !dx) return fail(WF2HIP_EINVAL, "null pointer");
+  // dx may be dy or z (element for element); any other overlap would race
+  auto meets = [&](const float* a, int64_t na) { return a < dx + n && dx < a + na; };
+  if (meets(labels, n)) return fail(WF2HIP_EOVERLAP, "softmax cross entropy backward: dx overlaps labels");
+  if (meets(z, n) && dx != z) return fail(WF2HIP_EOVERLAP, "softmax cross entropy backward: dx overlaps z without being z");
+  if (dy_is_scalar ? meets(dy, 1) : (meets(dy, n) && dx != dy))
+    return fail(WF2HIP_EOVERLAP, "softmax cross entropy backward: dx overlaps dy without being dy");
+  return dy_is_scalar ? launch_xent_bwd<true>(dy, z, labels, dx, n, batch)
+                      : launch_xent_bwd<false>(dy, z, labels, dx, n, batch);
 }

@@ -655,22 +655,45 @@ static int launch_maxmin(long n, const float* x, long incx, float* out) {
 // takes a single row has 1 - 2 KB in flight and leaves the memory system idle (rows
 // of 256: 68 % of the HBM peak for softmax, 53 % for LayerNorm at 2^26 elements); the
 // rows' loads are all issued first and their reductions interleave.
-template <int NV, bool VEC, bool NT, int RW = 1>
+//
+// XENT: the cross entropy of Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126,
+// 158) in the same pass.  The softmax z goes to `out` (the node saves it for its backward)
+// and loss = -1 (labels log(z + delta)), each operation rounded to binary32 as the nodes
+// of cross-entropy-loss round them, goes to xe.loss; labels and loss are rows of ncols.
+struct Xent {
+  const float* labels;
+  float* loss;
+  float delta;
+};
+
+__device__ __forceinline__ float xent_term(float label, float z, float delta) {
+  return -1.0f * (label * logf_(z + delta));
+}
+
+template <int NV, bool VEC, bool NT, int RW = 1, bool XENT = false>
 __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restrict__ x, int64_t ldx,
                                                             float* __restrict__ out, int64_t ldo,
                                                             int64_t nrows, int64_t ncols,
-                                                            int64_t causal_seq, float scale) {
+                                                            int64_t causal_seq, float scale, Xent xe) {
   const int64_t row0 = ((int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * RW;
   if (row0 >= nrows) return;
   const int lane = threadIdx.x & (kWave - 1);
   const float ninf = -__builtin_inff();
   RowRegs<NV, VEC, NT> r[RW];
+  RowRegs<NV, VEC, NT> t[XENT ? RW : 1];
   int64_t valid[RW];
 #pragma unroll
   for (int w = 0; w < RW; w++) {
     const int64_t row = row0 + w < nrows ? row0 + w : nrows - 1;  // a repeated last row is computed and not stored
     valid[w] = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
     r[w].load(x + row * ldx, valid[w], lane, ninf);
+  }
+  if (XENT) {
+#pragma unroll
+    for (int w = 0; w < RW; w++) {
+      const int64_t row = row0 + w < nrows ? row0 + w : nrows - 1;
+      t[w].load(xe.labels + row * ncols, ncols, lane, 0.0f);
+    }
   }
 #pragma unroll
   for (int w = 0; w < RW; w++) {
@@ -718,6 +741,16 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
 #pragma unroll
   for (int w = 0; w < RW; w++)
     if (row0 + w < nrows) r[w].store(out + (row0 + w) * ldo, ncols, lane);
+  if (XENT) {
+#pragma unroll
+    for (int w = 0; w < RW; w++) {
+#pragma unroll
+      for (int g = 0; g < NV; g++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) t[w].v[g][c] = xent_term(t[w].v[g][c], r[w].v[g][c], xe.delta);
+      if (row0 + w < nrows) t[w].store(xe.loss + (row0 + w) * ncols, ncols, lane);
+    }
+  }
 }
 
 // Rows of 769 ... 1024 columns: two wavefronts per row, each holding half of it (two
@@ -725,11 +758,11 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_wave(const float* __restr
 // LDS.  Twice the wavefronts of the one-per-row form at half the registers and half
 // the arithmetic between a wavefront's loads and its stores: (32768, 1024) 44.5 ->
 // 43.1 us, where a plain copy of the same rows by one wavefront each takes 43.9 us.
-template <bool VEC, bool NT>
+template <bool VEC, bool NT, bool XENT = false>
 __global__ __launch_bounds__(kBlock) void softmax_rows_pair(const float* __restrict__ x, int64_t ldx,
                                                             float* __restrict__ out, int64_t ldo,
                                                             int64_t nrows, int64_t ncols,
-                                                            int64_t causal_seq, float scale) {
+                                                            int64_t causal_seq, float scale, Xent xe) {
   constexpr int NVH = 2;
   constexpr int64_t kHalf = (int64_t)NVH * kWave * 4;  // 512 columns
   __shared__ float lmax[kWavesPerBlock];
@@ -741,8 +774,9 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_pair(const float* __restr
   const int64_t valid = causal_seq > 0 ? (row % causal_seq) + 1 : ncols;
   auto part = [&](int64_t n) { n -= half * kHalf; return n < 0 ? (int64_t)0 : (n > kHalf ? kHalf : n); };
   const int64_t valid_here = part(valid);
-  RowRegs<NVH, VEC, NT> r;
+  RowRegs<NVH, VEC, NT> r, t;
   r.load(x + row * ldx + half * kHalf, valid_here, lane, ninf);
+  if (XENT) t.load(xe.labels + row * ncols + half * kHalf, part(ncols), lane, 0.0f);
   float m = ninf;
 #pragma unroll
   for (int g = 0; g < NVH; g++)
@@ -782,13 +816,21 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_pair(const float* __restr
 #pragma unroll
     for (int c = 0; c < 4; c++) r.v[g][c] *= inv;
   if (row_raw < nrows) r.store(out + row * ldo + half * kHalf, part(ncols), lane);
+  if (XENT) {
+#pragma unroll
+    for (int g = 0; g < NVH; g++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) t.v[g][c] = xent_term(t.v[g][c], r.v[g][c], xe.delta);
+    if (row_raw < nrows) t.store(xe.loss + row * ncols + half * kHalf, part(ncols), lane);
+  }
 }
 
 // Rows too long for registers: one workgroup per row, three passes (the second
 // and third hit L2).
+template <bool XENT>
 __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __restrict__ x, int64_t ldx,
                                                              float* __restrict__ out, int64_t ldo,
-                                                             int64_t ncols) {
+                                                             int64_t ncols, Xent xe) {
   __shared__ float lmax[kWavesPerBlock];
   __shared__ double lsum[kWavesPerBlock];
   const float* xr = x + (int64_t)blockIdx.x * ldx;
@@ -814,7 +856,12 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __rest
   for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
     double d = (double)xr[c] - (double)m;
     double ed = (d < -104.0) ? 0.0 : exp_core(d);
-    orow[c] = (float)(ed * inv);
+    const float z = (float)(ed * inv);
+    orow[c] = z;
+    if (XENT) {
+      const int64_t at = (int64_t)blockIdx.x * ncols + c;
+      xe.loss[at] = xent_term(xe.labels[at], z, xe.delta);
+    }
   }
 }
 
@@ -928,29 +975,29 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_block(const float* __re
     outr[c] = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
 }
 
-template <bool VEC, bool NT>
+template <bool VEC, bool NT, bool XENT>
 static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t ldx, float* out,
                                int64_t ldo, int64_t nrows, int64_t ncols, int64_t causal_seq,
-                               float scale) {
+                               float scale, Xent xe) {
   hipStream_t st = rt().stream;
-#define WF2_SOFTMAX_CASE(N)                                                                   \
-  case N:                                                                                     \
-    softmax_rows_wave<N, VEC, NT><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,   \
-                                                             causal_seq, scale);              \
+#define WF2_SOFTMAX_CASE(N)                                                                            \
+  case N:                                                                                              \
+    softmax_rows_wave<N, VEC, NT, 1, XENT><<<blocks, kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,   \
+                                                                      causal_seq, scale, xe);          \
     break;
   if (nv == 4) {
-    softmax_rows_pair<VEC, NT><<<(uint32_t)ceil_div(nrows, 2), kBlock, 0, st>>>(x, ldx, out, ldo, nrows, ncols,
-                                                                            causal_seq, scale);
+    softmax_rows_pair<VEC, NT, XENT><<<(uint32_t)ceil_div(nrows, 2), kBlock, 0, st>>>(
+        x, ldx, out, ldo, nrows, ncols, causal_seq, scale, xe);
     return after_launch("softmax_rows_pair");
   }
   switch (nv) {
     case 1:
-      softmax_rows_wave<1, VEC, NT, 4><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 4), kBlock, 0, st>>>(
-          x, ldx, out, ldo, nrows, ncols, causal_seq, scale);
+      softmax_rows_wave<1, VEC, NT, 4, XENT><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 4), kBlock, 0, st>>>(
+          x, ldx, out, ldo, nrows, ncols, causal_seq, scale, xe);
       break;
     case 2:
-      softmax_rows_wave<2, VEC, NT, 2><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 2), kBlock, 0, st>>>(
-          x, ldx, out, ldo, nrows, ncols, causal_seq, scale);
+      softmax_rows_wave<2, VEC, NT, 2, XENT><<<(uint32_t)ceil_div(nrows, kWavesPerBlock * 2), kBlock, 0, st>>>(
+          x, ldx, out, ldo, nrows, ncols, causal_seq, scale, xe);
       break;
     WF2_SOFTMAX_CASE(3)
     WF2_SOFTMAX_CASE(4)
@@ -964,31 +1011,40 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
   return after_launch("softmax_rows_wave");
 }
 
+// xe == nullptr: the plain softmax.  Otherwise the cross-entropy epilogue as well
+// (no causal form; labels and loss are contiguous rows of ncols).
+template <bool XENT>
+static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
+                               int64_t ldo, int64_t causal_seq, float scale, Xent xe) {
+  const int nv = pick_nv(ncols);
+  if (nv == 0) {
+    if (causal_seq > 0) return fail(WF2HIP_EUNSUPPORTED, "causal softmax rows longer than 4096");
+    if (nrows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+    softmax_rows_block<XENT><<<(uint32_t)nrows, kBlock, 0, rt().stream>>>(x, ldx, out, ldo, ncols, xe);
+    return after_launch("softmax_rows_block");
+  }
+  int64_t blocks = ceil_div(nrows, kWavesPerBlock);
+  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
+  bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0;
+  if (XENT) vec = vec && aligned16(xe.labels) && aligned16(xe.loss) && ncols % 4 == 0;
+  const bool streaming = nrows * ncols * (XENT ? 16 : 8) >= ((int64_t)192 << 20);
+  if (vec && streaming)
+    return launch_softmax_wave<true, true, XENT>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                                 causal_seq, scale, xe);
+  if (vec)
+    return launch_softmax_wave<true, false, XENT>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                                  causal_seq, scale, xe);
+  return launch_softmax_wave<false, false, XENT>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
+                                                 causal_seq, scale, xe);
+}
+
 static int softmax_dispatch(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
                             int64_t ldo, int64_t causal_seq, float scale) {
   if (nrows < 0 || ncols < 0) return fail(WF2HIP_EINVAL, "negative extent");
   if (nrows == 0 || ncols == 0) return 0;
   if (!x || !out) return fail(WF2HIP_EINVAL, "null pointer");
   if (ldx < ncols || ldo < ncols) return fail(WF2HIP_EINVAL, "row pitch smaller than the row");
-  const int nv = pick_nv(ncols);
-  if (nv == 0) {
-    if (causal_seq > 0) return fail(WF2HIP_EUNSUPPORTED, "causal softmax rows longer than 4096");
-    if (nrows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
-    softmax_rows_block<<<(uint32_t)nrows, kBlock, 0, rt().stream>>>(x, ldx, out, ldo, ncols);
-    return after_launch("softmax_rows_block");
-  }
-  int64_t blocks = ceil_div(nrows, kWavesPerBlock);
-  if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
-  const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0;
-  const bool streaming = nrows * ncols * 8 >= ((int64_t)192 << 20);
-  if (vec && streaming)
-    return launch_softmax_wave<true, true>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
-                                           causal_seq, scale);
-  if (vec)
-    return launch_softmax_wave<true, false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
-                                            causal_seq, scale);
-  return launch_softmax_wave<false, false>(nv, (uint32_t)blocks, x, ldx, out, ldo, nrows, ncols,
-                                           causal_seq, scale);
+  return softmax_dispatch_as<false>(nrows, ncols, x, ldx, out, ldo, causal_seq, scale, Xent{nullptr, nullptr, 0.0f});
 }
 
 template <bool VEC, bool NT>
@@ -1136,6 +1192,19 @@ WF2_API int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long l
                                     long ldo) {
   WF2_TRY(require_init());
   return softmax_dispatch(rows, cols, x, ldx, out, ldo, 0, 1.0f);
+}
+
+WF2_API int wf2hip_softmax_cross_entropy_f32(long rows, long cols, const float* x, const float* labels, float delta,
+                                             float* z, float* loss) {
+  WF2_TRY(require_init());
+  if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
+  if (rows == 0 || cols == 0) return 0;
+  if (!x || !labels || !z || !loss) return fail(WF2HIP_EINVAL, "null pointer");
+  const int64_t n = (int64_t)rows * cols;
+  auto meet = [n](const float* a, const float* b) { return a < b + n && b < a + n; };
+  if (meet(z, x) || meet(z, labels) || meet(z, loss) || meet(loss, x) || meet(loss, labels))
+    return fail(WF2HIP_EOVERLAP, "softmax cross entropy: z and loss must overlap neither the inputs nor each other");
+  return softmax_dispatch_as<true>(rows, cols, x, cols, z, cols, 0, 1.0f, Xent{labels, loss, delta});
 }
 
 WF2_API int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,

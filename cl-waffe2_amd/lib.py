@@ -172,6 +172,8 @@ _SIGNATURES = {
     "wf2hip_layernorm_rows_f32": ([_L, _L, _P, _P, _P, _F, _P], C.c_int),
     "wf2hip_softmax_backward_rows_f32": ([_L, _L, _P, _L, _P, _L, _P, _L, _F, _L], C.c_int),
     "wf2hip_layernorm_backward_f32": ([_L, _L, _P, _P, _P, _F, _P, _P, _P], C.c_int),
+    "wf2hip_softmax_cross_entropy_f32": ([_L, _L, _P, _P, _F, _P, _P], C.c_int),
+    "wf2hip_softmax_cross_entropy_backward_f32": ([_L, _P, C.c_int, _P, _P, _F, _P], C.c_int),
     "wf2hip_activation_backward_nd": ([C.c_int, C.POINTER(View2), _P, _P, _F], C.c_int),
     "wf2hip_sgemm": ([C.c_char, C.c_char, _L, _L, _L, _F, _P, _L, _P, _L, _F, _P, _L], C.c_int),
     "wf2hip_sgemm_strided_batched": (

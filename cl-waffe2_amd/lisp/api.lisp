@@ -56,12 +56,18 @@
 (defcfun "wf2hip_sum_nd" :int (view (:pointer (:struct view2))) (a :pointer) (b :pointer) (divisor :float))
 (defcfun "wf2hip_softmax_rows_f32" :int (rows :long) (cols :long) (x :pointer) (ldx :long) (out :pointer) (ldo :long))
 (defcfun "wf2hip_layernorm_rows_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (b :pointer) (eps :float) (out :pointer))
+;; Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126): softmax and -labels log(z + delta) in one pass
+(defcfun "wf2hip_softmax_cross_entropy_f32" :int (rows :long) (cols :long) (x :pointer) (labels :pointer) (delta :float)
+  (z :pointer) (loss :pointer))
 ;; backward of the fused layers, one kernel each
 (defcfun "wf2hip_softmax_backward_rows_f32" :int (rows :long) (cols :long) (y :pointer) (ldy :long) (dy :pointer) (lddy :long)
   (dx :pointer) (lddx :long) (scale :float) (causal-seq :long))
 (defcfun "wf2hip_layernorm_backward_f32" :int (rows :long) (cols :long) (x :pointer) (g :pointer) (dy :pointer) (eps :float)
   (dx :pointer) (dg :pointer) (db :pointer))
 (defcfun "wf2hip_activation_backward_nd" :int (op :int) (view :pointer) (dout :pointer) (x :pointer) (p :float))
+;; sce-diff-static (source/nn/criterion.lisp:82-88) in one pass
+(defcfun "wf2hip_softmax_cross_entropy_backward_f32" :int (n :long) (dy :pointer) (dy-is-scalar :int) (z :pointer)
+  (labels :pointer) (batch :float) (dx :pointer))
 
 ;; struct wf2hip_view3 and the compare kernels (counterparts of waffe2_s{eq,lt,le,gt,ge}[_scal],
 ;; cl-waffe2-simd/api.lisp:143-209)

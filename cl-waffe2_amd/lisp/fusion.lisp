@@ -171,6 +171,67 @@ composed recipe."
         (call (HIP-Softmax-Node) x (make-input (shape x) nil :dtype :float :order (order x))))
       (call-composed 'cl-waffe2/nn:!softmax x :avoid-overflow avoid-overflow :axis axis)))
 
+;; ---- softmax cross entropy --------------------------------------------------------------------
+(defun softmax-cross-entropy-gradient (dout z label)
+  "(dout (z - label)) / batch, the SubNode, MulNode and DivNode of sce-diff-static
+(source/nn/criterion.lisp:82-88) in one kernel; batch is the second-to-last extent of Z."
+  (ensure-extension)
+  (let ((dout (eager-contiguous dout))
+        (dx (fresh-like z)))
+    (check (wf2hip-softmax-cross-entropy-backward-f32 (apply #'* (shape z)) (tensor-device-pointer dout) 0
+                                                      (tensor-device-pointer z) (tensor-device-pointer label)
+                                                      (coerce (car (last (shape z) 2)) 'single-float)
+                                                      (tensor-device-pointer dx)))
+    dx))
+
+(define-op (HIP-Softmax-Cross-Entropy-Node (self delta)
+            :slots ((delta :initform 1e-7 :accessor cross-entropy-delta))
+            :save-for-backward-names (z label)
+            :where (X[rows cols] Labels[rows cols] Z[rows cols] OUT[rows cols] -> OUT[rows cols])
+            :documentation "Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126) on contiguous
+matrices as one kernel (wf2hip_softmax_cross_entropy_f32): Z <- softmax over the last axis of X, saved
+for the backward as the reference saves it, OUT <- -1 (Labels log(Z + delta)).  Backward: one kernel
+as well (wf2hip_softmax_cross_entropy_backward_f32)."
+            :forward ((self x label z out)
+                      (ensure-extension)
+                      (check (wf2hip-softmax-cross-entropy-f32 (first (shape x)) (second (shape x))
+                                                               (tensor-device-pointer x)
+                                                               (tensor-device-pointer label)
+                                                               (coerce (cross-entropy-delta self) 'single-float)
+                                                               (tensor-device-pointer z)
+                                                               (tensor-device-pointer out)))
+                      (with-setting-save4bw ((z z) (label label)) out))
+            :backward ((self dout)
+                       (with-reading-save4bw ((z z) (label label))
+                         (if *compose-backward*
+                             (values (proceed (!div (!mul dout (!sub z label))
+                                                    (make-tensor (car (last (shape z) 2)) :dtype :float)))
+                                     nil nil nil)
+                             (values (softmax-cross-entropy-gradient dout z label) nil nil nil)))))
+  (setf (cross-entropy-delta self) delta))
+
+(defun softmax-cross-entropy-hip (x labels &key (axis 1) (delta 1e-7) (avoid-overflow nil) (reduction t))
+  "(softmax-cross-entropy x labels) on contiguous :float matrices with the classes on axis 1 as one
+kernel; the reductions stay outside the node (source/nn/criterion.lisp:192-196).  Anything else takes
+the reference's node."
+  (if (and (hip-float-tensor-p x)
+           (hip-float-tensor-p labels)
+           (= (length (shape x)) 2)
+           (equal (shape x) (shape labels))
+           (eql axis 1)
+           (every #'numberp (shape x)))
+      (let* ((x (->contiguous x))
+             (labels (->contiguous labels))
+             (out (call (HIP-Softmax-Cross-Entropy-Node delta) x labels
+                        (make-input (shape x) nil :dtype :float :order (order x))
+                        (make-input (shape x) nil :dtype :float :order (order x)))))
+        (case reduction
+          (:sum (!sum-hip out))
+          (:mean (!mean-hip out))
+          (t out)))
+      (call-composed 'cl-waffe2/nn:softmax-cross-entropy x labels :axis axis :delta delta
+                                                              :avoid-overflow avoid-overflow :reduction reduction)))
+
 ;; ---- LayerNorm over the last axis ------------------------------------------------------------
 (defun layer-norm-gradients (x g dout eps)
   "Gradients of y = (x - u) / sqrt(s + eps) * g + b per row (source/nn/norms.lisp:72-82) from the
@@ -522,5 +583,6 @@ pass :scale (/ 1.0 seq) for its numbers, :causal t for a decoder)."
 (define-bypass HIPTensor cl-waffe2/nn:!sigmoid !sigmoid-hip)
 (define-bypass HIPTensor cl-waffe2/nn:!gelu !gelu-hip)
 (define-bypass HIPTensor cl-waffe2/nn:!softmax !softmax-hip)
+(define-bypass HIPTensor cl-waffe2/nn:softmax-cross-entropy softmax-cross-entropy-hip)
 (define-bypass HIPTensor cl-waffe2/base-impl:!sum !sum-hip)
 (define-bypass HIPTensor cl-waffe2/base-impl:!mean !mean-hip)

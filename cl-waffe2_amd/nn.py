@@ -9,6 +9,7 @@ device without a kernel of their own.
 from __future__ import annotations
 
 from . import functional as F
+from . import nodes
 from .tensor import HIPTensor
 
 
@@ -98,3 +99,28 @@ def softmax_cross_entropy_backward(dy, z: HIPTensor, labels: HIPTensor) -> HIPTe
     ``z``; ``dy`` is the upstream gradient (a tensor of z's shape or a number)."""
     batch = float(z.shape[-2])
     return F.div(F.mul(F.sub(z, labels), dy), batch)
+
+
+def softmax_cross_entropy_fused(x: HIPTensor, labels: HIPTensor, delta: float = 1e-7, reduction=True):
+    """``(softmax-cross-entropy x labels)`` with the classes on the last axis as ONE node
+    (HIP-Softmax-Cross-Entropy-Node; ``softmax-cross-entropy-hip`` of the Lisp glue): the softmax is
+    max-subtracted (the kernel of HIP-Softmax-Node) where !softmax subtracts the mean or nothing, the
+    cross entropy rounds like the reference's nodes.  Returns ``(loss, z)`` like
+    :func:`softmax_cross_entropy`."""
+    x, labels = F.to_contiguous(x), F.to_contiguous(labels)
+    z = HIPTensor(list(x.shape), initial_element=None)
+    out = HIPTensor(list(x.shape), initial_element=None)
+    nodes.forward("HIP-Softmax-Cross-Entropy-Node", x, labels, z, out, float(delta))
+    return _reduce(out, reduction), z
+
+
+def softmax_cross_entropy_backward_fused(dy, z: HIPTensor, labels: HIPTensor, in_place: bool = False) -> HIPTensor:
+    """:func:`softmax_cross_entropy_backward` as ONE node (HIP-Softmax-Cross-Entropy-Node-backward), bit for
+    bit the same result.  ``dy``: a tensor of z's shape, a one-element tensor or a number.  With
+    ``in_place`` the gradient overwrites a full-shape ``dy``."""
+    if not isinstance(dy, HIPTensor):
+        dy = HIPTensor([1], initial_element=float(dy))
+    dy, labels = F.to_contiguous(dy), F.to_contiguous(labels)
+    full = list(dy.shape) == list(z.shape)
+    dx = dy if (in_place and full) else HIPTensor(list(z.shape), initial_element=None)
+    return nodes.forward("HIP-Softmax-Cross-Entropy-Node-backward", dy, z, labels, dx)

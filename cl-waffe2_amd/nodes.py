@@ -37,10 +37,10 @@ NODE_NAMES = (
     "Im2ColNode", "Col2ImNode",
     # the define-op nodes of lisp/fusion.lisp (one kernel each)
     "HIP-Sum-Node", "HIP-Activation-Node", "HIP-Softmax-Node", "HIP-LayerNorm-Node", "HIP-Linear-Node",
-    "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node",
+    "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node", "HIP-Softmax-Cross-Entropy-Node",
     # the -backward nodes define-op generates for them, where the backward is one kernel too
     "HIP-Activation-Node-backward", "HIP-Softmax-Node-backward", "HIP-Causal-Softmax-Node-backward",
-    "HIP-LayerNorm-Node-backward", "HIP-Attention-Node-backward",
+    "HIP-LayerNorm-Node-backward", "HIP-Attention-Node-backward", "HIP-Softmax-Cross-Entropy-Node-backward",
     # the node of the reference's GPT-2 example (examples/gpt-2/utils.lisp:68-72)
     "GPT2PositionalEmbedding",
 )
@@ -561,6 +561,42 @@ def _softmax_node(x: HIPTensor, out: HIPTensor) -> HIPTensor:
     rows = x.size // max(cols, 1)
     _lib.check(_lib.get().wf2hip_softmax_rows_f32(rows, cols, C.c_void_p(x.ptr), cols, C.c_void_p(out.ptr), cols))
     return out
+
+
+@define_impl("HIP-Softmax-Cross-Entropy-Node", HIPTensor, _only_float)
+def _softmax_cross_entropy_node(x: HIPTensor, labels: HIPTensor, z: HIPTensor, out: HIPTensor,
+                                delta: float = 1.0e-7) -> HIPTensor:
+    """``X[rows cols] Labels[rows cols] Z[rows cols] OUT[rows cols] -> OUT``: Softmax-Cross-Entropy-Node
+    (``source/nn/criterion.lisp:90-126``) as one kernel.  z <- softmax over the last axis (what the node
+    saves for its backward), out <- -1 (labels log(z + delta))."""
+    name = "HIP-Softmax-Cross-Entropy-Node"
+    _require_rows(f"{name}: x", x)
+    for what, t in (("labels", labels), ("z", z), ("out", out)):
+        _require_rows(f"{name}: {what}", t, x.shape)
+    cols = x.shape[-1]
+    rows = x.size // max(cols, 1)
+    _lib.check(_lib.get().wf2hip_softmax_cross_entropy_f32(rows, cols, C.c_void_p(x.ptr), C.c_void_p(labels.ptr),
+                                                          float(delta), C.c_void_p(z.ptr), C.c_void_p(out.ptr)))
+    return out
+
+
+@define_impl("HIP-Softmax-Cross-Entropy-Node-backward", HIPTensor, _only_float)
+def _softmax_cross_entropy_backward_node(dout: HIPTensor, z: HIPTensor, labels: HIPTensor, dx: HIPTensor) -> HIPTensor:
+    """``DOUT[rows cols] Z[rows cols] Labels[rows cols] DX[rows cols] -> DX``: sce-diff-static
+    (``source/nn/criterion.lisp:82-88``), (dout (z - labels)) / batch with batch the second-to-last extent
+    of z.  A one-element ``dout`` is the number every element uses (the gradient under a !sum or !mean of
+    the loss).  dx may be dout or z."""
+    name = "HIP-Softmax-Cross-Entropy-Node-backward"
+    _require_rows(f"{name}: z", z)
+    _require_rows(f"{name}: labels", labels, z.shape)
+    _require_rows(f"{name}: dx", dx, z.shape)
+    scalar = dout.size == 1 and z.size != 1
+    _require_rows(f"{name}: dout", dout, None if scalar else z.shape)
+    batch = float(z.shape[-2]) if len(z.shape) >= 2 else 1.0
+    _lib.check(_lib.get().wf2hip_softmax_cross_entropy_backward_f32(z.size, C.c_void_p(dout.ptr), int(scalar),
+                                                                   C.c_void_p(z.ptr), C.c_void_p(labels.ptr), batch,
+                                                                   C.c_void_p(dx.ptr)))
+    return dx
 
 
 @define_impl("HIP-LayerNorm-Node", HIPTensor, _only_float)

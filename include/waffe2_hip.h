@@ -606,6 +606,17 @@ int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
  * (source/nn/norms.lisp:44-82; examples/gpt-2/utils.lisp:114-127). */
 int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
                               const float* beta, float eps, float* out);
+/* Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126) over the last axis
+ * in one pass: z[r, c] <- softmax over c of x[r, c] (max-subtracted, the bits of
+ * wf2hip_softmax_rows_f32; the node saves it for its backward) and
+ * loss[r, c] <- -1 * (labels[r, c] * log(z[r, c] + delta)), each operation
+ * rounded to binary32 like the nodes of cross-entropy-loss (criterion.lisp:158).
+ * All four arrays are contiguous (rows, cols); z and loss overlap neither the
+ * inputs nor each other (WF2HIP_EOVERLAP).  The reductions :sum / :mean stay
+ * outside the node, as in the reference (criterion.lisp:192-196). */
+int wf2hip_softmax_cross_entropy_f32(long rows, long cols, const float* x,
+                                     const float* labels, float delta, float* z,
+                                     float* loss);
 
 /* ---- backward of the fused layers ------------------------------------------ */
 /* The reference differentiates !softmax, LayerNorm and the activations through
@@ -621,6 +632,16 @@ int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float*
 int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* y, long ldy,
                                      const float* dy, long lddy, float* dx, long lddx,
                                      float scale, long causal_seq);
+/* The backward of Softmax-Cross-Entropy-Node, sce-diff-static
+ * (source/nn/criterion.lisp:82-88, 103-110): dx[i] <- (dy[i] * (z[i] - labels[i])) / batch
+ * for i < n, the SubNode, MulNode and DivNode of the reference in one pass with
+ * the same binary32 roundings.  `batch` is the second-to-last extent of z as a
+ * float.  dy_is_scalar != 0: dy points to ONE float on the device that every
+ * element uses (the gradient a !sum or !mean of the loss hands down through its
+ * broadcasting view).  dx may be dy or z; it overlaps nothing else. */
+int wf2hip_softmax_cross_entropy_backward_f32(long n, const float* dy, int dy_is_scalar,
+                                              const float* z, const float* labels,
+                                              float batch, float* dx);
 /* Gradients of wf2hip_layernorm_rows_f32 from the saved input: with
  * xh = (x - mean) rstd and dyh = dy gamma,
  *   dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),

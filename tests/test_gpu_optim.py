@@ -164,13 +164,16 @@ def test_weights_round_trip(gpu, tmp_path):
     assert_bit_equal(back["bias"].numpy(), a[0, 0], "wf2model flat tensor")
 
 
-def test_classifier_training_step_by_step(gpu):
+@pytest.mark.parametrize("fused_loss", [False, True])
+def test_classifier_training_step_by_step(gpu, fused_loss):
     """A two-layer classifier trained entirely on the device with the
     reference's recipes: Linear = matmul + bias (AddNode with a broadcast row),
     !relu = x * (x > 0), Softmax-Cross-Entropy-Node forward and backward
     (nn/criterion.lisp:82-126), bias gradients as !sum over the batch, matmul
     backward products, Adam.  Every step is compared with the same recipe in
-    float64 on the host (loss and weights), and the loss must fall."""
+    float64 on the host (loss and weights), and the loss must fall.  With
+    `fused_loss` the criterion is HIP-Softmax-Cross-Entropy-Node and its one-kernel
+    backward instead of the node compositions."""
     W = gpu
     F = W.functional
     nn = W.nn
@@ -215,8 +218,12 @@ def test_classifier_training_step_by_step(gpu):
         mask = F.where(a1, ">", 0.0)
         h1 = F.mul(a1, mask)
         a2 = F.add(F.matmul(h1, dev["w2"]), dev["b2"])
-        loss, z = nn.softmax_cross_entropy(a2, dl, avoid_overflow=True, reduction="mean")
-        dz = nn.softmax_cross_entropy_backward(1.0 / labels.size, z, dl)
+        if fused_loss:
+            loss, z = nn.softmax_cross_entropy_fused(a2, dl, reduction="mean")
+            dz = nn.softmax_cross_entropy_backward_fused(1.0 / labels.size, z, dl)
+        else:
+            loss, z = nn.softmax_cross_entropy(a2, dl, avoid_overflow=True, reduction="mean")
+            dz = nn.softmax_cross_entropy_backward(1.0 / labels.size, z, dl)
         grads = {"w2": F.matmul(F.t(h1), dz), "b2": F.sum(dz, axis=0)}  # (1, c): the reduced axis stays, size 1
         dh = F.mul_(F.matmul(dz, F.t(dev["w2"])), mask)
         grads["w1"], grads["b1"] = F.matmul(F.t(dx), dh), F.sum(dh, axis=0)
