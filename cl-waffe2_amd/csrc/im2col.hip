@@ -16,12 +16,19 @@
 // (possible with dilation > 1) make the result of the sequential loop depend on
 // write order and are refused.
 //
-// im2col: one thread per written element of col, gathers from im.
+// im2col: a workgroup stages the image rows of a band of output rows in LDS and
+// writes the band of every (kh, kw) plane from there (im2col_lds); im2col_flat,
+// which gathers from im through the caches, where there is no reuse to gain
+// (k <= stride) or the rows do not fit; im2col_kernel beyond 2^31 elements.
 // col2im: im is the sum, over kh then kw ascending (the reference's order of
 // accumulation, so the binary32 result is identical), of the col elements that
-// land on it: one thread per element of im, no atomics.
-// HBM-bound: about 4 (k-h k-w + 1) bytes per image element.
+// land on it: gathered per element of im, no atomics (col2im_gather; col2im_single
+// where windows do not overlap; col2im_kernel beyond 2^31 elements).
+// HBM-bound: 4 (k-h k-w h-out w-out + H W) bytes per image plane.
+#include <algorithm>
+
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 
 namespace wf2 {
 
@@ -71,6 +78,256 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(UnfoldParams p) {
   p.dst[t] = acc;
 }
 
+// The same two maps for tensors below 2^31 elements, in 32-bit index arithmetic with the
+// divisions by extents turned into multiplications on the host (wf2_fastdiv.h).
+struct Unfold32 {
+  const float* src;
+  float* dst;
+  uint32_t H, W, H_out, W_out, K_H, K_W, s_h, s_w;
+  uint32_t d_h, d_w, pad_h, pad_w;
+  uint32_t total;          // elements of the destination
+  uint32_t plane_elems;    // H_out * W_out
+  FastDiv by_plane, by_w_out, by_kw, by_kh;  // im2col: col index -> (n c) kh kw i j
+  FastDiv by_w, by_h, by_sh, by_sw;          // col2im: im index -> (n c) y x; steps of the walk
+};
+
+// Where the reference's walk of kernel offset k stops: y < d k - pad + s out (im2col.c:75-80).
+__device__ __forceinline__ uint32_t walk_end(uint32_t d, uint32_t k, uint32_t pad, uint32_t s, uint32_t out) {
+  return d * k + s * out - pad;  // the host has refused geometries where this would be negative
+}
+
+// im2col: U elements of col per thread, kBlock apart, so that the lanes of a wavefront read
+// (with a unit stride along W) and write consecutive addresses: four consecutive elements per
+// lane and one 16-byte store measured no better, because a lane's four loads then lie 16
+// bytes from its neighbour's and the L1 handles nine times the accesses (231 MB of col from a
+// (32, 64, 58, 58) image, 3 x 3: 73 us).  The first element is decoded in full; the others
+// follow by adding kBlock to the position in mixed radix, which costs additions and compares
+// where a decode costs eight quarter-rate integer multiplications.
+struct ColCursor {
+  uint32_t nc, kh, kw, i, j;  // position in col[(n c) kh kw i j]
+};
+
+struct ColStep {  // kBlock = ((dnc K_H + dkh) K_W + dkw) plane + di W_out + dj
+  uint32_t dnc, dkh, dkw, di, dj;
+};
+
+__device__ __forceinline__ ColCursor cursor_at(const Unfold32& p, uint32_t e) {
+  ColCursor c;
+  uint32_t r;
+  const uint32_t plane = fd_divmod(e, p.by_plane, &r);
+  c.i = fd_divmod(r, p.by_w_out, &c.j);
+  const uint32_t rest = fd_divmod(plane, p.by_kw, &c.kw);
+  c.nc = fd_divmod(rest, p.by_kh, &c.kh);
+  return c;
+}
+
+__device__ __forceinline__ void cursor_advance(const Unfold32& p, const ColStep& d, ColCursor& c) {
+  uint32_t carry;
+  c.j += d.dj;
+  carry = c.j >= p.W_out;
+  c.j -= carry ? p.W_out : 0;
+  c.i += d.di + carry;
+  carry = c.i >= p.H_out;
+  c.i -= carry ? p.H_out : 0;
+  c.kw += d.dkw + carry;
+  carry = c.kw >= p.K_W;
+  c.kw -= carry ? p.K_W : 0;
+  c.kh += d.dkh + carry;
+  carry = c.kh >= p.K_H;
+  c.kh -= carry ? p.K_H : 0;
+  c.nc += d.dnc + carry;
+}
+
+// Workgroup b takes chunk (b mod 8) * per_xcd + b / 8: workgroups are dealt to the eight XCDs in
+// turn and each XCD has its own L2, so an XCD walks a contiguous range of col and the K_H K_W
+// planes that re-read one image plane find it in that XCD's L2.
+// M24: every factor of the index products is below 2^24 (one-pass multiplications).
+template <int U, bool M24>
+__global__ __launch_bounds__(kBlock) void im2col_flat(Unfold32 p, ColStep d, uint32_t per_xcd) {
+  const uint32_t chunk = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+  const uint32_t e0 = chunk * (kBlock * U) + threadIdx.x;
+  if ((blockIdx.x >> 3) >= per_xcd || e0 >= p.total) return;
+  auto mul = [](uint32_t a, uint32_t b) -> uint32_t { return M24 ? __umul24(a, b) : a * b; };
+  ColCursor c = cursor_at(p, e0);
+  float v[U];
+  bool on[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t y = c.kh + mul(c.i, p.s_h), x = c.kw + mul(c.j, p.s_w);
+    // what the reference's walk does not reach stays as it was
+    on[u] = e0 + u * kBlock < p.total && y < walk_end(p.d_h, c.kh, p.pad_h, p.s_h, p.H_out) &&
+            x < walk_end(p.d_w, c.kw, p.pad_w, p.s_w, p.W_out);
+    if (on[u]) v[u] = p.src[mul(mul(c.nc, p.H) + y, p.W) + x];
+    if (u + 1 < U) cursor_advance(p, d, c);
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++)
+    if (on[u]) p.dst[e0 + u * kBlock] = v[u];
+}
+
+// im2col through LDS: a workgroup owns `band_rows` output rows of one image plane (n c), reads
+// the image rows they touch once (they are adjacent in memory: one contiguous run) and writes the
+// band of all K_H K_W planes of col from LDS, lanes on consecutive addresses on both sides.
+// Reads that hit the L2 cost the memory system about what reads from HBM cost (the flat kernel
+// above takes as long as a copy of col, 79 us for the 231 MB of a (32, 64, 58, 58) image with a
+// 3 x 3 kernel, although it fetches only the 28 MB of the image from HBM), so the K_H K_W-fold
+// reuse has to happen inside the workgroup.
+__global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands, uint32_t band_rows) {
+  extern __shared__ float tile[];  // the image rows y0 ..., W floats each
+  const uint32_t nc = blockIdx.x / bands, band = blockIdx.x - nc * bands;
+  const uint32_t i0 = band * band_rows;
+  const uint32_t rows_here = p.H_out - i0 < band_rows ? p.H_out - i0 : band_rows;
+  const uint32_t y0 = i0 * p.s_h;
+  if (y0 >= p.H) return;  // uniform; the walk of no kernel row reaches this band
+  const uint32_t want = (rows_here - 1) * p.s_h + p.K_H;
+  const uint32_t need = want < p.H - y0 ? want : p.H - y0;
+  const float* src = p.src + ((size_t)nc * p.H + y0) * p.W;
+  {  // eight loads in flight per thread
+    const uint32_t count = need * p.W;
+    uint32_t e = threadIdx.x;
+    for (; e + 7 * kBlock < count; e += 8 * kBlock) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+#pragma unroll
+      for (int u = 0; u < 8; u++) tile[e + u * kBlock] = v[u];
+    }
+    for (; e < count; e += kBlock) tile[e] = src[e];
+  }
+  __syncthreads();
+  const uint32_t band_elems = rows_here * p.W_out;
+  for (uint32_t kh = 0; kh < p.K_H; kh++) {
+    const uint32_t end_h = walk_end(p.d_h, kh, p.pad_h, p.s_h, p.H_out);
+    for (uint32_t kw = 0; kw < p.K_W; kw++) {
+      const uint32_t end_w = walk_end(p.d_w, kw, p.pad_w, p.s_w, p.W_out);
+      float* dst = p.dst + (((size_t)nc * p.K_H + kh) * p.K_W + kw) * p.plane_elems + i0 * p.W_out;
+      for (uint32_t e = threadIdx.x; e < band_elems; e += kBlock) {
+        uint32_t j;
+        const uint32_t il = fd_divmod(e, p.by_w_out, &j);
+        const uint32_t y = kh + (i0 + il) * p.s_h, x = kw + j * p.s_w;
+        // What the reference's walk does not reach stays as it was.  (With padding every row
+        // of col ends in such an element, and stores that leave four bytes of a line out are
+        // merged by the memory system at about half the rate: 100 us where the same image
+        // without padding takes 54 us.  Reading the old value and writing it back is slower
+        // still.)
+        if (y < end_h && x < end_w) dst[e] = tile[(y - y0) * p.W + x];
+      }
+    }
+  }
+}
+
+// col2im: U elements of im per thread, kBlock apart; the kernel offsets are walked kh ascending,
+// then kw ascending (the reference's order of accumulation), and every load of a thread is
+// issued before its first addition.  A term the walk does not produce enters as +0, which
+// leaves a sum that started at +0 unchanged.  The step i along H depends on kh alone and the
+// step j along W on kw alone, so an element costs K_H + K_W divisions, not K_H K_W.
+// KH, KW > 0: the kernel extents, loops unrolled; 0: extents from p, one element per thread.
+// UNIT: both strides are 1.
+template <int KH, int KW, bool UNIT, int U>
+__global__ __launch_bounds__(kBlock) void col2im_gather(Unfold32 p) {
+  const uint32_t k_h = KH > 0 ? KH : p.K_H, k_w = KW > 0 ? KW : p.K_W;
+  // kernel row kh reaches (y, .) at step i when y = kh + i s_h and the walk gets that far
+  auto step_h = [&](uint32_t y, uint32_t kh, uint32_t* at) -> bool {
+    if (kh > y) return false;
+    const uint32_t dy = y - kh;
+    const uint32_t i = UNIT ? dy : fd_div(dy, p.by_sh);
+    *at = i * p.W_out;
+    return (UNIT || i * p.s_h == dy) && i < p.H_out && y < walk_end(p.d_h, kh, p.pad_h, p.s_h, p.H_out);
+  };
+  auto step_w = [&](uint32_t x, uint32_t kw, uint32_t* at) -> bool {
+    if (kw > x) return false;
+    const uint32_t dx = x - kw;
+    const uint32_t j = UNIT ? dx : fd_div(dx, p.by_sw);
+    *at = j;
+    return (UNIT || j * p.s_w == dx) && j < p.W_out && x < walk_end(p.d_w, kw, p.pad_w, p.s_w, p.W_out);
+  };
+  if (KH > 0) {
+    constexpr int NH = KH > 0 ? KH : 1, NW = KW > 0 ? KW : 1;
+    float v[U][NH][NW];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const uint32_t t = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+      uint32_t x, y;
+      const uint32_t row = fd_divmod(t, p.by_w, &x);
+      const uint32_t nc = fd_divmod(row, p.by_h, &y);
+      const float* src = p.src + (size_t)nc * (NH * NW) * p.plane_elems;
+      uint32_t ai[NH], aj[NW];
+      bool oh[NH], ow[NW];
+#pragma unroll
+      for (int kh = 0; kh < NH; kh++) oh[kh] = t < p.total && step_h(y, kh, &ai[kh]);
+#pragma unroll
+      for (int kw = 0; kw < NW; kw++) ow[kw] = step_w(x, kw, &aj[kw]);
+#pragma unroll
+      for (int kh = 0; kh < NH; kh++)
+#pragma unroll
+        for (int kw = 0; kw < NW; kw++)
+          v[u][kh][kw] = (oh[kh] && ow[kw]) ? src[(kh * NW + kw) * p.plane_elems + ai[kh] + aj[kw]] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const uint32_t t = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+      float acc = 0.0f;
+#pragma unroll
+      for (int kh = 0; kh < NH; kh++)
+#pragma unroll
+        for (int kw = 0; kw < NW; kw++) acc += v[u][kh][kw];
+      if (t < p.total) p.dst[t] = acc;
+    }
+  } else {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= p.total) return;
+    uint32_t x, y;
+    const uint32_t row = fd_divmod(t, p.by_w, &x);
+    const uint32_t nc = fd_divmod(row, p.by_h, &y);
+    const float* src = p.src + (size_t)nc * k_h * k_w * p.plane_elems;
+    float acc = 0.0f;
+    for (uint32_t kh = 0; kh < k_h && kh <= y; kh++) {
+      uint32_t ai, aj;
+      if (!step_h(y, kh, &ai)) continue;
+      const float* rowp = src + kh * k_w * p.plane_elems + ai;
+      for (uint32_t kw = 0; kw < k_w && kw <= x; kw++)
+        if (step_w(x, kw, &aj)) acc += rowp[kw * p.plane_elems + aj];
+    }
+    p.dst[t] = acc;
+  }
+}
+
+// col2im when the windows do not overlap (K_H <= s_h and K_W <= s_w, as in pooling): an element
+// of im belongs to at most one window, so it is one load, not a sum.  FAST: the strides are
+// powers of two (shifts instead of divisions) and every factor of the index products is below
+// 2^24 (one-pass multiplications); the index arithmetic is what bounds this kernel.
+template <bool FAST, int U>
+__global__ __launch_bounds__(kBlock) void col2im_single(Unfold32 p, uint32_t log_sh, uint32_t log_sw) {
+  auto mul = [](uint32_t a, uint32_t b) -> uint32_t { return FAST ? __umul24(a, b) : a * b; };
+  float v[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {  // the loads of a thread are all issued before its stores
+    const uint32_t t = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+    uint32_t x, y, kh, kw, i, j;
+    const uint32_t row = fd_divmod(t, p.by_w, &x);
+    const uint32_t nc = fd_divmod(row, p.by_h, &y);
+    if (FAST) {
+      i = y >> log_sh;
+      kh = y & (p.s_h - 1);
+      j = x >> log_sw;
+      kw = x & (p.s_w - 1);
+    } else {
+      i = fd_divmod(y, p.by_sh, &kh);
+      j = fd_divmod(x, p.by_sw, &kw);
+    }
+    const bool on = t < p.total && kh < p.K_H && kw < p.K_W && i < p.H_out && j < p.W_out &&
+                    y < walk_end(p.d_h, kh, p.pad_h, p.s_h, p.H_out) &&
+                    x < walk_end(p.d_w, kw, p.pad_w, p.s_w, p.W_out);
+    v[u] = 0.0f;
+    if (on) v[u] += p.src[mul(mul(mul(nc, p.K_H) + kh, p.K_W) + kw, p.plane_elems) + mul(i, p.W_out) + j];
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t t = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+    if (t < p.total) p.dst[t] = v[u];
+  }
+}
+
 static int make_params(long N, long C, long H, long W, long H_out, long W_out, long K_H, long K_W,
                        long pad_h, long pad_w, long stride_h, long stride_w, long dilation_h,
                        long dilation_w, UnfoldParams* p) {
@@ -102,6 +359,47 @@ static int make_params(long N, long C, long H, long W, long H_out, long W_out, l
   return 0;
 }
 
+// The 32-bit form of a validated geometry; false when an index would not fit.
+static bool make_unfold32(long N, long C, long H, long W, long H_out, long W_out, long K_H, long K_W, long pad_h,
+                          long pad_w, long stride_h, long stride_w, long dilation_h, long dilation_w, Unfold32* q) {
+  const int64_t limit = (int64_t)1 << 31;
+  const int64_t n_im = (int64_t)N * C * H * W, n_col = (int64_t)N * C * K_H * K_W * H_out * W_out;
+  // the ends of the walks are formed in 32 bits too
+  const int64_t end_h = dilation_h * (K_H - 1) + stride_h * H_out, end_w = dilation_w * (K_W - 1) + stride_w * W_out;
+  if (n_im >= limit || n_col >= limit || end_h >= limit || end_w >= limit || pad_h >= limit || pad_w >= limit)
+    return false;
+  q->H = (uint32_t)H; q->W = (uint32_t)W; q->H_out = (uint32_t)H_out; q->W_out = (uint32_t)W_out;
+  q->K_H = (uint32_t)K_H; q->K_W = (uint32_t)K_W; q->s_h = (uint32_t)stride_h; q->s_w = (uint32_t)stride_w;
+  q->d_h = (uint32_t)dilation_h; q->d_w = (uint32_t)dilation_w; q->pad_h = (uint32_t)pad_h; q->pad_w = (uint32_t)pad_w;
+  q->plane_elems = (uint32_t)(H_out * W_out);
+  q->by_plane = make_fastdiv(q->plane_elems);
+  q->by_w_out = make_fastdiv(q->W_out);
+  q->by_kw = make_fastdiv(q->K_W);
+  q->by_kh = make_fastdiv(q->K_H);
+  q->by_w = make_fastdiv(q->W);
+  q->by_h = make_fastdiv(q->H);
+  q->by_sh = make_fastdiv(q->s_h);
+  q->by_sw = make_fastdiv(q->s_w);
+  return true;
+}
+
+template <bool UNIT>
+static void launch_col2im(const Unfold32& q, hipStream_t st) {
+  auto blocks = [&](int u) { return (uint32_t)ceil_div((int64_t)q.total, (int64_t)kBlock * u); };
+  if (q.K_H == q.K_W && q.K_H == 1)
+    col2im_gather<1, 1, UNIT, 4><<<blocks(4), kBlock, 0, st>>>(q);
+  else if (q.K_H == q.K_W && q.K_H == 2)
+    col2im_gather<2, 2, UNIT, 4><<<blocks(4), kBlock, 0, st>>>(q);
+  else if (q.K_H == q.K_W && q.K_H == 3)
+    col2im_gather<3, 3, UNIT, (UNIT ? 1 : 4)><<<blocks(UNIT ? 1 : 4), kBlock, 0, st>>>(q);
+  else if (q.K_H == q.K_W && q.K_H == 5)
+    col2im_gather<5, 5, UNIT, (UNIT ? 1 : 2)><<<blocks(UNIT ? 1 : 2), kBlock, 0, st>>>(q);
+  else if (q.K_H == q.K_W && q.K_H == 7)
+    col2im_gather<7, 7, UNIT, 1><<<blocks(1), kBlock, 0, st>>>(q);
+  else
+    col2im_gather<0, 0, UNIT, 1><<<blocks(1), kBlock, 0, st>>>(q);
+}
+
 }  // namespace wf2
 
 using namespace wf2;
@@ -118,6 +416,48 @@ WF2_API int wf2hip_im2col_f32(float* col, long N, long C, long H, long W, long H
   if (!col || !im) return fail(WF2HIP_EINVAL, "null tensor pointer");
   p.src = im;
   p.dst = col;
+  Unfold32 q;
+  if (make_unfold32(N, C, H, W, H_out, W_out, K_H, K_W, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, &q)) {
+    q.src = im;
+    q.dst = col;
+    q.total = (uint32_t)p.total;
+    // the band of output rows whose image rows fit 16 KB of LDS, so that eight workgroups share a
+    // compute unit and the loading of one overlaps the storing of the others (48 KB where K_H
+    // image rows need more)
+    const int64_t lds_floats = (int64_t)K_H * W * 4 <= (16 << 10) ? (16 << 10) / 4 : (48 << 10) / 4;
+    const int64_t rows_fit = W > 0 ? lds_floats / W : 0;  // image rows
+    if (rows_fit >= K_H && K_H * K_W > stride_h * stride_w) {  // some reuse of the image to gain from
+      int64_t band_rows = std::min<int64_t>((rows_fit - K_H) / stride_h + 1, H_out);
+      // at least two workgroups per compute unit where the planes are few
+      const int64_t planes = (int64_t)N * C;
+      const int64_t cus = std::max(rt().num_cus, 1);
+      while (band_rows > 8 && planes * ceil_div(H_out, band_rows) < 2 * cus) band_rows = (band_rows + 1) / 2;
+      const int64_t bands = ceil_div(H_out, band_rows);
+      const int64_t tile_rows = std::min<int64_t>((band_rows - 1) * stride_h + K_H, H);
+      if (planes * bands < ((int64_t)1 << 31)) {
+        im2col_lds<<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
+            q, (uint32_t)bands, (uint32_t)band_rows);
+        return after_launch("im2col_lds");
+      }
+    }
+    constexpr int U = 4;  // 8 and 16 measure the same
+    const uint32_t per_xcd = (uint32_t)ceil_div(ceil_div(p.total, (int64_t)kBlock * U), 8);
+    ColStep d;  // kBlock in the mixed radix of col's index
+    uint32_t rest = kBlock / q.plane_elems, in_plane = kBlock % q.plane_elems;
+    d.di = in_plane / q.W_out;
+    d.dj = in_plane % q.W_out;
+    d.dkw = rest % q.K_W;
+    rest /= q.K_W;
+    d.dkh = rest % q.K_H;
+    d.dnc = rest / q.K_H;
+    const int64_t u24 = (int64_t)1 << 24;
+    const bool m24 = (int64_t)N * C * H < u24 && W < u24 && H_out < u24 && W_out < u24 && stride_h < u24 && stride_w < u24;
+    if (m24)
+      im2col_flat<U, true><<<per_xcd * 8, kBlock, 0, rt().stream>>>(q, d, per_xcd);
+    else
+      im2col_flat<U, false><<<per_xcd * 8, kBlock, 0, rt().stream>>>(q, d, per_xcd);
+    return after_launch("im2col_flat");
+  }
   const int64_t blocks = ceil_div(p.total, kBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "im2col: too many elements");
   im2col_kernel<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(p);
@@ -138,6 +478,29 @@ WF2_API int wf2hip_col2im_f32(const float* col, long N, long C, long H, long W, 
   p.dst = im;
   const int64_t blocks = ceil_div(p.total, kBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "col2im: too many elements");
+  Unfold32 q;
+  if (make_unfold32(N, C, H, W, H_out, W_out, K_H, K_W, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w, &q)) {
+    q.src = col;
+    q.dst = im;
+    q.total = (uint32_t)p.total;
+    if (K_H <= stride_h && K_W <= stride_w && !(stride_h == 1 && stride_w == 1)) {
+      auto pow2 = [](long v) { return (v & (v - 1)) == 0; };
+      auto log2 = [](long v) { uint32_t l = 0; while ((1L << l) < v) l++; return l; };
+      const int64_t u24 = (int64_t)1 << 24;
+      const bool fast = pow2(stride_h) && pow2(stride_w) && (int64_t)N * C * K_H * K_W < u24 &&
+                        (int64_t)H_out * W_out < u24;
+      const uint32_t blocks4 = (uint32_t)ceil_div(p.total, (int64_t)kBlock * 4);  // 16 per thread: slower
+      if (fast)
+        col2im_single<true, 4><<<blocks4, kBlock, 0, rt().stream>>>(q, log2(stride_h), log2(stride_w));
+      else
+        col2im_single<false, 4><<<blocks4, kBlock, 0, rt().stream>>>(q, 0, 0);
+    }
+    else if (stride_h == 1 && stride_w == 1)
+      launch_col2im<true>(q, rt().stream);
+    else
+      launch_col2im<false>(q, rt().stream);
+    return after_launch("col2im_gather");
+  }
   col2im_kernel<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(p);
   return after_launch("col2im_kernel");
 }

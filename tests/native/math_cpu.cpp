@@ -6,11 +6,15 @@
 //   wf2cpu_scan(op, first, last, stride, &max_ulp, &worst_bits)
 //       walks the binary32 bit patterns first, first+stride, ... <= last and
 //       returns the largest error in ulps against libm evaluated in binary64.
+//   wf2cpu_fastdiv_mismatches(d, n, count)
+//       how many of the numerators n[i] < 2^31, and of the multiples of d and their
+//       neighbours up to 2^31 - 1, the multiply-and-shift division gets wrong.
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
 
 #include "../../cl-waffe2_amd/csrc/wf2_math.h"
+#include "../../cl-waffe2_amd/csrc/wf2_fastdiv.h"
 
 enum { OP_SIN = 16, OP_COS, OP_TANH, OP_LOG, OP_EXP, OP_SQRT, OP_ABS, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN,
        OP_SINH, OP_COSH, OP_LOG2, OP_LOG10, OP_LOG1P, OP_SIGN = 34, OP_SQUARE, OP_ASINH, OP_ACOSH, OP_ATANH,
@@ -134,6 +138,32 @@ void wf2cpu_scan(int op, uint32_t first, uint32_t last, uint32_t stride,
   }
   *max_ulp = best;
   *worst_bits = best_bits;
+}
+
+long wf2cpu_fastdiv_mismatches(uint32_t d, const uint32_t* n, long count) {
+  const wf2::FastDiv f = wf2::make_fastdiv(d);
+  long bad = 0;
+  auto check = [&](uint32_t v) {
+    uint32_t rem;
+    const uint32_t q = wf2::fd_divmod(v, f, &rem);
+    if (q != v / d || rem != v % d) bad++;
+  };
+  for (long i = 0; i < count; i++) check(n[i]);
+  // k d - 1, k d, k d + 1 for up to 2^16 values of k spread over the range, the largest included
+  const uint64_t top = ((uint64_t)1 << 31) - 1;
+  const uint64_t kmax = top / d;
+  const uint64_t step = kmax / 65536 + 1;
+  for (uint64_t k = 0; k <= kmax; k += step) {
+    const uint64_t m = k * d;
+    if (m >= 1) check((uint32_t)(m - 1));
+    check((uint32_t)m);
+    if (m + 1 <= top) check((uint32_t)(m + 1));
+  }
+  const uint64_t m = kmax * d;
+  if (m >= 1) check((uint32_t)(m - 1));
+  check((uint32_t)m);
+  check((uint32_t)top);
+  return bad;
 }
 
 }  // extern "C"

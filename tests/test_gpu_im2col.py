@@ -38,16 +38,22 @@ def test_im2col_col2im_golden(gpu):
         assert_bit_equal(back.numpy(), gold[f"col2im_{idx}_im"], f"col2im case {idx}")
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(6))
 def test_im2col_random_geometries_match_oracle(gpu, O, seed):
+    """Kernels of 1 ... 7 rows and columns (square ones of 1, 2, 3, 5 and 7 take unrolled loops in
+    col2im, the others the loops over the extents), strides 1 ... 3, padding 0 ... 2; the later
+    seeds draw images of several workgroups."""
     W = gpu
     rng = np.random.default_rng(40 + seed)
+    top = 20 if seed < 3 else 45
     for case in range(10):
         N, Cc = int(rng.integers(1, 4)), int(rng.integers(1, 5))
-        k = (int(rng.integers(1, 5)), int(rng.integers(1, 5)))
+        k = (int(rng.integers(1, 8)), int(rng.integers(1, 8)))
+        if case % 2:
+            k = (k[0], k[0])
         s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
         p = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
-        Hin, Win = int(rng.integers(k[0], 20)), int(rng.integers(k[1], 20))
+        Hin, Win = int(rng.integers(k[0], top)), int(rng.integers(k[1], top))
         out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((Hin, Win))]
         H, Wd = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((Hin, Win))]
         im = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
@@ -62,6 +68,37 @@ def test_im2col_random_geometries_match_oracle(gpu, O, seed):
         back = W.HIPTensor([N, Cc, H, Wd])
         W.forward("Col2ImNode", W.HIPTensor.from_numpy(cin), back, s, p, (1, 1))
         assert_bit_equal(back.numpy(), want_im, f"col2im {N, Cc, H, Wd, k, s, p}")
+
+
+@pytest.mark.parametrize("N,Cc,Hin,Win,k,s,p", [
+    (2, 3, 130, 200, (3, 3), (1, 1), (1, 1)),     # several bands of rows per image plane
+    (1, 2, 40, 5000, (3, 3), (1, 1), (0, 0)),     # rows too wide for the staged kernel
+    (1, 2, 9, 3000, (5, 2), (1, 1), (2, 0)),      # the larger tile
+    (2, 2, 64, 64, (2, 2), (2, 2), (0, 0)),       # pooling windows: no overlap, strides powers of two
+    (2, 2, 63, 66, (3, 3), (3, 3), (0, 0)),       # no overlap, stride 3
+    (2, 2, 61, 67, (2, 3), (3, 4), (1, 1)),       # kernel smaller than the stride
+    (3, 2, 57, 57, (3, 3), (2, 2), (1, 1)),       # overlap with stride 2
+    (1, 1, 300, 300, (7, 7), (2, 2), (3, 3)),
+])
+def test_im2col_larger_geometries_match_oracle(gpu, O, N, Cc, Hin, Win, k, s, p):
+    """Each dispatch of the two kernels at sizes of many workgroups, bit for bit against the compiled
+    restatement of the reference's loops (elements its walk does not reach keep the 3.0 they held)."""
+    W = gpu
+    rng = np.random.default_rng(Hin * 1000 + Win)
+    out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((Hin, Win))]
+    H, Wd = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((Hin, Win))]
+    im = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
+    want = np.full((N, Cc, k[0], k[1], out[0], out[1]), 3.0, np.float32)
+    O.im2col(want, im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
+    col = W.HIPTensor.from_numpy(np.full(want.shape, 3.0, np.float32))
+    W.forward("Im2ColNode", W.HIPTensor.from_numpy(im), col, s, p, (1, 1))
+    assert_bit_equal(col.numpy(), want, "im2col")
+    cin = rng.standard_normal(want.shape).astype(np.float32)
+    want_im = np.zeros_like(im)
+    O.col2im(cin, want_im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
+    back = W.HIPTensor.from_numpy(np.full(im.shape, 9.0, np.float32))
+    W.forward("Col2ImNode", W.HIPTensor.from_numpy(cin), back, s, p, (1, 1))
+    assert_bit_equal(back.numpy(), want_im, "col2im")
 
 
 def test_unfold_and_adjoint(gpu):

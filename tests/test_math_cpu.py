@@ -25,14 +25,16 @@ OPS = {"sin": 16, "cos": 17, "tanh": 18, "log": 19, "exp": 20, "sqrt": 21, "abs"
 def M():
     so = os.path.join(HERE, "native", "libwf2_math_cpu.so")
     src = os.path.join(HERE, "native", "math_cpu.cpp")
-    hdr = os.path.join(HERE, "..", "cl-waffe2_amd", "csrc", "wf2_math.h")
-    if not os.path.exists(so) or os.path.getmtime(so) < max(os.path.getmtime(src), os.path.getmtime(hdr)):
+    hdrs = [os.path.join(HERE, "..", "cl-waffe2_amd", "csrc", h) for h in ("wf2_math.h", "wf2_fastdiv.h")]
+    if not os.path.exists(so) or os.path.getmtime(so) < max(os.path.getmtime(f) for f in [src] + hdrs):
         subprocess.check_call(["make", "-C", os.path.join(HERE, "native"), "-B"], stdout=subprocess.DEVNULL)
     L = C.CDLL(so)
     L.wf2cpu_unary.argtypes = [C.c_int, C.c_long, C.c_void_p, C.c_void_p]
     L.wf2cpu_pow.argtypes = [C.c_long, C.c_void_p, C.c_float, C.c_void_p]
     L.wf2cpu_scan.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_double),
                               C.POINTER(C.c_uint32)]
+    L.wf2cpu_fastdiv_mismatches.argtypes = [C.c_uint32, C.c_void_p, C.c_long]
+    L.wf2cpu_fastdiv_mismatches.restype = C.c_long
     return L
 
 
@@ -184,3 +186,18 @@ def test_gelu_gradient_core(M):
     t = np.linspace(-8, 8, 4001)
     g = lambda z: z / (1.0 + np.exp(-2.0 * np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))  # noqa: E731
     assert np.max(np.abs((g(t + 1e-6) - g(t - 1e-6)) / 2e-6 - gelu_grad_truth(t)[0])) < 1e-8
+
+
+def test_index_division_by_multiplication(M):
+    """The multiply-and-shift division of the unfold kernels' index maps (wf2_fastdiv.h) equals n / d and
+    n % d for every numerator below 2^31 it is tried on: random ones, and the multiples of d with their two
+    neighbours across the whole range, for small divisors, powers of two and their neighbours, primes and
+    divisors near 2^31."""
+    rng = np.random.default_rng(77)
+    divisors = set(range(1, 1030)) | {2 ** k + o for k in range(10, 31) for o in (-1, 0, 1)}
+    divisors |= {3136, 12544, 50257, 65521, 1000003, 2 ** 31 - 1, 2 ** 31 - 2, 2 ** 30 + 12345, 715827883}
+    divisors |= {int(v) for v in rng.integers(1, 2 ** 31, 300)}
+    n = np.concatenate([rng.integers(0, 2 ** 31, 4096), np.arange(0, 2048), 2 ** 31 - 1 - np.arange(0, 2048)]).astype(np.uint32)
+    for d in sorted(divisors):
+        if 1 <= d < 2 ** 31:
+            assert M.wf2cpu_fastdiv_mismatches(d, n.ctypes.data, n.size) == 0, d
