@@ -534,6 +534,30 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
             lambda s: W.nn.softmax_cross_entropy_backward(s[0], s[1], s[2]), 16 * R * Cn,
             note="sub, mul, div as separate nodes; rate quoted on the 16 B/elem of the fused form")
     del x0, t0
+    # unfold of a (32, 64, 56, 56) image for a 3 x 3 convolution with padding 1 (source/nn/im2col.lisp:51-95),
+    # and the two nodes it is composed from and differentiated through
+    Nb, Cc, Hh, Kk = 32, 64, 56, 3
+    img = normal([Nb, Cc, Hh, Hh])
+    ncol, nim = Nb * Cc * Kk * Kk * Hh * Hh, Nb * Cc * Hh * Hh
+    ring = ring_of(lambda: T([Nb * Hh * Hh, Cc * Kk * Kk], initial_element=None), 4 * ncol)
+    measure("unfold (32,64,56,56) 3x3 pad 1, one kernel: the (N h w) x (C kh kw) matrix", ring,
+            lambda s: W.nodes.forward("HIP-Unfold-Node", img, s, (Kk, Kk), (1, 1), (1, 1)), 4 * (ncol + nim))
+    measure("unfold (32,64,56,56) 3x3 pad 1, node for node", [None],
+            lambda s: F.unfold_composed(img, (1, 1), (Kk, Kk), (1, 1), (1, 1)), 4 * (ncol + nim),
+            note="padding copy, zero fill of col, Im2ColNode, permuting copy; rate quoted on the bytes of the one-kernel form")
+    padded = normal([Nb, Cc, Hh + 2, Hh + 2])
+    ring = ring_of(lambda: T([Nb, Cc, Kk, Kk, Hh, Hh], initial_element=None), 4 * ncol)
+    measure("Im2ColNode (32,64,58,58) -> (32,64,3,3,56,56), no padding argument", ring,
+            lambda s: W.nodes.forward("Im2ColNode", padded, s, (1, 1), (0, 0), (1, 1)), 4 * (ncol + nim))
+    ring = ring_of(lambda: T([Nb, Cc, Kk, Kk, Hh, Hh], initial_element=None), 4 * ncol)
+    measure("Im2ColNode, padding 1: the walk leaves the last row and column of every plane untouched", ring,
+            lambda s: W.nodes.forward("Im2ColNode", padded, s, (1, 1), (1, 1), (1, 1)), 4 * (ncol + nim),
+            note="stores that leave 4 bytes of a line out are merged by the memory system at about half the rate")
+    back = T([Nb, Cc, Hh + 2, Hh + 2], initial_element=None)
+    ring = ring_of(lambda: normal([Nb, Cc, Kk, Kk, Hh, Hh]), 4 * ncol)
+    measure("Col2ImNode (32,64,3,3,56,56) -> (32,64,58,58)", ring,
+            lambda s: W.nodes.forward("Col2ImNode", s, back, (1, 1), (1, 1), (1, 1)), 4 * (ncol + nim))
+    del img, padded, back
 
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),

@@ -26,6 +26,8 @@
 // where windows do not overlap; col2im_kernel beyond 2^31 elements).
 // HBM-bound: 4 (k-h k-w h-out w-out + H W) bytes per image plane.
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 #include "wf2_common.h"
 #include "wf2_fastdiv.h"
@@ -400,6 +402,106 @@ static void launch_col2im(const Unfold32& q, hipStream_t st) {
     col2im_gather<0, 0, UNIT, 1><<<blocks(1), kBlock, 0, st>>>(q);
 }
 
+// ---- unfold as one kernel -----------------------------------------------------------------------
+// (unfold input dilation kernel-size stride padding) of source/nn/im2col.lisp:51-95 composes a
+// zero-padded copy of the image, Im2ColNode into a zeroed col[N C kh kw i j], a permuting copy to
+// (N i j C kh kw) and a reshape to [(N h-out w-out) (C k-h k-w)]: four passes over tensors of
+// col's size.  Here the matrix is written once, from image rows staged in LDS:
+//   out[(n i j), (c kh kw)] = reached(i, j) ? padded[n c, kh + i s_h, kw + j s_w] : 0
+// with `padded` zero outside the image and reached(i, j) what Im2ColNode's walk visits
+// (dilation 1: i s_h + pad_h < s_h h-out and j s_w + pad_w < s_w w-out, whatever kh and kw are).
+// A workgroup owns `band` output rows i of one image n and `cc` channels: its part of the matrix
+// is, per (i, j), a run of cc K_H K_W consecutive floats (the whole band is one run when it owns
+// every channel).  Two small tables in LDS turn the position in the run, and the position (i, j),
+// into offsets into the staged tile.
+struct UnfoldFused {
+  const float* src;
+  float* dst;
+  uint32_t C, H, W, H_out, W_out, K_H, K_W, s_h, s_w, pad_h, pad_w;
+  uint32_t band, bands, cc, chunks;  // output rows per workgroup, channels per workgroup
+  uint32_t TR, TW;                   // rows and columns of the staged tile per channel
+  uint32_t Q;                        // C K_H K_W
+  FastDiv by_kk, by_kw, by_w_out, by_plane, by_tw;  // K_H K_W, K_W, W_out, TR TW, TW
+};
+
+template <int NQ>  // entries of a run per lane: cc K_H K_W <= 64 NQ
+__global__ __launch_bounds__(kBlock) void unfold_kernel(UnfoldFused p) {
+  extern __shared__ float lds[];
+  const uint32_t KK = p.K_H * p.K_W;
+  const uint32_t plane = p.TR * p.TW;
+  float* tile = lds;                                                   // [cc][TR][TW]
+  uint32_t* qoff = reinterpret_cast<uint32_t*>(lds + p.cc * plane);    // [cc KK]
+  uint32_t* roff = qoff + p.cc * KK;                                   // [band W_out]
+  const uint32_t chunk = blockIdx.x % p.chunks;
+  const uint32_t rest = blockIdx.x / p.chunks;
+  const uint32_t band = rest % p.bands, n = rest / p.bands;
+  const uint32_t c0 = chunk * p.cc;
+  const uint32_t cc = p.C - c0 < p.cc ? p.C - c0 : p.cc;
+  const uint32_t run = cc * KK;
+  const uint32_t i0 = band * p.band;
+  const uint32_t rows_here = p.H_out - i0 < p.band ? p.H_out - i0 : p.band;
+  const uint32_t R = rows_here * p.W_out;
+  constexpr uint32_t kSkipped = 0xffffffffu;
+  for (uint32_t q = threadIdx.x; q < run; q += kBlock) {
+    uint32_t r, kw;
+    const uint32_t c = fd_divmod(q, p.by_kk, &r);
+    const uint32_t kh = fd_divmod(r, p.by_kw, &kw);
+    qoff[q] = (c * p.TR + kh) * p.TW + kw;
+  }
+  for (uint32_t r = threadIdx.x; r < R; r += kBlock) {
+    uint32_t j;
+    const uint32_t il = fd_divmod(r, p.by_w_out, &j);
+    const bool reached = (i0 + il) * p.s_h + p.pad_h < p.s_h * p.H_out && j * p.s_w + p.pad_w < p.s_w * p.W_out;
+    roff[r] = reached ? il * p.s_h * p.TW + j * p.s_w : kSkipped;
+  }
+  // the tile: rows i0 s_h - pad_h ... of the image, columns -pad_w ..., zero outside the image
+  const int32_t y_first = (int32_t)(i0 * p.s_h) - (int32_t)p.pad_h;
+  const float* img = p.src + ((size_t)n * p.C + c0) * p.H * p.W;
+  auto fetch = [&](uint32_t e) -> float {
+    uint32_t r, tx;
+    const uint32_t c = fd_divmod(e, p.by_plane, &r);
+    const uint32_t ty = fd_divmod(r, p.by_tw, &tx);
+    const int32_t y = y_first + (int32_t)ty, x = (int32_t)tx - (int32_t)p.pad_w;
+    const bool inside = y >= 0 && y < (int32_t)p.H && x >= 0 && x < (int32_t)p.W;
+    return inside ? img[((size_t)c * p.H + y) * p.W + x] : 0.0f;
+  };
+  {  // eight loads in flight per thread
+    const uint32_t count = cc * plane;
+    uint32_t e = threadIdx.x;
+    for (; e + 7 * kBlock < count; e += 8 * kBlock) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = fetch(e + u * kBlock);
+#pragma unroll
+      for (int u = 0; u < 8; u++) tile[e + u * kBlock] = v[u];
+    }
+    for (; e < count; e += kBlock) tile[e] = fetch(e);
+  }
+  __syncthreads();
+  float* out = p.dst + ((size_t)n * p.H_out + i0) * p.W_out * p.Q + (size_t)c0 * KK;
+  // A wavefront owns the positions r = wave, wave + 4, ...; its lanes sweep the run, NQ entries
+  // each, whose tile offsets stay in registers: an element is one LDS read and one store.
+  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t off[NQ];
+#pragma unroll
+  for (int m = 0; m < NQ; m++) {
+    const uint32_t qc = lane + m * kWave;
+    off[m] = qc < run ? qoff[qc] : 0;
+  }
+  for (uint32_t r = wave; r < R; r += kBlock / kWave) {
+    const uint32_t ro = roff[r];  // uniform over the wavefront
+    float* row = out + (size_t)r * p.Q;
+    float v[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; m++) v[m] = ro == kSkipped ? 0.0f : tile[off[m] + ro];
+#pragma unroll
+    for (int m = 0; m < NQ; m++) {
+      const uint32_t qc = lane + m * kWave;
+      if (qc < run) row[qc] = v[m];
+    }
+  }
+}
+
 }  // namespace wf2
 
 using namespace wf2;
@@ -503,4 +605,108 @@ WF2_API int wf2hip_col2im_f32(const float* col, long N, long C, long H, long W, 
   }
   col2im_kernel<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(p);
   return after_launch("col2im_kernel");
+}
+
+WF2_API int wf2hip_unfold_f32(long N, long C, long H, long W, long K_H, long K_W, long stride_h, long stride_w,
+                              long pad_h, long pad_w, const float* x, float* out) {
+  WF2_TRY(require_init());
+  if (N < 0 || C < 0 || H < 0 || W < 0 || K_H < 1 || K_W < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0)
+    return fail(WF2HIP_EINVAL, "unfold: negative extent or non-positive kernel / stride");
+  if (H + 2 * pad_h < K_H || W + 2 * pad_w < K_W) return fail(WF2HIP_EINVAL, "unfold: kernel larger than the padded image");
+  const long H_out = (H + 2 * pad_h - K_H) / stride_h + 1, W_out = (W + 2 * pad_w - K_W) / stride_w + 1;
+  const int64_t limit = (int64_t)1 << 31;
+  const int64_t Q = (int64_t)C * K_H * K_W, rows = (int64_t)N * H_out * W_out;
+  if (rows == 0 || Q == 0) return 0;
+  if (!x || !out) return fail(WF2HIP_EINVAL, "null tensor pointer");
+  if (Q >= limit || H_out * W_out >= limit || (int64_t)H * W >= limit || stride_h * H_out + pad_h >= limit ||
+      stride_w * W_out + pad_w >= limit)
+    return fail(WF2HIP_EUNSUPPORTED, "unfold: extent beyond 2^31");
+  {  // out must not overlap x
+    const float* xe = x + (int64_t)N * C * H * W;
+    const float* oe = out + rows * Q;
+    if (x < oe && out < xe) return fail(WF2HIP_EOVERLAP, "unfold: the matrix overlaps the image");
+  }
+  UnfoldFused p;
+  p.src = x; p.dst = out;
+  p.C = (uint32_t)C; p.H = (uint32_t)H; p.W = (uint32_t)W; p.H_out = (uint32_t)H_out; p.W_out = (uint32_t)W_out;
+  p.K_H = (uint32_t)K_H; p.K_W = (uint32_t)K_W; p.s_h = (uint32_t)stride_h; p.s_w = (uint32_t)stride_w;
+  p.pad_h = (uint32_t)pad_h; p.pad_w = (uint32_t)pad_w;
+  p.Q = (uint32_t)Q;
+  const int64_t KK = K_H * K_W;
+  const int64_t TW = (W_out - 1) * stride_w + K_W;
+  // The split into bands of output rows and chunks of channels, among those whose tile and tables
+  // fit 60 KB of LDS.  Measured on (32, 64, 56, 56) with a 3 x 3 kernel (231 MB written): runs whose
+  // length is not a multiple of 64 bytes double the time (104 us against 55 us), more than 32 KB
+  // of LDS per workgroup costs a fifth (66 us), idle lanes at the end of a run and the image rows
+  // that neighbouring bands both read cost little.
+  if (KK > 1024) return fail(WF2HIP_EUNSUPPORTED, "unfold: kernels up to 1024 elements");
+  auto tile_rows = [&](int64_t b) { return (b - 1) * stride_h + K_H; };
+  auto lds_floats = [&](int64_t b, int64_t c) { return c * tile_rows(b) * TW + c * KK + b * W_out; };
+  const int64_t ceiling = (60 << 10) / 4, roomy = (32 << 10) / 4;
+  int64_t band = 0, cc = 0;
+  double best = 0.0;
+  for (int64_t b = std::max<int64_t>(1, std::min<int64_t>(256 / W_out, H_out)); b >= 1; b = b > 1 ? (b + 1) / 2 : 0) {
+    const int64_t most = std::min<int64_t>({C, 1024 / KK, (ceiling - b * W_out) / (tile_rows(b) * TW + KK)});
+    for (int64_t c = most; c >= 1; c--) {
+      const int64_t whole = C / c, last = C - whole * c;  // chunks of c channels and a shorter one
+      const int64_t slots = whole * ceil_div(c * KK, kWave) + (last ? ceil_div(last * KK, kWave) : 0);
+      const double lanes = (double)Q / (double)(slots * kWave);
+      const double reads = (double)(tile_rows(b) * TW) / (double)(b * W_out * KK);
+      const bool aligned = (c * KK) % 16 == 0 || c == C;
+      const double score = lanes * (aligned ? 1.0 : 0.5) * (lds_floats(b, c) <= roomy ? 1.0 : 0.85) / (1.0 + 0.3 * reads);
+      if (band == 0 || score > best * 1.02) {  // near ties go to the longer run, tried first
+        best = score;
+        band = b;
+        cc = c;
+      }
+    }
+  }
+  if (const char* force = getenv("WF2HIP_UNFOLD_SPLIT")) {  // experiment knob: "band,cc"
+    long fb = 0, fc = 0;
+    if (sscanf(force, "%ld,%ld", &fb, &fc) == 2 && fb >= 1 && fc >= 1 && fc * KK <= 1024 &&
+        lds_floats(fb, fc) <= (60 << 10) / 4) {
+      band = std::min<int64_t>(fb, H_out);
+      cc = std::min<int64_t>(fc, C);
+    }
+  }
+  if (band == 0)
+    return fail(WF2HIP_EUNSUPPORTED, "unfold: one channel of one output row needs more than 60 KB of LDS (compose it from nodes)");
+  p.band = (uint32_t)band;
+  p.bands = (uint32_t)ceil_div(H_out, band);
+  p.cc = (uint32_t)cc;
+  p.chunks = (uint32_t)ceil_div(C, cc);
+  p.TR = (uint32_t)tile_rows(band);
+  p.TW = (uint32_t)TW;
+  p.by_kk = make_fastdiv((uint32_t)KK);
+  p.by_kw = make_fastdiv(p.K_W);
+  p.by_w_out = make_fastdiv(p.W_out);
+  p.by_plane = make_fastdiv(p.TR * p.TW);
+  p.by_tw = make_fastdiv(p.TW);
+  const int64_t blocks = (int64_t)N * p.bands * p.chunks;
+  if (blocks >= limit) return fail(WF2HIP_EUNSUPPORTED, "unfold: too many workgroups");
+  const size_t bytes = (size_t)lds_floats(band, cc) * sizeof(float);
+  const int64_t per_lane = ceil_div(cc * KK, kWave);
+  hipStream_t st = rt().stream;
+#define WF2_CASE(NQ_)                                                                                            \
+  if (per_lane <= NQ_) {                                                                                         \
+    static bool configured = false;                                                                              \
+    if (!configured) {                                                                                           \
+      WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&unfold_kernel<NQ_>),                  \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 64 << 10),              \
+                        "hipFuncSetAttribute(unfold_kernel)"));                                                  \
+      configured = true;                                                                                         \
+    }                                                                                                            \
+    unfold_kernel<NQ_><<<(uint32_t)blocks, kBlock, bytes, st>>>(p);                                              \
+    return after_launch("unfold_kernel");                                                                        \
+  }
+  WF2_CASE(1)
+  WF2_CASE(2)
+  WF2_CASE(3)
+  WF2_CASE(4)
+  WF2_CASE(6)
+  WF2_CASE(8)
+  WF2_CASE(12)
+  WF2_CASE(16)
+#undef WF2_CASE
+  return fail(WF2HIP_EINVAL, "unfold: bad run length");
 }

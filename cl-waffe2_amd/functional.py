@@ -292,12 +292,12 @@ def im2col(padded_x: HIPTensor, kernel_size, h_out: int, w_out: int, stride, pad
     return reshape(col.permute(0, 4, 5, 1, 2, 3), N * h_out * w_out, Cc * kernel_size[0] * kernel_size[1])
 
 
-def unfold(x: HIPTensor, dilation, kernel_size, stride, pad) -> HIPTensor:
+def unfold_composed(x: HIPTensor, dilation, kernel_size, stride, pad) -> HIPTensor:
     """``(unfold input dilation kernel-size stride padding)``
-    (``source/nn/im2col.lisp:51-95``): sliding local blocks of a ``[N C H W]``
-    tensor as rows of a ``[(N h-out w-out) (C k-h k-w)]`` matrix.  The input is
-    padded by ``(pad, pad + out mod stride)`` on each spatial axis first, as the
-    reference does."""
+    (``source/nn/im2col.lisp:51-95``) node for node: sliding local blocks of a
+    ``[N C H W]`` tensor as rows of a ``[(N h-out w-out) (C k-h k-w)]`` matrix.  The
+    input is padded by ``(pad, pad + out mod stride)`` on each spatial axis first, as
+    the reference does."""
     if len(x.shape) != 4:
         raise ValueError("unfold takes a [N C H W] tensor")
     H, W = x.shape[2:]
@@ -305,6 +305,44 @@ def unfold(x: HIPTensor, dilation, kernel_size, stride, pad) -> HIPTensor:
     w_out = conv_out_size(W, pad[1], dilation[0], kernel_size[1], stride[1])   # (car dilation) twice: sic
     px = padding(x, [True, True, (pad[0], pad[0] + h_out % stride[0]), (pad[1], pad[1] + w_out % stride[1])])
     return im2col(px, kernel_size, h_out, w_out, stride, pad, dilation)
+
+
+def unfold(x: HIPTensor, dilation, kernel_size, stride, pad) -> HIPTensor:
+    """``(unfold input dilation kernel-size stride padding)``.  On :float tensors with
+    dilation 1 and the symbolic path enabled this is ONE node (HIP-Unfold-Node, the
+    bypass ``unfold-hip`` of the Lisp glue), bit for bit the matrix the composition
+    leaves (`unfold_composed`); otherwise the composition itself."""
+    if len(x.shape) != 4:
+        raise ValueError("unfold takes a [N C H W] tensor")
+    if not (ENABLE_SYMBOLIC_PATH and x.dtype == "float" and tuple(dilation) == (1, 1)):
+        return unfold_composed(x, dilation, kernel_size, stride, pad)
+    N, Cc, H, W = x.shape
+    h_out = conv_out_size(H, pad[0], 1, kernel_size[0], stride[0])
+    w_out = conv_out_size(W, pad[1], 1, kernel_size[1], stride[1])
+    out = HIPTensor([N * h_out * w_out, Cc * kernel_size[0] * kernel_size[1]], initial_element=None)
+    try:
+        return nodes.forward("HIP-Unfold-Node", to_contiguous(x), out, kernel_size, stride, pad)
+    except _lib.HIPError as err:
+        if err.code != _lib.EUNSUPPORTED:  # rows too wide for the kernel's staging memory: compose
+            raise
+        return unfold_composed(x, dilation, kernel_size, stride, pad)
+
+
+def unfold_backward(dcol: HIPTensor, x_shape, kernel_size, stride, pad) -> HIPTensor:
+    """The gradient of :func:`unfold` with respect to its input, as the reference's nodes derive it:
+    the reshape and the permutation undone (a copy into ``[N C k-h k-w h-out w-out]``),
+    Col2ImNode into the padded image, the interior of the padding."""
+    N, Cc, H, W = x_shape
+    kh, kw = kernel_size
+    h_out = conv_out_size(H, pad[0], 1, kh, stride[0])
+    w_out = conv_out_size(W, pad[1], 1, kw, stride[1])
+    col = to_contiguous(reshape(dcol, N, h_out, w_out, Cc, kh, kw).permute(0, 3, 4, 5, 1, 2))
+    Hp, Wp = H + 2 * pad[0] + h_out % stride[0], W + 2 * pad[1] + w_out % stride[1]
+    px = HIPTensor([N, Cc, Hp, Wp], initial_element=None)
+    nodes.forward("Col2ImNode", col, px, stride, pad, (1, 1))
+    if (Hp, Wp) == (H, W):
+        return px
+    return to_contiguous(px.view(True, True, (pad[0], pad[0] + H), (pad[1], pad[1] + W)))
 
 
 # ---------------------------------------------------------------------------

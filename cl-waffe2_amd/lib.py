@@ -190,6 +190,7 @@ _SIGNATURES = {
        for n in ("eq", "lt", "le", "gt", "ge")},
     "wf2hip_im2col_f32": ([_P] + [_L] * 14 + [_P], C.c_int),
     "wf2hip_col2im_f32": ([_P] + [_L] * 14 + [_P], C.c_int),
+    "wf2hip_unfold_f32": ([_L] * 10 + [_P, _P], C.c_int),
     "wf2hip_sgd_step_f32": ([_L, _P, _P, _F], C.c_int),
     "wf2hip_adam_step_f32": ([_L, _P, _P, _P, _P, _F, _F, _F, _F], C.c_int),
     "wf2hip_embedding_add_f32": ([_L, _L, _L, _P, _P, _L, _P, _L, _P], C.c_int),

@@ -155,6 +155,9 @@
 (defcfun "wf2hip_col2im_f32" :int
   (col :pointer) (n :long) (c :long) (h :long) (w :long) (h-out :long) (w-out :long) (k-h :long) (k-w :long)
   (pad-h :long) (pad-w :long) (stride-h :long) (stride-w :long) (dilation-h :long) (dilation-w :long) (im :pointer))
+;; unfold (source/nn/im2col.lisp:51-95) with dilation 1 as one kernel: padding, Im2ColNode, permutation and reshape
+(defcfun "wf2hip_unfold_f32" :int (n :long) (c :long) (h :long) (w :long) (k-h :long) (k-w :long) (stride-h :long)
+  (stride-w :long) (pad-h :long) (pad-w :long) (x :pointer) (out :pointer))
 (defcfun "wf2hip_sgd_step_f32" :int (n :long) (param :pointer) (grad :pointer) (lr :float))
 (defcfun "wf2hip_adam_step_f32" :int
   (n :long) (param :pointer) (grad :pointer) (m :pointer) (v :pointer)

@@ -232,6 +232,76 @@ the reference's node."
       (call-composed 'cl-waffe2/nn:softmax-cross-entropy x labels :axis axis :delta delta
                                                               :avoid-overflow avoid-overflow :reduction reduction)))
 
+;; ---- unfold ------------------------------------------------------------------------------------
+(defun unfold-out-size (size pad kernel stride)
+  "conv-out-size (source/nn/pool.lisp:10-17) with dilation 1."
+  (1+ (floor (- (+ size (* 2 pad)) kernel) stride)))
+
+(defun unfold-gradient (dout input-shape kernel-size stride padding)
+  "The gradient of unfold with respect to its input as the reference's nodes derive it: the reshape and
+the permutation undone (a copy into [N C k-h k-w h-out w-out]), Col2ImNode's kernel into the padded image,
+the interior of the padding."
+  (ensure-extension)
+  (destructuring-bind (n c h w) input-shape
+    (let* ((k-h (first kernel-size)) (k-w (second kernel-size))
+           (s-h (first stride)) (s-w (second stride))
+           (p-h (first padding)) (p-w (second padding))
+           (h-out (unfold-out-size h p-h k-h s-h))
+           (w-out (unfold-out-size w p-w k-w s-w))
+           (hp (+ h (* 2 p-h) (mod h-out s-h)))
+           (wp (+ w (* 2 p-w) (mod w-out s-w)))
+           (col (eager-contiguous (!permute (!reshape dout n h-out w-out c k-h k-w) (torch-order 0 3 4 5 1 2))))
+           (padded (make-tensor (list n c hp wp) :dtype :float :order (order dout) :device 'HIPTensor)))
+      (check (wf2hip-col2im-f32 (tensor-device-pointer col) n c hp wp h-out w-out k-h k-w p-h p-w s-h s-w 1 1
+                                (tensor-device-pointer padded)))
+      (if (and (= hp h) (= wp w))
+          padded
+          (eager-contiguous (view padded t t (list p-h (+ p-h h)) (list p-w (+ p-w w))))))))
+
+(define-op (HIP-Unfold-Node (self kernel-size stride padding)
+            :slots ((kernel-size :initform nil :accessor unfold-kernel-size)
+                    (stride :initform nil :accessor unfold-stride)
+                    (padding :initform nil :accessor unfold-padding)
+                    (input-shape :initform nil :accessor unfold-input-shape))
+            :where (X[N C H W] OUT[rows cols] -> OUT[rows cols])
+            :documentation "OUT[(N h-out w-out) (C k-h k-w)] <- unfold of the contiguous image X with dilation 1
+(source/nn/im2col.lisp:51-95): the padding, Im2ColNode, the permutation and the reshape as one kernel
+(wf2hip_unfold_f32), bit for bit the matrix the composition leaves.  Backward: the reference's own."
+            :forward ((self x out)
+                      (ensure-extension)
+                      (setf (unfold-input-shape self) (copy-list (shape x)))
+                      (destructuring-bind (n c h w) (shape x)
+                        (check (wf2hip-unfold-f32 n c h w
+                                                  (first (unfold-kernel-size self)) (second (unfold-kernel-size self))
+                                                  (first (unfold-stride self)) (second (unfold-stride self))
+                                                  (first (unfold-padding self)) (second (unfold-padding self))
+                                                  (tensor-device-pointer x) (tensor-device-pointer out))))
+                      out)
+            :backward ((self dout)
+                       (values (unfold-gradient dout (unfold-input-shape self) (unfold-kernel-size self)
+                                                (unfold-stride self) (unfold-padding self))
+                               nil)))
+  (setf (unfold-kernel-size self) kernel-size
+        (unfold-stride self) stride
+        (unfold-padding self) padding))
+
+(defun unfold-hip (input dilation kernel-size stride padding)
+  "(unfold input dilation kernel-size stride padding) on a :float device image of static shape with
+dilation 1 as one kernel; anything else takes the reference's composition."
+  (if (and (hip-float-tensor-p input)
+           (= (length (shape input)) 4)
+           (every #'numberp (shape input))
+           (equal dilation '(1 1))
+           (every #'integerp (append kernel-size stride padding)))
+      (destructuring-bind (n c h w) (shape input)
+        (let ((h-out (unfold-out-size h (first padding) (first kernel-size) (first stride)))
+              (w-out (unfold-out-size w (second padding) (second kernel-size) (second stride))))
+          (call (HIP-Unfold-Node kernel-size stride padding)
+                (->contiguous input)
+                (make-input (list (* n h-out w-out) (* c (first kernel-size) (second kernel-size))) nil
+                            :dtype :float :order (order input)))))
+      (call-composed 'cl-waffe2/nn:unfold input dilation kernel-size stride padding)))
+
 ;; ---- LayerNorm over the last axis ------------------------------------------------------------
 (defun layer-norm-gradients (x g dout eps)
   "Gradients of y = (x - u) / sqrt(s + eps) * g + b per row (source/nn/norms.lisp:72-82) from the
@@ -584,5 +654,6 @@ pass :scale (/ 1.0 seq) for its numbers, :causal t for a decoder)."
 (define-bypass HIPTensor cl-waffe2/nn:!gelu !gelu-hip)
 (define-bypass HIPTensor cl-waffe2/nn:!softmax !softmax-hip)
 (define-bypass HIPTensor cl-waffe2/nn:softmax-cross-entropy softmax-cross-entropy-hip)
+(define-bypass HIPTensor cl-waffe2/nn:unfold unfold-hip)
 (define-bypass HIPTensor cl-waffe2/base-impl:!sum !sum-hip)
 (define-bypass HIPTensor cl-waffe2/base-impl:!mean !mean-hip)

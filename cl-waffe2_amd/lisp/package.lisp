@@ -15,7 +15,7 @@ kernels are the hand-written gfx950 kernels of libwaffe2-hip.so.")
    #:hip-error
    #:!relu-hip #:!leaky-relu-hip #:!sigmoid-hip #:!gelu-hip #:!softmax-hip #:!layer-norm-hip
    #:!sum-hip #:!mean-hip #:!linear-hip #:!causal-softmax-hip #:!attention-hip
-   #:softmax-cross-entropy-hip))
+   #:softmax-cross-entropy-hip #:unfold-hip))
 
 (in-package :cl-waffe2/backends.hip)
 

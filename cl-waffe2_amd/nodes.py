@@ -38,6 +38,7 @@ NODE_NAMES = (
     # the define-op nodes of lisp/fusion.lisp (one kernel each)
     "HIP-Sum-Node", "HIP-Activation-Node", "HIP-Softmax-Node", "HIP-LayerNorm-Node", "HIP-Linear-Node",
     "HIP-Linear-Residual-Node", "HIP-Causal-Softmax-Node", "HIP-Attention-Node", "HIP-Softmax-Cross-Entropy-Node",
+    "HIP-Unfold-Node",
     # the -backward nodes define-op generates for them, where the backward is one kernel too
     "HIP-Activation-Node-backward", "HIP-Softmax-Node-backward", "HIP-Causal-Softmax-Node-backward",
     "HIP-LayerNorm-Node-backward", "HIP-Attention-Node-backward", "HIP-Softmax-Cross-Entropy-Node-backward",
@@ -336,6 +337,23 @@ def _col2im(col: HIPTensor, x: HIPTensor, stride, padding, dilation) -> HIPTenso
     args = _unfold_args(x.shape, col.shape, stride, padding, dilation)
     _lib.check(_lib.get().wf2hip_col2im_f32(C.c_void_p(col.ptr), *args, C.c_void_p(x.ptr)))
     return x
+
+
+@define_impl("HIP-Unfold-Node", HIPTensor, _only_float)
+def _unfold_node(x: HIPTensor, out: HIPTensor, kernel_size, stride, padding) -> HIPTensor:
+    """``X[N C H W] OUT[(N h-out w-out) (C k-h k-w)] -> OUT``: ``unfold`` with dilation 1
+    (``source/nn/im2col.lisp:51-95``: padding, Im2ColNode, permutation, reshape) as one kernel."""
+    if len(x.shape) != 4:
+        raise ValueError("HIP-Unfold-Node takes a [N C H W] tensor")
+    _require_rows("HIP-Unfold-Node: x", x)
+    N, Cc, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = ((int(v[0]), int(v[1])) for v in (kernel_size, stride, padding))
+    if min(kh, kw, sh, sw) < 1 or min(ph, pw) < 0 or H + 2 * ph < kh or W + 2 * pw < kw:
+        raise ValueError(f"HIP-Unfold-Node: kernel {kh, kw}, stride {sh, sw}, padding {ph, pw} on a {H} x {W} image")
+    h_out, w_out = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    _require_rows("HIP-Unfold-Node: out", out, [N * h_out * w_out, Cc * kh * kw])
+    _lib.check(_lib.get().wf2hip_unfold_f32(N, Cc, H, W, kh, kw, sh, sw, ph, pw, C.c_void_p(x.ptr), C.c_void_p(out.ptr)))
+    return out
 
 
 def _matrix_geometry(t: HIPTensor, what: str):

@@ -746,6 +746,18 @@ int wf2hip_im2col_f32(float* col, long N, long C, long H, long W, long H_out, lo
 int wf2hip_col2im_f32(const float* col, long N, long C, long H, long W, long H_out, long W_out,
                       long K_H, long K_W, long pad_h, long pad_w, long stride_h, long stride_w,
                       long dilation_h, long dilation_w, float* im);
+/* (unfold input dilation kernel-size stride padding) of source/nn/im2col.lisp:51-95
+ * with dilation 1 as one kernel: out[(n i j), (c kh kw)], a row-major
+ * (N H_out W_out) x (C K_H K_W) matrix, from the unpadded image x[N C H W], with
+ * H_out = (H + 2 pad_h - K_H) / stride_h + 1 (conv-out-size, source/nn/pool.lisp:10-17)
+ * and W_out likewise.  Bit for bit what the reference's composition leaves in a
+ * fresh matrix: the zero padding, Im2ColNode's walk (positions it does not reach
+ * hold 0), the permuting copy and the reshape.  Its backward is the reference's own
+ * (permute back, wf2hip_col2im_f32, the interior of the padded image).
+ * WF2HIP_EUNSUPPORTED when one channel of one output row does not fit the kernel's
+ * staging memory (compose it from the nodes then). */
+int wf2hip_unfold_f32(long N, long C, long H, long W, long K_H, long K_W, long stride_h,
+                      long stride_w, long pad_h, long pad_w, const float* x, float* out);
 
 /* ---- optimiser steps (extension) ------------------------------------------ */
 /* One pass per parameter tensor, performing the binary32 operations of the

@@ -183,3 +183,87 @@ def test_conv_and_pooling_layers(gpu, stride):
     assert_bit_equal(W.nn.max_pool2d(F.from_numpy(x), 2).numpy(), pw.max(axis=(4, 5)), "max pool")
     np.testing.assert_allclose(W.nn.avg_pool2d(F.from_numpy(x), 2).numpy(),
                                pw.astype(np.float64).mean(axis=(4, 5)), rtol=1e-6, atol=1e-6)
+
+
+UNFOLD_CASES = [
+    # N, C, H, W, kernel, stride, padding
+    (2, 3, 12, 11, (3, 2), (1, 1), (0, 0)),
+    (2, 3, 12, 11, (3, 3), (1, 1), (1, 1)),      # padded: the walk leaves the last row and column of every plane at 0
+    (3, 5, 17, 19, (3, 3), (2, 2), (1, 1)),
+    (2, 4, 16, 16, (2, 2), (2, 2), (0, 0)),      # pooling windows
+    (1, 1, 28, 28, (5, 5), (1, 1), (2, 2)),
+    (2, 2, 9, 40, (1, 1), (1, 1), (0, 0)),
+    (2, 70, 20, 20, (3, 3), (1, 1), (1, 1)),     # channels in chunks, the last one short
+    (1, 3, 70, 300, (3, 3), (1, 1), (1, 1)),     # rows wider than a band of 256 positions
+    (1, 2, 33, 31, (7, 7), (3, 2), (3, 3)),
+    (2, 3, 15, 14, (4, 3), (3, 4), (2, 1)),      # kernel smaller than the stride along W
+    (4, 64, 56, 56, (3, 3), (1, 1), (1, 1)),     # a ResNet-style layer
+    (1, 2, 6, 2200, (3, 3), (1, 1), (0, 0)),     # one channel of one output row needs more than the first budget
+]
+
+
+@pytest.mark.parametrize("N,Cc,H,Wd,k,s,p", UNFOLD_CASES)
+def test_unfold_as_one_node_is_the_composition(gpu, N, Cc, H, Wd, k, s, p):
+    """HIP-Unfold-Node against the node composition of unfold (padding, Im2ColNode into a zeroed col,
+    permutation, reshape), which the reference's vectors and the compiled im2col pin: pure data
+    movement, so bit for bit, -0.0 and NaN included."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(H * 131 + Wd)
+    x = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
+    x.flat[:3] = [-0.0, np.nan, np.inf]
+    dx = F.from_numpy(x)
+    want = F.unfold_composed(dx, (1, 1), k, s, p).numpy()
+    out = F.unfold(dx, (1, 1), k, s, p)
+    assert out.shape == list(want.shape)
+    assert_bit_equal(out.numpy(), want, "unfold")
+    assert_bit_equal(dx.numpy(), x, "x untouched")
+
+
+def test_unfold_node_arguments_and_fallback(gpu):
+    W = gpu
+    F = W.functional
+    import ctypes as C
+    lib = W.lib.get()
+    x = W.HIPTensor([1, 1, 4, 4])
+    out = W.HIPTensor([9, 4])
+    ptr = lambda t: C.c_void_p(t.ptr)  # noqa: E731
+    assert lib.wf2hip_unfold_f32(1, 1, 4, 4, 2, 2, 1, 1, 0, 0, ptr(x), ptr(out)) == 0
+    assert lib.wf2hip_unfold_f32(1, 1, 4, 4, 5, 2, 1, 1, 0, 0, ptr(x), ptr(out)) == W.lib.EINVAL    # kernel taller than the image
+    assert lib.wf2hip_unfold_f32(1, 1, 4, 4, 2, 2, 0, 1, 0, 0, ptr(x), ptr(out)) == W.lib.EINVAL
+    assert lib.wf2hip_unfold_f32(1, 1, 4, 4, 2, 2, 1, 1, 0, 0, ptr(x), None) == W.lib.EINVAL
+    assert lib.wf2hip_unfold_f32(1, 1, 4, 4, 2, 2, 1, 1, 0, 0, ptr(x), ptr(x)) == W.lib.EOVERLAP
+    assert lib.wf2hip_unfold_f32(0, 1, 4, 4, 2, 2, 1, 1, 0, 0, ptr(x), ptr(out)) == 0
+    with pytest.raises(ValueError):
+        W.forward("HIP-Unfold-Node", x, W.HIPTensor([9, 5]), (2, 2), (1, 1), (0, 0))
+    # a row too wide for the kernel's staging memory: the library refuses, unfold composes
+    wide = F.from_numpy(np.random.default_rng(1).standard_normal((1, 1, 3, 20000)).astype(np.float32))
+    tall_out = W.HIPTensor([19998, 9])
+    assert lib.wf2hip_unfold_f32(1, 1, 3, 20000, 3, 3, 1, 1, 0, 0, ptr(wide), ptr(tall_out)) == W.lib.EUNSUPPORTED
+    assert_bit_equal(F.unfold(wide, (1, 1), (3, 3), (1, 1), (0, 0)).numpy(),
+                     F.unfold_composed(wide, (1, 1), (3, 3), (1, 1), (0, 0)).numpy(), "fallback")
+
+
+@pytest.mark.parametrize("N,Cc,H,Wd,k,s,p", UNFOLD_CASES[:10])
+def test_unfold_backward_is_the_adjoint(gpu, N, Cc, H, Wd, k, s, p):
+    """<unfold(x), c> = <x, unfold_backward(c)> where the walk reaches every position (no padding), and in
+    general unfold_backward(c) is the float64 gradient of sum(unfold(x) * c) by its definition: each
+    element of x collects the c of the matrix entries that hold it."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(H * 7 + Wd)
+    x = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
+    col = F.unfold(F.from_numpy(x), (1, 1), k, s, p).numpy()
+    c = rng.standard_normal(col.shape).astype(np.float32)
+    back = F.unfold_backward(F.from_numpy(c), x.shape, k, s, p).numpy()
+    assert back.shape == x.shape
+    # the matrix entries as a linear map of x: push an index image through the same unfold
+    idx = np.arange(1, x.size + 1, dtype=np.float32).reshape(x.shape)       # exact below 2^24
+    assert x.size < 2 ** 24
+    where = F.unfold(F.from_numpy(idx), (1, 1), k, s, p).numpy().astype(np.int64)   # 0: padding or not reached
+    want = np.zeros(x.size + 1, np.float64)
+    np.add.at(want, where.ravel(), c.astype(np.float64).ravel())
+    want = want[1:].reshape(x.shape)
+    mag = np.zeros(x.size + 1, np.float64)
+    np.add.at(mag, where.ravel(), np.abs(c).astype(np.float64).ravel())
+    assert np.all(np.abs(back - want) <= 1e-6 * mag[1:].reshape(x.shape) + 1e-30)
