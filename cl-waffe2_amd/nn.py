@@ -60,6 +60,55 @@ def avg_pool2d(x: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
 
 
 # ---------------------------------------------------------------------------
+# backward of the layers above, as the nodes' own backward definitions compose it
+# ---------------------------------------------------------------------------
+
+def conv2d_backward(x: HIPTensor, weight: HIPTensor, dout: HIPTensor, stride=1, padding=0, bias: bool = True):
+    """``(dx, dweight, dbias)`` of :func:`conv2d` for the upstream gradient ``dout[N C_out H_out W_out]``:
+    the permutation of the output undone, MatMulNode's two backward products (dY^T . col and dY . W,
+    ``base-impl/matrix-ops.lisp:10-15``), the column sums the AddNode of the bias sends back, and the
+    backward of unfold.  ``col`` is recomputed (the reference saves it)."""
+    stride, padding = _pair(stride), _pair(padding)
+    N, _, H, W = x.shape
+    c_out, c_in, kh, kw = weight.shape
+    col = F.unfold(x, (1, 1), (kh, kw), stride, padding)                 # [(N h w) (C k-h k-w)]
+    dy = F.reshape(dout.permute(0, 2, 3, 1), -1, c_out)                  # [(N h w) C_out], a copy
+    col_w = F.reshape(weight, c_out, -1)
+    dweight = F.reshape(F.matmul(F.t(dy), col), c_out, c_in, kh, kw)
+    dbias = F.sum(dy, axis=0) if bias else None
+    dcol = F.matmul(dy, col_w)
+    return F.unfold_backward(dcol, x.shape, (kh, kw), stride, padding), dweight, dbias
+
+
+def _pool_backward(x: HIPTensor, dout: HIPTensor, kernel_size, stride, padding, spread) -> HIPTensor:
+    kernel_size, stride, padding = _pair(kernel_size), _pair(stride), _pair(padding)
+    N, Cc, H, W = x.shape
+    k = kernel_size[0] * kernel_size[1]
+    windows = F.reshape(F.unfold(x, (1, 1), kernel_size, stride, padding), -1, k)   # [(N h w C) (k-h k-w)]
+    d = F.reshape(dout.permute(0, 2, 3, 1), -1, 1)                                    # [(N h w C) 1], a copy
+    dwin = spread(windows, d.view(True, (":broadcast", k)))
+    return F.unfold_backward(F.reshape(dwin, -1, Cc * k), x.shape, kernel_size, stride, padding)
+
+
+def max_pool2d_backward(x: HIPTensor, dout: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
+    """The gradient of :func:`max_pool2d`: MaxValue-Node sends ``dout`` to every element of a window that
+    equals its maximum (the mask ``A=B a max(a)``, ``base-impl/matrix-ops.lisp:312-334``), unfold's backward
+    folds the windows."""
+    def spread(windows, d):
+        top = F.max(windows, axis=1, keepdims=True)
+        return F.mul_(F.compare(windows, top, "="), d)
+    return _pool_backward(x, dout, kernel_size, kernel_size if stride is None else stride, padding, spread)
+
+
+def avg_pool2d_backward(x: HIPTensor, dout: HIPTensor, kernel_size, stride=None, padding=0) -> HIPTensor:
+    """The gradient of :func:`avg_pool2d`: ``dout / (k-h k-w)`` to every element of the window."""
+    k = _pair(kernel_size)
+    def spread(windows, d):
+        return F.div_(F.copy(d), float(k[0] * k[1]))
+    return _pool_backward(x, dout, kernel_size, kernel_size if stride is None else stride, padding, spread)
+
+
+# ---------------------------------------------------------------------------
 # criteria (source/nn/criterion.lisp), composed from the backend's nodes
 # ---------------------------------------------------------------------------
 
