@@ -271,6 +271,26 @@ def row_probe(W, reps: int = 5):
     dg, db = T([Cn], initial_element=None), T([Cn], initial_element=None)
     run("LayerNorm backward (65536,1024)", 12 * R * Cn, lambda: (F.copy(a0), F.copy(a0), T([R, Cn], initial_element=None)),
         lambda s: W.nodes.forward("HIP-LayerNorm-Node-backward", s[0], g0, s[1], s[2], dg, db, 1e-5), launches=3)
+    del a0, g0, dg, db
+    R, Cn = 32768, 1024
+    a0 = normal([R, Cn], 3.0)
+    t0 = F.softmax_fused(normal([R, Cn]))
+    run("softmax cross entropy (32768,1024)", 16 * R * Cn,
+        lambda: (F.copy(a0), F.copy(t0), T([R, Cn], initial_element=None), T([R, Cn], initial_element=None)),
+        lambda s: W.nodes.forward("HIP-Softmax-Cross-Entropy-Node", s[0], s[1], s[2], s[3], 1e-7))
+    run("softmax cross entropy backward (32768,1024)", 16 * R * Cn, lambda: (F.copy(a0), F.copy(t0), F.copy(t0)),
+        lambda s: W.nn.softmax_cross_entropy_backward_fused(s[0], s[1], s[2], in_place=True))
+    del a0, t0
+    Nb, Cc, Hh, Kk = 32, 64, 56, 3
+    img, padded = normal([Nb, Cc, Hh, Hh]), normal([Nb, Cc, Hh + 2, Hh + 2])
+    ncol, nim = Nb * Cc * Kk * Kk * Hh * Hh, Nb * Cc * Hh * Hh
+    run("unfold (32,64,56,56) 3x3 pad 1", 4 * (ncol + nim), lambda: T([Nb * Hh * Hh, Cc * Kk * Kk], initial_element=None),
+        lambda s: W.nodes.forward("HIP-Unfold-Node", img, s, (Kk, Kk), (1, 1), (1, 1)))
+    run("Im2ColNode (32,64,58,58) 3x3", 4 * (ncol + nim), lambda: T([Nb, Cc, Kk, Kk, Hh, Hh], initial_element=None),
+        lambda s: W.nodes.forward("Im2ColNode", padded, s, (1, 1), (0, 0), (1, 1)))
+    back = T([Nb, Cc, Hh + 2, Hh + 2], initial_element=None)
+    run("Col2ImNode (32,64,3,3,56,56)", 4 * (ncol + nim), lambda: normal([Nb, Cc, Kk, Kk, Hh, Hh]),
+        lambda s: W.nodes.forward("Col2ImNode", s, back, (1, 1), (1, 1), (1, 1)))
     print(json.dumps({"probe_rows": order}))
 
 

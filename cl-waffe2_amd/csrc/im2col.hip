@@ -26,8 +26,6 @@
 // where windows do not overlap; col2im_kernel beyond 2^31 elements).
 // HBM-bound: 4 (k-h k-w h-out w-out + H W) bytes per image plane.
 #include <algorithm>
-#include <cstdio>
-#include <cstdlib>
 
 #include "wf2_common.h"
 #include "wf2_fastdiv.h"
@@ -659,14 +657,6 @@ WF2_API int wf2hip_unfold_f32(long N, long C, long H, long W, long K_H, long K_W
         band = b;
         cc = c;
       }
-    }
-  }
-  if (const char* force = getenv("WF2HIP_UNFOLD_SPLIT")) {  // experiment knob: "band,cc"
-    long fb = 0, fc = 0;
-    if (sscanf(force, "%ld,%ld", &fb, &fc) == 2 && fb >= 1 && fc >= 1 && fc * KK <= 1024 &&
-        lds_floats(fb, fc) <= (60 << 10) / 4) {
-      band = std::min<int64_t>(fb, H_out);
-      cc = std::min<int64_t>(fc, C);
     }
   }
   if (band == 0)
