@@ -272,7 +272,7 @@ static int launch_layernorm_bwd(int nv, uint32_t blocks, const float* x, const f
 // sce-diff-static of Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:82-88, 103-110): the
 // SubNode, MulNode and DivNode of dx = (dy (z - labels)) / batch in one pass, every operation
 // rounded to binary32 as those nodes round them.  BCAST: dy is one number (the gradient that a
-// !sum or !mean of the loss hands down through its broadcasting view).  Two 16-byte vectors per
+// !sum or !mean of the loss hands down through its broadcasting view).  Four 16-byte vectors per
 // thread and stream, all loads issued before the arithmetic.
 __device__ __forceinline__ float xent_grad(float dy, float z, float label, float batch) {
   return (dy * (z - label)) / batch;
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kBlock) void xent_bwd_kernel(const float* dy, const
                                                           float batch) {
   const float d0 = BCAST ? dy[0] : 0.0f;
   if (VEC) {
-    constexpr int U = 2;
+    constexpr int U = 4;
     const size_t nvec = n / 4;
     const size_t base = ((size_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kWave * U + (threadIdx.x & (kWave - 1));
     f4 dv[U], zv[U], tv[U];
@@ -324,12 +324,12 @@ template <bool BCAST>
 static int launch_xent_bwd(const float* dy, const float* z, const float* labels, float* dx, int64_t n, float batch) {
   const bool vec = aligned16(z) && aligned16(labels) && aligned16(dx) && (BCAST || aligned16(dy));
   const int64_t nvec = n / 4 > 0 ? n / 4 : 1;
-  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 2) : ceil_div(n, kBlock);
+  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 4) : ceil_div(n, kBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
   hipStream_t st = rt().stream;
   const bool streaming = n * (BCAST ? 12 : 16) >= ((int64_t)192 << 20);
   // every workgroup full: no bounds tests, so a thread's loads are all issued before its first wait
-  if (vec && streaming && n % (4 * kBlock * 2) == 0)
+  if (vec && streaming && n % (4 * kBlock * 4) == 0)
     xent_bwd_kernel<true, true, BCAST, true><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);
   else if (vec && streaming)
     xent_bwd_kernel<true, true, BCAST><<<(uint32_t)blocks, kBlock, 0, st>>>(dy, z, labels, dx, (size_t)n, batch);

@@ -23,15 +23,15 @@ __device__ __forceinline__ void adam1(float& p, float g, float& m, float& v, flo
   p = p - (m * lr_t) / (eps + __builtin_sqrtf(v));
 }
 
-// VEC: two 16-byte vectors per thread and stream, all loads issued before the
-// arithmetic; NT: streaming hint for tensors far beyond the Infinity Cache.
+// VEC: four 16-byte vectors per thread and stream (2^26 parameters: one 65 %, two 76 %, four 78 %,
+// eight 67 % of the HBM peak), all loads issued before the arithmetic; NT: streaming hint for tensors far beyond the Infinity Cache.
 template <bool VEC, bool NT, bool FULL = false>
 __global__ __launch_bounds__(kBlock) void adam_kernel(float* __restrict__ p, const float* __restrict__ g,
                                                       float* __restrict__ m, float* __restrict__ v,
                                                       size_t n, float omb1, float omb2, float lr_t,
                                                       float eps) {
   if (VEC) {
-    constexpr int U = 2;
+    constexpr int U = 4;
     const size_t nvec = n / 4;
     // each wavefront on 1 KB of its own per access and stream
     const size_t base = ((size_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWave * U +
@@ -149,13 +149,13 @@ WF2_API int wf2hip_adam_step_f32(long n, float* param, const float* grad, float*
         return fail(WF2HIP_EOVERLAP, "adam step: parameter, gradient and moments must not overlap");
   const bool vec = aligned16(param) && aligned16(grad) && aligned16(m) && aligned16(v);
   const int64_t nvec = n / 4 > 0 ? n / 4 : 1;
-  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 2) : ceil_div(n, kBlock);
+  const int64_t blocks = vec ? ceil_div(nvec, (int64_t)kBlock * 4) : ceil_div(n, kBlock);
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many elements for one launch");
   hipStream_t st = rt().stream;
   const bool streaming = (int64_t)n * 28 >= ((int64_t)192 << 20);
-  // every workgroup full: no bounds tests, so all eight loads of a thread are issued before its first
-  // wait (2^26 parameters: 315.4 -> 304.2 us, 74.4 -> 77.3 % of the HBM peak)
-  if (vec && streaming && n % (4 * kBlock * 2) == 0)
+  // every workgroup full: no bounds tests, so all sixteen loads of a thread are issued before its first
+  // wait (2^26 parameters with two vectors per thread and stream: 315.4 -> 304.2 us)
+  if (vec && streaming && n % (4 * kBlock * 4) == 0)
     adam_kernel<true, true, true><<<(uint32_t)blocks, kBlock, 0, st>>>(param, grad, m, v, (size_t)n,
                                                                       one_minus_beta1, one_minus_beta2, lr_t, eps);
   else if (vec && streaming)
