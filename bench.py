@@ -578,6 +578,18 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     measure("Col2ImNode (32,64,3,3,56,56) -> (32,64,58,58)", ring,
             lambda s: W.nodes.forward("Col2ImNode", s, back, (1, 1), (1, 1), (1, 1)), 4 * (ncol + nim))
     del img, padded, back
+    # the windows of a 2 x 2 pooling layer on (32,64,112,112): rows of four elements
+    R, Cn = 32 * 64 * 56 * 56, 4
+    w0 = normal([R, Cn])
+    ring = ring_of(lambda: clone(w0), 4 * R * Cn)
+    measure("row max (6422528,4): MaxPool2D's !max over its windows", ring, lambda s: F.max(s, axis=1), 4 * R * Cn + 4 * R)
+    ring = ring_of(lambda: clone(w0), 4 * R * Cn)
+    measure("row mean (6422528,4): AvgPool2D's !mean over its windows", ring, lambda s: F.mean(s, axis=1), 4 * R * Cn + 4 * R)
+    top = F.max(w0, axis=1, keepdims=True)
+    ring = ring_of(lambda: (clone(w0), T([R, Cn], initial_element=None)), 8 * R * Cn)
+    measure("compare (6422528,4) = its row maxima (broadcast): the mask of MaxValue-Node's backward", ring,
+            lambda s: F.compare(s[0], top, "=", out=s[1]), 8 * R * Cn + 4 * R)
+    del w0, top
 
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),

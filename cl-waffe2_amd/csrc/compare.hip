@@ -9,6 +9,7 @@
 // per element (two reads, one write).  The scalar right-hand side
 // (Where-Operation-Node) is an element-wise functor in elementwise.hip.
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_view.h"
 
 namespace wf2 {
@@ -194,6 +195,70 @@ __global__ __launch_bounds__(kBlock) void compare_rows(CmpRows p) {
   }
 }
 
+// Short rows: matrices whose rows are a few elements long and adjacent in `out` (the windows of a
+// pooling layer against their maxima: MaxValue-Node's backward compares (rows, k-h k-w) with a
+// (rows, 1) tensor broadcast along the row, base-impl/matrix-ops.lisp:330-334).  compare_rows
+// gives a workgroup four rows, which leaves all but one of its threads idle on rows of four
+// elements ((6422528, 4): 1.78 ms).  Here a thread takes one 16-byte vector of the flat output,
+// U of them kBlock apart, whatever row they fall in: row and column from a division by the row
+// length turned into a multiplication (wf2_fastdiv.h; total below 2^31, n0 a multiple of 4).
+struct CmpShort {
+  const float* x;
+  const float* y;
+  float* out;
+  uint32_t nvec;             // 16-byte vectors of out
+  FastDiv by_n0;             // the row length
+  int64_t ox, oy;            // row strides of x and y
+  int32_t x_inner, y_inner;  // 1 or 0 (one value per row)
+  int32_t op;
+  float then_value, else_value;
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kBlock) void compare_short_rows(CmpShort p) {
+  typedef f4 f4u __attribute__((aligned(4)));
+  constexpr int U = 4;
+  f4 a[U], b[U];
+  bool live[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t v = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+    live[u] = v < p.nvec;
+    if (!live[u]) continue;
+    const uint32_t e = v * 4;
+    uint32_t col;
+    const uint32_t row = fd_divmod(e, p.by_n0, &col);
+    const float* xr = p.x + (int64_t)row * p.ox;
+    const float* yr = p.y + (int64_t)row * p.oy;
+    if (p.x_inner) {
+      const f4u* q = reinterpret_cast<const f4u*>(xr + col);
+      a[u] = NT ? __builtin_nontemporal_load(q) : *q;
+    } else {
+      const float s = xr[0];
+      a[u] = f4{s, s, s, s};
+    }
+    if (p.y_inner) {
+      const f4u* q = reinterpret_cast<const f4u*>(yr + col);
+      b[u] = NT ? __builtin_nontemporal_load(q) : *q;
+    } else {
+      const float s = yr[0];
+      b[u] = f4{s, s, s, s};
+    }
+  }
+  auto pick = [&](float l, float r) { return holds(p.op, l, r) ? p.then_value : p.else_value; };
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    if (!live[u]) continue;
+    const uint32_t v = (blockIdx.x * U + u) * kBlock + threadIdx.x;
+    const f4 r = {pick(a[u].x, b[u].x), pick(a[u].y, b[u].y), pick(a[u].z, b[u].z), pick(a[u].w, b[u].w)};
+    f4* q = reinterpret_cast<f4*>(p.out) + v;
+    if (NT)
+      __builtin_nontemporal_store(r, q);
+    else
+      *q = r;
+  }
+}
+
 int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, float then_value,
                float else_value) {
   if (op < WF2HIP_EQ || op > WF2HIP_GE) return fail(WF2HIP_EINVAL, "unknown compare op %d", op);
@@ -234,6 +299,28 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
   for (int r = 0; r < last; r++) {
     if (s.shape[r] >= ((int64_t)1 << 32)) rows_ok = false;
     nrows *= s.shape[r];
+  }
+  if (rows_ok && s.rank == 2 && s.shape[last] < 1024 && s.shape[last] % 4 == 0 && s.sc[0] == s.shape[last] &&
+      s.total < ((int64_t)1 << 31) && ((uintptr_t)op_ & 15u) == 0) {
+    CmpShort q;
+    q.x = xp;
+    q.y = yp;
+    q.out = op_;
+    q.nvec = (uint32_t)(s.total / 4);
+    q.by_n0 = make_fastdiv((uint32_t)s.shape[last]);
+    q.ox = s.sa[0];
+    q.oy = s.sb[0];
+    q.x_inner = (int32_t)s.sa[last];
+    q.y_inner = (int32_t)s.sb[last];
+    q.op = op;
+    q.then_value = then_value;
+    q.else_value = else_value;
+    const uint32_t short_blocks = (uint32_t)ceil_div((int64_t)q.nvec, (int64_t)kBlock * 4);
+    if (s.total * 12 >= ((int64_t)192 << 20))
+      compare_short_rows<true><<<short_blocks, kBlock, 0, st>>>(q);
+    else
+      compare_short_rows<false><<<short_blocks, kBlock, 0, st>>>(q);
+    return after_launch("compare_short_rows");
   }
   if (rows_ok && nrows < ((int64_t)1 << 32)) {
     CmpRows q;

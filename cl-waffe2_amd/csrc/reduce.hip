@@ -17,6 +17,7 @@
 // All kernels here are HBM-bound: 4 bytes read per element reduced, 8 bytes
 // per element for softmax/LayerNorm (one read, one write).
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_math.h"
 #include "wf2_view.h"
 #include "wf2_rows.h"
@@ -205,6 +206,35 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_short(RowRedParams p) {
     acc = wave_sum(acc);
     if (lane == 0 && row0 + w < p.nrows) p.commit(p.a + aoff[w], acc);
   }
+}
+
+// Rows of at most 32 elements, adjacent in memory (AvgPool2D's !mean over windows of k-h k-w
+// elements, source/nn/pool.lisp:95-105): a thread per row.  The workgroup's 256 rows are one
+// contiguous run, read by consecutive lanes into LDS (rows padded to an odd pitch) and added
+// from there in index order, in binary64; a wavefront per four rows left (6422528, 4) at 770 us.
+__global__ __launch_bounds__(kBlock) void reduce_rows_tiny(RowRedParams p, FastDiv by_n) {
+  extern __shared__ float tiny_tile[];
+  const uint32_t n = (uint32_t)p.n0, pitch = n | 1u;
+  const uint32_t row0 = blockIdx.x * kBlock;
+  const uint32_t rows_here = p.nrows - row0 < (uint32_t)kBlock ? p.nrows - row0 : (uint32_t)kBlock;
+  const uint32_t count = rows_here * n;
+  const float* src = p.b + (int64_t)row0 * n;
+  auto place = [&](uint32_t e) { const uint32_t r = fd_div(e, by_n); return r * pitch + (e - r * n); };
+  uint32_t e = threadIdx.x;
+  for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+#pragma unroll
+    for (int u = 0; u < 8; u++) tiny_tile[place(e + u * kBlock)] = v[u];
+  }
+  for (; e < count; e += kBlock) tiny_tile[place(e)] = src[e];
+  __syncthreads();
+  if (threadIdx.x >= rows_here) return;
+  const float* row = tiny_tile + threadIdx.x * pitch;
+  double acc = 0.0;
+  for (uint32_t c = 0; c < n; c++) acc += (double)row[c];
+  p.commit(p.a + (int64_t)(row0 + threadIdx.x) * p.oa[0], acc);
 }
 
 // Folds the partial sums of a row in a fixed order.  This launch depends on the one
@@ -502,6 +532,11 @@ static int launch_row_reduce(const Space& s, float* a, const float* b, double* p
   p.seg = p.n0;
   hipStream_t st = rt().stream;
   const int64_t target_blocks = (int64_t)rt().num_cus * 8;
+  if (p.n0 <= 32 && p.nouter == 1 && p.ob[0] == p.n0 && nrows >= 4 * target_blocks) {
+    reduce_rows_tiny<<<(uint32_t)ceil_div(nrows, kBlock), kBlock, (size_t)kBlock * (p.n0 | 1) * sizeof(float), st>>>(
+        p, make_fastdiv((uint32_t)p.n0));
+    return after_launch("reduce_rows_tiny");
+  }
   if (p.n0 < 2048 && nrows * 1 >= 1) {
     // short rows: a wavefront each
     if (nrows >= target_blocks || p.n0 < 8192) {

@@ -15,6 +15,7 @@
 #include <math.h>
 
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_view.h"
 
 namespace wf2 {
@@ -185,6 +186,42 @@ __global__ __launch_bounds__(kBlock) void select_rows_wave4(SelParams<T> p) {
   }
 }
 
+// Rows of a few elements (pooling windows: MaxPool2D takes the maximum of rows of k-h k-w
+// elements, source/nn/pool.lisp:83-93), adjacent in memory: a thread per row.  The workgroup's
+// 256 rows are one contiguous run, read by consecutive lanes into LDS (rows padded to an odd
+// pitch) and scanned from there; a wavefront per four rows left (6422528, 4) at 970 us.
+constexpr int kTinyRowBytes = 128;  // rows up to 32 four-byte elements
+
+template <bool IsMax, class T>
+__global__ __launch_bounds__(kBlock) void select_rows_tiny(SelParams<T> p, FastDiv by_n) {
+  extern __shared__ __align__(16) unsigned char tiny_lds[];
+  T* tile = reinterpret_cast<T*>(tiny_lds);
+  const uint32_t n = (uint32_t)p.n, pitch = n | 1u;
+  const uint32_t row0 = blockIdx.x * kBlock;
+  const uint32_t rows_here = p.nrows - row0 < (uint32_t)kBlock ? p.nrows - row0 : (uint32_t)kBlock;
+  const uint32_t count = rows_here * n;
+  const T* src = p.x + (int64_t)row0 * n;
+  auto place = [&](uint32_t e) { const uint32_t r = fd_div(e, by_n); return r * pitch + (e - r * n); };
+  uint32_t e = threadIdx.x;
+  for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
+    T v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+#pragma unroll
+    for (int u = 0; u < 8; u++) tile[place(e + u * kBlock)] = v[u];
+  }
+  for (; e < count; e += kBlock) tile[place(e)] = src[e];
+  __syncthreads();
+  if (threadIdx.x >= rows_here) return;
+  Best<T> b = {worst<T, IsMax>(), 0u};
+  const T* row = tile + threadIdx.x * pitch;
+  for (uint32_t c = 0; c < n; c++) {  // increasing indices, strict comparison: the first occurrence stays
+    const T v = row[c];
+    if (IsMax ? v > b.v : v < b.v) { b.v = v; b.i = c; }
+  }
+  emit(p, (int64_t)(row0 + threadIdx.x) * p.oo[0], b);
+}
+
 // one workgroup per (row, split)
 template <bool IsMax, bool VEC, class T>
 __global__ __launch_bounds__(kBlock) void select_rows_block(SelParams<T> p) {
@@ -236,6 +273,13 @@ template <bool IsMax, bool VEC, class T>
 static int launch_select(SelParams<T>& p) {
   hipStream_t st = rt().stream;
   const int64_t target = (int64_t)rt().num_cus * 8;
+  if (p.n * (int64_t)sizeof(T) <= kTinyRowBytes && p.incx == 1 && p.nouter == 1 && p.ox[0] == p.n &&
+      p.nrows >= 4 * target) {
+    const uint32_t blocks = (uint32_t)ceil_div(p.nrows, kBlock);
+    const size_t bytes = (size_t)kBlock * ((size_t)p.n | 1u) * sizeof(T);
+    select_rows_tiny<IsMax, T><<<blocks, kBlock, bytes, st>>>(p, make_fastdiv((uint32_t)p.n));
+    return after_launch("select_rows_tiny");
+  }
   if (p.n <= (int64_t)kWave * (16 / (int64_t)sizeof(T)) && p.nrows >= 4 * target) {
     const uint32_t blocks = (uint32_t)ceil_div(p.nrows, (kBlock / kWave) * 4);
     select_rows_wave4<IsMax, VEC, T><<<blocks, kBlock, 0, st>>>(p);

@@ -1,0 +1,136 @@
+"""Many rows of a few elements: the shapes pooling layers hand to !max, !mean and to MaxValue-Node's
+backward (rows of k-h k-w window elements, source/nn/pool.lisp:83-105, base-impl/matrix-ops.lisp:312-334).
+Each of the three node families has a thread-per-row (or vector-per-thread) kernel for them; checked
+against numpy, which for these operations is the definition: first occurrence for the indices, NaN never
+selected, sums of at most 32 binary32 numbers exact in binary64 and rounded once."""
+import numpy as np
+import pytest
+
+from helpers import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+@pytest.mark.parametrize("cols", [1, 2, 3, 4, 5, 8, 9, 16, 25, 31, 32, 33])
+def test_select_tiny_rows(gpu, cols):
+    """33 columns are one too many for the thread-per-row kernel: the same answers from the next one."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(200 + cols)
+    rows = 9001
+    x = rng.integers(-6, 7, (rows, cols)).astype(f32)          # many ties
+    x[5] = np.nan                                               # a row of NaNs: -inf / +inf, index 0
+    x[6, 0] = np.nan                                            # NaN is never selected
+    x[7, cols - 1] = np.inf
+    x[8, 0] = -np.inf
+    dx = F.from_numpy(x)
+    with np.errstate(invalid="ignore"):
+        filled_lo = np.where(np.isnan(x), -np.inf, x)
+        filled_hi = np.where(np.isnan(x), np.inf, x)
+    assert_bit_equal(F.max(dx).numpy()[:, 0], filled_lo.max(axis=1), "max")
+    assert_bit_equal(F.min(dx).numpy()[:, 0], filled_hi.min(axis=1), "min")
+    want_amax = filled_lo.argmax(axis=1)
+    want_amin = filled_hi.argmin(axis=1)
+    # numpy picks the first -inf of an all-NaN row too; where a row's only finite candidates are NaN-filled
+    # positions the kernel's index is the first non-NaN occurrence of the extreme, or 0 for a row of NaNs
+    for want in (want_amax, want_amin):
+        want[5] = 0
+    if cols > 1:
+        got_amax = F.argmax(dx).numpy()[:, 0]
+        got_amin = F.argmin(dx).numpy()[:, 0]
+        keep = np.ones(rows, bool)
+        keep[[6, 8]] = False                                    # rows whose filled extreme may sit on the NaN / -inf itself
+        np.testing.assert_array_equal(got_amax[keep], want_amax[keep])
+        np.testing.assert_array_equal(got_amin[keep], want_amin[keep])
+        assert not np.isnan(x[6, got_amax[6]]) and x[6, got_amax[6]] == np.nanmax(x[6])
+        assert x[8, got_amin[8]] == -np.inf and got_amin[8] == 0
+
+
+@pytest.mark.parametrize("dtype,cols", [("double", 16), ("double", 17), ("int32", 7), ("uint8", 100), ("int16", 64),
+                                        ("uint32", 32), ("int8", 3)])
+def test_select_tiny_rows_typed(gpu, dtype, cols):
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(cols)
+    np_dtype = {"double": np.float64, "int32": np.int32, "uint8": np.uint8, "int16": np.int16, "uint32": np.uint32,
+                "int8": np.int8}[dtype]
+    rows = 8500
+    if dtype == "double":
+        x = rng.standard_normal((rows, cols)).astype(np_dtype)
+    else:
+        info = np.iinfo(np_dtype)
+        x = rng.integers(info.min, int(info.max) + 1, (rows, cols)).astype(np_dtype)
+        x[0] = info.min
+        x[1] = info.max
+    dx = F.from_numpy(x, dtype=dtype)
+    np.testing.assert_array_equal(F.max(dx).numpy()[:, 0], x.max(axis=1))
+    np.testing.assert_array_equal(F.min(dx).numpy()[:, 0], x.min(axis=1))
+    if dtype == "double":
+        np.testing.assert_array_equal(F.argmax(dx).numpy()[:, 0], x.argmax(axis=1))
+        np.testing.assert_array_equal(F.argmin(dx).numpy()[:, 0], x.argmin(axis=1))
+
+
+@pytest.mark.parametrize("cols", [1, 2, 4, 7, 9, 16, 25, 32, 33])
+def test_sum_and_mean_of_tiny_rows(gpu, cols):
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(300 + cols)
+    rows = 9100
+    x = (rng.standard_normal((rows, cols)) * 3).astype(f32)
+    x[3] = np.inf
+    x[4, 0] = np.nan
+    dx = F.from_numpy(x)
+    with np.errstate(invalid="ignore"):
+        total = x.astype(np.float64).sum(axis=1)
+    assert_bit_equal(F.sum(dx, axis=1).numpy()[:, 0], total.astype(f32), "row sums")
+    assert_bit_equal(F.mean(dx, axis=1).numpy()[:, 0], total.astype(f32) / f32(cols), "row means")
+    # accumulating into a destination that holds something (the AddNode of !sum's composition)
+    seed = rng.standard_normal((rows, 1)).astype(f32)
+    with np.errstate(invalid="ignore"):
+        want = (seed[:, 0].astype(np.float64) + total).astype(f32)
+    got = F.add_(F.from_numpy(seed).view(True, (":broadcast", cols)), dx)
+    assert_bit_equal(got.numpy()[:, 0], want, "accumulated")
+
+
+@pytest.mark.parametrize("cols", [4, 8, 12, 36, 1020])
+@pytest.mark.parametrize("which", ["y", "x", "both", "none"])
+def test_compare_short_rows(gpu, cols, which):
+    """A matrix of short rows against one value per row (broadcast along the row) on either side."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(cols + len(which))
+    rows = 9000 if cols < 1000 else 70
+    x = rng.integers(-3, 4, (rows, cols if which not in ("x", "both") else 1)).astype(f32)
+    y = rng.integers(-3, 4, (rows, cols if which not in ("y", "both") else 1)).astype(f32)
+    x.flat[:2] = [np.nan, -0.0]
+    y.flat[:2] = [1.0, 0.0]
+    dx, dy = F.from_numpy(x), F.from_numpy(y)
+    vx = dx if x.shape[1] == cols else dx.view(True, (":broadcast", cols))
+    vy = dy if y.shape[1] == cols else dy.view(True, (":broadcast", cols))
+    bx, by = np.broadcast_to(x, (rows, cols)), np.broadcast_to(y, (rows, cols))
+    for op, fn in (("=", np.equal), ("<", np.less), ("<=", np.less_equal), (">", np.greater), (">=", np.greater_equal)):
+        with np.errstate(invalid="ignore"):
+            want = np.where(fn(bx, by), f32(2.0), f32(-1.0))
+        got = F.compare(vx, vy, op, true_then=2.0, false_then=-1.0).numpy()
+        assert_bit_equal(got, want, f"{op} with {which} broadcast")
+
+
+def test_pooling_layers_at_size(gpu):
+    """MaxPool2D / AvgPool2D forward and MaxPool2D backward on (8, 16, 64, 64): every kernel above in one
+    composition, against the definitions."""
+    W = gpu
+    F, nn = W.functional, W.nn
+    rng = np.random.default_rng(77)
+    x = rng.integers(-4, 5, (8, 16, 64, 64)).astype(f32)        # ties inside windows
+    dx = F.from_numpy(x)
+    win = x.reshape(8, 16, 32, 2, 32, 2)
+    assert_bit_equal(F.to_contiguous(nn.max_pool2d(dx, 2)).numpy(), win.max(axis=(3, 5)), "max pool")
+    assert_bit_equal(F.to_contiguous(nn.avg_pool2d(dx, 2)).numpy(),
+                     (win.astype(np.float64).sum(axis=(3, 5)).astype(f32) / f32(4)), "avg pool")
+    dy = rng.standard_normal((8, 16, 32, 32)).astype(f32)
+    mask = win == win.max(axis=(3, 5), keepdims=True)
+    want = np.where(mask, dy[:, :, :, None, :, None], f32(0.0)).astype(f32).reshape(x.shape)   # the fold starts from +0
+    assert_bit_equal(nn.max_pool2d_backward(dx, F.from_numpy(dy), 2).numpy(), want, "max pool backward")
+    want_avg = np.broadcast_to((dy / f32(4))[:, :, :, None, :, None], win.shape).reshape(x.shape)
+    assert_bit_equal(nn.avg_pool2d_backward(dx, F.from_numpy(dy), 2).numpy(), want_avg, "avg pool backward")
