@@ -201,12 +201,12 @@ __global__ __launch_bounds__(kBlock) void compare_rows(CmpRows p) {
 // gives a workgroup four rows, which leaves all but one of its threads idle on rows of four
 // elements ((6422528, 4): 1.78 ms).  Here a thread takes one 16-byte vector of the flat output,
 // U of them kBlock apart, whatever row they fall in: row and column from a division by the row
-// length turned into a multiplication (wf2_fastdiv.h; total below 2^31, n0 a multiple of 4).
+// length turned into a multiplication (wf2_fastdiv.h; total below 2^31).
 struct CmpShort {
   const float* x;
   const float* y;
   float* out;
-  uint32_t nvec;             // 16-byte vectors of out
+  uint32_t nvec, total;      // 16-byte vectors of out (the last one may be partial); elements
   FastDiv by_n0;             // the row length
   int64_t ox, oy;            // row strides of x and y
   int32_t x_inner, y_inner;  // 1 or 0 (one value per row)
@@ -214,7 +214,8 @@ struct CmpShort {
   float then_value, else_value;
 };
 
-template <bool NT>
+// ALIGNED: the row length is a multiple of 4, so a thread's vector lies in one row.
+template <bool NT, bool ALIGNED>
 __global__ __launch_bounds__(kBlock) void compare_short_rows(CmpShort p) {
   typedef f4 f4u __attribute__((aligned(4)));
   constexpr int U = 4;
@@ -226,23 +227,34 @@ __global__ __launch_bounds__(kBlock) void compare_short_rows(CmpShort p) {
     live[u] = v < p.nvec;
     if (!live[u]) continue;
     const uint32_t e = v * 4;
-    uint32_t col;
-    const uint32_t row = fd_divmod(e, p.by_n0, &col);
-    const float* xr = p.x + (int64_t)row * p.ox;
-    const float* yr = p.y + (int64_t)row * p.oy;
-    if (p.x_inner) {
-      const f4u* q = reinterpret_cast<const f4u*>(xr + col);
-      a[u] = NT ? __builtin_nontemporal_load(q) : *q;
-    } else {
-      const float s = xr[0];
-      a[u] = f4{s, s, s, s};
-    }
-    if (p.y_inner) {
-      const f4u* q = reinterpret_cast<const f4u*>(yr + col);
-      b[u] = NT ? __builtin_nontemporal_load(q) : *q;
-    } else {
-      const float s = yr[0];
-      b[u] = f4{s, s, s, s};
+    if (ALIGNED) {
+      uint32_t col;
+      const uint32_t row = fd_divmod(e, p.by_n0, &col);
+      const float* xr = p.x + (int64_t)row * p.ox;
+      const float* yr = p.y + (int64_t)row * p.oy;
+      if (p.x_inner) {
+        const f4u* q = reinterpret_cast<const f4u*>(xr + col);
+        a[u] = NT ? __builtin_nontemporal_load(q) : *q;
+      } else {
+        const float s = xr[0];
+        a[u] = f4{s, s, s, s};
+      }
+      if (p.y_inner) {
+        const f4u* q = reinterpret_cast<const f4u*>(yr + col);
+        b[u] = NT ? __builtin_nontemporal_load(q) : *q;
+      } else {
+        const float s = yr[0];
+        b[u] = f4{s, s, s, s};
+      }
+    } else {  // the four elements may lie in two rows (or four, with rows of one to three elements)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        uint32_t col;
+        const uint32_t at = e + c < p.total ? e + c : p.total - 1;
+        const uint32_t row = fd_divmod(at, p.by_n0, &col);
+        a[u][c] = p.x[(int64_t)row * p.ox + (p.x_inner ? col : 0)];
+        b[u][c] = p.y[(int64_t)row * p.oy + (p.y_inner ? col : 0)];
+      }
     }
   }
   auto pick = [&](float l, float r) { return holds(p.op, l, r) ? p.then_value : p.else_value; };
@@ -251,11 +263,15 @@ __global__ __launch_bounds__(kBlock) void compare_short_rows(CmpShort p) {
     if (!live[u]) continue;
     const uint32_t v = (blockIdx.x * U + u) * kBlock + threadIdx.x;
     const f4 r = {pick(a[u].x, b[u].x), pick(a[u].y, b[u].y), pick(a[u].z, b[u].z), pick(a[u].w, b[u].w)};
-    f4* q = reinterpret_cast<f4*>(p.out) + v;
-    if (NT)
-      __builtin_nontemporal_store(r, q);
-    else
-      *q = r;
+    if (ALIGNED || v * 4 + 4 <= p.total) {
+      f4* q = reinterpret_cast<f4*>(p.out) + v;
+      if (NT)
+        __builtin_nontemporal_store(r, q);
+      else
+        *q = r;
+    } else {
+      for (uint32_t c = 0; v * 4 + c < p.total; c++) p.out[v * 4 + c] = r[c];
+    }
   }
 }
 
@@ -300,13 +316,16 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
     if (s.shape[r] >= ((int64_t)1 << 32)) rows_ok = false;
     nrows *= s.shape[r];
   }
-  if (rows_ok && s.rank == 2 && s.shape[last] < 1024 && s.shape[last] % 4 == 0 && s.sc[0] == s.shape[last] &&
-      s.total < ((int64_t)1 << 31) && ((uintptr_t)op_ & 15u) == 0) {
+  const bool short_rows = s.rank == 2 && s.sc[last] == 1 && (s.sa[last] == 1 || s.sa[last] == 0) &&
+                          (s.sb[last] == 1 || s.sb[last] == 0) && s.shape[last] < 1024 && s.sc[0] == s.shape[last] &&
+                          s.total < ((int64_t)1 << 31) - 4 && ((uintptr_t)op_ & 15u) == 0;
+  if (short_rows) {
     CmpShort q;
     q.x = xp;
     q.y = yp;
     q.out = op_;
-    q.nvec = (uint32_t)(s.total / 4);
+    q.nvec = (uint32_t)ceil_div(s.total, 4);
+    q.total = (uint32_t)s.total;
     q.by_n0 = make_fastdiv((uint32_t)s.shape[last]);
     q.ox = s.sa[0];
     q.oy = s.sb[0];
@@ -316,10 +335,12 @@ int compare_nd(int op, Space3 s, const float* x, const float* y, float* out, flo
     q.then_value = then_value;
     q.else_value = else_value;
     const uint32_t short_blocks = (uint32_t)ceil_div((int64_t)q.nvec, (int64_t)kBlock * 4);
-    if (s.total * 12 >= ((int64_t)192 << 20))
-      compare_short_rows<true><<<short_blocks, kBlock, 0, st>>>(q);
+    if (s.shape[last] % 4 != 0)
+      compare_short_rows<false, false><<<short_blocks, kBlock, 0, st>>>(q);
+    else if (s.total * 12 >= ((int64_t)192 << 20))
+      compare_short_rows<true, true><<<short_blocks, kBlock, 0, st>>>(q);
     else
-      compare_short_rows<false><<<short_blocks, kBlock, 0, st>>>(q);
+      compare_short_rows<false, true><<<short_blocks, kBlock, 0, st>>>(q);
     return after_launch("compare_short_rows");
   }
   if (rows_ok && nrows < ((int64_t)1 << 32)) {

@@ -845,6 +845,33 @@ __global__ __launch_bounds__(kBlock) void splitk_fold(const float* __restrict__ 
   *c = beta == 0.0f ? acc : beta * *c + acc;
 }
 
+// More than 16 partial products: a wavefront per output element, lane l adds slices l, l + 64, ...
+// in binary64 with eight loads in flight, the lanes meet by shuffles -- a fixed order.
+__global__ __launch_bounds__(kBlock) void splitk_fold_wide(const float* __restrict__ partials, int splits, int64_t m,
+                                                           int64_t n, float beta, float* __restrict__ C, int64_t ldc) {
+  const int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (e >= m * n) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t plane = m * n;
+  double acc = 0.0;
+  int s = lane;
+  for (; s + 7 * kWave < splits; s += 8 * kWave) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = partials[(int64_t)(s + u * kWave) * plane + e];
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc += (double)v[u];
+  }
+  for (; s < splits; s += kWave) acc += (double)partials[(int64_t)s * plane + e];
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) {
+    const int64_t j = e / m, i = e - j * m;
+    float* c = C + i + j * ldc;
+    *c = beta == 0.0f ? (float)acc : beta * *c + (float)acc;
+  }
+}
+
 int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha, const float* A,
                    long lda, long strideA, long strideA2, const float* B, long ldb, long strideB,
                    long strideB2, float beta, float* C, long ldc, long strideC, long strideC2,
@@ -860,8 +887,11 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
   const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128);
   const int64_t cus = rt().num_cus;
   if (k < 2048 || tiles >= cus || m < 1 || n < 1) return false;
+  // Few output tiles and a very long K (the weight gradient of a layer with few outputs:
+  // (10 x N) . (N x 256) over a batch of 65536 ran 150 us on 16 slices): as many slices of at
+  // least 512 as keep the launch within four workgroups per compute unit.
   int splits = 0;
-  for (int cand : {16, 8, 4, 2})
+  for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
     if (k % ((long)cand * 32) == 0 && k / cand >= 512 && tiles * cand <= 4 * cus) {
       splits = cand;
       break;
@@ -875,9 +905,15 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
   *rc = sgemm_batched2(transa, transb, m, n, kc, alpha, A, lda, sa, 0, B, ldb, sb, 0, 0.0f,
                        static_cast<float*>(scratch), m, (long)m * n, 0, splits, 1);
   if (*rc == 0) {
-    const int64_t blocks = ceil_div((int64_t)m * n, kBlock);
-    splitk_fold<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m, n, beta,
-                                                               C, ldc);
+    if (splits <= 16) {
+      const int64_t blocks = ceil_div((int64_t)m * n, kBlock);
+      splitk_fold<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m, n,
+                                                                 beta, C, ldc);
+    } else {
+      const int64_t blocks = ceil_div((int64_t)m * n, kBlock / kWave);
+      splitk_fold_wide<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m,
+                                                                      n, beta, C, ldc);
+    }
     *rc = after_launch("splitk_fold");
   }
   (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above

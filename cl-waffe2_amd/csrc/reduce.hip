@@ -391,6 +391,46 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_partial(ColRedParams q) {
   }
 }
 
+// Narrow dense matrices (bias gradients of a layer with few outputs: the column sums of
+// (N h w, C_out) or (N, classes)): up to 128 columns, rows adjacent in memory.  The 256-column
+// tiles above leave most lanes without a column, and below 64 columns the kept axis was handed
+// to the wavefront-per-output kernel, which walks a column with the row pitch as its stride
+// ((4194304, 4): 30 ms).  Here the workgroup reads k = 256 / ncols whole rows per step, one
+// contiguous run of k ncols floats: thread t adds column t mod ncols of every k-th row in
+// binary64, eight loads in flight, and the k threads of a column meet in LDS in a fixed order.
+__global__ __launch_bounds__(kBlock) void reduce_cols_narrow(ColRedParams q) {
+  __shared__ double lds[kBlock];
+  const AccParams& p = q.acc;
+  const uint32_t ncols = (uint32_t)q.ncols;
+  const uint32_t k = kBlock / ncols;  // rows per step
+  const uint32_t phase = threadIdx.x / ncols, col = threadIdx.x - phase * ncols;
+  const int64_t lo = (int64_t)blockIdx.x * q.seg;
+  const int64_t hi = lo + q.seg < p.nred ? lo + q.seg : p.nred;
+  double acc = 0.0;
+  if (phase < k) {
+    const float* src = p.b + col;
+    int64_t j = lo + phase;
+    for (; j + 7 * (int64_t)k < hi; j += 8 * (int64_t)k) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = src[(j + u * (int64_t)k) * ncols];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc += (double)v[u];
+    }
+    for (; j < hi; j += k) acc += (double)src[j * ncols];
+  }
+  lds[threadIdx.x] = acc;
+  __syncthreads();
+  if (threadIdx.x < ncols) {
+    double total = lds[threadIdx.x];
+    for (uint32_t r = 1; r < k; r++) total += lds[r * ncols + threadIdx.x];
+    if (q.splits == 1)
+      p.commit(p.a + threadIdx.x, total);
+    else
+      q.scratch[(int64_t)blockIdx.x * ncols + threadIdx.x] = total;
+  }
+}
+
 // Folds the splits' partial sums: 64 columns per workgroup, its four wavefronts take every
 // fourth split with eight loads in flight, then meet in LDS -- a fixed order.  (One thread per
 // column walking all splits in turn waits for memory once per split: 32 us for 128 splits of
@@ -418,14 +458,16 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_finish(ColRedParams q) {
     q.acc.commit(q.acc.a + c, (lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane]));
 }
 
-static int launch_col_reduce(const AccParams& p, int64_t ncols) {
+static int launch_col_reduce(const AccParams& p, int64_t ncols, bool narrow = false) {
   ColRedParams q;
   q.acc = p;
   q.ncols = ncols;
-  const int64_t ctiles = ceil_div(ncols, 256);
+  const int64_t ctiles = narrow ? 1 : ceil_div(ncols, 256);
   const int64_t target = (int64_t)rt().num_cus * 8;
   int64_t splits = ceil_div(target, ctiles);
-  if (splits > p.nred / 64) splits = p.nred / 64;  // at least 64 reduced indices per workgroup
+  // at least 64 reduced indices per workgroup (64 steps of whole rows in the narrow form)
+  const int64_t least = narrow ? 64 * (kBlock / ncols) : 64;
+  if (splits > p.nred / least) splits = p.nred / least;
   if (splits < 1) splits = 1;
   q.seg = ceil_div(ceil_div(p.nred, splits), 16) * 16;
   splits = ceil_div(p.nred, q.seg);
@@ -446,7 +488,9 @@ static int launch_col_reduce(const AccParams& p, int64_t ncols) {
     }
   }
   hipStream_t st = rt().stream;
-  if (p.nred * ncols * 4 >= ((int64_t)192 << 20))
+  if (narrow)
+    reduce_cols_narrow<<<(uint32_t)splits, kBlock, 0, st>>>(q);
+  else if (p.nred * ncols * 4 >= ((int64_t)192 << 20))
     reduce_cols_partial<true><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(q);
   else
     reduce_cols_partial<false><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(q);
@@ -632,7 +676,10 @@ static int launch_accumulate_with(int op, const Space& s, float* a, const float*
     if (s.shape[r] >= ((int64_t)1 << 32)) row_form = false;
   if (row_form) return launch_row_reduce(s, a, b, row_partials, commit);
   // column form: the only kept axis is the last one, contiguous on both sides
-  if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 16)
+  if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] <= 128 && p.nr == 1 &&
+      p.rb[0] == s.shape[last] && p.nred >= 16)
+    return launch_col_reduce(p, s.shape[last], true);  // a dense narrow matrix
+  if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 2)
     return launch_col_reduce(p, s.shape[last]);
   int64_t blocks = ceil_div(p.nout, kWavesPerBlock);
   if (blocks >= ((int64_t)1 << 31))

@@ -389,7 +389,10 @@ def test_matmul_few_tiles_long_k(gpu, ta, tb):
     W = gpu
     F = W.functional
     rng = np.random.default_rng(303 + ta + 2 * tb)
-    for m, n, k in [(768, 640, 8192), (200, 300, 4096), (130, 1000, 2048)]:
+    # the last four: tiny outputs over a very long K (the weight gradients of layers with few outputs),
+    # which run as up to 1024 slices folded by a wavefront per output element
+    for m, n, k in [(768, 640, 8192), (200, 300, 4096), (130, 1000, 2048), (10, 256, 65536), (256, 10, 65536),
+                    (4, 9, 100352), (3, 3, 1 << 20)]:
         A = rng.standard_normal((m, k)).astype(np.float32)
         B = rng.standard_normal((k, n)).astype(np.float32)
         dA = F.t(F.from_numpy(np.ascontiguousarray(A.T))) if ta else F.from_numpy(A)

@@ -93,14 +93,14 @@ def test_sum_and_mean_of_tiny_rows(gpu, cols):
     assert_bit_equal(got.numpy()[:, 0], want, "accumulated")
 
 
-@pytest.mark.parametrize("cols", [4, 8, 12, 36, 1020])
+@pytest.mark.parametrize("cols", [2, 3, 4, 5, 8, 10, 12, 33, 36, 1020, 1023])
 @pytest.mark.parametrize("which", ["y", "x", "both", "none"])
 def test_compare_short_rows(gpu, cols, which):
     """A matrix of short rows against one value per row (broadcast along the row) on either side."""
     W = gpu
     F = W.functional
     rng = np.random.default_rng(cols + len(which))
-    rows = 9000 if cols < 1000 else 70
+    rows = 9001 if cols < 1000 else 71
     x = rng.integers(-3, 4, (rows, cols if which not in ("x", "both") else 1)).astype(f32)
     y = rng.integers(-3, 4, (rows, cols if which not in ("y", "both") else 1)).astype(f32)
     x.flat[:2] = [np.nan, -0.0]
@@ -114,6 +114,30 @@ def test_compare_short_rows(gpu, cols, which):
             want = np.where(fn(bx, by), f32(2.0), f32(-1.0))
         got = F.compare(vx, vy, op, true_then=2.0, false_then=-1.0).numpy()
         assert_bit_equal(got, want, f"{op} with {which} broadcast")
+
+
+@pytest.mark.parametrize("rows,cols", [(400003, 3), (300000, 4), (100001, 10), (100352, 64), (70000, 100), (50000, 128),
+                                       (40000, 129), (3, 100000), (2, 70001), (15, 4097)])
+def test_column_sums_of_narrow_and_of_flat_matrices(gpu, rows, cols):
+    """!sum :axis 0 (bias gradients: the column sums of (N h w, C_out) or (N, classes)) where the matrix is
+    tall and narrow, and where it has only a few rows: binary64 partial sums, so the result is the float64 sum
+    rounded (exact for these magnitudes up to the last rounding, compared with one unit of slack)."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(f32)
+    dx = F.from_numpy(x)
+    want = x.astype(np.float64).sum(axis=0)
+    got = F.sum(dx, axis=0).numpy().ravel()
+    from helpers import ulp_distance
+    assert np.max(ulp_distance(got, want.astype(f32))) <= 1
+    assert np.max(np.abs(got - want)) <= 2.0 ** -23 * np.max(np.abs(x).astype(np.float64).sum(axis=0))
+    mean = F.mean(dx, axis=0).numpy().ravel()
+    assert np.max(np.abs(mean - want / rows)) <= 2.0 ** -22 * np.max(np.abs(want / rows)) + 1e-12
+    # into a destination that already holds values (AddNode into the broadcast view)
+    seed = rng.standard_normal((1, cols)).astype(f32)
+    acc = F.add_(F.from_numpy(seed).view((":broadcast", rows), True), dx).numpy()[0]
+    assert np.max(np.abs(acc - (seed[0] + want))) <= 2.0 ** -22 * (np.abs(seed[0]) + np.abs(want)).max()
 
 
 def test_pooling_layers_at_size(gpu):
