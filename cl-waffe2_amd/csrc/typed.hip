@@ -456,6 +456,25 @@ __global__ __launch_bounds__(kBlock) void typed_accumulate_add(T* a, const T* b,
   }
 }
 
+// Many destinations, few terms each (sums over a short trailing axis: (2097152, 4) rows): a thread
+// per destination adds its terms in index order.  A workgroup per destination takes 1.3 ms for
+// those two million sums of four.
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_thread(T* a, const T* b, TypedAcc p) {
+  using S = typename SumOf<T>::type;
+  const int64_t out = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (out >= p.nout) return;
+  int64_t aoff, boff;
+  acc_kept(p, out, &aoff, &boff);
+  S acc = S(0);
+  if (p.nr == 1) {
+    for (int64_t j = 0; j < p.nred; j++) acc += (S)b[boff + j * p.rb[0]];
+  } else {
+    for (int64_t j = 0; j < p.nred; j++) acc += (S)b[boff + acc_reduced(p, j)];
+  }
+  a[aoff] = (T)((S)a[aoff] + acc);
+}
+
 // Column form: the only kept axis is contiguous on both sides (sums over the leading
 // axes).  A thread owns one destination column, consecutive threads consecutive columns,
 // so every reduced index is one coalesced row segment; the reduced indices are split
@@ -589,7 +608,7 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
     using S = typename SumOf<T>::type;
     const int64_t target = (int64_t)rt().num_cus * 8;
     const int last = s.rank - 1;
-    if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 16) {
+    if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 2) {
       const int64_t ncols = s.shape[last];
       const int64_t ctiles = ceil_div(ncols, kBlock);
       int64_t splits = ceil_div(target, ctiles);
@@ -630,6 +649,10 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
       WF2_TRY(after_launch("typed_accumulate_partial"));
       typed_accumulate_fold<T><<<(uint32_t)ceil_div(p.nout, kWave), kWave, 0, st>>>(ap, p, (uint32_t)splits, partials);
       return after_launch("typed_accumulate_fold");
+    }
+    if (p.nred <= 128 && p.nout >= 64 * target) {
+      typed_accumulate_thread<T><<<(uint32_t)ceil_div(p.nout, kBlock), kBlock, 0, st>>>(ap, bp, p);
+      return after_launch("typed_accumulate_thread");
     }
     typed_accumulate_add<T><<<(uint32_t)p.nout, kBlock, 0, st>>>(ap, bp, p);
     return after_launch("typed_accumulate_add");

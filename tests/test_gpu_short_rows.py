@@ -140,6 +140,31 @@ def test_column_sums_of_narrow_and_of_flat_matrices(gpu, rows, cols):
     assert np.max(np.abs(acc - (seed[0] + want))) <= 2.0 ** -22 * (np.abs(seed[0]) + np.abs(want)).max()
 
 
+@pytest.mark.parametrize("dtype", ["double", "int32", "uint8", "int16"])
+@pytest.mark.parametrize("rows,cols", [(200001, 4), (140000, 9), (3, 70000)])
+def test_typed_sums_of_short_rows_and_of_flat_matrices(gpu, dtype, rows, cols):
+    """!sum on :double and the integer types (wrap-around sums, as the reference's C loops produce) along a
+    short trailing axis of very many rows, and down the few rows of a flat matrix."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(rows + cols)
+    np_dtype = {"double": np.float64, "int32": np.int32, "uint8": np.uint8, "int16": np.int16}[dtype]
+    if dtype == "double":
+        x = rng.standard_normal((rows, cols))
+    else:
+        info = np.iinfo(np_dtype)
+        x = rng.integers(info.min, int(info.max) + 1, (rows, cols)).astype(np_dtype)
+    dx = F.from_numpy(x, dtype=dtype)
+    for axis in (1, 0):
+        got = F.sum(dx, axis=axis).numpy().ravel()
+        if dtype == "double":
+            want = x.sum(axis=axis)
+            assert np.max(np.abs(got - want)) <= 1e-13 * np.abs(x).sum(axis=axis).max()
+        else:
+            want = x.astype(np.int64).sum(axis=axis).astype(np_dtype)    # modulo 2^bits
+            np.testing.assert_array_equal(got, want)
+
+
 def test_pooling_layers_at_size(gpu):
     """MaxPool2D / AvgPool2D forward and MaxPool2D backward on (8, 16, 64, 64): every kernel above in one
     composition, against the definitions."""
