@@ -165,6 +165,27 @@ def test_typed_sums_of_short_rows_and_of_flat_matrices(gpu, dtype, rows, cols):
             np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("shape,axes", [((32, 64, 28, 28), (0, 2, 3)), ((16, 3, 64, 64), (0, 2, 3)), ((6, 40, 50, 60), (1, 3)),
+                                        ((5, 70, 9, 1000), (0, 1, 3)), ((2, 3, 400000), (0, 2))])
+def test_sums_that_keep_a_middle_axis(gpu, shape, axes):
+    """Few destinations, each a long sum over axes on both sides of the kept ones: the per-channel sums of an
+    (N, C, H, W) tensor (batch-normalisation statistics, a channel-first bias gradient).  The reduced indices
+    of a destination are shared out over several workgroups and folded in binary64."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(f32)
+    dx = F.from_numpy(x)
+    want = x.astype(np.float64).sum(axis=axes, keepdims=True)
+    mag = np.abs(x).astype(np.float64).sum(axis=axes, keepdims=True)
+    got = F.sum(dx, axis=axes).numpy()
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= 2.0 ** -23 * mag)
+    count = np.prod([shape[a] for a in axes])
+    mean = F.mean(dx, axis=axes).numpy()
+    assert np.all(np.abs(mean - want / count) <= 2.0 ** -22 * mag / count)
+
+
 def test_pooling_layers_at_size(gpu):
     """MaxPool2D / AvgPool2D forward and MaxPool2D backward on (8, 16, 64, 64): every kernel above in one
     composition, against the definitions."""
