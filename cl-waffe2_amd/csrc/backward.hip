@@ -90,7 +90,9 @@ static int launch_softmax_bwd(int nv, const float* y, int64_t ldy, const float* 
     WF2_CASE(2)
     WF2_CASE(3)
     WF2_CASE(4)
+    WF2_CASE(5)
     WF2_CASE(6)
+    WF2_CASE(7)
     WF2_CASE(8)
     default: return fail(WF2HIP_EINVAL, "bad register tile");
   }
@@ -198,6 +200,114 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_rows(const float* __rest
   }
 }
 
+// Rows of 2049 ... 8192 columns: a workgroup per row, thread t holding the NG 16-byte vectors
+// (g 256 + t) 4 ... of x, dy and gamma and its share of the two column sums in registers; the
+// row statistics meet in LDS (three exchanges per row).  Workgroup b walks rows b, b + B, ...
+// and leaves its column sums in row b of `partial`, folded like the narrower kernel's.  Same
+// formulas as above: the mean from binary64 sums, deviations and squares in binary32.
+template <int NG, bool NT>
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __restrict__ x,
+                                                             const float* __restrict__ gamma,
+                                                             const float* dy, float eps,  // dx may be dy
+                                                             float* dx, float* __restrict__ partial,
+                                                             int64_t nrows, int64_t ncols) {
+  __shared__ double red[2][kWavesPerBlock];
+  const int wave = threadIdx.x / kWave;
+  // sum of v (and w) over the workgroup, in every thread; a fixed order
+  auto all_sum2 = [&](double v, double w, double* out_w) -> double {
+    v = wave_sum(v);
+    w = wave_sum(w);
+    __syncthreads();  // the previous exchange has been read
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      red[0][wave] = v;
+      red[1][wave] = w;
+    }
+    __syncthreads();
+    *out_w = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    return (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+  };
+  bool in[NG];
+  f4 g[NG], dg[NG], db[NG];
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    in[i] = c < ncols;  // ncols is a multiple of 4: a vector is wholly inside or outside
+    g[i] = in[i] ? *reinterpret_cast<const f4*>(gamma + c) : f4{0.f, 0.f, 0.f, 0.f};
+    dg[i] = db[i] = f4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float inv_n = 1.0f / (float)ncols;
+  for (int64_t row = blockIdx.x; row < nrows; row += gridDim.x) {
+    f4 xr[NG], dr[NG];
+#pragma unroll
+    for (int i = 0; i < NG; i++) {
+      const int64_t at = row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4;
+      xr[i] = dr[i] = f4{0.f, 0.f, 0.f, 0.f};
+      if (in[i]) {
+        const f4* px = reinterpret_cast<const f4*>(x + at);
+        const f4* pd = reinterpret_cast<const f4*>(dy + at);
+        xr[i] = NT ? __builtin_nontemporal_load(px) : *px;
+        dr[i] = NT ? __builtin_nontemporal_load(pd) : *pd;
+      }
+    }
+    double sum = 0.0, unused;
+#pragma unroll
+    for (int i = 0; i < NG; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) sum += (double)xr[i][c];
+    const float mean = (float)(all_sum2(sum, 0.0, &unused) / (double)ncols);
+    float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NG; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float d = in[i] ? xr[i][c] - mean : 0.0f;
+        xr[i][c] = d;
+        sq[c] = __builtin_fmaf(d, d, sq[c]);
+      }
+    const double var =
+        all_sum2(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3]), 0.0, &unused) / (double)ncols;
+    const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
+    float s1[2] = {0.0f, 0.0f}, s2[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NG; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float xh = xr[i][c] * rstd;
+        const float d = dr[i][c];
+        xr[i][c] = xh;
+        dg[i][c] = __builtin_fmaf(d, xh, dg[i][c]);
+        db[i][c] += d;
+        const float dyh = d * g[i][c];
+        dr[i][c] = dyh;
+        s1[c & 1] += dyh;
+        s2[c & 1] = __builtin_fmaf(dyh, xh, s2[c & 1]);
+      }
+    double t2;
+    const double t1 = all_sum2((double)s1[0] + (double)s1[1], (double)s2[0] + (double)s2[1], &t2);
+    const float m1 = (float)t1 * inv_n, m2 = (float)t2 * inv_n;
+#pragma unroll
+    for (int i = 0; i < NG; i++) {
+      if (!in[i]) continue;
+      f4 r;
+#pragma unroll
+      for (int c = 0; c < 4; c++) r[c] = rstd * ((dr[i][c] - m1) - xr[i][c] * m2);
+      f4* q = reinterpret_cast<f4*>(dx + row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4);
+      if (NT)
+        __builtin_nontemporal_store(r, q);
+      else
+        *q = r;
+    }
+  }
+  float* out = partial + (int64_t)blockIdx.x * 2 * ncols;
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    if (!in[i]) continue;
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    *reinterpret_cast<f4*>(out + c) = dg[i];
+    *reinterpret_cast<f4*>(out + ncols + c) = db[i];
+  }
+}
+
 // Column sums of the workgroups' rows in two small steps, so that the first has enough
 // workgroups to pull the few megabytes of `partial` at speed: the rows are cut into kFoldGroups
 // groups; workgroup (x, g) adds the rows of group g for 64 of the 2 ncols columns (its four
@@ -260,7 +370,9 @@ static int launch_layernorm_bwd(int nv, uint32_t blocks, const float* x, const f
     WF2_CASE(2)
     WF2_CASE(3)
     WF2_CASE(4)
+    WF2_CASE(5)
     WF2_CASE(6)
+    WF2_CASE(7)
     WF2_CASE(8)
     default: return fail(WF2HIP_EUNSUPPORTED, "LayerNorm backward: rows longer than 2048 are not built");
   }
@@ -389,9 +501,15 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
     return wf2hip_fill_f32(dbeta, (size_t)cols, 0.0f);
   }
   if (!x || !dy || !dx) return fail(WF2HIP_EINVAL, "null pointer");
-  const int nv = pick_nv(cols);
-  if (nv == 0 || nv > 8)
-    return fail(WF2HIP_EUNSUPPORTED, "LayerNorm backward: rows longer than 2048 are not built (compose it from nodes)");
+  int nv = pick_nv(cols);
+  // seven groups only where they fill the tile: rows of 1537 ... 1791 columns run at 2.1 TB/s on the
+  // guarded seven-group tile and at 3.9 TB/s on the guarded eight-group one ((32768, 1600))
+  if (nv == 7 && cols != 7 * kWave * 4) nv = 8;
+  const bool wide = nv == 0 || nv > 8;  // more than 2048 columns: a workgroup per row
+  if (wide && (cols > 8192 || cols % 4 != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(gamma)))
+    return fail(WF2HIP_EUNSUPPORTED,
+                "LayerNorm backward: rows longer than 2048 need a multiple of 4 up to 8192 columns and 16-byte aligned "
+                "tensors (compose it from nodes)");
   const int64_t total = (int64_t)rows * cols;
   if ((x < dx + total && dx < x + total) || (dgamma < dbeta + cols && dbeta < dgamma + cols))
     return fail(WF2HIP_EOVERLAP, "LayerNorm backward: dx overlaps x, or dgamma overlaps dbeta");
@@ -400,7 +518,8 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // two workgroups per compute unit, at most one wavefront per row: (65536, 1024) runs at 74 % of
   // the HBM peak (both small folds included), 66 % with one workgroup per unit, 65 - 67 % with
   // three to eight (more rows of `partial` to write and fold)
-  const int64_t blocks = std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
+  const int64_t blocks = wide ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
+                              : std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
   const size_t partial_bytes = (size_t)blocks * 2 * cols * sizeof(float);
   const size_t level2_bytes = (size_t)kFoldGroups * 2 * cols * sizeof(double);
   void* partial = nullptr;
@@ -409,7 +528,26 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
   const bool streaming = total * 12 >= ((int64_t)192 << 20);
   int rc;
-  if (vec && streaming)
+  if (wide) {
+    hipStream_t st = rt().stream;
+    const int ng = (int)ceil_div(cols, (int64_t)kBlock * 4);
+#define WF2_WIDE(NG_)                                                                                              \
+  if (streaming)                                                                                                   \
+    layernorm_bwd_wide<NG_, true><<<(uint32_t)blocks, kBlock, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols); \
+  else                                                                                                             \
+    layernorm_bwd_wide<NG_, false><<<(uint32_t)blocks, kBlock, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+    if (ng <= 3) {
+      WF2_WIDE(3)
+    } else if (ng <= 4) {
+      WF2_WIDE(4)
+    } else if (ng <= 6) {
+      WF2_WIDE(6)
+    } else {
+      WF2_WIDE(8)
+    }
+#undef WF2_WIDE
+    rc = after_launch("layernorm_bwd_wide");
+  } else if (vec && streaming)
     rc = launch_layernorm_bwd<true, true>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
   else if (vec)
     rc = launch_layernorm_bwd<true, false>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);

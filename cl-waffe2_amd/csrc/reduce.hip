@@ -1137,6 +1137,71 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_block(const float* __re
     outr[c] = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
 }
 
+// Rows of 2049 ... 8192 columns that are a multiple of 4: a workgroup per row with the row in
+// registers (thread t holds the NG 16-byte vectors (g 256 + t) 4 ...), one read and one write
+// where the three-pass form above reads the row three times ((8192, 4096): 82 us).  The
+// arithmetic of the wavefront form: the mean from binary64 sums, deviations, squares and the
+// output in binary32; the statistics meet in LDS.
+template <int NG, bool NT>
+__global__ __launch_bounds__(kBlock) void layernorm_rows_wide(const float* __restrict__ x,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta, float eps,
+                                                              float* __restrict__ out, int64_t ncols) {
+  __shared__ double red[2][kWavesPerBlock];
+  const int wave = threadIdx.x / kWave;
+  const int64_t base = (int64_t)blockIdx.x * ncols;
+  bool in[NG];
+  f4 r[NG];
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    in[i] = c < ncols;  // a vector is wholly inside or outside
+    r[i] = f4{0.f, 0.f, 0.f, 0.f};
+    if (in[i]) {
+      const f4* p = reinterpret_cast<const f4*>(x + base + c);
+      r[i] = NT ? __builtin_nontemporal_load(p) : *p;
+    }
+  }
+  double sum = 0.0;
+#pragma unroll
+  for (int i = 0; i < NG; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) sum += (double)r[i][c];
+  sum = wave_sum(sum);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[0][wave] = sum;
+  __syncthreads();
+  const float meanf = (float)(((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (double)ncols);
+  float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < NG; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const float d = in[i] ? r[i][c] - meanf : 0.0f;
+      r[i][c] = d;
+      sq[c] = __builtin_fmaf(d, d, sq[c]);
+    }
+  const double part = wave_sum(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3]));
+  if ((threadIdx.x & (kWave - 1)) == 0) red[1][wave] = part;
+  __syncthreads();
+  const double var = ((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (double)ncols;
+  const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    if (!in[i]) continue;
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    const f4 g = *reinterpret_cast<const f4*>(gamma + c);
+    const f4 b = *reinterpret_cast<const f4*>(beta + c);
+    f4 o;
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = __builtin_fmaf(r[i][k] * rstd, g[k], b[k]);
+    f4* q = reinterpret_cast<f4*>(out + base + c);
+    if (NT)
+      __builtin_nontemporal_store(o, q);
+    else
+      *q = o;
+  }
+}
+
 template <bool VEC, bool NT, bool XENT>
 static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t ldx, float* out,
                                int64_t ldo, int64_t nrows, int64_t ncols, int64_t causal_seq,
@@ -1163,7 +1228,9 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
       break;
     WF2_SOFTMAX_CASE(3)
     WF2_SOFTMAX_CASE(4)
+    WF2_SOFTMAX_CASE(5)
     WF2_SOFTMAX_CASE(6)
+    WF2_SOFTMAX_CASE(7)
     WF2_SOFTMAX_CASE(8)
     WF2_SOFTMAX_CASE(12)
     WF2_SOFTMAX_CASE(16)
@@ -1229,7 +1296,9 @@ static int launch_layernorm_wave(int nv, uint32_t blocks, const float* x, const 
       break;
     WF2_LN_CASE(3)
     WF2_LN_CASE(4)
+    WF2_LN_CASE(5)
     WF2_LN_CASE(6)
+    WF2_LN_CASE(7)
     WF2_LN_CASE(8)
     default: return fail(WF2HIP_EUNSUPPORTED, "LayerNorm rows longer than 2048 are not supported");
   }
@@ -1385,7 +1454,28 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   int nv = pick_nv(cols);
   if (nv == 0 || nv > 8) {
     if (rows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
-    layernorm_rows_block<<<(uint32_t)rows, kBlock, 0, rt().stream>>>(x, gamma, beta, eps, out, cols);
+    hipStream_t st = rt().stream;
+    if (cols <= 8192 && cols % 4 == 0 && aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta)) {
+      const bool nt = (int64_t)rows * cols * 8 >= ((int64_t)192 << 20);
+      const int ng = (int)ceil_div(cols, (int64_t)kBlock * 4);
+#define WF2_WIDE(NG_)                                                                                      \
+  if (nt)                                                                                                  \
+    layernorm_rows_wide<NG_, true><<<(uint32_t)rows, kBlock, 0, st>>>(x, gamma, beta, eps, out, cols);      \
+  else                                                                                                     \
+    layernorm_rows_wide<NG_, false><<<(uint32_t)rows, kBlock, 0, st>>>(x, gamma, beta, eps, out, cols);
+      if (ng <= 3) {
+        WF2_WIDE(3)
+      } else if (ng <= 4) {
+        WF2_WIDE(4)
+      } else if (ng <= 6) {
+        WF2_WIDE(6)
+      } else {
+        WF2_WIDE(8)
+      }
+#undef WF2_WIDE
+      return after_launch("layernorm_rows_wide");
+    }
+    layernorm_rows_block<<<(uint32_t)rows, kBlock, 0, st>>>(x, gamma, beta, eps, out, cols);
     return after_launch("layernorm_rows_block");
   }
   int64_t blocks = ceil_div(rows, kWavesPerBlock);

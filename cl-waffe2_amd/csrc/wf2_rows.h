@@ -116,11 +116,11 @@ struct RowRegs {
   }
 };
 
-// Register tiles: NV groups of 256 columns per wavefront.  Sizes 3, 6 and 12
-// make rows of 768, 1536 and 3072 columns (transformer widths) fill the tile
-// exactly, which selects the unguarded load path.
+// Register tiles: NV groups of 256 columns per wavefront.  Sizes 3, 5, 6 and 12
+// make rows of 768, 1280, 1536 and 3072 columns (transformer widths) fill the tile
+// exactly, which selects the unguarded load path; 7 holds rows of 1600.
 inline int pick_nv(int64_t ncols) {
-  static const int sizes[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  static const int sizes[] = {1, 2, 3, 4, 5, 6, 7, 8, 12, 16};
   for (int nv : sizes)
     if ((int64_t)nv * kWave * 4 >= ncols) return nv;
   return 0;

@@ -646,8 +646,9 @@ int wf2hip_softmax_cross_entropy_backward_f32(long n, const float* dy, int dy_is
  * xh = (x - mean) rstd and dyh = dy gamma,
  *   dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),
  *   dgamma[c] = sum over rows of dy xh,  dbeta[c] = sum over rows of dy.
- * Contiguous (rows, cols) operands, cols <= 2048 (longer rows return
- * WF2HIP_EUNSUPPORTED: compose them from nodes).  dx may be dy.  Allocates
+ * Contiguous (rows, cols) operands, cols <= 8192; beyond 2048 columns cols must
+ * be a multiple of 4 and the tensors 16-byte aligned (otherwise, and for longer
+ * rows, WF2HIP_EUNSUPPORTED: compose them from nodes).  dx may be dy.  Allocates
  * 8 * cols bytes per workgroup of scratch from the library's pool. */
 int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, const float* gamma,
                                   const float* dy, float eps, float* dx, float* dgamma,

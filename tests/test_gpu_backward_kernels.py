@@ -114,7 +114,9 @@ def test_causal_softmax_backward(gpu, batch, seq):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 4), (5, 60), (37, 768), (1000, 1024), (300, 2048), (4099, 768),
-                                       (257, 1001), (8192, 768)])
+                                       (257, 1001), (8192, 768),
+                                       # beyond 2048 columns: a workgroup per row, 3 ... 8 vectors per thread
+                                       (6, 2052), (700, 3072), (33, 4096), (1100, 5120), (5, 6148), (600, 8192)])
 def test_layernorm_backward(gpu, rows, cols):
     from oracle import gpt2_block_ref as ref
     W = gpu
@@ -136,12 +138,14 @@ def test_layernorm_backward(gpu, rows, cols):
         assert np.max(np.abs(cg.numpy() - gg.numpy()) / (mag_g + 1e-30)) <= 5e-6
 
 
-def test_layernorm_backward_wide_rows_take_the_composition(gpu):
+@pytest.mark.parametrize("cols", [8196, 4098])
+def test_layernorm_backward_rows_the_kernels_leave_to_the_composition(gpu, cols):
+    """More than 8192 columns, or more than 2048 that are not a multiple of 4."""
     from oracle import gpt2_block_ref as ref
     W = gpu
     F = W.functional
     rng = np.random.default_rng(5)
-    rows, cols = 6, 4096
+    rows = 6
     x = rng.standard_normal((rows, cols)).astype(f32)
     g = (1 + 0.1 * rng.standard_normal(cols)).astype(f32)
     dy = rng.standard_normal((rows, cols)).astype(f32)
