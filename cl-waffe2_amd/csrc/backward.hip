@@ -75,6 +75,44 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_block(const float* __
   for (int64_t c = threadIdx.x; c < ncols; c += kBlock) xr[c] = c < valid ? scale * (yr[c] * (dr[c] - dot)) : 0.0f;
 }
 
+// Rows of 2049 ... 32768 columns: a workgroup of 1024 threads per row with y and dy in registers
+// (thread t holds columns t, t + 1024, ...), one read of each and one write; the two-pass form
+// above reads both rows twice ((4096, 50257): 832 us).
+constexpr int kLongBlock = 1024;
+
+template <int E>
+__global__ __launch_bounds__(kLongBlock) void softmax_bwd_rows_long(const float* __restrict__ y, int64_t ldy,
+                                                                    const float* dy, int64_t lddy,  // dx may be dy
+                                                                    float* dx, int64_t lddx, int64_t ncols,
+                                                                    float scale) {
+  __shared__ double lds[kLongBlock / kWave];
+  const float* yr = y + (int64_t)blockIdx.x * ldy;
+  const float* dr = dy + (int64_t)blockIdx.x * lddy;
+  float a[E], b[E];
+  float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < E; k++) {
+    const int64_t c = (int64_t)k * kLongBlock + threadIdx.x;
+    a[k] = c < ncols ? yr[c] : 0.0f;
+    b[k] = c < ncols ? dr[c] : 0.0f;
+  }
+#pragma unroll
+  for (int k = 0; k < E; k++) part[k & 3] = __builtin_fmaf(b[k], a[k], part[k & 3]);
+  const double w = wave_sum(((double)part[0] + (double)part[1]) + ((double)part[2] + (double)part[3]));
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = w;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int i = 0; i < kLongBlock / kWave; i++) total += lds[i];
+  const float dot = (float)total;
+  float* xr = dx + (int64_t)blockIdx.x * lddx;
+#pragma unroll
+  for (int k = 0; k < E; k++) {
+    const int64_t c = (int64_t)k * kLongBlock + threadIdx.x;
+    if (c < ncols) xr[c] = scale * (a[k] * (b[k] - dot));
+  }
+}
+
 template <bool VEC, bool NT>
 static int launch_softmax_bwd(int nv, const float* y, int64_t ldy, const float* dy, int64_t lddy, float* dx,
                               int64_t lddx, int64_t nrows, int64_t ncols, int64_t causal_seq, float scale) {
@@ -479,8 +517,19 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
     return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps dy without being dy");
   int nv = pick_nv(cols);
   if (nv == 0 || nv > 8) {
-    softmax_bwd_rows_block<<<(uint32_t)rows, kBlock, 0, rt().stream>>>(y, ldy, dy, lddy, dx, lddx, cols, causal_seq,
-                                                                     scale);
+    hipStream_t st = rt().stream;
+    if (causal_seq == 0 && cols <= 32 * kLongBlock) {  // beyond: y and dy of a row exceed the registers of 1024 threads
+      if (cols <= 4 * kLongBlock)
+        softmax_bwd_rows_long<4><<<(uint32_t)rows, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, scale);
+      else if (cols <= 8 * kLongBlock)
+        softmax_bwd_rows_long<8><<<(uint32_t)rows, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, scale);
+      else if (cols <= 16 * kLongBlock)
+        softmax_bwd_rows_long<16><<<(uint32_t)rows, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, scale);
+      else
+        softmax_bwd_rows_long<32><<<(uint32_t)rows, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, scale);
+      return after_launch("softmax_bwd_rows_long");
+    }
+    softmax_bwd_rows_block<<<(uint32_t)rows, kBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, causal_seq, scale);
     return after_launch("softmax_bwd_rows_block");
   }
   const bool vec = aligned16(y) && aligned16(dy) && aligned16(dx) && ldy % 4 == 0 && lddy % 4 == 0 && lddx % 4 == 0;

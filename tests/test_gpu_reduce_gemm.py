@@ -267,13 +267,16 @@ def test_config4_softmax(gpu):
     np.testing.assert_allclose(shifted, _softmax64(X[:256] + np.float32(8.0)), rtol=1e-5, atol=1e-12)
 
 
-@pytest.mark.parametrize("cols", [1, 3, 64, 100, 255, 256, 1000, 1024, 2050, 4096, 5000, 20000])
+@pytest.mark.parametrize("cols", [1, 3, 64, 100, 255, 256, 1000, 1024, 2050, 4096, 4097, 5000, 8192, 8193, 20000,
+                                  32768, 40000, 50257, 53249, 65536, 70000])
 def test_softmax_widths(gpu, cols):
+    """Every row form: 1 ... 4096 columns in a wavefront's registers, 4097 ... 65536 in those of a workgroup of
+    1024 threads (8, 16, 32, 52 or 64 elements per thread), longer rows in three passes."""
     F = gpu.functional
     rng = np.random.default_rng(cols)
-    X = (rng.standard_normal((37, cols)) * 4).astype(np.float32)
+    X = (rng.standard_normal((37 if cols < 30000 else 5, cols)) * 4).astype(np.float32)
     got = F.softmax_fused(F.from_numpy(X)).numpy()
-    if cols <= 4096:
+    if cols <= 65536:
         _assert_softmax(got, _softmax64(X), f"{cols} columns")
     else:  # rows too long for registers: the three-pass binary64 kernel
         assert ulp_distance(got, _softmax64(X).astype(np.float32)).max() <= 2
