@@ -9,6 +9,8 @@
 // per wavefront, K in steps of 16 with the next step prefetched into registers): the :double path is there so that
 // models keep running on the device, the tuned kernels are the :float ones in
 // gemm.hip.
+#include <algorithm>
+
 #include "wf2_common.h"
 
 namespace wf2 {
@@ -21,6 +23,7 @@ struct DgemmParams {
   int64_t sA, sB, sC, sA2, sB2, sC2;  // batch strides: inner / outer level
   uint32_t batch_inner;
   double alpha, beta;
+  int64_t kslice;  // > 0: blockIdx.z names a slice of K of this length (a single product split over K)
 };
 
 typedef double d4 __attribute__((ext_vector_type(4)));
@@ -40,6 +43,11 @@ __global__ __launch_bounds__(kBlock) void dgemm_kernel(DgemmParams p) {
   const double* A = p.A + (int64_t)bi * p.sA + (int64_t)bo * p.sA2;
   const double* B = p.B + (int64_t)bi * p.sB + (int64_t)bo * p.sB2;
   double* C = p.C + (int64_t)bi * p.sC + (int64_t)bo * p.sC2;
+  int64_t kbeg = 0, kend = p.k;
+  if (p.kslice > 0) {  // batch_inner is the slice count and only sC is set: slice z writes its own m x n plane
+    kbeg = (int64_t)blockIdx.z * p.kslice;
+    kend = kbeg + p.kslice < p.k ? kbeg + p.kslice : p.k;
+  }
   const int64_t i0 = (int64_t)blockIdx.x * TILE, j0 = (int64_t)blockIdx.y * TILE;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wr = (wave & 1) * (TILE / 2), wc = (wave >> 1) * (TILE / 2);
@@ -60,16 +68,16 @@ __global__ __launch_bounds__(kBlock) void dgemm_kernel(DgemmParams p) {
       int i, kk;
       a_pos(r, i, kk);
       const int64_t gi = i0 + i, gk = k0 + kk;
-      ra[r] = (gi < p.m && gk < p.k) ? (TA ? A[gk + gi * p.lda] : A[gi + gk * p.lda]) : 0.0;
+      ra[r] = (gi < p.m && gk < kend) ? (TA ? A[gk + gi * p.lda] : A[gi + gk * p.lda]) : 0.0;
       int j, kb;
       b_pos(r, j, kb);
       const int64_t gj = j0 + j, gkb = k0 + kb;
-      rb[r] = (gj < p.n && gkb < p.k) ? (TB ? B[gj + gkb * p.ldb] : B[gkb + gj * p.ldb]) : 0.0;
+      rb[r] = (gj < p.n && gkb < kend) ? (TB ? B[gj + gkb * p.ldb] : B[gkb + gj * p.ldb]) : 0.0;
     }
   };
   d4 acc[NT][NT] = {};
-  if (p.k > 0) fetch(0);
-  for (int64_t k0 = 0; k0 < p.k; k0 += kDK) {
+  if (kend > kbeg) fetch(kbeg);
+  for (int64_t k0 = kbeg; k0 < kend; k0 += kDK) {
 #pragma unroll
     for (int r = 0; r < PER; r++) {
       int i, kk, j, kb;
@@ -79,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void dgemm_kernel(DgemmParams p) {
       Bs[kb][j] = rb[r];
     }
     __syncthreads();
-    if (k0 + kDK < p.k) fetch(k0 + kDK);
+    if (k0 + kDK < kend) fetch(k0 + kDK);
 #pragma unroll
     for (int kk = 0; kk < kDK; kk += 4) {
       // v_mfma_f64_16x16x4: D(16 x 16) += L(16 x 4) R(4 x 16); lane l supplies L[l%16][l/16] and
@@ -123,6 +131,26 @@ static void launch_dgemm(const DgemmParams& p, bool ta, bool tb, dim3 grid, hipS
   else dgemm_kernel<false, false, TILE><<<grid, kBlock, 0, st>>>(p);
 }
 
+// C <- beta C + the sum of the `splits` planes of a product split over K (planes packed m x n, already
+// scaled by alpha): a wavefront per output element, lane l adds planes l, l + 64, ... and the lanes meet by
+// shuffles -- a fixed order.
+__global__ __launch_bounds__(kBlock) void dgemm_fold(const double* __restrict__ partials, int splits, int64_t m,
+                                                     int64_t n, double beta, double* __restrict__ C, int64_t ldc) {
+  const int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (e >= m * n) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t plane = m * n;
+  double acc = 0.0;
+  for (int s = lane; s < splits; s += kWave) acc += partials[(int64_t)s * plane + e];
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) {
+    const int64_t j = e / m, i = e - j * m;
+    double* c = C + i + j * ldc;
+    *c = beta == 0.0 ? acc : beta * *c + acc;
+  }
+}
+
 static bool dn(char c) { return c == 'N' || c == 'n'; }
 static bool dt(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
@@ -146,14 +174,46 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
   p.sA2 = strideA2; p.sB2 = strideB2; p.sC2 = strideC2;
   p.batch_inner = (uint32_t)batch;
   p.alpha = alpha; p.beta = beta;
+  p.kslice = 0;
+  hipStream_t st = rt().stream;
+  const bool ta = !dn(transa), tb = !dn(transb);
+  // A single product with few output tiles over a long K ((10 x 1048576) . (1048576 x 10) ran 66 ms on one
+  // workgroup): slices of K of at least 512, as many as keep four workgroups per compute unit, each into a
+  // plane of its own, folded in a fixed order afterwards.
+  const int64_t small_tiles = ceil_div(m, 64) * ceil_div(n, 64);
+  if (batch == 1 && batch2 == 1 && k >= 2048 && small_tiles < (int64_t)rt().num_cus) {
+    int64_t splits = std::min<int64_t>(k / 512, 4 * (int64_t)rt().num_cus / small_tiles);
+    splits = std::min<int64_t>(splits, 4096);
+    const int64_t kslice = ceil_div(ceil_div(k, splits), (int64_t)kDK) * kDK;
+    splits = ceil_div(k, kslice);
+    void* scratch = nullptr;
+    if (splits >= 2 && wf2hip_malloc_uninitialized(&scratch, (size_t)splits * m * n * sizeof(double)) == 0) {
+      DgemmParams q = p;
+      q.C = static_cast<double*>(scratch);
+      q.ldc = m;
+      q.sA = q.sB = q.sA2 = q.sB2 = q.sC2 = 0;
+      q.sC = (int64_t)m * n;
+      q.batch_inner = (uint32_t)splits;
+      q.beta = 0.0;
+      q.kslice = kslice;
+      dim3 grid((uint32_t)ceil_div(m, 64), (uint32_t)ceil_div(n, 64), (uint32_t)splits);
+      launch_dgemm<64>(q, ta, tb, grid, st);
+      int rc = after_launch("dgemm_kernel");
+      if (rc == 0) {
+        dgemm_fold<<<(uint32_t)ceil_div((int64_t)m * n, kBlock / kWave), kBlock, 0, st>>>(
+            static_cast<const double*>(scratch), (int)splits, m, n, beta, C, ldc);
+        rc = after_launch("dgemm_fold");
+      }
+      (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
+      return rc;
+    }
+  }
   // 128 x 128 tiles once they fill the chip twice over, 64 x 64 below that
   const int64_t big = ceil_div(m, 128) * ceil_div(n, 128) * batch * batch2;
   const int tile = big >= 2 * (int64_t)rt().num_cus ? 128 : 64;
   const int64_t gx = ceil_div(m, tile), gy = ceil_div(n, tile);
   if (gx >= ((int64_t)1 << 31) || gy > 65535) return fail(WF2HIP_EUNSUPPORTED, "matrix too large for one launch");
   dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)(batch * batch2));
-  hipStream_t st = rt().stream;
-  const bool ta = !dn(transa), tb = !dn(transb);
   if (tile == 128) launch_dgemm<128>(p, ta, tb, grid, st);
   else launch_dgemm<64>(p, ta, tb, grid, st);
   return after_launch("dgemm_kernel");

@@ -152,3 +152,39 @@ def test_double_matmul_large_tiles(gpu, ta, tb):
     assert np.max(np.abs(got - want) / scale) <= 8 * k * EPS
     _check(got[0], opA[0], opB[0], what="first matrix, extended precision")
     _check(got[-1], opA[-1], opB[-1], what="last matrix, extended precision")
+
+
+@pytest.mark.parametrize("m,n,k", [(10, 10, 1 << 17), (64, 64, 40000), (3, 200, 2048), (130, 70, 5003)])
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_double_matmul_few_outputs_long_k(gpu, m, n, k, ta, tb):
+    """Few output tiles over a long K run as slices of K folded afterwards: K on and off the slice length,
+    every transpose form, and alpha, beta and a padded ldc through the C-ABI."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(m + n + k)
+    A = rng.standard_normal((k, m) if ta else (m, k))
+    B = rng.standard_normal((n, k) if tb else (k, n))
+    a, b = D(A), D(B)
+    out = F.matmul(F.t(a) if ta else a, F.t(b) if tb else b)
+    opA, opB = (A.T if ta else A), (B.T if tb else B)
+    _check(out.numpy(), opA, opB, what=f"{m}x{n}x{k} {ta} {tb}")
+    # column-major call: C (m x n, ldc = m + 3) <- 0.5 op(A) op(B) - 2 C; the row-major arrays above are the
+    # column-major transposes, so op(A) here is opB^T ... use the Fortran reading directly instead
+    lib = W.lib.get()
+    dp = lambda t: C.c_void_p(t.ptr)
+    ldc = m + 3
+    Cm = rng.standard_normal(ldc * n)
+    dC = D(Cm)
+    # A as stored is (k, m) row-major when ta, i.e. column-major m x k with lda = m: op = 'N'
+    Acm = np.ascontiguousarray(opA.T) if not ta else np.ascontiguousarray(opA)   # column-major m x k / k x m
+    Bcm = np.ascontiguousarray(opB.T) if not tb else np.ascontiguousarray(opB)
+    dA, dB = D(Acm.ravel()), D(Bcm.ravel())
+    # Acm (not ta): array (k, m) row-major = column-major m x k, lda = m, 'N'.  (ta): array (m, k) = column-major
+    # k x m, lda = k, 'T'.
+    W.lib.check(lib.wf2hip_dgemm(b"T" if ta else b"N", b"T" if tb else b"N", m, n, k, 0.5, dp(dA), k if ta else m,
+                                 dp(dB), n if tb else k, -2.0, dp(dC), ldc))
+    got = dC.numpy().reshape(n, ldc).T
+    C2 = Cm.reshape(n, ldc).T
+    _check(got[:m, :], 0.5 * opA, opB, extra=-2.0 * C2[:m, :], what="column-major call")
+    np.testing.assert_array_equal(got[m:, :], C2[m:, :])
