@@ -19,6 +19,7 @@
 // Arithmetic is IEEE binary32 with contraction disabled at build time
 // (-ffp-contract=off) so a+b, a*b ... are bit-identical to _mm256_*_ps.
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_math.h"
 #include "wf2_view.h"
 
@@ -838,6 +839,77 @@ static int launch_tile128(const TileParams& p, uint32_t blocks, F f) {
   return 0;
 }
 
+// ---- narrow tile kernel: the source's contiguous axis is short ---------------------------------------
+// (N, 12) -> (12, N), NHWC -> NCHW of images: the axis J along which src is contiguous has fewer than 32
+// elements.  A 64 x 64 tile would leave most of its lanes idle, and an element per lane reads every line of
+// src once per element of J ((1398101, 12) transposed: 126 us).  Here a workgroup takes `tl` positions of
+// dst's contiguous axis I with the whole of J: src is walked in storage order (whole lines when its rows are
+// adjacent), dst is written in 16-byte vectors, and LDS (element (j, i) at j * (tl + 4) + i) sits between
+// them.  tl is 512 for up to 15 elements of J and 256 for up to 31: at most 32 KB of LDS.  (The mirrored
+// case -- dst contiguous along the short axis -- is served well by an element per lane: dst is then written
+// in storage order and neighbouring wavefronts use up the lines of src.)
+constexpr int kNarrowMax = 31;
+constexpr int kNarrowFloats = 8064;  // >= 15 * 516 and 31 * 260
+
+template <class F, bool ReadDst, bool VEC>
+__global__ __launch_bounds__(kBlock) void ew_tile_narrow(TileParams p, F f, FastDiv by_nj, int tl) {
+  __shared__ __attribute__((aligned(16))) float tile[kNarrowFloats];
+  const int pitch = tl + 4;
+  uint32_t rem = blockIdx.x / p.tiles_i;
+  const int64_t i0 = (int64_t)(blockIdx.x - rem * p.tiles_i) * tl;
+  int64_t doff = 0, soff = 0;
+  for (int i = 0; i < p.nouter; i++) {
+    uint32_t q = rem / p.oshape[i];
+    uint32_t idx = rem - q * p.oshape[i];
+    rem = q;
+    doff += (int64_t)idx * p.odst[i];
+    soff += (int64_t)idx * p.osrc[i];
+  }
+  const int nj = (int)p.nj;
+  const int live = (int)(p.ni - i0 < tl ? p.ni - i0 : tl);  // positions of I in this tile
+  const uint32_t cells = (uint32_t)live * (uint32_t)nj;
+  float* dst = p.dst + doff;
+  const float* src = p.src + soff;
+  constexpr int U = 4;
+  // src (i, j) at i * s_i + j  ->  LDS
+  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+    float v[U];
+    uint32_t i[U], j[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const uint32_t e = e0 + u * kBlock;
+      i[u] = fd_divmod(e < cells ? e : 0u, by_nj, &j[u]);
+      v[u] = e < cells ? src[(i0 + i[u]) * p.s_i + j[u]] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (e0 + u * kBlock < cells) tile[j[u] * pitch + i[u]] = v[u];
+  }
+  __syncthreads();
+  // LDS -> dst (j, i) at j * d_j + i
+  const uint32_t per_row = (uint32_t)tl / 4;
+  const uint32_t vecs = (uint32_t)nj * per_row;
+  for (uint32_t q = threadIdx.x; q < vecs; q += kBlock) {
+    const uint32_t j = q / per_row;  // tl / 4 is a power of two
+    const int i4 = (int)(q - j * per_row) * 4;
+    if (i4 >= live) continue;
+    float* dp = dst + (int64_t)j * p.d_j + i0 + i4;
+    const float* t = tile + j * pitch + i4;
+    if (VEC && i4 + 4 <= live) {
+      const f4 a = ReadDst ? *reinterpret_cast<const f4*>(dp) : f4{0.f, 0.f, 0.f, 0.f};
+      const f4 b = *reinterpret_cast<const f4*>(t);
+      f4 o;
+      o.x = f(a.x, b.x);
+      o.y = f(a.y, b.y);
+      o.z = f(a.z, b.z);
+      o.w = f(a.w, b.w);
+      *reinterpret_cast<f4*>(dp) = o;
+    } else {
+      for (int u = 0; u < 4 && i4 + u < live; u++) dp[u] = f(ReadDst ? dp[u] : 0.0f, t[u]);
+    }
+  }
+}
+
 // ---- dispatch -------------------------------------------------------------------
 static inline int ilog2_ceil(int64_t v) {
   int l = 0;
@@ -990,7 +1062,9 @@ static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, i
   int J = -1;
   for (int r = 0; r < last; r++)
     if (s.sb[r] == 1 && s.sa[r] > 0) J = r;
-  if (J < 0 || s.shape[last] < 16 || s.shape[J] < 16) return false;
+  if (J < 0) return false;
+  const bool narrow = s.shape[J] <= kNarrowMax && s.shape[last] >= 256;
+  if (!narrow && (s.shape[last] < 32 || s.shape[J] < 16)) return false;  // an element per lane serves a short dst axis
   TileParams p;
   p.dst = dst + s.off_a;
   p.src = src + s.off_b;
@@ -1010,6 +1084,24 @@ static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, i
     p.osrc[p.nouter] = s.sb[r];
     p.nouter++;
     blocks *= s.shape[r];
+  }
+  if (narrow) {
+    const int tl = p.nj <= 15 ? 512 : 256;
+    const int64_t tiles = ceil_div(p.ni, tl);
+    int64_t nblocks = tiles;
+    for (int i = 0; i < p.nouter; i++) nblocks *= p.oshape[i];
+    if (nblocks >= ((int64_t)1 << 31)) return false;
+    p.tiles_i = (uint32_t)tiles;
+    bool v16 = aligned16(p.dst) && p.d_j % 4 == 0;  // 16-byte accesses on dst
+    for (int i = 0; i < p.nouter; i++)
+      if (p.odst[i] % 4 != 0) v16 = false;
+    const FastDiv by_nj = make_fastdiv((uint32_t)p.nj);
+    if (v16)
+      ew_tile_narrow<F, ReadDst, true><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+    else
+      ew_tile_narrow<F, ReadDst, false><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+    *rc = after_launch("ew_tile_narrow");
+    return true;
   }
   if (blocks >= ((int64_t)1 << 31)) return false;
   bool vec = aligned16(p.dst) && aligned16(p.src) && p.ni % 4 == 0 && p.nj % 4 == 0 &&
@@ -1144,8 +1236,53 @@ static bool try_launch_gather2(const Space& s, float* dst, const float* src, F f
 
 // `s` describes dst through (sa, off_a) and src through (sb, off_b); dst has
 // no broadcast axis.
+// The destination's unit-stride axis moved to the end (x^T += y): an elementwise pass may visit its index
+// space in any order as long as no destination element is visited twice, which holds when the axes sorted by
+// stride each step over everything the smaller ones cover.  False when there is nothing to move.
+static bool dst_unit_axis_last(const Space& s, Space* out) {
+  const int last = s.rank - 1;
+  if (s.rank < 2 || s.sa[last] == 1) return false;
+  int unit = -1;
+  for (int r = 0; r < last; r++)
+    if (s.sa[r] == 1 && s.shape[r] >= 16) unit = r;
+  if (unit < 0) return false;
+  int order[WF2HIP_MAX_RANK];
+  for (int r = 0; r < s.rank; r++) {
+    if (s.sa[r] <= 0) return false;
+    order[r] = r;
+  }
+  for (int i = 1; i < s.rank; i++)
+    for (int j = i; j > 0 && s.sa[order[j]] < s.sa[order[j - 1]]; j--) {
+      const int t = order[j];
+      order[j] = order[j - 1];
+      order[j - 1] = t;
+    }
+  int64_t covered = 1;  // elements spanned by the axes so far
+  for (int i = 0; i < s.rank; i++) {
+    const int r = order[i];
+    if (s.sa[r] < covered) return false;
+    covered = s.sa[r] * (s.shape[r] - 1) + covered;
+  }
+  *out = s;
+  int w = 0;
+  for (int r = 0; r < s.rank; r++) {
+    if (r == unit) continue;
+    out->shape[w] = s.shape[r];
+    out->sa[w] = s.sa[r];
+    out->sb[w] = s.sb[r];
+    w++;
+  }
+  out->shape[w] = s.shape[unit];
+  out->sa[w] = s.sa[unit];
+  out->sb[w] = s.sb[unit];
+  normalise(out);
+  return true;
+}
+
 template <class F, bool ReadDst>
-static int launch_elementwise(const Space& s, float* dst, const float* src, F f) {
+static int launch_elementwise(const Space& s_in, float* dst, const float* src, F f) {
+  Space turned;
+  const Space& s = dst_unit_axis_last(s_in, &turned) ? turned : s_in;
   const int last = s.rank - 1;
   int64_t nrows = s.total / (s.shape[last] ? s.shape[last] : 1);
   bool rows_ok = s.sa[last] == 1 && (s.sb[last] == 1 || s.sb[last] == 0) &&

@@ -204,3 +204,57 @@ def test_pooling_layers_at_size(gpu):
     assert_bit_equal(nn.max_pool2d_backward(dx, F.from_numpy(dy), 2).numpy(), want, "max pool backward")
     want_avg = np.broadcast_to((dy / f32(4))[:, :, :, None, :, None], win.shape).reshape(x.shape)
     assert_bit_equal(nn.avg_pool2d_backward(dx, F.from_numpy(dy), 2).numpy(), want_avg, "avg pool backward")
+
+
+@pytest.mark.parametrize("narrow", [2, 3, 5, 8, 12, 15, 16, 24, 31])
+@pytest.mark.parametrize("long", [256, 511, 1000, 4099])
+def test_transposing_passes_with_one_short_axis(gpu, narrow, long):
+    """(long, narrow) <-> (narrow, long): the exchange whose short axis has fewer than 16 elements takes long
+    tiles with the whole short axis.  Copies in both directions, an accumulating pass, batches in front,
+    a sliced (unaligned, padded) operand; data movement and one rounding each: bit-exact."""
+    F = gpu.functional
+    rng = np.random.default_rng(narrow * 10000 + long)
+    a = rng.standard_normal((3, long, narrow)).astype(np.float32)
+    da = F.from_numpy(a)
+    # src contiguous along the short axis
+    np.testing.assert_array_equal(F.copy(da.permute(0, 2, 1)).numpy(), a.transpose(0, 2, 1))
+    # dst contiguous along the short axis
+    b = rng.standard_normal((3, narrow, long)).astype(np.float32)
+    db = F.from_numpy(b)
+    np.testing.assert_array_equal(F.copy(db.permute(0, 2, 1)).numpy(), b.transpose(0, 2, 1))
+    # accumulate: b += a^T and a += b^T
+    got = F.add_(F.copy(db), da.permute(0, 2, 1)).numpy()
+    np.testing.assert_array_equal(got, b + a.transpose(0, 2, 1))
+    got = F.add_(F.copy(da), db.permute(0, 2, 1)).numpy()
+    np.testing.assert_array_equal(got, a + b.transpose(0, 2, 1))
+    # a window of a wider tensor (rows not adjacent, base off 16 bytes)
+    wide = rng.standard_normal((long + 2, narrow + 3)).astype(np.float32)
+    dw = F.from_numpy(wide)
+    win = dw.view((1, long + 1), (1, narrow + 1))
+    np.testing.assert_array_equal(F.copy(win.permute(1, 0)).numpy(), wide[1:long + 1, 1:narrow + 1].T)
+
+
+def test_image_layout_exchange(gpu):
+    """NCHW <-> NHWC with three channels, both directions."""
+    F = gpu.functional
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((5, 3, 37, 53)).astype(np.float32)
+    dx = F.from_numpy(x)
+    nhwc = F.copy(dx.permute(0, 2, 3, 1))
+    np.testing.assert_array_equal(nhwc.numpy(), x.transpose(0, 2, 3, 1))
+    np.testing.assert_array_equal(F.copy(nhwc.permute(0, 3, 1, 2)).numpy(), x)
+
+
+@pytest.mark.parametrize("shape", [(300, 500), (64, 64), (7, 129, 65), (1000, 17)])
+def test_passes_into_a_transposed_destination(gpu, shape):
+    """x^T += y and a copy into x^T: the destination's unit-stride axis is not the last one."""
+    F = gpu.functional
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    perm = tuple(range(len(shape) - 2)) + (len(shape) - 1, len(shape) - 2)
+    y = rng.standard_normal(tuple(shape[p] for p in perm)).astype(np.float32)
+    dx, dy = F.from_numpy(x), F.from_numpy(y)
+    F.add_(dx.permute(*perm), dy)
+    np.testing.assert_array_equal(dx.numpy(), x + y.transpose(perm))
+    F.move_(dx.permute(*perm), dy)
+    np.testing.assert_array_equal(dx.numpy(), y.transpose(perm))
