@@ -14,6 +14,7 @@
 #include <algorithm>
 
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_rows.h"
 
 namespace wf2 {
@@ -52,6 +53,60 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_wave(const float* __r
       a.v[g][c] = in ? t : 0.0f;
     }
   a.store(dx + row * lddx, ncols, lane);
+}
+
+// Many rows of at most 64 columns (class scores): a wavefront per row leaves most lanes idle ((1677721, 10):
+// 292 us).  A workgroup takes 128 adjacent rows (64 beyond 32 columns): y and dy, one contiguous run each, are staged into LDS in
+// storage order (row r at r * (ncols | 1), the odd pitch keeps a wavefront's rows on different banks), thread
+// r works through row r, and dx is written in storage order.  Rows must be adjacent (pitch == ncols) in all
+// three.
+constexpr int kTinyCols = 64;
+constexpr int kTinyFloats = 128 * 33;  // >= 64 * 65
+__host__ __device__ inline int tiny_rows_per_group(int ncols) { return ncols <= 32 ? 128 : 64; }
+
+__global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __restrict__ y, const float* dy,  // dx may be dy
+                                                                float* dx, int64_t nrows, int ncols, float scale,
+                                                                FastDiv by_c) {
+  __shared__ float ty[kTinyFloats];
+  __shared__ float td[kTinyFloats];
+  const int pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  const int64_t row0 = (int64_t)blockIdx.x * group;
+  const int rows_here = (int)(nrows - row0 < group ? nrows - row0 : group);
+  const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
+  const int64_t base = row0 * ncols;
+  constexpr int U = 4;
+  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+    float a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const bool live = e0 + u * kBlock < cells;
+      a[u] = live ? y[base + e0 + u * kBlock] : 0.0f;
+      b[u] = live ? dy[base + e0 + u * kBlock] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (e0 + u * kBlock < cells) {
+        uint32_t col;
+        const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+        ty[row * pitch + col] = a[u];
+        td[row * pitch + col] = b[u];
+      }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < rows_here) {
+    float* a = ty + threadIdx.x * pitch;
+    const float* b = td + threadIdx.x * pitch;
+    double acc = 0.0;
+    for (int j = 0; j < ncols; j++) acc += (double)(b[j] * a[j]);
+    const float dot = (float)acc;
+    for (int j = 0; j < ncols; j++) a[j] = scale * (a[j] * (b[j] - dot));
+  }
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < cells; e += kBlock) {
+    uint32_t col;
+    const uint32_t row = fd_divmod(e, by_c, &col);
+    dx[base + e] = ty[row * pitch + col];
+  }
 }
 
 // Rows beyond the register tile: a workgroup per row, two passes (the second one from the L2).
@@ -515,6 +570,11 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
   if (xlo < yhi && ylo < xhi) return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps y");
   if (xlo < dhi && dlo < xhi && !(dx == dy && lddx == lddy))
     return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps dy without being dy");
+  if (cols <= kTinyCols && causal_seq == 0 && rows >= 16384 && ldy == cols && lddy == cols && lddx == cols) {
+    softmax_bwd_rows_tiny<<<(uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols)), kBlock, 0, rt().stream>>>(
+        y, dy, dx, rows, (int)cols, scale, make_fastdiv((uint32_t)cols));
+    return after_launch("softmax_bwd_rows_tiny");
+  }
   int nv = pick_nv(cols);
   if (nv == 0 || nv > 8) {
     hipStream_t st = rt().stream;

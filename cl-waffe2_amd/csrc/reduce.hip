@@ -1321,9 +1321,115 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
 
 // xe == nullptr: the plain softmax.  Otherwise the cross-entropy epilogue as well
 // (no causal form; labels and loss are contiguous rows of ncols).
+// ---- rows of at most 64 columns (class scores: softmax over 10 classes) -----------------------------
+// A wavefront per row -- or per four rows -- leaves most lanes idle on such rows ((1677721, 10): softmax 361
+// us, 11 % of what its bytes take).  Here a workgroup takes 256 adjacent rows (128 beyond 32 columns): their storage, one contiguous
+// run, is staged into LDS in storage order (row r at r * (ncols | 1): the odd pitch keeps the 64 rows of a
+// wavefront on different banks), thread r works through row r there, and the run is written back in storage
+// order.  Rows must be adjacent in x and in every output (pitch == ncols).
+constexpr int kTinyCols = 64;
+constexpr int kTinyFloats = 256 * 33;  // >= 128 * 65
+__host__ __device__ inline int tiny_rows_per_group(int ncols) { return ncols <= 32 ? 256 : 128; }
+enum { kTinySoftmax = 0, kTinyXent = 1, kTinyLayerNorm = 2 };
+
+struct TinyRows {
+  const float* x;
+  float* out;
+  const float* aux0;  // Xent: labels; LayerNorm: gamma
+  const float* aux1;  // LayerNorm: beta
+  float* loss;        // Xent
+  float param;        // Xent: delta; LayerNorm: eps
+  int64_t nrows;
+  int ncols;
+};
+
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
+  __shared__ float tile[kTinyFloats];
+  const int ncols = a.ncols, pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  const int64_t row0 = (int64_t)blockIdx.x * group;
+  const int rows_here = (int)(a.nrows - row0 < group ? a.nrows - row0 : group);
+  const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
+  const int64_t base = row0 * ncols;
+  constexpr int U = 4;
+  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = e0 + u * kBlock < cells ? a.x[base + e0 + u * kBlock] : 0.0f;
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (e0 + u * kBlock < cells) {
+        uint32_t col;
+        const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+        tile[row * pitch + col] = v[u];
+      }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < rows_here) {
+    float* r = tile + threadIdx.x * pitch;
+    if constexpr (MODE == kTinyLayerNorm) {
+      // binary32 statistics, as the several-rows-per-wavefront form of layernorm_rows_wave
+      float sum = 0.0f;
+      for (int j = 0; j < ncols; j++) sum += r[j];
+      const float mean = sum / (float)ncols;
+      float sq = 0.0f;
+      for (int j = 0; j < ncols; j++) {
+        const float d = r[j] - mean;
+        sq = __builtin_fmaf(d, d, sq);
+      }
+      const float var = sq / (float)ncols;
+      const float rstd = (float)(1.0 / __builtin_sqrt((double)var + (double)a.param));
+      for (int j = 0; j < ncols; j++) r[j] = __builtin_fmaf((r[j] - mean) * rstd, a.aux0[j], a.aux1[j]);
+    } else {
+      float m = -__builtin_inff();
+      for (int j = 0; j < ncols; j++) m = fmaxf(m, r[j]);
+      double total = 0.0;
+      for (int j = 0; j < ncols; j++) {  // the exponential of softmax_rows_wave
+        const float d = fmaxf(r[j] - m, -160.0f);
+        const float t = d * 1.44269502f;
+        float tl = __builtin_fmaf(d, 1.44269502f, -t);
+        tl = __builtin_fmaf(d, 1.92596299e-8f, tl);
+        const float e = __builtin_amdgcn_exp2f(t);
+        const float ed = __builtin_fmaf(e, tl * 0.693147182f, e);
+        r[j] = ed;
+        total += (double)ed;
+      }
+      const float inv = (float)(1.0 / total);
+      for (int j = 0; j < ncols; j++) r[j] *= inv;
+    }
+  }
+  __syncthreads();
+  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+    float lab[U];
+    if constexpr (MODE == kTinyXent) {
+#pragma unroll
+      for (int u = 0; u < U; u++) lab[u] = e0 + u * kBlock < cells ? a.aux0[base + e0 + u * kBlock] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (e0 + u * kBlock < cells) {
+        uint32_t col;
+        const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+        const float z = tile[row * pitch + col];
+        a.out[base + e0 + u * kBlock] = z;
+        if constexpr (MODE == kTinyXent) a.loss[base + e0 + u * kBlock] = xent_term(lab[u], z, a.param);
+      }
+  }
+}
+
+// at least this many rows: below it the wavefront forms already finish within a launch's floor
+constexpr int64_t kTinyMinRows = 16384;
+
 template <bool XENT>
 static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
                                int64_t ldo, int64_t causal_seq, float scale, Xent xe) {
+  if (ncols <= kTinyCols && ldx == ncols && ldo == ncols && causal_seq == 0 && nrows >= kTinyMinRows &&
+      ceil_div(nrows, 128) < ((int64_t)1 << 31)) {
+    TinyRows a{x, out, xe.labels, nullptr, xe.loss, xe.delta, nrows, (int)ncols};
+    rows_tiny<XENT ? kTinyXent : kTinySoftmax><<<(uint32_t)ceil_div(nrows, tiny_rows_per_group((int)ncols)), kBlock, 0, rt().stream>>>(
+        a, make_fastdiv((uint32_t)ncols));
+    return after_launch("rows_tiny");
+  }
   const int nv = pick_nv(ncols);
   if (nv == 0) {
     if (causal_seq > 0) return fail(WF2HIP_EUNSUPPORTED, "causal softmax rows longer than 4096");
@@ -1542,6 +1648,12 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   if (rows < 0 || cols < 0) return fail(WF2HIP_EINVAL, "negative extent");
   if (rows == 0 || cols == 0) return 0;
   if (!x || !gamma || !beta || !out) return fail(WF2HIP_EINVAL, "null pointer");
+  if (cols <= kTinyCols && rows >= kTinyMinRows) {
+    TinyRows a{x, out, gamma, beta, nullptr, eps, rows, (int)cols};
+    rows_tiny<kTinyLayerNorm><<<(uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols)), kBlock, 0, rt().stream>>>(
+        a, make_fastdiv((uint32_t)cols));
+    return after_launch("rows_tiny");
+  }
   int nv = pick_nv(cols);
   if (nv == 0 || nv > 8) {
     if (rows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");

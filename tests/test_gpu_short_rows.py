@@ -258,3 +258,40 @@ def test_passes_into_a_transposed_destination(gpu, shape):
     np.testing.assert_array_equal(dx.numpy(), x + y.transpose(perm))
     F.move_(dx.permute(*perm), dy)
     np.testing.assert_array_equal(dx.numpy(), y.transpose(perm))
+
+
+@pytest.mark.parametrize("cols", [1, 2, 3, 7, 10, 16, 17, 31, 32, 33, 48, 63, 64])
+@pytest.mark.parametrize("rows", [16384, 20001])
+def test_softmax_and_layernorm_of_tiny_rows(gpu, rows, cols):
+    """Many rows of at most 64 columns take a thread per row (staged through LDS): against float64, the bars
+    of the wavefront-per-row kernels; the row count just below the switch gives the same values to rounding."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    x[5] *= 40                                    # underflowing tail
+    if cols > 1:
+        x[6, : cols // 2] = -np.inf
+    dx = F.from_numpy(x)
+    got = F.softmax_fused(dx).numpy()
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    want = e / e.sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(got, want, rtol=4e-6, atol=1.2e-38)
+    few = F.softmax_fused(F.from_numpy(x[:300])).numpy()      # wavefront form
+    np.testing.assert_allclose(got[:300], few, rtol=1e-6, atol=1.2e-38)
+    # in place
+    inplace = F.from_numpy(x)
+    F.softmax_fused(inplace, out=inplace)
+    np.testing.assert_array_equal(inplace.numpy(), got)
+    # LayerNorm
+    xl = rng.standard_normal((rows, cols)).astype(np.float32) * 2 + 1
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    got = F.layer_norm_fused(F.from_numpy(xl), F.from_numpy(g), F.from_numpy(b), eps=1e-5).numpy()
+    x64 = xl.astype(np.float64)
+    mean = x64.mean(axis=1, keepdims=True)
+    var = ((x64 - mean) ** 2).mean(axis=1, keepdims=True)
+    want = (x64 - mean) / np.sqrt(var + np.float64(np.float32(1e-5))) * g + b
+    # the deviation x - mean is rounded in binary32: an absolute error of about 2^-24 |x| / std per element
+    scale = np.abs(x64).max(axis=1, keepdims=True) / np.sqrt(var + 1e-5)
+    assert np.all(np.abs(got - want) <= 4e-7 * scale * np.abs(g) + 2e-6 * np.abs(want) + 1e-6)
