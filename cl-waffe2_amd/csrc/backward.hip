@@ -168,6 +168,75 @@ __global__ __launch_bounds__(kLongBlock) void softmax_bwd_rows_long(const float*
   }
 }
 
+// Rows beyond 32768 columns, or a few long rows that would leave most compute units without a workgroup:
+// the row in pieces of 8192 columns, a workgroup of 1024 threads each.  The first kernel leaves every piece's
+// sum of dy y in binary64, the second adds the pieces of its row in a fixed order and writes its piece of dx.
+constexpr int kSplitE = 8;
+constexpr int64_t kSplitPiece = (int64_t)kLongBlock * kSplitE;
+
+__global__ __launch_bounds__(kLongBlock) void softmax_bwd_split_dot(const float* __restrict__ y, int64_t ldy,
+                                                                    const float* __restrict__ dy, int64_t lddy,
+                                                                    int64_t ncols, uint32_t pieces,
+                                                                    double* __restrict__ pdot) {
+  __shared__ double lds[kLongBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const float* yr = y + (int64_t)row * ldy;
+  const float* dr = dy + (int64_t)row * lddy;
+  const int64_t c0 = (int64_t)piece * kSplitPiece + threadIdx.x;
+  float a[kSplitE], b[kSplitE];
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    a[k] = c < ncols ? yr[c] : 0.0f;
+    b[k] = c < ncols ? dr[c] : 0.0f;
+  }
+  float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) part[k & 3] = __builtin_fmaf(b[k], a[k], part[k & 3]);
+  const double w = wave_sum(((double)part[0] + (double)part[1]) + ((double)part[2] + (double)part[3]));
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = w;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double total = 0.0;
+    for (int i = 0; i < kLongBlock / kWave; i++) total += lds[i];
+    pdot[blockIdx.x] = total;
+  }
+}
+
+__global__ __launch_bounds__(kLongBlock) void softmax_bwd_split_apply(const float* __restrict__ y, int64_t ldy,
+                                                                      const float* dy, int64_t lddy,  // dx may be dy
+                                                                      float* dx, int64_t lddx, int64_t ncols,
+                                                                      uint32_t pieces,
+                                                                      const double* __restrict__ pdot, float scale) {
+  __shared__ double lds[kLongBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  double s = 0.0;
+  for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock) s += pdot[row * pieces + i];
+  s = wave_sum(s);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = s;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int i = 0; i < kLongBlock / kWave; i++) total += lds[i];
+  const float dot = (float)total;
+  const float* yr = y + (int64_t)row * ldy;
+  const float* dr = dy + (int64_t)row * lddy;
+  float* xr = dx + (int64_t)row * lddx;
+  const int64_t c0 = (int64_t)piece * kSplitPiece + threadIdx.x;
+  float a[kSplitE], b[kSplitE];
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    a[k] = c < ncols ? yr[c] : 0.0f;
+    b[k] = c < ncols ? dr[c] : 0.0f;
+  }
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    if (c < ncols) xr[c] = scale * (a[k] * (b[k] - dot));
+  }
+}
+
 template <bool VEC, bool NT>
 static int launch_softmax_bwd(int nv, const float* y, int64_t ldy, const float* dy, int64_t lddy, float* dx,
                               int64_t lddx, int64_t nrows, int64_t ncols, int64_t causal_seq, float scale) {
@@ -578,6 +647,24 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
   int nv = pick_nv(cols);
   if (nv == 0 || nv > 8) {
     hipStream_t st = rt().stream;
+    const int64_t pieces = ceil_div((int64_t)cols, kSplitPiece);
+    if (causal_seq == 0 && (cols > 32 * kLongBlock || (pieces >= 2 && rows < rt().num_cus)) &&
+        rows * pieces < ((int64_t)1 << 31)) {
+      void* pdot = nullptr;
+      if (wf2hip_malloc_uninitialized(&pdot, (size_t)(rows * pieces) * sizeof(double)) == 0) {
+        const uint32_t grid = (uint32_t)(rows * pieces);
+        softmax_bwd_split_dot<<<grid, kLongBlock, 0, st>>>(y, ldy, dy, lddy, cols, (uint32_t)pieces,
+                                                           static_cast<double*>(pdot));
+        int rc = after_launch("softmax_bwd_split_dot");
+        if (rc == 0) {
+          softmax_bwd_split_apply<<<grid, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, (uint32_t)pieces,
+                                                               static_cast<const double*>(pdot), scale);
+          rc = after_launch("softmax_bwd_split_apply");
+        }
+        (void)wf2hip_free(pdot);  // stream order keeps it alive for the launches above
+        return rc;
+      }
+    }
     if (causal_seq == 0 && cols <= 32 * kLongBlock) {  // beyond: y and dy of a row exceed the registers of 1024 threads
       if (cols <= 4 * kLongBlock)
         softmax_bwd_rows_long<4><<<(uint32_t)rows, kLongBlock, 0, st>>>(y, ldy, dy, lddy, dx, lddx, cols, scale);

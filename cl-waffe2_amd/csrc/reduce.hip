@@ -987,51 +987,11 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_pair(const float* __restr
   }
 }
 
-// Rows too long for registers: one workgroup per row, three passes (the second
-// and third hit L2).
-template <bool XENT>
-__global__ __launch_bounds__(kBlock) void softmax_rows_block(const float* __restrict__ x, int64_t ldx,
-                                                             float* __restrict__ out, int64_t ldo,
-                                                             int64_t ncols, Xent xe) {
-  __shared__ float lmax[kWavesPerBlock];
-  __shared__ double lsum[kWavesPerBlock];
-  const float* xr = x + (int64_t)blockIdx.x * ldx;
-  float* orow = out + (int64_t)blockIdx.x * ldo;
-  float m = -__builtin_inff();
-  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) m = fmaxf(m, xr[c]);
-  m = wave_max(m);
-  if ((threadIdx.x & (kWave - 1)) == 0) lmax[threadIdx.x / kWave] = m;
-  __syncthreads();
-  m = lmax[0];
-  for (int i = 1; i < kWavesPerBlock; i++) m = fmaxf(m, lmax[i]);
-  double s = 0.0;
-  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
-    double d = (double)xr[c] - (double)m;
-    s += (d < -104.0) ? 0.0 : exp_core(d);
-  }
-  s = wave_sum(s);
-  if ((threadIdx.x & (kWave - 1)) == 0) lsum[threadIdx.x / kWave] = s;
-  __syncthreads();
-  s = 0.0;
-  for (int i = 0; i < kWavesPerBlock; i++) s += lsum[i];
-  const double inv = 1.0 / s;
-  for (int64_t c = threadIdx.x; c < ncols; c += kBlock) {
-    double d = (double)xr[c] - (double)m;
-    double ed = (d < -104.0) ? 0.0 : exp_core(d);
-    const float z = (float)(ed * inv);
-    orow[c] = z;
-    if (XENT) {
-      const int64_t at = (int64_t)blockIdx.x * ncols + c;
-      xe.loss[at] = xent_term(xe.labels[at], z, xe.delta);
-    }
-  }
-}
-
 // Rows of 4097 ... 65536 columns (a vocabulary: the logits of a language model): a workgroup of
 // 1024 threads per row, thread t holding columns t, t + 1024, ... in registers, so the row is read
 // once and written once; maxima and sums meet in LDS.  The three-pass form above reads the row three
-// times from wherever it lies (reads that hit the L2 cost the memory system what misses cost) and
-// evaluates its exponentials in binary64: (4096, 50257) 982 us.  The exponential of softmax_rows_wave.
+// times from wherever it lies (reads that hit the L2 cost the memory system what misses cost):
+// (4096, 50257) 982 us.  The exponential of softmax_rows_wave.
 constexpr int kLongBlock = 1024;
 
 template <int E, bool XENT>
@@ -1102,6 +1062,123 @@ __global__ __launch_bounds__(kLongBlock) void softmax_rows_long(const float* __r
         if (c < ncols) xe.loss[base + c] = xent_term(lab[u], v[k0 + u], xe.delta);
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+// Rows beyond 65536 columns, or a few long rows that would leave most compute units without a workgroup
+// ((1, 16777216): 62 ms on one workgroup): the row in pieces of 16384 columns, a workgroup of 1024 threads
+// each.  softmax_split_stats leaves every piece's maximum m_p and s_p = sum exp(x - m_p) (its 16 elements
+// per thread in registers, one read); softmax_split_apply folds the pieces of its row -- M = max m_p,
+// S = sum s_p exp(m_p - M) in binary64, in a fixed order -- and writes exp(x - M) / S: two reads and a
+// write of the row.  The exponential of softmax_rows_wave.
+constexpr int kSplitE = 16;
+constexpr int64_t kSplitPiece = (int64_t)kLongBlock * kSplitE;
+
+__device__ __forceinline__ float exp_below_max(float v, float m) {
+  const float d = fmaxf(v - m, -160.0f);
+  const float t = d * 1.44269502f;
+  float tl = __builtin_fmaf(d, 1.44269502f, -t);
+  tl = __builtin_fmaf(d, 1.92596299e-8f, tl);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(e, tl * 0.693147182f, e);
+}
+
+__device__ __forceinline__ float long_block_max(float m, float* lmax) {
+  m = wave_max(m);
+  __syncthreads();  // lmax may still be read from an earlier use
+  if ((threadIdx.x & (kWave - 1)) == 0) lmax[threadIdx.x / kWave] = m;
+  __syncthreads();
+  m = lmax[0];
+#pragma unroll
+  for (int w = 1; w < kLongBlock / kWave; w++) m = fmaxf(m, lmax[w]);
+  return m;
+}
+
+__device__ __forceinline__ double long_block_sum(double s, double* lsum) {
+  s = wave_sum(s);
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) lsum[threadIdx.x / kWave] = s;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int w = 0; w < kLongBlock / kWave; w++) total += lsum[w];
+  return total;
+}
+
+__global__ __launch_bounds__(kLongBlock) void softmax_split_stats(const float* __restrict__ x, int64_t ldx,
+                                                                  int64_t ncols, uint32_t pieces,
+                                                                  float* __restrict__ pmax,
+                                                                  double* __restrict__ psum) {
+  __shared__ float lmax[kLongBlock / kWave];
+  __shared__ double lsum[kLongBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const float* xr = x + (int64_t)row * ldx;
+  const int64_t c0 = (int64_t)piece * kSplitPiece + threadIdx.x;
+  const float ninf = -__builtin_inff();
+  float v[kSplitE];
+  float m = ninf;
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    v[k] = c < ncols ? xr[c] : ninf;
+    m = fmaxf(m, v[k]);
+  }
+  m = long_block_max(m, lmax);
+  float sum = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) sum += exp_below_max(v[k], m);
+  const double total = long_block_sum((double)sum, lsum);
+  if (threadIdx.x == 0) {
+    pmax[blockIdx.x] = m;
+    psum[blockIdx.x] = total;
+  }
+}
+
+template <bool XENT>
+__global__ __launch_bounds__(kLongBlock) void softmax_split_apply(const float* x, int64_t ldx,  // out may be x
+                                                                  float* out, int64_t ldo, int64_t ncols,
+                                                                  uint32_t pieces, const float* __restrict__ pmax,
+                                                                  const double* __restrict__ psum, Xent xe) {
+  __shared__ float lmax[kLongBlock / kWave];
+  __shared__ double lsum[kLongBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const float ninf = -__builtin_inff();
+  float m = ninf;
+  for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock) m = fmaxf(m, pmax[row * pieces + i]);
+  m = long_block_max(m, lmax);
+  double s = 0.0;
+  for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock)
+    s += psum[row * pieces + i] * (double)exp_below_max(pmax[row * pieces + i], m);
+  const float inv = (float)(1.0 / long_block_sum(s, lsum));
+  const float* xr = x + (int64_t)row * ldx;
+  float* orow = out + (int64_t)row * ldo;
+  const int64_t c0 = (int64_t)piece * kSplitPiece + threadIdx.x;
+  float v[kSplitE];
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    v[k] = c < ncols ? xr[c] : ninf;
+  }
+  float lab[XENT ? kSplitE : 1];
+  if (XENT) {
+#pragma unroll
+    for (int k = 0; k < kSplitE; k++) {
+      const int64_t c = c0 + (int64_t)k * kLongBlock;
+      lab[k] = c < ncols ? xe.labels[(int64_t)row * ncols + c] : 0.0f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kSplitE; k++) {
+    const int64_t c = c0 + (int64_t)k * kLongBlock;
+    v[k] = exp_below_max(v[k], m) * inv;
+    if (c < ncols) orow[c] = v[k];
+  }
+  if (XENT) {
+#pragma unroll
+    for (int k = 0; k < kSplitE; k++) {
+      const int64_t c = c0 + (int64_t)k * kLongBlock;
+      if (c < ncols) xe.loss[(int64_t)row * ncols + c] = xent_term(lab[k], v[k], xe.delta);
     }
   }
 }
@@ -1435,6 +1512,23 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
     if (causal_seq > 0) return fail(WF2HIP_EUNSUPPORTED, "causal softmax rows longer than 4096");
     if (nrows >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many rows");
     hipStream_t st = rt().stream;
+    const int64_t pieces = ceil_div(ncols, kSplitPiece);
+    if (ncols > 64 * kLongBlock || (pieces >= 2 && nrows < rt().num_cus)) {
+      if (nrows * pieces >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many row pieces for one launch");
+      void* stats = nullptr;  // nrows x pieces sums (binary64), then as many maxima
+      WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(nrows * pieces) * (sizeof(double) + sizeof(float))));
+      double* psum = static_cast<double*>(stats);
+      float* pmax = reinterpret_cast<float*>(psum + nrows * pieces);
+      const uint32_t grid = (uint32_t)(nrows * pieces);
+      softmax_split_stats<<<grid, kLongBlock, 0, st>>>(x, ldx, ncols, (uint32_t)pieces, pmax, psum);
+      int rc = after_launch("softmax_split_stats");
+      if (rc == 0) {
+        softmax_split_apply<XENT><<<grid, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, (uint32_t)pieces, pmax, psum, xe);
+        rc = after_launch("softmax_split_apply");
+      }
+      (void)wf2hip_free(stats);  // stream order keeps it alive for the launches above
+      return rc;
+    }
     if (ncols <= 8 * kLongBlock)
       softmax_rows_long<8, XENT><<<(uint32_t)nrows, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
     else if (ncols <= 16 * kLongBlock)
@@ -1443,10 +1537,8 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
       softmax_rows_long<32, XENT><<<(uint32_t)nrows, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
     else if (ncols <= 52 * kLongBlock)  // GPT-2's vocabulary of 50257 with fewer register spills than 64
       softmax_rows_long<52, XENT><<<(uint32_t)nrows, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
-    else if (ncols <= 64 * kLongBlock)
-      softmax_rows_long<64, XENT><<<(uint32_t)nrows, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
     else
-      softmax_rows_block<XENT><<<(uint32_t)nrows, kBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
+      softmax_rows_long<64, XENT><<<(uint32_t)nrows, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, xe);
     return after_launch("softmax_rows_long");
   }
   int64_t blocks = ceil_div(nrows, kWavesPerBlock);

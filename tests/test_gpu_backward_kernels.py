@@ -74,7 +74,8 @@ def _softmax_bwd_truth(y, dy, scale, causal):
 
 
 @pytest.mark.parametrize("rows,cols", [(16384, 1), (16385, 2), (20001, 10), (16500, 31), (16384, 32), (16400, 33), (16390, 64), (5, 7), (33, 256), (100, 1000), (64, 1024), (17, 1537), (9, 2048), (6, 5000),
-                                       (7, 2049), (5, 4096), (9, 8193), (4, 16385), (3, 32768), (3, 50257)])
+                                       (7, 2049), (5, 4096), (9, 8193), (4, 16385), (3, 32768), (3, 50257), (1, 1 << 21), (300, 8192),
+                                       (300, 40001), (2, 1234567)])
 def test_softmax_backward_rows(gpu, rows, cols):
     W = gpu
     F = W.functional

@@ -268,18 +268,36 @@ def test_config4_softmax(gpu):
 
 
 @pytest.mark.parametrize("cols", [1, 3, 64, 100, 255, 256, 1000, 1024, 2050, 4096, 4097, 5000, 8192, 8193, 20000,
-                                  32768, 40000, 50257, 53249, 65536, 70000])
+                                  32768, 40000, 50257, 53249, 65536, 70000, 200001])
 def test_softmax_widths(gpu, cols):
     """Every row form: 1 ... 4096 columns in a wavefront's registers, 4097 ... 65536 in those of a workgroup of
-    1024 threads (8, 16, 32, 52 or 64 elements per thread), longer rows in three passes."""
+    1024 threads (8, 16, 32, 52 or 64 elements per thread; a few rows beyond 16384 columns in pieces of 16384),
+    longer rows in pieces."""
     F = gpu.functional
     rng = np.random.default_rng(cols)
     X = (rng.standard_normal((37 if cols < 30000 else 5, cols)) * 4).astype(np.float32)
     got = F.softmax_fused(F.from_numpy(X)).numpy()
-    if cols <= 65536:
-        _assert_softmax(got, _softmax64(X), f"{cols} columns")
-    else:  # rows too long for registers: the three-pass binary64 kernel
-        assert ulp_distance(got, _softmax64(X).astype(np.float32)).max() <= 2
+    _assert_softmax(got, _softmax64(X), f"{cols} columns")
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 16385), (1, 1 << 22), (3, 16384 * 5 + 7), (300, 32768), (300, 70001), (2, 1234567)])
+def test_softmax_rows_in_pieces(gpu, rows, cols):
+    """Rows handled as pieces of 16384 columns whose maxima and sums are folded afterwards: pieces that hold the
+    row's maximum first, last and in the middle, a piece of -inf only, a ragged last piece, in place, and an
+    unaligned row pitch; rows sum to 1."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows + cols)
+    X = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    X[0, cols - 1] = 30.0                       # the maximum in the last piece
+    if rows > 1:
+        X[1, 0] = 40.0                          # ... in the first
+        X[1, 16384:min(cols, 32768)] = -np.inf  # a piece that contributes nothing
+    d = F.from_numpy(X)
+    got = F.softmax_fused(d).numpy()
+    _assert_softmax(got, _softmax64(X), f"({rows}, {cols})")
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
+    F.softmax_fused(d, out=d)
+    np.testing.assert_array_equal(d.numpy(), got)
 
 
 def test_softmax_reference_composition(gpu, O):
