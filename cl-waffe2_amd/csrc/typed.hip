@@ -508,15 +508,76 @@ __global__ __launch_bounds__(kBlock) void typed_accumulate_cols(T* a, const T* b
     partials[(int64_t)split * ncols + c] = total;
 }
 
+// Narrow dense matrices (at most 128 columns, rows adjacent in memory): the 256-column tiles above leave most
+// lanes without a column ((131072, 64) :double: 518 us).  The workgroup reads k = 256 / ncols whole rows per
+// step, one contiguous run: thread t adds column t mod ncols of every k-th row with eight loads in flight, and
+// the k threads of a column meet in LDS in a fixed order.
+template <class T>
+__global__ __launch_bounds__(kBlock) void typed_accumulate_cols_narrow(T* a, const T* b, int64_t nred, uint32_t ncols,
+                                                                       uint32_t splits, int64_t seg,
+                                                                       typename SumOf<T>::type* partials) {
+  using S = typename SumOf<T>::type;
+  __shared__ S lds[kBlock];
+  const uint32_t k = kBlock / ncols;  // rows per step
+  const uint32_t phase = threadIdx.x / ncols, col = threadIdx.x - phase * ncols;
+  const int64_t lo = (int64_t)blockIdx.x * seg;
+  const int64_t hi = lo + seg < nred ? lo + seg : nred;
+  S acc = S(0);
+  if (phase < k) {
+    const T* src = b + col;
+    int64_t j = lo + phase;
+    for (; j + 7 * (int64_t)k < hi; j += 8 * (int64_t)k) {
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = src[(j + u * (int64_t)k) * ncols];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc += (S)v[u];
+    }
+    for (; j < hi; j += k) acc += (S)src[j * ncols];
+  }
+  lds[threadIdx.x] = acc;
+  __syncthreads();
+  if (threadIdx.x < ncols) {
+    S total = lds[threadIdx.x];
+    for (uint32_t r = 1; r < k; r++) total += lds[r * ncols + threadIdx.x];
+    if (splits == 1)
+      a[threadIdx.x] = (T)((S)a[threadIdx.x] + total);
+    else
+      partials[(int64_t)blockIdx.x * ncols + threadIdx.x] = total;
+  }
+}
+
+// Folds the splits' partial sums: 64 columns per workgroup, its four wavefronts take every fourth split with
+// eight loads in flight, then meet in LDS -- a fixed order.  (One thread per column walking all splits in
+// turn waits for memory once per split.)
 template <class T>
 __global__ __launch_bounds__(kBlock) void typed_accumulate_cols_fold(T* a, int64_t ncols, uint32_t splits,
                                                                      const typename SumOf<T>::type* partials) {
   using S = typename SumOf<T>::type;
-  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (c >= ncols) return;
-  S total = S(0);
-  for (uint32_t s = 0; s < splits; s++) total += partials[(int64_t)s * ncols + c];
-  a[c] = (T)((S)a[c] + total);
+  constexpr int kWaves = kBlock / kWave;
+  __shared__ S lds[kWaves][kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t c = (int64_t)blockIdx.x * kWave + lane;
+  S acc = S(0);
+  if (c < ncols) {
+    uint32_t sp = (uint32_t)wave;
+    for (; sp + 7 * kWaves < splits; sp += 8 * kWaves) {
+      S t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) t[u] = partials[(int64_t)(sp + u * kWaves) * ncols + c];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc += t[u];
+    }
+    for (; sp < splits; sp += kWaves) acc += partials[(int64_t)sp * ncols + c];
+  }
+  lds[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && c < ncols) {
+    S total = lds[0][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) total += lds[w][lane];
+    a[c] = (T)((S)a[c] + total);
+  }
 }
 
 // Few destinations, long reductions: `splits` workgroups per destination each sum a
@@ -608,11 +669,15 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
     using S = typename SumOf<T>::type;
     const int64_t target = (int64_t)rt().num_cus * 8;
     const int last = s.rank - 1;
-    if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 2) {
+    // a dense matrix of at most 128 columns with at least 64 steps of whole rows
+    const bool narrow = p.nk == 1 && p.nr == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] <= 128 &&
+                        p.rb[0] == s.shape[last] && p.nred >= 64 * (kBlock / s.shape[last]);
+    if (narrow || (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] >= 64 && p.nred >= 2)) {
       const int64_t ncols = s.shape[last];
-      const int64_t ctiles = ceil_div(ncols, kBlock);
+      const int64_t ctiles = narrow ? 1 : ceil_div(ncols, kBlock);
       int64_t splits = ceil_div(target, ctiles);
-      if (splits > p.nred / 32) splits = p.nred / 32;
+      const int64_t least = narrow ? 64 * (kBlock / ncols) : 32;  // reduced indices per workgroup
+      if (splits > p.nred / least) splits = p.nred / least;
       if (splits < 1) splits = 1;
       int64_t seg = ceil_div(p.nred, splits);
       splits = ceil_div(p.nred, seg);
@@ -623,12 +688,16 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
         seg = p.nred;
       }
       if (ctiles * splits < ((int64_t)1 << 31)) {
-        typed_accumulate_cols<T><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(ap, bp, p, ncols, (uint32_t)splits, seg,
-                                                                               static_cast<S*>(scratch));
+        if (narrow)
+          typed_accumulate_cols_narrow<T><<<(uint32_t)splits, kBlock, 0, st>>>(ap, bp, p.nred, (uint32_t)ncols,
+                                                                             (uint32_t)splits, seg, static_cast<S*>(scratch));
+        else
+          typed_accumulate_cols<T><<<(uint32_t)(ctiles * splits), kBlock, 0, st>>>(ap, bp, p, ncols, (uint32_t)splits, seg,
+                                                                                 static_cast<S*>(scratch));
         int rc = after_launch("typed_accumulate_cols");
         if (rc == 0 && splits > 1) {
-          typed_accumulate_cols_fold<T><<<(uint32_t)ctiles, kBlock, 0, st>>>(ap, ncols, (uint32_t)splits,
-                                                                            static_cast<const S*>(scratch));
+          typed_accumulate_cols_fold<T><<<(uint32_t)ceil_div(ncols, kWave), kBlock, 0, st>>>(ap, ncols, (uint32_t)splits,
+                                                                                         static_cast<const S*>(scratch));
           rc = after_launch("typed_accumulate_cols_fold");
         }
         if (scratch) (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above

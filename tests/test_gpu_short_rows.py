@@ -141,7 +141,8 @@ def test_column_sums_of_narrow_and_of_flat_matrices(gpu, rows, cols):
 
 
 @pytest.mark.parametrize("dtype", ["double", "int32", "uint8", "int16"])
-@pytest.mark.parametrize("rows,cols", [(200001, 4), (140000, 9), (3, 70000)])
+@pytest.mark.parametrize("rows,cols", [(200001, 4), (140000, 9), (3, 70000), (70001, 64), (30000, 100), (20000, 128), (9000, 129),
+                                       (5000, 1)])
 def test_typed_sums_of_short_rows_and_of_flat_matrices(gpu, dtype, rows, cols):
     """!sum on :double and the integer types (wrap-around sums, as the reference's C loops produce) along a
     short trailing axis of very many rows, and down the few rows of a flat matrix."""
