@@ -832,42 +832,48 @@ struct Epilogue {
   int causal = 0;
 };
 
-// C <- beta C + sum over the `splits` partial products of a split-K run (column-major,
-// partials packed m x n each, already scaled by alpha)
+// C[b] <- beta C[b] + sum over the `splits` partial products of a split-K run (column-major; the partial
+// of slice s and matrix b is the packed m x n plane s * batch + b, already scaled by alpha);
+// blockIdx.y is the matrix of the batch
 __global__ __launch_bounds__(kBlock) void splitk_fold(const float* __restrict__ partials, int splits, int64_t m,
-                                                      int64_t n, float beta, float* __restrict__ C, int64_t ldc) {
+                                                      int64_t n, float beta, float* __restrict__ C, int64_t ldc,
+                                                      int64_t strideC) {
   const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (e >= m * n) return;
   const int64_t j = e / m, i = e - j * m;
+  const int64_t plane = m * n, step = plane * gridDim.y;
+  partials += (int64_t)blockIdx.y * plane;
   float acc = 0.0f;
-  for (int s = 0; s < splits; s++) acc += partials[(int64_t)s * m * n + e];
-  float* c = C + i + j * ldc;
+  for (int s = 0; s < splits; s++) acc += partials[(int64_t)s * step + e];
+  float* c = C + (int64_t)blockIdx.y * strideC + i + j * ldc;
   *c = beta == 0.0f ? acc : beta * *c + acc;
 }
 
 // More than 16 partial products: a wavefront per output element, lane l adds slices l, l + 64, ...
 // in binary64 with eight loads in flight, the lanes meet by shuffles -- a fixed order.
 __global__ __launch_bounds__(kBlock) void splitk_fold_wide(const float* __restrict__ partials, int splits, int64_t m,
-                                                           int64_t n, float beta, float* __restrict__ C, int64_t ldc) {
+                                                           int64_t n, float beta, float* __restrict__ C, int64_t ldc,
+                                                           int64_t strideC) {
   const int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (e >= m * n) return;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t plane = m * n;
+  const int64_t plane = m * n, step = plane * gridDim.y;
+  partials += (int64_t)blockIdx.y * plane;
   double acc = 0.0;
   int s = lane;
   for (; s + 7 * kWave < splits; s += 8 * kWave) {
     float v[8];
 #pragma unroll
-    for (int u = 0; u < 8; u++) v[u] = partials[(int64_t)(s + u * kWave) * plane + e];
+    for (int u = 0; u < 8; u++) v[u] = partials[(int64_t)(s + u * kWave) * step + e];
 #pragma unroll
     for (int u = 0; u < 8; u++) acc += (double)v[u];
   }
-  for (; s < splits; s += kWave) acc += (double)partials[(int64_t)s * plane + e];
+  for (; s < splits; s += kWave) acc += (double)partials[(int64_t)s * step + e];
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
   if (lane == 0) {
     const int64_t j = e / m, i = e - j * m;
-    float* c = C + i + j * ldc;
+    float* c = C + (int64_t)blockIdx.y * strideC + i + j * ldc;
     *c = beta == 0.0f ? (float)acc : beta * *c + (float)acc;
   }
 }
@@ -879,40 +885,65 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
 
 int binary_nd(int op, Space s, float* a, const float* b);  // elementwise.hip
 
-// A single product with few output tiles and a long K (weight gradients: 768 x 3072
-// outputs over K = 8192 are 144 tiles for 256 compute units) runs as `splits` products
-// over slices of K in one batched launch, folded in a fixed order afterwards.
+// Products with few output tiles and a long K (weight gradients: 768 x 3072 outputs over K = 8192 are
+// 144 tiles for 256 compute units) run as `splits` products over slices of K, the slices as the outer
+// batch level of one launch, folded in a fixed order afterwards.  One batch level of such products
+// ((12, 3, 100000) . (12, 100000, 3)) is split the same way.
 static bool try_split_k(char transa, char transb, long m, long n, long k, float alpha, const float* A, long lda,
-                        const float* B, long ldb, float beta, float* C, long ldc, int* rc) {
-  const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128);
+                        long strideA, const float* B, long ldb, long strideB, float beta, float* C, long ldc,
+                        long strideC, long batch, int* rc) {
+  static thread_local bool splitting = false;  // the slices themselves are not split again
+  struct Guard {
+    bool& flag;
+    explicit Guard(bool& f) : flag(f) { flag = true; }
+    ~Guard() { flag = false; }
+  };
+  const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128) * batch;
   const int64_t cus = rt().num_cus;
-  if (k < 2048 || tiles >= cus || m < 1 || n < 1) return false;
-  // Few output tiles and a very long K (the weight gradient of a layer with few outputs:
-  // (10 x N) . (N x 256) over a batch of 65536 ran 150 us on 16 slices): as many slices of at
-  // least 512 as keep the launch within four workgroups per compute unit.
-  int splits = 0;
-  for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
-    if (k % ((long)cand * 32) == 0 && k / cand >= 512 && tiles * cand <= 4 * cus) {
-      splits = cand;
-      break;
-    }
-  if (splits == 0) return false;
-  const long kc = k / splits;
+  if (splitting || k < 2048 || tiles >= cus || m < 1 || n < 1) return false;
+  Guard guard(splitting);
+  // Equal slices where K allows it.  Few output tiles and a very long K (the weight gradient of a layer
+  // with few outputs: (10 x N) . (N x 256) over a batch of 65536 ran 150 us on 16 slices): as many slices
+  // of at least 512 as keep the launch within four workgroups per compute unit.
+  long splits = 0, kc = 0;
+  if (batch == 1)
+    for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
+      if (k % ((long)cand * 32) == 0 && k / cand >= 512 && tiles * cand <= 4 * cus) {
+        splits = cand;
+        kc = k / cand;
+        break;
+      }
+  long rest = 0;  // length of a shorter last slice
+  if (splits == 0) {
+    // any K ((127 x 100000) . (100000 x 127) ran 5.9 ms as one product): slices of a multiple of 32, the
+    // last one shorter, in a launch of its own
+    long most = std::min<long>(k / 512, (long)(4 * cus / tiles));
+    most = std::min<long>(most, 1024);
+    if (most < 2) return false;
+    kc = ceil_div(ceil_div(k, most), 32L) * 32;
+    splits = k / kc;
+    rest = k - splits * kc;
+    if (splits + (rest ? 1 : 0) < 2) return false;
+  }
+  const long planes = splits + (rest ? 1 : 0);
+  const int64_t plane = (int64_t)m * n;
   void* scratch = nullptr;
-  if (wf2hip_malloc_uninitialized(&scratch, (size_t)splits * m * n * sizeof(float)) != 0) return false;
+  if (wf2hip_malloc_uninitialized(&scratch, (size_t)(planes * batch * plane) * sizeof(float)) != 0) return false;
+  float* part = static_cast<float*>(scratch);
   const long sa = is_n(transa) ? kc * lda : kc;  // op(A) is m x k: a K slice starts kc columns / rows further
   const long sb = is_n(transb) ? kc : kc * ldb;
-  *rc = sgemm_batched2(transa, transb, m, n, kc, alpha, A, lda, sa, 0, B, ldb, sb, 0, 0.0f,
-                       static_cast<float*>(scratch), m, (long)m * n, 0, splits, 1);
+  *rc = sgemm_batched2(transa, transb, m, n, kc, alpha, A, lda, strideA, sa, B, ldb, strideB, sb, 0.0f, part, m,
+                       (long)plane, (long)(plane * batch), batch, splits);
+  if (*rc == 0 && rest)
+    *rc = sgemm_batched2(transa, transb, m, n, rest, alpha, A + splits * sa, lda, strideA, 0, B + splits * sb, ldb,
+                         strideB, 0, 0.0f, part + splits * batch * plane, m, (long)plane, 0, batch, 1);
   if (*rc == 0) {
-    if (splits <= 16) {
-      const int64_t blocks = ceil_div((int64_t)m * n, kBlock);
-      splitk_fold<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m, n,
-                                                                 beta, C, ldc);
+    if (planes <= 16) {
+      const dim3 grid((uint32_t)ceil_div(plane, (int64_t)kBlock), (uint32_t)batch);
+      splitk_fold<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC);
     } else {
-      const int64_t blocks = ceil_div((int64_t)m * n, kBlock / kWave);
-      splitk_fold_wide<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(static_cast<const float*>(scratch), splits, m,
-                                                                      n, beta, C, ldc);
+      const dim3 grid((uint32_t)ceil_div(plane, (int64_t)(kBlock / kWave)), (uint32_t)batch);
+      splitk_fold_wide<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC);
     }
     *rc = after_launch("splitk_fold");
   }
@@ -962,9 +993,10 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
       return rc;
     }
   }
-  if (batch == 1 && batch2 == 1 && !ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
+  if (batch2 == 1 && batch <= 65535 && !ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
     int rc = 0;
-    if (try_split_k(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, &rc)) return rc;
+    if (try_split_k(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, &rc))
+      return rc;
   }
 
   GemmParams p;

@@ -415,12 +415,22 @@ def test_matmul_few_tiles_long_k(gpu, ta, tb):
     # the last four: tiny outputs over a very long K (the weight gradients of layers with few outputs),
     # which run as up to 1024 slices folded by a wavefront per output element
     for m, n, k in [(768, 640, 8192), (200, 300, 4096), (130, 1000, 2048), (10, 256, 65536), (256, 10, 65536),
-                    (4, 9, 100352), (3, 3, 1 << 20)]:
+                    (4, 9, 100352), (3, 3, 1 << 20), (127, 127, 100000), (33, 65, 5003), (200, 100, 2049),
+                    (5, 7, 300001)]:   # the last four: K that no equal slices divide, a shorter last slice
         A = rng.standard_normal((m, k)).astype(np.float32)
         B = rng.standard_normal((k, n)).astype(np.float32)
         dA = F.t(F.from_numpy(np.ascontiguousarray(A.T))) if ta else F.from_numpy(A)
         dB = F.t(F.from_numpy(np.ascontiguousarray(B.T))) if tb else F.from_numpy(B)
         _gemm_check(F.matmul(dA, dB).numpy(), A.astype(np.float64), B.astype(np.float64))
+    # one batch level of such products, K on and off equal slices
+    for batch, m, n, k in [(12, 3, 5, 100000), (5, 130, 40, 4096), (3, 64, 64, 6001)]:
+        A = rng.standard_normal((batch, m, k)).astype(np.float32)
+        B = rng.standard_normal((batch, k, n)).astype(np.float32)
+        dA = F.t(F.from_numpy(np.ascontiguousarray(A.transpose(0, 2, 1)))) if ta else F.from_numpy(A)
+        dB = F.t(F.from_numpy(np.ascontiguousarray(B.transpose(0, 2, 1)))) if tb else F.from_numpy(B)
+        got = F.matmul(dA, dB).numpy()
+        for b in range(batch):
+            _gemm_check(got[b], A[b].astype(np.float64), B[b].astype(np.float64))
     # column-major contract with beta and padded leading dimensions
     lib = W.lib.get()
     m, n, k = 96, 200, 4096
