@@ -884,6 +884,9 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
                    long batch, long batch2, const Epilogue& ep = Epilogue());
 
 int binary_nd(int op, Space s, float* a, const float* b);  // elementwise.hip
+bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float alpha, const float* W, long ldw,
+                      const float* X, long ldx, float beta, float* C, long ldc, const float* bias,
+                      const float* residual, long ldres, int activation, int* rc);  // gemm_skinny.hip
 
 // Products with few output tiles and a long K (weight gradients: 768 x 3072 outputs over K = 8192 are
 // 144 tiles for 256 compute units) run as `splits` products over slices of K, the slices as the outer
@@ -969,6 +972,13 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
   if ((int64_t)batch * batch2 > 65535)
     return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  // at most 64 rows in the row-major product (a few tokens through a layer): one read of the other operand
+  if (batch == 1 && batch2 == 1 && n <= 64 && is_n(transb) && ep.causal == 0) {
+    int rc = 0;
+    if (try_sgemm_skinny(!is_n(transa), n, m, k, alpha, A, lda, B, ldb, beta, C, ldc, ep.bias, ep.residual, ep.ldres,
+                         ep.activation, &rc))
+      return rc;
+  }
   // x^T . dY (weight gradients): the left operand of the row-major product arrives stored
   // (k, rows), which only the register-staged kernel reads.  One transposing pass over it
   // (k x rows elements) puts the product on the streaming kernel.

@@ -1,0 +1,264 @@
+// gemm_skinny.hip -- MatMulNode when the left operand of the row-major product has at most 64 rows
+// (a few tokens through a Linear layer: x (rows, k) . W, W being (k, cols) or the (cols, k) storage that
+// `(!matmul x (!t w))` hands to sgemm_, source/backends/cpu/matrix-ops.lisp:12-112).
+//
+// Such a product is one read of W.  The tiled kernel of gemm.hip pads the rows to its 128 x 128 tile, so
+// its matrix cores and LDS do the work of 128 rows whatever the row count and W streams at 1.4 - 1.7 TB/s
+// ((1 ... 64, 8192) . (8192, 8192): 155 - 175 us).  Here a wavefront owns 16 CB columns of the output
+// (CB = 4 blocks; eight halve x's share of the requests but cost more in registers than that returns:
+// 32 rows of 8192 x 8192 74 -> 97 us, 64 rows 124 -> 164 us) and a slice of K and feeds
+// v_mfma_f32_16x16x4 straight from global memory, 16 steps of K at a time:
+//   W operand, lane (kk = lane / 16, jj = lane % 16):
+//     (cols, k) storage: CB 16-byte loads, W[j0 + 16 b + jj][k0 + 4 kk ... + 3], b = 0 .. CB - 1
+//     (k, cols) storage: CB 16-byte loads, W[k0 + 4 kk + s][j0 + 64 h + 4 jj ... + 3], s = 0 .. 3, h < CB / 4
+//   x operand: one 16-byte load per 16 rows, x[16 t + jj][k0 + 4 kk ... + 3]
+//   the product for step s (k = k0 + 4 kk + s on lane group kk) and column block b adds into the 16 x 16
+//   tile D of rows 16 t ... and columns j0 + 16 b + jj, or j0 + 64 (b / 4) + 4 jj + b % 4 (columns
+//   interleaved by four, so that a lane's four tiles are four neighbouring columns).
+// The four wavefronts of a workgroup take a quarter of the workgroup's slice of K each and meet in LDS;
+// with several slices of K over the grid each writes a plane of its own and skinny_finish adds the planes
+// in a fixed order.  alpha, beta, bias, activation and residual are applied once, at the end.
+#include "wf2_common.h"
+#include "wf2_math.h"
+
+namespace wf2 {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct SkinnyParams {
+  const float* W;
+  const float* X;
+  float* C;             // row-major rows x cols, pitch ldc
+  int64_t ldw, ldx, ldc;
+  int32_t rows;
+  int64_t cols;
+  int32_t k;
+  int32_t kslice;       // K per workgroup, a multiple of 64
+  uint32_t cgroups;     // groups of 16 CB columns
+  uint32_t gsplit;      // slices of K over the grid
+  float* partial;       // gsplit planes of rows x cols (packed) when gsplit > 1
+  float alpha, beta;
+  const float* bias;      // cols floats or null
+  const float* residual;  // rows x cols, pitch ldres, or null
+  int64_t ldres;
+  int32_t activation;     // 0 none, 1 tanh-form GELU
+};
+
+__device__ __forceinline__ void skinny_finish_store(const SkinnyParams& p, int row, int64_t col, float acc) {
+  float* c = p.C + (int64_t)row * p.ldc + col;
+  float v = p.alpha * acc;
+  if (p.beta != 0.0f) v += p.beta * *c;
+  if (p.bias) v += p.bias[col];
+  if (p.activation == 1) v = gelu_tanh_fast(v);
+  if (p.residual) v += p.residual[(int64_t)row * p.ldres + col];
+  *c = v;
+}
+
+// TW: W stored (cols, k), k contiguous; otherwise (k, cols), columns contiguous.  MT tiles of 16 rows,
+// CB blocks of 16 columns.
+template <bool TW, int MT, int CB>
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
+  __shared__ float meet[MT * CB * 4 * kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int kk = lane >> 4, jj = lane & 15;
+  const uint32_t ks = blockIdx.x / p.cgroups, cg = blockIdx.x - ks * p.cgroups;
+  const int64_t j0 = (int64_t)cg * (16 * CB);
+  const int quarter = p.kslice / 4;
+  const int kbeg = (int)ks * p.kslice + wave * quarter;
+  const int kend = kbeg + quarter < p.k ? kbeg + quarter : p.k;
+  const f4 zero = {0.f, 0.f, 0.f, 0.f};
+  f4 acc[MT][CB];
+#pragma unroll
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int b = 0; b < CB; b++) acc[t][b] = zero;
+
+  // row pointers (columns / rows past the end read a valid address and are not stored)
+  const float* wrow[CB];
+  if (TW) {
+#pragma unroll
+    for (int b = 0; b < CB; b++) {
+      int64_t j = j0 + 16 * b + jj;
+      if (j >= p.cols) j = p.cols - 1;
+      wrow[b] = p.W + j * p.ldw + 4 * kk;
+    }
+  } else {
+#pragma unroll
+    for (int h = 0; h < CB / 4; h++) {
+      int64_t j = j0 + 64 * h + 4 * jj;
+      if (j + 3 >= p.cols) j = p.cols - 4;  // cols is a multiple of 4 (host)
+#pragma unroll
+      for (int s = 0; s < 4; s++) wrow[4 * h + s] = p.W + (int64_t)(4 * kk + s) * p.ldw + j;
+    }
+  }
+  const float* xrow[MT];
+  bool xlive[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const int i = 16 * t + jj;
+    xlive[t] = i < p.rows;
+    xrow[t] = p.X + (int64_t)(xlive[t] ? i : 0) * p.ldx + 4 * kk;
+  }
+
+  f4 wv[2][CB], xv[2][MT];
+  auto fetch = [&](int k0, int buf) {
+    const bool in = k0 + 4 * kk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
+#pragma unroll
+    for (int q = 0; q < CB; q++) {
+      if (TW)
+        wv[buf][q] = in ? *reinterpret_cast<const f4*>(wrow[q] + k0) : zero;
+      else
+        wv[buf][q] = in ? *reinterpret_cast<const f4*>(wrow[q] + (int64_t)k0 * p.ldw) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++) xv[buf][t] = (in && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + k0) : zero;
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+#pragma unroll
+      for (int b = 0; b < CB; b++) {
+        // (k, cols) storage: block b = 4 h + c is component c of the load (s, h)
+        const float w = TW ? wv[buf][b][s] : wv[buf][4 * (b / 4) + s][b % 4];
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[buf][t][s], w, acc[t][b], 0, 0, 0);
+      }
+  };
+  if (kbeg < kend) {
+    fetch(kbeg, 0);
+    int k0 = kbeg;
+    for (; k0 + 32 < kend; k0 += 32) {
+      fetch(k0 + 16, 1);
+      multiply(0);
+      fetch(k0 + 32, 0);
+      multiply(1);
+    }
+    if (k0 + 16 < kend) {
+      fetch(k0 + 16, 1);
+      multiply(0);
+      multiply(1);
+    } else {
+      multiply(0);
+    }
+  }
+
+  // the four quarters of K meet in wavefront 0, in the order 1, 2, 3
+  for (int w = 1; w < kBlock / kWave; w++) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int b = 0; b < CB; b++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) meet[((t * CB + b) * 4 + r) * kWave + lane] = acc[t][b][r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int b = 0; b < CB; b++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) acc[t][b][r] += meet[((t * CB + b) * 4 + r) * kWave + lane];
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+  // D[4 (lane / 16) + r][lane % 16] of tile (t, b) in register r
+#pragma unroll
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int row = 16 * t + 4 * kk + r;
+      if (row >= p.rows) continue;
+#pragma unroll
+      for (int b = 0; b < CB; b++) {
+        const int64_t col = TW ? j0 + 16 * b + jj : j0 + 64 * (b / 4) + 4 * jj + b % 4;
+        if (col >= p.cols) continue;
+        if (p.gsplit == 1)
+          skinny_finish_store(p, row, col, acc[t][b][r]);
+        else
+          p.partial[((int64_t)ks * p.rows + row) * p.cols + col] = acc[t][b][r];
+      }
+    }
+}
+
+// the slices' planes added in the order 0, 1, ..., then alpha, beta, bias, activation, residual
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_finish(SkinnyParams p) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t plane = (int64_t)p.rows * p.cols;
+  if (e >= plane) return;
+  float acc = 0.0f;
+  for (uint32_t s = 0; s < p.gsplit; s++) acc += p.partial[(int64_t)s * plane + e];
+  const int row = (int)(e / p.cols);
+  skinny_finish_store(p, row, e - (int64_t)row * p.cols, acc);
+}
+
+static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; }
+
+// Row-major C (rows x cols) = act(alpha x . W + beta C + bias) + residual.  `w_is_cols_by_k`: W stored
+// (cols, k) with pitch ldw, else (k, cols).  Returns false (nothing launched) when the shape or the
+// alignment is not the kernel's; *rc holds the result of the launches otherwise.
+bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float alpha, const float* W, long ldw,
+                      const float* X, long ldx, float beta, float* C, long ldc, const float* bias,
+                      const float* residual, long ldres, int activation, int* rc) {
+  if (rows < 1 || rows > 64 || cols < 256 || k < 64 || k % 4 != 0 || k >= (1L << 30)) return false;
+  if (!aligned16(W) || !aligned16(X) || ldw % 4 != 0 || ldx % 4 != 0) return false;
+  if (!w_is_cols_by_k && cols % 4 != 0) return false;
+  SkinnyParams p;
+  p.W = W;
+  p.X = X;
+  p.C = C;
+  p.ldw = ldw;
+  p.ldx = ldx;
+  p.ldc = ldc;
+  p.rows = (int32_t)rows;
+  p.cols = cols;
+  p.k = (int32_t)k;
+  const int mt = rows <= 16 ? 1 : (rows <= 32 ? 2 : 4);
+  const int cb = 4;
+  p.cgroups = (uint32_t)ceil_div((int64_t)cols, (int64_t)(16 * cb));
+  // about four workgroups per compute unit, every wavefront at least four steps of 16
+  int64_t gsplit = (int64_t)rt().num_cus * 4 / p.cgroups;
+  if (gsplit > k / 256) gsplit = k / 256;
+  if (gsplit < 1) gsplit = 1;
+  p.kslice = (int32_t)(ceil_div(ceil_div((int64_t)k, gsplit), (int64_t)64) * 64);
+  gsplit = ceil_div((int64_t)k, (int64_t)p.kslice);
+  p.gsplit = (uint32_t)gsplit;
+  p.partial = nullptr;
+  p.alpha = alpha;
+  p.beta = beta;
+  p.bias = bias;
+  p.residual = residual;
+  p.ldres = ldres;
+  p.activation = activation;
+  const int64_t blocks = (int64_t)p.cgroups * gsplit;
+  if (blocks >= ((int64_t)1 << 31)) return false;
+  void* scratch = nullptr;
+  if (gsplit > 1) {
+    if (wf2hip_malloc_uninitialized(&scratch, (size_t)(gsplit * rows * cols) * sizeof(float)) != 0) return false;
+    p.partial = static_cast<float*>(scratch);
+  }
+  hipStream_t st = rt().stream;
+#define WF2_SKINNY(TW_)                                                                         \
+  do {                                                                                          \
+    if (mt == 1) sgemm_skinny_kernel<TW_, 1, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);        \
+    else if (mt == 2) sgemm_skinny_kernel<TW_, 2, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);   \
+    else sgemm_skinny_kernel<TW_, 4, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);                \
+  } while (0)
+  if (w_is_cols_by_k)
+    WF2_SKINNY(true);
+  else
+    WF2_SKINNY(false);
+#undef WF2_SKINNY
+  *rc = after_launch("sgemm_skinny_kernel");
+  if (*rc == 0 && gsplit > 1) {
+    sgemm_skinny_finish<<<(uint32_t)ceil_div((int64_t)rows * cols, (int64_t)kBlock), kBlock, 0, st>>>(p);
+    *rc = after_launch("sgemm_skinny_finish");
+  }
+  if (scratch) (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
+  return true;
+}
+
+}  // namespace wf2

@@ -641,3 +641,56 @@ def test_matmul_gelu_epilogue_edge_values(gpu):
     np.testing.assert_allclose(got[finite], truth[finite], rtol=4e-6, atol=1e-37)
     assert got[xs == np.inf][0] == np.inf and np.isnan(got[-1])
     assert got[xs == -np.inf][0] == 0.0 and got[list(xs).index(np.float32(-1e30))] == 0.0
+
+
+@pytest.mark.parametrize("rows", [1, 2, 7, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("cols,k", [(256, 64), (300, 100), (1000, 768), (5003, 260), (4096, 4100), (50257, 768)])
+def test_matmul_few_rows(gpu, rows, cols, k):
+    """At most 64 rows against a wide operand (a few tokens through a layer) take the kernel that reads the
+    wide operand once: both storages of it ((k, cols), and (cols, k) through !t), ragged column groups, K on
+    and off the slices and the 16-step, and the fused epilogue (bias, GELU, residual) on the same path."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows * 1000003 + cols * 7 + k)
+    X = rng.standard_normal((rows, k)).astype(np.float32)
+    Wkn = rng.standard_normal((k, cols)).astype(np.float32)
+    dX = F.from_numpy(X)
+    _gemm_check(F.matmul(dX, F.from_numpy(Wkn)).numpy(), X.astype(np.float64), Wkn.astype(np.float64))
+    dWt = F.from_numpy(np.ascontiguousarray(Wkn.T))
+    _gemm_check(F.matmul(dX, F.t(dWt)).numpy(), X.astype(np.float64), Wkn.astype(np.float64))
+    if cols <= 5003:
+        bias = rng.standard_normal(cols).astype(np.float32)
+        res = rng.standard_normal((rows, cols)).astype(np.float32)
+        z = X.astype(np.float64) @ Wkn.astype(np.float64) + bias
+        bound = REL * (np.abs(X.astype(np.float64)) @ np.abs(Wkn.astype(np.float64)) + np.abs(bias)) + 1e-30
+        got = F.linear(dX, F.from_numpy(Wkn), F.from_numpy(bias), residual=F.from_numpy(res)).numpy()
+        assert np.all(np.abs(got - (z + res)) <= bound + REL * np.abs(res))
+        got = F.linear(dX, F.from_numpy(Wkn), F.from_numpy(bias), activation="gelu").numpy()
+        gelu = 0.5 * z * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))
+        assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
+
+
+def test_sgemm_few_rows_column_major_contract(gpu):
+    """The same kernel through wf2hip_sgemm: column-major C (m x n, n <= 64) with padded leading dimensions,
+    alpha and beta, both storages of A; rows of padding stay untouched."""
+    W = gpu
+    lib = W.lib.get()
+    rng = np.random.default_rng(64)
+    for ca in "NT":
+        m, n, k = 1028, 5, 520
+        lda = (m if ca == "N" else k) + 4
+        ldb, ldc = k + 8, m + 3
+        A = rng.standard_normal(lda * (k if ca == "N" else m)).astype(np.float32)
+        B = rng.standard_normal(ldb * n).astype(np.float32)
+        Cm = rng.standard_normal(ldc * n).astype(np.float32)
+        A2 = A.reshape(-1, lda).T.astype(np.float64)
+        B2 = B.reshape(-1, ldb).T.astype(np.float64)
+        opA = A2[:m, :k] if ca == "N" else A2[:k, :m].T
+        opB = B2[:k, :n]
+        C2 = Cm.reshape(-1, ldc).T.astype(np.float64)
+        dA, dB, dC = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B), W.HIPTensor.from_numpy(Cm)
+        W.lib.check(lib.wf2hip_sgemm(ca.encode(), b"N", m, n, k, 0.5, dptr(dA), lda, dptr(dB), ldb, -2.0, dptr(dC), ldc))
+        got = dC.numpy().reshape(-1, ldc).T
+        want = 0.5 * opA @ opB - 2.0 * C2[:m, :n]
+        scale = 0.5 * np.abs(opA) @ np.abs(opB) + 2.0 * np.abs(C2[:m, :n])
+        assert np.max(np.abs(got[:m, :n] - want) / scale) < 1e-5
+        np.testing.assert_array_equal(got[m:, :], C2[m:, :].astype(np.float32))
