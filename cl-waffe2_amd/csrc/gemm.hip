@@ -832,12 +832,29 @@ struct Epilogue {
   int causal = 0;
 };
 
+// What the folds of a split-K run add after the sum (row-major terms, as the product's own epilogue):
+// act(sum + beta C + bias[col]) + residual[row][col]; the column-major element (i, j) is row j, column i.
+struct FoldEpilogue {
+  const float* bias;
+  const float* residual;
+  int64_t ldres;
+  int32_t activation;
+};
+
+__device__ __forceinline__ void fold_store(float* c, float acc, float beta, const FoldEpilogue& ep, int64_t i, int64_t j) {
+  float v = beta == 0.0f ? acc : beta * *c + acc;
+  if (ep.bias) v += ep.bias[i];
+  if (ep.activation == 1) v = gelu_tanh_fast(v);
+  if (ep.residual) v += ep.residual[j * ep.ldres + i];
+  *c = v;
+}
+
 // C[b] <- beta C[b] + sum over the `splits` partial products of a split-K run (column-major; the partial
 // of slice s and matrix b is the packed m x n plane s * batch + b, already scaled by alpha);
 // blockIdx.y is the matrix of the batch
 __global__ __launch_bounds__(kBlock) void splitk_fold(const float* __restrict__ partials, int splits, int64_t m,
                                                       int64_t n, float beta, float* __restrict__ C, int64_t ldc,
-                                                      int64_t strideC) {
+                                                      int64_t strideC, FoldEpilogue ep) {
   const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (e >= m * n) return;
   const int64_t j = e / m, i = e - j * m;
@@ -845,15 +862,14 @@ __global__ __launch_bounds__(kBlock) void splitk_fold(const float* __restrict__ 
   partials += (int64_t)blockIdx.y * plane;
   float acc = 0.0f;
   for (int s = 0; s < splits; s++) acc += partials[(int64_t)s * step + e];
-  float* c = C + (int64_t)blockIdx.y * strideC + i + j * ldc;
-  *c = beta == 0.0f ? acc : beta * *c + acc;
+  fold_store(C + (int64_t)blockIdx.y * strideC + i + j * ldc, acc, beta, ep, i, j);
 }
 
 // More than 16 partial products: a wavefront per output element, lane l adds slices l, l + 64, ...
 // in binary64 with eight loads in flight, the lanes meet by shuffles -- a fixed order.
 __global__ __launch_bounds__(kBlock) void splitk_fold_wide(const float* __restrict__ partials, int splits, int64_t m,
                                                            int64_t n, float beta, float* __restrict__ C, int64_t ldc,
-                                                           int64_t strideC) {
+                                                           int64_t strideC, FoldEpilogue ep) {
   const int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (e >= m * n) return;
   const int lane = threadIdx.x & (kWave - 1);
@@ -873,8 +889,7 @@ __global__ __launch_bounds__(kBlock) void splitk_fold_wide(const float* __restri
   for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
   if (lane == 0) {
     const int64_t j = e / m, i = e - j * m;
-    float* c = C + (int64_t)blockIdx.y * strideC + i + j * ldc;
-    *c = beta == 0.0f ? (float)acc : beta * *c + (float)acc;
+    fold_store(C + (int64_t)blockIdx.y * strideC + i + j * ldc, (float)acc, beta, ep, i, j);
   }
 }
 
@@ -894,7 +909,7 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
 // ((12, 3, 100000) . (12, 100000, 3)) is split the same way.
 static bool try_split_k(char transa, char transb, long m, long n, long k, float alpha, const float* A, long lda,
                         long strideA, const float* B, long ldb, long strideB, float beta, float* C, long ldc,
-                        long strideC, long batch, int* rc) {
+                        long strideC, long batch, const Epilogue& ep, int* rc) {
   static thread_local bool splitting = false;  // the slices themselves are not split again
   struct Guard {
     bool& flag;
@@ -903,19 +918,45 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
   };
   const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128) * batch;
   const int64_t cus = rt().num_cus;
-  if (splitting || k < 2048 || tiles >= cus || m < 1 || n < 1) return false;
+  if (splitting || tiles >= cus || m < 1 || n < 1) return false;
+  long splits = 0, kc = 0;
+  if (k < 2048) {
+    // A short K with few tiles (a few hundred rows through a layer: (256 x 768) . (768 x 2304) is 36 tiles
+    // of 48 steps each, one workgroup on a compute unit in seven): equal slices of at least 128 that bring
+    // the launch to about half the compute units -- more slices cost in the fold what they save ((256 x 768)
+    // . (768 x 2304) with its bias: 30.5 us whole, 22.6 us in 3 slices, 28.3 us in 6), and from a quarter
+    // of the compute units in tiles on the whole product is as fast ((512 x 768) . (768 x 2304): 31.9 / 33.5 us).
+    // Slices of at least 256 keep the streaming kernel; where those leave the launch below a quarter of the
+    // compute units, slices of at least 128 ((128 x 768) . (768 x 2304): 3 slices 19.6 us, 6 slices 16.6 us).
+    // Single products only (the layers of a model).
+    if (batch != 1 || k < 512 || tiles > cus / 4) return false;
+    const long want = (cus / 2 + tiles / 2) / tiles;
+    auto equal_slices = [&](long least) {
+      for (long cand = std::min<long>(want, k / least); cand >= 2; cand--)
+        if (k % (cand * 32) == 0) return cand;
+      return 0L;
+    };
+    splits = equal_slices(256);
+    if (splits * tiles < cus / 4) splits = equal_slices(128);
+    if (splits == 0) return false;
+    kc = k / splits;
+  }
   Guard guard(splitting);
   // Equal slices where K allows it.  Few output tiles and a very long K (the weight gradient of a layer
   // with few outputs: (10 x N) . (N x 256) over a batch of 65536 ran 150 us on 16 slices): as many slices
   // of at least 512 as keep the launch within four workgroups per compute unit.
-  long splits = 0, kc = 0;
-  if (batch == 1)
-    for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
-      if (k % ((long)cand * 32) == 0 && k / cand >= 512 && tiles * cand <= 4 * cus) {
-        splits = cand;
-        kc = k / cand;
-        break;
-      }
+  // (shorter slices, 256 and then 128, where those of 512 leave the launch below a quarter of the compute
+  // units: (96 x 3072) . (3072 x 768), 6 tiles: 36 us in 4 slices, 20 us in 24)
+  if (splits == 0 && batch == 1)
+    for (long least : {512L, 256L, 128L}) {
+      for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
+        if (k % ((long)cand * 32) == 0 && k / cand >= least && tiles * cand <= 4 * cus) {
+          splits = cand;
+          kc = k / cand;
+          break;
+        }
+      if (splits * tiles >= cus / 4) break;
+    }
   long rest = 0;  // length of a shorter last slice
   if (splits == 0) {
     // any K ((127 x 100000) . (100000 x 127) ran 5.9 ms as one product): slices of a multiple of 32, the
@@ -941,12 +982,13 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
     *rc = sgemm_batched2(transa, transb, m, n, rest, alpha, A + splits * sa, lda, strideA, 0, B + splits * sb, ldb,
                          strideB, 0, 0.0f, part + splits * batch * plane, m, (long)plane, 0, batch, 1);
   if (*rc == 0) {
+    const FoldEpilogue fe{ep.bias, ep.residual, ep.ldres, ep.activation};
     if (planes <= 16) {
       const dim3 grid((uint32_t)ceil_div(plane, (int64_t)kBlock), (uint32_t)batch);
-      splitk_fold<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC);
+      splitk_fold<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC, fe);
     } else {
       const dim3 grid((uint32_t)ceil_div(plane, (int64_t)(kBlock / kWave)), (uint32_t)batch);
-      splitk_fold_wide<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC);
+      splitk_fold_wide<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, strideC, fe);
     }
     *rc = after_launch("splitk_fold");
   }
@@ -1003,9 +1045,11 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
       return rc;
     }
   }
-  if (batch2 == 1 && batch <= 65535 && !ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
+  // (the fused epilogue of a single product goes into the fold; batches with one keep the plain route)
+  if (batch2 == 1 && batch <= 65535 && ep.causal == 0 && (batch == 1 || (!ep.bias && !ep.residual && ep.activation == 0))) {
     int rc = 0;
-    if (try_split_k(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, &rc))
+    if (try_split_k(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, ep,
+                    &rc))
       return rc;
   }
 

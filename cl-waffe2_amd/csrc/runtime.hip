@@ -13,6 +13,7 @@
 #include <string.h>
 #include <iterator>
 #include <unordered_map>
+#include <vector>
 
 #include "wf2_common.h"
 
@@ -66,6 +67,7 @@ struct Graph {
   std::multimap<size_t, void*> held;
 };
 static Graph* g_capture = nullptr;  // non-null between graph_begin and graph_end
+static std::vector<Graph*> g_destroy_after_capture;  // graphs released while another was being recorded (guarded by g_pool.mu)
 static std::unordered_map<void*, Graph*> g_graph_blocks;  // block -> the live graph recorded with it (guarded by g_pool.mu)
 
 struct Pool {
@@ -401,6 +403,14 @@ WF2_API int wf2hip_graph_end(void** graph) {
   }
   if (!g) return fail(WF2HIP_ECAPTURE, "no capture in progress");
   int rc = check_hip(hipStreamEndCapture(g_rt.stream, &g->graph), "hipStreamEndCapture");
+  {
+    std::vector<Graph*> waiting;
+    {
+      std::lock_guard<std::mutex> lock(g_pool.mu);
+      waiting.swap(g_destroy_after_capture);
+    }
+    for (Graph* old : waiting) (void)wf2hip_graph_destroy(old);
+  }
   if (rc == 0) rc = check_hip(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0),
                               "hipGraphInstantiate");
   if (rc != 0) {
@@ -422,6 +432,15 @@ WF2_API int wf2hip_graph_launch(void* graph) {
 WF2_API int wf2hip_graph_destroy(void* graph) {
   Graph* g = (Graph*)graph;
   if (!g) return 0;
+  {
+    // Destroying a graph synchronises the stream, which a capture in progress does not survive (a handle
+    // rebound inside a recording, `with Graph() as g:` over an older g): it waits for wf2hip_graph_end.
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    if (g_capture && g != g_capture) {
+      g_destroy_after_capture.push_back(g);
+      return 0;
+    }
+  }
   // replays still in flight read and write the held blocks
   if (g_rt.initialised) (void)hipStreamSynchronize(g_rt.stream);
   if (g->exec) (void)hipGraphExecDestroy(g->exec);

@@ -127,3 +127,27 @@ def test_block_dropped_after_the_capture_stays_with_the_graph(gpu):
     parked = W.lib.get().wf2hip_pool_idle_bytes()
     g.destroy()
     assert W.lib.get().wf2hip_pool_idle_bytes() >= parked + 4 * n  # the parked block is back
+
+
+def test_graph_released_during_a_recording(gpu):
+    """A graph handle rebound while the next graph is being recorded (`with Graph() as g:` over an older g)
+    releases the older graph inside the recording: its destruction waits for the end of the recording, and
+    the new graph records and replays as usual."""
+    W = gpu
+    F = W.functional
+    x = F.from_numpy(np.arange(4096, dtype=np.float32))
+
+    def run():
+        return F.exp(F.mul(x, 1.0 / 4096))
+
+    eager = run().numpy()
+    with W.lib.Graph() as g:
+        first = run()
+    g.launch()
+    assert_bit_equal(first.numpy(), eager, "first graph")
+    run()                          # the first graph keeps its blocks: the pool needs a set for the second
+    with W.lib.Graph() as g:       # the first graph loses its last reference here, inside the recording
+        second = run()
+    for i in range(2):
+        g.launch()
+        assert_bit_equal(second.numpy(), eager, f"second graph, replay {i}")

@@ -644,7 +644,7 @@ def test_matmul_gelu_epilogue_edge_values(gpu):
 
 
 @pytest.mark.parametrize("rows", [1, 2, 7, 16, 17, 32, 33, 64])
-@pytest.mark.parametrize("cols,k", [(256, 64), (300, 100), (1000, 768), (5003, 260), (4096, 4100), (50257, 768)])
+@pytest.mark.parametrize("cols,k", [(256, 64), (300, 100), (1000, 768), (5003, 260), (4096, 4100), (50257, 768), (8200, 4100)])
 def test_matmul_few_rows(gpu, rows, cols, k):
     """At most 64 rows against a wide operand (a few tokens through a layer) take the kernel that reads the
     wide operand once: both storages of it ((k, cols), and (cols, k) through !t), ragged column groups, K on
@@ -694,3 +694,28 @@ def test_sgemm_few_rows_column_major_contract(gpu):
         scale = 0.5 * np.abs(opA) @ np.abs(opB) + 2.0 * np.abs(C2[:m, :n])
         assert np.max(np.abs(got[:m, :n] - want) / scale) < 1e-5
         np.testing.assert_array_equal(got[m:, :], C2[m:, :].astype(np.float32))
+
+
+@pytest.mark.parametrize("rows,k,cols", [(96, 768, 2304), (256, 768, 768), (256, 3072, 768), (130, 1024, 1000),
+                                         (512, 800, 260), (300, 2080, 515)])
+def test_linear_of_a_few_hundred_rows(gpu, rows, k, cols):
+    """A layer applied to a few hundred rows: few output tiles over a K of several hundred, which runs as
+    slices of K whose fold applies the bias, the GELU and the residual -- against float64, and bit for bit
+    against the same product with its epilogue taken node for node (the fold adds what the nodes add)."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows + k + cols)
+    X = rng.standard_normal((rows, k)).astype(np.float32)
+    Wm = (rng.standard_normal((k, cols)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    res = rng.standard_normal((rows, cols)).astype(np.float32)
+    dX, dW, db, dr = F.from_numpy(X), F.from_numpy(Wm), F.from_numpy(bias), F.from_numpy(res)
+    z = X.astype(np.float64) @ Wm.astype(np.float64) + bias
+    bound = REL * (np.abs(X.astype(np.float64)) @ np.abs(Wm.astype(np.float64)) + np.abs(bias)) + 1e-30
+    plain = F.matmul(dX, dW)
+    _gemm_check(plain.numpy(), X.astype(np.float64), Wm.astype(np.float64))
+    got = F.linear(dX, dW, db, residual=dr).numpy()
+    assert np.all(np.abs(got - (z + res)) <= bound + REL * np.abs(res))
+    assert_bit_equal(got, F.add_(F.add_(plain, db), dr).numpy(), "bias and residual in the fold against the nodes")
+    got = F.linear(dX, dW, db, activation="gelu").numpy()
+    gelu = 0.5 * z * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))
+    assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
