@@ -239,6 +239,30 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tiny(RowRedParams p, FastD
   p.commit(p.a + (int64_t)(row0 + threadIdx.x) * p.oa[0], acc);
 }
 
+// Rows of exactly four floats, 16-byte aligned (2 x 2 pooling windows): the row is one vector load, four
+// rows per thread in flight, no LDS; the same sum in index order, in binary64.
+__global__ __launch_bounds__(kBlock) void reduce_rows_vec4(RowRedParams p) {
+  constexpr int U = 4;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4* src = reinterpret_cast<const f4*>(p.b);
+  const uint32_t first = blockIdx.x * (kBlock * U) + threadIdx.x;
+  f4 r[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t row = first + u * kBlock;
+    r[u] = row < p.nrows ? src[row] : f4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t row = first + u * kBlock;
+    if (row >= p.nrows) continue;
+    double acc = 0.0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc += (double)r[u][c];
+    p.commit(p.a + (int64_t)row * p.oa[0], acc);
+  }
+}
+
 // Folds the partial sums of a row in a fixed order.  This launch depends on the one
 // before it, so its own latency is all that counts: a thread issues its (up to 16)
 // loads together instead of one after the other (full sum of 2^25 elements: 25.0 ->
@@ -635,6 +659,10 @@ static int launch_row_reduce(const Space& s, float* a, const float* b, double* p
   hipStream_t st = rt().stream;
   const int64_t target_blocks = (int64_t)rt().num_cus * 8;
   if (p.n0 <= 32 && p.nouter == 1 && p.ob[0] == p.n0 && nrows >= 4 * target_blocks) {
+    if (p.n0 == 4 && aligned16(p.b)) {
+      reduce_rows_vec4<<<(uint32_t)ceil_div(nrows, (int64_t)kBlock * 4), kBlock, 0, st>>>(p);
+      return after_launch("reduce_rows_vec4");
+    }
     reduce_rows_tiny<<<(uint32_t)ceil_div(nrows, kBlock), kBlock, (size_t)kBlock * (p.n0 | 1) * sizeof(float), st>>>(
         p, make_fastdiv((uint32_t)p.n0));
     return after_launch("reduce_rows_tiny");

@@ -48,7 +48,9 @@ def test_select_tiny_rows(gpu, cols):
 
 
 @pytest.mark.parametrize("dtype,cols", [("double", 16), ("double", 17), ("int32", 7), ("uint8", 100), ("int16", 64),
-                                        ("uint32", 32), ("int8", 3)])
+                                        ("uint32", 32), ("int8", 3),
+                                        # rows of exactly 16 bytes: one vector load per row
+                                        ("double", 2), ("int32", 4), ("uint8", 16), ("int16", 8), ("uint32", 4)])
 def test_select_tiny_rows_typed(gpu, dtype, cols):
     W = gpu
     F = W.functional
