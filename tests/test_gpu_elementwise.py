@@ -645,3 +645,44 @@ def test_nodes_the_cpu_backend_leaves_to_lisptensor(gpu, O, op, lo, hi):
     ge = getattr(F, op)(F.from_numpy(edge)).numpy()
     assert ulp_distance(ge, te).max() <= limit, (edge, ge, te)
     assert np.array_equal(np.signbit(ge[~np.isnan(te)]), np.signbit(te[~np.isnan(te)]))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_permuted_and_sliced_passes(gpu, seed):
+    """Random ranks, extents (short, odd, just past a tile), axis orders and windows: copies out of and into
+    permuted views, an accumulating pass into a permuted destination and a unary pass over one, against
+    numpy's indexing.  Data movement and single roundings: bit-exact.  Whatever kernel the dispatcher picks
+    for the layout (rows, tiles, narrow tiles, strided gathers, an element per lane) must agree."""
+    F = gpu.functional
+    rng = np.random.default_rng(1000 + seed)
+    extents = [1, 2, 3, 5, 8, 13, 16, 17, 31, 32, 33, 64, 100, 257, 300, 513]
+    rank = int(rng.integers(2, 5))
+    while True:
+        shape = [int(rng.choice(extents)) for _ in range(rank)]
+        if np.prod(shape) <= 300000:
+            break
+    perm = tuple(int(p) for p in rng.permutation(rank))
+    x = rng.standard_normal(shape).astype(np.float32)
+    dx = F.from_numpy(x)
+    # a window on one axis (start past 0, so that the base pointer loses its alignment)
+    axis = int(rng.integers(0, rank))
+    lo = int(rng.integers(0, max(1, shape[axis] // 3) + 1)) if shape[axis] > 1 else 0
+    hi = shape[axis] - int(rng.integers(0, 2)) if shape[axis] - lo > 1 else shape[axis]
+    subs = [True] * rank
+    subs[axis] = (lo, hi)
+    index = tuple(slice(lo, hi) if a == axis else slice(None) for a in range(rank))
+    xv, dv = x[index], dx.view(*subs)
+    # copy out of a permuted window
+    assert_bit_equal(F.copy(dv.permute(*perm)).numpy(), xv.transpose(perm), f"copy {shape} {perm} axis {axis} [{lo}:{hi}]")
+    # unary pass over it
+    assert_bit_equal(F.abs(dv.permute(*perm)).numpy(), np.abs(xv.transpose(perm)), "abs")
+    # accumulate into the permuted window, then copy into it
+    y = rng.standard_normal(xv.transpose(perm).shape).astype(np.float32)
+    dy = F.from_numpy(y)
+    want = x.copy()
+    want[index] = xv + y.transpose(np.argsort(perm))
+    F.add_(dv.permute(*perm), dy)
+    assert_bit_equal(dx.numpy(), want, "accumulate into the permuted window")
+    want[index] = y.transpose(np.argsort(perm))
+    F.move_(dv.permute(*perm), dy)
+    assert_bit_equal(dx.numpy(), want, "copy into the permuted window")
