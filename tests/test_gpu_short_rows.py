@@ -298,3 +298,46 @@ def test_softmax_and_layernorm_of_tiny_rows(gpu, rows, cols):
     # the deviation x - mean is rounded in binary32: an absolute error of about 2^-24 |x| / std per element
     scale = np.abs(x64).max(axis=1, keepdims=True) / np.sqrt(var + 1e-5)
     assert np.all(np.abs(got - want) <= 4e-7 * scale * np.abs(g) + 2e-6 * np.abs(want) + 1e-6)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_sums_and_selections(gpu, seed):
+    """Random shapes (a few long axes, many short ones) and random kept / reduced axes: !sum, !mean, !max and
+    argmax against float64 / numpy, on :float and, for the sums, on :double and :int32 too.  Whatever kernel
+    the dispatcher picks (rows, tiny rows, columns, narrow columns, middle axes, pieces of long reductions)
+    must agree."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(5000 + seed)
+    extents = [1, 2, 3, 4, 7, 10, 32, 33, 64, 100, 128, 129, 1000, 4099, 20000, 70000]
+    rank = int(rng.integers(1, 5))
+    while True:
+        shape = [int(rng.choice(extents)) for _ in range(rank)]
+        if 1 <= np.prod(shape) <= 3000000:
+            break
+    x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    dx = F.from_numpy(x)
+    x64 = x.astype(np.float64)
+    naxes = int(rng.integers(1, rank + 1))
+    axes = tuple(sorted(int(a) for a in rng.choice(rank, naxes, replace=False)))
+    what = f"{shape} over {axes}"
+    got = F.sum(dx, axis=axes if len(axes) > 1 else axes[0]).numpy().reshape(-1)
+    want = x64.sum(axis=axes).reshape(-1)
+    bar = 2e-6 * np.abs(x64).sum(axis=axes).reshape(-1) + 1e-30
+    assert np.all(np.abs(got - want) <= bar), what
+    got = F.mean(dx, axis=axes if len(axes) > 1 else axes[0]).numpy().reshape(-1)
+    count = np.prod([shape[a] for a in axes])
+    assert np.all(np.abs(got - want / count) <= bar / count + 1e-30), what
+    # !max / !argmax reduce the trailing `t` axes as one run ((butlast (shape tensor) t) is kept)
+    t = int(rng.integers(1, rank + 1))
+    runs = x.reshape(shape[:rank - t] + [-1]) if t < rank else x.reshape(1, -1)
+    got_max = F.max(dx, axis=t).numpy().reshape(-1) if t < rank else F.max(F.reshape(dx, 1, -1)).numpy().reshape(-1)
+    assert_bit_equal(got_max, runs.max(axis=-1).reshape(-1), f"max of the trailing {t} axes, {what}")
+    got_arg = (F.argmax(dx, axis=t) if t < rank else F.argmax(F.reshape(dx, 1, -1))).numpy().reshape(-1).astype(np.int64)
+    np.testing.assert_array_equal(got_arg, runs.argmax(axis=-1).reshape(-1))   # the first maximum
+    xd = F.from_numpy(x64, dtype="double")
+    got = F.sum(xd, axis=axes if len(axes) > 1 else axes[0]).numpy().reshape(-1)
+    assert np.all(np.abs(got - want) <= 1e-13 * np.abs(x64).sum(axis=axes).reshape(-1) + 1e-300), what
+    xi = rng.integers(-2 ** 31, 2 ** 31, shape).astype(np.int32)
+    got = F.sum(F.from_numpy(xi, dtype="int32"), axis=axes if len(axes) > 1 else axes[0]).numpy().reshape(-1)
+    np.testing.assert_array_equal(got, xi.astype(np.int64).sum(axis=axes).astype(np.int32).reshape(-1))
