@@ -719,3 +719,37 @@ def test_linear_of_a_few_hundred_rows(gpu, rows, k, cols):
     got = F.linear(dX, dW, db, activation="gelu").numpy()
     gelu = 0.5 * z * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))
     assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_matmul_random_shapes_and_layouts(gpu, seed):
+    """Random extents (1, a few, just past a tile, hundreds, thousands), transposes, an optional batch and an
+    optional fused epilogue: whatever route the product takes (tiles, slices of K with the fold, the
+    few-rows kernel, batches) is held to the same bound against float64."""
+    F = gpu.functional
+    rng = np.random.default_rng(9000 + seed)
+    mn = [1, 2, 7, 16, 33, 64, 65, 128, 200, 256, 300, 1000, 2304]
+    ks = [1, 4, 17, 64, 100, 256, 768, 1024, 2049, 3072, 5000]
+    while True:
+        m, n, k = int(rng.choice(mn)), int(rng.choice(mn)), int(rng.choice(ks))
+        batch = int(rng.choice([0, 0, 1, 3]))
+        if 2.0 * m * n * k * max(batch, 1) <= 3e9:
+            break
+    ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    lead = (batch,) if batch else ()
+    A = rng.standard_normal(lead + (m, k)).astype(np.float32)
+    B = rng.standard_normal(lead + (k, n)).astype(np.float32)
+    swap = lambda a: np.ascontiguousarray(np.swapaxes(a, -1, -2))  # noqa: E731
+    dA = F.t(F.from_numpy(swap(A))) if ta else F.from_numpy(A)
+    dB = F.t(F.from_numpy(swap(B))) if tb else F.from_numpy(B)
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    want = A64 @ B64
+    bound = REL * (np.abs(A64) @ np.abs(B64)) + 1e-30
+    got = F.matmul(dA, dB).numpy()
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= bound), (m, n, k, batch, ta, tb, float(np.max(np.abs(got - want) / bound)))
+    if not batch:
+        bias = rng.standard_normal(n).astype(np.float32)
+        res = rng.standard_normal((m, n)).astype(np.float32)
+        got = F.matmul(dA, dB, bias=F.from_numpy(bias), residual=F.from_numpy(res)).numpy()
+        assert np.all(np.abs(got - (want + bias + res)) <= bound + REL * (np.abs(bias) + np.abs(res))), (m, n, k, ta, tb)
