@@ -358,8 +358,97 @@ static int dispatch_1d(int op, int64_t n, T* x, int64_t incx, const T* y, int64_
   }
 }
 
+// Transposing passes: dst has stride 1 along its last axis I, src along another axis J.  A 64 x 64 tile is
+// read with lanes running along J, parked in LDS (pitch 65) and written with lanes running along I: both
+// sides in whole lines, where an element per lane leaves one of them at a stride ((8192, 8192) transposed:
+// :double 414 us, :int32 329 us, :uint8 272 us).
+struct TypedTile {
+  int64_t ni, nj, d_j, s_i;  // extents of I and J, dst stride along J, src stride along I
+  uint32_t tiles_i, tiles_j;
+  int32_t nouter;
+  uint32_t oshape[WF2HIP_MAX_RANK];
+  int64_t odst[WF2HIP_MAX_RANK], osrc[WF2HIP_MAX_RANK];
+};
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void typed_tile(T* dst, const T* src, TypedTile p) {
+  constexpr int kEdge = 64;
+  __shared__ T tile[kEdge][kEdge + 1];
+  uint32_t rem = blockIdx.x / p.tiles_i;
+  const int64_t i0 = (int64_t)(blockIdx.x - rem * p.tiles_i) * kEdge;
+  const uint32_t tj = rem % p.tiles_j;
+  rem /= p.tiles_j;
+  const int64_t j0 = (int64_t)tj * kEdge;
+  int64_t doff = 0, soff = 0;
+  for (int i = 0; i < p.nouter; i++) {
+    const uint32_t q = rem / p.oshape[i];
+    const uint32_t idx = rem - q * p.oshape[i];
+    rem = q;
+    doff += (int64_t)idx * p.odst[i];
+    soff += (int64_t)idx * p.osrc[i];
+  }
+  const int tx = threadIdx.x & (kEdge - 1), ty = threadIdx.x / kEdge;
+  constexpr int kRows = kBlock / kEdge;  // rows of the tile per pass
+  {
+    T v[kEdge / kRows];
+#pragma unroll
+    for (int q = 0; q < kEdge / kRows; q++) {
+      const int64_t i = i0 + ty + q * kRows, j = j0 + tx;
+      v[q] = (i < p.ni && j < p.nj) ? src[soff + i * p.s_i + j] : T(0);
+    }
+#pragma unroll
+    for (int q = 0; q < kEdge / kRows; q++) tile[ty + q * kRows][tx] = v[q];
+  }
+  __syncthreads();
+  T old[kEdge / kRows];
+#pragma unroll
+  for (int q = 0; q < kEdge / kRows; q++) {
+    const int64_t i = i0 + tx, j = j0 + ty + q * kRows;
+    old[q] = (OP != WF2HIP_MOVE && i < p.ni && j < p.nj) ? dst[doff + j * p.d_j + i] : T(0);
+  }
+#pragma unroll
+  for (int q = 0; q < kEdge / kRows; q++) {
+    const int64_t i = i0 + tx, j = j0 + ty + q * kRows;
+    if (i < p.ni && j < p.nj) dst[doff + j * p.d_j + i] = apply<T, OP>(old[q], tile[tx][ty + q * kRows]);
+  }
+}
+
+template <class T, int OP>
+static bool try_typed_tile(const Space& s, T* a, const T* b, int* rc) {
+  const int last = s.rank - 1;
+  if (s.rank < 2 || s.sa[last] != 1 || s.sb[last] <= 1) return false;
+  int J = -1;
+  for (int r = 0; r < last; r++)
+    if (s.sb[r] == 1 && s.sa[r] > 0) J = r;
+  if (J < 0 || s.shape[last] < 16 || s.shape[J] < 16) return false;
+  TypedTile p;
+  p.ni = s.shape[last];
+  p.nj = s.shape[J];
+  p.d_j = s.sa[J];
+  p.s_i = s.sb[last];
+  p.tiles_i = (uint32_t)ceil_div(p.ni, (int64_t)64);
+  p.tiles_j = (uint32_t)ceil_div(p.nj, (int64_t)64);
+  p.nouter = 0;
+  int64_t blocks = (int64_t)p.tiles_i * p.tiles_j;
+  for (int r = last - 1; r >= 0; r--) {
+    if (r == J) continue;
+    if (s.shape[r] >= ((int64_t)1 << 32)) return false;
+    p.oshape[p.nouter] = (uint32_t)s.shape[r];
+    p.odst[p.nouter] = s.sa[r];
+    p.osrc[p.nouter] = s.sb[r];
+    p.nouter++;
+    blocks *= s.shape[r];
+  }
+  if (blocks >= ((int64_t)1 << 31)) return false;
+  typed_tile<T, OP><<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
+  *rc = after_launch("typed_tile");
+  return true;
+}
+
 template <class T, int OP>
 static int run_generic(const Space& s, T* a, const T* b) {
+  int rc = 0;
+  if (try_typed_tile<T, OP>(s, a, b, &rc)) return rc;
   TypedGen p;
   p.rank = s.rank;
   p.total = s.total;

@@ -238,3 +238,51 @@ def test_1d_entry_refuses_overlapping_runs(gpu, dtype):
     assert np.all(dx.numpy() == 7)
     W.lib.check(lib.wf2hip_binary_1d_typed(code, W.lib.ADD, n, C.c_void_p(dx.ptr), 1, C.c_void_p(dx.ptr), 1))
     assert np.all(dx.numpy() == 14)
+
+
+@pytest.mark.parametrize("dtype", ["double", "int32", "uint32", "int16", "uint16", "int8", "uint8"])
+@pytest.mark.parametrize("seed", range(6))
+def test_typed_random_permuted_passes(gpu, dtype, seed):
+    """Copies out of and into permuted windows and accumulating passes over them on every element type, random
+    ranks, extents and axis orders: the tiled transposing kernel and the element-per-lane kernel against
+    numpy's indexing (integer sums wrap, as the reference's C loops do); bit-exact."""
+    F = gpu.functional
+    np_dtype = {"double": np.float64, "int32": np.int32, "uint32": np.uint32, "int16": np.int16, "uint16": np.uint16,
+                "int8": np.int8, "uint8": np.uint8}[dtype]
+    rng = np.random.default_rng(77 * seed + len(dtype))
+    extents = [1, 2, 3, 15, 16, 17, 63, 64, 65, 100, 257, 300]
+    rank = int(rng.integers(2, 5))
+    while True:
+        shape = [int(rng.choice(extents)) for _ in range(rank)]
+        if np.prod(shape) <= 300000:
+            break
+    perm = tuple(int(p) for p in rng.permutation(rank))
+
+    def draw(sh):
+        if dtype == "double":
+            return rng.standard_normal(sh)
+        info = np.iinfo(np_dtype)
+        return rng.integers(info.min, int(info.max) + 1, sh).astype(np_dtype)
+
+    x = draw(shape)
+    dx = F.from_numpy(x, dtype=dtype)
+    axis = int(rng.integers(0, rank))
+    lo = 1 if shape[axis] > 2 else 0
+    subs = [True] * rank
+    subs[axis] = (lo, shape[axis])
+    index = tuple(slice(lo, None) if a == axis else slice(None) for a in range(rank))
+    xv, dv = x[index], dx.view(*subs)
+    what = f"{dtype} {shape} {perm} axis {axis} from {lo}"
+    np.testing.assert_array_equal(F.copy(dv.permute(*perm)).numpy(), xv.transpose(perm), err_msg="copy " + what)
+    y = draw(xv.transpose(perm).shape)
+    dy = F.from_numpy(y, dtype=dtype)
+    back = np.argsort(perm)
+    want = x.copy()
+    with np.errstate(over="ignore"):
+        want[index] = xv + y.transpose(back)
+    F.add_(dv.permute(*perm), dy)
+    np.testing.assert_array_equal(dx.numpy(), want, err_msg="accumulate into the permuted window, " + what)
+    with np.errstate(over="ignore"):
+        want2 = y - want[index].transpose(perm)
+    F.sub_(dy, dv.permute(*perm))
+    np.testing.assert_array_equal(dy.numpy(), want2, err_msg="subtract a permuted window, " + what)
