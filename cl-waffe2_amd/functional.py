@@ -69,9 +69,9 @@ def reshape(x: HIPTensor, *shape: int) -> HIPTensor:
     -1."""
     shape = list(shape)
     if shape.count(-1) == 1:
-        known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+        known = math.prod(s for s in shape if s != -1)
         shape[shape.index(-1)] = x.size // _builtins.max(known, 1)
-    if int(np.prod(shape, dtype=np.int64)) != x.size:
+    if math.prod(shape) != x.size:
         raise ValueError(f"reshape: cannot reshape {x.shape} into {shape}")
     src = to_contiguous(x)
     return HIPTensor(shape, vec=src.vec, dtype=src.dtype)

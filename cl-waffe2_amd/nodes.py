@@ -106,10 +106,10 @@ def _only_float(dtype) -> bool:
 
 
 def view2(a: HIPTensor, b: HIPTensor) -> _lib.View2:
-    sa, sta, oa = a.geometry()
-    sb, stb, ob = b.geometry()
+    sa, sta, oa = a._geom()
+    sb, stb, ob = b._geom()
     if sa != sb:
-        raise ValueError(f"shape mismatch: {sa} and {sb} (the node's :where is A[~] B[~] -> A[~])")
+        raise ValueError(f"shape mismatch: {list(sa)} and {list(sb)} (the node's :where is A[~] B[~] -> A[~])")
     v = _lib.View2()
     v.rank = len(sa)
     for r, (n, x, y) in enumerate(zip(sa, sta, stb)):

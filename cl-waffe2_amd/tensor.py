@@ -23,6 +23,8 @@ import ctypes as C
 from dataclasses import dataclass
 from typing import Sequence
 
+import math
+
 import numpy as np
 
 from . import lib as _lib
@@ -131,6 +133,9 @@ DTYPES = {"float": np.float32, "double": np.float64, "int32": np.int32, "uint32"
           "int16": np.int16, "uint16": np.uint16, "int8": np.int8, "uint8": np.uint8}
 
 
+ITEMSIZE = {name: np.dtype(t).itemsize for name, t in DTYPES.items()}
+
+
 class HIPTensor:
     """A tensor on the GPU, possibly a view of another one's storage.  Every node
     of the path runs on :float; the other dtypes have the arithmetic / move
@@ -142,7 +147,7 @@ class HIPTensor:
         if dtype not in DTYPES:
             raise ValueError(f"HIPTensor has no dtype {dtype}; known: {sorted(DTYPES)}")
         self.dtype = dtype
-        self.itemsize = np.dtype(DTYPES[dtype]).itemsize
+        self.itemsize = ITEMSIZE[dtype]
         self.orig_shape = [int(s) for s in shape]
         if len(self.orig_shape) < 1 or len(self.orig_shape) > _lib.MAX_RANK:
             raise ValueError(f"HIPTensor rank must be 1..{_lib.MAX_RANK}")
@@ -152,8 +157,10 @@ class HIPTensor:
         self.views = list(views) if views is not None else [
             Subscript(True, False, make_range(0, s)) for s in self.orig_shape]
         self.initial_offset = int(offset)
+        self._geometry = None  # (shape, strides, offset), computed once: a tensor's views never change
+        self._contiguous = None
         if vec is None:
-            n = int(np.prod(self.orig_shape, dtype=np.int64))
+            n = math.prod(self.orig_shape)
             # initial_element None = an InputTensor temporary (make-input): its
             # first use overwrites it, so it is not zero-filled
             vec = DeviceBuffer(self.itemsize * n, zero=initial_element is not None and initial_element == 0)
@@ -170,7 +177,7 @@ class HIPTensor:
     @property
     def shape(self) -> list[int]:
         """Visible shape (``compute-visible-shape``, ``view.lisp:216-221``)."""
-        return [v.repeat if v.broadcast else v.range.size for v in self.views]
+        return list(self._geom()[0])
 
     @property
     def ndim(self) -> int:
@@ -178,29 +185,40 @@ class HIPTensor:
 
     @property
     def size(self) -> int:
-        return int(np.prod(self.shape, dtype=np.int64))
+        n = 1
+        for extent in self._geom()[0]:
+            n *= extent
+        return n
 
     def geometry(self):
         """(shape, effective strides, start offset) in elements: what
         call-with-view computes per axis as stride x step and
         initial-offset + stride x range-nth(view, 0)
         (``call-with-view.lisp:120-137,168-195``)."""
-        shape, strides, off = [], [], self.initial_offset
-        for v, st in zip(self.views, self.stride):
-            if v.broadcast:
-                shape.append(v.repeat)
-                strides.append(0)
-                off += st * v.range.nth(0)
-            else:
-                shape.append(v.range.size)
-                strides.append(st * (v.range.nth(1) - v.range.nth(0)))
-                off += st * v.range.nth(0)
-        return shape, strides, off
+        shape, strides, off = self._geom()
+        return list(shape), list(strides), off
+
+    def _geom(self):
+        if self._geometry is None:
+            shape, strides, off = [], [], self.initial_offset
+            for v, st in zip(self.views, self.stride):
+                if v.broadcast:
+                    shape.append(v.repeat)
+                    strides.append(0)
+                    off += st * v.range.nth(0)
+                else:
+                    shape.append(v.range.size)
+                    strides.append(st * (v.range.nth(1) - v.range.nth(0)))
+                    off += st * v.range.nth(0)
+            self._geometry = (tuple(shape), tuple(strides), off)
+        return self._geometry
 
     def is_contiguous(self) -> bool:
-        shape, strides, off = self.geometry()
-        return off == 0 and strides == column_major_strides(shape) and \
-            int(np.prod(shape, dtype=np.int64)) * self.itemsize == self.vec.nbytes
+        if self._contiguous is None:
+            shape, strides, off = self._geom()
+            self._contiguous = off == 0 and list(strides) == column_major_strides(shape) and \
+                math.prod(shape) * self.itemsize == self.vec.nbytes
+        return self._contiguous
 
     @property
     def ptr(self) -> int:
