@@ -154,10 +154,11 @@ class HIPTensor:
         if any(s < 0 for s in self.orig_shape):
             raise ValueError("negative extent")
         self.stride = list(strides) if strides is not None else column_major_strides(self.orig_shape)
-        self.views = list(views) if views is not None else [
-            Subscript(True, False, make_range(0, s)) for s in self.orig_shape]
+        # full views are built on first use: most tensors are temporaries that are never viewed
+        self._views = list(views) if views is not None else None
         self.initial_offset = int(offset)
-        self._geometry = None  # (shape, strides, offset), computed once: a tensor's views never change
+        # (shape, strides, offset), computed once: a tensor's views never change
+        self._geometry = None if views is not None else (tuple(self.orig_shape), tuple(self.stride), self.initial_offset)
         self._contiguous = None
         if vec is None:
             n = math.prod(self.orig_shape)
@@ -180,8 +181,14 @@ class HIPTensor:
         return list(self._geom()[0])
 
     @property
+    def views(self) -> list:
+        if self._views is None:
+            self._views = [Subscript(True, False, make_range(0, s)) for s in self.orig_shape]
+        return self._views
+
+    @property
     def ndim(self) -> int:
-        return len(self.views)
+        return len(self.orig_shape)
 
     @property
     def size(self) -> int:
