@@ -902,6 +902,8 @@ int binary_nd(int op, Space s, float* a, const float* b);  // elementwise.hip
 bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float alpha, const float* W, long ldw,
                       const float* X, long ldx, float beta, float* C, long ldc, const float* bias,
                       const float* residual, long ldres, int activation, int* rc);  // gemm_skinny.hip
+bool try_sgemm_tiny_out(long rows, long cols, long k, float alpha, const float* L, long ldl, const float* R, long ldr,
+                        float** partial, long* planes, int* rc);  // gemm_skinny.hip
 
 // Products with few output tiles and a long K (weight gradients: 768 x 3072 outputs over K = 8192 are
 // 144 tiles for 256 compute units) run as `splits` products over slices of K, the slices as the outer
@@ -1020,6 +1022,23 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
     if (try_sgemm_skinny(!is_n(transa), n, m, k, alpha, A, lda, B, ldb, beta, C, ldc, ep.bias, ep.residual, ep.ldres,
                          ep.activation, &rc))
       return rc;
+  }
+  // a small output over a long K with both operands stored K-major (the weight gradient of a convolution
+  // with few channels): partial planes by slices of K, folded like the split-K planes
+  if (batch == 1 && batch2 == 1 && is_n(transa) && !is_n(transb) && ep.causal == 0) {
+    int rc = 0;
+    float* part = nullptr;
+    long planes = 0;
+    if (try_sgemm_tiny_out(n, m, k, alpha, B, ldb, A, lda, &part, &planes, &rc)) {
+      if (rc == 0) {
+        const FoldEpilogue fe{ep.bias, ep.residual, ep.ldres, ep.activation};
+        const dim3 grid((uint32_t)ceil_div((int64_t)m * n, (int64_t)(kBlock / kWave)), 1);
+        splitk_fold_wide<<<grid, kBlock, 0, rt().stream>>>(part, (int)planes, m, n, beta, C, ldc, 0, fe);
+        rc = after_launch("splitk_fold");
+      }
+      (void)wf2hip_free(part);  // stream order keeps it alive for the launches above
+      return rc;
+    }
   }
   // x^T . dY (weight gradients): the left operand of the row-major product arrives stored
   // (k, rows), which only the register-staged kernel reads.  One transposing pass over it

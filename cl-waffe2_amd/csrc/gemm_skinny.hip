@@ -18,7 +18,10 @@
 // The four wavefronts of a workgroup take a quarter of the workgroup's slice of K each and meet in LDS;
 // with several slices of K over the grid each writes a plane of its own and skinny_finish adds the planes
 // in a fixed order.  alpha, beta, bias, activation and residual are applied once, at the end.
+#include <algorithm>
+
 #include "wf2_common.h"
+#include "wf2_fastdiv.h"
 #include "wf2_math.h"
 
 namespace wf2 {
@@ -261,6 +264,109 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
     *rc = after_launch("sgemm_skinny_finish");
   }
   if (scratch) (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
+  return true;
+}
+
+// ---- a small output over a long K, both operands stored K-major -----------------------------------------
+// out (rows x cols) = sum over k of L[k][i] R[k][j] with rows x cols <= 512 and thousands of k: the weight
+// gradient of a convolution with few channels (dY^T . col: (N h w, O)^T . (N h w, C kh kw); the first layer of
+// the MNIST example is 4 x 9 outputs over K = 173056).  The tiled kernel spends a 128 x 128 tile's work per
+// slice of K on them (240 us for 5 MFLOP).  Here the grid splits K; a workgroup stages 64 rows of L and of R at
+// a time into LDS (both are contiguous runs when the rows are adjacent), thread t owns outputs t and t + 256
+// in registers, and every workgroup leaves a plane of partial sums that the split-K fold adds in a
+// fixed order.
+struct TinyOutParams {
+  const float* L;  // (k, rows), pitch ldl
+  const float* R;  // (k, cols), pitch ldr
+  int64_t ldl, ldr, k, kslice;
+  int32_t rows, cols, chunk;  // chunk: rows of K per LDS stage
+  float alpha;
+  float* partial;  // gridDim.x planes of rows x cols, row-major
+};
+
+template <int U>
+__global__ __launch_bounds__(kBlock) void sgemm_tiny_out_kernel(TinyOutParams p, FastDiv by_rows, FastDiv by_cols) {
+  extern __shared__ float stage[];
+  float* ls = stage;                            // chunk x rows
+  float* rs = stage + (size_t)p.chunk * p.rows;  // chunk x cols
+  const int64_t kbeg = (int64_t)blockIdx.x * p.kslice;
+  const int64_t kend = kbeg + p.kslice < p.k ? kbeg + p.kslice : p.k;
+  const uint32_t outputs = (uint32_t)p.rows * (uint32_t)p.cols;
+  uint32_t li[U], rj[U];
+  float acc[U];
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t o = threadIdx.x + u * kBlock;
+    uint32_t j;
+    const uint32_t i = fd_divmod(o < outputs ? o : 0u, by_cols, &j);
+    li[u] = i;
+    rj[u] = j;
+    acc[u] = 0.0f;
+  }
+  for (int64_t k0 = kbeg; k0 < kend; k0 += p.chunk) {
+    const uint32_t live = (uint32_t)(kend - k0 < p.chunk ? kend - k0 : p.chunk);
+    __syncthreads();  // the previous stage has been read
+    for (uint32_t e = threadIdx.x; e < live * (uint32_t)p.rows; e += kBlock) {
+      uint32_t i;
+      const uint32_t kk = fd_divmod(e, by_rows, &i);
+      ls[e] = p.L[(k0 + kk) * p.ldl + i];
+    }
+    for (uint32_t e = threadIdx.x; e < live * (uint32_t)p.cols; e += kBlock) {
+      uint32_t j;
+      const uint32_t kk = fd_divmod(e, by_cols, &j);
+      rs[e] = p.R[(k0 + kk) * p.ldr + j];
+    }
+    __syncthreads();
+    for (uint32_t kk = 0; kk < live; kk++) {
+      const float* lrow = ls + kk * p.rows;
+      const float* rrow = rs + kk * p.cols;
+#pragma unroll
+      for (int u = 0; u < U; u++) acc[u] = __builtin_fmaf(lrow[li[u]], rrow[rj[u]], acc[u]);
+    }
+  }
+  float* plane = p.partial + (size_t)blockIdx.x * outputs;
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t o = threadIdx.x + u * kBlock;
+    if (o < outputs) plane[o] = p.alpha * acc[u];
+  }
+}
+
+// Returns false (nothing launched) when the shape is not the kernel's.  On success *planes partial planes
+// of rows x cols (row-major, scaled by alpha) lie at *partial (pool memory, to be folded and freed by the
+// caller).
+bool try_sgemm_tiny_out(long rows, long cols, long k, float alpha, const float* L, long ldl, const float* R, long ldr,
+                        float** partial, long* planes, int* rc) {
+  // up to two outputs per thread: with more, the two LDS reads per multiply-add cost more than the tiled
+  // kernel's padding ((32 x 75) outputs over K = 65536: 257 us here, 160 us tiled)
+  if (rows < 1 || cols < 1 || rows * cols > 2 * kBlock || rows + cols > 192 || k < 8192) return false;
+  TinyOutParams p;
+  p.L = L;
+  p.R = R;
+  p.ldl = ldl;
+  p.ldr = ldr;
+  p.k = k;
+  p.rows = (int32_t)rows;
+  p.cols = (int32_t)cols;
+  p.chunk = 64;
+  p.alpha = alpha;
+  // about four workgroups per compute unit, each at least four stages
+  int64_t groups = std::min<int64_t>((int64_t)rt().num_cus * 4, k / (4 * p.chunk));
+  if (groups < 1) groups = 1;
+  p.kslice = ceil_div(ceil_div((int64_t)k, groups), (int64_t)p.chunk) * p.chunk;
+  groups = ceil_div((int64_t)k, p.kslice);
+  void* scratch = nullptr;
+  if (wf2hip_malloc_uninitialized(&scratch, (size_t)(groups * rows * cols) * sizeof(float)) != 0) return false;
+  p.partial = static_cast<float*>(scratch);
+  const size_t lds = (size_t)p.chunk * (rows + cols) * sizeof(float);
+  const FastDiv by_rows = make_fastdiv((uint32_t)rows), by_cols = make_fastdiv((uint32_t)cols);
+  hipStream_t st = rt().stream;
+  const int per_thread = (int)ceil_div((int64_t)rows * cols, (int64_t)kBlock);
+  if (per_thread <= 1) sgemm_tiny_out_kernel<1><<<(uint32_t)groups, kBlock, lds, st>>>(p, by_rows, by_cols);
+  else sgemm_tiny_out_kernel<2><<<(uint32_t)groups, kBlock, lds, st>>>(p, by_rows, by_cols);
+  *rc = after_launch("sgemm_tiny_out_kernel");
+  *partial = p.partial;
+  *planes = (long)groups;
   return true;
 }
 

@@ -753,3 +753,35 @@ def test_matmul_random_shapes_and_layouts(gpu, seed):
         res = rng.standard_normal((m, n)).astype(np.float32)
         got = F.matmul(dA, dB, bias=F.from_numpy(bias), residual=F.from_numpy(res)).numpy()
         assert np.all(np.abs(got - (want + bias + res)) <= bound + REL * (np.abs(bias) + np.abs(res))), (m, n, k, ta, tb)
+
+
+@pytest.mark.parametrize("rows,cols,k", [(4, 9, 173056), (16, 100, 43264), (1, 1, 8192), (64, 64, 9000), (7, 73, 8200), (2, 190, 9000),
+                                         (3, 3, 100001)])
+def test_matmul_small_output_long_k_both_k_major(gpu, rows, cols, k):
+    """x^T . y with x (k, rows) and y (k, cols): a small output over a long K with both operands stored K-major
+    (the weight gradient of a convolution with few channels) -- workgroups over slices of K, outputs in
+    registers, planes folded in a fixed order; also with alpha, beta and padded leading dimensions through
+    wf2hip_sgemm."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(rows + cols + k)
+    X = rng.standard_normal((k, rows)).astype(np.float32)
+    Y = rng.standard_normal((k, cols)).astype(np.float32)
+    got = F.matmul(F.t(F.from_numpy(X)), F.from_numpy(Y)).numpy()
+    _gemm_check(got, X.T.astype(np.float64), Y.astype(np.float64))
+    # column-major: C (cols x rows, ldc padded) <- 0.5 A B^T - 2 C with A (cols x k, lda) and B (rows x k, ldb)
+    lib = W.lib.get()
+    lda, ldb, ldc = cols + 3, rows + 2, cols + 1
+    A = rng.standard_normal(lda * k).astype(np.float32)
+    B = rng.standard_normal(ldb * k).astype(np.float32)
+    Cm = rng.standard_normal(ldc * rows).astype(np.float32)
+    A2 = A.reshape(k, lda).T.astype(np.float64)[:cols]       # cols x k
+    B2 = B.reshape(k, ldb).T.astype(np.float64)[:rows]       # rows x k
+    C2 = Cm.reshape(rows, ldc).T.astype(np.float64)
+    dA, dB, dC = W.HIPTensor.from_numpy(A), W.HIPTensor.from_numpy(B), W.HIPTensor.from_numpy(Cm)
+    W.lib.check(lib.wf2hip_sgemm(b"N", b"T", cols, rows, k, 0.5, dptr(dA), lda, dptr(dB), ldb, -2.0, dptr(dC), ldc))
+    got = dC.numpy().reshape(rows, ldc).T
+    want = 0.5 * A2 @ B2.T - 2.0 * C2[:cols]
+    scale = 0.5 * np.abs(A2) @ np.abs(B2.T) + 2.0 * np.abs(C2[:cols])
+    assert np.max(np.abs(got[:cols] - want) / scale) < 1e-5
+    np.testing.assert_array_equal(got[cols:], C2[cols:].astype(np.float32))
