@@ -949,14 +949,24 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
   // of at least 512 as keep the launch within four workgroups per compute unit.
   // (shorter slices, 256 and then 128, where those of 512 leave the launch below a quarter of the compute
   // units: (96 x 3072) . (3072 x 768), 6 tiles: 36 us in 4 slices, 20 us in 24)
+  // Where the powers of two leave most compute units idle, any count of equal slices will do: the weight
+  // gradient of a convolution over K = 43264 = 2^8 13^2 (one tile) ran as 8 slices, 106 us; 52 divide it too.
   if (splits == 0 && batch == 1)
     for (long least : {512L, 256L, 128L}) {
       for (int cand : {1024, 512, 256, 128, 64, 32, 16, 8, 4, 2})
         if (k % ((long)cand * 32) == 0 && k / cand >= least && tiles * cand <= 4 * cus) {
           splits = cand;
-          kc = k / cand;
           break;
         }
+      if (splits * tiles < cus / 2) {
+        const long most = std::min<long>(std::min<long>(k / least, (long)(4 * cus / tiles)), 1024);
+        for (long cand = most; cand > splits && cand >= 2; cand--)
+          if (k % (cand * 32) == 0) {
+            splits = cand;
+            break;
+          }
+      }
+      if (splits) kc = k / splits;
       if (splits * tiles >= cus / 4) break;
     }
   long rest = 0;  // length of a shorter last slice
