@@ -613,6 +613,24 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     measure(f"matmul {m}x{n}x{k}, left operand stored ({k},{m}) (!t), split over K", ring,
             lambda s: F.matmul(F.t(s[0]), s[1], out=s[2]), 2.0 * m * n * k, bound="mfma")
     del a0, b0
+    # a few rows against a wide operand (a few tokens through a layer): one read of that operand, bound by HBM
+    for m, n, k, stored in ((16, 8192, 8192, "kn"), (16, 50257, 768, "nk"), (64, 50257, 768, "nk")):
+        a0 = normal([m, k])
+        w0 = normal([k, n]) if stored == "kn" else normal([n, k])
+        ring = ring_of(lambda: (clone(a0), clone(w0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
+        label = (f"matmul {m}x{n}x{k}, few rows" if stored == "kn" else
+                 f"matmul {m}x{n}x{k}, few rows, right operand stored ({n},{k}) (!t): GPT-2's token projection")
+        measure(label, ring, (lambda s: F.matmul(s[0], s[1], out=s[2])) if stored == "kn" else
+                (lambda s: F.matmul(s[0], F.t(s[1]), out=s[2])), 4 * (m * k + k * n + m * n))
+        del a0, w0
+    # class scores: very many rows of ten columns; and one row of 2^24 columns
+    for rows_, cols_ in ((1677721, 10), (1, 1 << 24)):
+        x0 = normal([rows_, cols_])
+        ring = ring_of(lambda: (clone(x0), T([rows_, cols_], initial_element=None)), 8 * rows_ * cols_)
+        measure(f"row softmax ({rows_},{cols_}), one kernel" if rows_ > 1 else
+                f"row softmax ({rows_},{cols_}): pieces of the row over the grid, two launches", ring,
+                lambda s: F.softmax_fused(s[0], out=s[1]), (8 if rows_ > 1 else 12) * rows_ * cols_)
+        del x0
     B, H, S, hd = 8, 12, 1024, 64
     q0 = normal([B, H, S, hd])
     for causal in (True, False):

@@ -225,8 +225,13 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   const int mt = rows <= 16 ? 1 : (rows <= 32 ? 2 : 4);
   const int cb = 4;
   p.cgroups = (uint32_t)ceil_div((int64_t)cols, (int64_t)(16 * cb));
-  // about four workgroups per compute unit, every wavefront at least four steps of 16
-  int64_t gsplit = (int64_t)rt().num_cus * 4 / p.cgroups;
+  // about two workgroups per compute unit (on operands that are not in any cache, (16, 8192) . (8192, 8192):
+  // 58.5 us with two, 62.4 with four, 70.1 with sixteen: longer slices, fewer planes), every wavefront at
+  // least four steps of 16.  Tried without gain: two neighbouring vectors per lane for the (cols, k) storage,
+  // so that the four lanes of a row use up a 128-byte line in one step (76 against 74 us); a group of columns
+  // per wavefront with the whole K instead of quarters of K (GPT-2's token projection 48.3 against 49.6 us,
+  // everything else slower).
+  int64_t gsplit = (int64_t)rt().num_cus * 2 / p.cgroups;
   if (gsplit > k / 256) gsplit = k / 256;
   if (gsplit < 1) gsplit = 1;
   p.kslice = (int32_t)(ceil_div(ceil_div((int64_t)k, gsplit), (int64_t)64) * 64);
