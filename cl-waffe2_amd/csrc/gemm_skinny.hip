@@ -103,7 +103,11 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
     xrow[t] = p.X + (int64_t)(xlive[t] ? i : 0) * p.ldx + 4 * kk;
   }
 
-  f4 wv[2][CB], xv[2][MT];
+  // NB fetches of 16 steps in flight per wavefront; fetches past the end of the slice load nothing and multiply
+  // zeros, so the loop runs in whole rounds of NB.  (Four in flight, or 128 columns per wavefront to halve x's
+  // share of the requests, left (16, 8192) . (8192, 8192) on operands in no cache at 59 us.)
+  constexpr int NB = 2;
+  f4 wv[NB][CB], xv[NB][MT];
   auto fetch = [&](int k0, int buf) {
     const bool in = k0 + 4 * kk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
 #pragma unroll
@@ -129,20 +133,14 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
       }
   };
   if (kbeg < kend) {
-    fetch(kbeg, 0);
-    int k0 = kbeg;
-    for (; k0 + 32 < kend; k0 += 32) {
-      fetch(k0 + 16, 1);
-      multiply(0);
-      fetch(k0 + 32, 0);
-      multiply(1);
-    }
-    if (k0 + 16 < kend) {
-      fetch(k0 + 16, 1);
-      multiply(0);
-      multiply(1);
-    } else {
-      multiply(0);
+#pragma unroll
+    for (int b = 0; b < NB - 1; b++) fetch(kbeg + 16 * b, b);
+    for (int k0 = kbeg; k0 < kend; k0 += 16 * NB) {
+#pragma unroll
+      for (int b = 0; b < NB; b++) {
+        fetch(k0 + 16 * (b + NB - 1), (b + NB - 1) % NB);
+        multiply(b);
+      }
     }
   }
 
