@@ -185,6 +185,129 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
     }
 }
 
+// W stored (cols, k) and at most 32 rows: the same product with W fetched as whole lines.  In the kernel above a
+// lane's 16-byte load covers a quarter of 64 bytes of its row, so a fetch touches 64 bytes of 64 rows and the
+// other half of every 128-byte line is asked for a step later (rocprofv3: 1.39 x the operand fetched, (16, 8192)
+// . (8192, 8192)^T 69 us against 51 us for the other storage).  Here eight lanes cover 128 bytes of a row (32
+// steps of K), a load instruction eight rows, and the wavefront's 64 x 32 piece goes through a region of LDS of
+// its own (row pitch 36 floats) from which every lane reads the 16 bytes the matrix-core layout wants: rows
+// 16 b + lane % 16, steps 16 h + 4 (lane / 16) ... + 3.  No barrier: a wavefront's LDS accesses execute in order.
+template <int MT>
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_lines_kernel(SkinnyParams p) {
+  constexpr int kPitch = 36, kPiece = 64 * kPitch;  // floats
+  __shared__ __attribute__((aligned(16))) float lds[(kBlock / kWave) * kPiece];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int kk = lane >> 4, jj = lane & 15;
+  const int lrow = lane >> 3, lk = (lane & 7) * 4;  // the loading layout: row within eight, step within 32
+  const uint32_t ks = blockIdx.x / p.cgroups, cg = blockIdx.x - ks * p.cgroups;
+  const int64_t j0 = (int64_t)cg * 64;
+  const int quarter = p.kslice / 4;  // a multiple of 32
+  const int kbeg = (int)ks * p.kslice + wave * quarter;
+  const int kend = kbeg + quarter < p.k ? kbeg + quarter : p.k;
+  float* piece = lds + wave * kPiece;
+  const f4 zero = {0.f, 0.f, 0.f, 0.f};
+  f4 acc[MT][4];
+#pragma unroll
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int b = 0; b < 4; b++) acc[t][b] = zero;
+  const float* wrow[8];
+#pragma unroll
+  for (int q = 0; q < 8; q++) {
+    int64_t j = j0 + 8 * q + lrow;
+    if (j >= p.cols) j = p.cols - 1;  // read, not stored
+    wrow[q] = p.W + j * p.ldw + lk;
+  }
+  const float* xrow[MT];
+  bool xlive[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const int i = 16 * t + jj;
+    xlive[t] = i < p.rows;
+    xrow[t] = p.X + (int64_t)(xlive[t] ? i : 0) * p.ldx + 4 * kk;
+  }
+  f4 wv[2][8], xv[2][MT][2];
+  auto fetch = [&](int k0, int buf) {
+    const bool in = k0 + lk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
+#pragma unroll
+    for (int q = 0; q < 8; q++) wv[buf][q] = in ? *reinterpret_cast<const f4*>(wrow[q] + k0) : zero;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const bool xin = k0 + 16 * h + 4 * kk < kend;
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+        xv[buf][t][h] = (xin && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + k0 + 16 * h) : zero;
+    }
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 8; q++) *reinterpret_cast<f4*>(piece + (8 * q + lrow) * kPitch + lk) = wv[buf][q];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      f4 w[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) w[b] = *reinterpret_cast<const f4*>(piece + (16 * b + jj) * kPitch + 16 * h + 4 * kk);
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int t = 0; t < MT; t++)
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[buf][t][h][s], w[b][s], acc[t][b], 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  if (kbeg < kend) {
+    fetch(kbeg, 0);
+    for (int k0 = kbeg; k0 < kend; k0 += 64) {  // fetches past the end load nothing and multiply zeros
+      fetch(k0 + 32, 1);
+      multiply(0);
+      fetch(k0 + 64, 0);
+      multiply(1);
+    }
+  }
+  // the four quarters of K meet in wavefront 0, in the order 1, 2, 3 (through the first piece of LDS)
+  float* meet = lds;
+  for (int w = 1; w < kBlock / kWave; w++) {
+    __syncthreads();
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) meet[((t * 4 + b) * 4 + r) * kWave + lane] = acc[t][b][r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) acc[t][b][r] += meet[((t * 4 + b) * 4 + r) * kWave + lane];
+    }
+  }
+  if (wave != 0) return;
+#pragma unroll
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int row = 16 * t + 4 * kk + r;
+      if (row >= p.rows) continue;
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const int64_t col = j0 + 16 * b + jj;
+        if (col >= p.cols) continue;
+        if (p.gsplit == 1)
+          skinny_finish_store(p, row, col, acc[t][b][r]);
+        else
+          p.partial[((int64_t)ks * p.rows + row) * p.cols + col] = acc[t][b][r];
+      }
+    }
+}
+
 // the slices' planes added in the order 0, 1, ..., then alpha, beta, bias, activation, residual
 __global__ __launch_bounds__(kBlock) void sgemm_skinny_finish(SkinnyParams p) {
   const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -232,7 +355,8 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   int64_t gsplit = (int64_t)rt().num_cus * 2 / p.cgroups;
   if (gsplit > k / 256) gsplit = k / 256;
   if (gsplit < 1) gsplit = 1;
-  p.kslice = (int32_t)(ceil_div(ceil_div((int64_t)k, gsplit), (int64_t)64) * 64);
+  // (128: a quarter per wavefront then starts on a 128-byte line of W's rows where those are stored along k)
+  p.kslice = (int32_t)(ceil_div(ceil_div((int64_t)k, gsplit), (int64_t)128) * 128);
   gsplit = ceil_div((int64_t)k, (int64_t)p.kslice);
   p.gsplit = (uint32_t)gsplit;
   p.partial = nullptr;
@@ -256,7 +380,11 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
     else if (mt == 2) sgemm_skinny_kernel<TW_, 2, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);   \
     else sgemm_skinny_kernel<TW_, 4, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);                \
   } while (0)
-  if (w_is_cols_by_k)
+  if (w_is_cols_by_k && mt == 1)
+    sgemm_skinny_lines_kernel<1><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else if (w_is_cols_by_k && mt == 2)
+    sgemm_skinny_lines_kernel<2><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else if (w_is_cols_by_k)
     WF2_SKINNY(true);
   else
     WF2_SKINNY(false);
