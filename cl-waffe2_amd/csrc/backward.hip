@@ -64,6 +64,8 @@ constexpr int kTinyCols = 64;
 constexpr int kTinyFloats = 128 * 33;  // >= 64 * 65
 __host__ __device__ inline int tiny_rows_per_group(int ncols) { return ncols <= 32 ? 128 : 64; }
 
+// VEC: y, dy and dx are 16-byte aligned: the runs are staged in 16-byte vectors.
+template <bool VEC>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __restrict__ y, const float* dy,  // dx may be dy
                                                                 float* dx, int64_t nrows, int ncols, float scale,
                                                                 FastDiv by_c) {
@@ -75,7 +77,35 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __r
   const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
   const int64_t base = row0 * ncols;
   constexpr int U = 4;
-  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const uint32_t whole = VEC ? cells / 4 : 0;
+  if constexpr (VEC) {
+    for (uint32_t q0 = threadIdx.x; q0 < whole; q0 += kBlock * 2) {
+      f4 a[2], b[2];
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const bool live = q0 + u * kBlock < whole;
+        a[u] = live ? *reinterpret_cast<const f4*>(y + base + 4 * (int64_t)(q0 + u * kBlock)) : f4{0.f, 0.f, 0.f, 0.f};
+        b[u] = live ? *reinterpret_cast<const f4*>(dy + base + 4 * (int64_t)(q0 + u * kBlock)) : f4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+        if (q0 + u * kBlock < whole) {
+          uint32_t col;
+          uint32_t row = fd_divmod(4 * (q0 + u * kBlock), by_c, &col);
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            ty[row * pitch + col] = a[u][c];
+            td[row * pitch + col] = b[u][c];
+            if (++col == (uint32_t)ncols) {
+              col = 0;
+              row++;
+            }
+          }
+        }
+    }
+  }
+  for (uint32_t e0 = 4 * whole + threadIdx.x; e0 < cells; e0 += kBlock * U) {
     float a[U], b[U];
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -102,7 +132,23 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __r
     for (int j = 0; j < ncols; j++) a[j] = scale * (a[j] * (b[j] - dot));
   }
   __syncthreads();
-  for (uint32_t e = threadIdx.x; e < cells; e += kBlock) {
+  if constexpr (VEC) {
+    for (uint32_t q = threadIdx.x; q < whole; q += kBlock) {
+      uint32_t col;
+      uint32_t row = fd_divmod(4 * q, by_c, &col);
+      f4 v;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        v[c] = ty[row * pitch + col];
+        if (++col == (uint32_t)ncols) {
+          col = 0;
+          row++;
+        }
+      }
+      *reinterpret_cast<f4*>(dx + base + 4 * (int64_t)q) = v;
+    }
+  }
+  for (uint32_t e = 4 * whole + threadIdx.x; e < cells; e += kBlock) {
     uint32_t col;
     const uint32_t row = fd_divmod(e, by_c, &col);
     dx[base + e] = ty[row * pitch + col];
@@ -640,8 +686,13 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
   if (xlo < dhi && dlo < xhi && !(dx == dy && lddx == lddy))
     return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps dy without being dy");
   if (cols <= kTinyCols && causal_seq == 0 && rows >= 16384 && ldy == cols && lddy == cols && lddx == cols) {
-    softmax_bwd_rows_tiny<<<(uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols)), kBlock, 0, rt().stream>>>(
-        y, dy, dx, rows, (int)cols, scale, make_fastdiv((uint32_t)cols));
+    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols));
+    if (aligned16(y) && aligned16(dy) && aligned16(dx))
+      softmax_bwd_rows_tiny<true><<<groups, kBlock, 0, rt().stream>>>(y, dy, dx, rows, (int)cols, scale,
+                                                                        make_fastdiv((uint32_t)cols));
+    else
+      softmax_bwd_rows_tiny<false><<<groups, kBlock, 0, rt().stream>>>(y, dy, dx, rows, (int)cols, scale,
+                                                                         make_fastdiv((uint32_t)cols));
     return after_launch("softmax_bwd_rows_tiny");
   }
   int nv = pick_nv(cols);

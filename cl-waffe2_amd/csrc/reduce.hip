@@ -1448,7 +1448,9 @@ struct TinyRows {
   int ncols;
 };
 
-template <int MODE>
+// VEC: x and every output are 16-byte aligned: the run is staged in 16-byte vectors (a group's run starts on
+// a multiple of 16 bytes: 256 or 128 rows), the last partial vector of a ragged last group element by element.
+template <int MODE, bool VEC>
 __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
   __shared__ float tile[kTinyFloats];
   const int ncols = a.ncols, pitch = ncols | 1, group = tiny_rows_per_group(ncols);
@@ -1457,17 +1459,48 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
   const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
   const int64_t base = row0 * ncols;
   constexpr int U = 4;
-  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
-    float v[U];
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  if constexpr (VEC) {
+    const uint32_t whole = cells / 4;
+    for (uint32_t q0 = threadIdx.x; q0 < whole; q0 += kBlock * U) {
+      f4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) v[u] = e0 + u * kBlock < cells ? a.x[base + e0 + u * kBlock] : 0.0f;
+      for (int u = 0; u < U; u++)
+        v[u] = q0 + u * kBlock < whole ? *reinterpret_cast<const f4*>(a.x + base + 4 * (int64_t)(q0 + u * kBlock))
+                                       : f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int u = 0; u < U; u++)
-      if (e0 + u * kBlock < cells) {
-        uint32_t col;
-        const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
-        tile[row * pitch + col] = v[u];
-      }
+      for (int u = 0; u < U; u++)
+        if (q0 + u * kBlock < whole) {
+          uint32_t col;
+          uint32_t row = fd_divmod(4 * (q0 + u * kBlock), by_c, &col);
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            tile[row * pitch + col] = v[u][c];
+            if (++col == (uint32_t)ncols) {
+              col = 0;
+              row++;
+            }
+          }
+        }
+    }
+    for (uint32_t e = 4 * whole + threadIdx.x; e < cells; e += kBlock) {
+      uint32_t col;
+      const uint32_t row = fd_divmod(e, by_c, &col);
+      tile[row * pitch + col] = a.x[base + e];
+    }
+  } else {
+    for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = e0 + u * kBlock < cells ? a.x[base + e0 + u * kBlock] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        if (e0 + u * kBlock < cells) {
+          uint32_t col;
+          const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+          tile[row * pitch + col] = v[u];
+        }
+    }
   }
   __syncthreads();
   if ((int)threadIdx.x < rows_here) {
@@ -1504,21 +1537,49 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
     }
   }
   __syncthreads();
-  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
-    float lab[U];
-    if constexpr (MODE == kTinyXent) {
+  auto finish = [&](uint32_t e, float z, float lab) {
+    a.out[base + e] = z;
+    if constexpr (MODE == kTinyXent) a.loss[base + e] = xent_term(lab, z, a.param);
+  };
+  if constexpr (VEC) {
+    const uint32_t whole = cells / 4;
+    for (uint32_t q = threadIdx.x; q < whole; q += kBlock) {
+      f4 lab = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (MODE == kTinyXent) lab = *reinterpret_cast<const f4*>(a.aux0 + base + 4 * (int64_t)q);
+      uint32_t col;
+      uint32_t row = fd_divmod(4 * q, by_c, &col);
+      f4 z, loss;
 #pragma unroll
-      for (int u = 0; u < U; u++) lab[u] = e0 + u * kBlock < cells ? a.aux0[base + e0 + u * kBlock] : 0.0f;
-    }
-#pragma unroll
-    for (int u = 0; u < U; u++)
-      if (e0 + u * kBlock < cells) {
-        uint32_t col;
-        const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
-        const float z = tile[row * pitch + col];
-        a.out[base + e0 + u * kBlock] = z;
-        if constexpr (MODE == kTinyXent) a.loss[base + e0 + u * kBlock] = xent_term(lab[u], z, a.param);
+      for (int c = 0; c < 4; c++) {
+        z[c] = tile[row * pitch + col];
+        if constexpr (MODE == kTinyXent) loss[c] = xent_term(lab[c], z[c], a.param);
+        if (++col == (uint32_t)ncols) {
+          col = 0;
+          row++;
+        }
       }
+      *reinterpret_cast<f4*>(a.out + base + 4 * (int64_t)q) = z;
+      if constexpr (MODE == kTinyXent) *reinterpret_cast<f4*>(a.loss + base + 4 * (int64_t)q) = loss;
+    }
+    for (uint32_t e = 4 * whole + threadIdx.x; e < cells; e += kBlock) {
+      uint32_t col;
+      const uint32_t row = fd_divmod(e, by_c, &col);
+      finish(e, tile[row * pitch + col], MODE == kTinyXent ? a.aux0[base + e] : 0.0f);
+    }
+  } else {
+    for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+      float lab[U];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        lab[u] = (MODE == kTinyXent && e0 + u * kBlock < cells) ? a.aux0[base + e0 + u * kBlock] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        if (e0 + u * kBlock < cells) {
+          uint32_t col;
+          const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+          finish(e0 + u * kBlock, tile[row * pitch + col], lab[u]);
+        }
+    }
   }
 }
 
@@ -1531,8 +1592,11 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
   if (ncols <= kTinyCols && ldx == ncols && ldo == ncols && causal_seq == 0 && nrows >= kTinyMinRows &&
       ceil_div(nrows, 128) < ((int64_t)1 << 31)) {
     TinyRows a{x, out, xe.labels, nullptr, xe.loss, xe.delta, nrows, (int)ncols};
-    rows_tiny<XENT ? kTinyXent : kTinySoftmax><<<(uint32_t)ceil_div(nrows, tiny_rows_per_group((int)ncols)), kBlock, 0, rt().stream>>>(
-        a, make_fastdiv((uint32_t)ncols));
+    const uint32_t groups = (uint32_t)ceil_div(nrows, tiny_rows_per_group((int)ncols));
+    if (aligned16(x) && aligned16(out) && (!XENT || (aligned16(xe.labels) && aligned16(xe.loss))))
+      rows_tiny<XENT ? kTinyXent : kTinySoftmax, true><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)ncols));
+    else
+      rows_tiny<XENT ? kTinyXent : kTinySoftmax, false><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)ncols));
     return after_launch("rows_tiny");
   }
   const int nv = pick_nv(ncols);
@@ -1770,8 +1834,11 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   if (!x || !gamma || !beta || !out) return fail(WF2HIP_EINVAL, "null pointer");
   if (cols <= kTinyCols && rows >= kTinyMinRows) {
     TinyRows a{x, out, gamma, beta, nullptr, eps, rows, (int)cols};
-    rows_tiny<kTinyLayerNorm><<<(uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols)), kBlock, 0, rt().stream>>>(
-        a, make_fastdiv((uint32_t)cols));
+    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols));
+    if (aligned16(x) && aligned16(out))
+      rows_tiny<kTinyLayerNorm, true><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)cols));
+    else
+      rows_tiny<kTinyLayerNorm, false><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)cols));
     return after_launch("rows_tiny");
   }
   int nv = pick_nv(cols);
