@@ -222,15 +222,42 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tiny(RowRedParams p, FastD
   const uint32_t count = rows_here * n;
   const float* src = p.b + (int64_t)row0 * n;
   auto place = [&](uint32_t e) { const uint32_t r = fd_div(e, by_n); return r * pitch + (e - r * n); };
-  uint32_t e = threadIdx.x;
-  for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
-    float v[8];
+  if (((uintptr_t)src & 15u) == 0) {
+    // the run in 16-byte vectors (a workgroup's run of 256 rows starts on a multiple of 16 bytes), four in
+    // flight per thread; the elements of a vector are placed one by one
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4* vsrc = reinterpret_cast<const f4*>(src);
+    const uint32_t whole = count / 4;
+    for (uint32_t q0 = threadIdx.x; q0 < whole; q0 += 4 * kBlock) {
+      f4 v[4];
 #pragma unroll
-    for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+      for (int u = 0; u < 4; u++) v[u] = q0 + u * kBlock < whole ? vsrc[q0 + u * kBlock] : f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int u = 0; u < 8; u++) tiny_tile[place(e + u * kBlock)] = v[u];
+      for (int u = 0; u < 4; u++)
+        if (q0 + u * kBlock < whole) {
+          uint32_t r = fd_div((q0 + u * kBlock) * 4, by_n), c = (q0 + u * kBlock) * 4 - r * n;
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            tiny_tile[r * pitch + c] = v[u][i];
+            if (++c == n) {
+              c = 0;
+              r++;
+            }
+          }
+        }
+    }
+    for (uint32_t e = whole * 4 + threadIdx.x; e < count; e += kBlock) tiny_tile[place(e)] = src[e];
+  } else {
+    uint32_t e = threadIdx.x;
+    for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+#pragma unroll
+      for (int u = 0; u < 8; u++) tiny_tile[place(e + u * kBlock)] = v[u];
+    }
+    for (; e < count; e += kBlock) tiny_tile[place(e)] = src[e];
   }
-  for (; e < count; e += kBlock) tiny_tile[place(e)] = src[e];
   __syncthreads();
   if (threadIdx.x >= rows_here) return;
   const float* row = tiny_tile + threadIdx.x * pitch;

@@ -202,15 +202,48 @@ __global__ __launch_bounds__(kBlock) void select_rows_tiny(SelParams<T> p, FastD
   const uint32_t count = rows_here * n;
   const T* src = p.x + (int64_t)row0 * n;
   auto place = [&](uint32_t e) { const uint32_t r = fd_div(e, by_n); return r * pitch + (e - r * n); };
-  uint32_t e = threadIdx.x;
-  for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
-    T v[8];
+  if (((uintptr_t)src & 15u) == 0) {
+    // the run in 16-byte vectors (a workgroup's run of 256 rows starts on a multiple of 16 bytes), four in
+    // flight per thread; the elements of a vector are placed one by one
+    constexpr int N = 16 / (int)sizeof(T);
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    union Vec {
+      u4 q;
+      T v[N];
+    };
+    const u4* vsrc = reinterpret_cast<const u4*>(src);
+    const uint32_t whole = count / N;
+    for (uint32_t q0 = threadIdx.x; q0 < whole; q0 += 4 * kBlock) {
+      Vec v[4];
 #pragma unroll
-    for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+      for (int u = 0; u < 4; u++)
+        if (q0 + u * kBlock < whole) v[u].q = vsrc[q0 + u * kBlock];
 #pragma unroll
-    for (int u = 0; u < 8; u++) tile[place(e + u * kBlock)] = v[u];
+      for (int u = 0; u < 4; u++)
+        if (q0 + u * kBlock < whole) {
+          uint32_t r = fd_div((q0 + u * kBlock) * N, by_n), c = (q0 + u * kBlock) * N - r * n;
+#pragma unroll
+          for (int i = 0; i < N; i++) {
+            tile[r * pitch + c] = v[u].v[i];
+            if (++c == n) {
+              c = 0;
+              r++;
+            }
+          }
+        }
+    }
+    for (uint32_t e = whole * N + threadIdx.x; e < count; e += kBlock) tile[place(e)] = src[e];
+  } else {
+    uint32_t e = threadIdx.x;
+    for (; e + 7 * kBlock < count; e += 8 * kBlock) {  // eight loads in flight per thread
+      T v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = src[e + u * kBlock];
+#pragma unroll
+      for (int u = 0; u < 8; u++) tile[place(e + u * kBlock)] = v[u];
+    }
+    for (; e < count; e += kBlock) tile[place(e)] = src[e];
   }
-  for (; e < count; e += kBlock) tile[place(e)] = src[e];
   __syncthreads();
   if (threadIdx.x >= rows_here) return;
   Best<T> b = {worst<T, IsMax>(), 0u};
