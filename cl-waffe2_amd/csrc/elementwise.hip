@@ -851,7 +851,8 @@ static int launch_tile128(const TileParams& p, uint32_t blocks, F f) {
 constexpr int kNarrowMax = 31;
 constexpr int kNarrowFloats = 8064;  // >= 15 * 516 and 31 * 260
 
-template <class F, bool ReadDst, bool VEC>
+// VECSRC: src's rows are adjacent (s_i == nj) and 16-byte aligned: its run is read in 16-byte vectors.
+template <class F, bool ReadDst, bool VEC, bool VECSRC>
 __global__ __launch_bounds__(kBlock) void ew_tile_narrow(TileParams p, F f, FastDiv by_nj, int tl) {
   __shared__ __attribute__((aligned(16))) float tile[kNarrowFloats];
   const int pitch = tl + 4;
@@ -871,8 +872,34 @@ __global__ __launch_bounds__(kBlock) void ew_tile_narrow(TileParams p, F f, Fast
   float* dst = p.dst + doff;
   const float* src = p.src + soff;
   constexpr int U = 4;
+  uint32_t staged = 0;  // cells already in LDS
+  if constexpr (VECSRC) {
+    const uint32_t whole = cells / 4;
+    const f4* vsrc = reinterpret_cast<const f4*>(src + i0 * p.s_i);
+    for (uint32_t q0 = threadIdx.x; q0 < whole; q0 += kBlock * U) {
+      f4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = q0 + u * kBlock < whole ? vsrc[q0 + u * kBlock] : f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        if (q0 + u * kBlock < whole) {
+          uint32_t j;
+          uint32_t i = fd_divmod(4 * (q0 + u * kBlock), by_nj, &j);
+          const float c4[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            tile[j * pitch + i] = c4[c];
+            if (++j == (uint32_t)nj) {
+              j = 0;
+              i++;
+            }
+          }
+        }
+    }
+    staged = 4 * whole;
+  }
   // src (i, j) at i * s_i + j  ->  LDS
-  for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+  for (uint32_t e0 = staged + threadIdx.x; e0 < cells; e0 += kBlock * U) {
     float v[U];
     uint32_t i[U], j[U];
 #pragma unroll
@@ -1096,10 +1123,17 @@ static bool try_launch_tile(const Space& s, float* dst, const float* src, F f, i
     for (int i = 0; i < p.nouter; i++)
       if (p.odst[i] % 4 != 0) v16 = false;
     const FastDiv by_nj = make_fastdiv((uint32_t)p.nj);
-    if (v16)
-      ew_tile_narrow<F, ReadDst, true><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+    bool vsrc = aligned16(p.src) && p.s_i == p.nj;  // a tile's rows of src are one run, on a multiple of 16 bytes
+    for (int i = 0; i < p.nouter; i++)
+      if (p.osrc[i] % 4 != 0) vsrc = false;
+    if (v16 && vsrc)
+      ew_tile_narrow<F, ReadDst, true, true><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+    else if (v16)
+      ew_tile_narrow<F, ReadDst, true, false><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+    else if (vsrc)
+      ew_tile_narrow<F, ReadDst, false, true><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
     else
-      ew_tile_narrow<F, ReadDst, false><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
+      ew_tile_narrow<F, ReadDst, false, false><<<(uint32_t)nblocks, kBlock, 0, rt().stream>>>(p, f, by_nj, tl);
     *rc = after_launch("ew_tile_narrow");
     return true;
   }
