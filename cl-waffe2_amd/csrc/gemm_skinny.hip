@@ -104,9 +104,10 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
   }
 
   // NB fetches of 16 steps in flight per wavefront; fetches past the end of the slice load nothing and multiply
-  // zeros, so the loop runs in whole rounds of NB.  (Four in flight, or 128 columns per wavefront to halve x's
-  // share of the requests, left (16, 8192) . (8192, 8192) on operands in no cache at 59 us.)
-  constexpr int NB = 2;
+  // zeros, so the loop runs in whole rounds of NB.  Three from 17 rows on ((32, 8192) . (8192, 8192): 75 -> 69 us;
+  // at 64 rows no change).  (Four in flight, or 128 columns per wavefront to halve x's share of the requests, left
+  // (16, 8192) . (8192, 8192) on operands in no cache at 59 us.)
+  constexpr int NB = MT >= 2 ? 3 : 2;
   f4 wv[NB][CB], xv[NB][MT];
   auto fetch = [&](int k0, int buf) {
     const bool in = k0 + 4 * kk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
