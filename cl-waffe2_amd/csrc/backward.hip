@@ -408,6 +408,95 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_rows(const float* __rest
   }
 }
 
+// Very many rows of at most 64 columns: a wavefront per row leaves most lanes idle ((1677721, 10): 1.4 ms).
+// A workgroup walks groups of 128 adjacent rows (64 beyond 32 columns): x and dy, one contiguous run each, are
+// staged into LDS in storage order (odd pitch), thread r works through row r (the formulas of layernorm_bwd_rows:
+// the mean from a binary64 sum, deviations and squares in binary32) and leaves xh in place of x and the row's
+// rstd and two means beside it; threads 0 .. ncols - 1 then add their column's dy xh and dy over the group's rows
+// into registers, and all threads write dx in storage order.  A workgroup's column sums go to its row of
+// `partial`, folded like the other kernels'.
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                             const float* dy, float eps,  // dx may be dy
+                                                             float* dx, float* __restrict__ partial, int64_t nrows,
+                                                             int ncols, FastDiv by_c) {
+  __shared__ float tx[kTinyFloats];
+  __shared__ float td[kTinyFloats];
+  __shared__ float row_rstd[128], row_m1[128], row_m2[128];
+  const int pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  const int64_t ngroups = (nrows + group - 1) / group;
+  const float inv_n = 1.0f / (float)ncols;
+  float dg = 0.0f, db = 0.0f;  // threads 0 .. ncols - 1: the column sums over this workgroup's rows
+  constexpr int U = 4;
+  for (int64_t grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+    const int64_t row0 = grp * group;
+    const int rows_here = (int)(nrows - row0 < group ? nrows - row0 : group);
+    const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
+    const int64_t base = row0 * ncols;
+    __syncthreads();  // the previous group has been written out
+    for (uint32_t e0 = threadIdx.x; e0 < cells; e0 += kBlock * U) {
+      float a[U], b[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const bool live = e0 + u * kBlock < cells;
+        a[u] = live ? x[base + e0 + u * kBlock] : 0.0f;
+        b[u] = live ? dy[base + e0 + u * kBlock] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        if (e0 + u * kBlock < cells) {
+          uint32_t col;
+          const uint32_t row = fd_divmod(e0 + u * kBlock, by_c, &col);
+          tx[row * pitch + col] = a[u];
+          td[row * pitch + col] = b[u];
+        }
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < rows_here) {
+      float* xr = tx + threadIdx.x * pitch;
+      const float* dr = td + threadIdx.x * pitch;
+      double sum = 0.0;
+      for (int j = 0; j < ncols; j++) sum += (double)xr[j];
+      const float mean = (float)(sum / (double)ncols);
+      float sq = 0.0f;
+      for (int j = 0; j < ncols; j++) {
+        const float d = xr[j] - mean;
+        xr[j] = d;
+        sq = __builtin_fmaf(d, d, sq);
+      }
+      const float rstd = (float)(1.0 / __builtin_sqrt((double)sq / (double)ncols + (double)eps));
+      float s1 = 0.0f, s2 = 0.0f;
+      for (int j = 0; j < ncols; j++) {
+        const float xh = xr[j] * rstd;
+        xr[j] = xh;
+        const float dyh = dr[j] * gamma[j];
+        s1 += dyh;
+        s2 = __builtin_fmaf(dyh, xh, s2);
+      }
+      row_rstd[threadIdx.x] = rstd;
+      row_m1[threadIdx.x] = s1 * inv_n;
+      row_m2[threadIdx.x] = s2 * inv_n;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < ncols) {
+      for (int r = 0; r < rows_here; r++) {
+        const float d = td[r * pitch + threadIdx.x];
+        dg = __builtin_fmaf(d, tx[r * pitch + threadIdx.x], dg);
+        db += d;
+      }
+    }
+    for (uint32_t e = threadIdx.x; e < cells; e += kBlock) {
+      uint32_t col;
+      const uint32_t row = fd_divmod(e, by_c, &col);
+      const float dyh = td[row * pitch + col] * gamma[col];
+      dx[base + e] = row_rstd[row] * ((dyh - row_m1[row]) - tx[row * pitch + col] * row_m2[row]);
+    }
+  }
+  if ((int)threadIdx.x < ncols) {
+    partial[((int64_t)blockIdx.x * 2 + 0) * ncols + threadIdx.x] = dg;
+    partial[((int64_t)blockIdx.x * 2 + 1) * ncols + threadIdx.x] = db;
+  }
+}
+
 // Rows of 2049 ... 8192 columns: a workgroup per row, thread t holding the NG 16-byte vectors
 // (g 256 + t) 4 ... of x, dy and gamma and its share of the two column sums in registers; the
 // row statistics meet in LDS (three exchanges per row).  Workgroup b walks rows b, b + B, ...
@@ -765,7 +854,10 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // two workgroups per compute unit, at most one wavefront per row: (65536, 1024) runs at 74 % of
   // the HBM peak (both small folds included), 66 % with one workgroup per unit, 65 - 67 % with
   // three to eight (more rows of `partial` to write and fold)
+  const bool tiny = cols <= kTinyCols && rows >= 16384;
   const int64_t blocks = wide ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
+                         : tiny ? std::min<int64_t>(ceil_div((int64_t)rows, (int64_t)tiny_rows_per_group((int)cols)),
+                                                    4 * (int64_t)std::max(rt().num_cus, 1))
                               : std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
   const size_t partial_bytes = (size_t)blocks * 2 * cols * sizeof(float);
   const size_t level2_bytes = (size_t)kFoldGroups * 2 * cols * sizeof(double);
@@ -775,7 +867,11 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
   const bool streaming = total * 12 >= ((int64_t)192 << 20);
   int rc;
-  if (wide) {
+  if (tiny) {
+    layernorm_bwd_tiny<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(x, gamma, dy, eps, dx, (float*)partial, rows, (int)cols,
+                                                                     make_fastdiv((uint32_t)cols));
+    rc = after_launch("layernorm_bwd_tiny");
+  } else if (wide) {
     hipStream_t st = rt().stream;
     const int ng = (int)ceil_div(cols, (int64_t)kBlock * 4);
 #define WF2_WIDE(NG_)                                                                                              \

@@ -118,7 +118,9 @@ def test_causal_softmax_backward(gpu, batch, seq):
 @pytest.mark.parametrize("rows,cols", [(1, 4), (5, 60), (37, 768), (1000, 1024), (300, 2048), (4099, 768),
                                        (257, 1001), (8192, 768),
                                        # beyond 2048 columns: a workgroup per row, 3 ... 8 vectors per thread
-                                       (6, 2052), (700, 3072), (33, 4096), (1100, 5120), (5, 6148), (600, 8192)])
+                                       (6, 2052), (700, 3072), (33, 4096), (1100, 5120), (5, 6148), (600, 8192),
+                                       # very many rows of at most 64 columns: a thread per row
+                                       (16384, 10), (20001, 33), (16400, 64), (16385, 5), (40000, 32)])
 def test_layernorm_backward(gpu, rows, cols):
     from oracle import gpt2_block_ref as ref
     W = gpu
