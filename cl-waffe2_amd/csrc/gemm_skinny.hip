@@ -59,8 +59,12 @@ __device__ __forceinline__ void skinny_finish_store(const SkinnyParams& p, int r
 
 // TW: W stored (cols, k), k contiguous; otherwise (k, cols), columns contiguous.  MT tiles of 16 rows,
 // CB blocks of 16 columns.
-template <bool TW, int MT, int CB>
+// ALIGNED (the (k, cols) storage only): W's rows are 16-byte aligned and cols is a multiple of 4.  Otherwise
+// W is read element by element, lane jj taking columns j0 + 16 b + jj (64-byte runs), and the tiles hold those
+// columns.
+template <bool TW, int MT, int CB, bool ALIGNED = true>
 __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
+  static_assert(ALIGNED || (!TW && CB == 4), "the element-by-element form exists for the (k, cols) storage");
   __shared__ float meet[MT * CB * 4 * kWave];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int kk = lane >> 4, jj = lane & 15;
@@ -84,6 +88,13 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
       int64_t j = j0 + 16 * b + jj;
       if (j >= p.cols) j = p.cols - 1;
       wrow[b] = p.W + j * p.ldw + 4 * kk;
+    }
+  } else if (!ALIGNED) {
+#pragma unroll
+    for (int b = 0; b < CB; b++) {
+      int64_t j = j0 + 16 * b + jj;
+      if (j >= p.cols) j = p.cols - 1;
+      wrow[b] = p.W + (int64_t)(4 * kk) * p.ldw + j;
     }
   } else {
 #pragma unroll
@@ -113,10 +124,14 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
     const bool in = k0 + 4 * kk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
 #pragma unroll
     for (int q = 0; q < CB; q++) {
-      if (TW)
+      if (TW) {
         wv[buf][q] = in ? *reinterpret_cast<const f4*>(wrow[q] + k0) : zero;
-      else
+      } else if (ALIGNED) {
         wv[buf][q] = in ? *reinterpret_cast<const f4*>(wrow[q] + (int64_t)k0 * p.ldw) : zero;
+      } else {  // q is the step s; component b is column block b
+#pragma unroll
+        for (int b = 0; b < 4; b++) wv[buf][q][b] = in ? wrow[b][(int64_t)(k0 + q) * p.ldw] : 0.0f;
+      }
     }
 #pragma unroll
     for (int t = 0; t < MT; t++) xv[buf][t] = (in && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + k0) : zero;
@@ -176,7 +191,7 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
       if (row >= p.rows) continue;
 #pragma unroll
       for (int b = 0; b < CB; b++) {
-        const int64_t col = TW ? j0 + 16 * b + jj : j0 + 64 * (b / 4) + 4 * jj + b % 4;
+        const int64_t col = (TW || !ALIGNED) ? j0 + 16 * b + jj : j0 + 64 * (b / 4) + 4 * jj + b % 4;
         if (col >= p.cols) continue;
         if (p.gsplit == 1)
           skinny_finish_store(p, row, col, acc[t][b][r]);
@@ -332,8 +347,9 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   // slices of K) only on a large W ((64, 768) . (768, 50304): 92 against 111 us; (768, 2304): 18.1 against 14.6)
   if (rows > 32 && (int64_t)k * cols < ((int64_t)1 << 25)) return false;
   if (rows < 1 || rows > 64 || cols < 256 || k < 64 || k % 4 != 0 || k >= (1L << 30)) return false;
-  if (!aligned16(W) || !aligned16(X) || ldw % 4 != 0 || ldx % 4 != 0) return false;
-  if (!w_is_cols_by_k && cols % 4 != 0) return false;
+  if (!aligned16(X) || ldx % 4 != 0) return false;
+  const bool w_aligned = aligned16(W) && ldw % 4 == 0 && (w_is_cols_by_k || cols % 4 == 0);
+  if (w_is_cols_by_k && !w_aligned) return false;
   SkinnyParams p;
   p.W = W;
   p.X = X;
@@ -387,8 +403,14 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
     sgemm_skinny_lines_kernel<2><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   else if (w_is_cols_by_k)
     WF2_SKINNY(true);
-  else
+  else if (w_aligned)
     WF2_SKINNY(false);
+  else if (mt == 1)
+    sgemm_skinny_kernel<false, 1, 4, false><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else if (mt == 2)
+    sgemm_skinny_kernel<false, 2, 4, false><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+  else
+    sgemm_skinny_kernel<false, 4, 4, false><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
 #undef WF2_SKINNY
   *rc = after_launch("sgemm_skinny_kernel");
   if (*rc == 0 && gsplit > 1) {
