@@ -335,6 +335,23 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_finish(SkinnyParams p) {
   skinny_finish_store(p, row, e - (int64_t)row * p.cols, acc);
 }
 
+// many slices (a few outputs over a very long K): a wavefront per output element, lane l adds planes l, l + 64,
+// ... in binary64 and the lanes meet by shuffles -- a fixed order
+__global__ __launch_bounds__(kBlock) void sgemm_skinny_finish_wide(SkinnyParams p) {
+  const int64_t e = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  const int64_t plane = (int64_t)p.rows * p.cols;
+  if (e >= plane) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  double acc = 0.0;
+  for (uint32_t s = (uint32_t)lane; s < p.gsplit; s += kWave) acc += (double)p.partial[(int64_t)s * plane + e];
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) {
+    const int row = (int)(e / p.cols);
+    skinny_finish_store(p, row, e - (int64_t)row * p.cols, (float)acc);
+  }
+}
+
 static inline bool aligned16(const void* q) { return ((uintptr_t)q & 15u) == 0; }
 
 // Row-major C (rows x cols) = act(alpha x . W + beta C + bias) + residual.  `w_is_cols_by_k`: W stored
@@ -346,7 +363,9 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   // 33 ... 64 rows keep the matrix cores busy about half the time here: ahead of the tiled kernel (with its
   // slices of K) only on a large W ((64, 768) . (768, 50304): 92 against 111 us; (768, 2304): 18.1 against 14.6)
   if (rows > 32 && (int64_t)k * cols < ((int64_t)1 << 25)) return false;
-  if (rows < 1 || rows > 64 || cols < 256 || k < 64 || k % 4 != 0 || k >= (1L << 30)) return false;
+  // a wide operand, or a narrow one over a long K ((1 x 4194304) . (4194304 x 1): the slices of K fill the grid)
+  if (rows < 1 || rows > 64 || (cols < 256 && k < 8192) || cols < 1 || k < 64 || k % 4 != 0 || k >= (1L << 30))
+    return false;
   if (!aligned16(X) || ldx % 4 != 0) return false;
   const bool w_aligned = aligned16(W) && ldw % 4 == 0 && (w_is_cols_by_k || cols % 4 == 0);
   if (w_is_cols_by_k && !w_aligned) return false;
@@ -413,7 +432,10 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
     sgemm_skinny_kernel<false, 4, 4, false><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
 #undef WF2_SKINNY
   *rc = after_launch("sgemm_skinny_kernel");
-  if (*rc == 0 && gsplit > 1) {
+  if (*rc == 0 && gsplit > 16) {
+    sgemm_skinny_finish_wide<<<(uint32_t)ceil_div((int64_t)rows * cols, (int64_t)(kBlock / kWave)), kBlock, 0, st>>>(p);
+    *rc = after_launch("sgemm_skinny_finish_wide");
+  } else if (*rc == 0 && gsplit > 1) {
     sgemm_skinny_finish<<<(uint32_t)ceil_div((int64_t)rows * cols, (int64_t)kBlock), kBlock, 0, st>>>(p);
     *rc = after_launch("sgemm_skinny_finish");
   }
