@@ -96,7 +96,10 @@ int wf2hip_event_destroy(void* event);
  * are served from the pool only: WF2HIP_ECAPTURE otherwise); host transfers and
  * wf2hip_sync are refused while capturing; tensors the replay reads or writes
  * (inputs, outputs) must stay allocated for as long as the graph is used; new
- * inputs are written into the same buffers. */
+ * inputs are written into the same buffers.  wf2hip_graph_destroy waits for
+ * the stream; called while another graph is being recorded it returns at once
+ * and the graph is destroyed when that recording ends (a live graph keeps its
+ * blocks: run the sequence once more before recording it again). */
 int wf2hip_graph_begin(void);
 int wf2hip_graph_end(void** graph);
 int wf2hip_graph_launch(void* graph);
