@@ -904,6 +904,9 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
                       const float* residual, long ldres, int activation, int* rc);  // gemm_skinny.hip
 bool try_sgemm_tiny_out(long rows, long cols, long k, float alpha, const float* L, long ldl, const float* R, long ldr,
                         float** partial, long* planes, int* rc);  // gemm_skinny.hip
+bool try_sgemm_small_batch(bool ta, bool tb, long m, long n, long k, float alpha, const float* A, long lda, long sA,
+                           long sA2, const float* B, long ldb, long sB, long sB2, float beta, float* C, long ldc,
+                           long sC, long sC2, long batch, long batch2, int* rc);  // gemm_skinny.hip
 
 // Products with few output tiles and a long K (weight gradients: 768 x 3072 outputs over K = 8192 are
 // 144 tiles for 256 compute units) run as `splits` products over slices of K, the slices as the outer
@@ -1026,6 +1029,13 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
   if ((int64_t)batch * batch2 > 65535)
     return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  // many small matrices: an output element per thread or wavefront
+  if (!ep.bias && !ep.residual && ep.activation == 0 && ep.causal == 0) {
+    int rc = 0;
+    if (try_sgemm_small_batch(!is_n(transa), !is_n(transb), m, n, k, alpha, A, lda, strideA, strideA2, B, ldb, strideB,
+                              strideB2, beta, C, ldc, strideC, strideC2, batch, batch2, &rc))
+      return rc;
+  }
   // at most 64 rows in the row-major product (a few tokens through a layer): one read of the other operand
   if (batch == 1 && batch2 == 1 && n <= 64 && is_n(transb) && ep.causal == 0) {
     int rc = 0;

@@ -785,3 +785,28 @@ def test_matmul_small_output_long_k_both_k_major(gpu, rows, cols, k):
     scale = 0.5 * np.abs(A2) @ np.abs(B2.T) + 2.0 * np.abs(C2[:cols])
     assert np.max(np.abs(got[:cols] - want) / scale) < 1e-5
     np.testing.assert_array_equal(got[cols:], C2[cols:].astype(np.float32))
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(65535, 8, 8, 8), (4096, 16, 16, 16), (1024, 3, 3, 1000), (300, 1, 1, 4096),
+                                         (2000, 10, 10, 10), (100, 32, 32, 50), (64, 16, 16, 200), (256, 2, 1, 5000)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_many_small_matrices(gpu, batch, m, n, k, ta, tb):
+    """Batches of products with a few output elements each: an output element per thread, or per wavefront
+    over a longer K; every transpose form, and a two-level batch with a broadcast right operand."""
+    F = gpu.functional
+    rng = np.random.default_rng(batch + m + n + k)
+    A = rng.standard_normal((batch, m, k)).astype(np.float32)
+    B = rng.standard_normal((batch, k, n)).astype(np.float32)
+    swap = lambda a: np.ascontiguousarray(np.swapaxes(a, -1, -2))  # noqa: E731
+    dA = F.t(F.from_numpy(swap(A))) if ta else F.from_numpy(A)
+    dB = F.t(F.from_numpy(swap(B))) if tb else F.from_numpy(B)
+    got = F.matmul(dA, dB).numpy()
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    want = A64 @ B64
+    bound = REL * (np.abs(A64) @ np.abs(B64)) + 1e-30
+    assert np.all(np.abs(got - want) <= bound)
+    if batch % 4 == 0 and not ta:
+        A4 = A.reshape(4, batch // 4, m, k)
+        got = F.matmul(F.from_numpy(A4), dB.tensor if False else (F.t(F.from_numpy(swap(B[0]))) if tb else F.from_numpy(B[0]))).numpy()
+        want = A4.astype(np.float64) @ B64[0]
+        assert np.all(np.abs(got - want) <= REL * (np.abs(A4.astype(np.float64)) @ np.abs(B64[0])) + 1e-30)
