@@ -151,6 +151,10 @@ __global__ __launch_bounds__(kBlock) void dgemm_fold(const double* __restrict__ 
   }
 }
 
+bool try_dgemm_small_batch(bool ta, bool tb, long m, long n, long k, double alpha, const double* A, long lda, long sA,
+                           long sA2, const double* B, long ldb, long sB, long sB2, double beta, double* C, long ldc,
+                           long sC, long sC2, long batch, long batch2, int* rc);  // gemm_skinny.hip
+
 static bool dn(char c) { return c == 'N' || c == 'n'; }
 static bool dt(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
@@ -166,6 +170,12 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
   if (m == 0 || n == 0 || batch == 0 || batch2 == 0) return 0;
   if (!A || !B || !C) return fail(WF2HIP_EINVAL, "null matrix pointer");
   if ((int64_t)batch * batch2 > 65535) return fail(WF2HIP_EUNSUPPORTED, "more than 65535 matrices in one batch");
+  {  // many small matrices: an output element per thread or wavefront
+    int rc = 0;
+    if (try_dgemm_small_batch(!dn(transa), !dn(transb), m, n, k, alpha, A, lda, strideA, strideA2, B, ldb, strideB,
+                              strideB2, beta, C, ldc, strideC, strideC2, batch, batch2, &rc))
+      return rc;
+  }
   DgemmParams p;
   p.A = A; p.B = B; p.C = C;
   p.m = m; p.n = n; p.k = k;

@@ -551,19 +551,23 @@ bool try_sgemm_tiny_out(long rows, long cols, long k, float alpha, const float* 
 // tile per matrix; 256 x (1 x 4096) . (4096 x 1): 0.23 ms).  One output element per thread, or per wavefront
 // from K = 128 on (lanes along K, meeting by shuffles in binary64); the operands of neighbouring outputs are
 // the same few lines.  Column-major terms, as sgemm_: C(i, j) at i + j ldc.
+template <class T>
 struct SmallBatchParams {
-  const float* A;
-  const float* B;
-  float* C;
+  const T* A;
+  const T* B;
+  T* C;
   int64_t lda, ldb, ldc, sA, sA2, sB, sB2, sC, sC2;
   int32_t m, n, k, ta, tb;
   uint32_t batch_inner;
   int64_t outputs;  // m n batch batch2
-  float alpha, beta;
+  T alpha, beta;
 };
 
-template <bool WAVE>
-__global__ __launch_bounds__(kBlock) void sgemm_small_batch_kernel(SmallBatchParams p, FastDiv by_m, FastDiv by_n) {
+__device__ __forceinline__ float small_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double small_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+template <class T, bool WAVE>
+__global__ __launch_bounds__(kBlock) void sgemm_small_batch_kernel(SmallBatchParams<T> p, FastDiv by_m, FastDiv by_n) {
   const int64_t o = WAVE ? (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave
                          : (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (o >= p.outputs) return;
@@ -571,36 +575,37 @@ __global__ __launch_bounds__(kBlock) void sgemm_small_batch_kernel(SmallBatchPar
   uint32_t rest = fd_divmod((uint32_t)o, by_m, &i);
   const uint32_t z = fd_divmod(rest, by_n, &j);
   const uint32_t bi = z % p.batch_inner, bo = z / p.batch_inner;
-  const float* a = p.A + (int64_t)bi * p.sA + (int64_t)bo * p.sA2 + (p.ta ? (int64_t)i * p.lda : (int64_t)i);
-  const float* b = p.B + (int64_t)bi * p.sB + (int64_t)bo * p.sB2 + (p.tb ? (int64_t)j : (int64_t)j * p.ldb);
+  const T* a = p.A + (int64_t)bi * p.sA + (int64_t)bo * p.sA2 + (p.ta ? (int64_t)i * p.lda : (int64_t)i);
+  const T* b = p.B + (int64_t)bi * p.sB + (int64_t)bo * p.sB2 + (p.tb ? (int64_t)j : (int64_t)j * p.ldb);
   const int64_t astep = p.ta ? 1 : p.lda, bstep = p.tb ? p.ldb : 1;
-  float* c = p.C + (int64_t)bi * p.sC + (int64_t)bo * p.sC2 + i + (int64_t)j * p.ldc;
+  T* c = p.C + (int64_t)bi * p.sC + (int64_t)bo * p.sC2 + i + (int64_t)j * p.ldc;
   if (WAVE) {
     const int lane = threadIdx.x & (kWave - 1);
-    float part = 0.0f;
-    for (int kk = lane; kk < p.k; kk += kWave) part = __builtin_fmaf(a[kk * astep], b[kk * bstep], part);
+    T part = T(0);
+    for (int kk = lane; kk < p.k; kk += kWave) part = small_fma(a[kk * astep], b[kk * bstep], part);
     double acc = (double)part;
 #pragma unroll
     for (int s = kWave / 2; s > 0; s >>= 1) acc += __shfl_xor(acc, s);
-    if (lane == 0) *c = p.beta == 0.0f ? p.alpha * (float)acc : p.alpha * (float)acc + p.beta * *c;
+    if (lane == 0) *c = p.beta == T(0) ? p.alpha * (T)acc : p.alpha * (T)acc + p.beta * *c;
   } else {
-    float acc = 0.0f;
-    for (int kk = 0; kk < p.k; kk++) acc = __builtin_fmaf(a[kk * astep], b[kk * bstep], acc);
-    *c = p.beta == 0.0f ? p.alpha * acc : p.alpha * acc + p.beta * *c;
+    T acc = T(0);
+    for (int kk = 0; kk < p.k; kk++) acc = small_fma(a[kk * astep], b[kk * bstep], acc);
+    *c = p.beta == T(0) ? p.alpha * acc : p.alpha * acc + p.beta * *c;
   }
 }
 
 // Returns false (nothing launched) when the batch is not of this kind.
-bool try_sgemm_small_batch(bool ta, bool tb, long m, long n, long k, float alpha, const float* A, long lda, long sA,
-                           long sA2, const float* B, long ldb, long sB, long sB2, float beta, float* C, long ldc,
-                           long sC, long sC2, long batch, long batch2, int* rc) {
+template <class T>
+static bool try_small_batch(bool ta, bool tb, long m, long n, long k, T alpha, const T* A, long lda, long sA, long sA2,
+                            const T* B, long ldb, long sB, long sB2, T beta, T* C, long ldc, long sC, long sC2,
+                            long batch, long batch2, int* rc) {
   const int64_t nb = (int64_t)batch * batch2, outputs = (int64_t)m * n * nb;
   // outputs of at most 16 x 16 (4096 x (32 x 32) . (32 x 32): 39 us tiled, 86 us here), enough of them to fill
   // the chip with threads or, from K = 128 on, with wavefronts; K within a few thousand
   if (nb < 64 || m * n > 256 || k < 1 || k > 8192 || outputs >= ((int64_t)1 << 31) ||
       outputs < (k >= 128 ? 256 : 16384))
     return false;
-  SmallBatchParams p;
+  SmallBatchParams<T> p;
   p.A = A; p.B = B; p.C = C;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.sA = sA; p.sA2 = sA2; p.sB = sB; p.sB2 = sB2; p.sC = sC; p.sC2 = sC2;
@@ -612,11 +617,25 @@ bool try_sgemm_small_batch(bool ta, bool tb, long m, long n, long k, float alpha
   const FastDiv by_m = make_fastdiv((uint32_t)m), by_n = make_fastdiv((uint32_t)n);
   hipStream_t st = rt().stream;
   if (k >= 128)
-    sgemm_small_batch_kernel<true><<<(uint32_t)ceil_div(outputs, (int64_t)(kBlock / kWave)), kBlock, 0, st>>>(p, by_m, by_n);
+    sgemm_small_batch_kernel<T, true><<<(uint32_t)ceil_div(outputs, (int64_t)(kBlock / kWave)), kBlock, 0, st>>>(p, by_m, by_n);
   else
-    sgemm_small_batch_kernel<false><<<(uint32_t)ceil_div(outputs, (int64_t)kBlock), kBlock, 0, st>>>(p, by_m, by_n);
+    sgemm_small_batch_kernel<T, false><<<(uint32_t)ceil_div(outputs, (int64_t)kBlock), kBlock, 0, st>>>(p, by_m, by_n);
   *rc = after_launch("sgemm_small_batch_kernel");
   return true;
+}
+
+bool try_sgemm_small_batch(bool ta, bool tb, long m, long n, long k, float alpha, const float* A, long lda, long sA,
+                           long sA2, const float* B, long ldb, long sB, long sB2, float beta, float* C, long ldc,
+                           long sC, long sC2, long batch, long batch2, int* rc) {
+  return try_small_batch<float>(ta, tb, m, n, k, alpha, A, lda, sA, sA2, B, ldb, sB, sB2, beta, C, ldc, sC, sC2, batch,
+                                batch2, rc);
+}
+
+bool try_dgemm_small_batch(bool ta, bool tb, long m, long n, long k, double alpha, const double* A, long lda, long sA,
+                           long sA2, const double* B, long ldb, long sB, long sB2, double beta, double* C, long ldc,
+                           long sC, long sC2, long batch, long batch2, int* rc) {
+  return try_small_batch<double>(ta, tb, m, n, k, alpha, A, lda, sA, sA2, B, ldb, sB, sB2, beta, C, ldc, sC, sC2, batch,
+                                 batch2, rc);
 }
 
 }  // namespace wf2

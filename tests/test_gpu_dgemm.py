@@ -188,3 +188,25 @@ def test_double_matmul_few_outputs_long_k(gpu, m, n, k, ta, tb):
     C2 = Cm.reshape(n, ldc).T
     _check(got[:m, :], 0.5 * opA, opB, extra=-2.0 * C2[:m, :], what="column-major call")
     np.testing.assert_array_equal(got[m:, :], C2[m:, :])
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(20000, 4, 4, 4), (4096, 8, 8, 8), (300, 2, 3, 1000), (64, 16, 16, 200)])
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_double_matmul_many_small_matrices(gpu, batch, m, n, k, ta, tb):
+    """Batches of products with a few output elements each (an output element per thread, or per wavefront over
+    a longer K), against the product in extended precision."""
+    F = gpu.functional
+    rng = np.random.default_rng(batch + m + n + k)
+    A = rng.standard_normal((batch, k, m) if ta else (batch, m, k))
+    B = rng.standard_normal((batch, n, k) if tb else (batch, k, n))
+    a, b = D(A), D(B)
+    got = F.matmul(F.t(a) if ta else a, F.t(b) if tb else b).numpy()
+    opA = A.transpose(0, 2, 1) if ta else A
+    opB = B.transpose(0, 2, 1) if tb else B
+    want = opA @ opB
+    scale = np.abs(opA) @ np.abs(opB)
+    assert got.shape == (batch, m, n)
+    assert np.max(np.abs(got - want) / scale) <= 8 * k * EPS
+    for i in (0, batch // 2, batch - 1):
+        _check(got[i], opA[i], opB[i], what=f"matrix {i}, extended precision")
