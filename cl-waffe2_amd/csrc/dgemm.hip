@@ -155,6 +155,19 @@ bool try_dgemm_small_batch(bool ta, bool tb, long m, long n, long k, double alph
                            long sA2, const double* B, long ldb, long sB, long sB2, double beta, double* C, long ldc,
                            long sC, long sC2, long batch, long batch2, int* rc);  // gemm_skinny.hip
 
+// up to 16 planes: an output element per thread, the planes added in order
+__global__ __launch_bounds__(kBlock) void dgemm_fold_few(const double* __restrict__ partials, int splits, int64_t m,
+                                                         int64_t n, double beta, double* __restrict__ C, int64_t ldc) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= m * n) return;
+  const int64_t plane = m * n;
+  double acc = 0.0;
+  for (int s = 0; s < splits; s++) acc += partials[(int64_t)s * plane + e];
+  const int64_t j = e / m, i = e - j * m;
+  double* c = C + i + j * ldc;
+  *c = beta == 0.0 ? acc : beta * *c + acc;
+}
+
 static bool dn(char c) { return c == 'N' || c == 'n'; }
 static bool dt(char c) { return c == 'T' || c == 't' || c == 'C' || c == 'c'; }
 
@@ -210,8 +223,12 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
       launch_dgemm<64>(q, ta, tb, grid, st);
       int rc = after_launch("dgemm_kernel");
       if (rc == 0) {
-        dgemm_fold<<<(uint32_t)ceil_div((int64_t)m * n, kBlock / kWave), kBlock, 0, st>>>(
-            static_cast<const double*>(scratch), (int)splits, m, n, beta, C, ldc);
+        if (splits <= 16)
+          dgemm_fold_few<<<(uint32_t)ceil_div((int64_t)m * n, (int64_t)kBlock), kBlock, 0, st>>>(
+              static_cast<const double*>(scratch), (int)splits, m, n, beta, C, ldc);
+        else
+          dgemm_fold<<<(uint32_t)ceil_div((int64_t)m * n, kBlock / kWave), kBlock, 0, st>>>(
+              static_cast<const double*>(scratch), (int)splits, m, n, beta, C, ldc);
         rc = after_launch("dgemm_fold");
       }
       (void)wf2hip_free(scratch);  // stream order keeps it alive for the launches above
