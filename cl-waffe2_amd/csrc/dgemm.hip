@@ -204,8 +204,9 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
   // workgroup): slices of K of at least 512, as many as keep four workgroups per compute unit, each into a
   // plane of its own, folded in a fixed order afterwards.
   const int64_t small_tiles = ceil_div(m, 64) * ceil_div(n, 64);
-  if (batch == 1 && batch2 == 1 && k >= 2048 && small_tiles < (int64_t)rt().num_cus) {
-    int64_t splits = std::min<int64_t>(k / 512, 4 * (int64_t)rt().num_cus / small_tiles);
+  // (K of 512 ... 2047, a layer applied to a few hundred rows: slices of at least 256)
+  if (batch == 1 && batch2 == 1 && k >= 512 && small_tiles < (int64_t)rt().num_cus) {
+    int64_t splits = std::min<int64_t>(k / (k >= 2048 ? 512 : 256), 4 * (int64_t)rt().num_cus / small_tiles);
     splits = std::min<int64_t>(splits, 4096);
     const int64_t kslice = ceil_div(ceil_div(k, splits), (int64_t)kDK) * kDK;
     splits = ceil_div(k, kslice);
