@@ -1455,13 +1455,20 @@ static int launch_softmax_wave(int nv, uint32_t blocks, const float* x, int64_t 
 // (no causal form; labels and loss are contiguous rows of ncols).
 // ---- rows of at most 64 columns (class scores: softmax over 10 classes) -----------------------------
 // A wavefront per row -- or per four rows -- leaves most lanes idle on such rows ((1677721, 10): softmax 361
-// us, 11 % of what its bytes take).  Here a workgroup takes 256 adjacent rows (128 beyond 32 columns): their storage, one contiguous
+// us, 11 % of what its bytes take).  Here a workgroup takes 256 adjacent rows (up to 1024 of a few columns, 128 beyond 32 columns): their storage, one contiguous
 // run, is staged into LDS in storage order (row r at r * (ncols | 1): the odd pitch keeps the 64 rows of a
 // wavefront on different banks), thread r works through row r there, and the run is written back in storage
 // order.  Rows must be adjacent in x and in every output (pitch == ncols).
 constexpr int kTinyCols = 64;
 constexpr int kTinyFloats = 256 * 33;  // >= 128 * 65
-__host__ __device__ inline int tiny_rows_per_group(int ncols) { return ncols <= 32 ? 256 : 128; }
+// rows per workgroup: as many whole rounds of 256 rows (at most four) as the tile holds -- rows of two columns
+// in groups of 256 are 2 KB of work per workgroup, and the launch rate bounds the kernel ((8388608, 2): 55 us)
+__host__ __device__ inline int tiny_rows_per_group(int ncols) {
+  if (ncols > 32) return 128;
+  if (ncols > 8) return 256;  // (1677721, 10): 26 us in groups of 256, 30 us in groups of 768
+  const int rounds = 33 / (ncols | 1);
+  return 256 * (rounds > 4 ? 4 : rounds);
+}
 enum { kTinySoftmax = 0, kTinyXent = 1, kTinyLayerNorm = 2 };
 
 struct TinyRows {
@@ -1530,8 +1537,8 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
     }
   }
   __syncthreads();
-  if ((int)threadIdx.x < rows_here) {
-    float* r = tile + threadIdx.x * pitch;
+  for (int mine = threadIdx.x; mine < rows_here; mine += kBlock) {
+    float* r = tile + mine * pitch;
     if constexpr (MODE == kTinyLayerNorm) {
       // binary32 statistics, as the several-rows-per-wavefront form of layernorm_rows_wave
       float sum = 0.0f;
