@@ -62,7 +62,14 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_wave(const float* __r
 // three.
 constexpr int kTinyCols = 64;
 constexpr int kTinyFloats = 128 * 33;  // >= 64 * 65
-__host__ __device__ inline int tiny_rows_per_group(int ncols) { return ncols <= 32 ? 128 : 64; }
+// rows per workgroup: up to four rounds of 128 rows on rows of at most 8 columns (a group of 128 rows of two
+// columns is 1 KB per tensor: the launch rate bounds the kernels)
+__host__ __device__ inline int tiny_rows_per_group(int ncols) {
+  if (ncols > 32) return 64;
+  if (ncols > 8) return 128;
+  const int rounds = 33 / (ncols | 1);
+  return 128 * (rounds > 4 ? 4 : rounds);
+}
 
 // VEC: y, dy and dx are 16-byte aligned: the runs are staged in 16-byte vectors.
 template <bool VEC>
@@ -123,9 +130,9 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __r
       }
   }
   __syncthreads();
-  if ((int)threadIdx.x < rows_here) {
-    float* a = ty + threadIdx.x * pitch;
-    const float* b = td + threadIdx.x * pitch;
+  for (int mine = threadIdx.x; mine < rows_here; mine += kBlock) {
+    float* a = ty + mine * pitch;
+    const float* b = td + mine * pitch;
     double acc = 0.0;
     for (int j = 0; j < ncols; j++) acc += (double)(b[j] * a[j]);
     const float dot = (float)acc;
@@ -422,7 +429,8 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __rest
   __shared__ float tx[kTinyFloats];
   __shared__ float td[kTinyFloats];
   __shared__ float row_rstd[128], row_m1[128], row_m2[128];
-  const int pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  // groups of 128 rows (64 beyond 32 columns) whatever the width
+  const int pitch = ncols | 1, group = ncols <= 32 ? 128 : 64;
   const int64_t ngroups = (nrows + group - 1) / group;
   const float inv_n = 1.0f / (float)ncols;
   float dg = 0.0f, db = 0.0f;  // threads 0 .. ncols - 1: the column sums over this workgroup's rows
@@ -451,9 +459,9 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __rest
         }
     }
     __syncthreads();
-    if ((int)threadIdx.x < rows_here) {
-      float* xr = tx + threadIdx.x * pitch;
-      const float* dr = td + threadIdx.x * pitch;
+    for (int mine = threadIdx.x; mine < rows_here; mine += kBlock) {
+      float* xr = tx + mine * pitch;
+      const float* dr = td + mine * pitch;
       double sum = 0.0;
       for (int j = 0; j < ncols; j++) sum += (double)xr[j];
       const float mean = (float)(sum / (double)ncols);
@@ -472,9 +480,9 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __rest
         s1 += dyh;
         s2 = __builtin_fmaf(dyh, xh, s2);
       }
-      row_rstd[threadIdx.x] = rstd;
-      row_m1[threadIdx.x] = s1 * inv_n;
-      row_m2[threadIdx.x] = s2 * inv_n;
+      row_rstd[mine] = rstd;
+      row_m1[mine] = s1 * inv_n;
+      row_m2[mine] = s2 * inv_n;
     }
     __syncthreads();
     if ((int)threadIdx.x < ncols) {
@@ -856,7 +864,7 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // three to eight (more rows of `partial` to write and fold)
   const bool tiny = cols <= kTinyCols && rows >= 16384;
   const int64_t blocks = wide ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
-                         : tiny ? std::min<int64_t>(ceil_div((int64_t)rows, (int64_t)tiny_rows_per_group((int)cols)),
+                         : tiny ? std::min<int64_t>(ceil_div((int64_t)rows, (int64_t)(cols <= 32 ? 128 : 64)),
                                                     4 * (int64_t)std::max(rt().num_cus, 1))
                               : std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
   const size_t partial_bytes = (size_t)blocks * 2 * cols * sizeof(float);
