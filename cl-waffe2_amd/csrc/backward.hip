@@ -64,7 +64,7 @@ constexpr int kTinyCols = 64;
 constexpr int kTinyFloats = 128 * 33;  // >= 64 * 65
 // rows per workgroup: up to four rounds of 128 rows on rows of at most 8 columns (a group of 128 rows of two
 // columns is 1 KB per tensor: the launch rate bounds the kernels)
-__host__ __device__ inline int tiny_rows_per_group(int ncols) {
+__host__ __device__ static inline int tiny_bwd_rows_per_group(int ncols) {
   if (ncols > 32) return 64;
   if (ncols > 8) return 128;
   const int rounds = 33 / (ncols | 1);
@@ -78,8 +78,9 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_tiny(const float* __r
                                                                 FastDiv by_c) {
   __shared__ float ty[kTinyFloats];
   __shared__ float td[kTinyFloats];
-  const int pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  const int pitch = ncols | 1, group = tiny_bwd_rows_per_group(ncols);
   const int64_t row0 = (int64_t)blockIdx.x * group;
+  if (row0 >= nrows) return;  // a grid sized for other groups must not index past the rows
   const int rows_here = (int)(nrows - row0 < group ? nrows - row0 : group);
   const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
   const int64_t base = row0 * ncols;
@@ -783,7 +784,7 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
   if (xlo < dhi && dlo < xhi && !(dx == dy && lddx == lddy))
     return fail(WF2HIP_EOVERLAP, "softmax backward: dx overlaps dy without being dy");
   if (cols <= kTinyCols && causal_seq == 0 && rows >= 16384 && ldy == cols && lddy == cols && lddx == cols) {
-    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols));
+    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_bwd_rows_per_group((int)cols));
     if (aligned16(y) && aligned16(dy) && aligned16(dx))
       softmax_bwd_rows_tiny<true><<<groups, kBlock, 0, rt().stream>>>(y, dy, dx, rows, (int)cols, scale,
                                                                         make_fastdiv((uint32_t)cols));
@@ -799,7 +800,10 @@ WF2_API int wf2hip_softmax_backward_rows_f32(long rows, long cols, const float* 
     if (causal_seq == 0 && (cols > 32 * kLongBlock || (pieces >= 2 && rows < rt().num_cus)) &&
         rows * pieces < ((int64_t)1 << 31)) {
       void* pdot = nullptr;
-      if (wf2hip_malloc_uninitialized(&pdot, (size_t)(rows * pieces) * sizeof(double)) == 0) {
+      int held_up = 0;
+      if (!scratch_block(&pdot, (size_t)(rows * pieces) * sizeof(double), &held_up)) {
+        if (held_up) return held_up;
+      } else {
         const uint32_t grid = (uint32_t)(rows * pieces);
         softmax_bwd_split_dot<<<grid, kLongBlock, 0, st>>>(y, ldy, dy, lddy, cols, (uint32_t)pieces,
                                                            static_cast<double*>(pdot));

@@ -211,7 +211,10 @@ static int dgemm_batched2(char transa, char transb, long m, long n, long k, doub
     const int64_t kslice = ceil_div(ceil_div(k, splits), (int64_t)kDK) * kDK;
     splits = ceil_div(k, kslice);
     void* scratch = nullptr;
-    if (splits >= 2 && wf2hip_malloc_uninitialized(&scratch, (size_t)splits * m * n * sizeof(double)) == 0) {
+    int held_up = 0;
+    if (splits >= 2 && !scratch_block(&scratch, (size_t)splits * m * n * sizeof(double), &held_up) && held_up)
+      return held_up;
+    if (scratch) {
       DgemmParams q = p;
       q.C = static_cast<double*>(scratch);
       q.ldc = m;

@@ -987,7 +987,7 @@ static bool try_split_k(char transa, char transb, long m, long n, long k, float 
   const long planes = splits + (rest ? 1 : 0);
   const int64_t plane = (int64_t)m * n;
   void* scratch = nullptr;
-  if (wf2hip_malloc_uninitialized(&scratch, (size_t)(planes * batch * plane) * sizeof(float)) != 0) return false;
+  if (!scratch_block(&scratch, (size_t)(planes * batch * plane) * sizeof(float), rc)) return *rc != 0;
   float* part = static_cast<float*>(scratch);
   const long sa = is_n(transa) ? kc * lda : kc;  // op(A) is m x k: a K slice starts kc columns / rows further
   const long sb = is_n(transb) ? kc : kc * ldb;
@@ -1066,7 +1066,9 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   if (batch == 1 && batch2 == 1 && !is_n(transb) && k >= 1024 && k % BK == 0 && n >= 128 && m >= 128 &&
       aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && (is_n(transa) ? m % 4 == 0 : true)) {
     void* turned = nullptr;
-    if (wf2hip_malloc_uninitialized(&turned, (size_t)k * n * sizeof(float)) == 0) {
+    int held_up = 0;
+    if (!scratch_block(&turned, (size_t)k * n * sizeof(float), &held_up) && held_up) return held_up;
+    if (turned) {
       Space sp;  // dst (k x n column-major): (kk, j) at kk + j k; src (n x k): j + kk ldb
       sp.rank = 2;
       sp.shape[0] = n;

@@ -406,7 +406,7 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   if (blocks >= ((int64_t)1 << 31)) return false;
   void* scratch = nullptr;
   if (gsplit > 1) {
-    if (wf2hip_malloc_uninitialized(&scratch, (size_t)(gsplit * rows * cols) * sizeof(float)) != 0) return false;
+    if (!scratch_block(&scratch, (size_t)(gsplit * rows * cols) * sizeof(float), rc)) return *rc != 0;
     p.partial = static_cast<float*>(scratch);
   }
   hipStream_t st = rt().stream;
@@ -532,7 +532,7 @@ bool try_sgemm_tiny_out(long rows, long cols, long k, float alpha, const float* 
   p.kslice = ceil_div(ceil_div((int64_t)k, groups), (int64_t)p.chunk) * p.chunk;
   groups = ceil_div((int64_t)k, p.kslice);
   void* scratch = nullptr;
-  if (wf2hip_malloc_uninitialized(&scratch, (size_t)(groups * rows * cols) * sizeof(float)) != 0) return false;
+  if (!scratch_block(&scratch, (size_t)(groups * rows * cols) * sizeof(float), rc)) return *rc != 0;
   p.partial = static_cast<float*>(scratch);
   const size_t lds = (size_t)p.chunk * (rows + cols) * sizeof(float);
   const FastDiv by_rows = make_fastdiv((uint32_t)rows), by_cols = make_fastdiv((uint32_t)cols);

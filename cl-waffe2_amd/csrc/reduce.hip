@@ -585,10 +585,10 @@ static int launch_col_reduce(const AccParams& p, int64_t ncols, bool narrow = fa
   if (ctiles * splits >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "iteration space too large");
   void* scratch = nullptr;
   if (splits > 1) {
-    // no block to be had (inside a graph capture the pool is the only source): one
-    // workgroup per column tile instead
-    if (wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(double)) != 0) {
-      scratch = nullptr;
+    // no block to be had (out of memory): one workgroup per column tile instead
+    int held_up = 0;
+    if (!scratch_block(&scratch, (size_t)(splits * ncols) * sizeof(double), &held_up)) {
+      if (held_up) return held_up;
       splits = 1;
       q.splits = 1;
       q.seg = p.nred;
@@ -758,8 +758,10 @@ static int launch_row_reduce(const Space& s, float* a, const float* b, double* p
 
 // a <- a op b where `a` has broadcast (stride-0) axes.  `s` is normalised.
 // `row_partials` replaces the library's partial-sum buffer for the row form.
+// may_allocate == false: only the paths that need no scratch beyond row_partials (the row form, the
+// sequential form and the wavefront-per-destination form) -- what the allocation-free entry point may use.
 static int launch_accumulate_with(int op, const Space& s, float* a, const float* b, double* row_partials,
-                                  Commit commit = Commit{0, 1.0f}) {
+                                  Commit commit = Commit{0, 1.0f}, bool may_allocate = true) {
   hipStream_t st = rt().stream;
   const bool sequential = op != WF2HIP_ADD || rt().reduce_mode == 1;
   AccParams p;
@@ -788,6 +790,13 @@ static int launch_accumulate_with(int op, const Space& s, float* a, const float*
   for (int r = 0; r < last; r++)
     if (s.shape[r] >= ((int64_t)1 << 32)) row_form = false;
   if (row_form) return launch_row_reduce(s, a, b, row_partials, commit);
+  if (!may_allocate) {
+    int64_t blocks = ceil_div(p.nout, kWavesPerBlock);
+    if (blocks >= ((int64_t)1 << 31))
+      return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
+    accumulate_generic<<<(uint32_t)blocks, kBlock, 0, st>>>(p);
+    return after_launch("accumulate_generic");
+  }
   // column form: the only kept axis is the last one, contiguous on both sides
   if (p.nk == 1 && s.sa[last] == 1 && s.sb[last] == 1 && s.shape[last] <= 128 && p.nr == 1 &&
       p.rb[0] == s.shape[last] && p.nred >= 16)
@@ -802,7 +811,10 @@ static int launch_accumulate_with(int op, const Space& s, float* a, const float*
       const int64_t seg = ceil_div(ceil_div(p.nred, splits), kBlock) * kBlock;
       splits = ceil_div(p.nred, seg);
       void* scratch = nullptr;
-      if (splits > 1 && wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * p.nout) * sizeof(double)) == 0) {
+      int held_up = 0;
+      if (splits > 1 && !scratch_block(&scratch, (size_t)(splits * p.nout) * sizeof(double), &held_up) && held_up)
+        return held_up;
+      if (scratch) {
         accumulate_partial<<<(uint32_t)(p.nout * splits), kBlock, 0, st>>>(p, (uint32_t)splits, (uint32_t)seg,
                                                                           static_cast<double*>(scratch));
         int rc = after_launch("accumulate_partial");
@@ -1463,7 +1475,7 @@ constexpr int kTinyCols = 64;
 constexpr int kTinyFloats = 256 * 33;  // >= 128 * 65
 // rows per workgroup: as many whole rounds of 256 rows (at most four) as the tile holds -- rows of two columns
 // in groups of 256 are 2 KB of work per workgroup, and the launch rate bounds the kernel ((8388608, 2): 55 us)
-__host__ __device__ inline int tiny_rows_per_group(int ncols) {
+__host__ __device__ static inline int tiny_fwd_rows_per_group(int ncols) {
   if (ncols > 32) return 128;
   if (ncols > 8) return 256;  // (1677721, 10): 26 us in groups of 256, 30 us in groups of 768
   const int rounds = 33 / (ncols | 1);
@@ -1487,8 +1499,9 @@ struct TinyRows {
 template <int MODE, bool VEC>
 __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
   __shared__ float tile[kTinyFloats];
-  const int ncols = a.ncols, pitch = ncols | 1, group = tiny_rows_per_group(ncols);
+  const int ncols = a.ncols, pitch = ncols | 1, group = tiny_fwd_rows_per_group(ncols);
   const int64_t row0 = (int64_t)blockIdx.x * group;
+  if (row0 >= a.nrows) return;  // a grid sized for other groups must not index past the rows
   const int rows_here = (int)(a.nrows - row0 < group ? a.nrows - row0 : group);
   const uint32_t cells = (uint32_t)rows_here * (uint32_t)ncols;
   const int64_t base = row0 * ncols;
@@ -1540,18 +1553,19 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
   for (int mine = threadIdx.x; mine < rows_here; mine += kBlock) {
     float* r = tile + mine * pitch;
     if constexpr (MODE == kTinyLayerNorm) {
-      // binary32 statistics, as the several-rows-per-wavefront form of layernorm_rows_wave
-      float sum = 0.0f;
-      for (int j = 0; j < ncols; j++) sum += r[j];
-      const float mean = sum / (float)ncols;
+      // the statistics of layernorm_bwd_tiny, operation for operation, so that the backward's xh is the
+      // forward's: the mean from a binary64 sum, deviations and their squares in binary32
+      double sum = 0.0;
+      for (int j = 0; j < ncols; j++) sum += (double)r[j];
+      const float mean = (float)(sum / (double)ncols);
       float sq = 0.0f;
       for (int j = 0; j < ncols; j++) {
         const float d = r[j] - mean;
+        r[j] = d;
         sq = __builtin_fmaf(d, d, sq);
       }
-      const float var = sq / (float)ncols;
-      const float rstd = (float)(1.0 / __builtin_sqrt((double)var + (double)a.param));
-      for (int j = 0; j < ncols; j++) r[j] = __builtin_fmaf((r[j] - mean) * rstd, a.aux0[j], a.aux1[j]);
+      const float rstd = (float)(1.0 / __builtin_sqrt((double)sq / (double)ncols + (double)a.param));
+      for (int j = 0; j < ncols; j++) r[j] = __builtin_fmaf(r[j] * rstd, a.aux0[j], a.aux1[j]);
     } else {
       float m = -__builtin_inff();
       for (int j = 0; j < ncols; j++) m = fmaxf(m, r[j]);
@@ -1626,7 +1640,7 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
   if (ncols <= kTinyCols && ldx == ncols && ldo == ncols && causal_seq == 0 && nrows >= kTinyMinRows &&
       ceil_div(nrows, 128) < ((int64_t)1 << 31)) {
     TinyRows a{x, out, xe.labels, nullptr, xe.loss, xe.delta, nrows, (int)ncols};
-    const uint32_t groups = (uint32_t)ceil_div(nrows, tiny_rows_per_group((int)ncols));
+    const uint32_t groups = (uint32_t)ceil_div(nrows, tiny_fwd_rows_per_group((int)ncols));
     if (aligned16(x) && aligned16(out) && (!XENT || (aligned16(xe.labels) && aligned16(xe.loss))))
       rows_tiny<XENT ? kTinyXent : kTinySoftmax, true><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)ncols));
     else
@@ -1831,7 +1845,7 @@ WF2_API int wf2hip_reduce_add_rows_f32_noalloc(long rows, long cols, const float
     return fail(WF2HIP_EOVERLAP, "row sums into a window that overlaps the source");
   // cols == 1 leaves no reduced axis: a plain strided add, which uses no scratch
   if (!has_broadcast_axis(s, s.sa)) return binary_nd(WF2HIP_ADD, s, out, x);
-  return launch_accumulate_with(WF2HIP_ADD, s, out, x, partials);
+  return launch_accumulate_with(WF2HIP_ADD, s, out, x, partials, Commit{0, 1.0f}, false);
 }
 
 WF2_API int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long ldx, float* out,
@@ -1868,7 +1882,7 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
   if (!x || !gamma || !beta || !out) return fail(WF2HIP_EINVAL, "null pointer");
   if (cols <= kTinyCols && rows >= kTinyMinRows) {
     TinyRows a{x, out, gamma, beta, nullptr, eps, rows, (int)cols};
-    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_rows_per_group((int)cols));
+    const uint32_t groups = (uint32_t)ceil_div((int64_t)rows, tiny_fwd_rows_per_group((int)cols));
     if (aligned16(x) && aligned16(out))
       rows_tiny<kTinyLayerNorm, true><<<groups, kBlock, 0, rt().stream>>>(a, make_fastdiv((uint32_t)cols));
     else

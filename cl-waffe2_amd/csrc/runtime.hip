@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "wf2_common.h"
+#include "wf2_pool.h"
 
 namespace wf2 {
 
@@ -46,83 +47,40 @@ int require_init() {
 }
 
 // ---- caching allocator -------------------------------------------------------
-// cl-waffe2 allocates a compiled model's temporaries once and reuses them on
-// every forward (maybe-allocate!, source/vm/allocation.lisp:121-145); a host
-// that allocates per call gets the same steady state from this pool.  Blocks
-// are recycled without synchronising: every kernel and copy of the library
-// runs on one stream, so a recycled block's new user is ordered after its old
-// one.  hipFree (which does synchronise) only happens on trim/shutdown or when
-// the device is out of memory.
-// A captured graph keeps the blocks its kernels were recorded with: every block
-// handed out during a capture is registered to that graph, and when such a block is
-// freed -- during the capture or at any time after it, e.g. when the host's collector
-// finalises a result it dropped -- it is parked in the graph's `held` list instead of
-// the idle pool.  Parked blocks are re-usable by later allocations of the same capture
-// (a replay preserves the recorded order) and only return to the pool when the graph
-// is destroyed: until then every replay still writes into them, and an eager
-// allocation that received one would be silently overwritten.
-struct Graph {
+// The bookkeeping (idle blocks, blocks that captured graphs still write into) is
+// BlockPool, wf2_pool.h.  Blocks are recycled without synchronising: every kernel and
+// copy of the library runs on one stream, so a recycled block's new user is ordered
+// after its old one.  hipFree (which does synchronise) only happens on trim/shutdown
+// or when the device is out of memory.
+struct Graph : GraphBlocks {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
-  std::multimap<size_t, void*> held;
 };
 static Graph* g_capture = nullptr;  // non-null between graph_begin and graph_end
-static std::vector<Graph*> g_destroy_after_capture;  // graphs released while another was being recorded (guarded by g_pool.mu)
-static std::unordered_map<void*, Graph*> g_graph_blocks;  // block -> the live graph recorded with it (guarded by g_pool.mu)
+static std::vector<Graph*> g_destroy_after_capture;  // graphs released while another was being recorded (guarded by g_pool_mu)
 
-struct Pool {
-  std::mutex mu;
-  std::multimap<size_t, void*> idle;          // size class -> block
-  std::unordered_map<void*, size_t> size_of;  // every block handed out or idle
-  size_t idle_bytes = 0;
-  bool enabled = true;
-};
-static Pool g_pool;
-
-static size_t size_class(size_t bytes) {
-  const size_t small = 512, large = (size_t)2 << 20;
-  if (bytes < ((size_t)1 << 20)) return (bytes + small - 1) / small * small;
-  return (bytes + large - 1) / large * large;
-}
+static std::mutex g_pool_mu;
+static BlockPool g_pool;  // guarded by g_pool_mu
+static size_t g_pool_requests = 0;  // guarded by g_pool_mu
 
 static void pool_release_idle_locked() {
-  for (auto& kv : g_pool.idle) {
-    (void)hipFree(kv.second);
-    g_pool.size_of.erase(kv.second);
-  }
-  g_pool.idle.clear();
-  g_pool.idle_bytes = 0;
+  std::vector<void*> release;
+  g_pool.drain_idle(&release);
+  for (void* ptr : release) (void)hipFree(ptr);
 }
 
 static int pool_alloc(void** ptr, size_t bytes) {
-  const size_t cls = size_class(bytes);
-  std::lock_guard<std::mutex> lock(g_pool.mu);
-  if (g_capture) {
-    auto held = g_capture->held.find(cls);
-    if (held != g_capture->held.end()) {
-      *ptr = held->second;
-      g_capture->held.erase(held);
-      return 0;
-    }
-  }
-  if (g_pool.enabled) {
-    auto it = g_pool.idle.find(cls);
-    if (it != g_pool.idle.end()) {
-      *ptr = it->second;
-      g_pool.idle.erase(it);
-      g_pool.idle_bytes -= cls;
-      if (g_capture) g_graph_blocks[*ptr] = g_capture;
-      return 0;
-    }
-  }
-  if (g_capture) {
-    *ptr = nullptr;
+  const size_t cls = BlockPool::size_class(bytes);
+  std::lock_guard<std::mutex> lock(g_pool_mu);
+  g_pool_requests++;
+  *ptr = g_pool.take(cls, g_capture);
+  if (*ptr) return 0;
+  if (g_capture)
     return fail(WF2HIP_ECAPTURE,
                 "a %zu-byte block is not in the pool and hipMalloc cannot run during graph "
                 "capture: run the sequence once before capturing it", bytes);
-  }
   hipError_t e = hipMalloc(ptr, cls);
-  if (e == hipErrorOutOfMemory && !g_pool.idle.empty()) {
+  if (e == hipErrorOutOfMemory && g_pool.has_idle()) {
     (void)hipGetLastError();
     (void)hipStreamSynchronize(g_rt.stream);
     pool_release_idle_locked();
@@ -134,31 +92,19 @@ static int pool_alloc(void** ptr, size_t bytes) {
     return fail(WF2HIP_ENOMEM, "out of device memory allocating %zu bytes", bytes);
   }
   WF2_TRY(check_hip(e, "hipMalloc"));
-  g_pool.size_of[*ptr] = cls;
+  g_pool.adopt(*ptr, cls);
   return 0;
 }
 
 static int pool_free(void* ptr) {
-  std::lock_guard<std::mutex> lock(g_pool.mu);
-  auto it = g_pool.size_of.find(ptr);
-  if (it == g_pool.size_of.end())
+  BlockPool::Outcome what;
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mu);
+    what = g_pool.give_back(ptr, g_capture);
+  }
+  if (what == BlockPool::kUnknown)
     return fail(WF2HIP_EINVAL, "wf2hip_free: %p was not allocated by wf2hip_malloc", ptr);
-  if (g_capture) {
-    g_graph_blocks[ptr] = g_capture;  // also a block from before the capture: its last use may be recorded
-    g_capture->held.emplace(it->second, ptr);
-    return 0;
-  }
-  auto owner = g_graph_blocks.find(ptr);
-  if (owner != g_graph_blocks.end()) {
-    owner->second->held.emplace(it->second, ptr);
-    return 0;
-  }
-  if (g_pool.enabled) {
-    g_pool.idle.emplace(it->second, ptr);
-    g_pool.idle_bytes += it->second;
-    return 0;
-  }
-  g_pool.size_of.erase(it);
+  if (what == BlockPool::kKept) return 0;
   WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
   return check_hip(hipFree(ptr), "hipFree");
 }
@@ -219,7 +165,7 @@ WF2_API int wf2hip_shutdown(void) {
   if (!g_rt.initialised) return 0;
   (void)hipStreamSynchronize(g_rt.stream);
   {
-    std::lock_guard<std::mutex> pool_lock(g_pool.mu);
+    std::lock_guard<std::mutex> pool_lock(g_pool_mu);
     pool_release_idle_locked();
   }
   if (g_rt.partials) (void)hipFree(g_rt.partials);
@@ -231,14 +177,19 @@ WF2_API int wf2hip_shutdown(void) {
 WF2_API int wf2hip_pool_trim(void) {
   WF2_TRY(require_init());
   WF2_TRY(check_hip(hipStreamSynchronize(g_rt.stream), "hipStreamSynchronize"));
-  std::lock_guard<std::mutex> lock(g_pool.mu);
+  std::lock_guard<std::mutex> lock(g_pool_mu);
   pool_release_idle_locked();
   return 0;
 }
 
 WF2_API size_t wf2hip_pool_idle_bytes(void) {
-  std::lock_guard<std::mutex> lock(g_pool.mu);
-  return g_pool.idle_bytes;
+  std::lock_guard<std::mutex> lock(g_pool_mu);
+  return g_pool.idle_bytes();
+}
+
+WF2_API size_t wf2hip_pool_requests(void) {
+  std::lock_guard<std::mutex> lock(g_pool_mu);
+  return g_pool_requests;
 }
 
 WF2_API int wf2hip_device_info(char* buf, size_t buflen) {
@@ -376,7 +327,7 @@ WF2_API int wf2hip_get_reduce_mode(void) { return g_rt.reduce_mode; }
 
 WF2_API int wf2hip_graph_begin(void) {
   WF2_TRY(require_init());
-  std::lock_guard<std::mutex> lock(g_pool.mu);
+  std::lock_guard<std::mutex> lock(g_pool_mu);
   if (g_capture) return fail(WF2HIP_ECAPTURE, "a capture is already in progress");
   if (g_rt.stream == nullptr)
     return fail(WF2HIP_ECAPTURE, "the null stream cannot be captured; use the library's own stream");
@@ -397,7 +348,7 @@ WF2_API int wf2hip_graph_end(void** graph) {
   *graph = nullptr;
   Graph* g;
   {
-    std::lock_guard<std::mutex> lock(g_pool.mu);
+    std::lock_guard<std::mutex> lock(g_pool_mu);
     g = g_capture;
     g_capture = nullptr;
   }
@@ -406,7 +357,7 @@ WF2_API int wf2hip_graph_end(void** graph) {
   {
     std::vector<Graph*> waiting;
     {
-      std::lock_guard<std::mutex> lock(g_pool.mu);
+      std::lock_guard<std::mutex> lock(g_pool_mu);
       waiting.swap(g_destroy_after_capture);
     }
     for (Graph* old : waiting) (void)wf2hip_graph_destroy(old);
@@ -435,7 +386,7 @@ WF2_API int wf2hip_graph_destroy(void* graph) {
   {
     // Destroying a graph synchronises the stream, which a capture in progress does not survive (a handle
     // rebound inside a recording, `with Graph() as g:` over an older g): it waits for wf2hip_graph_end.
-    std::lock_guard<std::mutex> lock(g_pool.mu);
+    std::lock_guard<std::mutex> lock(g_pool_mu);
     if (g_capture && g != g_capture) {
       g_destroy_after_capture.push_back(g);
       return 0;
@@ -446,18 +397,10 @@ WF2_API int wf2hip_graph_destroy(void* graph) {
   if (g->exec) (void)hipGraphExecDestroy(g->exec);
   if (g->graph) (void)hipGraphDestroy(g->graph);
   {
-    std::lock_guard<std::mutex> lock(g_pool.mu);
-    for (auto it = g_graph_blocks.begin(); it != g_graph_blocks.end();)
-      it = it->second == g ? g_graph_blocks.erase(it) : std::next(it);
-    for (auto& kv : g->held) {
-      if (g_pool.enabled) {
-        g_pool.idle.emplace(kv.first, kv.second);
-        g_pool.idle_bytes += kv.first;
-      } else {
-        g_pool.size_of.erase(kv.second);
-        (void)hipFree(kv.second);
-      }
-    }
+    std::lock_guard<std::mutex> lock(g_pool_mu);
+    std::vector<void*> release;
+    g_pool.forget_graph(g, &release);
+    for (void* ptr : release) (void)hipFree(ptr);
   }
   delete g;
   return 0;

@@ -771,8 +771,9 @@ static int run_accumulate(int op, const Space& s, T* a, const T* b) {
       int64_t seg = ceil_div(p.nred, splits);
       splits = ceil_div(p.nred, seg);
       void* scratch = nullptr;
-      if (splits > 1 && wf2hip_malloc_uninitialized(&scratch, (size_t)(splits * ncols) * sizeof(S)) != 0) {
-        scratch = nullptr;
+      int held_up = 0;
+      if (splits > 1 && !scratch_block(&scratch, (size_t)(splits * ncols) * sizeof(S), &held_up)) {
+        if (held_up) return held_up;
         splits = 1;
         seg = p.nred;
       }

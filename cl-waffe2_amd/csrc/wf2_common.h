@@ -43,6 +43,19 @@ inline int after_launch(const char* what) { return check_hip(hipGetLastError(), 
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Scratch for a faster route of a kernel that also has a route without scratch.  true: *ptr is the block
+// (release it with wf2hip_free once the launches that use it are enqueued).  false with *rc == 0: the device is
+// out of memory and the caller takes its other route.  false with *rc != 0: a graph capture is in progress and
+// the pool holds no such block -- the caller gives up with that code, because a route chosen by what the pool
+// happens to hold would let an eager run and a replay of the same node round differently.
+inline bool scratch_block(void** ptr, size_t bytes, int* rc) {
+  *rc = wf2hip_malloc_uninitialized(ptr, bytes);
+  if (*rc == 0) return true;
+  if (*rc != WF2HIP_ECAPTURE) *rc = 0;
+  *ptr = nullptr;
+  return false;
+}
+
 }  // namespace wf2
 
 #define WF2_TRY(expr)            \

@@ -116,6 +116,7 @@ _SIGNATURES = {
     "wf2hip_free": ([_P], C.c_int),
     "wf2hip_pool_trim": ([], C.c_int),
     "wf2hip_pool_idle_bytes": ([], C.c_size_t),
+    "wf2hip_pool_requests": ([], C.c_size_t),
     "wf2hip_memcpy_h2d": ([_P, _P, C.c_size_t], C.c_int),
     "wf2hip_memcpy_d2h": ([_P, _P, C.c_size_t], C.c_int),
     "wf2hip_memcpy_d2d": ([_P, _P, C.c_size_t], C.c_int),

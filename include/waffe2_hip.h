@@ -73,6 +73,10 @@ int wf2hip_free(void* ptr);
 /* Give idle pooled blocks back to the device (synchronises). */
 int wf2hip_pool_trim(void);
 size_t wf2hip_pool_idle_bytes(void);
+/* Number of block requests (wf2hip_malloc, wf2hip_malloc_uninitialized and the library's own scratch) served
+ * since the library was loaded, from the pool or from the device: a caller can check that a sequence it
+ * means to capture, or an entry point that promises not to allocate, asked for nothing. */
+size_t wf2hip_pool_requests(void);
 int wf2hip_memcpy_h2d(void* dst, const void* src, size_t bytes);
 int wf2hip_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int wf2hip_memcpy_d2d(void* dst, const void* src, size_t bytes);

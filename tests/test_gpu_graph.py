@@ -151,3 +151,49 @@ def test_graph_released_during_a_recording(gpu):
     for i in range(2):
         g.launch()
         assert_bit_equal(second.numpy(), eager, f"second graph, replay {i}")
+
+
+@pytest.mark.parametrize("rows", [128, 256, 512])
+def test_layer_replay_equals_eager_bit_for_bit(gpu, rows):
+    """A Linear layer on a few hundred rows runs as slices of K folded in a fixed order, the slice count chosen
+    from the shape (so its bits depend on the number of rows fed through it).  Captured after a warm-up, every
+    replay must equal the eager result bit for bit: the route never depends on what the pool happens to hold."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(rows)
+    x = F.from_numpy(rng.standard_normal((rows, 768)).astype(np.float32))
+    w = F.from_numpy((0.02 * rng.standard_normal((768, 2304))).astype(np.float32))
+    b = F.from_numpy(rng.standard_normal(2304).astype(np.float32))
+    eager = F.linear(x, w, b, activation="gelu").numpy()
+    with W.lib.Graph() as g:
+        out = F.linear(x, w, b, activation="gelu")
+    for i in range(2):
+        g.launch()
+        assert_bit_equal(out.numpy(), eager, f"rows {rows}, replay {i}")
+    g.destroy()
+    ref = x.numpy().astype(np.float64) @ w.numpy().astype(np.float64) + b.numpy()
+    ref = 0.5 * ref * (1 + np.tanh(np.sqrt(2 / np.pi) * (ref + 0.044715 * ref ** 3)))
+    assert np.abs(eager - ref).max() <= 2e-5 * max(1.0, np.abs(ref).max())
+
+
+def test_capture_without_scratch_fails_loudly(gpu):
+    """A product that splits K needs a scratch block.  Captured without a warm-up (the pool has never seen the
+    block) it must fail with WF2HIP_ECAPTURE rather than quietly take another route with other rounding."""
+    W = gpu
+    F = W.functional
+    rng = np.random.default_rng(11)
+    # shapes of their own, so that no earlier test has left a matching scratch block in the pool
+    x = F.from_numpy(rng.standard_normal((200, 1056)).astype(np.float32))
+    w = F.from_numpy(rng.standard_normal((1056, 1000)).astype(np.float32))
+    out = W.HIPTensor([200, 1000], initial_element=None)
+    W.lib.check(W.lib.get().wf2hip_pool_trim())
+    with pytest.raises(W.HIPError) as e:
+        with W.lib.Graph():
+            F.matmul(x, w, out=out)
+    assert e.value.code == W.lib.ECAPTURE
+    eager = F.matmul(x, w, out=out).numpy().copy()  # warm-up
+    with W.lib.Graph() as g:
+        F.matmul(x, w, out=out)
+    g.launch()
+    assert_bit_equal(out.numpy(), eager, "replay after the warm-up")
+    g.destroy()

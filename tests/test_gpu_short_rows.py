@@ -303,6 +303,38 @@ def test_softmax_and_layernorm_of_tiny_rows(gpu, rows, cols):
     assert np.all(np.abs(got - want) <= 4e-7 * scale * np.abs(g) + 2e-6 * np.abs(want) + 1e-6)
 
 
+@pytest.mark.parametrize("cols", [10, 64])
+def test_layernorm_tiny_rows_against_the_wavefront_form_and_its_own_backward(gpu, cols):
+    """The thread-per-row LayerNorm starts at 16384 rows.  The same rows through it (16384 rows) and through the
+    wavefront form (16383 rows) agree to the rounding of the row statistics, both agree with the reference's
+    ten-node recipe (source/nn/norms.lisp:72-82) run node for node, and the backward kernel of the same regime
+    recomputes exactly the x-hat the forward produced: with gamma = 1, beta = 0 the forward output is x-hat, and
+    with dy a single 1 the gradient of gamma is that row's x-hat."""
+    F = gpu.functional
+    rng = np.random.default_rng(cols)
+    x = (rng.standard_normal((16384, cols)) * 2 + 1).astype(np.float32)
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    dg, db = F.from_numpy(g), F.from_numpy(b)
+    tiny = F.layer_norm_fused(F.from_numpy(x), dg, db, eps=1e-5).numpy()
+    wave = F.layer_norm_fused(F.from_numpy(x[:16383]), dg, db, eps=1e-5).numpy()
+    nodes = F.layer_norm(F.from_numpy(x[:2000]), dg, db, eps=1e-5).numpy()
+    x64 = x.astype(np.float64)
+    std = np.sqrt(x64.var(axis=1, keepdims=True) + 1e-5)
+    scale = np.abs(x64).max(axis=1, keepdims=True) / std
+    bar = 6e-7 * scale * np.abs(g) + 3e-6 * np.abs(tiny) + 1e-6
+    assert np.all(np.abs(tiny[:16383] - wave) <= bar[:16383])
+    assert np.all(np.abs(tiny[:2000] - nodes) <= 4 * bar[:2000])
+    ones, zeros = F.from_numpy(np.ones(cols, np.float32)), F.from_numpy(np.zeros(cols, np.float32))
+    xh = F.layer_norm_fused(F.from_numpy(x), ones, zeros, eps=1e-5).numpy()
+    for row in (0, 777, 16383):
+        dy = np.zeros_like(x)
+        dy[row] = 1.0
+        _, dgamma, dbeta = F.layer_norm_backward(F.from_numpy(x), ones, F.from_numpy(dy), 1e-5)
+        np.testing.assert_array_equal(dgamma.numpy().ravel(), xh[row])
+        np.testing.assert_array_equal(dbeta.numpy().ravel(), np.ones(cols, np.float32))
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_random_sums_and_selections(gpu, seed):
     """Random shapes (a few long axes, many short ones) and random kept / reduced axes: !sum, !mean, !max and

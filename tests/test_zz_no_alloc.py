@@ -74,3 +74,40 @@ def test_noalloc_refuses_sizes_beyond_its_maximum(gpu):
     assert rc == W.lib.EUNSUPPORTED
     assert b"maximum" in lib.wf2hip_last_error()
     assert lib.wf2hip_reduce_add_rows_f32_noalloc(0, 5, None, 5, None, 1) == 0
+
+
+@pytest.mark.parametrize("rows, cols, ldx, inco", [
+    (64, 1 << 18, 1 << 18, 1),    # rows split over workgroups
+    (4096, 4096, 4096, 1),        # a wavefront or workgroup per row
+    (37, 29999, 30000, 1),        # padded rows
+    (37, 1, 30000, 1),            # one column: a strided add
+    (40, 50000, 50016, 0),        # every row into one number, padded rows: two reduced axes
+    (40, 50000, 50000, 0),        # the same, dense: one long run
+    (70000, 1, 3, 0),             # a strided column into one number
+])
+def test_noalloc_requests_no_block(gpu, rows, cols, ldx, inco):
+    """No block is requested from the allocator, whatever form the arguments normalise to; results agree with
+    the allocating entry to the bar of every reduction (bit equality where both run the same kernels)."""
+    W = gpu
+    lib = W.lib.get()
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((rows, ldx)).astype(np.float32)
+    nout = rows if inco else 1
+    start = rng.standard_normal(nout).astype(np.float32)
+    dx = W.HIPTensor.from_numpy(x)
+    got = W.HIPTensor.from_numpy(start.copy())
+    want = W.HIPTensor.from_numpy(start.copy())
+    W.lib.check(lib.wf2hip_sync())
+    before = lib.wf2hip_pool_requests()
+    W.lib.check(lib.wf2hip_reduce_add_rows_f32_noalloc(rows, cols, dptr(dx), ldx, dptr(got), inco))
+    assert lib.wf2hip_pool_requests() == before, "the allocation-free entry point asked the allocator for a block"
+    W.lib.check(lib.wf2hip_reduce_add_rows_f32(rows, cols, dptr(dx), ldx, dptr(want), inco))
+    got, want = got.numpy(), want.numpy()
+    x64 = x[:, :cols].astype(np.float64)
+    if inco:
+        assert_bit_equal(got, want, f"rows {rows} cols {cols} ldx {ldx}")
+        ref, mag = start + x64.sum(axis=1), np.abs(start) + np.abs(x64).sum(axis=1)
+    else:
+        ref, mag = start + x64.sum(), np.abs(start) + np.abs(x64).sum()
+        assert np.all(np.abs(want - ref) <= 1e-5 * mag)
+    assert np.all(np.abs(got - ref) <= 1e-5 * mag)
