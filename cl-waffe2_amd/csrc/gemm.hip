@@ -30,6 +30,8 @@
 // Bound: fp32 MFMA peak (157.3 TFLOP/s on MI355X); 2 m n k flop per product.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "wf2_common.h"
 #include "wf2_math.h"
 #include "wf2_view.h"
@@ -345,6 +347,22 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 //                     the order 0 4 1 5 2 6 3 7, so that the value lane l needs for
 //                     k = 8 g + 4 (l / 32) + s sits at float 64 s + l of the
 //                     instruction's 1 KB: plain conflict-free 32-bit reads.
+// One global -> LDS instruction: 64 lanes x 16 bytes from `base` + this lane's byte offset into the 1 KB of
+// LDS at byte address `lds_addr` (same for the whole wavefront).  Written out because the compiler's own
+// builtin always forms a 64-bit address per lane, which costs the matrix cores five times the issue time.
+// M0 holds the LDS destination; nothing else in these kernels uses it.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t lane_offset, const float* base) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(lane_offset), "s"(base)
+               : "memory", "m0");
+#endif
+}
+#pragma clang diagnostic pop
+
 template <bool RKIN, int TN, bool TALL = false>
 struct DmaLayout {
   static constexpr int BNt = TALL ? 32 * TN : 64 * TN;
@@ -387,20 +405,24 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const int wm = TALL ? wave * 32 : (wave >> 1) * 64;
   const int wn = TALL ? 0 : (wave & 1) * 32 * TN;
 
-  // Global source of every 16-byte piece this lane moves per K-step (k = 0);
-  // rows / columns beyond the matrix are clamped to its last ones: they only
-  // feed accumulators that are never stored.
+  // Global source of every 16-byte piece this lane moves per K-step: a base per operand that is the same
+  // for the whole workgroup and moves along K on the scalar unit, plus a byte offset per lane and
+  // instruction that never changes (32 bits: the host checks that a tile's rows span less than 4 GB).
+  // With the address in this form -- scalar base, 32-bit lane offset -- a load costs the matrix cores about
+  // 5 cycles of issue; with a 64-bit address per lane it costs 26, and the 64-bit add that forms it 10 more
+  // (measured between back-to-back MFMAs: seven or eight loads per K-step were 8 % of the loop).
+  // Rows / columns beyond the matrix are clamped to its last ones: they only feed accumulators that are
+  // never stored.
   constexpr int LI = 4;                   // left-operand instructions per wavefront
   constexpr int RI = Lay::R_INSTRS / 4;   // right-operand instructions per wavefront
-  const float* srcL[LI];
-  const float* srcR[RI];
+  uint32_t offL[LI], offR[RI];
 #pragma unroll
   for (int j = 0; j < LI; j++) {
     const int row = (wave * LI + j) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int64_t gr = m0 + row;
     gr = gr < p.M ? gr : p.M - 1;
-    srcL[j] = L + gr * p.ldl + chunk * 4;
+    offL[j] = (uint32_t)(((gr - m0) * p.ldl + chunk * 4) * (int64_t)sizeof(float));
   }
 #pragma unroll
   for (int j = 0; j < RI; j++) {
@@ -410,33 +432,37 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       const int chunk = (lane & 7) ^ ((row >> 1) & 7);
       int64_t gn = n0 + row;
       gn = gn < p.N ? gn : p.N - 1;
-      srcR[j] = R + gn * p.ldr + chunk * 4;
+      offR[j] = (uint32_t)(((gn - n0) * p.ldr + chunk * 4) * (int64_t)sizeof(float));
     } else if (TALL) {
       // instruction q: column block q / 4, k-rows 8 (q % 4) + {0 4 1 5 2 6 3 7}[lane / 8]
       const int slot = lane >> 3;
       const int krow = 8 * (q & 3) + (slot >> 1) + 4 * (slot & 1);
       int64_t gn = n0 + 32 * (q >> 2) + 4 * (lane & 7);
       gn = gn < p.N ? gn : p.N - 4;
-      srcR[j] = R + (int64_t)krow * p.ldr + gn;
+      offR[j] = (uint32_t)(((int64_t)krow * p.ldr + (gn - n0)) * (int64_t)sizeof(float));
     } else {
       constexpr int CPR = BNt / 4;  // 16-byte pieces per k-row; LDS keeps [k][BNt] densely
       const int piece = q * 64 + lane;
       const int krow = piece / CPR;
       int64_t gn = n0 + (piece % CPR) * 4;
       gn = gn < p.N ? gn : p.N - 4;
-      srcR[j] = R + (int64_t)krow * p.ldr + gn;
+      offR[j] = (uint32_t)(((int64_t)krow * p.ldr + (gn - n0)) * (int64_t)sizeof(float));
     }
   }
-  auto fetch = [&](int stage, int64_t k0) {
-#if defined(__HIP_DEVICE_COMPILE__)
+  const float* nextL = L + m0 * p.ldl;                          // K-step the next fetch reads
+  const float* nextR = RKIN ? R + n0 * p.ldr : R + n0;
+  const int64_t stepR = RKIN ? (int64_t)BK : (int64_t)BK * p.ldr;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)smem;
+  auto fetch = [&](int stage) {
 #pragma unroll
     for (int j = 0; j < LI; j++)
-      __builtin_amdgcn_global_load_lds(srcL[j] + k0, ldsL(stage) + (wave * LI + j) * 256, 16, 0, 0);
+      dma16(lds0 + (uint32_t)((stage * Lay::STAGE + (wave * LI + j) * 256) * sizeof(float)), offL[j], nextL);
 #pragma unroll
     for (int j = 0; j < RI; j++)
-      __builtin_amdgcn_global_load_lds(RKIN ? srcR[j] + k0 : srcR[j] + k0 * p.ldr,
-                                       ldsR(stage) + (wave * RI + j) * Lay::R_INSTR_PITCH, 16, 0, 0);
-#endif
+      dma16(lds0 + (uint32_t)((stage * Lay::STAGE + Lay::LFLOATS + (wave * RI + j) * Lay::R_INSTR_PITCH) * sizeof(float)),
+            offR[j], nextR);
+    nextL += BK;
+    nextR += stepR;
   };
 
   f16v acc[MI][TN];
@@ -538,15 +564,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   if (FUSED && p.causal == 2 && m0 + BMt < klimit) klimit = m0 + BMt;
   const int ksteps = (int)(klimit / BK);  // K and the tile height are multiples of BK
 
-  fetch(0, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  read_frags(0, 0, 0);
-  for (int ks = 0; ks < ksteps; ks++) {
-    const int cur = ks & 1;
-    const bool more = ks + 1 < ksteps;
+  // One K-step on the stage `cur` (a constant after inlining: the loop below is unrolled by two, so every LDS
+  // address is a register fixed for the kernel plus an immediate and the loop holds no vector-ALU
+  // instruction at all -- each one costs the matrix cores 5 - 12 cycles of issue).
+  auto k_step = [&](auto cur_c, bool more) {
+    constexpr int cur = decltype(cur_c)::value;
     // the other stage was last read before the barrier of the previous step
-    if (more) fetch(cur ^ 1, (int64_t)(ks + 1) * BK);
+    if (more) fetch(cur ^ 1);
     read_frags(cur, 1, 1); multiply(0); pin_order();
     read_frags(cur, 2, 0); multiply(1); pin_order();
     read_frags(cur, 3, 1); multiply(0); pin_order();
@@ -556,7 +580,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     __syncthreads();
     if (more) read_frags(cur ^ 1, 0, 0);
     multiply(1); pin_order();
+  };
+  fetch(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  read_frags(0, 0, 0);
+  int ks = 0;
+  for (; ks + 2 <= ksteps; ks += 2) {
+    k_step(std::integral_constant<int, 0>{}, true);
+    k_step(std::integral_constant<int, 1>{}, ks + 2 < ksteps);
   }
+  if (ks < ksteps) k_step(std::integral_constant<int, 0>{}, false);
 
   // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
@@ -1136,9 +1170,11 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   // global -> LDS streaming kernel: left operand k-innermost, whole K-steps
   // (with only a few K-steps per tile the set-up of the streaming kernel costs more
   // than it saves: 96 x 1024x1024x64 runs in 187 us staged, 243 us streamed)
-  bool dma = fast && lkin && k % BK == 0 && k >= 256;
+  // (the streaming kernel addresses a tile's rows by 32-bit byte offsets from a base of the workgroup)
+  const bool pitch32 = lda < ((long)1 << 22) && ldb < ((long)1 << 22);
+  bool dma = fast && lkin && k % BK == 0 && k >= 256 && pitch32;
   if (const char* force = getenv("WF2HIP_GEMM_STREAM"))  // testing knob: 0 never, 1 whenever possible
-    dma = force[0] == '1' ? (fast && lkin && k % BK == 0 && k > 0) : false;
+    dma = force[0] == '1' ? (fast && lkin && k % BK == 0 && k > 0 && pitch32) : false;
 
   // Tile choice: time ~ tiles on the busiest CU x tile width / efficiency.
   // Measured per unit of work 128x128 is about 6 % ahead of 128x64 (which
