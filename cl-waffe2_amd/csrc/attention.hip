@@ -31,7 +31,10 @@
 // Numerics: products and sums in binary32 on the matrix cores, exponentials by
 // v_exp_f32 (about 1 ulp) on max-subtracted arguments; the result agrees with
 // the float64 closed form to ~1e-6 relative to max|V|.
+#include <type_traits>
+
 #include "wf2_common.h"
+#include "wf2_dma.h"
 
 namespace wf2 {
 
@@ -59,11 +62,16 @@ struct AttnParams {
   float* lse;  // optional: log2 of the row sums of exp2(scores), (batch * heads, seq); what the backward needs
 };
 
+// How far the maximum a row's exponentials are taken against may lag behind the row's true maximum
+// (log2 units): the reference only moves when a block holds a score more than this above it, so after
+// the first blocks the accumulator is almost never rescaled.  Exponentials then reach 2^8 at most --
+// any reference gives the same quotient, and binary32 has the range.
+constexpr float kMaxLag = 8.0f;
+
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_kernel(
     AttnParams p) {  // two workgroups per CU: at most 256 registers per lane
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  auto lds_k = [&](int stage) { return smem + stage * kStageFloats; };
-  auto lds_v = [&](int stage) { return smem + stage * kStageFloats + kKBlock * kRowFloats; };
+  constexpr int kKeyFloats = kKBlock * kRowFloats;  // one tile: 64 rows of 64 floats
 
   // longest query blocks first: with a causal mask block qb needs qb+1 key spans
   const int nbh = p.batch * p.heads;
@@ -79,15 +87,17 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const int half = lane >> 5;
   const int col = lane & 31;
 
-  const int q_first = qb * kQBlock + wave * 32;  // first query of this wavefront
+  // With a causal mask the wavefronts of a workgroup walk 2 qb + 1, 2 qb + 1, 2 qb + 2, 2 qb + 2 key
+  // blocks.  Wavefront w of every workgroup sits on SIMD w, so every second workgroup hands its
+  // queries out in reverse: the two workgroups that share a compute unit then load its SIMDs evenly.
+  const int part = (p.causal && (blockIdx.x & 1)) ? 3 - wave : wave;
+  const int q_first = qb * kQBlock + part * 32;  // first query of this wavefront
   const int query = q_first + col;
   const int query_ld = query < p.seq ? query : p.seq - 1;
 
   const float* qp = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)query_ld * p.qs[2];
   const float* kp = p.k + b * p.ks[0] + h * p.ks[1];
   const float* vp = p.v + b * p.vs[0] + h * p.vs[1];
-  (void)kp;
-  (void)vp;  // only the device pass reads them (global -> LDS builtin)
 
   // Q fragment: qf[4 j + r] = Q[query][8 j + 4 half + r] * scale * log2(e)
   float qf[32];
@@ -108,7 +118,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const int q_last_wave = q_first + 31;
 
   f16v o0 = {0}, o1 = {0};
-  float m = -INFINITY;  // running maximum (log2 domain), shared by both halves
+  float m = -INFINITY;  // the maximum the exponentials are taken against (log2 domain), shared by both halves
   float lsum = 0.f;     // running sum of this half's keys
 
   // Key / value blocks go global -> LDS without passing through registers: one
@@ -118,23 +128,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   //           consecutive rows cover all 64 banks;
   //   values  the two 128-byte halves of a row are swapped when (row / 4) is odd:
   //           the half-waves read rows 4 apart and then hit different banks.
-  // Rows beyond the sequence are clamped (their scores are masked later); chunks
-  // beyond head_dim are not loaded and stay zero from the clear below.
-  auto fetch = [&](bool values, int stage, int key0) {
-#if defined(__HIP_DEVICE_COMPILE__)
+  // A block's base address stays on the scalar unit; per lane there are only the four byte offsets
+  // of its pieces (wf2_dma.h).  Rows beyond the sequence are clamped (their scores are masked later):
+  // only the last block of a ragged sequence computes offsets of its own.  Chunks beyond head_dim
+  // are not loaded and stay zero from the clear below.
+  const uint32_t lds0 = lds_address(smem);
+  const int drow = lane >> 4, dslot = lane & 15;
+  uint32_t koff[4], voff[4];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int q4 = wave * 4 + j;
-      const int row = q4 * 4 + (lane >> 4);
-      const int slot = lane & 15;
-      int key = key0 + row;
-      key = key < p.seq ? key : p.seq - 1;
-      const int chunk = values ? slot ^ (((row >> 2) & 1) << 3) : slot ^ (row & 15);
-      const float* src = values ? vp + (int64_t)key * p.vs[2] : kp + (int64_t)key * p.ks[2];
-      float* dst = (values ? lds_v(stage) : lds_k(stage)) + q4 * 256;
-      if (chunk * 4 < p.head_dim) __builtin_amdgcn_global_load_lds(src + chunk * 4, dst, 16, 0, 0);
+  for (int j = 0; j < 4; j++) {
+    const int row = (wave * 4 + j) * 4 + drow;
+    koff[j] = (uint32_t)((row * p.ks[2] + (dslot ^ (row & 15)) * 4) * (int64_t)sizeof(float));
+    voff[j] = (uint32_t)((row * p.vs[2] + (dslot ^ (((row >> 2) & 1) << 3)) * 4) * (int64_t)sizeof(float));
+  }
+  const bool whole_rows = p.head_dim == kHeadDim;
+  auto fetch = [&](bool values, int stage, int key0) {
+    const float* base = values ? vp + (int64_t)key0 * p.vs[2] : kp + (int64_t)key0 * p.ks[2];
+    const uint32_t dst = lds0 + (uint32_t)((stage * kStageFloats + (values ? kKeyFloats : 0) + wave * 1024) * sizeof(float));
+    const bool ragged = key0 + kKBlock > p.seq;
+    if (whole_rows && !ragged) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) dma16(dst + j * 1024, values ? voff[j] : koff[j], base);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int row = (wave * 4 + j) * 4 + drow;
+        const int chunk = values ? dslot ^ (((row >> 2) & 1) << 3) : dslot ^ (row & 15);
+        const int last = p.seq - 1 - key0;  // >= 0: key0 < seq
+        const int64_t r = row < last ? row : last;
+        const uint32_t off = (uint32_t)((r * (values ? p.vs[2] : p.ks[2]) + chunk * 4) * (int64_t)sizeof(float));
+        if (chunk * 4 < p.head_dim) dma16(dst + j * 1024, off, base);
+      }
     }
-#endif
   };
   if (p.head_dim < kHeadDim) {
     for (int i = threadIdx.x; i < 2 * kStageFloats / 4; i += kBlock)
@@ -142,32 +167,57 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     __syncthreads();
   }
 
-  const int kswz = col & 15;     // rows col and 32 + col share it
-  const int vswap = half << 5;   // keys read by the upper half-wave have (key / 4) odd
-
-  // S^T of one key block: two 32 x 32 tiles (keys 0-31 and 32-63 of the block)
-  auto scores = [&](const float* sk, f16v& s0, f16v& s1) {
+  // LDS addresses of the fragments, fixed for the kernel: everything that depends on the block or the
+  // stage is an immediate, so the loop holds no address arithmetic (a vector-ALU instruction costs the
+  // matrix cores 5 - 12 cycles of issue).
+  //   keys    row col (and 32 + col), 16-byte slot (2 j + half) ^ (col % 16) for contraction group j
+  //   values  row 4 half + ..., floats 2 col, 2 col + 1 with the halves swapped for the upper half-wave
+  const float* kfrag[8];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      s0[i] = 0.f;
-      s1[i] = 0.f;
-    }
+  for (int j = 0; j < 8; j++) kfrag[j] = smem + col * kRowFloats + (((2 * j + half) ^ (col & 15)) * 4);
+  const float* vfrag = smem + kKeyFloats + 4 * half * kRowFloats + ((2 * col) ^ (half << 5));
+
+  // S^T of one key block: two 32 x 32 tiles (keys 0-31 and 32-63 of the block).  The fragments of
+  // contraction group j + 1 are on their way while the matrix cores work on group j.
+  auto scores = [&](int stage, f16v& s0, f16v& s1) {
+    const int so = stage * kStageFloats;
+    f4 ka[2], kb[2];
+    ka[0] = *reinterpret_cast<const f4*>(kfrag[0] + so);
+    kb[0] = *reinterpret_cast<const f4*>(kfrag[0] + so + 32 * kRowFloats);
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-      const int slot = ((2 * j + half) ^ kswz) * 4;
-      f4 k0 = *reinterpret_cast<const f4*>(sk + col * kRowFloats + slot);
-      f4 k1 = *reinterpret_cast<const f4*>(sk + (32 + col) * kRowFloats + slot);
-      s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[4 * j + 0], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[4 * j + 0], s1, 0, 0, 0);
+      if (j + 1 < 8) {
+        ka[(j + 1) & 1] = *reinterpret_cast<const f4*>(kfrag[j + 1] + so);
+        kb[(j + 1) & 1] = *reinterpret_cast<const f4*>(kfrag[j + 1] + so + 32 * kRowFloats);
+      }
+      const f4 k0 = ka[j & 1], k1 = kb[j & 1];
+      if (j == 0) {
+        const f16v zero = {0};
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[0], zero, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[0], zero, 0, 0, 0);
+      } else {
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.x, qf[4 * j + 0], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.x, qf[4 * j + 0], s1, 0, 0, 0);
+      }
       s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.y, qf[4 * j + 1], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.y, qf[4 * j + 1], s1, 0, 0, 0);
       s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.z, qf[4 * j + 2], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.z, qf[4 * j + 2], s1, 0, 0, 0);
       s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(k0.w, qf[4 * j + 3], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1.w, qf[4 * j + 3], s1, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+      // the two reads of the next group go among this group's first MFMAs
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+#endif
     }
   };
-  // masks, running softmax statistics, P = exp2(S - max) in place
+  // masks, running softmax statistics, P = exp2(S - m) in place.  Per score: a share of a three-way
+  // maximum, a subtraction, an exponential and an addition; the accumulator is rescaled only when the
+  // reference maximum moves (kMaxLag), which a branch the whole wavefront takes or skips decides.
   auto normalise = [&](int key0, f16v& s0, f16v& s1) {
     // register i of tile t holds key key0 + 32 t + 8 (i/4) + 4 half + i%4
     const bool edge = (p.causal && key0 + kKBlock - 1 > q_first) || key0 + kKBlock > p.seq;
@@ -180,50 +230,66 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
         if (key + 32 > limit) s1[i] = -INFINITY;
       }
     }
-    float mloc = s0[0];
+    float mloc = fmaxf(s0[0], s1[0]);
 #pragma unroll
-    for (int i = 1; i < 16; i++) mloc = fmaxf(mloc, s0[i]);
-#pragma unroll
-    for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s1[i]);
+    for (int i = 1; i < 16; i++) mloc = fmaxf(fmaxf(mloc, s0[i]), s1[i]);  // v_max3_f32
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float mnew = fmaxf(m, mloc);
-    // key 0 is visible to every query, so mnew is finite from the first block on
-    const float alpha = __builtin_amdgcn_exp2f(m - mnew);
-    m = mnew;
-    float psum = 0.f;
+    // key 0 is visible to every query, so the reference is finite from the first block on
+    if (__any(mloc > m + kMaxLag)) {
+      const float mnew = mloc > m + kMaxLag ? mloc : m;
+      const float alpha = __builtin_amdgcn_exp2f(m - mnew);
+      m = mnew;
+      lsum *= alpha;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        o0[i] *= alpha;
+        o1[i] *= alpha;
+      }
+    }
+    float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      s0[i] = __builtin_amdgcn_exp2f(s0[i] - mnew);
-      s1[i] = __builtin_amdgcn_exp2f(s1[i] - mnew);
-      psum += s0[i] + s1[i];
+      s0[i] = __builtin_amdgcn_exp2f(s0[i] - m);
+      s1[i] = __builtin_amdgcn_exp2f(s1[i] - m);
+      ps[i & 3] += s0[i];
+      ps[i & 3] += s1[i];
     }
-    lsum = lsum * alpha + psum;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      o0[i] *= alpha;
-      o1[i] *= alpha;
-    }
+    lsum += (ps[0] + ps[1]) + (ps[2] + ps[3]);
   };
   // O^T += V^T . P^T.  Accumulator o0 owns the even head dimensions, o1 the odd
   // ones: a lane then needs V[key][2 col] and V[key][2 col + 1], one 64-bit read
   // (half as many LDS instructions as two tiles of 32 consecutive dimensions).
   typedef float f2 __attribute__((ext_vector_type(2)));
-  auto accumulate = [&](const float* sv, const f16v& s0, const f16v& s1) {
+  auto accumulate = [&](int stage, const f16v& s0, const f16v& s1) {
+    const float* sv = vfrag + stage * kStageFloats;
+    // register i <-> key 8 (i/4) + i%4 (+ 4 half, in vfrag) of each 32-key tile
+    f2 va[2], vb[2];
+    va[0] = *reinterpret_cast<const f2*>(sv);
+    vb[0] = *reinterpret_cast<const f2*>(sv + 32 * kRowFloats);
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      const int key = 8 * (i >> 2) + 4 * half + (i & 3);
-      const f2 v0 = *reinterpret_cast<const f2*>(sv + key * kRowFloats + ((2 * col) ^ vswap));
-      const f2 v1 = *reinterpret_cast<const f2*>(sv + (32 + key) * kRowFloats + ((2 * col) ^ vswap));
+      if (i + 1 < 16) {
+        const int key = 8 * ((i + 1) >> 2) + ((i + 1) & 3);
+        va[(i + 1) & 1] = *reinterpret_cast<const f2*>(sv + key * kRowFloats);
+        vb[(i + 1) & 1] = *reinterpret_cast<const f2*>(sv + (32 + key) * kRowFloats);
+      }
+      const f2 v0 = va[i & 1], v1 = vb[i & 1];
       o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v0.x, s0[i], o0, 0, 0, 0);
       o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v0.y, s0[i], o1, 0, 0, 0);
       o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(v1.x, s1[i], o0, 0, 0, 0);
       o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(v1.y, s1[i], o1, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+#endif
     }
   };
 
-  // Software pipeline over key blocks: while the vector units work through the
-  // softmax of block kb, the matrix cores already form the scores of block
-  // kb + 1; then P V of block kb follows.  Keys are therefore staged one block
+  // Software pipeline over key blocks: the scores of block kb + 1 are formed before
+  // the softmax of block kb, then P V of block kb follows.  Keys are therefore staged one block
   // further ahead than values:
   //   top of iteration kb   fetch K(kb + 2) into the stage K(kb) left (its scores
   //                         were formed before the last barrier), V(kb + 1) into
@@ -231,34 +297,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   //   body                  scores of kb + 1 from K(kb + 1), softmax of kb, P V of
   //                         kb from V(kb)
   //   end                   wait for this wavefront's fetches, barrier
+  // The loop is unrolled by two, so that stages are constants and the scores of consecutive blocks
+  // alternate between two pairs of accumulators instead of being copied.
+  f16v sa0, sa1, sb0, sb1;
+  auto block = [&](auto parity, int kb, f16v& c0, f16v& c1, f16v& n0, f16v& n1) {
+    constexpr int par = decltype(parity)::value;  // kb % 2
+    const int key0 = kb * kKBlock;
+    if (kb + 2 < nkb) fetch(false, par, key0 + 2 * kKBlock);
+    if (kb + 1 < nkb) fetch(true, par ^ 1, key0 + kKBlock);
+    // a wavefront whose queries all precede a key block has nothing to add there
+    const bool active = !(p.causal && key0 > q_last_wave);
+    const bool next_active = kb + 1 < nkb && !(p.causal && key0 + kKBlock > q_last_wave);
+    if (next_active) scores(par ^ 1, n0, n1);  // implies active
+    if (active) {
+      normalise(key0, c0, c1);
+      accumulate(par, c0, c1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's fetches have landed
+    __syncthreads();
+  };
   fetch(false, 0, 0);
   fetch(true, 0, 0);
   if (nkb > 1) fetch(false, 1, kKBlock);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  f16v n0, n1;  // scores of the next block
-  scores(lds_k(0), n0, n1);
+  scores(0, sa0, sa1);
   __syncthreads();  // every wavefront has read K(0) before its stage is refilled
-
-  for (int kb = 0; kb < nkb; kb++) {
-    const int key0 = kb * kKBlock;
-    if (kb + 2 < nkb) fetch(false, kb & 1, key0 + 2 * kKBlock);
-    if (kb + 1 < nkb) fetch(true, (kb + 1) & 1, key0 + kKBlock);
-    // a wavefront whose queries all precede a key block has nothing to add there
-    const bool active = !(p.causal && key0 > q_last_wave);
-    const bool next_active = kb + 1 < nkb && !(p.causal && key0 + kKBlock > q_last_wave);
-    f16v s0 = n0, s1 = n1;
-    if (next_active) {  // implies active
-      scores(lds_k((kb + 1) & 1), n0, n1);
-      normalise(key0, s0, s1);
-      accumulate(lds_v(kb & 1), s0, s1);
-    } else if (active) {
-      normalise(key0, s0, s1);
-      accumulate(lds_v(kb & 1), s0, s1);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's fetches have landed
-    __syncthreads();
+  int kb = 0;
+  for (; kb + 2 <= nkb; kb += 2) {
+    block(std::integral_constant<int, 0>{}, kb, sa0, sa1, sb0, sb1);
+    block(std::integral_constant<int, 1>{}, kb + 1, sb0, sb1, sa0, sa1);
   }
+  if (kb < nkb) block(std::integral_constant<int, 0>{}, kb, sa0, sa1, sb0, sb1);
 
   const float total = lsum + __shfl_xor(lsum, 32);
   const float inv = 1.0f / total;

@@ -33,6 +33,7 @@
 #include <type_traits>
 
 #include "wf2_common.h"
+#include "wf2_dma.h"
 #include "wf2_math.h"
 #include "wf2_view.h"
 
@@ -347,22 +348,6 @@ __global__ __launch_bounds__(kBlock) void sgemm_kernel(GemmParams p) {
 //                     the order 0 4 1 5 2 6 3 7, so that the value lane l needs for
 //                     k = 8 g + 4 (l / 32) + s sits at float 64 s + l of the
 //                     instruction's 1 KB: plain conflict-free 32-bit reads.
-// One global -> LDS instruction: 64 lanes x 16 bytes from `base` + this lane's byte offset into the 1 KB of
-// LDS at byte address `lds_addr` (same for the whole wavefront).  Written out because the compiler's own
-// builtin always forms a 64-bit address per lane, which costs the matrix cores five times the issue time.
-// M0 holds the LDS destination; nothing else in these kernels uses it.
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t lane_offset, const float* base) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(lane_offset), "s"(base)
-               : "memory", "m0");
-#endif
-}
-#pragma clang diagnostic pop
-
 template <bool RKIN, int TN, bool TALL = false>
 struct DmaLayout {
   static constexpr int BNt = TALL ? 32 * TN : 64 * TN;
@@ -452,7 +437,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const float* nextL = L + m0 * p.ldl;                          // K-step the next fetch reads
   const float* nextR = RKIN ? R + n0 * p.ldr : R + n0;
   const int64_t stepR = RKIN ? (int64_t)BK : (int64_t)BK * p.ldr;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)smem;
+  const uint32_t lds0 = lds_address(smem);
   auto fetch = [&](int stage) {
 #pragma unroll
     for (int j = 0; j < LI; j++)
