@@ -445,10 +445,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   const float* str2 = KEYS ? p.dout + b * p.os[0] + h * p.os[1] : p.v + b * p.vs[0] + h * p.vs[1];
   const int64_t pitch1 = KEYS ? p.qs[2] : p.ks[2];
   const int64_t pitch2 = KEYS ? p.os[2] : p.vs[2];
-  (void)str1;
-  (void)str2;
-  (void)pitch1;
-  (void)pitch2;  // only the device pass reads them (global -> LDS builtin)
   const float* lse = p.lse + (int64_t)bh * p.seq;
   const float* delta = p.delta + (int64_t)bh * p.seq;
 
@@ -488,21 +484,44 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
     }
   }
 
+  // The tiles go global -> LDS through scalar-base loads (wf2_dma.h): a base per stream that is the same
+  // for the workgroup, per lane the four byte offsets of its pieces in each stream.  Only a ragged last
+  // tile (rows clamped to the sequence) and heads narrower than 64 compute offsets of their own.
+  const uint32_t lds0 = lds_address(smem);
+  const int drow = lane >> 4, dslot = lane & 15;
+  uint32_t off1[4], off2[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int r = (wave * 4 + j) * 4 + drow;
+    const int chunk = dslot ^ (r & 15);
+    off1[j] = (uint32_t)((r * pitch1 + chunk * 4) * (int64_t)sizeof(float));
+    off2[j] = (uint32_t)((r * pitch2 + chunk * 4) * (int64_t)sizeof(float));
+  }
+  const bool whole_rows = p.head_dim == kHeadDim;
   float stat_value = 0.f;
   auto fetch = [&](int stage, int tile) {
-#if defined(__HIP_DEVICE_COMPILE__)
     const int row0 = tile * kKBlock;
+    const float* b1 = str1 + (int64_t)row0 * pitch1;
+    const float* b2 = str2 + (int64_t)row0 * pitch2;
+    const uint32_t d1 = lds0 + (uint32_t)((stage * kBwdStageFloats + wave * 1024) * sizeof(float));
+    const uint32_t d2 = d1 + (uint32_t)(kKBlock * kRowFloats * sizeof(float));
+    if (whole_rows && row0 + kKBlock <= p.seq) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int q4 = wave * 4 + j;
-      const int r = q4 * 4 + (lane >> 4);
-      const int slot = lane & 15;
-      int srow = row0 + r;
-      srow = srow < p.seq ? srow : p.seq - 1;
-      const int chunk = slot ^ (r & 15);
-      if (chunk * 4 < p.head_dim) {
-        __builtin_amdgcn_global_load_lds(str1 + (int64_t)srow * pitch1 + chunk * 4, tile1(stage) + q4 * 256, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(str2 + (int64_t)srow * pitch2 + chunk * 4, tile2(stage) + q4 * 256, 16, 0, 0);
+      for (int j = 0; j < 4; j++) {
+        dma16(d1 + j * 1024, off1[j], b1);
+        dma16(d2 + j * 1024, off2[j], b2);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int r = (wave * 4 + j) * 4 + drow;
+        const int chunk = dslot ^ (r & 15);
+        const int last = p.seq - 1 - row0;  // >= 0
+        const int64_t rr = r < last ? r : last;
+        if (chunk * 4 < p.head_dim) {
+          dma16(d1 + j * 1024, (uint32_t)((rr * pitch1 + chunk * 4) * (int64_t)sizeof(float)), b1);
+          dma16(d2 + j * 1024, (uint32_t)((rr * pitch2 + chunk * 4) * (int64_t)sizeof(float)), b2);
+        }
       }
     }
     if (KEYS && wave < 2) {  // L (wavefront 0) and D (wavefront 1) of the tile's 64 queries, parked in a register
@@ -510,7 +529,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       srow = srow < p.seq ? srow : p.seq - 1;
       stat_value = wave == 0 ? lse[srow] : delta[srow];
     }
-#endif
   };
   // ... and written to LDS only after the arithmetic of the current tile, so that waiting for that
   // load does not also wait for the tile loads issued before it
@@ -525,13 +543,29 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 
   f16v g1a = {0}, g1b = {0};  // dQ (KEYS false) or dK (KEYS true): even / odd head dimensions
   f16v g2a = {0}, g2b = {0};  // dV (KEYS true)
-  const int kswz = col & 15;
   typedef float f2 __attribute__((ext_vector_type(2)));
 
-  auto compute = [&](int stage, int tile) {
-    const float* s1 = tile1(stage);
-    const float* s2 = tile2(stage);
-    const float* st = stats + stage * kBwdStatFloats;
+  // LDS addresses of the fragments, fixed for the kernel (stage, sub-tile and register index enter as
+  // immediates, so the tile loop holds no address arithmetic):
+  //   products against the resident rows   row col of the sub-tile, 16-byte slot (2 j + half) ^ (col % 16)
+  //   products that accumulate gradients   row 4 half + e (e the part of the register's row that is a
+  //                                        constant), floats 2 (col % 2) of slot (col / 2) ^ ((e + 4 half) % 16)
+  const float* sfrag[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) sfrag[j] = smem + col * kRowFloats + (((2 * j + half) ^ (col & 15)) * 4);
+  const float* gfrag[8];
+#pragma unroll
+  for (int q = 0; q < 8; q++) {
+    const int e = 8 * (q >> 2) + (q & 3);  // (row of register i) % 16 - 4 half, for i % 8 == q
+    gfrag[q] = smem + 4 * half * kRowFloats + (((col >> 1) ^ (e + 4 * half)) * 4) + 2 * (col & 1);
+  }
+  const float* sthalf = stats + 4 * half;
+
+  auto compute = [&](auto stage_c, int tile) {
+    constexpr int stage = decltype(stage_c)::value;
+    constexpr int so = stage * kBwdStageFloats;               // tile 1 of the stage; tile 2 follows it
+    constexpr int t2 = kKBlock * kRowFloats;
+    const float* st = sthalf + stage * kBwdStatFloats;
 #pragma unroll
     for (int t = 0; t < 2; t++) {
       const int s_first = tile * kKBlock + 32 * t;  // first streamed row of this 32-row sub-tile
@@ -539,76 +573,122 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
       if (p.causal) active = active && (KEYS ? s_first + 31 >= r_first : s_first <= r_first + 31);
       if (!active) continue;  // uniform over the wavefront
       f16v sc, dp;
+      {
+        // the fragments of contraction group j + 1 are on their way while the matrix cores work on group j
+        f4 xa[2], xb[2];
+        xa[0] = *reinterpret_cast<const f4*>(sfrag[0] + so + 32 * t * kRowFloats);
+        xb[0] = *reinterpret_cast<const f4*>(sfrag[0] + so + t2 + 32 * t * kRowFloats);
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        sc[i] = 0.f;
-        dp[i] = 0.f;
+        for (int j = 0; j < 8; j++) {
+          if (j + 1 < 8) {
+            xa[(j + 1) & 1] = *reinterpret_cast<const f4*>(sfrag[j + 1] + so + 32 * t * kRowFloats);
+            xb[(j + 1) & 1] = *reinterpret_cast<const f4*>(sfrag[j + 1] + so + t2 + 32 * t * kRowFloats);
+          }
+          const f4 x1 = xa[j & 1], x2 = xb[j & 1];
+          if (j == 0) {
+            const f16v zero = {0};
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, a1[0], zero, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, a2[0], zero, 0, 0, 0);
+          } else {
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, a1[4 * j + 0], sc, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, a2[4 * j + 0], dp, 0, 0, 0);
+          }
+          sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, a1[4 * j + 1], sc, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, a2[4 * j + 1], dp, 0, 0, 0);
+          sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.z, a1[4 * j + 2], sc, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.z, a2[4 * j + 2], dp, 0, 0, 0);
+          sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.w, a1[4 * j + 3], sc, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.w, a2[4 * j + 3], dp, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+#endif
+        }
       }
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const int slot = ((2 * j + half) ^ kswz) * 4;
-        const f4 x1 = *reinterpret_cast<const f4*>(s1 + (32 * t + col) * kRowFloats + slot);
-        const f4 x2 = *reinterpret_cast<const f4*>(s2 + (32 * t + col) * kRowFloats + slot);
-        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, a1[4 * j + 0], sc, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, a2[4 * j + 0], dp, 0, 0, 0);
-        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, a1[4 * j + 1], sc, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, a2[4 * j + 1], dp, 0, 0, 0);
-        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.z, a1[4 * j + 2], sc, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.z, a2[4 * j + 2], dp, 0, 0, 0);
-        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.w, a1[4 * j + 3], sc, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.w, a2[4 * j + 3], dp, 0, 0, 0);
-      }
-      // register i holds streamed row s_first + 8 (i/4) + 4 half + i%4 against resident row `row`
+      // register i holds streamed row s_first + 8 (i/4) + 4 half + i%4 against resident row `row`.
+      // Only sub-tiles on the diagonal or past the end of the sequence hold hidden pairs; the others take
+      // four vector instructions per pair (subtract, exponential, subtract, multiply).
+      const bool edge = s_first + 32 > p.seq ||
+                        (p.causal && !(KEYS ? r_first + 31 <= s_first : s_first + 31 <= r_first));
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         f4 lvals = {l_res, l_res, l_res, l_res}, dvals = {d_res, d_res, d_res, d_res};
         if (KEYS) {
-          lvals = *reinterpret_cast<const f4*>(st + 32 * t + 8 * g + 4 * half);
-          dvals = *reinterpret_cast<const f4*>(st + kKBlock + 32 * t + 8 * g + 4 * half);
+          lvals = *reinterpret_cast<const f4*>(st + 32 * t + 8 * g);
+          dvals = *reinterpret_cast<const f4*>(st + kKBlock + 32 * t + 8 * g);
         }
 #pragma unroll
         for (int c = 0; c < 4; c++) {
           const int i = 4 * g + c;
-          const int srow = s_first + 8 * g + 4 * half + c;
-          const int query = KEYS ? srow : row;
-          const int key = KEYS ? row : srow;
-          const bool visible = srow < p.seq && (!p.causal || key <= query);
-          const float pe = visible ? __builtin_amdgcn_exp2f(sc[i] - lvals[c]) : 0.f;
+          float pe = __builtin_amdgcn_exp2f(sc[i] - lvals[c]);
+          if (edge) {
+            const int srow = s_first + 8 * g + 4 * half + c;
+            const int query = KEYS ? srow : row;
+            const int key = KEYS ? row : srow;
+            const bool visible = srow < p.seq && (!p.causal || key <= query);
+            pe = visible ? pe : 0.f;
+          }
           sc[i] = pe;
           dp[i] = pe * (dp[i] - dvals[c]);
         }
       }
       // (streamed tile)^T . dS and, with resident keys, (dO tile)^T . P
+      {
+        f2 ya[2], yb[2];
+        ya[0] = *reinterpret_cast<const f2*>(gfrag[0] + so + 32 * t * kRowFloats);
+        if (KEYS) yb[0] = *reinterpret_cast<const f2*>(gfrag[0] + so + t2 + 32 * t * kRowFloats);
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int lr = 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
-        const int pos = (col >> 1) ^ (lr & 15);
-        const int off = lr * kRowFloats + pos * 4 + 2 * (col & 1);
-        const f2 x1 = *reinterpret_cast<const f2*>(s1 + off);
-        g1a = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, dp[i], g1a, 0, 0, 0);
-        g1b = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, dp[i], g1b, 0, 0, 0);
-        if (KEYS) {
-          const f2 x2 = *reinterpret_cast<const f2*>(s2 + off);
-          g2a = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, sc[i], g2a, 0, 0, 0);
-          g2b = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, sc[i], g2b, 0, 0, 0);
+        for (int i = 0; i < 16; i++) {
+          if (i + 1 < 16) {
+            // register i + 1: row 32 t + 8 ((i+1)/4) + (i+1)%4 + 4 half, address register ((i+1)/4 % 2) 4 + (i+1)%4
+            const int n = i + 1;
+            const int q = 4 * ((n >> 2) & 1) + (n & 3);
+            const int imm = (32 * t + 8 * (n >> 2) + (n & 3)) * kRowFloats;
+            ya[n & 1] = *reinterpret_cast<const f2*>(gfrag[q] + so + imm);
+            if (KEYS) yb[n & 1] = *reinterpret_cast<const f2*>(gfrag[q] + so + t2 + imm);
+          }
+          const f2 x1 = ya[i & 1];
+          g1a = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.x, dp[i], g1a, 0, 0, 0);
+          g1b = __builtin_amdgcn_mfma_f32_32x32x2f32(x1.y, dp[i], g1b, 0, 0, 0);
+          if (KEYS) {
+            const f2 x2 = yb[i & 1];
+            g2a = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.x, sc[i], g2a, 0, 0, 0);
+            g2b = __builtin_amdgcn_mfma_f32_32x32x2f32(x2.y, sc[i], g2b, 0, 0, 0);
+          }
+#if defined(__HIP_DEVICE_COMPILE__)
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, KEYS ? 2 : 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, KEYS ? 3 : 1, 0);
+#endif
         }
       }
     }
   };
 
-  // two stages: the next tile is fetched while this one is worked on; one barrier per tile
-  fetch(t_begin & 1, t_begin);
-  publish(t_begin & 1);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  for (int tile = t_begin; tile < t_end; tile++) {
+  // two stages: the next tile is fetched while this one is worked on; one barrier per tile.  The loop is
+  // unrolled by two so that a tile's stage is a constant.
+  auto step = [&](auto stage_c, int tile) {
+    constexpr int stage = decltype(stage_c)::value;
     const bool more = tile + 1 < t_end;
-    if (more) fetch((tile + 1) & 1, tile + 1);
-    compute(tile & 1, tile);
-    if (more) publish((tile + 1) & 1);
+    if (more) fetch(stage ^ 1, tile + 1);
+    compute(stage_c, tile);
+    if (more) publish(stage ^ 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's fetches have landed
     __syncthreads();
+  };
+  fetch(0, t_begin);
+  publish(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int tile = t_begin;
+  for (; tile + 2 <= t_end; tile += 2) {
+    step(std::integral_constant<int, 0>{}, tile);
+    step(std::integral_constant<int, 1>{}, tile + 1);
   }
+  if (tile < t_end) step(std::integral_constant<int, 0>{}, tile);
 
   auto write = [&](float* out, const f16v& ea, const f16v& eb, float factor) {
     // register i of ea / eb holds head dimension 2 r / 2 r + 1, r = 8 (i/4) + 4 half + i%4
