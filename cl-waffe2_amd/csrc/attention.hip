@@ -355,7 +355,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
 // P = exp2(S - L) needs no second pass over the keys) and D = sum_d dO O = sum_j P dP.  Per tile
 //   S = scale log2e Q K^T,  P = exp2(S - L),  dP = dO V^T,  dS = P (dP - D),
 //   dQ += scale dS K,   dK += scale dS^T Q,   dV += P^T dO,
-// and no (seq, seq) tensor is ever written.  One kernel body serves two launches:
+// and no (seq, seq) tensor is ever written.  One body serves both kinds of workgroup of the launch:
 //   KEYS = false  a lane owns a QUERY (Q and dO rows in registers), key / value tiles stream
 //                 through LDS, the accumulator is dQ            (the forward kernel's frame);
 //   KEYS = true   a lane owns a KEY (K and V rows in registers), query / dO tiles stream, the
@@ -413,17 +413,13 @@ __global__ __launch_bounds__(kBlock) void attention_delta_kernel(const float* __
 }
 
 template <bool KEYS>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_bwd_kernel(
-    AttnBwdParams p) {
+__device__ __forceinline__ void attention_bwd_body(const AttnBwdParams& p, const int rank, const int bh) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   auto tile1 = [&](int stage) { return smem + stage * kBwdStageFloats; };
   auto tile2 = [&](int stage) { return smem + stage * kBwdStageFloats + kKBlock * kRowFloats; };
   float* const stats = smem + 2 * kBwdStageFloats;  // [stage][L: 64, D: 64]
 
-  // longest first: the last query block walks the most key tiles, the first key block the most query tiles
-  const int nbh = p.batch * p.heads;
-  const int rank = blockIdx.x / nbh;
-  const int bh = blockIdx.x - rank * nbh;
+  // rank 0 is the longest: the last query block walks the most key tiles, the first key block the most query tiles
   const int rb = KEYS ? rank : p.rblocks - 1 - rank;
   const int b = bh / p.heads;
   const int h = bh - b * p.heads;
@@ -711,6 +707,25 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   }
 }
 
+// Both kinds of workgroup in one launch, handed out by rank (longest first), keys-resident before
+// queries-resident within a rank (128 against 96 MFMAs per sub-tile): 2 x 768 workgroups of very unequal
+// length at (8, 12, 1024) leave a much shorter tail than two launches of 768 that each end with the compute
+// units that drew the longest workgroups finishing alone.
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) void attention_bwd_kernel(
+    AttnBwdParams p) {  // two workgroups per CU: at most 256 registers per lane
+  const int nbh = p.batch * p.heads;
+  const int group = blockIdx.x / nbh;
+  const int bh = blockIdx.x - group * nbh;
+  // Without a mask every workgroup of a kind is as long as the others: one kind after the other then (two
+  // code bodies resident side by side cost 4 % in instruction fetches and have no tail to make up for).
+  const bool keys = p.causal ? (group & 1) == 0 : group < p.rblocks;
+  const int rank = p.causal ? group >> 1 : (keys ? group : group - p.rblocks);
+  if (keys)
+    attention_bwd_body<true>(p, rank, bh);
+  else
+    attention_bwd_body<false>(p, rank, bh);
+}
+
 // [lo, hi) in elements touched through (batch, head, position) strides
 static void extent3(const float* base, const int64_t (&s)[3], int64_t nb, int64_t nh, int64_t nt,
                     int64_t head_dim, const float** lo, const float** hi) {
@@ -848,14 +863,12 @@ WF2_API int wf2hip_attention_backward_f32(const wf2hip_attention_desc* d, const 
   p.scale_log2e = d->scale * 1.44269504088896340736f;
   const int64_t blocks = (int64_t)p.rblocks * p.batch * p.heads;
   if (blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "attention backward: too many workgroups");
+  if (2 * blocks >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "attention backward: too many workgroups");
   static bool configured = false;
   if (!configured) {
-    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_kernel<false>),
+    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAttnBwdLdsBytes),
-                      "hipFuncSetAttribute(attention_bwd_kernel<false>)"));
-    WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_kernel<true>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAttnBwdLdsBytes),
-                      "hipFuncSetAttribute(attention_bwd_kernel<true>)"));
+                      "hipFuncSetAttribute(attention_bwd_kernel)"));
     configured = true;
   }
   const int64_t rows = d->batch * d->heads * d->seq;
@@ -869,12 +882,8 @@ WF2_API int wf2hip_attention_backward_f32(const wf2hip_attention_desc* d, const 
       o, dout, p.os[0], p.os[1], p.os[2], p.heads, p.seq, p.head_dim, rows, static_cast<float*>(delta));
   int rc = after_launch("attention_delta_kernel");
   if (rc == 0) {
-    attention_bwd_kernel<false><<<(uint32_t)blocks, kBlock, kAttnBwdLdsBytes, st>>>(p);
-    rc = after_launch("attention_bwd_kernel<false>");
-  }
-  if (rc == 0) {
-    attention_bwd_kernel<true><<<(uint32_t)blocks, kBlock, kAttnBwdLdsBytes, st>>>(p);
-    rc = after_launch("attention_bwd_kernel<true>");
+    attention_bwd_kernel<<<(uint32_t)(2 * blocks), kBlock, kAttnBwdLdsBytes, st>>>(p);
+    rc = after_launch("attention_bwd_kernel");
   }
   (void)wf2hip_free(delta);  // stream order keeps it alive for the launches above
   return rc;

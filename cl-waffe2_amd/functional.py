@@ -845,7 +845,7 @@ def attention_backward(q: HIPTensor, k: HIPTensor, v: HIPTensor, dout: HIPTensor
     products form their lower triangles only and dS K skips the tiles above the diagonal.
     ``fused=False`` takes the softmax gradient node for node and every product in full.
     With the forward pass's output ``out`` and row statistics ``lse`` (`attention(..., lse=)`) the
-    whole backward is HIP-Attention-Node-backward instead: three launches, no (seq, seq) tensor."""
+    whole backward is HIP-Attention-Node-backward instead: two launches, no (seq, seq) tensor."""
     hd = q.shape[-1]
     scale = 1.0 / math.sqrt(hd) if scale is None else float(scale)
     if out is not None and lse is not None:

@@ -810,8 +810,9 @@ int wf2hip_attention_forward_f32(const wf2hip_attention_desc* desc, const float*
 /* dQ, dK, dV of that forward pass from Q, K, V, its output O, the upstream gradient dO and
  * lse, without materialising a (seq, seq) tensor: the backward of the !matmul / !softmax /
  * !matmul chain (MatMulNode's backward, source/base-impl/matrix-ops.lisp:10-15; !softmax's
- * through its composition, source/nn/activation.lisp:126-159) in three launches
- * (D = sum_d dO O per query; dQ with queries resident; dK and dV with keys resident).
+ * through its composition, source/nn/activation.lisp:126-159) in two launches
+ * (D = sum_d dO O per query; then workgroups with queries resident that form dQ and
+ * workgroups with keys resident that form dK and dV, handed out longest first).
  * dO is addressed through o_stride; dQ, dK, dV through q_stride, k_stride, v_stride, so they
  * can be windows of one fused-projection gradient.  The gradients may not overlap anything
  * that is read.  Allocates 4 * batch * heads * seq bytes of scratch from the library's pool.
