@@ -67,6 +67,9 @@ struct GemmParams {
   //    K loop of a row tile stops at its last row
   int32_t causal;
   int32_t pair_ok;  // C (and residual) rows allow 8-byte stores at even columns
+  // 1: the tile (i, j) is stored at C[j * ldc + i] (bias indexed by i, residual laid out like C): the product
+  // was handed over with its operands exchanged; 2: the same, and C / residual allow 16-byte accesses along i
+  int32_t transposed;
 };
 
 // Loads this thread's share of a ROWS x BK operand tile into registers
@@ -580,6 +583,55 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(2))) voi
   // D layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile.
   const int64_t res_base = (int64_t)zo * p.sRes2 + (int64_t)zi * p.sRes;
+  if constexpr (RKIN && TN == 1 && !TALL) {
+    if (p.transposed) {
+      // The output of a product with few rows, computed with the operands exchanged so that the long
+      // operand is the one with 128 rows per tile (gemm.hip, sgemm_batched2): the 128 x 64 tile is turned
+      // over in LDS (the stages are free once every wavefront has passed the last barrier of the K loop:
+      // none reads LDS after it) and leaves in runs along its 128 rows, which are contiguous in C.
+      constexpr int TP = BMt + 1;  // pitch of a tile column: lanes hold 32 consecutive columns
+      float* turn = smem;
+#pragma unroll
+      for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          turn[(wn + col) * TP + wm + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3)] = acc[i][0][r];
+      __syncthreads();
+      const float* res = (FUSED && p.residual) ? p.residual + res_base : nullptr;
+      // thread t: rows 4 (t % 32) ... + 3 of columns t / 32, t / 32 + 8, ...
+      const int r4 = 4 * (threadIdx.x & 31);
+      const int64_t gi = m0 + r4;
+      float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (FUSED && p.bias) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) bias4[c] = gi + c < p.M ? p.bias[gi + c] : 0.f;
+      }
+      for (int cj = threadIdx.x >> 5; cj < BNt; cj += kBlock / 32) {
+        const int64_t gj = n0 + cj;
+        if (gj >= p.N || gi >= p.M) continue;
+        float* c_out = C + gj * p.ldc + gi;
+        const float* r_in = res ? res + gj * p.ldres + gi : nullptr;
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[c] = turn[cj * TP + r4 + c];
+        if (p.transposed == 2 && gi + 3 < p.M) {
+          f4 old = {0.f, 0.f, 0.f, 0.f}, rs = {0.f, 0.f, 0.f, 0.f};
+          if (p.beta != 0.0f) old = *reinterpret_cast<const f4*>(c_out);
+          if (r_in) rs = *reinterpret_cast<const f4*>(r_in);
+          f4 o;
+#pragma unroll
+          for (int c = 0; c < 4; c++) o[c] = finish_value<FUSED>(p, v[c], old[c], bias4[c], rs[c]);
+          *reinterpret_cast<f4*>(c_out) = o;
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; c++)
+            if (gi + c < p.M)
+              c_out[c] = finish_value<FUSED>(p, v[c], p.beta != 0.0f ? c_out[c] : 0.f, bias4[c], r_in ? r_in[c] : 0.f);
+        }
+      }
+      return;
+    }
+  }
   const bool pairs = !TALL && !RKIN && TN >= 2 && p.pair_ok;
   const float* res = (FUSED && p.residual) ? p.residual + res_base : nullptr;
   if constexpr (!TALL) {
@@ -1055,8 +1107,20 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
                               strideB2, beta, C, ldc, strideC, strideC2, batch, batch2, &rc))
       return rc;
   }
+  // 33 ... 64 rows of the row-major product against a weight stored (cols, k) (`(!matmul x (!t w))`: a few
+  // dozen tokens against the token table): the few-rows kernel below feeds the matrix cores from global
+  // memory and keeps them busy about a third of the time at this height, and the tiled kernels pad the rows
+  // to 128.  With the operands exchanged the weight is the operand with 128 rows per tile and the tokens are
+  // the 64 columns of a 128 x 64 tile, nothing padded; the streaming kernel turns each tile over in LDS on the
+  // way out ((64, 768) . (50257, 768)^T: 96 -> 62 us; with few tiles the slices of K below come first).
+  static const char* turn_env = getenv("WF2HIP_GEMM_TURN_ROWS");  // testing knob: least number of rows, 0 = never
+  const long turn_from = turn_env ? atol(turn_env) : 33;
+  const bool turned = turn_from > 0 && n >= turn_from && n <= 64 && m >= 1024 && is_n(transb) && !is_n(transa) &&
+                      ep.causal == 0 && k % BK == 0 && k >= 256 && aligned16(A) && aligned16(B) && lda % 4 == 0 &&
+                      ldb % 4 == 0 && lda < ((long)1 << 22) && ldb < ((long)1 << 22) && strideA % 4 == 0 &&
+                      strideB % 4 == 0 && strideA2 % 4 == 0 && strideB2 % 4 == 0;
   // at most 64 rows in the row-major product (a few tokens through a layer): one read of the other operand
-  if (batch == 1 && batch2 == 1 && n <= 64 && is_n(transb) && ep.causal == 0) {
+  if (!turned && batch == 1 && batch2 == 1 && n <= 64 && is_n(transb) && ep.causal == 0) {
     int rc = 0;
     if (try_sgemm_skinny(!is_n(transa), n, m, k, alpha, A, lda, B, ldb, beta, C, ldc, ep.bias, ep.residual, ep.ldres,
                          ep.activation, &rc))
@@ -1113,6 +1177,44 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
       return rc;
   }
 
+  if (turned) {
+    GemmParams p;
+    p.L = A;  // the weight: m rows of k
+    p.R = B;  // the tokens: n rows of k, the columns of the turned product
+    p.C = C;
+    p.M = m;
+    p.N = n;
+    p.K = k;
+    p.ldl = lda;
+    p.ldr = ldb;
+    p.ldc = ldc;
+    p.sL = strideA;
+    p.sR = strideB;
+    p.sC = strideC;
+    p.sL2 = strideA2;
+    p.sR2 = strideB2;
+    p.sC2 = strideC2;
+    p.batch_inner = (uint32_t)batch;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.bias = ep.bias;
+    p.residual = ep.residual;
+    p.ldres = ep.ldres;
+    p.sRes = ep.sRes;
+    p.sRes2 = ep.sRes2;
+    p.activation = ep.activation;
+    p.causal = 0;
+    p.pair_ok = 0;
+    auto by4 = [](int64_t v) { return (v & 3) == 0; };
+    const bool vec4 = ((uintptr_t)C % 16 == 0) && by4(ldc) && by4(strideC) && by4(strideC2) &&
+                      (!ep.residual || (((uintptr_t)ep.residual % 16 == 0) && by4(ep.ldres) && by4(ep.sRes) && by4(ep.sRes2)));
+    p.transposed = vec4 ? 2 : 1;
+    p.tiles_m = (uint32_t)ceil_div(p.M, 128);
+    p.tiles_n = 1;
+    WF2_TRY((launch_dma<1>(p, true, dim3(p.tiles_m, (uint32_t)((int64_t)batch * batch2)), rt().stream)));
+    return after_launch("sgemm_dma_kernel");
+  }
+
   GemmParams p;
   // row-major view: Cr[n][m] = Left[n][k] . Right[k][m]
   p.L = B;
@@ -1140,6 +1242,7 @@ int sgemm_batched2(char transa, char transb, long m, long n, long k, float alpha
   p.sRes2 = ep.sRes2;
   p.activation = ep.activation;
   p.causal = ep.causal;
+  p.transposed = 0;
   const bool lkin = is_n(transb);   // left stored [rows][k]
   const bool rkin = !is_n(transa);  // right stored [cols][k]
   bool fast = aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && strideA % 4 == 0 &&

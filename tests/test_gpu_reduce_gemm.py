@@ -669,6 +669,40 @@ def test_matmul_few_rows(gpu, rows, cols, k):
         assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
 
 
+@pytest.mark.parametrize("rows", [33, 48, 64])
+@pytest.mark.parametrize("cols,k", [(1024, 256), (4100, 768), (2051, 512), (2048, 4096), (50257, 768)])
+def test_matmul_33_to_64_rows_against_a_table(gpu, rows, cols, k):
+    """33 ... 64 rows against a weight stored (cols, k) (`(!matmul x (!t w))`, the token projection of the GPT-2
+    example, examples/gpt-2/model.lisp:137-196) run with the operands exchanged through the streaming kernel,
+    whose tiles are turned over on the way out: ragged last tiles, column counts that rule out 16-byte stores,
+    few tiles over a long K (slices of K first), and the fused epilogue -- bias per column of the row-major
+    product, GELU, residual -- on that path; all against float64 at the bar of every product."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows * 7919 + cols + k)
+    X = rng.standard_normal((rows, k)).astype(np.float32)
+    Wt = (rng.standard_normal((cols, k)) / np.sqrt(k)).astype(np.float32)
+    X64, W64 = X.astype(np.float64), Wt.astype(np.float64).T
+    dX, dW = F.from_numpy(X), F.from_numpy(Wt)
+    _gemm_check(F.matmul(dX, F.t(dW)).numpy(), X64, W64)
+    if cols > 5000:
+        return
+    bias = rng.standard_normal(cols).astype(np.float32)
+    res = rng.standard_normal((rows, cols)).astype(np.float32)
+    z = X64 @ W64 + bias
+    bound = REL * (np.abs(X64) @ np.abs(W64) + np.abs(bias)) + 1e-30
+    got = F.matmul(dX, F.t(dW), bias=F.from_numpy(bias), residual=F.from_numpy(res)).numpy()
+    assert np.all(np.abs(got - (z + res)) <= bound + REL * np.abs(res))
+    got = F.matmul(dX, F.t(dW), bias=F.from_numpy(bias), activation="gelu").numpy()
+    gelu = 0.5 * z * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))
+    assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
+    # an output that is a window of a wider tensor (rows of padding stay untouched) and starts off a 16-byte boundary
+    wide = F.from_numpy(np.full((rows, cols + 5), 7.0, np.float32))
+    F.matmul(dX, F.t(dW), out=wide.view(True, (1, cols + 1)))
+    got = wide.numpy()
+    _gemm_check(got[:, 1:cols + 1], X64, W64)
+    assert np.all(got[:, 0] == 7.0) and np.all(got[:, cols + 1:] == 7.0)
+
+
 def test_sgemm_few_rows_column_major_contract(gpu):
     """The same kernel through wf2hip_sgemm: column-major C (m x n, n <= 64) with padded leading dimensions,
     alpha and beta, both storages of A; rows of padding stay untouched."""
