@@ -593,7 +593,7 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
 
     # products on fp32 MFMA, random data
     for m, n, k in ((8192, 8192, 8192), (4096, 4096, 4096), (8192, 2304, 768), (8192, 3072, 768),
-                    (8192, 768, 3072)):
+                    (8192, 768, 3072), (8192, 768, 768)):
         a0, b0 = normal([m, k]), normal([k, n])
         ring = ring_of(lambda: (clone(a0), clone(b0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
         measure(f"matmul {m}x{n}x{k}", ring, lambda s: F.matmul(s[0], s[1], out=s[2]), 2.0 * m * n * k,
@@ -640,16 +640,16 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         measure(f"attention (8,12,1024,64) {'causal' if causal else 'full'}", ring,
                 lambda s, c=causal: F.attention(s[0], s[1], s[2], out=s[3], causal=c), flop, bound="mfma",
                 note="flop of the useful half of the score matrix" if causal else None)
-    # the backward of the same attention (three launches: D per query, dQ, dK and dV)
+    # the backward of the same attention (two launches: D per query; dQ, dK and dV)
     lse = T([B, H, S], initial_element=None)
     o0 = F.attention(q0, q0, q0, causal=True, lse=lse)
     ring = ring_of(lambda: (clone(q0), clone(q0), clone(q0), clone(q0), T([B, H, S, hd], initial_element=None),
                             T([B, H, S, hd], initial_element=None), T([B, H, S, hd], initial_element=None)),
                    28 * B * H * S * hd)
-    measure("attention backward (8,12,1024,64) causal: dQ, dK, dV (three launches)", ring,
+    measure("attention backward (8,12,1024,64) causal: dQ, dK, dV (two launches)", ring,
             lambda s: F.attention_backward(s[0], s[1], s[2], s[3], causal=True, dq=s[4], dk=s[5], dv=s[6], out=o0, lse=lse),
             10.0 * B * H * S * S * hd * 0.5, bound="mfma",
-            note="flop of the useful half of the five products a backward needs at least (the kernels form seven)")
+            note="flop of the useful half of the five products a backward needs at least (the kernel forms seven)")
     del q0, o0, lse
     return rows
 
@@ -784,6 +784,40 @@ def cpu_block_forward_ms():
     return out
 
 
+# Short names for the rows of the BASELINE configurations and of the kernels that bound the block, for
+# a compact last key of the JSON line: whoever keeps only the end of the line still sees every
+# configuration.  name -> the start of the row's label in `rows`.
+COMPACT_ROWS = (
+    ("cfg1_add", "add (1024,1024)"), ("cfg2_bcast_add", "A(4096,8192) += B"), ("cfg2_stride2_mul", "A[:, 0:8192:2] *= 0.5"),
+    ("cfg2_slice_copy", "copy of A[:, 0:8192:2]"), ("cfg2_offset_sub", "C = A[1024:3072]"),
+    ("cfg3_exp", "exp 2^26"), ("cfg3_tanh", "tanh 2^26"), ("cfg3_sin", "sin 2^26"), ("cfg3_log", "loge 2^26"),
+    ("cfg4_rowsum", "row sum (8192,4096), !sum as one node"), ("cfg4_fullsum", "full sum (8192,4096)"),
+    ("cfg4_softmax", "row softmax (32768,1024), one kernel"), ("copy_536MB", "copy 2^26"), ("copy_268MB", "copy (32768,1024)"),
+    ("layernorm", "LayerNorm (65536,1024)"), ("layernorm_bwd", "LayerNorm backward"), ("adam", "Adam step"),
+    ("transpose", "transposing copy"), ("unfold", "unfold (32,64,56,56) 3x3 pad 1, one kernel"),
+    ("im2col", "Im2ColNode (32,64,58,58)"), ("im2col_pad", "Im2ColNode, padding 1"), ("col2im", "Col2ImNode"),
+    ("mm_8192x2304x768", "matmul 8192x2304x768"), ("mm_8192x3072x768", "matmul 8192x3072x768"),
+    ("mm_8192x768x3072", "matmul 8192x768x3072"), ("mm_8192x768x768", "matmul 8192x768x768"), ("mm_4096^3", "matmul 4096x4096x4096"),
+    ("mm_dW_splitK", "matmul 768x3072x8192"), ("mm_16x50257x768", "matmul 16x50257x768"), ("mm_64x50257x768", "matmul 64x50257x768"),
+    ("attn_causal", "attention (8,12,1024,64) causal"), ("attn_full", "attention (8,12,1024,64) full"),
+    ("attn_bwd_causal", "attention backward"),
+)
+
+
+def compact_rows(rows, block):
+    """{short name: [ms, fraction of the bounding peak]} for COMPACT_ROWS, plus the fused block forward."""
+    out = {}
+    for name, start in COMPACT_ROWS:
+        for label, row in rows.items():
+            if label.startswith(start):
+                out[name] = [round(row["ms"], 4), round(row["frac"], 3)]
+                break
+    if block:
+        out["cfg5_block_fused_ms"] = round(block.get("fused_graph", block.get("fused", 0.0)), 4)
+        out["cfg5_block_fused_eager_ms"] = round(block.get("fused", 0.0), 4)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -881,6 +915,8 @@ def main():
                 k: round(flop / v / 1e9, 1) for k, v in blk.items() if "backward" not in k}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
+    if "rows" in result:  # last, and short
+        result["baseline_rows"] = compact_rows(result["rows"], result.get("gpt2_block_fwd_ms"))
     print(json.dumps(result))
 
 
