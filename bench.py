@@ -314,14 +314,73 @@ def matrix_core_probe(W, reps: int = 4):
             F.attention(q, k, v, out=out, causal=causal, lse=lse)
     for _ in range(reps):
         F.attention_backward(q, k, v, dout, causal=True, dq=dq, dk=dk, dv=dv, out=out, lse=lse)
-    a = T.from_numpy(rng.standard_normal((B * S, 768)).astype(np.float32))
-    b = T.from_numpy(rng.standard_normal((768, 3072)).astype(np.float32))
-    c = T([B * S, 3072], initial_element=None)
-    for _ in range(reps):
-        F.matmul(a, b, out=c)
+    # the four projections of the block with their epilogues (bias; bias + residual; bias + GELU), the
+    # plain product of the widest one, and a cube
+    M = B * S
+    names = []
+    for m, n, k, bias, res, act in ((M, 2304, 768, True, False, None), (M, 768, 768, True, True, None),
+                                    (M, 3072, 768, True, False, "gelu"), (M, 768, 3072, True, True, None),
+                                    (M, 3072, 768, False, False, None), (4096, 4096, 4096, False, False, None)):
+        a = T.from_numpy(rng.standard_normal((m, k)).astype(np.float32))
+        b = T.from_numpy((rng.standard_normal((k, n)) * 0.02).astype(np.float32))
+        c = T([m, n], initial_element=None)
+        bv = T.from_numpy(rng.standard_normal(n).astype(np.float32)) if bias else None
+        rv = T.from_numpy(rng.standard_normal((m, n)).astype(np.float32)) if res else None
+        for _ in range(reps):
+            F.matmul(a, b, out=c, bias=bv, residual=rv, activation=act)
+        names.append(f"matmul {m}x{n}x{k}" + (" + bias" if bias else "") + (" + residual" if res else "") +
+                     (" + GELU" if act else ""))
+        del a, b, c, bv, rv
     W.lib.synchronize()
     print(json.dumps({"probe_matrix_cores": ["attention (8,12,1024,64) full", "attention causal",
-                                             "attention backward causal", "matmul 8192x3072x768"],
+                                             "attention backward causal (D, then dQ / dK / dV)"] + names,
+                      "launches_each": reps}))
+
+
+def size_probe(W, reps: int = 6):
+    """The launch sequence behind profiles/short_kernel_fit.txt: four kernels of the path (plain copy,
+    row-broadcast add, row sum as one node, row softmax) at six sizes from 32 MB to 1 GB moved per launch,
+    `reps` launches each on a ring of buffer sets larger than the Infinity Cache.  Their durations under
+    `rocprofv3 --kernel-trace`, fitted as t = t0 + bytes / rate, separate the fixed cost of a launch (ramp
+    and drain) from the rate the kernel streams at."""
+    F = W.functional
+    T = W.HIPTensor
+    rng = np.random.Generator(np.random.PCG64(6))
+    cases = []
+    for mb in (32, 64, 128, 256, 512, 1024):
+        moved = mb << 20
+        n = moved // 8                      # elements of a kernel that reads and writes each once
+        count = max(2, -(-(768 << 20) // moved) + 1)
+        src = T.from_numpy(rng.standard_normal(1 << 22).astype(np.float32))
+
+        def fresh(shape):
+            t = T(list(shape), initial_element=None)
+            flat = F.reshape(t, -1)
+            for lo in range(0, flat.shape[0], 1 << 22):  # fill from the 16 MB sample
+                hi = min(lo + (1 << 22), flat.shape[0])
+                F.move_(flat.view((lo, hi)), src.view((0, hi - lo)))
+            return t
+
+        ring = [(fresh([n]), T([n], initial_element=None)) for _ in range(count)]
+        for i in range(reps):
+            F.move_(ring[i % count][1], ring[i % count][0])
+        cases.append(("copy", moved, n))
+        row = fresh([1, 8192]).view((":broadcast", n // 8192), True)
+        for i in range(reps):
+            F.add_(F.reshape(ring[i % count][0], n // 8192, 8192), row)
+        cases.append(("row-broadcast add, rows of 8192", moved, n))
+        for i in range(reps):
+            F.softmax_fused(F.reshape(ring[i % count][0], n // 1024, 1024), out=F.reshape(ring[i % count][1], n // 1024, 1024))
+        cases.append(("row softmax, rows of 1024", moved, n))
+        del ring, row
+        n4 = moved // 4                     # the row sum reads every element once
+        ring = [(fresh([n4 // 4096, 4096]), T([n4 // 4096, 1])) for _ in range(count)]
+        for i in range(reps):
+            F.sum(ring[i % count][0], axis=1, out=ring[i % count][1], keepdims=True)
+        cases.append(("row sum, rows of 4096", moved, n4))
+        del ring
+        W.lib.synchronize()
+    print(json.dumps({"probe_sizes": [{"kernel": k, "bytes": b, "elements": e} for k, b, e in cases],
                       "launches_each": reps}))
 
 
@@ -833,6 +892,8 @@ def main():
                     help="run the launch sequence of the other kernels of the path for rocprofv3 --pmc runs and exit")
     ap.add_argument("--probe-matrix-cores", action="store_true",
                     help="run the launch sequence of the attention kernels and one projection for rocprofv3 --pmc runs and exit")
+    ap.add_argument("--probe-sizes", action="store_true",
+                    help="run four kernels of the path at six sizes (32 MB ... 1 GB moved) for a rocprofv3 --kernel-trace run and exit")
     ap.add_argument("--probe", action="store_true",
                     help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
@@ -851,6 +912,9 @@ def main():
         return
     if args.probe_matrix_cores:
         matrix_core_probe(W)
+        return
+    if args.probe_sizes:
+        size_probe(W)
         return
 
     step_ms, wall_ms, per_kernel, binary_ms, sustained_ms = gpu_steps(W, args.steps, args.warmup)
