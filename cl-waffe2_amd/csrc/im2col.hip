@@ -172,6 +172,9 @@ __global__ __launch_bounds__(kBlock) void im2col_flat(Unfold32 p, ColStep d, uin
 // above takes as long as a copy of col, 79 us for the 231 MB of a (32, 64, 58, 58) image with a
 // 3 x 3 kernel, although it fetches only the 28 MB of the image from HBM), so the K_H K_W-fold
 // reuse has to happen inside the workgroup.
+// VEC: every band of every plane of col starts on a 16-byte boundary: a lane takes four consecutive
+// elements and they leave in one 16-byte nontemporal store (single stores where the walk skips one of them).
+template <bool VEC>
 __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands, uint32_t band_rows) {
   extern __shared__ float tile[];  // the image rows y0 ..., W floats each
   const uint32_t nc = blockIdx.x / bands, band = blockIdx.x - nc * bands;
@@ -196,6 +199,81 @@ __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands,
   }
   __syncthreads();
   const uint32_t band_elems = rows_here * p.W_out;
+  if constexpr (VEC) {
+    // A thread's vectors (four consecutive elements of the band) are the same in every (kh, kw) plane:
+    // their positions in the band and in the tile are worked out once, and a plane costs four LDS reads,
+    // a few additions and one store per vector.  Planes the walk covers whole (no padding argument) skip
+    // the tests; elsewhere the elements the walk does not reach are stored one by one around the hole.
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int NV = 8;  // vectors per thread and pass
+    for (uint32_t base = 0; base < band_elems; base += 4 * kBlock * NV) {
+      uint32_t toff[NV][4];   // tile offset of element c of vector u for kh = kw = 0
+      uint32_t xs[NV][4], ys[NV][4];
+      bool live[NV];
+#pragma unroll
+      for (int u = 0; u < NV; u++) {
+        const uint32_t e = base + 4 * (threadIdx.x + u * kBlock);
+        live[u] = e < band_elems;
+        uint32_t j;
+        uint32_t il = fd_divmod(live[u] ? e : 0, p.by_w_out, &j);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          ys[u][c] = (i0 + il) * p.s_h;
+          xs[u][c] = j * p.s_w;
+          toff[u][c] = (ys[u][c] - y0) * p.W + xs[u][c];
+          if (++j == p.W_out) {
+            j = 0;
+            il++;
+          }
+        }
+      }
+      for (uint32_t kh = 0; kh < p.K_H; kh++) {
+        const uint32_t end_h = walk_end(p.d_h, kh, p.pad_h, p.s_h, p.H_out);
+        for (uint32_t kw = 0; kw < p.K_W; kw++) {
+          const uint32_t end_w = walk_end(p.d_w, kw, p.pad_w, p.s_w, p.W_out);
+          float* dst = p.dst + (((size_t)nc * p.K_H + kh) * p.K_W + kw) * p.plane_elems + i0 * p.W_out + base;
+          const uint32_t shift = kh * p.W + kw;
+          // the whole band of this plane is reached: the last element of the band lies inside both walks
+          // (a band is a whole number of vectors: a vector lies inside it or outside)
+          const bool whole = kh + (i0 + rows_here - 1) * p.s_h < end_h && kw + (p.W_out - 1) * p.s_w < end_w;
+          if (whole) {
+#pragma unroll
+            for (int u = 0; u < NV; u++) {
+              if (!live[u]) continue;
+              f4 v;
+#pragma unroll
+              for (int c = 0; c < 4; c++) v[c] = tile[toff[u][c] + shift];
+              __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst + 4 * (threadIdx.x + u * kBlock)));
+            }
+          } else {
+#pragma unroll
+            for (int u = 0; u < NV; u++) {
+              if (!live[u]) continue;
+              const uint32_t e = base + 4 * (threadIdx.x + u * kBlock);
+              f4 v;
+              bool on[4];
+#pragma unroll
+              for (int c = 0; c < 4; c++) {
+                on[c] = e + c < band_elems && kh + ys[u][c] < end_h && kw + xs[u][c] < end_w;
+                v[c] = on[c] ? tile[toff[u][c] + shift] : 0.0f;
+              }
+              float* d = dst + 4 * (threadIdx.x + u * kBlock);
+              if (on[0] && on[1] && on[2] && on[3]) {
+                __builtin_nontemporal_store(v, reinterpret_cast<f4*>(d));
+              } else {
+                // around a hole: single stores (reading the vector, merging and writing it back whole is
+                // slower: 114 against 98 us for the padded walk of a (32, 64, 58, 58) image)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                  if (on[c]) d[c] = v[c];
+              }
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
   for (uint32_t kh = 0; kh < p.K_H; kh++) {
     const uint32_t end_h = walk_end(p.d_h, kh, p.pad_h, p.s_h, p.H_out);
     for (uint32_t kw = 0; kw < p.K_W; kw++) {
@@ -422,7 +500,10 @@ struct UnfoldFused {
   FastDiv by_kk, by_kw, by_w_out, by_plane, by_tw;  // K_H K_W, K_W, W_out, TR TW, TW
 };
 
-template <int NQ>  // entries of a run per lane: cc K_H K_W <= 64 NQ
+// VEC: runs are whole 16-byte vectors on 16-byte boundaries (cc K_H K_W and C K_H K_W multiples of 4, dst
+// aligned): a lane then owns NQ vectors of four consecutive entries and the matrix leaves in 16-byte
+// nontemporal stores, a quarter of the store instructions of the element form.
+template <int NQ, bool VEC = false>  // entries (VEC: vectors) of a run per lane: cc K_H K_W <= 64 NQ (256 NQ)
 __global__ __launch_bounds__(kBlock) void unfold_kernel(UnfoldFused p) {
   extern __shared__ float lds[];
   const uint32_t KK = p.K_H * p.K_W;
@@ -480,6 +561,31 @@ __global__ __launch_bounds__(kBlock) void unfold_kernel(UnfoldFused p) {
   // A wavefront owns the positions r = wave, wave + 4, ...; its lanes sweep the run, NQ entries
   // each, whose tile offsets stay in registers: an element is one LDS read and one store.
   const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if constexpr (VEC) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    uint32_t off[NQ][4];
+#pragma unroll
+    for (int m = 0; m < NQ; m++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const uint32_t qc = 4 * (lane + m * kWave) + c;
+        off[m][c] = qc < run ? qoff[qc] : 0;
+      }
+    for (uint32_t r = wave; r < R; r += kBlock / kWave) {
+      const uint32_t ro = roff[r];  // uniform over the wavefront
+      float* row = out + (size_t)r * p.Q;
+      f4 v[NQ];
+#pragma unroll
+      for (int m = 0; m < NQ; m++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[m][c] = ro == kSkipped ? 0.0f : tile[off[m][c] + ro];
+#pragma unroll
+      for (int m = 0; m < NQ; m++) {
+        const uint32_t qc = 4 * (lane + m * kWave);
+        if (qc < run) __builtin_nontemporal_store(v[m], reinterpret_cast<f4*>(row + qc));
+      }
+    }
+  } else {
   uint32_t off[NQ];
 #pragma unroll
   for (int m = 0; m < NQ; m++) {
@@ -497,6 +603,7 @@ __global__ __launch_bounds__(kBlock) void unfold_kernel(UnfoldFused p) {
       const uint32_t qc = lane + m * kWave;
       if (qc < run) row[qc] = v[m];
     }
+  }
   }
 }
 
@@ -535,8 +642,15 @@ WF2_API int wf2hip_im2col_f32(float* col, long N, long C, long H, long W, long H
       const int64_t bands = ceil_div(H_out, band_rows);
       const int64_t tile_rows = std::min<int64_t>((band_rows - 1) * stride_h + K_H, H);
       if (planes * bands < ((int64_t)1 << 31)) {
-        im2col_lds<<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
-            q, (uint32_t)bands, (uint32_t)band_rows);
+        static const char* vec_env = getenv("WF2HIP_UNFOLD_VEC");  // testing knob: 0 = stores of single elements
+        const bool vec = ((uintptr_t)col % 16) == 0 && (H_out * W_out) % 4 == 0 && (band_rows * W_out) % 4 == 0 &&
+                         !(vec_env && vec_env[0] == '0');
+        if (vec)
+          im2col_lds<true><<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
+              q, (uint32_t)bands, (uint32_t)band_rows);
+        else
+          im2col_lds<false><<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
+              q, (uint32_t)bands, (uint32_t)band_rows);
         return after_launch("im2col_lds");
       }
     }
@@ -675,8 +789,31 @@ WF2_API int wf2hip_unfold_f32(long N, long C, long H, long W, long K_H, long K_W
   const int64_t blocks = (int64_t)N * p.bands * p.chunks;
   if (blocks >= limit) return fail(WF2HIP_EUNSUPPORTED, "unfold: too many workgroups");
   const size_t bytes = (size_t)lds_floats(band, cc) * sizeof(float);
-  const int64_t per_lane = ceil_div(cc * KK, kWave);
   hipStream_t st = rt().stream;
+  static const char* vec_env = getenv("WF2HIP_UNFOLD_VEC");  // testing knob: 0 = stores of single elements
+  const bool vec = (cc * KK) % 4 == 0 && ((int64_t)C * KK) % 4 == 0 && ((uintptr_t)out % 16) == 0 &&
+                   !(vec_env && vec_env[0] == '0');
+  if (vec) {
+    const int64_t vecs_per_lane = ceil_div(cc * KK, (int64_t)kWave * 4);
+#define WF2_VCASE(NQ_)                                                                                           \
+  if (vecs_per_lane <= NQ_) {                                                                                    \
+    static bool configured = false;                                                                              \
+    if (!configured) {                                                                                           \
+      WF2_TRY(check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&unfold_kernel<NQ_, true>),            \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 64 << 10),              \
+                        "hipFuncSetAttribute(unfold_kernel)"));                                                  \
+      configured = true;                                                                                         \
+    }                                                                                                            \
+    unfold_kernel<NQ_, true><<<(uint32_t)blocks, kBlock, bytes, st>>>(p);                                        \
+    return after_launch("unfold_kernel");                                                                        \
+  }
+    WF2_VCASE(1)
+    WF2_VCASE(2)
+    WF2_VCASE(3)
+    WF2_VCASE(4)
+#undef WF2_VCASE
+  }
+  const int64_t per_lane = ceil_div(cc * KK, kWave);
 #define WF2_CASE(NQ_)                                                                                            \
   if (per_lane <= NQ_) {                                                                                         \
     static bool configured = false;                                                                              \
