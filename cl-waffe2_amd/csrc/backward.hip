@@ -614,6 +614,128 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __rest
   }
 }
 
+// Rows beyond 8192 columns, and rows beyond 2048 that cannot be read with 16-byte loads: the row in
+// pieces of 16384 columns.  layernorm_bwd_piece_sums reads x, dy and gamma once and leaves, per piece,
+// S_p = sum x, Q_p = sum (x - a_p)^2, D_p = sum gamma dy and C_p = sum gamma dy (x - a_p) about the
+// piece's own a_p = (float)(S_p / n_p); the row's sums follow from them without a pass that knows the
+// mean: sum gamma dy (x - mean) = sum_p [C_p + (a_p - mean) D_p].  layernorm_bwd_piece_apply folds them
+// per row and writes dx, 512 threads on a quarter of a piece each.  Its workgroup (quarter, group) walks
+// rows group, group + G, ... and leaves its column sums in row `group` of `partial`, folded like the narrower kernels' (with one group they are
+// dgamma and dbeta themselves).  The formulas of layernorm_bwd_rows.
+template <bool VEC>
+__global__ __launch_bounds__(kPieceBlock) void layernorm_bwd_piece_sums(const float* __restrict__ x,
+                                                                       const float* __restrict__ gamma,
+                                                                       const float* __restrict__ dy, int64_t ncols,
+                                                                       uint32_t pieces, double* __restrict__ psum,
+                                                                       double* __restrict__ pdev,
+                                                                       double* __restrict__ pd, double* __restrict__ pc) {
+  __shared__ double lds[2 * kPieceBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const int64_t c0 = (int64_t)piece * kPieceCols;
+  const int64_t left = ncols - c0;
+  const int64_t n = left < kPieceCols ? left : kPieceCols;
+  PieceRegs<VEC> xr, dr, g;
+  xr.load(x + (int64_t)row * ncols + c0, left, 0.0f);
+  dr.load(dy + (int64_t)row * ncols + c0, left, 0.0f);
+  g.load(gamma + c0, left, 0.0f);
+  double sum = 0.0;
+  float s1[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < kPieceE; k++) {
+    sum += (double)xr.v[k];
+    dr.v[k] *= g.v[k];
+    s1[k & 1] += dr.v[k];
+  }
+  double d_total;
+  const double total = piece_sum2(sum, (double)s1[0] + (double)s1[1], lds, &d_total);
+  const float a = (float)(total / (double)n);
+  float sq[2] = {0.0f, 0.0f}, s2[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < kPieceE; k++) {
+    const float d = PieceRegs<VEC>::col(k) < left ? xr.v[k] - a : 0.0f;
+    sq[k & 1] = __builtin_fmaf(d, d, sq[k & 1]);
+    s2[k & 1] = __builtin_fmaf(dr.v[k], d, s2[k & 1]);
+  }
+  double c_total;
+  const double dev = piece_sum2((double)sq[0] + (double)sq[1], (double)s2[0] + (double)s2[1], lds, &c_total);
+  if (threadIdx.x == 0) {
+    psum[blockIdx.x] = total;
+    pdev[blockIdx.x] = dev;
+    pd[blockIdx.x] = d_total;
+    pc[blockIdx.x] = c_total;
+  }
+}
+
+// five registers per element: 512 threads on 4096 columns, so that two workgroups per compute unit
+// cover each other's exchanges
+constexpr int kApplyBlock = 512;
+constexpr int kApplyE = 8;
+constexpr int64_t kApplyCols = (int64_t)kApplyBlock * kApplyE;
+
+template <bool VEC>
+__global__ __launch_bounds__(kApplyBlock) void layernorm_bwd_piece_apply(const float* __restrict__ x,
+                                                                        const float* __restrict__ gamma,
+                                                                        const float* dy,  // dx may be dy
+                                                                        float eps, float* dx, float* __restrict__ out_g,
+                                                                        float* __restrict__ out_b, int64_t nrows,
+                                                                        int64_t ncols, uint32_t pieces,
+                                                                        const double* __restrict__ psum,
+                                                                        const double* __restrict__ pdev,
+                                                                        const double* __restrict__ pd,
+                                                                        const double* __restrict__ pc) {
+  __shared__ double lds[2 * kApplyBlock / kWave];
+  const uint32_t piece = blockIdx.x;
+  const int64_t c0 = (int64_t)piece * kApplyCols;
+  const int64_t left = ncols - c0;
+  typedef PieceRegs<VEC, kApplyBlock, kApplyE> Regs;
+  Regs g, dg, db;
+  g.load(gamma + c0, left, 0.0f);
+#pragma unroll
+  for (int k = 0; k < kApplyE; k++) dg.v[k] = db.v[k] = 0.0f;
+  for (int64_t row = blockIdx.y; row < nrows; row += gridDim.y) {
+    Regs xr, dr;
+    xr.load(x + row * ncols + c0, left, 0.0f);
+    dr.load(dy + row * ncols + c0, left, 0.0f);
+    const double* rs = psum + row * pieces;
+    const double* rq = pdev + row * pieces;
+    const double* rd = pd + row * pieces;
+    const double* rc = pc + row * pieces;
+    double s = 0.0, d_sum = 0.0;
+    for (uint32_t i = threadIdx.x; i < pieces; i += kApplyBlock) {
+      s += rs[i];
+      d_sum += rd[i];
+    }
+    double t1;
+    const double mean = piece_sum2<kApplyBlock>(s, d_sum, lds, &t1) / (double)ncols;
+    double q = 0.0, c_sum = 0.0;
+    for (uint32_t i = threadIdx.x; i < pieces; i += kApplyBlock) {
+      const int64_t l = ncols - (int64_t)i * kPieceCols;
+      const double n = (double)(l < kPieceCols ? l : kPieceCols);
+      const double mu = rs[i] / n;
+      const double a = (double)(float)mu;
+      q += rq[i] + n * ((mu - mean) * (mu - mean) - (mu - a) * (mu - a));
+      c_sum += rc[i] + (a - mean) * rd[i];
+    }
+    double t2;
+    const double var = piece_sum2<kApplyBlock>(q, c_sum, lds, &t2) / (double)ncols;
+    const float meanf = (float)mean;
+    const double rstd64 = 1.0 / __builtin_sqrt((var > 0.0 ? var : 0.0) + (double)eps);
+    const float rstd = (float)rstd64;
+    const float m1 = (float)(t1 / (double)ncols), m2 = (float)(t2 * rstd64 / (double)ncols);
+#pragma unroll
+    for (int k = 0; k < kApplyE; k++) {
+      const float xh = Regs::col(k) < left ? (xr.v[k] - meanf) * rstd : 0.0f;
+      const float d = dr.v[k];
+      dg.v[k] = __builtin_fmaf(d, xh, dg.v[k]);
+      db.v[k] += d;
+      xr.v[k] = rstd * ((d * g.v[k] - m1) - xh * m2);
+    }
+    xr.store(dx + row * ncols + c0, left);
+  }
+  dg.store(out_g + (int64_t)blockIdx.y * 2 * ncols + c0, left);
+  db.store(out_b + (int64_t)blockIdx.y * 2 * ncols + c0, left);
+}
+
 // Column sums of the workgroups' rows in two small steps, so that the first has enough
 // workgroups to pull the few megabytes of `partial` at speed: the rows are cut into kFoldGroups
 // groups; workgroup (x, g) adds the rows of group g for 64 of the 2 ncols columns (its four
@@ -647,13 +769,16 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_fold1(const float* __res
     level2[(int64_t)blockIdx.y * width + col] = (lds[0][lane] + lds[1][lane]) + (lds[2][lane] + lds[3][lane]);
 }
 
-__global__ __launch_bounds__(kWave) void layernorm_bwd_fold2(const double* __restrict__ level2, int64_t ncols,
+// `groups` rows (at most kFoldGroups) of 2 ncols sums each: binary64 ones from the first step, or
+// the kernels' own binary32 rows when there are few enough of them to skip that step.
+template <typename T>
+__global__ __launch_bounds__(kWave) void layernorm_bwd_fold2(const T* __restrict__ level2, int groups, int64_t ncols,
                                                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
   const int64_t col = (int64_t)blockIdx.x * kWave + threadIdx.x;
   if (col >= 2 * ncols) return;
   double t[kFoldGroups];
 #pragma unroll
-  for (int g = 0; g < kFoldGroups; g++) t[g] = level2[(int64_t)g * 2 * ncols + col];
+  for (int g = 0; g < kFoldGroups; g++) t[g] = g < groups ? (double)level2[(int64_t)g * 2 * ncols + col] : 0.0;
   double acc = 0.0;
 #pragma unroll
   for (int g = 0; g < kFoldGroups; g++) acc += t[g];
@@ -854,10 +979,8 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // guarded seven-group tile and at 3.9 TB/s on the guarded eight-group one ((32768, 1600))
   if (nv == 7 && cols != 7 * kWave * 4) nv = 8;
   const bool wide = nv == 0 || nv > 8;  // more than 2048 columns: a workgroup per row
-  if (wide && (cols > 8192 || cols % 4 != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(gamma)))
-    return fail(WF2HIP_EUNSUPPORTED,
-                "LayerNorm backward: rows longer than 2048 need a multiple of 4 up to 8192 columns and 16-byte aligned "
-                "tensors (compose it from nodes)");
+  const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
+  const bool in_pieces = wide && (cols > 8192 || !vec);
   const int64_t total = (int64_t)rows * cols;
   if ((x < dx + total && dx < x + total) || (dgamma < dbeta + cols && dbeta < dgamma + cols))
     return fail(WF2HIP_EOVERLAP, "LayerNorm backward: dx overlaps x, or dgamma overlaps dbeta");
@@ -867,19 +990,58 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // the HBM peak (both small folds included), 66 % with one workgroup per unit, 65 - 67 % with
   // three to eight (more rows of `partial` to write and fold)
   const bool tiny = cols <= kTinyCols && rows >= 16384;
-  const int64_t blocks = wide ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
+  const int64_t pieces = ceil_div((int64_t)cols, kPieceCols);
+  if (in_pieces && (rows * pieces >= ((int64_t)1 << 31) || pieces >= ((int64_t)1 << 31)))
+    return fail(WF2HIP_EUNSUPPORTED, "too many row pieces for one launch");
+  // in pieces: enough row groups for two workgroups of 512 threads per compute unit
+  const int64_t quarters = ceil_div((int64_t)cols, kApplyCols);
+  const int64_t blocks = in_pieces ? std::min<int64_t>({(int64_t)rows, ceil_div(2 * (int64_t)std::max(rt().num_cus, 1), quarters), 65535})
+                         : wide  ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
                          : tiny ? std::min<int64_t>(ceil_div((int64_t)rows, (int64_t)(cols <= 32 ? 128 : 64)),
                                                     4 * (int64_t)std::max(rt().num_cus, 1))
                               : std::min<int64_t>(ceil_div(rows, kWavesPerBlock), 2 * (int64_t)std::max(rt().num_cus, 1));
-  const size_t partial_bytes = (size_t)blocks * 2 * cols * sizeof(float);
-  const size_t level2_bytes = (size_t)kFoldGroups * 2 * cols * sizeof(double);
+  // few enough rows of column sums go to the last fold as they are; one row is the result itself
+  const bool direct = in_pieces && blocks == 1;
+  const bool two_folds = blocks > kFoldGroups;
+  const size_t partial_bytes = direct ? 0 : (size_t)blocks * 2 * cols * sizeof(float);
+  const size_t level2_bytes = two_folds ? (size_t)kFoldGroups * 2 * cols * sizeof(double) : 0;
   void* partial = nullptr;
-  WF2_TRY(wf2hip_malloc_uninitialized(&partial, partial_bytes + level2_bytes));  // partial_bytes is a multiple of 8
+  if (!direct) WF2_TRY(wf2hip_malloc_uninitialized(&partial, partial_bytes + level2_bytes));  // partial_bytes is a multiple of 8
   double* level2 = reinterpret_cast<double*>(static_cast<char*>(partial) + partial_bytes);
-  const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
   const bool streaming = total * 12 >= ((int64_t)192 << 20);
   int rc;
-  if (tiny) {
+  if (in_pieces) {
+    hipStream_t st = rt().stream;
+    void* stats = nullptr;  // four binary64 values per (row, piece)
+    const size_t np = (size_t)(rows * pieces);
+    rc = wf2hip_malloc_uninitialized(&stats, np * 4 * sizeof(double));
+    if (rc != 0) {
+      if (partial) (void)wf2hip_free(partial);
+      return rc;
+    }
+    double* psum = static_cast<double*>(stats);
+    double *pdev = psum + np, *pd = psum + 2 * np, *pc = psum + 3 * np;
+    float* out_g = direct ? dgamma : static_cast<float*>(partial);
+    float* out_b = direct ? dbeta : static_cast<float*>(partial) + cols;
+    const uint32_t grid = (uint32_t)np;
+    const dim3 grid2((uint32_t)quarters, (uint32_t)blocks);
+    if (vec)
+      layernorm_bwd_piece_sums<true><<<grid, kPieceBlock, 0, st>>>(x, gamma, dy, cols, (uint32_t)pieces, psum, pdev, pd, pc);
+    else
+      layernorm_bwd_piece_sums<false><<<grid, kPieceBlock, 0, st>>>(x, gamma, dy, cols, (uint32_t)pieces, psum, pdev, pd, pc);
+    rc = after_launch("layernorm_bwd_piece_sums");
+    if (rc == 0) {
+      if (vec)
+        layernorm_bwd_piece_apply<true><<<grid2, kApplyBlock, 0, st>>>(x, gamma, dy, eps, dx, out_g, out_b, rows, cols,
+                                                                      (uint32_t)pieces, psum, pdev, pd, pc);
+      else
+        layernorm_bwd_piece_apply<false><<<grid2, kApplyBlock, 0, st>>>(x, gamma, dy, eps, dx, out_g, out_b, rows, cols,
+                                                                       (uint32_t)pieces, psum, pdev, pd, pc);
+      rc = after_launch("layernorm_bwd_piece_apply");
+    }
+    (void)wf2hip_free(stats);  // stream order keeps it alive for the launches above
+    if (direct) return rc;
+  } else if (tiny) {
     layernorm_bwd_tiny<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(x, gamma, dy, eps, dx, (float*)partial, rows, (int)cols,
                                                                      make_fastdiv((uint32_t)cols));
     rc = after_launch("layernorm_bwd_tiny");
@@ -908,15 +1070,18 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
     rc = launch_layernorm_bwd<true, false>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
   else
     rc = launch_layernorm_bwd<false, false>(nv, (uint32_t)blocks, x, gamma, dy, eps, dx, (float*)partial, rows, cols);
-  if (rc == 0) {
+  if (rc == 0 && two_folds) {
     const uint32_t strips = (uint32_t)ceil_div(2 * (int64_t)cols, kWave);
     layernorm_bwd_fold1<<<dim3(strips, kFoldGroups), kBlock, 0, rt().stream>>>((const float*)partial, blocks,
                                                                               2 * (int64_t)cols, level2);
     rc = after_launch("layernorm_bwd_fold1");
   }
   if (rc == 0) {
-    layernorm_bwd_fold2<<<(uint32_t)ceil_div(2 * (int64_t)cols, kWave), kWave, 0, rt().stream>>>(level2, cols, dgamma,
-                                                                                               dbeta);
+    const uint32_t grid = (uint32_t)ceil_div(2 * (int64_t)cols, kWave);
+    if (two_folds)
+      layernorm_bwd_fold2<double><<<grid, kWave, 0, rt().stream>>>(level2, kFoldGroups, cols, dgamma, dbeta);
+    else
+      layernorm_bwd_fold2<float><<<grid, kWave, 0, rt().stream>>>((const float*)partial, (int)blocks, cols, dgamma, dbeta);
     rc = after_launch("layernorm_bwd_fold2");
   }
   (void)wf2hip_free(partial);  // stream order keeps it alive for the launches above

@@ -1360,6 +1360,89 @@ __global__ __launch_bounds__(kBlock) void layernorm_rows_block(const float* __re
     outr[c] = (float)(((double)xr[c] - mean) * rstd * (double)gamma[c] + (double)beta[c]);
 }
 
+// Rows of 8196 ... 65536 columns (multiples of 4), at least one per compute unit: a workgroup of 1024
+// threads per row, thread t holding the E / 4 16-byte vectors (g 1024 + t) 4 of the row in registers --
+// one read and one write.  The arithmetic of layernorm_rows_wide.
+template <int E, bool NT>
+__global__ __launch_bounds__(kPieceBlock) void layernorm_rows_long(const float* __restrict__ x,
+                                                                  const float* __restrict__ gamma,
+                                                                  const float* __restrict__ beta, float eps,
+                                                                  float* __restrict__ out, int64_t ncols) {
+  __shared__ double lds[2 * kPieceBlock / kWave];
+  const int64_t base = (int64_t)blockIdx.x * ncols;
+  f4 v[E / 4];
+  bool in[E / 4];
+#pragma unroll
+  for (int g = 0; g < E / 4; g++) {
+    const int64_t c = ((int64_t)g * kPieceBlock + threadIdx.x) * 4;
+    in[g] = c < ncols;
+    v[g] = f4{0.f, 0.f, 0.f, 0.f};
+    if (in[g]) {
+      const f4* q = reinterpret_cast<const f4*>(x + base + c);
+      v[g] = NT ? __builtin_nontemporal_load(q) : *q;
+    }
+  }
+  double sum = 0.0, unused;
+#pragma unroll
+  for (int g = 0; g < E / 4; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) sum += (double)v[g][c];
+  const float mean = (float)(piece_sum2(sum, 0.0, lds, &unused) / (double)ncols);
+  float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int g = 0; g < E / 4; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const float d = in[g] ? v[g][c] - mean : 0.0f;
+      v[g][c] = d;
+      sq[c] = __builtin_fmaf(d, d, sq[c]);
+    }
+  const double var =
+      piece_sum2(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3]), 0.0, lds, &unused) / (double)ncols;
+  const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
+#pragma unroll
+  for (int g = 0; g < E / 4; g++) {
+    if (!in[g]) continue;
+    const int64_t c = ((int64_t)g * kPieceBlock + threadIdx.x) * 4;
+    const f4 gm = *reinterpret_cast<const f4*>(gamma + c);
+    const f4 bt = *reinterpret_cast<const f4*>(beta + c);
+    f4 r;
+#pragma unroll
+    for (int k = 0; k < 4; k++) r[k] = __builtin_fmaf(v[g][k] * rstd, gm[k], bt[k]);
+    f4* q = reinterpret_cast<f4*>(out + base + c);
+    if (NT)
+      __builtin_nontemporal_store(r, q);
+    else
+      *q = r;
+  }
+}
+
+// Rows beyond 8192 columns: the row in pieces of 16384 columns (layernorm_piece_stats), then every
+// piece folds its row's statistics and writes its share of the output: two reads and a write of the
+// row, on as many workgroups as there are pieces ((1, 16777216) on 1024 of them where the three-pass
+// kernel above has one).
+template <bool VEC>
+__global__ __launch_bounds__(kPieceBlock) void layernorm_piece_apply(const float* __restrict__ x,
+                                                                    const float* __restrict__ gamma,
+                                                                    const float* __restrict__ beta, float eps,
+                                                                    float* __restrict__ out, int64_t ncols,
+                                                                    uint32_t pieces, const double* __restrict__ psum,
+                                                                    const double* __restrict__ pdev) {
+  __shared__ double lds[2 * kPieceBlock / kWave];
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const int64_t c0 = (int64_t)piece * kPieceCols;
+  const int64_t left = ncols - c0;
+  PieceRegs<VEC> r, g, b;
+  r.load(x + (int64_t)row * ncols + c0, left, 0.0f);
+  g.load(gamma + c0, left, 0.0f);
+  b.load(beta + c0, left, 0.0f);
+  float mean, rstd;
+  piece_row_stats(psum + (int64_t)row * pieces, pdev + (int64_t)row * pieces, pieces, ncols, eps, lds, &mean, &rstd);
+#pragma unroll
+  for (int k = 0; k < kPieceE; k++) r.v[k] = __builtin_fmaf((r.v[k] - mean) * rstd, g.v[k], b.v[k]);
+  r.store(out + (int64_t)row * ncols + c0, left);
+}
+
 // Rows of 2049 ... 8192 columns that are a multiple of 4: a workgroup per row with the row in
 // registers (thread t holds the NG 16-byte vectors (g 256 + t) 4 ...), one read and one write
 // where the three-pass form above reads the row three times ((8192, 4096): 82 us).  The
@@ -1912,6 +1995,50 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
       }
 #undef WF2_WIDE
       return after_launch("layernorm_rows_wide");
+    }
+    const bool aligned = cols % 4 == 0 && aligned16(x) && aligned16(out) && aligned16(gamma) && aligned16(beta);
+    if (cols > 8192 && cols <= 64 * (int64_t)kPieceBlock && aligned && rows >= rt().num_cus) {
+      const bool nt = (int64_t)rows * cols * 8 >= ((int64_t)192 << 20);
+#define WF2_LONG(E_)                                                                                       \
+  if (nt)                                                                                                  \
+    layernorm_rows_long<E_, true><<<(uint32_t)rows, kPieceBlock, 0, st>>>(x, gamma, beta, eps, out, cols); \
+  else                                                                                                     \
+    layernorm_rows_long<E_, false><<<(uint32_t)rows, kPieceBlock, 0, st>>>(x, gamma, beta, eps, out, cols);
+      if (cols <= 16 * (int64_t)kPieceBlock) {
+        WF2_LONG(16)
+      } else if (cols <= 32 * (int64_t)kPieceBlock) {
+        WF2_LONG(32)
+      } else if (cols <= 48 * (int64_t)kPieceBlock) {
+        WF2_LONG(48)
+      } else {
+        WF2_LONG(64)
+      }
+#undef WF2_LONG
+      return after_launch("layernorm_rows_long");
+    }
+    if (cols > 8192) {
+      const int64_t pieces = ceil_div((int64_t)cols, kPieceCols);
+      if (rows * pieces >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many row pieces for one launch");
+      void* stats = nullptr;  // rows x pieces sums, then as many sums of squared deviations
+      WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(rows * pieces) * 2 * sizeof(double)));
+      double* psum = static_cast<double*>(stats);
+      double* pdev = psum + rows * pieces;
+      const uint32_t grid = (uint32_t)(rows * pieces);
+      const bool vec = aligned;
+      if (vec)
+        layernorm_piece_stats<true><<<grid, kPieceBlock, 0, st>>>(x, cols, (uint32_t)pieces, psum, pdev);
+      else
+        layernorm_piece_stats<false><<<grid, kPieceBlock, 0, st>>>(x, cols, (uint32_t)pieces, psum, pdev);
+      int rc = after_launch("layernorm_piece_stats");
+      if (rc == 0) {
+        if (vec)
+          layernorm_piece_apply<true><<<grid, kPieceBlock, 0, st>>>(x, gamma, beta, eps, out, cols, (uint32_t)pieces, psum, pdev);
+        else
+          layernorm_piece_apply<false><<<grid, kPieceBlock, 0, st>>>(x, gamma, beta, eps, out, cols, (uint32_t)pieces, psum, pdev);
+        rc = after_launch("layernorm_piece_apply");
+      }
+      (void)wf2hip_free(stats);  // stream order keeps it alive for the launches above
+      return rc;
     }
     layernorm_rows_block<<<(uint32_t)rows, kBlock, 0, st>>>(x, gamma, beta, eps, out, cols);
     return after_launch("layernorm_rows_block");

@@ -720,10 +720,10 @@ def layer_norm_fused(x: HIPTensor, g: HIPTensor, b: HIPTensor, eps: float = 1.0e
 
 def layer_norm_backward(x: HIPTensor, g: HIPTensor, dout: HIPTensor, eps: float = 1.0e-5):
     """(dx, dgamma, dbeta) of LayerNorm over the last axis from the saved input: one row kernel and a
-    small fold (HIP-LayerNorm-Node-backward) for rows up to 8192 wide (a multiple of 4 beyond 2048), the node
-    composition otherwise."""
+    small fold (HIP-LayerNorm-Node-backward); rows beyond 8192 columns in pieces over several workgroups.
+    The node composition for the other element types."""
     cols = x.shape[-1]
-    if x.dtype != "float" or not (cols <= 2048 or (cols <= 8192 and cols % 4 == 0)):
+    if x.dtype != "float":
         return layer_norm_backward_composed(x, g, dout, eps)
     x2, d2 = to_contiguous(x), to_contiguous(dout)
     dx = HIPTensor(list(x.shape), initial_element=None)

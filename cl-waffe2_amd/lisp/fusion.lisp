@@ -321,13 +321,9 @@ Composed from ! functions (!mean and !sum are one node each on the device)."
          (db   (!sum-hip dout :axis 0)))
     (values dx dg db)))
 
-(defun layer-norm-kernel-width-p (cols)
-  "Row widths wf2hip_layernorm_backward_f32 takes: up to 2048, or a multiple of 4 up to 8192."
-  (or (<= cols 2048) (and (<= cols 8192) (zerop (mod cols 4)))))
-
 (defun layer-norm-gradients-fused (x g dout eps)
   "The same three gradients from one row kernel and two small folds (wf2hip_layernorm_backward_f32;
-rows up to 8192 wide, a multiple of 4 beyond 2048)."
+rows beyond 8192 columns in pieces over several workgroups)."
   (ensure-extension)
   (let* ((dout (eager-contiguous dout))
          (rows (first (shape x)))
@@ -346,8 +342,9 @@ rows up to 8192 wide, a multiple of 4 beyond 2048)."
             :save-for-backward-names (x g)
             :where (X[rows cols] G[cols] B[cols] OUT[rows cols] -> OUT[rows cols])
             :documentation "OUT <- (x - mean) / sqrt(var + eps) * g + b per row, one kernel
-(wf2hip_layernorm_rows_f32).  Backward: the three gradients from the saved input, one kernel for
-rows up to 8192 wide (layer-norm-gradients-fused), composed beyond (layer-norm-gradients)."
+(wf2hip_layernorm_rows_f32).  Backward: the three gradients from the saved input by
+wf2hip_layernorm_backward_f32 (layer-norm-gradients-fused), or composed from nodes
+(layer-norm-gradients) under *compose-backward*."
             :forward ((self x g b out)
                       (ensure-extension)
                       (check (wf2hip-layernorm-rows-f32 (first (shape x)) (second (shape x))
@@ -358,7 +355,7 @@ rows up to 8192 wide (layer-norm-gradients-fused), composed beyond (layer-norm-g
                       (with-setting-save4bw ((x x) (g g)) out))
             :backward ((self dout)
                        (with-reading-save4bw ((x x) (g g))
-                         (if (or *compose-backward* (not (layer-norm-kernel-width-p (second (shape x)))))
+                         (if *compose-backward*
                              (multiple-value-bind (dx dg db) (layer-norm-gradients x g dout (layernorm-eps self))
                                (values (proceed dx)
                                        (proceed (!reshape dg (second (shape x))))

@@ -555,7 +555,7 @@ def _causal_softmax_backward_node(y: HIPTensor, dout: HIPTensor, dx: HIPTensor, 
 @define_impl("HIP-LayerNorm-Node-backward", HIPTensor, _only_float)
 def _layernorm_backward_node(x: HIPTensor, g: HIPTensor, dout: HIPTensor, dx: HIPTensor, dg: HIPTensor,
                              db: HIPTensor, eps: float = 1.0e-5) -> HIPTensor:
-    """``X[rows cols] G[cols] DOUT[rows cols] DX[rows cols] DG[cols] DB[cols] -> DX DG DB`` (rows up to 8192 wide; a multiple of 4 beyond 2048)."""
+    """``X[rows cols] G[cols] DOUT[rows cols] DX[rows cols] DG[cols] DB[cols] -> DX DG DB``."""
     cols = x.shape[-1]
     name = "HIP-LayerNorm-Node-backward"
     _require_rows(f"{name}: x", x)

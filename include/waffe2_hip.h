@@ -610,7 +610,9 @@ int wf2hip_softmax_rows_f32(long rows, long cols, const float* x, long ldx,
 int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
                               float scale);
 /* LayerNorm over the last axis: out = (x - mean)/sqrt(var + eps) * g + b
- * (source/nn/norms.lisp:44-82; examples/gpt-2/utils.lisp:114-127). */
+ * (source/nn/norms.lisp:44-82; examples/gpt-2/utils.lisp:114-127).  Rows beyond
+ * 8192 columns run in pieces of 16384 columns over several workgroups: two
+ * launches and 16 bytes per piece of scratch from the library's pool. */
 int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
                               const float* beta, float eps, float* out);
 /* Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126) over the last axis
@@ -653,10 +655,12 @@ int wf2hip_softmax_cross_entropy_backward_f32(long n, const float* dy, int dy_is
  * xh = (x - mean) rstd and dyh = dy gamma,
  *   dx = rstd (dyh - mean(dyh) - xh mean(dyh xh)),
  *   dgamma[c] = sum over rows of dy xh,  dbeta[c] = sum over rows of dy.
- * Contiguous (rows, cols) operands, cols <= 8192; beyond 2048 columns cols must
- * be a multiple of 4 and the tensors 16-byte aligned (otherwise, and for longer
- * rows, WF2HIP_EUNSUPPORTED: compose them from nodes).  dx may be dy.  Allocates
- * 8 * cols bytes per workgroup of scratch from the library's pool. */
+ * Contiguous (rows, cols) operands of any width: up to 8192 columns one row
+ * kernel and two small folds; beyond that (and beyond 2048 columns that are no
+ * multiple of 4 or lie off a 16-byte boundary) the row in pieces of 16384
+ * columns over several workgroups, three row kernels.  dx may be dy.  Allocates
+ * 8 * cols bytes per workgroup of scratch from the library's pool (and 32 bytes
+ * per piece for rows in pieces). */
 int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, const float* gamma,
                                   const float* dy, float eps, float* dx, float* dgamma,
                                   float* dbeta);

@@ -142,27 +142,46 @@ def test_layernorm_backward(gpu, rows, cols):
         assert np.max(np.abs(cg.numpy() - gg.numpy()) / (mag_g + 1e-30)) <= 5e-6
 
 
-@pytest.mark.parametrize("cols", [8196, 4098])
-def test_layernorm_backward_rows_the_kernels_leave_to_the_composition(gpu, cols):
-    """More than 8192 columns, or more than 2048 that are not a multiple of 4."""
+@pytest.mark.parametrize("rows,cols,shift", [(6, 8196, 0), (6, 4098, 0), (3, 16384, 0), (2, 40001, 0), (1, 262144 + 8, 0),
+                                             (700, 8200, 0), (1100, 2050, 0), (5, 32768, 1), (4, 3072, 3)])
+def test_layernorm_backward_in_pieces(gpu, rows, cols, shift):
+    """More than 8192 columns, or more than 2048 that cannot be read with 16-byte loads (a column count that is no
+    multiple of 4, or tensors `shift` elements off a 16-byte boundary): the row in pieces of 16384 columns over several
+    workgroups, through the C ABI, against binary64 and against the node composition."""
     from oracle import gpt2_block_ref as ref
+    import ctypes as C
     W = gpu
     F = W.functional
-    rng = np.random.default_rng(5)
-    rows = 6
-    x = rng.standard_normal((rows, cols)).astype(f32)
+    rng = np.random.default_rng(rows + 7 * cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(f32)
     g = (1 + 0.1 * rng.standard_normal(cols)).astype(f32)
     dy = rng.standard_normal((rows, cols)).astype(f32)
     lib = W.lib.get()
-    import ctypes as C
-    p = lambda t: C.c_void_p(t.ptr)  # noqa: E731
-    tx, tg, td = F.from_numpy(x), F.from_numpy(g), F.from_numpy(dy)
-    ox, og, ob = W.HIPTensor([rows, cols]), W.HIPTensor([cols]), W.HIPTensor([cols])
-    rc = lib.wf2hip_layernorm_backward_f32(rows, cols, p(tx), p(tg), p(td), 1e-5, p(ox), p(og), p(ob))
-    assert rc == W.lib.EUNSUPPORTED
+    total = rows * cols
+    hold = [F.from_numpy(np.concatenate([np.zeros(shift, f32), a.ravel()])) for a in (x, g, dy)]
+    outs = [W.HIPTensor([n + shift]) for n in (total, cols, cols)]
+    p = lambda t: C.c_void_p(t.ptr + 4 * shift)  # noqa: E731
+    rc = lib.wf2hip_layernorm_backward_f32(rows, cols, p(hold[0]), p(hold[1]), p(hold[2]), 1e-5, p(outs[0]), p(outs[1]),
+                                           p(outs[2]))
+    assert rc == 0
+    gx = outs[0].numpy()[shift:].reshape(rows, cols)
+    gg, gb = outs[1].numpy()[shift:], outs[2].numpy()[shift:]
     dx, dg, db, mag, mag_g = ref.layer_norm_backward(x.astype(np.float64), g.astype(np.float64), dy.astype(np.float64), 1e-5)
-    gx, gg, gb = F.layer_norm_backward(tx, tg, td, 1e-5)
-    assert np.max(np.abs(gx.numpy() - dx) / mag) <= 5e-6 and np.max(np.abs(gg.numpy() - dg) / mag_g) <= 5e-6
+    assert np.max(np.abs(gx - dx) / mag) <= 3e-6
+    # xhat comes from x - (float)mean: where x is close to the mean the rounding of the mean (6e-8 |mean| rstd, about
+    # 1.5e-8 here) is large against |xhat| itself, and with a row or two nothing averages it out
+    assert np.max(np.abs(gg - dg) / (mag_g + 0.03 * np.abs(dy).sum(0) + 1e-30)) <= 3e-6
+    assert np.max(np.abs(gb - db) / (np.abs(dy).sum(0) + 1e-30)) <= 1e-6
+    if total <= 1 << 20:
+        cx, cg, cb = F.layer_norm_backward_composed(F.from_numpy(x), F.from_numpy(g), F.from_numpy(dy), 1e-5)
+        assert np.max(np.abs(cx.numpy() - gx) / mag) <= 5e-6
+        assert np.max(np.abs(cg.numpy() - gg) / (mag_g + 0.03 * np.abs(dy).sum(0) + 1e-30)) <= 5e-6
+    # dx may be dy
+    rc = lib.wf2hip_layernorm_backward_f32(rows, cols, p(hold[0]), p(hold[1]), p(hold[2]), 1e-5, p(hold[2]), p(outs[1]),
+                                           p(outs[2]))
+    assert rc == 0
+    assert np.array_equal(hold[2].numpy()[shift:].reshape(rows, cols), gx)
+    assert np.array_equal(outs[1].numpy()[shift:], gg)
 
 
 def test_backward_entries_on_empty_operands(gpu):

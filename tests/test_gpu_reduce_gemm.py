@@ -349,10 +349,12 @@ def test_layernorm(gpu):
     W = gpu
     F = W.functional
     rng = np.random.default_rng(7)
-    # 2052 ... 8192 (multiples of 4): a workgroup per row holding it in registers; 4101, 8196, 20000: three passes
+    # 2052 ... 8192 (multiples of 4): a workgroup per row holding it in registers; 4101: three passes;
+    # beyond 8192: the row in pieces of 16384 columns over several workgroups
     for rows, cols in [(64, 768), (10, 100), (5, 1), (33, 2048), (7, 255), (9, 3072), (3, 4101), (2, 20000),
                        (1001, 1024), (513, 1000), (300, 1536), (5, 2052), (300, 4096), (7, 5120), (40, 6148),
-                       (129, 8192), (3, 8196)]:
+                       (129, 8192), (3, 8196), (700, 8200), (5, 16384), (3, 16388), (2, 40001), (1, (1 << 20) + 4),
+                       (40, 32768)]:
         X = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
         g = rng.standard_normal(cols).astype(np.float32)
         b = rng.standard_normal(cols).astype(np.float32)
