@@ -24,8 +24,9 @@
 // the reference's vector body does.
 //
 // These are bandwidth kernels like their :float counterparts: 16-byte vectors
-// when both runs are contiguous (or y is one value), one element per lane with
-// four in flight otherwise.  A destination with incx = 0 accumulates in the
+// when both runs are contiguous (or y is one value) and on the rows of sliced
+// views of the 8- and 16-bit types, tiles through LDS for transposing passes,
+// one element per lane with four in flight otherwise.  A destination with incx = 0 accumulates in the
 // reference's order on one lane.
 #include <math.h>
 
@@ -445,9 +446,129 @@ static bool try_typed_tile(const Space& s, T* a, const T* b, int* rc) {
   return true;
 }
 
+// Sliced views of the 8- and 16-bit types: both sides have stride 1 along the last axis, rows of `len`
+// elements at any pitch and any (element-aligned) start.  An element per lane moves 64 or 128 bytes per
+// wavefront and access; here a lane takes 16 bytes of the destination row: `lanes` (a power of two up to
+// 256) lanes share a row, the elements before the row's first 16-byte boundary and after its last one
+// go one to a lane, the vectors between them are read and written whole.  The source row starts wherever
+// it starts: its vectors are read at element alignment, which the hardware serves.
+struct TypedRows {
+  int64_t len, nrows;
+  uint32_t lane_shift;  // log2(lanes)
+  int32_t nouter;
+  uint32_t oshape[WF2HIP_MAX_RANK];  // innermost outer axis first
+  int64_t odst[WF2HIP_MAX_RANK], osrc[WF2HIP_MAX_RANK];
+};
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void typed_rows(T* dst, const T* src, TypedRows p) {
+  constexpr int N = 16 / (int)sizeof(T);
+  constexpr int U = 2;
+  using P = Pack<T, N>;
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const uint32_t lanes = 1u << p.lane_shift;
+  const uint32_t sub = threadIdx.x & (lanes - 1);
+  const int64_t row = (int64_t)blockIdx.x * (kBlock >> p.lane_shift) + (threadIdx.x >> p.lane_shift);
+  if (row >= p.nrows) return;
+  int64_t doff = 0, soff = 0;
+  {
+    uint64_t rem = (uint64_t)row;
+    for (int i = 0; i < p.nouter; i++) {
+      const uint64_t q = rem / p.oshape[i];
+      const int64_t idx = (int64_t)(rem - q * p.oshape[i]);
+      rem = q;
+      doff += idx * p.odst[i];
+      soff += idx * p.osrc[i];
+    }
+  }
+  T* d = dst + doff;
+  const T* s = src + soff;
+  int64_t head = (int64_t)((16 - ((uintptr_t)d & 15)) & 15) / (int64_t)sizeof(T);
+  if (head > p.len) head = p.len;
+  const int64_t nvec = (p.len - head) / N;
+  const int64_t tail0 = head + nvec * N;
+  if (blockIdx.y == 0) {
+    // at most N - 1 elements on either side of the vectors
+    const int64_t loose = head + (p.len - tail0);
+    for (int64_t e = sub; e < loose; e += lanes) {
+      const int64_t i = e < head ? e : tail0 + (e - head);
+      const T yv = s[i];
+      d[i] = apply<T, OP>(OP != WF2HIP_MOVE ? d[i] : yv, yv);
+    }
+  }
+  const int64_t step = (int64_t)lanes * gridDim.y;
+  for (int64_t v0 = (int64_t)blockIdx.y * lanes + sub; v0 < nvec; v0 += step * U) {
+    u4 a[U], b[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t v = v0 + u * step;
+      if (v < nvec) {
+        if (OP != WF2HIP_MOVE) a[u] = *reinterpret_cast<const u4*>(d + head + v * N);
+        __builtin_memcpy(&b[u], s + head + v * N, 16);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t v = v0 + u * step;
+      if (v < nvec) {
+        u4 r;
+        if constexpr (OP == WF2HIP_MOVE) {
+          r = b[u];
+        } else if constexpr (kWordOp<T, OP>) {
+#pragma unroll
+          for (int k = 0; k < 4; k++) r[k] = apply_word<(int)sizeof(T), OP>(a[u][k], b[u][k]);
+        } else {
+          const P pa = __builtin_bit_cast(P, a[u]), pb = __builtin_bit_cast(P, b[u]);
+          P pr;
+#pragma unroll
+          for (int k = 0; k < N; k++) pr.v[k] = apply<T, OP>(pa.v[k], pb.v[k]);
+          r = __builtin_bit_cast(u4, pr);
+        }
+        *reinterpret_cast<u4*>(d + head + v * N) = r;
+      }
+    }
+  }
+}
+
+template <class T, int OP>
+static bool try_typed_rows(const Space& s, T* a, const T* b, int* rc) {
+  const int last = s.rank - 1;
+  if (sizeof(T) > 2 || s.rank < 2 || s.sa[last] != 1 || s.sb[last] != 1) return false;
+  constexpr int N = 16 / (int)sizeof(T);
+  const int64_t len = s.shape[last];
+  if (len < 4 * N) return false;  // rows under 64 bytes: mostly loose elements
+  TypedRows p;
+  p.len = len;
+  p.nrows = s.total / len;
+  p.nouter = 0;
+  for (int r = last - 1; r >= 0; r--) {
+    if (s.shape[r] >= ((int64_t)1 << 32)) return false;
+    p.oshape[p.nouter] = (uint32_t)s.shape[r];
+    p.odst[p.nouter] = s.sa[r];
+    p.osrc[p.nouter] = s.sb[r];
+    p.nouter++;
+  }
+  const int64_t vecs = ceil_div(len, (int64_t)N);
+  p.lane_shift = 0;
+  while (p.lane_shift < 8 && ((int64_t)1 << p.lane_shift) < vecs) p.lane_shift++;
+  const int64_t lanes = (int64_t)1 << p.lane_shift;
+  const int64_t gx = ceil_div(p.nrows, (int64_t)kBlock / lanes);
+  if (gx >= ((int64_t)1 << 31)) return false;
+  // along a long row: workgroups of two vectors per lane, as many as fill the device with few rows
+  int64_t gy = ceil_div(vecs, lanes * 2);
+  const int64_t fill = ceil_div((int64_t)rt().num_cus * 16, gx);
+  if (gy > fill) gy = fill;
+  if (gy > 65535) gy = 65535;
+  if (gy < 1) gy = 1;
+  typed_rows<T, OP><<<dim3((uint32_t)gx, (uint32_t)gy), kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
+  *rc = after_launch("typed_rows");
+  return true;
+}
+
 template <class T, int OP>
 static int run_generic(const Space& s, T* a, const T* b) {
   int rc = 0;
+  if (try_typed_rows<T, OP>(s, a, b, &rc)) return rc;
   if (try_typed_tile<T, OP>(s, a, b, &rc)) return rc;
   TypedGen p;
   p.rank = s.rank;

@@ -286,3 +286,64 @@ def test_typed_random_permuted_passes(gpu, dtype, seed):
         want2 = y - want[index].transpose(perm)
     F.sub_(dy, dv.permute(*perm))
     np.testing.assert_array_equal(dy.numpy(), want2, err_msg="subtract a permuted window, " + what)
+
+
+@pytest.mark.parametrize("dtype", ["int16", "uint16", "int8", "uint8"])
+@pytest.mark.parametrize("seed", range(5))
+def test_sliced_rows_of_the_narrow_types(gpu, dtype, seed):
+    """Windows with stride 1 along the last axis (a slice of every row, of several leading axes, a row broadcast
+    as the other operand): rows of 64 bytes and more run 16 bytes per lane, whatever byte the rows of either
+    side start on -- every start and length modulo 16 appears; bit-exact against numpy (sums wrap, quotients
+    truncate, as in the reference's loops, cl-waffe2-simd.c:252-288)."""
+    F = gpu.functional
+    npt = {"int16": np.int16, "uint16": np.uint16, "int8": np.int8, "uint8": np.uint8}[dtype]
+    rng = np.random.default_rng(1000 * seed + len(dtype) + npt().itemsize)
+    info = np.iinfo(npt)
+
+    def draw(sh, nonzero=False):
+        if nonzero:
+            return rng.integers(1, 12, sh).astype(npt)
+        return rng.integers(info.min, int(info.max) + 1, sh).astype(npt)
+
+    for case in range(6):
+        rank = int(rng.integers(2, 5))
+        width = int(rng.choice([70, 129, 300, 1024, 4099, 70000 if rank == 2 else 513]))
+        shape = [int(rng.integers(2, 7)) for _ in range(rank - 1)] + [width]
+        lo = int(rng.integers(0, 19))
+        hi = width - int(rng.integers(0, 19))
+        lead_lo = int(rng.integers(0, 2))
+        x, y = draw(shape), draw(shape)
+        dx, dy = F.from_numpy(x, dtype=dtype), F.from_numpy(y, dtype=dtype)
+        lo_y = int(rng.integers(0, 19))  # the other side starts on another byte
+        lo_y = min(lo_y, width - (hi - lo))
+        subs_x = [(lead_lo, shape[0])] + [True] * (rank - 2) + [(lo, hi)]
+        subs_y = [(lead_lo, shape[0])] + [True] * (rank - 2) + [(lo_y, lo_y + hi - lo)]
+        ix = (slice(lead_lo, None),) + (slice(None),) * (rank - 2) + (slice(lo, hi),)
+        iy = (slice(lead_lo, None),) + (slice(None),) * (rank - 2) + (slice(lo_y, lo_y + hi - lo),)
+        what = f"{dtype} {shape} x[{lo}:{hi}] y[{lo_y}:] lead {lead_lo}"
+        with np.errstate(over="ignore"):
+            want = x.copy()
+            want[ix] = x[ix] + y[iy]
+            F.add_(dx.view(*subs_x), dy.view(*subs_y))
+            np.testing.assert_array_equal(dx.numpy(), want, err_msg="add " + what)
+            want[ix] = want[ix] * y[iy]
+            F.mul_(dx.view(*subs_x), dy.view(*subs_y))
+            np.testing.assert_array_equal(dx.numpy(), want, err_msg="mul " + what)
+            want2 = y.copy()
+            want2[iy] = y[iy] - want[ix]
+            F.sub_(dy.view(*subs_y), dx.view(*subs_x))
+            np.testing.assert_array_equal(dy.numpy(), want2, err_msg="sub " + what)
+        d = draw(shape, nonzero=True)
+        dd = F.from_numpy(d, dtype=dtype)
+        F.div_(dx.view(*subs_x), dd.view(*subs_y))
+        want[ix] = np.trunc(want[ix].astype(np.float64) / d[iy]).astype(npt)
+        np.testing.assert_array_equal(dx.numpy(), want, err_msg="div " + what)
+        # a copy out of the window, and one row added to every row of it
+        np.testing.assert_array_equal(F.copy(dx.view(*subs_x)).numpy(), want[ix], err_msg="copy " + what)
+        row = draw((hi - lo,))
+        bview = F.from_numpy(row.reshape((1,) * (rank - 1) + (-1,)), dtype=dtype).view(
+            *([(":broadcast", shape[0] - lead_lo)] + [(":broadcast", n) for n in shape[1:-1]] + [True]))
+        with np.errstate(over="ignore"):
+            want[ix] = want[ix] + row
+        F.add_(dx.view(*subs_x), bview)
+        np.testing.assert_array_equal(dx.numpy(), want, err_msg="row broadcast " + what)
