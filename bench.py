@@ -347,7 +347,7 @@ def size_probe(W, reps: int = 6):
     T = W.HIPTensor
     rng = np.random.Generator(np.random.PCG64(6))
     cases = []
-    for mb in (32, 64, 128, 256, 512, 1024):
+    for mb in SIZE_PROBE_MB:
         moved = mb << 20
         n = moved // 8                      # elements of a kernel that reads and writes each once
         count = max(2, -(-(768 << 20) // moved) + 1)
@@ -382,6 +382,56 @@ def size_probe(W, reps: int = 6):
         W.lib.synchronize()
     print(json.dumps({"probe_sizes": [{"kernel": k, "bytes": b, "elements": e} for k, b, e in cases],
                       "launches_each": reps}))
+
+
+SIZE_PROBE_MB = (32, 64, 128, 256, 512, 1024)
+
+
+def size_fit(trace_csv: str, reps: int = 6) -> str:
+    """The table of profiles/short_kernel_fit.txt from the kernel trace (csv) of a `--probe-sizes` run: per kernel
+    the median of the last `reps` - 1 launches at each size, the least-squares line t = t0 + bytes / rate through
+    the six sizes, and what that line says of a launch that moves 128 MB (2^24 elements read and written)."""
+    import csv
+    with open(trace_csv, newline="") as f:
+        launches = sorted(csv.DictReader(f), key=lambda r: int(r["Start_Timestamp"]))
+    runs = []  # consecutive launches of one kernel at one grid: [name, durations in us]
+    for r in launches:
+        key = (r["Kernel_Name"], r["Grid_Size_X"])
+        us = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+        if runs and runs[-1][0] == key:
+            runs[-1][1].append(us)
+        else:
+            runs.append([key, [us]])
+    # per size, in launch order: fills and `reps` copies (ew_flat<OpMove>) end where the broadcast row is written
+    # (ew_rows<OpMove>); then `reps` row-broadcast adds, `reps` softmaxes, fills, `reps` row sums
+    picked = {"copy": [], "row-broadcast add, rows of 8192": [], "row softmax, rows of 1024": [],
+              "row sum, rows of 4096": []}
+    for i, (key, times) in enumerate(runs):
+        name = key[0]
+        if "ew_rows<wf2::OpMove" in name and i > 0:
+            picked["copy"].append(runs[i - 1][1][-reps:])
+        elif "ew_rows<wf2::OpAdd" in name and len(times) == reps:
+            picked["row-broadcast add, rows of 8192"].append(times)
+        elif "softmax_rows" in name and len(times) == reps:
+            picked["row softmax, rows of 1024"].append(times)
+        elif "reduce_rows" in name and len(times) == reps:
+            picked["row sum, rows of 4096"].append(times)
+    lines = []
+    for kernel, per_size in picked.items():
+        if len(per_size) != len(SIZE_PROBE_MB):
+            raise SystemExit(f"bench.py --fit-sizes: {len(per_size)} runs of '{kernel}' in the trace, "
+                             f"{len(SIZE_PROBE_MB)} expected")
+        x = np.array([mb * float(1 << 20) for mb in SIZE_PROBE_MB])
+        t = np.array([float(np.median(times[1:])) for times in per_size])
+        slope, t0 = np.polyfit(x, t, 1)           # us per byte, us
+        rate = 1.0 / slope / 1e6                  # TB/s
+        lines.append(f"{kernel}: t = {t0:.2f} us + bytes / {rate:.2f} TB/s  ({rate / 8.0 * 100:.1f} % of 8 TB/s)")
+        for mb, got in zip(SIZE_PROBE_MB, t):
+            fit = t0 + mb * float(1 << 20) * slope
+            frac = mb * float(1 << 20) / got / 1e6 / 8.0 * 100
+            lines.append(f"    {mb:5d} MB  measured {got:8.2f} us ({frac:4.1f} %)   line {fit:8.2f} us   "
+                         f"fixed share {t0 / got * 100:4.1f} %")
+    return "\n".join(lines)
 
 
 def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
@@ -894,9 +944,14 @@ def main():
                     help="run the launch sequence of the attention kernels and one projection for rocprofv3 --pmc runs and exit")
     ap.add_argument("--probe-sizes", action="store_true",
                     help="run four kernels of the path at six sizes (32 MB ... 1 GB moved) for a rocprofv3 --kernel-trace run and exit")
+    ap.add_argument("--fit-sizes", metavar="KERNEL_TRACE_CSV",
+                    help="fit t = t0 + bytes / rate to the kernel trace of a --probe-sizes run, print the table and exit (no GPU)")
     ap.add_argument("--probe", action="store_true",
                     help="run the short fixed launch sequence used for rocprofv3 --pmc runs and exit")
     args = ap.parse_args()
+    if args.fit_sizes:
+        print(size_fit(args.fit_sizes))
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on ONE GPU (no collectives, no sharding); "
                  "--gpus must be 1")

@@ -733,14 +733,20 @@ static int launch_row_reduce(const Space& s, float* a, const float* b, double* p
   int64_t blocks = nrows * p.splits;
   if (blocks >= ((int64_t)1 << 31))
     return fail(WF2HIP_EUNSUPPORTED, "iteration space too large for one launch");
-  // far beyond the Infinity Cache: stream with non-temporal loads
-  // Footprints that do not stay in the 256 MB Infinity Cache: rows (or row segments) of
-  // 4096 elements and more through the streaming kernel; shorter ones, which do not fill
-  // one of its 4096-element batches, through the 256-thread kernel.  Measured cold,
-  // (32768, 2048): 42.1 us against 67.1 us through the streaming kernel; (16384, 4096):
-  // 39.2 us streaming against 45.5 us; (8192, 4096), 128 MiB: 21.6 us against 24.4 us.
+  // From 16 MiB on, rows (or row segments) of 4096 elements and more go through the streaming
+  // kernel; shorter ones, which do not fill one of its 4096-element batches, through the
+  // 256-thread kernel.  Kernel durations on operands that are not in a cache, (32768, 2048):
+  // 42.1 us against 67.1 us through the streaming kernel; (16384, 4096): 39.2 us streaming
+  // against 45.5 us; (8192, 4096): 21.6 us against 24.4 us; (4096, 4096): 13.0 us against
+  // 24.6 us; (2048, 4096): 8.6 us against 13.8 us.  On operands the Infinity Cache holds the
+  // two are within 10 % of each other up to 32 MiB and the streaming kernel ahead beyond
+  // ((4096, 4096): 8.1 us against 11.9 us).  WF2HIP_ROWSUM_STREAM_MB moves the threshold.
   const int64_t bytes = nrows * p.n0 * 4;
-  if (vec_ok && p.seg >= 4096 && bytes >= ((int64_t)128 << 20))
+  static const int64_t stream_from = [] {
+    const char* e = getenv("WF2HIP_ROWSUM_STREAM_MB");
+    return (int64_t)(e ? atoi(e) : 16) << 20;
+  }();
+  if (vec_ok && p.seg >= 4096 && bytes >= stream_from)
     reduce_rows_stream<<<(uint32_t)blocks, kStreamBlock, 0, st>>>(p);
   else if (vec_ok && bytes >= ((int64_t)192 << 20))  // nontemporal loads: (32768, 2048) 39.0 us against 41.7 us
     reduce_rows_block<4, true><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
