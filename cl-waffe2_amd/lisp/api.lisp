@@ -169,6 +169,8 @@
 (defcfun "wf2hip_graph_launch" :int (graph :pointer))
 (defcfun "wf2hip_graph_destroy" :int (graph :pointer))
 (defcfun "wf2hip_pool_trim" :int)
+(defcfun "wf2hip_pool_idle_bytes" :size)
+(defcfun "wf2hip_pool_requests" :size)
 
 (defmacro with-captured-graph ((graph) &body body)
   "Runs BODY once with every kernel launch recorded instead of executed and binds GRAPH to the

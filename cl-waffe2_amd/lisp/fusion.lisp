@@ -187,7 +187,7 @@ composed recipe."
 (define-op (HIP-Softmax-Cross-Entropy-Node (self delta)
             :slots ((delta :initform 1e-7 :accessor cross-entropy-delta))
             :save-for-backward-names (z label)
-            :where (X[rows cols] Labels[rows cols] Z[rows cols] OUT[rows cols] -> OUT[rows cols])
+            :where (X[rows cols] Label[rows cols] Z[rows cols] OUT[rows cols] -> OUT[rows cols])
             :documentation "Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126) on contiguous
 matrices as one kernel (wf2hip_softmax_cross_entropy_f32): Z <- softmax over the last axis of X, saved
 for the backward as the reference saves it, OUT <- -1 (Labels log(Z + delta)).  Backward: one kernel
