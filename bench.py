@@ -297,7 +297,8 @@ def row_probe(W, reps: int = 5):
 def matrix_core_probe(W, reps: int = 4):
     """The launch sequence for `rocprofv3 --pmc` runs of the kernels bound by the matrix cores, at the block's
     shapes: `reps` launches each of attention forward (full, then causal), attention backward (causal:
-    D, dQ, dK and dV) and one projection, printed in order at the end."""
+    D, then dQ / dK / dV in one launch), the block's projections and the products of a few rows, printed in order
+    at the end."""
     F = W.functional
     T = W.HIPTensor
     rng = np.random.Generator(np.random.PCG64(6))
@@ -331,6 +332,16 @@ def matrix_core_probe(W, reps: int = 4):
         names.append(f"matmul {m}x{n}x{k}" + (" + bias" if bias else "") + (" + residual" if res else "") +
                      (" + GELU" if act else ""))
         del a, b, c, bv, rv
+    # a few rows against a wide operand: the streaming kernel of 16 rows, and the token projection of 64 rows
+    # with the operands exchanged
+    for m, n, k, stored in ((16, 8192, 8192, "kn"), (16, 50257, 768, "nk"), (64, 50257, 768, "nk")):
+        a = T.from_numpy(rng.standard_normal((m, k)).astype(np.float32))
+        w = T.from_numpy((rng.standard_normal((k, n) if stored == "kn" else (n, k)) * 0.02).astype(np.float32))
+        c = T([m, n], initial_element=None)
+        for _ in range(reps):
+            F.matmul(a, w if stored == "kn" else F.t(w), out=c)
+        names.append(f"matmul {m}x{n}x{k}, few rows" + (", right operand stored (n, k)" if stored == "nk" else ""))
+        del a, w, c
     W.lib.synchronize()
     print(json.dumps({"probe_matrix_cores": ["attention (8,12,1024,64) full", "attention causal",
                                              "attention backward causal (D, then dQ / dK / dV)"] + names,
@@ -729,8 +740,16 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         ring = ring_of(lambda: (clone(a0), clone(w0), T([m, n], initial_element=None)), 4 * (m * k + k * n + m * n))
         label = (f"matmul {m}x{n}x{k}, few rows" if stored == "kn" else
                  f"matmul {m}x{n}x{k}, few rows, right operand stored ({n},{k}) (!t): GPT-2's token projection")
+        # 2 m flop per 4 bytes of the wide operand: beyond 39 rows (157.3 TFLOP/s / 8 TB/s = 19.7 flop per byte)
+        # the matrix cores bound the product, not the one read of the operand
+        flop_us = 2.0 * m * n * k / FP32_MFMA_PEAK_TFLOPS / 1e6
+        byte_us = 4.0 * (m * k + k * n + m * n) / HBM_PEAK_GBS / 1e3
         measure(label, ring, (lambda s: F.matmul(s[0], s[1], out=s[2])) if stored == "kn" else
-                (lambda s: F.matmul(s[0], F.t(s[1]), out=s[2])), 4 * (m * k + k * n + m * n))
+                (lambda s: F.matmul(s[0], F.t(s[1]), out=s[2])), 4 * (m * k + k * n + m * n),
+                note=(f"at the peaks: {byte_us:.1f} us of HBM traffic, {flop_us:.1f} us of fp32 matrix-core work"
+                      + ("; bound by the matrix cores" if flop_us > byte_us else "")))
+        if flop_us > byte_us:
+            rows[label]["frac_mfma_peak"] = round(flop_us * 1e-3 / rows[label]["ms"], 4)
         del a0, w0
     # class scores: very many rows of ten columns; and one row of 2^24 columns
     for rows_, cols_ in ((1677721, 10), (1, 1 << 24)):
