@@ -324,6 +324,114 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_lines_kernel(SkinnyParams
     }
 }
 
+// The same product with a workgroup of ONE wavefront per 16 CB columns (rows of W) and slice of K.  The kernel
+// above hands a workgroup 64 columns, so GPT-2's token projection (50257 columns) is 786 workgroups, all
+// resident at once, three on most compute units and four on some: the counters show a compute unit holding a
+// wave for 57 % of the launch only.  1571 one-wavefront workgroups of 32 columns are dealt out as compute units
+// fall free.  Each keeps KSTEPS steps of 32 of K in flight per buffer (8 KB of W with CB = 2, KSTEPS = 2); x
+// comes from the L2 cache, once per workgroup (16 columns per wavefront read x as often as W and run 15 %
+// slower).  No meeting in LDS: a wavefront covers its slice of K alone.
+template <int MT, int CB, int KSTEPS>
+__global__ __launch_bounds__(kWave) void sgemm_skinny_wave_kernel(SkinnyParams p) {
+  constexpr int kPitch = 36;
+  __shared__ __attribute__((aligned(16))) float piece[KSTEPS][16 * CB * kPitch];
+  const int lane = threadIdx.x;
+  const int kk = lane >> 4, jj = lane & 15;
+  const int lrow = lane >> 3, lk = (lane & 7) * 4;  // the loading layout: row within eight, step within 32
+  const uint32_t ks = blockIdx.x / p.cgroups, cg = blockIdx.x - ks * p.cgroups;
+  const int64_t j0 = (int64_t)cg * 16 * CB;
+  const int kbeg = (int)ks * p.kslice;
+  const int kend = kbeg + p.kslice < p.k ? kbeg + p.kslice : p.k;
+  const f4 zero = {0.f, 0.f, 0.f, 0.f};
+  f4 acc[MT][CB];
+#pragma unroll
+  for (int t = 0; t < MT; t++)
+#pragma unroll
+    for (int b = 0; b < CB; b++) acc[t][b] = zero;
+  const float* wrow[2 * CB];
+#pragma unroll
+  for (int q = 0; q < 2 * CB; q++) {
+    int64_t j = j0 + 8 * q + lrow;
+    if (j >= p.cols) j = p.cols - 1;  // read, not stored
+    wrow[q] = p.W + j * p.ldw + lk;
+  }
+  const float* xrow[MT];
+  bool xlive[MT];
+#pragma unroll
+  for (int t = 0; t < MT; t++) {
+    const int i = 16 * t + jj;
+    xlive[t] = i < p.rows;
+    xrow[t] = p.X + (int64_t)(xlive[t] ? i : 0) * p.ldx + 4 * kk;
+  }
+  f4 wv[2][KSTEPS][2 * CB], xv[2][KSTEPS][MT][2];
+  auto fetch = [&](int k0, int buf) {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) {
+      const int kq = k0 + 32 * s;
+      const bool in = kq + lk < kend;  // k and the slices are multiples of 4: a vector is wholly in or out
+#pragma unroll
+      for (int q = 0; q < 2 * CB; q++)
+        wv[buf][s][q] = in ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(wrow[q] + kq)) : zero;
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const bool xin = kq + 16 * h + 4 * kk < kend;
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+          xv[buf][s][t][h] = (xin && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + kq + 16 * h) : zero;
+      }
+    }
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+      for (int q = 0; q < 2 * CB; q++) *reinterpret_cast<f4*>(&piece[s][(8 * q + lrow) * kPitch + lk]) = wv[buf][s][q];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        f4 w[CB];
+#pragma unroll
+        for (int b = 0; b < CB; b++) w[b] = *reinterpret_cast<const f4*>(&piece[s][(16 * b + jj) * kPitch + 16 * h + 4 * kk]);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+          for (int b = 0; b < CB; b++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+              acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[buf][s][t][h][e], w[b][e], acc[t][b], 0, 0, 0);
+      }
+    __builtin_amdgcn_wave_barrier();
+  };
+  if (kbeg < kend) {
+    fetch(kbeg, 0);
+    for (int k0 = kbeg; k0 < kend; k0 += 64 * KSTEPS) {  // fetches past the end load nothing and multiply zeros
+      fetch(k0 + 32 * KSTEPS, 1);
+      multiply(0);
+      fetch(k0 + 64 * KSTEPS, 0);
+      multiply(1);
+    }
+  }
+  // D[4 (lane / 16) + r][lane % 16] of tile (t, b) in register r
+#pragma unroll
+  for (int b = 0; b < CB; b++) {
+    const int64_t col = j0 + 16 * b + jj;
+    if (col >= p.cols) continue;
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = 16 * t + 4 * kk + r;
+        if (row >= p.rows) continue;
+        if (p.gsplit == 1)
+          skinny_finish_store(p, row, col, acc[t][b][r]);
+        else
+          p.partial[((int64_t)ks * p.rows + row) * p.cols + col] = acc[t][b][r];
+      }
+  }
+}
+
 // the slices' planes added in the order 0, 1, ..., then alpha, beta, bias, activation, residual
 __global__ __launch_bounds__(kBlock) void sgemm_skinny_finish(SkinnyParams p) {
   const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -389,6 +497,19 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
   // per wavefront with the whole K instead of quarters of K (GPT-2's token projection 48.3 against 49.6 us,
   // everything else slower).
   int64_t gsplit = (int64_t)rt().num_cus * 2 / p.cgroups;
+  // W stored along k, at most 32 rows, and enough columns to fill the device without slicing K (from 32768
+  // columns on): a wavefront per 32 columns.  GPT-2's token projection, 1 / 16 / 32 rows: 30.6 / 33.8 / 50.9 us
+  // against 40.9 / 42.7 / 58.5 us; with slices of K ((8192, 8192)^T) the workgroups of four wavefronts above
+  // are level or ahead (32 rows: 75 against 86 us) and keep the work.
+  static const bool wave_env = [] {
+    const char* e = getenv("WF2HIP_SKINNY_WAVE");
+    return !e || atoi(e) != 0;
+  }();
+  const bool by_wave = w_is_cols_by_k && mt <= 2 && wave_env && cols >= (int64_t)128 * rt().num_cus;
+  if (by_wave) {
+    p.cgroups = (uint32_t)ceil_div((int64_t)cols, (int64_t)32);
+    gsplit = 1;
+  }
   if (gsplit > k / 256) gsplit = k / 256;
   if (gsplit < 1) gsplit = 1;
   // (128: a quarter per wavefront then starts on a 128-byte line of W's rows where those are stored along k)
@@ -416,7 +537,11 @@ bool try_sgemm_skinny(bool w_is_cols_by_k, long rows, long cols, long k, float a
     else if (mt == 2) sgemm_skinny_kernel<TW_, 2, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);   \
     else sgemm_skinny_kernel<TW_, 4, 4><<<(uint32_t)blocks, kBlock, 0, st>>>(p);                \
   } while (0)
-  if (w_is_cols_by_k && mt == 1)
+  if (by_wave && mt == 1)
+    sgemm_skinny_wave_kernel<1, 2, 2><<<(uint32_t)blocks, kWave, 0, st>>>(p);
+  else if (by_wave)
+    sgemm_skinny_wave_kernel<2, 2, 2><<<(uint32_t)blocks, kWave, 0, st>>>(p);
+  else if (w_is_cols_by_k && mt == 1)
     sgemm_skinny_lines_kernel<1><<<(uint32_t)blocks, kBlock, 0, st>>>(p);
   else if (w_is_cols_by_k && mt == 2)
     sgemm_skinny_lines_kernel<2><<<(uint32_t)blocks, kBlock, 0, st>>>(p);

@@ -671,6 +671,30 @@ def test_matmul_few_rows(gpu, rows, cols, k):
         assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
 
 
+@pytest.mark.parametrize("rows", [1, 9, 16, 25, 32])
+@pytest.mark.parametrize("cols,k", [(32768, 64), (40001, 100), (50257, 768), (33000, 1028)])
+def test_matmul_few_rows_against_a_table_of_many_rows(gpu, rows, cols, k):
+    """At most 32 rows against a table of 32768 rows and more stored (cols, k) -- GPT-2's token projection,
+    `(!matmul x (!t wte))`: a wavefront per 32 columns with the whole of K.  Ragged last group, K on and off the
+    steps of 64, and the fused epilogue on the same path; float64 with the bound of the other gemm tests."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows * 31 + cols + k)
+    X = rng.standard_normal((rows, k)).astype(np.float32)
+    Wt = rng.standard_normal((cols, k)).astype(np.float32)
+    dX, dW = F.from_numpy(X), F.from_numpy(Wt)
+    X64, W64 = X.astype(np.float64), Wt.astype(np.float64).T
+    _gemm_check(F.matmul(dX, F.t(dW)).numpy(), X64, W64)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    res = rng.standard_normal((rows, cols)).astype(np.float32)
+    z = X64 @ W64 + bias
+    bound = REL * (np.abs(X64) @ np.abs(W64) + np.abs(bias)) + 1e-30
+    got = F.matmul(dX, F.t(dW), bias=F.from_numpy(bias), residual=F.from_numpy(res)).numpy()
+    assert np.all(np.abs(got - (z + res)) <= bound + REL * np.abs(res))
+    got = F.matmul(dX, F.t(dW), bias=F.from_numpy(bias), activation="gelu").numpy()
+    gelu = 0.5 * z * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (z + 0.044715 * z ** 3)))
+    assert np.all(np.abs(got - gelu) <= 2.0 * bound + 4e-6 * np.abs(gelu) + 1e-6)
+
+
 @pytest.mark.parametrize("rows", [33, 48, 64])
 @pytest.mark.parametrize("cols,k", [(1024, 256), (4100, 768), (2051, 512), (2048, 4096), (50257, 768)])
 def test_matmul_33_to_64_rows_against_a_table(gpu, rows, cols, k):
