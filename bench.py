@@ -756,8 +756,8 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         x0 = normal([rows_, cols_])
         ring = ring_of(lambda: (clone(x0), T([rows_, cols_], initial_element=None)), 8 * rows_ * cols_)
         measure(f"row softmax ({rows_},{cols_}), one kernel" if rows_ > 1 else
-                f"row softmax ({rows_},{cols_}): pieces of the row over the grid, two launches", ring,
-                lambda s: F.softmax_fused(s[0], out=s[1]), (8 if rows_ > 1 else 12) * rows_ * cols_)
+                f"row softmax ({rows_},{cols_}): pieces of the row over the grid, one launch", ring,
+                lambda s: F.softmax_fused(s[0], out=s[1]), 8 * rows_ * cols_)
         del x0
     B, H, S, hd = 8, 12, 1024, 64
     q0 = normal([B, H, S, hd])

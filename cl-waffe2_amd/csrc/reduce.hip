@@ -1256,6 +1256,111 @@ __global__ __launch_bounds__(kLongBlock) void softmax_split_apply(const float* x
   }
 }
 
+// A few very long rows in ONE launch: a workgroup of 1024 threads holds a piece of 65536 columns in registers,
+// leaves the piece's maximum and sum, waits until every piece of the launch has done so, folds its row's pieces
+// like softmax_split_apply and writes its share -- one read and one write of the row where the two launches
+// above read it twice.
+//
+// The wait needs every workgroup of the grid on the device at the same time: the host launches this form only
+// when the grid is no larger than what the device holds at once (one such workgroup per compute unit).  Even
+// so a workgroup never waits without bound: after kMeetSpins polls it stops waiting and works out the row's
+// maximum and sum from the row itself -- which is why x and out must not overlap here.  The two counters are
+// left at zero by the last workgroup to pass, for the next launch; launches of this kernel that overlap in
+// time on one device (several streams) would share them and must not happen: the library launches on one stream.
+constexpr int kOneE = 64;
+constexpr int64_t kOnePiece = (int64_t)kLongBlock * kOneE;
+constexpr uint32_t kMeetSpins = 1u << 20;  // about a second
+__device__ unsigned int g_softmax_meet[2];  // [0]: pieces that left their statistics, [1]: workgroups past the wait
+
+__global__ __launch_bounds__(kLongBlock) void softmax_one_launch(const float* __restrict__ x, int64_t ldx,
+                                                                 float* __restrict__ out, int64_t ldo, int64_t ncols,
+                                                                 uint32_t pieces, float* pmax, double* psum,
+                                                                 uint32_t spins) {
+  __shared__ float lmax[kLongBlock / kWave];
+  __shared__ double lsum[kLongBlock / kWave];
+  __shared__ int met;
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const float* xr = x + (int64_t)row * ldx;
+  const int64_t c0 = (int64_t)piece * kOnePiece;
+  const float ninf = -__builtin_inff();
+  // thread t holds the 16-byte vectors (g 1024 + t) 4 of the piece (16-byte aligned rows, ncols a multiple of 4)
+  float v[kOneE];
+  const uint32_t first = threadIdx.x * 4;                            // within the piece
+  const uint32_t left = (uint32_t)((ncols - c0 < kOnePiece ? ncols - c0 : kOnePiece));  // columns of this piece
+  const float* xp = xr + c0;
+  float m = ninf;
+#pragma unroll
+  for (int g = 0; g < kOneE / 4; g++) {
+    f4 t = {ninf, ninf, ninf, ninf};
+    if (first + g * 4 * kLongBlock < left) t = __builtin_nontemporal_load(reinterpret_cast<const f4*>(xp + first + g * 4 * kLongBlock));
+    v[4 * g] = t.x; v[4 * g + 1] = t.y; v[4 * g + 2] = t.z; v[4 * g + 3] = t.w;
+  }
+  // exponentials once, against the thread's own maximum (no exchange between the loads and this pass): the
+  // output is e_k exp(m_thread - M) / S
+#pragma unroll
+  for (int k = 0; k < kOneE; k++) m = fmaxf(m, v[k]);
+  float sum = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kOneE; k++) {
+    v[k] = exp_below_max(v[k], m);
+    sum += v[k];
+  }
+  const float mine = m;
+  m = long_block_max(mine, lmax);
+  const double total = long_block_sum((double)sum * (double)exp_below_max(mine, m), lsum);
+  if (threadIdx.x == 0) {
+    // The statistics go to memory past the caches (device-scope atomic stores), are waited for, and only then
+    // is the arrival counted: the order a release would give, without its write-back of the whole L2 (2.6 us
+    // per workgroup here).  The readers below use device-scope loads, which no stale cache line serves.
+    __hip_atomic_store(&pmax[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&psum[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __hip_atomic_fetch_add(&g_softmax_meet[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t polls = 0;
+    while (__hip_atomic_load(&g_softmax_meet[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x && polls < spins) {
+      __builtin_amdgcn_s_sleep(8);
+      polls++;
+    }
+    met = __hip_atomic_load(&g_softmax_meet[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= gridDim.x;
+  }
+  __syncthreads();
+  float big = ninf;
+  double s = 0.0;
+  if (met) {
+    // the fold of softmax_split_apply; the statistics were written by other workgroups during this launch:
+    // read them past the caches this compute unit may hold stale lines in
+    for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock)
+      big = fmaxf(big, __hip_atomic_load(&pmax[row * pieces + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    big = long_block_max(big, lmax);
+    for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock)
+      s += __hip_atomic_load(&psum[row * pieces + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) *
+           (double)exp_below_max(__hip_atomic_load(&pmax[row * pieces + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), big);
+  } else {
+    // gave up waiting: the row's maximum and sum from the row itself (x is not written by this launch)
+    for (int64_t c = threadIdx.x; c < ncols; c += kLongBlock) big = fmaxf(big, xr[c]);
+    big = long_block_max(big, lmax);
+    float part = 0.0f;
+    for (int64_t c = threadIdx.x; c < ncols; c += kLongBlock) part += exp_below_max(xr[c], big);
+    s = (double)part;
+  }
+  const float factor = exp_below_max(mine, big) * (float)(1.0 / long_block_sum(s, lsum));
+  float* op = out + (int64_t)row * ldo + c0;
+#pragma unroll
+  for (int g = 0; g < kOneE / 4; g++) {
+    f4 t;
+#pragma unroll
+    for (int c = 0; c < 4; c++) t[c] = v[4 * g + c] * factor;
+    if (first + g * 4 * kLongBlock < left) __builtin_nontemporal_store(t, reinterpret_cast<f4*>(op + first + g * 4 * kLongBlock));
+  }
+  if (threadIdx.x == 0) {
+    const unsigned int before = __hip_atomic_fetch_add(&g_softmax_meet[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (before + 1 == gridDim.x) {  // everyone has arrived and is past the wait: zero for the next launch
+      __hip_atomic_store(&g_softmax_meet[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&g_softmax_meet[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 template <int NV, bool VEC, bool NT, int RW = 1>
 __global__ __launch_bounds__(kBlock) void layernorm_rows_wave(const float* __restrict__ x,
                                                               const float* __restrict__ gamma,
@@ -1723,6 +1828,19 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
 // at least this many rows: below it the wavefront forms already finish within a launch's floor
 constexpr int64_t kTinyMinRows = 16384;
 
+// How many workgroups of softmax_one_launch the device holds at once (0: the form is not used).
+static int64_t softmax_one_launch_capacity() {
+  static const int64_t capacity = [] {
+    int held = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&held, softmax_one_launch, kLongBlock, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      return (int64_t)0;
+    }
+    return (int64_t)held * rt().num_cus;
+  }();
+  return capacity;
+}
+
 template <bool XENT>
 static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int64_t ldx, float* out,
                                int64_t ldo, int64_t causal_seq, float scale, Xent xe) {
@@ -1744,6 +1862,29 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
     const int64_t pieces = ceil_div(ncols, kSplitPiece);
     if (ncols > 64 * kLongBlock || (pieces >= 2 && nrows < rt().num_cus)) {
       if (nrows * pieces >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many row pieces for one launch");
+      // one launch when every workgroup of it is on the device at once, and x and out are apart
+      const int64_t big_pieces = ceil_div(ncols, kOnePiece);
+      const float* x_end = x + (nrows - 1) * ldx + ncols;
+      const float* out_end = out + (nrows - 1) * ldo + ncols;
+      static const bool one_env = [] {
+        const char* e = getenv("WF2HIP_SOFTMAX_ONE_LAUNCH");
+        return !e || atoi(e) != 0;
+      }();
+      // testing knob, read at every call: with 0 polls every workgroup takes the path of one that gave up waiting
+      const char* spins_env = getenv("WF2HIP_SOFTMAX_MEET_SPINS");
+      const uint32_t meet_spins = spins_env ? (uint32_t)atol(spins_env) : kMeetSpins;
+      const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0 && ncols % 4 == 0;
+      if (!XENT && one_env && vec && nrows * big_pieces <= softmax_one_launch_capacity() && (x_end <= out || out_end <= x)) {
+        void* stats = nullptr;
+        WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(nrows * big_pieces) * (sizeof(double) + sizeof(float))));
+        double* psum = static_cast<double*>(stats);
+        float* pmax = reinterpret_cast<float*>(psum + nrows * big_pieces);
+        const uint32_t grid = (uint32_t)(nrows * big_pieces);
+        softmax_one_launch<<<grid, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, (uint32_t)big_pieces, pmax, psum, meet_spins);
+        const int rc = after_launch("softmax_one_launch");
+        (void)wf2hip_free(stats);  // stream order keeps it alive for the launch above
+        return rc;
+      }
       void* stats = nullptr;  // nrows x pieces sums (binary64), then as many maxima
       WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(nrows * pieces) * (sizeof(double) + sizeof(float))));
       double* psum = static_cast<double*>(stats);

@@ -296,8 +296,38 @@ def test_softmax_rows_in_pieces(gpu, rows, cols):
     got = F.softmax_fused(d).numpy()
     _assert_softmax(got, _softmax64(X), f"({rows}, {cols})")
     assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
-    F.softmax_fused(d, out=d)
-    np.testing.assert_array_equal(d.numpy(), got)
+    F.softmax_fused(d, out=d)  # in place: always the two launches, whose pieces are shorter
+    np.testing.assert_allclose(d.numpy(), got, rtol=8e-6, atol=1.2e-38)  # each within 4e-6 of the truth
+    _assert_softmax(d.numpy(), _softmax64(X), f"({rows}, {cols}) in place")
+
+
+def test_softmax_long_rows_in_one_launch(gpu, monkeypatch):
+    """A few rows whose pieces of 65536 columns all fit on the device at once go through one launch in which
+    every workgroup waits for the others' statistics: (1, 2^24) is one workgroup on every compute unit.  Twice in
+    a row and then a smaller one (the counters of the meeting are left at zero by each launch); the same with
+    no polls allowed, where every workgroup takes the path of one that gave up waiting and works out the row's
+    statistics by itself."""
+    F = gpu.functional
+    rng = np.random.default_rng(24)
+    big = (rng.standard_normal((1, 1 << 24)) * 3).astype(np.float32)
+    big[0, 12345678] = 25.0
+    want_big = _softmax64(big)
+    d, o = F.from_numpy(big), gpu.HIPTensor([1, 1 << 24])
+    for _ in range(2):
+        F.softmax_fused(d, out=o)
+        _assert_softmax(o.numpy(), want_big, "(1, 2^24)")
+    small = (rng.standard_normal((3, 65536 * 3 + 8)) * 3).astype(np.float32)
+    small[1, :65536] = -np.inf
+    want_small = _softmax64(small)
+    got = F.softmax_fused(F.from_numpy(small)).numpy()
+    _assert_softmax(got, want_small, "(3, 196616)")
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
+    monkeypatch.setenv("WF2HIP_SOFTMAX_MEET_SPINS", "0")
+    alone = F.softmax_fused(F.from_numpy(small)).numpy()
+    _assert_softmax(alone, want_small, "(3, 196616), nobody waits")
+    monkeypatch.delenv("WF2HIP_SOFTMAX_MEET_SPINS")
+    again = F.softmax_fused(F.from_numpy(small)).numpy()
+    np.testing.assert_array_equal(again, got)
 
 
 def test_softmax_reference_composition(gpu, O):
