@@ -1272,10 +1272,11 @@ constexpr int64_t kOnePiece = (int64_t)kLongBlock * kOneE;
 constexpr uint32_t kMeetSpins = 1u << 20;  // about a second
 __device__ unsigned int g_softmax_meet[2];  // [0]: pieces that left their statistics, [1]: workgroups past the wait
 
+template <bool XENT>
 __global__ __launch_bounds__(kLongBlock) void softmax_one_launch(const float* __restrict__ x, int64_t ldx,
                                                                  float* __restrict__ out, int64_t ldo, int64_t ncols,
                                                                  uint32_t pieces, float* pmax, double* psum,
-                                                                 uint32_t spins) {
+                                                                 uint32_t spins, Xent xe) {
   __shared__ float lmax[kLongBlock / kWave];
   __shared__ double lsum[kLongBlock / kWave];
   __shared__ int met;
@@ -1350,7 +1351,17 @@ __global__ __launch_bounds__(kLongBlock) void softmax_one_launch(const float* __
     f4 t;
 #pragma unroll
     for (int c = 0; c < 4; c++) t[c] = v[4 * g + c] * factor;
-    if (first + g * 4 * kLongBlock < left) __builtin_nontemporal_store(t, reinterpret_cast<f4*>(op + first + g * 4 * kLongBlock));
+    if (first + g * 4 * kLongBlock < left) {
+      __builtin_nontemporal_store(t, reinterpret_cast<f4*>(op + first + g * 4 * kLongBlock));
+      if constexpr (XENT) {  // labels and loss are packed (rows, ncols)
+        const int64_t at = (int64_t)row * ncols + c0 + first + g * 4 * kLongBlock;
+        const f4 lab = __builtin_nontemporal_load(reinterpret_cast<const f4*>(xe.labels + at));
+        f4 l;
+#pragma unroll
+        for (int c = 0; c < 4; c++) l[c] = xent_term(lab[c], t[c], xe.delta);
+        __builtin_nontemporal_store(l, reinterpret_cast<f4*>(xe.loss + at));
+      }
+    }
   }
   if (threadIdx.x == 0) {
     const unsigned int before = __hip_atomic_fetch_add(&g_softmax_meet[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1831,12 +1842,13 @@ constexpr int64_t kTinyMinRows = 16384;
 // How many workgroups of softmax_one_launch the device holds at once (0: the form is not used).
 static int64_t softmax_one_launch_capacity() {
   static const int64_t capacity = [] {
-    int held = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&held, softmax_one_launch, kLongBlock, 0) != hipSuccess) {
+    int plain = 0, xent = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, softmax_one_launch<false>, kLongBlock, 0) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&xent, softmax_one_launch<true>, kLongBlock, 0) != hipSuccess) {
       (void)hipGetLastError();
       return (int64_t)0;
     }
-    return (int64_t)held * rt().num_cus;
+    return (int64_t)std::min(plain, xent) * rt().num_cus;
   }();
   return capacity;
 }
@@ -1874,13 +1886,14 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
       const char* spins_env = getenv("WF2HIP_SOFTMAX_MEET_SPINS");
       const uint32_t meet_spins = spins_env ? (uint32_t)atol(spins_env) : kMeetSpins;
       const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0 && ncols % 4 == 0;
-      if (!XENT && one_env && vec && nrows * big_pieces <= softmax_one_launch_capacity() && (x_end <= out || out_end <= x)) {
+      const bool xent_ok = !XENT || (aligned16(xe.labels) && aligned16(xe.loss));
+      if (one_env && vec && xent_ok && nrows * big_pieces <= softmax_one_launch_capacity() && (x_end <= out || out_end <= x)) {
         void* stats = nullptr;
         WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(nrows * big_pieces) * (sizeof(double) + sizeof(float))));
         double* psum = static_cast<double*>(stats);
         float* pmax = reinterpret_cast<float*>(psum + nrows * big_pieces);
         const uint32_t grid = (uint32_t)(nrows * big_pieces);
-        softmax_one_launch<<<grid, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, (uint32_t)big_pieces, pmax, psum, meet_spins);
+        softmax_one_launch<XENT><<<grid, kLongBlock, 0, st>>>(x, ldx, out, ldo, ncols, (uint32_t)big_pieces, pmax, psum, meet_spins, xe);
         const int rc = after_launch("softmax_one_launch");
         (void)wf2hip_free(stats);  // stream order keeps it alive for the launch above
         return rc;
