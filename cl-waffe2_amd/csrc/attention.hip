@@ -415,8 +415,6 @@ __global__ __launch_bounds__(kBlock) void attention_delta_kernel(const float* __
 template <bool KEYS>
 __device__ __forceinline__ void attention_bwd_body(const AttnBwdParams& p, const int rank, const int bh) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  auto tile1 = [&](int stage) { return smem + stage * kBwdStageFloats; };
-  auto tile2 = [&](int stage) { return smem + stage * kBwdStageFloats + kKBlock * kRowFloats; };
   float* const stats = smem + 2 * kBwdStageFloats;  // [stage][L: 64, D: 64]
 
   // rank 0 is the longest: the last query block walks the most key tiles, the first key block the most query tiles
