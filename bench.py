@@ -556,6 +556,13 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
         ring = ring_of(lambda: (clone(x0), clone(x0)), 2 * 4 * N)
         measure(f"x += y, :{dtype}, 256 MiB per tensor", ring, lambda s: F.add_(s[0], s[1]), 12 * N)
         del x0
+    # the same on a sliced view of an 8-bit tensor: rows that start and end off every 16-byte boundary
+    rows8, wide8 = 16384, 16448
+    x0 = T.from_numpy(rng.integers(0, 100, (rows8, wide8)).astype(np.uint8), dtype="uint8")
+    ring = ring_of(lambda: (clone(x0), clone(x0)), 2 * rows8 * wide8)
+    measure("x += y on the window [:, 3:16387] of :uint8 (16384,16448) tensors", ring,
+            lambda s: F.add_(s[0].view(True, (3, 16387)), s[1].view(True, (5, 16389))), 3 * rows8 * 16384)
+    del x0
 
     # transposing copy through LDS tiles
     a0 = normal([SIDE, SIDE])
@@ -627,6 +634,18 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     measure("LayerNorm (65536,1024), one kernel", ring, lambda s: F.layer_norm_fused(s[0], g0, b0, out=s[1]),
             8 * R * Cn)
     del x0, g0, b0
+    # rows beyond 8192 columns: a workgroup of 1024 threads per row, forward and backward
+    R, Cn = 4096, 16384
+    x0, g0, b0 = normal([R, Cn]), normal([Cn]), normal([Cn])
+    ring = ring_of(lambda: (clone(x0), T([R, Cn], initial_element=None)), 8 * R * Cn)
+    measure("LayerNorm (4096,16384), one kernel", ring, lambda s: F.layer_norm_fused(s[0], g0, b0, out=s[1]),
+            8 * R * Cn)
+    dg0, db0 = T([Cn], initial_element=None), T([Cn], initial_element=None)
+    ring = ring_of(lambda: (clone(x0), clone(x0), T([R, Cn], initial_element=None)), 12 * R * Cn)
+    measure("LayerNorm backward (4096,16384): dx, dgamma, dbeta (three launches)", ring,
+            lambda s: W.nodes.forward("HIP-LayerNorm-Node-backward", s[0], g0, s[1], s[2], dg0, db0, 1e-5),
+            12 * R * Cn)
+    del x0, g0, b0, dg0, db0
     p0 = normal([N])
     for name, make, per in (("Adam", lambda p: W.optimizers.Adam(p, lr=1e-3), 28), ("SGD", lambda p: W.optimizers.SGD(p, lr=1e-3), 16)):
         ring = ring_of(lambda: (make(clone(p0)), clone(p0)), per * N)
@@ -921,7 +940,8 @@ COMPACT_ROWS = (
     ("cfg3_exp", "exp 2^26"), ("cfg3_tanh", "tanh 2^26"), ("cfg3_sin", "sin 2^26"), ("cfg3_log", "loge 2^26"),
     ("cfg4_rowsum", "row sum (8192,4096), !sum as one node"), ("cfg4_fullsum", "full sum (8192,4096)"),
     ("cfg4_softmax", "row softmax (32768,1024), one kernel"), ("copy_536MB", "copy 2^26"), ("copy_268MB", "copy (32768,1024)"),
-    ("layernorm", "LayerNorm (65536,1024)"), ("layernorm_bwd", "LayerNorm backward"), ("adam", "Adam step"),
+    ("layernorm", "LayerNorm (65536,1024)"), ("layernorm_bwd", "LayerNorm backward (65536"), ("ln_16384", "LayerNorm (4096,16384)"),
+    ("ln_16384_bwd", "LayerNorm backward (4096,16384)"), ("u8_window_add", "x += y on the window"), ("adam", "Adam step"),
     ("transpose", "transposing copy"), ("unfold", "unfold (32,64,56,56) 3x3 pad 1, one kernel"),
     ("im2col", "Im2ColNode (32,64,58,58)"), ("im2col_pad", "Im2ColNode, padding 1"), ("col2im", "Col2ImNode"),
     ("mm_8192x2304x768", "matmul 8192x2304x768"), ("mm_8192x3072x768", "matmul 8192x3072x768"),

@@ -506,18 +506,19 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __rest
   }
 }
 
-// Rows of 2049 ... 8192 columns: a workgroup per row, thread t holding the NG 16-byte vectors
+// Rows of 2049 ... 8192 columns (BLOCK = 1024 threads: up to 16384): a workgroup per row, thread t holding the NG 16-byte vectors
 // (g 256 + t) 4 ... of x, dy and gamma and its share of the two column sums in registers; the
 // row statistics meet in LDS (three exchanges per row).  Workgroup b walks rows b, b + B, ...
 // and leaves its column sums in row b of `partial`, folded like the narrower kernel's.  Same
 // formulas as above: the mean from binary64 sums, deviations and squares in binary32.
-template <int NG, bool NT>
-__global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __restrict__ x,
+template <int NG, bool NT, int BLOCK = kBlock>
+__global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restrict__ x,
                                                              const float* __restrict__ gamma,
                                                              const float* dy, float eps,  // dx may be dy
                                                              float* dx, float* __restrict__ partial,
                                                              int64_t nrows, int64_t ncols) {
-  __shared__ double red[2][kWavesPerBlock];
+  constexpr int kWaves = BLOCK / kWave;
+  __shared__ double red[2][kWaves];
   const int wave = threadIdx.x / kWave;
   // sum of v (and w) over the workgroup, in every thread; a fixed order
   auto all_sum2 = [&](double v, double w, double* out_w) -> double {
@@ -529,14 +530,21 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __rest
       red[1][wave] = w;
     }
     __syncthreads();
-    *out_w = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
-    return (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    double tv = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    double tw = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+#pragma unroll
+    for (int i = 4; i < kWaves; i += 4) {
+      tv += (red[0][i] + red[0][i + 1]) + (red[0][i + 2] + red[0][i + 3]);
+      tw += (red[1][i] + red[1][i + 1]) + (red[1][i + 2] + red[1][i + 3]);
+    }
+    *out_w = tw;
+    return tv;
   };
   bool in[NG];
   f4 g[NG], dg[NG], db[NG];
 #pragma unroll
   for (int i = 0; i < NG; i++) {
-    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    const int64_t c = ((int64_t)i * BLOCK + threadIdx.x) * 4;
     in[i] = c < ncols;  // ncols is a multiple of 4: a vector is wholly inside or outside
     g[i] = in[i] ? *reinterpret_cast<const f4*>(gamma + c) : f4{0.f, 0.f, 0.f, 0.f};
     dg[i] = db[i] = f4{0.f, 0.f, 0.f, 0.f};
@@ -546,7 +554,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __rest
     f4 xr[NG], dr[NG];
 #pragma unroll
     for (int i = 0; i < NG; i++) {
-      const int64_t at = row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4;
+      const int64_t at = row * ncols + ((int64_t)i * BLOCK + threadIdx.x) * 4;
       xr[i] = dr[i] = f4{0.f, 0.f, 0.f, 0.f};
       if (in[i]) {
         const f4* px = reinterpret_cast<const f4*>(x + at);
@@ -597,7 +605,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __rest
       f4 r;
 #pragma unroll
       for (int c = 0; c < 4; c++) r[c] = rstd * ((dr[i][c] - m1) - xr[i][c] * m2);
-      f4* q = reinterpret_cast<f4*>(dx + row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4);
+      f4* q = reinterpret_cast<f4*>(dx + row * ncols + ((int64_t)i * BLOCK + threadIdx.x) * 4);
       if (NT)
         __builtin_nontemporal_store(r, q);
       else
@@ -608,7 +616,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __rest
 #pragma unroll
   for (int i = 0; i < NG; i++) {
     if (!in[i]) continue;
-    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
+    const int64_t c = ((int64_t)i * BLOCK + threadIdx.x) * 4;
     *reinterpret_cast<f4*>(out + c) = dg[i];
     *reinterpret_cast<f4*>(out + ncols + c) = db[i];
   }
@@ -980,7 +988,8 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   if (nv == 7 && cols != 7 * kWave * 4) nv = 8;
   const bool wide = nv == 0 || nv > 8;  // more than 2048 columns: a workgroup per row
   const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
-  const bool in_pieces = wide && (cols > 8192 || !vec);
+  const bool long_rows = wide && vec && cols > 8192 && cols <= 16384 && rows >= rt().num_cus;  // 1024 threads per row
+  const bool in_pieces = wide && (cols > 8192 || !vec) && !long_rows;
   const int64_t total = (int64_t)rows * cols;
   if ((x < dx + total && dx < x + total) || (dgamma < dbeta + cols && dbeta < dgamma + cols))
     return fail(WF2HIP_EOVERLAP, "LayerNorm backward: dx overlaps x, or dgamma overlaps dbeta");
@@ -996,6 +1005,7 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   // in pieces: enough row groups for two workgroups of 512 threads per compute unit
   const int64_t quarters = ceil_div((int64_t)cols, kApplyCols);
   const int64_t blocks = in_pieces ? std::min<int64_t>({(int64_t)rows, ceil_div(2 * (int64_t)std::max(rt().num_cus, 1), quarters), 65535})
+                         : long_rows ? std::min<int64_t>(rows, (int64_t)std::max(rt().num_cus, 1))
                          : wide  ? std::min<int64_t>(rows, 2 * (int64_t)std::max(rt().num_cus, 1))
                          : tiny ? std::min<int64_t>(ceil_div((int64_t)rows, (int64_t)(cols <= 32 ? 128 : 64)),
                                                     4 * (int64_t)std::max(rt().num_cus, 1))
@@ -1045,6 +1055,13 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
     layernorm_bwd_tiny<<<(uint32_t)blocks, kBlock, 0, rt().stream>>>(x, gamma, dy, eps, dx, (float*)partial, rows, (int)cols,
                                                                      make_fastdiv((uint32_t)cols));
     rc = after_launch("layernorm_bwd_tiny");
+  } else if (long_rows) {
+    hipStream_t st = rt().stream;
+    if (streaming)
+      layernorm_bwd_wide<4, true, 1024><<<(uint32_t)blocks, 1024, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+    else
+      layernorm_bwd_wide<4, false, 1024><<<(uint32_t)blocks, 1024, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+    rc = after_launch("layernorm_bwd_wide");
   } else if (wide) {
     hipStream_t st = rt().stream;
     const int ng = (int)ceil_div(cols, (int64_t)kBlock * 4);

@@ -119,6 +119,8 @@ def test_causal_softmax_backward(gpu, batch, seq):
                                        (257, 1001), (8192, 768),
                                        # beyond 2048 columns: a workgroup per row, 3 ... 8 vectors per thread
                                        (6, 2052), (700, 3072), (33, 4096), (1100, 5120), (5, 6148), (600, 8192),
+                                       # 8196 ... 16384 columns and at least a row per compute unit: the same with 1024 threads
+                                       (300, 16384), (260, 9000), (513, 12292),
                                        # very many rows of at most 64 columns: a thread per row
                                        (16384, 10), (20001, 33), (16400, 64), (16385, 5), (40000, 32)])
 def test_layernorm_backward(gpu, rows, cols):
