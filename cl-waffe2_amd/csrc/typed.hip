@@ -460,16 +460,17 @@ struct TypedRows {
   int64_t odst[WF2HIP_MAX_RANK], osrc[WF2HIP_MAX_RANK];
 };
 
-template <class T, int OP>
+template <class T, int OP, bool NT>
 __global__ __launch_bounds__(kBlock) void typed_rows(T* dst, const T* src, TypedRows p) {
   constexpr int N = 16 / (int)sizeof(T);
-  constexpr int U = 2;
+  constexpr int U = 4;
   using P = Pack<T, N>;
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   const uint32_t lanes = 1u << p.lane_shift;
   const uint32_t sub = threadIdx.x & (lanes - 1);
-  const int64_t row = (int64_t)blockIdx.x * (kBlock >> p.lane_shift) + (threadIdx.x >> p.lane_shift);
-  if (row >= p.nrows) return;
+  const int64_t rows_per_pass = (int64_t)gridDim.x * (kBlock >> p.lane_shift);
+  for (int64_t row = (int64_t)blockIdx.x * (kBlock >> p.lane_shift) + (threadIdx.x >> p.lane_shift); row < p.nrows;
+       row += rows_per_pass) {
   int64_t doff = 0, soff = 0;
   {
     uint64_t rem = (uint64_t)row;
@@ -503,7 +504,10 @@ __global__ __launch_bounds__(kBlock) void typed_rows(T* dst, const T* src, Typed
     for (int u = 0; u < U; u++) {
       const int64_t v = v0 + u * step;
       if (v < nvec) {
-        if (OP != WF2HIP_MOVE) a[u] = *reinterpret_cast<const u4*>(d + head + v * N);
+        if (OP != WF2HIP_MOVE) {
+          const u4* q = reinterpret_cast<const u4*>(d + head + v * N);
+          a[u] = NT ? __builtin_nontemporal_load(q) : *q;
+        }
         __builtin_memcpy(&b[u], s + head + v * N, 16);
       }
     }
@@ -524,9 +528,14 @@ __global__ __launch_bounds__(kBlock) void typed_rows(T* dst, const T* src, Typed
           for (int k = 0; k < N; k++) pr.v[k] = apply<T, OP>(pa.v[k], pb.v[k]);
           r = __builtin_bit_cast(u4, pr);
         }
-        *reinterpret_cast<u4*>(d + head + v * N) = r;
+        u4* q = reinterpret_cast<u4*>(d + head + v * N);
+        if (NT)
+          __builtin_nontemporal_store(r, q);
+        else
+          *q = r;
       }
     }
+  }
   }
 }
 
@@ -552,15 +561,20 @@ static bool try_typed_rows(const Space& s, T* a, const T* b, int* rc) {
   p.lane_shift = 0;
   while (p.lane_shift < 8 && ((int64_t)1 << p.lane_shift) < vecs) p.lane_shift++;
   const int64_t lanes = (int64_t)1 << p.lane_shift;
-  const int64_t gx = ceil_div(p.nrows, (int64_t)kBlock / lanes);
-  if (gx >= ((int64_t)1 << 31)) return false;
-  // along a long row: workgroups of two vectors per lane, as many as fill the device with few rows
-  int64_t gy = ceil_div(vecs, lanes * 2);
+  // at most 64 workgroups per compute unit and position along the row: a workgroup then walks several rows
+  int64_t gx = ceil_div(p.nrows, (int64_t)kBlock / lanes);
+  if (gx > (int64_t)rt().num_cus * 64) gx = (int64_t)rt().num_cus * 64;
+  // along a long row: workgroups of four vectors per lane, as many as fill the device with few rows
+  int64_t gy = ceil_div(vecs, lanes * 4);
   const int64_t fill = ceil_div((int64_t)rt().num_cus * 16, gx);
   if (gy > fill) gy = fill;
   if (gy > 65535) gy = 65535;
   if (gy < 1) gy = 1;
-  typed_rows<T, OP><<<dim3((uint32_t)gx, (uint32_t)gy), kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
+  // far beyond the Infinity Cache: the destination's side nontemporal, as in the contiguous kernels
+  if (s.total * (int64_t)sizeof(T) * (OP != WF2HIP_MOVE ? 3 : 2) >= ((int64_t)192 << 20))
+    typed_rows<T, OP, true><<<dim3((uint32_t)gx, (uint32_t)gy), kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
+  else
+    typed_rows<T, OP, false><<<dim3((uint32_t)gx, (uint32_t)gy), kBlock, 0, rt().stream>>>(a + s.off_a, b + s.off_b, p);
   *rc = after_launch("typed_rows");
   return true;
 }
