@@ -326,9 +326,9 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_lines_kernel(SkinnyParams
 
 // The same product with a workgroup of ONE wavefront per 16 CB columns (rows of W) and slice of K.  The kernel
 // above hands a workgroup 64 columns, so GPT-2's token projection (50257 columns) is 786 workgroups, all
-// resident at once, three on most compute units and four on some: the counters show a compute unit holding a
-// wave for 57 % of the launch only.  1571 one-wavefront workgroups of 32 columns are dealt out as compute units
-// fall free.  Each keeps KSTEPS steps of 32 of K in flight per buffer (8 KB of W with CB = 2, KSTEPS = 2); x
+// resident at once, three on most compute units and four on some, with nothing to even them out, and over
+// K = 768 each of their wavefronts runs three iterations before the four meet in LDS.  1571 one-wavefront
+// workgroups of 32 columns are dealt out as compute units fall free.  Each keeps KSTEPS steps of 32 of K in flight per buffer (8 KB of W with CB = 2, KSTEPS = 2); x
 // comes from the L2 cache, once per workgroup (16 columns per wavefront read x as often as W and run 15 %
 // slower).  No meeting in LDS: a wavefront covers its slice of K alone.
 template <int MT, int CB, int KSTEPS>
