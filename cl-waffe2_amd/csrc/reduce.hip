@@ -1565,6 +1565,114 @@ __global__ __launch_bounds__(kPieceBlock) void layernorm_piece_apply(const float
   r.store(out + (int64_t)row * ncols + c0, left);
 }
 
+// A few very long rows in ONE launch, like softmax_one_launch: a workgroup of 1024 threads holds a piece of
+// 65536 columns in registers, leaves the piece's sum S_p and squared deviations Q_p about a_p = (float)(S_p / n_p),
+// waits -- bounded -- until every piece of the launch has, folds its row's pieces as layernorm_piece_apply does
+// and writes its share: one read and one write of the row.  The same conditions: every workgroup of the grid on
+// the device at once, x and out apart (a workgroup that gives up waiting reads the row itself), one stream.
+__device__ unsigned int g_layernorm_meet[2];
+
+__global__ __launch_bounds__(kLongBlock) void layernorm_one_launch(const float* __restrict__ x,
+                                                                   const float* __restrict__ gamma,
+                                                                   const float* __restrict__ beta, float eps,
+                                                                   float* __restrict__ out, int64_t ncols, uint32_t pieces,
+                                                                   double* psum, double* pdev, uint32_t spins) {
+  __shared__ double lsum[kLongBlock / kWave];
+  __shared__ int met;
+  const uint32_t row = blockIdx.x / pieces, piece = blockIdx.x - row * pieces;
+  const float* xr = x + (int64_t)row * ncols;
+  const int64_t c0 = (int64_t)piece * kOnePiece;
+  float v[kOneE];
+  const uint32_t first = threadIdx.x * 4;
+  const uint32_t left = (uint32_t)((ncols - c0 < kOnePiece ? ncols - c0 : kOnePiece));
+  const float* xp = xr + c0;
+#pragma unroll
+  for (int g = 0; g < kOneE / 4; g++) {
+    f4 t = {0.f, 0.f, 0.f, 0.f};
+    if (first + g * 4 * kLongBlock < left) t = __builtin_nontemporal_load(reinterpret_cast<const f4*>(xp + first + g * 4 * kLongBlock));
+    v[4 * g] = t.x; v[4 * g + 1] = t.y; v[4 * g + 2] = t.z; v[4 * g + 3] = t.w;
+  }
+  double sum = 0.0;
+#pragma unroll
+  for (int k = 0; k < kOneE; k++) sum += (double)v[k];
+  const double total = long_block_sum(sum, lsum);
+  const float a = (float)(total / (double)left);
+  float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int g = 0; g < kOneE / 4; g++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const float d = first + g * 4 * kLongBlock < left ? v[4 * g + c] - a : 0.0f;
+      sq[c] = __builtin_fmaf(d, d, sq[c]);
+    }
+  const double dev = long_block_sum(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3]), lsum);
+  if (threadIdx.x == 0) {
+    // statistics past the caches, waited for, then the arrival (see softmax_one_launch)
+    __hip_atomic_store(&psum[blockIdx.x], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&pdev[blockIdx.x], dev, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __hip_atomic_fetch_add(&g_layernorm_meet[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t polls = 0;
+    while (__hip_atomic_load(&g_layernorm_meet[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x && polls < spins) {
+      __builtin_amdgcn_s_sleep(8);
+      polls++;
+    }
+    met = __hip_atomic_load(&g_layernorm_meet[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= gridDim.x;
+  }
+  __syncthreads();
+  double mean, var;
+  if (met) {
+    const double* rs = psum + (int64_t)row * pieces;
+    const double* rq = pdev + (int64_t)row * pieces;
+    double s = 0.0;
+    for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock)
+      s += __hip_atomic_load(&rs[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    mean = long_block_sum(s, lsum) / (double)ncols;
+    double q = 0.0;
+    for (uint32_t i = threadIdx.x; i < pieces; i += kLongBlock) {
+      const int64_t l = ncols - (int64_t)i * kOnePiece;
+      const double n = (double)(l < kOnePiece ? l : kOnePiece);
+      const double mu = __hip_atomic_load(&rs[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) / n;
+      const double ap = (double)(float)mu;
+      q += __hip_atomic_load(&rq[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + n * ((mu - mean) * (mu - mean) - (mu - ap) * (mu - ap));
+    }
+    var = long_block_sum(q, lsum) / (double)ncols;
+  } else {
+    // gave up waiting: the row's statistics from the row itself (x is not written by this launch)
+    double s = 0.0;
+    for (int64_t c = threadIdx.x; c < ncols; c += kLongBlock) s += (double)xr[c];
+    mean = long_block_sum(s, lsum) / (double)ncols;
+    double q = 0.0;
+    for (int64_t c = threadIdx.x; c < ncols; c += kLongBlock) {
+      const double d = (double)xr[c] - mean;
+      q += d * d;
+    }
+    var = long_block_sum(q, lsum) / (double)ncols;
+  }
+  const float meanf = (float)mean;
+  const float rstd = (float)(1.0 / __builtin_sqrt((var > 0.0 ? var : 0.0) + (double)eps));
+  float* op = out + (int64_t)row * ncols + c0;
+#pragma unroll
+  for (int g = 0; g < kOneE / 4; g++) {
+    const uint32_t at = first + g * 4 * kLongBlock;
+    if (at < left) {
+      const f4 gm = *reinterpret_cast<const f4*>(gamma + c0 + at);
+      const f4 bt = *reinterpret_cast<const f4*>(beta + c0 + at);
+      f4 t;
+#pragma unroll
+      for (int c = 0; c < 4; c++) t[c] = __builtin_fmaf((v[4 * g + c] - meanf) * rstd, gm[c], bt[c]);
+      __builtin_nontemporal_store(t, reinterpret_cast<f4*>(op + at));
+    }
+  }
+  if (threadIdx.x == 0) {
+    const unsigned int before = __hip_atomic_fetch_add(&g_layernorm_meet[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (before + 1 == gridDim.x) {  // everyone has arrived and is past the wait: zero for the next launch
+      __hip_atomic_store(&g_layernorm_meet[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&g_layernorm_meet[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 // Rows of 2049 ... 8192 columns that are a multiple of 4: a workgroup per row with the row in
 // registers (thread t holds the NG 16-byte vectors (g 256 + t) 4 ...), one read and one write
 // where the three-pass form above reads the row three times ((8192, 4096): 82 us).  The
@@ -1838,6 +1946,18 @@ __global__ __launch_bounds__(kBlock) void rows_tiny(TinyRows a, FastDiv by_c) {
 
 // at least this many rows: below it the wavefront forms already finish within a launch's floor
 constexpr int64_t kTinyMinRows = 16384;
+
+static int64_t layernorm_one_launch_capacity() {
+  static const int64_t capacity = [] {
+    int held = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&held, layernorm_one_launch, kLongBlock, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      return (int64_t)0;
+    }
+    return (int64_t)held * rt().num_cus;
+  }();
+  return capacity;
+}
 
 // How many workgroups of softmax_one_launch the device holds at once (0: the form is not used).
 static int64_t softmax_one_launch_capacity() {
@@ -2179,6 +2299,29 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
     if (cols > 8192) {
       const int64_t pieces = ceil_div((int64_t)cols, kPieceCols);
       if (rows * pieces >= ((int64_t)1 << 31)) return fail(WF2HIP_EUNSUPPORTED, "too many row pieces for one launch");
+      // one launch when every workgroup of it is on the device at once, and x and out are apart
+      const int64_t big_pieces = ceil_div((int64_t)cols, kOnePiece);
+      const float* x_end = x + (int64_t)rows * cols;
+      const float* out_end = out + (int64_t)rows * cols;
+      static const bool one_env = [] {
+        const char* e = getenv("WF2HIP_LAYERNORM_ONE_LAUNCH");
+        return !e || atoi(e) != 0;
+      }();
+      // (below 2^22 elements the meeting costs more than the second launch: (100, 20000) 15.7 against 12.8 us)
+      if (one_env && aligned && (int64_t)rows * cols >= ((int64_t)1 << 22) && rows * big_pieces <= layernorm_one_launch_capacity() &&
+          (x_end <= out || out_end <= x)) {
+        const char* spins_env = getenv("WF2HIP_SOFTMAX_MEET_SPINS");  // testing knob, read at every call
+        const uint32_t meet_spins = spins_env ? (uint32_t)atol(spins_env) : kMeetSpins;
+        void* stats = nullptr;
+        WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(rows * big_pieces) * 2 * sizeof(double)));
+        double* psum = static_cast<double*>(stats);
+        double* pdev = psum + rows * big_pieces;
+        layernorm_one_launch<<<(uint32_t)(rows * big_pieces), kLongBlock, 0, st>>>(x, gamma, beta, eps, out, cols,
+                                                                                  (uint32_t)big_pieces, psum, pdev, meet_spins);
+        const int rc = after_launch("layernorm_one_launch");
+        (void)wf2hip_free(stats);  // stream order keeps it alive for the launch above
+        return rc;
+      }
       void* stats = nullptr;  // rows x pieces sums, then as many sums of squared deviations
       WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(rows * pieces) * 2 * sizeof(double)));
       double* psum = static_cast<double*>(stats);

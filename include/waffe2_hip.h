@@ -612,7 +612,8 @@ int wf2hip_causal_softmax_f32(long batch, long seq, const float* x, float* out,
 /* LayerNorm over the last axis: out = (x - mean)/sqrt(var + eps) * g + b
  * (source/nn/norms.lisp:44-82; examples/gpt-2/utils.lisp:114-127).  Rows beyond
  * 8192 columns run in pieces of 16384 columns over several workgroups: two
- * launches and 16 bytes per piece of scratch from the library's pool. */
+ * launches (one where all pieces fit on the device at once and x and out are
+ * apart) and 16 bytes per piece of scratch from the library's pool. */
 int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, const float* gamma,
                               const float* beta, float eps, float* out);
 /* Softmax-Cross-Entropy-Node (source/nn/criterion.lisp:90-126) over the last axis

@@ -398,6 +398,42 @@ def test_layernorm(gpu):
         np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
 
 
+def test_layernorm_long_rows_in_one_launch(gpu, monkeypatch):
+    """A few rows whose pieces of 65536 columns all fit on the device at once: one launch in which every workgroup
+    waits for the others' statistics.  (1, 2^24) fills the device; twice in a row, then a smaller one (the counters
+    of the meeting are left at zero), then with no polls allowed: every workgroup works out the row's statistics by
+    itself.  Against float64."""
+    F = gpu.functional
+    rng = np.random.default_rng(42)
+
+    def check(X, g, b, what):
+        X64 = X.astype(np.float64)
+        mu = X64.mean(axis=1, keepdims=True)
+        var = ((X64 - mu) ** 2).mean(axis=1, keepdims=True)
+        want = (X64 - mu) / np.sqrt(var + 1e-5) * g + b
+        got = F.layer_norm_fused(F.from_numpy(X), F.from_numpy(g), F.from_numpy(b)).numpy()
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=2e-6, err_msg=what)
+        return got
+
+    n = 1 << 24
+    X = (rng.standard_normal((1, n)) * 2 + 0.5).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    for _ in range(2):
+        check(X, g, b, "(1, 2^24)")
+    del X, g, b
+    cols = 65536 * 3 + 8
+    X = (rng.standard_normal((3, cols)) * 3 - 1.0).astype(np.float32)
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    first = check(X, g, b, "(3, 196616)")
+    monkeypatch.setenv("WF2HIP_SOFTMAX_MEET_SPINS", "0")
+    check(X, g, b, "(3, 196616), nobody waits")
+    monkeypatch.delenv("WF2HIP_SOFTMAX_MEET_SPINS")
+    again = check(X, g, b, "(3, 196616) again")
+    np.testing.assert_array_equal(again, first)
+
+
 # ---------------------------------------------------------------------------
 # gemm
 # ---------------------------------------------------------------------------
