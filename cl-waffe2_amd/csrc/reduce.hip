@@ -2003,7 +2003,7 @@ static int softmax_dispatch_as(int64_t nrows, int64_t ncols, const float* x, int
         return !e || atoi(e) != 0;
       }();
       // testing knob, read at every call: with 0 polls every workgroup takes the path of one that gave up waiting
-      const char* spins_env = getenv("WF2HIP_SOFTMAX_MEET_SPINS");
+      const char* spins_env = getenv("WF2HIP_MEET_SPINS");
       const uint32_t meet_spins = spins_env ? (uint32_t)atol(spins_env) : kMeetSpins;
       const bool vec = aligned16(x) && aligned16(out) && ldx % 4 == 0 && ldo % 4 == 0 && ncols % 4 == 0;
       const bool xent_ok = !XENT || (aligned16(xe.labels) && aligned16(xe.loss));
@@ -2310,7 +2310,7 @@ WF2_API int wf2hip_layernorm_rows_f32(long rows, long cols, const float* x, cons
       // (below 2^22 elements the meeting costs more than the second launch: (100, 20000) 15.7 against 12.8 us)
       if (one_env && aligned && (int64_t)rows * cols >= ((int64_t)1 << 22) && rows * big_pieces <= layernorm_one_launch_capacity() &&
           (x_end <= out || out_end <= x)) {
-        const char* spins_env = getenv("WF2HIP_SOFTMAX_MEET_SPINS");  // testing knob, read at every call
+        const char* spins_env = getenv("WF2HIP_MEET_SPINS");  // testing knob, read at every call
         const uint32_t meet_spins = spins_env ? (uint32_t)atol(spins_env) : kMeetSpins;
         void* stats = nullptr;
         WF2_TRY(wf2hip_malloc_uninitialized(&stats, (size_t)(rows * big_pieces) * 2 * sizeof(double)));

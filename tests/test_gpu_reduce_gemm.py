@@ -322,10 +322,10 @@ def test_softmax_long_rows_in_one_launch(gpu, monkeypatch):
     got = F.softmax_fused(F.from_numpy(small)).numpy()
     _assert_softmax(got, want_small, "(3, 196616)")
     assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
-    monkeypatch.setenv("WF2HIP_SOFTMAX_MEET_SPINS", "0")
+    monkeypatch.setenv("WF2HIP_MEET_SPINS", "0")
     alone = F.softmax_fused(F.from_numpy(small)).numpy()
     _assert_softmax(alone, want_small, "(3, 196616), nobody waits")
-    monkeypatch.delenv("WF2HIP_SOFTMAX_MEET_SPINS")
+    monkeypatch.delenv("WF2HIP_MEET_SPINS")
     again = F.softmax_fused(F.from_numpy(small)).numpy()
     np.testing.assert_array_equal(again, got)
 
@@ -427,9 +427,9 @@ def test_layernorm_long_rows_in_one_launch(gpu, monkeypatch):
     g = rng.standard_normal(cols).astype(np.float32)
     b = rng.standard_normal(cols).astype(np.float32)
     first = check(X, g, b, "(3, 196616)")
-    monkeypatch.setenv("WF2HIP_SOFTMAX_MEET_SPINS", "0")
+    monkeypatch.setenv("WF2HIP_MEET_SPINS", "0")
     check(X, g, b, "(3, 196616), nobody waits")
-    monkeypatch.delenv("WF2HIP_SOFTMAX_MEET_SPINS")
+    monkeypatch.delenv("WF2HIP_MEET_SPINS")
     again = check(X, g, b, "(3, 196616) again")
     np.testing.assert_array_equal(again, first)
 
