@@ -711,7 +711,8 @@ def row_table(W, reps: int = 10, warm: int = 3, replay: bool = True):
     ring = ring_of(lambda: T([Nb, Cc, Kk, Kk, Hh, Hh], initial_element=None), 4 * ncol)
     measure("Im2ColNode, padding 1: the walk leaves the last row and column of every plane untouched", ring,
             lambda s: W.nodes.forward("Im2ColNode", padded, s, (1, 1), (1, 1), (1, 1)), 4 * (ncol + nim),
-            note="stores that leave 4 bytes of a line out are merged by the memory system at about half the rate")
+            note="the old values of the elements the walk leaves out are read first (whole lines, four of every seven of col) "
+                 "and written back inside whole 16-byte stores; rate quoted on the bytes of the walk alone")
     back = T([Nb, Cc, Hh + 2, Hh + 2], initial_element=None)
     ring = ring_of(lambda: normal([Nb, Cc, Kk, Kk, Hh, Hh]), 4 * ncol)
     measure("Col2ImNode (32,64,3,3,56,56) -> (32,64,58,58)", ring,

@@ -174,9 +174,23 @@ __global__ __launch_bounds__(kBlock) void im2col_flat(Unfold32 p, ColStep d, uin
 // reuse has to happen inside the workgroup.
 // VEC: every band of every plane of col starts on a 16-byte boundary: a lane takes four consecutive
 // elements and they leave in one 16-byte nontemporal store (single stores where the walk skips one of them).
-template <bool VEC>
-__global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands, uint32_t band_rows) {
-  extern __shared__ float tile[];  // the image rows y0 ..., W floats each
+// SAME (VEC only): without dilation the walk of every kernel offset takes the same steps (i s_h < s_h H_out -
+// pad_h whatever kh is, and likewise along W), so which elements of a vector are reached is worked out once per
+// vector, not once per vector and plane.
+// HOLES (with SAME): the walk along W stops hole_w elements short of the end of every row of col, and what it
+// does not reach keeps its value.  Stores that leave four bytes of a 128-byte line out are merged by the memory
+// system at about half the rate of whole lines, so the workgroup reads those elements of its band of every plane
+// first (kHolesPerThread per thread at most, in flight while the image rows are staged), keeps them in LDS behind
+// the tile -- [plane][row of the band][hole_w], which is the order they come in along the band -- and writes them
+// back inside whole 16-byte stores.  Nothing else writes them during the launch: a band of a plane belongs to
+// one workgroup.  (The padded walk of a (32, 64, 58, 58) image, 3 x 3: 71 us against 94 with single stores
+// around them and 47 without a padding argument; the reads fetch whole 128-byte lines, four of every seven of
+// col, and the kernel moves those bytes at the rate it moves the others.)
+constexpr int kHolesPerThread = 4;
+
+template <bool VEC, bool SAME, bool HOLES>
+__device__ __forceinline__ void im2col_band(float* tile, const Unfold32& p, uint32_t bands, uint32_t band_rows,
+                                            uint32_t tile_floats, uint32_t hole_w) {
   const uint32_t nc = blockIdx.x / bands, band = blockIdx.x - nc * bands;
   const uint32_t i0 = band * band_rows;
   const uint32_t rows_here = p.H_out - i0 < band_rows ? p.H_out - i0 : band_rows;
@@ -185,6 +199,23 @@ __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands,
   const uint32_t want = (rows_here - 1) * p.s_h + p.K_H;
   const uint32_t need = want < p.H - y0 ? want : p.H - y0;
   const float* src = p.src + ((size_t)nc * p.H + y0) * p.W;
+  float* holes = tile + tile_floats;
+  float old[kHolesPerThread];
+  if constexpr (HOLES) {
+    const uint32_t per_plane = rows_here * hole_w, holes_here = p.K_H * p.K_W * per_plane;
+#pragma unroll
+    for (int u = 0; u < kHolesPerThread; u++) {
+      const uint32_t idx = threadIdx.x + u * kBlock;
+      old[u] = 0.0f;
+      if (idx < holes_here) {
+        const uint32_t plane = idx / per_plane, slot = idx - plane * per_plane;
+        const uint32_t il = hole_w == 1 ? slot : slot / hole_w, h = slot - il * hole_w;
+        // rows the walk along H does not reach are left alone altogether
+        if ((i0 + il) * p.s_h < walk_end(1, 0, p.pad_h, p.s_h, p.H_out))
+          old[u] = p.dst[((size_t)nc * p.K_H * p.K_W + plane) * p.plane_elems + (i0 + il) * p.W_out + p.W_out - hole_w + h];
+      }
+    }
+  }
   {  // eight loads in flight per thread
     const uint32_t count = need * p.W;
     uint32_t e = threadIdx.x;
@@ -197,8 +228,74 @@ __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands,
     }
     for (; e < count; e += kBlock) tile[e] = src[e];
   }
+  if constexpr (HOLES) {
+#pragma unroll
+    for (int u = 0; u < kHolesPerThread; u++) holes[threadIdx.x + u * kBlock] = old[u];
+  }
   __syncthreads();
   const uint32_t band_elems = rows_here * p.W_out;
+  if constexpr (SAME) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int NV = 4;  // vectors per thread and pass
+    const uint32_t end_h = walk_end(1, 0, p.pad_h, p.s_h, p.H_out), end_w = walk_end(1, 0, p.pad_w, p.s_w, p.W_out);
+    for (uint32_t base = 0; base < band_elems; base += 4 * kBlock * NV) {
+      uint32_t toff[NV][4];  // tile offset of element c of vector u for kh = kw = 0
+      // bit c: element c of vector u lies inside the band and both walks; bit 4 + c: inside the band and the
+      // walk along H but beyond the one along W (its old value is staged); from bit 8: how many such elements
+      // of the band come before the vector
+      uint32_t reached[NV];
+#pragma unroll
+      for (int u = 0; u < NV; u++) {
+        const uint32_t e = base + 4 * (threadIdx.x + u * kBlock);
+        const bool live = e < band_elems;
+        uint32_t j;
+        uint32_t il = fd_divmod(live ? e : 0, p.by_w_out, &j);
+        reached[u] = 0;
+        if constexpr (HOLES) reached[u] = (il * hole_w + (j > p.W_out - hole_w ? j - (p.W_out - hole_w) : 0)) << 8;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          toff[u][c] = il * p.s_h * p.W + j * p.s_w;
+          if (live && e + c < band_elems && (i0 + il) * p.s_h < end_h) reached[u] |= (j * p.s_w < end_w ? 1u : 16u) << c;
+          if (++j == p.W_out) {
+            j = 0;
+            il++;
+          }
+        }
+      }
+      for (uint32_t plane = 0; plane < p.K_H * p.K_W; plane++) {
+        const uint32_t kh = plane / p.K_W, kw = plane - kh * p.K_W;
+        float* dst = p.dst + ((size_t)nc * p.K_H * p.K_W + plane) * p.plane_elems + i0 * p.W_out + base;
+        const uint32_t shift = kh * p.W + kw;
+        const uint32_t staged0 = tile_floats + plane * rows_here * hole_w;
+#pragma unroll
+        for (int u = 0; u < NV; u++) {
+          float* d = dst + 4 * (threadIdx.x + u * kBlock);
+          if (HOLES ? ((reached[u] | reached[u] >> 4) & 15u) == 15u : (reached[u] & 15u) == 15u) {
+            // one gather for reached elements (from the image rows) and staged ones (behind them)
+            uint32_t at = staged0 + (reached[u] >> 8);
+            f4 v;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+              if constexpr (HOLES) {
+                const bool staged = reached[u] >> (4 + c) & 1;
+                v[c] = tile[staged ? at : toff[u][c] + shift];
+                at += staged;
+              } else {
+                v[c] = tile[toff[u][c] + shift];
+              }
+            }
+            __builtin_nontemporal_store(v, reinterpret_cast<f4*>(d));
+          } else {
+            // around what the walk leaves as it was: single stores
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+              if (reached[u] >> c & 1) d[c] = tile[toff[u][c] + shift];
+          }
+        }
+      }
+    }
+    return;
+  }
   if constexpr (VEC) {
     // A thread's vectors (four consecutive elements of the band) are the same in every (kh, kw) plane:
     // their positions in the band and in the tile are worked out once, and a plane costs four LDS reads,
@@ -261,8 +358,7 @@ __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands,
               if (on[0] && on[1] && on[2] && on[3]) {
                 __builtin_nontemporal_store(v, reinterpret_cast<f4*>(d));
               } else {
-                // around a hole: single stores (reading the vector, merging and writing it back whole is
-                // slower: 114 against 98 us for the padded walk of a (32, 64, 58, 58) image)
+                // around what the walk leaves as it was: single stores
 #pragma unroll
                 for (int c = 0; c < 4; c++)
                   if (on[c]) d[c] = v[c];
@@ -283,15 +379,24 @@ __global__ __launch_bounds__(kBlock) void im2col_lds(Unfold32 p, uint32_t bands,
         uint32_t j;
         const uint32_t il = fd_divmod(e, p.by_w_out, &j);
         const uint32_t y = kh + (i0 + il) * p.s_h, x = kw + j * p.s_w;
-        // What the reference's walk does not reach stays as it was.  (With padding every row
-        // of col ends in such an element, and stores that leave four bytes of a line out are
-        // merged by the memory system at about half the rate: 100 us where the same image
-        // without padding takes 54 us.  Reading the old value and writing it back is slower
-        // still.)
+        // what the reference's walk does not reach stays as it was
         if (y < end_h && x < end_w) dst[e] = tile[(y - y0) * p.W + x];
       }
     }
   }
+}
+
+// (four wavefronts per SIMD: the general form sits at the edge of 128 registers)
+template <bool VEC, bool SAME = false>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 8))) void im2col_lds(Unfold32 p, uint32_t bands, uint32_t band_rows) {
+  extern __shared__ float tile[];  // the image rows y0 ..., W floats each
+  im2col_band<VEC, SAME, false>(tile, p, bands, band_rows, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock)
+void im2col_lds_holes(Unfold32 p, uint32_t bands, uint32_t band_rows, uint32_t tile_floats, uint32_t hole_w) {
+  extern __shared__ float tile[];  // the image rows, then the staged old values
+  im2col_band<true, true, true>(tile, p, bands, band_rows, tile_floats, hole_w);
 }
 
 // col2im: U elements of im per thread, kBlock apart; the kernel offsets are walked kh ascending,
@@ -645,7 +750,23 @@ WF2_API int wf2hip_im2col_f32(float* col, long N, long C, long H, long W, long H
         static const char* vec_env = getenv("WF2HIP_UNFOLD_VEC");  // testing knob: 0 = stores of single elements
         const bool vec = ((uintptr_t)col % 16) == 0 && (H_out * W_out) % 4 == 0 && (band_rows * W_out) % 4 == 0 &&
                          !(vec_env && vec_env[0] == '0');
-        if (vec)
+        bool untouched = false;  // does the walk leave elements of col as they were?
+        for (long k = 0; k < K_H; k++) untouched |= (long)p.count_h[k] < H_out;
+        for (long k = 0; k < K_W; k++) untouched |= (long)p.count_w[k] < W_out;
+        const bool same = vec && untouched && dilation_h == 1 && dilation_w == 1;
+        const int64_t hole_w = W_out - (int64_t)p.count_w[0];  // without dilation: of every kw
+        static const char* holes_env = getenv("WF2HIP_IM2COL_HOLES");  // testing knob: 0 = single stores around them
+        const bool holes = same && hole_w > 0 && hole_w < W_out &&
+                           K_H * K_W * band_rows * hole_w <= (int64_t)kHolesPerThread * kBlock &&
+                           !(holes_env && holes_env[0] == '0');
+        if (holes)
+          im2col_lds_holes<<<(uint32_t)(planes * bands), kBlock,
+                             ((size_t)tile_rows * W + kHolesPerThread * kBlock) * sizeof(float), rt().stream>>>(
+              q, (uint32_t)bands, (uint32_t)band_rows, (uint32_t)(tile_rows * W), (uint32_t)hole_w);
+        else if (same)
+          im2col_lds<true, true><<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
+              q, (uint32_t)bands, (uint32_t)band_rows);
+        else if (vec)
           im2col_lds<true><<<(uint32_t)(planes * bands), kBlock, (size_t)tile_rows * W * sizeof(float), rt().stream>>>(
               q, (uint32_t)bands, (uint32_t)band_rows);
         else

@@ -57,9 +57,10 @@ def test_im2col_random_geometries_match_oracle(gpu, O, seed):
         out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((Hin, Win))]
         H, Wd = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((Hin, Win))]
         im = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
-        want = np.full((N, Cc, k[0], k[1], out[0], out[1]), 3.0, np.float32)
+        start = rng.standard_normal((N, Cc, k[0], k[1], out[0], out[1])).astype(np.float32)
+        want = start.copy()  # what the walk does not reach keeps the value it held
         O.im2col(want, im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
-        col = W.HIPTensor.from_numpy(np.full(want.shape, 3.0, np.float32))
+        col = W.HIPTensor.from_numpy(start)
         W.forward("Im2ColNode", W.HIPTensor.from_numpy(im), col, s, p, (1, 1))
         assert_bit_equal(col.numpy(), want, f"im2col {N, Cc, H, Wd, k, s, p}")
         cin = rng.standard_normal(want.shape).astype(np.float32)
@@ -79,18 +80,24 @@ def test_im2col_random_geometries_match_oracle(gpu, O, seed):
     (2, 2, 61, 67, (2, 3), (3, 4), (1, 1)),       # kernel smaller than the stride
     (3, 2, 57, 57, (3, 3), (2, 2), (1, 1)),       # overlap with stride 2
     (1, 1, 300, 300, (7, 7), (2, 2), (3, 3)),
+    (3, 5, 56, 56, (3, 3), (1, 1), (1, 1)),       # one band per plane, one element short at the end of every row
+    (2, 3, 60, 64, (3, 5), (1, 1), (2, 2)),       # two elements short
+    (2, 2, 120, 98, (5, 5), (1, 1), (1, 3)),      # several bands, three short
+    (8, 64, 56, 56, (3, 3), (1, 1), (1, 1)),      # a whole plane per workgroup, the old values staged
+    (8, 64, 28, 28, (5, 5), (1, 1), (1, 3)),      # more old values than a workgroup stages: single stores around them
 ])
 def test_im2col_larger_geometries_match_oracle(gpu, O, N, Cc, Hin, Win, k, s, p):
     """Each dispatch of the two kernels at sizes of many workgroups, bit for bit against the compiled
-    restatement of the reference's loops (elements its walk does not reach keep the 3.0 they held)."""
+    restatement of the reference's loops (elements its walk does not reach keep the values they held)."""
     W = gpu
     rng = np.random.default_rng(Hin * 1000 + Win)
     out = [(size + 2 * p[a] - (k[a] - 1) - 1) // s[a] + 1 for a, size in enumerate((Hin, Win))]
     H, Wd = [size + 2 * p[a] + out[a] % s[a] for a, size in enumerate((Hin, Win))]
     im = rng.standard_normal((N, Cc, H, Wd)).astype(np.float32)
-    want = np.full((N, Cc, k[0], k[1], out[0], out[1]), 3.0, np.float32)
+    start = rng.standard_normal((N, Cc, k[0], k[1], out[0], out[1])).astype(np.float32)
+    want = start.copy()
     O.im2col(want, im, N, Cc, H, Wd, out[0], out[1], k[0], k[1], p, s, (1, 1))
-    col = W.HIPTensor.from_numpy(np.full(want.shape, 3.0, np.float32))
+    col = W.HIPTensor.from_numpy(start)
     W.forward("Im2ColNode", W.HIPTensor.from_numpy(im), col, s, p, (1, 1))
     assert_bit_equal(col.numpy(), want, "im2col")
     cin = rng.standard_normal(want.shape).astype(np.float32)
