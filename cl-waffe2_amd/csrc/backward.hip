@@ -506,18 +506,18 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_tiny(const float* __rest
   }
 }
 
-// Rows of 2049 ... 8192 columns (BLOCK = 1024 threads: up to 16384): a workgroup per row, thread t holding the NG 16-byte vectors
+// Rows of 2049 ... 8192 columns: a workgroup per row, thread t holding the NG 16-byte vectors
 // (g 256 + t) 4 ... of x, dy and gamma and its share of the two column sums in registers; the
 // row statistics meet in LDS (three exchanges per row).  Workgroup b walks rows b, b + B, ...
 // and leaves its column sums in row b of `partial`, folded like the narrower kernel's.  Same
 // formulas as above: the mean from binary64 sums, deviations and squares in binary32.
-template <int NG, bool NT, int BLOCK = kBlock>
-__global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restrict__ x,
+template <int NG, bool NT>
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_wide(const float* __restrict__ x,
                                                              const float* __restrict__ gamma,
                                                              const float* dy, float eps,  // dx may be dy
                                                              float* dx, float* __restrict__ partial,
                                                              int64_t nrows, int64_t ncols) {
-  constexpr int kWaves = BLOCK / kWave;
+  constexpr int kWaves = kBlock / kWave;
   __shared__ double red[2][kWaves];
   const int wave = threadIdx.x / kWave;
   // sum of v (and w) over the workgroup, in every thread; a fixed order
@@ -544,7 +544,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restr
   f4 g[NG], dg[NG], db[NG];
 #pragma unroll
   for (int i = 0; i < NG; i++) {
-    const int64_t c = ((int64_t)i * BLOCK + threadIdx.x) * 4;
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
     in[i] = c < ncols;  // ncols is a multiple of 4: a vector is wholly inside or outside
     g[i] = in[i] ? *reinterpret_cast<const f4*>(gamma + c) : f4{0.f, 0.f, 0.f, 0.f};
     dg[i] = db[i] = f4{0.f, 0.f, 0.f, 0.f};
@@ -554,7 +554,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restr
     f4 xr[NG], dr[NG];
 #pragma unroll
     for (int i = 0; i < NG; i++) {
-      const int64_t at = row * ncols + ((int64_t)i * BLOCK + threadIdx.x) * 4;
+      const int64_t at = row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4;
       xr[i] = dr[i] = f4{0.f, 0.f, 0.f, 0.f};
       if (in[i]) {
         const f4* px = reinterpret_cast<const f4*>(x + at);
@@ -605,7 +605,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restr
       f4 r;
 #pragma unroll
       for (int c = 0; c < 4; c++) r[c] = rstd * ((dr[i][c] - m1) - xr[i][c] * m2);
-      f4* q = reinterpret_cast<f4*>(dx + row * ncols + ((int64_t)i * BLOCK + threadIdx.x) * 4);
+      f4* q = reinterpret_cast<f4*>(dx + row * ncols + ((int64_t)i * kBlock + threadIdx.x) * 4);
       if (NT)
         __builtin_nontemporal_store(r, q);
       else
@@ -616,9 +616,177 @@ __global__ __launch_bounds__(BLOCK) void layernorm_bwd_wide(const float* __restr
 #pragma unroll
   for (int i = 0; i < NG; i++) {
     if (!in[i]) continue;
-    const int64_t c = ((int64_t)i * BLOCK + threadIdx.x) * 4;
+    const int64_t c = ((int64_t)i * kBlock + threadIdx.x) * 4;
     *reinterpret_cast<f4*>(out + c) = dg[i];
     *reinterpret_cast<f4*>(out + ncols + c) = db[i];
+  }
+}
+
+// Rows of 8193 ... 16384 columns, 16-byte aligned, at least a row per compute unit: layernorm_bwd_wide's row
+// per 1024-thread workgroup with the next row's loads issued before the current row is reduced.  One such
+// workgroup fills a compute unit, and its sixteen wavefronts move through a row in step (load, three exchanges,
+// store), so without the second set of registers nothing is in flight while a row is reduced.  The registers
+// come from the two column sums, which live in LDS instead (2 x 16384 floats, each element read and written by
+// the one thread that owns the column).  Same formulas, same order of accumulation, same layout of `partial`.
+constexpr int kLongNG = 4;  // vectors per thread of the kLongBlock = 1024 threads
+constexpr int kLongCols = kLongBlock * kLongNG * 4;
+constexpr size_t kLongLdsBytes = 2 * (size_t)kLongCols * sizeof(float) + 4 * (kLongBlock / kWave) * sizeof(double);
+
+template <bool NT>
+__global__ __launch_bounds__(kLongBlock) void layernorm_bwd_long(const float* __restrict__ x,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* dy, float eps,  // dx may be dy
+                                                                 float* dx, float* __restrict__ partial,
+                                                                 uint32_t nrows, int64_t ncols) {  // rows are counted in 32 bits: the SALU compares no wider
+  constexpr int kWaves = kLongBlock / kWave, NG = kLongNG;
+  extern __shared__ double long_lds[];
+  double* red = long_lds;                                          // two buffers of [2][kWaves], used in turn
+  f4* acc = reinterpret_cast<f4*>(long_lds + 4 * kWaves);         // [2][NG][kLongBlock]: dgamma, dbeta
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  int turn = 0;
+  // Sums of v and w over the workgroup, in every thread, in a fixed order.  The barrier waits for this
+  // wavefront's LDS traffic only (__syncthreads would also wait for the loads of the next row, which is what
+  // they are issued early to avoid); two buffers in turn, so a wavefront that runs ahead into the next exchange
+  // writes where nobody still reads (it has passed this barrier, so everyone has finished the exchange before).
+  // Lane l reads the partial of wavefront l mod 16 and four butterfly steps leave the total in every lane.
+  auto all_sum2 = [&](double v, double w, double* out_w) -> double {
+    static_assert(kWaves == 16, "the butterfly below folds sixteen partials");
+    v = wave_sum(v);
+    w = wave_sum(w);
+    double* buf = red + turn * 2 * kWaves;
+    turn ^= 1;
+    if (lane == 0) {
+      buf[wave] = v;
+      buf[kWaves + wave] = w;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    double tv = buf[lane & (kWaves - 1)], tw = buf[kWaves + (lane & (kWaves - 1))];
+#pragma unroll
+    for (int o = kWaves / 2; o > 0; o >>= 1) {
+      tv += __shfl_xor(tv, o);
+      tw += __shfl_xor(tw, o);
+    }
+    *out_w = tw;
+    return tv;
+  };
+  auto all_sum = [&](double v) -> double {
+    v = wave_sum(v);
+    double* buf = red + turn * 2 * kWaves;
+    turn ^= 1;
+    if (lane == 0) buf[wave] = v;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    double tv = buf[lane & (kWaves - 1)];
+#pragma unroll
+    for (int o = kWaves / 2; o > 0; o >>= 1) tv += __shfl_xor(tv, o);
+    return tv;
+  };
+  bool in[NG];
+  f4 g[NG];
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    const int64_t c = ((int64_t)i * kLongBlock + threadIdx.x) * 4;
+    in[i] = c < ncols;  // ncols is a multiple of 4: a vector is wholly inside or outside
+    g[i] = in[i] ? *reinterpret_cast<const f4*>(gamma + c) : f4{0.f, 0.f, 0.f, 0.f};
+    acc[i * kLongBlock + threadIdx.x] = f4{0.f, 0.f, 0.f, 0.f};
+    acc[(NG + i) * kLongBlock + threadIdx.x] = f4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float inv_n = 1.0f / (float)ncols;
+  // A row of x, dy or dx is a buffer of ncols floats: loads take a scalar descriptor, one 32-bit lane offset and
+  // a scalar offset per vector (no 64-bit address per load held in registers), a lane past the end of the row
+  // reads zeros and its store is dropped.  No branch around a load, so the loads are straight-line code and
+  // the wait for this row's registers can leave the next row's loads in flight.
+  constexpr int kRawBuffer = 0x00020000;  // dword 3 of a raw buffer descriptor: 32-bit data, no swizzle, no stride
+  constexpr int kAux = NT ? 2 : 0;        // the nt bit
+  const uint32_t lane_off = threadIdx.x * 16;
+  auto row_of = [&](const float* base, uint32_t row) {  // a row past the last one: an empty buffer
+    const bool there = row < nrows;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base + (int64_t)(there ? row : 0u) * ncols), 0,
+                                             there ? (int)(ncols * 4) : 0, kRawBuffer);
+  };
+  // (issued for the row after the last one too, where it reads nothing: with the same instructions on every
+  // path the compiler's wait before a row's first use counts exactly the loads issued after it)
+  auto load = [&](f4 (&xr)[NG], f4 (&dr)[NG], uint32_t row) {
+    const __amdgpu_buffer_rsrc_t rx = row_of(x, row), rd = row_of(dy, row);
+#pragma unroll
+    for (int i = 0; i < NG; i++) {
+      xr[i] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(rx, lane_off, i * kLongBlock * 16, kAux));
+      dr[i] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(rd, lane_off, i * kLongBlock * 16, kAux));
+    }
+  };
+  auto reduce_row = [&](f4 (&xr)[NG], f4 (&dr)[NG], uint32_t row) {
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < NG; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) sum += (double)xr[i][c];
+    const float mean = (float)(all_sum(sum) / (double)ncols);
+    float sq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NG; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float d = in[i] ? xr[i][c] - mean : 0.0f;
+        xr[i][c] = d;
+        sq[c] = __builtin_fmaf(d, d, sq[c]);
+      }
+    const double var = all_sum(((double)sq[0] + (double)sq[1]) + ((double)sq[2] + (double)sq[3])) / (double)ncols;
+    const float rstd = (float)(1.0 / __builtin_sqrt(var + (double)eps));
+    float s1[2] = {0.0f, 0.0f}, s2[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < NG; i++) {
+      f4 dg = acc[i * kLongBlock + threadIdx.x], db = acc[(NG + i) * kLongBlock + threadIdx.x];
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float xh = xr[i][c] * rstd;
+        const float d = dr[i][c];
+        xr[i][c] = xh;
+        dg[c] = __builtin_fmaf(d, xh, dg[c]);
+        db[c] += d;
+        const float dyh = d * g[i][c];
+        dr[i][c] = dyh;
+        s1[c & 1] += dyh;
+        s2[c & 1] = __builtin_fmaf(dyh, xh, s2[c & 1]);
+      }
+      acc[i * kLongBlock + threadIdx.x] = dg;
+      acc[(NG + i) * kLongBlock + threadIdx.x] = db;
+    }
+    double t2;
+    const double t1 = all_sum2((double)s1[0] + (double)s1[1], (double)s2[0] + (double)s2[1], &t2);
+    const float m1 = (float)t1 * inv_n, m2 = (float)t2 * inv_n;
+#pragma unroll
+    for (int i = 0; i < NG; i++) {
+      f4 r;
+#pragma unroll
+      for (int c = 0; c < 4; c++) r[c] = rstd * ((dr[i][c] - m1) - xr[i][c] * m2);
+      if (in[i]) {
+        f4* q = reinterpret_cast<f4*>(dx + (int64_t)row * ncols + ((int64_t)i * kLongBlock + threadIdx.x) * 4);
+        if (NT)
+          __builtin_nontemporal_store(r, q);
+        else
+          *q = r;
+      }
+    }
+  };
+  const uint32_t step = gridDim.x;  // rows + step stays below 2^32: the host keeps rows below 2^31
+  f4 xa[NG], da[NG], xb[NG], db_[NG];
+  uint32_t row = blockIdx.x;
+  load(xa, da, row);
+  while (row < nrows) {
+    load(xb, db_, row + step);
+    reduce_row(xa, da, row);
+    row += step;
+    if (row >= nrows) break;
+    load(xa, da, row + step);
+    reduce_row(xb, db_, row);
+    row += step;
+  }
+  float* out = partial + (int64_t)blockIdx.x * 2 * ncols;
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    if (!in[i]) continue;
+    const int64_t c = ((int64_t)i * kLongBlock + threadIdx.x) * 4;
+    *reinterpret_cast<f4*>(out + c) = acc[i * kLongBlock + threadIdx.x];
+    *reinterpret_cast<f4*>(out + ncols + c) = acc[(NG + i) * kLongBlock + threadIdx.x];
   }
 }
 
@@ -988,7 +1156,7 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
   if (nv == 7 && cols != 7 * kWave * 4) nv = 8;
   const bool wide = nv == 0 || nv > 8;  // more than 2048 columns: a workgroup per row
   const bool vec = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gamma) && cols % 4 == 0;
-  const bool long_rows = wide && vec && cols > 8192 && cols <= 16384 && rows >= rt().num_cus;  // 1024 threads per row
+  const bool long_rows = wide && vec && cols > 8192 && cols <= 16384 && rows >= rt().num_cus && rows < ((int64_t)1 << 31);  // 1024 threads per row
   const bool in_pieces = wide && (cols > 8192 || !vec) && !long_rows;
   const int64_t total = (int64_t)rows * cols;
   if ((x < dx + total && dx < x + total) || (dgamma < dbeta + cols && dbeta < dgamma + cols))
@@ -1057,11 +1225,27 @@ WF2_API int wf2hip_layernorm_backward_f32(long rows, long cols, const float* x, 
     rc = after_launch("layernorm_bwd_tiny");
   } else if (long_rows) {
     hipStream_t st = rt().stream;
+    static bool configured = false;
+    rc = 0;
+    if (!configured) {
+      rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&layernorm_bwd_long<true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongLdsBytes),
+                     "hipFuncSetAttribute(layernorm_bwd_long)");
+      if (rc == 0)
+        rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&layernorm_bwd_long<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongLdsBytes),
+                       "hipFuncSetAttribute(layernorm_bwd_long)");
+      configured = rc == 0;
+    }
+    if (rc != 0) {
+      (void)wf2hip_free(partial);
+      return rc;
+    }
     if (streaming)
-      layernorm_bwd_wide<4, true, 1024><<<(uint32_t)blocks, 1024, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols);
+      layernorm_bwd_long<true><<<(uint32_t)blocks, kLongBlock, kLongLdsBytes, st>>>(x, gamma, dy, eps, dx, (float*)partial, (uint32_t)rows, cols);
     else
-      layernorm_bwd_wide<4, false, 1024><<<(uint32_t)blocks, 1024, 0, st>>>(x, gamma, dy, eps, dx, (float*)partial, rows, cols);
-    rc = after_launch("layernorm_bwd_wide");
+      layernorm_bwd_long<false><<<(uint32_t)blocks, kLongBlock, kLongLdsBytes, st>>>(x, gamma, dy, eps, dx, (float*)partial, (uint32_t)rows, cols);
+    rc = after_launch("layernorm_bwd_long");
   } else if (wide) {
     hipStream_t st = rt().stream;
     const int ng = (int)ceil_div(cols, (int64_t)kBlock * 4);
