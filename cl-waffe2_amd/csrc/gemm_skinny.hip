@@ -381,6 +381,23 @@ __global__ __launch_bounds__(kWave) void sgemm_skinny_wave_kernel(SkinnyParams p
       }
     }
   };
+  // The same for a chunk that lies wholly inside [kbeg, kend): no test and so no branch around a load.  With
+  // branches the compiler's wait before a buffer's first use cannot count the loads issued after it and
+  // waits for all of them, the other buffer's included, which undoes the double buffering.  (Rows of x beyond
+  // the matrix read row 0 and feed accumulator rows that are never stored.)
+  auto fetch_full = [&](int k0, int buf) {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) {
+      const int kq = k0 + 32 * s;
+#pragma unroll
+      for (int q = 0; q < 2 * CB; q++)
+        wv[buf][s][q] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(wrow[q] + kq));
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) xv[buf][s][t][h] = *reinterpret_cast<const f4*>(xrow[t] + kq + 16 * h);
+    }
+  };
   auto multiply = [&](int buf) {
 #pragma unroll
     for (int s = 0; s < KSTEPS; s++)
@@ -405,8 +422,15 @@ __global__ __launch_bounds__(kWave) void sgemm_skinny_wave_kernel(SkinnyParams p
     __builtin_amdgcn_wave_barrier();
   };
   if (kbeg < kend) {
-    fetch(kbeg, 0);
-    for (int k0 = kbeg; k0 < kend; k0 += 64 * KSTEPS) {  // fetches past the end load nothing and multiply zeros
+    int k0 = kbeg;
+    fetch(k0, 0);
+    for (; k0 + 96 * KSTEPS <= kend; k0 += 64 * KSTEPS) {  // the next two chunks are whole
+      fetch_full(k0 + 32 * KSTEPS, 1);
+      multiply(0);
+      fetch_full(k0 + 64 * KSTEPS, 0);
+      multiply(1);
+    }
+    for (; k0 < kend; k0 += 64 * KSTEPS) {  // fetches past the end load nothing and multiply zeros
       fetch(k0 + 32 * KSTEPS, 1);
       multiply(0);
       fetch(k0 + 64 * KSTEPS, 0);
