@@ -136,6 +136,25 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
 #pragma unroll
     for (int t = 0; t < MT; t++) xv[buf][t] = (in && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + k0) : zero;
   };
+  // The same for 16 steps wholly inside the wavefront's part of K: no test, so no branch around a load.  With
+  // branches the compiler's wait before a buffer's first use cannot count the loads issued after it and
+  // waits for all of them -- the fetches meant to stay in flight included.  (Rows of x beyond the matrix read
+  // row 0 and feed accumulator rows that are never stored.)
+  auto fetch_full = [&](int k0, int buf) {
+#pragma unroll
+    for (int q = 0; q < CB; q++) {
+      if (TW) {
+        wv[buf][q] = *reinterpret_cast<const f4*>(wrow[q] + k0);
+      } else if (ALIGNED) {
+        wv[buf][q] = *reinterpret_cast<const f4*>(wrow[q] + (int64_t)k0 * p.ldw);
+      } else {
+#pragma unroll
+        for (int b = 0; b < 4; b++) wv[buf][q][b] = wrow[b][(int64_t)(k0 + q) * p.ldw];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++) xv[buf][t] = *reinterpret_cast<const f4*>(xrow[t] + k0);
+  };
   auto multiply = [&](int buf) {
 #pragma unroll
     for (int s = 0; s < 4; s++)
@@ -151,7 +170,15 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_kernel(SkinnyParams p) {
   if (kbeg < kend) {
 #pragma unroll
     for (int b = 0; b < NB - 1; b++) fetch(kbeg + 16 * b, b);
-    for (int k0 = kbeg; k0 < kend; k0 += 16 * NB) {
+    int k0 = kbeg;
+    for (; k0 + 16 * (2 * NB - 1) <= kend; k0 += 16 * NB) {  // every fetch of the round is whole
+#pragma unroll
+      for (int b = 0; b < NB; b++) {
+        fetch_full(k0 + 16 * (b + NB - 1), (b + NB - 1) % NB);
+        multiply(b);
+      }
+    }
+    for (; k0 < kend; k0 += 16 * NB) {
 #pragma unroll
       for (int b = 0; b < NB; b++) {
         fetch(k0 + 16 * (b + NB - 1), (b + NB - 1) % NB);
@@ -255,6 +282,14 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_lines_kernel(SkinnyParams
         xv[buf][t][h] = (xin && xlive[t]) ? *reinterpret_cast<const f4*>(xrow[t] + k0 + 16 * h) : zero;
     }
   };
+  auto fetch_full = [&](int k0, int buf) {  // 32 steps wholly inside: no branch around a load (see above)
+#pragma unroll
+    for (int q = 0; q < 8; q++) wv[buf][q] = *reinterpret_cast<const f4*>(wrow[q] + k0);
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int t = 0; t < MT; t++) xv[buf][t][h] = *reinterpret_cast<const f4*>(xrow[t] + k0 + 16 * h);
+  };
   auto multiply = [&](int buf) {
 #pragma unroll
     for (int q = 0; q < 8; q++) *reinterpret_cast<f4*>(piece + (8 * q + lrow) * kPitch + lk) = wv[buf][q];
@@ -275,8 +310,17 @@ __global__ __launch_bounds__(kBlock) void sgemm_skinny_lines_kernel(SkinnyParams
     __builtin_amdgcn_wave_barrier();
   };
   if (kbeg < kend) {
-    fetch(kbeg, 0);
-    for (int k0 = kbeg; k0 < kend; k0 += 64) {  // fetches past the end load nothing and multiply zeros
+    int k0 = kbeg;
+    fetch(k0, 0);
+    // (from 17 rows on: (32, 8192) . (8192, 8192)^T 74.7 -> 71.9 us; with one tile of rows the loads this keeps
+    // in flight slow the kernel down, 58.8 -> 65.6 us at 16 rows)
+    for (; MT >= 2 && k0 + 96 <= kend; k0 += 64) {  // the next two pieces are whole
+      fetch_full(k0 + 32, 1);
+      multiply(0);
+      fetch_full(k0 + 64, 0);
+      multiply(1);
+    }
+    for (; k0 < kend; k0 += 64) {  // fetches past the end load nothing and multiply zeros
       fetch(k0 + 32, 1);
       multiply(0);
       fetch(k0 + 64, 0);
