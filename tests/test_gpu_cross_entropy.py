@@ -55,12 +55,14 @@ def test_truth_identities():
 
 
 # every row form of the kernel: four rows per wavefront (256 columns and fewer), two (512), one (768 ... 4096,
-# 1024 as two wavefronts per row), a workgroup of 1024 threads per row up to 65536 columns (8, 16, 32, 52, 64
-# elements per thread), three passes beyond; row counts that leave ragged last workgroups; from 16384 rows of at
+# 1024 as two wavefronts per row), a workgroup of 1024 threads per row up to 65536 columns (2, 4, 8, 13, 16
+# vectors per thread), three passes beyond; row counts that leave ragged last workgroups; from 16384 rows of at
 # most 64 columns on, a thread per row
 SHAPES = [(20001, 10), (16390, 33), (16384, 64), (16384, 32), (16390, 1), (17000, 31), (40000, 4), (100, 10), (7, 3), (1, 1), (257, 256), (65, 500), (33, 768), (101, 1000), (64, 1024), (9, 1537),
           (11, 2048), (6, 3072), (5, 4096), (4, 5000), (3, 50257), (5, 8192), (4, 8197), (3, 20000), (3, 32768),
-          (3, 60000), (3, 66000)]
+          (3, 60000), (3, 66000),
+          # at least a row per compute unit: a workgroup per row up to 65536 columns, rows off a 16-byte boundary
+          (260, 8195), (257, 20001), (258, 40001), (257, 50257), (256, 65536)]
 
 
 @pytest.mark.parametrize("rows,cols", SHAPES)

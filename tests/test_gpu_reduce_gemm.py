@@ -280,6 +280,22 @@ def test_softmax_widths(gpu, cols):
     _assert_softmax(got, _softmax64(X), f"{cols} columns")
 
 
+@pytest.mark.parametrize("rows,cols", [(300, 4100), (260, 8195), (258, 16384), (257, 20001), (260, 32770), (260, 50257),
+                                       (257, 53248), (257, 53249), (256, 65536), (258, 65535)])
+def test_softmax_a_workgroup_per_row(gpu, rows, cols):
+    """At least a row per compute unit and 4097 ... 65536 columns: a workgroup of 1024 threads per row holding
+    2, 4, 8, 13 or 16 vectors of four columns per thread, rows that start off a 16-byte boundary (odd lengths),
+    lengths that are no multiple of four, and the largest row of every form."""
+    F = gpu.functional
+    rng = np.random.default_rng(rows * 31 + cols)
+    X = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    X[0, cols - 1] = 30.0          # the maximum in the last column
+    X[1, : cols // 2] = -np.inf    # half a row that contributes nothing
+    got = F.softmax_fused(F.from_numpy(X)).numpy()
+    _assert_softmax(got, _softmax64(X), f"({rows}, {cols})")
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < 1e-5
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 16385), (1, 1 << 22), (3, 16384 * 5 + 7), (300, 32768), (300, 70001), (2, 1234567)])
 def test_softmax_rows_in_pieces(gpu, rows, cols):
     """Rows handled as pieces of 16384 columns whose maxima and sums are folded afterwards: pieces that hold the
