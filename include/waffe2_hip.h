@@ -749,7 +749,9 @@ int wf2hip_matmul_fused(const wf2hip_matmul_desc* desc, const float* A, const fl
  * (cl-waffe2-simd/kernels/im2col.c:63-115, 395-448), same argument order and the
  * same walk: for kernel offset k the positions k, k + stride, ... below
  * dilation * k - pad + stride * out are visited.  Elements of Col the walk does
- * not reach are left untouched; col2im overwrites X and accumulates in the
+ * not reach keep their values (with a padding argument the call may read them and
+ * store them back unchanged, so Col must be readable and nothing else may write
+ * it during the call); col2im overwrites X and accumulates in the
  * reference's order (kernel rows, then kernel columns, ascending).  Geometries
  * whose walk would leave its plane of Col (dilation > 1) return
  * WF2HIP_EUNSUPPORTED.  Tensors in cl-waffe2's default (:column) order. */
